@@ -1,0 +1,123 @@
+"""ctypes binding of ``libcueq_amd.so`` (the C ABI declared in ``include/cueq_amd.h``).
+
+The library is loaded from inside the package directory.  There is no fallback: if the
+shared object is missing or an entry point fails, an exception is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libcueq_amd.so"
+
+# enum cueq_dtype
+F32, F64, F16, BF16 = 0, 1, 2, 3
+# enum cueq_batch_dim
+BATCH_DIM_AUTO, BATCH_DIM_SHARED, BATCH_DIM_BATCHED, BATCH_DIM_INDEXED = -1, 0, 1, 2
+
+EXPORTED_SYMBOLS = (
+    "cueq_last_error",
+    "cueq_version",
+    "cueq_u1d_plan_create",
+    "cueq_u1d_plan_destroy",
+    "cueq_u1d_workspace_size",
+    "cueq_u1d_run",
+    "cueq_segment_csr_workspace",
+    "cueq_segment_csr_build",
+)
+
+
+class U1dDesc(C.Structure):
+    _fields_ = [
+        ("math_dtype", C.c_int32),
+        ("operand_extent", C.c_int64),
+        ("num_inputs", C.c_int32),
+        ("num_outputs", C.c_int32),
+        ("buffer_dim", C.POINTER(C.c_int32)),
+        ("buffer_num_segments", C.POINTER(C.c_int32)),
+        ("num_operations", C.c_int32),
+        ("num_operands", C.POINTER(C.c_int32)),
+        ("operations", C.POINTER(C.c_int32)),
+        ("num_paths", C.POINTER(C.c_int32)),
+        ("path_indices_start", C.POINTER(C.c_int64)),
+        ("path_coefficients_start", C.POINTER(C.c_int64)),
+        ("path_indices", C.POINTER(C.c_int32)),
+        ("path_indices_len", C.c_int64),
+        ("path_coefficients", C.POINTER(C.c_double)),
+        ("path_coefficients_len", C.c_int64),
+    ]
+
+
+class U1dBuffer(C.Structure):
+    _fields_ = [
+        ("data", C.c_void_p),
+        ("rows", C.c_int64),
+        ("dtype", C.c_int32),
+        ("batch_dim", C.c_int32),
+        ("index", C.c_void_p),
+        ("index_is_64", C.c_int32),
+        ("csr_offsets", C.c_void_p),
+        ("csr_perm", C.c_void_p),
+    ]
+
+
+class CueqError(RuntimeError):
+    pass
+
+
+_lock = threading.Lock()
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library once and declare the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m cuequivariance_amd.build` "
+                "(hipcc, gfx950). This package has no non-HIP execution path."
+            )
+        lib = C.CDLL(str(LIB_PATH))
+        lib.cueq_last_error.restype = C.c_char_p
+        lib.cueq_version.restype = C.c_char_p
+        lib.cueq_u1d_plan_create.argtypes = [C.POINTER(U1dDesc), C.POINTER(C.c_void_p)]
+        lib.cueq_u1d_plan_create.restype = C.c_int
+        lib.cueq_u1d_plan_destroy.argtypes = [C.c_void_p]
+        lib.cueq_u1d_plan_destroy.restype = None
+        lib.cueq_u1d_workspace_size.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64]
+        lib.cueq_u1d_workspace_size.restype = C.c_int64
+        lib.cueq_u1d_run.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]
+        lib.cueq_u1d_run.restype = C.c_int
+        lib.cueq_segment_csr_workspace.argtypes = [C.c_int64, C.c_int64]
+        lib.cueq_segment_csr_workspace.restype = C.c_int64
+        lib.cueq_segment_csr_build.argtypes = [
+            C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
+        ]
+        lib.cueq_segment_csr_build.restype = C.c_int
+        _lib = lib
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().cueq_last_error().decode("utf-8", "replace")
+        raise CueqError(f"{what} failed (status {status}): {msg}")
+
+
+def int32_array(values):
+    return (C.c_int32 * max(1, len(values)))(*values)
+
+
+def int64_array(values):
+    return (C.c_int64 * max(1, len(values)))(*values)
+
+
+def double_array(values):
+    return (C.c_double * max(1, len(values)))(*values)

@@ -1,0 +1,414 @@
+// uniform-1d executor: plan creation and the table-driven kernels.
+//
+// A plan regroups the descriptor's paths by (output buffer, output segment) and uploads
+// them once.  Every output element is owned by one thread (or one wavefront when a
+// scalar output contracts the channel mode), which walks the batch rows that
+// contribute to it and the paths of its segment in a fixed order: no atomics, results
+// are bit-reproducible from run to run.
+//
+// Semantics follow the reference's PyTorch executor,
+// cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_naive.py:61-160
+// (per path: coefficient * product of the operand segments, summed per output segment) and
+// :376-433 (gather of indexed inputs, scatter-add of indexed outputs, sum over the batch
+// for a one-row output).
+
+#include <algorithm>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace cueq {
+
+static thread_local std::string g_error;
+
+void set_error(const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_error = buf;
+}
+
+constexpr int kMaxBuffers = 16;   // inputs + outputs of one polynomial
+constexpr int kMaxInOperands = 7; // input operands of one path
+constexpr int kShareChunk = 128;  // batch rows folded by one thread when an output is shared
+
+struct DevBuffer {
+  const void* data;
+  const void* index;
+  int64_t rows;
+  int32_t dtype;
+  int32_t mode;
+  int32_t index_is_64;
+  int32_t dim;
+  int32_t nseg;
+  int32_t pad;
+};
+
+struct KernelArgs {
+  DevBuffer buf[kMaxBuffers];
+  // path tables of the output buffer being computed
+  const double* coeff;
+  const int32_t* nin;       // inputs of each path
+  const int32_t* in;        // [npaths * kMaxInOperands] packed (buffer << 24) | segment
+  const int32_t* seg_start; // [nseg_out + 1]
+  void* out;                // output tensor, or the partial buffer when chunking a shared output
+  const int64_t* csr_offsets;
+  const int64_t* csr_perm;
+  int64_t out_rows;  // rows of `out` as addressed by this launch
+  int64_t batch;
+  int32_t out_dtype;
+  int32_t out_mode;  // CUEQ_BATCH_*; SHARED here means "row r folds batch rows [r*chunk, (r+1)*chunk)"
+  int32_t out_dim;
+  int32_t out_nseg;
+  int32_t extent;
+  int32_t chunk;
+};
+
+template <typename M>
+__device__ __forceinline__ M path_product(const KernelArgs& a, int p, int64_t z, int u) {
+  M prod = static_cast<M>(a.coeff[p]);
+  const int n = a.nin[p];
+  for (int k = 0; k < n; ++k) {
+    const int32_t packed = a.in[p * kMaxInOperands + k];
+    const DevBuffer& b = a.buf[packed >> 24];
+    const int seg = packed & 0xffffff;
+    int64_t row = 0;
+    if (b.mode == CUEQ_BATCH_BATCHED) row = z;
+    else if (b.mode == CUEQ_BATCH_INDEXED) row = load_index(b.index, b.index_is_64, z);
+    const int64_t width = b.dim ? static_cast<int64_t>(b.nseg) * a.extent : b.nseg;
+    const int64_t off = row * width + (b.dim ? static_cast<int64_t>(seg) * a.extent + u : seg);
+    prod *= load_as<M>(b.data, b.dtype, off);
+  }
+  return prod;
+}
+
+template <typename M>
+__device__ __forceinline__ void z_range(const KernelArgs& a, int64_t r, int64_t& z0, int64_t& z1) {
+  if (a.out_mode == CUEQ_BATCH_BATCHED) { z0 = r; z1 = r + 1; }
+  else if (a.out_mode == CUEQ_BATCH_INDEXED) { z0 = a.csr_offsets[r]; z1 = a.csr_offsets[r + 1]; }
+  else { z0 = r * a.chunk; z1 = min(z0 + a.chunk, a.batch); }
+}
+
+// One thread per output element (row, segment, channel).
+template <typename M>
+__global__ void __launch_bounds__(256) u1d_generic_elem(KernelArgs a) {
+  const int ext_out = a.out_dim ? a.extent : 1;
+  const int64_t per_row = static_cast<int64_t>(a.out_nseg) * ext_out;
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= a.out_rows * per_row) return;
+  const int64_t r = tid / per_row;
+  const int rem = static_cast<int>(tid - r * per_row);
+  const int s = rem / ext_out, u = rem - s * ext_out;
+  int64_t z0, z1;
+  z_range<M>(a, r, z0, z1);
+  const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
+  M acc = 0;
+  for (int64_t zz = z0; zz < z1; ++zz) {
+    const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
+    for (int p = p0; p < p1; ++p) acc += path_product<M>(a, p, z, u);
+  }
+  store_as<M>(a.out, a.out_dtype, tid, acc);
+}
+
+// One wavefront per scalar output element (row, segment): lanes stride over the channel
+// mode, then a fixed-shape butterfly reduction.
+template <typename M>
+__global__ void __launch_bounds__(256) u1d_generic_wave(KernelArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wid = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+  if (wid >= a.out_rows * a.out_nseg) return;
+  const int64_t r = wid / a.out_nseg;
+  const int s = static_cast<int>(wid - r * a.out_nseg);
+  int64_t z0, z1;
+  z_range<M>(a, r, z0, z1);
+  const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
+  M acc = 0;
+  for (int64_t zz = z0; zz < z1; ++zz) {
+    const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
+    for (int p = p0; p < p1; ++p)
+      for (int u = lane; u < a.extent; u += 64) acc += path_product<M>(a, p, z, u);
+  }
+  for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 64);
+  if (lane == 0) store_as<M>(a.out, a.out_dtype, wid, acc);
+}
+
+// out[e] = sum over chunks c (ascending) of partial[c, e]
+template <typename M>
+__global__ void __launch_bounds__(256) u1d_fold_chunks(const M* partial, int64_t nchunks, int64_t width, void* out,
+                                                       int out_dtype) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (e >= width) return;
+  M acc = 0;
+  for (int64_t c = 0; c < nchunks; ++c) acc += partial[c * width + e];
+  store_as<M>(out, out_dtype, e, acc);
+}
+
+struct OutTables {
+  int32_t npaths = 0;
+  double* coeff = nullptr;
+  int32_t* nin = nullptr;
+  int32_t* in = nullptr;
+  int32_t* seg_start = nullptr;
+  bool contracts_channel = false;  // scalar output fed by channel-carrying inputs
+};
+
+}  // namespace cueq
+
+using namespace cueq;
+
+struct cueq_u1d_plan {
+  int32_t math_dtype;
+  int32_t extent;
+  int32_t num_inputs, num_outputs;
+  std::vector<int32_t> buffer_dim, buffer_nseg;
+  std::vector<OutTables> out;  // one per output buffer
+  void* device_blob = nullptr;
+  int device = 0;
+};
+
+extern "C" const char* cueq_last_error(void) { return g_error.c_str(); }
+extern "C" const char* cueq_version(void) { return "cueq_amd 0.1 (gfx950)"; }
+
+extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_plan) {
+  CUEQ_REQUIRE(d && out_plan, CUEQ_ERR_INVALID, "null argument");
+  CUEQ_REQUIRE(d->math_dtype == CUEQ_F32 || d->math_dtype == CUEQ_F64, CUEQ_ERR_INVALID,
+               "math_dtype must be f32 or f64");
+  const int nbuf = d->num_inputs + d->num_outputs;
+  CUEQ_REQUIRE(d->num_inputs >= 0 && d->num_outputs >= 1 && nbuf <= kMaxBuffers, CUEQ_ERR_UNSUPPORTED,
+               "polynomial has %d buffers, at most %d are supported", nbuf, kMaxBuffers);
+  CUEQ_REQUIRE(d->operand_extent >= 1 && d->operand_extent < (1 << 24), CUEQ_ERR_INVALID, "bad operand_extent");
+  for (int b = 0; b < nbuf; ++b) {
+    CUEQ_REQUIRE(d->buffer_dim[b] == 0 || d->buffer_dim[b] == 1, CUEQ_ERR_INVALID, "buffer_dim must be 0 or 1");
+    CUEQ_REQUIRE(d->buffer_num_segments[b] >= 0 && d->buffer_num_segments[b] < (1 << 24), CUEQ_ERR_INVALID,
+                 "bad segment count for buffer %d", b);
+  }
+
+  struct HostPath { int out_seg; double c; int nin; int32_t in[kMaxInOperands]; };
+  std::vector<std::vector<HostPath>> per_out(d->num_outputs);
+  std::vector<bool> contracts(d->num_outputs, false);
+
+  int64_t op_off = 0;
+  for (int o = 0; o < d->num_operations; ++o) {
+    const int nop = d->num_operands[o];
+    CUEQ_REQUIRE(nop >= 1 && nop <= kMaxInOperands + 1, CUEQ_ERR_UNSUPPORTED, "operation %d has %d operands", o, nop);
+    const int32_t* bufs = d->operations + op_off;
+    op_off += nop;
+    int out_pos = -1;
+    for (int k = 0; k < nop; ++k) {
+      CUEQ_REQUIRE(bufs[k] >= 0 && bufs[k] < nbuf, CUEQ_ERR_INVALID, "operation %d: buffer id out of range", o);
+      if (bufs[k] >= d->num_inputs) {
+        CUEQ_REQUIRE(out_pos < 0, CUEQ_ERR_INVALID, "operation %d has more than one output buffer", o);
+        out_pos = k;
+      }
+    }
+    CUEQ_REQUIRE(out_pos >= 0, CUEQ_ERR_INVALID, "operation %d has no output buffer", o);
+    const int ob = bufs[out_pos] - d->num_inputs;
+    const int64_t pi0 = d->path_indices_start[o], pc0 = d->path_coefficients_start[o];
+    CUEQ_REQUIRE(pi0 >= 0 && pi0 + static_cast<int64_t>(d->num_paths[o]) * nop <= d->path_indices_len &&
+                     pc0 >= 0 && pc0 + d->num_paths[o] <= d->path_coefficients_len,
+                 CUEQ_ERR_INVALID, "operation %d: path tables out of range", o);
+    for (int p = 0; p < d->num_paths[o]; ++p) {
+      HostPath hp{};
+      hp.c = d->path_coefficients[pc0 + p];
+      hp.nin = 0;
+      for (int k = 0; k < nop; ++k) {
+        const int seg = d->path_indices[pi0 + static_cast<int64_t>(p) * nop + k];
+        CUEQ_REQUIRE(seg >= 0 && seg < d->buffer_num_segments[bufs[k]], CUEQ_ERR_INVALID,
+                     "operation %d path %d: segment %d out of range for buffer %d", o, p, seg, bufs[k]);
+        if (k == out_pos) hp.out_seg = seg;
+        else {
+          hp.in[hp.nin++] = (bufs[k] << 24) | seg;
+          if (d->buffer_dim[bufs[k]] == 1 && d->buffer_dim[bufs[out_pos]] == 0 && d->operand_extent > 1)
+            contracts[ob] = true;
+        }
+      }
+      per_out[ob].push_back(hp);
+    }
+  }
+
+  auto* plan = new cueq_u1d_plan();
+  plan->math_dtype = d->math_dtype;
+  plan->extent = static_cast<int32_t>(d->operand_extent);
+  plan->num_inputs = d->num_inputs;
+  plan->num_outputs = d->num_outputs;
+  plan->buffer_dim.assign(d->buffer_dim, d->buffer_dim + nbuf);
+  plan->buffer_nseg.assign(d->buffer_num_segments, d->buffer_num_segments + nbuf);
+  plan->out.resize(d->num_outputs);
+  if (hipGetDevice(&plan->device) != hipSuccess) plan->device = 0;
+
+  // Lay all tables out in one host blob, then one upload.
+  size_t total = 0;
+  auto reserve = [&](size_t bytes) { size_t o = total; total += (bytes + 15) & ~size_t(15); return o; };
+  struct Off { size_t coeff, nin, in, seg; };
+  std::vector<Off> offs(d->num_outputs);
+  for (int ob = 0; ob < d->num_outputs; ++ob) {
+    auto& v = per_out[ob];
+    std::stable_sort(v.begin(), v.end(), [](const HostPath& x, const HostPath& y) { return x.out_seg < y.out_seg; });
+    const int nseg = d->buffer_num_segments[d->num_inputs + ob];
+    offs[ob].coeff = reserve(v.size() * sizeof(double));
+    offs[ob].nin = reserve(v.size() * sizeof(int32_t));
+    offs[ob].in = reserve(v.size() * kMaxInOperands * sizeof(int32_t));
+    offs[ob].seg = reserve((nseg + 1) * sizeof(int32_t));
+  }
+  std::vector<char> host(total ? total : 16, 0);
+  for (int ob = 0; ob < d->num_outputs; ++ob) {
+    auto& v = per_out[ob];
+    const int nseg = d->buffer_num_segments[d->num_inputs + ob];
+    auto* coeff = reinterpret_cast<double*>(host.data() + offs[ob].coeff);
+    auto* nin = reinterpret_cast<int32_t*>(host.data() + offs[ob].nin);
+    auto* in = reinterpret_cast<int32_t*>(host.data() + offs[ob].in);
+    auto* seg = reinterpret_cast<int32_t*>(host.data() + offs[ob].seg);
+    std::vector<int32_t> count(nseg + 1, 0);
+    for (size_t p = 0; p < v.size(); ++p) {
+      coeff[p] = v[p].c;
+      nin[p] = v[p].nin;
+      std::memcpy(in + p * kMaxInOperands, v[p].in, sizeof(v[p].in));
+      count[v[p].out_seg + 1]++;
+    }
+    seg[0] = 0;
+    for (int s = 0; s < nseg; ++s) seg[s + 1] = seg[s] + count[s + 1];
+  }
+  hipError_t e = hipMalloc(&plan->device_blob, host.size());
+  if (e == hipSuccess) e = hipMemcpy(plan->device_blob, host.data(), host.size(), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    set_error("uploading plan tables failed: %s", hipGetErrorString(e));
+    if (plan->device_blob) (void)hipFree(plan->device_blob);
+    delete plan;
+    return CUEQ_ERR_HIP;
+  }
+  char* base = static_cast<char*>(plan->device_blob);
+  for (int ob = 0; ob < d->num_outputs; ++ob) {
+    OutTables& t = plan->out[ob];
+    t.npaths = static_cast<int32_t>(per_out[ob].size());
+    t.coeff = reinterpret_cast<double*>(base + offs[ob].coeff);
+    t.nin = reinterpret_cast<int32_t*>(base + offs[ob].nin);
+    t.in = reinterpret_cast<int32_t*>(base + offs[ob].in);
+    t.seg_start = reinterpret_cast<int32_t*>(base + offs[ob].seg);
+    t.contracts_channel = contracts[ob];
+  }
+  *out_plan = plan;
+  return CUEQ_OK;
+}
+
+extern "C" void cueq_u1d_plan_destroy(cueq_u1d_plan* plan) {
+  if (!plan) return;
+  if (plan->device_blob) (void)hipFree(plan->device_blob);
+  delete plan;
+}
+
+static int64_t share_chunks(int64_t batch) { return (batch + kShareChunk - 1) / kShareChunk; }
+
+extern "C" int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch) {
+  if (!plan || !buffers) return 0;
+  const int msize = plan->math_dtype == CUEQ_F64 ? 8 : 4;
+  int64_t need = 0;
+  for (int ob = 0; ob < plan->num_outputs; ++ob) {
+    const int b = plan->num_inputs + ob;
+    if (buffers[b].batch_dim != CUEQ_BATCH_SHARED) continue;
+    const int64_t nch = share_chunks(batch);
+    if (nch <= 1) continue;
+    const int64_t width = static_cast<int64_t>(plan->buffer_nseg[b]) * (plan->buffer_dim[b] ? plan->extent : 1);
+    need = std::max<int64_t>(need, nch * width * msize);
+  }
+  return need;
+}
+
+template <typename M>
+static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch, void* workspace,
+                     int64_t workspace_bytes, hipStream_t stream) {
+  const int nbuf = plan->num_inputs + plan->num_outputs;
+  KernelArgs a{};
+  for (int b = 0; b < nbuf; ++b) {
+    const cueq_u1d_buffer& s = buffers[b];
+    CUEQ_REQUIRE(s.batch_dim == CUEQ_BATCH_SHARED || s.batch_dim == CUEQ_BATCH_BATCHED ||
+                     s.batch_dim == CUEQ_BATCH_INDEXED,
+                 CUEQ_ERR_INVALID, "buffer %d: batch_dim must be resolved (shared/batched/indexed)", b);
+    CUEQ_REQUIRE(s.dtype >= CUEQ_F32 && s.dtype <= CUEQ_BF16, CUEQ_ERR_INVALID, "buffer %d: bad dtype", b);
+    CUEQ_REQUIRE(s.rows >= 0, CUEQ_ERR_INVALID, "buffer %d: negative row count", b);
+    const int64_t width = static_cast<int64_t>(plan->buffer_nseg[b]) * (plan->buffer_dim[b] ? plan->extent : 1);
+    CUEQ_REQUIRE(s.data != nullptr || s.rows * width == 0, CUEQ_ERR_INVALID, "buffer %d: null data", b);
+    if (s.batch_dim == CUEQ_BATCH_SHARED) CUEQ_REQUIRE(s.rows == 1, CUEQ_ERR_INVALID, "buffer %d: shared buffer must have one row", b);
+    if (s.batch_dim == CUEQ_BATCH_BATCHED) CUEQ_REQUIRE(s.rows == batch, CUEQ_ERR_INVALID, "buffer %d: %lld rows, batch size is %lld", b, (long long)s.rows, (long long)batch);
+    if (s.batch_dim == CUEQ_BATCH_INDEXED) {
+      CUEQ_REQUIRE(s.index != nullptr || batch == 0, CUEQ_ERR_INVALID, "buffer %d: indexed without index tensor", b);
+      if (b >= plan->num_inputs)
+        CUEQ_REQUIRE(s.csr_offsets != nullptr && (s.csr_perm != nullptr || batch == 0), CUEQ_ERR_INVALID,
+                     "output buffer %d is indexed: csr_offsets/csr_perm are required", b);
+    }
+    DevBuffer& dbuf = a.buf[b];
+    dbuf.data = s.data;
+    dbuf.index = s.index;
+    dbuf.rows = s.rows;
+    dbuf.dtype = s.dtype;
+    dbuf.mode = s.batch_dim;
+    dbuf.index_is_64 = s.index_is_64;
+    dbuf.dim = plan->buffer_dim[b];
+    dbuf.nseg = plan->buffer_nseg[b];
+  }
+  a.batch = batch;
+  a.extent = plan->extent;
+  a.chunk = kShareChunk;
+
+  for (int ob = 0; ob < plan->num_outputs; ++ob) {
+    const int b = plan->num_inputs + ob;
+    const OutTables& t = plan->out[ob];
+    const cueq_u1d_buffer& o = buffers[b];
+    const int ext_out = plan->buffer_dim[b] ? plan->extent : 1;
+    const int64_t width = static_cast<int64_t>(plan->buffer_nseg[b]) * ext_out;
+    if (o.rows * width == 0) continue;
+    a.coeff = t.coeff;
+    a.nin = t.nin;
+    a.in = t.in;
+    a.seg_start = t.seg_start;
+    a.out_dim = plan->buffer_dim[b];
+    a.out_nseg = plan->buffer_nseg[b];
+    a.out_mode = o.batch_dim;
+    a.csr_offsets = o.csr_offsets;
+    a.csr_perm = o.csr_perm;
+    a.out = o.data;
+    a.out_dtype = o.dtype;
+    a.out_rows = o.rows;
+    int64_t nchunks = 0;
+    if (o.batch_dim == CUEQ_BATCH_SHARED) {
+      nchunks = share_chunks(batch);
+      if (nchunks > 1) {
+        const int64_t need = nchunks * width * static_cast<int64_t>(sizeof(M));
+        CUEQ_REQUIRE(workspace != nullptr && workspace_bytes >= need, CUEQ_ERR_INVALID,
+                     "workspace too small: need %lld bytes", (long long)need);
+        a.out = workspace;
+        a.out_dtype = sizeof(M) == 8 ? CUEQ_F64 : CUEQ_F32;
+        a.out_rows = nchunks;
+      } else {
+        a.out_rows = 1;  // zero or one chunk: fold straight into the output
+      }
+    }
+    const bool wave = t.contracts_channel;
+    const int64_t work = a.out_rows * (wave ? static_cast<int64_t>(a.out_nseg) * 64 : width);
+    const int64_t blocks = (work + 255) / 256;
+    CUEQ_REQUIRE(blocks < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "output %d too large for one launch", ob);
+    if (wave) hipLaunchKernelGGL(u1d_generic_wave<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(u1d_generic_elem<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    CUEQ_CHECK_HIP(hipGetLastError());
+    if (nchunks > 1) {
+      const int64_t fb = (width + 255) / 256;
+      hipLaunchKernelGGL(u1d_fold_chunks<M>, dim3(static_cast<unsigned>(fb)), dim3(256), 0, stream,
+                         static_cast<const M*>(workspace), nchunks, width, o.data, o.dtype);
+      CUEQ_CHECK_HIP(hipGetLastError());
+    }
+  }
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch, void* workspace,
+                            int64_t workspace_bytes, void* stream) {
+  CUEQ_REQUIRE(plan && buffers, CUEQ_ERR_INVALID, "null argument");
+  CUEQ_REQUIRE(batch >= 0, CUEQ_ERR_INVALID, "negative batch size");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (plan->math_dtype == CUEQ_F64) return run_typed<double>(plan, buffers, batch, workspace, workspace_bytes, s);
+  return run_typed<float>(plan, buffers, batch, workspace, workspace_bytes, s);
+}

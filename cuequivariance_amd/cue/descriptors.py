@@ -1,0 +1,184 @@
+"""Ready-made equivariant polynomials: channel-wise / fully-connected tensor products, linear maps.
+
+Reference behaviour followed (``cuequivariance/cuequivariance/group_theory/descriptors``):
+
+* ``irreps_tp.py:22-91``    fully_connected_tensor_product  ``"uvw,iu,jv,kw+ijk"``
+* ``irreps_tp.py:232-321``  channelwise_tensor_product      ``"uv,iu,jv,kuv+ijk"``
+* ``irreps_tp.py:505-545``  linear                          ``"uv,iu,iv"``
+* ``spherical_harmonics_.py:119-156`` recursion and normalisation of the spherical harmonics
+
+All descriptors use the ``ir_mul`` layout (component index outside, multiplicity inside).
+"""
+
+from __future__ import annotations
+
+import itertools
+from typing import Optional, Sequence
+
+import numpy as np
+
+from .irreps import Irrep, Irreps, IrrepsAndLayout, clebsch_gordan, into_list_of_irrep, ir_mul
+from .polynomial import EquivariantPolynomial, SegmentedPolynomial
+from .stp import SegmentedTensorProduct
+
+__all__ = [
+    "channelwise_tensor_product",
+    "fully_connected_tensor_product",
+    "linear",
+    "spherical_harmonics_values",
+]
+
+
+def _scalar_weights(irreps: Irreps, poly: SegmentedPolynomial) -> IrrepsAndLayout:
+    return IrrepsAndLayout(irreps.new_scalars(poly.inputs[0].size), ir_mul)
+
+
+def channelwise_tensor_product(
+    irreps1: Irreps,
+    irreps2: Irreps,
+    irreps3_filter=None,
+    simplify_irreps3: bool = False,
+) -> EquivariantPolynomial:
+    """``weights[uv], lhs[iu], rhs[jv] -> output[kuv]``: one weighted path per allowed (ir1, ir2, ir3).
+
+    Every path owns a weight segment and an output segment.  Output irreps are
+    stable-sorted with the group's order and the weight/output segments are
+    renumbered accordingly while the paths keep their generation order.
+    """
+    G = irreps1.irrep_class
+    if irreps3_filter is not None:
+        irreps3_filter = into_list_of_irrep(G, irreps3_filter)
+
+    d = SegmentedTensorProduct.from_subscripts("uv,iu,jv,kuv+ijk")
+    for mul, ir in irreps1:
+        d.add_segment(1, (ir.dim, mul))
+    for mul, ir in irreps2:
+        d.add_segment(2, (ir.dim, mul))
+
+    out = []
+    for (i1, (mul1, ir1)), (i2, (mul2, ir2)) in itertools.product(enumerate(irreps1), enumerate(irreps2)):
+        for ir3 in ir1 * ir2:
+            if irreps3_filter is not None and ir3 not in irreps3_filter:
+                continue
+            for cg in clebsch_gordan(ir1, ir2, ir3):
+                d.add_path(None, i1, i2, None, c=cg, dims={"u": mul1, "v": mul2})
+                out.append((mul1 * mul2, ir3))
+
+    irreps3, _perm, inv = Irreps(G, out).sort()
+    d = d.permute_segments(0, inv)
+    d = d.permute_segments(3, inv)
+    d = d.normalize_paths_for_operand(-1)
+
+    if simplify_irreps3:
+        d = d.flatten_coefficient_modes()
+        segs = [(ir, k) for _m, ir in irreps3 for k in range(ir.dim)]
+        order = sorted(range(len(segs)), key=lambda s: (_Key(segs[s][0]), segs[s][1], s))
+        d = d.permute_segments(3, order)
+        irreps3 = irreps3.simplify()
+
+    poly = SegmentedPolynomial.eval_last_operand(d)
+    return EquivariantPolynomial(
+        [_scalar_weights(irreps1, poly), IrrepsAndLayout(irreps1, ir_mul), IrrepsAndLayout(irreps2, ir_mul)],
+        [IrrepsAndLayout(irreps3, ir_mul)],
+        poly,
+    )
+
+
+class _Key:
+    __slots__ = ("ir",)
+
+    def __init__(self, ir):
+        self.ir = ir
+
+    def __eq__(self, o):
+        return self.ir == o.ir
+
+    def __lt__(self, o):
+        return self.ir < o.ir
+
+
+def fully_connected_tensor_product(irreps1: Irreps, irreps2: Irreps, irreps3: Irreps) -> EquivariantPolynomial:
+    """``weights[uvw], lhs[iu], rhs[jv] -> output[kw]``: every allowed (ir1, ir2, ir3) triple gets a weight block."""
+    d = SegmentedTensorProduct.from_subscripts("uvw,iu,jv,kw+ijk")
+    for mul, ir in irreps1:
+        d.add_segment(1, (ir.dim, mul))
+    for mul, ir in irreps2:
+        d.add_segment(2, (ir.dim, mul))
+    for mul, ir in irreps3:
+        d.add_segment(3, (ir.dim, mul))
+    for (i1, (mul1, ir1)), (i2, (mul2, ir2)), (i3, (mul3, ir3)) in itertools.product(
+        enumerate(irreps1), enumerate(irreps2), enumerate(irreps3)
+    ):
+        if ir3 not in ir1 * ir2:
+            continue
+        for cg in clebsch_gordan(ir1, ir2, ir3):
+            d.add_path((mul1, mul2, mul3), i1, i2, i3, c=cg)
+    d = d.normalize_paths_for_operand(-1)
+    poly = SegmentedPolynomial.eval_last_operand(d)
+    return EquivariantPolynomial(
+        [_scalar_weights(irreps1, poly), IrrepsAndLayout(irreps1, ir_mul), IrrepsAndLayout(irreps2, ir_mul)],
+        [IrrepsAndLayout(irreps3, ir_mul)],
+        poly,
+    )
+
+
+def linear(irreps_in: Irreps, irreps_out: Irreps) -> EquivariantPolynomial:
+    """``weights[uv], input[iu] -> output[iv]``: a weight matrix between every pair of equal irreps."""
+    d = SegmentedTensorProduct.from_subscripts("uv_iu_iv")
+    for mul, ir in irreps_in:
+        d.add_segment(1, (ir.dim, mul))
+    for mul, ir in irreps_out:
+        d.add_segment(2, (ir.dim, mul))
+    for (i1, (mul1, ir1)), (i2, (mul2, ir2)) in itertools.product(enumerate(irreps_in), enumerate(irreps_out)):
+        if ir1 == ir2:
+            d.add_path((mul1, mul2), i1, i2, c=1.0)
+    d = d.normalize_paths_for_operand(-1)
+    poly = SegmentedPolynomial.eval_last_operand(d)
+    return EquivariantPolynomial(
+        [_scalar_weights(irreps_in, poly), IrrepsAndLayout(irreps_in, ir_mul)],
+        [IrrepsAndLayout(irreps_out, ir_mul)],
+        poly,
+    )
+
+
+def spherical_harmonics_values(ir_vec: Irrep, ls: Sequence[int], vectors: np.ndarray) -> np.ndarray:
+    """Component-normalised real spherical harmonics ``Y_l(x)`` as homogeneous polynomials of ``x``.
+
+    ``Y_0 = 1``, ``Y_1 = sqrt(3) x``, ``Y_l = sqrt(2l+1) CG(Y_l1, Y_l2) / norm`` with ``l1 = l - l//2``,
+    ``l2 = l//2`` and ``norm`` fixed by evaluating at ``(0, 1, 0)``.  On unit vectors
+    ``sum_m Y_lm^2 = 2l+1``.  Output: ``(..., sum(2l+1))`` in the order of ``ls``.
+    """
+    vectors = np.asarray(vectors, dtype=np.float64)
+    assert vectors.shape[-1] == 3
+    return np.concatenate([_normalised_sh(ir_vec, ell, vectors) for ell in ls], axis=-1)
+
+
+def _normalised_sh(ir_vec: Irrep, ell: int, x: np.ndarray) -> np.ndarray:
+    if ell == 0:
+        return np.ones(x.shape[:-1] + (1,))
+    if ell == 1:
+        return np.sqrt(3.0) * x
+    l2 = ell // 2
+    l1 = ell - l2
+    north = np.array([0.0, 1.0, 0.0])
+
+    def raw(v):
+        y1, y2 = _normalised_sh(ir_vec, l1, v), _normalised_sh(ir_vec, l2, v)
+        ir1 = _sh_irrep(ir_vec, l1)
+        ir2 = _sh_irrep(ir_vec, l2)
+        ir = sorted(ir1 * ir2, key=_Key)[-1]
+        cg = clebsch_gordan(ir1, ir2, ir)[0]
+        return np.einsum("...i,...j,ijk->...k", y1, y2, cg)
+
+    norm = np.sqrt(np.sum(raw(north) ** 2))
+    return np.sqrt(2 * ell + 1) * raw(x) / norm
+
+
+def _sh_irrep(ir_vec: Irrep, ell: int) -> Irrep:
+    if ell == 0:
+        return ir_vec.trivial()
+    if ell == 1:
+        return ir_vec
+    l2 = ell // 2
+    l1 = ell - l2
+    return sorted(_sh_irrep(ir_vec, l1) * _sh_irrep(ir_vec, l2), key=_Key)[-1]

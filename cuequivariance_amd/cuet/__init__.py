@@ -1,0 +1,16 @@
+"""Torch-facing layer: the drop-in mirror of ``cuequivariance_torch`` running on HIP kernels."""
+
+from .transpose import TransposeSegments, TransposeIrrepsLayout
+from .segmented_polynomial import SegmentedPolynomial
+from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear
+from .uniform_1d import uniform_1d
+
+__all__ = [
+    "TransposeSegments",
+    "TransposeIrrepsLayout",
+    "SegmentedPolynomial",
+    "ChannelWiseTensorProduct",
+    "FullyConnectedTensorProduct",
+    "Linear",
+    "uniform_1d",
+]

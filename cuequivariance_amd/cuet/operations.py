@@ -1,0 +1,308 @@
+"""High-level equivariant layers: channel-wise and fully-connected tensor products, linear.
+
+Constructor arguments, attributes (``irreps_*``, ``weight_numel``, ``weight``, ``shared_weights``,
+``internal_weights``, ``method``) and ``forward`` signatures mirror
+
+* ``cuequivariance_torch/cuequivariance_torch/operations/tp_channel_wise.py:30-258``
+* ``cuequivariance_torch/cuequivariance_torch/operations/tp_fully_connected.py:30-207``
+* ``cuequivariance_torch/cuequivariance_torch/operations/linear.py:30-191``
+
+Defaults differ where the reference defaults to its PyTorch executor: every layer here runs HIP
+kernels (``uniform_1d`` for the channel-wise product, the dense executor ``fused_tp`` for the other two).
+"""
+
+from __future__ import annotations
+
+import warnings
+from typing import Dict, Optional, Sequence
+
+import torch
+
+from .. import cue
+from ..cue import descriptors
+from .segmented_polynomial import SegmentedPolynomial
+from .transpose import TransposeIrrepsLayout
+
+__all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear"]
+
+
+def _default_irreps(*irreps_list):
+    out = []
+    for irreps in irreps_list:
+        if isinstance(irreps, str):
+            irreps = cue.Irreps(irreps)
+        elif not isinstance(irreps, cue.Irreps):
+            irreps = cue.Irreps(irreps)
+        out.append(irreps)
+    return tuple(out)
+
+
+def _assert_same_group(*irreps_list):
+    g = irreps_list[0].irrep_class
+    for irreps in irreps_list[1:]:
+        if irreps.irrep_class is not g:
+            raise ValueError("The provided irreps are not of the same group.")
+
+
+def _default_layout(layout) -> cue.IrrepsLayout:
+    if layout is None:
+        warnings.warn("layout is not specified, defaulting to cue.mul_ir (the e3nn layout)")
+        return cue.mul_ir
+    return cue.IrrepsLayout.as_layout(layout)
+
+
+def _method_from_fallback(method, use_fallback, default: str) -> str:
+    if method is not None:
+        return method
+    if use_fallback is None:
+        return default
+    warnings.warn("`use_fallback` is deprecated, please use `method` instead", DeprecationWarning)
+    if use_fallback:
+        raise ValueError("use_fallback=True asks for the PyTorch executor, which this engine does not have")
+    return default
+
+
+class ChannelWiseTensorProduct(torch.nn.Module):
+    """``out[k u v] = w[u v] * sum_ij C[i j k] x1[i u] x2[j v]`` for every allowed irrep triple.
+
+    ``forward(x1, x2, weight=None, indices_1=None, indices_2=None, indices_out=None, size_out=None)``:
+    ``indices_1`` / ``indices_2`` gather rows of ``x1`` / ``x2`` per batch element, ``indices_out`` scatter-adds
+    the batch elements into ``size_out`` output rows (deterministically).
+    """
+
+    def __init__(
+        self,
+        irreps_in1: cue.Irreps,
+        irreps_in2: cue.Irreps,
+        filter_irreps_out: Sequence[cue.Irrep] = None,
+        *,
+        layout: Optional[cue.IrrepsLayout] = None,
+        layout_in1: Optional[cue.IrrepsLayout] = None,
+        layout_in2: Optional[cue.IrrepsLayout] = None,
+        layout_out: Optional[cue.IrrepsLayout] = None,
+        shared_weights: bool = True,
+        internal_weights: bool = None,
+        device: Optional[torch.device] = None,
+        dtype: Optional[torch.dtype] = None,
+        math_dtype=None,
+        use_fallback: Optional[bool] = None,
+        method: Optional[str] = None,
+    ):
+        super().__init__()
+        irreps_in1, irreps_in2 = _default_irreps(irreps_in1, irreps_in2)
+        _assert_same_group(irreps_in1, irreps_in2)
+        e = descriptors.channelwise_tensor_product(irreps_in1, irreps_in2, filter_irreps_out)
+        descriptor, irreps_out = e.polynomial.operations[0][1], e.outputs[0].irreps
+        assert descriptor.subscripts == "uv,iu,jv,kuv+ijk"
+        e2 = e.flatten_coefficient_modes().squeeze_modes()
+        u1d_compatible = (
+            e2.all_same_segment_shape() and len(e2.polynomial.operations[0][1].subscripts.modes()) == 1
+        )
+        self.irreps_in1, self.irreps_in2, self.irreps_out = irreps_in1, irreps_in2, irreps_out
+        self.weight_numel = descriptor.operands[0].size
+        self.shared_weights = shared_weights
+        self.internal_weights = internal_weights if internal_weights is not None else shared_weights
+        if self.internal_weights:
+            if not self.shared_weights:
+                raise ValueError("Internal weights should be shared")
+            self.weight = torch.nn.Parameter(torch.randn(1, self.weight_numel, device=device, dtype=dtype))
+        else:
+            self.weight = None
+        self.transpose_in1 = TransposeIrrepsLayout(
+            e.inputs[1].irreps, source=_default_layout(layout_in1 or layout), target=e.inputs[1].layout, device=device
+        )
+        self.transpose_in2 = TransposeIrrepsLayout(
+            e.inputs[2].irreps, source=_default_layout(layout_in2 or layout), target=e.inputs[2].layout, device=device
+        )
+        self.transpose_out = TransposeIrrepsLayout(
+            e.outputs[0].irreps, source=e.outputs[0].layout, target=_default_layout(layout_out or layout), device=device
+        )
+        self.method = _method_from_fallback(method, use_fallback, "uniform_1d")
+        if self.method == "uniform_1d" and not u1d_compatible:
+            raise ValueError(
+                "`uniform_1d` method requires segments to be the same shape\n"
+                "You can consider making the segments uniform in the descriptor."
+            )
+        self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+
+    def extra_repr(self) -> str:
+        return (
+            f"shared_weights={self.shared_weights}, internal_weights={self.internal_weights}, "
+            f"weight_numel={self.weight_numel}"
+        )
+
+    def forward(
+        self,
+        x1: torch.Tensor,
+        x2: torch.Tensor,
+        weight: Optional[torch.Tensor] = None,
+        indices_1: Optional[torch.Tensor] = None,
+        indices_2: Optional[torch.Tensor] = None,
+        indices_out: Optional[torch.Tensor] = None,
+        size_out: Optional[int] = None,
+    ) -> torch.Tensor:
+        x1 = self.transpose_in1(x1)
+        x2 = self.transpose_in2(x2)
+        indices_in: Dict[int, torch.Tensor] = {}
+        if indices_1 is not None:
+            indices_in[1] = indices_1
+        if indices_2 is not None:
+            indices_in[2] = indices_2
+        indices_o: Dict[int, torch.Tensor] = {}
+        sizes_out: Dict[int, torch.Tensor] = {}
+        if indices_out is not None:
+            if size_out is None:
+                raise ValueError("size_out should be provided if indices_out is provided")
+            indices_o = {0: indices_out}
+            sizes_out = {0: torch.empty(size_out, 1, device="meta")}  # only .shape[0] is read
+        if self.weight is not None:
+            if weight is not None:
+                raise ValueError("Internal weights are used, weight should be None")
+            weight = self.weight
+        elif weight is None:
+            raise ValueError("Internal weights are not used, weight should not be None")
+        out = self.f([weight, x1, x2], input_indices=indices_in, output_shapes=sizes_out, output_indices=indices_o)
+        return self.transpose_out(out[0])
+
+
+class FullyConnectedTensorProduct(torch.nn.Module):
+    """``out[k w] = sum_{u v i j} w[u v w] C[i j k] x1[i u] x2[j v]`` over every allowed irrep triple."""
+
+    def __init__(
+        self,
+        irreps_in1: cue.Irreps,
+        irreps_in2: cue.Irreps,
+        irreps_out: cue.Irreps,
+        *,
+        layout: Optional[cue.IrrepsLayout] = None,
+        layout_in1: Optional[cue.IrrepsLayout] = None,
+        layout_in2: Optional[cue.IrrepsLayout] = None,
+        layout_out: Optional[cue.IrrepsLayout] = None,
+        shared_weights: bool = True,
+        internal_weights: bool = None,
+        device: Optional[torch.device] = None,
+        dtype: Optional[torch.dtype] = None,
+        math_dtype=None,
+        use_fallback: Optional[bool] = None,
+        method: Optional[str] = None,
+    ):
+        super().__init__()
+        irreps_in1, irreps_in2, irreps_out = _default_irreps(irreps_in1, irreps_in2, irreps_out)
+        _assert_same_group(irreps_in1, irreps_in2, irreps_out)
+        if dtype is None:
+            dtype = torch.get_default_dtype()
+        e = descriptors.fully_connected_tensor_product(irreps_in1, irreps_in2, irreps_out)
+        assert e.polynomial.operations[0][1].subscripts == "uvw,iu,jv,kw+ijk"
+        self.irreps_in1, self.irreps_in2, self.irreps_out = irreps_in1, irreps_in2, irreps_out
+        self.weight_numel = e.polynomial.operations[0][1].operands[0].size
+        self.shared_weights = shared_weights
+        self.internal_weights = internal_weights if internal_weights is not None else shared_weights
+        if self.internal_weights:
+            if not self.shared_weights:
+                raise ValueError("Internal weights should be shared")
+            self.weight = torch.nn.Parameter(torch.randn(1, self.weight_numel, device=device, dtype=dtype))
+        else:
+            self.weight = None
+        self.transpose_in1 = TransposeIrrepsLayout(
+            e.inputs[1].irreps, source=_default_layout(layout_in1 or layout), target=e.inputs[1].layout, device=device
+        )
+        self.transpose_in2 = TransposeIrrepsLayout(
+            e.inputs[2].irreps, source=_default_layout(layout_in2 or layout), target=e.inputs[2].layout, device=device
+        )
+        self.transpose_out = TransposeIrrepsLayout(
+            e.outputs[0].irreps, source=e.outputs[0].layout, target=_default_layout(layout_out or layout), device=device
+        )
+        self.method = _method_from_fallback(method, use_fallback, "fused_tp")
+        self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+
+    def extra_repr(self) -> str:
+        return (
+            f"shared_weights={self.shared_weights}, internal_weights={self.internal_weights}, "
+            f"weight_numel={self.weight_numel}"
+        )
+
+    def forward(self, x1: torch.Tensor, x2: torch.Tensor, weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+        x1 = self.transpose_in1(x1)
+        x2 = self.transpose_in2(x2)
+        if self.weight is not None:
+            if weight is not None:
+                raise ValueError("Internal weights are used, weight should be None")
+            weight = self.weight
+        elif weight is None:
+            raise ValueError("Internal weights are not used, weight should not be None")
+        return self.transpose_out(self.f([weight, x1, x2])[0])
+
+
+class Linear(torch.nn.Module):
+    """Equivariant linear map: one ``mul_in x mul_out`` weight block per pair of equal irreps, scaled ``1/sqrt(mul_in)``.
+
+    ``forward(x, weight=None, weight_indices=None)``; with ``weight_classes > 1`` the weights have one row per
+    class and ``weight_indices`` selects the row used by each batch element.
+    """
+
+    def __init__(
+        self,
+        irreps_in: cue.Irreps,
+        irreps_out: cue.Irreps,
+        *,
+        layout: Optional[cue.IrrepsLayout] = None,
+        layout_in: Optional[cue.IrrepsLayout] = None,
+        layout_out: Optional[cue.IrrepsLayout] = None,
+        shared_weights: bool = True,
+        internal_weights: bool = None,
+        weight_classes: Optional[int] = 1,
+        device: Optional[torch.device] = None,
+        dtype: Optional[torch.dtype] = None,
+        math_dtype=None,
+        use_fallback: Optional[bool] = None,
+        method: Optional[str] = None,
+    ):
+        super().__init__()
+        irreps_in, irreps_out = _default_irreps(irreps_in, irreps_out)
+        _assert_same_group(irreps_in, irreps_out)
+        e = descriptors.linear(irreps_in, irreps_out)
+        assert e.polynomial.operations[0][1].subscripts == "uv,iu,iv"
+        self.irreps_in, self.irreps_out = irreps_in, irreps_out
+        self.weight_numel = e.inputs[0].dim
+        self.weight_classes = weight_classes
+        self.shared_weights = shared_weights
+        if weight_classes > 1 and not shared_weights:
+            raise ValueError("Weight classes require shared weights.")
+        self.internal_weights = internal_weights if internal_weights is not None else shared_weights
+        if self.internal_weights:
+            if not self.shared_weights:
+                raise ValueError("Internal weights should be shared")
+            self.weight = torch.nn.Parameter(torch.randn(weight_classes, self.weight_numel, device=device, dtype=dtype))
+        else:
+            self.weight = None
+        self.transpose_in = TransposeIrrepsLayout(
+            e.inputs[1].irreps, source=_default_layout(layout_in or layout), target=e.inputs[1].layout, device=device
+        )
+        self.transpose_out = TransposeIrrepsLayout(
+            e.outputs[0].irreps, source=e.outputs[0].layout, target=_default_layout(layout_out or layout), device=device
+        )
+        self.method = _method_from_fallback(method, use_fallback, "fused_tp")
+        self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+
+    def extra_repr(self) -> str:
+        return (
+            f"shared_weights={self.shared_weights}, internal_weights={self.internal_weights}, "
+            f"weight_numel={self.weight_numel}"
+        )
+
+    def forward(
+        self, x: torch.Tensor, weight: Optional[torch.Tensor] = None, weight_indices: Optional[torch.Tensor] = None
+    ) -> torch.Tensor:
+        if self.internal_weights:
+            if weight is not None:
+                raise ValueError("Internal weights are used, weight should be None")
+            weight = self.weight
+        input_indices: Dict[int, torch.Tensor] = {}
+        if self.weight_classes > 1:
+            if weight_indices is None:
+                raise ValueError("weight_indices should be provided if weight_classes > 1")
+            input_indices[0] = weight_indices
+        if weight is None:
+            raise ValueError("Weights should not be None")
+        out = self.f([weight, self.transpose_in(x)], input_indices=input_indices)
+        return self.transpose_out(out[0])

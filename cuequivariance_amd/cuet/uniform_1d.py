@@ -1,0 +1,459 @@
+"""The ``uniform_1d`` operator on MI355X: same call signature as the reference's closed op.
+
+``uniform_1d(name, math_dtype, operand_extent, ..., batch_size, tensors)`` takes exactly the
+21 positional arguments of ``torch.ops.cuequivariance.uniform_1d`` as called at
+``cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_uniform_1d.py:55-77,294-316``
+and returns the list of output tensors.  It differs from the reference in how it runs:
+
+* the path tables are compiled once into a device-resident plan (``cueq_u1d_plan_create``);
+* scatter into indexed outputs is a gather over rows grouped by output row (no atomics);
+* backward is the same operator applied to the transposed tables (the path table is reused,
+  only the roles of the buffers change, as in
+  ``cuequivariance/cuequivariance/segmented_polynomials/segmented_polynomial.py:1003-1133``),
+  so gradients of any order work.
+
+Everything executes through the C ABI in ``libcueq_amd.so``; CPU tensors are rejected.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from collections import OrderedDict
+from typing import List, Optional, Sequence
+
+import torch
+
+from .. import _lib
+from .._lib import BATCH_DIM_AUTO, BATCH_DIM_BATCHED, BATCH_DIM_INDEXED, BATCH_DIM_SHARED
+
+__all__ = [
+    "uniform_1d",
+    "BATCH_DIM_AUTO",
+    "BATCH_DIM_SHARED",
+    "BATCH_DIM_BATCHED",
+    "BATCH_DIM_INDEXED",
+    "Uniform1dPlan",
+]
+
+_DTYPE_CODE = {
+    torch.float32: _lib.F32,
+    torch.float64: _lib.F64,
+    torch.float16: _lib.F16,
+    torch.bfloat16: _lib.BF16,
+}
+
+
+class Uniform1dPlan:
+    """Flat descriptor tables + lazily created device plans (one per GPU) + derived backward plans."""
+
+    def __init__(
+        self,
+        math_dtype: torch.dtype,
+        operand_extent: int,
+        num_inputs: int,
+        num_outputs: int,
+        buffer_dim: Sequence[int],
+        buffer_num_segments: Sequence[int],
+        dtypes: Sequence[int],
+        num_operands: Sequence[int],
+        operations: Sequence[int],
+        num_paths: Sequence[int],
+        path_indices_start: Sequence[int],
+        path_coefficients_start: Sequence[int],
+        path_indices: Sequence[int],
+        path_coefficients: Sequence[float],
+        name: str = "segmented_polynomial",
+    ):
+        if math_dtype not in (torch.float32, torch.float64):
+            raise ValueError(f"uniform_1d: math_dtype must be float32 or float64, got {math_dtype}")
+        self.name = name
+        self.math_dtype = math_dtype
+        self.operand_extent = int(operand_extent)
+        self.num_inputs = int(num_inputs)
+        self.num_outputs = int(num_outputs)
+        self.buffer_dim = tuple(int(x) for x in buffer_dim)
+        self.buffer_num_segments = tuple(int(x) for x in buffer_num_segments)
+        self.dtypes = tuple(int(x) for x in dtypes)
+        self.num_operands = tuple(int(x) for x in num_operands)
+        self.operations = tuple(int(x) for x in operations)
+        self.num_paths = tuple(int(x) for x in num_paths)
+        self.path_indices_start = tuple(int(x) for x in path_indices_start)
+        self.path_coefficients_start = tuple(int(x) for x in path_coefficients_start)
+        self.path_indices = tuple(int(x) for x in path_indices)
+        self.path_coefficients = tuple(float(x) for x in path_coefficients)
+        nbuf = self.num_inputs + self.num_outputs
+        if len(self.buffer_dim) != nbuf or len(self.buffer_num_segments) != nbuf or len(self.dtypes) != nbuf:
+            raise ValueError("uniform_1d: per-buffer lists must have num_inputs + num_outputs entries")
+        if not (len(self.num_operands) == len(self.num_paths) == len(self.path_indices_start)
+                == len(self.path_coefficients_start)):
+            raise ValueError("uniform_1d: per-operation lists have inconsistent lengths")
+        if sum(self.num_operands) != len(self.operations):
+            raise ValueError("uniform_1d: `operations` does not match `num_operands`")
+        self._handles: dict[int, int] = {}
+        self._backward: dict[tuple, "Uniform1dPlan"] = {}
+        self._lock = threading.Lock()
+
+    # ------------------------------------------------------------------ geometry
+    def width(self, b: int) -> int:
+        return self.buffer_num_segments[b] * (self.operand_extent if self.buffer_dim[b] else 1)
+
+    def key(self) -> tuple:
+        return (
+            self.math_dtype, self.operand_extent, self.num_inputs, self.num_outputs, self.buffer_dim,
+            self.buffer_num_segments, self.dtypes, self.num_operands, self.operations, self.num_paths,
+            self.path_indices_start, self.path_coefficients_start, self.path_indices, self.path_coefficients,
+        )
+
+    # ------------------------------------------------------------------ device plan
+    def handle(self, device: torch.device) -> int:
+        idx = device.index if device.index is not None else torch.cuda.current_device()
+        h = self._handles.get(idx)
+        if h is not None:
+            return h
+        with self._lock:
+            h = self._handles.get(idx)
+            if h is not None:
+                return h
+            lib = _lib.load()
+            keep = dict(
+                buffer_dim=_lib.int32_array(self.buffer_dim),
+                nseg=_lib.int32_array(self.buffer_num_segments),
+                num_operands=_lib.int32_array(self.num_operands),
+                operations=_lib.int32_array(self.operations),
+                num_paths=_lib.int32_array(self.num_paths),
+                pis=_lib.int64_array(self.path_indices_start),
+                pcs=_lib.int64_array(self.path_coefficients_start),
+                pi=_lib.int32_array(self.path_indices),
+                pc=_lib.double_array(self.path_coefficients),
+            )
+            desc = _lib.U1dDesc(
+                math_dtype=_DTYPE_CODE[self.math_dtype],
+                operand_extent=self.operand_extent,
+                num_inputs=self.num_inputs,
+                num_outputs=self.num_outputs,
+                buffer_dim=keep["buffer_dim"],
+                buffer_num_segments=keep["nseg"],
+                num_operations=len(self.num_operands),
+                num_operands=keep["num_operands"],
+                operations=keep["operations"],
+                num_paths=keep["num_paths"],
+                path_indices_start=keep["pis"],
+                path_coefficients_start=keep["pcs"],
+                path_indices=keep["pi"],
+                path_indices_len=len(self.path_indices),
+                path_coefficients=keep["pc"],
+                path_coefficients_len=len(self.path_coefficients),
+            )
+            out = C.c_void_p()
+            with torch.cuda.device(idx):
+                _lib.check(lib.cueq_u1d_plan_create(C.byref(desc), C.byref(out)), "cueq_u1d_plan_create")
+            self._handles[idx] = out.value
+            return out.value
+
+    def __del__(self):
+        try:
+            lib = _lib.load()
+            for h in self._handles.values():
+                lib.cueq_u1d_plan_destroy(h)
+        except Exception:
+            pass
+
+    # ------------------------------------------------------------------ transposition
+    def backward_plan(self, needs_grad: tuple) -> "Uniform1dPlan":
+        """Plan computing the gradients of the inputs flagged in ``needs_grad``.
+
+        Buffers of the new plan: the original inputs, one cotangent per original output, then
+        one gradient per flagged input.  For every operation and every operand slot bound to a
+        flagged input, an operation with the same path table is emitted in which that slot
+        becomes the output and the original output slot reads the cotangent.
+        """
+        needs_grad = tuple(bool(x) for x in needs_grad)
+        plan = self._backward.get(needs_grad)
+        if plan is not None:
+            return plan
+        nin, nout = self.num_inputs, self.num_outputs
+        grad_buf, k = {}, nin + nout
+        for i, g in enumerate(needs_grad):
+            if g:
+                grad_buf[i] = k
+                k += 1
+        buf_dim = list(self.buffer_dim) + [self.buffer_dim[i] for i in grad_buf]
+        buf_nseg = list(self.buffer_num_segments) + [self.buffer_num_segments[i] for i in grad_buf]
+        # inputs inherit their own dtype; cotangents are inputs too; a gradient takes its primal's dtype
+        dtypes = list(range(nin + nout)) + [i for i in grad_buf]
+        num_operands, operations, num_paths, pis, pcs = [], [], [], [], []
+        off = 0
+        for o, nop in enumerate(self.num_operands):
+            bufs = self.operations[off: off + nop]
+            off += nop
+            out_pos = [s for s, b in enumerate(bufs) if b >= nin]
+            assert len(out_pos) == 1
+            out_pos = out_pos[0]
+            for s, b in enumerate(bufs):
+                if s == out_pos or not needs_grad[b]:
+                    continue
+                nb = list(bufs)
+                nb[s] = grad_buf[b]
+                # nb[out_pos] keeps its id: cotangent of output j sits at position nin + j
+                num_operands.append(nop)
+                operations += nb
+                num_paths.append(self.num_paths[o])
+                pis.append(self.path_indices_start[o])
+                pcs.append(self.path_coefficients_start[o])
+        plan = Uniform1dPlan(
+            self.math_dtype, self.operand_extent, nin + nout, len(grad_buf), buf_dim, buf_nseg, dtypes,
+            num_operands, operations, num_paths, pis, pcs, self.path_indices, self.path_coefficients,
+            name=self.name + "_bwd",
+        )
+        self._backward[needs_grad] = plan
+        return plan
+
+
+_plan_cache: "OrderedDict[tuple, Uniform1dPlan]" = OrderedDict()
+_plan_cache_lock = threading.Lock()
+
+
+def _cached_plan(plan: Uniform1dPlan) -> Uniform1dPlan:
+    k = plan.key()
+    with _plan_cache_lock:
+        hit = _plan_cache.get(k)
+        if hit is not None:
+            _plan_cache.move_to_end(k)
+            return hit
+        _plan_cache[k] = plan
+        while len(_plan_cache) > 256:
+            _plan_cache.popitem(last=False)
+        return plan
+
+
+# ---------------------------------------------------------------------- CSR cache
+_csr_cache: "OrderedDict[tuple, tuple]" = OrderedDict()
+
+
+def _segment_csr(index: torch.Tensor, nrows: int):
+    """(offsets[nrows+1], perm[n]) grouping batch ids by output row; cached per index tensor."""
+    key = (index.data_ptr(), index._version, index.numel(), int(nrows), index.dtype, index.device)
+    hit = _csr_cache.get(key)
+    if hit is not None:
+        _csr_cache.move_to_end(key)
+        return hit[1], hit[2]
+    lib = _lib.load()
+    n = index.numel()
+    offsets = torch.empty(nrows + 1, dtype=torch.int64, device=index.device)
+    perm = torch.empty(max(n, 1), dtype=torch.int64, device=index.device)
+    ws_bytes = lib.cueq_segment_csr_workspace(n, nrows)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=index.device)
+    stream = torch.cuda.current_stream(index.device).cuda_stream
+    _lib.check(
+        lib.cueq_segment_csr_build(
+            index.data_ptr(), 1 if index.dtype == torch.int64 else 0, n, nrows,
+            offsets.data_ptr(), perm.data_ptr(), ws.data_ptr(), ws_bytes, stream,
+        ),
+        "cueq_segment_csr_build",
+    )
+    # the index tensor is kept alive with the entry so its address cannot be reused meanwhile
+    _csr_cache[key] = (index, offsets, perm)
+    while len(_csr_cache) > 32:
+        _csr_cache.popitem(last=False)
+    return offsets, perm
+
+
+# ---------------------------------------------------------------------- execution
+class _CallConfig:
+    """Resolved batching of one call: per buffer the mode, the index tensor slot and the row count."""
+
+    __slots__ = ("modes", "index_of", "rows", "batch")
+
+    def __init__(self, modes, index_of, rows, batch):
+        self.modes = tuple(modes)
+        self.index_of = tuple(index_of)
+        self.rows = tuple(rows)
+        self.batch = int(batch)
+
+
+def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor],
+            indices: Sequence[torch.Tensor]) -> List[torch.Tensor]:
+    nin, nout = plan.num_inputs, plan.num_outputs
+    device = inputs[0].device if nin else indices[0].device
+    if device.type != "cuda":
+        raise RuntimeError("uniform_1d runs on the GPU only; got tensors on " + str(device))
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        handle = plan.handle(device)
+        bufs = (_lib.U1dBuffer * (nin + nout))()
+        keep = []
+        for b in range(nin):
+            t = inputs[b]
+            if t.dtype not in _DTYPE_CODE:
+                raise ValueError(f"uniform_1d: unsupported dtype {t.dtype} for input {b}")
+            if t.dim() != 2 or t.shape[1] != plan.width(b):
+                raise ValueError(f"uniform_1d: input {b} has shape {tuple(t.shape)}, expected (rows, {plan.width(b)})")
+            t = t.contiguous()
+            keep.append(t)
+            bufs[b].data = t.data_ptr()
+            bufs[b].rows = t.shape[0]
+            bufs[b].dtype = _DTYPE_CODE[t.dtype]
+            bufs[b].batch_dim = cfg.modes[b]
+            if cfg.modes[b] == BATCH_DIM_INDEXED:
+                idx = indices[cfg.index_of[b]]
+                bufs[b].index = idx.data_ptr()
+                bufs[b].index_is_64 = 1 if idx.dtype == torch.int64 else 0
+        outputs = []
+        for o in range(nout):
+            b = nin + o
+            src = plan.dtypes[b]
+            dtype = plan.math_dtype if src < 0 else inputs[src].dtype
+            out = torch.empty((cfg.rows[b], plan.width(b)), dtype=dtype, device=device)
+            outputs.append(out)
+            bufs[b].data = out.data_ptr()
+            bufs[b].rows = out.shape[0]
+            bufs[b].dtype = _DTYPE_CODE[dtype]
+            bufs[b].batch_dim = cfg.modes[b]
+            if cfg.modes[b] == BATCH_DIM_INDEXED:
+                idx = indices[cfg.index_of[b]]
+                bufs[b].index = idx.data_ptr()
+                bufs[b].index_is_64 = 1 if idx.dtype == torch.int64 else 0
+                offsets, perm = _segment_csr(idx, cfg.rows[b])
+                keep += [offsets, perm]
+                bufs[b].csr_offsets = offsets.data_ptr()
+                bufs[b].csr_perm = perm.data_ptr()
+        ws_bytes = lib.cueq_u1d_workspace_size(handle, bufs, cfg.batch)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes > 0 else None
+        stream = torch.cuda.current_stream(device).cuda_stream
+        _lib.check(
+            lib.cueq_u1d_run(handle, bufs, cfg.batch, ws.data_ptr() if ws is not None else None, ws_bytes, stream),
+            f"cueq_u1d_run[{plan.name}]",
+        )
+    return outputs
+
+
+class _Uniform1dFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, plan: Uniform1dPlan, cfg: _CallConfig, num_index: int, *tensors):
+        nin = plan.num_inputs
+        inputs, indices = tensors[:nin], tensors[nin: nin + num_index]
+        ctx.plan, ctx.cfg, ctx.num_index = plan, cfg, num_index
+        ctx.save_for_backward(*tensors)
+        outs = _launch(plan, cfg, [t.detach() for t in inputs], indices)
+        return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        plan, cfg, num_index = ctx.plan, ctx.cfg, ctx.num_index
+        nin, nout = plan.num_inputs, plan.num_outputs
+        tensors = ctx.saved_tensors
+        inputs, indices = tensors[:nin], tensors[nin:]
+        needs = tuple(ctx.needs_input_grad[3: 3 + nin])
+        if not any(needs):
+            return (None,) * (3 + len(tensors))
+        bplan = plan.backward_plan(needs)
+        cots = []
+        for o, g in enumerate(grad_outputs):
+            b = nin + o
+            if g is None:
+                src = plan.dtypes[b]
+                g = torch.zeros((cfg.rows[b], plan.width(b)), device=inputs[0].device,
+                                dtype=plan.math_dtype if src < 0 else inputs[src].dtype)
+            cots.append(g)
+        flagged = [i for i, n in enumerate(needs) if n]
+        modes = list(cfg.modes) + [cfg.modes[i] for i in flagged]
+        index_of = list(cfg.index_of) + [cfg.index_of[i] for i in flagged]
+        rows = list(cfg.rows) + [cfg.rows[i] for i in flagged]
+        bcfg = _CallConfig(modes, index_of, rows, cfg.batch)
+        grads = _Uniform1dFunction.apply(bplan, bcfg, num_index, *inputs, *cots, *indices)
+        out = [None, None, None] + [None] * len(tensors)
+        for g, i in zip(grads, flagged):
+            out[3 + i] = g
+        return tuple(out)
+
+
+def run_plan(plan: Uniform1dPlan, batch_dim: Sequence[int], index_buffer: Sequence[int], batch_size: int,
+             num_index: int, tensors: Sequence[torch.Tensor]) -> List[torch.Tensor]:
+    """Resolve AUTO batch dims and sizes (same rules as the reference op's caller) and execute."""
+    nin, nout = plan.num_inputs, plan.num_outputs
+    if len(tensors) != nin + num_index:
+        raise ValueError(f"uniform_1d: expected {nin} inputs + {num_index} index tensors, got {len(tensors)}")
+    inputs, indices = list(tensors[:nin]), list(tensors[nin:])
+    for k, idx in enumerate(indices):
+        if idx.dtype not in (torch.int32, torch.int64) or idx.dim() != 1:
+            raise ValueError(f"uniform_1d: index tensor {k} must be a 1-D int32/int64 tensor")
+        indices[k] = idx.contiguous()
+    modes = list(batch_dim)
+    batch = batch_size
+    # batch size: the common length of index tensors and of batched (multi-row) inputs
+    candidates = [idx.shape[0] for idx in indices]
+    for b in range(nin):
+        if modes[b] == BATCH_DIM_INDEXED:
+            continue
+        r = inputs[b].shape[0]
+        if modes[b] == BATCH_DIM_BATCHED or (modes[b] == BATCH_DIM_AUTO and r != 1):
+            candidates.append(r)
+    if batch == BATCH_DIM_AUTO:
+        batch = candidates[0] if candidates else 1
+    for c in candidates:
+        if c != batch:
+            raise ValueError(f"uniform_1d: inconsistent batch sizes {sorted(set(candidates + [batch]))}")
+    rows = [0] * (nin + nout)
+    for b in range(nin):
+        rows[b] = inputs[b].shape[0]
+        if modes[b] == BATCH_DIM_AUTO:
+            modes[b] = BATCH_DIM_SHARED if (rows[b] == 1 and batch != 1) else BATCH_DIM_BATCHED
+        if modes[b] == BATCH_DIM_BATCHED and rows[b] == 1 and batch != 1:
+            modes[b] = BATCH_DIM_SHARED
+        if modes[b] == BATCH_DIM_INDEXED:
+            assert index_buffer[b] >= 0
+    for o in range(nout):
+        b = nin + o
+        if modes[b] == BATCH_DIM_INDEXED:
+            rows[b] = int(index_buffer[nin + nout + index_buffer[b]])
+        elif modes[b] == BATCH_DIM_SHARED:
+            rows[b] = 1
+        else:
+            modes[b] = BATCH_DIM_BATCHED
+            rows[b] = batch
+    cfg = _CallConfig(modes, list(index_buffer[: nin + nout]), rows, batch)
+    outs = _Uniform1dFunction.apply(plan, cfg, num_index, *inputs, *indices)
+    return list(outs)
+
+
+def uniform_1d(
+    name: str,
+    math_dtype: torch.dtype,
+    operand_extent: int,
+    num_inputs: int,
+    num_outputs: int,
+    num_index: int,
+    buffer_dim: List[int],
+    buffer_num_segments: List[int],
+    batch_dim: List[int],
+    index_buffer: List[int],
+    dtypes: List[int],
+    num_operations: int,
+    num_operands: List[int],
+    operations: List[int],
+    num_paths: List[int],
+    path_indices_start: List[int],
+    path_coefficients_start: List[int],
+    path_indices: List[int],
+    path_coefficients: List[float],
+    batch_size: int,
+    tensors: List[torch.Tensor],
+) -> List[torch.Tensor]:
+    """Drop-in for ``torch.ops.cuequivariance.uniform_1d`` (argument meaning unchanged).
+
+    ``tensors`` = the inputs followed by the index tensors; ``index_buffer`` maps every buffer to
+    its index tensor (or -1) and then lists, per index tensor, the row count of the buffer it
+    addresses; ``dtypes[num_inputs + k]`` names the input whose dtype output ``k`` inherits
+    (-1: the math dtype).  Differentiable to any order.
+    """
+    if len(num_operands) != num_operations:
+        raise ValueError("uniform_1d: num_operations does not match num_operands")
+    plan = _cached_plan(
+        Uniform1dPlan(
+            math_dtype, operand_extent, num_inputs, num_outputs, buffer_dim, buffer_num_segments, dtypes,
+            num_operands, operations, num_paths, path_indices_start, path_coefficients_start, path_indices,
+            path_coefficients, name=name,
+        )
+    )
+    return run_plan(plan, batch_dim, index_buffer, batch_size, num_index, tensors)

@@ -1,0 +1,111 @@
+/*
+ * C ABI of the MI355X (gfx950) segmented-polynomial engine.
+ *
+ * Every entry point takes plain pointers and sizes, launches asynchronously on
+ * the given HIP stream (passed as void*), never allocates device memory unless
+ * stated, never throws, and returns 0 on success or a negative error code;
+ * cueq_last_error() returns a thread-local message for the last failure.
+ *
+ * The entry points replace the closed native ops that the reference's Python
+ * frontend calls; each declaration cites the reference call site it stands for
+ * (paths relative to the reference checkout).
+ */
+#ifndef CUEQ_AMD_H
+#define CUEQ_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of tensors crossing the boundary */
+enum cueq_dtype { CUEQ_F32 = 0, CUEQ_F64 = 1, CUEQ_F16 = 2, CUEQ_BF16 = 3 };
+
+/* How a buffer's rows relate to the batch index z.
+ * Mirrors BATCH_DIM_{AUTO,SHARED,BATCHED,INDEXED} imported at
+ * cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_uniform_1d.py:25-30
+ * (the reference does not publish the numeric values; these are this library's). */
+enum cueq_batch_dim { CUEQ_BATCH_AUTO = -1, CUEQ_BATCH_SHARED = 0, CUEQ_BATCH_BATCHED = 1, CUEQ_BATCH_INDEXED = 2 };
+
+enum cueq_status {
+  CUEQ_OK = 0,
+  CUEQ_ERR_INVALID = -1,     /* malformed tables / arguments                      */
+  CUEQ_ERR_UNSUPPORTED = -2, /* valid request this build has no kernel for        */
+  CUEQ_ERR_HIP = -3,         /* a HIP runtime call failed                         */
+  CUEQ_ERR_TOO_LARGE = -4    /* size beyond a documented limit                    */
+};
+
+const char* cueq_last_error(void);
+const char* cueq_version(void);
+
+/* ------------------------------------------------------------------------- */
+/* uniform-1d executor                                                        */
+/* ------------------------------------------------------------------------- */
+
+typedef struct cueq_u1d_plan cueq_u1d_plan;
+
+/* Descriptor tables, exactly the flat lists the reference builds at
+ * cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_uniform_1d.py:188-218
+ * and passes positionally to torch.ops.cuequivariance.uniform_1d (same file, :55-77). */
+typedef struct {
+  int32_t math_dtype;                  /* CUEQ_F32 or CUEQ_F64                                   */
+  int64_t operand_extent;              /* u: extent of the single mode                            */
+  int32_t num_inputs;
+  int32_t num_outputs;
+  const int32_t* buffer_dim;           /* [num_inputs+num_outputs] 0: scalar segments, 1: u-vectors */
+  const int32_t* buffer_num_segments;  /* [num_inputs+num_outputs]                                */
+  int32_t num_operations;
+  const int32_t* num_operands;         /* [num_operations]                                        */
+  const int32_t* operations;           /* concatenated buffer ids, sum(num_operands) entries      */
+  const int32_t* num_paths;            /* [num_operations]                                        */
+  const int64_t* path_indices_start;   /* [num_operations] offset into path_indices               */
+  const int64_t* path_coefficients_start; /* [num_operations] offset into path_coefficients      */
+  const int32_t* path_indices;         /* row-major (path, operand) segment ids                   */
+  int64_t path_indices_len;
+  const double* path_coefficients;
+  int64_t path_coefficients_len;
+} cueq_u1d_desc;
+
+/* One tensor at the boundary. */
+typedef struct {
+  void* data;            /* device pointer, row-major (rows, num_segments * (dim ? extent : 1))   */
+  int64_t rows;
+  int32_t dtype;         /* cueq_dtype                                                            */
+  int32_t batch_dim;     /* cueq_batch_dim (never AUTO here)                                      */
+  const void* index;     /* INDEXED: device pointer to batch_size row ids, else NULL              */
+  int32_t index_is_64;   /* 1: int64 ids, 0: int32                                                */
+  /* Outputs that are INDEXED or SHARED are reduced without atomics.  For INDEXED the
+   * caller passes the grouping of batch rows by output row: csr_offsets[rows+1] and
+   * csr_perm[batch_size] (batch ids of row r are csr_perm[csr_offsets[r] .. csr_offsets[r+1]),
+   * ascending inside a row), e.g. from cueq_segment_csr_build.  NULL otherwise.              */
+  const int64_t* csr_offsets;
+  const int64_t* csr_perm;
+} cueq_u1d_buffer;
+
+/* Compiles the tables into device-resident path tables (sorted and grouped by output
+ * segment).  Allocates device memory owned by the plan.  The plan is immutable and may be
+ * run concurrently from several threads/streams of the device it was created on. */
+int cueq_u1d_plan_create(const cueq_u1d_desc* desc, cueq_u1d_plan** plan);
+void cueq_u1d_plan_destroy(cueq_u1d_plan* plan);
+
+/* Bytes of device workspace cueq_u1d_run needs for this call shape (0 if none). */
+int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size);
+
+/* Evaluates every operation of the plan:
+ *   out[b_out][row_out(z), seg_out(p), :] += coeff[p] * prod_k in[b_k][row_k(z), seg_k(p), :]
+ * buffers = inputs then outputs; outputs are fully overwritten.  Stands for the call at
+ * cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_uniform_1d.py:294-316. */
+int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size,
+                 void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Stable grouping of n row ids (values in [0, nrows)) by value: offsets[nrows+1], perm[n].
+ * Deterministic (no atomics decide the order).  workspace: cueq_segment_csr_workspace(n, nrows) bytes. */
+int64_t cueq_segment_csr_workspace(int64_t n, int64_t nrows);
+int cueq_segment_csr_build(const void* index, int32_t index_is_64, int64_t n, int64_t nrows,
+                           int64_t* offsets, int64_t* perm, void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUEQ_AMD_H */
