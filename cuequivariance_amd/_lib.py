@@ -22,6 +22,7 @@ EXPORTED_SYMBOLS = (
     "cueq_version",
     "cueq_u1d_plan_create",
     "cueq_u1d_plan_destroy",
+    "cueq_u1d_plan_info",
     "cueq_u1d_workspace_size",
     "cueq_u1d_run",
     "cueq_segment_csr_workspace",
@@ -91,6 +92,8 @@ def load() -> C.CDLL:
         lib.cueq_u1d_plan_create.restype = C.c_int
         lib.cueq_u1d_plan_destroy.argtypes = [C.c_void_p]
         lib.cueq_u1d_plan_destroy.restype = None
+        lib.cueq_u1d_plan_info.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
+        lib.cueq_u1d_plan_info.restype = C.c_int
         lib.cueq_u1d_workspace_size.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64]
         lib.cueq_u1d_workspace_size.restype = C.c_int64
         lib.cueq_u1d_run.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]

@@ -55,6 +55,10 @@ def _compile(src: Path, obj: Path) -> None:
 
 def build_library(force: bool = False, jobs: int | None = None, verbose: bool = True) -> Path:
     BUILD.mkdir(exist_ok=True)
+    sys.path.insert(0, str(ROOT))
+    from cuequivariance_amd.codegen import registry as _registry
+
+    _registry.generate()
     srcs = sources()
     todo = []
     for s in srcs:

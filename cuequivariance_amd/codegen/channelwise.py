@@ -1,0 +1,525 @@
+"""Generator of straight-line gfx950 kernels for weighted channel-wise tensor products.
+
+Input: the flat uniform-1d tables of one operation with operands
+``[w (u-vector), x1 (u-vector), x2 (scalar), out (u-vector)]`` — the form a channel-wise
+tensor product takes after flattening the Clebsch-Gordan modes — i.e. for every path ``p``
+
+    out[k_p, u] += c_p * w[b_p, u] * x1[i_p, u] * x2[j_p]
+
+Output: HIP source with the path table unrolled into the instruction stream.
+
+Forward kernel (one wavefront = one output row x 64 channels):
+  * channels across lanes, so every HBM access is a contiguous 256-byte (fp32) line;
+  * the uniform factor ``c_p * x2[j_p]`` of each path lives in a table register: lane ``n`` of each
+    16-lane row holds the factor of a path whose ``x2`` index is ``n``; the FMA reads it with the DPP
+    ``row_newbcast:n`` modifier, which broadcasts lane ``n`` of every row to the row - no LDS traffic,
+    no scalar float arithmetic, one VALU instruction per path;
+  * ``w[b] * x1[i]`` is formed once per (block, i) and reused by all paths of the block;
+  * the batch rows that scatter into one output row are summed in registers in CSR order, then
+    stored once: deterministic, nothing of batch size is materialised.
+
+Backward kernel (one wavefront = a chunk of consecutive batch rows x 64 channels) computes the three
+gradients in one pass over the inputs.  With ``G[b][i][j] = sum_k C[i,j,k] g[k]`` (literal
+coefficients), ``D[b][i] = sum_j G[b][i][j] x2[j]`` and ``F[b][j] = sum_i G[b][i][j] x1[i]``:
+``dw[b] = sum_i x1[i] D[b][i]``, ``dx1[i] += w[b] D[b][i]``, ``dx2[j] = sum_u w[b] F[b][j]``.
+"""
+
+from __future__ import annotations
+
+import struct
+from collections import defaultdict
+from dataclasses import dataclass, field
+from typing import Sequence
+
+MASK64 = (1 << 64) - 1
+
+
+# ---------------------------------------------------------------------------------------------
+# descriptor hash (must match cueq::hash_u1d_desc in csrc/uniform1d.hip)
+# ---------------------------------------------------------------------------------------------
+def fnv64_words(words) -> int:
+    h = 1469598103934665603
+    for w in words:
+        w &= MASK64
+        for i in range(8):
+            h ^= (w >> (8 * i)) & 0xFF
+            h = (h * 1099511628211) & MASK64
+    return h
+
+
+def hash_tables(math_code: int, extent: int, nin: int, nout: int, buffer_dim, nseg, num_operands, operations,
+                num_paths, path_indices_start, path_coefficients_start, path_indices, path_coefficients) -> int:
+    words = [math_code, extent, nin, nout, *buffer_dim, *nseg, len(num_operands)]
+    off = 0
+    for o, nop in enumerate(num_operands):
+        words.append(nop)
+        words += list(operations[off: off + nop])
+        off += nop
+        words.append(num_paths[o])
+        pi0, pc0 = path_indices_start[o], path_coefficients_start[o]
+        words += list(path_indices[pi0: pi0 + num_paths[o] * nop])
+        for p in range(num_paths[o]):
+            words.append(struct.unpack("<Q", struct.pack("<d", float(path_coefficients[pc0 + p])))[0])
+    return fnv64_words(words)
+
+
+# ---------------------------------------------------------------------------------------------
+# structure analysis
+# ---------------------------------------------------------------------------------------------
+@dataclass
+class Block:
+    """All paths sharing one weight segment."""
+
+    b: int
+    entries: list = field(default_factory=list)  # (i, j, k, c)
+
+    @property
+    def i_list(self):
+        return sorted({e[0] for e in self.entries})
+
+    @property
+    def j_list(self):
+        return sorted({e[1] for e in self.entries})
+
+    @property
+    def k_list(self):
+        return sorted({e[2] for e in self.entries})
+
+
+@dataclass
+class ChannelwiseStructure:
+    extent: int
+    nseg_w: int
+    nseg_x1: int
+    nseg_x2: int
+    nseg_out: int
+    blocks: list
+
+    @property
+    def num_paths(self):
+        return sum(len(b.entries) for b in self.blocks)
+
+
+def analyze(extent: int, nseg: Sequence[int], paths: Sequence[tuple]) -> ChannelwiseStructure:
+    """``paths``: (w_seg, x1_seg, x2_seg, out_seg, coefficient)."""
+    blocks: dict[int, Block] = {}
+    for b, i, j, k, c in paths:
+        if c == 0.0:
+            continue
+        blocks.setdefault(b, Block(b)).entries.append((i, j, k, float(c)))
+    out = [blocks[b] for b in sorted(blocks)]
+    # Order blocks so that blocks reading the same x1 segments are neighbours (register reuse).
+    out.sort(key=lambda blk: (blk.i_list, blk.j_list, blk.b))
+    return ChannelwiseStructure(extent, nseg[0], nseg[1], nseg[2], nseg[3], out)
+
+
+def _lit(c: float, T: str) -> str:
+    s = repr(float(c))
+    if "e" not in s and "." not in s and "inf" not in s and "nan" not in s:
+        s += ".0"
+    return s + ("f" if T == "float" else "")
+
+
+# ---------------------------------------------------------------------------------------------
+# forward
+# ---------------------------------------------------------------------------------------------
+def _split_blocks(st: ChannelwiseStructure, nsplit: int) -> list[list[Block]]:
+    """Greedy balance of blocks over ``nsplit`` groups by path count, keeping the sorted order inside groups."""
+    groups = [[] for _ in range(nsplit)]
+    load = [0] * nsplit
+    for blk in sorted(st.blocks, key=lambda b: -len(b.entries)):
+        g = load.index(min(load))
+        groups[g].append(blk)
+        load[g] += len(blk.entries) + 2 * len(blk.k_list)
+    for g in groups:
+        g.sort(key=lambda blk: (blk.i_list, blk.j_list, blk.b))
+    return groups
+
+
+def _tables_for(blocks: Sequence[Block]):
+    """Assign every path a slot (table t, lane n): n = x2 index mod 16, one Y register per 16 x2 segments.
+
+    Returns (slots: {(b, idx_in_block): (t, n)}, table rows: list of (m, [coeff for n in 0..15])).
+    """
+    per_j = defaultdict(list)
+    for blk in blocks:
+        for e_idx, (i, j, k, c) in enumerate(blk.entries):
+            per_j[j].append((blk.b, e_idx, c))
+    tables = []  # (m, coeffs[16])
+    slots = {}
+    ms = sorted({j // 16 for j in per_j})
+    for m in ms:
+        depth = max(len(per_j[j]) for j in per_j if j // 16 == m)
+        base = len(tables)
+        for t in range(depth):
+            tables.append((m, [0.0] * 16))
+        for j in per_j:
+            if j // 16 != m:
+                continue
+            for t, (b, e_idx, c) in enumerate(per_j[j]):
+                tables[base + t][1][j % 16] = c
+                slots[(b, e_idx)] = (base + t, j % 16)
+    return slots, tables
+
+
+def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: int, ns: str) -> str:
+    """HIP source of the forward kernels (one ``__device__`` body per block group) in namespace ``ns``."""
+    fp = T
+    dpp = "v_fmac_f32_dpp" if T == "float" else "v_fmac_f64_dpp"
+    groups = _split_blocks(st, nsplit)
+    L = []
+    A = L.append
+    A(f"// forward: {st.num_paths} paths, {len(st.blocks)} blocks, split over {nsplit} wave group(s)")
+    all_tables = []
+    group_meta = []
+    for q, blocks in enumerate(groups):
+        slots, tables = _tables_for(blocks)
+        group_meta.append((slots, len(all_tables), len(tables)))
+        all_tables += tables
+    A(f"__device__ const {fp} fwd_ctab[{max(1, len(all_tables)) * 16}] = {{")
+    for m, row in all_tables:
+        A("  " + ", ".join(_lit(c, T) for c in row) + ",")
+    A("};")
+    A(f"constexpr int kFwdTables = {len(all_tables)};")
+    A("")
+    for q, blocks in enumerate(groups):
+        slots, tbase, ntab = group_meta[q]
+        tables = all_tables[tbase: tbase + ntab]
+        ks = sorted({k for blk in blocks for k in blk.k_list})
+        i_used = sorted({i for blk in blocks for i in blk.i_list})
+        ms = sorted({m for m, _ in tables})
+        A(f"template <bool X1_IDX, bool W_SHARED>")
+        A(f"__device__ __forceinline__ void fwd_group{q}(FWD_PARAMS, const {fp}* s_c, int64_t r, int lane, int uu, bool active) {{")
+        for k in ks:
+            A(f"  {fp} acc{k} = 0;")
+        A("  int64_t z0, z1;")
+        A("  if (csr_offsets) { z0 = csr_offsets[r]; z1 = csr_offsets[r + 1]; } else { z0 = r; z1 = r + 1; }")
+        A("  const int n16 = lane & 15;")
+        A("  for (int64_t zz = z0; zz < z1; ++zz) {")
+        A("    const int64_t z = csr_perm ? csr_perm[zz] : zz;")
+        A("    int64_t srow = z;")
+        A("    if (X1_IDX) srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
+        A(f"    const {fp}* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
+        A(f"    const {fp}* __restrict__ wp = w + (W_SHARED ? 0 : z * {st.nseg_w * st.extent}ll);")
+        A(f"    const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
+        for m in ms:
+            nvalid = min(16, st.nseg_x2 - 16 * m)
+            A(f"    const {fp} yv{m} = x2p[{16 * m} + (n16 < {nvalid} ? n16 : 0)];")
+        for i in i_used:
+            A(f"    const {fp} xv{i} = x1p[{i * st.extent} + uu];")
+        for blk in blocks:
+            A(f"    const {fp} wv{blk.b} = wp[{blk.b * st.extent} + uu];")
+        # tables
+        for t, (m, _row) in enumerate(tables):
+            A(f"    {fp} t{t} = s_c[{(tbase + t) * 16} + n16] * yv{m};")
+        # fence: table registers are produced by VALU and consumed through DPP
+        names = [f"t{t}" for t in range(ntab)]
+        for c0 in range(0, len(names), 12):
+            ops = ", ".join(f'"+v"({n})' for n in names[c0: c0 + 12])
+            A(f'    asm volatile("s_nop 1" : {ops});')
+        for blk in blocks:
+            A(f"    {{  // block w[{blk.b}]: x1 {blk.i_list} x x2 {blk.j_list} -> out {blk.k_list}")
+            for i in blk.i_list:
+                A(f"      const {fp} wx{i} = wv{blk.b} * xv{i};")
+            for e_idx, (i, j, k, c) in enumerate(blk.entries):
+                t, n = slots[(blk.b, e_idx)]
+                A(f'      asm("{dpp} %0, %1, %2 row_newbcast:{n} row_mask:0xf bank_mask:0xf" : "+v"(acc{k}) : "v"(t{t}), "v"(wx{i}));')
+            A("    }")
+        A("  }")
+        A("  if (active) {")
+        A(f"    {fp}* __restrict__ op = out + r * {st.nseg_out * st.extent}ll;")
+        for k in ks:
+            A(f"    op[{k * st.extent} + uu] = acc{k};")
+        A("  }")
+        A("}")
+        A("")
+    # kernel
+    nch = (st.extent + 63) // 64
+    A("template <bool X1_IDX, bool W_SHARED>")
+    A(f"__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu({waves_per_eu}))) fwd_kernel(FWD_PARAMS) {{")
+    A(f"  __shared__ {fp} s_c[{max(1, len(all_tables)) * 16}];")
+    A("  const int lane = threadIdx.x;")
+    A(f"  for (int i = lane; i < {len(all_tables) * 16}; i += 64) s_c[i] = fwd_ctab[i];")
+    A("  __syncthreads();")
+    A("  int64_t wid = blockIdx.x;")
+    A(f"  const int q = static_cast<int>(wid % {nsplit}); wid /= {nsplit};")
+    A(f"  const int ch = static_cast<int>(wid % {nch}); const int64_t r = wid / {nch};")
+    if st.extent % 64 == 0:
+        A("  const int uu = ch * 64 + lane; constexpr bool active = true;")
+    else:
+        A(f"  const int u = ch * 64 + lane; const bool active = u < {st.extent}; const int uu = active ? u : 0;")
+    A("  switch (q) {")
+    for q in range(nsplit):
+        A(f"    case {q}: fwd_group{q}<X1_IDX, W_SHARED>(FWD_ARGS, s_c, r, lane, uu, active); break;")
+    A("  }")
+    A("}")
+    A(f"constexpr int kFwdSplit = {nsplit};")
+    A(f"constexpr int kChunks = {nch};")
+    return "\n".join(L)
+
+
+# ---------------------------------------------------------------------------------------------
+# backward
+# ---------------------------------------------------------------------------------------------
+def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: int) -> str:
+    """HIP source of the fused backward kernel (dw, dx1, dx2 in one pass)."""
+    fp = T
+    L = []
+    A = L.append
+    A(f"// backward: fused dw / dx1 / dx2, {chunk} batch rows per wavefront")
+    A("template <bool X1_IDX, bool G_IDX, bool ATOMIC_DX1>")
+    A(f"__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu({waves_per_eu}))) bwd_kernel(BWD_PARAMS) {{")
+    nch = (st.extent + 63) // 64
+    A("  const int lane = threadIdx.x;")
+    A("  int64_t wid = blockIdx.x;")
+    A(f"  const int ch = static_cast<int>(wid % {nch}); const int64_t cid = wid / {nch};")
+    if st.extent % 64 == 0:
+        A("  const int uu = ch * 64 + lane; constexpr bool active = true;")
+    else:
+        A(f"  const int u = ch * 64 + lane; const bool active = u < {st.extent}; const int uu = active ? u : 0;")
+    A(f"  const int64_t z0 = cid * {chunk}ll; const int64_t z1 = (z0 + {chunk} < batch) ? z0 + {chunk} : batch;")
+    for k in range(st.nseg_out):
+        A(f"  {fp} gr{k} = 0;")
+    A("  int64_t grow_cur = -1;")
+    A("  for (int64_t z = z0; z < z1; ++z) {")
+    A("    int64_t grow = z;")
+    A("    if (G_IDX) grow = g_idx64 ? static_cast<const int64_t*>(g_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(g_index)[z]);")
+    A("    if (grow != grow_cur) {")
+    A("      grow_cur = grow;")
+    A(f"      const {fp}* __restrict__ gp = g + grow * {st.nseg_out * st.extent}ll;")
+    for k in range(st.nseg_out):
+        A(f"      gr{k} = gp[{k * st.extent} + uu];")
+    A("    }")
+    A("    int64_t srow = z;")
+    A("    if (X1_IDX) srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
+    A(f"    const {fp}* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
+    A(f"    const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
+    A(f"    const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
+    A(f"    {fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
+    i_used = sorted({i for blk in st.blocks for i in blk.i_list})
+    j_used = sorted({j for blk in st.blocks for j in blk.j_list})
+    for i in i_used:
+        A(f"    const {fp} xv{i} = x1p[{i * st.extent} + uu];")
+    for blk in st.blocks:
+        A(f"    const {fp} wv{blk.b} = wp[{blk.b * st.extent} + uu];")
+    for j in j_used:
+        A(f"    const {fp} yv{j} = x2p[{j}];")
+    for i in i_used:
+        A(f"    {fp} dxa{i} = 0;")
+    for j in j_used:
+        A(f"    {fp} pj{j} = 0;")
+    for blk in st.blocks:
+        A(f"    {{  // block w[{blk.b}]")
+        A(f"      const {fp} wb = wv{blk.b};")
+        gij = defaultdict(list)
+        for i, j, k, c in blk.entries:
+            gij[(i, j)].append((k, c))
+        A(f"      {fp} dwb = 0;")
+        for j in blk.j_list:
+            A(f"      {fp} F{j} = 0;")
+        # per x1 component: G = sum_k c g_k is a temporary feeding both D (with x2) and F (with x1)
+        for i in blk.i_list:
+            A("      {")
+            A(f"        {fp} D = 0;")
+            for j in blk.j_list:
+                if (i, j) not in gij:
+                    continue
+                expr = None
+                for k, c in gij[(i, j)]:
+                    expr = f"{_lit(c, T)} * gr{k}" if expr is None else f"fma({_lit(c, T)}, gr{k}, {expr})"
+                A(f"        {{ const {fp} G = {expr}; D = fma(G, yv{j}, D); F{j} = fma(G, xv{i}, F{j}); }}")
+            A(f"        dwb = fma(xv{i}, D, dwb); dxa{i} = fma(wb, D, dxa{i});")
+            A("      }")
+        A(f"      if (active) dwp[{blk.b * st.extent} + uu] = dwb;")
+        for j in blk.j_list:
+            A(f"      pj{j} = fma(wb, F{j}, pj{j});")
+        A("    }")
+        A("    __builtin_amdgcn_sched_barrier(0);")
+    # dx1: scatter
+    A("    if (active) {")
+    A("      if (ATOMIC_DX1) {")
+    A(f"        {fp}* dp = dx1 + srow * {st.nseg_x1 * st.extent}ll;")
+    for i in i_used:
+        A(f"        unsafeAtomicAdd(dp + ({i * st.extent} + uu), dxa{i});")
+    A("      } else {")
+    A(f"        {fp}* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
+    for i in range(st.nseg_x1):
+        A(f"        dp[{i * st.extent} + uu] = " + (f"dxa{i};" if i in i_used else "0;"))
+    A("      }")
+    A("    }")
+    # dx2: reduce over the 64 lanes, then combine channel chunks
+    A("    if (!active) {" + " ".join(f"pj{j} = 0;" for j in j_used) + "}")
+    for j in j_used:
+        A(f"    pj{j} = wave_sum(pj{j});")
+    if nch == 1:
+        A("    if (lane == 0) {")
+        A(f"      {fp}* __restrict__ d2 = dx2 + z * {st.nseg_x2}ll;")
+        for j in range(st.nseg_x2):
+            A(f"      d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+        A("    }")
+    else:
+        A("    if (lane == 0) {")
+        A(f"      {fp}* __restrict__ d2 = dx2_partial + (z * {nch} + ch) * {st.nseg_x2}ll;")
+        for j in range(st.nseg_x2):
+            A(f"      d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+        A("    }")
+    A("  }")
+    A("}")
+    A(f"constexpr int kBwdChunk = {chunk};")
+    return "\n".join(L)
+
+
+
+# ---------------------------------------------------------------------------------------------
+# translation unit
+# ---------------------------------------------------------------------------------------------
+FWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}* __restrict__ x2, {T}* __restrict__ out, "
+              "const void* __restrict__ x1_index, int x1_idx64, const int64_t* __restrict__ csr_offsets, "
+              "const int64_t* __restrict__ csr_perm")
+FWD_ARGS = "w, x1, x2, out, x1_index, x1_idx64, csr_offsets, csr_perm"
+BWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}* __restrict__ x2, const {T}* __restrict__ g, "
+              "{T}* __restrict__ dw, {T}* dx1, {T}* __restrict__ dx1_partial, {T}* __restrict__ dx2, "
+              "{T}* __restrict__ dx2_partial, const void* __restrict__ x1_index, int x1_idx64, "
+              "const void* __restrict__ g_index, int g_idx64, int64_t batch")
+
+
+def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_hash: int, *, fwd_split: int = 1,
+              fwd_waves: int = 2, bwd_waves: int = 2, bwd_chunk: int = 16) -> str:
+    """Complete .hip translation unit: kernels, host launchers, registration under both table hashes."""
+    ns = f"cw_{name}"
+    nch = (st.extent + 63) // 64
+    W1, WW, W2, WO = st.nseg_x1 * st.extent, st.nseg_w * st.extent, st.nseg_x2, st.nseg_out * st.extent
+    out = []
+    A = out.append
+    A("// GENERATED by cuequivariance_amd/codegen/channelwise.py - do not edit.")
+    A(f"// channel-wise tensor product '{name}': extent {st.extent}, segments w/x1/x2/out = "
+      f"{st.nseg_w}/{st.nseg_x1}/{st.nseg_x2}/{st.nseg_out}, {st.num_paths} paths, math {T}")
+    A('#include "cw_common.h"')
+    A("")
+    A("namespace cueq {")
+    A(f"namespace {ns} {{")
+    A(f"#define FWD_PARAMS {FWD_PARAMS.format(T=T)}")
+    A(f"#define FWD_ARGS {FWD_ARGS}")
+    A(f"#define BWD_PARAMS {BWD_PARAMS.format(T=T)}")
+    A("")
+    A(emit_forward(st, T, fwd_split, fwd_waves, ns))
+    A("")
+    A(emit_backward(st, T, bwd_waves, bwd_chunk))
+    A("")
+    code = f"dtype_code<{T}>::value"
+    A(f"""
+static bool all_dtype(const cueq_u1d_buffer* b, int n) {{
+  for (int i = 0; i < n; ++i) if (b[i].dtype != {code}) return false;
+  return true;
+}}
+
+// buffers: w, x1, x2 | out
+static int run_fwd(const SpecCall& c) {{
+  const cueq_u1d_buffer* b = c.buffers;
+  if (!all_dtype(b, 4)) return CUEQ_ERR_UNSUPPORTED;
+  if (b[2].batch_dim != CUEQ_BATCH_BATCHED) return CUEQ_ERR_UNSUPPORTED;
+  if (b[0].batch_dim == CUEQ_BATCH_INDEXED || b[1].batch_dim == CUEQ_BATCH_SHARED) return CUEQ_ERR_UNSUPPORTED;
+  if (b[3].batch_dim == CUEQ_BATCH_SHARED) return CUEQ_ERR_UNSUPPORTED;
+  const bool x1_idx = b[1].batch_dim == CUEQ_BATCH_INDEXED, w_shared = b[0].batch_dim == CUEQ_BATCH_SHARED;
+  const bool out_idx = b[3].batch_dim == CUEQ_BATCH_INDEXED;
+  if (out_idx && (!b[3].csr_offsets || (!b[3].csr_perm && c.batch > 0))) return CUEQ_ERR_UNSUPPORTED;
+  const int64_t rows = b[3].rows;
+  if (rows == 0) return CUEQ_OK;
+  const int64_t grid = rows * {nch} * kFwdSplit;
+  CUEQ_REQUIRE(grid < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "too many output rows for one launch");
+  const {T}* w = static_cast<const {T}*>(b[0].data);
+  const {T}* x1 = static_cast<const {T}*>(b[1].data);
+  const {T}* x2 = static_cast<const {T}*>(b[2].data);
+  {T}* o = static_cast<{T}*>(b[3].data);
+  const int64_t* offs = out_idx ? b[3].csr_offsets : nullptr;
+  const int64_t* perm = out_idx ? b[3].csr_perm : nullptr;
+  const dim3 g(static_cast<unsigned>(grid)), t(64);
+#define LAUNCH_FWD(XI, WS) hipLaunchKernelGGL((fwd_kernel<XI, WS>), g, t, 0, c.stream, w, x1, x2, o, b[1].index, b[1].index_is_64, offs, perm)
+  if (x1_idx && w_shared) LAUNCH_FWD(true, true);
+  else if (x1_idx) LAUNCH_FWD(true, false);
+  else if (w_shared) LAUNCH_FWD(false, true);
+  else LAUNCH_FWD(false, false);
+#undef LAUNCH_FWD
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}}
+
+// buffers: w, x1, x2, g | dw, dx1, dx2
+static int64_t bwd_workspace(const cueq_u1d_buffer* b, int64_t batch) {{
+  int64_t need = 0;
+  if ({nch} > 1) need += batch * {nch} * {W2}ll * sizeof({T});
+  need = (need + 255) & ~int64_t(255);
+  if (b[1].batch_dim == CUEQ_BATCH_INDEXED && deterministic_scatter()) need += batch * {W1}ll * sizeof({T});
+  return need;
+}}
+
+static int run_bwd(const SpecCall& c) {{
+  const cueq_u1d_buffer* b = c.buffers;
+  if (!all_dtype(b, 7)) return CUEQ_ERR_UNSUPPORTED;
+  if (b[0].batch_dim != CUEQ_BATCH_BATCHED || b[2].batch_dim != CUEQ_BATCH_BATCHED) return CUEQ_ERR_UNSUPPORTED;
+  if (b[1].batch_dim == CUEQ_BATCH_SHARED || b[3].batch_dim == CUEQ_BATCH_SHARED) return CUEQ_ERR_UNSUPPORTED;
+  if (b[4].batch_dim != CUEQ_BATCH_BATCHED || b[6].batch_dim != CUEQ_BATCH_BATCHED) return CUEQ_ERR_UNSUPPORTED;
+  if (b[5].batch_dim != b[1].batch_dim) return CUEQ_ERR_UNSUPPORTED;
+  const bool x1_idx = b[1].batch_dim == CUEQ_BATCH_INDEXED, g_idx = b[3].batch_dim == CUEQ_BATCH_INDEXED;
+  if (x1_idx && (b[5].index != b[1].index || b[5].rows != b[1].rows)) return CUEQ_ERR_UNSUPPORTED;
+  const bool det = deterministic_scatter();
+  if (x1_idx && det && (!b[5].csr_offsets || (!b[5].csr_perm && c.batch > 0))) return CUEQ_ERR_UNSUPPORTED;
+  const int64_t batch = c.batch;
+  const {T}* w = static_cast<const {T}*>(b[0].data);
+  const {T}* x1 = static_cast<const {T}*>(b[1].data);
+  const {T}* x2 = static_cast<const {T}*>(b[2].data);
+  const {T}* g = static_cast<const {T}*>(b[3].data);
+  {T}* dw = static_cast<{T}*>(b[4].data);
+  {T}* dx1 = static_cast<{T}*>(b[5].data);
+  {T}* dx2 = static_cast<{T}*>(b[6].data);
+  const int64_t need = bwd_workspace(b, batch);
+  CUEQ_REQUIRE(need == 0 || (c.workspace && c.workspace_bytes >= need), CUEQ_ERR_INVALID, "workspace too small: need %lld bytes", (long long)need);
+  char* ws = static_cast<char*>(c.workspace);
+  {T}* dx2_partial = nullptr;
+  int64_t off = 0;
+  if ({nch} > 1) {{ dx2_partial = reinterpret_cast<{T}*>(ws); off = (batch * {nch} * {W2}ll * sizeof({T}) + 255) & ~int64_t(255); }}
+  {T}* dx1_partial = nullptr;
+  bool atomic = false;
+  if (!x1_idx) dx1_partial = dx1;  // one row per batch element: plain stores
+  else if (det) dx1_partial = reinterpret_cast<{T}*>(ws + off);
+  else atomic = true;
+  if (atomic && b[5].rows > 0) {{
+    const int64_t n = b[5].rows * {W1}ll;
+    hipLaunchKernelGGL(fill_zero<{T}>, dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1, n);
+    CUEQ_CHECK_HIP(hipGetLastError());
+  }}
+  if (batch > 0) {{
+    const int64_t nchunks = (batch + kBwdChunk - 1) / kBwdChunk;
+    const int64_t grid = nchunks * {nch};
+    CUEQ_REQUIRE(grid < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "batch too large for one launch");
+    const dim3 gd(static_cast<unsigned>(grid)), t(64);
+#define LAUNCH_BWD(XI, GI, AT) hipLaunchKernelGGL((bwd_kernel<XI, GI, AT>), gd, t, 0, c.stream, w, x1, x2, g, dw, dx1, dx1_partial, dx2, dx2_partial, b[1].index, b[1].index_is_64, b[3].index, b[3].index_is_64, batch)
+    if (x1_idx && g_idx && atomic) LAUNCH_BWD(true, true, true);
+    else if (x1_idx && g_idx) LAUNCH_BWD(true, true, false);
+    else if (x1_idx && atomic) LAUNCH_BWD(true, false, true);
+    else if (x1_idx) LAUNCH_BWD(true, false, false);
+    else if (g_idx) LAUNCH_BWD(false, true, false);
+    else LAUNCH_BWD(false, false, false);
+#undef LAUNCH_BWD
+    CUEQ_CHECK_HIP(hipGetLastError());
+    if ({nch} > 1) {{
+      hipLaunchKernelGGL(fold_parts<{T}>, dim3(blocks_for(batch * {W2}ll)), dim3(256), 0, c.stream, dx2_partial, batch, {nch}, {W2}, dx2);
+      CUEQ_CHECK_HIP(hipGetLastError());
+    }}
+  }}
+  if (x1_idx && det && b[5].rows > 0) {{
+    const int64_t n = b[5].rows * {W1}ll;
+    hipLaunchKernelGGL(segment_sum_rows<{T}>, dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1_partial, b[5].csr_offsets, b[5].csr_perm, b[5].rows, {W1}, dx1);
+    CUEQ_CHECK_HIP(hipGetLastError());
+  }}
+  return CUEQ_OK;
+}}
+
+static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{T}", run_fwd, nullptr}};
+static const U1dSpec spec_bwd = {{0x{bwd_hash:016x}ull, "{name}_bwd_{T}", run_bwd, bwd_workspace}};
+static SpecRegistrar reg_fwd(&spec_fwd);
+static SpecRegistrar reg_bwd(&spec_bwd);
+""")
+    A(f"}}  // namespace {ns}")
+    A("}  // namespace cueq")
+    return "\n".join(out) + "\n"

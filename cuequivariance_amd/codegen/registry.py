@@ -1,0 +1,52 @@
+"""Descriptors for which specialised kernels are generated when the library is built.
+
+Each entry yields one translation unit in ``csrc/generated`` holding a forward kernel and a fused
+backward kernel (all three gradients).  Anything not listed runs on the table-driven kernels.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+
+from .. import cue
+from ..tables import U1dTables
+from . import channelwise as cw
+
+GENERATED_DIR = Path(__file__).resolve().parent.parent / "csrc" / "generated"
+
+# (name, irreps_in1, irreps_in2, filter, tuning)
+CHANNELWISE = [
+    ("c128_l3", "128x0e+128x1o+128x2e+128x3o", "0e+1o+2e+3o", "0e+1o+2e+3o", {}),
+    ("c32_l2", "32x0e+32x1o+32x2e", "0e+1o+2e", "0e+1o+2e", {}),
+]
+
+MATH = (("float", 0), ("double", 1))
+
+
+def channelwise_tables(irreps1: str, irreps2: str, filt) -> U1dTables:
+    e = cue.descriptors.channelwise_tensor_product(cue.Irreps("O3", irreps1), cue.Irreps("O3", irreps2), filt)
+    return U1dTables.from_polynomial(e.polynomial.flatten_coefficient_modes().squeeze_modes())
+
+
+def generate(verbose: bool = False) -> list[Path]:
+    GENERATED_DIR.mkdir(parents=True, exist_ok=True)
+    written = []
+    for name, ir1, ir2, filt, tuning in CHANNELWISE:
+        t = channelwise_tables(ir1, ir2, filt)
+        assert t.operations == (0, 1, 2, 3) and t.buffer_dim == (1, 1, 0, 1)
+        _, paths = t.operation(0)
+        st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
+        tb = t.backward((True, True, True))
+        for T, code in MATH:
+            src = cw.emit_unit(st, T, name, t.content_hash(code), tb.content_hash(code), **tuning.get(T, {}))
+            path = GENERATED_DIR / f"cw_{name}_{T}.hip"
+            if not path.exists() or path.read_text() != src:
+                path.write_text(src)
+            written.append(path)
+            if verbose:
+                print(f"generated {path.name}: {st.num_paths} paths")
+    return written
+
+
+if __name__ == "__main__":
+    generate(verbose=True)

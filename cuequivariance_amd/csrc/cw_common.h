@@ -1,0 +1,83 @@
+// Helpers shared by the generated channel-wise kernels: wavefront reductions and the small
+// streaming kernels that finish a backward pass (row gather-sum, partial folding, zero fill).
+#pragma once
+
+#include "common.h"
+#include "u1d_spec.h"
+
+namespace cueq {
+
+// ---- DPP lane exchange ------------------------------------------------------------------------
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ double dpp_move(double v) {
+  const uint64_t b = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b & 0xffffffffu), CTRL, ROW_MASK, 0xf, true));
+  const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b >> 32), CTRL, ROW_MASK, 0xf, true));
+  return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// Sum over the 64 lanes, result valid in every lane.  Fixed butterfly: bit-reproducible.
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+  v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_move<0x141>(v);  // row_half_mirror
+  v += dpp_move<0x140>(v);  // row_mirror: every lane holds its row's sum
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// ---- finishing kernels ------------------------------------------------------------------------
+// out[r, :] = sum over zz in [offsets[r], offsets[r+1]) of partial[perm[zz], :]   (width elements per row)
+template <typename T>
+__global__ void __launch_bounds__(256) segment_sum_rows(const T* __restrict__ partial, const int64_t* __restrict__ offsets,
+                                                        const int64_t* __restrict__ perm, int64_t nrows, int width,
+                                                        T* __restrict__ out) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t r = tid / width;
+  if (r >= nrows) return;
+  const int c = static_cast<int>(tid - r * width);
+  T acc = 0;
+  for (int64_t zz = offsets[r]; zz < offsets[r + 1]; ++zz) acc += partial[perm[zz] * width + c];
+  out[tid] = acc;
+}
+
+// out[z, j] = sum over c in [0, nparts) of partial[(z * nparts + c), j]
+template <typename T>
+__global__ void __launch_bounds__(256) fold_parts(const T* __restrict__ partial, int64_t n, int nparts, int width,
+                                                  T* __restrict__ out) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= n * width) return;
+  const int64_t z = tid / width;
+  const int j = static_cast<int>(tid - z * width);
+  T acc = 0;
+  for (int c = 0; c < nparts; ++c) acc += partial[(z * nparts + c) * width + j];
+  out[tid] = acc;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) fill_zero(T* __restrict__ p, int64_t n) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid < n) p[tid] = 0;
+}
+
+inline unsigned blocks_for(int64_t n, int per_block = 256) { return static_cast<unsigned>((n + per_block - 1) / per_block); }
+
+// Scatter policy of the fused backward for the gradient of a gathered operand:
+// hardware floating-point atomics (fast, summation order varies) or per-row partials
+// followed by a gather-sum in index order (bit-reproducible, one extra pass over batch x row).
+inline bool deterministic_scatter() {
+  const char* e = getenv("CUEQ_DETERMINISTIC");
+  return e && e[0] == '1';
+}
+
+template <typename T> struct dtype_code;
+template <> struct dtype_code<float> { static constexpr int value = CUEQ_F32; };
+template <> struct dtype_code<double> { static constexpr int value = CUEQ_F64; };
+
+}  // namespace cueq

@@ -1,0 +1,52 @@
+// Registry of descriptor-specialised uniform-1d kernels.
+//
+// The generic executor interprets path tables at run time.  For descriptors known when the
+// library is built, straight-line kernels are generated (cuequivariance_amd/codegen) with the
+// path table baked into the instruction stream; each generated translation unit registers
+// itself here under a content hash of the descriptor tables.  cueq_u1d_plan_create computes the
+// same hash and, when it finds an entry, cueq_u1d_run tries it first; the entry may decline a
+// call shape (returns CUEQ_ERR_UNSUPPORTED), in which case the generic kernels run.
+#pragma once
+
+#include <cstdint>
+
+#include "common.h"
+
+namespace cueq {
+
+struct SpecCall {
+  const cueq_u1d_buffer* buffers;  // inputs then outputs
+  int64_t batch;
+  void* workspace;
+  int64_t workspace_bytes;
+  hipStream_t stream;
+};
+
+struct U1dSpec {
+  uint64_t hash;
+  const char* name;
+  int (*run)(const SpecCall& call);                                    // CUEQ_OK / CUEQ_ERR_UNSUPPORTED / error
+  int64_t (*workspace)(const cueq_u1d_buffer* buffers, int64_t batch);  // bytes, may be null
+};
+
+void register_u1d_spec(const U1dSpec* spec);
+const U1dSpec* find_u1d_spec(uint64_t hash);
+
+// FNV-1a over a stream of 64-bit words (little endian bytes); the generator computes the same.
+struct Fnv64 {
+  uint64_t h = 1469598103934665603ull;
+  void word(uint64_t w) {
+    for (int i = 0; i < 8; ++i) {
+      h ^= (w >> (8 * i)) & 0xff;
+      h *= 1099511628211ull;
+    }
+  }
+};
+
+uint64_t hash_u1d_desc(const cueq_u1d_desc* d);
+
+struct SpecRegistrar {
+  explicit SpecRegistrar(const U1dSpec* s) { register_u1d_spec(s); }
+};
+
+}  // namespace cueq

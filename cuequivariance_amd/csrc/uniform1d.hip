@@ -13,16 +13,59 @@
 // for a one-row output).
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
 #include <vector>
 
 #include "common.h"
+#include "u1d_spec.h"
 
 namespace cueq {
 
 static thread_local std::string g_error;
+
+// ---- registry of specialised kernels (filled by static initialisers of generated files) ----
+static std::vector<const U1dSpec*>& spec_list() {
+  static std::vector<const U1dSpec*> v;
+  return v;
+}
+void register_u1d_spec(const U1dSpec* spec) { spec_list().push_back(spec); }
+const U1dSpec* find_u1d_spec(uint64_t hash) {
+  for (const U1dSpec* s : spec_list())
+    if (s->hash == hash) return s;
+  return nullptr;
+}
+
+uint64_t hash_u1d_desc(const cueq_u1d_desc* d) {
+  Fnv64 f;
+  const int nbuf = d->num_inputs + d->num_outputs;
+  f.word(static_cast<uint64_t>(d->math_dtype));
+  f.word(static_cast<uint64_t>(d->operand_extent));
+  f.word(static_cast<uint64_t>(d->num_inputs));
+  f.word(static_cast<uint64_t>(d->num_outputs));
+  for (int b = 0; b < nbuf; ++b) f.word(static_cast<uint64_t>(d->buffer_dim[b]));
+  for (int b = 0; b < nbuf; ++b) f.word(static_cast<uint64_t>(d->buffer_num_segments[b]));
+  f.word(static_cast<uint64_t>(d->num_operations));
+  int64_t off = 0;
+  for (int o = 0; o < d->num_operations; ++o) {
+    const int nop = d->num_operands[o];
+    f.word(static_cast<uint64_t>(nop));
+    for (int k = 0; k < nop; ++k) f.word(static_cast<uint64_t>(d->operations[off + k]));
+    off += nop;
+    f.word(static_cast<uint64_t>(d->num_paths[o]));
+    const int64_t pi0 = d->path_indices_start[o], pc0 = d->path_coefficients_start[o];
+    for (int64_t i = 0; i < static_cast<int64_t>(d->num_paths[o]) * nop; ++i)
+      f.word(static_cast<uint64_t>(d->path_indices[pi0 + i]));
+    for (int p = 0; p < d->num_paths[o]; ++p) {
+      uint64_t bits;
+      std::memcpy(&bits, &d->path_coefficients[pc0 + p], 8);
+      f.word(bits);
+    }
+  }
+  return f.h;
+}
 
 void set_error(const char* fmt, ...) {
   char buf[1024];
@@ -167,6 +210,8 @@ struct cueq_u1d_plan {
   int32_t num_inputs, num_outputs;
   std::vector<int32_t> buffer_dim, buffer_nseg;
   std::vector<OutTables> out;  // one per output buffer
+  const cueq::U1dSpec* spec = nullptr;  // descriptor-specialised kernels, if any were built
+  uint64_t hash = 0;
   void* device_blob = nullptr;
   int device = 0;
 };
@@ -291,8 +336,17 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
     t.seg_start = reinterpret_cast<int32_t*>(base + offs[ob].seg);
     t.contracts_channel = contracts[ob];
   }
+  plan->hash = hash_u1d_desc(d);
+  plan->spec = find_u1d_spec(plan->hash);
   *out_plan = plan;
   return CUEQ_OK;
+}
+
+// 1 when descriptor-specialised kernels exist for this plan, else 0; *hash receives the table hash.
+extern "C" int cueq_u1d_plan_info(const cueq_u1d_plan* plan, uint64_t* hash) {
+  if (!plan) return 0;
+  if (hash) *hash = plan->hash;
+  return plan->spec ? 1 : 0;
 }
 
 extern "C" void cueq_u1d_plan_destroy(cueq_u1d_plan* plan) {
@@ -307,6 +361,7 @@ extern "C" int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq
   if (!plan || !buffers) return 0;
   const int msize = plan->math_dtype == CUEQ_F64 ? 8 : 4;
   int64_t need = 0;
+  if (plan->spec && plan->spec->workspace) need = plan->spec->workspace(buffers, batch);
   for (int ob = 0; ob < plan->num_outputs; ++ob) {
     const int b = plan->num_inputs + ob;
     if (buffers[b].batch_dim != CUEQ_BATCH_SHARED) continue;
@@ -409,6 +464,11 @@ extern "C" int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* bu
   CUEQ_REQUIRE(plan && buffers, CUEQ_ERR_INVALID, "null argument");
   CUEQ_REQUIRE(batch >= 0, CUEQ_ERR_INVALID, "negative batch size");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (plan->spec && !getenv("CUEQ_FORCE_GENERIC")) {
+    SpecCall call{buffers, batch, workspace, workspace_bytes, s};
+    const int rc = plan->spec->run(call);
+    if (rc != CUEQ_ERR_UNSUPPORTED) return rc;
+  }
   if (plan->math_dtype == CUEQ_F64) return run_typed<double>(plan, buffers, batch, workspace, workspace_bytes, s);
   return run_typed<float>(plan, buffers, batch, workspace, workspace_bytes, s);
 }

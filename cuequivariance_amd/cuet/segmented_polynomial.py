@@ -13,13 +13,13 @@ Mirror of ``cuequivariance_torch/cuequivariance_torch/primitives/segmented_polyn
 from __future__ import annotations
 
 import warnings
-from itertools import accumulate
 from typing import Any, Dict, List, Optional
 
 import torch
 import torch.nn as nn
 
 from .. import cue
+from ..tables import U1dTables
 from . import uniform_1d as u1d
 
 __all__ = ["SegmentedPolynomial", "SegmentedPolynomialFromUniform1d"]
@@ -64,7 +64,6 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
             ) from e
         polynomial = polynomial.squeeze_modes()
 
-        operand_extent = None
         for o in polynomial.operands:
             torch._assert(o.ndim in [0, 1], "For method 'uniform_1d', only 0D (scalar) or 1D operands are supported.")
             torch._assert(
@@ -73,41 +72,34 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
                 "If segment extents differ but share a common divisor, preprocess the polynomial with "
                 "'split_mode()' to obtain uniform segment extents.",
             )
-            if o.ndim == 1 and len(o.segments) > 0:
-                if operand_extent is None:
-                    (operand_extent,) = o.segment_shape
-                else:
-                    torch._assert(
-                        (operand_extent,) == o.segment_shape,
-                        "For method 'uniform_1d', all 1D operands must share the same segment extent.",
-                    )
-        if operand_extent is None:
-            operand_extent = 1
         for ope, stp in polynomial.operations:
             torch._assert(stp.num_operands == len(ope.buffers), "operation/operand count mismatch")
             torch._assert(
                 stp.coefficient_subscripts == "",
                 "In method 'uniform_1d', coefficients must be scalar (coefficient_subscripts must be empty).",
             )
-
+        try:
+            tables = U1dTables.from_polynomial(polynomial, output_dtype_map)
+        except ValueError as e:
+            raise ValueError(f"For method 'uniform_1d': {e}") from e
+        self.tables = tables
         self.num_inputs = polynomial.num_inputs
         self.num_outputs = polynomial.num_outputs
         self.name = name
         self.math_dtype = _resolve_math_dtype(math_dtype, "uniform_1d")
-        self.operand_extent = operand_extent
-        self.buffer_dim = [o.ndim for o in polynomial.operands]
-        self.buffer_num_segments = [len(o.segments) for o in polynomial.operands]
-        default_map = [0 if polynomial.num_inputs >= 1 else -1] * polynomial.num_outputs
-        self.dtypes = list(range(self.num_inputs)) + (default_map if output_dtype_map is None else list(output_dtype_map))
-        ops = polynomial.operations
-        self.num_operations = len(ops)
-        self.num_operands = [len(o.buffers) for o, _ in ops]
-        self.operations = [b for o, _ in ops for b in o.buffers]
-        self.num_paths = [s.num_paths for _, s in ops]
-        self.path_indices_start = [0] + list(accumulate(s.num_paths * s.num_operands for _, s in ops))[:-1]
-        self.path_coefficients_start = [0] + list(accumulate(s.num_paths for _, s in ops))[:-1]
-        self.path_indices = [i for _, s in ops for p in s.paths for i in p.indices]
-        self.path_coefficients = [float(p.coefficients) for _, s in ops for p in s.paths]
+        # the flat lists, under the reference's attribute names
+        self.operand_extent = tables.operand_extent
+        self.buffer_dim = list(tables.buffer_dim)
+        self.buffer_num_segments = list(tables.buffer_num_segments)
+        self.dtypes = list(tables.dtypes)
+        self.num_operations = len(tables.num_operands)
+        self.num_operands = list(tables.num_operands)
+        self.operations = list(tables.operations)
+        self.num_paths = list(tables.num_paths)
+        self.path_indices_start = list(tables.path_indices_start)
+        self.path_coefficients_start = list(tables.path_coefficients_start)
+        self.path_indices = list(tables.path_indices)
+        self.path_coefficients = list(tables.path_coefficients)
 
         self.BATCH_DIM_AUTO = u1d.BATCH_DIM_AUTO
         self.BATCH_DIM_SHARED = u1d.BATCH_DIM_SHARED
@@ -125,12 +117,7 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
     def _plan(self, math_dtype: torch.dtype) -> u1d.Uniform1dPlan:
         plan = self._plans.get(math_dtype)
         if plan is None:
-            plan = u1d.Uniform1dPlan(
-                math_dtype, self.operand_extent, self.num_inputs, self.num_outputs, self.buffer_dim,
-                self.buffer_num_segments, self.dtypes, self.num_operands, self.operations, self.num_paths,
-                self.path_indices_start, self.path_coefficients_start, self.path_indices, self.path_coefficients,
-                name=self.name,
-            )
+            plan = u1d.Uniform1dPlan(self.tables, math_dtype, name=self.name)
             self._plans[math_dtype] = plan
         return plan
 

@@ -26,6 +26,7 @@ import torch
 
 from .. import _lib
 from .._lib import BATCH_DIM_AUTO, BATCH_DIM_BATCHED, BATCH_DIM_INDEXED, BATCH_DIM_SHARED
+from ..tables import U1dTables
 
 __all__ = [
     "uniform_1d",
@@ -47,63 +48,33 @@ _DTYPE_CODE = {
 class Uniform1dPlan:
     """Flat descriptor tables + lazily created device plans (one per GPU) + derived backward plans."""
 
-    def __init__(
-        self,
-        math_dtype: torch.dtype,
-        operand_extent: int,
-        num_inputs: int,
-        num_outputs: int,
-        buffer_dim: Sequence[int],
-        buffer_num_segments: Sequence[int],
-        dtypes: Sequence[int],
-        num_operands: Sequence[int],
-        operations: Sequence[int],
-        num_paths: Sequence[int],
-        path_indices_start: Sequence[int],
-        path_coefficients_start: Sequence[int],
-        path_indices: Sequence[int],
-        path_coefficients: Sequence[float],
-        name: str = "segmented_polynomial",
-    ):
+    def __init__(self, tables: U1dTables, math_dtype: torch.dtype, name: str = "segmented_polynomial"):
         if math_dtype not in (torch.float32, torch.float64):
             raise ValueError(f"uniform_1d: math_dtype must be float32 or float64, got {math_dtype}")
+        self.tables = tables
         self.name = name
         self.math_dtype = math_dtype
-        self.operand_extent = int(operand_extent)
-        self.num_inputs = int(num_inputs)
-        self.num_outputs = int(num_outputs)
-        self.buffer_dim = tuple(int(x) for x in buffer_dim)
-        self.buffer_num_segments = tuple(int(x) for x in buffer_num_segments)
-        self.dtypes = tuple(int(x) for x in dtypes)
-        self.num_operands = tuple(int(x) for x in num_operands)
-        self.operations = tuple(int(x) for x in operations)
-        self.num_paths = tuple(int(x) for x in num_paths)
-        self.path_indices_start = tuple(int(x) for x in path_indices_start)
-        self.path_coefficients_start = tuple(int(x) for x in path_coefficients_start)
-        self.path_indices = tuple(int(x) for x in path_indices)
-        self.path_coefficients = tuple(float(x) for x in path_coefficients)
-        nbuf = self.num_inputs + self.num_outputs
-        if len(self.buffer_dim) != nbuf or len(self.buffer_num_segments) != nbuf or len(self.dtypes) != nbuf:
-            raise ValueError("uniform_1d: per-buffer lists must have num_inputs + num_outputs entries")
-        if not (len(self.num_operands) == len(self.num_paths) == len(self.path_indices_start)
-                == len(self.path_coefficients_start)):
-            raise ValueError("uniform_1d: per-operation lists have inconsistent lengths")
-        if sum(self.num_operands) != len(self.operations):
-            raise ValueError("uniform_1d: `operations` does not match `num_operands`")
         self._handles: dict[int, int] = {}
         self._backward: dict[tuple, "Uniform1dPlan"] = {}
         self._lock = threading.Lock()
 
+    def __getattr__(self, item):
+        # table fields (operand_extent, num_inputs, buffer_dim, ...) read through
+        if item == "tables":
+            raise AttributeError(item)
+        return getattr(self.tables, item)
+
     # ------------------------------------------------------------------ geometry
     def width(self, b: int) -> int:
-        return self.buffer_num_segments[b] * (self.operand_extent if self.buffer_dim[b] else 1)
+        return self.tables.width(b)
 
     def key(self) -> tuple:
-        return (
-            self.math_dtype, self.operand_extent, self.num_inputs, self.num_outputs, self.buffer_dim,
-            self.buffer_num_segments, self.dtypes, self.num_operands, self.operations, self.num_paths,
-            self.path_indices_start, self.path_coefficients_start, self.path_indices, self.path_coefficients,
-        )
+        return (self.math_dtype, self.tables)
+
+    def specialised(self, device: torch.device) -> bool:
+        """True when kernels generated for exactly these tables are linked into the library."""
+        h = self.handle(device)
+        return bool(_lib.load().cueq_u1d_plan_info(h, None))
 
     # ------------------------------------------------------------------ device plan
     def handle(self, device: torch.device) -> int:
@@ -161,52 +132,12 @@ class Uniform1dPlan:
 
     # ------------------------------------------------------------------ transposition
     def backward_plan(self, needs_grad: tuple) -> "Uniform1dPlan":
-        """Plan computing the gradients of the inputs flagged in ``needs_grad``.
-
-        Buffers of the new plan: the original inputs, one cotangent per original output, then
-        one gradient per flagged input.  For every operation and every operand slot bound to a
-        flagged input, an operation with the same path table is emitted in which that slot
-        becomes the output and the original output slot reads the cotangent.
-        """
+        """Plan computing the gradients of the flagged inputs (see ``U1dTables.backward``)."""
         needs_grad = tuple(bool(x) for x in needs_grad)
         plan = self._backward.get(needs_grad)
-        if plan is not None:
-            return plan
-        nin, nout = self.num_inputs, self.num_outputs
-        grad_buf, k = {}, nin + nout
-        for i, g in enumerate(needs_grad):
-            if g:
-                grad_buf[i] = k
-                k += 1
-        buf_dim = list(self.buffer_dim) + [self.buffer_dim[i] for i in grad_buf]
-        buf_nseg = list(self.buffer_num_segments) + [self.buffer_num_segments[i] for i in grad_buf]
-        # inputs inherit their own dtype; cotangents are inputs too; a gradient takes its primal's dtype
-        dtypes = list(range(nin + nout)) + [i for i in grad_buf]
-        num_operands, operations, num_paths, pis, pcs = [], [], [], [], []
-        off = 0
-        for o, nop in enumerate(self.num_operands):
-            bufs = self.operations[off: off + nop]
-            off += nop
-            out_pos = [s for s, b in enumerate(bufs) if b >= nin]
-            assert len(out_pos) == 1
-            out_pos = out_pos[0]
-            for s, b in enumerate(bufs):
-                if s == out_pos or not needs_grad[b]:
-                    continue
-                nb = list(bufs)
-                nb[s] = grad_buf[b]
-                # nb[out_pos] keeps its id: cotangent of output j sits at position nin + j
-                num_operands.append(nop)
-                operations += nb
-                num_paths.append(self.num_paths[o])
-                pis.append(self.path_indices_start[o])
-                pcs.append(self.path_coefficients_start[o])
-        plan = Uniform1dPlan(
-            self.math_dtype, self.operand_extent, nin + nout, len(grad_buf), buf_dim, buf_nseg, dtypes,
-            num_operands, operations, num_paths, pis, pcs, self.path_indices, self.path_coefficients,
-            name=self.name + "_bwd",
-        )
-        self._backward[needs_grad] = plan
+        if plan is None:
+            plan = Uniform1dPlan(self.tables.backward(needs_grad), self.math_dtype, name=self.name + "_bwd")
+            self._backward[needs_grad] = plan
         return plan
 
 
@@ -451,9 +382,12 @@ def uniform_1d(
         raise ValueError("uniform_1d: num_operations does not match num_operands")
     plan = _cached_plan(
         Uniform1dPlan(
-            math_dtype, operand_extent, num_inputs, num_outputs, buffer_dim, buffer_num_segments, dtypes,
-            num_operands, operations, num_paths, path_indices_start, path_coefficients_start, path_indices,
-            path_coefficients, name=name,
+            U1dTables.make(
+                operand_extent, num_inputs, num_outputs, buffer_dim, buffer_num_segments, dtypes, num_operands,
+                operations, num_paths, path_indices_start, path_coefficients_start, path_indices, path_coefficients,
+            ),
+            math_dtype,
+            name=name,
         )
     )
     return run_plan(plan, batch_dim, index_buffer, batch_size, num_index, tensors)

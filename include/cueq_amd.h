@@ -89,6 +89,12 @@ typedef struct {
 int cueq_u1d_plan_create(const cueq_u1d_desc* desc, cueq_u1d_plan** plan);
 void cueq_u1d_plan_destroy(cueq_u1d_plan* plan);
 
+/* Introspection: returns 1 when kernels specialised for this descriptor were compiled into the
+ * library (0: the table-driven kernels will run); *hash receives the descriptor's content hash.
+ * No counterpart in the reference, whose op compiles its kernel at run time
+ * (CHANGELOG.md:38 "NVRTC"); here specialisation happens when the library is built. */
+int cueq_u1d_plan_info(const cueq_u1d_plan* plan, uint64_t* hash);
+
 /* Bytes of device workspace cueq_u1d_run needs for this call shape (0 if none). */
 int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size);
 
