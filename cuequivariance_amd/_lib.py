@@ -23,6 +23,7 @@ EXPORTED_SYMBOLS = (
     "cueq_u1d_plan_create",
     "cueq_u1d_plan_destroy",
     "cueq_u1d_plan_info",
+    "cueq_u1d_desc_info",
     "cueq_u1d_workspace_size",
     "cueq_u1d_run",
     "cueq_segment_csr_workspace",
@@ -94,6 +95,8 @@ def load() -> C.CDLL:
         lib.cueq_u1d_plan_destroy.restype = None
         lib.cueq_u1d_plan_info.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
         lib.cueq_u1d_plan_info.restype = C.c_int
+        lib.cueq_u1d_desc_info.argtypes = [C.POINTER(U1dDesc), C.POINTER(C.c_uint64)]
+        lib.cueq_u1d_desc_info.restype = C.c_int
         lib.cueq_u1d_workspace_size.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64]
         lib.cueq_u1d_workspace_size.restype = C.c_int64
         lib.cueq_u1d_run.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]
@@ -124,3 +127,37 @@ def int64_array(values):
 
 def double_array(values):
     return (C.c_double * max(1, len(values)))(*values)
+
+
+def make_desc(tables, math_code: int):
+    """(U1dDesc, keep-alive arrays) for a ``U1dTables``."""
+    keep = dict(
+        buffer_dim=int32_array(tables.buffer_dim),
+        nseg=int32_array(tables.buffer_num_segments),
+        num_operands=int32_array(tables.num_operands),
+        operations=int32_array(tables.operations),
+        num_paths=int32_array(tables.num_paths),
+        pis=int64_array(tables.path_indices_start),
+        pcs=int64_array(tables.path_coefficients_start),
+        pi=int32_array(tables.path_indices),
+        pc=double_array(tables.path_coefficients),
+    )
+    desc = U1dDesc(
+        math_dtype=math_code,
+        operand_extent=tables.operand_extent,
+        num_inputs=tables.num_inputs,
+        num_outputs=tables.num_outputs,
+        buffer_dim=keep["buffer_dim"],
+        buffer_num_segments=keep["nseg"],
+        num_operations=len(tables.num_operands),
+        num_operands=keep["num_operands"],
+        operations=keep["operations"],
+        num_paths=keep["num_paths"],
+        path_indices_start=keep["pis"],
+        path_coefficients_start=keep["pcs"],
+        path_indices=keep["pi"],
+        path_indices_len=len(tables.path_indices),
+        path_coefficients=keep["pc"],
+        path_coefficients_len=len(tables.path_coefficients),
+    )
+    return desc, keep

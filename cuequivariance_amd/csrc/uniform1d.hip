@@ -342,6 +342,14 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
   return CUEQ_OK;
 }
 
+// Host-only: content hash of the descriptor tables and whether specialised kernels are linked in.
+extern "C" int cueq_u1d_desc_info(const cueq_u1d_desc* d, uint64_t* hash) {
+  if (!d) return 0;
+  const uint64_t h = hash_u1d_desc(d);
+  if (hash) *hash = h;
+  return find_u1d_spec(h) ? 1 : 0;
+}
+
 // 1 when descriptor-specialised kernels exist for this plan, else 0; *hash receives the table hash.
 extern "C" int cueq_u1d_plan_info(const cueq_u1d_plan* plan, uint64_t* hash) {
   if (!plan) return 0;

@@ -181,6 +181,11 @@ class Irrep:
     def is_trivial(self) -> bool:
         return self.is_scalar()
 
+    @property
+    def X(self):
+        """Generators of the Lie algebra in this representation, shape ``(3, dim, dim)``."""
+        return self.continuous_generators()
+
     def __le__(self, other) -> bool:
         return self == other or self < other
 

@@ -198,6 +198,17 @@ class Path:
         return Path([self.indices[i] for i in perm], self.coefficients)
 
 
+def _format_dims(dims: dict) -> str:
+    def fmt(dd):
+        if len(dd) == 0:
+            return ""
+        if len(dd) == 1:
+            return str(next(iter(dd)))
+        return "{" + ", ".join(str(i) for i in sorted(dd)) + "}"
+
+    return " ".join(f"{m}={fmt(dd)}" for m, dd in sorted(dims.items()))
+
+
 def _canon(i: int, n: int, what: str) -> int:
     if not -n <= i < n:
         raise ValueError(f"{what} {i} out of range [-{n}, {n})")
@@ -222,6 +233,11 @@ class SegmentedTensorProduct:
     def from_subscripts(cls, subscripts) -> "SegmentedTensorProduct":
         s = Subscripts(subscripts)
         return cls([(None, ss) for ss in s.operands], s.coefficients)
+
+    @classmethod
+    def empty_segments(cls, num_segments: Sequence[int]) -> "SegmentedTensorProduct":
+        """Descriptor whose operands are ``num_segments[k]`` scalar segments each, no paths yet."""
+        return cls([(SegmentedOperand.empty_segments(n), "") for n in num_segments], "")
 
     @classmethod
     def from_dict(cls, data: dict) -> "SegmentedTensorProduct":
@@ -325,13 +341,41 @@ class SegmentedTensorProduct:
     def __repr__(self):
         sizes = ",".join(str(o.size) for o in self.operands)
         nseg = ",".join(str(len(o)) for o in self.operands)
-        dims = " ".join(
-            f"{m}={next(iter(d))}" if len(d) == 1 else f"{m}={{{', '.join(map(str, sorted(d)))}}}"
-            for m, d in sorted(self.get_dimensions_dict().items())
-        )
+        dims = _format_dims(self.get_dimensions_dict())
         return f"{self.subscripts} sizes={sizes} num_segments={nseg} num_paths={self.num_paths}" + (
             f" {dims}" if dims else ""
         )
+
+    def to_text(self, coefficient_formatter=lambda x: f"{x}") -> str:
+        """Multi-line dump: header, per-operand mode extents, memory cost, path indices and coefficients.
+
+        Same layout as the reference's ``to_text`` except that the ``Flop cost`` line is omitted.
+        """
+        out = f"{self}"
+        dims = self.get_dimensions_dict()
+        for oid, (ope, ss) in enumerate(self.operands_and_subscripts):
+            out += f"\noperand #{oid} subscripts={ss}"
+            for i, ch in enumerate(ss):
+                if len(dims[ch]) == 1:
+                    out += f"\n  | {ch}: [{ope.segments[0][i]}] * {len(ope.segments)}"
+                else:
+                    out += f"\n  | {ch}: [" + ", ".join(str(s[i]) for s in ope.segments) + "]"
+        out += f"\nMemory cost: {sum(o.size for o in self.operands)}"
+        if self.paths:
+            out += "\nPath indices: " + ", ".join(" ".join(str(i) for i in row) for row in self.indices)
+            if all(len(dims[ch]) == 1 for ch in self.coefficient_subscripts):
+                out += "\nPath coefficients: " + np.array2string(
+                    self.stacked_coefficients, max_line_width=np.inf, formatter={"float": coefficient_formatter},
+                    threshold=np.inf,
+                )
+            else:
+                out += "\nPath coefficients:\n" + "\n".join(
+                    np.array2string(p.coefficients, formatter={"float": coefficient_formatter}, threshold=np.inf)
+                    for p in self.paths
+                )
+        else:
+            out += "\nNo paths."
+        return out
 
     def get_dimensions_dict(self) -> dict[str, set[int]]:
         dims = {m: set() for m in self.subscripts.modes()}
@@ -363,6 +407,13 @@ class SegmentedTensorProduct:
     def all_same_segment_shape(self) -> bool:
         return all(o.all_same_segment_shape() for o in self.operands)
 
+    def all_segments_are_used(self) -> bool:
+        return all(
+            any(s == p.indices[o] for p in self.paths)
+            for o, ope in enumerate(self.operands)
+            for s in range(ope.num_segments)
+        )
+
     def assert_valid(self):
         for m in self.subscripts.modes():
             if self.subscripts.count(m) == 1:
@@ -381,6 +432,8 @@ class SegmentedTensorProduct:
         if isinstance(segment, dict):
             segment = tuple(segment[m] for m in self._ops[operand][1])
         ope = self._ops[operand][0]
+        if len(segment) != ope.ndim:
+            raise ValueError(f"segment has {len(segment)} dimensions, expected {ope.ndim}.")
         self._ops[operand][0] = ope.with_segments(ope.segments + (tuple(segment),))
         return ope.num_segments
 

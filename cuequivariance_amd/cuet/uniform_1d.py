@@ -87,35 +87,7 @@ class Uniform1dPlan:
             if h is not None:
                 return h
             lib = _lib.load()
-            keep = dict(
-                buffer_dim=_lib.int32_array(self.buffer_dim),
-                nseg=_lib.int32_array(self.buffer_num_segments),
-                num_operands=_lib.int32_array(self.num_operands),
-                operations=_lib.int32_array(self.operations),
-                num_paths=_lib.int32_array(self.num_paths),
-                pis=_lib.int64_array(self.path_indices_start),
-                pcs=_lib.int64_array(self.path_coefficients_start),
-                pi=_lib.int32_array(self.path_indices),
-                pc=_lib.double_array(self.path_coefficients),
-            )
-            desc = _lib.U1dDesc(
-                math_dtype=_DTYPE_CODE[self.math_dtype],
-                operand_extent=self.operand_extent,
-                num_inputs=self.num_inputs,
-                num_outputs=self.num_outputs,
-                buffer_dim=keep["buffer_dim"],
-                buffer_num_segments=keep["nseg"],
-                num_operations=len(self.num_operands),
-                num_operands=keep["num_operands"],
-                operations=keep["operations"],
-                num_paths=keep["num_paths"],
-                path_indices_start=keep["pis"],
-                path_coefficients_start=keep["pcs"],
-                path_indices=keep["pi"],
-                path_indices_len=len(self.path_indices),
-                path_coefficients=keep["pc"],
-                path_coefficients_len=len(self.path_coefficients),
-            )
+            desc, keep = _lib.make_desc(self.tables, _DTYPE_CODE[self.math_dtype])
             out = C.c_void_p()
             with torch.cuda.device(idx):
                 _lib.check(lib.cueq_u1d_plan_create(C.byref(desc), C.byref(out)), "cueq_u1d_plan_create")

@@ -94,6 +94,8 @@ void cueq_u1d_plan_destroy(cueq_u1d_plan* plan);
  * No counterpart in the reference, whose op compiles its kernel at run time
  * (CHANGELOG.md:38 "NVRTC"); here specialisation happens when the library is built. */
 int cueq_u1d_plan_info(const cueq_u1d_plan* plan, uint64_t* hash);
+/* Same answer from the tables alone; touches no device (usable on a host without a GPU). */
+int cueq_u1d_desc_info(const cueq_u1d_desc* desc, uint64_t* hash);
 
 /* Bytes of device workspace cueq_u1d_run needs for this call shape (0 if none). */
 int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size);
