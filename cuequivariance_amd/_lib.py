@@ -20,6 +20,8 @@ BATCH_DIM_AUTO, BATCH_DIM_SHARED, BATCH_DIM_BATCHED, BATCH_DIM_INDEXED = -1, 0, 
 EXPORTED_SYMBOLS = (
     "cueq_last_error",
     "cueq_version",
+    "cueq_timing_begin",
+    "cueq_timing_end",
     "cueq_u1d_plan_create",
     "cueq_u1d_plan_destroy",
     "cueq_u1d_plan_info",
@@ -65,6 +67,10 @@ class U1dBuffer(C.Structure):
     ]
 
 
+class TimingEntry(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("launches", C.c_int64), ("total_ms", C.c_double)]
+
+
 class CueqError(RuntimeError):
     pass
 
@@ -89,6 +95,9 @@ def load() -> C.CDLL:
         lib = C.CDLL(str(LIB_PATH))
         lib.cueq_last_error.restype = C.c_char_p
         lib.cueq_version.restype = C.c_char_p
+        lib.cueq_timing_begin.restype = C.c_int
+        lib.cueq_timing_end.argtypes = [C.POINTER(TimingEntry), C.c_int]
+        lib.cueq_timing_end.restype = C.c_int
         lib.cueq_u1d_plan_create.argtypes = [C.POINTER(U1dDesc), C.POINTER(C.c_void_p)]
         lib.cueq_u1d_plan_create.restype = C.c_int
         lib.cueq_u1d_plan_destroy.argtypes = [C.c_void_p]
@@ -161,3 +170,14 @@ def make_desc(tables, math_code: int):
         path_coefficients_len=len(tables.path_coefficients),
     )
     return desc, keep
+
+
+def timing_begin() -> None:
+    check(load().cueq_timing_begin(), "cueq_timing_begin")
+
+
+def timing_end() -> dict:
+    """{kernel name: (launches, total milliseconds)} of the kernels launched since ``timing_begin``."""
+    buf = (TimingEntry * 64)()
+    n = load().cueq_timing_end(buf, 64)
+    return {buf[i].name.decode(): (int(buf[i].launches), float(buf[i].total_ms)) for i in range(n)}

@@ -434,6 +434,7 @@ static int run_fwd(const SpecCall& c) {{
   const int64_t* offs = out_idx ? b[3].csr_offsets : nullptr;
   const int64_t* perm = out_idx ? b[3].csr_perm : nullptr;
   const dim3 g(static_cast<unsigned>(grid)), t(64);
+  KernelTimer timer("{name}_fwd_{T}", c.stream);
 #define LAUNCH_FWD(XI, WS) hipLaunchKernelGGL((fwd_kernel<XI, WS>), g, t, 0, c.stream, w, x1, x2, o, b[1].index, b[1].index_is_64, offs, perm)
   if (x1_idx && w_shared) LAUNCH_FWD(true, true);
   else if (x1_idx) LAUNCH_FWD(true, false);
@@ -493,6 +494,8 @@ static int run_bwd(const SpecCall& c) {{
     const int64_t grid = nchunks * {nch};
     CUEQ_REQUIRE(grid < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "batch too large for one launch");
     const dim3 gd(static_cast<unsigned>(grid)), t(64);
+    {{
+    KernelTimer timer("{name}_bwd_{T}", c.stream);
 #define LAUNCH_BWD(XI, GI, AT) hipLaunchKernelGGL((bwd_kernel<XI, GI, AT>), gd, t, 0, c.stream, w, x1, x2, g, dw, dx1, dx1_partial, dx2, dx2_partial, b[1].index, b[1].index_is_64, b[3].index, b[3].index_is_64, batch)
     if (x1_idx && g_idx && atomic) LAUNCH_BWD(true, true, true);
     else if (x1_idx && g_idx) LAUNCH_BWD(true, true, false);
@@ -501,6 +504,7 @@ static int run_bwd(const SpecCall& c) {{
     else if (g_idx) LAUNCH_BWD(false, true, false);
     else LAUNCH_BWD(false, false, false);
 #undef LAUNCH_BWD
+    }}
     CUEQ_CHECK_HIP(hipGetLastError());
     if ({nch} > 1) {{
       hipLaunchKernelGGL(fold_parts<{T}>, dim3(blocks_for(batch * {W2}ll)), dim3(256), 0, c.stream, dx2_partial, batch, {nch}, {W2}, dx2);

@@ -45,6 +45,22 @@ struct Fnv64 {
 
 uint64_t hash_u1d_desc(const cueq_u1d_desc* d);
 
+// Optional per-kernel timing with HIP events (cueq_timing_begin / cueq_timing_end).
+bool timing_enabled();
+void timing_mark(const char* name, hipStream_t stream, bool begin);
+
+struct KernelTimer {
+  const char* name;
+  hipStream_t stream;
+  bool on;
+  KernelTimer(const char* n, hipStream_t s) : name(n), stream(s), on(timing_enabled()) {
+    if (on) timing_mark(name, stream, true);
+  }
+  ~KernelTimer() {
+    if (on) timing_mark(name, stream, false);
+  }
+};
+
 struct SpecRegistrar {
   explicit SpecRegistrar(const U1dSpec* s) { register_u1d_spec(s); }
 };

@@ -67,6 +67,31 @@ uint64_t hash_u1d_desc(const cueq_u1d_desc* d) {
   return f.h;
 }
 
+// ---- event timing -----------------------------------------------------------------------
+struct TimingRecord { const char* name; hipEvent_t start, stop; };
+static std::mutex g_timing_mutex;
+static bool g_timing_on = false;
+static std::vector<TimingRecord> g_timing;
+static thread_local hipEvent_t g_pending_start = nullptr;
+
+bool timing_enabled() { return g_timing_on; }
+
+void timing_mark(const char* name, hipStream_t stream, bool begin) {
+  if (begin) {
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    (void)hipEventRecord(e, stream);
+    g_pending_start = e;
+  } else if (g_pending_start) {
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    (void)hipEventRecord(e, stream);
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    g_timing.push_back({name, g_pending_start, e});
+    g_pending_start = nullptr;
+  }
+}
+
 void set_error(const char* fmt, ...) {
   char buf[1024];
   va_list ap;
@@ -217,6 +242,36 @@ struct cueq_u1d_plan {
 };
 
 extern "C" const char* cueq_last_error(void) { return g_error.c_str(); }
+
+extern "C" int cueq_timing_begin(void) {
+  std::lock_guard<std::mutex> lock(g_timing_mutex);
+  for (auto& r : g_timing) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }
+  g_timing.clear();
+  g_timing_on = true;
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_timing_end(cueq_timing_entry* out, int max_entries) {
+  std::lock_guard<std::mutex> lock(g_timing_mutex);
+  g_timing_on = false;
+  int n = 0;
+  for (auto& r : g_timing) {
+    float ms = 0.f;
+    if (hipEventSynchronize(r.stop) == hipSuccess && hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+      int k = 0;
+      for (; k < n; ++k) if (std::strcmp(out[k].name, r.name) == 0) break;
+      if (k == n) {
+        if (n >= max_entries) { k = -1; }
+        else { std::snprintf(out[n].name, sizeof(out[n].name), "%s", r.name); out[n].launches = 0; out[n].total_ms = 0; ++n; }
+      }
+      if (k >= 0) { out[k].launches += 1; out[k].total_ms += ms; }
+    }
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_timing.clear();
+  return n;
+}
 extern "C" const char* cueq_version(void) { return "cueq_amd 0.1 (gfx950)"; }
 
 extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_plan) {

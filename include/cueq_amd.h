@@ -39,6 +39,20 @@ enum cueq_status {
 const char* cueq_last_error(void);
 const char* cueq_version(void);
 
+/* Per-kernel timing with HIP events recorded on the stream each kernel is launched on.
+ * Between cueq_timing_begin() and cueq_timing_end() the main kernel of every call is bracketed by a
+ * pair of events; cueq_timing_end waits for them and returns, per kernel name, the number of launches
+ * and their summed duration.  Same purpose as the reference's event-based helper
+ * cuequivariance_torch/cuequivariance_torch/benchmarking.py:24-158; unlike it, the events sit directly
+ * around the kernel inside the library, so host-side launch work is excluded. */
+typedef struct {
+  char name[64];
+  int64_t launches;
+  double total_ms;
+} cueq_timing_entry;
+int cueq_timing_begin(void);
+int cueq_timing_end(cueq_timing_entry* entries, int max_entries); /* returns the number of entries filled */
+
 /* ------------------------------------------------------------------------- */
 /* uniform-1d executor                                                        */
 /* ------------------------------------------------------------------------- */
