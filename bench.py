@@ -94,6 +94,8 @@ def main() -> int:
     ap.add_argument("--edges", type=int, default=100_000)
     ap.add_argument("--cpu-sample-edges", type=int, default=4000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--deterministic", action="store_true",
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
     args = ap.parse_args()
@@ -112,6 +114,15 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
     dev = torch.device("cuda:0")
+    if args.calibration_copy:
+        n = 1 << 28  # 2^28 floats = 1 GiB read and 1 GiB written per copy
+        a = torch.ones(n, dtype=torch.float32, device=dev)
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "copy", "bytes_read": n * 4, "bytes_written": n * 4, "launches": 5}))
+        return 0
     dtype = torch.float32 if args.dtype == "fp32" else torch.float64
     N, E = args.nodes, args.edges
 

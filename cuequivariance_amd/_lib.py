@@ -10,7 +10,10 @@ import ctypes as C
 import threading
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libcueq_amd.so"
+import os
+
+# The in-tree build; CUEQ_AMD_LIBRARY may point at another build of the same ABI.
+LIB_PATH = Path(os.environ.get("CUEQ_AMD_LIBRARY") or (Path(__file__).resolve().parent / "libcueq_amd.so"))
 
 # enum cueq_dtype
 F32, F64, F16, BF16 = 0, 1, 2, 3

@@ -162,7 +162,7 @@ def _tables_for(blocks: Sequence[Block]):
     return slots, tables
 
 
-def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: int, ns: str) -> str:
+def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: int, ns: str, prefetch: bool = True) -> str:
     """HIP source of the forward kernels (one ``__device__`` body per block group) in namespace ``ns``."""
     fp = T
     dpp = "v_fmac_f32_dpp" if T == "float" else "v_fmac_f64_dpp"
@@ -188,6 +188,41 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
         ks = sorted({k for blk in blocks for k in blk.k_list})
         i_used = sorted({i for blk in blocks for i in blk.i_list})
         ms = sorted({m for m, _ in tables})
+
+        def load(S: str, zz: str, ind: str):
+            A(f"{ind}{{")
+            A(f"{ind}  const int64_t z = csr_perm ? csr_perm[{zz}] : ({zz});")
+            A(f"{ind}  int64_t srow = z;")
+            A(f"{ind}  if (X1_IDX) srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
+            A(f"{ind}  const {fp}* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
+            A(f"{ind}  const {fp}* __restrict__ wp = w + (W_SHARED ? 0 : z * {st.nseg_w * st.extent}ll);")
+            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
+            for m in ms:
+                nvalid = min(16, st.nseg_x2 - 16 * m)
+                A(f"{ind}  {S}_yv{m} = x2p[{16 * m} + (n16 < {nvalid} ? n16 : 0)];")
+            for i in i_used:
+                A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
+            for blk in blocks:
+                A(f"{ind}  {S}_wv{blk.b} = wp[{blk.b * st.extent} + uu];")
+            A(f"{ind}}}")
+
+        def body(S: str, ind: str):
+            for t, (m, _row) in enumerate(tables):
+                A(f"{ind}{fp} t{t} = s_c[{(tbase + t) * 16} + n16] * {S}_yv{m};")
+            # fence: table registers are produced by VALU and consumed through DPP
+            names = [f"t{t}" for t in range(ntab)]
+            for c0 in range(0, len(names), 12):
+                ops = ", ".join(f'"+v"({n})' for n in names[c0: c0 + 12])
+                A(f'{ind}asm volatile("s_nop 1" : {ops});')
+            for blk in blocks:
+                A(f"{ind}{{  // block w[{blk.b}]: x1 {blk.i_list} x x2 {blk.j_list} -> out {blk.k_list}")
+                for i in blk.i_list:
+                    A(f"{ind}  const {fp} wx{i} = {S}_wv{blk.b} * {S}_xv{i};")
+                for e_idx, (i, j, k, c) in enumerate(blk.entries):
+                    t, n = slots[(blk.b, e_idx)]
+                    A(f'{ind}  asm("{dpp} %0, %1, %2 row_newbcast:{n} row_mask:0xf bank_mask:0xf" : "+v"(acc{k}) : "v"(t{t}), "v"(wx{i}));')
+                A(f"{ind}}}")
+
         A(f"template <bool X1_IDX, bool W_SHARED>")
         A(f"__device__ __forceinline__ void fwd_group{q}(FWD_PARAMS, const {fp}* s_c, int64_t r, int lane, int uu, bool active) {{")
         for k in ks:
@@ -195,37 +230,36 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
         A("  int64_t z0, z1;")
         A("  if (csr_offsets) { z0 = csr_offsets[r]; z1 = csr_offsets[r + 1]; } else { z0 = r; z1 = r + 1; }")
         A("  const int n16 = lane & 15;")
-        A("  for (int64_t zz = z0; zz < z1; ++zz) {")
-        A("    const int64_t z = csr_perm ? csr_perm[zz] : zz;")
-        A("    int64_t srow = z;")
-        A("    if (X1_IDX) srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
-        A(f"    const {fp}* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
-        A(f"    const {fp}* __restrict__ wp = w + (W_SHARED ? 0 : z * {st.nseg_w * st.extent}ll);")
-        A(f"    const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
-        for m in ms:
-            nvalid = min(16, st.nseg_x2 - 16 * m)
-            A(f"    const {fp} yv{m} = x2p[{16 * m} + (n16 < {nvalid} ? n16 : 0)];")
-        for i in i_used:
-            A(f"    const {fp} xv{i} = x1p[{i * st.extent} + uu];")
-        for blk in blocks:
-            A(f"    const {fp} wv{blk.b} = wp[{blk.b * st.extent} + uu];")
-        # tables
-        for t, (m, _row) in enumerate(tables):
-            A(f"    {fp} t{t} = s_c[{(tbase + t) * 16} + n16] * yv{m};")
-        # fence: table registers are produced by VALU and consumed through DPP
-        names = [f"t{t}" for t in range(ntab)]
-        for c0 in range(0, len(names), 12):
-            ops = ", ".join(f'"+v"({n})' for n in names[c0: c0 + 12])
-            A(f'    asm volatile("s_nop 1" : {ops});')
-        for blk in blocks:
-            A(f"    {{  // block w[{blk.b}]: x1 {blk.i_list} x x2 {blk.j_list} -> out {blk.k_list}")
-            for i in blk.i_list:
-                A(f"      const {fp} wx{i} = wv{blk.b} * xv{i};")
-            for e_idx, (i, j, k, c) in enumerate(blk.entries):
-                t, n = slots[(blk.b, e_idx)]
-                A(f'      asm("{dpp} %0, %1, %2 row_newbcast:{n} row_mask:0xf bank_mask:0xf" : "+v"(acc{k}) : "v"(t{t}), "v"(wx{i}));')
+        sets = ("a", "b") if prefetch else ("a",)
+        for S in sets:
+            A(f"  {fp} " + ", ".join([f"{S}_yv{m} = 0" for m in ms] + [f"{S}_xv{i} = 0" for i in i_used]
+                                      + [f"{S}_wv{blk.b} = 0" for blk in blocks]) + ";")
+        if prefetch:
+            A("  if (z0 < z1) {")
+            load("a", "z0", "    ")
+            A("  }")
+            A("  for (int64_t zz = z0; zz < z1; zz += 2) {")
+            A("    if (zz + 1 < z1) {")
+            load("b", "zz + 1", "      ")
             A("    }")
-        A("  }")
+            A("    __builtin_amdgcn_sched_barrier(0);")
+            A("    {")
+            body("a", "      ")
+            A("    }")
+            A("    if (zz + 1 >= z1) break;")
+            A("    if (zz + 2 < z1) {")
+            load("a", "zz + 2", "      ")
+            A("    }")
+            A("    __builtin_amdgcn_sched_barrier(0);")
+            A("    {")
+            body("b", "      ")
+            A("    }")
+            A("  }")
+        else:
+            A("  for (int64_t zz = z0; zz < z1; ++zz) {")
+            load("a", "zz", "    ")
+            body("a", "    ")
+            A("  }")
         A("  if (active) {")
         A(f"    {fp}* __restrict__ op = out + r * {st.nseg_out * st.extent}ll;")
         for k in ks:
@@ -384,7 +418,7 @@ BWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}*
 
 
 def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_hash: int, *, fwd_split: int = 1,
-              fwd_waves: int = 2, bwd_waves: int = 2, bwd_chunk: int = 16) -> str:
+              fwd_waves: int = 2, fwd_prefetch: bool = True, bwd_waves: int = 2, bwd_chunk: int = 16) -> str:
     """Complete .hip translation unit: kernels, host launchers, registration under both table hashes."""
     ns = f"cw_{name}"
     nch = (st.extent + 63) // 64
@@ -402,7 +436,7 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     A(f"#define FWD_ARGS {FWD_ARGS}")
     A(f"#define BWD_PARAMS {BWD_PARAMS.format(T=T)}")
     A("")
-    A(emit_forward(st, T, fwd_split, fwd_waves, ns))
+    A(emit_forward(st, T, fwd_split, fwd_waves, ns, fwd_prefetch))
     A("")
     A(emit_backward(st, T, bwd_waves, bwd_chunk))
     A("")
