@@ -33,6 +33,10 @@ EXPORTED_SYMBOLS = (
     "cueq_u1d_run",
     "cueq_segment_csr_workspace",
     "cueq_segment_csr_build",
+    "cueq_seg_gemm",
+    "cueq_seg_outer_workspace",
+    "cueq_seg_outer",
+    "cueq_seg_rowdot",
 )
 
 
@@ -68,6 +72,18 @@ class U1dBuffer(C.Structure):
         ("csr_offsets", C.c_void_p),
         ("csr_perm", C.c_void_p),
     ]
+
+
+class GemmProblem(C.Structure):
+    _fields_ = [
+        ("a_off", C.c_int64), ("c_off", C.c_int64), ("b_off", C.c_int64), ("alpha", C.c_double),
+        ("s_col", C.c_int32), ("trans_b", C.c_int32), ("accumulate", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
+class OuterEntry(C.Structure):
+    _fields_ = [("a_off", C.c_int64), ("c_off", C.c_int64), ("alpha", C.c_double), ("s_col", C.c_int32),
+                ("reserved", C.c_int32)]
 
 
 class TimingEntry(C.Structure):
@@ -119,6 +135,24 @@ def load() -> C.CDLL:
             C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
         ]
         lib.cueq_segment_csr_build.restype = C.c_int
+        lib.cueq_seg_gemm.argtypes = [
+            C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
+            C.c_int64, C.c_int64, C.POINTER(GemmProblem), C.c_int32, C.c_void_p,
+        ]
+        lib.cueq_seg_gemm.restype = C.c_int
+        lib.cueq_seg_outer_workspace.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int64]
+        lib.cueq_seg_outer_workspace.restype = C.c_int64
+        lib.cueq_seg_outer.argtypes = [
+            C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64,
+            C.c_void_p, C.c_int64, C.POINTER(OuterEntry), C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64,
+            C.c_void_p,
+        ]
+        lib.cueq_seg_outer.restype = C.c_int
+        lib.cueq_seg_rowdot.argtypes = [
+            C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
+            C.c_int64, C.c_int64, C.POINTER(GemmProblem), C.c_void_p,
+        ]
+        lib.cueq_seg_rowdot.restype = C.c_int
         _lib = lib
     return _lib
 

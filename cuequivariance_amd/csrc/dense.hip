@@ -1,0 +1,557 @@
+// Dense segmented contractions on the matrix cores (MFMA), for equivariant Linear and
+// fully-connected tensor products with shared weights.
+//
+// After the Clebsch-Gordan modes are flattened, every path of such a polynomial is a small GEMM
+//     C[z, c_seg, :] (+)= alpha * s[z] * A[z, a_seg, :] @ W_p            (K x N weight block W_p)
+// with an optional per-row scalar s[z] (the second operand of a fully-connected product, whose
+// multiplicity is 1).  Stands for the closed modules the reference calls at
+// cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_fused_tp.py:27-72
+// (FusedTensorProductOp3 / Op4).
+//
+// seg_gemm: one workgroup per (weight block, persistent slot).  Each wavefront owns 32 output
+// columns and keeps its K x 32 slice of the weight block in registers for the whole kernel; row
+// tiles of A (32 rows x K) stream through LDS (double buffered, 16-byte coalesced global loads).
+// The contraction index is permuted so that each lane reads contiguous LDS words.
+// seg_outer: weight gradient, contraction over the batch; both MFMA operands are read straight
+// from global memory (the batch index is the MFMA k index), per-workgroup partial sums are folded
+// in a fixed order: no atomics.
+
+#include <vector>
+
+#include "common.h"
+#include "u1d_spec.h"
+
+namespace cueq {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+struct GemmProblem {
+  int64_t a_off, c_off, b_off;
+  double alpha;
+  int32_t s_col, trans_b;
+  int32_t accumulate, pad;
+};
+
+constexpr int kMaxProblems = 32;
+struct GemmProblems {
+  GemmProblem p[kMaxProblems];
+};
+
+// The problem table travels by value in the kernel arguments; selecting with a uniform compare
+// chain keeps it in scalar registers (a dynamic index would force a copy to scratch memory).
+__device__ __forceinline__ GemmProblem select_problem(const GemmProblems& probs, int idx) {
+  GemmProblem pr = probs.p[0];
+#pragma unroll
+  for (int i = 1; i < kMaxProblems; ++i)
+    if (i == idx) pr = probs.p[i];
+  return pr;
+}
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(uint16_t v) { return bf16_bits_to_float(v); }
+__device__ __forceinline__ void from_float(float& d, float v) { d = v; }
+__device__ __forceinline__ void from_float(uint16_t& d, float v) { d = float_to_bf16_bits(v); }
+__device__ __forceinline__ double to_float(double v) { return v; }
+__device__ __forceinline__ void from_float(double& d, double v) { d = v; }
+__device__ __forceinline__ void from_float(float& d, double v) { d = static_cast<float>(v); }
+
+// ------------------------------------------------------------------------------------------------
+// fp32: v_mfma_f32_32x32x2_f32.  A operand lane l holds A[l%32][k(l/32, step)], B operand B[k][l%32].
+// ------------------------------------------------------------------------------------------------
+template <int K, int NW>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3))) seg_gemm_f32(const float* __restrict__ A, int64_t lda, const float* __restrict__ B,
+                                                    const float* __restrict__ S, int64_t lds_, float* __restrict__ C,
+                                                    int64_t ldc, int64_t rows, int N, GemmProblems probs) {
+  constexpr int KH = K / 2;        // contraction indices handled by one lane half
+  constexpr int LDA = K + 4;       // padded LDS row (floats)
+  extern __shared__ float smem[];  // 2 x 32 x LDA
+  const GemmProblem pr = select_problem(probs, blockIdx.y);
+  constexpr int nthreads = 64 * NW;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int n0 = wave * 32;
+
+  float breg[KH];
+#pragma unroll
+  for (int s = 0; s < KH; ++s) {
+    const int k = h * KH + s;
+    breg[s] = pr.trans_b ? B[pr.b_off + static_cast<int64_t>(n0 + c) * K + k] : B[pr.b_off + static_cast<int64_t>(k) * N + n0 + c];
+  }
+
+  const int64_t ntiles = (rows + 31) / 32;
+  constexpr int V4_PER_ROW = K / 4;
+  constexpr int total_v4 = 32 * V4_PER_ROW;
+  constexpr int per_thread = (total_v4 + nthreads - 1) / nthreads;
+  float4 stage[per_thread];
+
+  auto load_tile = [&](int64_t t) {
+#pragma unroll
+    for (int q = 0; q < per_thread; ++q) {
+      const int e = tid + q * nthreads;
+      if (e < total_v4) {
+        const int r = e / V4_PER_ROW, v = e - r * V4_PER_ROW;
+        int64_t row = t * 32 + r;
+        if (row >= rows) row = rows - 1;
+        stage[q] = *reinterpret_cast<const float4*>(A + row * lda + pr.a_off + v * 4);
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+    float* dst = smem + buf * 32 * LDA;
+#pragma unroll
+    for (int q = 0; q < per_thread; ++q) {
+      const int e = tid + q * nthreads;
+      if (e < total_v4) {
+        const int r = e / V4_PER_ROW, v = e - r * V4_PER_ROW;
+        *reinterpret_cast<float4*>(dst + r * LDA + v * 4) = stage[q];
+      }
+    }
+  };
+
+  int64_t t = blockIdx.x;
+  if (t < ntiles) load_tile(t);
+  int buf = 0;
+  for (; t < ntiles; t += gridDim.x) {
+    store_tile(buf);
+    __syncthreads();
+    const int64_t tn = t + gridDim.x;
+    if (tn < ntiles) load_tile(tn);
+    const float* a = smem + buf * 32 * LDA + c * LDA + h * KH;
+    floatx16 acc = {0};
+#pragma unroll
+    for (int s4 = 0; s4 < KH; s4 += 4) {
+      const float4 av = *reinterpret_cast<const float4*>(a + s4);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, breg[s4 + 0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, breg[s4 + 1], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, breg[s4 + 2], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, breg[s4 + 3], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int64_t row = t * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+      if (row < rows) {
+        float val = static_cast<float>(pr.alpha) * acc[v];
+        if (pr.s_col >= 0) val *= S[row * lds_ + pr.s_col];
+        float* dst = C + row * ldc + pr.c_off + n0 + c;
+        *dst = pr.accumulate ? *dst + val : val;
+      }
+    }
+    buf ^= 1;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// bf16 in / bf16 out, fp32 accumulate: v_mfma_f32_32x32x16_bf16 (lane half h supplies 8 of the 16 k)
+// ------------------------------------------------------------------------------------------------
+template <int K, int NW>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4))) seg_gemm_bf16(const uint16_t* __restrict__ A, int64_t lda,
+                                                     const uint16_t* __restrict__ B, const uint16_t* __restrict__ S,
+                                                     int64_t lds_, uint16_t* __restrict__ C, int64_t ldc, int64_t rows,
+                                                     int N, GemmProblems probs) {
+  constexpr int KH = K / 2;
+  constexpr int STEPS = K / 16;
+  constexpr int LDA = K + 8;  // padded LDS row (bf16)
+  extern __shared__ float smem[];
+  uint16_t* sm = reinterpret_cast<uint16_t*>(smem);
+  const GemmProblem pr = select_problem(probs, blockIdx.y);
+  constexpr int nthreads = 64 * NW;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int n0 = wave * 32;
+
+  bf16x8 breg[STEPS];
+#pragma unroll
+  for (int q = 0; q < STEPS; ++q) {
+    uint16_t tmp[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int k = h * KH + q * 8 + e;
+      tmp[e] = pr.trans_b ? B[pr.b_off + static_cast<int64_t>(n0 + c) * K + k] : B[pr.b_off + static_cast<int64_t>(k) * N + n0 + c];
+    }
+    breg[q] = *reinterpret_cast<bf16x8*>(tmp);
+  }
+
+  const int64_t ntiles = (rows + 31) / 32;
+  constexpr int V8_PER_ROW = K / 8;  // 16-byte chunks per row
+  constexpr int total = 32 * V8_PER_ROW;
+  constexpr int per_thread = (total + nthreads - 1) / nthreads;
+  uint4 stage[per_thread];
+
+  auto load_tile = [&](int64_t t) {
+#pragma unroll
+    for (int q = 0; q < per_thread; ++q) {
+      const int e = tid + q * nthreads;
+      if (e < total) {
+        const int r = e / V8_PER_ROW, v = e - r * V8_PER_ROW;
+        int64_t row = t * 32 + r;
+        if (row >= rows) row = rows - 1;
+        stage[q] = *reinterpret_cast<const uint4*>(A + row * lda + pr.a_off + v * 8);
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+    uint16_t* dst = sm + buf * 32 * LDA;
+#pragma unroll
+    for (int q = 0; q < per_thread; ++q) {
+      const int e = tid + q * nthreads;
+      if (e < total) {
+        const int r = e / V8_PER_ROW, v = e - r * V8_PER_ROW;
+        *reinterpret_cast<uint4*>(dst + r * LDA + v * 8) = stage[q];
+      }
+    }
+  };
+
+  int64_t t = blockIdx.x;
+  if (t < ntiles) load_tile(t);
+  int buf = 0;
+  for (; t < ntiles; t += gridDim.x) {
+    store_tile(buf);
+    __syncthreads();
+    const int64_t tn = t + gridDim.x;
+    if (tn < ntiles) load_tile(tn);
+    const uint16_t* a = sm + buf * 32 * LDA + c * LDA + h * KH;
+    floatx16 acc = {0};
+#pragma unroll
+    for (int q = 0; q < STEPS; ++q) {
+      const bf16x8 av = *reinterpret_cast<const bf16x8*>(a + q * 8);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, breg[q], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int64_t row = t * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+      if (row < rows) {
+        float val = static_cast<float>(pr.alpha) * acc[v];
+        if (pr.s_col >= 0) val *= bf16_bits_to_float(S[row * lds_ + pr.s_col]);
+        uint16_t* dst = C + row * ldc + pr.c_off + n0 + c;
+        if (pr.accumulate) val += bf16_bits_to_float(*dst);
+        *dst = float_to_bf16_bits(val);
+      }
+    }
+    buf ^= 1;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// generic fallback (any K, N; float, double, bf16): one thread per output element
+// ------------------------------------------------------------------------------------------------
+template <typename IO, typename ACC>
+__global__ void __launch_bounds__(256) seg_gemm_simple(const IO* __restrict__ A, int64_t lda, const IO* __restrict__ B,
+                                                       const IO* __restrict__ S, int64_t lds_, IO* __restrict__ C,
+                                                       int64_t ldc, int64_t rows, int K, int N, GemmProblems probs) {
+  const GemmProblem pr = select_problem(probs, blockIdx.y);
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= rows * N) return;
+  const int64_t row = tid / N;
+  const int n = static_cast<int>(tid - row * N);
+  ACC acc = 0;
+  for (int k = 0; k < K; ++k) {
+    const ACC b = pr.trans_b ? static_cast<ACC>(to_float(B[pr.b_off + static_cast<int64_t>(n) * K + k]))
+                             : static_cast<ACC>(to_float(B[pr.b_off + static_cast<int64_t>(k) * N + n]));
+    acc += static_cast<ACC>(to_float(A[row * lda + pr.a_off + k])) * b;
+  }
+  acc *= static_cast<ACC>(pr.alpha);
+  if (pr.s_col >= 0) acc *= static_cast<ACC>(to_float(S[row * lds_ + pr.s_col]));
+  IO* dst = C + row * ldc + pr.c_off + n;
+  if (pr.accumulate) acc += static_cast<ACC>(to_float(*dst));
+  from_float(*dst, acc);
+}
+
+// ------------------------------------------------------------------------------------------------
+// weight gradient: dW[k][n] = sum over entries e and rows z of alpha_e * s_e[z] * A[z, a_off_e + k] * G[z, c_off_e + n]
+// partial[slot][k][n] per workgroup, folded afterwards.
+// ------------------------------------------------------------------------------------------------
+struct OuterEntry {
+  int64_t a_off, c_off;
+  double alpha;
+  int32_t s_col, pad;
+};
+constexpr int kMaxOuterEntries = 32;
+struct OuterProblem {
+  OuterEntry e[kMaxOuterEntries];
+  int32_t n_entries;
+  int32_t trans_out;  // 0: dW[k][n], 1: dW[n][k]
+};
+
+template <typename IO, int NB>
+__global__ void __launch_bounds__(512) seg_outer_mfma(const IO* __restrict__ A, int64_t lda, const IO* __restrict__ G,
+                                                      int64_t ldg, const IO* __restrict__ S, int64_t lds_,
+                                                      float* __restrict__ partial, int64_t rows, int K,
+                                                      int64_t rows_per_block, OuterProblem pr) {
+  // wavefront w owns k-block w (32 rows of dW) and all NB column blocks; the batch index is the MFMA k
+  // index: lane half h feeds row zi + 2q + h.  Eight row pairs are loaded before their MFMAs are issued.
+  constexpr int N = NB * 32;
+  constexpr int UNROLL = 8;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int k0 = wave * 32;
+  floatx16 acc[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) acc[j] = floatx16{0};
+  const int64_t z_begin = static_cast<int64_t>(blockIdx.x) * rows_per_block;
+  const int64_t z_end = z_begin + rows_per_block < rows ? z_begin + rows_per_block : rows;
+  for (int ent = 0; ent < pr.n_entries; ++ent) {
+    OuterEntry en = pr.e[0];
+#pragma unroll
+    for (int i = 1; i < kMaxOuterEntries; ++i)
+      if (i == ent) en = pr.e[i];
+    const float alpha = static_cast<float>(en.alpha);
+    for (int64_t zi = z_begin; zi < z_end; zi += 2 * UNROLL) {
+      float a[UNROLL], g[UNROLL][NB];
+#pragma unroll
+      for (int q = 0; q < UNROLL; ++q) {
+        const int64_t z = zi + 2 * q + h;
+        const bool ok = z < z_end;
+        const int64_t zz = ok ? z : z_end - 1;
+        float av = to_float(A[zz * lda + en.a_off + k0 + c]) * alpha;
+        if (en.s_col >= 0) av *= to_float(S[zz * lds_ + en.s_col]);
+        a[q] = ok ? av : 0.f;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) g[q][j] = to_float(G[zz * ldg + en.c_off + j * 32 + c]);
+      }
+#pragma unroll
+      for (int q = 0; q < UNROLL; ++q)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q], g[q][j], acc[j], 0, 0, 0);
+    }
+  }
+  float* out = partial + static_cast<int64_t>(blockIdx.x) * K * N;
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int k = k0 + 8 * (v >> 2) + 4 * h + (v & 3);
+      const int n = j * 32 + c;
+      out[pr.trans_out ? static_cast<int64_t>(n) * K + k : static_cast<int64_t>(k) * N + n] = acc[j][v];
+    }
+  }
+}
+
+template <typename IO, typename ACC>
+__global__ void __launch_bounds__(256) seg_outer_simple(const IO* __restrict__ A, int64_t lda, const IO* __restrict__ G,
+                                                        int64_t ldg, const IO* __restrict__ S, int64_t lds_,
+                                                        ACC* __restrict__ partial, int64_t rows, int K, int N,
+                                                        int64_t rows_per_block, OuterProblem pr) {
+  const int64_t z_begin = static_cast<int64_t>(blockIdx.y) * rows_per_block;
+  const int64_t z_end = z_begin + rows_per_block < rows ? z_begin + rows_per_block : rows;
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= K * N) return;
+  const int k = e / N, n = e - k * N;
+  ACC acc = 0;
+  for (int ent = 0; ent < pr.n_entries; ++ent) {
+    const OuterEntry en = pr.e[ent];
+    for (int64_t z = z_begin; z < z_end; ++z) {
+      ACC a = static_cast<ACC>(to_float(A[z * lda + en.a_off + k])) * static_cast<ACC>(en.alpha);
+      if (en.s_col >= 0) a *= static_cast<ACC>(to_float(S[z * lds_ + en.s_col]));
+      acc += a * static_cast<ACC>(to_float(G[z * ldg + en.c_off + n]));
+    }
+  }
+  partial[static_cast<int64_t>(blockIdx.y) * K * N + (pr.trans_out ? static_cast<int64_t>(n) * K + k : static_cast<int64_t>(k) * N + n)] = acc;
+}
+
+// out[e] (+)= sum over slots (ascending) of partial[slot][e]
+template <typename IO, typename ACC>
+__global__ void __launch_bounds__(256) fold_slots(const ACC* __restrict__ partial, int nslots, int64_t n, IO* __restrict__ out,
+                                                  int accumulate) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (e >= n) return;
+  ACC acc = 0;
+  for (int s = 0; s < nslots; ++s) acc += partial[static_cast<int64_t>(s) * n + e];
+  if (accumulate) acc += static_cast<ACC>(to_float(out[e]));
+  from_float(out[e], acc);
+}
+
+// row-wise dot: dS[z, s_col] (+)= alpha * sum_n G[z, c_off + n] * (A[z, a_off:a_off+K] @ W)[n]
+template <typename IO, typename ACC>
+__global__ void __launch_bounds__(256) seg_rowdot(const IO* __restrict__ A, int64_t lda, const IO* __restrict__ B,
+                                                  const IO* __restrict__ G, int64_t ldg, IO* __restrict__ dS, int64_t lds_,
+                                                  int64_t rows, int K, int N, GemmProblem pr) {
+  // one wavefront per row: lanes over n, loop over k
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+  if (row >= rows) return;
+  ACC acc = 0;
+  for (int n = lane; n < N; n += 64) {
+    ACC t = 0;
+    for (int k = 0; k < K; ++k) {
+      const ACC b = pr.trans_b ? static_cast<ACC>(to_float(B[pr.b_off + static_cast<int64_t>(n) * K + k]))
+                               : static_cast<ACC>(to_float(B[pr.b_off + static_cast<int64_t>(k) * N + n]));
+      t += static_cast<ACC>(to_float(A[row * lda + pr.a_off + k])) * b;
+    }
+    acc += t * static_cast<ACC>(to_float(G[row * ldg + pr.c_off + n]));
+  }
+  for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 64);
+  if (lane == 0) {
+    acc *= static_cast<ACC>(pr.alpha);
+    IO* dst = dS + row * lds_ + pr.s_col;
+    if (pr.accumulate) acc += static_cast<ACC>(to_float(*dst));
+    from_float(*dst, acc);
+  }
+}
+
+static int device_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+}  // namespace cueq
+
+using namespace cueq;
+
+extern "C" int cueq_seg_gemm(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* S,
+                             int64_t lds_, void* C, int64_t ldc, int64_t rows, const cueq_gemm_problem* problems,
+                             int32_t nproblems, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(K > 0 && N > 0 && rows >= 0 && nproblems >= 0, CUEQ_ERR_INVALID, "bad sizes");
+  CUEQ_REQUIRE(nproblems <= kMaxProblems, CUEQ_ERR_TOO_LARGE, "at most %d problems per call", kMaxProblems);
+  if (rows == 0 || nproblems == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(A && B && C && problems, CUEQ_ERR_INVALID, "null pointer");
+  GemmProblems pp;
+  for (int i = 0; i < nproblems; ++i) {
+    pp.p[i] = {problems[i].a_off, problems[i].c_off, problems[i].b_off, problems[i].alpha, problems[i].s_col,
+               problems[i].trans_b, problems[i].accumulate, 0};
+    CUEQ_REQUIRE(problems[i].s_col < 0 || S, CUEQ_ERR_INVALID, "row scale requested without S");
+  }
+  const bool mfma_ok = (K == 32 || K == 64 || K == 128) && (N == 32 || N == 64 || N == 128) && (lda % 8 == 0);
+  bool aligned = mfma_ok;
+  for (int i = 0; i < nproblems && aligned; ++i) aligned = (problems[i].a_off % 8 == 0);
+  if (aligned && (dtype == CUEQ_F32 || dtype == CUEQ_BF16)) {
+    const int threads = 64 * (N / 32);
+    const int64_t ntiles = (rows + 31) / 32;
+    int64_t gx = (static_cast<int64_t>(device_cus()) * 4 + nproblems - 1) / nproblems;
+    if (gx > ntiles) gx = ntiles;
+    if (gx < 1) gx = 1;
+    const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(nproblems));
+    KernelTimer timer(dtype == CUEQ_F32 ? "seg_gemm_f32" : "seg_gemm_bf16", stream);
+    if (dtype == CUEQ_F32) {
+      const size_t sh = 2 * 32 * (K + 4) * sizeof(float);
+#define LAUNCH(KK, NW) hipLaunchKernelGGL((seg_gemm_f32<KK, NW>), grid, dim3(threads), sh, stream, static_cast<const float*>(A), lda, static_cast<const float*>(B), static_cast<const float*>(S), lds_, static_cast<float*>(C), ldc, rows, N, pp)
+#define LAUNCH_N(KK) switch (N) { case 32: LAUNCH(KK, 1); break; case 64: LAUNCH(KK, 2); break; default: LAUNCH(KK, 4); }
+      switch (K) { case 32: LAUNCH_N(32); break; case 64: LAUNCH_N(64); break; default: LAUNCH_N(128); }
+#undef LAUNCH_N
+#undef LAUNCH
+    } else {
+      const size_t sh = 2 * 32 * (K + 8) * sizeof(uint16_t);
+#define LAUNCH(KK, NW) hipLaunchKernelGGL((seg_gemm_bf16<KK, NW>), grid, dim3(threads), sh, stream, static_cast<const uint16_t*>(A), lda, static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(S), lds_, static_cast<uint16_t*>(C), ldc, rows, N, pp)
+#define LAUNCH_N(KK) switch (N) { case 32: LAUNCH(KK, 1); break; case 64: LAUNCH(KK, 2); break; default: LAUNCH(KK, 4); }
+      switch (K) { case 32: LAUNCH_N(32); break; case 64: LAUNCH_N(64); break; default: LAUNCH_N(128); }
+#undef LAUNCH_N
+#undef LAUNCH
+    }
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
+  const int64_t total = rows * N;
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256), static_cast<unsigned>(nproblems));
+  CUEQ_REQUIRE((total + 255) / 256 < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "too many rows");
+  KernelTimer timer("seg_gemm_simple", stream);
+  if (dtype == CUEQ_F32)
+    hipLaunchKernelGGL((seg_gemm_simple<float, float>), grid, dim3(256), 0, stream, static_cast<const float*>(A), lda, static_cast<const float*>(B), static_cast<const float*>(S), lds_, static_cast<float*>(C), ldc, rows, K, N, pp);
+  else if (dtype == CUEQ_F64)
+    hipLaunchKernelGGL((seg_gemm_simple<double, double>), grid, dim3(256), 0, stream, static_cast<const double*>(A), lda, static_cast<const double*>(B), static_cast<const double*>(S), lds_, static_cast<double*>(C), ldc, rows, K, N, pp);
+  else if (dtype == CUEQ_BF16)
+    hipLaunchKernelGGL((seg_gemm_simple<uint16_t, float>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(A), lda, static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(S), lds_, static_cast<uint16_t*>(C), ldc, rows, K, N, pp);
+  else {
+    set_error("seg_gemm: unsupported dtype %d", dtype);
+    return CUEQ_ERR_UNSUPPORTED;
+  }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+static int64_t outer_slots(int64_t rows) {
+  int64_t slots = static_cast<int64_t>(device_cus()) * 2;
+  const int64_t max_by_rows = (rows + 255) / 256;  // at least 256 rows per slot
+  if (slots > max_by_rows) slots = max_by_rows;
+  return slots < 1 ? 1 : slots;
+}
+
+extern "C" int64_t cueq_seg_outer_workspace(int32_t dtype, int32_t K, int32_t N, int64_t rows) {
+  const int64_t acc = dtype == CUEQ_F64 ? 8 : 4;
+  return outer_slots(rows) * K * N * acc;
+}
+
+extern "C" int cueq_seg_outer(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* G, int64_t ldg,
+                              const void* S, int64_t lds_, void* dW, int64_t rows, const cueq_outer_entry* entries,
+                              int32_t nentries, int32_t trans_out, int32_t accumulate, void* workspace,
+                              int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(K > 0 && N > 0 && rows >= 0 && nentries >= 1, CUEQ_ERR_INVALID, "bad sizes");
+  CUEQ_REQUIRE(nentries <= kMaxOuterEntries, CUEQ_ERR_TOO_LARGE, "at most %d entries per call", kMaxOuterEntries);
+  CUEQ_REQUIRE(dW && entries && (rows == 0 || (A && G)), CUEQ_ERR_INVALID, "null pointer");
+  OuterProblem pr;
+  pr.n_entries = nentries;
+  pr.trans_out = trans_out;
+  for (int i = 0; i < nentries; ++i) {
+    pr.e[i] = {entries[i].a_off, entries[i].c_off, entries[i].alpha, entries[i].s_col, 0};
+    CUEQ_REQUIRE(entries[i].s_col < 0 || S, CUEQ_ERR_INVALID, "row scale requested without S");
+  }
+  const int64_t slots = outer_slots(rows);
+  const int64_t need = cueq_seg_outer_workspace(dtype, K, N, rows);
+  CUEQ_REQUIRE(workspace && workspace_bytes >= need, CUEQ_ERR_INVALID, "workspace too small: need %lld bytes", (long long)need);
+  const int64_t rows_per_block = ((rows + slots - 1) / slots + 15) & ~int64_t(15);
+  const int64_t kn = static_cast<int64_t>(K) * N;
+  const bool mfma_ok = (K % 32 == 0) && K <= 256 && (N == 32 || N == 64 || N == 128) && (dtype == CUEQ_F32 || dtype == CUEQ_BF16);
+  {
+    KernelTimer timer(mfma_ok ? "seg_outer_mfma" : "seg_outer_simple", stream);
+    if (mfma_ok) {
+      const dim3 grid(static_cast<unsigned>(slots)), block(64 * (K / 32));
+#define LAUNCH_OUTER(IO, NB) hipLaunchKernelGGL((seg_outer_mfma<IO, NB>), grid, block, 0, stream, static_cast<const IO*>(A), lda, static_cast<const IO*>(G), ldg, static_cast<const IO*>(S), lds_, static_cast<float*>(workspace), rows, K, rows_per_block, pr)
+      if (dtype == CUEQ_F32) { switch (N) { case 32: LAUNCH_OUTER(float, 1); break; case 64: LAUNCH_OUTER(float, 2); break; default: LAUNCH_OUTER(float, 4); } }
+      else { switch (N) { case 32: LAUNCH_OUTER(uint16_t, 1); break; case 64: LAUNCH_OUTER(uint16_t, 2); break; default: LAUNCH_OUTER(uint16_t, 4); } }
+#undef LAUNCH_OUTER
+    } else {
+      const dim3 grid(static_cast<unsigned>((kn + 255) / 256), static_cast<unsigned>(slots));
+      if (dtype == CUEQ_F32)
+        hipLaunchKernelGGL((seg_outer_simple<float, float>), grid, dim3(256), 0, stream, static_cast<const float*>(A), lda, static_cast<const float*>(G), ldg, static_cast<const float*>(S), lds_, static_cast<float*>(workspace), rows, K, N, rows_per_block, pr);
+      else if (dtype == CUEQ_F64)
+        hipLaunchKernelGGL((seg_outer_simple<double, double>), grid, dim3(256), 0, stream, static_cast<const double*>(A), lda, static_cast<const double*>(G), ldg, static_cast<const double*>(S), lds_, static_cast<double*>(workspace), rows, K, N, rows_per_block, pr);
+      else if (dtype == CUEQ_BF16)
+        hipLaunchKernelGGL((seg_outer_simple<uint16_t, float>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(A), lda, static_cast<const uint16_t*>(G), ldg, static_cast<const uint16_t*>(S), lds_, static_cast<float*>(workspace), rows, K, N, rows_per_block, pr);
+      else {
+        set_error("seg_outer: unsupported dtype %d", dtype);
+        return CUEQ_ERR_UNSUPPORTED;
+      }
+    }
+  }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  const dim3 fgrid(static_cast<unsigned>((kn + 255) / 256));
+  if (dtype == CUEQ_F32)
+    hipLaunchKernelGGL((fold_slots<float, float>), fgrid, dim3(256), 0, stream, static_cast<const float*>(workspace), static_cast<int>(slots), kn, static_cast<float*>(dW), accumulate);
+  else if (dtype == CUEQ_F64)
+    hipLaunchKernelGGL((fold_slots<double, double>), fgrid, dim3(256), 0, stream, static_cast<const double*>(workspace), static_cast<int>(slots), kn, static_cast<double*>(dW), accumulate);
+  else
+    hipLaunchKernelGGL((fold_slots<uint16_t, float>), fgrid, dim3(256), 0, stream, static_cast<const float*>(workspace), static_cast<int>(slots), kn, static_cast<uint16_t*>(dW), accumulate);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_seg_rowdot(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* G,
+                               int64_t ldg, void* dS, int64_t lds_, int64_t rows, const cueq_gemm_problem* problem,
+                               void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(K > 0 && N > 0 && rows >= 0 && problem, CUEQ_ERR_INVALID, "bad arguments");
+  if (rows == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(A && B && G && dS && problem->s_col >= 0, CUEQ_ERR_INVALID, "null pointer or missing scale column");
+  const GemmProblem pr{problem->a_off, problem->c_off, problem->b_off, problem->alpha, problem->s_col, problem->trans_b,
+                       problem->accumulate, 0};
+  const dim3 grid(static_cast<unsigned>((rows * 64 + 255) / 256));
+  if (dtype == CUEQ_F32)
+    hipLaunchKernelGGL((seg_rowdot<float, float>), grid, dim3(256), 0, stream, static_cast<const float*>(A), lda, static_cast<const float*>(B), static_cast<const float*>(G), ldg, static_cast<float*>(dS), lds_, rows, K, N, pr);
+  else if (dtype == CUEQ_F64)
+    hipLaunchKernelGGL((seg_rowdot<double, double>), grid, dim3(256), 0, stream, static_cast<const double*>(A), lda, static_cast<const double*>(B), static_cast<const double*>(G), ldg, static_cast<double*>(dS), lds_, rows, K, N, pr);
+  else if (dtype == CUEQ_BF16)
+    hipLaunchKernelGGL((seg_rowdot<uint16_t, float>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(A), lda, static_cast<const uint16_t*>(B), static_cast<const uint16_t*>(G), ldg, static_cast<uint16_t*>(dS), lds_, rows, K, N, pr);
+  else {
+    set_error("seg_rowdot: unsupported dtype %d", dtype);
+    return CUEQ_ERR_UNSUPPORTED;
+  }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}

@@ -1,0 +1,245 @@
+"""Dense executor (``method="fused_tp"``): Linear and fully-connected tensor products on the matrix cores.
+
+Mirror of ``cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_fused_tp.py:75-262``
+for the polynomial forms the high-level layers produce:
+
+* 3 operands ``weights[uv], x[iu] -> out[iv]``          (equivariant Linear, ``descriptors/irreps_tp.py:505-521``)
+* 4 operands ``weights[uvw], x1[iu], x2[jv] -> out[kw]`` with ``v = 1`` (fully-connected product whose second
+  operand has multiplicity one, e.g. spherical harmonics; ``descriptors/irreps_tp.py:22-47``)
+
+with weights shared over the batch.  After the Clebsch-Gordan modes are flattened every path is a small
+GEMM ``out[:, k_seg] += c * x2[:, j] * x1[:, i_seg] @ W_p``; they are grouped into launches of
+``cueq_seg_gemm`` (MFMA).  The backward pass calls ``cueq_seg_gemm`` with transposed blocks (input
+gradient), ``cueq_seg_outer`` (weight gradient, batch reduction without atomics) and ``cueq_seg_rowdot``
+(gradient of the multiplicity-one operand).  First-order gradients only.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn as nn
+
+from .. import _lib, cue
+
+__all__ = ["SegmentedPolynomialDense"]
+
+_DTYPE_CODE = {torch.float32: _lib.F32, torch.float64: _lib.F64, torch.bfloat16: _lib.BF16}
+
+
+class _Path:
+    __slots__ = ("w_off", "a_off", "j", "c_off", "K", "N", "coeff")
+
+    def __init__(self, w_off, a_off, j, c_off, K, N, coeff):
+        self.w_off, self.a_off, self.j, self.c_off, self.K, self.N, self.coeff = w_off, a_off, j, c_off, K, N, coeff
+
+
+def _analyse(polynomial: cue.SegmentedPolynomial):
+    """Flatten to per-path GEMMs.  Returns (paths, has_x2)."""
+    if polynomial.num_outputs != 1 or len(polynomial.operations) != 1:
+        raise NotImplementedError("fused_tp: exactly one operation with one output is supported")
+    ope, stp = polynomial.operations[0]
+    if tuple(ope.buffers) != tuple(range(stp.num_operands)) or stp.num_operands not in (3, 4):
+        raise NotImplementedError(f"fused_tp supports 3 or 4 operands in buffer order. Got {stp.subscripts}.")
+    if stp.num_paths == 0:
+        raise NotImplementedError("fused_tp does not support empty paths.")
+    # every mode that does not index the weights (the irrep components i, j, k) is flattened away
+    d = stp.flatten_modes([m for m in stp.subscripts.modes() if m not in stp.subscripts.operands[0]])
+    ss = d.subscripts.operands
+    if stp.num_operands == 3:
+        if not (len(ss[0]) == 2 and ss[1] == ss[0][0] and ss[2] == ss[0][1]):
+            raise NotImplementedError(f"fused_tp does not support {d.subscripts} (expected uv,u,v)")
+    else:
+        if not (len(ss[0]) == 3 and ss[1] == ss[0][0] and ss[2] == ss[0][1] and ss[3] == ss[0][2]):
+            raise NotImplementedError(f"fused_tp does not support {d.subscripts} (expected uvw,u,v,w)")
+        if d.get_dims(ss[2]) - {1}:
+            raise NotImplementedError(
+                "fused_tp: the second operand of a 4-operand contraction must have multiplicity 1 "
+                f"(got extents {sorted(d.get_dims(ss[2]))})"
+            )
+    offs = [o.segment_offsets() for o in d.operands]
+    paths = []
+    for p in d.paths:
+        c = float(p.coefficients)
+        if c == 0.0:
+            continue
+        wshape = d.operands[0][p.indices[0]]
+        K, N = wshape[0], wshape[-1]
+        j = offs[2][p.indices[2]] if stp.num_operands == 4 else -1
+        paths.append(_Path(offs[0][p.indices[0]], offs[1][p.indices[1]], j, offs[-1][p.indices[-1]], K, N, c))
+    return paths, stp.num_operands == 4
+
+
+def _problem_array(items):
+    arr = (_lib.GemmProblem * max(1, len(items)))()
+    for n, (a_off, c_off, b_off, s_col, trans_b, alpha, acc) in enumerate(items):
+        arr[n].a_off, arr[n].c_off, arr[n].b_off = a_off, c_off, b_off
+        arr[n].s_col, arr[n].trans_b, arr[n].alpha, arr[n].accumulate = s_col, trans_b, alpha, acc
+    return arr
+
+
+def _launch_gemms(dtype, A, B, S, Cout, items_by_shape):
+    """items_by_shape: {(K, N): [(a_off, c_off, b_off, s_col, trans_b, alpha)]}; resolves overwrite/accumulate."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(A.device).cuda_stream
+    written = set()
+    for (K, N), items in items_by_shape.items():
+        pending = list(items)
+        while pending:
+            launch, rest, seen = [], [], set()
+            for it in pending:
+                if it[1] in seen or len(launch) >= 32:
+                    rest.append(it)
+                else:
+                    seen.add(it[1])
+                    launch.append(it + (1 if it[1] in written else 0,))
+            written |= seen
+            arr = _problem_array(launch)
+            _lib.check(
+                lib.cueq_seg_gemm(
+                    _DTYPE_CODE[dtype], K, N, A.data_ptr(), A.stride(0), B.data_ptr(),
+                    S.data_ptr() if S is not None else None, S.stride(0) if S is not None else 0,
+                    Cout.data_ptr(), Cout.stride(0), A.shape[0], arr, len(launch), stream,
+                ),
+                "cueq_seg_gemm",
+            )
+            pending = rest
+    return written
+
+
+class _DenseFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, mod: "SegmentedPolynomialDense", w, x1, x2):
+        dtype = x1.dtype
+        Z = x1.shape[0]
+        out = torch.zeros((Z, mod.out_size), dtype=dtype, device=x1.device)
+        wd = w.detach().to(dtype).contiguous()
+        x1d = x1.detach().contiguous()
+        x2d = x2.detach().contiguous() if x2 is not None else None
+        if Z > 0:
+            with torch.cuda.device(x1.device):
+                by_shape: Dict[tuple, list] = {}
+                for p in mod.paths:
+                    by_shape.setdefault((p.K, p.N), []).append((p.a_off, p.c_off, p.w_off, p.j, 0, p.coeff))
+                _launch_gemms(dtype, x1d, wd, x2d, out, by_shape)
+        ctx.mod = mod
+        ctx.save_for_backward(w, x1, x2 if x2 is not None else torch.empty(0))
+        ctx.has_x2 = x2 is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        mod = ctx.mod
+        w, x1, x2 = ctx.saved_tensors
+        x2 = x2 if ctx.has_x2 else None
+        dtype = x1.dtype
+        lib = _lib.load()
+        g = g.contiguous()
+        wd = w.detach().to(dtype).contiguous()
+        x1d = x1.detach().contiguous()
+        x2d = x2.detach().contiguous() if x2 is not None else None
+        Z = x1.shape[0]
+        gw = gx1 = gx2 = None
+        with torch.cuda.device(x1.device):
+            stream = torch.cuda.current_stream(x1.device).cuda_stream
+            if ctx.needs_input_grad[2]:
+                gx1 = torch.zeros_like(x1d)
+                if Z > 0:
+                    by_shape: Dict[tuple, list] = {}
+                    for p in mod.paths:  # dx1[:, i_seg] += c * x2[:, j] * g[:, k_seg] @ W_p^T
+                        by_shape.setdefault((p.N, p.K), []).append((p.c_off, p.a_off, p.w_off, p.j, 1, p.coeff))
+                    _launch_gemms(dtype, g, wd, x2d, gx1, by_shape)
+            if ctx.needs_input_grad[1]:
+                gwd = torch.zeros_like(wd)
+                if Z > 0:
+                    groups: Dict[tuple, list] = {}
+                    for p in mod.paths:
+                        groups.setdefault((p.w_off, p.K, p.N), []).append(p)
+                    for (w_off, K, N), plist in groups.items():
+                        ws_bytes = lib.cueq_seg_outer_workspace(_DTYPE_CODE[dtype], K, N, Z)
+                        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x1.device)
+                        for c0 in range(0, len(plist), 32):
+                            chunk = plist[c0: c0 + 32]
+                            ent = (_lib.OuterEntry * len(chunk))()
+                            for n, p in enumerate(chunk):
+                                ent[n].a_off, ent[n].c_off, ent[n].s_col, ent[n].alpha = p.a_off, p.c_off, p.j, p.coeff
+                            _lib.check(
+                                lib.cueq_seg_outer(
+                                    _DTYPE_CODE[dtype], K, N, x1d.data_ptr(), x1d.stride(0), g.data_ptr(), g.stride(0),
+                                    x2d.data_ptr() if x2d is not None else None,
+                                    x2d.stride(0) if x2d is not None else 0,
+                                    gwd.data_ptr() + w_off * gwd.element_size(), Z, ent, len(chunk), 0,
+                                    1 if c0 > 0 else 0, ws.data_ptr(), ws_bytes, stream,
+                                ),
+                                "cueq_seg_outer",
+                            )
+                gw = gwd.to(w.dtype).reshape(w.shape)
+            if x2 is not None and ctx.needs_input_grad[3]:
+                gx2 = torch.zeros_like(x2d)
+                touched = set()
+                for p in mod.paths:
+                    if Z == 0:
+                        break
+                    pr = _problem_array([(p.a_off, p.c_off, p.w_off, p.j, 0, p.coeff, 1 if p.j in touched else 0)])
+                    touched.add(p.j)
+                    _lib.check(
+                        lib.cueq_seg_rowdot(
+                            _DTYPE_CODE[dtype], p.K, p.N, x1d.data_ptr(), x1d.stride(0), wd.data_ptr(), g.data_ptr(),
+                            g.stride(0), gx2.data_ptr(), gx2.stride(0), Z, pr, stream,
+                        ),
+                        "cueq_seg_rowdot",
+                    )
+        return None, gw, gx1, gx2
+
+
+class SegmentedPolynomialDense(nn.Module):
+    """Dense (MFMA) executor for Linear / fully-connected polynomials with weights shared over the batch."""
+
+    def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype=None, output_dtype_map: List[int] = None,
+                 name: str = "segmented_polynomial"):
+        super().__init__()
+        self._polynomial_orig = polynomial
+        self._output_dtype_map_orig = output_dtype_map
+        self.name = name
+        if isinstance(math_dtype, str):
+            math_dtype = getattr(torch, math_dtype)
+        if math_dtype not in (None, torch.float32, torch.float64):
+            raise ValueError("Fused TP only supports math_dtype==float32 or math_dtype==float64")
+        self.math_dtype = math_dtype
+        self.num_inputs, self.num_outputs = polynomial.num_inputs, polynomial.num_outputs
+        self.input_sizes = [o.size for o in polynomial.inputs]
+        self.out_size = polynomial.outputs[0].size
+        self.paths, self.has_x2 = _analyse(polynomial)
+
+    def __reduce__(self):
+        from .segmented_polynomial import SegmentedPolynomial
+
+        return (SegmentedPolynomial, (self._polynomial_orig, "fused_tp", self.math_dtype, self._output_dtype_map_orig, self.name))
+
+    def forward(self, inputs: List[torch.Tensor], input_indices: Dict[int, torch.Tensor],
+                output_shapes: Dict[int, torch.Tensor], output_indices: Dict[int, torch.Tensor]):
+        for i, (x, size) in enumerate(zip(inputs, self.input_sizes)):
+            if x.ndim != 2 or x.shape[-1] != size:
+                raise ValueError(f"Input {i} has shape {tuple(x.shape)} but expected shape (rows, {size}).")
+        if input_indices or output_indices or output_shapes:
+            raise NotImplementedError("fused_tp: indexed operands are not implemented by the dense executor")
+        w, x1 = inputs[0], inputs[1]
+        x2 = inputs[2] if self.has_x2 else None
+        if x1.device.type != "cuda":
+            raise RuntimeError("fused_tp runs on the GPU only; got tensors on " + str(x1.device))
+        if w.shape[0] != 1:
+            raise NotImplementedError("fused_tp: weights must be shared over the batch (one row)")
+        if x1.dtype not in _DTYPE_CODE:
+            raise ValueError(f"fused_tp: unsupported dtype {x1.dtype}")
+        if self.math_dtype == torch.float32 and x1.dtype == torch.float64:
+            raise ValueError("Fused TP does not support float32 math_dtype with float64 inputs.")
+        if x2 is not None:
+            if x2.dtype != x1.dtype:
+                raise ValueError("fused_tp: both operands must have the same dtype")
+            if x2.shape[0] == 1 and x1.shape[0] != 1:
+                x2 = x2.expand(x1.shape[0], x2.shape[1])
+            elif x1.shape[0] == 1 and x2.shape[0] != 1:
+                x1 = x1.expand(x2.shape[0], x1.shape[1])
+        return [_DenseFunction.apply(self, w, x1, x2)]

@@ -127,6 +127,48 @@ int64_t cueq_segment_csr_workspace(int64_t n, int64_t nrows);
 int cueq_segment_csr_build(const void* index, int32_t index_is_64, int64_t n, int64_t nrows,
                            int64_t* offsets, int64_t* perm, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* dense segmented contractions (matrix cores)                                */
+/* ------------------------------------------------------------------------- */
+
+/* One small GEMM of a flattened Linear / fully-connected polynomial:
+ *   C[z, c_off : c_off+N] (+)= alpha * S[z, s_col] * A[z, a_off : a_off+K] @ W,   W = K x N block of B at b_off
+ * (trans_b: the block is stored N x K).  Replaces the closed modules FusedTensorProductOp3 / Op4 constructed at
+ * cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_fused_tp.py:27-72. */
+typedef struct {
+  int64_t a_off, c_off, b_off;
+  double alpha;
+  int32_t s_col;      /* column of the per-row scalar in S, -1: none */
+  int32_t trans_b;
+  int32_t accumulate; /* 0: overwrite the output segment, 1: add to it */
+  int32_t reserved;
+} cueq_gemm_problem;
+
+/* At most 32 problems per call; all share K, N, the row strides lda/lds/ldc (in elements) and must write disjoint
+ * output segments.  dtype: CUEQ_F32 / CUEQ_BF16 run on MFMA when K, N are in {32, 64, 128}; otherwise, and for
+ * CUEQ_F64, a plain kernel runs.  Accumulation is in fp32 (fp64 for CUEQ_F64). */
+int cueq_seg_gemm(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* S,
+                  int64_t lds, void* C, int64_t ldc, int64_t rows, const cueq_gemm_problem* problems, int32_t nproblems,
+                  void* stream);
+
+/* Weight gradient of the same contraction, summed over the batch without atomics:
+ *   dW[k][n] (+)= sum_e sum_z alpha_e * S[z, s_col_e] * A[z, a_off_e + k] * G[z, c_off_e + n]
+ * (trans_out: dW stored N x K).  workspace: cueq_seg_outer_workspace bytes. */
+typedef struct {
+  int64_t a_off, c_off;
+  double alpha;
+  int32_t s_col;
+  int32_t reserved;
+} cueq_outer_entry;
+int64_t cueq_seg_outer_workspace(int32_t dtype, int32_t K, int32_t N, int64_t rows);
+int cueq_seg_outer(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* G, int64_t ldg,
+                   const void* S, int64_t lds, void* dW, int64_t rows, const cueq_outer_entry* entries, int32_t nentries,
+                   int32_t trans_out, int32_t accumulate, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Gradient of the per-row scalar:  dS[z, s_col] (+)= alpha * sum_n G[z, c_off + n] * (A[z, a_off : a_off+K] @ W)[n]. */
+int cueq_seg_rowdot(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* G,
+                    int64_t ldg, void* dS, int64_t lds, int64_t rows, const cueq_gemm_problem* problem, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
