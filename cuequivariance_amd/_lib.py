@@ -137,14 +137,14 @@ def load() -> C.CDLL:
         lib.cueq_segment_csr_build.restype = C.c_int
         lib.cueq_seg_gemm.argtypes = [
             C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
-            C.c_int64, C.c_int64, C.POINTER(GemmProblem), C.c_int32, C.c_void_p,
+            C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p,
         ]
         lib.cueq_seg_gemm.restype = C.c_int
         lib.cueq_seg_outer_workspace.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int64]
         lib.cueq_seg_outer_workspace.restype = C.c_int64
         lib.cueq_seg_outer.argtypes = [
             C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64,
-            C.c_void_p, C.c_int64, C.POINTER(OuterEntry), C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64,
+            C.c_void_p, C.c_int64, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64,
             C.c_void_p,
         ]
         lib.cueq_seg_outer.restype = C.c_int

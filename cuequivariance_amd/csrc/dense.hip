@@ -33,20 +33,7 @@ struct GemmProblem {
   int32_t accumulate, pad;
 };
 
-constexpr int kMaxProblems = 32;
-struct GemmProblems {
-  GemmProblem p[kMaxProblems];
-};
-
-// The problem table travels by value in the kernel arguments; selecting with a uniform compare
-// chain keeps it in scalar registers (a dynamic index would force a copy to scratch memory).
-__device__ __forceinline__ GemmProblem select_problem(const GemmProblems& probs, int idx) {
-  GemmProblem pr = probs.p[0];
-#pragma unroll
-  for (int i = 1; i < kMaxProblems; ++i)
-    if (i == idx) pr = probs.p[i];
-  return pr;
-}
+constexpr int kMaxProblems = 65535;  // grid.y
 
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(uint16_t v) { return bf16_bits_to_float(v); }
@@ -58,15 +45,17 @@ __device__ __forceinline__ void from_float(float& d, double v) { d = static_cast
 
 // ------------------------------------------------------------------------------------------------
 // fp32: v_mfma_f32_32x32x2_f32.  A operand lane l holds A[l%32][k(l/32, step)], B operand B[k][l%32].
+// A row tile is RT x 32 rows; one barrier per tile.
 // ------------------------------------------------------------------------------------------------
-template <int K, int NW>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3))) seg_gemm_f32(const float* __restrict__ A, int64_t lda, const float* __restrict__ B,
-                                                    const float* __restrict__ S, int64_t lds_, float* __restrict__ C,
-                                                    int64_t ldc, int64_t rows, int N, GemmProblems probs) {
+template <int K, int NW, int RT>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) seg_gemm_f32(
+    const float* __restrict__ A, int64_t lda, const float* __restrict__ B, const float* __restrict__ S, int64_t lds_,
+    float* __restrict__ C, int64_t ldc, int64_t rows, int N, const GemmProblem* __restrict__ probs) {
   constexpr int KH = K / 2;        // contraction indices handled by one lane half
   constexpr int LDA = K + 4;       // padded LDS row (floats)
-  extern __shared__ float smem[];  // 2 x 32 x LDA
-  const GemmProblem pr = select_problem(probs, blockIdx.y);
+  constexpr int TM = 32 * RT;      // rows per tile
+  extern __shared__ float smem[];  // 2 x TM x LDA
+  const GemmProblem pr = probs[blockIdx.y];
   constexpr int nthreads = 64 * NW;
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
@@ -79,9 +68,9 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3)
     breg[s] = pr.trans_b ? B[pr.b_off + static_cast<int64_t>(n0 + c) * K + k] : B[pr.b_off + static_cast<int64_t>(k) * N + n0 + c];
   }
 
-  const int64_t ntiles = (rows + 31) / 32;
+  const int64_t ntiles = (rows + TM - 1) / TM;
   constexpr int V4_PER_ROW = K / 4;
-  constexpr int total_v4 = 32 * V4_PER_ROW;
+  constexpr int total_v4 = TM * V4_PER_ROW;
   constexpr int per_thread = (total_v4 + nthreads - 1) / nthreads;
   float4 stage[per_thread];
 
@@ -91,14 +80,14 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3)
       const int e = tid + q * nthreads;
       if (e < total_v4) {
         const int r = e / V4_PER_ROW, v = e - r * V4_PER_ROW;
-        int64_t row = t * 32 + r;
+        int64_t row = t * TM + r;
         if (row >= rows) row = rows - 1;
         stage[q] = *reinterpret_cast<const float4*>(A + row * lda + pr.a_off + v * 4);
       }
     }
   };
   auto store_tile = [&](int buf) {
-    float* dst = smem + buf * 32 * LDA;
+    float* dst = smem + buf * TM * LDA;
 #pragma unroll
     for (int q = 0; q < per_thread; ++q) {
       const int e = tid + q * nthreads;
@@ -109,6 +98,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3)
     }
   };
 
+  const float alpha = static_cast<float>(pr.alpha);
   int64_t t = blockIdx.x;
   if (t < ntiles) load_tile(t);
   int buf = 0;
@@ -117,24 +107,36 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(3)
     __syncthreads();
     const int64_t tn = t + gridDim.x;
     if (tn < ntiles) load_tile(tn);
-    const float* a = smem + buf * 32 * LDA + c * LDA + h * KH;
-    floatx16 acc = {0};
 #pragma unroll
-    for (int s4 = 0; s4 < KH; s4 += 4) {
-      const float4 av = *reinterpret_cast<const float4*>(a + s4);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, breg[s4 + 0], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, breg[s4 + 1], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, breg[s4 + 2], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, breg[s4 + 3], acc, 0, 0, 0);
-    }
+    for (int rt = 0; rt < RT; ++rt) {
+      const float* a = smem + (buf * TM + rt * 32 + c) * LDA + h * KH;
+      // all LDS reads of the sub-tile are issued before the first MFMA; they return in order
+      float4 av[KH / 4];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int64_t row = t * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-      if (row < rows) {
-        float val = static_cast<float>(pr.alpha) * acc[v];
-        if (pr.s_col >= 0) val *= S[row * lds_ + pr.s_col];
-        float* dst = C + row * ldc + pr.c_off + n0 + c;
-        *dst = pr.accumulate ? *dst + val : val;
+      for (int q = 0; q < KH / 4; ++q) av[q] = *reinterpret_cast<const float4*>(a + 4 * q);
+      floatx16 acc = {0};
+#pragma unroll
+      for (int q = 0; q < KH / 4; ++q) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].x, breg[4 * q + 0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].y, breg[4 * q + 1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].z, breg[4 * q + 2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[q].w, breg[4 * q + 3], acc, 0, 0, 0);
+      }
+      // epilogue: uniform sub-tile base + 32-bit lane offset
+      const int64_t r0 = t * TM + rt * 32;
+      float* __restrict__ ctile = C + r0 * ldc + pr.c_off + n0;
+      const float* __restrict__ stile = S + r0 * lds_ + (pr.s_col >= 0 ? pr.s_col : 0);
+      const int64_t rows_left = rows - r0;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int r = 8 * (v >> 2) + 4 * h + (v & 3);
+        if (r < rows_left) {
+          float val = alpha * acc[v];
+          if (pr.s_col >= 0) val *= stile[r * static_cast<int>(lds_)];
+          const int off = r * static_cast<int>(ldc) + c;
+          if (pr.accumulate) val += ctile[off];
+          ctile[off] = val;
+        }
       }
     }
     buf ^= 1;
@@ -148,13 +150,13 @@ template <int K, int NW>
 __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4))) seg_gemm_bf16(const uint16_t* __restrict__ A, int64_t lda,
                                                      const uint16_t* __restrict__ B, const uint16_t* __restrict__ S,
                                                      int64_t lds_, uint16_t* __restrict__ C, int64_t ldc, int64_t rows,
-                                                     int N, GemmProblems probs) {
+                                                     int N, const GemmProblem* __restrict__ probs) {
   constexpr int KH = K / 2;
   constexpr int STEPS = K / 16;
   constexpr int LDA = K + 8;  // padded LDS row (bf16)
   extern __shared__ float smem[];
   uint16_t* sm = reinterpret_cast<uint16_t*>(smem);
-  const GemmProblem pr = select_problem(probs, blockIdx.y);
+  const GemmProblem pr = probs[blockIdx.y];
   constexpr int nthreads = 64 * NW;
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
@@ -238,8 +240,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4)
 template <typename IO, typename ACC>
 __global__ void __launch_bounds__(256) seg_gemm_simple(const IO* __restrict__ A, int64_t lda, const IO* __restrict__ B,
                                                        const IO* __restrict__ S, int64_t lds_, IO* __restrict__ C,
-                                                       int64_t ldc, int64_t rows, int K, int N, GemmProblems probs) {
-  const GemmProblem pr = select_problem(probs, blockIdx.y);
+                                                       int64_t ldc, int64_t rows, int K, int N, const GemmProblem* __restrict__ probs) {
+  const GemmProblem pr = probs[blockIdx.y];
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= rows * N) return;
   const int64_t row = tid / N;
@@ -266,9 +268,8 @@ struct OuterEntry {
   double alpha;
   int32_t s_col, pad;
 };
-constexpr int kMaxOuterEntries = 32;
 struct OuterProblem {
-  OuterEntry e[kMaxOuterEntries];
+  const OuterEntry* e;  // device pointer
   int32_t n_entries;
   int32_t trans_out;  // 0: dW[k][n], 1: dW[n][k]
 };
@@ -291,10 +292,7 @@ __global__ void __launch_bounds__(512) seg_outer_mfma(const IO* __restrict__ A, 
   const int64_t z_begin = static_cast<int64_t>(blockIdx.x) * rows_per_block;
   const int64_t z_end = z_begin + rows_per_block < rows ? z_begin + rows_per_block : rows;
   for (int ent = 0; ent < pr.n_entries; ++ent) {
-    OuterEntry en = pr.e[0];
-#pragma unroll
-    for (int i = 1; i < kMaxOuterEntries; ++i)
-      if (i == ent) en = pr.e[i];
+    const OuterEntry en = pr.e[ent];
     const float alpha = static_cast<float>(en.alpha);
     for (int64_t zi = z_begin; zi < z_end; zi += 2 * UNROLL) {
       float a[UNROLL], g[UNROLL][NB];
@@ -406,32 +404,27 @@ using namespace cueq;
 
 extern "C" int cueq_seg_gemm(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* S,
                              int64_t lds_, void* C, int64_t ldc, int64_t rows, const cueq_gemm_problem* problems,
-                             int32_t nproblems, void* stream_) {
+                             int32_t nproblems, int32_t force_simple, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   CUEQ_REQUIRE(K > 0 && N > 0 && rows >= 0 && nproblems >= 0, CUEQ_ERR_INVALID, "bad sizes");
   CUEQ_REQUIRE(nproblems <= kMaxProblems, CUEQ_ERR_TOO_LARGE, "at most %d problems per call", kMaxProblems);
+  static_assert(sizeof(GemmProblem) == sizeof(cueq_gemm_problem), "ABI struct mismatch");
   if (rows == 0 || nproblems == 0) return CUEQ_OK;
   CUEQ_REQUIRE(A && B && C && problems, CUEQ_ERR_INVALID, "null pointer");
-  GemmProblems pp;
-  for (int i = 0; i < nproblems; ++i) {
-    pp.p[i] = {problems[i].a_off, problems[i].c_off, problems[i].b_off, problems[i].alpha, problems[i].s_col,
-               problems[i].trans_b, problems[i].accumulate, 0};
-    CUEQ_REQUIRE(problems[i].s_col < 0 || S, CUEQ_ERR_INVALID, "row scale requested without S");
-  }
+  const GemmProblem* pp = reinterpret_cast<const GemmProblem*>(problems);
   const bool mfma_ok = (K == 32 || K == 64 || K == 128) && (N == 32 || N == 64 || N == 128) && (lda % 8 == 0);
-  bool aligned = mfma_ok;
-  for (int i = 0; i < nproblems && aligned; ++i) aligned = (problems[i].a_off % 8 == 0);
-  if (aligned && (dtype == CUEQ_F32 || dtype == CUEQ_BF16)) {
+  if (mfma_ok && !force_simple && (dtype == CUEQ_F32 || dtype == CUEQ_BF16)) {
     const int threads = 64 * (N / 32);
-    const int64_t ntiles = (rows + 31) / 32;
-    int64_t gx = (static_cast<int64_t>(device_cus()) * 4 + nproblems - 1) / nproblems;
+    const int rt = 1;
+    const int64_t ntiles = (rows + 32 * rt - 1) / (32 * rt);
+    int64_t gx = (static_cast<int64_t>(device_cus()) * 8 + nproblems - 1) / nproblems;
     if (gx > ntiles) gx = ntiles;
     if (gx < 1) gx = 1;
     const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(nproblems));
     KernelTimer timer(dtype == CUEQ_F32 ? "seg_gemm_f32" : "seg_gemm_bf16", stream);
     if (dtype == CUEQ_F32) {
       const size_t sh = 2 * 32 * (K + 4) * sizeof(float);
-#define LAUNCH(KK, NW) hipLaunchKernelGGL((seg_gemm_f32<KK, NW>), grid, dim3(threads), sh, stream, static_cast<const float*>(A), lda, static_cast<const float*>(B), static_cast<const float*>(S), lds_, static_cast<float*>(C), ldc, rows, N, pp)
+#define LAUNCH(KK, NW) hipLaunchKernelGGL((seg_gemm_f32<KK, NW, 1>), grid, dim3(threads), sh, stream, static_cast<const float*>(A), lda, static_cast<const float*>(B), static_cast<const float*>(S), lds_, static_cast<float*>(C), ldc, rows, N, pp)
 #define LAUNCH_N(KK) switch (N) { case 32: LAUNCH(KK, 1); break; case 64: LAUNCH(KK, 2); break; default: LAUNCH(KK, 4); }
       switch (K) { case 32: LAUNCH_N(32); break; case 64: LAUNCH_N(64); break; default: LAUNCH_N(128); }
 #undef LAUNCH_N
@@ -483,15 +476,13 @@ extern "C" int cueq_seg_outer(int32_t dtype, int32_t K, int32_t N, const void* A
                               int64_t workspace_bytes, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   CUEQ_REQUIRE(K > 0 && N > 0 && rows >= 0 && nentries >= 1, CUEQ_ERR_INVALID, "bad sizes");
-  CUEQ_REQUIRE(nentries <= kMaxOuterEntries, CUEQ_ERR_TOO_LARGE, "at most %d entries per call", kMaxOuterEntries);
+  static_assert(sizeof(OuterEntry) == sizeof(cueq_outer_entry), "ABI struct mismatch");
   CUEQ_REQUIRE(dW && entries && (rows == 0 || (A && G)), CUEQ_ERR_INVALID, "null pointer");
+  (void)S;
   OuterProblem pr;
   pr.n_entries = nentries;
   pr.trans_out = trans_out;
-  for (int i = 0; i < nentries; ++i) {
-    pr.e[i] = {entries[i].a_off, entries[i].c_off, entries[i].alpha, entries[i].s_col, 0};
-    CUEQ_REQUIRE(entries[i].s_col < 0 || S, CUEQ_ERR_INVALID, "row scale requested without S");
-  }
+  pr.e = reinterpret_cast<const OuterEntry*>(entries);
   const int64_t slots = outer_slots(rows);
   const int64_t need = cueq_seg_outer_workspace(dtype, K, N, rows);
   CUEQ_REQUIRE(workspace && workspace_bytes >= need, CUEQ_ERR_INVALID, "workspace too small: need %lld bytes", (long long)need);

@@ -80,33 +80,56 @@ def _problem_array(items):
     return arr
 
 
-def _launch_gemms(dtype, A, B, S, Cout, items_by_shape):
-    """items_by_shape: {(K, N): [(a_off, c_off, b_off, s_col, trans_b, alpha)]}; resolves overwrite/accumulate."""
-    lib = _lib.load()
-    stream = torch.cuda.current_stream(A.device).cuda_stream
-    written = set()
+def _plan_gemm_launches(items_by_shape):
+    """[(K, N, [problem tuples with the accumulate flag], aligned)]: problems of a launch write disjoint segments."""
+    launches, written = [], set()
     for (K, N), items in items_by_shape.items():
         pending = list(items)
         while pending:
             launch, rest, seen = [], [], set()
             for it in pending:
-                if it[1] in seen or len(launch) >= 32:
+                if it[1] in seen:
                     rest.append(it)
                 else:
                     seen.add(it[1])
                     launch.append(it + (1 if it[1] in written else 0,))
             written |= seen
-            arr = _problem_array(launch)
-            _lib.check(
-                lib.cueq_seg_gemm(
-                    _DTYPE_CODE[dtype], K, N, A.data_ptr(), A.stride(0), B.data_ptr(),
-                    S.data_ptr() if S is not None else None, S.stride(0) if S is not None else 0,
-                    Cout.data_ptr(), Cout.stride(0), A.shape[0], arr, len(launch), stream,
-                ),
-                "cueq_seg_gemm",
-            )
+            launches.append((K, N, launch, all(it[0] % 8 == 0 for it in launch)))
             pending = rest
-    return written
+    return launches
+
+
+class _DeviceTables:
+    """Problem tables of one module uploaded to one device (read by the kernels with scalar loads)."""
+
+    def __init__(self, mod: "SegmentedPolynomialDense", device: torch.device):
+        def upload(ctypes_array):
+            raw = bytes(ctypes_array)
+            return torch.frombuffer(bytearray(raw), dtype=torch.uint8).to(device)
+
+        self.fwd = [(K, N, upload(_problem_array(items)), len(items), ok) for K, N, items, ok in mod.fwd_launches]
+        self.dx1 = [(K, N, upload(_problem_array(items)), len(items), ok) for K, N, items, ok in mod.dx1_launches]
+        self.dw = []
+        for (w_off, K, N), plist in mod.dw_groups.items():
+            ent = (_lib.OuterEntry * len(plist))()
+            for n, p in enumerate(plist):
+                ent[n].a_off, ent[n].c_off, ent[n].s_col, ent[n].alpha = p.a_off, p.c_off, p.j, p.coeff
+            self.dw.append((w_off, K, N, upload(ent), len(plist)))
+
+
+def _run_gemms(dtype, A, B, S, Cout, launches):
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(A.device).cuda_stream
+    for K, N, table, n, aligned in launches:
+        force_simple = 0 if (aligned and A.stride(0) % 8 == 0) else 1
+        _lib.check(
+            lib.cueq_seg_gemm(
+                _DTYPE_CODE[dtype], K, N, A.data_ptr(), A.stride(0), B.data_ptr(),
+                S.data_ptr() if S is not None else None, S.stride(0) if S is not None else 0,
+                Cout.data_ptr(), Cout.stride(0), A.shape[0], table.data_ptr(), n, force_simple, stream,
+            ),
+            "cueq_seg_gemm",
+        )
 
 
 class _DenseFunction(torch.autograd.Function):
@@ -114,16 +137,13 @@ class _DenseFunction(torch.autograd.Function):
     def forward(ctx, mod: "SegmentedPolynomialDense", w, x1, x2):
         dtype = x1.dtype
         Z = x1.shape[0]
-        out = torch.zeros((Z, mod.out_size), dtype=dtype, device=x1.device)
+        out = (torch.empty if mod.fwd_covers_output else torch.zeros)((Z, mod.out_size), dtype=dtype, device=x1.device)
         wd = w.detach().to(dtype).contiguous()
         x1d = x1.detach().contiguous()
         x2d = x2.detach().contiguous() if x2 is not None else None
         if Z > 0:
             with torch.cuda.device(x1.device):
-                by_shape: Dict[tuple, list] = {}
-                for p in mod.paths:
-                    by_shape.setdefault((p.K, p.N), []).append((p.a_off, p.c_off, p.w_off, p.j, 0, p.coeff))
-                _launch_gemms(dtype, x1d, wd, x2d, out, by_shape)
+                _run_gemms(dtype, x1d, wd, x2d, out, mod.tables(x1.device).fwd)
         ctx.mod = mod
         ctx.save_for_backward(w, x1, x2 if x2 is not None else torch.empty(0))
         ctx.has_x2 = x2 is not None
@@ -143,38 +163,28 @@ class _DenseFunction(torch.autograd.Function):
         Z = x1.shape[0]
         gw = gx1 = gx2 = None
         with torch.cuda.device(x1.device):
+            tables = mod.tables(x1.device)
             stream = torch.cuda.current_stream(x1.device).cuda_stream
             if ctx.needs_input_grad[2]:
-                gx1 = torch.zeros_like(x1d)
+                # dx1[:, i_seg] += c * x2[:, j] * g[:, k_seg] @ W_p^T
+                gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
                 if Z > 0:
-                    by_shape: Dict[tuple, list] = {}
-                    for p in mod.paths:  # dx1[:, i_seg] += c * x2[:, j] * g[:, k_seg] @ W_p^T
-                        by_shape.setdefault((p.N, p.K), []).append((p.c_off, p.a_off, p.w_off, p.j, 1, p.coeff))
-                    _launch_gemms(dtype, g, wd, x2d, gx1, by_shape)
+                    _run_gemms(dtype, g, wd, x2d, gx1, tables.dx1)
             if ctx.needs_input_grad[1]:
                 gwd = torch.zeros_like(wd)
                 if Z > 0:
-                    groups: Dict[tuple, list] = {}
-                    for p in mod.paths:
-                        groups.setdefault((p.w_off, p.K, p.N), []).append(p)
-                    for (w_off, K, N), plist in groups.items():
+                    for w_off, K, N, ent, n in tables.dw:
                         ws_bytes = lib.cueq_seg_outer_workspace(_DTYPE_CODE[dtype], K, N, Z)
                         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x1.device)
-                        for c0 in range(0, len(plist), 32):
-                            chunk = plist[c0: c0 + 32]
-                            ent = (_lib.OuterEntry * len(chunk))()
-                            for n, p in enumerate(chunk):
-                                ent[n].a_off, ent[n].c_off, ent[n].s_col, ent[n].alpha = p.a_off, p.c_off, p.j, p.coeff
-                            _lib.check(
-                                lib.cueq_seg_outer(
-                                    _DTYPE_CODE[dtype], K, N, x1d.data_ptr(), x1d.stride(0), g.data_ptr(), g.stride(0),
-                                    x2d.data_ptr() if x2d is not None else None,
-                                    x2d.stride(0) if x2d is not None else 0,
-                                    gwd.data_ptr() + w_off * gwd.element_size(), Z, ent, len(chunk), 0,
-                                    1 if c0 > 0 else 0, ws.data_ptr(), ws_bytes, stream,
-                                ),
-                                "cueq_seg_outer",
-                            )
+                        _lib.check(
+                            lib.cueq_seg_outer(
+                                _DTYPE_CODE[dtype], K, N, x1d.data_ptr(), x1d.stride(0), g.data_ptr(), g.stride(0),
+                                x2d.data_ptr() if x2d is not None else None, x2d.stride(0) if x2d is not None else 0,
+                                gwd.data_ptr() + w_off * gwd.element_size(), Z, ent.data_ptr(), n, 0, 0,
+                                ws.data_ptr(), ws_bytes, stream,
+                            ),
+                            "cueq_seg_outer",
+                        )
                 gw = gwd.to(w.dtype).reshape(w.shape)
             if x2 is not None and ctx.needs_input_grad[3]:
                 gx2 = torch.zeros_like(x2d)
@@ -212,6 +222,26 @@ class SegmentedPolynomialDense(nn.Module):
         self.input_sizes = [o.size for o in polynomial.inputs]
         self.out_size = polynomial.outputs[0].size
         self.paths, self.has_x2 = _analyse(polynomial)
+        fwd, dx1 = {}, {}
+        self.dw_groups: Dict[tuple, list] = {}
+        for p in self.paths:
+            fwd.setdefault((p.K, p.N), []).append((p.a_off, p.c_off, p.w_off, p.j, 0, p.coeff))
+            dx1.setdefault((p.N, p.K), []).append((p.c_off, p.a_off, p.w_off, p.j, 1, p.coeff))
+            self.dw_groups.setdefault((p.w_off, p.K, p.N), []).append(p)
+        self.fwd_launches = _plan_gemm_launches(fwd)
+        self.dx1_launches = _plan_gemm_launches(dx1)
+        out_cols = sum(N for _, N, items, _ in self.fwd_launches for it in items if it[6] == 0)
+        in_cols = sum(N for _, N, items, _ in self.dx1_launches for it in items if it[6] == 0)
+        self.fwd_covers_output = out_cols == self.out_size
+        self.dx1_covers_input = in_cols == self.input_sizes[1]
+        self._tables: Dict[int, _DeviceTables] = {}
+
+    def tables(self, device: torch.device) -> _DeviceTables:
+        idx = device.index if device.index is not None else torch.cuda.current_device()
+        t = self._tables.get(idx)
+        if t is None:
+            t = self._tables[idx] = _DeviceTables(self, torch.device("cuda", idx))
+        return t
 
     def __reduce__(self):
         from .segmented_polynomial import SegmentedPolynomial

@@ -144,16 +144,18 @@ typedef struct {
   int32_t reserved;
 } cueq_gemm_problem;
 
-/* At most 32 problems per call; all share K, N, the row strides lda/lds/ldc (in elements) and must write disjoint
- * output segments.  dtype: CUEQ_F32 / CUEQ_BF16 run on MFMA when K, N are in {32, 64, 128}; otherwise, and for
- * CUEQ_F64, a plain kernel runs.  Accumulation is in fp32 (fp64 for CUEQ_F64). */
+/* `problems` is a DEVICE pointer to nproblems entries (uploaded once by the caller when the layer is built; the
+ * kernels read it with scalar loads).  All problems of one call share K, N, the row strides lda/lds/ldc (in
+ * elements, lda a multiple of 8, every a_off a multiple of 8 for the MFMA kernels) and must write disjoint output
+ * segments.  dtype: CUEQ_F32 / CUEQ_BF16 run on MFMA when K, N are in {32, 64, 128} and force_simple is 0;
+ * otherwise, and for CUEQ_F64, a plain kernel runs.  Accumulation is in fp32 (fp64 for CUEQ_F64). */
 int cueq_seg_gemm(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* S,
                   int64_t lds, void* C, int64_t ldc, int64_t rows, const cueq_gemm_problem* problems, int32_t nproblems,
-                  void* stream);
+                  int32_t force_simple, void* stream);
 
 /* Weight gradient of the same contraction, summed over the batch without atomics:
  *   dW[k][n] (+)= sum_e sum_z alpha_e * S[z, s_col_e] * A[z, a_off_e + k] * G[z, c_off_e + n]
- * (trans_out: dW stored N x K).  workspace: cueq_seg_outer_workspace bytes. */
+ * (trans_out: dW stored N x K).  `entries` is a DEVICE pointer.  workspace: cueq_seg_outer_workspace bytes. */
 typedef struct {
   int64_t a_off, c_off;
   double alpha;

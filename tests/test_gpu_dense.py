@@ -1,0 +1,130 @@
+"""GPU parity tests of the dense (MFMA) executor behind ``method="fused_tp"`` against the CPU oracle.
+
+``Linear`` and ``FullyConnectedTensorProduct`` follow the reference's operation tests
+(``cuequivariance_torch/tests/operations/linear_test.py:37-96``,
+``cuequivariance_torch/tests/operations/tensor_product_test.py:30-108``): outputs and first
+derivatives, several dtypes, shared and batched weights.
+
+Tolerances (max-norm relative to ``max|ref|``): float64 1e-12, float32 1e-5, bfloat16 2e-2.  The
+float64 oracle is evaluated on the inputs after rounding to the tested dtype.
+"""
+
+import pytest
+import torch
+
+from cuequivariance_amd import cue
+from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float64: 1e-12, torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def rel_err(got, ref):
+    got, ref = got.detach().cpu().double(), ref.detach().cpu().double()
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    return (got - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
+
+
+def check_against_oracle(device, module, inputs, dtype):
+    """inputs: float64 host tensors in the polynomial's operand order (weights first)."""
+    rounded = [t.to(dtype).double() for t in inputs]
+    spec = spec_from_polynomial(module.f._polynomial_orig)
+    a = [t.clone().requires_grad_(True) for t in rounded]
+    ref = naive_segmented_polynomial(spec, a)[0]
+    cot = torch.randn(ref.shape, dtype=torch.float64, generator=torch.Generator().manual_seed(99)).to(dtype).double()
+    ref_grads = torch.autograd.grad(ref, a, cot)
+    b = [t.to(dtype).to(device).requires_grad_(True) for t in rounded]
+    out = module.f(b)[0]
+    assert out.dtype == dtype
+    grads = torch.autograd.grad(out, b, cot.to(dtype).to(device))
+    tol = TOL[dtype]
+    assert rel_err(out, ref) <= tol, ("out", rel_err(out, ref))
+    for i, (g, r) in enumerate(zip(grads, ref_grads)):
+        assert g.dtype == dtype and g.shape == b[i].shape
+        assert rel_err(g, r) <= tol, (f"grad {i}", rel_err(g, r))
+
+
+def linear_module(irreps_in, irreps_out, **kw):
+    from cuequivariance_amd import cuet
+
+    return cuet.Linear(cue.Irreps("O3", irreps_in), cue.Irreps("O3", irreps_out), layout=cue.ir_mul,
+                       internal_weights=False, method="fused_tp", **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize(
+    "irreps_in,irreps_out,Z",
+    [
+        ("128x0e+128x1o+128x2e", "128x0e+128x1o+128x2e", 1000),  # MFMA path, K = N = 128
+        ("64x0e+32x1o+48x2e", "32x0e+64x1o+16x2e", 333),  # mixed multiplicities, ragged row count
+        ("32x0e+32x1o", "64x0e+96x1o", 65),
+        ("8x0e+3x1o", "5x0e+7x1o", 17),  # sizes the MFMA tiling does not cover
+    ],
+)
+def test_linear_matches_oracle(device, dtype, irreps_in, irreps_out, Z):
+    m = linear_module(irreps_in, irreps_out)
+    g = torch.Generator().manual_seed(Z)
+    w = torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g)
+    x = torch.randn(Z, m.irreps_in.dim, dtype=torch.float64, generator=g)
+    check_against_oracle(device, m, [w, x], dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+def test_fully_connected_matches_oracle(device, dtype):
+    from cuequivariance_amd import cuet
+
+    m = cuet.FullyConnectedTensorProduct(
+        cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e"), cue.Irreps("O3", "64x0e+64x1o"),
+        layout=cue.ir_mul, internal_weights=False,
+    )
+    g = torch.Generator().manual_seed(5)
+    w = torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g)
+    x1 = torch.randn(777, 256, dtype=torch.float64, generator=g)
+    x2 = torch.randn(777, 9, dtype=torch.float64, generator=g)
+    check_against_oracle(device, m, [w, x1, x2], dtype)
+
+
+def test_linear_module_call_and_internal_weights(device):
+    """The module call path (x, weight) and internal weights give what the functional core gives."""
+    from cuequivariance_amd import cuet
+
+    irreps = cue.Irreps("O3", "32x0e+32x1o")
+    m = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=True, method="fused_tp", device=device)
+    x = torch.randn(40, irreps.dim, device=device)
+    y = m(x)
+    y2 = m.f([m.weight, x])[0]
+    assert torch.equal(y, y2)
+    with pytest.raises(ValueError):
+        m(x, torch.randn(1, m.weight_numel, device=device))
+
+
+def test_linear_empty_batch(device):
+    m = linear_module("32x0e+32x1o", "32x0e+32x1o")
+    w = torch.randn(1, m.weight_numel, device=device, requires_grad=True)
+    x = torch.zeros(0, m.irreps_in.dim, device=device, requires_grad=True)
+    y = m(x, w)
+    assert y.shape == (0, m.irreps_out.dim)
+    gw, gx = torch.autograd.grad(y, [w, x], torch.zeros_like(y))
+    assert gx.shape == x.shape and torch.count_nonzero(gw) == 0
+
+
+def test_linear_full_size_properties(device):
+    """At the benchmark's size (200 000 rows x 128 channels x l<=2): linearity in x and in w, and
+    agreement of the weight gradient with the adjoint identity <dy, L_w x> = <dL/dw, w>."""
+    m = linear_module("128x0e+128x1o+128x2e", "128x0e+128x1o+128x2e")
+    Z = 200_000
+    g = torch.Generator(device=device).manual_seed(3)
+    w = torch.randn(1, m.weight_numel, device=device, generator=g, requires_grad=True)
+    x = torch.randn(Z, 1152, device=device, generator=g, requires_grad=True)
+    x2 = torch.randn(Z, 1152, device=device, generator=g)
+    y = m(x, w)
+    y2 = m(x2, w)
+    ysum = m(x + 2 * x2, w)
+    scale = y.abs().max().item()
+    assert (ysum - (y + 2 * y2)).abs().max().item() <= 2e-5 * scale
+    cot = torch.randn(Z, 1152, device=device, generator=g)
+    gw, gx = torch.autograd.grad(y, [w, x], cot)
+    lhs = (cot.double() * y.detach().double()).sum().item()
+    assert abs((gw.double() * w.detach().double()).sum().item() - lhs) <= 1e-4 * abs(lhs) + 1e-3 * scale
+    assert abs((gx.double() * x.detach().double()).sum().item() - lhs) <= 1e-4 * abs(lhs) + 1e-3 * scale
