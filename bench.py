@@ -92,7 +92,7 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["fp32", "fp64"], default="fp32")
     ap.add_argument("--nodes", type=int, default=5000)
     ap.add_argument("--edges", type=int, default=100_000)
-    ap.add_argument("--cpu-sample-edges", type=int, default=4000)
+    ap.add_argument("--cpu-sample-edges", type=int, default=12000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")

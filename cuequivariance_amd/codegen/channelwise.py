@@ -18,8 +18,8 @@ Forward kernel (one wavefront = one output row x 64 channels):
   * the batch rows that scatter into one output row are summed in registers in CSR order, then
     stored once: deterministic, nothing of batch size is materialised.
 
-Backward kernel (one wavefront = a chunk of consecutive batch rows x 64 channels) computes the three
-gradients in one pass over the inputs.  With ``G[b][i][j] = sum_k C[i,j,k] g[k]`` (literal
+Backward kernel (one wavefront per resident slot, each owning a contiguous range of batch rows x 64
+channels) computes the three gradients in one pass over the inputs.  With ``G[b][i][j] = sum_k C[i,j,k] g[k]`` (literal
 coefficients), ``D[b][i] = sum_j G[b][i][j] x2[j]`` and ``F[b][j] = sum_i G[b][i][j] x1[i]``:
 ``dw[b] = sum_i x1[i] D[b][i]``, ``dx1[i] += w[b] D[b][i]``, ``dx2[j] = sum_u w[b] F[b][j]``.
 """
@@ -300,7 +300,7 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
     fp = T
     L = []
     A = L.append
-    A(f"// backward: fused dw / dx1 / dx2, {chunk} batch rows per wavefront")
+    A("// backward: fused dw / dx1 / dx2; every wavefront owns one contiguous, equally sized range of batch rows")
     A("template <bool X1_IDX, bool G_IDX, bool ATOMIC_DX1>")
     A(f"__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu({waves_per_eu}))) bwd_kernel(BWD_PARAMS) {{")
     nch = (st.extent + 63) // 64
@@ -311,7 +311,8 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
         A("  const int uu = ch * 64 + lane; constexpr bool active = true;")
     else:
         A(f"  const int u = ch * 64 + lane; const bool active = u < {st.extent}; const int uu = active ? u : 0;")
-    A(f"  const int64_t z0 = cid * {chunk}ll; const int64_t z1 = (z0 + {chunk} < batch) ? z0 + {chunk} : batch;")
+    A(f"  const int64_t nranges = gridDim.x / {nch};")
+    A("  const int64_t z0 = cid * batch / nranges, z1 = (cid + 1) * batch / nranges;")
     for k in range(st.nseg_out):
         A(f"  {fp} gr{k} = 0;")
     A("  int64_t grow_cur = -1;")
@@ -399,7 +400,8 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
         A("    }")
     A("  }")
     A("}")
-    A(f"constexpr int kBwdChunk = {chunk};")
+    A(f"constexpr int kBwdMinRange = {chunk};   // fewest batch rows worth a wavefront of their own")
+    A(f"constexpr int kBwdWaves = {waves_per_eu};")
     return "\n".join(L)
 
 
@@ -524,9 +526,12 @@ static int run_bwd(const SpecCall& c) {{
     CUEQ_CHECK_HIP(hipGetLastError());
   }}
   if (batch > 0) {{
-    const int64_t nchunks = (batch + kBwdChunk - 1) / kBwdChunk;
-    const int64_t grid = nchunks * {nch};
-    CUEQ_REQUIRE(grid < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "batch too large for one launch");
+    // one launch round of resident wavefronts; short batches get fewer, not shorter than kBwdMinRange rows
+    int64_t nranges = wave_slots(kBwdWaves) / {nch};
+    const int64_t most = (batch + kBwdMinRange - 1) / kBwdMinRange;
+    if (nranges > most) nranges = most;
+    if (nranges < 1) nranges = 1;
+    const int64_t grid = nranges * {nch};
     const dim3 gd(static_cast<unsigned>(grid)), t(64);
     {{
     KernelTimer timer("{name}_bwd_{T}", c.stream);

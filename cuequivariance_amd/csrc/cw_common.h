@@ -66,6 +66,21 @@ __global__ void __launch_bounds__(256) fill_zero(T* __restrict__ p, int64_t n) {
   if (tid < n) p[tid] = 0;
 }
 
+// Compute units of the current device (cached for the first device queried).
+inline int device_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
+}
+
+// Number of resident wavefront slots to fill: compute units x 4 SIMDs x waves per SIMD.
+inline int64_t wave_slots(int waves_per_simd) { return static_cast<int64_t>(device_cus()) * 4 * waves_per_simd; }
+
 inline unsigned blocks_for(int64_t n, int per_block = 256) { return static_cast<unsigned>((n + per_block - 1) / per_block); }
 
 // Scatter policy of the fused backward for the gradient of a gathered operand:

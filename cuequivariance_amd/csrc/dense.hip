@@ -19,6 +19,7 @@
 #include <vector>
 
 #include "common.h"
+#include "cw_common.h"
 #include "u1d_spec.h"
 
 namespace cueq {
@@ -385,17 +386,6 @@ __global__ void __launch_bounds__(256) seg_rowdot(const IO* __restrict__ A, int6
     if (pr.accumulate) acc += static_cast<ACC>(to_float(*dst));
     from_float(*dst, acc);
   }
-}
-
-static int device_cus() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;
-    if (cus <= 0) cus = 256;
-  }
-  return cus;
 }
 
 }  // namespace cueq
