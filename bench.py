@@ -27,6 +27,15 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# Bytes that left the L2 per launch at the default workload (5000 nodes, 100000 edges, fp32), from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE; KiB per dispatch) scaled by what the same
+# counters read for a 1 GiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Summary and commands:
+# profiles/channelwise_c128_l3_fp32_cfg2_hbm_traffic.txt.  Not measurable from inside this process.
+MEASURED_TRAFFIC_BYTES = {
+    ("c128_l3_bwd_float", 5000, 100_000): 4.314e9,
+    ("c128_l3_fwd_float", 5000, 100_000): 2.214e9,
+}
+
 
 def algorithmic_bytes(E: int, N: int, W: int, D1: int, D2: int, D3: int, s: int) -> dict:
     """Compulsory traffic: every distinct input element read once, every output element written once."""
@@ -169,7 +178,7 @@ def main() -> int:
         a = dominant[1]["achieved_GBps"]
         roofline = {
             "bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
-            "traffic": None, "kernel": dominant[0], "avg_ms": dominant[1]["avg_ms"],
+            "traffic": MEASURED_TRAFFIC_BYTES.get((dominant[0], N, E)), "kernel": dominant[0], "avg_ms": dominant[1]["avg_ms"],
             "algorithmic_bytes_per_launch": dominant[1]["algorithmic_bytes"],
         }
     total_alg = alg["fwd"] + alg["bwd"]
