@@ -5,6 +5,7 @@ from .irreps import (
     SU2,
     SO3,
     O3,
+    O3_e3nn,
     MulIrrep,
     Irreps,
     IrrepsLayout,
@@ -16,11 +17,21 @@ from .irreps import (
 )
 from .stp import Subscripts, SegmentedOperand, Path, SegmentedTensorProduct
 from .polynomial import Operation, SegmentedPolynomial, EquivariantPolynomial
+from .reduced_basis import (
+    IrrepsArray,
+    reduced_tensor_product_basis,
+    reduced_symmetric_tensor_product_basis,
+    reduced_antisymmetric_tensor_product_basis,
+    selection_rule_product,
+    selection_rule_power,
+)
 from . import descriptors
+from . import mace
 
 __all__ = [
-    "Irrep", "SU2", "SO3", "O3", "MulIrrep", "Irreps", "IrrepsLayout", "mul_ir", "ir_mul",
+    "Irrep", "SU2", "SO3", "O3", "O3_e3nn", "MulIrrep", "Irreps", "IrrepsLayout", "mul_ir", "ir_mul",
     "IrrepsAndLayout", "clebsch_gordan", "into_list_of_irrep", "Subscripts", "SegmentedOperand",
     "Path", "SegmentedTensorProduct", "Operation", "SegmentedPolynomial", "EquivariantPolynomial",
-    "descriptors",
+    "descriptors", "mace", "IrrepsArray", "reduced_tensor_product_basis", "reduced_symmetric_tensor_product_basis",
+    "reduced_antisymmetric_tensor_product_basis", "selection_rule_product", "selection_rule_power",
 ]

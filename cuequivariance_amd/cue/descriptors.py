@@ -6,26 +6,30 @@ Reference behaviour followed (``cuequivariance/cuequivariance/group_theory/descr
 * ``irreps_tp.py:232-321``  channelwise_tensor_product      ``"uv,iu,jv,kuv+ijk"``
 * ``irreps_tp.py:505-545``  linear                          ``"uv,iu,iv"``
 * ``spherical_harmonics_.py:119-156`` recursion and normalisation of the spherical harmonics
+* ``symmetric_contractions.py:20-134``  symmetric_contraction  ``"w_a_b_c_i+abciw"`` per degree
 
 All descriptors use the ``ir_mul`` layout (component index outside, multiplicity inside).
 """
 
 from __future__ import annotations
 
+import functools
 import itertools
 from typing import Optional, Sequence
 
 import numpy as np
 
 from .irreps import Irrep, Irreps, IrrepsAndLayout, clebsch_gordan, into_list_of_irrep, ir_mul
-from .polynomial import EquivariantPolynomial, SegmentedPolynomial
-from .stp import SegmentedTensorProduct
+from .polynomial import EquivariantPolynomial, Operation, SegmentedPolynomial
+from .reduced_basis import reduced_symmetric_tensor_product_basis
+from .stp import SegmentedOperand, SegmentedTensorProduct
 
 __all__ = [
     "channelwise_tensor_product",
     "fully_connected_tensor_product",
     "linear",
     "spherical_harmonics_values",
+    "symmetric_contraction",
 ]
 
 
@@ -182,3 +186,71 @@ def _sh_irrep(ir_vec: Irrep, ell: int) -> Irrep:
     l2 = ell // 2
     l1 = ell - l2
     return sorted(_sh_irrep(ir_vec, l1) * _sh_irrep(ir_vec, l2), key=_Key)[-1]
+
+
+# ---------------------------------------------------------------------------------------------
+# symmetric contraction
+# ---------------------------------------------------------------------------------------------
+@functools.lru_cache(maxsize=None)
+def _symmetric_contraction_core(irreps_in: Irreps, irreps_out: Irreps, degrees: tuple) -> SegmentedPolynomial:
+    """Polynomial ``weights[u], x[u] -> out[u]``: for every degree n the symmetric part of ``x^n`` is mapped
+    onto ``irreps_out`` with one weight per independent coupling (reference
+    ``descriptors/symmetric_contractions.py:20-88``)."""
+    degrees = list(degrees)
+    if len(degrees) != 1:
+        return SegmentedPolynomial.stack(
+            [_symmetric_contraction_core(irreps_in, irreps_out, (n,)) for n in degrees], [True, False, False]
+        )
+    [degree] = degrees
+    mul = irreps_in.muls[0]
+    assert all(m == mul for m in irreps_in.muls) and all(m == mul for m in irreps_out.muls)
+    irreps_in, irreps_out = irreps_in.set_mul(1), irreps_out.set_mul(1)
+    x_operands = range(1, degree + 1)
+    out_operand = degree + 1
+    x_operand = SegmentedOperand([(mul,)] * irreps_in.dim, ndim=1)
+
+    if degree == 0:
+        d = SegmentedTensorProduct.from_subscripts("i_i")
+        for _, ir in irreps_out:
+            if not ir.is_scalar():
+                d.add_segment(out_operand, {"i": ir.dim})
+            else:
+                d.add_path(None, None, c=1, dims={"i": ir.dim})
+        d = d.flatten_modes("i")
+    else:
+        abc = "abcdefgh"[:degree]
+        d = SegmentedTensorProduct.from_subscripts(f"w_{'_'.join(abc)}_i+{abc}iw")
+        for i in x_operands:
+            d.add_segment(i, (irreps_in.dim,))
+        U = reduced_symmetric_tensor_product_basis(irreps_in, degree, keep_ir=irreps_out, layout=ir_mul)
+        for _, ir in irreps_out:
+            u = U.filter(keep=[ir])
+            if len(u.segments) == 0:
+                d.add_segment(out_operand, {"i": ir.dim})
+            else:
+                [u] = u.segments  # (a, b, c, ..., i, w)
+                d.add_path(None, *(0,) * degree, None, c=u)
+        d = d.normalize_paths_for_operand(out_operand)
+        d = d.flatten_coefficient_modes()
+
+    d = d.append_modes_to_all_operands("u", {"u": mul})
+    for i in x_operands:
+        assert d.operands[i] == x_operand
+    return SegmentedPolynomial(
+        [d.operands[0], x_operand], [d.operands[-1]], [(Operation([0] + [1] * degree + [2]), d)]
+    )
+
+
+def symmetric_contraction(irreps_in: Irreps, irreps_out: Irreps, degrees) -> EquivariantPolynomial:
+    """Weighted sum of the input contracted with itself ``degree`` times, for every degree in ``degrees``.
+
+    Operands: ``weights[u], input[u] -> output[u]`` (all ``ir_mul``); the multiplicities of ``irreps_in`` and
+    ``irreps_out`` must all be equal and are carried as the parallel mode ``u``.  For ``16x(0+1+2) -> 16x(0+1)`` of SO3
+    and degrees (1, 2, 3): 32 + 80 + 176 weights and 4 / 37 / 437 paths (reference
+    ``descriptors/symmetric_contractions.py:91-134``)."""
+    poly = _symmetric_contraction_core(irreps_in, irreps_out, tuple(degrees))
+    return EquivariantPolynomial(
+        [IrrepsAndLayout(irreps_in.new_scalars(poly.inputs[0].size), ir_mul), IrrepsAndLayout(irreps_in, ir_mul)],
+        [IrrepsAndLayout(irreps_out, ir_mul)],
+        poly,
+    )

@@ -350,6 +350,30 @@ class O3(Irrep):
         return SO3(l=self.l).continuous_generators()
 
 
+class O3_e3nn(O3):
+    """O(3) irreps ordered the e3nn way, ``(l, p)`` ascending: ``0e < 0o < 1e < 1o < ...`` (reference
+    ``group_theory/experimental/e3nn.py:23-52``).  The reference takes the coefficients of this group from
+    ``e3nn.o3.wigner_3j(l1, l2, l3) * sqrt(2 l3 + 1)``; they are the same real-basis tensors as :class:`O3`'s
+    (same ``(-i)^l`` change of basis, same normalisation), which is what is used here."""
+
+    def __mul__(self, other) -> list["O3_e3nn"]:
+        return [O3_e3nn(l=ir.l, p=ir.p) for ir in O3.__mul__(self, other)]
+
+    def _key(self):
+        return (self.l, self.p)
+
+    def __lt__(self, other) -> bool:
+        return self._key() < O3_e3nn._from(other)._key()
+
+    @classmethod
+    def iterator(cls):
+        ell = 0
+        while True:
+            yield cls(l=ell, p=(-1) ** ell)
+            yield cls(l=ell, p=-((-1) ** ell))
+            ell += 1
+
+
 _IRREP_CLASSES = {"SU2": SU2, "SO3": SO3, "O3": O3}
 
 

@@ -162,6 +162,38 @@ class SegmentedPolynomial:
         return cls(stp.operands[:-1], (stp.operands[-1],), ((Operation(range(stp.num_operands)), stp),))
 
     @classmethod
+    def stack(cls, polys, stacked) -> "SegmentedPolynomial":
+        """Stack polynomials: operands flagged in ``stacked`` are concatenated over ``polys`` (every tensor product keeps
+        addressing its own slice), the others must be identical.  Operations with equal buffers are then fused
+        (reference ``segmented_polynomial.py:167-232``)."""
+        polys = list(polys)
+        assert len(polys) > 0
+        n_in, n_out = polys[0].num_inputs, polys[0].num_outputs
+        assert all(p.num_inputs == n_in and p.num_outputs == n_out for p in polys)
+        assert len(stacked) == n_in + n_out
+        operands = []
+        for bid in range(n_in + n_out):
+            if stacked[bid]:
+                parts = [p.operands[bid] for p in polys if p.operands[bid] is not None]
+                operands.append(SegmentedOperand(sum([list(o.segments) for o in parts], []), ndim=parts[0].ndim))
+            else:
+                ope = polys[0].operands[bid]
+                assert all(p.operands[bid] == ope for p in polys)
+                operands.append(ope)
+        ops = []
+        for index, pol in enumerate(polys):
+            for ope, stp in pol.operations:
+                stp = stp.copy()
+                for oid, b in enumerate(ope.buffers):
+                    if stacked[b]:
+                        for p in reversed(polys[:index]):
+                            stp.insert_segments(oid, 0, p.operands[b].segments)
+                        for p in polys[index + 1:]:
+                            stp.insert_segments(oid, -1, p.operands[b].segments)
+                ops.append((ope, stp))
+        return cls(operands[:n_in], operands[n_in:], ops).consolidate()
+
+    @classmethod
     def stack_tensor_products(cls, inputs, outputs, operations) -> "SegmentedPolynomial":
         """Operands given as ``None`` are the concatenation of that operand over all operations."""
         inputs, outputs = list(inputs), list(outputs)

@@ -2,7 +2,7 @@
 
 from .transpose import TransposeSegments, TransposeIrrepsLayout
 from .segmented_polynomial import SegmentedPolynomial
-from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear
+from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction
 from .uniform_1d import uniform_1d
 
 __all__ = [
@@ -12,5 +12,6 @@ __all__ = [
     "ChannelWiseTensorProduct",
     "FullyConnectedTensorProduct",
     "Linear",
+    "SymmetricContraction",
     "uniform_1d",
 ]

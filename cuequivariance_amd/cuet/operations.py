@@ -6,6 +6,7 @@ Constructor arguments, attributes (``irreps_*``, ``weight_numel``, ``weight``, `
 * ``cuequivariance_torch/cuequivariance_torch/operations/tp_channel_wise.py:30-258``
 * ``cuequivariance_torch/cuequivariance_torch/operations/tp_fully_connected.py:30-207``
 * ``cuequivariance_torch/cuequivariance_torch/operations/linear.py:30-191``
+* ``cuequivariance_torch/cuequivariance_torch/operations/symmetric_contraction.py:32-242``
 
 Defaults differ where the reference defaults to its PyTorch executor: every layer here runs HIP
 kernels (``uniform_1d`` for the channel-wise product, the dense executor ``fused_tp`` for the other two).
@@ -23,7 +24,7 @@ from ..cue import descriptors
 from .segmented_polynomial import SegmentedPolynomial
 from .transpose import TransposeIrrepsLayout
 
-__all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear"]
+__all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear", "SymmetricContraction"]
 
 
 def _default_irreps(*irreps_list):
@@ -305,4 +306,75 @@ class Linear(torch.nn.Module):
         if weight is None:
             raise ValueError("Weights should not be None")
         out = self.f([weight, self.transpose_in(x)], input_indices=input_indices)
+        return self.transpose_out(out[0])
+
+
+class SymmetricContraction(torch.nn.Module):
+    """Symmetric contraction of MACE (https://arxiv.org/abs/2206.07697): for every degree ``n`` up to
+    ``contraction_degree`` the symmetric part of ``x ⊗ ... ⊗ x`` (``n`` factors) is mapped onto ``irreps_out`` with
+    one learned weight per independent coupling, channel and element type.
+
+    ``weight`` has shape ``(num_elements, weight_shape[0], mul)``; ``forward(x, indices)`` picks the weight row of each
+    batch element by ``indices`` (int32 or int64, one per row of ``x``).  With ``original_mace=True`` the weights are
+    those of the original MACE parametrisation and are projected onto the standard basis at every call.
+    All multiplicities of ``irreps_in`` and ``irreps_out`` must be equal.
+    """
+
+    def __init__(
+        self,
+        irreps_in: cue.Irreps,
+        irreps_out: cue.Irreps,
+        contraction_degree: int,
+        num_elements: int,
+        *,
+        layout: Optional[cue.IrrepsLayout] = None,
+        layout_in: Optional[cue.IrrepsLayout] = None,
+        layout_out: Optional[cue.IrrepsLayout] = None,
+        device: Optional[torch.device] = None,
+        dtype: Optional[torch.dtype] = None,
+        math_dtype=None,
+        original_mace: bool = False,
+        use_fallback: Optional[bool] = None,
+        method: Optional[str] = None,
+    ):
+        super().__init__()
+        irreps_in, irreps_out = _default_irreps(irreps_in, irreps_out)
+        _assert_same_group(irreps_in, irreps_out)
+        self.contraction_degree = contraction_degree
+        if len(set(irreps_in.muls) | set(irreps_out.muls)) != 1:
+            raise ValueError("Input/Output irreps must have the same mul")
+        mul = irreps_in.muls[0]
+        self.irreps_in, self.irreps_out = irreps_in, irreps_out
+        self.etp, p = cue.mace.symmetric_contraction(irreps_in, irreps_out, range(1, contraction_degree + 1))
+        if original_mace:
+            self.register_buffer("projection", torch.tensor(p, dtype=dtype, device=device))
+            self.weight_shape = (p.shape[0], mul)
+        else:
+            self.projection = None
+            self.weight_shape = (self.etp.inputs[0].dim // mul, mul)
+        self.num_elements = num_elements
+        self.weight = torch.nn.Parameter(torch.randn(num_elements, *self.weight_shape, device=device, dtype=dtype))
+        self.transpose_in = TransposeIrrepsLayout(
+            self.etp.inputs[1].irreps, source=_default_layout(layout_in or layout), target=self.etp.inputs[1].layout,
+            device=device,
+        )
+        self.transpose_out = TransposeIrrepsLayout(
+            self.etp.outputs[0].irreps, source=self.etp.outputs[0].layout,
+            target=_default_layout(layout_out or layout), device=device,
+        )
+        if method == "uniform_1d" and not self.etp.polynomial.all_same_segment_shape():
+            raise ValueError("`uniform_1d` method requires segments to be the same shape")
+        self.method = _method_from_fallback(method, use_fallback, "uniform_1d")
+        self.f = SegmentedPolynomial(self.etp.polynomial, method=self.method, math_dtype=math_dtype)
+
+    def extra_repr(self) -> str:
+        return f"contraction_degree={self.contraction_degree}, weight_shape={self.weight_shape}"
+
+    def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+        """``x``: ``(batch, irreps_in.dim)``; ``indices``: ``(batch,)``; returns ``(batch, irreps_out.dim)``."""
+        if self.projection is not None:
+            weight = torch.einsum("zau,ab->zbu", self.weight, self.projection)
+        else:
+            weight = self.weight
+        out = self.f([weight.flatten(1), self.transpose_in(x)], input_indices={0: indices})
         return self.transpose_out(out[0])
