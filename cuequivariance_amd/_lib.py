@@ -37,6 +37,16 @@ EXPORTED_SYMBOLS = (
     "cueq_seg_outer_workspace",
     "cueq_seg_outer",
     "cueq_seg_rowdot",
+    "cueq_gemm_nt",
+    "cueq_transpose",
+    "cueq_layer_norm_fwd",
+    "cueq_layer_norm_bwd_workspace",
+    "cueq_layer_norm_bwd",
+    "cueq_gate_fwd",
+    "cueq_gate_bwd",
+    "cueq_sum_cols",
+    "cueq_sum_rows_workspace",
+    "cueq_sum_rows",
 )
 
 
@@ -153,6 +163,27 @@ def load() -> C.CDLL:
             C.c_int64, C.c_int64, C.POINTER(GemmProblem), C.c_void_p,
         ]
         lib.cueq_seg_rowdot.restype = C.c_int
+        i32, i64, ptr, f64 = C.c_int32, C.c_int64, C.c_void_p, C.c_double
+        lib.cueq_gemm_nt.argtypes = [i32, i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, ptr, i64, i64, i64, f64, i32, ptr]
+        lib.cueq_gemm_nt.restype = C.c_int
+        lib.cueq_transpose.argtypes = [i32, i64, i64, i64, ptr, ptr, ptr]
+        lib.cueq_transpose.restype = C.c_int
+        lib.cueq_layer_norm_fwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, f64, ptr, ptr, ptr, ptr]
+        lib.cueq_layer_norm_fwd.restype = C.c_int
+        lib.cueq_layer_norm_bwd_workspace.argtypes = [i64, i64]
+        lib.cueq_layer_norm_bwd_workspace.restype = i64
+        lib.cueq_layer_norm_bwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, i64, ptr]
+        lib.cueq_layer_norm_bwd.restype = C.c_int
+        lib.cueq_gate_fwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, ptr, i32, ptr, i32, ptr, ptr]
+        lib.cueq_gate_fwd.restype = C.c_int
+        lib.cueq_gate_bwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, ptr, ptr, i32, ptr, i32, ptr, ptr, ptr]
+        lib.cueq_gate_bwd.restype = C.c_int
+        lib.cueq_sum_cols.argtypes = [i32, i64, i64, ptr, ptr, ptr]
+        lib.cueq_sum_cols.restype = C.c_int
+        lib.cueq_sum_rows_workspace.argtypes = [i64, i64]
+        lib.cueq_sum_rows_workspace.restype = i64
+        lib.cueq_sum_rows.argtypes = [i32, i64, i64, ptr, ptr, ptr, i64, ptr]
+        lib.cueq_sum_rows.restype = C.c_int
         _lib = lib
     return _lib
 

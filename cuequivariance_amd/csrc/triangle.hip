@@ -1,0 +1,579 @@
+// Kernels of the triangle multiplicative update (AlphaFold-style pair update):
+//   LayerNorm over the hidden dimension, sigmoid-gated dual projection, the triangular contraction
+//   t[d,b,i,j] = sum_k a[d,b,i,k] b[d,b,j,k], LayerNorm across d with a layout change, output gate.
+// The stages are separate launches composed by the host (cuequivariance_amd/cuet/triangle.py):
+//   cueq_gemm_nt        batched C = alpha * A * B^T (+ C), both operands contraction-contiguous, MFMA
+//   cueq_transpose      batched 2-D transpose through LDS
+//   cueq_layer_norm_*   row LayerNorm forward / backward (one wavefront per row)
+//   cueq_gate_*         out = sigmoid(u + bu) * (v + bv) * mask and its backward
+//   cueq_sum_rows/cols  reductions for the bias / affine gradients
+// Math is fp32 throughout; tensors are fp32 or bf16.
+//
+// Algorithm reference: cuequivariance_jax/cuequivariance_jax/triangle/_triangle_multiplicative_update.py:371-417,
+// _layer_norm_transpose.py:162-227, _sigmoid_gated_dual_gemm.py:111-218 (the torch entry point
+// cuequivariance_torch/primitives/triangle.py:138-262 forwards to a closed kernel).
+
+#include <algorithm>
+
+#include "common.h"
+#include "cw_common.h"
+#include "u1d_spec.h"
+
+namespace cueq {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float tri_load(const float* p, int64_t i) { return p[i]; }
+__device__ __forceinline__ float tri_load(const uint16_t* p, int64_t i) { return bf16_bits_to_float(p[i]); }
+__device__ __forceinline__ void tri_store(float* p, int64_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void tri_store(uint16_t* p, int64_t i, float v) { p[i] = float_to_bf16_bits(v); }
+
+// ------------------------------------------------------------------------------------------------
+// C[b] (M x N) = alpha * A[b] (M x K, row stride lda) * B[b]^T (N x K, row stride ldb)  (+ C[b])
+// 128 x 128 block tile, 4 wavefronts of 64 x 64, 64 bytes of k per row and step, double-buffered LDS.
+// Lane half h of a wavefront supplies the same k subset to both MFMA operands, so the k order
+// inside a step is free and every operand read is one or two ds_read_b128.
+// ------------------------------------------------------------------------------------------------
+constexpr int kTile = 128;
+constexpr int kRowBytes = 80;  // 64 bytes of data + 16 bytes of padding
+
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
+                                                      const TI* __restrict__ B, int64_t ldb, int64_t sB,
+                                                      TO* __restrict__ C, int64_t ldc, int64_t sC, int M, int N, int K,
+                                                      float alpha, int accumulate) {
+  constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
+  constexpr int BK = 64 / sizeof(TI);   // k extent of one step
+  __shared__ __align__(16) char smem[2][2][kTile * kRowBytes];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
+  A += static_cast<int64_t>(blockIdx.z) * sA;
+  B += static_cast<int64_t>(blockIdx.z) * sB;
+  C += static_cast<int64_t>(blockIdx.z) * sC;
+
+  // every thread stages two 16-byte vectors of A and two of B per step
+  uint4 stA[2], stB[2];
+  int ldrow[2], ldpart[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int e = tid + q * 256;
+    ldrow[q] = e >> 2;
+    ldpart[q] = e & 3;
+  }
+  auto load_step = [&](int ks) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int k = ks * BK + ldpart[q] * EPV;
+      const int ra = min(m0 + ldrow[q], M - 1), rb = min(n0 + ldrow[q], N - 1);
+      if (k < K) {
+        stA[q] = *reinterpret_cast<const uint4*>(A + static_cast<int64_t>(ra) * lda + k);
+        stB[q] = *reinterpret_cast<const uint4*>(B + static_cast<int64_t>(rb) * ldb + k);
+      } else {
+        stA[q] = make_uint4(0, 0, 0, 0);
+        stB[q] = make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  auto store_step = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      *reinterpret_cast<uint4*>(&smem[buf][0][ldrow[q] * kRowBytes + ldpart[q] * 16]) = stA[q];
+      *reinterpret_cast<uint4*>(&smem[buf][1][ldrow[q] * kRowBytes + ldpart[q] * 16]) = stB[q];
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = floatx16{0};
+
+  const int nsteps = (K + BK - 1) / BK;
+  load_step(0);
+  int buf = 0;
+  for (int ks = 0; ks < nsteps; ++ks) {
+    store_step(buf);
+    __syncthreads();
+    if (ks + 1 < nsteps) load_step(ks + 1);
+    const char* sa = &smem[buf][0][(wm * 64 + c) * kRowBytes + h * 32];
+    const char* sb = &smem[buf][1][(wn * 64 + c) * kRowBytes + h * 32];
+    uint4 fa[2][2], fb[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        fa[t][q] = *reinterpret_cast<const uint4*>(sa + t * 32 * kRowBytes + q * 16);
+        fb[t][q] = *reinterpret_cast<const uint4*>(sb + t * 32 * kRowBytes + q * 16);
+      }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if constexpr (sizeof(TI) == 2) {
+#pragma unroll
+          for (int q = 0; q < 2; ++q)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[i][q]),
+                                                                __builtin_bit_cast(bf16x8_t, fb[j][q]), acc[i][j], 0, 0, 0);
+        } else {
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const float* pa = reinterpret_cast<const float*>(&fa[i][q]);
+            const float* pb = reinterpret_cast<const float*>(&fb[j][q]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[s], pb[s], acc[i][j], 0, 0, 0);
+          }
+        }
+      }
+    buf ^= 1;
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + c;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (row < M && col < N) {
+          const int64_t o = static_cast<int64_t>(row) * ldc + col;
+          float val = alpha * acc[i][j][v];
+          if (accumulate) val += tri_load(C, o);
+          tri_store(C, o, val);
+        }
+      }
+    }
+}
+
+// any shape / alignment: one thread per output element
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256) gemm_nt_simple(const TI* __restrict__ A, int64_t lda, int64_t sA, const TI* __restrict__ B,
+                                                      int64_t ldb, int64_t sB, TO* __restrict__ C, int64_t ldc, int64_t sC,
+                                                      int M, int N, int K, float alpha, int accumulate) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= static_cast<int64_t>(M) * N) return;
+  const int row = static_cast<int>(tid / N), col = static_cast<int>(tid - static_cast<int64_t>(row) * N);
+  A += static_cast<int64_t>(blockIdx.z) * sA + static_cast<int64_t>(row) * lda;
+  B += static_cast<int64_t>(blockIdx.z) * sB + static_cast<int64_t>(col) * ldb;
+  C += static_cast<int64_t>(blockIdx.z) * sC;
+  float acc = 0;
+  for (int k = 0; k < K; ++k) acc = fmaf(tri_load(A, k), tri_load(B, k), acc);
+  const int64_t o = static_cast<int64_t>(row) * ldc + col;
+  float val = alpha * acc;
+  if (accumulate) val += tri_load(C, o);
+  tri_store(C, o, val);
+}
+
+// ------------------------------------------------------------------------------------------------
+// batched transpose  out[b][c][r] = in[b][r][c]  (32 x 32 tiles through LDS)
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ in, T* __restrict__ out, int R, int Ccols) {
+  __shared__ T tile[32][33];
+  const int64_t base = static_cast<int64_t>(blockIdx.z) * R * Ccols;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = r0 + ty + q * 8, cc = c0 + tx;
+    if (r < R && cc < Ccols) tile[ty + q * 8][tx] = in[base + static_cast<int64_t>(r) * Ccols + cc];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int cc = c0 + ty + q * 8, r = r0 + tx;
+    if (r < R && cc < Ccols) out[base + static_cast<int64_t>(cc) * R + r] = tile[tx][ty + q * 8];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// LayerNorm over rows of length D (D <= 1024): one wavefront per row, biased variance
+// ------------------------------------------------------------------------------------------------
+constexpr int kLnMaxPerLane = 16;
+
+template <typename T>
+__global__ void __launch_bounds__(256) ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                     T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd,
+                                                     int64_t rows, int D, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * D;
+  float v[kLnMaxPerLane];
+  float s = 0;
+#pragma unroll
+  for (int q = 0; q < kLnMaxPerLane; ++q) {
+    const int e = lane + q * 64;
+    v[q] = e < D ? tri_load(xr, e) : 0.f;
+    s += v[q];
+  }
+  const float mu = wave_sum(s) / D;
+  float ss = 0;
+#pragma unroll
+  for (int q = 0; q < kLnMaxPerLane; ++q) {
+    const int e = lane + q * 64;
+    const float d = e < D ? v[q] - mu : 0.f;
+    ss += d * d;
+  }
+  const float rs = 1.0f / sqrtf(wave_sum(ss) / D + eps);
+  T* yr = y + row * D;
+#pragma unroll
+  for (int q = 0; q < kLnMaxPerLane; ++q) {
+    const int e = lane + q * 64;
+    if (e < D) {
+      float o = (v[q] - mu) * rs;
+      if (gamma) o *= tri_load(gamma, e);
+      if (beta) o += tri_load(beta, e);
+      tri_store(yr, e, o);
+    }
+  }
+  if (lane == 0) {
+    mean[row] = mu;
+    rstd[row] = rs;
+  }
+}
+
+// dx = rstd * (g - mean(g) - xhat * mean(g * xhat)),  g = dy * gamma;   per-block partial sums of
+// dgamma = sum dy * xhat and dbeta = sum dy go to part[2][blocks][D].
+template <typename T>
+__global__ void __launch_bounds__(256) ln_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ mean,
+                                                     const float* __restrict__ rstd, const T* __restrict__ gamma,
+                                                     T* __restrict__ dx, float* __restrict__ part, int64_t rows, int D,
+                                                     int rows_per_block) {
+  extern __shared__ float sred[];  // [4 waves][2][D]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float ag[kLnMaxPerLane], ab[kLnMaxPerLane];
+#pragma unroll
+  for (int q = 0; q < kLnMaxPerLane; ++q) ag[q] = ab[q] = 0.f;
+  const int64_t r_begin = static_cast<int64_t>(blockIdx.x) * rows_per_block;
+  const int64_t r_end = min(r_begin + rows_per_block, rows);
+  for (int64_t row = r_begin + wave; row < r_end; row += 4) {
+    const T* xr = x + row * D;
+    const T* gr = dy + row * D;
+    const float mu = mean[row], rs = rstd[row];
+    float xh[kLnMaxPerLane], g[kLnMaxPerLane];
+    float s1 = 0, s2 = 0;
+#pragma unroll
+    for (int q = 0; q < kLnMaxPerLane; ++q) {
+      const int e = lane + q * 64;
+      if (e < D) {
+        xh[q] = (tri_load(xr, e) - mu) * rs;
+        const float d = tri_load(gr, e);
+        ag[q] += d * xh[q];
+        ab[q] += d;
+        g[q] = gamma ? d * tri_load(gamma, e) : d;
+        s1 += g[q];
+        s2 += g[q] * xh[q];
+      } else {
+        xh[q] = g[q] = 0.f;
+      }
+    }
+    s1 = wave_sum(s1) / D;
+    s2 = wave_sum(s2) / D;
+    T* dr = dx + row * D;
+#pragma unroll
+    for (int q = 0; q < kLnMaxPerLane; ++q) {
+      const int e = lane + q * 64;
+      if (e < D) tri_store(dr, e, rs * (g[q] - s1 - xh[q] * s2));
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < kLnMaxPerLane; ++q) {
+    const int e = lane + q * 64;
+    if (e < D) {
+      sred[(wave * 2 + 0) * D + e] = ag[q];
+      sred[(wave * 2 + 1) * D + e] = ab[q];
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 2 * D; e += 256) {
+    const int which = e / D, d = e - which * D;
+    float s = 0;
+    for (int w = 0; w < 4; ++w) s += sred[(w * 2 + which) * D + d];
+    part[(static_cast<int64_t>(which) * gridDim.x + blockIdx.x) * D + d] = s;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// gate: out[r][c] = sigmoid(u + bu) * (v + bv) * mask;  biases and mask are indexed by row (axis 0) or column (axis 1)
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) gate_fwd_kernel(const float* __restrict__ u, const float* __restrict__ v, const T* __restrict__ bu,
+                                                       const T* __restrict__ bv, int bias_axis, const T* __restrict__ mask, int mask_axis,
+                                                       T* __restrict__ out, int64_t R, int64_t Ccols) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= R * Ccols) return;
+  const int64_t r = tid / Ccols, cc = tid - r * Ccols;
+  const int64_t ib = bias_axis == 0 ? r : cc;
+  const float uu = u[tid] + (bu ? tri_load(bu, ib) : 0.f);
+  const float vv = v[tid] + (bv ? tri_load(bv, ib) : 0.f);
+  float o = vv / (1.0f + __expf(-uu));
+  if (mask) o *= tri_load(mask, mask_axis == 0 ? r : cc);
+  tri_store(out, tid, o);
+}
+
+// du = dout * mask * (v + bv) * s * (1 - s),  dv = dout * mask * s,  s = sigmoid(u + bu)
+template <typename T>
+__global__ void __launch_bounds__(256) gate_bwd_kernel(const T* __restrict__ dout, const float* __restrict__ u, const float* __restrict__ v,
+                                                       const T* __restrict__ bu, const T* __restrict__ bv, int bias_axis,
+                                                       const T* __restrict__ mask, int mask_axis, T* __restrict__ du, T* __restrict__ dv,
+                                                       int64_t R, int64_t Ccols) {
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tid >= R * Ccols) return;
+  const int64_t r = tid / Ccols, cc = tid - r * Ccols;
+  const int64_t ib = bias_axis == 0 ? r : cc;
+  const float uu = u[tid] + (bu ? tri_load(bu, ib) : 0.f);
+  const float vv = v[tid] + (bv ? tri_load(bv, ib) : 0.f);
+  const float s = 1.0f / (1.0f + __expf(-uu));
+  float d = tri_load(dout, tid);
+  if (mask) d *= tri_load(mask, mask_axis == 0 ? r : cc);
+  tri_store(du, tid, d * vv * s * (1.0f - s));
+  tri_store(dv, tid, d * s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// reductions of an (R x C) array: sum over columns -> [R] (one wavefront per row);
+// sum over rows -> [C] (two stages through per-block partials)
+// ------------------------------------------------------------------------------------------------
+template <typename TI>
+__global__ void __launch_bounds__(256) sum_cols_kernel(const TI* __restrict__ in, float* __restrict__ out, int64_t R, int64_t Ccols) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= R) return;
+  float s = 0;
+  for (int64_t cc = lane; cc < Ccols; cc += 64) s += tri_load(in, row * Ccols + cc);
+  s = wave_sum(s);
+  if (lane == 0) out[row] = s;
+}
+
+template <typename TI>
+__global__ void __launch_bounds__(256) sum_rows_partial_kernel(const TI* __restrict__ in, float* __restrict__ part, int64_t R, int64_t Ccols,
+                                                               int64_t rows_per_block) {
+  const int64_t cc = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (cc >= Ccols) return;
+  const int64_t r0 = blockIdx.y * rows_per_block, r1 = min(r0 + rows_per_block, R);
+  float s = 0;
+  for (int64_t r = r0; r < r1; ++r) s += tri_load(in, r * Ccols + cc);
+  part[static_cast<int64_t>(blockIdx.y) * Ccols + cc] = s;
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(256) fold_partials_kernel(const float* __restrict__ part, TO* __restrict__ out, int64_t nparts, int64_t n,
+                                                            int accumulate) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = 0;
+  for (int64_t p = 0; p < nparts; ++p) s += part[p * n + i];
+  if (accumulate) s += tri_load(out, i);
+  tri_store(out, i, s);
+}
+
+static bool is_io(int dt) { return dt == CUEQ_F32 || dt == CUEQ_BF16; }
+
+}  // namespace cueq
+
+using namespace cueq;
+
+#define TRI_DISPATCH(dt, CALL_F32, CALL_BF16)      \
+  do {                                             \
+    if ((dt) == CUEQ_F32) { CALL_F32; } else { CALL_BF16; } \
+  } while (0)
+
+extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                            int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
+                            int64_t batch, double alpha, int32_t accumulate, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm_nt: dtypes must be float32 or bfloat16");
+  CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, CUEQ_ERR_INVALID, "gemm_nt: negative extent");
+  if (M == 0 || N == 0 || batch == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(A && B && C, CUEQ_ERR_INVALID, "gemm_nt: null operand");
+  CUEQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch < 65536, CUEQ_ERR_TOO_LARGE, "gemm_nt: extent too large");
+  const int epv = in_dtype == CUEQ_F32 ? 4 : 8;
+  const bool aligned = K % epv == 0 && lda % epv == 0 && ldb % epv == 0 && stride_a % epv == 0 && stride_b % epv == 0 &&
+                       reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 && K > 0;
+  const float al = static_cast<float>(alpha);
+  const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
+  if (aligned) {
+    const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(batch));
+    CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm_nt: too many row tiles (M <= 8388480)");
+    KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
+#define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_nt_kernel<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate)
+    if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_LAUNCH(float, float);
+    else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t);
+    else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float);
+    else GEMM_LAUNCH(uint16_t, uint16_t);
+#undef GEMM_LAUNCH
+  } else {
+    const int64_t total = M * N;
+    CUEQ_REQUIRE((total + 255) / 256 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gemm_nt: output too large for the unaligned path");
+    const dim3 grid(static_cast<unsigned>((total + 255) / 256), 1, static_cast<unsigned>(batch));
+    KernelTimer timer("gemm_nt_simple", stream);
+#define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_nt_simple<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate)
+    if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_LAUNCH(float, float);
+    else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t);
+    else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float);
+    else GEMM_LAUNCH(uint16_t, uint16_t);
+#undef GEMM_LAUNCH
+  }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_t cols, const void* in, void* out, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "transpose: dtype must be float32 or bfloat16");
+  if (batch <= 0 || rows <= 0 || cols <= 0) return CUEQ_OK;
+  CUEQ_REQUIRE(in && out, CUEQ_ERR_INVALID, "transpose: null operand");
+  const int64_t gy = (rows + 31) / 32, gx = (cols + 31) / 32;
+  CUEQ_REQUIRE(gy < 65536 && batch < 65536 && gx < (1ll << 31), CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
+  const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy), static_cast<unsigned>(batch));
+  KernelTimer timer("transpose", stream);
+  TRI_DISPATCH(dtype,
+               hipLaunchKernelGGL(transpose_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), static_cast<float*>(out), static_cast<int>(rows), static_cast<int>(cols)),
+               hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols)));
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_layer_norm_fwd(int32_t dtype, int64_t rows, int64_t D, const void* x, const void* gamma, const void* beta, double eps,
+                                   void* y, float* mean, float* rstd, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "layer_norm: dtype must be float32 or bfloat16");
+  CUEQ_REQUIRE(D > 0 && D <= 64 * kLnMaxPerLane, CUEQ_ERR_UNSUPPORTED, "layer_norm: hidden size must be in [1, %d]", 64 * kLnMaxPerLane);
+  if (rows <= 0) return CUEQ_OK;
+  CUEQ_REQUIRE(x && y && mean && rstd, CUEQ_ERR_INVALID, "layer_norm: null operand");
+  CUEQ_REQUIRE((rows + 3) / 4 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "layer_norm: too many rows");
+  const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
+  KernelTimer timer("layer_norm_fwd", stream);
+  TRI_DISPATCH(dtype,
+               hipLaunchKernelGGL(ln_fwd_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), static_cast<const float*>(gamma), static_cast<const float*>(beta), static_cast<float*>(y), mean, rstd, rows, static_cast<int>(D), static_cast<float>(eps)),
+               hipLaunchKernelGGL(ln_fwd_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, rows, static_cast<int>(D), static_cast<float>(eps)));
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+static int64_t ln_bwd_blocks(int64_t rows) {
+  int64_t nb = static_cast<int64_t>(device_cus()) * 4;
+  const int64_t most = (rows + 15) / 16;
+  if (nb > most) nb = most;
+  return nb < 1 ? 1 : nb;
+}
+
+extern "C" int64_t cueq_layer_norm_bwd_workspace(int64_t rows, int64_t D) { return ln_bwd_blocks(rows) * 2 * D * static_cast<int64_t>(sizeof(float)); }
+
+// dgamma / dbeta (float32, length D) may be null; workspace as sized by cueq_layer_norm_bwd_workspace.
+extern "C" int cueq_layer_norm_bwd(int32_t dtype, int64_t rows, int64_t D, const void* dy, const void* x, const float* mean, const float* rstd,
+                                   const void* gamma, void* dx, float* dgamma, float* dbeta, void* workspace, int64_t workspace_bytes,
+                                   void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "layer_norm: dtype must be float32 or bfloat16");
+  CUEQ_REQUIRE(D > 0 && D <= 64 * kLnMaxPerLane, CUEQ_ERR_UNSUPPORTED, "layer_norm: hidden size must be in [1, %d]", 64 * kLnMaxPerLane);
+  const int64_t nb = ln_bwd_blocks(rows);
+  if (rows <= 0) {
+    if (dgamma) CUEQ_CHECK_HIP(hipMemsetAsync(dgamma, 0, D * sizeof(float), stream));
+    if (dbeta) CUEQ_CHECK_HIP(hipMemsetAsync(dbeta, 0, D * sizeof(float), stream));
+    return CUEQ_OK;
+  }
+  CUEQ_REQUIRE(dy && x && mean && rstd && dx, CUEQ_ERR_INVALID, "layer_norm: null operand");
+  CUEQ_REQUIRE(workspace && workspace_bytes >= cueq_layer_norm_bwd_workspace(rows, D), CUEQ_ERR_INVALID, "layer_norm: workspace too small");
+  float* part = static_cast<float*>(workspace);
+  const int rpb = static_cast<int>((rows + nb - 1) / nb);
+  const size_t sh = 4 * 2 * D * sizeof(float);
+  {
+    KernelTimer timer("layer_norm_bwd", stream);
+    TRI_DISPATCH(dtype,
+                 hipLaunchKernelGGL(ln_bwd_kernel<float>, dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const float*>(dy), static_cast<const float*>(x), mean, rstd, static_cast<const float*>(gamma), static_cast<float*>(dx), part, rows, static_cast<int>(D), rpb),
+                 hipLaunchKernelGGL(ln_bwd_kernel<uint16_t>, dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const uint16_t*>(dy), static_cast<const uint16_t*>(x), mean, rstd, static_cast<const uint16_t*>(gamma), static_cast<uint16_t*>(dx), part, rows, static_cast<int>(D), rpb));
+  }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  const unsigned g = static_cast<unsigned>((D + 255) / 256);
+  if (dgamma) hipLaunchKernelGGL(fold_partials_kernel<float>, dim3(g), dim3(256), 0, stream, part, dgamma, nb, D, 0);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  if (dbeta) hipLaunchKernelGGL(fold_partials_kernel<float>, dim3(g), dim3(256), 0, stream, part + nb * D, dbeta, nb, D, 0);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_gate_fwd(int32_t dtype, int64_t rows, int64_t cols, const float* u, const float* v, const void* bias_u, const void* bias_v,
+                             int32_t bias_axis, const void* mask, int32_t mask_axis, void* out, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "gate: dtype must be float32 or bfloat16");
+  const int64_t n = rows * cols;
+  if (n <= 0) return CUEQ_OK;
+  CUEQ_REQUIRE(u && v && out, CUEQ_ERR_INVALID, "gate: null operand");
+  CUEQ_REQUIRE((n + 255) / 256 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gate: too many elements");
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  KernelTimer timer("gate_fwd", stream);
+  TRI_DISPATCH(dtype,
+               hipLaunchKernelGGL(gate_fwd_kernel<float>, grid, dim3(256), 0, stream, u, v, static_cast<const float*>(bias_u), static_cast<const float*>(bias_v), bias_axis, static_cast<const float*>(mask), mask_axis, static_cast<float*>(out), rows, cols),
+               hipLaunchKernelGGL(gate_fwd_kernel<uint16_t>, grid, dim3(256), 0, stream, u, v, static_cast<const uint16_t*>(bias_u), static_cast<const uint16_t*>(bias_v), bias_axis, static_cast<const uint16_t*>(mask), mask_axis, static_cast<uint16_t*>(out), rows, cols));
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_gate_bwd(int32_t dtype, int64_t rows, int64_t cols, const void* dout, const float* u, const float* v, const void* bias_u,
+                             const void* bias_v, int32_t bias_axis, const void* mask, int32_t mask_axis, void* du, void* dv, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "gate: dtype must be float32 or bfloat16");
+  const int64_t n = rows * cols;
+  if (n <= 0) return CUEQ_OK;
+  CUEQ_REQUIRE(dout && u && v && du && dv, CUEQ_ERR_INVALID, "gate: null operand");
+  CUEQ_REQUIRE((n + 255) / 256 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gate: too many elements");
+  const dim3 grid(static_cast<unsigned>((n + 255) / 256));
+  KernelTimer timer("gate_bwd", stream);
+  TRI_DISPATCH(dtype,
+               hipLaunchKernelGGL(gate_bwd_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(dout), u, v, static_cast<const float*>(bias_u), static_cast<const float*>(bias_v), bias_axis, static_cast<const float*>(mask), mask_axis, static_cast<float*>(du), static_cast<float*>(dv), rows, cols),
+               hipLaunchKernelGGL(gate_bwd_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(dout), u, v, static_cast<const uint16_t*>(bias_u), static_cast<const uint16_t*>(bias_v), bias_axis, static_cast<const uint16_t*>(mask), mask_axis, static_cast<uint16_t*>(du), static_cast<uint16_t*>(dv), rows, cols));
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+// out[r] = sum_c in[r][c]   (float32 result)
+extern "C" int cueq_sum_cols(int32_t dtype, int64_t rows, int64_t cols, const void* in, float* out, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "sum_cols: dtype must be float32 or bfloat16");
+  if (rows <= 0) return CUEQ_OK;
+  CUEQ_REQUIRE(in && out, CUEQ_ERR_INVALID, "sum_cols: null operand");
+  const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
+  TRI_DISPATCH(dtype,
+               hipLaunchKernelGGL(sum_cols_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), out, rows, cols),
+               hipLaunchKernelGGL(sum_cols_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), out, rows, cols));
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+static int64_t sum_rows_blocks(int64_t rows) {
+  int64_t nb = (rows + 255) / 256;
+  if (nb > 1024) nb = 1024;
+  return nb < 1 ? 1 : nb;
+}
+
+extern "C" int64_t cueq_sum_rows_workspace(int64_t rows, int64_t cols) { return sum_rows_blocks(rows) * cols * static_cast<int64_t>(sizeof(float)); }
+
+// out[c] = sum_r in[r][c]   (float32 result, deterministic two-stage reduction)
+extern "C" int cueq_sum_rows(int32_t dtype, int64_t rows, int64_t cols, const void* in, float* out, void* workspace, int64_t workspace_bytes,
+                             void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "sum_rows: dtype must be float32 or bfloat16");
+  if (cols <= 0) return CUEQ_OK;
+  CUEQ_REQUIRE(out, CUEQ_ERR_INVALID, "sum_rows: null output");
+  if (rows <= 0) {
+    CUEQ_CHECK_HIP(hipMemsetAsync(out, 0, cols * sizeof(float), stream));
+    return CUEQ_OK;
+  }
+  CUEQ_REQUIRE(in && workspace && workspace_bytes >= cueq_sum_rows_workspace(rows, cols), CUEQ_ERR_INVALID, "sum_rows: workspace too small");
+  const int64_t nb = sum_rows_blocks(rows);
+  const int64_t rpb = (rows + nb - 1) / nb;
+  float* part = static_cast<float*>(workspace);
+  const dim3 grid(static_cast<unsigned>((cols + 255) / 256), static_cast<unsigned>(nb));
+  TRI_DISPATCH(dtype,
+               hipLaunchKernelGGL(sum_rows_partial_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), part, rows, cols, rpb),
+               hipLaunchKernelGGL(sum_rows_partial_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), part, rows, cols, rpb));
+  CUEQ_CHECK_HIP(hipGetLastError());
+  hipLaunchKernelGGL(fold_partials_kernel<float>, dim3(static_cast<unsigned>((cols + 255) / 256)), dim3(256), 0, stream, part, out, nb, cols, 0);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}

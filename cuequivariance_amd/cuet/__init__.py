@@ -4,6 +4,7 @@ from .transpose import TransposeSegments, TransposeIrrepsLayout
 from .segmented_polynomial import SegmentedPolynomial
 from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction
 from .uniform_1d import uniform_1d
+from .triangle import triangle_multiplicative_update, TriMulPrecision
 
 __all__ = [
     "TransposeSegments",
@@ -14,4 +15,6 @@ __all__ = [
     "Linear",
     "SymmetricContraction",
     "uniform_1d",
+    "triangle_multiplicative_update",
+    "TriMulPrecision",
 ]

@@ -1,0 +1,382 @@
+"""Triangle multiplicative update (pair-representation update of AlphaFold-style models) on HIP kernels.
+
+``triangle_multiplicative_update`` keeps the signature, defaults and error behaviour of
+``cuequivariance_torch/cuequivariance_torch/primitives/triangle.py:138-262``; the computation is the one the
+reference states in the open
+``cuequivariance_jax/cuequivariance_jax/triangle/_triangle_multiplicative_update.py:371-417``::
+
+    xh  = LayerNorm(x; norm_in)                                            (B, N, N, D)
+    ab  = sigmoid(xh G_in^T + b) * (xh P_in^T + b) * mask, stored (2D, B, N, N);  a, b = split(ab)
+    t   = einsum("dbik,dbjk->dbij", a, b)   (outgoing)   /  einsum("dbki,dbkj->dbij", a, b)   (incoming)
+    y   = LayerNorm over d of t, stored (B, N, N, D)
+    out = sigmoid(xh G_out^T + b) * (y P_out^T + b)       -- the output gate reads the normalised input xh
+
+Every stage is a HIP kernel reached through the C ABI (``cueq_gemm_nt``, ``cueq_layer_norm_*``, ``cueq_gate_*``,
+``cueq_transpose``, ``cueq_sum_*``); torch only owns the buffers.  Inputs float32 or bfloat16, fp32 accumulation;
+intermediate tensors are kept in the input dtype like the reference does, the projection accumulators in float32.
+"""
+
+from __future__ import annotations
+
+import enum
+import math
+from typing import Optional
+
+import torch
+
+from .. import _lib
+
+__all__ = ["triangle_multiplicative_update", "TriMulPrecision"]
+
+
+class TriMulPrecision(enum.IntEnum):
+    """Matrix-multiplication precision request (reference ``primitives/triangle.py:24-31``).  The MFMA kernels
+    here compute float32 inputs in IEEE float32 and bfloat16 inputs with float32 accumulation whatever is asked."""
+
+    NONE = -1
+    DEFAULT = 0
+    TF32 = 1
+    TF32x3 = 2
+    IEEE = 3
+
+
+_CODE = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+# ---------------------------------------------------------------------------------------------
+# thin wrappers over the C ABI (shapes checked here, before any launch)
+# ---------------------------------------------------------------------------------------------
+def gemm_nt(A: torch.Tensor, B: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
+            accumulate: bool = False, alpha: float = 1.0) -> torch.Tensor:
+    """``C[b] = alpha * A[b] @ B[b]^T (+ C[b])`` for ``A (batch, M, K)``, ``B (batch, N, K)`` (or 2-D, batch 1)."""
+    squeeze = A.dim() == 2
+    if squeeze:
+        A, B = A.unsqueeze(0), B.unsqueeze(0)
+    assert A.dim() == 3 and B.dim() == 3 and A.shape[0] == B.shape[0] and A.shape[2] == B.shape[2], (A.shape, B.shape)
+    assert A.dtype == B.dtype and A.stride(2) == 1 and B.stride(2) == 1
+    batch, M, K = A.shape
+    N = B.shape[1]
+    if out is None:
+        assert not accumulate
+        out = torch.empty(batch, M, N, dtype=out_dtype, device=A.device)
+    else:
+        out = out.view(batch, M, N)
+        assert out.dtype == out_dtype and out.is_contiguous()
+    _lib.check(
+        _lib.load().cueq_gemm_nt(
+            _CODE[A.dtype], _CODE[out_dtype], M, N, K, A.data_ptr(), A.stride(1), A.stride(0) if batch > 1 else 0,
+            B.data_ptr(), B.stride(1), B.stride(0) if batch > 1 else 0, out.data_ptr(), N, M * N, batch, float(alpha),
+            int(accumulate), _stream(A),
+        ),
+        "cueq_gemm_nt",
+    )
+    return out[0] if squeeze else out
+
+
+def transpose(x: torch.Tensor) -> torch.Tensor:
+    """Swap the last two axes of a contiguous 2-D or 3-D tensor into a new contiguous tensor."""
+    assert x.is_contiguous() and x.dim() in (2, 3)
+    batch = x.shape[0] if x.dim() == 3 else 1
+    R, Cc = x.shape[-2], x.shape[-1]
+    out = torch.empty(x.shape[:-2] + (Cc, R), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.load().cueq_transpose(_CODE[x.dtype], batch, R, Cc, x.data_ptr(), out.data_ptr(), _stream(x)), "cueq_transpose")
+    return out
+
+
+def layer_norm_fwd(x: torch.Tensor, gamma, beta, eps: float):
+    rows, D = x.shape
+    y = torch.empty_like(x)
+    mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+    _lib.check(
+        _lib.load().cueq_layer_norm_fwd(_CODE[x.dtype], rows, D, x.data_ptr(), _ptr(gamma), _ptr(beta), float(eps), y.data_ptr(),
+                                        mean.data_ptr(), rstd.data_ptr(), _stream(x)),
+        "cueq_layer_norm_fwd",
+    )
+    return y, mean, rstd
+
+
+def layer_norm_bwd(dy: torch.Tensor, x: torch.Tensor, mean, rstd, gamma, need_affine: bool):
+    rows, D = x.shape
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    dgamma = torch.empty(D, dtype=torch.float32, device=x.device) if need_affine else None
+    dbeta = torch.empty(D, dtype=torch.float32, device=x.device) if need_affine else None
+    ws_bytes = lib.cueq_layer_norm_bwd_workspace(rows, D)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    _lib.check(
+        lib.cueq_layer_norm_bwd(_CODE[x.dtype], rows, D, dy.data_ptr(), x.data_ptr(), mean.data_ptr(), rstd.data_ptr(), _ptr(gamma),
+                                dx.data_ptr(), _ptr(dgamma), _ptr(dbeta), ws.data_ptr(), ws_bytes, _stream(x)),
+        "cueq_layer_norm_bwd",
+    )
+    return dx, dgamma, dbeta
+
+
+def gate_fwd(u, v, bias_u, bias_v, bias_axis: int, mask, mask_axis: int, dtype) -> torch.Tensor:
+    rows, cols = u.shape
+    out = torch.empty(rows, cols, dtype=dtype, device=u.device)
+    _lib.check(
+        _lib.load().cueq_gate_fwd(_CODE[dtype], rows, cols, u.data_ptr(), v.data_ptr(), _ptr(bias_u), _ptr(bias_v), bias_axis,
+                                  _ptr(mask), mask_axis, out.data_ptr(), _stream(u)),
+        "cueq_gate_fwd",
+    )
+    return out
+
+
+def gate_bwd(dout, u, v, bias_u, bias_v, bias_axis: int, mask, mask_axis: int):
+    rows, cols = u.shape
+    du, dv = torch.empty_like(dout), torch.empty_like(dout)
+    _lib.check(
+        _lib.load().cueq_gate_bwd(_CODE[dout.dtype], rows, cols, dout.data_ptr(), u.data_ptr(), v.data_ptr(), _ptr(bias_u),
+                                  _ptr(bias_v), bias_axis, _ptr(mask), mask_axis, du.data_ptr(), dv.data_ptr(), _stream(u)),
+        "cueq_gate_bwd",
+    )
+    return du, dv
+
+
+def sum_cols(x: torch.Tensor) -> torch.Tensor:
+    rows, cols = x.shape
+    out = torch.empty(rows, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().cueq_sum_cols(_CODE[x.dtype], rows, cols, x.data_ptr(), out.data_ptr(), _stream(x)), "cueq_sum_cols")
+    return out
+
+
+def sum_rows(x: torch.Tensor) -> torch.Tensor:
+    rows, cols = x.shape
+    lib = _lib.load()
+    out = torch.empty(cols, dtype=torch.float32, device=x.device)
+    ws_bytes = lib.cueq_sum_rows_workspace(rows, cols)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    _lib.check(lib.cueq_sum_rows(_CODE[x.dtype], rows, cols, x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, _stream(x)), "cueq_sum_rows")
+    return out
+
+
+def _split_k_chunks(K: int, align: int) -> int:
+    """Number of equal chunks (each a multiple of ``align``) to split a long contraction into."""
+    for n in range(min(512, max(1, K // 512)), 1, -1):
+        if K % n == 0 and (K // n) % align == 0:
+            return n
+    return 1
+
+
+def gemm_long_k(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """``A (P, K) @ B (Q, K)^T`` in float32 for a very long ``K``: equal k-chunks as a batched GEMM, then an ordered
+    sum of the partial products (no atomics)."""
+    P, K = A.shape
+    Q = B.shape[0]
+    n = _split_k_chunks(K, 8 if A.dtype == torch.bfloat16 else 4)
+    if n == 1:
+        return gemm_nt(A, B, torch.float32)
+    ck = K // n
+    Ab = A.as_strided((n, P, ck), (ck, A.stride(0), 1))
+    Bb = B.as_strided((n, Q, ck), (ck, B.stride(0), 1))
+    part = gemm_nt(Ab, Bb, torch.float32)
+    return sum_rows(part.view(n, P * Q)).view(P, Q)
+
+
+# ---------------------------------------------------------------------------------------------
+# autograd
+# ---------------------------------------------------------------------------------------------
+class _TriMul(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, mask, nin_w, nin_b, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, nout_b, p_out_w, p_out_b, g_out_w, g_out_b,
+                outgoing: bool, eps: float):
+        T = x.dtype
+        Bsz, N, _, D = x.shape
+        M = Bsz * N * N
+        Do = p_out_w.shape[0]
+        x2 = x.reshape(M, D)
+        xh, mean1, rstd1 = layer_norm_fwd(x2, nin_w, nin_b, eps)
+        u1 = gemm_nt(g_in_w, xh, torch.float32)  # (2D, M): the "transposed output" of the reference comes for free
+        v1 = gemm_nt(p_in_w, xh, torch.float32)
+        mflat = None if mask is None else mask.reshape(M)
+        ab = gate_fwd(u1, v1, g_in_b, p_in_b, 0, mflat, 1, T)  # (2D, M) == (2D, B, N, N)
+        a = ab[:D].view(D * Bsz, N, N)
+        b = ab[D:].view(D * Bsz, N, N)
+        if outgoing:
+            t = gemm_nt(a, b, T)  # t[i, j] = sum_k a[i, k] b[j, k]
+        else:
+            t = gemm_nt(transpose(a), transpose(b), T)  # t[i, j] = sum_k a[k, i] b[k, j]
+        tT = transpose(t.view(D, M))  # (M, D)
+        y, mean2, rstd2 = layer_norm_fwd(tT, nout_w, nout_b, eps)
+        u2 = gemm_nt(xh, g_out_w, torch.float32)  # (M, Do)
+        v2 = gemm_nt(y, p_out_w, torch.float32)
+        out = gate_fwd(u2, v2, g_out_b, p_out_b, 1, None, 0, T)
+        ctx.save_for_backward(x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
+                              xh, mean1, rstd1, u1, v1, ab, tT, mean2, rstd2, y, u2, v2)
+        ctx.outgoing, ctx.dims = outgoing, (Bsz, N, D, Do)
+        ctx.has = (nin_w is not None, nin_b is not None, nout_w is not None, nout_b is not None)
+        return out.view(Bsz, N, N, Do)
+
+    @staticmethod
+    def backward(ctx, dout):
+        (x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
+         xh, mean1, rstd1, u1, v1, ab, tT, mean2, rstd2, y, u2, v2) = ctx.saved_tensors
+        Bsz, N, D, Do = ctx.dims
+        M = Bsz * N * N
+        T = x2.dtype
+        need = ctx.needs_input_grad
+        dout = dout.contiguous().view(M, Do).to(T)
+
+        # output gate
+        du2, dv2 = gate_bwd(dout, u2, v2, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
+        dxh = gemm_nt(du2, transpose(g_out_w), T)  # (M, D)
+        dy = gemm_nt(dv2, transpose(p_out_w), T)
+        xhT = transpose(xh)  # (D, M)
+        d_g_out_w = d_p_out_w = d_g_out_b = d_p_out_b = None
+        if need[12]:
+            d_g_out_w = gemm_long_k(transpose(du2), xhT).to(g_out_w.dtype)
+        if need[10]:
+            d_p_out_w = gemm_long_k(transpose(dv2), transpose(y)).to(p_out_w.dtype)
+        if g_out_b is not None and need[13]:
+            d_g_out_b = sum_rows(du2).to(g_out_b.dtype)
+        if p_out_b is not None and need[11]:
+            d_p_out_b = sum_rows(dv2).to(p_out_b.dtype)
+
+        # LayerNorm across d
+        affine_out = (ctx.has[2] and need[8]) or (ctx.has[3] and need[9])
+        dtT, d_nout_w, d_nout_b = layer_norm_bwd(dy, tT, mean2, rstd2, nout_w, affine_out)
+        dt = transpose(dtT).view(D * Bsz, N, N)  # (D, M) viewed per (d, b)
+
+        # triangular contraction
+        a = ab[:D].view(D * Bsz, N, N)
+        b = ab[D:].view(D * Bsz, N, N)
+        dab = torch.empty_like(ab)
+        da = dab[:D].view(D * Bsz, N, N)
+        db = dab[D:].view(D * Bsz, N, N)
+        if ctx.outgoing:  # t = a b^T
+            gemm_nt(dt, transpose(b), T, out=da)  # da[i, k] = sum_j dt[i, j] b[j, k]
+            gemm_nt(transpose(dt), transpose(a), T, out=db)  # db[j, k] = sum_i dt[i, j] a[i, k]
+        else:  # t = a^T b
+            gemm_nt(b, dt, T, out=da)  # da[k, i] = sum_j b[k, j] dt[i, j]
+            gemm_nt(a, transpose(dt), T, out=db)  # db[k, j] = sum_i a[k, i] dt[i, j]
+
+        # input gate and projections
+        du1, dv1 = gate_bwd(dab, u1, v1, g_in_b, p_in_b, 0, mflat, 1)  # (2D, M)
+        gemm_nt(transpose(du1), transpose(g_in_w), T, out=dxh, accumulate=True)
+        gemm_nt(transpose(dv1), transpose(p_in_w), T, out=dxh, accumulate=True)
+        d_g_in_w = d_p_in_w = d_g_in_b = d_p_in_b = None
+        if need[6]:
+            d_g_in_w = gemm_long_k(du1, xhT).to(g_in_w.dtype)
+        if need[4]:
+            d_p_in_w = gemm_long_k(dv1, xhT).to(p_in_w.dtype)
+        if g_in_b is not None and need[7]:
+            d_g_in_b = sum_cols(du1).to(g_in_b.dtype)
+        if p_in_b is not None and need[5]:
+            d_p_in_b = sum_cols(dv1).to(p_in_b.dtype)
+
+        # input LayerNorm
+        affine_in = (ctx.has[0] and need[2]) or (ctx.has[1] and need[3])
+        dx, d_nin_w, d_nin_b = layer_norm_bwd(dxh, x2, mean1, rstd1, nin_w, affine_in)
+        dx = dx.view(Bsz, N, N, D) if need[0] else None
+
+        def cast(g, like, have):
+            return g.to(like.dtype) if (g is not None and have) else None
+
+        return (dx, None, cast(d_nin_w, x2, ctx.has[0]), cast(d_nin_b, x2, ctx.has[1]), d_p_in_w, d_p_in_b, d_g_in_w, d_g_in_b,
+                cast(d_nout_w, x2, ctx.has[2]), cast(d_nout_b, x2, ctx.has[3]), d_p_out_w, d_p_out_b, d_g_out_w, d_g_out_b, None, None)
+
+
+def _lecun_normal(shape, device, dtype) -> torch.Tensor:
+    """Truncated normal with variance 1 / fan_in (the reference's default projection initialiser,
+    ``_triangle_multiplicative_update.py:60-96``)."""
+    w = torch.empty(shape, device=device, dtype=torch.float32)
+    std = math.sqrt(1.0 / shape[1]) / 0.87962566103423978
+    torch.nn.init.trunc_normal_(w, mean=0.0, std=std, a=-2.0 * std, b=2.0 * std)
+    return w.to(dtype)
+
+
+def triangle_multiplicative_update(
+    x: torch.Tensor,
+    direction: str = "outgoing",
+    mask: Optional[torch.Tensor] = None,
+    norm_in_weight: Optional[torch.Tensor] = None,
+    norm_in_bias: Optional[torch.Tensor] = None,
+    p_in_weight: Optional[torch.Tensor] = None,
+    p_in_bias: Optional[torch.Tensor] = None,
+    g_in_weight: Optional[torch.Tensor] = None,
+    g_in_bias: Optional[torch.Tensor] = None,
+    norm_out_weight: Optional[torch.Tensor] = None,
+    norm_out_bias: Optional[torch.Tensor] = None,
+    p_out_weight: Optional[torch.Tensor] = None,
+    p_out_bias: Optional[torch.Tensor] = None,
+    g_out_weight: Optional[torch.Tensor] = None,
+    g_out_bias: Optional[torch.Tensor] = None,
+    eps: float = 1e-5,
+    precision: Optional[TriMulPrecision] = None,
+) -> torch.Tensor:
+    """Triangle multiplicative update of a pair tensor ``x (..., N, N, D)``; see the module docstring.
+
+    ``mask (..., N, N)`` multiplies the gated projections; norm weights default to 1 / biases to 0, projection
+    biases to none; projection weights that are not given are drawn (truncated normal, variance ``1 / D``) at
+    every call, as a stand-in for the reference's initialiser - pass them for anything but a shape test.
+    ``D`` must be a multiple of 32 (reference ``primitives/triangle.py:207``).  Differentiable with respect to
+    ``x`` and every weight given.
+    """
+    if direction not in ("outgoing", "incoming"):
+        raise ValueError("direction must be either 'outgoing' or 'incoming'")
+    if precision is not None and not isinstance(precision, (TriMulPrecision, int)):
+        raise ValueError("precision must be a TriMulPrecision or None")
+    if x.dim() < 3:
+        raise ValueError("x must have shape (..., N, N, D)")
+    if x.dim() == 3:
+        x = x.unsqueeze(0)
+        if mask is not None and mask.dim() == 2:
+            mask = mask.unsqueeze(0)
+    lead = x.shape[:-3]
+    N, N2, D = x.shape[-3:]
+    if N != N2:
+        raise ValueError(f"x must be square in its two sequence dimensions, got {N} x {N2}")
+    if D % 32 != 0:
+        raise ValueError("hidden dimension must be a multiple of 32")
+    if not x.is_cuda:
+        raise ValueError("triangle_multiplicative_update runs on the GPU only: x is on " + str(x.device))
+    if x.dtype not in _CODE:
+        raise ValueError(f"x must be float32 or bfloat16, got {x.dtype}")
+    T, dev = x.dtype, x.device
+    if mask is not None and tuple(mask.shape) != tuple(lead) + (N, N):
+        raise ValueError(f"mask must have shape {tuple(lead) + (N, N)}, got {tuple(mask.shape)}")
+
+    def vec(t, n, name):
+        if t is None:
+            return None
+        if tuple(t.shape) != (n,):
+            raise ValueError(f"{name} must have shape ({n},), got {tuple(t.shape)}")
+        return t.to(T).contiguous()
+
+    def mat(t, shape, name):
+        if t is None:
+            with torch.no_grad():
+                return _lecun_normal(shape, dev, T)
+        if tuple(t.shape) != shape and not (shape[0] is None and t.dim() == 2 and t.shape[1] == shape[1]):
+            raise ValueError(f"{name} must have shape {shape}, got {tuple(t.shape)}")
+        return t.to(T).contiguous()
+
+    Do = D
+    if p_out_weight is not None:
+        Do = p_out_weight.shape[0]
+    elif g_out_weight is not None:
+        Do = g_out_weight.shape[0]
+    args = (
+        vec(norm_in_weight, D, "norm_in_weight"), vec(norm_in_bias, D, "norm_in_bias"),
+        mat(p_in_weight, (2 * D, D), "p_in_weight"), vec(p_in_bias, 2 * D, "p_in_bias"),
+        mat(g_in_weight, (2 * D, D), "g_in_weight"), vec(g_in_bias, 2 * D, "g_in_bias"),
+        vec(norm_out_weight, D, "norm_out_weight"), vec(norm_out_bias, D, "norm_out_bias"),
+        mat(p_out_weight, (Do, D), "p_out_weight"), vec(p_out_bias, Do, "p_out_bias"),
+        mat(g_out_weight, (Do, D), "g_out_weight"), vec(g_out_bias, Do, "g_out_bias"),
+    )
+    Bsz = 1
+    for s in lead:
+        Bsz *= s
+    xf = x.reshape(Bsz, N, N, D).contiguous()
+    mf = None if mask is None else mask.reshape(Bsz, N, N).to(T).contiguous()
+    out = _TriMul.apply(xf, mf, *args, direction == "outgoing", float(eps))
+    return out.view(tuple(lead) + (N, N, Do))

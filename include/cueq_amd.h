@@ -171,6 +171,55 @@ int cueq_seg_outer(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t l
 int cueq_seg_rowdot(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* G,
                     int64_t ldg, void* dS, int64_t lds, int64_t rows, const cueq_gemm_problem* problem, void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* triangle multiplicative update: the stages behind                           */
+/*   cuequivariance_torch/cuequivariance_torch/primitives/triangle.py:138-262   */
+/* (closed kernel; open algorithm cuequivariance_jax/cuequivariance_jax/triangle/  */
+/*  _triangle_multiplicative_update.py:371-417).  dtype arguments are CUEQ_F32 or  */
+/* CUEQ_BF16, arithmetic is fp32, all pointers are device pointers.                */
+/* ------------------------------------------------------------------------- */
+
+/* Batched C[b] = alpha * A[b] * B[b]^T (+ C[b]):  A is M x K (row stride lda), B is N x K (row stride ldb), both with the
+ * contraction index contiguous; C is M x N (row stride ldc); strides between batch items in elements.  MFMA path when
+ * K, lda, ldb and the batch strides are multiples of 16 bytes worth of elements, otherwise a plain kernel.
+ * Stands for the projections (_sigmoid_gated_dual_gemm.py:111-150) and the contraction
+ * einsum("dbik,dbjk->dbij") (_triangle_multiplicative_update.py:393-397). */
+int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                 int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
+                 int64_t batch, double alpha, int32_t accumulate, void* stream);
+
+/* out[b][c][r] = in[b][r][c] (layout changes "bijd<->dbij" of _layer_norm_transpose.py:162-227 and operand
+ * re-orientation for the incoming direction and the backward contractions). */
+int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_t cols, const void* in, void* out, void* stream);
+
+/* Row LayerNorm with biased variance, rstd = 1/sqrt(var + eps) (_layer_norm_transpose.py:196-209); gamma / beta may
+ * be NULL; mean and rstd (float32, one per row) are kept for the backward.  D <= 1024. */
+int cueq_layer_norm_fwd(int32_t dtype, int64_t rows, int64_t D, const void* x, const void* gamma, const void* beta,
+                        double eps, void* y, float* mean, float* rstd, void* stream);
+int64_t cueq_layer_norm_bwd_workspace(int64_t rows, int64_t D);
+/* dx from dy, the forward input x and the saved statistics; dgamma / dbeta (float32[D], may be NULL) are summed
+ * over rows without atomics through the workspace. */
+int cueq_layer_norm_bwd(int32_t dtype, int64_t rows, int64_t D, const void* dy, const void* x, const float* mean,
+                        const float* rstd, const void* gamma, void* dx, float* dgamma, float* dbeta, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+
+/* out = sigmoid(u + bias_u) * (v + bias_v) * mask on a rows x cols array (u, v float32 accumulators of the two
+ * projections); biases (may be NULL) are indexed by row (bias_axis 0) or column (1), the mask (may be NULL)
+ * likewise (_sigmoid_gated_dual_gemm.py:135-150).  cueq_gate_bwd returns the gradients of u and v
+ * (_sigmoid_gated_dual_gemm.py:153-218). */
+int cueq_gate_fwd(int32_t dtype, int64_t rows, int64_t cols, const float* u, const float* v, const void* bias_u,
+                  const void* bias_v, int32_t bias_axis, const void* mask, int32_t mask_axis, void* out, void* stream);
+int cueq_gate_bwd(int32_t dtype, int64_t rows, int64_t cols, const void* dout, const float* u, const float* v,
+                  const void* bias_u, const void* bias_v, int32_t bias_axis, const void* mask, int32_t mask_axis,
+                  void* du, void* dv, void* stream);
+
+/* Deterministic reductions of a rows x cols array into float32: over columns (one value per row) and over rows
+ * (one value per column; workspace of cueq_sum_rows_workspace bytes).  Used for bias and affine gradients. */
+int cueq_sum_cols(int32_t dtype, int64_t rows, int64_t cols, const void* in, float* out, void* stream);
+int64_t cueq_sum_rows_workspace(int64_t rows, int64_t cols);
+int cueq_sum_rows(int32_t dtype, int64_t rows, int64_t cols, const void* in, float* out, void* workspace,
+                  int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
