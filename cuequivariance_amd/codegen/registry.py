@@ -1,7 +1,7 @@
 """Descriptors for which specialised kernels are generated when the library is built.
 
-Each entry yields one translation unit in ``csrc/generated`` holding a forward kernel and a fused
-backward kernel (all three gradients).  Anything not listed runs on the table-driven kernels.
+Each entry yields one translation unit per math type in ``csrc/generated`` holding a forward kernel and a fused
+backward kernel.  Anything not listed runs on the table-driven kernels.
 """
 
 from __future__ import annotations
@@ -11,6 +11,7 @@ from pathlib import Path
 from .. import cue
 from ..tables import U1dTables
 from . import channelwise as cw
+from . import symmetric as sc
 
 GENERATED_DIR = Path(__file__).resolve().parent.parent / "csrc" / "generated"
 
@@ -18,6 +19,12 @@ GENERATED_DIR = Path(__file__).resolve().parent.parent / "csrc" / "generated"
 CHANNELWISE = [
     ("c128_l3", "128x0e+128x1o+128x2e+128x3o", "0e+1o+2e+3o", "0e+1o+2e+3o", {}),
     ("c32_l2", "32x0e+32x1o+32x2e", "0e+1o+2e", "0e+1o+2e", {}),
+]
+
+# (name, irreps_in, irreps_out, contraction degree)
+SYMMETRIC = [
+    ("s128_l3", "128x0e+128x1o+128x2e+128x3o", "128x0e+128x1o", 3),
+    ("s32_l2", "32x0e+32x1o+32x2e", "32x0e+32x1o", 3),
 ]
 
 MATH = (("float", 0), ("double", 1))
@@ -28,9 +35,29 @@ def channelwise_tables(irreps1: str, irreps2: str, filt) -> U1dTables:
     return U1dTables.from_polynomial(e.polynomial.flatten_coefficient_modes().squeeze_modes())
 
 
+def symmetric_polynomial(irreps_in: str, irreps_out: str, degree: int):
+    e = cue.descriptors.symmetric_contraction(cue.Irreps("O3", irreps_in), cue.Irreps("O3", irreps_out), range(1, degree + 1))
+    return e.polynomial.flatten_coefficient_modes().squeeze_modes()
+
+
+def _write(path: Path, src: str, written: list) -> None:
+    if not path.exists() or path.read_text() != src:
+        path.write_text(src)
+    written.append(path)
+
+
 def generate(verbose: bool = False) -> list[Path]:
     GENERATED_DIR.mkdir(parents=True, exist_ok=True)
     written = []
+    for name, irreps_in, irreps_out, degree in SYMMETRIC:
+        poly = symmetric_polynomial(irreps_in, irreps_out, degree)
+        t = U1dTables.from_polynomial(poly)
+        st = sc.analyze(poly)
+        for T, code in MATH:
+            bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
+            _write(GENERATED_DIR / f"sc_{name}_{T}.hip", sc.emit_unit(st, T, name, t.content_hash(code), bwd), written)
+            if verbose:
+                print(f"generated sc_{name}_{T}.hip: {len(st.terms)} folded terms")
     for name, ir1, ir2, filt, tuning in CHANNELWISE:
         t = channelwise_tables(ir1, ir2, filt)
         assert t.operations == (0, 1, 2, 3) and t.buffer_dim == (1, 1, 0, 1)

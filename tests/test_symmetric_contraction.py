@@ -203,3 +203,54 @@ def test_module_forward_signature_and_layouts(device):
     torch.testing.assert_close(to_mul_ir(ya), yb, atol=1e-5, rtol=1e-5)
     with pytest.raises(ValueError):
         cuet.SymmetricContraction(cue.Irreps("O3", "8x0e+4x1o"), irreps_out, 2, 3, layout=cue.ir_mul)
+
+
+@pytest.mark.gpu
+def test_generated_kernels_full_size(device, monkeypatch):
+    """cfg3 shape (50 000 nodes, 128 channels, l <= 3 -> 0e+1o, 10 element types): the descriptor-specialised kernels are
+    the ones running, repeat bit-identically (no atomics in the weight gradient), and agree with the table-driven
+    kernels on a slice; element types that never occur get a zero gradient; int64 and pre-sorted indices work."""
+    from cuequivariance_amd import cuet
+
+    m = cuet.SymmetricContraction(
+        cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "128x0e+128x1o"), 3, 10, layout=cue.ir_mul,
+        dtype=torch.float32, device=device,
+    )
+    plan = m.f.m._plan(torch.float32)
+    assert plan.specialised(device) and plan.backward_plan((True, True)).specialised(device)
+    assert plan.backward_plan((False, True)).specialised(device) and plan.backward_plan((True, False)).specialised(device)
+    Z = 50_000
+    gen = torch.Generator(device=device).manual_seed(0)
+    x = torch.randn(Z, 2048, device=device, generator=gen, requires_grad=True)
+    idx = torch.randint(0, 9, (Z,), device=device, generator=gen, dtype=torch.int32)  # type 9 never occurs
+    cot = torch.randn(Z, 512, device=device, generator=gen)
+
+    def step(xx, ii, cc):
+        out = m(xx, ii)
+        return [out] + list(torch.autograd.grad(out, [m.weight, xx], cc))
+
+    a, b = step(x, idx, cot), step(x, idx, cot)
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
+    assert torch.count_nonzero(a[1][9]) == 0 and torch.count_nonzero(a[1][3]) > 0
+    # int64 indices; sorted indices (identity permutation in the grouping)
+    c = step(x, idx.long(), cot)
+    assert torch.equal(a[0], c[0]) and torch.equal(a[2], c[2])
+    order = torch.sort(idx.long(), stable=True)[1]
+    d = step(x[order].detach().requires_grad_(True), idx[order].contiguous(), cot[order].contiguous())
+    assert torch.equal(d[0], a[0][order]) and torch.equal(d[2], a[2][order])
+    assert (d[1] - a[1]).abs().max().item() <= 1e-5 * a[1].abs().max().item()
+    # slice against the generic kernels
+    Zs = 2000
+    xs = x[:Zs].detach().requires_grad_(True)
+    got = step(xs, idx[:Zs].contiguous(), cot[:Zs].contiguous())
+    monkeypatch.setenv("CUEQ_FORCE_GENERIC", "1")
+    want = step(xs, idx[:Zs].contiguous(), cot[:Zs].contiguous())
+    for name, u, v in zip(("out", "dw", "dx"), got, want):
+        assert (u - v).abs().max().item() <= 5e-5 * v.abs().max().item(), name
+    # only the input gradient (frozen weights) and only the weight gradient
+    monkeypatch.delenv("CUEQ_FORCE_GENERIC")
+    out = m(xs, idx[:Zs].contiguous())
+    (gx,) = torch.autograd.grad(out, [xs], cot[:Zs].contiguous(), retain_graph=True)
+    (gw,) = torch.autograd.grad(out, [m.weight], cot[:Zs].contiguous())
+    assert torch.equal(gx, got[2]) and torch.equal(gw, got[1])
