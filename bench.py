@@ -93,12 +93,102 @@ def cpu_baseline(torch, cue, module, host, sample_edges: int, sample_nodes: int)
     }
 
 
+def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
+    """Secondary workloads (BASELINE.json configs[2..4]); same timing discipline as the headline line."""
+    wl = args.workload
+    if wl == "cfg3":
+        Z = 50_000
+        m = cuet.SymmetricContraction(cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "128x0e+128x1o"),
+                                      3, 10, layout=cue.ir_mul, dtype=torch.float32, device=dev)
+        g = torch.Generator(device=dev).manual_seed(0)
+        x = torch.randn(Z, 2048, device=dev, generator=g, requires_grad=True)
+        idx = torch.randint(0, 10, (Z,), device=dev, generator=g, dtype=torch.int32)
+        with torch.no_grad():
+            m.weight.mul_(1.0 / m.weight.shape[1] ** 0.5)
+        cot = torch.randn(Z, 512, device=dev, generator=g)
+
+        def step():
+            return torch.autograd.grad(m(x, idx), [m.weight, x], cot)
+
+        unit, units, dt = "nodes/s", Z, "f32"
+        # every distinct element once: fwd reads x and writes out; bwd reads x, g and writes dx (weights 10 x 3712 negligible)
+        alg = {"fwd": Z * (2048 + 512) * 4, "bwd": Z * (2048 + 512 + 2048) * 4}
+        bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
+        desc = ("configs[2]: symmetric contraction 128x(0e+1o+2e+3o) -> 128x(0e+1o), degree 3, 10 element types, "
+                "50000 nodes, int32 element index, fwd + bwd (dw, dx)")
+    elif wl == "cfg4":
+        Z = 200_000
+        dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+        irreps = cue.Irreps("O3", "128x0e+128x1o+128x2e")
+        m = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=False, method="fused_tp")
+        g = torch.Generator(device=dev).manual_seed(0)
+        x = torch.randn(Z, 1152, device=dev, generator=g).to(dtype).requires_grad_(True)
+        w = torch.randn(1, m.weight_numel, device=dev, generator=g).to(dtype).requires_grad_(True)
+        cot = torch.randn(Z, 1152, device=dev, generator=g).to(dtype)
+
+        def step():
+            return torch.autograd.grad(m(x, w), [w, x], cot)
+
+        unit, units, dt = "rows/s", Z, "bf16" if dtype == torch.bfloat16 else "f32"
+        f = 2 * Z * 128 * 128 * 9
+        alg = {"fwd": f, "bwd": 2 * f}
+        bound, pu = "mfma", "TFLOP/s"
+        peak = 2500.0 if dtype == torch.bfloat16 else 157.3
+        desc = "configs[3]: Linear 128x0e+128x1o+128x2e -> same, batch 200000, shared weights, fwd + bwd (dw, dx)"
+    else:
+        dtype = torch.float32 if args.dtype == "fp32" else torch.bfloat16
+        n, D = 512, 128
+        g = torch.Generator(device=dev).manual_seed(0)
+
+        def r(*shape, scale=1.0):
+            return (torch.randn(*shape, device=dev, generator=g) * scale).to(dtype)
+
+        x = r(1, n, n, D).requires_grad_(True)
+        kw = dict(mask=(torch.rand(1, n, n, device=dev, generator=g) < 0.9).to(dtype),
+                  norm_in_weight=torch.ones(D, device=dev, dtype=dtype), norm_in_bias=torch.zeros(D, device=dev, dtype=dtype),
+                  p_in_weight=r(2 * D, D, scale=D ** -0.5), g_in_weight=r(2 * D, D, scale=D ** -0.5),
+                  norm_out_weight=torch.ones(D, device=dev, dtype=dtype), norm_out_bias=torch.zeros(D, device=dev, dtype=dtype),
+                  p_out_weight=r(D, D, scale=D ** -0.5), g_out_weight=r(D, D, scale=D ** -0.5))
+        cot = r(1, n, n, D)
+
+        def step():
+            return torch.autograd.grad(cuet.triangle_multiplicative_update(x, "outgoing", **kw), [x], cot)
+
+        unit, units, dt = "pair rows/s", n * n, "bf16" if dtype == torch.bfloat16 else "f32"
+        f = 2 * n * n * D * 4 * D + 2 * D * n ** 3 + 2 * n * n * D * 2 * D  # projections in, contraction, projections out
+        alg = {"fwd": f, "bwd": 2 * f}
+        bound, pu = "mfma", "TFLOP/s"
+        peak = 2500.0 if dtype == torch.bfloat16 else 157.3
+        desc = "configs[4]: triangle multiplicative update, outgoing, z [1,512,512,128], mask Bernoulli(0.9), fwd + bwd w.r.t. z"
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.timing_begin()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = (time.perf_counter() - t0) / args.steps
+    kernels = {n_: {"launches": l, "avg_ms": t / max(l, 1), "ms_per_step": t / args.steps} for n_, (l, t) in _lib.timing_end().items()}
+    total = alg["fwd"] + alg["bwd"]
+    achieved = total / elapsed / (1e9 if bound == "hbm" else 1e12)
+    return {
+        "metric": f"{unit.split('/')[0]}/sec, {wl} fwd+bwd (secondary workload)", "value": units / elapsed, "unit": unit, "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dt, "data": "synthetic", "config": {"workload": desc},
+        "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": pu, "frac": achieved / peak, "traffic": None,
+                     "scope": "whole step: algorithmic bytes or flops of forward + backward over the step time"},
+        "kernels": kernels,
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--dtype", choices=["fp32", "fp64"], default="fp32")
+    ap.add_argument("--dtype", choices=["fp32", "fp64", "bf16"], default=None,
+                    help="cfg2: fp32 (default) or fp64; cfg3: fp32; cfg4: fp32 (default) or bf16; cfg5: bf16 (default) or fp32")
     ap.add_argument("--nodes", type=int, default=5000)
     ap.add_argument("--edges", type=int, default=100_000)
     ap.add_argument("--cpu-sample-edges", type=int, default=12000)
@@ -107,6 +197,9 @@ def main() -> int:
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--deterministic", action="store_true",
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
+    ap.add_argument("--workload", choices=["cfg2", "cfg3", "cfg4", "cfg5"], default="cfg2",
+                    help="cfg2 (default) is the headline metric; the others print a secondary line for the same "
+                         "library: cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg5 triangle update")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
@@ -132,7 +225,13 @@ def main() -> int:
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "copy", "bytes_read": n * 4, "bytes_written": n * 4, "launches": 5}))
         return 0
-    dtype = torch.float32 if args.dtype == "fp32" else torch.float64
+    if args.workload != "cfg2":
+        print(json.dumps(secondary(torch, cue, cuet, _lib, dev, args)))
+        return 0
+    if args.dtype == "bf16":
+        print("bench.py: cfg2 is measured in fp32 or fp64 (the uniform-1d math types)", file=sys.stderr)
+        return 2
+    dtype = torch.float64 if args.dtype == "fp64" else torch.float32
     N, E = args.nodes, args.edges
 
     m = cuet.ChannelWiseTensorProduct(

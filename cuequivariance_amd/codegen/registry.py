@@ -17,7 +17,8 @@ GENERATED_DIR = Path(__file__).resolve().parent.parent / "csrc" / "generated"
 
 # (name, irreps_in1, irreps_in2, filter, tuning)
 CHANNELWISE = [
-    ("c128_l3", "128x0e+128x1o+128x2e+128x3o", "0e+1o+2e+3o", "0e+1o+2e+3o", {}),
+    # float64 needs the whole register file of a SIMD lane (one wavefront per SIMD): with two, both kernels spill
+    ("c128_l3", "128x0e+128x1o+128x2e+128x3o", "0e+1o+2e+3o", "0e+1o+2e+3o", {"double": {"fwd_waves": 1, "bwd_waves": 1}}),
     ("c32_l2", "32x0e+32x1o+32x2e", "0e+1o+2e", "0e+1o+2e", {}),
 ]
 
