@@ -38,6 +38,8 @@ EXPORTED_SYMBOLS = (
     "cueq_seg_outer",
     "cueq_seg_rowdot",
     "cueq_gemm_nt",
+    "cueq_gemm_tn_items",
+    "cueq_gemm_tn",
     "cueq_transpose",
     "cueq_layer_norm_fwd",
     "cueq_layer_norm_bwd_workspace",
@@ -166,6 +168,10 @@ def load() -> C.CDLL:
         i32, i64, ptr, f64 = C.c_int32, C.c_int64, C.c_void_p, C.c_double
         lib.cueq_gemm_nt.argtypes = [i32, i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, ptr, i64, i64, i64, f64, i32, ptr]
         lib.cueq_gemm_nt.restype = C.c_int
+        lib.cueq_gemm_tn_items.argtypes = [i64, i32]
+        lib.cueq_gemm_tn_items.restype = i64
+        lib.cueq_gemm_tn.argtypes = [i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, i32, ptr, f64, ptr]
+        lib.cueq_gemm_tn.restype = C.c_int
         lib.cueq_transpose.argtypes = [i32, i64, i64, i64, ptr, ptr, ptr]
         lib.cueq_transpose.restype = C.c_int
         lib.cueq_layer_norm_fwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, f64, ptr, ptr, ptr, ptr]

@@ -148,6 +148,116 @@ __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, 
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Partial products of C (M x N) = sum_z A[z, :M]^T B[z, :N] over a long row range: item (chunk, part) of
+// grid.z covers rows [chunk * rows_per_chunk, ...) of the column blocks A + part * stride_a, B + part * stride_b
+// and writes alpha * partial to P[item] (float32, M x N).  The caller sums the items in order (no atomics).
+// Rows are staged through LDS as float32 (bf16 inputs are widened on the way), MFMA 32x32x2 f32.
+// ------------------------------------------------------------------------------------------------
+constexpr int kTnRows = 16;  // rows (contraction) per step
+
+__device__ __forceinline__ void tn_load8(const float* p, float* r) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w; r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+}
+__device__ __forceinline__ void tn_load8(const uint16_t* p, float* r) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    r[2 * e] = __uint_as_float(w[e] << 16);
+    r[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+  }
+}
+
+template <typename TI, bool VEC>
+__global__ void __launch_bounds__(256) gemm_tn_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA, const TI* __restrict__ B,
+                                                      int64_t ldb, int64_t sB, float* __restrict__ P, int M, int N, int64_t rows,
+                                                      int64_t rows_per_chunk, int nparts, float alpha) {
+  __shared__ __align__(16) float sa[kTnRows][kTile + 4];
+  __shared__ __align__(16) float sb[kTnRows][kTile + 4];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
+  const int64_t item = blockIdx.z;
+  const int64_t chunk = item / nparts;
+  const int part = static_cast<int>(item - chunk * nparts);
+  A += part * sA;
+  B += part * sB;
+  P += item * static_cast<int64_t>(M) * N;
+  const int64_t z_begin = chunk * rows_per_chunk;
+  const int64_t z_end = min(z_begin + rows_per_chunk, rows);
+
+  // staging: 16 rows x 128 columns per operand; a thread owns (row, 8 consecutive columns)
+  const int srow = tid >> 4, scol = (tid & 15) * 8;
+  float ra[8], rb[8];
+  auto load_step = [&](int64_t z) {
+    const int64_t zr = z + srow;
+    if constexpr (VEC) {  // M, N multiples of 8 and 16-byte aligned rows: whole vectors are in or out
+      if (zr < z_end && m0 + scol < M) tn_load8(A + zr * lda + m0 + scol, ra);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ra[e] = 0.f;
+      }
+      if (zr < z_end && n0 + scol < N) tn_load8(B + zr * ldb + n0 + scol, rb);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rb[e] = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const bool ok = zr < z_end;
+        ra[e] = (ok && m0 + scol + e < M) ? tri_load(A, zr * lda + m0 + scol + e) : 0.f;
+        rb[e] = (ok && n0 + scol + e < N) ? tri_load(B, zr * ldb + n0 + scol + e) : 0.f;
+      }
+    }
+  };
+  auto store_step = [&]() {
+#pragma unroll
+    for (int e = 0; e < 8; e += 4) {
+      *reinterpret_cast<float4*>(&sa[srow][scol + e]) = make_float4(ra[e], ra[e + 1], ra[e + 2], ra[e + 3]);
+      *reinterpret_cast<float4*>(&sb[srow][scol + e]) = make_float4(rb[e], rb[e + 1], rb[e + 2], rb[e + 3]);
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = floatx16{0};
+
+  if (z_begin < z_end) load_step(z_begin);
+  for (int64_t z = z_begin; z < z_end; z += kTnRows) {
+    __syncthreads();  // the previous step's reads are done
+    store_step();
+    __syncthreads();
+    if (z + kTnRows < z_end) load_step(z + kTnRows);
+#pragma unroll
+    for (int s = 0; s < kTnRows / 2; ++s) {
+      const int zr = h * (kTnRows / 2) + s;  // lane half h covers its own half of the rows
+      const float a0 = sa[zr][wm * 64 + c], a1 = sa[zr][wm * 64 + 32 + c];
+      const float b0 = sb[zr][wn * 64 + c], b1 = sb[zr][wn * 64 + 32 + c];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + c;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (row < M && col < N) P[static_cast<int64_t>(row) * N + col] = alpha * acc[i][j][v];
+      }
+    }
+}
+
 // any shape / alignment: one thread per output element
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(256) gemm_nt_simple(const TI* __restrict__ A, int64_t lda, int64_t sA, const TI* __restrict__ B,
@@ -418,6 +528,38 @@ extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int6
     else GEMM_LAUNCH(uint16_t, uint16_t);
 #undef GEMM_LAUNCH
   }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int64_t cueq_gemm_tn_items(int64_t rows, int32_t nparts) {
+  if (nparts < 1) nparts = 1;
+  int64_t chunks = (static_cast<int64_t>(device_cus()) * 2 + nparts - 1) / nparts;
+  const int64_t most = (rows + 4 * kTnRows - 1) / (4 * kTnRows);  // at least 64 rows per chunk
+  if (chunks > most) chunks = most;
+  if (chunks < 1) chunks = 1;
+  return chunks * nparts;
+}
+
+extern "C" int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows, const void* A, int64_t lda, int64_t stride_a,
+                            const void* B, int64_t ldb, int64_t stride_b, int32_t nparts, float* partials, double alpha, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(in_dtype), CUEQ_ERR_UNSUPPORTED, "gemm_tn: dtype must be float32 or bfloat16");
+  CUEQ_REQUIRE(M > 0 && N > 0 && rows >= 0 && nparts >= 1, CUEQ_ERR_INVALID, "gemm_tn: bad extents");
+  CUEQ_REQUIRE(A && B && partials, CUEQ_ERR_INVALID, "gemm_tn: null operand");
+  CUEQ_REQUIRE(M < (1ll << 20) && N < (1ll << 20), CUEQ_ERR_TOO_LARGE, "gemm_tn: result too large");
+  const int64_t items = cueq_gemm_tn_items(rows, nparts);
+  const int64_t chunks = items / nparts;
+  const int64_t rpc = rows == 0 ? 0 : (((rows + chunks - 1) / chunks + kTnRows - 1) / kTnRows) * kTnRows;
+  CUEQ_REQUIRE(items < 65536, CUEQ_ERR_TOO_LARGE, "gemm_tn: too many items");
+  const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(items));
+  const bool vec = M % 8 == 0 && N % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0;
+  KernelTimer timer("gemm_tn", stream);
+#define TN_LAUNCH(TI, V) hipLaunchKernelGGL((gemm_tn_kernel<TI, V>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, partials, static_cast<int>(M), static_cast<int>(N), rows, rpc, nparts, static_cast<float>(alpha))
+  if (in_dtype == CUEQ_F32) { if (vec) TN_LAUNCH(float, true); else TN_LAUNCH(float, false); }
+  else { if (vec) TN_LAUNCH(uint16_t, true); else TN_LAUNCH(uint16_t, false); }
+#undef TN_LAUNCH
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }

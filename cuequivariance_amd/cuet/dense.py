@@ -132,6 +132,51 @@ def _run_gemms(dtype, A, B, S, Cout, launches):
         )
 
 
+def _batched_groups(paths, a_key, c_key):
+    """Group paths that share the weight block and scale into launches whose operand / result column offsets advance
+    by constant strides: [(first path, count, stride of a, stride of c)]."""
+    by_block: Dict[tuple, list] = {}
+    for p in paths:
+        by_block.setdefault((p.w_off, p.K, p.N, p.coeff), []).append(p)
+    groups = []
+    for plist in by_block.values():
+        plist = sorted(plist, key=a_key)
+        n = len(plist)
+        da = a_key(plist[1]) - a_key(plist[0]) if n > 1 else 0
+        dc = c_key(plist[1]) - c_key(plist[0]) if n > 1 else 0
+        regular = n > 1 and da > 0 and dc > 0 and all(
+            a_key(plist[t + 1]) - a_key(plist[t]) == da and c_key(plist[t + 1]) - c_key(plist[t]) == dc for t in range(n - 1)
+        )
+        if regular:
+            groups.append((plist[0], n, da, dc))
+        else:
+            groups += [(q, 1, 0, 0) for q in plist]
+    return groups
+
+
+def _run_tiled(dtype, A, a_key, B_of, Cout, c_key, groups, Kdim, Ndim):
+    """``Cout[:, c : c + N] (+)= coeff * A[:, a : a + K] @ B^T`` per group through the 128 x 128 tiled MFMA kernel
+    (``cueq_gemm_nt``; ``B_of(path)`` gives the pointer of the ``N x K`` block)."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(A.device).cuda_stream
+    code = _DTYPE_CODE[dtype]
+    es = A.element_size()
+    written = set()
+    for p, count, da, dc in groups:
+        cols = tuple(c_key(p) + t * dc for t in range(count))
+        acc = 1 if any(c in written for c in cols) else 0
+        if acc and count > 1 and not all(c in written for c in cols):
+            raise NotImplementedError("fused_tp: irregular overlap of output segments")
+        written.update(cols)
+        _lib.check(
+            lib.cueq_gemm_nt(code, code, A.shape[0], Ndim(p), Kdim(p), A.data_ptr() + a_key(p) * es, A.stride(0), da,
+                             B_of(p), Kdim(p), 0, Cout.data_ptr() + c_key(p) * es, Cout.stride(0), dc, count, p.coeff, acc,
+                             stream),
+            "cueq_gemm_nt",
+        )
+    return written
+
+
 class _DenseFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, mod: "SegmentedPolynomialDense", w, x1, x2):
@@ -143,7 +188,14 @@ class _DenseFunction(torch.autograd.Function):
         x2d = x2.detach().contiguous() if x2 is not None else None
         if Z > 0:
             with torch.cuda.device(x1.device):
-                _run_gemms(dtype, x1d, wd, x2d, out, mod.tables(x1.device).fwd)
+                if mod.tiled(dtype, x1d, out):
+                    # out[:, k_seg] (+)= c * x1[:, i_seg] @ W_p: the kernel wants W_p^T (N x K, contraction contiguous)
+                    wt = mod.transposed_weights(wd)
+                    es = wd.element_size()
+                    _run_tiled(dtype, x1d, lambda p: p.a_off, lambda p: wt.data_ptr() + p.w_off * es, out, lambda p: p.c_off,
+                               mod.fwd_groups, lambda p: p.K, lambda p: p.N)
+                else:
+                    _run_gemms(dtype, x1d, wd, x2d, out, mod.tables(x1.device).fwd)
         ctx.mod = mod
         ctx.save_for_backward(w, x1, x2 if x2 is not None else torch.empty(0))
         ctx.has_x2 = x2 is not None
@@ -169,10 +221,33 @@ class _DenseFunction(torch.autograd.Function):
                 # dx1[:, i_seg] += c * x2[:, j] * g[:, k_seg] @ W_p^T
                 gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
                 if Z > 0:
-                    _run_gemms(dtype, g, wd, x2d, gx1, tables.dx1)
+                    if mod.tiled(dtype, g, gx1):
+                        # dx1[:, i_seg] (+)= c * g[:, k_seg] @ W_p^T: W_p (K x N) is already "N x K" for this product
+                        es = wd.element_size()
+                        _run_tiled(dtype, g, lambda p: p.c_off, lambda p: wd.data_ptr() + p.w_off * es, gx1, lambda p: p.a_off,
+                                   mod.dx1_groups, lambda p: p.N, lambda p: p.K)
+                    else:
+                        _run_gemms(dtype, g, wd, x2d, gx1, tables.dx1)
             if ctx.needs_input_grad[1]:
                 gwd = torch.zeros_like(wd)
-                if Z > 0:
+                if Z > 0 and mod.tiled(dtype, x1d, g):
+                    # dW_p[k][n] += c * sum_z x1[z, i_seg + k] g[z, k_seg + n]: chunked partial products, ordered sum
+                    code, es = _DTYPE_CODE[dtype], x1d.element_size()
+                    for p, count, da, dc in mod.fwd_groups:
+                        items = lib.cueq_gemm_tn_items(Z, count)
+                        part = torch.empty(items, p.K * p.N, dtype=torch.float32, device=x1.device)
+                        _lib.check(
+                            lib.cueq_gemm_tn(code, p.K, p.N, Z, x1d.data_ptr() + p.a_off * es, x1d.stride(0), da,
+                                             g.data_ptr() + p.c_off * es, g.stride(0), dc, count, part.data_ptr(), p.coeff, stream),
+                            "cueq_gemm_tn",
+                        )
+                        total = torch.empty(p.K * p.N, dtype=torch.float32, device=x1.device)
+                        ws_bytes = lib.cueq_sum_rows_workspace(items, p.K * p.N)
+                        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x1.device)
+                        _lib.check(lib.cueq_sum_rows(_lib.F32, items, p.K * p.N, part.data_ptr(), total.data_ptr(), ws.data_ptr(),
+                                                     ws_bytes, stream), "cueq_sum_rows")
+                        gwd.view(-1)[p.w_off: p.w_off + p.K * p.N] += total.to(dtype)
+                elif Z > 0:
                     for w_off, K, N, ent, n in tables.dw:
                         ws_bytes = lib.cueq_seg_outer_workspace(_DTYPE_CODE[dtype], K, N, Z)
                         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x1.device)
@@ -235,6 +310,25 @@ class SegmentedPolynomialDense(nn.Module):
         self.fwd_covers_output = out_cols == self.out_size
         self.dx1_covers_input = in_cols == self.input_sizes[1]
         self._tables: Dict[int, _DeviceTables] = {}
+        # launches of the 128 x 128 tiled kernel (3-operand form only: no per-row scale there)
+        self.fwd_groups = _batched_groups(self.paths, lambda p: p.a_off, lambda p: p.c_off)
+        self.dx1_groups = _batched_groups(self.paths, lambda p: p.c_off, lambda p: p.a_off)
+        self.weight_blocks = sorted({(p.w_off, p.K, p.N) for p in self.paths})
+
+    def tiled(self, dtype, A: torch.Tensor, Cout: torch.Tensor) -> bool:
+        """The tiled kernel serves fp32 / bf16 contractions without a per-row scale."""
+        return (not self.has_x2) and dtype in (torch.float32, torch.bfloat16)
+
+    def transposed_weights(self, wd: torch.Tensor) -> torch.Tensor:
+        """Every ``K x N`` weight block transposed in place of itself (same offsets) by ``cueq_transpose``."""
+        lib = _lib.load()
+        wt = torch.empty_like(wd)
+        stream = torch.cuda.current_stream(wd.device).cuda_stream
+        es = wd.element_size()
+        for w_off, K, N in self.weight_blocks:
+            _lib.check(lib.cueq_transpose(_DTYPE_CODE[wd.dtype], 1, K, N, wd.data_ptr() + w_off * es, wt.data_ptr() + w_off * es, stream),
+                       "cueq_transpose")
+        return wt
 
     def tables(self, device: torch.device) -> _DeviceTables:
         idx = device.index if device.index is not None else torch.cuda.current_device()

@@ -188,6 +188,15 @@ int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int6
                  int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
                  int64_t batch, double alpha, int32_t accumulate, void* stream);
 
+/* Weight-gradient shaped product C (M x N) = sum over rows z and parts p of A[z, p*stride_a : +M]^T B[z, p*stride_b : +N]
+ * (both operands row-major with the long index z as rows).  The rows are cut into chunks; item (chunk, part) writes
+ * alpha * its partial product to partials[item] (float32, M x N); the caller adds the cueq_gemm_tn_items(rows, nparts)
+ * items in order (e.g. cueq_sum_rows over an items x (M*N) view): no atomics.  Serves the weight gradients of the dense
+ * layers (reference: the backward of FusedTensorProductOp3, primitives/segmented_polynomial_fused_tp.py:32-48). */
+int64_t cueq_gemm_tn_items(int64_t rows, int32_t nparts);
+int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows, const void* A, int64_t lda, int64_t stride_a,
+                 const void* B, int64_t ldb, int64_t stride_b, int32_t nparts, float* partials, double alpha, void* stream);
+
 /* out[b][c][r] = in[b][r][c] (layout changes "bijd<->dbij" of _layer_norm_transpose.py:162-227 and operand
  * re-orientation for the incoming direction and the backward contractions). */
 int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_t cols, const void* in, void* out, void* stream);
