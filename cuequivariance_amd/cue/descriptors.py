@@ -5,7 +5,7 @@ Reference behaviour followed (``cuequivariance/cuequivariance/group_theory/descr
 * ``irreps_tp.py:22-91``    fully_connected_tensor_product  ``"uvw,iu,jv,kw+ijk"``
 * ``irreps_tp.py:232-321``  channelwise_tensor_product      ``"uv,iu,jv,kuv+ijk"``
 * ``irreps_tp.py:505-545``  linear                          ``"uv,iu,iv"``
-* ``spherical_harmonics_.py:119-156`` recursion and normalisation of the spherical harmonics
+* ``spherical_harmonics_.py:23-85,119-156`` spherical-harmonics polynomial, recursion and normalisation
 * ``symmetric_contractions.py:20-134``  symmetric_contraction  ``"w_a_b_c_i+abciw"`` per degree
 
 All descriptors use the ``ir_mul`` layout (component index outside, multiplicity inside).
@@ -28,6 +28,7 @@ __all__ = [
     "channelwise_tensor_product",
     "fully_connected_tensor_product",
     "linear",
+    "spherical_harmonics",
     "spherical_harmonics_values",
     "symmetric_contraction",
 ]
@@ -253,4 +254,81 @@ def symmetric_contraction(irreps_in: Irreps, irreps_out: Irreps, degrees) -> Equ
         [IrrepsAndLayout(irreps_in.new_scalars(poly.inputs[0].size), ir_mul), IrrepsAndLayout(irreps_in, ir_mul)],
         [IrrepsAndLayout(irreps_out, ir_mul)],
         poly,
+    )
+
+
+# ---------------------------------------------------------------------------------------------
+# spherical harmonics as a polynomial of the vector
+# ---------------------------------------------------------------------------------------------
+@functools.lru_cache(maxsize=None)
+def _sh_monomials(ir_vec: Irrep, ell: int) -> tuple:
+    """``Y_l`` component by component as ``{(d0, d1, d2): coefficient}`` (homogeneous of degree ``l``); same
+    recursion and normalisation as :func:`spherical_harmonics_values`, carried out on polynomials."""
+    from .linalg import round_to_sqrt_rational
+
+    if ell == 0:
+        return ({(0, 0, 0): 1.0},)
+    if ell == 1:
+        return tuple({tuple(int(a == i) for a in range(3)): float(np.sqrt(3.0))} for i in range(3))
+    l2 = ell // 2
+    l1 = ell - l2
+    y1, y2 = _sh_monomials(ir_vec, l1), _sh_monomials(ir_vec, l2)
+    ir1, ir2 = _sh_irrep(ir_vec, l1), _sh_irrep(ir_vec, l2)
+    ir = sorted(ir1 * ir2, key=_Key)[-1]
+    cg = clebsch_gordan(ir1, ir2, ir)[0]
+    comps = []
+    for k in range(ir.dim):
+        acc: dict = {}
+        for i in range(ir1.dim):
+            for j in range(ir2.dim):
+                c = cg[i, j, k]
+                if c == 0.0:
+                    continue
+                for da, ca in y1[i].items():
+                    for db, cb in y2[j].items():
+                        key = (da[0] + db[0], da[1] + db[1], da[2] + db[2])
+                        acc[key] = acc.get(key, 0.0) + c * ca * cb
+        comps.append(acc)
+    # normalise on the point (0, 1, 0): only the pure x1^l monomials survive there
+    north = np.array([comp.get((0, ell, 0), 0.0) for comp in comps])
+    scale = np.sqrt(2 * ell + 1) / np.sqrt(np.sum(north**2))
+    out = []
+    for comp in comps:
+        cleaned = {}
+        for key, c in comp.items():
+            c = float(round_to_sqrt_rational(np.asarray(c * scale), 2**20))
+            if abs(c) > 1e-12:
+                cleaned[key] = c
+        out.append(cleaned)
+    return tuple(out)
+
+
+@functools.lru_cache(maxsize=None)
+def _spherical_harmonics_core(ir_vec: Irrep, ls: tuple):
+    if len(ls) != 1:
+        results = [_spherical_harmonics_core(ir_vec, (ell,)) for ell in ls]
+        poly = SegmentedPolynomial.stack([r[0] for r in results], [False, True])
+        return poly, Irreps(type(ir_vec), sum([list(r[1]) for r in results], []))
+    [ell] = ls
+    ir = _sh_irrep(ir_vec, ell)
+    assert ir_vec.dim == 3
+    d = SegmentedTensorProduct.empty_segments([3] * ell + [ir.dim])
+    for i, comp in enumerate(_sh_monomials(ir_vec, ell)):
+        for degrees in sorted(comp, reverse=True):  # lexicographic, highest power of x0 first
+            indices = sum(((a,) * n for a, n in enumerate(degrees)), ())
+            d.add_path(*indices, i, c=comp[degrees])
+    d = d.symmetrize_operands(range(ell))
+    poly = SegmentedPolynomial(
+        [SegmentedOperand([()] * 3, ndim=0)], [SegmentedOperand([()] * ir.dim, ndim=0)], [(Operation([0] * ell + [1]), d)]
+    )
+    return poly, Irreps(type(ir_vec), [(1, ir)])
+
+
+def spherical_harmonics(ir_vec: Irrep, ls, layout=ir_mul) -> EquivariantPolynomial:
+    """Spherical harmonics ``Y_l(x)`` for every ``l`` in ``ls`` as a polynomial of the vector ``x`` (component
+    normalisation: ``sum_m Y_lm(x)^2 = 2l+1`` on unit vectors, ``Y_1 = sqrt(3) x``).  Operands ``vector[] ... -> Y[]``;
+    ``[0, 1, 2]`` gives 1 / 3 / 11 paths (reference ``descriptors/spherical_harmonics_.py:56-85``)."""
+    poly, irreps_out = _spherical_harmonics_core(ir_vec, tuple(ls))
+    return EquivariantPolynomial(
+        [IrrepsAndLayout(Irreps(type(ir_vec), [(1, ir_vec)]), ir_mul)], [IrrepsAndLayout(irreps_out, ir_mul)], poly
     )

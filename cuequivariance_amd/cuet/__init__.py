@@ -2,7 +2,7 @@
 
 from .transpose import TransposeSegments, TransposeIrrepsLayout
 from .segmented_polynomial import SegmentedPolynomial
-from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction
+from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction, SphericalHarmonics
 from .uniform_1d import uniform_1d
 from .triangle import triangle_multiplicative_update, TriMulPrecision
 
@@ -14,6 +14,7 @@ __all__ = [
     "FullyConnectedTensorProduct",
     "Linear",
     "SymmetricContraction",
+    "SphericalHarmonics",
     "uniform_1d",
     "triangle_multiplicative_update",
     "TriMulPrecision",

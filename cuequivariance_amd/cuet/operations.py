@@ -7,6 +7,7 @@ Constructor arguments, attributes (``irreps_*``, ``weight_numel``, ``weight``, `
 * ``cuequivariance_torch/cuequivariance_torch/operations/tp_fully_connected.py:30-207``
 * ``cuequivariance_torch/cuequivariance_torch/operations/linear.py:30-191``
 * ``cuequivariance_torch/cuequivariance_torch/operations/symmetric_contraction.py:32-242``
+* ``cuequivariance_torch/cuequivariance_torch/operations/spherical_harmonics.py:26-93``
 
 Defaults differ where the reference defaults to its PyTorch executor: every layer here runs HIP
 kernels (``uniform_1d`` for the channel-wise product, the dense executor ``fused_tp`` for the other two).
@@ -24,7 +25,7 @@ from ..cue import descriptors
 from .segmented_polynomial import SegmentedPolynomial
 from .transpose import TransposeIrrepsLayout
 
-__all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear", "SymmetricContraction"]
+__all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear", "SymmetricContraction", "SphericalHarmonics"]
 
 
 def _default_irreps(*irreps_list):
@@ -378,3 +379,26 @@ class SymmetricContraction(torch.nn.Module):
             weight = self.weight
         out = self.f([weight.flatten(1), self.transpose_in(x)], input_indices={0: indices})
         return self.transpose_out(out[0])
+
+
+class SphericalHarmonics(torch.nn.Module):
+    """Spherical harmonics of 3-vectors: ``forward(vectors (batch, 3)) -> (batch, sum(2l+1))`` for the degrees ``ls``
+    (ascending, unique); component normalisation, ``Y_1 = sqrt(3) x``.  ``normalize=True`` divides the vectors by their
+    norm first."""
+
+    def __init__(self, ls, normalize: bool = True, device: Optional[torch.device] = None, math_dtype=None,
+                 use_fallback: Optional[bool] = None, method: Optional[str] = None):
+        super().__init__()
+        self.ls = ls if isinstance(ls, list) else [ls]
+        assert self.ls == sorted(set(self.ls))
+        self.normalize = normalize
+        e = descriptors.spherical_harmonics(cue.SO3(1), self.ls)
+        self.method = _method_from_fallback(method, use_fallback, "uniform_1d")
+        self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+
+    def forward(self, vectors: torch.Tensor) -> torch.Tensor:
+        torch._assert(vectors.ndim == 2, f"Input must have shape (batch, 3) - got {vectors.shape}")
+        if self.normalize:
+            vectors = torch.nn.functional.normalize(vectors, dim=1)
+        [output] = self.f([vectors])
+        return output

@@ -73,6 +73,14 @@ def _tensor_product(op: dict, out_pos: int, inputs: List[torch.Tensor], math_dty
     formula = ",".join([op["coefficient_subscripts"]] + ["Z" + ss[k] for k in in_pos]) + "->Z" + ss[out_pos]
     offs = [_offsets(segs) for segs in op["segments"]]
     out_segments = op["segments"][out_pos]
+    if not in_pos:
+        # an operation without inputs is a constant row (segmented_polynomial_naive.py:184-240), broadcast by the caller
+        row = torch.zeros(sum(math.prod(sh) for sh in out_segments), dtype=math_dtype or torch.float64)
+        for idx, coeff in zip(op["path_indices"], op["path_coefficients"]):
+            shape = out_segments[idx[out_pos]]
+            o = offs[out_pos][idx[out_pos]]
+            row[o: o + math.prod(shape)] += torch.tensor(coeff, dtype=row.dtype).reshape(-1)
+        return row.to(first_dtype).reshape(1, -1)
     per_segment: List[List[torch.Tensor]] = [[] for _ in out_segments]
     for idx, coeff in zip(op["path_indices"], op["path_coefficients"]):
         if not np.any(coeff != 0):

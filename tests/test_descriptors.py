@@ -360,3 +360,23 @@ def test_cfg2_tables():
     np.testing.assert_allclose(t.path_coefficients[:4], [1.0, 1.0, 1.0, 1.0], atol=1e-12)
     # element offset of segment s of buffer b in a row is s * extent (or s for scalars)
     assert t.width(0) == 2944 and t.width(1) == 2048 and t.width(2) == 16 and t.width(3) == 12672
+
+
+def test_spherical_harmonics_polynomial():
+    """Path counts of the doc example (``descriptors/spherical_harmonics_.py:70-76``), the value at (0, 1, 0)
+    (``cuequivariance_jax/segmented_polynomials/segmented_polynomial.py:112-117``), the norm on unit vectors and agreement
+    with the independent value recursion."""
+    e = cue.descriptors.spherical_harmonics(cue.SO3(1), [0, 1, 2])
+    assert [d.num_paths for _, d in e.polynomial.operations] == [1, 3, 11]
+    [y] = e.polynomial(np.array([0.0, 1.0, 0.0]))
+    np.testing.assert_allclose(y, [1, 0, np.sqrt(3), 0, 0, 0, np.sqrt(5), 0, 0], atol=1e-14)
+    ls = [0, 1, 2, 3, 4]
+    p = cue.descriptors.spherical_harmonics(cue.O3(1, -1), ls).polynomial
+    x = np.random.default_rng(0).normal(size=(7, 3))
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    [y] = p(x)
+    np.testing.assert_allclose(y, cue.descriptors.spherical_harmonics_values(cue.O3(1, -1), ls, x), atol=1e-13)
+    off = 0
+    for ell in ls:
+        np.testing.assert_allclose((y[:, off: off + 2 * ell + 1] ** 2).sum(1), 2 * ell + 1, atol=1e-12)
+        off += 2 * ell + 1

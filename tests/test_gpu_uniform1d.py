@@ -401,3 +401,27 @@ def test_segment_csr_bit_exact(device, sorted_ids, index_dtype):
     assert torch.equal(perm.cpu()[:n], exp_perm)
     with pytest.raises(Exception):
         _segment_csr(torch.tensor([0, nrows], dtype=index_dtype, device=device), nrows)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_spherical_harmonics_module(device, dtype):
+    """``cuet.SphericalHarmonics`` (reference ``operations/spherical_harmonics.py:26-93``): values and the gradient
+    with respect to the vectors against the oracle, with and without normalisation."""
+    from cuequivariance_amd import cuet
+
+    ls = [0, 1, 2, 3]
+    g = torch.Generator().manual_seed(0)
+    v = torch.randn(301, 3, dtype=torch.float64, generator=g).to(dtype)
+    cot = torch.randn(301, 16, dtype=torch.float64, generator=g).to(dtype)
+    for normalize in (True, False):
+        m = cuet.SphericalHarmonics(ls, normalize=normalize)
+        spec = spec_from_polynomial(m.f._polynomial_orig)
+        a = v.clone().requires_grad_(True)
+        vin = torch.nn.functional.normalize(a, dim=1) if normalize else a
+        ref = naive_segmented_polynomial(spec, [vin])[0]
+        (ref_grad,) = torch.autograd.grad(ref, [a], cot)
+        b = v.clone().to(device).requires_grad_(True)
+        out = m(b)
+        (grad,) = torch.autograd.grad(out, [b], cot.to(device))
+        assert_close(out, ref, TOL[dtype], "Y")
+        assert_close(grad, ref_grad, 4 * TOL[dtype], "dY/dx")
