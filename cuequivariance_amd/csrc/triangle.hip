@@ -299,12 +299,38 @@ __global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ in
   }
 }
 
+// 2-byte elements, even extents: 64 x 64 tiles moved as pairs (4-byte accesses on both sides)
+__global__ void __launch_bounds__(256) transpose16_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, int R, int Ccols) {
+  __shared__ uint16_t tile[64][66];
+  const int64_t base = static_cast<int64_t>(blockIdx.z) * R * Ccols;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 pairs x 8
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int r = r0 + ty + q * 8, cc = c0 + 2 * tx;
+    if (r < R && cc < Ccols) {
+      const uint32_t v = *reinterpret_cast<const uint32_t*>(in + base + static_cast<int64_t>(r) * Ccols + cc);
+      tile[ty + q * 8][2 * tx] = static_cast<uint16_t>(v & 0xffffu);
+      tile[ty + q * 8][2 * tx + 1] = static_cast<uint16_t>(v >> 16);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int cc = c0 + ty + q * 8, r = r0 + 2 * tx;
+    if (r < R && cc < Ccols) {
+      const uint32_t v = static_cast<uint32_t>(tile[2 * tx][ty + q * 8]) | (static_cast<uint32_t>(tile[2 * tx + 1][ty + q * 8]) << 16);
+      *reinterpret_cast<uint32_t*>(out + base + static_cast<int64_t>(cc) * R + r) = v;
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // LayerNorm over rows of length D (D <= 1024): one wavefront per row, biased variance
 // ------------------------------------------------------------------------------------------------
 constexpr int kLnMaxPerLane = 16;
 
-template <typename T>
+template <typename T, int NQ>
 __global__ void __launch_bounds__(256) ln_fwd_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
                                                      T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd,
                                                      int64_t rows, int D, float eps) {
@@ -312,10 +338,10 @@ __global__ void __launch_bounds__(256) ln_fwd_kernel(const T* __restrict__ x, co
   const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const T* xr = x + row * D;
-  float v[kLnMaxPerLane];
+  float v[NQ];
   float s = 0;
 #pragma unroll
-  for (int q = 0; q < kLnMaxPerLane; ++q) {
+  for (int q = 0; q < NQ; ++q) {
     const int e = lane + q * 64;
     v[q] = e < D ? tri_load(xr, e) : 0.f;
     s += v[q];
@@ -323,7 +349,7 @@ __global__ void __launch_bounds__(256) ln_fwd_kernel(const T* __restrict__ x, co
   const float mu = wave_sum(s) / D;
   float ss = 0;
 #pragma unroll
-  for (int q = 0; q < kLnMaxPerLane; ++q) {
+  for (int q = 0; q < NQ; ++q) {
     const int e = lane + q * 64;
     const float d = e < D ? v[q] - mu : 0.f;
     ss += d * d;
@@ -331,7 +357,7 @@ __global__ void __launch_bounds__(256) ln_fwd_kernel(const T* __restrict__ x, co
   const float rs = 1.0f / sqrtf(wave_sum(ss) / D + eps);
   T* yr = y + row * D;
 #pragma unroll
-  for (int q = 0; q < kLnMaxPerLane; ++q) {
+  for (int q = 0; q < NQ; ++q) {
     const int e = lane + q * 64;
     if (e < D) {
       float o = (v[q] - mu) * rs;
@@ -348,26 +374,26 @@ __global__ void __launch_bounds__(256) ln_fwd_kernel(const T* __restrict__ x, co
 
 // dx = rstd * (g - mean(g) - xhat * mean(g * xhat)),  g = dy * gamma;   per-block partial sums of
 // dgamma = sum dy * xhat and dbeta = sum dy go to part[2][blocks][D].
-template <typename T>
+template <typename T, int NQ>
 __global__ void __launch_bounds__(256) ln_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ mean,
                                                      const float* __restrict__ rstd, const T* __restrict__ gamma,
                                                      T* __restrict__ dx, float* __restrict__ part, int64_t rows, int D,
                                                      int rows_per_block) {
   extern __shared__ float sred[];  // [4 waves][2][D]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float ag[kLnMaxPerLane], ab[kLnMaxPerLane];
+  float ag[NQ], ab[NQ];
 #pragma unroll
-  for (int q = 0; q < kLnMaxPerLane; ++q) ag[q] = ab[q] = 0.f;
+  for (int q = 0; q < NQ; ++q) ag[q] = ab[q] = 0.f;
   const int64_t r_begin = static_cast<int64_t>(blockIdx.x) * rows_per_block;
   const int64_t r_end = min(r_begin + rows_per_block, rows);
   for (int64_t row = r_begin + wave; row < r_end; row += 4) {
     const T* xr = x + row * D;
     const T* gr = dy + row * D;
     const float mu = mean[row], rs = rstd[row];
-    float xh[kLnMaxPerLane], g[kLnMaxPerLane];
+    float xh[NQ], g[NQ];
     float s1 = 0, s2 = 0;
 #pragma unroll
-    for (int q = 0; q < kLnMaxPerLane; ++q) {
+    for (int q = 0; q < NQ; ++q) {
       const int e = lane + q * 64;
       if (e < D) {
         xh[q] = (tri_load(xr, e) - mu) * rs;
@@ -385,17 +411,152 @@ __global__ void __launch_bounds__(256) ln_bwd_kernel(const T* __restrict__ dy, c
     s2 = wave_sum(s2) / D;
     T* dr = dx + row * D;
 #pragma unroll
-    for (int q = 0; q < kLnMaxPerLane; ++q) {
+    for (int q = 0; q < NQ; ++q) {
       const int e = lane + q * 64;
       if (e < D) tri_store(dr, e, rs * (g[q] - s1 - xh[q] * s2));
     }
   }
 #pragma unroll
-  for (int q = 0; q < kLnMaxPerLane; ++q) {
+  for (int q = 0; q < NQ; ++q) {
     const int e = lane + q * 64;
     if (e < D) {
       sred[(wave * 2 + 0) * D + e] = ag[q];
       sred[(wave * 2 + 1) * D + e] = ab[q];
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 2 * D; e += 256) {
+    const int which = e / D, d = e - which * D;
+    float s = 0;
+    for (int w = 0; w < 4; ++w) s += sred[(w * 2 + which) * D + d];
+    part[(static_cast<int64_t>(which) * gridDim.x + blockIdx.x) * D + d] = s;
+  }
+}
+
+// ---- rows of D = 8 L elements: L lanes per row, 8 consecutive elements (16 or 32 bytes) per lane, 64 / L rows
+//      per wavefront; reductions stay inside the L lanes ------------------------------------------------------------
+__device__ __forceinline__ void ln_store8(float* p, const float* r) {
+  *reinterpret_cast<float4*>(p) = make_float4(r[0], r[1], r[2], r[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(r[4], r[5], r[6], r[7]);
+}
+__device__ __forceinline__ void ln_store8(uint16_t* p, const float* r) {
+  uint4 o;
+  o.x = float_to_bf16_bits(r[0]) | (static_cast<uint32_t>(float_to_bf16_bits(r[1])) << 16);
+  o.y = float_to_bf16_bits(r[2]) | (static_cast<uint32_t>(float_to_bf16_bits(r[3])) << 16);
+  o.z = float_to_bf16_bits(r[4]) | (static_cast<uint32_t>(float_to_bf16_bits(r[5])) << 16);
+  o.w = float_to_bf16_bits(r[6]) | (static_cast<uint32_t>(float_to_bf16_bits(r[7])) << 16);
+  *reinterpret_cast<uint4*>(p) = o;
+}
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {  // sum over aligned groups of L lanes, valid in every lane
+  if (L >= 2) v += dpp_move<0xB1>(v);
+  if (L >= 4) v += dpp_move<0x4E>(v);
+  if (L >= 8) v += dpp_move<0x141>(v);
+  if (L >= 16) v += dpp_move<0x140>(v);
+  if (L >= 32) v += __shfl_xor(v, 16, 64);
+  if (L >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+template <typename T, int L>
+__global__ void __launch_bounds__(256) ln_fwd_rows8(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                    T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd, int64_t rows,
+                                                    float eps) {
+  constexpr int D = 8 * L, RPW = 64 / L;
+  const int lane = threadIdx.x & 63, sub = lane / L, col = (lane % L) * 8;
+  const int64_t row = (static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6)) * RPW + sub;
+  const bool ok = row < rows;
+  float v[8], gm[8], bt[8];
+  if (ok) tn_load8(x + row * D + col, v);
+  else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0.f;
+  }
+  float s = 0;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) s += v[e];
+  const float mu = group_sum<L>(s) * (1.0f / D);
+  float ss = 0;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    v[e] -= mu;
+    ss += v[e] * v[e];
+  }
+  const float rs = 1.0f / sqrtf(group_sum<L>(ss) * (1.0f / D) + eps);
+  if (gamma) tn_load8(gamma + col, gm);
+  if (beta) tn_load8(beta + col, bt);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    v[e] *= rs;
+    if (gamma) v[e] *= gm[e];
+    if (beta) v[e] += bt[e];
+  }
+  if (ok) {
+    ln_store8(y + row * D + col, v);
+    if (lane % L == 0) {
+      mean[row] = mu;
+      rstd[row] = rs;
+    }
+  }
+}
+
+template <typename T, int L>
+__global__ void __launch_bounds__(256) ln_bwd_rows8(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ mean,
+                                                    const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
+                                                    float* __restrict__ part, int64_t rows, int rows_per_block) {
+  constexpr int D = 8 * L, RPW = 64 / L;
+  extern __shared__ float sred[];  // [4 waves][2][D]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane / L, col = (lane % L) * 8;
+  float ag[8], ab[8], gm[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ag[e] = ab[e] = 0.f;
+  if (gamma) tn_load8(gamma + col, gm);
+  const int64_t r_begin = static_cast<int64_t>(blockIdx.x) * rows_per_block;
+  const int64_t r_end = min(r_begin + rows_per_block, rows);
+  for (int64_t r0 = r_begin + wave * RPW; r0 < r_end; r0 += 4 * RPW) {
+    const int64_t row = r0 + sub;
+    const bool ok = row < r_end;
+    float xh[8], g[8];
+    float mu = 0.f, rs = 0.f;
+    if (ok) {
+      tn_load8(x + row * D + col, xh);
+      tn_load8(dy + row * D + col, g);
+      mu = mean[row];
+      rs = rstd[row];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xh[e] = g[e] = 0.f;
+    }
+    float s1 = 0, s2 = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      xh[e] = (xh[e] - mu) * rs;
+      ag[e] += g[e] * xh[e];
+      ab[e] += g[e];
+      if (gamma) g[e] *= gm[e];
+      s1 += g[e];
+      s2 += g[e] * xh[e];
+    }
+    s1 = group_sum<L>(s1) * (1.0f / D);
+    s2 = group_sum<L>(s2) * (1.0f / D);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] = rs * (g[e] - s1 - xh[e] * s2);
+    if (ok) ln_store8(dx + row * D + col, g);
+  }
+  // rows of one wavefront -> one lane group, then the four wavefronts through LDS
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+#pragma unroll
+    for (int off = L; off < 64; off *= 2) {
+      ag[e] += __shfl_xor(ag[e], off, 64);
+      ab[e] += __shfl_xor(ab[e], off, 64);
+    }
+  }
+  if (lane < L) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      sred[(wave * 2 + 0) * D + col + e] = ag[e];
+      sred[(wave * 2 + 1) * D + col + e] = ab[e];
     }
   }
   __syncthreads();
@@ -569,6 +730,16 @@ extern "C" int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_
   CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "transpose: dtype must be float32 or bfloat16");
   if (batch <= 0 || rows <= 0 || cols <= 0) return CUEQ_OK;
   CUEQ_REQUIRE(in && out, CUEQ_ERR_INVALID, "transpose: null operand");
+  CUEQ_REQUIRE(rows < (1ll << 31) && cols < (1ll << 31), CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
+  if (dtype == CUEQ_BF16 && rows % 2 == 0 && cols % 2 == 0 && reinterpret_cast<uintptr_t>(in) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0) {
+    const int64_t gy2 = (rows + 63) / 64, gx2 = (cols + 63) / 64;
+    CUEQ_REQUIRE(gy2 < 65536 && batch < 65536, CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
+    KernelTimer timer("transpose", stream);
+    hipLaunchKernelGGL(transpose16_kernel, dim3(static_cast<unsigned>(gx2), static_cast<unsigned>(gy2), static_cast<unsigned>(batch)), dim3(256), 0, stream,
+                       static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols));
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
   const int64_t gy = (rows + 31) / 32, gx = (cols + 31) / 32;
   CUEQ_REQUIRE(gy < 65536 && batch < 65536 && gx < (1ll << 31), CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
   const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy), static_cast<unsigned>(batch));
@@ -590,9 +761,25 @@ extern "C" int cueq_layer_norm_fwd(int32_t dtype, int64_t rows, int64_t D, const
   CUEQ_REQUIRE((rows + 3) / 4 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "layer_norm: too many rows");
   const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
   KernelTimer timer("layer_norm_fwd", stream);
-  TRI_DISPATCH(dtype,
-               hipLaunchKernelGGL(ln_fwd_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), static_cast<const float*>(gamma), static_cast<const float*>(beta), static_cast<float*>(y), mean, rstd, rows, static_cast<int>(D), static_cast<float>(eps)),
-               hipLaunchKernelGGL(ln_fwd_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, rows, static_cast<int>(D), static_cast<float>(eps)));
+  const bool al16 = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(gamma) | reinterpret_cast<uintptr_t>(beta)) & 15) == 0;
+  if (al16 && (D == 32 || D == 64 || D == 128 || D == 256 || D == 512)) {
+    const int L = static_cast<int>(D / 8);
+    const int64_t rpb = 4 * (64 / L);
+    const dim3 g8(static_cast<unsigned>((rows + rpb - 1) / rpb));
+#define LN8(T, LL) hipLaunchKernelGGL((ln_fwd_rows8<T, LL>), g8, dim3(256), 0, stream, static_cast<const T*>(x), static_cast<const T*>(gamma), static_cast<const T*>(beta), static_cast<T*>(y), mean, rstd, rows, static_cast<float>(eps))
+#define LN8_L(T) do { switch (L) { case 4: LN8(T, 4); break; case 8: LN8(T, 8); break; case 16: LN8(T, 16); break; case 32: LN8(T, 32); break; default: LN8(T, 64); } } while (0)
+    TRI_DISPATCH(dtype, LN8_L(float), LN8_L(uint16_t));
+#undef LN8_L
+#undef LN8
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
+  const int nq = static_cast<int>((D + 63) / 64);
+#define LN_FWD(T, NQ) hipLaunchKernelGGL((ln_fwd_kernel<T, NQ>), grid, dim3(256), 0, stream, static_cast<const T*>(x), static_cast<const T*>(gamma), static_cast<const T*>(beta), static_cast<T*>(y), mean, rstd, rows, static_cast<int>(D), static_cast<float>(eps))
+#define LN_FWD_NQ(T) do { if (nq <= 1) LN_FWD(T, 1); else if (nq <= 2) LN_FWD(T, 2); else if (nq <= 4) LN_FWD(T, 4); else if (nq <= 8) LN_FWD(T, 8); else LN_FWD(T, 16); } while (0)
+  TRI_DISPATCH(dtype, LN_FWD_NQ(float), LN_FWD_NQ(uint16_t));
+#undef LN_FWD_NQ
+#undef LN_FWD
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }
@@ -626,9 +813,22 @@ extern "C" int cueq_layer_norm_bwd(int32_t dtype, int64_t rows, int64_t D, const
   const size_t sh = 4 * 2 * D * sizeof(float);
   {
     KernelTimer timer("layer_norm_bwd", stream);
-    TRI_DISPATCH(dtype,
-                 hipLaunchKernelGGL(ln_bwd_kernel<float>, dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const float*>(dy), static_cast<const float*>(x), mean, rstd, static_cast<const float*>(gamma), static_cast<float*>(dx), part, rows, static_cast<int>(D), rpb),
-                 hipLaunchKernelGGL(ln_bwd_kernel<uint16_t>, dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const uint16_t*>(dy), static_cast<const uint16_t*>(x), mean, rstd, static_cast<const uint16_t*>(gamma), static_cast<uint16_t*>(dx), part, rows, static_cast<int>(D), rpb));
+    const bool al16 = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(dx) | reinterpret_cast<uintptr_t>(gamma)) & 15) == 0;
+    const int nq = static_cast<int>((D + 63) / 64);
+    if (al16 && (D == 32 || D == 64 || D == 128 || D == 256 || D == 512)) {
+      const int L = static_cast<int>(D / 8);
+#define LNB8(T, LL) hipLaunchKernelGGL((ln_bwd_rows8<T, LL>), dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const T*>(dy), static_cast<const T*>(x), mean, rstd, static_cast<const T*>(gamma), static_cast<T*>(dx), part, rows, rpb)
+#define LNB8_L(T) do { switch (L) { case 4: LNB8(T, 4); break; case 8: LNB8(T, 8); break; case 16: LNB8(T, 16); break; case 32: LNB8(T, 32); break; default: LNB8(T, 64); } } while (0)
+      TRI_DISPATCH(dtype, LNB8_L(float), LNB8_L(uint16_t));
+#undef LNB8_L
+#undef LNB8
+    } else {
+#define LN_BWD(T, NQ) hipLaunchKernelGGL((ln_bwd_kernel<T, NQ>), dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const T*>(dy), static_cast<const T*>(x), mean, rstd, static_cast<const T*>(gamma), static_cast<T*>(dx), part, rows, static_cast<int>(D), rpb)
+#define LN_BWD_NQ(T) do { if (nq <= 1) LN_BWD(T, 1); else if (nq <= 2) LN_BWD(T, 2); else if (nq <= 4) LN_BWD(T, 4); else if (nq <= 8) LN_BWD(T, 8); else LN_BWD(T, 16); } while (0)
+    TRI_DISPATCH(dtype, LN_BWD_NQ(float), LN_BWD_NQ(uint16_t));
+#undef LN_BWD_NQ
+#undef LN_BWD
+    }
   }
   CUEQ_CHECK_HIP(hipGetLastError());
   const unsigned g = static_cast<unsigned>((D + 255) / 256);
