@@ -38,6 +38,20 @@ __device__ __forceinline__ void tri_store(uint16_t* p, int64_t i, float v) { p[i
 constexpr int kTile = 128;
 constexpr int kRowBytes = 80;  // 64 bytes of data + 16 bytes of padding
 
+// Workgroups are handed to the 8 XCDs round-robin in launch order and every XCD has its own L2.  This maps the
+// launch-order index to a tile index so that each XCD works through one contiguous range of tiles (column tile
+// fastest, then row tile, then batch): tiles that read the same operand rows then share an L2.
+__device__ __forceinline__ void xcd_tile(int& bx, int& by, int& bz) {
+  const uint64_t gx = gridDim.x, gy = gridDim.y;
+  const uint64_t total = gx * gy * gridDim.z;
+  const uint64_t L = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+  const uint64_t q = total >> 3, r = total & 7, x = L & 7;
+  const uint64_t P = x * q + (x < r ? x : r) + (L >> 3);
+  bx = static_cast<int>(P % gx);
+  by = static_cast<int>((P / gx) % gy);
+  bz = static_cast<int>(P / (gx * gy));
+}
+
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
                                                       const TI* __restrict__ B, int64_t ldb, int64_t sB,
@@ -49,10 +63,12 @@ __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
-  A += static_cast<int64_t>(blockIdx.z) * sA;
-  B += static_cast<int64_t>(blockIdx.z) * sB;
-  C += static_cast<int64_t>(blockIdx.z) * sC;
+  int bx, by, bz;
+  xcd_tile(bx, by, bz);
+  const int m0 = by * kTile, n0 = bx * kTile;
+  A += static_cast<int64_t>(bz) * sA;
+  B += static_cast<int64_t>(bz) * sB;
+  C += static_cast<int64_t>(bz) * sC;
 
   // every thread stages two 16-byte vectors of A and two of B per step
   uint4 stA[2], stB[2];
@@ -256,6 +272,128 @@ __global__ void __launch_bounds__(256) gemm_tn_kernel(const TI* __restrict__ A, 
         if (row < M && col < N) P[static_cast<int64_t>(row) * N + col] = alpha * acc[i][j][v];
       }
     }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Two products of the same shape and the sigmoid gate in one kernel:
+//   u = A1 * B1^T,  v = A2 * B2^T   (A* M x K, B* N x K, contraction contiguous, fp32 accumulate)
+//   BWD == false:  C = sigmoid(u + b1) * (v + b2) * mask
+//   BWD == true :  dU = dC * mask * (v + b2) * s * (1 - s),  dV = dC * mask * s,   s = sigmoid(u + b1)
+// so the two accumulators never travel through memory (the backward recomputes them).  Biases and mask are
+// indexed by row (axis 0) or column (axis 1) of C.  Same 128 x 128 tiling as gemm_nt_kernel; SHARE_B: B2 == B1.
+// ------------------------------------------------------------------------------------------------
+template <typename TI, bool BWD, bool SHARE_B>
+__global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict__ A1, const TI* __restrict__ A2, int64_t lda,
+                                                           const TI* __restrict__ B1, const TI* __restrict__ B2, int64_t ldb,
+                                                           const TI* __restrict__ bias1, const TI* __restrict__ bias2, int bias_axis,
+                                                           const TI* __restrict__ mask, int mask_axis, const TI* __restrict__ dC,
+                                                           TI* __restrict__ out1, TI* __restrict__ out2, int64_t ldc, int M, int N, int K) {
+  // 8 wavefronts of 64 x 32 (both products): half the accumulators per wavefront of the plain GEMM tiling, so two
+  // blocks fit a CU and one block's epilogue overlaps the other's loads.
+  constexpr int EPV = 16 / sizeof(TI);
+  constexpr int BK = 64 / sizeof(TI);
+  constexpr int NT = SHARE_B ? 3 : 4;  // staged tiles per step: A1, A2, B1 (, B2)
+  __shared__ __align__(16) char smem[2][NT][kTile * kRowBytes];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wm = wave >> 2, wn = wave & 3;
+  int bx, by, bz;
+  xcd_tile(bx, by, bz);
+  const int m0 = by * kTile, n0 = bx * kTile;
+
+  uint4 st[NT];
+  const int ldrow = tid >> 2, ldpart = tid & 3;
+  const int64_t offa = static_cast<int64_t>(min(m0 + ldrow, M - 1)) * lda + ldpart * EPV;
+  const int64_t offb = static_cast<int64_t>(min(n0 + ldrow, N - 1)) * ldb + ldpart * EPV;
+  auto load_step = [&](int ks) {
+    const int k = ks * BK;
+    if (k + ldpart * EPV < K) {
+      st[0] = *reinterpret_cast<const uint4*>(A1 + offa + k);
+      st[1] = *reinterpret_cast<const uint4*>(A2 + offa + k);
+      st[2] = *reinterpret_cast<const uint4*>(B1 + offb + k);
+      if constexpr (!SHARE_B) st[3] = *reinterpret_cast<const uint4*>(B2 + offb + k);
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) st[t] = make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_step = [&](int buf) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) *reinterpret_cast<uint4*>(&smem[buf][t][ldrow * kRowBytes + ldpart * 16]) = st[t];
+  };
+
+  floatx16 acc[2][2];  // [product][i]
+#pragma unroll
+  for (int p = 0; p < 2; ++p)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) acc[p][i] = floatx16{0};
+
+  const int nsteps = (K + BK - 1) / BK;
+  load_step(0);
+  int buf = 0;
+  for (int ks = 0; ks < nsteps; ++ks) {
+    store_step(buf);
+    __syncthreads();
+    if (ks + 1 < nsteps) load_step(ks + 1);
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      const char* sa = &smem[buf][p][(wm * 64 + c) * kRowBytes + h * 32];
+      const char* sb = &smem[buf][(SHARE_B || p == 0) ? 2 : 3][(wn * 32 + c) * kRowBytes + h * 32];
+      uint4 fa[2][2], fb[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        fa[0][q] = *reinterpret_cast<const uint4*>(sa + q * 16);
+        fa[1][q] = *reinterpret_cast<const uint4*>(sa + 32 * kRowBytes + q * 16);
+        fb[q] = *reinterpret_cast<const uint4*>(sb + q * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if constexpr (sizeof(TI) == 2) {
+#pragma unroll
+          for (int q = 0; q < 2; ++q)
+            acc[p][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[i][q]),
+                                                                __builtin_bit_cast(bf16x8_t, fb[q]), acc[p][i], 0, 0, 0);
+        } else {
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const float* pa = reinterpret_cast<const float*>(&fa[i][q]);
+            const float* pb = reinterpret_cast<const float*>(&fb[q]);
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) acc[p][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[s2], pb[s2], acc[p][i], 0, 0, 0);
+          }
+        }
+      }
+    }
+    buf ^= 1;
+  }
+
+  const int col = n0 + wn * 32 + c;
+  if (col >= N) return;
+  const float cb1 = (bias1 && bias_axis == 1) ? tri_load(bias1, col) : 0.f;
+  const float cb2 = (bias2 && bias_axis == 1) ? tri_load(bias2, col) : 0.f;
+  const float cmk = (mask && mask_axis == 1) ? tri_load(mask, col) : 1.f;
+  const bool rowb1 = bias1 && bias_axis == 0, rowb2 = bias2 && bias_axis == 0, rowmk = mask && mask_axis == 0;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+      if (row < M) {
+        const int64_t o = static_cast<int64_t>(row) * ldc + col;
+        const float uu = acc[0][i][v] + (rowb1 ? tri_load(bias1, row) : cb1);
+        const float vv = acc[1][i][v] + (rowb2 ? tri_load(bias2, row) : cb2);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-uu));
+        const float mk = rowmk ? tri_load(mask, row) : cmk;
+        if constexpr (!BWD) {
+          tri_store(out1, o, sg * vv * mk);
+        } else {
+          const float d = tri_load(dC, o) * mk;
+          tri_store(out1, o, d * vv * sg * (1.0f - sg));
+          tri_store(out2, o, d * sg);
+        }
+      }
+    }
+  }
 }
 
 // any shape / alignment: one thread per output element
@@ -689,6 +827,32 @@ extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int6
     else GEMM_LAUNCH(uint16_t, uint16_t);
 #undef GEMM_LAUNCH
   }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_t K, const void* A1, const void* A2, int64_t lda,
+                              const void* B1, const void* B2, int64_t ldb, const void* bias1, const void* bias2, int32_t bias_axis,
+                              const void* mask, int32_t mask_axis, const void* dC, void* out1, void* out2, int64_t ldc, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "dual_gate: dtype must be float32 or bfloat16");
+  CUEQ_REQUIRE(M >= 0 && N >= 0 && K > 0, CUEQ_ERR_INVALID, "dual_gate: bad extents");
+  if (M == 0 || N == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(A1 && A2 && B1 && out1 && (!backward || (dC && out2)), CUEQ_ERR_INVALID, "dual_gate: null operand");
+  const int epv = dtype == CUEQ_F32 ? 4 : 8;
+  const bool aligned = K % epv == 0 && lda % epv == 0 && ldb % epv == 0 &&
+                       ((reinterpret_cast<uintptr_t>(A1) | reinterpret_cast<uintptr_t>(A2) | reinterpret_cast<uintptr_t>(B1) | reinterpret_cast<uintptr_t>(B2)) & 15) == 0;
+  CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "dual_gate: K, row strides and pointers must be multiples of 16 bytes");
+  const int64_t gy = (M + kTile - 1) / kTile, gx = (N + kTile - 1) / kTile;
+  CUEQ_REQUIRE(gy < 65536 && gx < (1ll << 31) && M < (1ll << 31) && N < (1ll << 31), CUEQ_ERR_TOO_LARGE, "dual_gate: extent too large");
+  const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy));
+  const bool share = B2 == nullptr || B2 == B1;
+  KernelTimer timer(backward ? "dual_gate_bwd" : "dual_gate_fwd", stream);
+#define DG(TI, BW, SH) hipLaunchKernelGGL((dual_gate_kernel<TI, BW, SH>), grid, dim3(512), 0, stream, static_cast<const TI*>(A1), static_cast<const TI*>(A2), lda, static_cast<const TI*>(B1), static_cast<const TI*>(B2), ldb, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), bias_axis, static_cast<const TI*>(mask), mask_axis, static_cast<const TI*>(dC), static_cast<TI*>(out1), static_cast<TI*>(out2), ldc, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K))
+#define DG_T(TI) do { if (backward) { if (share) DG(TI, true, true); else DG(TI, true, false); } else { if (share) DG(TI, false, true); else DG(TI, false, false); } } while (0)
+  TRI_DISPATCH(dtype, DG_T(float), DG_T(uint16_t));
+#undef DG_T
+#undef DG
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }

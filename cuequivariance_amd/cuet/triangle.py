@@ -13,7 +13,8 @@ reference states in the open
 
 Every stage is a HIP kernel reached through the C ABI (``cueq_gemm_nt``, ``cueq_layer_norm_*``, ``cueq_gate_*``,
 ``cueq_transpose``, ``cueq_sum_*``); torch only owns the buffers.  Inputs float32 or bfloat16, fp32 accumulation;
-intermediate tensors are kept in the input dtype like the reference does, the projection accumulators in float32.
+intermediate tensors are kept in the input dtype like the reference does; the projection accumulators stay in registers
+(``cueq_dual_gate`` fuses both projections with the gate and recomputes them in the backward).
 """
 
 from __future__ import annotations
@@ -142,6 +143,55 @@ def gate_bwd(dout, u, v, bias_u, bias_v, bias_axis: int, mask, mask_axis: int):
     return du, dv
 
 
+def _fusable(*tensors) -> bool:
+    """The fused projection + gate kernel moves 16-byte vectors: row strides and addresses must allow it."""
+    for t in tensors:
+        if t is None:
+            continue
+        if t.data_ptr() % 16 or (t.dim() == 2 and (t.stride(0) * t.element_size()) % 16):
+            return False
+    return True
+
+
+def dual_gate_fwd(A1, A2, B1, B2, bias1, bias2, bias_axis: int, mask, mask_axis: int) -> torch.Tensor:
+    """``sigmoid(A1 B1^T + bias1) * (A2 B2^T + bias2) * mask`` (``B2 is None``: same as ``B1``); the two products stay
+    in registers when the operands allow the fused kernel, otherwise they go through float32 buffers."""
+    M, K = A1.shape
+    N = B1.shape[0]
+    T = A1.dtype
+    if _fusable(A1, A2, B1, B2) and (K * A1.element_size()) % 16 == 0:
+        out = torch.empty(M, N, dtype=T, device=A1.device)
+        _lib.check(
+            _lib.load().cueq_dual_gate(_CODE[T], 0, M, N, K, A1.data_ptr(), A2.data_ptr(), A1.stride(0), B1.data_ptr(), _ptr(B2),
+                                       B1.stride(0), _ptr(bias1), _ptr(bias2), bias_axis, _ptr(mask), mask_axis, None,
+                                       out.data_ptr(), None, N, _stream(A1)),
+            "cueq_dual_gate",
+        )
+        return out
+    u = gemm_nt(A1, B1, torch.float32)
+    v = gemm_nt(A2, B1 if B2 is None else B2, torch.float32)
+    return gate_fwd(u, v, bias1, bias2, bias_axis, mask, mask_axis, T)
+
+
+def dual_gate_bwd(dout, A1, A2, B1, B2, bias1, bias2, bias_axis: int, mask, mask_axis: int):
+    """Gradients of the two products of :func:`dual_gate_fwd` (they are recomputed, not read back)."""
+    M, K = A1.shape
+    N = B1.shape[0]
+    T = A1.dtype
+    if _fusable(A1, A2, B1, B2, dout) and (K * A1.element_size()) % 16 == 0:
+        du, dv = torch.empty(M, N, dtype=T, device=A1.device), torch.empty(M, N, dtype=T, device=A1.device)
+        _lib.check(
+            _lib.load().cueq_dual_gate(_CODE[T], 1, M, N, K, A1.data_ptr(), A2.data_ptr(), A1.stride(0), B1.data_ptr(), _ptr(B2),
+                                       B1.stride(0), _ptr(bias1), _ptr(bias2), bias_axis, _ptr(mask), mask_axis, dout.data_ptr(),
+                                       du.data_ptr(), dv.data_ptr(), N, _stream(A1)),
+            "cueq_dual_gate",
+        )
+        return du, dv
+    u = gemm_nt(A1, B1, torch.float32)
+    v = gemm_nt(A2, B1 if B2 is None else B2, torch.float32)
+    return gate_bwd(dout, u, v, bias1, bias2, bias_axis, mask, mask_axis)
+
+
 def sum_cols(x: torch.Tensor) -> torch.Tensor:
     rows, cols = x.shape
     out = torch.empty(rows, dtype=torch.float32, device=x.device)
@@ -195,10 +245,9 @@ class _TriMul(torch.autograd.Function):
         Do = p_out_w.shape[0]
         x2 = x.reshape(M, D)
         xh, mean1, rstd1 = layer_norm_fwd(x2, nin_w, nin_b, eps)
-        u1 = gemm_nt(g_in_w, xh, torch.float32)  # (2D, M): the "transposed output" of the reference comes for free
-        v1 = gemm_nt(p_in_w, xh, torch.float32)
         mflat = None if mask is None else mask.reshape(M)
-        ab = gate_fwd(u1, v1, g_in_b, p_in_b, 0, mflat, 1, T)  # (2D, M) == (2D, B, N, N)
+        # (2D, M) == (2D, B, N, N): the "transposed output" of the reference comes for free with the weights as rows
+        ab = dual_gate_fwd(g_in_w, p_in_w, xh, None, g_in_b, p_in_b, 0, mflat, 1)
         a = ab[:D].view(D * Bsz, N, N)
         b = ab[D:].view(D * Bsz, N, N)
         if outgoing:
@@ -207,11 +256,9 @@ class _TriMul(torch.autograd.Function):
             t = gemm_nt(transpose(a), transpose(b), T)  # t[i, j] = sum_k a[k, i] b[k, j]
         tT = transpose(t.view(D, M))  # (M, D)
         y, mean2, rstd2 = layer_norm_fwd(tT, nout_w, nout_b, eps)
-        u2 = gemm_nt(xh, g_out_w, torch.float32)  # (M, Do)
-        v2 = gemm_nt(y, p_out_w, torch.float32)
-        out = gate_fwd(u2, v2, g_out_b, p_out_b, 1, None, 0, T)
+        out = dual_gate_fwd(xh, y, g_out_w, p_out_w, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
         ctx.save_for_backward(x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
-                              xh, mean1, rstd1, u1, v1, ab, tT, mean2, rstd2, y, u2, v2)
+                              xh, mean1, rstd1, ab, tT, mean2, rstd2, y)
         ctx.outgoing, ctx.dims = outgoing, (Bsz, N, D, Do)
         ctx.has = (nin_w is not None, nin_b is not None, nout_w is not None, nout_b is not None)
         return out.view(Bsz, N, N, Do)
@@ -219,7 +266,7 @@ class _TriMul(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout):
         (x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
-         xh, mean1, rstd1, u1, v1, ab, tT, mean2, rstd2, y, u2, v2) = ctx.saved_tensors
+         xh, mean1, rstd1, ab, tT, mean2, rstd2, y) = ctx.saved_tensors
         Bsz, N, D, Do = ctx.dims
         M = Bsz * N * N
         T = x2.dtype
@@ -227,7 +274,7 @@ class _TriMul(torch.autograd.Function):
         dout = dout.contiguous().view(M, Do).to(T)
 
         # output gate
-        du2, dv2 = gate_bwd(dout, u2, v2, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
+        du2, dv2 = dual_gate_bwd(dout, xh, y, g_out_w, p_out_w, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
         dxh = gemm_nt(du2, transpose(g_out_w), T)  # (M, D)
         dy = gemm_nt(dv2, transpose(p_out_w), T)
         xhT = transpose(xh)  # (D, M)
@@ -260,7 +307,7 @@ class _TriMul(torch.autograd.Function):
             gemm_nt(a, transpose(dt), T, out=db)  # db[k, j] = sum_i a[k, i] dt[i, j]
 
         # input gate and projections
-        du1, dv1 = gate_bwd(dab, u1, v1, g_in_b, p_in_b, 0, mflat, 1)  # (2D, M)
+        du1, dv1 = dual_gate_bwd(dab, g_in_w, p_in_w, xh, None, g_in_b, p_in_b, 0, mflat, 1)  # (2D, M)
         gemm_nt(transpose(du1), transpose(g_in_w), T, out=dxh, accumulate=True)
         gemm_nt(transpose(dv1), transpose(p_in_w), T, out=dxh, accumulate=True)
         d_g_in_w = d_p_in_w = d_g_in_b = d_p_in_b = None

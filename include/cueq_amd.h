@@ -188,6 +188,16 @@ int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int6
                  int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
                  int64_t batch, double alpha, int32_t accumulate, void* stream);
 
+/* The gated dual projection in one kernel (_sigmoid_gated_dual_gemm.py:111-218): u = A1 B1^T, v = A2 B2^T (A* M x K, B* N x K,
+ * contraction contiguous; B2 NULL: same as B1), then
+ *   backward == 0:  out1 = sigmoid(u + bias1) * (v + bias2) * mask
+ *   backward != 0:  out1 = d u, out2 = d v from the cotangent dC of that output (u, v are recomputed, never stored).
+ * Biases / mask (may be NULL) are indexed by the row (axis 0) or column (axis 1) of the M x N result; ldc is the row
+ * stride of dC, out1, out2.  K, lda, ldb and the operand pointers must be multiples of 16 bytes. */
+int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_t K, const void* A1, const void* A2, int64_t lda,
+                   const void* B1, const void* B2, int64_t ldb, const void* bias1, const void* bias2, int32_t bias_axis,
+                   const void* mask, int32_t mask_axis, const void* dC, void* out1, void* out2, int64_t ldc, void* stream);
+
 /* Weight-gradient shaped product C (M x N) = sum over rows z and parts p of A[z, p*stride_a : +M]^T B[z, p*stride_b : +N]
  * (both operands row-major with the long index z as rows).  The rows are cut into chunks; item (chunk, part) writes
  * alpha * its partial product to partials[item] (float32, M x N); the caller adds the cueq_gemm_tn_items(rows, nparts)
