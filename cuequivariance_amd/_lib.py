@@ -39,6 +39,7 @@ EXPORTED_SYMBOLS = (
     "cueq_seg_rowdot",
     "cueq_gemm_nt",
     "cueq_dual_gate",
+    "cueq_gate_bwd_input",
     "cueq_gemm_tn_items",
     "cueq_gemm_tn",
     "cueq_transpose",
@@ -171,6 +172,9 @@ def load() -> C.CDLL:
         lib.cueq_gemm_nt.restype = C.c_int
         lib.cueq_dual_gate.argtypes = [i32, i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i32, ptr, i32, ptr, ptr, ptr, i64, ptr]
         lib.cueq_dual_gate.restype = C.c_int
+        lib.cueq_gate_bwd_input.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, ptr, ptr, i64,
+                                            i32, ptr, ptr, i64, i32, ptr, ptr, ptr]
+        lib.cueq_gate_bwd_input.restype = C.c_int
         lib.cueq_gemm_tn_items.argtypes = [i64, i32]
         lib.cueq_gemm_tn_items.restype = i64
         lib.cueq_gemm_tn.argtypes = [i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, i32, ptr, f64, ptr]

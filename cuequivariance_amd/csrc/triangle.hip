@@ -396,6 +396,247 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Backward of the gated dual projection down to the projection inputs, in one kernel:
+//   u[c][m] = W1[c,:] . X1[m,:],  v[c][m] = W2[c,:] . X2[m,:]        (recomputed, K = 32 * KT)
+//   s = sigmoid(u + b1[c]),  d = dC * mask[m],  du = d (v + b2[c]) s (1 - s),  dv = d s
+//   dX1[m,:] (+)= sum_c du[c][m] W1[c,:] (+ sum_c dv[c][m] W2[c,:] unless SPLIT),   SPLIT: dX2[m,:] = sum_c dv[c][m] W2[c,:]
+// A wavefront owns 32 columns m for the whole kernel and walks the rows c in chunks of 32.  The 32 x 32 MFMA result
+// holds, per lane, one m and 16 values of c - exactly an operand of the next MFMA with m as the row and c as the
+// contraction - so du and dv go from the accumulator straight into the second product and never touch memory
+// (they are written only when the caller asks for them, for the weight gradients).  X fragments stay in registers;
+// weight chunks are double-buffered in LDS (row-major for the first product; for 2-byte types a transposed copy
+// W^T supplies the second product's operand, float32 reads the row-major chunk column-wise).
+// ------------------------------------------------------------------------------------------------
+template <typename TI>
+__device__ __forceinline__ void mma_step(floatx16& acc, const uint4& a, const uint4& b) {
+  if constexpr (sizeof(TI) == 2) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+  } else {
+    const float* pa = reinterpret_cast<const float*>(&a);
+    const float* pb = reinterpret_cast<const float*>(&b);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[e], pb[e], acc, 0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
+}
+
+template <typename TI, int KT, bool SPLIT>
+__global__ void __launch_bounds__(256, SPLIT ? 1 : 2)
+    gate_bwd_input_kernel(const TI* __restrict__ W1, const TI* __restrict__ W2, int64_t ldw, const TI* __restrict__ W1T,
+                          const TI* __restrict__ W2T, int64_t ldwt, const TI* __restrict__ X1, const TI* __restrict__ X2, int64_t ldx,
+                          const TI* __restrict__ bias1, const TI* __restrict__ bias2, const TI* __restrict__ mask,
+                          const TI* __restrict__ dC, int64_t ldc, int dc_by_row, TI* __restrict__ dX1, TI* __restrict__ dX2,
+                          int64_t lddx, int accumulate, TI* __restrict__ dU, TI* __restrict__ dV, int C, int M) {
+  constexpr bool BF = sizeof(TI) == 2;
+  constexpr int EPV = 16 / sizeof(TI);
+  constexpr int K = 32 * KT;
+  constexpr int ROWB = K * sizeof(TI);  // bytes of one weight row
+  constexpr int WSTR = ROWB + 16;       // LDS row stride of a row-major chunk (32 rows)
+  constexpr int NS = ROWB / 64;         // 64-byte contraction steps of the first product
+  constexpr int WBYTES = 32 * WSTR;
+  constexpr int TSTR = 72;              // LDS row stride of a transposed chunk: 32 c = 64 bytes + 8 (conflict-free 8-byte reads)
+  constexpr int TBYTES = BF ? K * TSTR : 0;
+  constexpr int BUF = 2 * WBYTES + 2 * TBYTES;
+  constexpr int VPR = ROWB / 16, NWV = 32 * VPR, NW = (NWV + 255) / 256;
+  constexpr int NTV = BF ? K * 4 : 0, NTQ = BF ? (NTV + 255) / 256 : 1;
+  __shared__ __align__(16) char smem[2][BUF];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int mcol = blockIdx.x * kTile + wave * 32 + c;  // this lane's m in the first product (column) ...
+  const int mld = min(mcol, M - 1);
+  const int mrow0 = blockIdx.x * kTile + wave * 32;     // ... and the wavefront's first m in the second (rows by v)
+
+  uint4 stw[2][NW], stt[2][NTQ];
+  auto load_chunk = [&](int c0) {
+#pragma unroll
+    for (int q = 0; q < NW; ++q) {
+      const int e = tid + q * 256;
+      if (NWV % 256 == 0 || e < NWV) {
+        const int64_t o = static_cast<int64_t>(c0 + e / VPR) * ldw + (e % VPR) * EPV;
+        stw[0][q] = *reinterpret_cast<const uint4*>(W1 + o);
+        stw[1][q] = *reinterpret_cast<const uint4*>(W2 + o);
+      }
+    }
+    if constexpr (BF) {
+#pragma unroll
+      for (int q = 0; q < NTQ; ++q) {
+        const int e = tid + q * 256;
+        if (NTV % 256 == 0 || e < NTV) {
+          const int64_t o = static_cast<int64_t>(e >> 2) * ldwt + c0 + (e & 3) * 8;
+          stt[0][q] = *reinterpret_cast<const uint4*>(W1T + o);
+          stt[1][q] = *reinterpret_cast<const uint4*>(W2T + o);
+        }
+      }
+    }
+  };
+  auto store_chunk = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < NW; ++q) {
+      const int e = tid + q * 256;
+      if (NWV % 256 == 0 || e < NWV) {
+        const int o = (e / VPR) * WSTR + (e % VPR) * 16;
+        *reinterpret_cast<uint4*>(&smem[buf][o]) = stw[0][q];
+        *reinterpret_cast<uint4*>(&smem[buf][WBYTES + o]) = stw[1][q];
+      }
+    }
+    if constexpr (BF) {
+#pragma unroll
+      for (int q = 0; q < NTQ; ++q) {
+        const int e = tid + q * 256;
+        if (NTV % 256 == 0 || e < NTV) {
+          const int o = 2 * WBYTES + (e >> 2) * TSTR + (e & 3) * 16;
+          *reinterpret_cast<uint2*>(&smem[buf][o]) = make_uint2(stt[0][q].x, stt[0][q].y);
+          *reinterpret_cast<uint2*>(&smem[buf][o + 8]) = make_uint2(stt[0][q].z, stt[0][q].w);
+          *reinterpret_cast<uint2*>(&smem[buf][TBYTES + o]) = make_uint2(stt[1][q].x, stt[1][q].y);
+          *reinterpret_cast<uint2*>(&smem[buf][TBYTES + o + 8]) = make_uint2(stt[1][q].z, stt[1][q].w);
+        }
+      }
+    }
+  };
+
+  // fragments of X for this lane's m: lane half h holds bytes [64 s + 32 h, +32) of the row
+  uint4 xf1[NS][2], xf2[SPLIT ? NS : 1][2];
+#pragma unroll
+  for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int64_t o = static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / static_cast<int>(sizeof(TI));
+      xf1[s2][q] = *reinterpret_cast<const uint4*>(X1 + o);
+      if constexpr (SPLIT) xf2[s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
+    }
+  const float mk = mask ? tri_load(mask, mld) : 1.0f;
+
+  floatx16 ax1[KT], ax2[SPLIT ? KT : 1];
+#pragma unroll
+  for (int t = 0; t < KT; ++t) ax1[t] = floatx16{0};
+#pragma unroll
+  for (int t = 0; t < (SPLIT ? KT : 1); ++t) ax2[t] = floatx16{0};
+
+  const int nchunks = C / 32;
+  load_chunk(0);
+  store_chunk(0);
+  __syncthreads();
+  for (int ci = 0; ci < nchunks; ++ci) {
+    const int c0 = ci * 32, buf = ci & 1;
+    if (ci + 1 < nchunks) load_chunk(c0 + 32);
+
+    // cotangent of this chunk: value v of the lane belongs to row c0 + 8 (v >> 2) + 4 h + (v & 3)
+    float dc[16];
+    if (dc_by_row) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dc[v] = tri_load(dC, static_cast<int64_t>(c0 + 8 * (v >> 2) + 4 * h + (v & 3)) * ldc + mld);
+    } else {
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const TI* p = dC + static_cast<int64_t>(mld) * ldc + c0 + 8 * a + 4 * h;
+        if constexpr (BF) {
+          const uint2 w = *reinterpret_cast<const uint2*>(p);
+          dc[4 * a] = __uint_as_float(w.x << 16); dc[4 * a + 1] = __uint_as_float(w.x & 0xffff0000u);
+          dc[4 * a + 2] = __uint_as_float(w.y << 16); dc[4 * a + 3] = __uint_as_float(w.y & 0xffff0000u);
+        } else {
+          const float4 w = *reinterpret_cast<const float4*>(p);
+          dc[4 * a] = w.x; dc[4 * a + 1] = w.y; dc[4 * a + 2] = w.z; dc[4 * a + 3] = w.w;
+        }
+      }
+    }
+
+    // first product: u, v for 32 rows c x 32 columns m
+    floatx16 au = floatx16{0}, av = floatx16{0};
+    {
+      const char* w1 = &smem[buf][c * WSTR + h * 32];
+#pragma unroll
+      for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const uint4 a1 = *reinterpret_cast<const uint4*>(w1 + s2 * 64 + q * 16);
+          const uint4 a2 = *reinterpret_cast<const uint4*>(w1 + WBYTES + s2 * 64 + q * 16);
+          mma_step<TI>(au, a1, xf1[s2][q]);
+          mma_step<TI>(av, a2, SPLIT ? xf2[s2][q] : xf1[s2][q]);
+        }
+    }
+
+    // gate backward in registers
+    float du[16], dv[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = c0 + 8 * (v >> 2) + 4 * h + (v & 3);
+      const float uu = au[v] + (bias1 ? tri_load(bias1, row) : 0.f);
+      const float vv = av[v] + (bias2 ? tri_load(bias2, row) : 0.f);
+      const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-uu));
+      const float d = dc[v] * mk;
+      du[v] = d * vv * sg * (1.0f - sg);
+      dv[v] = d * sg;
+    }
+    if (dU != nullptr && mcol < M) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = c0 + 8 * (v >> 2) + 4 * h + (v & 3);
+        const int64_t o = dc_by_row ? static_cast<int64_t>(row) * ldc + mcol : static_cast<int64_t>(mcol) * ldc + row;
+        tri_store(dU, o, du[v]);
+        tri_store(dV, o, dv[v]);
+      }
+    }
+
+    // second product: rows m (lanes of the operand), contraction over the 32 rows c of the chunk
+    if constexpr (BF) {
+      uint4 pu[2], pv[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        pu[t] = make_uint4(pack_bf16(du[8 * t], du[8 * t + 1]), pack_bf16(du[8 * t + 2], du[8 * t + 3]),
+                           pack_bf16(du[8 * t + 4], du[8 * t + 5]), pack_bf16(du[8 * t + 6], du[8 * t + 7]));
+        pv[t] = make_uint4(pack_bf16(dv[8 * t], dv[8 * t + 1]), pack_bf16(dv[8 * t + 2], dv[8 * t + 3]),
+                           pack_bf16(dv[8 * t + 4], dv[8 * t + 5]), pack_bf16(dv[8 * t + 6], dv[8 * t + 7]));
+      }
+      const char* t1 = &smem[buf][2 * WBYTES + c * TSTR + h * 8];
+#pragma unroll
+      for (int ds = 0; ds < KT; ++ds)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const char* p1 = t1 + ds * 32 * TSTR + t * 32;
+          const uint2 l1 = *reinterpret_cast<const uint2*>(p1), h1 = *reinterpret_cast<const uint2*>(p1 + 16);
+          const uint2 l2 = *reinterpret_cast<const uint2*>(p1 + TBYTES), h2 = *reinterpret_cast<const uint2*>(p1 + TBYTES + 16);
+          mma_step<TI>(ax1[ds], pu[t], make_uint4(l1.x, l1.y, h1.x, h1.y));
+          mma_step<TI>(SPLIT ? ax2[ds] : ax1[ds], pv[t], make_uint4(l2.x, l2.y, h2.x, h2.y));
+        }
+    } else {
+#pragma unroll
+      for (int ds = 0; ds < KT; ++ds)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const char* p1 = &smem[buf][(8 * (v >> 2) + 4 * h + (v & 3)) * WSTR + (ds * 32 + c) * 4];
+          const float w1 = *reinterpret_cast<const float*>(p1), w2 = *reinterpret_cast<const float*>(p1 + WBYTES);
+          ax1[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(du[v], w1, ax1[ds], 0, 0, 0);
+          if constexpr (SPLIT) ax2[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(dv[v], w2, ax2[ds], 0, 0, 0);
+          else ax1[ds] = __builtin_amdgcn_mfma_f32_32x32x2f32(dv[v], w2, ax1[ds], 0, 0, 0);
+        }
+    }
+
+    if (ci + 1 < nchunks) store_chunk(buf ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int ds = 0; ds < KT; ++ds) {
+    const int col = ds * 32 + c;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = mrow0 + 8 * (v >> 2) + 4 * h + (v & 3);
+      if (row < M) {
+        const int64_t o = static_cast<int64_t>(row) * lddx + col;
+        float val = ax1[ds][v];
+        if (accumulate) val += tri_load(dX1, o);
+        tri_store(dX1, o, val);
+        if constexpr (SPLIT) tri_store(dX2, o, ax2[ds][v]);
+      }
+    }
+  }
+}
+
 // any shape / alignment: one thread per output element
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(256) gemm_nt_simple(const TI* __restrict__ A, int64_t lda, int64_t sA, const TI* __restrict__ B,
@@ -853,6 +1094,43 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
   TRI_DISPATCH(dtype, DG_T(float), DG_T(uint16_t));
 #undef DG_T
 #undef DG
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
+                                   const void* W1T, const void* W2T, int64_t ldwt, const void* X1, const void* X2, int64_t ldx,
+                                   const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
+                                   int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
+                                   void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: dtype must be float32 or bfloat16");
+  CUEQ_REQUIRE(C >= 0 && M >= 0 && K > 0, CUEQ_ERR_INVALID, "gate_bwd_input: bad extents");
+  if (M == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(K % 32 == 0 && K <= 128, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: K must be 32, 64, 96 or 128");
+  CUEQ_REQUIRE(C % 32 == 0 && C > 0, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: C must be a positive multiple of 32");
+  CUEQ_REQUIRE(M < (1ll << 31) - kTile && C < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gate_bwd_input: extent too large");
+  CUEQ_REQUIRE(W1 && W2 && X1 && dC && dX1 && (!dU == !dV), CUEQ_ERR_INVALID, "gate_bwd_input: null operand");
+  const bool bf = dtype == CUEQ_BF16;
+  CUEQ_REQUIRE(!bf || (W1T && W2T), CUEQ_ERR_INVALID, "gate_bwd_input: bfloat16 needs the transposed weights");
+  const bool split = X2 != nullptr && X2 != X1;
+  CUEQ_REQUIRE(!split || dX2, CUEQ_ERR_INVALID, "gate_bwd_input: two inputs need two gradients");
+  CUEQ_REQUIRE(!(split && accumulate), CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: accumulate needs a single input");
+  const int epv = bf ? 8 : 4;
+  const uintptr_t ptrs = reinterpret_cast<uintptr_t>(W1) | reinterpret_cast<uintptr_t>(W2) | reinterpret_cast<uintptr_t>(W1T) |
+                         reinterpret_cast<uintptr_t>(W2T) | reinterpret_cast<uintptr_t>(X1) | reinterpret_cast<uintptr_t>(X2) |
+                         (dc_by_row ? 0 : reinterpret_cast<uintptr_t>(dC));
+  const bool aligned = (ptrs & 15) == 0 && ldw % epv == 0 && ldx % epv == 0 && (!bf || ldwt % epv == 0) && (dc_by_row || ldc % epv == 0);
+  CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: row strides and pointers must be multiples of 16 bytes");
+  const dim3 grid(static_cast<unsigned>((M + kTile - 1) / kTile));
+  KernelTimer timer("gate_bwd_input", stream);
+#define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP>), grid, dim3(256), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(W1T), static_cast<const TI*>(W2T), ldwt, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, dc_by_row, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
+#define GBI_K(TI, SP) do { switch (K / 32) { case 1: GBI(TI, 1, SP); break; case 2: GBI(TI, 2, SP); break; case 3: GBI(TI, 3, SP); break; default: GBI(TI, 4, SP); break; } } while (0)
+#define GBI_T(TI) do { if (split) GBI_K(TI, true); else GBI_K(TI, false); } while (0)
+  TRI_DISPATCH(dtype, GBI_T(float), GBI_T(uint16_t));
+#undef GBI_T
+#undef GBI_K
+#undef GBI
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }

@@ -192,6 +192,36 @@ def dual_gate_bwd(dout, A1, A2, B1, B2, bias1, bias2, bias_axis: int, mask, mask
     return gate_bwd(dout, u, v, bias1, bias2, bias_axis, mask, mask_axis)
 
 
+def gate_bwd_input(dC, dc_by_row: bool, W1, W2, X1, X2, bias1, bias2, mask, dX1=None, want_gate_grads: bool = False):
+    """Backward of ``sigmoid(W1 X1^T + b1) * (W2 X2^T + b2) * mask`` (rows ``c``, columns ``m``) down to ``X1``/``X2``
+    in one kernel (``cueq_gate_bwd_input``); ``dC`` is ``(C, M)`` when ``dc_by_row`` else ``(M, C)``.  ``X2 is None``: one
+    input, whose gradient is added to ``dX1`` when that is given.  Returns ``(dX1, dX2, dU, dV)`` (``dU, dV`` in the layout
+    of ``dC``, only when ``want_gate_grads``), or ``None`` when the shapes do not allow the fused kernel."""
+    Cn, K = W1.shape
+    M = X1.shape[0]
+    T = W1.dtype
+    es = W1.element_size()
+    if K % 32 or K > 128 or Cn % 32 or not _fusable(W1, W2, X1, X2, dC, dX1):
+        return None
+    bf = T == torch.bfloat16
+    W1T = transpose(W1) if bf else None
+    W2T = transpose(W2) if bf else None
+    accumulate = dX1 is not None
+    if dX1 is None:
+        dX1 = torch.empty(M, K, dtype=T, device=W1.device)
+    dX2 = torch.empty(M, K, dtype=T, device=W1.device) if X2 is not None else None
+    dU = torch.empty_like(dC) if want_gate_grads else None
+    dV = torch.empty_like(dC) if want_gate_grads else None
+    _lib.check(
+        _lib.load().cueq_gate_bwd_input(_CODE[T], Cn, M, K, W1.data_ptr(), W2.data_ptr(), W1.stride(0), _ptr(W1T), _ptr(W2T), Cn,
+                                        X1.data_ptr(), _ptr(X2), X1.stride(0), _ptr(bias1), _ptr(bias2), _ptr(mask), dC.data_ptr(),
+                                        dC.stride(0), int(dc_by_row), dX1.data_ptr(), _ptr(dX2), dX1.stride(0), int(accumulate),
+                                        _ptr(dU), _ptr(dV), _stream(W1)),
+        "cueq_gate_bwd_input",
+    )
+    return dX1, dX2, dU, dV
+
+
 def sum_cols(x: torch.Tensor) -> torch.Tensor:
     rows, cols = x.shape
     out = torch.empty(rows, dtype=torch.float32, device=x.device)
@@ -274,10 +304,16 @@ class _TriMul(torch.autograd.Function):
         dout = dout.contiguous().view(M, Do).to(T)
 
         # output gate
-        du2, dv2 = dual_gate_bwd(dout, xh, y, g_out_w, p_out_w, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
-        dxh = gemm_nt(du2, transpose(g_out_w), T)  # (M, D)
-        dy = gemm_nt(dv2, transpose(p_out_w), T)
-        xhT = transpose(xh)  # (D, M)
+        w_out = need[10] or need[11] or need[12] or need[13]
+        fused = gate_bwd_input(dout, False, g_out_w, p_out_w, xh, y, g_out_b, p_out_b, None, None, w_out)
+        if fused is not None:
+            dxh, dy, du2, dv2 = fused
+        else:
+            du2, dv2 = dual_gate_bwd(dout, xh, y, g_out_w, p_out_w, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
+            dxh = gemm_nt(du2, transpose(g_out_w), T)  # (M, D)
+            dy = gemm_nt(dv2, transpose(p_out_w), T)
+        w_in = need[4] or need[5] or need[6] or need[7]
+        xhT = transpose(xh) if (w_in or need[12]) else None  # (D, M)
         d_g_out_w = d_p_out_w = d_g_out_b = d_p_out_b = None
         if need[12]:
             d_g_out_w = gemm_long_k(transpose(du2), xhT).to(g_out_w.dtype)
@@ -307,9 +343,13 @@ class _TriMul(torch.autograd.Function):
             gemm_nt(a, transpose(dt), T, out=db)  # db[k, j] = sum_i a[k, i] dt[i, j]
 
         # input gate and projections
-        du1, dv1 = dual_gate_bwd(dab, g_in_w, p_in_w, xh, None, g_in_b, p_in_b, 0, mflat, 1)  # (2D, M)
-        gemm_nt(transpose(du1), transpose(g_in_w), T, out=dxh, accumulate=True)
-        gemm_nt(transpose(dv1), transpose(p_in_w), T, out=dxh, accumulate=True)
+        fused = gate_bwd_input(dab, True, g_in_w, p_in_w, xh, None, g_in_b, p_in_b, mflat, dxh, w_in)
+        if fused is not None:
+            du1, dv1 = fused[2], fused[3]
+        else:
+            du1, dv1 = dual_gate_bwd(dab, g_in_w, p_in_w, xh, None, g_in_b, p_in_b, 0, mflat, 1)  # (2D, M)
+            gemm_nt(transpose(du1), transpose(g_in_w), T, out=dxh, accumulate=True)
+            gemm_nt(transpose(dv1), transpose(p_in_w), T, out=dxh, accumulate=True)
         d_g_in_w = d_p_in_w = d_g_in_b = d_p_in_b = None
         if need[6]:
             d_g_in_w = gemm_long_k(du1, xhT).to(g_in_w.dtype)

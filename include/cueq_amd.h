@@ -198,6 +198,21 @@ int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_
                    const void* B1, const void* B2, int64_t ldb, const void* bias1, const void* bias2, int32_t bias_axis,
                    const void* mask, int32_t mask_axis, const void* dC, void* out1, void* out2, int64_t ldc, void* stream);
 
+/* Backward of the gated dual projection down to the projection inputs (_sigmoid_gated_dual_gemm.py:153-218), one kernel:
+ *   u[c][m] = W1[c,:] . X1[m,:],  v[c][m] = W2[c,:] . X2[m,:]   (W* C x K row-major with row stride ldw, X* M x K; recomputed)
+ *   s = sigmoid(u + bias1[c]),  d = dC * mask[m],  du = d (v + bias2[c]) s (1 - s),  dv = d s
+ *   X2 NULL or == X1:  dX1[m,:] (+)= sum_c du W1[c,:] + dv W2[c,:]          (accumulate != 0 adds to dX1)
+ *   otherwise:         dX1[m,:]  =  sum_c du W1[c,:],   dX2[m,:] = sum_c dv W2[c,:]
+ * dC (and dU, dV when not NULL: the gate gradients for the weight / bias gradients) are C x M with row stride ldc when
+ * dc_by_row != 0, M x C otherwise.  bfloat16 also takes the transposed weights W1T, W2T (K x C, row stride ldwt).
+ * K must be 32, 64, 96 or 128 and C a multiple of 32; strides and pointers multiples of 16 bytes, else
+ * CUEQ_ERR_UNSUPPORTED (compose cueq_dual_gate and cueq_gemm_nt instead). */
+int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
+                        const void* W1T, const void* W2T, int64_t ldwt, const void* X1, const void* X2, int64_t ldx,
+                        const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
+                        int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
+                        void* stream);
+
 /* Weight-gradient shaped product C (M x N) = sum over rows z and parts p of A[z, p*stride_a : +M]^T B[z, p*stride_b : +N]
  * (both operands row-major with the long index z as rows).  The rows are cut into chunks; item (chunk, part) writes
  * alpha * its partial product to partials[item] (float32, M x N); the caller adds the cueq_gemm_tn_items(rows, nparts)

@@ -107,6 +107,25 @@ def test_hip_path_matches_oracle(device, dtype, direction, shape):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 40, 128, None), (1, 33, 96, 64), (1, 16, 160, None)])
+def test_input_gradient_only(device, dtype, shape):
+    """Only x asks for a gradient (the benchmark's case): the gate gradients then stay in registers (D <= 128) or go
+    through the unfused kernels (D = 160)."""
+    from cuequivariance_amd import cuet
+
+    Bsz, N, D, Do = shape
+    p, cot = make_case(Bsz, N, D, dtype, 5, Do=Do)
+    pr = {k: v.clone() for k, v in p.items()}
+    pr["x"].requires_grad_(True)
+    (want,) = torch.autograd.grad(oracle_trimul(direction="outgoing", **pr), [pr["x"]], cot)
+    pg = {k: v.to(dtype).to(device) for k, v in p.items()}
+    pg["x"].requires_grad_(True)
+    (got,) = torch.autograd.grad(cuet.triangle_multiplicative_update(direction="outgoing", **pg), [pg["x"]], cot.to(dtype).to(device))
+    assert rel_err(got, want) <= TOL[dtype], rel_err(got, want)
+
+
+@pytest.mark.gpu
 def test_defaults_shapes_and_errors(device):
     """The reference's own test: no weights given, shapes only (triangle_test.py:97-118); plus argument checks."""
     from cuequivariance_amd import cuet
