@@ -420,16 +420,53 @@ __device__ __forceinline__ void mma_step(floatx16& acc, const uint4& a, const ui
   }
 }
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
+// A wavefront-uniform address, pinned to scalar registers so that loads take the "scalar base + 32-bit lane offset" form
+// instead of one 64-bit vector address per access.
+__device__ __forceinline__ const char* uniform_ptr(const void* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+  return reinterpret_cast<const char*>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
-template <typename TI, int KT, bool SPLIT>
-__global__ void __launch_bounds__(256, SPLIT ? 1 : 2)
+template <typename V>
+__device__ __forceinline__ V load_global(const char* uniform_base, uint32_t lane_offset) {
+  typedef const __attribute__((address_space(1))) V* gptr;
+  return *reinterpret_cast<gptr>(reinterpret_cast<uint64_t>(uniform_base) + lane_offset);
+}
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+template <>
+__device__ __forceinline__ uint4 load_global<uint4>(const char* uniform_base, uint32_t lane_offset) {
+  const u32x4_t v = load_global<u32x4_t>(uniform_base, lane_offset);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+template <>
+__device__ __forceinline__ uint2 load_global<uint2>(const char* uniform_base, uint32_t lane_offset) {
+  const u32x2_t v = load_global<u32x2_t>(uniform_base, lane_offset);
+  return make_uint2(v.x, v.y);
+}
+
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {  // round to nearest even, one v_cvt_pk_bf16_f32
+  const floatx2_t f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
+// 2-byte single-input case: 8 wavefronts (256 columns m) per block at 2 wavefronts per SIMD; the others need more
+// registers per wavefront and run 4 wavefronts per block at 1 per SIMD.
+template <typename TI, bool SPLIT>
+constexpr int gbi_threads() { return (sizeof(TI) == 2 && !SPLIT) ? 512 : 256; }
+
+// DC_BY_ROW: dC, dU, dV are C x M (else M x C).  Addresses inside the loop are a uniform 64-bit base plus a 32-bit
+// lane offset (the host checks the extents), which keeps them out of the vector registers.
+template <typename TI, int KT, bool SPLIT, bool DC_BY_ROW>
+__global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_threads<TI, SPLIT>() == 512 ? 2 : 1))
     gate_bwd_input_kernel(const TI* __restrict__ W1, const TI* __restrict__ W2, int64_t ldw, const TI* __restrict__ W1T,
                           const TI* __restrict__ W2T, int64_t ldwt, const TI* __restrict__ X1, const TI* __restrict__ X2, int64_t ldx,
                           const TI* __restrict__ bias1, const TI* __restrict__ bias2, const TI* __restrict__ mask,
-                          const TI* __restrict__ dC, int64_t ldc, int dc_by_row, TI* __restrict__ dX1, TI* __restrict__ dX2,
+                          const TI* __restrict__ dC, int64_t ldc, TI* __restrict__ dX1, TI* __restrict__ dX2,
                           int64_t lddx, int accumulate, TI* __restrict__ dU, TI* __restrict__ dV, int C, int M) {
   constexpr bool BF = sizeof(TI) == 2;
   constexpr int EPV = 16 / sizeof(TI);
@@ -440,55 +477,86 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2)
   constexpr int WBYTES = 32 * WSTR;
   constexpr int TSTR = 72;              // LDS row stride of a transposed chunk: 32 c = 64 bytes + 8 (conflict-free 8-byte reads)
   constexpr int TBYTES = BF ? K * TSTR : 0;
-  constexpr int BUF = 2 * WBYTES + 2 * TBYTES;
-  constexpr int VPR = ROWB / 16, NWV = 32 * VPR, NW = (NWV + 255) / 256;
-  constexpr int NTV = BF ? K * 4 : 0, NTQ = BF ? (NTV + 255) / 256 : 1;
+  constexpr int BIAS = 2 * WBYTES + 2 * TBYTES;  // offset of the chunk's biases (2 x 32 float)
+  constexpr int BUF = BIAS + 256;
+  constexpr int NTH = gbi_threads<TI, SPLIT>(), BM = NTH / 2;  // threads and columns m per block
+  constexpr int VPR = ROWB / 16, NWV = 32 * VPR, NW = (NWV + NTH - 1) / NTH;
+  constexpr int NTV = BF ? K * 4 : 0, NTQ = BF ? (NTV + NTH - 1) / NTH : 1;
   __shared__ __align__(16) char smem[2][BUF];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
-  const int mcol = blockIdx.x * kTile + wave * 32 + c;  // this lane's m in the first product (column) ...
+  const int mcol = blockIdx.x * BM + wave * 32 + c;  // this lane's m in the first product (column) ...
   const int mld = min(mcol, M - 1);
-  const int mrow0 = blockIdx.x * kTile + wave * 32;     // ... and the wavefront's first m in the second (rows by v)
+  const int mrow0 = blockIdx.x * BM + wave * 32;     // ... and the wavefront's first m in the second (rows by v)
 
+  constexpr int ES = sizeof(TI);
   uint4 stw[2][NW], stt[2][NTQ];
-  auto load_chunk = [&](int c0) {
+  uint32_t wofs[NW], tofs[NTQ];
+#pragma unroll
+  for (int q = 0; q < NW; ++q) {
+    const int e = min(tid + q * NTH, NWV - 1);
+    wofs[q] = static_cast<uint32_t>(((e / VPR) * ldw + (e % VPR) * EPV) * ES);
+  }
+#pragma unroll
+  for (int q = 0; q < NTQ; ++q) {
+    const int e = min(tid + q * NTH, (BF ? NTV : 1) - 1);
+    tofs[q] = static_cast<uint32_t>(((e >> 2) * ldwt + (e & 3) * 8) * ES);
+  }
+  // biases of the chunk: threads 0..31 / 32..63 (of every 64) fetch bias1 / bias2, the first 64 threads store them
+  const TI* bsrc = (tid & 32) ? bias2 : bias1;
+  const bool has_bias = bsrc != nullptr;
+  const char* bptr = reinterpret_cast<const char*>(has_bias ? bsrc : W1);
+  const uint32_t bofs = has_bias ? static_cast<uint32_t>((tid & 31) * ES) : 0u;
+  TI stb;
+  // the row-major chunk and the biases are fetched at the top of an iteration and stored after the first product,
+  // the transposed chunk is fetched then and stored at the end: half the staging registers are live at a time
+  auto load_rows = [&](int c0) {
+    stb = *reinterpret_cast<const TI*>(bptr + (has_bias ? static_cast<int64_t>(c0) * ES : 0) + bofs);  // bptr differs by lane
+    const char* w1 = uniform_ptr(reinterpret_cast<const char*>(W1) + static_cast<int64_t>(c0) * ldw * ES);
+    const char* w2 = uniform_ptr(reinterpret_cast<const char*>(W2) + static_cast<int64_t>(c0) * ldw * ES);
 #pragma unroll
     for (int q = 0; q < NW; ++q) {
-      const int e = tid + q * 256;
-      if (NWV % 256 == 0 || e < NWV) {
-        const int64_t o = static_cast<int64_t>(c0 + e / VPR) * ldw + (e % VPR) * EPV;
-        stw[0][q] = *reinterpret_cast<const uint4*>(W1 + o);
-        stw[1][q] = *reinterpret_cast<const uint4*>(W2 + o);
-      }
+      stw[0][q] = load_global<uint4>(w1, wofs[q]);
+      stw[1][q] = load_global<uint4>(w2, wofs[q]);
     }
+  };
+  auto load_cols = [&](int c0) {
     if constexpr (BF) {
+      const char* t1 = uniform_ptr(reinterpret_cast<const char*>(W1T) + static_cast<int64_t>(c0) * ES);
+      const char* t2 = uniform_ptr(reinterpret_cast<const char*>(W2T) + static_cast<int64_t>(c0) * ES);
 #pragma unroll
       for (int q = 0; q < NTQ; ++q) {
-        const int e = tid + q * 256;
-        if (NTV % 256 == 0 || e < NTV) {
-          const int64_t o = static_cast<int64_t>(e >> 2) * ldwt + c0 + (e & 3) * 8;
-          stt[0][q] = *reinterpret_cast<const uint4*>(W1T + o);
-          stt[1][q] = *reinterpret_cast<const uint4*>(W2T + o);
-        }
+        stt[0][q] = load_global<uint4>(t1, tofs[q]);
+        stt[1][q] = load_global<uint4>(t2, tofs[q]);
       }
     }
   };
-  auto store_chunk = [&](int buf) {
+  auto store_rows = [&](int buf) {
+    if (tid < 64) {
+      float bv = 0.f;
+      if (has_bias) {
+        if constexpr (BF) bv = bf16_bits_to_float(stb);
+        else bv = stb;
+      }
+      *reinterpret_cast<float*>(&smem[buf][BIAS + tid * 4]) = bv;
+    }
 #pragma unroll
     for (int q = 0; q < NW; ++q) {
-      const int e = tid + q * 256;
-      if (NWV % 256 == 0 || e < NWV) {
+      const int e = tid + q * NTH;
+      if (NWV % NTH == 0 || e < NWV) {
         const int o = (e / VPR) * WSTR + (e % VPR) * 16;
         *reinterpret_cast<uint4*>(&smem[buf][o]) = stw[0][q];
         *reinterpret_cast<uint4*>(&smem[buf][WBYTES + o]) = stw[1][q];
       }
     }
+  };
+  auto store_cols = [&](int buf) {
     if constexpr (BF) {
 #pragma unroll
       for (int q = 0; q < NTQ; ++q) {
-        const int e = tid + q * 256;
-        if (NTV % 256 == 0 || e < NTV) {
+        const int e = tid + q * NTH;
+        if (NTV % NTH == 0 || e < NTV) {
           const int o = 2 * WBYTES + (e >> 2) * TSTR + (e & 3) * 16;
           *reinterpret_cast<uint2*>(&smem[buf][o]) = make_uint2(stt[0][q].x, stt[0][q].y);
           *reinterpret_cast<uint2*>(&smem[buf][o + 8]) = make_uint2(stt[0][q].z, stt[0][q].w);
@@ -517,33 +585,52 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2)
 #pragma unroll
   for (int t = 0; t < (SPLIT ? KT : 1); ++t) ax2[t] = floatx16{0};
 
-  const int nchunks = C / 32;
-  load_chunk(0);
-  store_chunk(0);
-  __syncthreads();
-  for (int ci = 0; ci < nchunks; ++ci) {
-    const int c0 = ci * 32, buf = ci & 1;
-    if (ci + 1 < nchunks) load_chunk(c0 + 32);
-
-    // cotangent of this chunk: value v of the lane belongs to row c0 + 8 (v >> 2) + 4 h + (v & 3)
-    float dc[16];
-    if (dc_by_row) {
+  // cotangent of a chunk: value v of the lane belongs to row c0 + 8 (v >> 2) + 4 h + (v & 3); fetched one chunk ahead
+  // (kept as loaded - one register per value, or packed pairs when read along c - and widened where it is used)
+  uint32_t dcr[16];
+  const uint32_t dcofs = DC_BY_ROW ? static_cast<uint32_t>((4 * h * ldc + mld) * ES) : static_cast<uint32_t>((mld * ldc + 4 * h) * ES);
+  auto load_dc = [&](int c0) {
+    if constexpr (DC_BY_ROW) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) dc[v] = tri_load(dC, static_cast<int64_t>(c0 + 8 * (v >> 2) + 4 * h + (v & 3)) * ldc + mld);
+      for (int v = 0; v < 16; ++v) {
+        const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * (v >> 2) + (v & 3)) * ldc * ES);
+        if constexpr (BF) dcr[v] = load_global<uint16_t>(base, dcofs);
+        else dcr[v] = load_global<uint32_t>(base, dcofs);
+      }
     } else {
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
-        const TI* p = dC + static_cast<int64_t>(mld) * ldc + c0 + 8 * a + 4 * h;
+        const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * a) * ES);
         if constexpr (BF) {
-          const uint2 w = *reinterpret_cast<const uint2*>(p);
-          dc[4 * a] = __uint_as_float(w.x << 16); dc[4 * a + 1] = __uint_as_float(w.x & 0xffff0000u);
-          dc[4 * a + 2] = __uint_as_float(w.y << 16); dc[4 * a + 3] = __uint_as_float(w.y & 0xffff0000u);
+          const uint2 w = load_global<uint2>(base, dcofs);
+          dcr[4 * a] = w.x; dcr[4 * a + 1] = w.y;  // values 4a..4a+3 in two registers
         } else {
-          const float4 w = *reinterpret_cast<const float4*>(p);
-          dc[4 * a] = w.x; dc[4 * a + 1] = w.y; dc[4 * a + 2] = w.z; dc[4 * a + 3] = w.w;
+          const uint4 w = load_global<uint4>(base, dcofs);
+          dcr[4 * a] = w.x; dcr[4 * a + 1] = w.y; dcr[4 * a + 2] = w.z; dcr[4 * a + 3] = w.w;
         }
       }
     }
+  };
+  auto dc_value = [&](int v) -> float {
+    if constexpr (!BF) return __uint_as_float(dcr[v]);
+    else {
+      if constexpr (DC_BY_ROW) return __uint_as_float(dcr[v] << 16);
+      const uint32_t w = dcr[4 * (v >> 2) + ((v & 3) >> 1)];
+      return (v & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+    }
+  };
+
+  const int nchunks = C / 32;
+  load_rows(0);
+  load_cols(0);
+  load_dc(0);
+  store_rows(0);
+  store_cols(0);
+  __syncthreads();
+  for (int ci = 0; ci < nchunks; ++ci) {
+    const int c0 = ci * 32, buf = ci & 1;
+    const bool more = ci + 1 < nchunks;
+    if (more) load_rows(c0 + 32);
 
     // first product: u, v for 32 rows c x 32 columns m
     floatx16 au = floatx16{0}, av = floatx16{0};
@@ -560,38 +647,45 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2)
         }
     }
 
-    // gate backward in registers
-    float du[16], dv[16];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = c0 + 8 * (v >> 2) + 4 * h + (v & 3);
-      const float uu = au[v] + (bias1 ? tri_load(bias1, row) : 0.f);
-      const float vv = av[v] + (bias2 ? tri_load(bias2, row) : 0.f);
-      const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-uu));
-      const float d = dc[v] * mk;
-      du[v] = d * vv * sg * (1.0f - sg);
-      dv[v] = d * sg;
+    if (more) {
+      store_rows(buf ^ 1);  // the other buffer was last read before the previous barrier
+      load_cols(c0 + 32);
     }
-    if (dU != nullptr && mcol < M) {
+
+    // gate backward in registers; du, dv are packed (2-byte types) as soon as they exist
+    float du[BF ? 4 : 16], dv[BF ? 4 : 16];
+    uint32_t pu[BF ? 8 : 1], pv[BF ? 8 : 1];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = c0 + 8 * (v >> 2) + 4 * h + (v & 3);
-        const int64_t o = dc_by_row ? static_cast<int64_t>(row) * ldc + mcol : static_cast<int64_t>(mcol) * ldc + row;
-        tri_store(dU, o, du[v]);
-        tri_store(dV, o, dv[v]);
+    for (int a = 0; a < 4; ++a) {
+      const float4 b1 = *reinterpret_cast<const float4*>(&smem[buf][BIAS + (8 * a + 4 * h) * 4]);
+      const float4 b2 = *reinterpret_cast<const float4*>(&smem[buf][BIAS + 128 + (8 * a + 4 * h) * 4]);
+      const float b1v[4] = {b1.x, b1.y, b1.z, b1.w}, b2v[4] = {b2.x, b2.y, b2.z, b2.w};
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int v = 4 * a + b;
+        const float uu = au[v] + b1v[b];
+        const float vv = av[v] + b2v[b];
+        const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-uu));
+        const float d = dc_value(v) * mk;
+        const float duv = d * vv * sg * (1.0f - sg), dvv = d * sg;
+        du[BF ? b : v] = duv;
+        dv[BF ? b : v] = dvv;
+        if (dU != nullptr && mcol < M) {
+          const int row = c0 + 8 * a + 4 * h + b;
+          const int64_t o = DC_BY_ROW ? static_cast<int64_t>(row) * ldc + mcol : static_cast<int64_t>(mcol) * ldc + row;
+          tri_store(dU, o, duv);
+          tri_store(dV, o, dvv);
+        }
+      }
+      if constexpr (BF) {
+        pu[2 * a] = pack_bf16(du[0], du[1]); pu[2 * a + 1] = pack_bf16(du[2], du[3]);
+        pv[2 * a] = pack_bf16(dv[0], dv[1]); pv[2 * a + 1] = pack_bf16(dv[2], dv[3]);
       }
     }
+    if (more) load_dc(c0 + 32);
 
     // second product: rows m (lanes of the operand), contraction over the 32 rows c of the chunk
     if constexpr (BF) {
-      uint4 pu[2], pv[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        pu[t] = make_uint4(pack_bf16(du[8 * t], du[8 * t + 1]), pack_bf16(du[8 * t + 2], du[8 * t + 3]),
-                           pack_bf16(du[8 * t + 4], du[8 * t + 5]), pack_bf16(du[8 * t + 6], du[8 * t + 7]));
-        pv[t] = make_uint4(pack_bf16(dv[8 * t], dv[8 * t + 1]), pack_bf16(dv[8 * t + 2], dv[8 * t + 3]),
-                           pack_bf16(dv[8 * t + 4], dv[8 * t + 5]), pack_bf16(dv[8 * t + 6], dv[8 * t + 7]));
-      }
       const char* t1 = &smem[buf][2 * WBYTES + c * TSTR + h * 8];
 #pragma unroll
       for (int ds = 0; ds < KT; ++ds)
@@ -600,8 +694,9 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2)
           const char* p1 = t1 + ds * 32 * TSTR + t * 32;
           const uint2 l1 = *reinterpret_cast<const uint2*>(p1), h1 = *reinterpret_cast<const uint2*>(p1 + 16);
           const uint2 l2 = *reinterpret_cast<const uint2*>(p1 + TBYTES), h2 = *reinterpret_cast<const uint2*>(p1 + TBYTES + 16);
-          mma_step<TI>(ax1[ds], pu[t], make_uint4(l1.x, l1.y, h1.x, h1.y));
-          mma_step<TI>(SPLIT ? ax2[ds] : ax1[ds], pv[t], make_uint4(l2.x, l2.y, h2.x, h2.y));
+          mma_step<TI>(ax1[ds], make_uint4(pu[4 * t], pu[4 * t + 1], pu[4 * t + 2], pu[4 * t + 3]), make_uint4(l1.x, l1.y, h1.x, h1.y));
+          mma_step<TI>(SPLIT ? ax2[ds] : ax1[ds], make_uint4(pv[4 * t], pv[4 * t + 1], pv[4 * t + 2], pv[4 * t + 3]),
+                       make_uint4(l2.x, l2.y, h2.x, h2.y));
         }
     } else {
 #pragma unroll
@@ -616,7 +711,7 @@ __global__ void __launch_bounds__(256, SPLIT ? 1 : 2)
         }
     }
 
-    if (ci + 1 < nchunks) store_chunk(buf ^ 1);
+    if (more) store_cols(buf ^ 1);
     __syncthreads();
   }
 
@@ -1122,9 +1217,13 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
                          (dc_by_row ? 0 : reinterpret_cast<uintptr_t>(dC));
   const bool aligned = (ptrs & 15) == 0 && ldw % epv == 0 && ldx % epv == 0 && (!bf || ldwt % epv == 0) && (dc_by_row || ldc % epv == 0);
   CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: row strides and pointers must be multiples of 16 bytes");
-  const dim3 grid(static_cast<unsigned>((M + kTile - 1) / kTile));
+  CUEQ_REQUIRE(split == !dc_by_row, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: built for one input with dC by rows (C x M) and two inputs with dC by columns (M x C)");
+  const int64_t es = bf ? 2 : 4;
+  CUEQ_REQUIRE(ldc >= 0 && ldw >= 0 && ldwt >= 0 && 32 * ldw * es < (1ll << 31) && (K + 1) * ldwt * es < (1ll << 31) &&
+                   (dc_by_row ? (4 * ldc + M) : (M * ldc + 8)) * es < (1ll << 32),
+               CUEQ_ERR_TOO_LARGE, "gate_bwd_input: strides too large for 32-bit lane offsets");
   KernelTimer timer("gate_bwd_input", stream);
-#define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP>), grid, dim3(256), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(W1T), static_cast<const TI*>(W2T), ldwt, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, dc_by_row, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
+#define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP, !SP>), dim3(static_cast<unsigned>((M + gbi_threads<TI, SP>() / 2 - 1) / (gbi_threads<TI, SP>() / 2))), dim3(gbi_threads<TI, SP>()), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(W1T), static_cast<const TI*>(W2T), ldwt, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
 #define GBI_K(TI, SP) do { switch (K / 32) { case 1: GBI(TI, 1, SP); break; case 2: GBI(TI, 2, SP); break; case 3: GBI(TI, 3, SP); break; default: GBI(TI, 4, SP); break; } } while (0)
 #define GBI_T(TI) do { if (split) GBI_K(TI, true); else GBI_K(TI, false); } while (0)
   TRI_DISPATCH(dtype, GBI_T(float), GBI_T(uint16_t));
