@@ -52,11 +52,71 @@ __device__ __forceinline__ void xcd_tile(int& bx, int& by, int& bz) {
   bz = static_cast<int>(P / (gx * gy));
 }
 
+// ------------------------------------------------------------------------------------------------
+// Results leave the MFMA register layout (a lane holds one column and 16 rows of a 32 x 32 tile) through LDS, so
+// that global memory sees 16-byte vectors on contiguous row segments: 2-byte stores straight from that layout reach
+// only a fraction of the write bandwidth.  put: one 32 x 32 accumulator into a staging tile whose rows are
+// `row_stride` bytes apart; flush: a wavefront moves 32 rows x NCOLS staged elements to C (optionally adding what is
+// there).  A staging tile is private to one wavefront, whose LDS operations execute in program order.
+// ------------------------------------------------------------------------------------------------
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {  // round to nearest even, one v_cvt_pk_bf16_f32
+  const floatx2_t f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
+template <typename TO>
+__device__ __forceinline__ void stage_put(char* tile, int row_stride, int col, int h, const floatx16& acc, float alpha) {
+#pragma unroll
+  for (int v = 0; v < 16; v += 2) {
+    char* p = tile + (8 * (v >> 2) + 4 * h + (v & 3)) * row_stride + col * static_cast<int>(sizeof(TO));
+    if constexpr (sizeof(TO) == 2) {
+      const uint32_t w = pack_bf16(alpha * acc[v], alpha * acc[v + 1]);
+      *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(w & 0xffffu);
+      *reinterpret_cast<uint16_t*>(p + row_stride) = static_cast<uint16_t>(w >> 16);
+    } else {
+      *reinterpret_cast<float*>(p) = alpha * acc[v];
+      *reinterpret_cast<float*>(p + row_stride) = alpha * acc[v + 1];
+    }
+  }
+}
+
+template <typename TO>
+__device__ __forceinline__ uint4 add_vec(uint4 a, uint4 b) {
+  if constexpr (sizeof(TO) == 2) {
+    const uint32_t x[4] = {a.x, a.y, a.z, a.w}, y[4] = {b.x, b.y, b.z, b.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      r[e] = pack_bf16(__uint_as_float(x[e] << 16) + __uint_as_float(y[e] << 16),
+                       __uint_as_float(x[e] & 0xffff0000u) + __uint_as_float(y[e] & 0xffff0000u));
+    return make_uint4(r[0], r[1], r[2], r[3]);
+  } else {
+    return make_uint4(__float_as_uint(__uint_as_float(a.x) + __uint_as_float(b.x)), __float_as_uint(__uint_as_float(a.y) + __uint_as_float(b.y)),
+                      __float_as_uint(__uint_as_float(a.z) + __uint_as_float(b.z)), __float_as_uint(__uint_as_float(a.w) + __uint_as_float(b.w)));
+  }
+}
+
+// nthreads threads (index t) move `rows` staged rows of NCOLS elements to C (row stride ldc elements)
+template <typename TO, int NCOLS>
+__device__ __forceinline__ void stage_flush(const char* tile, int row_stride, int rows, TO* __restrict__ C, int64_t ldc, int t, int nthreads,
+                                            bool accumulate) {
+  constexpr int EPV = 16 / sizeof(TO), VPR = NCOLS / EPV;
+  for (int idx = t; idx < rows * VPR; idx += nthreads) {
+    const int r = idx / VPR, cv = idx % VPR;
+    uint4 val = *reinterpret_cast<const uint4*>(tile + r * row_stride + cv * 16);
+    uint4* g = reinterpret_cast<uint4*>(C + static_cast<int64_t>(r) * ldc + cv * EPV);
+    if (accumulate) val = add_vec<TO>(val, *g);
+    *g = val;
+  }
+}
+
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
                                                       const TI* __restrict__ B, int64_t ldb, int64_t sB,
                                                       TO* __restrict__ C, int64_t ldc, int64_t sC, int M, int N, int K,
-                                                      float alpha, int accumulate) {
+                                                      float alpha, int accumulate, int vec_out) {
   constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
   constexpr int BK = 64 / sizeof(TI);   // k extent of one step
   __shared__ __align__(16) char smem[2][2][kTile * kRowBytes];
@@ -146,6 +206,21 @@ __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, 
     buf ^= 1;
   }
 
+  __syncthreads();  // every wavefront is done with the operand tiles, which become staging space
+  // whole wavefront tile inside C and 16-byte aligned rows: through LDS, 32 rows at a time
+  if (vec_out && m0 + wm * 64 + 64 <= M && n0 + wn * 64 + 64 <= N) {
+    constexpr int RS = 64 * sizeof(TO) + 16;
+    char* tile = &smem[0][0][0] + wave * (32 * RS);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      stage_put<TO>(tile, RS, c, h, acc[i][0], alpha);
+      stage_put<TO>(tile, RS, 32 + c, h, acc[i][1], alpha);
+      __builtin_amdgcn_wave_barrier();
+      stage_flush<TO, 64>(tile, RS, 32, C + static_cast<int64_t>(m0 + wm * 64 + i * 32) * ldc + n0 + wn * 64, ldc, lane, 64, accumulate != 0);
+      __builtin_amdgcn_wave_barrier();
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -287,7 +362,8 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
                                                            const TI* __restrict__ B1, const TI* __restrict__ B2, int64_t ldb,
                                                            const TI* __restrict__ bias1, const TI* __restrict__ bias2, int bias_axis,
                                                            const TI* __restrict__ mask, int mask_axis, const TI* __restrict__ dC,
-                                                           TI* __restrict__ out1, TI* __restrict__ out2, int64_t ldc, int M, int N, int K) {
+                                                           TI* __restrict__ out1, TI* __restrict__ out2, int64_t ldc, int M, int N, int K,
+                                                           int vec_out) {
   // 8 wavefronts of 64 x 32 (both products): half the accumulators per wavefront of the plain GEMM tiling, so two
   // blocks fit a CU and one block's epilogue overlaps the other's loads.
   constexpr int EPV = 16 / sizeof(TI);
@@ -368,11 +444,42 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
   }
 
   const int col = n0 + wn * 32 + c;
-  if (col >= N) return;
-  const float cb1 = (bias1 && bias_axis == 1) ? tri_load(bias1, col) : 0.f;
-  const float cb2 = (bias2 && bias_axis == 1) ? tri_load(bias2, col) : 0.f;
-  const float cmk = (mask && mask_axis == 1) ? tri_load(mask, col) : 1.f;
+  const int colc = min(col, N - 1);
+  const float cb1 = (bias1 && bias_axis == 1) ? tri_load(bias1, colc) : 0.f;
+  const float cb2 = (bias2 && bias_axis == 1) ? tri_load(bias2, colc) : 0.f;
+  const float cmk = (mask && mask_axis == 1) ? tri_load(mask, colc) : 1.f;
   const bool rowb1 = bias1 && bias_axis == 0, rowb2 = bias2 && bias_axis == 0, rowmk = mask && mask_axis == 0;
+
+  if constexpr (!BWD) {
+    // whole block tile inside the output and 16-byte aligned rows: 64 rows at a time through LDS
+    if (vec_out && m0 + kTile <= M && n0 + kTile <= N) {
+      constexpr int RS = kTile * sizeof(TI) + 16;
+      static_assert(64 * RS <= 2 * NT * kTile * kRowBytes, "staging tile must fit the operand buffers");
+      char* tile = &smem[0][0][0];
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+        __syncthreads();  // operand reads / the previous flush are done
+        if (wm == pass) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            floatx16 g;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+              const float uu = acc[0][i][v] + (rowb1 ? tri_load(bias1, row) : cb1);
+              const float vv = acc[1][i][v] + (rowb2 ? tri_load(bias2, row) : cb2);
+              g[v] = __builtin_amdgcn_rcpf(1.0f + __expf(-uu)) * vv * (rowmk ? tri_load(mask, row) : cmk);
+            }
+            stage_put<TI>(tile + i * 32 * RS, RS, wn * 32 + c, h, g, 1.0f);
+          }
+        }
+        __syncthreads();
+        stage_flush<TI, kTile>(tile, RS, 64, out1 + static_cast<int64_t>(m0 + pass * 64) * ldc + n0, ldc, tid, 512, false);
+      }
+      return;
+    }
+  }
+  if (col >= N) return;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -447,22 +554,18 @@ __device__ __forceinline__ uint2 load_global<uint2>(const char* uniform_base, ui
   return make_uint2(v.x, v.y);
 }
 
-typedef float floatx2_t __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {  // round to nearest even, one v_cvt_pk_bf16_f32
-  const floatx2_t f = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
-}
 
-// 2-byte single-input case: 8 wavefronts (256 columns m) per block at 2 wavefronts per SIMD; the others need more
-// registers per wavefront and run 4 wavefronts per block at 1 per SIMD.
+// 4 wavefronts (128 columns m) per block; the 2-byte single-input case fits 2 wavefronts per SIMD (two blocks per
+// CU, so one block's waits overlap the other's work), the others need more registers and run 1 per SIMD.
 template <typename TI, bool SPLIT>
-constexpr int gbi_threads() { return (sizeof(TI) == 2 && !SPLIT) ? 512 : 256; }
+constexpr int gbi_threads() { return 256; }
+template <typename TI, bool SPLIT>
+constexpr int gbi_waves_per_simd() { return (sizeof(TI) == 2 && !SPLIT) ? 2 : 1; }
 
 // DC_BY_ROW: dC, dU, dV are C x M (else M x C).  Addresses inside the loop are a uniform 64-bit base plus a 32-bit
 // lane offset (the host checks the extents), which keeps them out of the vector registers.
 template <typename TI, int KT, bool SPLIT, bool DC_BY_ROW>
-__global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_threads<TI, SPLIT>() == 512 ? 2 : 1))
+__global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_simd<TI, SPLIT>()))
     gate_bwd_input_kernel(const TI* __restrict__ W1, const TI* __restrict__ W2, int64_t ldw, const TI* __restrict__ W1T,
                           const TI* __restrict__ W2T, int64_t ldwt, const TI* __restrict__ X1, const TI* __restrict__ X2, int64_t ldx,
                           const TI* __restrict__ bias1, const TI* __restrict__ bias2, const TI* __restrict__ mask,
@@ -587,15 +690,15 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_threads<TI, S
 
   // cotangent of a chunk: value v of the lane belongs to row c0 + 8 (v >> 2) + 4 h + (v & 3); fetched one chunk ahead
   // (kept as loaded - one register per value, or packed pairs when read along c - and widened where it is used)
-  uint32_t dcr[16];
+  uint32_t dcr[16], dcn[16];
   const uint32_t dcofs = DC_BY_ROW ? static_cast<uint32_t>((4 * h * ldc + mld) * ES) : static_cast<uint32_t>((mld * ldc + 4 * h) * ES);
   auto load_dc = [&](int c0) {
     if constexpr (DC_BY_ROW) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * (v >> 2) + (v & 3)) * ldc * ES);
-        if constexpr (BF) dcr[v] = load_global<uint16_t>(base, dcofs);
-        else dcr[v] = load_global<uint32_t>(base, dcofs);
+        if constexpr (BF) dcn[v] = load_global<uint16_t>(base, dcofs);
+        else dcn[v] = load_global<uint32_t>(base, dcofs);
       }
     } else {
 #pragma unroll
@@ -603,10 +706,10 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_threads<TI, S
         const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * a) * ES);
         if constexpr (BF) {
           const uint2 w = load_global<uint2>(base, dcofs);
-          dcr[4 * a] = w.x; dcr[4 * a + 1] = w.y;  // values 4a..4a+3 in two registers
+          dcn[4 * a] = w.x; dcn[4 * a + 1] = w.y;  // values 4a..4a+3 in two registers
         } else {
           const uint4 w = load_global<uint4>(base, dcofs);
-          dcr[4 * a] = w.x; dcr[4 * a + 1] = w.y; dcr[4 * a + 2] = w.z; dcr[4 * a + 3] = w.w;
+          dcn[4 * a] = w.x; dcn[4 * a + 1] = w.y; dcn[4 * a + 2] = w.z; dcn[4 * a + 3] = w.w;
         }
       }
     }
@@ -630,7 +733,12 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_threads<TI, S
   for (int ci = 0; ci < nchunks; ++ci) {
     const int c0 = ci * 32, buf = ci & 1;
     const bool more = ci + 1 < nchunks;
-    if (more) load_rows(c0 + 32);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dcr[v] = dcn[v];
+    if (more) {
+      load_rows(c0 + 32);
+      load_dc(c0 + 32);  // a whole iteration ahead of its use
+    }
 
     // first product: u, v for 32 rows c x 32 columns m
     floatx16 au = floatx16{0}, av = floatx16{0};
@@ -682,8 +790,6 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_threads<TI, S
         pv[2 * a] = pack_bf16(dv[0], dv[1]); pv[2 * a + 1] = pack_bf16(dv[2], dv[3]);
       }
     }
-    if (more) load_dc(c0 + 32);
-
     // second product: rows m (lanes of the operand), contraction over the 32 rows c of the chunk
     if constexpr (BF) {
       const char* t1 = &smem[buf][2 * WBYTES + c * TSTR + h * 8];
@@ -715,6 +821,24 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_threads<TI, S
     __syncthreads();
   }
 
+  // (the loop's last barrier has passed: the weight buffers are free for staging)
+  if (mrow0 + 32 <= M) {
+    constexpr int RS = ROWB + 16;
+    static_assert(4 * 32 * RS <= 2 * BUF, "staging tiles must fit the weight buffers");
+    char* tile = &smem[0][0] + wave * (32 * RS);
+#pragma unroll
+    for (int ds = 0; ds < KT; ++ds) stage_put<TI>(tile, RS, ds * 32 + c, h, ax1[ds], 1.0f);
+    __builtin_amdgcn_wave_barrier();
+    stage_flush<TI, K>(tile, RS, 32, dX1 + static_cast<int64_t>(mrow0) * lddx, lddx, lane, 64, accumulate != 0);
+    if constexpr (SPLIT) {
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int ds = 0; ds < KT; ++ds) stage_put<TI>(tile, RS, ds * 32 + c, h, ax2[ds], 1.0f);
+      __builtin_amdgcn_wave_barrier();
+      stage_flush<TI, K>(tile, RS, 32, dX2 + static_cast<int64_t>(mrow0) * lddx, lddx, lane, 64, false);
+    }
+    return;
+  }
 #pragma unroll
   for (int ds = 0; ds < KT; ++ds) {
     const int col = ds * 32 + c;
@@ -1145,7 +1269,9 @@ extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int6
     const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(batch));
     CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm_nt: too many row tiles (M <= 8388480)");
     KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
-#define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_nt_kernel<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate)
+    const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
+    const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
+#define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_nt_kernel<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_LAUNCH(float, float);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t);
     else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float);
@@ -1183,8 +1309,9 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
   CUEQ_REQUIRE(gy < 65536 && gx < (1ll << 31) && M < (1ll << 31) && N < (1ll << 31), CUEQ_ERR_TOO_LARGE, "dual_gate: extent too large");
   const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy));
   const bool share = B2 == nullptr || B2 == B1;
+  const int vec_out = (reinterpret_cast<uintptr_t>(out1) % 16 == 0 && ldc % epv == 0) ? 1 : 0;
   KernelTimer timer(backward ? "dual_gate_bwd" : "dual_gate_fwd", stream);
-#define DG(TI, BW, SH) hipLaunchKernelGGL((dual_gate_kernel<TI, BW, SH>), grid, dim3(512), 0, stream, static_cast<const TI*>(A1), static_cast<const TI*>(A2), lda, static_cast<const TI*>(B1), static_cast<const TI*>(B2), ldb, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), bias_axis, static_cast<const TI*>(mask), mask_axis, static_cast<const TI*>(dC), static_cast<TI*>(out1), static_cast<TI*>(out2), ldc, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K))
+#define DG(TI, BW, SH) hipLaunchKernelGGL((dual_gate_kernel<TI, BW, SH>), grid, dim3(512), 0, stream, static_cast<const TI*>(A1), static_cast<const TI*>(A2), lda, static_cast<const TI*>(B1), static_cast<const TI*>(B2), ldb, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), bias_axis, static_cast<const TI*>(mask), mask_axis, static_cast<const TI*>(dC), static_cast<TI*>(out1), static_cast<TI*>(out2), ldc, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), vec_out)
 #define DG_T(TI) do { if (backward) { if (share) DG(TI, true, true); else DG(TI, true, false); } else { if (share) DG(TI, false, true); else DG(TI, false, false); } } while (0)
   TRI_DISPATCH(dtype, DG_T(float), DG_T(uint16_t));
 #undef DG_T
@@ -1214,8 +1341,8 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
   const int epv = bf ? 8 : 4;
   const uintptr_t ptrs = reinterpret_cast<uintptr_t>(W1) | reinterpret_cast<uintptr_t>(W2) | reinterpret_cast<uintptr_t>(W1T) |
                          reinterpret_cast<uintptr_t>(W2T) | reinterpret_cast<uintptr_t>(X1) | reinterpret_cast<uintptr_t>(X2) |
-                         (dc_by_row ? 0 : reinterpret_cast<uintptr_t>(dC));
-  const bool aligned = (ptrs & 15) == 0 && ldw % epv == 0 && ldx % epv == 0 && (!bf || ldwt % epv == 0) && (dc_by_row || ldc % epv == 0);
+                         (dc_by_row ? 0 : reinterpret_cast<uintptr_t>(dC)) | reinterpret_cast<uintptr_t>(dX1) | reinterpret_cast<uintptr_t>(dX2);
+  const bool aligned = (ptrs & 15) == 0 && ldw % epv == 0 && ldx % epv == 0 && lddx % epv == 0 && (!bf || ldwt % epv == 0) && (dc_by_row || ldc % epv == 0);
   CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: row strides and pointers must be multiples of 16 bytes");
   CUEQ_REQUIRE(split == !dc_by_row, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: built for one input with dC by rows (C x M) and two inputs with dC by columns (M x C)");
   const int64_t es = bf ? 2 : 4;
