@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "cueq_seg_outer",
     "cueq_seg_rowdot",
     "cueq_gemm_nt",
+    "cueq_gemm",
     "cueq_dual_gate",
     "cueq_gate_bwd_input",
     "cueq_gemm_tn_items",
@@ -170,6 +171,8 @@ def load() -> C.CDLL:
         i32, i64, ptr, f64 = C.c_int32, C.c_int64, C.c_void_p, C.c_double
         lib.cueq_gemm_nt.argtypes = [i32, i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, ptr, i64, i64, i64, f64, i32, ptr]
         lib.cueq_gemm_nt.restype = C.c_int
+        lib.cueq_gemm.argtypes = [i32, i32, i32, i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, ptr, i64, i64, i64, f64, i32, ptr]
+        lib.cueq_gemm.restype = C.c_int
         lib.cueq_dual_gate.argtypes = [i32, i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i32, ptr, i32, ptr, ptr, ptr, i64, ptr]
         lib.cueq_dual_gate.restype = C.c_int
         lib.cueq_gate_bwd_input.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, ptr, ptr, i64,

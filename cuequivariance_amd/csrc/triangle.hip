@@ -112,13 +112,51 @@ __device__ __forceinline__ void stage_flush(const char* tile, int row_stride, in
   }
 }
 
-template <typename TI, typename TO>
-__global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
-                                                      const TI* __restrict__ B, int64_t ldb, int64_t sB,
-                                                      TO* __restrict__ C, int64_t ldc, int64_t sC, int M, int N, int K,
-                                                      float alpha, int accumulate, int vec_out) {
+// TA / TB: the operand is given contraction-major (K x M resp. K x N, row stride lda / ldb) instead of the default
+// contraction-contiguous M x K / N x K.  Such a tile is staged as it lies in memory (rows of k) and the MFMA operand
+// is assembled on the way out of LDS: 2-byte types with the transposing read ds_read_b64_tr_b16 (within 16 lanes,
+// lane 4g+p receives element p of the four 8-byte rows addressed by lanes g, 4+g, 8+g, 12+g), 4-byte types with
+// plain reads along the row.  The row strides (320 / 640 bytes) spread the rows of one read over all banks.
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+constexpr int kTransStride16 = 320, kTransStride32 = 640;
+
+template <typename TI, bool TR>
+__device__ __forceinline__ void gemm_stage_offsets(int e, int& row, int& part) {
+  constexpr int VPRN = kTile * sizeof(TI) / 16;  // vectors per k row of a contraction-major tile
+  if constexpr (TR) { row = e / VPRN; part = e % VPRN; }
+  else { row = e >> 2; part = e & 3; }
+}
+
+// fragment of subtile rows [base, base + 32) for MFMA step half q: 16 bytes of k per lane
+template <typename TI, bool TR>
+__device__ __forceinline__ uint4 gemm_fragment(const char* tile, int base, int q, int lane) {
+  const int c = lane & 31, h = lane >> 5;
+  if constexpr (!TR) {
+    return *reinterpret_cast<const uint4*>(tile + (base + c) * kRowBytes + h * 32 + q * 16);
+  } else if constexpr (sizeof(TI) == 2) {
+    const int s = lane & 15, g16 = (lane >> 4) & 1;
+    const char* p = tile + (16 * h + 8 * q + (s >> 2)) * kTransStride16 + (base + 16 * g16 + 4 * (s & 3)) * 2;  // k as in the other layout
+    typedef shortx4_t __attribute__((address_space(3))) * lptr;
+    const shortx4_t r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p));
+    const shortx4_t r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p + 4 * kTransStride16));
+    const uint2 a = __builtin_bit_cast(uint2, r0), b = __builtin_bit_cast(uint2, r1);
+    return make_uint4(a.x, a.y, b.x, b.y);
+  } else {
+    const char* p = tile + (8 * h + 4 * q) * kTransStride32 + (base + c) * 4;
+    return make_uint4(*reinterpret_cast<const uint32_t*>(p), *reinterpret_cast<const uint32_t*>(p + kTransStride32),
+                      *reinterpret_cast<const uint32_t*>(p + 2 * kTransStride32), *reinterpret_cast<const uint32_t*>(p + 3 * kTransStride32));
+  }
+}
+
+template <typename TI, typename TO, bool TA, bool TB>
+__global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
+                                                   const TI* __restrict__ B, int64_t ldb, int64_t sB,
+                                                   TO* __restrict__ C, int64_t ldc, int64_t sC, int M, int N, int K,
+                                                   float alpha, int accumulate, int vec_out) {
   constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
   constexpr int BK = 64 / sizeof(TI);   // k extent of one step
+  constexpr int TS = sizeof(TI) == 2 ? kTransStride16 : kTransStride32;
+  static_assert(BK * TS == kTile * kRowBytes, "both tile layouts take the same space");
   __shared__ __align__(16) char smem[2][2][kTile * kRowBytes];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
@@ -132,32 +170,36 @@ __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, 
 
   // every thread stages two 16-byte vectors of A and two of B per step
   uint4 stA[2], stB[2];
-  int ldrow[2], ldpart[2];
+  int arow[2], apart[2], brow[2], bpart[2];
 #pragma unroll
   for (int q = 0; q < 2; ++q) {
-    const int e = tid + q * 256;
-    ldrow[q] = e >> 2;
-    ldpart[q] = e & 3;
+    gemm_stage_offsets<TI, TA>(tid + q * 256, arow[q], apart[q]);
+    gemm_stage_offsets<TI, TB>(tid + q * 256, brow[q], bpart[q]);
   }
+  auto load_one = [&](const TI* __restrict__ P, int64_t ld, bool tr, int row, int part, int x0, int X, int ks) -> uint4 {
+    if (tr) {  // row = k within the step, part = vector along the tile's 128 columns (extent X is a multiple of EPV)
+      const int k = ks * BK + row, x = x0 + part * EPV;
+      const bool ok = k < K && x < X;
+      const uint4 v = *reinterpret_cast<const uint4*>(P + static_cast<int64_t>(ok ? k : 0) * ld + (ok ? x : 0));
+      return ok ? v : make_uint4(0, 0, 0, 0);
+    }
+    const int k = ks * BK + part * EPV;
+    const bool ok = k < K;
+    const uint4 v = *reinterpret_cast<const uint4*>(P + static_cast<int64_t>(min(x0 + row, X - 1)) * ld + (ok ? k : 0));
+    return ok ? v : make_uint4(0, 0, 0, 0);
+  };
   auto load_step = [&](int ks) {
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
-      const int k = ks * BK + ldpart[q] * EPV;
-      const int ra = min(m0 + ldrow[q], M - 1), rb = min(n0 + ldrow[q], N - 1);
-      if (k < K) {
-        stA[q] = *reinterpret_cast<const uint4*>(A + static_cast<int64_t>(ra) * lda + k);
-        stB[q] = *reinterpret_cast<const uint4*>(B + static_cast<int64_t>(rb) * ldb + k);
-      } else {
-        stA[q] = make_uint4(0, 0, 0, 0);
-        stB[q] = make_uint4(0, 0, 0, 0);
-      }
+      stA[q] = load_one(A, lda, TA, arow[q], apart[q], m0, M, ks);
+      stB[q] = load_one(B, ldb, TB, brow[q], bpart[q], n0, N, ks);
     }
   };
   auto store_step = [&](int buf) {
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
-      *reinterpret_cast<uint4*>(&smem[buf][0][ldrow[q] * kRowBytes + ldpart[q] * 16]) = stA[q];
-      *reinterpret_cast<uint4*>(&smem[buf][1][ldrow[q] * kRowBytes + ldpart[q] * 16]) = stB[q];
+      *reinterpret_cast<uint4*>(&smem[buf][0][arow[q] * (TA ? TS : kRowBytes) + apart[q] * 16]) = stA[q];
+      *reinterpret_cast<uint4*>(&smem[buf][1][brow[q] * (TB ? TS : kRowBytes) + bpart[q] * 16]) = stB[q];
     }
   };
 
@@ -174,15 +216,13 @@ __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, 
     store_step(buf);
     __syncthreads();
     if (ks + 1 < nsteps) load_step(ks + 1);
-    const char* sa = &smem[buf][0][(wm * 64 + c) * kRowBytes + h * 32];
-    const char* sb = &smem[buf][1][(wn * 64 + c) * kRowBytes + h * 32];
     uint4 fa[2][2], fb[2][2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        fa[t][q] = *reinterpret_cast<const uint4*>(sa + t * 32 * kRowBytes + q * 16);
-        fb[t][q] = *reinterpret_cast<const uint4*>(sb + t * 32 * kRowBytes + q * 16);
+        fa[t][q] = gemm_fragment<TI, TA>(&smem[buf][0][0], wm * 64 + t * 32, q, lane);
+        fb[t][q] = gemm_fragment<TI, TB>(&smem[buf][1][0], wn * 64 + t * 32, q, lane);
       }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -206,9 +246,10 @@ __global__ void __launch_bounds__(256) gemm_nt_kernel(const TI* __restrict__ A, 
     buf ^= 1;
   }
 
-  __syncthreads();  // every wavefront is done with the operand tiles, which become staging space
-  // whole wavefront tile inside C and 16-byte aligned rows: through LDS, 32 rows at a time
-  if (vec_out && m0 + wm * 64 + 64 <= M && n0 + wn * 64 + 64 <= N) {
+  // 2-byte results, whole wavefront tile inside C, 16-byte aligned rows: through LDS, 32 rows at a time (4-byte
+  // results already leave as 128-byte row segments and gain nothing from the detour)
+  if constexpr (sizeof(TO) == 2) __syncthreads();  // every wavefront is done with the operand tiles, which become staging space
+  if (sizeof(TO) == 2 && vec_out && m0 + wm * 64 + 64 <= M && n0 + wn * 64 + 64 <= N) {
     constexpr int RS = 64 * sizeof(TO) + 16;
     char* tile = &smem[0][0][0] + wave * (32 * RS);
 #pragma unroll
@@ -856,19 +897,20 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
   }
 }
 
-// any shape / alignment: one thread per output element
+// any shape / alignment / operand order: one thread per output element (rs*: stride between rows of the operand,
+// ks*: stride along the contraction)
 template <typename TI, typename TO>
-__global__ void __launch_bounds__(256) gemm_nt_simple(const TI* __restrict__ A, int64_t lda, int64_t sA, const TI* __restrict__ B,
-                                                      int64_t ldb, int64_t sB, TO* __restrict__ C, int64_t ldc, int64_t sC,
-                                                      int M, int N, int K, float alpha, int accumulate) {
+__global__ void __launch_bounds__(256) gemm_simple(const TI* __restrict__ A, int64_t rsa, int64_t ksa, int64_t sA, const TI* __restrict__ B,
+                                                   int64_t rsb, int64_t ksb, int64_t sB, TO* __restrict__ C, int64_t ldc, int64_t sC,
+                                                   int M, int N, int K, float alpha, int accumulate) {
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= static_cast<int64_t>(M) * N) return;
   const int row = static_cast<int>(tid / N), col = static_cast<int>(tid - static_cast<int64_t>(row) * N);
-  A += static_cast<int64_t>(blockIdx.z) * sA + static_cast<int64_t>(row) * lda;
-  B += static_cast<int64_t>(blockIdx.z) * sB + static_cast<int64_t>(col) * ldb;
+  A += static_cast<int64_t>(blockIdx.z) * sA + static_cast<int64_t>(row) * rsa;
+  B += static_cast<int64_t>(blockIdx.z) * sB + static_cast<int64_t>(col) * rsb;
   C += static_cast<int64_t>(blockIdx.z) * sC;
   float acc = 0;
-  for (int k = 0; k < K; ++k) acc = fmaf(tri_load(A, k), tri_load(B, k), acc);
+  for (int k = 0; k < K; ++k) acc = fmaf(tri_load(A, k * ksa), tri_load(B, k * ksb), acc);
   const int64_t o = static_cast<int64_t>(row) * ldc + col;
   float val = alpha * acc;
   if (accumulate) val += tri_load(C, o);
@@ -1251,38 +1293,44 @@ using namespace cueq;
     if ((dt) == CUEQ_F32) { CALL_F32; } else { CALL_BF16; } \
   } while (0)
 
-extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
-                            int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
-                            int64_t batch, double alpha, int32_t accumulate, void* stream_) {
+extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
+                         const void* A, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C,
+                         int64_t ldc, int64_t stride_c, int64_t batch, double alpha, int32_t accumulate, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm_nt: dtypes must be float32 or bfloat16");
-  CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, CUEQ_ERR_INVALID, "gemm_nt: negative extent");
+  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm: dtypes must be float32 or bfloat16");
+  CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, CUEQ_ERR_INVALID, "gemm: negative extent");
   if (M == 0 || N == 0 || batch == 0) return CUEQ_OK;
-  CUEQ_REQUIRE(A && B && C, CUEQ_ERR_INVALID, "gemm_nt: null operand");
-  CUEQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch < 65536, CUEQ_ERR_TOO_LARGE, "gemm_nt: extent too large");
+  CUEQ_REQUIRE(A && B && C, CUEQ_ERR_INVALID, "gemm: null operand");
+  CUEQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch < 65536, CUEQ_ERR_TOO_LARGE, "gemm: extent too large");
   const int epv = in_dtype == CUEQ_F32 ? 4 : 8;
-  const bool aligned = K % epv == 0 && lda % epv == 0 && ldb % epv == 0 && stride_a % epv == 0 && stride_b % epv == 0 &&
-                       reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 && K > 0;
+  // vectors run along k for a contraction-contiguous operand, along its other extent for a contraction-major one
+  const bool aligned = K > 0 && (trans_a ? M : K) % epv == 0 && (trans_b ? N : K) % epv == 0 && lda % epv == 0 && ldb % epv == 0 &&
+                       stride_a % epv == 0 && stride_b % epv == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(B) % 16 == 0;
   const float al = static_cast<float>(alpha);
   const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
-  if (aligned) {
+  const bool mixed = in_dtype != out_dtype;
+  if (aligned && !(mixed && (trans_a || trans_b))) {
     const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(batch));
-    CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm_nt: too many row tiles (M <= 8388480)");
+    CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm: too many row tiles (M <= 8388480)");
     KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
     const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
     const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
-#define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_nt_kernel<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out)
-    if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_LAUNCH(float, float);
-    else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t);
-    else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float);
-    else GEMM_LAUNCH(uint16_t, uint16_t);
+#define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out)
+#define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_LAUNCH(TI, TI, true, true); else if (trans_a) GEMM_LAUNCH(TI, TI, true, false); else if (trans_b) GEMM_LAUNCH(TI, TI, false, true); else GEMM_LAUNCH(TI, TI, false, false); } while (0)
+    if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_TR(float);
+    else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t, false, false);
+    else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float, false, false);
+    else GEMM_TR(uint16_t);
+#undef GEMM_TR
 #undef GEMM_LAUNCH
   } else {
     const int64_t total = M * N;
-    CUEQ_REQUIRE((total + 255) / 256 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gemm_nt: output too large for the unaligned path");
+    CUEQ_REQUIRE((total + 255) / 256 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gemm: output too large for the unaligned path");
     const dim3 grid(static_cast<unsigned>((total + 255) / 256), 1, static_cast<unsigned>(batch));
     KernelTimer timer("gemm_nt_simple", stream);
-#define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_nt_simple<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate)
+    const int64_t rsa = trans_a ? 1 : lda, ksa = trans_a ? lda : 1, rsb = trans_b ? 1 : ldb, ksb = trans_b ? ldb : 1;
+#define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_simple<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), rsa, ksa, stride_a, static_cast<const TI*>(B), rsb, ksb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_LAUNCH(float, float);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t);
     else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float);
@@ -1291,6 +1339,12 @@ extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int6
   }
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
+}
+
+extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                            int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
+                            int64_t batch, double alpha, int32_t accumulate, void* stream_) {
+  return cueq_gemm(in_dtype, out_dtype, 0, 0, M, N, K, A, lda, stride_a, B, ldb, stride_b, C, ldc, stride_c, batch, alpha, accumulate, stream_);
 }
 
 extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_t K, const void* A1, const void* A2, int64_t lda,

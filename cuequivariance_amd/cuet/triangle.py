@@ -56,15 +56,18 @@ def _ptr(t: Optional[torch.Tensor]):
 # thin wrappers over the C ABI (shapes checked here, before any launch)
 # ---------------------------------------------------------------------------------------------
 def gemm_nt(A: torch.Tensor, B: torch.Tensor, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None,
-            accumulate: bool = False, alpha: float = 1.0) -> torch.Tensor:
-    """``C[b] = alpha * A[b] @ B[b]^T (+ C[b])`` for ``A (batch, M, K)``, ``B (batch, N, K)`` (or 2-D, batch 1)."""
+            accumulate: bool = False, alpha: float = 1.0, trans_a: bool = False, trans_b: bool = False) -> torch.Tensor:
+    """``C[b] = alpha * A[b] @ B[b]^T (+ C[b])`` for ``A (batch, M, K)``, ``B (batch, N, K)`` (or 2-D, batch 1);
+    ``trans_a`` / ``trans_b``: that operand is given as ``(batch, K, M)`` / ``(batch, K, N)`` instead."""
     squeeze = A.dim() == 2
     if squeeze:
         A, B = A.unsqueeze(0), B.unsqueeze(0)
-    assert A.dim() == 3 and B.dim() == 3 and A.shape[0] == B.shape[0] and A.shape[2] == B.shape[2], (A.shape, B.shape)
+    assert A.dim() == 3 and B.dim() == 3 and A.shape[0] == B.shape[0], (A.shape, B.shape)
     assert A.dtype == B.dtype and A.stride(2) == 1 and B.stride(2) == 1
-    batch, M, K = A.shape
-    N = B.shape[1]
+    batch = A.shape[0]
+    K, M = (A.shape[1], A.shape[2]) if trans_a else (A.shape[2], A.shape[1])
+    Kb, N = (B.shape[1], B.shape[2]) if trans_b else (B.shape[2], B.shape[1])
+    assert K == Kb, (A.shape, B.shape, trans_a, trans_b)
     if out is None:
         assert not accumulate
         out = torch.empty(batch, M, N, dtype=out_dtype, device=A.device)
@@ -72,12 +75,12 @@ def gemm_nt(A: torch.Tensor, B: torch.Tensor, out_dtype: torch.dtype, out: Optio
         out = out.view(batch, M, N)
         assert out.dtype == out_dtype and out.is_contiguous()
     _lib.check(
-        _lib.load().cueq_gemm_nt(
-            _CODE[A.dtype], _CODE[out_dtype], M, N, K, A.data_ptr(), A.stride(1), A.stride(0) if batch > 1 else 0,
-            B.data_ptr(), B.stride(1), B.stride(0) if batch > 1 else 0, out.data_ptr(), N, M * N, batch, float(alpha),
-            int(accumulate), _stream(A),
+        _lib.load().cueq_gemm(
+            _CODE[A.dtype], _CODE[out_dtype], int(trans_a), int(trans_b), M, N, K, A.data_ptr(), A.stride(1),
+            A.stride(0) if batch > 1 else 0, B.data_ptr(), B.stride(1), B.stride(0) if batch > 1 else 0, out.data_ptr(), N, M * N,
+            batch, float(alpha), int(accumulate), _stream(A),
         ),
-        "cueq_gemm_nt",
+        "cueq_gemm",
     )
     return out[0] if squeeze else out
 
@@ -283,7 +286,7 @@ class _TriMul(torch.autograd.Function):
         if outgoing:
             t = gemm_nt(a, b, T)  # t[i, j] = sum_k a[i, k] b[j, k]
         else:
-            t = gemm_nt(transpose(a), transpose(b), T)  # t[i, j] = sum_k a[k, i] b[k, j]
+            t = gemm_nt(a, b, T, trans_a=True, trans_b=True)  # t[i, j] = sum_k a[k, i] b[k, j]
         tT = transpose(t.view(D, M))  # (M, D)
         y, mean2, rstd2 = layer_norm_fwd(tT, nout_w, nout_b, eps)
         out = dual_gate_fwd(xh, y, g_out_w, p_out_w, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
@@ -336,11 +339,11 @@ class _TriMul(torch.autograd.Function):
         da = dab[:D].view(D * Bsz, N, N)
         db = dab[D:].view(D * Bsz, N, N)
         if ctx.outgoing:  # t = a b^T
-            gemm_nt(dt, transpose(b), T, out=da)  # da[i, k] = sum_j dt[i, j] b[j, k]
-            gemm_nt(transpose(dt), transpose(a), T, out=db)  # db[j, k] = sum_i dt[i, j] a[i, k]
+            gemm_nt(dt, b, T, out=da, trans_b=True)  # da[i, k] = sum_j dt[i, j] b[j, k]
+            gemm_nt(dt, a, T, out=db, trans_a=True, trans_b=True)  # db[j, k] = sum_i dt[i, j] a[i, k]
         else:  # t = a^T b
             gemm_nt(b, dt, T, out=da)  # da[k, i] = sum_j b[k, j] dt[i, j]
-            gemm_nt(a, transpose(dt), T, out=db)  # db[k, j] = sum_i a[k, i] dt[i, j]
+            gemm_nt(a, dt, T, out=db, trans_b=True)  # db[k, j] = sum_i a[k, i] dt[i, j]
 
         # input gate and projections
         fused = gate_bwd_input(dab, True, g_in_w, p_in_w, xh, None, g_in_b, p_in_b, mflat, dxh, w_in)

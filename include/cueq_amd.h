@@ -188,6 +188,14 @@ int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int6
                  int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
                  int64_t batch, double alpha, int32_t accumulate, void* stream);
 
+/* cueq_gemm_nt with a choice of operand order: trans_a != 0 takes A as K x M (row stride lda, batch stride stride_a)
+ * instead of M x K, trans_b != 0 takes B as K x N.  Serves the gradients of the triangular contraction
+ * (da = dt b, db = dt^T a; _triangle_multiplicative_update.py:393-397) and its "incoming" form without transposed
+ * copies.  Mixed input / output types are supported for trans_a == trans_b == 0 only. */
+int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
+              const void* A, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc,
+              int64_t stride_c, int64_t batch, double alpha, int32_t accumulate, void* stream);
+
 /* The gated dual projection in one kernel (_sigmoid_gated_dual_gemm.py:111-218): u = A1 B1^T, v = A2 B2^T (A* M x K, B* N x K,
  * contraction contiguous; B2 NULL: same as B1), then
  *   backward == 0:  out1 = sigmoid(u + bias1) * (v + bias2) * mask

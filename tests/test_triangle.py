@@ -108,6 +108,29 @@ def test_hip_path_matches_oracle(device, dtype, direction, shape):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21)])
+def test_gemm_operand_orders(device, dtype, trans_a, trans_b, dims):
+    """cueq_gemm against torch.matmul in float64 for the four operand orders: tiled MFMA path (aligned extents,
+    partial tiles included) and the element-wise path (odd extents)."""
+    from cuequivariance_amd.cuet import triangle as tri
+
+    batch, M, N, K = dims
+    g = torch.Generator().manual_seed(M * 7 + N)
+    A = torch.randn((batch, K, M) if trans_a else (batch, M, K), generator=g).to(dtype)
+    B = torch.randn((batch, K, N) if trans_b else (batch, N, K), generator=g).to(dtype)
+    A64 = A.double().transpose(1, 2) if trans_a else A.double()
+    B64 = B.double() if trans_b else B.double().transpose(1, 2)
+    ref = 0.5 * A64 @ B64
+    got = tri.gemm_nt(A.to(device), B.to(device), dtype, alpha=0.5, trans_a=trans_a, trans_b=trans_b)
+    assert rel_err(got, ref) <= TOL[dtype], rel_err(got, ref)
+    prev = torch.randn(batch, M, N, generator=g).to(dtype)
+    got2 = tri.gemm_nt(A.to(device), B.to(device), dtype, out=prev.to(device).clone(), accumulate=True, trans_a=trans_a, trans_b=trans_b)
+    assert rel_err(got2, 2 * ref + prev.double()) <= TOL[dtype]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(1, 40, 128, None), (1, 33, 96, 64), (1, 16, 160, None)])
 def test_input_gradient_only(device, dtype, shape):
     """Only x asks for a gradient (the benchmark's case): the gate gradients then stay in registers (D <= 128) or go
