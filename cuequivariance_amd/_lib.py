@@ -175,7 +175,7 @@ def load() -> C.CDLL:
         lib.cueq_gemm.restype = C.c_int
         lib.cueq_dual_gate.argtypes = [i32, i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i32, ptr, i32, ptr, ptr, ptr, i64, ptr]
         lib.cueq_dual_gate.restype = C.c_int
-        lib.cueq_gate_bwd_input.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, ptr, ptr, i64,
+        lib.cueq_gate_bwd_input.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, ptr, ptr, i64,
                                             i32, ptr, ptr, i64, i32, ptr, ptr, ptr]
         lib.cueq_gate_bwd_input.restype = C.c_int
         lib.cueq_gemm_tn_items.argtypes = [i64, i32]

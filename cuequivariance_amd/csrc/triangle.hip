@@ -553,8 +553,8 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
 // holds, per lane, one m and 16 values of c - exactly an operand of the next MFMA with m as the row and c as the
 // contraction - so du and dv go from the accumulator straight into the second product and never touch memory
 // (they are written only when the caller asks for them, for the weight gradients).  X fragments stay in registers;
-// weight chunks are double-buffered in LDS (row-major for the first product; for 2-byte types a transposed copy
-// W^T supplies the second product's operand, float32 reads the row-major chunk column-wise).
+// weight chunks are double-buffered in LDS, row-major; the second product reads them along the columns (2-byte
+// types with the transposing LDS read).
 // ------------------------------------------------------------------------------------------------
 template <typename TI>
 __device__ __forceinline__ void mma_step(floatx16& acc, const uint4& a, const uint4& b) {
@@ -607,8 +607,8 @@ constexpr int gbi_waves_per_simd() { return (sizeof(TI) == 2 && !SPLIT) ? 2 : 1;
 // lane offset (the host checks the extents), which keeps them out of the vector registers.
 template <typename TI, int KT, bool SPLIT, bool DC_BY_ROW>
 __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_simd<TI, SPLIT>()))
-    gate_bwd_input_kernel(const TI* __restrict__ W1, const TI* __restrict__ W2, int64_t ldw, const TI* __restrict__ W1T,
-                          const TI* __restrict__ W2T, int64_t ldwt, const TI* __restrict__ X1, const TI* __restrict__ X2, int64_t ldx,
+    gate_bwd_input_kernel(const TI* __restrict__ W1, const TI* __restrict__ W2, int64_t ldw, const TI* __restrict__ X1,
+                          const TI* __restrict__ X2, int64_t ldx,
                           const TI* __restrict__ bias1, const TI* __restrict__ bias2, const TI* __restrict__ mask,
                           const TI* __restrict__ dC, int64_t ldc, TI* __restrict__ dX1, TI* __restrict__ dX2,
                           int64_t lddx, int accumulate, TI* __restrict__ dU, TI* __restrict__ dV, int C, int M) {
@@ -619,13 +619,10 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
   constexpr int WSTR = ROWB + 16;       // LDS row stride of a row-major chunk (32 rows)
   constexpr int NS = ROWB / 64;         // 64-byte contraction steps of the first product
   constexpr int WBYTES = 32 * WSTR;
-  constexpr int TSTR = 72;              // LDS row stride of a transposed chunk: 32 c = 64 bytes + 8 (conflict-free 8-byte reads)
-  constexpr int TBYTES = BF ? K * TSTR : 0;
-  constexpr int BIAS = 2 * WBYTES + 2 * TBYTES;  // offset of the chunk's biases (2 x 32 float)
+  constexpr int BIAS = 2 * WBYTES;      // offset of the chunk's biases (2 x 32 float)
   constexpr int BUF = BIAS + 256;
   constexpr int NTH = gbi_threads<TI, SPLIT>(), BM = NTH / 2;  // threads and columns m per block
   constexpr int VPR = ROWB / 16, NWV = 32 * VPR, NW = (NWV + NTH - 1) / NTH;
-  constexpr int NTV = BF ? K * 4 : 0, NTQ = BF ? (NTV + NTH - 1) / NTH : 1;
   __shared__ __align__(16) char smem[2][BUF];
 
   const int tid = threadIdx.x;
@@ -635,17 +632,12 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
   const int mrow0 = blockIdx.x * BM + wave * 32;     // ... and the wavefront's first m in the second (rows by v)
 
   constexpr int ES = sizeof(TI);
-  uint4 stw[2][NW], stt[2][NTQ];
-  uint32_t wofs[NW], tofs[NTQ];
+  uint4 stw[2][NW];
+  uint32_t wofs[NW];
 #pragma unroll
   for (int q = 0; q < NW; ++q) {
     const int e = min(tid + q * NTH, NWV - 1);
     wofs[q] = static_cast<uint32_t>(((e / VPR) * ldw + (e % VPR) * EPV) * ES);
-  }
-#pragma unroll
-  for (int q = 0; q < NTQ; ++q) {
-    const int e = min(tid + q * NTH, (BF ? NTV : 1) - 1);
-    tofs[q] = static_cast<uint32_t>(((e >> 2) * ldwt + (e & 3) * 8) * ES);
   }
   // biases of the chunk: threads 0..31 / 32..63 (of every 64) fetch bias1 / bias2, the first 64 threads store them
   const TI* bsrc = (tid & 32) ? bias2 : bias1;
@@ -653,8 +645,7 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
   const char* bptr = reinterpret_cast<const char*>(has_bias ? bsrc : W1);
   const uint32_t bofs = has_bias ? static_cast<uint32_t>((tid & 31) * ES) : 0u;
   TI stb;
-  // the row-major chunk and the biases are fetched at the top of an iteration and stored after the first product,
-  // the transposed chunk is fetched then and stored at the end: half the staging registers are live at a time
+  // the next chunk and its biases are fetched at the top of an iteration and stored after the first product
   auto load_rows = [&](int c0) {
     stb = *reinterpret_cast<const TI*>(bptr + (has_bias ? static_cast<int64_t>(c0) * ES : 0) + bofs);  // bptr differs by lane
     const char* w1 = uniform_ptr(reinterpret_cast<const char*>(W1) + static_cast<int64_t>(c0) * ldw * ES);
@@ -663,17 +654,6 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
     for (int q = 0; q < NW; ++q) {
       stw[0][q] = load_global<uint4>(w1, wofs[q]);
       stw[1][q] = load_global<uint4>(w2, wofs[q]);
-    }
-  };
-  auto load_cols = [&](int c0) {
-    if constexpr (BF) {
-      const char* t1 = uniform_ptr(reinterpret_cast<const char*>(W1T) + static_cast<int64_t>(c0) * ES);
-      const char* t2 = uniform_ptr(reinterpret_cast<const char*>(W2T) + static_cast<int64_t>(c0) * ES);
-#pragma unroll
-      for (int q = 0; q < NTQ; ++q) {
-        stt[0][q] = load_global<uint4>(t1, tofs[q]);
-        stt[1][q] = load_global<uint4>(t2, tofs[q]);
-      }
     }
   };
   auto store_rows = [&](int buf) {
@@ -695,22 +675,6 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
       }
     }
   };
-  auto store_cols = [&](int buf) {
-    if constexpr (BF) {
-#pragma unroll
-      for (int q = 0; q < NTQ; ++q) {
-        const int e = tid + q * NTH;
-        if (NTV % NTH == 0 || e < NTV) {
-          const int o = 2 * WBYTES + (e >> 2) * TSTR + (e & 3) * 16;
-          *reinterpret_cast<uint2*>(&smem[buf][o]) = make_uint2(stt[0][q].x, stt[0][q].y);
-          *reinterpret_cast<uint2*>(&smem[buf][o + 8]) = make_uint2(stt[0][q].z, stt[0][q].w);
-          *reinterpret_cast<uint2*>(&smem[buf][TBYTES + o]) = make_uint2(stt[1][q].x, stt[1][q].y);
-          *reinterpret_cast<uint2*>(&smem[buf][TBYTES + o + 8]) = make_uint2(stt[1][q].z, stt[1][q].w);
-        }
-      }
-    }
-  };
-
   // fragments of X for this lane's m: lane half h holds bytes [64 s + 32 h, +32) of the row
   uint4 xf1[NS][2], xf2[SPLIT ? NS : 1][2];
 #pragma unroll
@@ -766,10 +730,8 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
 
   const int nchunks = C / 32;
   load_rows(0);
-  load_cols(0);
   load_dc(0);
   store_rows(0);
-  store_cols(0);
   __syncthreads();
   for (int ci = 0; ci < nchunks; ++ci) {
     const int c0 = ci * 32, buf = ci & 1;
@@ -796,10 +758,7 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
         }
     }
 
-    if (more) {
-      store_rows(buf ^ 1);  // the other buffer was last read before the previous barrier
-      load_cols(c0 + 32);
-    }
+    if (more) store_rows(buf ^ 1);  // the other buffer was last read before the previous barrier
 
     // gate backward in registers; du, dv are packed (2-byte types) as soon as they exist
     float du[BF ? 4 : 16], dv[BF ? 4 : 16];
@@ -833,14 +792,20 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
     }
     // second product: rows m (lanes of the operand), contraction over the 32 rows c of the chunk
     if constexpr (BF) {
-      const char* t1 = &smem[buf][2 * WBYTES + c * TSTR + h * 8];
+      // operand of the second product: for column d = 32 ds + (lane & 31), the 8 rows c that this lane's du / dv
+      // values belong to (16 t + 4 h + 0..3 and + 8), gathered from the row-major chunk by two transposing reads
+      typedef shortx4_t __attribute__((address_space(3))) * lptr;
+      const int s16 = lane & 15, g16 = (lane >> 4) & 1;
+      const char* t1 = &smem[buf][(4 * h + (s16 >> 2)) * WSTR + (16 * g16 + 4 * (s16 & 3)) * 2];
 #pragma unroll
       for (int ds = 0; ds < KT; ++ds)
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          const char* p1 = t1 + ds * 32 * TSTR + t * 32;
-          const uint2 l1 = *reinterpret_cast<const uint2*>(p1), h1 = *reinterpret_cast<const uint2*>(p1 + 16);
-          const uint2 l2 = *reinterpret_cast<const uint2*>(p1 + TBYTES), h2 = *reinterpret_cast<const uint2*>(p1 + TBYTES + 16);
+          const char* p1 = t1 + t * 16 * WSTR + ds * 64;
+          const uint2 l1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p1)));
+          const uint2 h1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p1 + 8 * WSTR)));
+          const uint2 l2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p1 + WBYTES)));
+          const uint2 h2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p1 + WBYTES + 8 * WSTR)));
           mma_step<TI>(ax1[ds], make_uint4(pu[4 * t], pu[4 * t + 1], pu[4 * t + 2], pu[4 * t + 3]), make_uint4(l1.x, l1.y, h1.x, h1.y));
           mma_step<TI>(SPLIT ? ax2[ds] : ax1[ds], make_uint4(pv[4 * t], pv[4 * t + 1], pv[4 * t + 2], pv[4 * t + 3]),
                        make_uint4(l2.x, l2.y, h2.x, h2.y));
@@ -858,7 +823,6 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
         }
     }
 
-    if (more) store_cols(buf ^ 1);
     __syncthreads();
   }
 
@@ -1375,7 +1339,7 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
 }
 
 extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
-                                   const void* W1T, const void* W2T, int64_t ldwt, const void* X1, const void* X2, int64_t ldx,
+                                   const void* X1, const void* X2, int64_t ldx,
                                    const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
                                    int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
                                    void* stream_) {
@@ -1388,23 +1352,21 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
   CUEQ_REQUIRE(M < (1ll << 31) - kTile && C < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gate_bwd_input: extent too large");
   CUEQ_REQUIRE(W1 && W2 && X1 && dC && dX1 && (!dU == !dV), CUEQ_ERR_INVALID, "gate_bwd_input: null operand");
   const bool bf = dtype == CUEQ_BF16;
-  CUEQ_REQUIRE(!bf || (W1T && W2T), CUEQ_ERR_INVALID, "gate_bwd_input: bfloat16 needs the transposed weights");
   const bool split = X2 != nullptr && X2 != X1;
   CUEQ_REQUIRE(!split || dX2, CUEQ_ERR_INVALID, "gate_bwd_input: two inputs need two gradients");
   CUEQ_REQUIRE(!(split && accumulate), CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: accumulate needs a single input");
   const int epv = bf ? 8 : 4;
-  const uintptr_t ptrs = reinterpret_cast<uintptr_t>(W1) | reinterpret_cast<uintptr_t>(W2) | reinterpret_cast<uintptr_t>(W1T) |
-                         reinterpret_cast<uintptr_t>(W2T) | reinterpret_cast<uintptr_t>(X1) | reinterpret_cast<uintptr_t>(X2) |
+  const uintptr_t ptrs = reinterpret_cast<uintptr_t>(W1) | reinterpret_cast<uintptr_t>(W2) | reinterpret_cast<uintptr_t>(X1) | reinterpret_cast<uintptr_t>(X2) |
                          (dc_by_row ? 0 : reinterpret_cast<uintptr_t>(dC)) | reinterpret_cast<uintptr_t>(dX1) | reinterpret_cast<uintptr_t>(dX2);
-  const bool aligned = (ptrs & 15) == 0 && ldw % epv == 0 && ldx % epv == 0 && lddx % epv == 0 && (!bf || ldwt % epv == 0) && (dc_by_row || ldc % epv == 0);
+  const bool aligned = (ptrs & 15) == 0 && ldw % epv == 0 && ldx % epv == 0 && lddx % epv == 0 && (dc_by_row || ldc % epv == 0);
   CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: row strides and pointers must be multiples of 16 bytes");
   CUEQ_REQUIRE(split == !dc_by_row, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: built for one input with dC by rows (C x M) and two inputs with dC by columns (M x C)");
   const int64_t es = bf ? 2 : 4;
-  CUEQ_REQUIRE(ldc >= 0 && ldw >= 0 && ldwt >= 0 && 32 * ldw * es < (1ll << 31) && (K + 1) * ldwt * es < (1ll << 31) &&
+  CUEQ_REQUIRE(ldc >= 0 && ldw >= 0 && 32 * ldw * es < (1ll << 31) &&
                    (dc_by_row ? (4 * ldc + M) : (M * ldc + 8)) * es < (1ll << 32),
                CUEQ_ERR_TOO_LARGE, "gate_bwd_input: strides too large for 32-bit lane offsets");
   KernelTimer timer("gate_bwd_input", stream);
-#define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP, !SP>), dim3(static_cast<unsigned>((M + gbi_threads<TI, SP>() / 2 - 1) / (gbi_threads<TI, SP>() / 2))), dim3(gbi_threads<TI, SP>()), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(W1T), static_cast<const TI*>(W2T), ldwt, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
+#define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP, !SP>), dim3(static_cast<unsigned>((M + gbi_threads<TI, SP>() / 2 - 1) / (gbi_threads<TI, SP>() / 2))), dim3(gbi_threads<TI, SP>()), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
 #define GBI_K(TI, SP) do { switch (K / 32) { case 1: GBI(TI, 1, SP); break; case 2: GBI(TI, 2, SP); break; case 3: GBI(TI, 3, SP); break; default: GBI(TI, 4, SP); break; } } while (0)
 #define GBI_T(TI) do { if (split) GBI_K(TI, true); else GBI_K(TI, false); } while (0)
   TRI_DISPATCH(dtype, GBI_T(float), GBI_T(uint16_t));

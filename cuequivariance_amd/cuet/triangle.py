@@ -206,9 +206,6 @@ def gate_bwd_input(dC, dc_by_row: bool, W1, W2, X1, X2, bias1, bias2, mask, dX1=
     es = W1.element_size()
     if K % 32 or K > 128 or Cn % 32 or not _fusable(W1, W2, X1, X2, dC, dX1):
         return None
-    bf = T == torch.bfloat16
-    W1T = transpose(W1) if bf else None
-    W2T = transpose(W2) if bf else None
     accumulate = dX1 is not None
     if dX1 is None:
         dX1 = torch.empty(M, K, dtype=T, device=W1.device)
@@ -216,7 +213,7 @@ def gate_bwd_input(dC, dc_by_row: bool, W1, W2, X1, X2, bias1, bias2, mask, dX1=
     dU = torch.empty_like(dC) if want_gate_grads else None
     dV = torch.empty_like(dC) if want_gate_grads else None
     _lib.check(
-        _lib.load().cueq_gate_bwd_input(_CODE[T], Cn, M, K, W1.data_ptr(), W2.data_ptr(), W1.stride(0), _ptr(W1T), _ptr(W2T), Cn,
+        _lib.load().cueq_gate_bwd_input(_CODE[T], Cn, M, K, W1.data_ptr(), W2.data_ptr(), W1.stride(0),
                                         X1.data_ptr(), _ptr(X2), X1.stride(0), _ptr(bias1), _ptr(bias2), _ptr(mask), dC.data_ptr(),
                                         dC.stride(0), int(dc_by_row), dX1.data_ptr(), _ptr(dX2), dX1.stride(0), int(accumulate),
                                         _ptr(dU), _ptr(dV), _stream(W1)),

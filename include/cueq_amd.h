@@ -212,11 +212,11 @@ int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_
  *   X2 NULL or == X1:  dX1[m,:] (+)= sum_c du W1[c,:] + dv W2[c,:]          (accumulate != 0 adds to dX1)
  *   otherwise:         dX1[m,:]  =  sum_c du W1[c,:],   dX2[m,:] = sum_c dv W2[c,:]
  * dC (and dU, dV when not NULL: the gate gradients for the weight / bias gradients) are C x M with row stride ldc when
- * dc_by_row != 0, M x C otherwise.  bfloat16 also takes the transposed weights W1T, W2T (K x C, row stride ldwt).
+ * dc_by_row != 0, M x C otherwise (built for one input with dC by rows and for two inputs with dC by columns).
  * K must be 32, 64, 96 or 128 and C a multiple of 32; strides and pointers multiples of 16 bytes, else
  * CUEQ_ERR_UNSUPPORTED (compose cueq_dual_gate and cueq_gemm_nt instead). */
 int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
-                        const void* W1T, const void* W2T, int64_t ldwt, const void* X1, const void* X2, int64_t ldx,
+                        const void* X1, const void* X2, int64_t ldx,
                         const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
                         int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
                         void* stream);
