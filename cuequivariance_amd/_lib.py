@@ -39,6 +39,9 @@ EXPORTED_SYMBOLS = (
     "cueq_seg_rowdot",
     "cueq_gemm_nt",
     "cueq_gemm",
+    "cueq_layer_norm_t_fwd",
+    "cueq_layer_norm_t_bwd_workspace",
+    "cueq_layer_norm_t_bwd",
     "cueq_dual_gate",
     "cueq_gate_bwd_input",
     "cueq_gemm_tn_items",
@@ -173,6 +176,12 @@ def load() -> C.CDLL:
         lib.cueq_gemm_nt.restype = C.c_int
         lib.cueq_gemm.argtypes = [i32, i32, i32, i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, ptr, i64, i64, i64, f64, i32, ptr]
         lib.cueq_gemm.restype = C.c_int
+        lib.cueq_layer_norm_t_fwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, f64, ptr, ptr, ptr, ptr]
+        lib.cueq_layer_norm_t_fwd.restype = C.c_int
+        lib.cueq_layer_norm_t_bwd_workspace.argtypes = [i32, i64, i64]
+        lib.cueq_layer_norm_t_bwd_workspace.restype = C.c_int64
+        lib.cueq_layer_norm_t_bwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, i64, ptr]
+        lib.cueq_layer_norm_t_bwd.restype = C.c_int
         lib.cueq_dual_gate.argtypes = [i32, i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i32, ptr, i32, ptr, ptr, ptr, i64, ptr]
         lib.cueq_dual_gate.restype = C.c_int
         lib.cueq_gate_bwd_input.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, ptr, ptr, i64,

@@ -1173,6 +1173,226 @@ __global__ void __launch_bounds__(256) ln_bwd_rows8(const T* __restrict__ dy, co
 }
 
 // ------------------------------------------------------------------------------------------------
+// LayerNorm over d of a tensor stored d-major, x_t (D x M, row d contiguous in m), with the result row-major
+// y (M x D): the "LayerNorm with a layout change" of the triangle update (_layer_norm_transpose.py:162-227) in one
+// pass instead of a transpose and a row LayerNorm.  A block takes MT = 128 / sizeof(T) bytes-worth of consecutive m
+// (64 two-byte or 32 four-byte elements: 128-byte row segments of x_t) for all d through an LDS tile.
+// The backward takes dy (M x D) and x_t and writes dx_t (D x M); blocks walk tiles with a stride so that the
+// gamma / beta partial sums stay few.
+// ------------------------------------------------------------------------------------------------
+constexpr int kLnTMaxD = 256;
+template <typename T>
+struct LnT {
+  static constexpr int MT = 128 / sizeof(T);       // m per tile
+  static constexpr int RS = 132;                   // bytes between d rows of the x tile (33 dwords: no bank conflicts along d)
+  static constexpr int G = 256 / MT;               // thread groups along d
+  static constexpr int EPV = 16 / sizeof(T);
+};
+
+template <typename T>
+__device__ __forceinline__ float lnt_tile(const char* tile, int d, int m) {
+  if constexpr (sizeof(T) == 2) return bf16_bits_to_float(*reinterpret_cast<const uint16_t*>(tile + d * LnT<T>::RS + m * 2));
+  else return *reinterpret_cast<const float*>(tile + d * LnT<T>::RS + m * 4);
+}
+
+// x_t tile [D][MT] -> LDS (vectors beyond M are zero)
+template <typename T>
+__device__ __forceinline__ void lnt_load_tile(char* tile, const T* __restrict__ xt, int64_t M, int D, int64_t m0, int tid) {
+  constexpr int VPRM = 8;  // 16-byte vectors per 128-byte row segment
+  for (int idx = tid; idx < D * VPRM; idx += 256) {
+    const int d = idx / VPRM, v = idx % VPRM;
+    const int64_t m = m0 + v * LnT<T>::EPV;
+    uint4 val = make_uint4(0, 0, 0, 0);
+    if (m < M) val = *reinterpret_cast<const uint4*>(xt + static_cast<int64_t>(d) * M + m);
+    uint32_t* p = reinterpret_cast<uint32_t*>(tile + d * LnT<T>::RS + v * 16);
+    p[0] = val.x; p[1] = val.y; p[2] = val.z; p[3] = val.w;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) ln_t_fwd_kernel(const T* __restrict__ xt, const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                       T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int D,
+                                                       float eps) {
+  using L = LnT<T>;
+  extern __shared__ __align__(16) char lnt_dyn[];  // D * RS bytes: the x tile
+  char* tile = lnt_dyn;
+  __shared__ float red[L::G][L::MT];
+  __shared__ float smean[L::MT], srstd[L::MT];
+  __shared__ __align__(16) float sgam[kLnTMaxD], sbet[kLnTMaxD];
+  const int tid = threadIdx.x;
+  const int64_t m0 = static_cast<int64_t>(blockIdx.x) * L::MT;
+  lnt_load_tile<T>(tile, xt, M, D, m0, tid);
+  if (tid < D) {
+    sgam[tid] = gamma ? tri_load(gamma, tid) : 1.0f;
+    sbet[tid] = beta ? tri_load(beta, tid) : 0.0f;
+  }
+  __syncthreads();
+  const int m = tid % L::MT, g = tid / L::MT;
+  float s = 0;
+  for (int d = g; d < D; d += L::G) s += lnt_tile<T>(tile, d, m);
+  red[g][m] = s;
+  __syncthreads();
+  if (tid < L::MT) {
+    float t = 0;
+#pragma unroll
+    for (int k = 0; k < L::G; ++k) t += red[k][tid];
+    smean[tid] = t / D;
+  }
+  __syncthreads();
+  const float mu = smean[m];
+  s = 0;
+  for (int d = g; d < D; d += L::G) {
+    const float c = lnt_tile<T>(tile, d, m) - mu;
+    s += c * c;
+  }
+  red[g][m] = s;
+  __syncthreads();
+  if (tid < L::MT) {
+    float t = 0;
+#pragma unroll
+    for (int k = 0; k < L::G; ++k) t += red[k][tid];
+    const float r = rsqrtf(t / D + eps);
+    srstd[tid] = r;
+    if (m0 + tid < M) {
+      mean[m0 + tid] = smean[tid];
+      rstd[m0 + tid] = r;
+    }
+  }
+  __syncthreads();
+  // rows of y: 16-byte vectors along d
+  const int vpr = D / L::EPV;
+  for (int idx = tid; idx < L::MT * vpr; idx += 256) {
+    const int r = idx / vpr, v = idx % vpr;
+    if (m0 + r >= M) continue;
+    const float mu2 = smean[r], rs = srstd[r];
+    float o[L::EPV];
+#pragma unroll
+    for (int e = 0; e < L::EPV; ++e) {
+      const int d = v * L::EPV + e;
+      o[e] = (lnt_tile<T>(tile, d, r) - mu2) * rs * sgam[d] + sbet[d];
+    }
+    uint4 out;
+    if constexpr (sizeof(T) == 2) out = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+    else out = make_uint4(__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3]));
+    *reinterpret_cast<uint4*>(y + (m0 + r) * D + v * L::EPV) = out;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) ln_t_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ xt, const float* __restrict__ mean,
+                                                       const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dxt,
+                                                       float* __restrict__ part, int64_t M, int D, int64_t ntiles, int need_affine) {
+  using L = LnT<T>;
+  constexpr int PW = 4 / sizeof(T);  // elements per 4-byte store along m
+  extern __shared__ __align__(16) char lnt_dyn[];  // the x tile (D * RS bytes, rounded up to 16), then the dy tile (MT * DS)
+  char* tile = lnt_dyn;
+  char* dtile = lnt_dyn + ((D * L::RS + 15) & ~15);
+  __shared__ float red1[L::G][L::MT], red2[L::G][L::MT];
+  __shared__ float smean[L::MT], srstd[L::MT], c1[L::MT], c2[L::MT];
+  __shared__ float sgam[kLnTMaxD];
+  const int tid = threadIdx.x;
+  if (tid < D) sgam[tid] = gamma ? tri_load(gamma, tid) : 1.0f;  // visible after the first barrier of the tile loop
+  const int DS = D * static_cast<int>(sizeof(T)) + 4;  // bytes between rows of the dy tile
+  const int vpr = D / L::EPV;
+  auto dyv = [&](int m, int d) -> float {
+    if constexpr (sizeof(T) == 2) return bf16_bits_to_float(*reinterpret_cast<const uint16_t*>(dtile + m * DS + d * 2));
+    else return *reinterpret_cast<const float*>(dtile + m * DS + d * 4);
+  };
+  float sg[(kLnTMaxD + 255) / 256] = {0}, sb[(kLnTMaxD + 255) / 256] = {0};  // this thread's d: partial dgamma / dbeta
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int64_t m0 = t * L::MT;
+    __syncthreads();  // the previous tile is no longer read
+    lnt_load_tile<T>(tile, xt, M, D, m0, tid);
+    for (int idx = tid; idx < L::MT * vpr; idx += 256) {
+      const int r = idx / vpr, v = idx % vpr;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (m0 + r < M) val = *reinterpret_cast<const uint4*>(dy + (m0 + r) * D + v * L::EPV);
+      uint32_t* p = reinterpret_cast<uint32_t*>(dtile + r * DS + v * 16);
+      p[0] = val.x; p[1] = val.y; p[2] = val.z; p[3] = val.w;
+    }
+    if (tid < L::MT) {
+      const bool ok = m0 + tid < M;
+      smean[tid] = ok ? mean[m0 + tid] : 0.f;
+      srstd[tid] = ok ? rstd[m0 + tid] : 0.f;
+    }
+    __syncthreads();
+    const int m = tid % L::MT, g = tid / L::MT;
+    {
+      const float mu = smean[m], rs = srstd[m];
+      float s1 = 0, s2 = 0;
+      for (int d = g; d < D; d += L::G) {
+        const float xh = (lnt_tile<T>(tile, d, m) - mu) * rs;
+        const float gg = dyv(m, d) * sgam[d];
+        s1 += gg;
+        s2 += gg * xh;
+      }
+      red1[g][m] = s1;
+      red2[g][m] = s2;
+    }
+    __syncthreads();
+    if (tid < L::MT) {
+      float a = 0, b = 0;
+#pragma unroll
+      for (int k = 0; k < L::G; ++k) { a += red1[k][tid]; b += red2[k][tid]; }
+      c1[tid] = a / D;
+      c2[tid] = b / D;
+    }
+    __syncthreads();
+    // dx_t[d][m]: 4-byte stores along m
+    {
+      constexpr int MP = L::MT / PW;  // stores per d row
+      const int mp = tid % MP, dg = tid / MP;
+      const int64_t mg = m0 + mp * PW;
+      if (mg < M) {
+        float rs[PW], mu[PW], k1[PW], k2[PW];
+#pragma unroll
+        for (int e = 0; e < PW; ++e) {
+          rs[e] = srstd[mp * PW + e]; mu[e] = smean[mp * PW + e]; k1[e] = c1[mp * PW + e]; k2[e] = c2[mp * PW + e];
+        }
+#pragma unroll 4
+        for (int d = dg; d < D; d += 256 / MP) {
+          const float gmm = sgam[d];
+          float o[PW];
+#pragma unroll
+          for (int e = 0; e < PW; ++e) {
+            const int mm = mp * PW + e;
+            const float xh = (lnt_tile<T>(tile, d, mm) - mu[e]) * rs[e];
+            o[e] = rs[e] * (dyv(mm, d) * gmm - k1[e] - xh * k2[e]);
+          }
+          uint32_t w;
+          if constexpr (sizeof(T) == 2) w = pack_bf16(o[0], o[1]);
+          else w = __float_as_uint(o[0]);
+          *reinterpret_cast<uint32_t*>(dxt + static_cast<int64_t>(d) * M + mg) = w;
+        }
+      }
+    }
+    if (need_affine) {
+#pragma unroll
+      for (int q = 0; q < (kLnTMaxD + 255) / 256; ++q) {
+        const int d = tid + q * 256;
+        if (d < D) {
+          for (int mm = 0; mm < L::MT; ++mm) {  // rows beyond M hold zeros in the dy tile
+            const float v = dyv(mm, d);
+            sg[q] += v * (lnt_tile<T>(tile, d, mm) - smean[mm]) * srstd[mm];
+            sb[q] += v;
+          }
+        }
+      }
+    }
+  }
+  if (need_affine) {
+#pragma unroll
+    for (int q = 0; q < (kLnTMaxD + 255) / 256; ++q) {
+      const int d = tid + q * 256;
+      if (d < D) {
+        part[static_cast<int64_t>(blockIdx.x) * D + d] = sg[q];
+        part[(static_cast<int64_t>(gridDim.x) + blockIdx.x) * D + d] = sb[q];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // gate: out[r][c] = sigmoid(u + bu) * (v + bv) * mask;  biases and mask are indexed by row (axis 0) or column (axis 1)
 // ------------------------------------------------------------------------------------------------
 template <typename T>
@@ -1513,6 +1733,80 @@ extern "C" int cueq_layer_norm_bwd(int32_t dtype, int64_t rows, int64_t D, const
 #undef LN_BWD_NQ
 #undef LN_BWD
     }
+  }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  const unsigned g = static_cast<unsigned>((D + 255) / 256);
+  if (dgamma) hipLaunchKernelGGL(fold_partials_kernel<float>, dim3(g), dim3(256), 0, stream, part, dgamma, nb, D, 0);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  if (dbeta) hipLaunchKernelGGL(fold_partials_kernel<float>, dim3(g), dim3(256), 0, stream, part + nb * D, dbeta, nb, D, 0);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+static bool ln_t_ok(int32_t dtype, int64_t M, int64_t D, const void* a, const void* b, const void* c) {
+  const int epv = dtype == CUEQ_F32 ? 4 : 8;
+  return D > 0 && D <= kLnTMaxD && D % epv == 0 && M % epv == 0 &&
+         ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15) == 0;
+}
+
+extern "C" int cueq_layer_norm_t_fwd(int32_t dtype, int64_t M, int64_t D, const void* x_t, const void* gamma, const void* beta, double eps,
+                                     void* y, float* mean, float* rstd, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "layer_norm_t: dtype must be float32 or bfloat16");
+  if (M <= 0) return CUEQ_OK;
+  CUEQ_REQUIRE(x_t && y && mean && rstd, CUEQ_ERR_INVALID, "layer_norm_t: null operand");
+  CUEQ_REQUIRE(ln_t_ok(dtype, M, D, x_t, y, nullptr), CUEQ_ERR_UNSUPPORTED,
+               "layer_norm_t: D must be at most %d, D and M multiples of 16 bytes of elements, pointers 16-byte aligned", kLnTMaxD);
+  const int64_t mt = dtype == CUEQ_F32 ? 32 : 64;
+  const int64_t ntiles = (M + mt - 1) / mt;
+  CUEQ_REQUIRE(ntiles < (1ll << 31), CUEQ_ERR_TOO_LARGE, "layer_norm_t: too many rows");
+  const size_t fwd_lds = static_cast<size_t>(D) * 132;
+  KernelTimer timer("layer_norm_t_fwd", stream);
+  TRI_DISPATCH(dtype,
+               hipLaunchKernelGGL(ln_t_fwd_kernel<float>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const float*>(x_t), static_cast<const float*>(gamma), static_cast<const float*>(beta), static_cast<float*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)),
+               hipLaunchKernelGGL(ln_t_fwd_kernel<uint16_t>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const uint16_t*>(x_t), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)));
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+static int64_t ln_t_bwd_blocks(int32_t dtype, int64_t M) {
+  const int64_t mt = dtype == CUEQ_F32 ? 32 : 64;
+  const int64_t ntiles = (M + mt - 1) / mt;
+  const int64_t nb = static_cast<int64_t>(device_cus()) * 8;
+  return ntiles < nb ? (ntiles < 1 ? 1 : ntiles) : nb;
+}
+
+extern "C" int64_t cueq_layer_norm_t_bwd_workspace(int32_t dtype, int64_t M, int64_t D) {
+  return ln_t_bwd_blocks(dtype, M) * 2 * D * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int cueq_layer_norm_t_bwd(int32_t dtype, int64_t M, int64_t D, const void* dy, const void* x_t, const float* mean, const float* rstd,
+                                     const void* gamma, void* dx_t, float* dgamma, float* dbeta, void* workspace, int64_t workspace_bytes,
+                                     void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "layer_norm_t: dtype must be float32 or bfloat16");
+  if (M <= 0) {
+    if (dgamma) CUEQ_CHECK_HIP(hipMemsetAsync(dgamma, 0, D * sizeof(float), stream));
+    if (dbeta) CUEQ_CHECK_HIP(hipMemsetAsync(dbeta, 0, D * sizeof(float), stream));
+    return CUEQ_OK;
+  }
+  CUEQ_REQUIRE(dy && x_t && mean && rstd && dx_t, CUEQ_ERR_INVALID, "layer_norm_t: null operand");
+  CUEQ_REQUIRE(ln_t_ok(dtype, M, D, x_t, dy, dx_t), CUEQ_ERR_UNSUPPORTED,
+               "layer_norm_t: D must be at most %d, D and M multiples of 16 bytes of elements, pointers 16-byte aligned", kLnTMaxD);
+  const int need_affine = (dgamma || dbeta) ? 1 : 0;
+  CUEQ_REQUIRE(!need_affine || (workspace && workspace_bytes >= cueq_layer_norm_t_bwd_workspace(dtype, M, D)), CUEQ_ERR_INVALID,
+               "layer_norm_t: workspace too small");
+  const int64_t mt = dtype == CUEQ_F32 ? 32 : 64;
+  const int64_t ntiles = (M + mt - 1) / mt;
+  const int64_t nb = ln_t_bwd_blocks(dtype, M);
+  float* part = static_cast<float*>(workspace);
+  const int64_t es = dtype == CUEQ_F32 ? 4 : 2;
+  const size_t bwd_lds = static_cast<size_t>(((D * 132 + 15) & ~15ll) + mt * (D * es + 4));
+  {
+    KernelTimer timer("layer_norm_t_bwd", stream);
+    TRI_DISPATCH(dtype,
+                 hipLaunchKernelGGL(ln_t_bwd_kernel<float>, dim3(static_cast<unsigned>(nb)), dim3(256), bwd_lds, stream, static_cast<const float*>(dy), static_cast<const float*>(x_t), mean, rstd, static_cast<const float*>(gamma), static_cast<float*>(dx_t), part, M, static_cast<int>(D), ntiles, need_affine),
+                 hipLaunchKernelGGL(ln_t_bwd_kernel<uint16_t>, dim3(static_cast<unsigned>(nb)), dim3(256), bwd_lds, stream, static_cast<const uint16_t*>(dy), static_cast<const uint16_t*>(x_t), mean, rstd, static_cast<const uint16_t*>(gamma), static_cast<uint16_t*>(dx_t), part, M, static_cast<int>(D), ntiles, need_affine));
   }
   CUEQ_CHECK_HIP(hipGetLastError());
   const unsigned g = static_cast<unsigned>((D + 255) / 256);

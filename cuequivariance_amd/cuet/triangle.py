@@ -124,6 +124,43 @@ def layer_norm_bwd(dy: torch.Tensor, x: torch.Tensor, mean, rstd, gamma, need_af
     return dx, dgamma, dbeta
 
 
+def _ln_t_ok(xt: torch.Tensor) -> bool:
+    D, M = xt.shape
+    epv = 16 // xt.element_size()
+    return D <= 256 and D % epv == 0 and M % epv == 0 and xt.data_ptr() % 16 == 0
+
+
+def layer_norm_t_fwd(xt: torch.Tensor, gamma, beta, eps: float):
+    """LayerNorm over d of ``xt (D, M)`` into ``y (M, D)`` (one kernel, no transposed copy)."""
+    D, M = xt.shape
+    y = torch.empty(M, D, dtype=xt.dtype, device=xt.device)
+    mean = torch.empty(M, dtype=torch.float32, device=xt.device)
+    rstd = torch.empty(M, dtype=torch.float32, device=xt.device)
+    _lib.check(
+        _lib.load().cueq_layer_norm_t_fwd(_CODE[xt.dtype], M, D, xt.data_ptr(), _ptr(gamma), _ptr(beta), float(eps), y.data_ptr(),
+                                          mean.data_ptr(), rstd.data_ptr(), _stream(xt)),
+        "cueq_layer_norm_t_fwd",
+    )
+    return y, mean, rstd
+
+
+def layer_norm_t_bwd(dy: torch.Tensor, xt: torch.Tensor, mean, rstd, gamma, need_affine: bool):
+    """Backward of :func:`layer_norm_t_fwd`: ``dy (M, D)`` -> ``dxt (D, M)`` (+ float32 ``dgamma``, ``dbeta``)."""
+    D, M = xt.shape
+    lib = _lib.load()
+    dxt = torch.empty_like(xt)
+    dgamma = torch.empty(D, dtype=torch.float32, device=xt.device) if need_affine else None
+    dbeta = torch.empty(D, dtype=torch.float32, device=xt.device) if need_affine else None
+    ws_bytes = lib.cueq_layer_norm_t_bwd_workspace(_CODE[xt.dtype], M, D) if need_affine else 0
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=xt.device) if need_affine else None
+    _lib.check(
+        lib.cueq_layer_norm_t_bwd(_CODE[xt.dtype], M, D, dy.data_ptr(), xt.data_ptr(), mean.data_ptr(), rstd.data_ptr(), _ptr(gamma),
+                                  dxt.data_ptr(), _ptr(dgamma), _ptr(dbeta), _ptr(ws), ws_bytes, _stream(xt)),
+        "cueq_layer_norm_t_bwd",
+    )
+    return dxt, dgamma, dbeta
+
+
 def gate_fwd(u, v, bias_u, bias_v, bias_axis: int, mask, mask_axis: int, dtype) -> torch.Tensor:
     rows, cols = u.shape
     out = torch.empty(rows, cols, dtype=dtype, device=u.device)
@@ -284,11 +321,14 @@ class _TriMul(torch.autograd.Function):
             t = gemm_nt(a, b, T)  # t[i, j] = sum_k a[i, k] b[j, k]
         else:
             t = gemm_nt(a, b, T, trans_a=True, trans_b=True)  # t[i, j] = sum_k a[k, i] b[k, j]
-        tT = transpose(t.view(D, M))  # (M, D)
-        y, mean2, rstd2 = layer_norm_fwd(tT, nout_w, nout_b, eps)
+        t2 = t.view(D, M)
+        if _ln_t_ok(t2):
+            y, mean2, rstd2 = layer_norm_t_fwd(t2, nout_w, nout_b, eps)  # (M, D)
+        else:
+            y, mean2, rstd2 = layer_norm_fwd(transpose(t2), nout_w, nout_b, eps)
         out = dual_gate_fwd(xh, y, g_out_w, p_out_w, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
         ctx.save_for_backward(x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
-                              xh, mean1, rstd1, ab, tT, mean2, rstd2, y)
+                              xh, mean1, rstd1, ab, t2, mean2, rstd2, y)
         ctx.outgoing, ctx.dims = outgoing, (Bsz, N, D, Do)
         ctx.has = (nin_w is not None, nin_b is not None, nout_w is not None, nout_b is not None)
         return out.view(Bsz, N, N, Do)
@@ -296,7 +336,7 @@ class _TriMul(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout):
         (x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
-         xh, mean1, rstd1, ab, tT, mean2, rstd2, y) = ctx.saved_tensors
+         xh, mean1, rstd1, ab, t2, mean2, rstd2, y) = ctx.saved_tensors
         Bsz, N, D, Do = ctx.dims
         M = Bsz * N * N
         T = x2.dtype
@@ -326,8 +366,12 @@ class _TriMul(torch.autograd.Function):
 
         # LayerNorm across d
         affine_out = (ctx.has[2] and need[8]) or (ctx.has[3] and need[9])
-        dtT, d_nout_w, d_nout_b = layer_norm_bwd(dy, tT, mean2, rstd2, nout_w, affine_out)
-        dt = transpose(dtT).view(D * Bsz, N, N)  # (D, M) viewed per (d, b)
+        if _ln_t_ok(t2):
+            dt, d_nout_w, d_nout_b = layer_norm_t_bwd(dy, t2, mean2, rstd2, nout_w, affine_out)  # (D, M)
+        else:
+            dtT, d_nout_w, d_nout_b = layer_norm_bwd(dy, transpose(t2), mean2, rstd2, nout_w, affine_out)
+            dt = transpose(dtT)
+        dt = dt.view(D * Bsz, N, N)  # (D, M) viewed per (d, b)
 
         # triangular contraction
         a = ab[:D].view(D * Bsz, N, N)

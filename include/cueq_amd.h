@@ -245,6 +245,18 @@ int cueq_layer_norm_bwd(int32_t dtype, int64_t rows, int64_t D, const void* dy, 
                         const float* rstd, const void* gamma, void* dx, float* dgamma, float* dbeta, void* workspace,
                         int64_t workspace_bytes, void* stream);
 
+/* LayerNorm over d of a tensor stored d-major, x_t (D x M), into row-major y (M x D), and its backward from
+ * dy (M x D) to dx_t (D x M): the LayerNorm with a layout change after the triangular contraction
+ * (_layer_norm_transpose.py:162-227) without a transposed copy.  mean, rstd: M floats.  D at most 256; D and M
+ * multiples of 16 bytes of elements and 16-byte aligned pointers, else CUEQ_ERR_UNSUPPORTED (use cueq_transpose and the
+ * row versions).  The workspace (cueq_layer_norm_t_bwd_workspace bytes) is needed when dgamma or dbeta is asked for. */
+int cueq_layer_norm_t_fwd(int32_t dtype, int64_t M, int64_t D, const void* x_t, const void* gamma, const void* beta, double eps,
+                          void* y, float* mean, float* rstd, void* stream);
+int64_t cueq_layer_norm_t_bwd_workspace(int32_t dtype, int64_t M, int64_t D);
+int cueq_layer_norm_t_bwd(int32_t dtype, int64_t M, int64_t D, const void* dy, const void* x_t, const float* mean, const float* rstd,
+                          const void* gamma, void* dx_t, float* dgamma, float* dbeta, void* workspace, int64_t workspace_bytes,
+                          void* stream);
+
 /* out = sigmoid(u + bias_u) * (v + bias_v) * mask on a rows x cols array (u, v float32 accumulators of the two
  * projections); biases (may be NULL) are indexed by row (bias_axis 0) or column (1), the mask (may be NULL)
  * likewise (_sigmoid_gated_dual_gemm.py:135-150).  cueq_gate_bwd returns the gradients of u and v
