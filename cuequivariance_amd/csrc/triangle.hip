@@ -151,8 +151,9 @@ __device__ __forceinline__ uint4 gemm_fragment(const char* tile, int base, int q
 template <typename TI, typename TO, bool TA, bool TB>
 __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
                                                    const TI* __restrict__ B, int64_t ldb, int64_t sB,
-                                                   TO* __restrict__ C, int64_t ldc, int64_t sC, int M, int N, int K,
-                                                   float alpha, int accumulate, int vec_out) {
+                                                   TO* __restrict__ C, int64_t ldc, int64_t sC, int M, int N, int Kfull,
+                                                   float alpha, int accumulate, int vec_out, int64_t k_total, int nparts, int64_t pA,
+                                                   int64_t pB, int64_t pC) {
   constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
   constexpr int BK = 64 / sizeof(TI);   // k extent of one step
   constexpr int TS = sizeof(TI) == 2 ? kTransStride16 : kTransStride32;
@@ -164,9 +165,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
   int bx, by, bz;
   xcd_tile(bx, by, bz);
   const int m0 = by * kTile, n0 = bx * kTile;
-  A += static_cast<int64_t>(bz) * sA;
-  B += static_cast<int64_t>(bz) * sB;
-  C += static_cast<int64_t>(bz) * sC;
+  // batch item = (chunk, part): strides s* between chunks, p* between parts (nparts == 1: a plain batch)
+  const int chunk = bz / nparts, part = bz - chunk * nparts;
+  A += static_cast<int64_t>(chunk) * sA + static_cast<int64_t>(part) * pA;
+  B += static_cast<int64_t>(chunk) * sB + static_cast<int64_t>(part) * pB;
+  C += static_cast<int64_t>(chunk) * sC + static_cast<int64_t>(part) * pC;
+  // k_total > 0: the chunks are consecutive k ranges of one long contraction; the last ones may be short or empty
+  const int K = k_total > 0 ? static_cast<int>(max<int64_t>(0, min<int64_t>(Kfull, k_total - static_cast<int64_t>(chunk) * Kfull))) : Kfull;
 
   // every thread stages two 16-byte vectors of A and two of B per step
   uint4 stA[2], stB[2];
@@ -210,7 +215,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
     for (int j = 0; j < 2; ++j) acc[i][j] = floatx16{0};
 
   const int nsteps = (K + BK - 1) / BK;
-  load_step(0);
+  if (nsteps > 0) load_step(0);
   int buf = 0;
   for (int ks = 0; ks < nsteps; ++ks) {
     store_step(buf);
@@ -1500,7 +1505,7 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
     KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
     const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
     const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
-#define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out)
+#define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0)
 #define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_LAUNCH(TI, TI, true, true); else if (trans_a) GEMM_LAUNCH(TI, TI, true, false); else if (trans_b) GEMM_LAUNCH(TI, TI, false, true); else GEMM_LAUNCH(TI, TI, false, false); } while (0)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_TR(float);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t, false, false);
@@ -1621,6 +1626,16 @@ extern "C" int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows
   const bool vec = M % 8 == 0 && N % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0 &&
                    reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0;
   KernelTimer timer("gemm_tn", stream);
+  if (in_dtype == CUEQ_BF16 && vec && rows > 0) {
+    // 2-byte inputs: bf16 MFMA on contraction-major tiles (transposing LDS reads); batch items = (row chunk, part)
+    const int64_t rpc32 = (((rows + chunks - 1) / chunks + 31) / 32) * 32;
+    hipLaunchKernelGGL((gemm_kernel<uint16_t, float, true, true>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(A), lda,
+                       rpc32 * lda, static_cast<const uint16_t*>(B), ldb, rpc32 * ldb, partials, N, static_cast<int64_t>(nparts) * M * N,
+                       static_cast<int>(M), static_cast<int>(N), static_cast<int>(rpc32), static_cast<float>(alpha), 0, 0, rows, nparts,
+                       stride_a, stride_b, static_cast<int64_t>(M) * N);
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
 #define TN_LAUNCH(TI, V) hipLaunchKernelGGL((gemm_tn_kernel<TI, V>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, partials, static_cast<int>(M), static_cast<int>(N), rows, rpc, nparts, static_cast<float>(alpha))
   if (in_dtype == CUEQ_F32) { if (vec) TN_LAUNCH(float, true); else TN_LAUNCH(float, false); }
   else { if (vec) TN_LAUNCH(uint16_t, true); else TN_LAUNCH(uint16_t, false); }
