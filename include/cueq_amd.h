@@ -234,6 +234,13 @@ int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows, const voi
  * re-orientation for the incoming direction and the backward contractions). */
 int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_t cols, const void* in, void* out, void* stream);
 
+/* Per-segment (u, v) -> (v, u) transposition of every row, one pass: out[r][o] = in[r][src_index[o]] with the row
+ * permutation src_index (device, int32, length total) built once by the caller from the segment list.  Stands for the
+ * native segmented_transpose op behind cuequivariance_torch/primitives/transpose.py:83-183 (mul_ir <-> ir_mul).
+ * element_size 2, 4 or 8 bytes; in and out must not alias. */
+int cueq_segmented_transpose(int32_t element_size, int64_t rows, int64_t total, const int32_t* src_index, const void* in, void* out,
+                             void* stream);
+
 /* Row LayerNorm with biased variance, rstd = 1/sqrt(var + eps) (_layer_norm_transpose.py:196-209); gamma / beta may
  * be NULL; mean and rstd (float32, one per row) are kept for the backward.  D <= 1024. */
 int cueq_layer_norm_fwd(int32_t dtype, int64_t rows, int64_t D, const void* x, const void* gamma, const void* beta,
