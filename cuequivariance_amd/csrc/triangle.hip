@@ -151,9 +151,10 @@ __device__ __forceinline__ uint4 gemm_fragment(const char* tile, int base, int q
 template <typename TI, typename TO, bool TA, bool TB>
 __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
                                                    const TI* __restrict__ B, int64_t ldb, int64_t sB,
-                                                   TO* __restrict__ C, int64_t ldc, int64_t sC, int M, int N, int Kfull,
+                                                   TO* __restrict__ C, int64_t ldc, int64_t sC, int Mfull, int N, int Kfull,
                                                    float alpha, int accumulate, int vec_out, int64_t k_total, int nparts, int64_t pA,
-                                                   int64_t pB, int64_t pC) {
+                                                   int64_t pB, int64_t pC, const int64_t* __restrict__ goff, int ngroups, int gmode,
+                                                   int64_t gsB, int64_t gsC) {
   constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
   constexpr int BK = 64 / sizeof(TI);   // k extent of one step
   constexpr int TS = sizeof(TI) == 2 ? kTransStride16 : kTransStride32;
@@ -164,14 +165,39 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
   const int wm = wave >> 1, wn = wave & 1;
   int bx, by, bz;
   xcd_tile(bx, by, bz);
-  const int m0 = by * kTile, n0 = bx * kTile;
+  int m0 = by * kTile, M = Mfull;
+  const int n0 = bx * kTile;
   // batch item = (chunk, part): strides s* between chunks, p* between parts (nparts == 1: a plain batch)
   const int chunk = bz / nparts, part = bz - chunk * nparts;
   A += static_cast<int64_t>(chunk) * sA + static_cast<int64_t>(part) * pA;
   B += static_cast<int64_t>(chunk) * sB + static_cast<int64_t>(part) * pB;
   C += static_cast<int64_t>(chunk) * sC + static_cast<int64_t>(part) * pC;
   // k_total > 0: the chunks are consecutive k ranges of one long contraction; the last ones may be short or empty
-  const int K = k_total > 0 ? static_cast<int>(max<int64_t>(0, min<int64_t>(Kfull, k_total - static_cast<int64_t>(chunk) * Kfull))) : Kfull;
+  int K = k_total > 0 ? static_cast<int>(max<int64_t>(0, min<int64_t>(Kfull, k_total - static_cast<int64_t>(chunk) * Kfull))) : Kfull;
+  if (gmode == 1) {
+    // rows grouped: rows [goff[g], goff[g+1]) of A and C use the B of group g; the row-tile index walks the groups'
+    // tiles in order (a tile never straddles two groups; the grid has one spare tile per group)
+    int t = by, g = 0;
+    for (; g < ngroups; ++g) {
+      const int64_t lo = goff[g], n = goff[g + 1] - lo;
+      const int nt = static_cast<int>((n + kTile - 1) / kTile);
+      if (t < nt) {
+        m0 = static_cast<int>(lo) + t * kTile;
+        break;
+      }
+      t -= nt;
+    }
+    if (g == ngroups) return;  // the whole block leaves before any barrier
+    M = static_cast<int>(goff[g + 1]);
+    B += static_cast<int64_t>(g) * gsB;
+  } else if (gmode == 2) {
+    // contraction grouped: chunk g contracts rows [goff[g], goff[g+1]) of the contraction-major operands into its own C
+    const int64_t k0 = goff[chunk];
+    K = static_cast<int>(goff[chunk + 1] - k0);
+    A += k0 * lda;
+    B += k0 * ldb;
+    C += static_cast<int64_t>(chunk) * gsC;
+  }
 
   // every thread stages two 16-byte vectors of A and two of B per step
   uint4 stA[2], stB[2];
@@ -1505,7 +1531,7 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
     KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
     const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
     const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
-#define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0)
+#define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0, nullptr, 0, 0, 0, 0)
 #define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_LAUNCH(TI, TI, true, true); else if (trans_a) GEMM_LAUNCH(TI, TI, true, false); else if (trans_b) GEMM_LAUNCH(TI, TI, false, true); else GEMM_LAUNCH(TI, TI, false, false); } while (0)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_TR(float);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t, false, false);
@@ -1534,6 +1560,54 @@ extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int6
                             int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
                             int64_t batch, double alpha, int32_t accumulate, void* stream_) {
   return cueq_gemm(in_dtype, out_dtype, 0, 0, M, N, K, A, lda, stride_a, B, ldb, stride_b, C, ldc, stride_c, batch, alpha, accumulate, stream_);
+}
+
+extern "C" int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mode, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                                 int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
+                                 int64_t batch, const int64_t* offsets, int64_t ngroups, int32_t trans_b, int64_t group_stride, double alpha,
+                                 int32_t accumulate, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm_grouped: dtypes must be float32 or bfloat16");
+  CUEQ_REQUIRE(mode == 1 || mode == 2, CUEQ_ERR_INVALID, "gemm_grouped: mode must be 1 (rows grouped) or 2 (contraction grouped)");
+  CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 1 && ngroups >= 0, CUEQ_ERR_INVALID, "gemm_grouped: bad extents");
+  if (M == 0 || N == 0 || ngroups == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(A && B && C && offsets, CUEQ_ERR_INVALID, "gemm_grouped: null operand");
+  CUEQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch * (mode == 2 ? ngroups : 1) < 65536 && ngroups < 65536,
+               CUEQ_ERR_TOO_LARGE, "gemm_grouped: extent too large");
+  const int epv = in_dtype == CUEQ_F32 ? 4 : 8;
+  const float al = static_cast<float>(alpha);
+  const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
+  const bool ptrs_ok = reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 && lda % epv == 0 && ldb % epv == 0 &&
+                       stride_a % epv == 0 && stride_b % epv == 0 && group_stride % epv == 0;
+  KernelTimer timer(mode == 1 ? "gemm_grouped_rows" : "gemm_grouped_k", stream);
+  if (mode == 1) {
+    // C[z, :] = alpha * A[z, :] . B_g^T for the rows z of group g; B_g = B + g * group_stride is N x K, or K x N with trans_b
+    CUEQ_REQUIRE(in_dtype == out_dtype, CUEQ_ERR_UNSUPPORTED, "gemm_grouped: rows-grouped products keep the dtype");
+    CUEQ_REQUIRE(ptrs_ok && K % epv == 0 && (!trans_b || N % epv == 0), CUEQ_ERR_UNSUPPORTED,
+                 "gemm_grouped: extents, strides and pointers must be multiples of 16 bytes");
+    const int64_t gy = (M + kTile - 1) / kTile + ngroups;
+    CUEQ_REQUIRE(gy < 65536, CUEQ_ERR_TOO_LARGE, "gemm_grouped: too many row tiles");
+    const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>(gy), static_cast<unsigned>(batch));
+    const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
+#define GG(TI, TB) hipLaunchKernelGGL((gemm_kernel<TI, TI, false, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TI*>(C), ldc, stride_c, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), al, accumulate, vec_out, 0, 1, 0, 0, 0, offsets, static_cast<int>(ngroups), 1, group_stride, 0)
+    if (in_dtype == CUEQ_F32) { if (trans_b) GG(float, true); else GG(float, false); }
+    else { if (trans_b) GG(uint16_t, true); else GG(uint16_t, false); }
+#undef GG
+  } else {
+    // C_g (M x N, at C + g * group_stride) (+)= alpha * sum over the rows z of group g of A[z, :M]^T B[z, :N]
+    // (A, B row-major with z as rows: contraction-major operands); batch items are separate column blocks (stride_*)
+    CUEQ_REQUIRE(ptrs_ok && M % epv == 0 && N % epv == 0, CUEQ_ERR_UNSUPPORTED,
+                 "gemm_grouped: extents, strides and pointers must be multiples of 16 bytes");
+    CUEQ_REQUIRE(in_dtype == out_dtype || out_dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "gemm_grouped: the result is the input dtype or float32");
+    const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(ngroups * batch));
+#define GK(TI, TO) hipLaunchKernelGGL((gemm_kernel<TI, TO, true, true>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, 0, static_cast<const TI*>(B), ldb, 0, static_cast<TO*>(C), ldc, 0, static_cast<int>(M), static_cast<int>(N), 0, al, accumulate, 0, 0, static_cast<int>(batch), stride_a, stride_b, stride_c, offsets, static_cast<int>(ngroups), 2, 0, group_stride)
+    if (in_dtype == CUEQ_F32) GK(float, float);
+    else if (out_dtype == CUEQ_F32) GK(uint16_t, float);
+    else GK(uint16_t, uint16_t);
+#undef GK
+  }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
 }
 
 extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_t K, const void* A1, const void* A2, int64_t lda,
@@ -1632,7 +1706,7 @@ extern "C" int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows
     hipLaunchKernelGGL((gemm_kernel<uint16_t, float, true, true>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(A), lda,
                        rpc32 * lda, static_cast<const uint16_t*>(B), ldb, rpc32 * ldb, partials, N, static_cast<int64_t>(nparts) * M * N,
                        static_cast<int>(M), static_cast<int>(N), static_cast<int>(rpc32), static_cast<float>(alpha), 0, 0, rows, nparts,
-                       stride_a, stride_b, static_cast<int64_t>(M) * N);
+                       stride_a, stride_b, static_cast<int64_t>(M) * N, nullptr, 0, 0, 0, 0);
     CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }

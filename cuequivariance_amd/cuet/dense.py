@@ -279,15 +279,91 @@ class _DenseFunction(torch.autograd.Function):
         return None, gw, gx1, gx2
 
 
+class _IndexedDenseFunction(torch.autograd.Function):
+    """Linear with one weight row per class and the batch rows sorted by class (``offsets[c] .. offsets[c+1]`` are the rows
+    of class ``c``): grouped GEMMs on the tiled MFMA kernel (``cueq_gemm_grouped``), no host synchronisation."""
+
+    @staticmethod
+    def forward(ctx, mod: "SegmentedPolynomialDense", w, x1, offsets):
+        dtype = x1.dtype
+        Z, Cn, W = x1.shape[0], w.shape[0], w.shape[1]
+        lib = _lib.load()
+        out = (torch.empty if mod.fwd_covers_output else torch.zeros)((Z, mod.out_size), dtype=dtype, device=x1.device)
+        wd = w.detach().to(dtype).contiguous()
+        x1d = x1.detach().contiguous()
+        if Z > 0:
+            with torch.cuda.device(x1.device):
+                stream = torch.cuda.current_stream(x1.device).cuda_stream
+                code, es = _DTYPE_CODE[dtype], x1d.element_size()
+                written = set()
+                for p, count, da, dc in mod.fwd_groups:
+                    cols = tuple(p.c_off + t * dc for t in range(count))
+                    acc = 1 if any(c in written for c in cols) else 0
+                    written.update(cols)
+                    # out[z, k_seg] (+)= c * x1[z, i_seg] @ W_p[class(z)]; the K x N block is contraction-major as it lies
+                    _lib.check(
+                        lib.cueq_gemm_grouped(code, code, 1, Z, p.N, p.K, x1d.data_ptr() + p.a_off * es, x1d.stride(0), da,
+                                              wd.data_ptr() + p.w_off * es, p.N, 0, out.data_ptr() + p.c_off * es, out.stride(0), dc,
+                                              count, offsets.data_ptr(), Cn, 1, W, p.coeff, acc, stream),
+                        "cueq_gemm_grouped",
+                    )
+        ctx.mod = mod
+        ctx.save_for_backward(w, x1, offsets)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        mod = ctx.mod
+        w, x1, offsets = ctx.saved_tensors
+        dtype = x1.dtype
+        Z, Cn, W = x1.shape[0], w.shape[0], w.shape[1]
+        lib = _lib.load()
+        g = g.contiguous()
+        wd = w.detach().to(dtype).contiguous()
+        x1d = x1.detach().contiguous()
+        gw = gx1 = None
+        with torch.cuda.device(x1.device):
+            stream = torch.cuda.current_stream(x1.device).cuda_stream
+            code, es = _DTYPE_CODE[dtype], x1d.element_size()
+            if ctx.needs_input_grad[2]:
+                gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
+                written = set()
+                for p, count, dc, da in mod.dx1_groups if Z > 0 else []:
+                    cols = tuple(p.a_off + t * da for t in range(count))
+                    acc = 1 if any(c in written for c in cols) else 0
+                    written.update(cols)
+                    # dx1[z, i_seg] (+)= c * g[z, k_seg] @ W_p[class(z)]^T: the K x N block is "N' x K'" for this product
+                    _lib.check(
+                        lib.cueq_gemm_grouped(code, code, 1, Z, p.K, p.N, g.data_ptr() + p.c_off * es, g.stride(0), dc,
+                                              wd.data_ptr() + p.w_off * es, p.N, 0, gx1.data_ptr() + p.a_off * es, gx1.stride(0), da,
+                                              count, offsets.data_ptr(), Cn, 0, W, p.coeff, acc, stream),
+                        "cueq_gemm_grouped",
+                    )
+            if ctx.needs_input_grad[1]:
+                # dW_p[c] += coeff * sum over the rows z of class c of x1[z, i_seg]^T g[z, k_seg]: float32 accumulation
+                gw32 = torch.zeros(Cn, W, dtype=torch.float32, device=x1.device)
+                for p, count, da, dc in mod.fwd_groups if Z > 0 else []:
+                    for t in range(count):
+                        _lib.check(
+                            lib.cueq_gemm_grouped(code, _lib.F32, 2, p.K, p.N, 0, x1d.data_ptr() + (p.a_off + t * da) * es, x1d.stride(0), 0,
+                                                  g.data_ptr() + (p.c_off + t * dc) * es, g.stride(0), 0,
+                                                  gw32.data_ptr() + p.w_off * 4, p.N, 0, 1, offsets.data_ptr(), Cn, 0, W, p.coeff, 1, stream),
+                            "cueq_gemm_grouped",
+                        )
+                gw = gw32.to(w.dtype)
+        return None, gw, gx1, None
+
+
 class SegmentedPolynomialDense(nn.Module):
     """Dense (MFMA) executor for Linear / fully-connected polynomials with weights shared over the batch."""
 
     def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype=None, output_dtype_map: List[int] = None,
-                 name: str = "segmented_polynomial"):
+                 name: str = "segmented_polynomial", method: str = "fused_tp"):
         super().__init__()
         self._polynomial_orig = polynomial
         self._output_dtype_map_orig = output_dtype_map
         self.name = name
+        self.method = method
         if isinstance(math_dtype, str):
             math_dtype = getattr(torch, math_dtype)
         if math_dtype not in (None, torch.float32, torch.float64):
@@ -340,16 +416,41 @@ class SegmentedPolynomialDense(nn.Module):
     def __reduce__(self):
         from .segmented_polynomial import SegmentedPolynomial
 
-        return (SegmentedPolynomial, (self._polynomial_orig, "fused_tp", self.math_dtype, self._output_dtype_map_orig, self.name))
+        return (SegmentedPolynomial, (self._polynomial_orig, self.method, self.math_dtype, self._output_dtype_map_orig, self.name))
+
+    def _indexed(self, w: torch.Tensor, x1: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+        """One weight row per class, rows of ``x1`` sorted by class (reference
+        ``primitives/segmented_polynomial_indexed_linear.py:247-339``: sorted indices are required there too)."""
+        if self.has_x2:
+            raise NotImplementedError("indexed_linear: only the 3-operand (Linear) form is supported")
+        if x1.device.type != "cuda":
+            raise RuntimeError("indexed_linear runs on the GPU only; got tensors on " + str(x1.device))
+        if x1.dtype not in (torch.float32, torch.bfloat16):
+            raise NotImplementedError(f"indexed_linear: float32 and bfloat16 are implemented, got {x1.dtype}")
+        if index.ndim != 1 or index.shape[0] != x1.shape[0]:
+            raise ValueError("indexed_linear: the index must have one entry per batch row")
+        Cn = w.shape[0]
+        if index.numel() > 1:
+            assert bool(torch.all(index[1:] - index[:-1] >= 0)), "Indexed_linear does not support non-sorted indices."
+        counts = torch.bincount(index, minlength=Cn)
+        if counts.shape[0] != Cn:
+            raise ValueError("indexed_linear: an index is out of range of the weight rows")
+        offsets = torch.zeros(Cn + 1, dtype=torch.int64, device=x1.device)
+        offsets[1:] = torch.cumsum(counts, 0)
+        return _IndexedDenseFunction.apply(self, w, x1, offsets)
 
     def forward(self, inputs: List[torch.Tensor], input_indices: Dict[int, torch.Tensor],
                 output_shapes: Dict[int, torch.Tensor], output_indices: Dict[int, torch.Tensor]):
         for i, (x, size) in enumerate(zip(inputs, self.input_sizes)):
             if x.ndim != 2 or x.shape[-1] != size:
                 raise ValueError(f"Input {i} has shape {tuple(x.shape)} but expected shape (rows, {size}).")
-        if input_indices or output_indices or output_shapes:
-            raise NotImplementedError("fused_tp: indexed operands are not implemented by the dense executor")
         w, x1 = inputs[0], inputs[1]
+        if self.method == "indexed_linear" and set(input_indices) == {0} and not output_indices and not output_shapes:
+            return [self._indexed(w, x1, input_indices[0])]
+        if input_indices or output_indices or output_shapes:
+            raise NotImplementedError(
+                f"{self.method}: the dense executor takes weights shared over the batch, or (method='indexed_linear') "
+                "weights indexed by a sorted class index; other indexed operands are not implemented")
         x2 = inputs[2] if self.has_x2 else None
         if x1.device.type != "cuda":
             raise RuntimeError("fused_tp runs on the GPU only; got tensors on " + str(x1.device))

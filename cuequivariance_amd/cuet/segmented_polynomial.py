@@ -205,7 +205,7 @@ class SegmentedPolynomial(nn.Module):
         if method == "":
             warnings.warn(
                 "SegmentedPolynomial() was called without `method`; defaulting to 'uniform_1d'. "
-                "Available methods: 'uniform_1d', 'fused_tp'."
+                "Available methods: 'uniform_1d', 'fused_tp', 'indexed_linear'."
             )
             method = "uniform_1d"
         if method == "uniform_1d":
@@ -220,7 +220,11 @@ class SegmentedPolynomial(nn.Module):
                 "Use 'uniform_1d' or 'fused_tp'."
             )
         elif method == "indexed_linear":
-            raise NotImplementedError("method='indexed_linear' is not implemented by this engine yet")
+            from .dense import SegmentedPolynomialDense
+
+            if math_dtype is not None:
+                warnings.warn("`indexed_linear` does not support explicit `math_dtype`.This will be ignored.")
+            self.m = SegmentedPolynomialDense(polynomial, None, output_dtype_map, name, method="indexed_linear")
         else:
             raise ValueError(f"Invalid method: {method}")
         self.method = method

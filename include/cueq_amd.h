@@ -196,6 +196,19 @@ int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t tran
               const void* A, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc,
               int64_t stride_c, int64_t batch, double alpha, int32_t accumulate, void* stream);
 
+/* Grouped products on the tiled kernel, for a Linear whose weights are chosen per row by a sorted class index
+ * (the closed indexed_linear op behind cuequivariance_torch/primitives/segmented_polynomial_indexed_linear.py:116-156):
+ * offsets (device, int64, ngroups + 1) gives the row range [offsets[g], offsets[g+1]) of group g.
+ *   mode 1, rows grouped:        C[z, :] (+)= alpha * A[z, :K] . B_g^T for the rows z of group g, B_g = B + g * group_stride
+ *                                (N x K, or K x N with trans_b); batch items advance A, B, C by stride_* (column blocks).
+ *   mode 2, contraction grouped: C_g (M x N at C + g * group_stride) (+)= alpha * sum over the rows z of group g of
+ *                                A[z, :M]^T B[z, :N]; K is ignored; out_dtype may be float32 for bfloat16 inputs.
+ * Extents along vectors, strides and pointers must be multiples of 16 bytes (CUEQ_ERR_UNSUPPORTED otherwise). */
+int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mode, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                      int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
+                      int64_t batch, const int64_t* offsets, int64_t ngroups, int32_t trans_b, int64_t group_stride, double alpha,
+                      int32_t accumulate, void* stream);
+
 /* The gated dual projection in one kernel (_sigmoid_gated_dual_gemm.py:111-218): u = A1 B1^T, v = A2 B2^T (A* M x K, B* N x K,
  * contraction contiguous; B2 NULL: same as B1), then
  *   backward == 0:  out1 = sigmoid(u + bias1) * (v + bias2) * mask

@@ -128,3 +128,47 @@ def test_linear_full_size_properties(device):
     lhs = (cot.double() * y.detach().double()).sum().item()
     assert abs((gw.double() * w.detach().double()).sum().item() - lhs) <= 1e-4 * abs(lhs) + 1e-3 * scale
     assert abs((gx.double() * x.detach().double()).sum().item() - lhs) <= 1e-4 * abs(lhs) + 1e-3 * scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(
+    "irreps,classes,sizes",
+    [
+        # the reference's own case (segmented_polynomial_test.py:480-486: linear 16x0e+16x1o+16x2e, first input indexed)
+        ("16x0e+16x1o+16x2e", 4, [70, 0, 1, 200]),
+        # MACE-style per-species Linear: 128 channels, 10 species, ragged class sizes around the 128-row tile
+        ("128x0e+128x1o+128x2e", 10, [128, 5, 0, 300, 129, 127, 256, 0, 1, 64]),
+    ],
+)
+def test_indexed_linear_matches_oracle(device, dtype, irreps, classes, sizes):
+    """``method="indexed_linear"``: one weight row per class, rows sorted by class (grouped MFMA GEMMs), forward and
+    the gradients w.r.t. weights and input against the oracle's gather-then-contract evaluation."""
+    from cuequivariance_amd import cuet
+
+    m = cuet.Linear(cue.Irreps("O3", irreps), cue.Irreps("O3", irreps), layout=cue.ir_mul, internal_weights=False,
+                    weight_classes=classes, method="indexed_linear")
+    Z = sum(sizes)
+    g = torch.Generator().manual_seed(Z)
+    idx = torch.repeat_interleave(torch.arange(classes), torch.tensor(sizes))
+    w = torch.randn(classes, m.weight_numel, dtype=torch.float64, generator=g).to(dtype).double()
+    x = torch.randn(Z, m.irreps_in.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+    a = [w.clone().requires_grad_(True), x.clone().requires_grad_(True)]
+    ref = naive_segmented_polynomial(spec, a, input_indices={0: idx})[0]
+    cot = torch.randn(ref.shape, dtype=torch.float64, generator=g).to(dtype).double()
+    ref_grads = torch.autograd.grad(ref, a, cot)
+    wg = w.to(dtype).to(device).requires_grad_(True)
+    xg = x.to(dtype).to(device).requires_grad_(True)
+    out = m(xg, wg, idx.to(torch.int32).to(device))
+    assert out.dtype == dtype and out.shape == ref.shape
+    grads = torch.autograd.grad(out, [wg, xg], cot.to(dtype).to(device))
+    tol = TOL[dtype]
+    assert rel_err(out, ref) <= tol, ("out", rel_err(out, ref))
+    for name, got, want in zip(("dw", "dx"), grads, ref_grads):
+        assert rel_err(got, want) <= tol, (name, rel_err(got, want))
+    # int64 indices give the same bits; unsorted indices are refused like in the reference
+    out64 = m(xg, wg, idx.to(device))
+    assert torch.equal(out64, out)
+    if Z > 2:
+        with pytest.raises(AssertionError):
+            m(xg, wg, idx.flip(0).to(device))
