@@ -138,7 +138,12 @@ def test_oracle_reproduces_original_mace_output():
     assert tuple(m.weight.shape) == tuple(w.shape)
     weight = torch.einsum("zau,ab->zbu", w.double(), m.projection.double()).flatten(1)
     out = naive_segmented_polynomial(spec_from_polynomial(m.etp.polynomial), [weight, x.double()], {0: idx})[0]
-    torch.testing.assert_close(m.transpose_out(out).float(), expected, atol=g["atol"], rtol=g["rtol"])
+    # the golden vector is in the mul_ir layout; the oracle works in ir_mul: per-segment (ir, mul) -> (mul, ir) by views
+    parts, off = [], 0
+    for mul, ir in m.irreps_out:
+        parts.append(out[:, off: off + mul * ir.dim].reshape(-1, ir.dim, mul).transpose(1, 2).reshape(-1, mul * ir.dim))
+        off += mul * ir.dim
+    torch.testing.assert_close(torch.cat(parts, dim=1).float(), expected, atol=g["atol"], rtol=g["rtol"])
 
 
 @pytest.mark.gpu
