@@ -470,11 +470,22 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
     for (int t = 0; t < NT; ++t) *reinterpret_cast<uint4*>(&smem[buf][t][ldrow * kRowBytes + ldpart * 16]) = st[t];
   };
 
+  // the accumulators start from the biases (by row or by column of the result)
+  const int col = n0 + wn * 32 + c;
+  const int colc = min(col, N - 1);
   floatx16 acc[2][2];  // [product][i]
 #pragma unroll
-  for (int p = 0; p < 2; ++p)
+  for (int p = 0; p < 2; ++p) {
+    const TI* bias = p == 0 ? bias1 : bias2;
+    const float cb = (bias && bias_axis == 1) ? tri_load(bias, colc) : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) acc[p][i] = floatx16{0};
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = min(m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * h + (v & 3), M - 1);
+        acc[p][i][v] = (bias && bias_axis == 0) ? tri_load(bias, row) : cb;
+      }
+  }
 
   const int nsteps = (K + BK - 1) / BK;
   load_step(0);
@@ -515,12 +526,8 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
     buf ^= 1;
   }
 
-  const int col = n0 + wn * 32 + c;
-  const int colc = min(col, N - 1);
-  const float cb1 = (bias1 && bias_axis == 1) ? tri_load(bias1, colc) : 0.f;
-  const float cb2 = (bias2 && bias_axis == 1) ? tri_load(bias2, colc) : 0.f;
   const float cmk = (mask && mask_axis == 1) ? tri_load(mask, colc) : 1.f;
-  const bool rowb1 = bias1 && bias_axis == 0, rowb2 = bias2 && bias_axis == 0, rowmk = mask && mask_axis == 0;
+  const bool rowmk = mask && mask_axis == 0;
 
   if constexpr (!BWD) {
     // whole block tile inside the output and 16-byte aligned rows: 64 rows at a time through LDS
@@ -538,9 +545,7 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
               const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-              const float uu = acc[0][i][v] + (rowb1 ? tri_load(bias1, row) : cb1);
-              const float vv = acc[1][i][v] + (rowb2 ? tri_load(bias2, row) : cb2);
-              g[v] = __builtin_amdgcn_rcpf(1.0f + __expf(-uu)) * vv * (rowmk ? tri_load(mask, row) : cmk);
+              g[v] = __builtin_amdgcn_rcpf(1.0f + __expf(-acc[0][i][v])) * acc[1][i][v] * (rowmk ? tri_load(mask, row) : cmk);
             }
             stage_put<TI>(tile + i * 32 * RS, RS, wn * 32 + c, h, g, 1.0f);
           }
@@ -559,9 +564,8 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
       const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
       if (row < M) {
         const int64_t o = static_cast<int64_t>(row) * ldc + col;
-        const float uu = acc[0][i][v] + (rowb1 ? tri_load(bias1, row) : cb1);
-        const float vv = acc[1][i][v] + (rowb2 ? tri_load(bias2, row) : cb2);
-        const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-uu));
+        const float vv = acc[1][i][v];
+        const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-acc[0][i][v]));
         const float mk = rowmk ? tri_load(mask, row) : cmk;
         if constexpr (!BWD) {
           tri_store(out1, o, sg * vv * mk);
@@ -774,8 +778,15 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
       load_dc(c0 + 32);  // a whole iteration ahead of its use
     }
 
-    // first product: u, v for 32 rows c x 32 columns m
-    floatx16 au = floatx16{0}, av = floatx16{0};
+    // first product: u, v for 32 rows c x 32 columns m; the accumulators start from the biases of their rows
+    floatx16 au, av;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const float4 b1 = *reinterpret_cast<const float4*>(&smem[buf][BIAS + (8 * a + 4 * h) * 4]);
+      const float4 b2 = *reinterpret_cast<const float4*>(&smem[buf][BIAS + 128 + (8 * a + 4 * h) * 4]);
+      au[4 * a] = b1.x; au[4 * a + 1] = b1.y; au[4 * a + 2] = b1.z; au[4 * a + 3] = b1.w;
+      av[4 * a] = b2.x; av[4 * a + 1] = b2.y; av[4 * a + 2] = b2.z; av[4 * a + 3] = b2.w;
+    }
     {
       const char* w1 = &smem[buf][c * WSTR + h * 32];
 #pragma unroll
@@ -796,17 +807,13 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
     uint32_t pu[BF ? 8 : 1], pv[BF ? 8 : 1];
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const float4 b1 = *reinterpret_cast<const float4*>(&smem[buf][BIAS + (8 * a + 4 * h) * 4]);
-      const float4 b2 = *reinterpret_cast<const float4*>(&smem[buf][BIAS + 128 + (8 * a + 4 * h) * 4]);
-      const float b1v[4] = {b1.x, b1.y, b1.z, b1.w}, b2v[4] = {b2.x, b2.y, b2.z, b2.w};
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const int v = 4 * a + b;
-        const float uu = au[v] + b1v[b];
-        const float vv = av[v] + b2v[b];
+        const float uu = au[v], vv = av[v];
         const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-uu));
-        const float d = dc_value(v) * mk;
-        const float duv = d * vv * sg * (1.0f - sg), dvv = d * sg;
+        const float dvv = dc_value(v) * mk * sg;           // dv = d s
+        const float duv = dvv * fmaf(-vv, sg, vv);          // du = d v s (1 - s)
         du[BF ? b : v] = duv;
         dv[BF ? b : v] = dvv;
         if (dU != nullptr && mcol < M) {
