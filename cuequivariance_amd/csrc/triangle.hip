@@ -118,18 +118,27 @@ __device__ __forceinline__ void stage_flush(const char* tile, int row_stride, in
 // lane 4g+p receives element p of the four 8-byte rows addressed by lanes g, 4+g, 8+g, 12+g), 4-byte types with
 // plain reads along the row.  The row strides (320 / 640 bytes) spread the rows of one read over all banks.
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
-constexpr int kTransStride16 = 320, kTransStride32 = 640;
+// bytes between the k rows of a contraction-major tile of EXT columns: the row plus 64 (2-byte) / 128 (4-byte) bytes
+template <typename TI, int EXT>
+constexpr int trans_stride() { return EXT * static_cast<int>(sizeof(TI)) + (sizeof(TI) == 2 ? 64 : 128); }
+// LDS bytes of one operand tile of EXT rows (either layout)
+template <typename TI, int EXT>
+constexpr int gemm_tile_bytes() {
+  constexpr int a = EXT * kRowBytes, b = (64 / static_cast<int>(sizeof(TI))) * trans_stride<TI, EXT>();
+  return a > b ? a : b;
+}
 
-template <typename TI, bool TR>
+template <typename TI, bool TR, int EXT>
 __device__ __forceinline__ void gemm_stage_offsets(int e, int& row, int& part) {
-  constexpr int VPRN = kTile * sizeof(TI) / 16;  // vectors per k row of a contraction-major tile
+  constexpr int VPRN = EXT * sizeof(TI) / 16;  // vectors per k row of a contraction-major tile
   if constexpr (TR) { row = e / VPRN; part = e % VPRN; }
   else { row = e >> 2; part = e & 3; }
 }
 
 // fragment of subtile rows [base, base + 32) for MFMA step half q: 16 bytes of k per lane
-template <typename TI, bool TR>
+template <typename TI, bool TR, int EXT>
 __device__ __forceinline__ uint4 gemm_fragment(const char* tile, int base, int q, int lane) {
+  constexpr int kTransStride16 = trans_stride<uint16_t, EXT>(), kTransStride32 = trans_stride<float, EXT>();
   const int c = lane & 31, h = lane >> 5;
   if constexpr (!TR) {
     return *reinterpret_cast<const uint4*>(tile + (base + c) * kRowBytes + h * 32 + q * 16);
@@ -148,8 +157,10 @@ __device__ __forceinline__ uint4 gemm_fragment(const char* tile, int base, int q
   }
 }
 
-template <typename TI, typename TO, bool TA, bool TB>
-__global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
+// WM x WN wavefronts of 64 x 64 per block: 2 x 2 (a 128 x 128 tile) by default; 4 x 4 (256 x 256, 16 wavefronts) halves
+// the operand traffic between L2 and the CUs for products whose both extents are large.
+template <typename TI, typename TO, bool TA, bool TB, int WM = 2, int WN = 2>
+__global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
                                                    const TI* __restrict__ B, int64_t ldb, int64_t sB,
                                                    TO* __restrict__ C, int64_t ldc, int64_t sC, int Mfull, int N, int Kfull,
                                                    float alpha, int accumulate, int vec_out, int64_t k_total, int nparts, int64_t pA,
@@ -157,16 +168,18 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
                                                    int64_t gsB, int64_t gsC) {
   constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
   constexpr int BK = 64 / sizeof(TI);   // k extent of one step
-  constexpr int TS = sizeof(TI) == 2 ? kTransStride16 : kTransStride32;
-  static_assert(BK * TS == kTile * kRowBytes, "both tile layouts take the same space");
-  __shared__ __align__(16) char smem[2][2][kTile * kRowBytes];
+  constexpr int TMR = 64 * WM, TNC = 64 * WN, NTH = 64 * WM * WN;  // tile rows, tile columns, threads
+  constexpr int TSA = trans_stride<TI, TMR>(), TSB = trans_stride<TI, TNC>();
+  constexpr int ABYTES = gemm_tile_bytes<TI, TMR>(), BBYTES = gemm_tile_bytes<TI, TNC>();
+  constexpr int NVA = TMR * 4 / NTH, NVB = TNC * 4 / NTH;  // 16-byte vectors per thread and step
+  __shared__ __align__(16) char smem[2][ABYTES + BBYTES];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   int bx, by, bz;
   xcd_tile(bx, by, bz);
-  int m0 = by * kTile, M = Mfull;
-  const int n0 = bx * kTile;
+  int m0 = by * TMR, M = Mfull;
+  const int n0 = bx * TNC;
   // batch item = (chunk, part): strides s* between chunks, p* between parts (nparts == 1: a plain batch)
   const int chunk = bz / nparts, part = bz - chunk * nparts;
   A += static_cast<int64_t>(chunk) * sA + static_cast<int64_t>(part) * pA;
@@ -180,9 +193,9 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
     int t = by, g = 0;
     for (; g < ngroups; ++g) {
       const int64_t lo = goff[g], n = goff[g + 1] - lo;
-      const int nt = static_cast<int>((n + kTile - 1) / kTile);
+      const int nt = static_cast<int>((n + TMR - 1) / TMR);
       if (t < nt) {
-        m0 = static_cast<int>(lo) + t * kTile;
+        m0 = static_cast<int>(lo) + t * TMR;
         break;
       }
       t -= nt;
@@ -199,16 +212,15 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
     C += static_cast<int64_t>(chunk) * gsC;
   }
 
-  // every thread stages two 16-byte vectors of A and two of B per step
-  uint4 stA[2], stB[2];
-  int arow[2], apart[2], brow[2], bpart[2];
+  // every thread stages NVA 16-byte vectors of A and NVB of B per step
+  uint4 stA[NVA], stB[NVB];
+  int arow[NVA], apart[NVA], brow[NVB], bpart[NVB];
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    gemm_stage_offsets<TI, TA>(tid + q * 256, arow[q], apart[q]);
-    gemm_stage_offsets<TI, TB>(tid + q * 256, brow[q], bpart[q]);
-  }
+  for (int q = 0; q < NVA; ++q) gemm_stage_offsets<TI, TA, TMR>(tid + q * NTH, arow[q], apart[q]);
+#pragma unroll
+  for (int q = 0; q < NVB; ++q) gemm_stage_offsets<TI, TB, TNC>(tid + q * NTH, brow[q], bpart[q]);
   auto load_one = [&](const TI* __restrict__ P, int64_t ld, bool tr, int row, int part, int x0, int X, int ks) -> uint4 {
-    if (tr) {  // row = k within the step, part = vector along the tile's 128 columns (extent X is a multiple of EPV)
+    if (tr) {  // row = k within the step, part = vector along the tile's columns (extent X is a multiple of EPV)
       const int k = ks * BK + row, x = x0 + part * EPV;
       const bool ok = k < K && x < X;
       const uint4 v = *reinterpret_cast<const uint4*>(P + static_cast<int64_t>(ok ? k : 0) * ld + (ok ? x : 0));
@@ -221,17 +233,16 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
   };
   auto load_step = [&](int ks) {
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      stA[q] = load_one(A, lda, TA, arow[q], apart[q], m0, M, ks);
-      stB[q] = load_one(B, ldb, TB, brow[q], bpart[q], n0, N, ks);
-    }
+    for (int q = 0; q < NVA; ++q) stA[q] = load_one(A, lda, TA, arow[q], apart[q], m0, M, ks);
+#pragma unroll
+    for (int q = 0; q < NVB; ++q) stB[q] = load_one(B, ldb, TB, brow[q], bpart[q], n0, N, ks);
   };
   auto store_step = [&](int buf) {
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      *reinterpret_cast<uint4*>(&smem[buf][0][arow[q] * (TA ? TS : kRowBytes) + apart[q] * 16]) = stA[q];
-      *reinterpret_cast<uint4*>(&smem[buf][1][brow[q] * (TB ? TS : kRowBytes) + bpart[q] * 16]) = stB[q];
-    }
+    for (int q = 0; q < NVA; ++q) *reinterpret_cast<uint4*>(&smem[buf][arow[q] * (TA ? TSA : kRowBytes) + apart[q] * 16]) = stA[q];
+#pragma unroll
+    for (int q = 0; q < NVB; ++q)
+      *reinterpret_cast<uint4*>(&smem[buf][ABYTES + brow[q] * (TB ? TSB : kRowBytes) + bpart[q] * 16]) = stB[q];
   };
 
   floatx16 acc[2][2];
@@ -252,8 +263,8 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        fa[t][q] = gemm_fragment<TI, TA>(&smem[buf][0][0], wm * 64 + t * 32, q, lane);
-        fb[t][q] = gemm_fragment<TI, TB>(&smem[buf][1][0], wn * 64 + t * 32, q, lane);
+        fa[t][q] = gemm_fragment<TI, TA, TMR>(&smem[buf][0], wm * 64 + t * 32, q, lane);
+        fb[t][q] = gemm_fragment<TI, TB, TNC>(&smem[buf][ABYTES], wn * 64 + t * 32, q, lane);
       }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -279,19 +290,22 @@ __global__ void __launch_bounds__(256) gemm_kernel(const TI* __restrict__ A, int
 
   // 2-byte results, whole wavefront tile inside C, 16-byte aligned rows: through LDS, 32 rows at a time (4-byte
   // results already leave as 128-byte row segments and gain nothing from the detour)
-  if constexpr (sizeof(TO) == 2) __syncthreads();  // every wavefront is done with the operand tiles, which become staging space
-  if (sizeof(TO) == 2 && vec_out && m0 + wm * 64 + 64 <= M && n0 + wn * 64 + 64 <= N) {
-    constexpr int RS = 64 * sizeof(TO) + 16;
-    char* tile = &smem[0][0][0] + wave * (32 * RS);
+  if constexpr (sizeof(TO) == 2) {
+    __syncthreads();  // every wavefront is done with the operand tiles, which become staging space
+    if (vec_out && m0 + wm * 64 + 64 <= M && n0 + wn * 64 + 64 <= N) {
+      constexpr int RS = 64 * sizeof(TO) + 16;
+      static_assert(WM * WN * 32 * RS <= 2 * (ABYTES + BBYTES), "staging tiles must fit the operand buffers");
+      char* tile = &smem[0][0] + wave * (32 * RS);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      stage_put<TO>(tile, RS, c, h, acc[i][0], alpha);
-      stage_put<TO>(tile, RS, 32 + c, h, acc[i][1], alpha);
-      __builtin_amdgcn_wave_barrier();
-      stage_flush<TO, 64>(tile, RS, 32, C + static_cast<int64_t>(m0 + wm * 64 + i * 32) * ldc + n0 + wn * 64, ldc, lane, 64, accumulate != 0);
-      __builtin_amdgcn_wave_barrier();
+      for (int i = 0; i < 2; ++i) {
+        stage_put<TO>(tile, RS, c, h, acc[i][0], alpha);
+        stage_put<TO>(tile, RS, 32 + c, h, acc[i][1], alpha);
+        __builtin_amdgcn_wave_barrier();
+        stage_flush<TO, 64>(tile, RS, 32, C + static_cast<int64_t>(m0 + wm * 64 + i * 32) * ldc + n0 + wn * 64, ldc, lane, 64, accumulate != 0);
+        __builtin_amdgcn_wave_barrier();
+      }
+      return;
     }
-    return;
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -1538,14 +1552,21 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
     KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
     const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
     const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
-#define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0, nullptr, 0, 0, 0, 0)
-#define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_LAUNCH(TI, TI, true, true); else if (trans_a) GEMM_LAUNCH(TI, TI, true, false); else if (trans_b) GEMM_LAUNCH(TI, TI, false, true); else GEMM_LAUNCH(TI, TI, false, false); } while (0)
+    // 256 x 256 tiles when both extents are multiples of 256 and there are enough of them to fill the chip
+    const bool big = !mixed && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) * batch >= 2 * static_cast<int64_t>(device_cus());
+    const dim3 grid_big(static_cast<unsigned>(N / 256), static_cast<unsigned>(M / 256), static_cast<unsigned>(batch));
+#define GEMM_ARGS(TI, TO) static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0, nullptr, 0, 0, 0, 0
+#define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, GEMM_ARGS(TI, TO))
+#define GEMM_SZ(TI, TA, TB) do { if (big) hipLaunchKernelGGL((gemm_kernel<TI, TI, TA, TB, 4, 4>), grid_big, dim3(1024), 0, stream, GEMM_ARGS(TI, TI)); else GEMM_LAUNCH(TI, TI, TA, TB); } while (0)
+#define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_SZ(TI, true, true); else if (trans_a) GEMM_SZ(TI, true, false); else if (trans_b) GEMM_SZ(TI, false, true); else GEMM_SZ(TI, false, false); } while (0)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_TR(float);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t, false, false);
     else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float, false, false);
     else GEMM_TR(uint16_t);
 #undef GEMM_TR
+#undef GEMM_SZ
 #undef GEMM_LAUNCH
+#undef GEMM_ARGS
   } else {
     const int64_t total = M * N;
     CUEQ_REQUIRE((total + 255) / 256 < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gemm: output too large for the unaligned path");

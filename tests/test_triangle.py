@@ -109,10 +109,11 @@ def test_hip_path_matches_oracle(device, dtype, direction, shape):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21)])
+@pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21), (160, 512, 256, 96)])
 def test_gemm_operand_orders(device, dtype, trans_a, trans_b, dims):
     """cueq_gemm against torch.matmul in float64 for the four operand orders: tiled MFMA path (aligned extents,
-    partial tiles included) and the element-wise path (odd extents)."""
+    partial tiles included), the 256 x 256 tiles (both extents multiples of 256, many tiles) and the element-wise
+    path (odd extents)."""
     from cuequivariance_amd.cuet import triangle as tri
 
     batch, M, N, K = dims
