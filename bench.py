@@ -135,6 +135,27 @@ def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
         bound, pu = "mfma", "TFLOP/s"
         peak = 2500.0 if dtype == torch.bfloat16 else 157.3
         desc = "configs[3]: Linear 128x0e+128x1o+128x2e -> same, batch 200000, shared weights, fwd + bwd (dw, dx)"
+    elif wl == "cfg4fc":
+        Z = 50_000
+        dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+        i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e")
+        m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, internal_weights=False)
+        g = torch.Generator(device=dev).manual_seed(0)
+        x1 = torch.randn(Z, i1.dim, device=dev, generator=g).to(dtype).requires_grad_(True)
+        x2 = torch.randn(Z, i2.dim, device=dev, generator=g).to(dtype).requires_grad_(True)
+        w = torch.randn(1, m.weight_numel, device=dev, generator=g).to(dtype).requires_grad_(True)
+        cot = torch.randn(Z, i1.dim, device=dev, generator=g).to(dtype)
+
+        def step():
+            return torch.autograd.grad(m(x1, x2, w), [w, x1, x2], cot)
+
+        unit, units, dt = "rows/s", Z, "bf16" if dtype == torch.bfloat16 else "f32"
+        es = 2 if dtype == torch.bfloat16 else 4
+        # every distinct element once: fwd reads x1, x2 and writes out; bwd reads x1, x2, g and writes dx1, dx2 (weights 20480 negligible)
+        alg = {"fwd": Z * (256 + 9 + 256) * es, "bwd": Z * (256 + 9 + 256 + 256 + 9) * es}
+        bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
+        desc = ("configs[3]: FullyConnectedTensorProduct 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, batch 50000, shared weights, "
+                "fwd + bwd (dw, dx1, dx2)")
     else:
         dtype = torch.float32 if args.dtype == "fp32" else torch.bfloat16
         n, D = 512, 128
@@ -197,9 +218,10 @@ def main() -> int:
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--deterministic", action="store_true",
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
-    ap.add_argument("--workload", choices=["cfg2", "cfg3", "cfg4", "cfg5"], default="cfg2",
+    ap.add_argument("--workload", choices=["cfg2", "cfg3", "cfg4", "cfg4fc", "cfg5"], default="cfg2",
                     help="cfg2 (default) is the headline metric; the others print a secondary line for the same "
-                         "library: cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg5 triangle update")
+                         "library: cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected product, "
+                         "cfg5 triangle update")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "

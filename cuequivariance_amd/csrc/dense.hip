@@ -388,6 +388,59 @@ __global__ void __launch_bounds__(256) seg_rowdot(const IO* __restrict__ A, int6
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Element-wise stages of the fully-connected product on the tiled GEMMs.  With T[:, t] = x1[:, i_seg] . W_p for every
+// distinct (weight block, x1 segment) computed by cueq_gemm, every flattened path is
+//   out[z, c_off + n] += coeff * x2[z, j] * T[z, t_off + n]
+// (a "use" of T); the backward has the same shape with g in place of x1.  fc_combine sums the uses of every output
+// block; fc_rowdot is the gradient of the multiplicity-one operand, dx2[z, j] += coeff * <x1[z, a_off : +K], G[z, g_off : +K]>.
+// ------------------------------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ constexpr int type_code() { return sizeof(T) == 4 ? CUEQ_F32 : CUEQ_BF16; }  // float / uint16_t (bf16 bits)
+struct FcBlock { int32_t out_off, n, first_use, num_uses; };
+struct FcUse { int32_t j, src_off; float coeff; int32_t pad; };
+
+template <typename TS, typename TT, typename TO>
+__global__ void __launch_bounds__(256) fc_combine_kernel(const TS* __restrict__ S, int64_t lds_, const TT* __restrict__ T, int64_t ldt,
+                                                         TO* __restrict__ O, int64_t ldo, const FcBlock* __restrict__ blocks,
+                                                         const FcUse* __restrict__ uses, int64_t Z, int max_n) {
+  const FcBlock b = blocks[blockIdx.y];
+  // a thread owns one column n of the block and walks rows; 256 threads cover 256 / max_n rows per pass
+  const int rows_per_pass = 256 / max_n;
+  const int n = threadIdx.x % max_n, r = threadIdx.x / max_n;
+  if (n >= b.n || r >= rows_per_pass) return;
+  for (int64_t z = static_cast<int64_t>(blockIdx.x) * rows_per_pass + r; z < Z; z += static_cast<int64_t>(gridDim.x) * rows_per_pass) {
+    float acc = 0.f;
+    for (int u = 0; u < b.num_uses; ++u) {
+      const FcUse use = uses[b.first_use + u];
+      acc = fmaf(use.coeff * load_as<float>(S, type_code<TS>(), z * lds_ + use.j), load_as<float>(T, type_code<TT>(), z * ldt + use.src_off + n), acc);
+    }
+    store_as<float>(O, type_code<TO>(), z * ldo + b.out_off + n, acc);
+  }
+}
+
+struct FcDotUse { int32_t j, a_off, g_off, k; float coeff; int32_t pad[3]; };
+
+template <typename TX, typename TG>
+__global__ void __launch_bounds__(256) fc_rowdot_kernel(const TX* __restrict__ X, int64_t ldx, const TG* __restrict__ G, int64_t ldg,
+                                                        TX* __restrict__ D, int64_t ldd, int n2, const FcDotUse* __restrict__ uses,
+                                                        int num_uses, int64_t Z) {
+  // one wavefront per row; lane j keeps the running sum of column j (n2 <= 64)
+  const int lane = threadIdx.x & 63;
+  for (int64_t z = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6); z < Z; z += static_cast<int64_t>(gridDim.x) * 4) {
+    float acc = 0.f;
+    for (int u = 0; u < num_uses; ++u) {
+      const FcDotUse use = uses[u];
+      float p = 0.f;
+      for (int k = lane; k < use.k; k += 64)
+        p = fmaf(load_as<float>(X, type_code<TX>(), z * ldx + use.a_off + k), load_as<float>(G, type_code<TG>(), z * ldg + use.g_off + k), p);
+      p = wave_sum(p);
+      if (lane == use.j) acc = fmaf(use.coeff, p, acc);
+    }
+    if (lane < n2) store_as<float>(D, type_code<TX>(), z * ldd + lane, acc);
+  }
+}
+
 }  // namespace cueq
 
 using namespace cueq;
@@ -533,6 +586,51 @@ extern "C" int cueq_seg_rowdot(int32_t dtype, int32_t K, int32_t N, const void* 
     set_error("seg_rowdot: unsupported dtype %d", dtype);
     return CUEQ_ERR_UNSUPPORTED;
   }
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+// dtype codes: s = x2 and the result (the tensor dtype), t = the GEMM results (float32 or the tensor dtype)
+extern "C" int cueq_fc_combine(int32_t dtype, int32_t t_dtype, int64_t rows, const void* S, int64_t lds_, const void* T, int64_t ldt, void* O,
+                               int64_t ldo, const void* blocks, int32_t num_blocks, const void* uses, int32_t max_n, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE((dtype == CUEQ_F32 || dtype == CUEQ_BF16) && (t_dtype == CUEQ_F32 || t_dtype == dtype), CUEQ_ERR_UNSUPPORTED,
+               "fc_combine: tensors float32 or bfloat16, GEMM results float32 or the tensor dtype");
+  CUEQ_REQUIRE(rows >= 0 && num_blocks >= 0 && max_n >= 1 && max_n <= 256, CUEQ_ERR_INVALID, "fc_combine: bad extents (block width at most 256)");
+  if (rows == 0 || num_blocks == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(S && T && O && blocks && uses, CUEQ_ERR_INVALID, "fc_combine: null operand");
+  const int rpp = 256 / max_n;
+  int64_t gx = (rows + rpp - 1) / rpp;
+  const int64_t cap = static_cast<int64_t>(device_cus()) * 32 / num_blocks + 1;
+  if (gx > cap) gx = cap;
+  const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(num_blocks));
+  KernelTimer timer("fc_combine", stream);
+#define FCC(TS, TT) hipLaunchKernelGGL((fc_combine_kernel<TS, TT, TS>), grid, dim3(256), 0, stream, static_cast<const TS*>(S), lds_, static_cast<const TT*>(T), ldt, static_cast<TS*>(O), ldo, static_cast<const FcBlock*>(blocks), static_cast<const FcUse*>(uses), rows, max_n)
+  if (dtype == CUEQ_F32) FCC(float, float);
+  else if (t_dtype == CUEQ_F32) FCC(uint16_t, float);
+  else FCC(uint16_t, uint16_t);
+#undef FCC
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+extern "C" int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, const void* X, int64_t ldx, const void* G, int64_t ldg, void* D,
+                              int64_t ldd, int32_t n2, const void* uses, int32_t num_uses, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE((dtype == CUEQ_F32 || dtype == CUEQ_BF16) && (g_dtype == CUEQ_F32 || g_dtype == dtype), CUEQ_ERR_UNSUPPORTED,
+               "fc_rowdot: tensors float32 or bfloat16, GEMM results float32 or the tensor dtype");
+  CUEQ_REQUIRE(rows >= 0 && n2 >= 1 && n2 <= 64 && num_uses >= 0, CUEQ_ERR_UNSUPPORTED, "fc_rowdot: the multiplicity-one operand has at most 64 elements");
+  if (rows == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(X && G && D && (uses || num_uses == 0), CUEQ_ERR_INVALID, "fc_rowdot: null operand");
+  int64_t gx = (rows + 3) / 4;
+  const int64_t cap = static_cast<int64_t>(device_cus()) * 32;
+  if (gx > cap) gx = cap;
+  KernelTimer timer("fc_rowdot", stream);
+#define FCD(TX, TG) hipLaunchKernelGGL((fc_rowdot_kernel<TX, TG>), dim3(static_cast<unsigned>(gx)), dim3(256), 0, stream, static_cast<const TX*>(X), ldx, static_cast<const TG*>(G), ldg, static_cast<TX*>(D), ldd, n2, static_cast<const FcDotUse*>(uses), num_uses, rows)
+  if (dtype == CUEQ_F32) FCD(float, float);
+  else if (g_dtype == CUEQ_F32) FCD(uint16_t, float);
+  else FCD(uint16_t, uint16_t);
+#undef FCD
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }

@@ -182,9 +182,15 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
   const int n0 = bx * TNC;
   // batch item = (chunk, part): strides s* between chunks, p* between parts (nparts == 1: a plain batch)
   const int chunk = bz / nparts, part = bz - chunk * nparts;
-  A += static_cast<int64_t>(chunk) * sA + static_cast<int64_t>(part) * pA;
-  B += static_cast<int64_t>(chunk) * sB + static_cast<int64_t>(part) * pB;
-  C += static_cast<int64_t>(chunk) * sC + static_cast<int64_t>(part) * pC;
+  if (gmode == 3) {  // the parts are unrelated blocks: element offsets of A, B, C per part from a table
+    A += static_cast<int64_t>(chunk) * sA + goff[3 * part];
+    B += static_cast<int64_t>(chunk) * sB + goff[3 * part + 1];
+    C += static_cast<int64_t>(chunk) * sC + goff[3 * part + 2];
+  } else {
+    A += static_cast<int64_t>(chunk) * sA + static_cast<int64_t>(part) * pA;
+    B += static_cast<int64_t>(chunk) * sB + static_cast<int64_t>(part) * pB;
+    C += static_cast<int64_t>(chunk) * sC + static_cast<int64_t>(part) * pC;
+  }
   // k_total > 0: the chunks are consecutive k ranges of one long contraction; the last ones may be short or empty
   int K = k_total > 0 ? static_cast<int>(max<int64_t>(0, min<int64_t>(Kfull, k_total - static_cast<int64_t>(chunk) * Kfull))) : Kfull;
   if (gmode == 1) {
@@ -1546,7 +1552,8 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
   const float al = static_cast<float>(alpha);
   const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
   const bool mixed = in_dtype != out_dtype;
-  if (aligned && !(mixed && (trans_a || trans_b))) {
+  const bool mixed_ok = !mixed || (!trans_a && !trans_b) || (in_dtype == CUEQ_BF16 && out_dtype == CUEQ_F32 && !trans_a && trans_b);
+  if (aligned && mixed_ok) {
     const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(batch));
     CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm: too many row tiles (M <= 8388480)");
     KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
@@ -1561,7 +1568,7 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
 #define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_SZ(TI, true, true); else if (trans_a) GEMM_SZ(TI, true, false); else if (trans_b) GEMM_SZ(TI, false, true); else GEMM_SZ(TI, false, false); } while (0)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_TR(float);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t, false, false);
-    else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float, false, false);
+    else if (out_dtype == CUEQ_F32) { if (trans_b) GEMM_LAUNCH(uint16_t, float, false, true); else GEMM_LAUNCH(uint16_t, float, false, false); }
     else GEMM_TR(uint16_t);
 #undef GEMM_TR
 #undef GEMM_SZ
@@ -1588,6 +1595,45 @@ extern "C" int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int6
                             int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc, int64_t stride_c,
                             int64_t batch, double alpha, int32_t accumulate, void* stream_) {
   return cueq_gemm(in_dtype, out_dtype, 0, 0, M, N, K, A, lda, stride_a, B, ldb, stride_b, C, ldc, stride_c, batch, alpha, accumulate, stream_);
+}
+
+extern "C" int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
+                               const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc, const int64_t* table,
+                               int64_t nparts, int64_t k_chunks, int64_t chunk_stride_c, double alpha, int32_t accumulate, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(is_io(in_dtype) && (out_dtype == in_dtype || out_dtype == CUEQ_F32), CUEQ_ERR_UNSUPPORTED,
+               "gemm_table: float32 or bfloat16 operands, result of the same type or float32");
+  CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && nparts >= 0 && k_chunks >= 1, CUEQ_ERR_INVALID, "gemm_table: bad extents");
+  if (M == 0 || N == 0 || nparts == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(A && B && C && table, CUEQ_ERR_INVALID, "gemm_table: null operand");
+  CUEQ_REQUIRE(k_chunks == 1 || (trans_a && trans_b), CUEQ_ERR_UNSUPPORTED, "gemm_table: the contraction is cut only for contraction-major operands");
+  CUEQ_REQUIRE(!(trans_a && !trans_b), CUEQ_ERR_UNSUPPORTED, "gemm_table: A contraction-major with B contraction-contiguous is not built");
+  CUEQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && nparts * k_chunks < 65536, CUEQ_ERR_TOO_LARGE, "gemm_table: extent too large");
+  const int epv = in_dtype == CUEQ_F32 ? 4 : 8;
+  // the table's offsets must keep the 16-byte alignment too: the caller builds it from segment offsets (checked there)
+  const bool aligned = K > 0 && (trans_a ? M : K) % epv == 0 && (trans_b ? N : K) % epv == 0 && lda % epv == 0 && ldb % epv == 0 &&
+                       reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0;
+  CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "gemm_table: extents along vectors, strides and pointers must be multiples of 16 bytes");
+  const int64_t kc = k_chunks == 1 ? K : (((K + k_chunks - 1) / k_chunks + 31) / 32) * 32;  // contraction per chunk
+  const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(nparts * k_chunks));
+  CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm_table: too many row tiles");
+  const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
+  const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0) ? 1 : 0;
+  KernelTimer timer("gemm_table", stream);
+  // results at most 64 columns wide take 256 x 64 tiles (4 x 1 wavefronts) instead of wasting half a 128 x 128 tile
+  const bool skinny = N <= 64;
+  const dim3 grid_s(1, static_cast<unsigned>((M + 255) / 256), static_cast<unsigned>(nparts * k_chunks));
+#define GT_ARGS(TI, TO) static_cast<const TI*>(A), lda, k_chunks == 1 ? 0 : kc * lda, static_cast<const TI*>(B), ldb, k_chunks == 1 ? 0 : kc * ldb, static_cast<TO*>(C), ldc, chunk_stride_c, static_cast<int>(M), static_cast<int>(N), static_cast<int>(kc), static_cast<float>(alpha), accumulate, vec_out, k_chunks == 1 ? 0 : K, static_cast<int>(nparts), 0, 0, 0, table, 0, 3, 0, 0
+#define GT(TI, TO, TA, TB) do { if (skinny) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB, 4, 1>), grid_s, dim3(256), 0, stream, GT_ARGS(TI, TO)); else hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, GT_ARGS(TI, TO)); } while (0)
+#define GT_T(TI, TO) do { if (trans_a && trans_b) GT(TI, TO, true, true); else if (trans_b) GT(TI, TO, false, true); else GT(TI, TO, false, false); } while (0)
+  if (in_dtype == CUEQ_F32) GT_T(float, float);
+  else if (out_dtype == CUEQ_F32) GT_T(uint16_t, float);
+  else GT_T(uint16_t, uint16_t);
+#undef GT_T
+#undef GT
+#undef GT_ARGS
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
 }
 
 extern "C" int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mode, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,

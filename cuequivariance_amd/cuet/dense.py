@@ -8,10 +8,10 @@ for the polynomial forms the high-level layers produce:
   operand has multiplicity one, e.g. spherical harmonics; ``descriptors/irreps_tp.py:22-47``)
 
 with weights shared over the batch.  After the Clebsch-Gordan modes are flattened every path is a small
-GEMM ``out[:, k_seg] += c * x2[:, j] * x1[:, i_seg] @ W_p``; they are grouped into launches of
-``cueq_seg_gemm`` (MFMA).  The backward pass calls ``cueq_seg_gemm`` with transposed blocks (input
-gradient), ``cueq_seg_outer`` (weight gradient, batch reduction without atomics) and ``cueq_seg_rowdot``
-(gradient of the multiplicity-one operand).  First-order gradients only.
+GEMM ``out[:, k_seg] += c * x2[:, j] * x1[:, i_seg] @ W_p``.  In float32 / bfloat16 the weight contractions run as a
+few batched launches of the 128 x 128 tiled kernel (``cueq_gemm``, ``cueq_gemm_tn``) and the scaling by ``x2`` and the
+sums over paths as one element-wise kernel per result (``cueq_fc_combine``, ``cueq_fc_rowdot``); float64 and shapes
+those kernels refuse go through ``cueq_seg_gemm`` / ``cueq_seg_outer`` / ``cueq_seg_rowdot``.  First-order gradients only.
 """
 
 from __future__ import annotations
@@ -279,6 +279,201 @@ class _DenseFunction(torch.autograd.Function):
         return None, gw, gx1, gx2
 
 
+def _progressions(items, key_a, key_c):
+    """Split ``items`` (sorted) into runs whose ``key_a`` and ``key_c`` advance by constant positive strides:
+    ``[(first item, count, stride a, stride c)]`` - one batched GEMM launch each."""
+    runs, i = [], 0
+    while i < len(items):
+        j = i + 1
+        da = dc = 0
+        if j < len(items):
+            da, dc = key_a(items[j]) - key_a(items[i]), key_c(items[j]) - key_c(items[i])
+            if da > 0 and dc > 0:
+                while j + 1 < len(items) and key_a(items[j + 1]) - key_a(items[j]) == da and key_c(items[j + 1]) - key_c(items[j]) == dc:
+                    j += 1
+                j += 1
+            else:
+                da = dc = 0
+        runs.append((items[i], j - i, da, dc))
+        i = j
+    return runs
+
+
+class _FcPlan:
+    """Host tables of the fully-connected product on the tiled GEMMs (see ``cueq_fc_combine`` in the header):
+    ``T[:, t] = x1[:, i_seg] @ W_p`` per distinct (weight block, x1 segment), ``G[:, g] = g[:, k_seg] @ W_p^T`` per distinct
+    (weight block, output segment); every flattened path is then one scaled use of a ``T`` (forward, ``H`` for the weight
+    gradient) or of a ``G`` (``dx1``, ``dx2``)."""
+
+    def __init__(self, paths, n2: int):
+        import numpy as np
+
+        self.n2 = n2
+        t_of, g_of = {}, {}
+        t_cols = g_cols = 0
+        for p in sorted(paths, key=lambda p: (p.w_off, p.a_off)):
+            if (p.w_off, p.a_off) not in t_of:
+                t_of[(p.w_off, p.a_off)] = (t_cols, p.K, p.N)
+                t_cols += p.N
+        for p in sorted(paths, key=lambda p: (p.w_off, p.c_off)):
+            if (p.w_off, p.c_off) not in g_of:
+                g_of[(p.w_off, p.c_off)] = (g_cols, p.K, p.N)
+                g_cols += p.K
+        self.t_cols, self.g_cols = t_cols, g_cols
+        # one table-driven GEMM launch per block shape: rows (operand offset, weight offset, result offset)
+        self.t_shapes, self.g_shapes = {}, {}
+        for (w_off, a_off), (t, K, N) in sorted(t_of.items()):
+            self.t_shapes.setdefault((K, N), []).append((a_off, w_off, t))
+        for (w_off, c_off), (gq, K, N) in sorted(g_of.items()):
+            self.g_shapes.setdefault((K, N), []).append((c_off, w_off, gq))
+        def tables(block_key, block_n, src):
+            blocks = {}
+            for p in paths:
+                blocks.setdefault((block_key(p), block_n(p)), []).append((p.j, src(p), p.coeff))
+            barr = np.zeros(len(blocks), dtype=[("off", "<i4"), ("n", "<i4"), ("first", "<i4"), ("num", "<i4")])
+            uarr = np.zeros(sum(len(u) for u in blocks.values()), dtype=[("j", "<i4"), ("src", "<i4"), ("coeff", "<f4"), ("pad", "<i4")])
+            first = 0
+            for b, ((off, n), us) in enumerate(sorted(blocks.items())):
+                barr[b] = (off, n, first, len(us))
+                for u in us:
+                    uarr[first] = (u[0], u[1], u[2], 0)
+                    first += 1
+            return barr, uarr, max(n for _, n in blocks)
+
+        self.fwd = tables(lambda p: p.c_off, lambda p: p.N, lambda p: t_of[(p.w_off, p.a_off)][0])
+        self.dx1 = tables(lambda p: p.a_off, lambda p: p.K, lambda p: g_of[(p.w_off, p.c_off)][0])
+        self.h = tables(lambda p: t_of[(p.w_off, p.a_off)][0], lambda p: p.N, lambda p: p.c_off)
+        darr = np.zeros(len(paths), dtype=[("j", "<i4"), ("a", "<i4"), ("g", "<i4"), ("k", "<i4"), ("coeff", "<f4"), ("pad", "<i4", 3)])
+        for u, p in enumerate(paths):
+            darr[u] = (p.j, p.a_off, g_of[(p.w_off, p.c_off)][0], p.K, p.coeff, (0, 0, 0))
+        self.dx2 = darr
+        self.ok = max(self.fwd[2], self.dx1[2], self.h[2]) <= 256 and n2 <= 64
+        self._device: Dict[int, dict] = {}
+
+    def device(self, dev: torch.device) -> dict:
+        idx = dev.index if dev.index is not None else torch.cuda.current_device()
+        d = self._device.get(idx)
+        if d is None:
+            def up(a):
+                return torch.from_numpy(a.view("u1").reshape(-1).copy()).to(torch.device("cuda", idx))
+
+            device = torch.device("cuda", idx)
+            t_tabs, g_tabs, w_tabs = {}, {}, {}
+            for (K, N), rows in self.t_shapes.items():
+                t_tabs[(K, N)] = torch.tensor(rows, dtype=torch.int64, device=device)
+                # weight gradient: part p contracts x1[:, a_off_p : +K] with H[:, t_p : +N] into block p of the partials
+                w_tabs[(K, N)] = (
+                    torch.tensor([(a, t, p * K * N) for p, (a, _, t) in enumerate(rows)], dtype=torch.int64, device=device),
+                    (torch.tensor([w for _, w, _ in rows], dtype=torch.int64, device=device)[:, None]
+                     + torch.arange(K * N, dtype=torch.int64, device=device)[None, :]).reshape(-1),
+                )
+            for (K, N), rows in self.g_shapes.items():
+                g_tabs[(K, N)] = torch.tensor(rows, dtype=torch.int64, device=device)
+            d = self._device[idx] = {
+                "t": t_tabs, "g": g_tabs, "w": w_tabs,
+                "fwd": (up(self.fwd[0]), up(self.fwd[1]), len(self.fwd[0]), self.fwd[2]),
+                "dx1": (up(self.dx1[0]), up(self.dx1[1]), len(self.dx1[0]), self.dx1[2]),
+                "h": (up(self.h[0]), up(self.h[1]), len(self.h[0]), self.h[2]),
+                "dx2": (up(self.dx2), len(self.dx2)),
+            }
+        return d
+
+
+def _fc_combine(lib, code, t_code, Z, S, T, O, table, stream):
+    blocks, uses, nblocks, max_n = table
+    _lib.check(lib.cueq_fc_combine(code, t_code, Z, S.data_ptr(), S.stride(0), T.data_ptr(), T.stride(0), O.data_ptr(), O.stride(0),
+                                   blocks.data_ptr(), nblocks, uses.data_ptr(), max_n, stream), "cueq_fc_combine")
+
+
+class _FcFunction(torch.autograd.Function):
+    """Fully-connected product (shared weights, second operand of multiplicity one) on the tiled GEMMs: a few batched
+    ``cueq_gemm`` launches for the weight contractions and one ``cueq_fc_combine`` / ``cueq_fc_rowdot`` per result."""
+
+    @staticmethod
+    def forward(ctx, mod: "SegmentedPolynomialDense", w, x1, x2):
+        dtype, dev = x1.dtype, x1.device
+        Z = x1.shape[0]
+        plan, lib = mod.fc_plan, _lib.load()
+        out = (torch.empty if mod.fwd_covers_output else torch.zeros)((Z, mod.out_size), dtype=dtype, device=dev)
+        if Z > 0:
+            wd, x1d, x2d = w.detach().to(dtype).contiguous(), x1.detach().contiguous(), x2.detach().contiguous()
+            with torch.cuda.device(dev):
+                stream = torch.cuda.current_stream(dev).cuda_stream
+                code, es = _DTYPE_CODE[dtype], x1d.element_size()
+                T = torch.empty(Z, plan.t_cols, dtype=torch.float32, device=dev)
+                tables = plan.device(dev)
+                for (K, N), tab in tables["t"].items():
+                    # T[:, t : + N] = x1[:, a_off : + K] @ W_p for every row (a_off, w_off, t) of the table; W_p is K x N:
+                    # contraction-major as it lies
+                    _lib.check(lib.cueq_gemm_table(code, _lib.F32, 0, 1, Z, N, K, x1d.data_ptr(), x1d.stride(0), wd.data_ptr(), N,
+                                                   T.data_ptr(), plan.t_cols, tab.data_ptr(), tab.shape[0], 1, 0, 1.0, 0, stream),
+                               "cueq_gemm_table")
+                _fc_combine(lib, code, _lib.F32, Z, x2d, T, out, tables["fwd"], stream)
+        ctx.mod = mod
+        ctx.save_for_backward(w, x1, x2)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        mod = ctx.mod
+        w, x1, x2 = ctx.saved_tensors
+        dtype, dev = x1.dtype, x1.device
+        Z = x1.shape[0]
+        plan, lib = mod.fc_plan, _lib.load()
+        g = g.contiguous()
+        wd, x1d, x2d = w.detach().to(dtype).contiguous(), x1.detach().contiguous(), x2.detach().contiguous()
+        gw = gx1 = gx2 = None
+        need_w, need_x1, need_x2 = ctx.needs_input_grad[1], ctx.needs_input_grad[2], ctx.needs_input_grad[3]
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            code, es = _DTYPE_CODE[dtype], x1d.element_size()
+            tables = plan.device(dev)
+            if need_x1:
+                gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
+            if need_x2:
+                gx2 = torch.zeros_like(x2d)
+            if (need_x1 or need_x2) and Z > 0:
+                G = torch.empty(Z, plan.g_cols, dtype=torch.float32, device=dev)
+                for (K, N), tab in tables["g"].items():
+                    # G[:, gq : + K] = g[:, c_off : + N] @ W_p^T for every row (c_off, w_off, gq); W_p (K x N) is
+                    # "rows x contraction" for this product
+                    _lib.check(lib.cueq_gemm_table(code, _lib.F32, 0, 0, Z, K, N, g.data_ptr(), g.stride(0), wd.data_ptr(), N,
+                                                   G.data_ptr(), plan.g_cols, tab.data_ptr(), tab.shape[0], 1, 0, 1.0, 0, stream),
+                               "cueq_gemm_table")
+                if need_x1:
+                    _fc_combine(lib, code, _lib.F32, Z, x2d, G, gx1, tables["dx1"], stream)
+                if need_x2:
+                    uses, nuses = tables["dx2"]
+                    _lib.check(lib.cueq_fc_rowdot(code, _lib.F32, Z, x1d.data_ptr(), x1d.stride(0), G.data_ptr(), plan.g_cols,
+                                                  gx2.data_ptr(), gx2.stride(0), plan.n2, uses.data_ptr(), nuses, stream), "cueq_fc_rowdot")
+            if need_w:
+                gwd = torch.zeros_like(wd)
+                if Z > 0:
+                    # H[:, t] = sum over the uses of T-block t of coeff * x2[:, j] * g[:, k_seg]; then dW_p = sum_i x1[:, i_seg]^T H[:, t_i]
+                    H = torch.empty(Z, plan.t_cols, dtype=dtype, device=dev)
+                    _fc_combine(lib, code, code, Z, x2d, g, H, tables["h"], stream)
+                    gw32 = torch.zeros(wd.numel(), dtype=torch.float32, device=dev)
+                    for (K, N), (tab, dst) in tables["w"].items():
+                        nparts = tab.shape[0]
+                        tiles = ((K + 127) // 128) * ((N + 127) // 128)
+                        chunks = max(1, min(-(-512 // (nparts * tiles)), Z // 256))
+                        part = torch.empty(chunks, nparts * K * N, dtype=torch.float32, device=dev)
+                        _lib.check(lib.cueq_gemm_table(code, _lib.F32, 1, 1, K, N, Z, x1d.data_ptr(), x1d.stride(0), H.data_ptr(),
+                                                       plan.t_cols, part.data_ptr(), N, tab.data_ptr(), nparts, chunks, nparts * K * N,
+                                                       1.0, 0, stream), "cueq_gemm_table")
+                        total = torch.empty(nparts * K * N, dtype=torch.float32, device=dev)
+                        ws_bytes = lib.cueq_sum_rows_workspace(chunks, nparts * K * N)
+                        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+                        _lib.check(lib.cueq_sum_rows(_lib.F32, chunks, nparts * K * N, part.data_ptr(), total.data_ptr(), ws.data_ptr(),
+                                                     ws_bytes, stream), "cueq_sum_rows")
+                        gw32.index_add_(0, dst, total)  # blocks of one path (its x1 components) land on the same weights
+                    gwd = gw32.to(dtype).view(wd.shape)
+                gw = gwd.to(w.dtype).reshape(w.shape)
+            if gx2 is not None and x2.shape[0] == 1 and Z != 1:
+                gx2 = gx2.sum(0, keepdim=True)
+        return None, gw, gx1, gx2
+
+
 class _IndexedDenseFunction(torch.autograd.Function):
     """Linear with one weight row per class and the batch rows sorted by class (``offsets[c] .. offsets[c+1]`` are the rows
     of class ``c``): grouped GEMMs on the tiled MFMA kernel (``cueq_gemm_grouped``), no host synchronisation."""
@@ -390,6 +585,7 @@ class SegmentedPolynomialDense(nn.Module):
         self.fwd_groups = _batched_groups(self.paths, lambda p: p.a_off, lambda p: p.c_off)
         self.dx1_groups = _batched_groups(self.paths, lambda p: p.c_off, lambda p: p.a_off)
         self.weight_blocks = sorted({(p.w_off, p.K, p.N) for p in self.paths})
+        self.fc_plan = _FcPlan(self.paths, self.input_sizes[2]) if self.has_x2 else None
 
     def tiled(self, dtype, A: torch.Tensor, Cout: torch.Tensor) -> bool:
         """The tiled kernel serves fp32 / bf16 contractions without a per-row scale."""
@@ -467,4 +663,6 @@ class SegmentedPolynomialDense(nn.Module):
                 x2 = x2.expand(x1.shape[0], x2.shape[1])
             elif x1.shape[0] == 1 and x2.shape[0] != 1:
                 x1 = x1.expand(x2.shape[0], x1.shape[1])
+        if x2 is not None and self.fc_plan.ok and x1.dtype in (torch.float32, torch.bfloat16):
+            return [_FcFunction.apply(self, w, x1, x2)]
         return [_DenseFunction.apply(self, w, x1, x2)]

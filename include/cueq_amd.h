@@ -171,6 +171,18 @@ int cueq_seg_outer(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t l
 int cueq_seg_rowdot(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t lda, const void* B, const void* G,
                     int64_t ldg, void* dS, int64_t lds, int64_t rows, const cueq_gemm_problem* problem, void* stream);
 
+/* Element-wise stages of the fully-connected product (uvw,iu,jv,kw with v = 1; FusedTensorProductOp4,
+ * primitives/segmented_polynomial_fused_tp.py:40-48) on top of the tiled GEMMs: with T[:, t] = x1[:, i_seg] . W_p from cueq_gemm,
+ *   cueq_fc_combine: O[z, out_off + n] = sum over the uses u of block b of coeff_u * S[z, j_u] * T[z, src_off_u + n],  n < n_b
+ *   cueq_fc_rowdot:  D[z, j] = sum over the uses u with j_u == j of coeff_u * <X[z, a_off_u : +k_u], G[z, g_off_u : +k_u]>
+ * blocks: device array of {int32 out_off, n, first_use, num_uses}; uses: device array of {int32 j, src_off; float coeff; int32 pad}
+ * (combine) or {int32 j, a_off, g_off, k; float coeff; int32 pad[3]} (rowdot).  dtype: S, O, X, D (float32 / bfloat16);
+ * t_dtype / g_dtype: T / G (float32 or the same).  Block widths at most max_n <= 256; D has n2 <= 64 columns. */
+int cueq_fc_combine(int32_t dtype, int32_t t_dtype, int64_t rows, const void* S, int64_t lds, const void* T, int64_t ldt, void* O,
+                    int64_t ldo, const void* blocks, int32_t num_blocks, const void* uses, int32_t max_n, void* stream);
+int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, const void* X, int64_t ldx, const void* G, int64_t ldg, void* D,
+                   int64_t ldd, int32_t n2, const void* uses, int32_t num_uses, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* triangle multiplicative update: the stages behind                           */
 /*   cuequivariance_torch/cuequivariance_torch/primitives/triangle.py:138-262   */
@@ -195,6 +207,16 @@ int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int6
 int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
               const void* A, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc,
               int64_t stride_c, int64_t batch, double alpha, int32_t accumulate, void* stream);
+
+/* The tiled product over unrelated blocks in one launch: part p computes C + table[3p+2] (+)= alpha * op(A + table[3p]) .
+ * op(B + table[3p+1])^T with the shared extents M, N, K and row strides (table: device, int64, element offsets).
+ * k_chunks > 1 (trans_a and trans_b only) cuts the contraction into k_chunks row ranges; chunk c writes its partial
+ * product to C + c * chunk_stride_c + table[3p+2] and the caller adds the chunks in order.  Serves the weight contractions
+ * of the fully-connected product (FusedTensorProductOp4, primitives/segmented_polynomial_fused_tp.py:40-48), whose blocks
+ * do not advance by constant strides. */
+int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
+                    const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc, const int64_t* table,
+                    int64_t nparts, int64_t k_chunks, int64_t chunk_stride_c, double alpha, int32_t accumulate, void* stream);
 
 /* Grouped products on the tiled kernel, for a Linear whose weights are chosen per row by a sorted class index
  * (the closed indexed_linear op behind cuequivariance_torch/primitives/segmented_polynomial_indexed_linear.py:116-156):
