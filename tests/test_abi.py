@@ -51,3 +51,36 @@ def test_table_hash_agrees_between_python_and_c(math_code):
         assert h.value == tables.content_hash(math_code)
         # kernels for this descriptor (forward and the all-gradients backward) are generated at build time
         assert has_spec == (0 if tables.num_outputs == 1 and tables.num_inputs == 4 else 1)
+
+
+def test_dense_entries_refuse_bad_arguments_before_any_launch():
+    """Argument checks of the tiled-GEMM family run on the host: no GPU is touched when a request is refused."""
+    lib = _lib.load()
+    F32, F64, BF16 = _lib.F32, _lib.F64, _lib.BF16
+    p = 4096  # a fake, 16-byte aligned address: never dereferenced by a refused call
+    # dtype outside float32 / bfloat16
+    assert lib.cueq_gemm(F64, F64, 0, 0, 8, 8, 8, p, 8, 0, p, 8, 0, p, 8, 0, 1, 1.0, 0, None) == -2
+    assert b"float32 or bfloat16" in lib.cueq_last_error()
+    # negative extent, null operand
+    assert lib.cueq_gemm(F32, F32, 0, 0, -1, 8, 8, p, 8, 0, p, 8, 0, p, 8, 0, 1, 1.0, 0, None) == -1
+    assert lib.cueq_gemm(F32, F32, 0, 0, 8, 8, 8, None, 8, 0, p, 8, 0, p, 8, 0, 1, 1.0, 0, None) == -1
+    # empty problems succeed without a launch
+    assert lib.cueq_gemm(F32, F32, 0, 0, 0, 8, 8, None, 8, 0, None, 8, 0, None, 8, 0, 1, 1.0, 0, None) == 0
+    # grouped: unknown mode; rows-grouped keeps the dtype
+    assert lib.cueq_gemm_grouped(F32, F32, 7, 8, 8, 8, p, 8, 0, p, 8, 0, p, 8, 0, 1, p, 2, 0, 64, 1.0, 0, None) == -1
+    assert lib.cueq_gemm_grouped(BF16, F32, 1, 8, 8, 8, p, 8, 0, p, 8, 0, p, 8, 0, 1, p, 2, 0, 64, 1.0, 0, None) == -2
+    # table-driven: the contraction is cut only for contraction-major operands
+    assert lib.cueq_gemm_table(F32, F32, 0, 0, 8, 8, 8, p, 8, p, 8, p, 8, p, 1, 4, 64, 1.0, 0, None) == -2
+    # fused gate backward: K beyond 128, C not a multiple of 32
+    args = (p, p, 160, p, None, 160, None, None, None, p, 64, 1, p, None, 160, 0, None, None, None)
+    assert lib.cueq_gate_bwd_input(BF16, 64, 128, 160, *args) == -2 and b"K must be" in lib.cueq_last_error()
+    args = (p, p, 128, p, None, 128, None, None, None, p, 64, 1, p, None, 128, 0, None, None, None)
+    assert lib.cueq_gate_bwd_input(BF16, 48, 128, 128, *args) == -2
+    # LayerNorm with layout change: D beyond 256
+    assert lib.cueq_layer_norm_t_fwd(F32, 64, 512, p, None, None, 1e-5, p, p, p, None) == -2
+    # segmented transpose: element size, aliasing
+    assert lib.cueq_segmented_transpose(3, 4, 4, p, p, 2 * p, None) == -2
+    assert lib.cueq_segmented_transpose(4, 4, 4, p, p, p, None) == -1 and b"in place" in lib.cueq_last_error()
+    # fully-connected stages: block width, operand width
+    assert lib.cueq_fc_combine(F32, F32, 4, p, 1, p, 1, p, 1, p, 1, p, 512, None) == -1
+    assert lib.cueq_fc_rowdot(F32, F32, 4, p, 1, p, 1, p, 1, 100, p, 1, None) == -2
