@@ -295,8 +295,11 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
 # ---------------------------------------------------------------------------------------------
 # backward
 # ---------------------------------------------------------------------------------------------
-def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: int) -> str:
-    """HIP source of the fused backward kernel (dw, dx1, dx2 in one pass)."""
+def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: int, prefetch: bool = False) -> str:
+    """HIP source of the fused backward kernel (dw, dx1, dx2 in one pass).  With ``prefetch`` the operands of the next
+    batch row (x1 row, weight row, x2 row, indices) are fetched into a second register set while the current row is
+    processed.  Measured on the 128-channel l <= 3 case: 219 instead of 178 registers, no spills, same time
+    (0.759 vs 0.757 ms): the loop does not wait on these loads, so the option is off."""
     fp = T
     L = []
     A = L.append
@@ -316,89 +319,122 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
     for k in range(st.nseg_out):
         A(f"  {fp} gr{k} = 0;")
     A("  int64_t grow_cur = -1;")
-    A("  for (int64_t z = z0; z < z1; ++z) {")
-    A("    int64_t grow = z;")
-    A("    if (G_IDX) grow = g_idx64 ? static_cast<const int64_t*>(g_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(g_index)[z]);")
-    A("    if (grow != grow_cur) {")
-    A("      grow_cur = grow;")
-    A(f"      const {fp}* __restrict__ gp = g + grow * {st.nseg_out * st.extent}ll;")
-    for k in range(st.nseg_out):
-        A(f"      gr{k} = gp[{k * st.extent} + uu];")
-    A("    }")
-    A("    int64_t srow = z;")
-    A("    if (X1_IDX) srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
-    A(f"    const {fp}* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
-    A(f"    const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
-    A(f"    const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
-    A(f"    {fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
     i_used = sorted({i for blk in st.blocks for i in blk.i_list})
     j_used = sorted({j for blk in st.blocks for j in blk.j_list})
-    for i in i_used:
-        A(f"    const {fp} xv{i} = x1p[{i * st.extent} + uu];")
-    for blk in st.blocks:
-        A(f"    const {fp} wv{blk.b} = wp[{blk.b * st.extent} + uu];")
-    for j in j_used:
-        A(f"    const {fp} yv{j} = x2p[{j}];")
-    for i in i_used:
-        A(f"    {fp} dxa{i} = 0;")
-    for j in j_used:
-        A(f"    {fp} pj{j} = 0;")
-    for blk in st.blocks:
-        A(f"    {{  // block w[{blk.b}]")
-        A(f"      const {fp} wb = wv{blk.b};")
-        gij = defaultdict(list)
-        for i, j, k, c in blk.entries:
-            gij[(i, j)].append((k, c))
-        A(f"      {fp} dwb = 0;")
-        for j in blk.j_list:
-            A(f"      {fp} F{j} = 0;")
-        # per x1 component: G = sum_k c g_k is a temporary feeding both D (with x2) and F (with x1)
-        for i in blk.i_list:
-            A("      {")
-            A(f"        {fp} D = 0;")
+
+    def load(S: str, zz: str, ind: str):
+        A(f"{ind}{{")
+        A(f"{ind}  const int64_t z = {zz};")
+        A(f"{ind}  {S}_grow = z;")
+        A(f"{ind}  if (G_IDX) {S}_grow = g_idx64 ? static_cast<const int64_t*>(g_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(g_index)[z]);")
+        A(f"{ind}  {S}_srow = z;")
+        A(f"{ind}  if (X1_IDX) {S}_srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
+        A(f"{ind}  const {fp}* __restrict__ x1p = x1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
+        A(f"{ind}  const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
+        A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
+        for i in i_used:
+            A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
+        for blk in st.blocks:
+            A(f"{ind}  {S}_wv{blk.b} = wp[{blk.b * st.extent} + uu];")
+        for j in j_used:
+            A(f"{ind}  {S}_yv{j} = x2p[{j}];")
+        A(f"{ind}}}")
+
+    def body(S: str, zz: str, ind: str):
+        A(f"{ind}const int64_t z = {zz};")
+        A(f"{ind}if ({S}_grow != grow_cur) {{")
+        A(f"{ind}  grow_cur = {S}_grow;")
+        A(f"{ind}  const {fp}* __restrict__ gp = g + grow_cur * {st.nseg_out * st.extent}ll;")
+        for k in range(st.nseg_out):
+            A(f"{ind}  gr{k} = gp[{k * st.extent} + uu];")
+        A(f"{ind}}}")
+        A(f"{ind}{fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
+        for i in i_used:
+            A(f"{ind}{fp} dxa{i} = 0;")
+        for j in j_used:
+            A(f"{ind}{fp} pj{j} = 0;")
+        for blk in st.blocks:
+            A(f"{ind}{{  // block w[{blk.b}]")
+            A(f"{ind}  const {fp} wb = {S}_wv{blk.b};")
+            gij = defaultdict(list)
+            for i, j, k, c in blk.entries:
+                gij[(i, j)].append((k, c))
+            A(f"{ind}  {fp} dwb = 0;")
             for j in blk.j_list:
-                if (i, j) not in gij:
-                    continue
-                expr = None
-                for k, c in gij[(i, j)]:
-                    expr = f"{_lit(c, T)} * gr{k}" if expr is None else f"fma({_lit(c, T)}, gr{k}, {expr})"
-                A(f"        {{ const {fp} G = {expr}; D = fma(G, yv{j}, D); F{j} = fma(G, xv{i}, F{j}); }}")
-            A(f"        dwb = fma(xv{i}, D, dwb); dxa{i} = fma(wb, D, dxa{i});")
-            A("      }")
-        A(f"      if (active) dwp[{blk.b * st.extent} + uu] = dwb;")
-        for j in blk.j_list:
-            A(f"      pj{j} = fma(wb, F{j}, pj{j});")
+                A(f"{ind}  {fp} F{j} = 0;")
+            # per x1 component: G = sum_k c g_k is a temporary feeding both D (with x2) and F (with x1)
+            for i in blk.i_list:
+                A(f"{ind}  {{")
+                A(f"{ind}    {fp} D = 0;")
+                for j in blk.j_list:
+                    if (i, j) not in gij:
+                        continue
+                    expr = None
+                    for k, c in gij[(i, j)]:
+                        expr = f"{_lit(c, T)} * gr{k}" if expr is None else f"fma({_lit(c, T)}, gr{k}, {expr})"
+                    A(f"{ind}    {{ const {fp} G = {expr}; D = fma(G, {S}_yv{j}, D); F{j} = fma(G, {S}_xv{i}, F{j}); }}")
+                A(f"{ind}    dwb = fma({S}_xv{i}, D, dwb); dxa{i} = fma(wb, D, dxa{i});")
+                A(f"{ind}  }}")
+            A(f"{ind}  if (active) dwp[{blk.b * st.extent} + uu] = dwb;")
+            for j in blk.j_list:
+                A(f"{ind}  pj{j} = fma(wb, F{j}, pj{j});")
+            A(f"{ind}}}")
+            A(f"{ind}__builtin_amdgcn_sched_barrier(0);")
+        # dx1: scatter
+        A(f"{ind}if (active) {{")
+        A(f"{ind}  if (ATOMIC_DX1) {{")
+        A(f"{ind}    {fp}* dp = dx1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
+        for i in i_used:
+            A(f"{ind}    unsafeAtomicAdd(dp + ({i * st.extent} + uu), dxa{i});")
+        A(f"{ind}  }} else {{")
+        A(f"{ind}    {fp}* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
+        for i in range(st.nseg_x1):
+            A(f"{ind}    dp[{i * st.extent} + uu] = " + (f"dxa{i};" if i in i_used else "0;"))
+        A(f"{ind}  }}")
+        A(f"{ind}}}")
+        # dx2: reduce over the 64 lanes, then combine channel chunks
+        A(f"{ind}if (!active) {{" + " ".join(f"pj{j} = 0;" for j in j_used) + "}")
+        for j in j_used:
+            A(f"{ind}pj{j} = wave_sum(pj{j});")
+        A(f"{ind}if (lane == 0) {{")
+        if nch == 1:
+            A(f"{ind}  {fp}* __restrict__ d2 = dx2 + z * {st.nseg_x2}ll;")
+        else:
+            A(f"{ind}  {fp}* __restrict__ d2 = dx2_partial + (z * {nch} + ch) * {st.nseg_x2}ll;")
+        for j in range(st.nseg_x2):
+            A(f"{ind}  d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+        A(f"{ind}}}")
+
+    sets = ("a", "b") if prefetch else ("a",)
+    for S in sets:
+        A(f"  int64_t {S}_grow = -1, {S}_srow = 0;")
+        A(f"  {fp} " + ", ".join([f"{S}_xv{i} = 0" for i in i_used] + [f"{S}_wv{blk.b} = 0" for blk in st.blocks]
+                                  + [f"{S}_yv{j} = 0" for j in j_used]) + ";")
+    if prefetch:
+        # one copy of the body (two copies drive the register allocator into hundreds of spills): set "a" is the row in
+        # work, set "b" the row being fetched; "a = b" at the end of the iteration
+        A("  if (z0 < z1) {")
+        load("a", "z0", "    ")
+        A("  }")
+        A("  for (int64_t zz = z0; zz < z1; ++zz) {")
+        A("    {")
+        load("b", "(zz + 1 < z1 ? zz + 1 : zz)", "      ")
         A("    }")
         A("    __builtin_amdgcn_sched_barrier(0);")
-    # dx1: scatter
-    A("    if (active) {")
-    A("      if (ATOMIC_DX1) {")
-    A(f"        {fp}* dp = dx1 + srow * {st.nseg_x1 * st.extent}ll;")
-    for i in i_used:
-        A(f"        unsafeAtomicAdd(dp + ({i * st.extent} + uu), dxa{i});")
-    A("      } else {")
-    A(f"        {fp}* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
-    for i in range(st.nseg_x1):
-        A(f"        dp[{i * st.extent} + uu] = " + (f"dxa{i};" if i in i_used else "0;"))
-    A("      }")
-    A("    }")
-    # dx2: reduce over the 64 lanes, then combine channel chunks
-    A("    if (!active) {" + " ".join(f"pj{j} = 0;" for j in j_used) + "}")
-    for j in j_used:
-        A(f"    pj{j} = wave_sum(pj{j});")
-    if nch == 1:
-        A("    if (lane == 0) {")
-        A(f"      {fp}* __restrict__ d2 = dx2 + z * {st.nseg_x2}ll;")
-        for j in range(st.nseg_x2):
-            A(f"      d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+        A("    {")
+        body("a", "zz", "      ")
         A("    }")
+        A("    a_grow = b_grow; a_srow = b_srow;")
+        A("    " + " ".join([f"a_xv{i} = b_xv{i};" for i in i_used] + [f"a_wv{blk.b} = b_wv{blk.b};" for blk in st.blocks]
+                             + [f"a_yv{j} = b_yv{j};" for j in j_used]))
+        A("  }")
     else:
-        A("    if (lane == 0) {")
-        A(f"      {fp}* __restrict__ d2 = dx2_partial + (z * {nch} + ch) * {st.nseg_x2}ll;")
-        for j in range(st.nseg_x2):
-            A(f"      d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+        A("  for (int64_t zz = z0; zz < z1; ++zz) {")
+        load("a", "zz", "    ")
+        A("    {")
+        body("a", "zz", "      ")
         A("    }")
-    A("  }")
+        A("  }")
     A("}")
     A(f"constexpr int kBwdMinRange = {chunk};   // fewest batch rows worth a wavefront of their own")
     A(f"constexpr int kBwdWaves = {waves_per_eu};")
@@ -420,7 +456,8 @@ BWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}*
 
 
 def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_hash: int, *, fwd_split: int = 1,
-              fwd_waves: int = 2, fwd_prefetch: bool = True, bwd_waves: int = 2, bwd_chunk: int = 16) -> str:
+              fwd_waves: int = 2, fwd_prefetch: bool = True, bwd_waves: int = 2, bwd_chunk: int = 16,
+              bwd_prefetch: bool = False) -> str:
     """Complete .hip translation unit: kernels, host launchers, registration under both table hashes."""
     ns = f"cw_{name}"
     nch = (st.extent + 63) // 64
@@ -440,7 +477,7 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     A("")
     A(emit_forward(st, T, fwd_split, fwd_waves, ns, fwd_prefetch))
     A("")
-    A(emit_backward(st, T, bwd_waves, bwd_chunk))
+    A(emit_backward(st, T, bwd_waves, bwd_chunk, bwd_prefetch))
     A("")
     code = f"dtype_code<{T}>::value"
     A(f"""
