@@ -203,7 +203,7 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
             for i in i_used:
                 A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
             for blk in blocks:
-                A(f"{ind}  {S}_wv{blk.b} = wp[{blk.b * st.extent} + uu];")
+                A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
             A(f"{ind}}}")
 
         def body(S: str, ind: str):
@@ -263,7 +263,7 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
         A("  if (active) {")
         A(f"    {fp}* __restrict__ op = out + r * {st.nseg_out * st.extent}ll;")
         for k in ks:
-            A(f"    op[{k * st.extent} + uu] = acc{k};")
+            A(f"    STREAM_STORE(acc{k}, op + {k * st.extent} + uu);")
         A("  }")
         A("}")
         A("")
@@ -335,7 +335,7 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
         for i in i_used:
             A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
         for blk in st.blocks:
-            A(f"{ind}  {S}_wv{blk.b} = wp[{blk.b * st.extent} + uu];")
+            A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
         for j in j_used:
             A(f"{ind}  {S}_yv{j} = x2p[{j}];")
         A(f"{ind}}}")
@@ -346,7 +346,7 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
         A(f"{ind}  grow_cur = {S}_grow;")
         A(f"{ind}  const {fp}* __restrict__ gp = g + grow_cur * {st.nseg_out * st.extent}ll;")
         for k in range(st.nseg_out):
-            A(f"{ind}  gr{k} = gp[{k * st.extent} + uu];")
+            A(f"{ind}  gr{k} = STREAM_LOAD(gp + {k * st.extent} + uu);")
         A(f"{ind}}}")
         A(f"{ind}{fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
         for i in i_used:
@@ -375,7 +375,7 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
                     A(f"{ind}    {{ const {fp} G = {expr}; D = fma(G, {S}_yv{j}, D); F{j} = fma(G, {S}_xv{i}, F{j}); }}")
                 A(f"{ind}    dwb = fma({S}_xv{i}, D, dwb); dxa{i} = fma(wb, D, dxa{i});")
                 A(f"{ind}  }}")
-            A(f"{ind}  if (active) dwp[{blk.b * st.extent} + uu] = dwb;")
+            A(f"{ind}  if (active) STREAM_STORE(dwb, dwp + {blk.b * st.extent} + uu);")
             for j in blk.j_list:
                 A(f"{ind}  pj{j} = fma(wb, F{j}, pj{j});")
             A(f"{ind}}}")
@@ -468,6 +468,15 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     A(f"// channel-wise tensor product '{name}': extent {st.extent}, segments w/x1/x2/out = "
       f"{st.nseg_w}/{st.nseg_x1}/{st.nseg_x2}/{st.nseg_out}, {st.num_paths} paths, math {T}")
     A('#include "cw_common.h"')
+    A("// operands that are read or written exactly once per launch (weights, weight gradients, the output rows) are")
+    A("// marked non-temporal so that they do not displace the gathered rows in the caches")
+    A("#ifndef CUEQ_CW_NO_STREAM")
+    A("#define STREAM_LOAD(p) __builtin_nontemporal_load(p)")
+    A("#define STREAM_STORE(v, p) __builtin_nontemporal_store(v, p)")
+    A("#else")
+    A("#define STREAM_LOAD(p) (*(p))")
+    A("#define STREAM_STORE(v, p) (*(p) = (v))")
+    A("#endif")
     A("")
     A("namespace cueq {")
     A(f"namespace {ns} {{")
