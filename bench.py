@@ -96,7 +96,27 @@ def cpu_baseline(torch, cue, module, host, sample_edges: int, sample_nodes: int)
 def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
     """Secondary workloads (BASELINE.json configs[2..4]); same timing discipline as the headline line."""
     wl = args.workload
-    if wl == "cfg3":
+    if wl == "cfg1":
+        Z = 4096
+        i1, i2 = cue.Irreps("O3", "32x0e+32x1o+32x2e"), cue.Irreps("O3", "0e+1o+2e")
+        m = cuet.ChannelWiseTensorProduct(i1, i2, ["0e", "1o", "2e"], layout=cue.ir_mul, shared_weights=False,
+                                          internal_weights=False, device=dev, dtype=torch.float32)
+        g = torch.Generator(device=dev).manual_seed(0)
+        x1 = torch.randn(Z, i1.dim, device=dev, generator=g, requires_grad=True)
+        x2 = torch.randn(Z, i2.dim, device=dev, generator=g, requires_grad=True)
+        w = torch.randn(Z, m.weight_numel, device=dev, generator=g, requires_grad=True)
+        cot = torch.randn(Z, m.irreps_out.dim, device=dev, generator=g)
+
+        def step():
+            return torch.autograd.grad(m(x1, x2, w), [x1, x2, w], cot)
+
+        unit, units, dt = "samples/s", Z, "f32"
+        d1, d2, dw, do = i1.dim, i2.dim, m.weight_numel, m.irreps_out.dim
+        alg = {"fwd": Z * (d1 + d2 + dw + do) * 4, "bwd": Z * (2 * (d1 + d2 + dw) + do) * 4}
+        bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
+        desc = ("configs[0]: channel-wise TP 32x0e+32x1o+32x2e (x) 0e+1o+2e, outputs up to l = 2, batch 4096, per-sample weights, "
+                "fwd + bwd (dx1, dx2, dw); 69 MB of traffic: launch-latency regime")
+    elif wl == "cfg3":
         Z = 50_000
         m = cuet.SymmetricContraction(cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "128x0e+128x1o"),
                                       3, 10, layout=cue.ir_mul, dtype=torch.float32, device=dev)
@@ -218,9 +238,9 @@ def main() -> int:
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--deterministic", action="store_true",
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
-    ap.add_argument("--workload", choices=["cfg2", "cfg3", "cfg4", "cfg4fc", "cfg5"], default="cfg2",
+    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4fc", "cfg5"], default="cfg2",
                     help="cfg2 (default) is the headline metric; the others print a secondary line for the same "
-                         "library: cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected product, "
+                         "library: cfg1 the reference's CPU-sized channel-wise case, cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected product, "
                          "cfg5 triangle update")
     args = ap.parse_args()
     if args.gpus != 1:
