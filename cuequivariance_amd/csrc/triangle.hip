@@ -1617,8 +1617,7 @@ extern "C" int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t tran
   const int64_t kc = k_chunks == 1 ? K : (((K + k_chunks - 1) / k_chunks + 31) / 32) * 32;  // contraction per chunk
   const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(nparts * k_chunks));
   CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm_table: too many row tiles");
-  const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
-  const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0) ? 1 : 0;
+  const int vec_out = 0;  // the result offsets come from the device table: their alignment is not known here
   KernelTimer timer("gemm_table", stream);
   // results at most 64 columns wide take 256 x 64 tiles (4 x 1 wavefronts) instead of wasting half a 128 x 128 tile
   const bool skinny = N <= 64;
