@@ -272,25 +272,27 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
         fa[t][q] = gemm_fragment<TI, TA, TMR>(&smem[buf][0], wm * 64 + t * 32, q, lane);
         fb[t][q] = gemm_fragment<TI, TB, TNC>(&smem[buf][ABYTES], wn * 64 + t * 32, q, lane);
       }
+    // consecutive MFMAs go to different accumulators: a dependent one would wait for its predecessor to drain
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int q = 0; q < 2; ++q) {
+      if constexpr (sizeof(TI) == 2) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if constexpr (sizeof(TI) == 2) {
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int q = 0; q < 2; ++q)
+          for (int j = 0; j < 2; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[i][q]),
                                                                 __builtin_bit_cast(bf16x8_t, fb[j][q]), acc[i][j], 0, 0, 0);
-        } else {
+      } else {
 #pragma unroll
-          for (int q = 0; q < 2; ++q) {
-            const float* pa = reinterpret_cast<const float*>(&fa[i][q]);
-            const float* pb = reinterpret_cast<const float*>(&fb[j][q]);
+        for (int s = 0; s < 4; ++s)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[s], pb[s], acc[i][j], 0, 0, 0);
-          }
-        }
+          for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(reinterpret_cast<const float*>(&fa[i][q])[s],
+                                                               reinterpret_cast<const float*>(&fb[j][q])[s], acc[i][j], 0, 0, 0);
       }
+    }
     buf ^= 1;
   }
 
