@@ -921,6 +921,213 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same computation for 2-byte types with the weights resident in LDS: one block per CU loads W1, W2 (C rows)
+// and the biases once, then its wavefronts walk 32-column tiles of m independently - no barrier and no weight
+// traffic inside the loop, and wavefronts of one SIMD drift into different phases (MFMA / gate math / memory).
+// LDS: 2 C (2 K + 16) bytes of weights + 8 C bytes of biases + a wave-private 8-row staging tile for the results.
+// ------------------------------------------------------------------------------------------------
+template <int KT, bool SPLIT, bool DC_BY_ROW>
+__global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
+    gate_bwd_input_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X1,
+                              const uint16_t* __restrict__ X2, int64_t ldx, const uint16_t* __restrict__ bias1,
+                              const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask, const uint16_t* __restrict__ dC,
+                              int64_t ldc, uint16_t* __restrict__ dX1, uint16_t* __restrict__ dX2, int64_t lddx, int accumulate,
+                              uint16_t* __restrict__ dU, uint16_t* __restrict__ dV, int C, int M) {
+  using TI = uint16_t;
+  constexpr int ES = 2, EPV = 8;
+  constexpr int K = 32 * KT, ROWB = K * ES, WSTR = ROWB + 16, NS = ROWB / 64, VPR = ROWB / 16;
+  constexpr int NTH = SPLIT ? 256 : 512, NWAVES = NTH / 64;
+  extern __shared__ __align__(16) char gbi_dsm[];
+  char* sw1 = gbi_dsm;
+  char* sw2 = gbi_dsm + C * WSTR;
+  float* sb = reinterpret_cast<float*>(gbi_dsm + 2 * C * WSTR);  // bias1[C], bias2[C]
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  char* stage = reinterpret_cast<char*>(sb + 2 * C) + wave * (8 * WSTR);
+
+  for (int e = tid; e < C * VPR; e += NTH) {
+    const int r = e / VPR, part = e % VPR;
+    *reinterpret_cast<uint4*>(sw1 + r * WSTR + part * 16) = *reinterpret_cast<const uint4*>(W1 + static_cast<int64_t>(r) * ldw + part * EPV);
+    *reinterpret_cast<uint4*>(sw2 + r * WSTR + part * 16) = *reinterpret_cast<const uint4*>(W2 + static_cast<int64_t>(r) * ldw + part * EPV);
+  }
+  for (int i = tid; i < C; i += NTH) {
+    sb[i] = bias1 ? tri_load(bias1, i) : 0.f;
+    sb[C + i] = bias2 ? tri_load(bias2, i) : 0.f;
+  }
+  __syncthreads();
+
+  const int nchunks = C / 32;
+  const int64_t ntiles = (static_cast<int64_t>(M) + 31) / 32;
+  // v_perm_b32 selectors (bytes 0-3 = own register, 4-7 = the neighbour's): even lane (own.lo, other.lo), odd lane (other.hi, own.hi)
+  const uint32_t pair_sel = (lane & 1) ? 0x03020706u : 0x05040100u;
+  const bool pair_ok = DC_BY_ROW && ((M | ldc) & 1) == 0;
+  for (int64_t tile = static_cast<int64_t>(blockIdx.x) * NWAVES + wave; tile < ntiles; tile += static_cast<int64_t>(gridDim.x) * NWAVES) {
+    const int mrow0 = static_cast<int>(tile * 32);
+    const int mcol = mrow0 + c;
+    const int mld = min(mcol, M - 1);
+    uint4 xf1[NS][2], xf2[SPLIT ? NS : 1][2];
+#pragma unroll
+    for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int64_t o = static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES;
+        xf1[s2][q] = *reinterpret_cast<const uint4*>(X1 + o);
+        if constexpr (SPLIT) xf2[s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
+      }
+    const float mk = mask ? tri_load(mask, mld) : 1.0f;
+    floatx16 ax1[KT], ax2[SPLIT ? KT : 1];
+#pragma unroll
+    for (int t = 0; t < KT; ++t) ax1[t] = floatx16{0};
+#pragma unroll
+    for (int t = 0; t < (SPLIT ? KT : 1); ++t) ax2[t] = floatx16{0};
+
+    uint32_t dcr[16], dcn[16];
+    const uint32_t dcofs = DC_BY_ROW ? static_cast<uint32_t>((4 * h * ldc + mld) * ES) : static_cast<uint32_t>((mld * ldc + 4 * h) * ES);
+    auto load_dc = [&](int c0) {
+      if constexpr (DC_BY_ROW) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * (v >> 2) + (v & 3)) * ldc * ES);
+          dcn[v] = load_global<uint16_t>(base, dcofs);
+        }
+      } else {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * a) * ES);
+          const uint2 w = load_global<uint2>(base, dcofs);
+          dcn[4 * a] = w.x; dcn[4 * a + 1] = w.y;  // values 4a..4a+3 in two registers
+        }
+      }
+    };
+    auto dc_value = [&](int v) -> float {
+      if constexpr (DC_BY_ROW) return __uint_as_float(dcr[v] << 16);
+      const uint32_t w = dcr[4 * (v >> 2) + ((v & 3) >> 1)];
+      return (v & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+    };
+
+    load_dc(0);
+    for (int ci = 0; ci < nchunks; ++ci) {
+      const int c0 = ci * 32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) dcr[v] = dcn[v];
+      if (ci + 1 < nchunks) load_dc(c0 + 32);
+
+      floatx16 au, av;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const float4 b1 = *reinterpret_cast<const float4*>(sb + c0 + 8 * a + 4 * h);
+        const float4 b2 = *reinterpret_cast<const float4*>(sb + C + c0 + 8 * a + 4 * h);
+        au[4 * a] = b1.x; au[4 * a + 1] = b1.y; au[4 * a + 2] = b1.z; au[4 * a + 3] = b1.w;
+        av[4 * a] = b2.x; av[4 * a + 1] = b2.y; av[4 * a + 2] = b2.z; av[4 * a + 3] = b2.w;
+      }
+      {
+        const char* w1 = sw1 + (c0 + c) * WSTR + h * 32;
+        const char* w2 = sw2 + (c0 + c) * WSTR + h * 32;
+#pragma unroll
+        for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const uint4 a1 = *reinterpret_cast<const uint4*>(w1 + s2 * 64 + q * 16);
+            const uint4 a2 = *reinterpret_cast<const uint4*>(w2 + s2 * 64 + q * 16);
+            mma_step<TI>(au, a1, xf1[s2][q]);
+            mma_step<TI>(av, a2, SPLIT ? xf2[s2][q] : xf1[s2][q]);
+          }
+      }
+      uint32_t pu[8], pv[8];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        float du[4], dv[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int v = 4 * a + b;
+          const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-au[v]));
+          dv[b] = dc_value(v) * mk * sg;
+          du[b] = dv[b] * fmaf(-av[v], sg, av[v]);
+        }
+        pu[2 * a] = pack_bf16(du[0], du[1]); pu[2 * a + 1] = pack_bf16(du[2], du[3]);
+        pv[2 * a] = pack_bf16(dv[0], dv[1]); pv[2 * a + 1] = pack_bf16(dv[2], dv[3]);
+        if (dU != nullptr) {
+          const int row = c0 + 8 * a + 4 * h;
+          if constexpr (!DC_BY_ROW) {
+            // the lane's four rows are adjacent elements of its m row: one 8-byte store per array
+            if (mcol < M) {
+              const int64_t o = static_cast<int64_t>(mcol) * ldc + row;
+              *reinterpret_cast<uint2*>(dU + o) = make_uint2(pu[2 * a], pu[2 * a + 1]);
+              *reinterpret_cast<uint2*>(dV + o) = make_uint2(pv[2 * a], pv[2 * a + 1]);
+            }
+          } else if (pair_ok) {
+            // neighbouring lanes swap halves: the even lane stores rows 0 and 2 for columns (m, m + 1), the odd
+            // lane rows 1 and 3 for columns (m - 1, m) - 4-byte stores, 128 contiguous bytes per half-wave
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const uint32_t ou = pu[2 * a + j], ov = pv[2 * a + j];
+              const uint32_t ru = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(ou), 0xB1, 0xF, 0xF, true));
+              const uint32_t rv = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(ov), 0xB1, 0xF, 0xF, true));
+              const uint32_t wu = __builtin_amdgcn_perm(ru, ou, pair_sel), wv = __builtin_amdgcn_perm(rv, ov, pair_sel);
+              if (mcol < M) {
+                const int64_t o = static_cast<int64_t>(row + 2 * j + (lane & 1)) * ldc + (mcol & ~1);
+                *reinterpret_cast<uint32_t*>(dU + o) = wu;
+                *reinterpret_cast<uint32_t*>(dV + o) = wv;
+              }
+            }
+          } else if (mcol < M) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              const int64_t o = static_cast<int64_t>(row + b) * ldc + mcol;
+              tri_store(dU, o, du[b]);
+              tri_store(dV, o, dv[b]);
+            }
+          }
+        }
+      }
+      {
+        typedef shortx4_t __attribute__((address_space(3))) * lptr;
+        const int s16 = lane & 15, g16 = (lane >> 4) & 1;
+        const int off = (c0 + 4 * h + (s16 >> 2)) * WSTR + (16 * g16 + 4 * (s16 & 3)) * 2;
+#pragma unroll
+        for (int ds = 0; ds < KT; ++ds)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const int o = off + t * 16 * WSTR + ds * 64;
+            const uint2 l1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw1 + o)));
+            const uint2 h1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw1 + o + 8 * WSTR)));
+            const uint2 l2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw2 + o)));
+            const uint2 h2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw2 + o + 8 * WSTR)));
+            mma_step<TI>(ax1[ds], make_uint4(pu[4 * t], pu[4 * t + 1], pu[4 * t + 2], pu[4 * t + 3]), make_uint4(l1.x, l1.y, h1.x, h1.y));
+            mma_step<TI>(SPLIT ? ax2[ds] : ax1[ds], make_uint4(pv[4 * t], pv[4 * t + 1], pv[4 * t + 2], pv[4 * t + 3]),
+                         make_uint4(l2.x, l2.y, h2.x, h2.y));
+          }
+      }
+    }
+
+    // results: 8 rows (one value group a) at a time through the wave-private staging tile, 16-byte row vectors out
+#pragma unroll
+    for (int which = 0; which < (SPLIT ? 2 : 1); ++which) {
+      uint16_t* dst = which == 0 ? dX1 : dX2;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int ds = 0; ds < KT; ++ds) {
+          const floatx16& acc = (which == 0) ? ax1[ds] : ax2[SPLIT ? ds : 0];
+          const uint32_t w01 = pack_bf16(acc[4 * a], acc[4 * a + 1]), w23 = pack_bf16(acc[4 * a + 2], acc[4 * a + 3]);
+          char* p = stage + (4 * h) * WSTR + (ds * 32 + c) * 2;
+          *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(w01 & 0xffffu);
+          *reinterpret_cast<uint16_t*>(p + WSTR) = static_cast<uint16_t>(w01 >> 16);
+          *reinterpret_cast<uint16_t*>(p + 2 * WSTR) = static_cast<uint16_t>(w23 & 0xffffu);
+          *reinterpret_cast<uint16_t*>(p + 3 * WSTR) = static_cast<uint16_t>(w23 >> 16);
+        }
+        __builtin_amdgcn_wave_barrier();
+        const int r0 = mrow0 + 8 * a;
+        const int rows = min(8, M - r0);
+        if (rows > 0)
+          stage_flush<TI, K>(stage, WSTR, rows, dst + static_cast<int64_t>(r0) * lddx, lddx, lane, 64, which == 0 && accumulate != 0);
+      }
+    }
+  }
+}
+
 // any shape / alignment / operand order: one thread per output element (rs*: stride between rows of the operand,
 // ks*: stride along the contraction)
 template <typename TI, typename TO>
@@ -1731,7 +1938,8 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
   CUEQ_REQUIRE(!(split && accumulate), CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: accumulate needs a single input");
   const int epv = bf ? 8 : 4;
   const uintptr_t ptrs = reinterpret_cast<uintptr_t>(W1) | reinterpret_cast<uintptr_t>(W2) | reinterpret_cast<uintptr_t>(X1) | reinterpret_cast<uintptr_t>(X2) |
-                         (dc_by_row ? 0 : reinterpret_cast<uintptr_t>(dC)) | reinterpret_cast<uintptr_t>(dX1) | reinterpret_cast<uintptr_t>(dX2);
+                         (dc_by_row ? 0 : reinterpret_cast<uintptr_t>(dC)) | reinterpret_cast<uintptr_t>(dX1) | reinterpret_cast<uintptr_t>(dX2) |
+                         reinterpret_cast<uintptr_t>(dU) | reinterpret_cast<uintptr_t>(dV);
   const bool aligned = (ptrs & 15) == 0 && ldw % epv == 0 && ldx % epv == 0 && lddx % epv == 0 && (dc_by_row || ldc % epv == 0);
   CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: row strides and pointers must be multiples of 16 bytes");
   CUEQ_REQUIRE(split == !dc_by_row, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: built for one input with dC by rows (C x M) and two inputs with dC by columns (M x C)");
@@ -1740,6 +1948,25 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
                    (dc_by_row ? (4 * ldc + M) : (M * ldc + 8)) * es < (1ll << 32),
                CUEQ_ERR_TOO_LARGE, "gate_bwd_input: strides too large for 32-bit lane offsets");
   KernelTimer timer("gate_bwd_input", stream);
+  if (bf) {
+    // weights resident in LDS when they fit (2 C rows of 2 K + 16 bytes, biases, staging tiles)
+    const int nwaves = split ? 4 : 8;
+    const size_t lds = static_cast<size_t>(2 * C * (2 * K + 16) + 8 * C + nwaves * 8 * (2 * K + 16));
+    if (lds <= 160 * 1024) {
+      const int64_t ntiles = (M + 31) / 32;
+      int64_t gx = (ntiles + nwaves - 1) / nwaves;
+      if (gx > device_cus()) gx = device_cus();
+#define GBR(KT, SP) do { auto kfn = gate_bwd_input_res_kernel<KT, SP, !SP>; \
+        CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(SP ? 256 : 512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X1), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<const uint16_t*>(dC), ldc, static_cast<uint16_t*>(dX1), static_cast<uint16_t*>(dX2), lddx, accumulate, static_cast<uint16_t*>(dU), static_cast<uint16_t*>(dV), static_cast<int>(C), static_cast<int>(M)); } while (0)
+#define GBR_K(SP) do { switch (K / 32) { case 1: GBR(1, SP); break; case 2: GBR(2, SP); break; case 3: GBR(3, SP); break; default: GBR(4, SP); break; } } while (0)
+      if (split) GBR_K(true); else GBR_K(false);
+#undef GBR_K
+#undef GBR
+      CUEQ_CHECK_HIP(hipGetLastError());
+      return CUEQ_OK;
+    }
+  }
 #define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP, !SP>), dim3(static_cast<unsigned>((M + gbi_threads<TI, SP>() / 2 - 1) / (gbi_threads<TI, SP>() / 2))), dim3(gbi_threads<TI, SP>()), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
 #define GBI_K(TI, SP) do { switch (K / 32) { case 1: GBI(TI, 1, SP); break; case 2: GBI(TI, 2, SP); break; case 3: GBI(TI, 3, SP); break; default: GBI(TI, 4, SP); break; } } while (0)
 #define GBI_T(TI) do { if (split) GBI_K(TI, true); else GBI_K(TI, false); } while (0)
