@@ -936,7 +936,13 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
                               uint16_t* __restrict__ dU, uint16_t* __restrict__ dV, int C, int M) {
   using TI = uint16_t;
   constexpr int ES = 2, EPV = 8;
-  constexpr int K = 32 * KT, ROWB = K * ES, WSTR = ROWB + 16, NS = ROWB / 64, VPR = ROWB / 16;
+  constexpr int K = 32 * KT, ROWB = K * ES, NS = ROWB / 64, VPR = ROWB / 16;
+  // weight rows in LDS: 256-byte rows keep their 16-byte units XOR-swizzled by a rotation of the row's low four bits
+  // (16 consecutive rows put one unit on 16 different bank groups for the row-operand reads; 4 consecutive rows put
+  // one 64-byte span on 4 different ones for the transposing reads); shorter rows are padded by 16 bytes instead
+  constexpr bool SWZ = KT == 4;
+  constexpr int WSTR = SWZ ? ROWB : ROWB + 16, SSTR = ROWB + 16;
+  auto swz = [](int row) -> int { return SWZ ? (((row & 3) << 2) | ((row >> 2) & 3)) : 0; };
   constexpr int NTH = SPLIT ? 256 : 512, NWAVES = NTH / 64;
   extern __shared__ __align__(16) char gbi_dsm[];
   char* sw1 = gbi_dsm;
@@ -944,12 +950,13 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   float* sb = reinterpret_cast<float*>(gbi_dsm + 2 * C * WSTR);  // bias1[C], bias2[C]
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
-  char* stage = reinterpret_cast<char*>(sb + 2 * C) + wave * (8 * WSTR);
+  char* stage = reinterpret_cast<char*>(sb + 2 * C) + wave * (8 * SSTR);
 
   for (int e = tid; e < C * VPR; e += NTH) {
     const int r = e / VPR, part = e % VPR;
-    *reinterpret_cast<uint4*>(sw1 + r * WSTR + part * 16) = *reinterpret_cast<const uint4*>(W1 + static_cast<int64_t>(r) * ldw + part * EPV);
-    *reinterpret_cast<uint4*>(sw2 + r * WSTR + part * 16) = *reinterpret_cast<const uint4*>(W2 + static_cast<int64_t>(r) * ldw + part * EPV);
+    const int po = (part ^ swz(r)) << 4;
+    *reinterpret_cast<uint4*>(sw1 + r * WSTR + po) = *reinterpret_cast<const uint4*>(W1 + static_cast<int64_t>(r) * ldw + part * EPV);
+    *reinterpret_cast<uint4*>(sw2 + r * WSTR + po) = *reinterpret_cast<const uint4*>(W2 + static_cast<int64_t>(r) * ldw + part * EPV);
   }
   for (int i = tid; i < C; i += NTH) {
     sb[i] = bias1 ? tri_load(bias1, i) : 0.f;
@@ -961,57 +968,88 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   const int64_t ntiles = (static_cast<int64_t>(M) + 31) / 32;
   // v_perm_b32 selectors (bytes 0-3 = own register, 4-7 = the neighbour's): even lane (own.lo, other.lo), odd lane (other.hi, own.hi)
   const uint32_t pair_sel = (lane & 1) ? 0x03020706u : 0x05040100u;
-  const bool pair_ok = DC_BY_ROW && ((M | ldc) & 1) == 0;
-  for (int64_t tile = static_cast<int64_t>(blockIdx.x) * NWAVES + wave; tile < ntiles; tile += static_cast<int64_t>(gridDim.x) * NWAVES) {
-    const int mrow0 = static_cast<int>(tile * 32);
-    const int mcol = mrow0 + c;
-    const int mld = min(mcol, M - 1);
-    uint4 xf1[NS][2], xf2[SPLIT ? NS : 1][2];
+  const int64_t tstep = static_cast<int64_t>(gridDim.x) * NWAVES;
+  auto tile_row = [&](int64_t t) -> int { return static_cast<int>(min(t * 32 + c, static_cast<int64_t>(M) - 1)); };
+
+  // cotangent values of a chunk, packed: register 2 a + j holds rows 8 a + 4 h + 2 j, + 1 of this lane's column.
+  // dC by rows (C x M): a lane pair loads 4-byte column pairs - the even lane of row 2 j, the odd lane of row
+  // 2 j + 1 - and swaps halves on use; dC by columns (M x C): the four rows are 8 adjacent bytes.
+  // The loads run a chunk ahead of their use, across tile boundaries: (ptile, pci) is the next chunk to request.
+  uint32_t dcr[8], dcn[8];
+  auto dc_lane_offset = [&](int mld) -> uint32_t {
+    return DC_BY_ROW ? static_cast<uint32_t>(((4 * h + (lane & 1)) * ldc + (mld & ~1)) * ES) : static_cast<uint32_t>((mld * ldc + 4 * h) * ES);
+  };
+  int64_t ptile = static_cast<int64_t>(blockIdx.x) * NWAVES + wave;
+  int pci = 0;
+  uint32_t pofs = ptile < ntiles ? dc_lane_offset(tile_row(ptile)) : 0u;
+  auto request_dc = [&](uint32_t (&dst)[8]) {
+    if (ptile >= ntiles) return;
+    const int c0 = pci * 32;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      if constexpr (DC_BY_ROW) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * a + 2 * j) * ldc * ES);
+          dst[2 * a + j] = load_global<uint32_t>(base, pofs);
+        }
+      } else {
+        const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * a) * ES);
+        const uint2 w = load_global<uint2>(base, pofs);
+        dst[2 * a] = w.x; dst[2 * a + 1] = w.y;
+      }
+    }
+    if (++pci == nchunks) {
+      pci = 0;
+      ptile += tstep;
+      if (ptile < ntiles) pofs = dc_lane_offset(tile_row(ptile));
+    }
+  };
+  auto dc_value = [&](int v) -> float {
+    const uint32_t w = dcr[v >> 1];
+    return (v & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+  };
+  // the rows of X of a tile, one row per lane, and its mask value; those of the next tile are requested a tile ahead
+  uint4 xf1[NS][2], xf2[SPLIT ? NS : 1][2], xn1[NS][2], xn2[SPLIT ? NS : 1][2];
+  float mk = 1.0f, mkn = 1.0f;
+  auto request_x = [&](int mld, uint4 (&x1)[NS][2], uint4 (&x2)[SPLIT ? NS : 1][2], float& m) {
 #pragma unroll
     for (int s2 = 0; s2 < NS; ++s2)
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const int64_t o = static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES;
-        xf1[s2][q] = *reinterpret_cast<const uint4*>(X1 + o);
-        if constexpr (SPLIT) xf2[s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
+        x1[s2][q] = *reinterpret_cast<const uint4*>(X1 + o);
+        if constexpr (SPLIT) x2[s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
       }
-    const float mk = mask ? tri_load(mask, mld) : 1.0f;
+    if (mask) m = tri_load(mask, mld);
+  };
+  int64_t tile = ptile;
+  if (tile < ntiles) request_x(tile_row(tile), xf1, xf2, mk);
+  request_dc(dcn);
+
+  for (; tile < ntiles; tile += tstep) {
+    const int mrow0 = static_cast<int>(tile * 32);
+    const int mcol = mrow0 + c;
+    const bool more = tile + tstep < ntiles;
+    if (more) request_x(tile_row(tile + tstep), xn1, xn2, mkn);
     floatx16 ax1[KT], ax2[SPLIT ? KT : 1];
 #pragma unroll
     for (int t = 0; t < KT; ++t) ax1[t] = floatx16{0};
 #pragma unroll
     for (int t = 0; t < (SPLIT ? KT : 1); ++t) ax2[t] = floatx16{0};
 
-    uint32_t dcr[16], dcn[16];
-    const uint32_t dcofs = DC_BY_ROW ? static_cast<uint32_t>((4 * h * ldc + mld) * ES) : static_cast<uint32_t>((mld * ldc + 4 * h) * ES);
-    auto load_dc = [&](int c0) {
-      if constexpr (DC_BY_ROW) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * (v >> 2) + (v & 3)) * ldc * ES);
-          dcn[v] = load_global<uint16_t>(base, dcofs);
-        }
-      } else {
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          const char* base = uniform_ptr(reinterpret_cast<const char*>(dC) + static_cast<int64_t>(c0 + 8 * a) * ES);
-          const uint2 w = load_global<uint2>(base, dcofs);
-          dcn[4 * a] = w.x; dcn[4 * a + 1] = w.y;  // values 4a..4a+3 in two registers
-        }
-      }
-    };
-    auto dc_value = [&](int v) -> float {
-      if constexpr (DC_BY_ROW) return __uint_as_float(dcr[v] << 16);
-      const uint32_t w = dcr[4 * (v >> 2) + ((v & 3) >> 1)];
-      return (v & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
-    };
-
-    load_dc(0);
     for (int ci = 0; ci < nchunks; ++ci) {
       const int c0 = ci * 32;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) dcr[v] = dcn[v];
-      if (ci + 1 < nchunks) load_dc(c0 + 32);
+      for (int v = 0; v < 8; ++v) {
+        if constexpr (DC_BY_ROW) {
+          const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(dcn[v]), 0xB1, 0xF, 0xF, true));
+          dcr[v] = __builtin_amdgcn_perm(other, dcn[v], pair_sel);
+        } else {
+          dcr[v] = dcn[v];
+        }
+      }
+      request_dc(dcn);
 
       floatx16 au, av;
 #pragma unroll
@@ -1022,14 +1060,14 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
         av[4 * a] = b2.x; av[4 * a + 1] = b2.y; av[4 * a + 2] = b2.z; av[4 * a + 3] = b2.w;
       }
       {
-        const char* w1 = sw1 + (c0 + c) * WSTR + h * 32;
-        const char* w2 = sw2 + (c0 + c) * WSTR + h * 32;
+        const int wrow = (c0 + c) * WSTR;
 #pragma unroll
         for (int s2 = 0; s2 < NS; ++s2)
 #pragma unroll
           for (int q = 0; q < 2; ++q) {
-            const uint4 a1 = *reinterpret_cast<const uint4*>(w1 + s2 * 64 + q * 16);
-            const uint4 a2 = *reinterpret_cast<const uint4*>(w2 + s2 * 64 + q * 16);
+            const int wo = wrow + ((((2 * h + q) ^ swz(c)) << 4) ^ (s2 << 6));
+            const uint4 a1 = *reinterpret_cast<const uint4*>(sw1 + wo);
+            const uint4 a2 = *reinterpret_cast<const uint4*>(sw2 + wo);
             mma_step<TI>(au, a1, xf1[s2][q]);
             mma_step<TI>(av, a2, SPLIT ? xf2[s2][q] : xf1[s2][q]);
           }
@@ -1056,7 +1094,7 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
               *reinterpret_cast<uint2*>(dU + o) = make_uint2(pu[2 * a], pu[2 * a + 1]);
               *reinterpret_cast<uint2*>(dV + o) = make_uint2(pv[2 * a], pv[2 * a + 1]);
             }
-          } else if (pair_ok) {
+          } else {
             // neighbouring lanes swap halves: the even lane stores rows 0 and 2 for columns (m, m + 1), the odd
             // lane rows 1 and 3 for columns (m - 1, m) - 4-byte stores, 128 contiguous bytes per half-wave
 #pragma unroll
@@ -1071,29 +1109,26 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
                 *reinterpret_cast<uint32_t*>(dV + o) = wv;
               }
             }
-          } else if (mcol < M) {
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-              const int64_t o = static_cast<int64_t>(row + b) * ldc + mcol;
-              tri_store(dU, o, du[b]);
-              tri_store(dV, o, dv[b]);
-            }
           }
         }
       }
       {
         typedef shortx4_t __attribute__((address_space(3))) * lptr;
         const int s16 = lane & 15, g16 = (lane >> 4) & 1;
-        const int off = (c0 + 4 * h + (s16 >> 2)) * WSTR + (16 * g16 + 4 * (s16 & 3)) * 2;
+        // rows 4 h + (s16 >> 2) (+ 8, + 16 t): a row 8 further flips bit 1 of the swizzle, 16 further leaves it
+        const int trow = 4 * h + (s16 >> 2), tunit = 2 * g16 + ((s16 & 3) >> 1);
+        const int off = (c0 + trow) * WSTR + 8 * (s16 & 1);
+        const int ulo = (tunit ^ swz(trow)) << 4, uhi = SWZ ? (ulo ^ 32) : ulo;
 #pragma unroll
         for (int ds = 0; ds < KT; ++ds)
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
-            const int o = off + t * 16 * WSTR + ds * 64;
+            const int o = off + t * 16 * WSTR + (ulo ^ (ds << 6));
+            const int o8 = off + (t * 16 + 8) * WSTR + (uhi ^ (ds << 6));
             const uint2 l1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw1 + o)));
-            const uint2 h1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw1 + o + 8 * WSTR)));
+            const uint2 h1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw1 + o8)));
             const uint2 l2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw2 + o)));
-            const uint2 h2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw2 + o + 8 * WSTR)));
+            const uint2 h2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw2 + o8)));
             mma_step<TI>(ax1[ds], make_uint4(pu[4 * t], pu[4 * t + 1], pu[4 * t + 2], pu[4 * t + 3]), make_uint4(l1.x, l1.y, h1.x, h1.y));
             mma_step<TI>(SPLIT ? ax2[ds] : ax1[ds], make_uint4(pv[4 * t], pv[4 * t + 1], pv[4 * t + 2], pv[4 * t + 3]),
                          make_uint4(l2.x, l2.y, h2.x, h2.y));
@@ -1112,18 +1147,28 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
         for (int ds = 0; ds < KT; ++ds) {
           const floatx16& acc = (which == 0) ? ax1[ds] : ax2[SPLIT ? ds : 0];
           const uint32_t w01 = pack_bf16(acc[4 * a], acc[4 * a + 1]), w23 = pack_bf16(acc[4 * a + 2], acc[4 * a + 3]);
-          char* p = stage + (4 * h) * WSTR + (ds * 32 + c) * 2;
+          char* p = stage + (4 * h) * SSTR + (ds * 32 + c) * 2;
           *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(w01 & 0xffffu);
-          *reinterpret_cast<uint16_t*>(p + WSTR) = static_cast<uint16_t>(w01 >> 16);
-          *reinterpret_cast<uint16_t*>(p + 2 * WSTR) = static_cast<uint16_t>(w23 & 0xffffu);
-          *reinterpret_cast<uint16_t*>(p + 3 * WSTR) = static_cast<uint16_t>(w23 >> 16);
+          *reinterpret_cast<uint16_t*>(p + SSTR) = static_cast<uint16_t>(w01 >> 16);
+          *reinterpret_cast<uint16_t*>(p + 2 * SSTR) = static_cast<uint16_t>(w23 & 0xffffu);
+          *reinterpret_cast<uint16_t*>(p + 3 * SSTR) = static_cast<uint16_t>(w23 >> 16);
         }
         __builtin_amdgcn_wave_barrier();
         const int r0 = mrow0 + 8 * a;
         const int rows = min(8, M - r0);
         if (rows > 0)
-          stage_flush<TI, K>(stage, WSTR, rows, dst + static_cast<int64_t>(r0) * lddx, lddx, lane, 64, which == 0 && accumulate != 0);
+          stage_flush<TI, K>(stage, SSTR, rows, dst + static_cast<int64_t>(r0) * lddx, lddx, lane, 64, which == 0 && accumulate != 0);
       }
+    }
+    if (more) {
+#pragma unroll
+      for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          xf1[s2][q] = xn1[s2][q];
+          if constexpr (SPLIT) xf2[s2][q] = xn2[s2][q];
+        }
+      mk = mkn;
     }
   }
 }
@@ -1951,8 +1996,10 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
   if (bf) {
     // weights resident in LDS when they fit (2 C rows of 2 K + 16 bytes, biases, staging tiles)
     const int nwaves = split ? 4 : 8;
-    const size_t lds = static_cast<size_t>(2 * C * (2 * K + 16) + 8 * C + nwaves * 8 * (2 * K + 16));
-    if (lds <= 160 * 1024) {
+    const size_t lds = static_cast<size_t>(2 * C * (K == 128 ? 2 * K : 2 * K + 16) + 8 * C + nwaves * 8 * (2 * K + 16));
+    // (dC by rows is read, and the gate gradients written, as 4-byte column pairs)
+    const bool pairs_ok = !dc_by_row || (M % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(dC) % 4 == 0);
+    if (lds <= 160 * 1024 && pairs_ok) {
       const int64_t ntiles = (M + 31) / 32;
       int64_t gx = (ntiles + nwaves - 1) / nwaves;
       if (gx > device_cus()) gx = device_cus();

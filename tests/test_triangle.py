@@ -196,3 +196,48 @@ def test_full_size_properties(device):
     scale = a.float().abs().max().item()
     assert (a.float() - b.float()).abs().max().item() <= 2e-2 * scale
     assert torch.isfinite(out_in.float()).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("M", [2048 * 32 + 37 * 32 + 8, 3 * 32 + 8])
+def test_gate_bwd_input_many_tiles(device, dtype, split, M):
+    """The fused gate backward on more row tiles than one launch holds wavefronts for (each wavefront then walks several
+    tiles, the last one partial), against the closed form d/dX of sum(dC * sigmoid(U) * V * mask) written with torch in
+    float64: U = W1 X1^T + b1, V = W2 X2^T + b2."""
+    from cuequivariance_amd.cuet import triangle as T
+
+    g = torch.Generator().manual_seed(11)
+    C, K = 64, 64
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    W1, W2, b1, b2 = r(C, K) / 8, r(C, K) / 8, r(C), r(C)
+    X1, X2 = r(M, K), (r(M, K) if split else None)
+    mask = (torch.rand(M, generator=g) > 0.2).double()
+    dC = r(C, M) if not split else r(M, C)
+    prior = r(M, K) if not split else None
+    q = lambda t: None if t is None else t.to(dtype)  # the kernel's inputs, rounded once
+    W1, W2, b1, b2, X1, X2, mask, dC, prior = map(q, (W1, W2, b1, b2, X1, X2, mask, dC, prior))
+    d = lambda t: None if t is None else t.double()
+    Xb = d(X2) if split else d(X1)
+    U = d(W1) @ d(X1).T + d(b1)[:, None]
+    V = d(W2) @ Xb.T + d(b2)[:, None]
+    dCm = (d(dC) if not split else d(dC).T) * d(mask)[None, :]
+    sg = torch.sigmoid(U)
+    dV = dCm * sg
+    dU = dCm * V * sg * (1 - sg)
+    if split:
+        want1, want2 = dU.T @ d(W1), dV.T @ d(W2)
+    else:
+        want1, want2 = d(prior) + dU.T @ d(W1) + dV.T @ d(W2), None
+    dev = lambda t: None if t is None else t.to(device)
+    got = T.gate_bwd_input(dev(dC), not split, dev(W1), dev(W2), dev(X1), dev(X2), dev(b1), dev(b2), dev(mask),
+                           dX1=dev(prior.clone()) if prior is not None else None, want_gate_grads=True)
+    assert got is not None
+    g1, g2, gU, gV = got
+    tol = TOL[dtype]
+    assert rel_err(g1, want1) <= tol, rel_err(g1, want1)
+    if split:
+        assert rel_err(g2, want2) <= tol, rel_err(g2, want2)
+    layout = (lambda t: t) if not split else (lambda t: t.T)
+    assert rel_err(gU, layout(dU)) <= tol and rel_err(gV, layout(dV)) <= tol
