@@ -46,7 +46,10 @@ def _analyse(polynomial: cue.SegmentedPolynomial):
     if stp.num_paths == 0:
         raise NotImplementedError("fused_tp does not support empty paths.")
     # every mode that does not index the weights (the irrep components i, j, k) is flattened away
-    d = stp.flatten_modes([m for m in stp.subscripts.modes() if m not in stp.subscripts.operands[0]])
+    try:
+        d = stp.flatten_modes([m for m in stp.subscripts.modes() if m not in stp.subscripts.operands[0]])
+    except ValueError as e:
+        raise NotImplementedError(f"fused_tp does not support {stp.subscripts} (the weights come first): {e}") from e
     ss = d.subscripts.operands
     if stp.num_operands == 3:
         if not (len(ss[0]) == 2 and ss[1] == ss[0][0] and ss[2] == ss[0][1]):
