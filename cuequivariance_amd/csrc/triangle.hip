@@ -1763,7 +1763,13 @@ __global__ void __launch_bounds__(256) sum_rows_partial_kernel(const TI* __restr
   if (cc >= Ccols) return;
   const int64_t r0 = blockIdx.y * rows_per_block, r1 = min(r0 + rows_per_block, R);
   float s = 0;
-  for (int64_t r = r0; r < r1; ++r) s += tri_load(in, r * Ccols + cc);
+  int64_t r = r0;
+  for (; r + 4 <= r1; r += 4) {  // four loads in flight, added in row order
+    const float v0 = tri_load(in, r * Ccols + cc), v1 = tri_load(in, (r + 1) * Ccols + cc);
+    const float v2 = tri_load(in, (r + 2) * Ccols + cc), v3 = tri_load(in, (r + 3) * Ccols + cc);
+    s += v0; s += v1; s += v2; s += v3;
+  }
+  for (; r < r1; ++r) s += tri_load(in, r * Ccols + cc);
   part[static_cast<int64_t>(blockIdx.y) * Ccols + cc] = s;
 }
 
@@ -1874,11 +1880,15 @@ extern "C" int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t tran
   const int vec_out = 0;  // the result offsets come from the device table: their alignment is not known here
   KernelTimer timer("gemm_table", stream);
   // results at most 64 columns wide take 256 x 64 tiles (4 x 1 wavefronts) instead of wasting half a 128 x 128 tile
+  // and products of at most 64 x 64 with both operands contraction-major (weight gradients of small blocks) take one
+  // wavefront each
   const bool skinny = N <= 64;
+  const bool small = skinny && M <= 64 && trans_a && trans_b;
   const dim3 grid_s(1, static_cast<unsigned>((M + 255) / 256), static_cast<unsigned>(nparts * k_chunks));
+  const dim3 grid_1(1, 1, static_cast<unsigned>(nparts * k_chunks));
 #define GT_ARGS(TI, TO) static_cast<const TI*>(A), lda, k_chunks == 1 ? 0 : kc * lda, static_cast<const TI*>(B), ldb, k_chunks == 1 ? 0 : kc * ldb, static_cast<TO*>(C), ldc, chunk_stride_c, static_cast<int>(M), static_cast<int>(N), static_cast<int>(kc), static_cast<float>(alpha), accumulate, vec_out, k_chunks == 1 ? 0 : K, static_cast<int>(nparts), 0, 0, 0, table, 0, 3, 0, 0
 #define GT(TI, TO, TA, TB) do { if (skinny) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB, 4, 1>), grid_s, dim3(256), 0, stream, GT_ARGS(TI, TO)); else hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, GT_ARGS(TI, TO)); } while (0)
-#define GT_T(TI, TO) do { if (trans_a && trans_b) GT(TI, TO, true, true); else if (trans_b) GT(TI, TO, false, true); else GT(TI, TO, false, false); } while (0)
+#define GT_T(TI, TO) do { if (small) hipLaunchKernelGGL((gemm_kernel<TI, TO, true, true, 1, 1>), grid_1, dim3(64), 0, stream, GT_ARGS(TI, TO)); else if (trans_a && trans_b) GT(TI, TO, true, true); else if (trans_b) GT(TI, TO, false, true); else GT(TI, TO, false, false); } while (0)
   if (in_dtype == CUEQ_F32) GT_T(float, float);
   else if (out_dtype == CUEQ_F32) GT_T(uint16_t, float);
   else GT_T(uint16_t, uint16_t);
@@ -2303,13 +2313,17 @@ extern "C" int cueq_sum_cols(int32_t dtype, int64_t rows, int64_t cols, const vo
   return CUEQ_OK;
 }
 
-static int64_t sum_rows_blocks(int64_t rows) {
-  int64_t nb = (rows + 255) / 256;
+// row blocks of the first stage: enough of them that the launch fills the chip (about 2048 workgroups with the column
+// blocks), at least 8 rows each, at most 1024
+static int64_t sum_rows_blocks(int64_t rows, int64_t cols) {
+  const int64_t col_blocks = (cols + 255) / 256;
+  int64_t nb = (2048 + col_blocks - 1) / col_blocks;
+  if (nb > (rows + 7) / 8) nb = (rows + 7) / 8;
   if (nb > 1024) nb = 1024;
   return nb < 1 ? 1 : nb;
 }
 
-extern "C" int64_t cueq_sum_rows_workspace(int64_t rows, int64_t cols) { return sum_rows_blocks(rows) * cols * static_cast<int64_t>(sizeof(float)); }
+extern "C" int64_t cueq_sum_rows_workspace(int64_t rows, int64_t cols) { return sum_rows_blocks(rows, cols) * cols * static_cast<int64_t>(sizeof(float)); }
 
 // out[c] = sum_r in[r][c]   (float32 result, deterministic two-stage reduction)
 extern "C" int cueq_sum_rows(int32_t dtype, int64_t rows, int64_t cols, const void* in, float* out, void* workspace, int64_t workspace_bytes,
@@ -2323,7 +2337,7 @@ extern "C" int cueq_sum_rows(int32_t dtype, int64_t rows, int64_t cols, const vo
     return CUEQ_OK;
   }
   CUEQ_REQUIRE(in && workspace && workspace_bytes >= cueq_sum_rows_workspace(rows, cols), CUEQ_ERR_INVALID, "sum_rows: workspace too small");
-  const int64_t nb = sum_rows_blocks(rows);
+  const int64_t nb = sum_rows_blocks(rows, cols);
   const int64_t rpb = (rows + nb - 1) / nb;
   float* part = static_cast<float*>(workspace);
   const dim3 grid(static_cast<unsigned>((cols + 255) / 256), static_cast<unsigned>(nb));

@@ -458,8 +458,11 @@ class _FcFunction(torch.autograd.Function):
                     gw32 = torch.zeros(wd.numel(), dtype=torch.float32, device=dev)
                     for (K, N), (tab, dst) in tables["w"].items():
                         nparts = tab.shape[0]
-                        tiles = ((K + 127) // 128) * ((N + 127) // 128)
-                        chunks = max(1, min(-(-512 // (nparts * tiles)), Z // 256))
+                        if K <= 64 and N <= 64:  # one wavefront per 64 x 64 product: about two of them per SIMD
+                            chunks = max(1, min(-(-2048 // nparts), Z // 64))
+                        else:
+                            tiles = ((K + 127) // 128) * ((N + 127) // 128)
+                            chunks = max(1, min(-(-512 // (nparts * tiles)), Z // 256))
                         part = torch.empty(chunks, nparts * K * N, dtype=torch.float32, device=dev)
                         _lib.check(lib.cueq_gemm_table(code, _lib.F32, 1, 1, K, N, Z, x1d.data_ptr(), x1d.stride(0), H.data_ptr(),
                                                        plan.t_cols, part.data_ptr(), N, tab.data_ptr(), nparts, chunks, nparts * K * N,
