@@ -175,6 +175,24 @@ class _CallConfig:
         self.batch = int(batch)
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device: torch.device):
+    """Context that makes ``device`` current; nothing to do (and nothing to pay) when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
+
+
 def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor],
             indices: Sequence[torch.Tensor]) -> List[torch.Tensor]:
     nin, nout = plan.num_inputs, plan.num_outputs
@@ -182,7 +200,7 @@ def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor
     if device.type != "cuda":
         raise RuntimeError("uniform_1d runs on the GPU only; got tensors on " + str(device))
     lib = _lib.load()
-    with torch.cuda.device(device):
+    with _on_device(device):
         handle = plan.handle(device)
         bufs = (_lib.U1dBuffer * (nin + nout))()
         keep = []
@@ -192,16 +210,18 @@ def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor
                 raise ValueError(f"uniform_1d: unsupported dtype {t.dtype} for input {b}")
             if t.dim() != 2 or t.shape[1] != plan.width(b):
                 raise ValueError(f"uniform_1d: input {b} has shape {tuple(t.shape)}, expected (rows, {plan.width(b)})")
-            t = t.contiguous()
+            if not t.is_contiguous():
+                t = t.contiguous()
             keep.append(t)
-            bufs[b].data = t.data_ptr()
-            bufs[b].rows = t.shape[0]
-            bufs[b].dtype = _DTYPE_CODE[t.dtype]
-            bufs[b].batch_dim = cfg.modes[b]
+            bb = bufs[b]  # (one ctypes proxy per buffer, not one per field)
+            bb.data = t.data_ptr()
+            bb.rows = t.shape[0]
+            bb.dtype = _DTYPE_CODE[t.dtype]
+            bb.batch_dim = cfg.modes[b]
             if cfg.modes[b] == BATCH_DIM_INDEXED:
                 idx = indices[cfg.index_of[b]]
-                bufs[b].index = idx.data_ptr()
-                bufs[b].index_is_64 = 1 if idx.dtype == torch.int64 else 0
+                bb.index = idx.data_ptr()
+                bb.index_is_64 = 1 if idx.dtype == torch.int64 else 0
         outputs = []
         for o in range(nout):
             b = nin + o
@@ -209,21 +229,22 @@ def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor
             dtype = plan.math_dtype if src < 0 else inputs[src].dtype
             out = torch.empty((cfg.rows[b], plan.width(b)), dtype=dtype, device=device)
             outputs.append(out)
-            bufs[b].data = out.data_ptr()
-            bufs[b].rows = out.shape[0]
-            bufs[b].dtype = _DTYPE_CODE[dtype]
-            bufs[b].batch_dim = cfg.modes[b]
+            bb = bufs[b]
+            bb.data = out.data_ptr()
+            bb.rows = out.shape[0]
+            bb.dtype = _DTYPE_CODE[dtype]
+            bb.batch_dim = cfg.modes[b]
             if cfg.modes[b] == BATCH_DIM_INDEXED:
                 idx = indices[cfg.index_of[b]]
-                bufs[b].index = idx.data_ptr()
-                bufs[b].index_is_64 = 1 if idx.dtype == torch.int64 else 0
+                bb.index = idx.data_ptr()
+                bb.index_is_64 = 1 if idx.dtype == torch.int64 else 0
                 offsets, perm = _segment_csr(idx, cfg.rows[b])
                 keep += [offsets, perm]
-                bufs[b].csr_offsets = offsets.data_ptr()
-                bufs[b].csr_perm = perm.data_ptr()
+                bb.csr_offsets = offsets.data_ptr()
+                bb.csr_perm = perm.data_ptr()
         ws_bytes = lib.cueq_u1d_workspace_size(handle, bufs, cfg.batch)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes > 0 else None
-        stream = torch.cuda.current_stream(device).cuda_stream
+        stream = torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device())
         _lib.check(
             lib.cueq_u1d_run(handle, bufs, cfg.batch, ws.data_ptr() if ws is not None else None, ws_bytes, stream),
             f"cueq_u1d_run[{plan.name}]",
