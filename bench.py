@@ -32,8 +32,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # counters read for a 1 GiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Summary and commands:
 # profiles/channelwise_c128_l3_fp32_cfg2_hbm_traffic.txt.  Not measurable from inside this process.
 MEASURED_TRAFFIC_BYTES = {
-    ("c128_l3_bwd_float", 5000, 100_000): 4.314e9,
-    ("c128_l3_fwd_float", 5000, 100_000): 2.214e9,
+    ("c128_l3_bwd_float", 5000, 100_000): 4.270e9,
+    ("c128_l3_fwd_float", 5000, 100_000): 2.135e9,
 }
 
 
