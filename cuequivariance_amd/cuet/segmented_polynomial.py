@@ -105,7 +105,9 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
         self.BATCH_DIM_SHARED = u1d.BATCH_DIM_SHARED
         self.BATCH_DIM_BATCHED = u1d.BATCH_DIM_BATCHED
         self.BATCH_DIM_INDEXED = u1d.BATCH_DIM_INDEXED
-        self._plans: dict = {}
+        # both math types up front (host-side tables only; device plans are made at the first launch), so that a
+        # traced forward only reads this dictionary
+        self._plans: dict = {dt: u1d.Uniform1dPlan(self.tables, dt, name=self.name) for dt in (torch.float32, torch.float64)}
 
     def __reduce__(self):
         return (

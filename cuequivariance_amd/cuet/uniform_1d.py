@@ -19,6 +19,7 @@ from __future__ import annotations
 
 import ctypes as C
 import threading
+import weakref
 from collections import OrderedDict
 from typing import List, Optional, Sequence
 
@@ -45,6 +46,17 @@ _DTYPE_CODE = {
 }
 
 
+_traced_plans: dict = {}
+_traced_lock = threading.Lock()
+
+
+def _plan_by_id(plan_id: int) -> "Uniform1dPlan":
+    plan = _traced_plans[plan_id]()
+    if plan is None:
+        raise RuntimeError("uniform_1d: the module this graph was traced from no longer exists")
+    return plan
+
+
 class Uniform1dPlan:
     """Flat descriptor tables + lazily created device plans (one per GPU) + derived backward plans."""
 
@@ -57,6 +69,10 @@ class Uniform1dPlan:
         self._handles: dict[int, int] = {}
         self._backward: dict[tuple, "Uniform1dPlan"] = {}
         self._lock = threading.Lock()
+        # small integer under which a traced graph (torch.compile / export) names this plan
+        with _traced_lock:
+            self.traced_id = len(_traced_plans)
+            _traced_plans[self.traced_id] = weakref.ref(self)
 
     def __getattr__(self, item):
         # table fields (operand_extent, num_inputs, buffer_dim, ...) read through
@@ -292,6 +308,66 @@ class _Uniform1dFunction(torch.autograd.Function):
         return tuple(out)
 
 
+# ---------------------------------------------------------------------- traced execution
+# Under torch.compile / torch.export the launch is one opaque operator (the Python above it - resolving batch modes
+# and row counts - is traced as ordinary integer arithmetic); eager calls keep the lighter autograd.Function path.
+@torch.library.custom_op("cuequivariance_amd::u1d_launch", mutates_args=(), device_types="cuda")
+def _u1d_launch_op(plan_id: int, modes: List[int], index_of: List[int], rows: List[int], batch: int,
+                   tensors: List[torch.Tensor]) -> List[torch.Tensor]:
+    plan = _plan_by_id(plan_id)
+    nin = plan.num_inputs
+    outs = _launch(plan, _CallConfig(modes, index_of, rows, batch), [t.detach() for t in tensors[:nin]], tensors[nin:])
+    return list(outs)
+
+
+@_u1d_launch_op.register_fake
+def _u1d_launch_fake(plan_id, modes, index_of, rows, batch, tensors):
+    plan = _plan_by_id(plan_id)
+    nin = plan.num_inputs
+    outs = []
+    for o in range(plan.num_outputs):
+        src = plan.dtypes[nin + o]
+        outs.append(tensors[0].new_empty((rows[nin + o], plan.width(nin + o)), dtype=plan.math_dtype if src < 0 else tensors[src].dtype))
+    return outs
+
+
+def _u1d_setup_context(ctx, inputs, output):
+    plan_id, modes, index_of, rows, batch, tensors = inputs
+    ctx.meta = (plan_id, tuple(modes), tuple(index_of), tuple(rows), batch)
+    ctx.save_for_backward(*tensors)
+
+
+def _u1d_backward(ctx, grad_outputs):
+    plan_id, modes, index_of, rows, batch = ctx.meta
+    plan = _plan_by_id(plan_id)
+    nin = plan.num_inputs
+    tensors = ctx.saved_tensors
+    inputs, indices = tensors[:nin], tensors[nin:]
+    flags = ctx.needs_input_grad[5]
+    if isinstance(flags, bool):
+        flags = [flags] * len(tensors)
+    needs = tuple(bool(f) for f in flags[:nin])
+    grads: List[Optional[torch.Tensor]] = [None] * len(tensors)
+    if any(needs):
+        bplan = plan.backward_plan(needs)
+        cots = []
+        for o, g in enumerate(grad_outputs):
+            if g is None:
+                src = plan.dtypes[nin + o]
+                g = torch.zeros((rows[nin + o], plan.width(nin + o)), device=inputs[0].device,
+                                dtype=plan.math_dtype if src < 0 else inputs[src].dtype)
+            cots.append(g)
+        flagged = [i for i, n in enumerate(needs) if n]
+        got = _u1d_launch_op(bplan.traced_id, list(modes) + [modes[i] for i in flagged], list(index_of) + [index_of[i] for i in flagged],
+                             list(rows) + [rows[i] for i in flagged], batch, [*inputs, *cots, *indices])
+        for g, i in zip(got, flagged):
+            grads[i] = g
+    return None, None, None, None, None, grads
+
+
+torch.library.register_autograd("cuequivariance_amd::u1d_launch", _u1d_backward, setup_context=_u1d_setup_context)
+
+
 def run_plan(plan: Uniform1dPlan, batch_dim: Sequence[int], index_buffer: Sequence[int], batch_size: int,
              num_index: int, tensors: Sequence[torch.Tensor]) -> List[torch.Tensor]:
     """Resolve AUTO batch dims and sizes (same rules as the reference op's caller) and execute."""
@@ -336,6 +412,8 @@ def run_plan(plan: Uniform1dPlan, batch_dim: Sequence[int], index_buffer: Sequen
         else:
             modes[b] = BATCH_DIM_BATCHED
             rows[b] = batch
+    if torch.compiler.is_compiling():
+        return list(_u1d_launch_op(plan.traced_id, modes, list(index_buffer[: nin + nout]), rows, batch, [*inputs, *indices]))
     cfg = _CallConfig(modes, list(index_buffer[: nin + nout]), rows, batch)
     outs = _Uniform1dFunction.apply(plan, cfg, num_index, *inputs, *indices)
     return list(outs)
