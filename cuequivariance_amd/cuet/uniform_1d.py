@@ -47,6 +47,7 @@ _DTYPE_CODE = {
 
 
 _traced_plans: dict = {}
+_PLAIN_TENSORS = (torch.Tensor, torch.nn.Parameter)
 _traced_lock = threading.Lock()
 
 
@@ -412,7 +413,8 @@ def run_plan(plan: Uniform1dPlan, batch_dim: Sequence[int], index_buffer: Sequen
         else:
             modes[b] = BATCH_DIM_BATCHED
             rows[b] = batch
-    if torch.compiler.is_compiling():
+    # (traced: under Dynamo, or called with the tracer's tensor subclasses when a composite operator is decomposed)
+    if torch.compiler.is_compiling() or (inputs and type(inputs[0]) not in _PLAIN_TENSORS):
         return list(_u1d_launch_op(plan.traced_id, modes, list(index_buffer[: nin + nout]), rows, batch, [*inputs, *indices]))
     cfg = _CallConfig(modes, list(index_buffer[: nin + nout]), rows, batch)
     outs = _Uniform1dFunction.apply(plan, cfg, num_index, *inputs, *indices)

@@ -80,6 +80,36 @@ def test_uniform_1d_through_torch_ops(device, dtype):
 
 
 @pytest.mark.gpu
+def test_uniform_1d_op_under_torch_compile(device):
+    """The registered operator inside ``torch.compile(fullgraph=True)``: it is decomposed into the opaque launch operator;
+    forward equals eager bit for bit (same kernels), and so do the gradients of this batched (atomic-free) case."""
+    from cuequivariance_amd import ops_torch
+
+    ops_torch.register_ops()
+    C = ops_torch.uniform_1d
+    poly = channelwise_poly()
+    t = U1dTables.from_polynomial(poly.flatten_coefficient_modes().squeeze_modes())
+    g = torch.Generator(device=device).manual_seed(6)
+    Z = 64
+    w = torch.randn(Z, t.width(0), device=device, generator=g, requires_grad=True)
+    x1 = torch.randn(Z, t.width(1), device=device, generator=g, requires_grad=True)
+    x2 = torch.randn(Z, t.width(2), device=device, generator=g)
+
+    def f(w, x1, x2):
+        return torch.ops.cuequivariance.uniform_1d(
+            "seam", torch.float32, t.operand_extent, t.num_inputs, t.num_outputs, 0, list(t.buffer_dim),
+            list(t.buffer_num_segments), [C.BATCH_DIM_AUTO] * 4, [-1] * 4, list(t.dtypes), len(t.num_operands),
+            list(t.num_operands), list(t.operations), list(t.num_paths), list(t.path_indices_start),
+            list(t.path_coefficients_start), list(t.path_indices), list(t.path_coefficients), C.BATCH_DIM_AUTO, [w, x1, x2])[0]
+
+    ref = f(w, x1, x2)
+    out = torch.compile(f, fullgraph=True, backend="aot_eager", dynamic=False)(w, x1, x2)
+    assert torch.equal(out, ref)
+    for a, b in zip(torch.autograd.grad(out.sum(), [w, x1]), torch.autograd.grad(ref.sum(), [w, x1])):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
 def test_segmented_transpose_with_frontend_info(device, dtype):
     """``segmented_transpose(x, info, True)`` with the int table of ``primitives/transpose.py:150-168``: every (u, v)
