@@ -1173,6 +1173,115 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// sigmoid(W1 X^T + b1) * (W2 X^T + b2) * mask for 2-byte types with W1, W2 (C rows) and the biases resident in LDS, the
+// forward twin of the kernel above: rows c of the result are weight rows, columns m are rows of X; one persistent
+// block per CU, every wavefront walks tiles of 64 columns m on its own (two 32-column MFMA tiles sharing each weight
+// fragment).  Results leave as 4-byte column pairs: neighbouring lanes swap halves (even lane: row 2 j for columns
+// m, m + 1; odd lane: row 2 j + 1 for m - 1, m), so N and ldc must be even.
+// ------------------------------------------------------------------------------------------------
+template <int KT>
+__global__ void __launch_bounds__(512, 2)
+    dual_gate_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X, int64_t ldx,
+                         const uint16_t* __restrict__ bias1, const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask,
+                         uint16_t* __restrict__ out, int64_t ldc, int C, int M) {
+  using TI = uint16_t;
+  constexpr int ES = 2, EPV = 8;
+  constexpr int K = 32 * KT, ROWB = K * ES, NS = ROWB / 64, VPR = ROWB / 16;
+  constexpr bool SWZ = KT == 4;  // (same layout of the weight rows as gate_bwd_input_res_kernel)
+  constexpr int WSTR = SWZ ? ROWB : ROWB + 16;
+  constexpr int NTH = 512, NWAVES = NTH / 64;
+  auto swz = [](int row) -> int { return SWZ ? (((row & 3) << 2) | ((row >> 2) & 3)) : 0; };
+  extern __shared__ __align__(16) char dgr_dsm[];
+  char* sw1 = dgr_dsm;
+  char* sw2 = dgr_dsm + C * WSTR;
+  float* sb = reinterpret_cast<float*>(dgr_dsm + 2 * C * WSTR);  // bias1[C], bias2[C]
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+
+  for (int e = tid; e < C * VPR; e += NTH) {
+    const int r = e / VPR, part = e % VPR;
+    const int po = (part ^ swz(r)) << 4;
+    *reinterpret_cast<uint4*>(sw1 + r * WSTR + po) = *reinterpret_cast<const uint4*>(W1 + static_cast<int64_t>(r) * ldw + part * EPV);
+    *reinterpret_cast<uint4*>(sw2 + r * WSTR + po) = *reinterpret_cast<const uint4*>(W2 + static_cast<int64_t>(r) * ldw + part * EPV);
+  }
+  for (int i = tid; i < C; i += NTH) {
+    sb[i] = bias1 ? tri_load(bias1, i) : 0.f;
+    sb[C + i] = bias2 ? tri_load(bias2, i) : 0.f;
+  }
+  __syncthreads();
+
+  const int nchunks = C / 32;
+  const int64_t ntiles = (static_cast<int64_t>(M) + 63) / 64;
+  const int64_t tstep = static_cast<int64_t>(gridDim.x) * NWAVES;
+  const uint32_t pair_sel = (lane & 1) ? 0x03020706u : 0x05040100u;
+  for (int64_t tile = static_cast<int64_t>(blockIdx.x) * NWAVES + wave; tile < ntiles; tile += tstep) {
+    uint4 xf[2][NS][2];
+    float mk[2];
+    int mcol[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      mcol[t] = static_cast<int>(tile * 64) + 32 * t + c;
+      const int mld = min(mcol[t], M - 1);
+#pragma unroll
+      for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+          xf[t][s2][q] = *reinterpret_cast<const uint4*>(X + static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES);
+      mk[t] = mask ? tri_load(mask, mld) : 1.0f;
+    }
+    for (int ci = 0; ci < nchunks; ++ci) {
+      const int c0 = ci * 32;
+      floatx16 au[2], av[2];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const float4 b1 = *reinterpret_cast<const float4*>(sb + c0 + 8 * a + 4 * h);
+        const float4 b2 = *reinterpret_cast<const float4*>(sb + C + c0 + 8 * a + 4 * h);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          au[t][4 * a] = b1.x; au[t][4 * a + 1] = b1.y; au[t][4 * a + 2] = b1.z; au[t][4 * a + 3] = b1.w;
+          av[t][4 * a] = b2.x; av[t][4 * a + 1] = b2.y; av[t][4 * a + 2] = b2.z; av[t][4 * a + 3] = b2.w;
+        }
+      }
+      const int wrow = (c0 + c) * WSTR;
+#pragma unroll
+      for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const int wo = wrow + ((((2 * h + q) ^ swz(c)) << 4) ^ (s2 << 6));
+          const uint4 a1 = *reinterpret_cast<const uint4*>(sw1 + wo);
+          const uint4 a2 = *reinterpret_cast<const uint4*>(sw2 + wo);
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            mma_step<TI>(au[t], a1, xf[t][s2][q]);
+            mma_step<TI>(av[t], a2, xf[t][s2][q]);
+          }
+        }
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          float g[4];
+#pragma unroll
+          for (int b = 0; b < 4; ++b) {
+            const int v = 4 * a + b;
+            g[b] = __builtin_amdgcn_rcpf(1.0f + __expf(-au[t][v])) * av[t][v] * mk[t];
+          }
+          const uint32_t own[2] = {pack_bf16(g[0], g[1]), pack_bf16(g[2], g[3])};
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(own[j]), 0xB1, 0xF, 0xF, true));
+            const uint32_t word = __builtin_amdgcn_perm(other, own[j], pair_sel);
+            if (mcol[t] < M) {
+              const int row = c0 + 8 * a + 4 * h + 2 * j + (lane & 1);
+              *reinterpret_cast<uint32_t*>(out + static_cast<int64_t>(row) * ldc + (mcol[t] & ~1)) = word;
+            }
+          }
+        }
+    }
+  }
+}
+
 // any shape / alignment / operand order: one thread per output element (rs*: stride between rows of the operand,
 // ks*: stride along the contraction)
 template <typename TI, typename TO>
@@ -1965,6 +2074,24 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
   const bool share = B2 == nullptr || B2 == B1;
   const int vec_out = (reinterpret_cast<uintptr_t>(out1) % 16 == 0 && ldc % epv == 0) ? 1 : 0;
   KernelTimer timer(backward ? "dual_gate_bwd" : "dual_gate_fwd", stream);
+  // forward with one shared right operand, biases along the rows and the mask along the columns, in a 2-byte type:
+  // the left operands (the weights, M rows) stay resident in LDS when they fit
+  if (dtype == CUEQ_BF16 && !backward && share && (!(bias1 || bias2) || bias_axis == 0) && (!mask || mask_axis == 1) && K % 32 == 0 && K <= 128 &&
+      M % 32 == 0 && N % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(out1) % 4 == 0 && N >= 4096) {
+    const size_t lds = static_cast<size_t>(2 * M * (K == 128 ? 2 * K : 2 * K + 16) + 8 * M);
+    if (lds <= 160 * 1024) {
+      const int64_t ntiles = (N + 63) / 64;
+      int64_t gx2 = (ntiles + 7) / 8;
+      if (gx2 > device_cus()) gx2 = device_cus();
+#define DGR(KT) do { auto kfn = dual_gate_res_kernel<KT>; \
+        CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx2)), dim3(512), lds, stream, static_cast<const uint16_t*>(A1), static_cast<const uint16_t*>(A2), lda, static_cast<const uint16_t*>(B1), ldb, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<uint16_t*>(out1), ldc, static_cast<int>(M), static_cast<int>(N)); } while (0)
+      switch (K / 32) { case 1: DGR(1); break; case 2: DGR(2); break; case 3: DGR(3); break; default: DGR(4); break; }
+#undef DGR
+      CUEQ_CHECK_HIP(hipGetLastError());
+      return CUEQ_OK;
+    }
+  }
 #define DG(TI, BW, SH) hipLaunchKernelGGL((dual_gate_kernel<TI, BW, SH>), grid, dim3(512), 0, stream, static_cast<const TI*>(A1), static_cast<const TI*>(A2), lda, static_cast<const TI*>(B1), static_cast<const TI*>(B2), ldb, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), bias_axis, static_cast<const TI*>(mask), mask_axis, static_cast<const TI*>(dC), static_cast<TI*>(out1), static_cast<TI*>(out2), ldc, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), vec_out)
 #define DG_T(TI) do { if (backward) { if (share) DG(TI, true, true); else DG(TI, true, false); } else { if (share) DG(TI, false, true); else DG(TI, false, false); } } while (0)
   TRI_DISPATCH(dtype, DG_T(float), DG_T(uint16_t));
