@@ -241,3 +241,29 @@ def test_gate_bwd_input_many_tiles(device, dtype, split, M):
         assert rel_err(g2, want2) <= tol, rel_err(g2, want2)
     layout = (lambda t: t) if not split else (lambda t: t.T)
     assert rel_err(gU, layout(dU)) <= tol and rel_err(gV, layout(dV)) <= tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("N", [64 * 2048 + 64 * 5 + 2, 4096 + 34])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_dual_gate_many_column_tiles(device, dtype, N, with_bias):
+    """The fused forward gate with a shared right operand on more 64-column tiles than one launch holds wavefronts for
+    (each wavefront then walks several tiles; the last tile is partial), against sigmoid(W1 X^T + b1) (W2 X^T + b2) mask
+    written with torch in float64 on the rounded inputs."""
+    from cuequivariance_amd.cuet import triangle as T
+
+    g = torch.Generator().manual_seed(17)
+    C, K = 96, 64
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    W1, W2, X = (r(C, K) / 8).to(dtype), (r(C, K) / 8).to(dtype), r(N, K).to(dtype)
+    b1, b2 = (r(C).to(dtype), r(C).to(dtype)) if with_bias else (None, None)
+    mask = (torch.rand(N, generator=g) > 0.2).to(dtype)
+    d = lambda t: t.double()
+    U = d(W1) @ d(X).T + (d(b1)[:, None] if with_bias else 0)
+    V = d(W2) @ d(X).T + (d(b2)[:, None] if with_bias else 0)
+    want = torch.sigmoid(U) * V * d(mask)[None, :]
+    dev = lambda t: None if t is None else t.to(device)
+    got = T.dual_gate_fwd(dev(W1), dev(W2), dev(X), None, dev(b1), dev(b2), 0, dev(mask), 1)
+    assert got.shape == (C, N) and got.dtype == dtype
+    assert rel_err(got, want) <= TOL[dtype], rel_err(got, want)
