@@ -113,6 +113,11 @@ class Uniform1dPlan:
 
     def __del__(self):
         try:
+            with _traced_lock:
+                _traced_plans.pop(self.traced_id, None)
+        except Exception:
+            pass
+        try:
             lib = _lib.load()
             for h in self._handles.values():
                 lib.cueq_u1d_plan_destroy(h)
