@@ -474,6 +474,16 @@ class Irreps:
     def __setattr__(self, *a):  # immutable
         raise AttributeError("Irreps is immutable")
 
+    # immutable value: copies are the object itself, pickles rebuild it from its parts
+    def __copy__(self):
+        return self
+
+    def __deepcopy__(self, memo):
+        return self
+
+    def __reduce__(self):
+        return (Irreps, (self.irrep_class, self._mulirreps))
+
     def __len__(self):
         return len(self._mulirreps)
 

@@ -5,6 +5,7 @@ from .segmented_polynomial import SegmentedPolynomial
 from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction, SphericalHarmonics
 from .uniform_1d import uniform_1d
 from .triangle import triangle_multiplicative_update, TriMulPrecision
+from . import layers
 
 __all__ = [
     "TransposeSegments",
@@ -18,4 +19,5 @@ __all__ = [
     "uniform_1d",
     "triangle_multiplicative_update",
     "TriMulPrecision",
+    "layers",
 ]

@@ -15,8 +15,9 @@ kernels (``uniform_1d`` for the channel-wise product, the dense executor ``fused
 
 from __future__ import annotations
 
+import math
 import warnings
-from typing import Dict, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -62,6 +63,32 @@ def _method_from_fallback(method, use_fallback, default: str) -> str:
     if use_fallback:
         raise ValueError("use_fallback=True asks for the PyTorch executor, which this engine does not have")
     return default
+
+
+class _FlattenedUniform(torch.nn.Module):
+    """The same polynomial with every mode but the output's last one flattened away (and that one split down to a
+    common extent), which the uniform-1d kernels take.  The dense executor wants one weight row shared by the batch (or
+    rows sorted by class); weights per sample or picked by an arbitrary class index are ordinary batched / indexed
+    operands here.  Built on first use."""
+
+    def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype):
+        super().__init__()
+        self._polynomial, self._math_dtype = polynomial, math_dtype
+        self.f = None
+
+    def forward(self, inputs: List[torch.Tensor], input_indices: Optional[Dict[int, torch.Tensor]] = None,
+                output_shapes: Optional[Dict[int, torch.Tensor]] = None, output_indices: Optional[Dict[int, torch.Tensor]] = None):
+        if self.f is None:
+            q = self._polynomial.flatten_coefficient_modes()
+            stp = q.operations[0][1]
+            keep = stp.subscripts.operands[-1][-1]
+            q = q.flatten_modes([m for m in stp.subscripts.modes() if m != keep])
+            extents = sorted(q.operations[0][1].get_dims(keep))
+            if len(extents) > 1:
+                q = q.split_mode(keep, math.gcd(*extents))
+            self.f = SegmentedPolynomial(q, method="uniform_1d", math_dtype=self._math_dtype)
+        return self.f(inputs, input_indices=input_indices or {}, output_shapes=output_shapes or {},
+                      output_indices=output_indices or {})
 
 
 class ChannelWiseTensorProduct(torch.nn.Module):
@@ -216,6 +243,7 @@ class FullyConnectedTensorProduct(torch.nn.Module):
         )
         self.method = _method_from_fallback(method, use_fallback, "fused_tp")
         self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+        self.f_per_sample = _FlattenedUniform(e.polynomial, math_dtype)  # weights of shape (batch, weight_numel)
 
     def extra_repr(self) -> str:
         return (
@@ -223,7 +251,11 @@ class FullyConnectedTensorProduct(torch.nn.Module):
             f"weight_numel={self.weight_numel}"
         )
 
-    def forward(self, x1: torch.Tensor, x2: torch.Tensor, weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x1: torch.Tensor, x2: torch.Tensor, weight: Optional[torch.Tensor] = None, *,
+                indices_1: Optional[torch.Tensor] = None, indices_out: Optional[torch.Tensor] = None,
+                size_out: Optional[int] = None) -> torch.Tensor:
+        """``indices_1`` (rows of ``x1`` per batch element) and ``indices_out`` / ``size_out`` (output row per batch
+        element, summed) are extensions over the reference's signature: gather and scatter-sum inside the kernel."""
         x1 = self.transpose_in1(x1)
         x2 = self.transpose_in2(x2)
         if self.weight is not None:
@@ -232,6 +264,16 @@ class FullyConnectedTensorProduct(torch.nn.Module):
             weight = self.weight
         elif weight is None:
             raise ValueError("Internal weights are not used, weight should not be None")
+        if indices_1 is not None or indices_out is not None:
+            if indices_out is not None and size_out is None:
+                raise ValueError("size_out should be provided if indices_out is provided")
+            out = self.f_per_sample(
+                [weight, x1, x2], {} if indices_1 is None else {1: indices_1},
+                {} if indices_out is None else {0: torch.empty(size_out, 1, device="meta")},
+                {} if indices_out is None else {0: indices_out})
+            return self.transpose_out(out[0])
+        if weight.shape[0] != 1:
+            return self.transpose_out(self.f_per_sample([weight, x1, x2])[0])
         return self.transpose_out(self.f([weight, x1, x2])[0])
 
 
@@ -285,6 +327,8 @@ class Linear(torch.nn.Module):
         )
         self.method = _method_from_fallback(method, use_fallback, "fused_tp")
         self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+        # weights per sample, or per class with an index in any order (sorted classes: method="indexed_linear")
+        self.f_per_sample = _FlattenedUniform(e.polynomial, math_dtype)
 
     def extra_repr(self) -> str:
         return (
@@ -306,7 +350,10 @@ class Linear(torch.nn.Module):
             input_indices[0] = weight_indices
         if weight is None:
             raise ValueError("Weights should not be None")
-        out = self.f([weight, self.transpose_in(x)], input_indices=input_indices)
+        if self.method != "indexed_linear" and (input_indices or weight.shape[0] != 1):
+            out = self.f_per_sample([weight, self.transpose_in(x)], input_indices)
+        else:
+            out = self.f([weight, self.transpose_in(x)], input_indices=input_indices)
         return self.transpose_out(out[0])
 
 

@@ -172,3 +172,52 @@ def test_indexed_linear_matches_oracle(device, dtype, irreps, classes, sizes):
     if Z > 2:
         with pytest.raises(AssertionError):
             m(xg, wg, idx.flip(0).to(device))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_weights_per_sample_and_unsorted_classes(device, dtype):
+    """``shared_weights=False`` (one weight row per sample) for the fully connected product and the linear map, and
+    ``weight_classes`` with an index in arbitrary order: served by the uniform-1d kernels on the flattened descriptor;
+    against the CPU oracle on the unflattened descriptor (reference behaviour:
+    ``cuequivariance_torch/operations/tp_fully_connected.py:30-207``, ``operations/linear.py:150-190``)."""
+    from cuequivariance_amd import cuet
+
+    g = torch.Generator().manual_seed(23)
+    Z = 77
+    tol = 1e-12 if dtype == torch.float64 else 1e-5
+    i1, i2, io = cue.Irreps("O3", "6x0e+4x1o"), cue.Irreps("O3", "0e+1o"), cue.Irreps("O3", "6x0e+4x1o+2x2e")
+    fc = cuet.FullyConnectedTensorProduct(i1, i2, io, layout=cue.ir_mul, shared_weights=False, device=device, dtype=dtype)
+    x1 = torch.randn(Z, i1.dim, generator=g, dtype=torch.float64).to(dtype)
+    x2 = torch.randn(Z, i2.dim, generator=g, dtype=torch.float64).to(dtype)
+    w = torch.randn(Z, fc.weight_numel, generator=g, dtype=torch.float64).to(dtype)
+    spec = spec_from_polynomial(cue.descriptors.fully_connected_tensor_product(i1, i2, io).polynomial)
+    a = [t.clone().requires_grad_(True) for t in (w, x1, x2)]
+    ref = naive_segmented_polynomial(spec, a)[0]
+    cot = torch.randn(ref.shape, generator=g, dtype=torch.float64).to(dtype)
+    ref_grads = torch.autograd.grad(ref, a, cot)
+    b = [t.clone().to(device).requires_grad_(True) for t in (w, x1, x2)]
+    out = fc(b[1], b[2], b[0])
+    grads = torch.autograd.grad(out, b, cot.to(device))
+    assert rel_err(out, ref) <= tol, "fc per-sample weights"
+    for p, q, name in zip(ref_grads, grads, ("dw", "dx1", "dx2")):
+        assert rel_err(q, p) <= tol, name
+
+    lin = cuet.Linear(i1, io, layout=cue.ir_mul, weight_classes=4, device=device, dtype=dtype)
+    idx = torch.randint(0, 4, (Z,), generator=g, dtype=torch.int32)  # not sorted
+    spec = spec_from_polynomial(cue.descriptors.linear(i1, io).polynomial)
+    wl = lin.weight.detach().cpu().clone().requires_grad_(True)
+    xl = x1.clone().requires_grad_(True)
+    ref = naive_segmented_polynomial(spec, [wl, xl], {0: idx})[0]
+    cot = torch.randn(ref.shape, generator=g, dtype=torch.float64).to(dtype)
+    ref_grads = torch.autograd.grad(ref, [wl, xl], cot)
+    xg = x1.clone().to(device).requires_grad_(True)
+    out = lin(xg, weight_indices=idx.to(device))
+    grads = torch.autograd.grad(out, [lin.weight, xg], cot.to(device))
+    assert rel_err(out, ref) <= tol, "linear with unsorted classes"
+    for p, q, name in zip(ref_grads, grads, ("dw", "dx")):
+        assert rel_err(q, p) <= tol, name
+
+    lin2 = cuet.Linear(i1, io, layout=cue.ir_mul, shared_weights=False, device=device, dtype=dtype)
+    wz = torch.randn(Z, lin2.weight_numel, generator=g, dtype=torch.float64).to(dtype)
+    ref = naive_segmented_polynomial(spec, [wz, x1])[0]
+    assert rel_err(lin2(x1.to(device), wz.to(device)), ref) <= tol, "linear per-sample weights"
