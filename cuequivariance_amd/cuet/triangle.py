@@ -21,7 +21,7 @@ from __future__ import annotations
 
 import enum
 import math
-from typing import Optional
+from typing import List, Optional
 
 import torch
 
@@ -302,10 +302,11 @@ def gemm_long_k(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
 # ---------------------------------------------------------------------------------------------
 # autograd
 # ---------------------------------------------------------------------------------------------
-class _TriMul(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, x, mask, nin_w, nin_b, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, nout_b, p_out_w, p_out_b, g_out_w, g_out_b,
+def _trimul_fwd(x, mask, nin_w, nin_b, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, nout_b, p_out_w, p_out_b, g_out_w, g_out_b,
                 outgoing: bool, eps: float):
+    """Forward of the update on ``x (B, N, N, D)``: returns the output, the tensors the backward reads (inputs first,
+    then the eight computed ones) and the extents."""
+    if True:
         T = x.dtype
         Bsz, N, _, D = x.shape
         M = Bsz * N * N
@@ -327,20 +328,20 @@ class _TriMul(torch.autograd.Function):
         else:
             y, mean2, rstd2 = layer_norm_fwd(transpose(t2), nout_w, nout_b, eps)
         out = dual_gate_fwd(xh, y, g_out_w, p_out_w, g_out_b, p_out_b, 1, None, 0)  # (M, Do)
-        ctx.save_for_backward(x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
-                              xh, mean1, rstd1, ab, t2, mean2, rstd2, y)
-        ctx.outgoing, ctx.dims = outgoing, (Bsz, N, D, Do)
-        ctx.has = (nin_w is not None, nin_b is not None, nout_w is not None, nout_b is not None)
-        return out.view(Bsz, N, N, Do)
+        saved = (x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
+                 xh, mean1, rstd1, ab, t2, mean2, rstd2, y)
+        has = (nin_w is not None, nin_b is not None, nout_w is not None, nout_b is not None)
+        return out.view(Bsz, N, N, Do), saved, (Bsz, N, D, Do), has
 
-    @staticmethod
-    def backward(ctx, dout):
+
+def _trimul_bwd(saved, dims, has, outgoing: bool, need, dout):
+    """Gradients for the 16 arguments of :func:`_trimul_fwd` (``need[k]``: whether argument ``k`` wants one)."""
+    if True:
         (x2, mflat, nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b, g_out_w, g_out_b,
-         xh, mean1, rstd1, ab, t2, mean2, rstd2, y) = ctx.saved_tensors
-        Bsz, N, D, Do = ctx.dims
+         xh, mean1, rstd1, ab, t2, mean2, rstd2, y) = saved
+        Bsz, N, D, Do = dims
         M = Bsz * N * N
         T = x2.dtype
-        need = ctx.needs_input_grad
         dout = dout.contiguous().view(M, Do).to(T)
 
         # output gate
@@ -365,7 +366,7 @@ class _TriMul(torch.autograd.Function):
             d_p_out_b = sum_rows(dv2).to(p_out_b.dtype)
 
         # LayerNorm across d
-        affine_out = (ctx.has[2] and need[8]) or (ctx.has[3] and need[9])
+        affine_out = (has[2] and need[8]) or (has[3] and need[9])
         if _ln_t_ok(t2):
             dt, d_nout_w, d_nout_b = layer_norm_t_bwd(dy, t2, mean2, rstd2, nout_w, affine_out)  # (D, M)
         else:
@@ -379,7 +380,7 @@ class _TriMul(torch.autograd.Function):
         dab = torch.empty_like(ab)
         da = dab[:D].view(D * Bsz, N, N)
         db = dab[D:].view(D * Bsz, N, N)
-        if ctx.outgoing:  # t = a b^T
+        if outgoing:  # t = a b^T
             gemm_nt(dt, b, T, out=da, trans_b=True)  # da[i, k] = sum_j dt[i, j] b[j, k]
             gemm_nt(dt, a, T, out=db, trans_a=True, trans_b=True)  # db[j, k] = sum_i dt[i, j] a[i, k]
         else:  # t = a^T b
@@ -405,15 +406,94 @@ class _TriMul(torch.autograd.Function):
             d_p_in_b = sum_cols(dv1).to(p_in_b.dtype)
 
         # input LayerNorm
-        affine_in = (ctx.has[0] and need[2]) or (ctx.has[1] and need[3])
+        affine_in = (has[0] and need[2]) or (has[1] and need[3])
         dx, d_nin_w, d_nin_b = layer_norm_bwd(dxh, x2, mean1, rstd1, nin_w, affine_in)
         dx = dx.view(Bsz, N, N, D) if need[0] else None
 
         def cast(g, like, have):
             return g.to(like.dtype) if (g is not None and have) else None
 
-        return (dx, None, cast(d_nin_w, x2, ctx.has[0]), cast(d_nin_b, x2, ctx.has[1]), d_p_in_w, d_p_in_b, d_g_in_w, d_g_in_b,
-                cast(d_nout_w, x2, ctx.has[2]), cast(d_nout_b, x2, ctx.has[3]), d_p_out_w, d_p_out_b, d_g_out_w, d_g_out_b, None, None)
+        return (dx, None, cast(d_nin_w, x2, has[0]), cast(d_nin_b, x2, has[1]), d_p_in_w, d_p_in_b, d_g_in_w, d_g_in_b,
+                cast(d_nout_w, x2, has[2]), cast(d_nout_b, x2, has[3]), d_p_out_w, d_p_out_b, d_g_out_w, d_g_out_b, None, None)
+
+
+class _TriMul(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, *args):
+        out, saved, dims, has = _trimul_fwd(*args)
+        ctx.save_for_backward(*saved)
+        ctx.outgoing, ctx.dims, ctx.has = args[14], dims, has
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        return _trimul_bwd(ctx.saved_tensors, ctx.dims, ctx.has, ctx.outgoing, ctx.needs_input_grad, dout)
+
+
+# ---------------------------------------------------------------------- traced execution (torch.compile / export)
+# Two opaque operators, forward and backward, around the same two functions.  Optional tensors travel as empty
+# placeholders plus a presence list (operator schemas have no optional entries inside tensor lists).
+def _placeholders(ref: torch.Tensor, tensors):
+    return [ref.new_empty(0) if t is None else t for t in tensors], [t is not None for t in tensors]
+
+
+@torch.library.custom_op("cuequivariance_amd::trimul_fwd", mutates_args=(), device_types="cuda")
+def _trimul_fwd_op(x: torch.Tensor, tensors: List[torch.Tensor], present: List[bool], outgoing: bool, eps: float) -> List[torch.Tensor]:
+    args = [t if p else None for t, p in zip(tensors, present)]  # mask, then the 12 weights
+    out, saved, _, _ = _trimul_fwd(x, *args, outgoing, eps)
+    return [out, *saved[12:]]  # + xh, mean1, rstd1, ab, t2, mean2, rstd2, y
+
+
+@_trimul_fwd_op.register_fake
+def _trimul_fwd_fake(x, tensors, present, outgoing, eps):
+    Bsz, N, _, D = x.shape
+    M = Bsz * N * N
+    Do = tensors[9].shape[0]  # p_out_weight
+    f32 = dict(dtype=torch.float32)
+    return [x.new_empty(Bsz, N, N, Do), x.new_empty(M, D), x.new_empty(M, **f32), x.new_empty(M, **f32), x.new_empty(2 * D, M),
+            x.new_empty(D, M), x.new_empty(M, **f32), x.new_empty(M, **f32), x.new_empty(M, D)]
+
+
+@torch.library.custom_op("cuequivariance_amd::trimul_bwd", mutates_args=(), device_types="cuda")
+def _trimul_bwd_op(dout: torch.Tensor, x: torch.Tensor, tensors: List[torch.Tensor], computed: List[torch.Tensor], present: List[bool],
+                   need: List[bool], outgoing: bool) -> List[torch.Tensor]:
+    mask, nin_w, nin_b, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, nout_b, p_out_w, p_out_b, g_out_w, g_out_b = [
+        t if p else None for t, p in zip(tensors, present)]
+    Bsz, N, _, D = x.shape
+    M = Bsz * N * N
+    saved = (x.reshape(M, D), None if mask is None else mask.reshape(M), nin_w, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, p_out_w, p_out_b,
+             g_out_w, g_out_b, *computed)
+    has = (nin_w is not None, nin_b is not None, nout_w is not None, nout_b is not None)
+    grads = _trimul_bwd(saved, (Bsz, N, D, p_out_w.shape[0]), has, outgoing, [*need, False, False], dout)
+    return [x.new_empty(0) if (g is None or not n) else g.contiguous() for g, n in zip(grads[:14], need)]
+
+
+@_trimul_bwd_op.register_fake
+def _trimul_bwd_fake(dout, x, tensors, computed, present, need, outgoing):
+    like = [x, *tensors]
+    return [torch.empty_like(t) if (n and (k == 0 or present[k - 1]) and k != 1) else x.new_empty(0) for k, (t, n) in enumerate(zip(like, need))]
+
+
+def _trimul_setup_context(ctx, inputs, output):
+    x, tensors, present, outgoing, eps = inputs
+    ctx.present, ctx.outgoing, ctx.ntensors = list(present), outgoing, len(tensors)
+    ctx.save_for_backward(x, *tensors, *output[1:])
+
+
+def _trimul_autograd(ctx, grads):
+    saved = ctx.saved_tensors
+    x, tensors, computed = saved[0], list(saved[1: 1 + ctx.ntensors]), list(saved[1 + ctx.ntensors:])
+    flags = ctx.needs_input_grad[1]
+    if isinstance(flags, bool):
+        flags = [flags] * len(tensors)
+    need = [bool(ctx.needs_input_grad[0]), *[bool(f) for f in flags]]
+    got = _trimul_bwd_op(grads[0], x, tensors, computed, ctx.present, need, ctx.outgoing)
+    pick = [g if g.numel() > 0 else None for g in got]
+    return pick[0], pick[1:], None, None, None
+
+
+torch.library.register_autograd("cuequivariance_amd::trimul_fwd", _trimul_autograd, setup_context=_trimul_setup_context)
+
 
 
 def _lecun_normal(shape, device, dtype) -> torch.Tensor:
@@ -509,5 +589,9 @@ def triangle_multiplicative_update(
         Bsz *= s
     xf = x.reshape(Bsz, N, N, D).contiguous()
     mf = None if mask is None else mask.reshape(Bsz, N, N).to(T).contiguous()
-    out = _TriMul.apply(xf, mf, *args, direction == "outgoing", float(eps))
+    if torch.compiler.is_compiling() or type(xf) not in (torch.Tensor, torch.nn.Parameter):
+        tensors, present = _placeholders(xf, [mf, *args])
+        out = _trimul_fwd_op(xf, tensors, present, direction == "outgoing", float(eps))[0]
+    else:
+        out = _TriMul.apply(xf, mf, *args, direction == "outgoing", float(eps))
     return out.view(tuple(lead) + (N, N, Do))
