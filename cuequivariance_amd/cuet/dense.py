@@ -17,6 +17,8 @@ those kernels refuse go through ``cueq_seg_gemm`` / ``cueq_seg_outer`` / ``cueq_
 from __future__ import annotations
 
 import ctypes as C
+import threading
+import weakref
 from typing import Dict, List, Optional
 
 import torch
@@ -365,9 +367,15 @@ class _FcPlan:
             for (K, N), rows in self.t_shapes.items():
                 t_tabs[(K, N)] = torch.tensor(rows, dtype=torch.int64, device=device)
                 # weight gradient: part p contracts x1[:, a_off_p : +K] with H[:, t_p : +N] into block p of the partials
+                # the parts of one weight block (its x1 components) are summed in a fixed order: for every distinct
+                # block the list of its parts, padded with the index of an all-zero extra part
+                blocks = sorted({w for _, w, _ in rows})
+                members = [[p for p, (_, w, _) in enumerate(rows) if w == wb] for wb in blocks]
+                width = max(len(m) for m in members)
                 w_tabs[(K, N)] = (
                     torch.tensor([(a, t, p * K * N) for p, (a, _, t) in enumerate(rows)], dtype=torch.int64, device=device),
-                    (torch.tensor([w for _, w, _ in rows], dtype=torch.int64, device=device)[:, None]
+                    torch.tensor([m + [len(rows)] * (width - len(m)) for m in members], dtype=torch.int64, device=device),
+                    (torch.tensor(blocks, dtype=torch.int64, device=device)[:, None]
                      + torch.arange(K * N, dtype=torch.int64, device=device)[None, :]).reshape(-1),
                 )
             for (K, N), rows in self.g_shapes.items():
@@ -456,7 +464,7 @@ class _FcFunction(torch.autograd.Function):
                     H = torch.empty(Z, plan.t_cols, dtype=dtype, device=dev)
                     _fc_combine(lib, code, code, Z, x2d, g, H, tables["h"], stream)
                     gw32 = torch.zeros(wd.numel(), dtype=torch.float32, device=dev)
-                    for (K, N), (tab, dst) in tables["w"].items():
+                    for (K, N), (tab, members, dst) in tables["w"].items():
                         nparts = tab.shape[0]
                         if K <= 64 and N <= 64:  # one wavefront per 64 x 64 product: about two of them per SIMD
                             chunks = max(1, min(-(-2048 // nparts), Z // 64))
@@ -467,12 +475,14 @@ class _FcFunction(torch.autograd.Function):
                         _lib.check(lib.cueq_gemm_table(code, _lib.F32, 1, 1, K, N, Z, x1d.data_ptr(), x1d.stride(0), H.data_ptr(),
                                                        plan.t_cols, part.data_ptr(), N, tab.data_ptr(), nparts, chunks, nparts * K * N,
                                                        1.0, 0, stream), "cueq_gemm_table")
-                        total = torch.empty(nparts * K * N, dtype=torch.float32, device=dev)
+                        total = torch.zeros((nparts + 1) * K * N, dtype=torch.float32, device=dev)  # (+ the all-zero part)
                         ws_bytes = lib.cueq_sum_rows_workspace(chunks, nparts * K * N)
                         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
                         _lib.check(lib.cueq_sum_rows(_lib.F32, chunks, nparts * K * N, part.data_ptr(), total.data_ptr(), ws.data_ptr(),
                                                      ws_bytes, stream), "cueq_sum_rows")
-                        gw32.index_add_(0, dst, total)  # blocks of one path (its x1 components) land on the same weights
+                        # blocks of one path (its x1 components) land on the same weights: ordered sum, then a copy
+                        # to distinct destinations (index_add_ would use atomics)
+                        gw32.index_copy_(0, dst, total.view(nparts + 1, K * N)[members].sum(1).reshape(-1))
                     gwd = gw32.to(dtype).view(wd.shape)
                 gw = gwd.to(w.dtype).reshape(w.shape)
             if gx2 is not None and x2.shape[0] == 1 and Z != 1:
@@ -555,6 +565,77 @@ class _IndexedDenseFunction(torch.autograd.Function):
         return None, gw, gx1, None
 
 
+# ---------------------------------------------------------------------- traced execution (torch.compile / export)
+# Forward and backward of the two shared-weight functions as opaque operators.  They call the static methods above with
+# a plain object in place of the autograd context; the module travels as a small integer.
+_traced_modules: dict = {}
+_traced_lock = threading.Lock()
+_FUNCTIONS = (_DenseFunction, _FcFunction)
+
+
+class _PlainContext:
+    def save_for_backward(self, *tensors):
+        self.saved_tensors = tensors
+
+
+def _module_by_id(mod_id: int) -> "SegmentedPolynomialDense":
+    mod = _traced_modules[mod_id]()
+    if mod is None:
+        raise RuntimeError("fused_tp: the module this graph was traced from no longer exists")
+    return mod
+
+
+@torch.library.custom_op("cuequivariance_amd::dense_fwd", mutates_args=(), device_types="cuda")
+def _dense_fwd_op(mod_id: int, kind: int, w: torch.Tensor, x1: torch.Tensor, x2: Optional[torch.Tensor]) -> torch.Tensor:
+    return _FUNCTIONS[kind].forward(_PlainContext(), _module_by_id(mod_id), w, x1, x2)
+
+
+@_dense_fwd_op.register_fake
+def _dense_fwd_fake(mod_id, kind, w, x1, x2):
+    return x1.new_empty(x1.shape[0], _module_by_id(mod_id).out_size)
+
+
+@torch.library.custom_op("cuequivariance_amd::dense_bwd", mutates_args=(), device_types="cuda")
+def _dense_bwd_op(mod_id: int, kind: int, w: torch.Tensor, x1: torch.Tensor, x2: Optional[torch.Tensor], g: torch.Tensor,
+                  need: List[bool]) -> List[torch.Tensor]:
+    ctx = _PlainContext()
+    ctx.mod, ctx.has_x2 = _module_by_id(mod_id), x2 is not None
+    ctx.saved_tensors = (w, x1, x2 if (x2 is not None or kind == 1) else torch.empty(0))
+    ctx.needs_input_grad = (False, *need)
+    grads = _FUNCTIONS[kind].backward(ctx, g)[1:4]
+    return [x1.new_empty(0) if (t is None or not n) else t.contiguous() for t, n in zip(grads, need)]
+
+
+@_dense_bwd_op.register_fake
+def _dense_bwd_fake(mod_id, kind, w, x1, x2, g, need):
+    return [torch.empty_like(t) if (n and t is not None) else x1.new_empty(0) for t, n in zip((w, x1, x2), need)]
+
+
+def _dense_setup_context(ctx, inputs, output):
+    mod_id, kind, w, x1, x2 = inputs
+    ctx.meta = (mod_id, kind, x2 is not None)
+    ctx.save_for_backward(w, x1, *([x2] if x2 is not None else []))
+
+
+def _dense_autograd(ctx, g):
+    mod_id, kind, has_x2 = ctx.meta
+    w, x1 = ctx.saved_tensors[:2]
+    x2 = ctx.saved_tensors[2] if has_x2 else None
+    need = [bool(n) for n in ctx.needs_input_grad[2:5]]
+    got = _dense_bwd_op(mod_id, kind, w, x1, x2, g.contiguous(), need)
+    gw, gx1, gx2 = [t if t.numel() > 0 else None for t in got]
+    return None, None, gw, gx1, gx2
+
+
+torch.library.register_autograd("cuequivariance_amd::dense_fwd", _dense_autograd, setup_context=_dense_setup_context)
+
+
+def _apply_dense(kind: int, mod: "SegmentedPolynomialDense", w, x1, x2):
+    if torch.compiler.is_compiling() or type(x1) not in (torch.Tensor, torch.nn.Parameter):
+        return _dense_fwd_op(mod.traced_id, kind, w, x1, x2)
+    return _FUNCTIONS[kind].apply(mod, w, x1, x2)
+
+
 class SegmentedPolynomialDense(nn.Module):
     """Dense (MFMA) executor for Linear / fully-connected polynomials with weights shared over the batch."""
 
@@ -592,6 +673,9 @@ class SegmentedPolynomialDense(nn.Module):
         self.dx1_groups = _batched_groups(self.paths, lambda p: p.c_off, lambda p: p.a_off)
         self.weight_blocks = sorted({(p.w_off, p.K, p.N) for p in self.paths})
         self.fc_plan = _FcPlan(self.paths, self.input_sizes[2]) if self.has_x2 else None
+        with _traced_lock:  # the integer under which a traced graph names this module
+            self.traced_id = len(_traced_modules)
+            _traced_modules[self.traced_id] = weakref.ref(self)
 
     def tiled(self, dtype, A: torch.Tensor, Cout: torch.Tensor) -> bool:
         """The tiled kernel serves fp32 / bf16 contractions without a per-row scale."""
@@ -670,5 +754,5 @@ class SegmentedPolynomialDense(nn.Module):
             elif x1.shape[0] == 1 and x2.shape[0] != 1:
                 x1 = x1.expand(x2.shape[0], x1.shape[1])
         if x2 is not None and self.fc_plan.ok and x1.dtype in (torch.float32, torch.bfloat16):
-            return [_FcFunction.apply(self, w, x1, x2)]
-        return [_DenseFunction.apply(self, w, x1, x2)]
+            return [_apply_dense(1, self, w, x1, x2)]
+        return [_apply_dense(0, self, w, x1, x2)]

@@ -117,3 +117,29 @@ def test_compiled_triangle_update_matches_eager(device, dtype):
     assert torch.equal(out, ref)
     for a, b in zip(torch.autograd.grad(out, leaves, cot), ref_grads):
         assert a.dtype == b.dtype and torch.equal(a, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_compiled_linear_and_fully_connected_match_eager(device, dtype):
+    """The MFMA executor (shared weights) under ``torch.compile(fullgraph=True)``: ``dense_fwd`` / ``dense_bwd``."""
+    from cuequivariance_amd import cuet
+
+    g = torch.Generator(device=device).manual_seed(21)
+    i1, i2, io = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e"), cue.Irreps("O3", "64x0e+64x1o")
+    lin = cuet.Linear(i1, io, layout=cue.ir_mul, device=device, dtype=dtype)
+    fc = cuet.FullyConnectedTensorProduct(i1, i2, io, layout=cue.ir_mul, device=device, dtype=dtype)
+    x1 = torch.randn(300, i1.dim, device=device, generator=g).to(dtype).requires_grad_(True)
+    x2 = torch.randn(300, i2.dim, device=device, generator=g).to(dtype).requires_grad_(True)
+
+    def f(x1, x2):
+        return fc(lin(x1), x2)
+
+    ref = f(x1, x2)
+    cot = torch.randn(ref.shape, device=device, generator=g).to(dtype)
+    leaves = [x1, x2, lin.weight, fc.weight]
+    ref_grads = torch.autograd.grad(ref, leaves, cot)
+    out = torch.compile(f, fullgraph=True, backend="aot_eager", dynamic=False)(x1, x2)
+    assert torch.equal(out, ref)
+    for a, b in zip(torch.autograd.grad(out, leaves, cot), ref_grads):
+        assert torch.equal(a, b)
