@@ -1882,6 +1882,33 @@ __global__ void __launch_bounds__(256) sum_rows_partial_kernel(const TI* __restr
   part[static_cast<int64_t>(blockIdx.y) * Ccols + cc] = s;
 }
 
+// out[c] = sum_r in[r][c] in one launch for a moderate number of rows: 64 columns x 16 row lanes per block, every lane
+// adds rows r = lane, lane + 16, ... in order, the 16 partial sums are added in lane order (fixed, reproducible)
+template <typename TI>
+__global__ void __launch_bounds__(1024) sum_rows_lds_kernel(const TI* __restrict__ in, float* __restrict__ out, int64_t R, int64_t Ccols) {
+  __shared__ float s_acc[16][64];
+  const int cl = threadIdx.x & 63, rl = threadIdx.x >> 6;
+  const int64_t cc = static_cast<int64_t>(blockIdx.x) * 64 + cl;
+  float s = 0;
+  if (cc < Ccols) {
+    int64_t r = rl;
+    for (; r + 48 < R; r += 64) {  // four loads in flight
+      const float v0 = tri_load(in, r * Ccols + cc), v1 = tri_load(in, (r + 16) * Ccols + cc);
+      const float v2 = tri_load(in, (r + 32) * Ccols + cc), v3 = tri_load(in, (r + 48) * Ccols + cc);
+      s += v0; s += v1; s += v2; s += v3;
+    }
+    for (; r < R; r += 16) s += tri_load(in, r * Ccols + cc);
+  }
+  s_acc[rl][cl] = s;
+  __syncthreads();
+  if (rl == 0 && cc < Ccols) {
+    float total = 0;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) total += s_acc[t][cl];
+    out[cc] = total;
+  }
+}
+
 template <typename TO>
 __global__ void __launch_bounds__(256) fold_partials_kernel(const float* __restrict__ part, TO* __restrict__ out, int64_t nparts, int64_t n,
                                                             int accumulate) {
@@ -2464,6 +2491,14 @@ extern "C" int cueq_sum_rows(int32_t dtype, int64_t rows, int64_t cols, const vo
     return CUEQ_OK;
   }
   CUEQ_REQUIRE(in && workspace && workspace_bytes >= cueq_sum_rows_workspace(rows, cols), CUEQ_ERR_INVALID, "sum_rows: workspace too small");
+  if (rows <= 4096 && (cols + 63) / 64 >= 128) {  // few rows, enough column blocks to fill the chip: one launch
+    const dim3 grid1(static_cast<unsigned>((cols + 63) / 64));
+    TRI_DISPATCH(dtype,
+                 hipLaunchKernelGGL(sum_rows_lds_kernel<float>, grid1, dim3(1024), 0, stream, static_cast<const float*>(in), out, rows, cols),
+                 hipLaunchKernelGGL(sum_rows_lds_kernel<uint16_t>, grid1, dim3(1024), 0, stream, static_cast<const uint16_t*>(in), out, rows, cols));
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
   const int64_t nb = sum_rows_blocks(rows, cols);
   const int64_t rpb = (rows + nb - 1) / nb;
   float* part = static_cast<float*>(workspace);

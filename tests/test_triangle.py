@@ -267,3 +267,22 @@ def test_dual_gate_many_column_tiles(device, dtype, N, with_bias):
     got = T.dual_gate_fwd(dev(W1), dev(W2), dev(X), None, dev(b1), dev(b2), 0, dev(mask), 1)
     assert got.shape == (C, N) and got.dtype == dtype
     assert rel_err(got, want) <= TOL[dtype], rel_err(got, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(513, 16384), (37, 8200), (3000, 700), (70000, 130), (1, 8192), (5, 3)])
+def test_sum_rows_paths(device, dtype, shape):
+    """Column sums of a (rows, cols) matrix in float32: the single-launch kernel (few rows, many columns), the two-stage
+    one (everything else), partial column blocks and single rows; against a float64 sum of the rounded input, and
+    bit-identical from run to run."""
+    from cuequivariance_amd.cuet import triangle as T
+
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(*shape, generator=g).to(dtype)
+    want = x.double().sum(0)
+    got = T.sum_rows(x.to(device))
+    assert got.dtype == torch.float32 and got.shape == (shape[1],)
+    scale = x.double().abs().sum(0).max().item()
+    assert (got.cpu().double() - want).abs().max().item() <= 1e-6 * scale
+    assert torch.equal(got, T.sum_rows(x.to(device)))
