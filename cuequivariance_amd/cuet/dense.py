@@ -234,10 +234,13 @@ class _DenseFunction(torch.autograd.Function):
                     else:
                         _run_gemms(dtype, g, wd, x2d, gx1, tables.dx1)
             if ctx.needs_input_grad[1]:
-                gwd = torch.zeros_like(wd)
+                gwd = None
                 if Z > 0 and mod.tiled(dtype, x1d, g):
                     # dW_p[k][n] += c * sum_z x1[z, i_seg + k] g[z, k_seg + n]: chunked partial products, ordered sum
+                    # straight into a float32 image of the weights (a block met a second time is added)
                     code, es = _DTYPE_CODE[dtype], x1d.element_size()
+                    gw32 = torch.zeros(wd.numel(), dtype=torch.float32, device=x1.device)
+                    written = set()
                     for p, count, da, dc in mod.fwd_groups:
                         items = lib.cueq_gemm_tn_items(Z, count)
                         part = torch.empty(items, p.K * p.N, dtype=torch.float32, device=x1.device)
@@ -246,13 +249,18 @@ class _DenseFunction(torch.autograd.Function):
                                              g.data_ptr() + p.c_off * es, g.stride(0), dc, count, part.data_ptr(), p.coeff, stream),
                             "cueq_gemm_tn",
                         )
-                        total = torch.empty(p.K * p.N, dtype=torch.float32, device=x1.device)
+                        first = p.w_off not in written
+                        written.add(p.w_off)
+                        total = gw32[p.w_off: p.w_off + p.K * p.N] if first else torch.empty(p.K * p.N, dtype=torch.float32, device=x1.device)
                         ws_bytes = lib.cueq_sum_rows_workspace(items, p.K * p.N)
                         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x1.device)
                         _lib.check(lib.cueq_sum_rows(_lib.F32, items, p.K * p.N, part.data_ptr(), total.data_ptr(), ws.data_ptr(),
                                                      ws_bytes, stream), "cueq_sum_rows")
-                        gwd.view(-1)[p.w_off: p.w_off + p.K * p.N] += total.to(dtype)
+                        if not first:
+                            gw32[p.w_off: p.w_off + p.K * p.N] += total
+                    gwd = gw32.view(wd.shape)
                 elif Z > 0:
+                    gwd = torch.zeros_like(wd)
                     for w_off, K, N, ent, n in tables.dw:
                         ws_bytes = lib.cueq_seg_outer_workspace(_DTYPE_CODE[dtype], K, N, Z)
                         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x1.device)
@@ -265,6 +273,8 @@ class _DenseFunction(torch.autograd.Function):
                             ),
                             "cueq_seg_outer",
                         )
+                if gwd is None:
+                    gwd = torch.zeros_like(wd)
                 gw = gwd.to(w.dtype).reshape(w.shape)
             if x2 is not None and ctx.needs_input_grad[3]:
                 gx2 = torch.zeros_like(x2d)
