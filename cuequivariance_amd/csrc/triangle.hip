@@ -300,7 +300,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
   // results already leave as 128-byte row segments and gain nothing from the detour)
   if constexpr (sizeof(TO) == 2) {
     __syncthreads();  // every wavefront is done with the operand tiles, which become staging space
-    if (vec_out && m0 + wm * 64 + 64 <= M && n0 + wn * 64 + 64 <= N) {
+    // (parts addressed through a table: every part checks the alignment of its own result block)
+    const bool vec_rows = gmode == 3 ? (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * sizeof(TO)) % 16 == 0) : vec_out != 0;
+    if (vec_rows && m0 + wm * 64 + 64 <= M && n0 + wn * 64 + 64 <= N) {
       constexpr int RS = 64 * sizeof(TO) + 16;
       static_assert(WM * WN * 32 * RS <= 2 * (ABYTES + BBYTES), "staging tiles must fit the operand buffers");
       char* tile = &smem[0][0] + wave * (32 * RS);

@@ -159,6 +159,54 @@ def _batched_groups(paths, a_key, c_key):
     return groups
 
 
+def _merged_tables(mod: "SegmentedPolynomialDense", device: torch.device):
+    """For the 3-operand form: the column blocks of all paths as parts of table-driven launches, one launch per distinct
+    (K, N, coefficient).  ``fwd``: rows (x offset, weight offset, out offset); ``dx``: rows (g offset, weight offset, dx
+    offset); ``None`` when two parts of one launch would write the same columns (those take the per-group launches)."""
+    key = (device.type, device.index)
+    hit = mod._merged.get(key)
+    if hit is None:
+        by = {}
+        for p in mod.paths:
+            by.setdefault((p.K, p.N, p.coeff), []).append(p)
+        ok = all(len({p.c_off for p in plist}) == len(plist) and len({p.a_off for p in plist}) == len(plist) for plist in by.values())
+        outs = [p.c_off for p in mod.paths]
+        ins = [p.a_off for p in mod.paths]
+        ok = ok and len(set(outs)) == len(outs) and len(set(ins)) == len(ins)
+        # the table-driven launch moves 16-byte vectors: extents and offsets in multiples of 8 elements
+        ok = ok and all(v % 8 == 0 for p in mod.paths for v in (p.K, p.N, p.a_off, p.c_off, p.w_off))
+        hit = None
+        if ok:
+            hit = [(K, N, coeff,
+                    torch.tensor([(p.a_off, p.w_off, p.c_off) for p in plist], dtype=torch.int64, device=device),
+                    torch.tensor([(p.c_off, p.w_off, p.a_off) for p in plist], dtype=torch.int64, device=device))
+                   for (K, N, coeff), plist in by.items()]
+        mod._merged[key] = hit if hit is not None else False
+        return hit
+    return hit or None
+
+
+def _vector_rows(*tensors) -> bool:
+    return all(t.data_ptr() % 16 == 0 and (t.dim() < 2 or (t.stride(0) * t.element_size()) % 16 == 0) for t in tensors)
+
+
+def _run_merged(dtype, A, B, Cout, launches, forward: bool):
+    """``Cout[:, c : c + N] = coeff * A[:, a : a + K] @ W_p`` (forward, W_p is K x N as it lies) or
+    ``Cout[:, a : a + K] = coeff * A[:, c : c + N] @ W_p^T`` (input gradient) for all parts of a launch at once."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(A.device).cuda_stream
+    code = _DTYPE_CODE[dtype]
+    for K, N, coeff, fwd_tab, dx_tab in launches:
+        if forward:
+            _lib.check(lib.cueq_gemm_table(code, code, 0, 1, A.shape[0], N, K, A.data_ptr(), A.stride(0), B.data_ptr(), N,
+                                           Cout.data_ptr(), Cout.stride(0), fwd_tab.data_ptr(), fwd_tab.shape[0], 1, 0, coeff, 0, stream),
+                       "cueq_gemm_table")
+        else:
+            _lib.check(lib.cueq_gemm_table(code, code, 0, 0, A.shape[0], K, N, A.data_ptr(), A.stride(0), B.data_ptr(), N,
+                                           Cout.data_ptr(), Cout.stride(0), dx_tab.data_ptr(), dx_tab.shape[0], 1, 0, coeff, 0, stream),
+                       "cueq_gemm_table")
+
+
 def _run_tiled(dtype, A, a_key, B_of, Cout, c_key, groups, Kdim, Ndim):
     """``Cout[:, c : c + N] (+)= coeff * A[:, a : a + K] @ B^T`` per group through the 128 x 128 tiled MFMA kernel
     (``cueq_gemm_nt``; ``B_of(path)`` gives the pointer of the ``N x K`` block)."""
@@ -193,7 +241,10 @@ class _DenseFunction(torch.autograd.Function):
         x2d = x2.detach().contiguous() if x2 is not None else None
         if Z > 0:
             with torch.cuda.device(x1.device):
-                if mod.tiled(dtype, x1d, out):
+                merged = _merged_tables(mod, x1.device) if (mod.tiled(dtype, x1d, out) and _vector_rows(x1d, wd, out)) else None
+                if merged is not None:
+                    _run_merged(dtype, x1d, wd, out, merged, True)
+                elif mod.tiled(dtype, x1d, out):
                     # out[:, k_seg] (+)= c * x1[:, i_seg] @ W_p: the kernel wants W_p^T (N x K, contraction contiguous)
                     wt = mod.transposed_weights(wd)
                     es = wd.element_size()
@@ -226,7 +277,10 @@ class _DenseFunction(torch.autograd.Function):
                 # dx1[:, i_seg] += c * x2[:, j] * g[:, k_seg] @ W_p^T
                 gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
                 if Z > 0:
-                    if mod.tiled(dtype, g, gx1):
+                    merged = _merged_tables(mod, x1.device) if (mod.tiled(dtype, g, gx1) and _vector_rows(g, wd, gx1)) else None
+                    if merged is not None:
+                        _run_merged(dtype, g, wd, gx1, merged, False)
+                    elif mod.tiled(dtype, g, gx1):
                         # dx1[:, i_seg] (+)= c * g[:, k_seg] @ W_p^T: W_p (K x N) is already "N x K" for this product
                         es = wd.element_size()
                         _run_tiled(dtype, g, lambda p: p.c_off, lambda p: wd.data_ptr() + p.w_off * es, gx1, lambda p: p.a_off,
@@ -683,6 +737,7 @@ class SegmentedPolynomialDense(nn.Module):
         self.dx1_groups = _batched_groups(self.paths, lambda p: p.c_off, lambda p: p.a_off)
         self.weight_blocks = sorted({(p.w_off, p.K, p.N) for p in self.paths})
         self.fc_plan = _FcPlan(self.paths, self.input_sizes[2]) if self.has_x2 else None
+        self._merged: dict = {}
         with _traced_lock:  # the integer under which a traced graph names this module
             self.traced_id = len(_traced_modules)
             _traced_modules[self.traced_id] = weakref.ref(self)
