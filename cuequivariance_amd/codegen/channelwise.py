@@ -568,7 +568,7 @@ static int run_bwd(const SpecCall& c) {{
   else atomic = true;
   if (atomic && b[5].rows > 0) {{
     const int64_t n = b[5].rows * {W1}ll;
-    hipLaunchKernelGGL(fill_zero<{T}>, dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1, n);
+    hipLaunchKernelGGL(fill_zero<{T}>, dim3(fill_blocks<{T}>(n)), dim3(256), 0, c.stream, dx1, n);
     CUEQ_CHECK_HIP(hipGetLastError());
   }}
   if (batch > 0) {{

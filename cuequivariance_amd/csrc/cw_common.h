@@ -60,10 +60,25 @@ __global__ void __launch_bounds__(256) fold_parts(const T* __restrict__ partial,
   out[tid] = acc;
 }
 
+// p[0 .. n) = 0, 16 bytes per thread (element by element when p is not 16-byte aligned, and for the tail);
+// launch with fill_blocks<T>(n) blocks of 256 threads
 template <typename T>
 __global__ void __launch_bounds__(256) fill_zero(T* __restrict__ p, int64_t n) {
-  const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (tid < n) p[tid] = 0;
+  constexpr int V = 16 / sizeof(T);
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * V;
+  if (i >= n) return;
+  if (i + V <= n && reinterpret_cast<uintptr_t>(p) % 16 == 0) {
+    *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
+  } else {
+    for (int64_t k = i; k < n && k < i + V; ++k) p[k] = 0;
+  }
+}
+
+template <typename T>
+inline unsigned fill_blocks(int64_t n) {
+  constexpr int V = 16 / sizeof(T);
+  const int64_t threads = (n + V - 1) / V;
+  return static_cast<unsigned>((threads + 255) / 256);
 }
 
 // Compute units of the current device (cached for the first device queried).
