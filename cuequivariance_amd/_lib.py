@@ -186,9 +186,9 @@ def load() -> C.CDLL:
         lib.cueq_gemm_grouped.restype = C.c_int
         lib.cueq_gemm_table.argtypes = [i32, i32, i32, i32, i64, i64, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i64, i64, i64, f64, i32, ptr]
         lib.cueq_gemm_table.restype = C.c_int
-        lib.cueq_fc_combine.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i32, ptr, i32, ptr]
+        lib.cueq_fc_combine.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i32, ptr, i32, i32, ptr]
         lib.cueq_fc_combine.restype = C.c_int
-        lib.cueq_fc_rowdot.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, i32, ptr, i32, ptr]
+        lib.cueq_fc_rowdot.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, i32, ptr, i32, i32, ptr]
         lib.cueq_fc_rowdot.restype = C.c_int
         lib.cueq_segmented_transpose.argtypes = [i32, i64, i64, ptr, ptr, ptr, ptr]
         lib.cueq_segmented_transpose.restype = C.c_int

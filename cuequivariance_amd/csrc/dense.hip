@@ -419,6 +419,41 @@ __global__ void __launch_bounds__(256) fc_combine_kernel(const TS* __restrict__ 
   }
 }
 
+// four adjacent columns per thread (16 / 8-byte accesses): blocks, offsets and row strides are multiples of four
+__device__ __forceinline__ float4 fc_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 fc_load4(const uint16_t* p) {
+  const uint2 w = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
+}
+__device__ __forceinline__ void fc_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void fc_store4(uint16_t* p, float4 v) {
+  uint16_t h[4];
+  from_float(h[0], v.x); from_float(h[1], v.y); from_float(h[2], v.z); from_float(h[3], v.w);
+  *reinterpret_cast<uint2*>(p) = make_uint2(static_cast<uint32_t>(h[0]) | (static_cast<uint32_t>(h[1]) << 16),
+                                            static_cast<uint32_t>(h[2]) | (static_cast<uint32_t>(h[3]) << 16));
+}
+
+template <typename TS, typename TT, typename TO>
+__global__ void __launch_bounds__(256) fc_combine_vec_kernel(const TS* __restrict__ S, int64_t lds_, const TT* __restrict__ T, int64_t ldt,
+                                                             TO* __restrict__ O, int64_t ldo, const FcBlock* __restrict__ blocks,
+                                                             const FcUse* __restrict__ uses, int64_t Z, int max_n) {
+  const FcBlock b = blocks[blockIdx.y];
+  const int tpr = max_n / 4;  // threads per row
+  const int rows_per_pass = 256 / tpr;
+  const int n = (threadIdx.x % tpr) * 4, r = threadIdx.x / tpr;
+  if (n >= b.n || r >= rows_per_pass) return;
+  for (int64_t z = static_cast<int64_t>(blockIdx.x) * rows_per_pass + r; z < Z; z += static_cast<int64_t>(gridDim.x) * rows_per_pass) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int u = 0; u < b.num_uses; ++u) {
+      const FcUse use = uses[b.first_use + u];
+      const float sc = use.coeff * load_as<float>(S, type_code<TS>(), z * lds_ + use.j);
+      const float4 t = fc_load4(T + z * ldt + use.src_off + n);
+      acc.x = fmaf(sc, t.x, acc.x); acc.y = fmaf(sc, t.y, acc.y); acc.z = fmaf(sc, t.z, acc.z); acc.w = fmaf(sc, t.w, acc.w);
+    }
+    fc_store4(O + z * ldo + b.out_off + n, acc);
+  }
+}
+
 struct FcDotUse { int32_t j, a_off, g_off, k; float coeff; int32_t pad[3]; };
 
 template <typename TX, typename TG>
@@ -428,16 +463,64 @@ __global__ void __launch_bounds__(256) fc_rowdot_kernel(const TX* __restrict__ X
   // one wavefront per row; lane j keeps the running sum of column j (n2 <= 64)
   const int lane = threadIdx.x & 63;
   for (int64_t z = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6); z < Z; z += static_cast<int64_t>(gridDim.x) * 4) {
-    float acc = 0.f;
+    // consecutive uses of one column j share a single reduction over the lanes (the caller may sort the uses by j)
+    float acc = 0.f, p = 0.f;
+    int cur = num_uses > 0 ? uses[0].j : 0;
     for (int u = 0; u < num_uses; ++u) {
       const FcDotUse use = uses[u];
-      float p = 0.f;
+      if (use.j != cur) {
+        p = wave_sum(p);
+        if (lane == cur) acc += p;
+        p = 0.f;
+        cur = use.j;
+      }
+      float q = 0.f;
       for (int k = lane; k < use.k; k += 64)
-        p = fmaf(load_as<float>(X, type_code<TX>(), z * ldx + use.a_off + k), load_as<float>(G, type_code<TG>(), z * ldg + use.g_off + k), p);
-      p = wave_sum(p);
-      if (lane == use.j) acc = fmaf(use.coeff, p, acc);
+        q = fmaf(load_as<float>(X, type_code<TX>(), z * ldx + use.a_off + k), load_as<float>(G, type_code<TG>(), z * ldg + use.g_off + k), q);
+      p = fmaf(use.coeff, q, p);
     }
+    p = wave_sum(p);
+    if (lane == cur) acc += p;
     if (lane < n2) store_as<float>(D, type_code<TX>(), z * ldd + lane, acc);
+  }
+}
+
+// The same with four rows per wavefront: 16 lanes per row, four adjacent elements per lane (k, the offsets and the row
+// strides are multiples of four); lane l of a row keeps the columns j = l, l + 16, l + 32, l + 48.
+template <typename TX, typename TG>
+__global__ void __launch_bounds__(256) fc_rowdot_vec_kernel(const TX* __restrict__ X, int64_t ldx, const TG* __restrict__ G, int64_t ldg,
+                                                            TX* __restrict__ D, int64_t ldd, int n2, const FcDotUse* __restrict__ uses,
+                                                            int num_uses, int64_t Z) {
+  const int lane = threadIdx.x & 63, l16 = lane & 15, sub = lane >> 4;
+  for (int64_t z0 = (static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6)) * 4; z0 < Z; z0 += static_cast<int64_t>(gridDim.x) * 16) {
+    const int64_t z = min(z0 + sub, Z - 1);
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f, p = 0.f;
+    int cur = num_uses > 0 ? uses[0].j : 0;
+    auto commit = [&]() {
+      p += __shfl_xor(p, 8, 64); p += __shfl_xor(p, 4, 64); p += __shfl_xor(p, 2, 64); p += __shfl_xor(p, 1, 64);
+      if (l16 == (cur & 15)) {
+        const int q = cur >> 4;
+        if (q == 0) a0 += p; else if (q == 1) a1 += p; else if (q == 2) a2 += p; else a3 += p;
+      }
+      p = 0.f;
+    };
+    for (int u = 0; u < num_uses; ++u) {
+      const FcDotUse use = uses[u];
+      if (use.j != cur) { commit(); cur = use.j; }
+      float q = 0.f;
+      for (int k = 4 * l16; k < use.k; k += 64) {
+        const float4 x = fc_load4(X + z * ldx + use.a_off + k), g = fc_load4(G + z * ldg + use.g_off + k);
+        q = fmaf(x.x, g.x, q); q = fmaf(x.y, g.y, q); q = fmaf(x.z, g.z, q); q = fmaf(x.w, g.w, q);
+      }
+      p = fmaf(use.coeff, q, p);
+    }
+    commit();
+    if (z0 + sub < Z) {
+      if (l16 < n2) store_as<float>(D, type_code<TX>(), z * ldd + l16, a0);
+      if (l16 + 16 < n2) store_as<float>(D, type_code<TX>(), z * ldd + l16 + 16, a1);
+      if (l16 + 32 < n2) store_as<float>(D, type_code<TX>(), z * ldd + l16 + 32, a2);
+      if (l16 + 48 < n2) store_as<float>(D, type_code<TX>(), z * ldd + l16 + 48, a3);
+    }
   }
 }
 
@@ -592,19 +675,33 @@ extern "C" int cueq_seg_rowdot(int32_t dtype, int32_t K, int32_t N, const void* 
 
 // dtype codes: s = x2 and the result (the tensor dtype), t = the GEMM results (float32 or the tensor dtype)
 extern "C" int cueq_fc_combine(int32_t dtype, int32_t t_dtype, int64_t rows, const void* S, int64_t lds_, const void* T, int64_t ldt, void* O,
-                               int64_t ldo, const void* blocks, int32_t num_blocks, const void* uses, int32_t max_n, void* stream_) {
+                               int64_t ldo, const void* blocks, int32_t num_blocks, const void* uses, int32_t max_n, int32_t vectorised,
+                               void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   CUEQ_REQUIRE((dtype == CUEQ_F32 || dtype == CUEQ_BF16) && (t_dtype == CUEQ_F32 || t_dtype == dtype), CUEQ_ERR_UNSUPPORTED,
                "fc_combine: tensors float32 or bfloat16, GEMM results float32 or the tensor dtype");
   CUEQ_REQUIRE(rows >= 0 && num_blocks >= 0 && max_n >= 1 && max_n <= 256, CUEQ_ERR_INVALID, "fc_combine: bad extents (block width at most 256)");
   if (rows == 0 || num_blocks == 0) return CUEQ_OK;
   CUEQ_REQUIRE(S && T && O && blocks && uses, CUEQ_ERR_INVALID, "fc_combine: null operand");
-  const int rpp = 256 / max_n;
+  // four columns per thread when every block width, column offset and row stride is a multiple of four and the rows are
+  // 16 / 8-byte aligned (the caller says so: it owns the tables)
+  const bool vec = vectorised != 0 && max_n % 4 == 0 && ldt % 4 == 0 && ldo % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(T) % 16 == 0 && reinterpret_cast<uintptr_t>(O) % 16 == 0;
+  const int rpp = vec ? 256 / (max_n / 4) : 256 / max_n;
   int64_t gx = (rows + rpp - 1) / rpp;
   const int64_t cap = static_cast<int64_t>(device_cus()) * 32 / num_blocks + 1;
   if (gx > cap) gx = cap;
   const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(num_blocks));
   KernelTimer timer("fc_combine", stream);
+  if (vec) {
+#define FCV(TS, TT) hipLaunchKernelGGL((fc_combine_vec_kernel<TS, TT, TS>), grid, dim3(256), 0, stream, static_cast<const TS*>(S), lds_, static_cast<const TT*>(T), ldt, static_cast<TS*>(O), ldo, static_cast<const FcBlock*>(blocks), static_cast<const FcUse*>(uses), rows, max_n)
+    if (dtype == CUEQ_F32) FCV(float, float);
+    else if (t_dtype == CUEQ_F32) FCV(uint16_t, float);
+    else FCV(uint16_t, uint16_t);
+#undef FCV
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
 #define FCC(TS, TT) hipLaunchKernelGGL((fc_combine_kernel<TS, TT, TS>), grid, dim3(256), 0, stream, static_cast<const TS*>(S), lds_, static_cast<const TT*>(T), ldt, static_cast<TS*>(O), ldo, static_cast<const FcBlock*>(blocks), static_cast<const FcUse*>(uses), rows, max_n)
   if (dtype == CUEQ_F32) FCC(float, float);
   else if (t_dtype == CUEQ_F32) FCC(uint16_t, float);
@@ -615,7 +712,7 @@ extern "C" int cueq_fc_combine(int32_t dtype, int32_t t_dtype, int64_t rows, con
 }
 
 extern "C" int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, const void* X, int64_t ldx, const void* G, int64_t ldg, void* D,
-                              int64_t ldd, int32_t n2, const void* uses, int32_t num_uses, void* stream_) {
+                              int64_t ldd, int32_t n2, const void* uses, int32_t num_uses, int32_t vectorised, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   CUEQ_REQUIRE((dtype == CUEQ_F32 || dtype == CUEQ_BF16) && (g_dtype == CUEQ_F32 || g_dtype == dtype), CUEQ_ERR_UNSUPPORTED,
                "fc_rowdot: tensors float32 or bfloat16, GEMM results float32 or the tensor dtype");
@@ -626,6 +723,18 @@ extern "C" int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, cons
   const int64_t cap = static_cast<int64_t>(device_cus()) * 32;
   if (gx > cap) gx = cap;
   KernelTimer timer("fc_rowdot", stream);
+  // four elements per lane when the caller states that every k, a_off and g_off of the table is a multiple of four
+  if (vectorised != 0 && ldx % 4 == 0 && ldg % 4 == 0 && reinterpret_cast<uintptr_t>(X) % 16 == 0 && reinterpret_cast<uintptr_t>(G) % 16 == 0) {
+    int64_t gv = (rows + 15) / 16;
+    if (gv > cap) gv = cap;
+#define FCDV(TX, TG) hipLaunchKernelGGL((fc_rowdot_vec_kernel<TX, TG>), dim3(static_cast<unsigned>(gv)), dim3(256), 0, stream, static_cast<const TX*>(X), ldx, static_cast<const TG*>(G), ldg, static_cast<TX*>(D), ldd, n2, static_cast<const FcDotUse*>(uses), num_uses, rows)
+    if (dtype == CUEQ_F32) FCDV(float, float);
+    else if (g_dtype == CUEQ_F32) FCDV(uint16_t, float);
+    else FCDV(uint16_t, uint16_t);
+#undef FCDV
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
 #define FCD(TX, TG) hipLaunchKernelGGL((fc_rowdot_kernel<TX, TG>), dim3(static_cast<unsigned>(gx)), dim3(256), 0, stream, static_cast<const TX*>(X), ldx, static_cast<const TG*>(G), ldg, static_cast<TX*>(D), ldd, n2, static_cast<const FcDotUse*>(uses), num_uses, rows)
   if (dtype == CUEQ_F32) FCD(float, float);
   else if (g_dtype == CUEQ_F32) FCD(uint16_t, float);

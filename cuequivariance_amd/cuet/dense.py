@@ -407,15 +407,18 @@ class _FcPlan:
                 for u in us:
                     uarr[first] = (u[0], u[1], u[2], 0)
                     first += 1
-            return barr, uarr, max(n for _, n in blocks)
+            # (last entry: every block width and column offset is a multiple of four - four columns per thread)
+            vec = all(off % 4 == 0 and n % 4 == 0 for off, n in blocks) and all(u[1] % 4 == 0 for us in blocks.values() for u in us)
+            return barr, uarr, max(n for _, n in blocks), vec
 
         self.fwd = tables(lambda p: p.c_off, lambda p: p.N, lambda p: t_of[(p.w_off, p.a_off)][0])
         self.dx1 = tables(lambda p: p.a_off, lambda p: p.K, lambda p: g_of[(p.w_off, p.c_off)][0])
         self.h = tables(lambda p: t_of[(p.w_off, p.a_off)][0], lambda p: p.N, lambda p: p.c_off)
         darr = np.zeros(len(paths), dtype=[("j", "<i4"), ("a", "<i4"), ("g", "<i4"), ("k", "<i4"), ("coeff", "<f4"), ("pad", "<i4", 3)])
-        for u, p in enumerate(paths):
+        for u, p in enumerate(sorted(paths, key=lambda p: p.j)):  # by column: uses of one column share a reduction
             darr[u] = (p.j, p.a_off, g_of[(p.w_off, p.c_off)][0], p.K, p.coeff, (0, 0, 0))
         self.dx2 = darr
+        self.dx2_vec = all(v % 4 == 0 for p in paths for v in (p.K, p.a_off, g_of[(p.w_off, p.c_off)][0]))
         self.ok = max(self.fwd[2], self.dx1[2], self.h[2]) <= 256 and n2 <= 64
         self._device: Dict[int, dict] = {}
 
@@ -446,18 +449,18 @@ class _FcPlan:
                 g_tabs[(K, N)] = torch.tensor(rows, dtype=torch.int64, device=device)
             d = self._device[idx] = {
                 "t": t_tabs, "g": g_tabs, "w": w_tabs,
-                "fwd": (up(self.fwd[0]), up(self.fwd[1]), len(self.fwd[0]), self.fwd[2]),
-                "dx1": (up(self.dx1[0]), up(self.dx1[1]), len(self.dx1[0]), self.dx1[2]),
-                "h": (up(self.h[0]), up(self.h[1]), len(self.h[0]), self.h[2]),
+                "fwd": (up(self.fwd[0]), up(self.fwd[1]), len(self.fwd[0]), self.fwd[2], self.fwd[3]),
+                "dx1": (up(self.dx1[0]), up(self.dx1[1]), len(self.dx1[0]), self.dx1[2], self.dx1[3]),
+                "h": (up(self.h[0]), up(self.h[1]), len(self.h[0]), self.h[2], self.h[3]),
                 "dx2": (up(self.dx2), len(self.dx2)),
             }
         return d
 
 
 def _fc_combine(lib, code, t_code, Z, S, T, O, table, stream):
-    blocks, uses, nblocks, max_n = table
+    blocks, uses, nblocks, max_n, vec = table
     _lib.check(lib.cueq_fc_combine(code, t_code, Z, S.data_ptr(), S.stride(0), T.data_ptr(), T.stride(0), O.data_ptr(), O.stride(0),
-                                   blocks.data_ptr(), nblocks, uses.data_ptr(), max_n, stream), "cueq_fc_combine")
+                                   blocks.data_ptr(), nblocks, uses.data_ptr(), max_n, 1 if vec else 0, stream), "cueq_fc_combine")
 
 
 class _FcFunction(torch.autograd.Function):
@@ -520,7 +523,8 @@ class _FcFunction(torch.autograd.Function):
                 if need_x2:
                     uses, nuses = tables["dx2"]
                     _lib.check(lib.cueq_fc_rowdot(code, _lib.F32, Z, x1d.data_ptr(), x1d.stride(0), G.data_ptr(), plan.g_cols,
-                                                  gx2.data_ptr(), gx2.stride(0), plan.n2, uses.data_ptr(), nuses, stream), "cueq_fc_rowdot")
+                                                  gx2.data_ptr(), gx2.stride(0), plan.n2, uses.data_ptr(), nuses,
+                                                  1 if plan.dx2_vec else 0, stream), "cueq_fc_rowdot")
             if need_w:
                 gwd = torch.zeros_like(wd)
                 if Z > 0:

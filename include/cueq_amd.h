@@ -177,11 +177,15 @@ int cueq_seg_rowdot(int32_t dtype, int32_t K, int32_t N, const void* A, int64_t 
  *   cueq_fc_rowdot:  D[z, j] = sum over the uses u with j_u == j of coeff_u * <X[z, a_off_u : +k_u], G[z, g_off_u : +k_u]>
  * blocks: device array of {int32 out_off, n, first_use, num_uses}; uses: device array of {int32 j, src_off; float coeff; int32 pad}
  * (combine) or {int32 j, a_off, g_off, k; float coeff; int32 pad[3]} (rowdot).  dtype: S, O, X, D (float32 / bfloat16);
- * t_dtype / g_dtype: T / G (float32 or the same).  Block widths at most max_n <= 256; D has n2 <= 64 columns. */
+ * t_dtype / g_dtype: T / G (float32 or the same).  Block widths at most max_n <= 256; D has n2 <= 64 columns.
+ * vectorised != 0: the caller states that every block width, out_off and src_off in the tables is a multiple of four
+ * (rowdot: every k, a_off and g_off) (then, with matching row strides and pointers, a thread moves four adjacent
+ * elements at a time). */
 int cueq_fc_combine(int32_t dtype, int32_t t_dtype, int64_t rows, const void* S, int64_t lds, const void* T, int64_t ldt, void* O,
-                    int64_t ldo, const void* blocks, int32_t num_blocks, const void* uses, int32_t max_n, void* stream);
+                    int64_t ldo, const void* blocks, int32_t num_blocks, const void* uses, int32_t max_n, int32_t vectorised,
+                    void* stream);
 int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, const void* X, int64_t ldx, const void* G, int64_t ldg, void* D,
-                   int64_t ldd, int32_t n2, const void* uses, int32_t num_uses, void* stream);
+                   int64_t ldd, int32_t n2, const void* uses, int32_t num_uses, int32_t vectorised, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* triangle multiplicative update: the stages behind                           */

@@ -82,5 +82,5 @@ def test_dense_entries_refuse_bad_arguments_before_any_launch():
     assert lib.cueq_segmented_transpose(3, 4, 4, p, p, 2 * p, None) == -2
     assert lib.cueq_segmented_transpose(4, 4, 4, p, p, p, None) == -1 and b"in place" in lib.cueq_last_error()
     # fully-connected stages: block width, operand width
-    assert lib.cueq_fc_combine(F32, F32, 4, p, 1, p, 1, p, 1, p, 1, p, 512, None) == -1
-    assert lib.cueq_fc_rowdot(F32, F32, 4, p, 1, p, 1, p, 1, 100, p, 1, None) == -2
+    assert lib.cueq_fc_combine(F32, F32, 4, p, 1, p, 1, p, 1, p, 1, p, 512, 0, None) == -1
+    assert lib.cueq_fc_rowdot(F32, F32, 4, p, 1, p, 1, p, 1, 100, p, 1, 0, None) == -2
