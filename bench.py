@@ -59,12 +59,12 @@ def make_inputs(torch, cue, N: int, E: int, dtype, seed: int = 0):
     return node.to(dtype), sh.to(dtype), w.to(dtype), senders, receivers, cot.to(dtype)
 
 
-def cpu_baseline(torch, cue, module, host, sample_edges: int, sample_nodes: int) -> dict:
+def cpu_baseline(torch, cue, module, host, sample_edges: int, sample_nodes: int, threads: int = 0) -> dict:
     """The CPU oracle (restatement of the reference's PyTorch executor) on a slice of the same inputs."""
     from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
 
     node, sh, w, senders, receivers, cot = host
-    cores = min(os.cpu_count() or 1, 16)
+    cores = threads if threads > 0 else min(os.cpu_count() or 1, 16)
     torch.set_num_threads(cores)
     spec = spec_from_polynomial(module.f._polynomial_orig)
     # a contiguous slice of edges (receivers stay sorted) with indices folded into the first sample_nodes rows
@@ -253,6 +253,7 @@ def main() -> int:
     ap.add_argument("--edges", type=int, default=100_000)
     ap.add_argument("--cpu-sample-edges", type=int, default=12000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (default: the box's share, at most 16)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     ap.add_argument("--deterministic", action="store_true",
@@ -369,7 +370,7 @@ def main() -> int:
         "kernels": per_kernel,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(torch, cue, m, host, min(args.cpu_sample_edges, E), min(200, N))
+        line["cpu_baseline"] = cpu_baseline(torch, cue, m, host, min(args.cpu_sample_edges, E), min(200, N), args.cpu_threads)
     print(json.dumps(line))
     return 0
 
