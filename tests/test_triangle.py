@@ -85,7 +85,8 @@ def rel_err(got, ref):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("direction", ["outgoing", "incoming"])
-@pytest.mark.parametrize("shape", [(1, 32, 32, None), (2, 48, 64, None), (1, 40, 128, 64), (1, 33, 32, None), (1, 20, 64, None)])
+@pytest.mark.parametrize("shape", [(1, 32, 32, None), (2, 48, 64, None), (1, 40, 128, 64), (1, 33, 32, None), (1, 20, 64, None),
+                                   (1, 66, 96, None)])
 def test_hip_path_matches_oracle(device, dtype, direction, shape):
     from cuequivariance_amd import cuet
 
