@@ -27,12 +27,22 @@ namespace cueq {
 static thread_local std::string g_error;
 
 // ---- registry of specialised kernels (filled by static initialisers of generated files) ----
+// (entries also arrive while the program runs: translation units compiled for a descriptor at first use register
+// themselves when their shared object is loaded, possibly while another thread creates a plan)
 static std::vector<const U1dSpec*>& spec_list() {
   static std::vector<const U1dSpec*> v;
   return v;
 }
-void register_u1d_spec(const U1dSpec* spec) { spec_list().push_back(spec); }
+static std::mutex& spec_mutex() {
+  static std::mutex m;
+  return m;
+}
+void register_u1d_spec(const U1dSpec* spec) {
+  std::lock_guard<std::mutex> lock(spec_mutex());
+  spec_list().push_back(spec);
+}
 const U1dSpec* find_u1d_spec(uint64_t hash) {
+  std::lock_guard<std::mutex> lock(spec_mutex());
   for (const U1dSpec* s : spec_list())
     if (s->hash == hash) return s;
   return nullptr;

@@ -108,6 +108,8 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
         # both math types up front (host-side tables only; device plans are made at the first launch), so that a
         # traced forward only reads this dictionary
         self._plans: dict = {dt: u1d.Uniform1dPlan(self.tables, dt, name=self.name) for dt in (torch.float32, torch.float64)}
+        for plan in self._plans.values():
+            plan.polynomial = polynomial  # (lets kernels for symmetric contractions be generated at first use)
 
     def __reduce__(self):
         return (

@@ -19,6 +19,7 @@ from __future__ import annotations
 
 import ctypes as C
 import threading
+import warnings
 import weakref
 from collections import OrderedDict
 from typing import List, Optional, Sequence
@@ -26,6 +27,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from .. import _lib
+from .. import jit as _jit
 from .._lib import BATCH_DIM_AUTO, BATCH_DIM_BATCHED, BATCH_DIM_INDEXED, BATCH_DIM_SHARED
 from ..tables import U1dTables
 
@@ -69,6 +71,8 @@ class Uniform1dPlan:
         self.math_dtype = math_dtype
         self._handles: dict[int, int] = {}
         self._backward: dict[tuple, "Uniform1dPlan"] = {}
+        self.jit_root = None  # for a backward plan: the forward plan, whose translation unit holds its kernels
+        self.polynomial = None  # the flattened polynomial the tables came from, when the caller has it
         self._lock = threading.Lock()
         # small integer under which a traced graph (torch.compile / export) names this plan
         with _traced_lock:
@@ -104,11 +108,21 @@ class Uniform1dPlan:
             if h is not None:
                 return h
             lib = _lib.load()
+            if _jit.enabled():  # kernels generated for this descriptor at first use (off by default)
+                root = self.jit_root or self
+                _jit.ensure_specialised(root.tables, _DTYPE_CODE[self.math_dtype], root.polynomial)
             desc, keep = _lib.make_desc(self.tables, _DTYPE_CODE[self.math_dtype])
             out = C.c_void_p()
             with torch.cuda.device(idx):
                 _lib.check(lib.cueq_u1d_plan_create(C.byref(desc), C.byref(out)), "cueq_u1d_plan_create")
             self._handles[idx] = out.value
+            if (not _jit.enabled() and self.jit_root is None and not lib.cueq_u1d_plan_info(out.value, None)
+                    and (_jit.is_channelwise(self.tables) or _jit.is_symmetric_contraction(self.polynomial))):
+                warnings.warn(
+                    f"uniform_1d[{self.name}]: no specialised kernels are built for this descriptor, the "
+                    "table-driven kernels (two orders of magnitude slower) will run; set CUEQ_AMD_JIT=1 or call "
+                    "cuequivariance_amd.jit.enable() to compile them at first use (a few seconds, cached on disk)",
+                    stacklevel=2)
             return out.value
 
     def __del__(self):
@@ -131,6 +145,7 @@ class Uniform1dPlan:
         plan = self._backward.get(needs_grad)
         if plan is None:
             plan = Uniform1dPlan(self.tables.backward(needs_grad), self.math_dtype, name=self.name + "_bwd")
+            plan.jit_root = self if self.jit_root is None else None
             self._backward[needs_grad] = plan
         return plan
 

@@ -1,0 +1,164 @@
+"""Descriptor-specialised kernels at first use.
+
+The library ships straight-line kernels for the descriptors listed in ``codegen/registry.py``; every other descriptor
+runs on the table-driven kernels, which are two to three orders of magnitude slower for channel-wise products.  With
+this module enabled (``CUEQ_AMD_JIT=1`` in the environment, or :func:`enable`), the first plan of a channel-wise
+descriptor that has no specialised kernels yet generates the same kind of translation unit the build generates
+(``codegen/channelwise.py``), compiles it with ``hipcc`` for gfx950 into a small shared object next to a cache key, and
+loads it: its static initialiser registers the kernels with the library (``cueq::register_u1d_spec``), and the plan that
+is created right afterwards finds them.  The reference's uniform-1d operator is compiled at first use as well
+(``SegmentedPolynomialFromUniform1dJit``, ``cuequivariance_torch/primitives/segmented_polynomial_uniform_1d.py:82``).
+
+Compiling takes a few seconds per descriptor and math type (tens for the largest), once per machine: shared objects are kept under
+``CUEQ_AMD_JIT_CACHE`` (default ``~/.cache/cuequivariance_amd``), keyed by the table hash and the library build.
+Off by default, so that a test suite that touches dozens of small descriptors does not compile each of them.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+from pathlib import Path
+from typing import Optional
+
+from . import _lib
+from .tables import U1dTables
+
+__all__ = ["enable", "enabled", "ensure_specialised", "is_channelwise", "cache_dir"]
+
+_enabled: Optional[bool] = None
+_lock = threading.Lock()
+_loaded: dict = {}  # table hash -> ctypes handle (kept: the registered kernels live in the object)
+_failed: set = set()
+
+PKG = Path(__file__).resolve().parent
+CSRC = PKG / "csrc"
+INCLUDE = PKG.parent / "include"
+
+
+def enable(on: bool = True) -> None:
+    """Turn compilation at first use on or off for this process (overrides ``CUEQ_AMD_JIT``)."""
+    global _enabled
+    _enabled = bool(on)
+
+
+def enabled() -> bool:
+    if _enabled is not None:
+        return _enabled
+    return os.environ.get("CUEQ_AMD_JIT", "0") not in ("", "0", "false", "False")
+
+
+def cache_dir() -> Path:
+    root = os.environ.get("CUEQ_AMD_JIT_CACHE")
+    base = Path(root) if root else Path.home() / ".cache" / "cuequivariance_amd"
+    st = _lib.LIB_PATH.stat()
+    build = hashlib.sha1(f"{_lib.LIB_PATH}:{st.st_size}:{st.st_mtime_ns}".encode()).hexdigest()[:12]
+    d = base / f"jit-{build}"
+    d.mkdir(parents=True, exist_ok=True)
+    return d
+
+
+def is_channelwise(t: U1dTables) -> bool:
+    return (t.num_inputs == 3 and t.num_outputs == 1 and tuple(t.operations) == (0, 1, 2, 3) and tuple(t.buffer_dim) == (1, 1, 0, 1)
+            and len(t.num_operands) == 1)
+
+
+def _tuning(st, T: str) -> dict:
+    """Wavefronts per SIMD and prefetching from a register estimate (accumulators + operand sets; doubles take two)."""
+    per = 2 if T == "double" else 1
+    operands = st.nseg_x1 + st.nseg_w + 4
+    fwd_two_sets = (st.nseg_out + 2 * operands + 30) * per
+    fwd_one_set = (st.nseg_out + operands + 30) * per
+    if fwd_two_sets <= 250:
+        fwd = dict(fwd_waves=2, fwd_prefetch=True)
+    elif fwd_one_set <= 250:
+        fwd = dict(fwd_waves=2, fwd_prefetch=False)
+    else:
+        fwd = dict(fwd_waves=1, fwd_prefetch=fwd_two_sets <= 500)
+    bwd_regs = (st.nseg_out + 2 * st.nseg_x1 + st.nseg_w + st.nseg_x2 + 30) * per
+    return dict(fwd, bwd_waves=2 if bwd_regs <= 250 else 1)
+
+
+def _has_spec(t: U1dTables, code: int) -> bool:
+    desc, keep = _lib.make_desc(t, code)
+    return bool(_lib.load().cueq_u1d_desc_info(C.byref(desc), None))
+
+
+def is_symmetric_contraction(poly) -> bool:
+    """``w[u], x[u] (one to three times) -> out[u]`` in every operation, one uniform extent: the form
+    ``codegen/symmetric.py`` generates kernels for."""
+    if poly is None or poly.num_inputs != 2 or poly.num_outputs != 1 or not poly.operations:
+        return False
+    extents = {s for ope in poly.operands for s in ope.segments}
+    if len(extents) != 1 or len(next(iter(extents))) != 1:
+        return False
+    for ope, stp in poly.operations:
+        bufs = tuple(ope.buffers)
+        if len(bufs) < 3 or len(bufs) > 5 or bufs[0] != 0 or bufs[-1] != 2 or any(b != 1 for b in bufs[1:-1]):
+            return False
+    return True
+
+
+def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None) -> bool:
+    """Make sure specialised kernels for ``tables`` (forward) and for its backward are registered with the library,
+    compiling them if this module is enabled and the descriptor is a channel-wise product or (given the flattened
+    ``polynomial`` the tables came from) a symmetric contraction.  Returns whether they are."""
+    if _has_spec(tables, math_code):
+        return True
+    if not enabled() or not (is_channelwise(tables) or is_symmetric_contraction(polynomial)):
+        return False
+    key = tables.content_hash(math_code)
+    with _lock:
+        if key in _loaded or _has_spec(tables, math_code):
+            return True
+        if key in _failed:
+            return False
+        try:
+            _loaded[key] = _build_and_load(tables, math_code, key, polynomial)
+        except Exception as e:  # compilation is an optimisation: the table-driven kernels still serve the plan
+            _failed.add(key)
+            print(f"[cueq_amd.jit] specialised kernels for descriptor {key:016x} not built: {e}", file=sys.stderr, flush=True)
+            return False
+    return _has_spec(tables, math_code)
+
+
+def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None):
+    from .codegen import channelwise as cw
+    from .codegen import symmetric as sc
+
+    T = "float" if code == _lib.F32 else "double"
+    name = f"jit_{key:016x}"
+    so = cache_dir() / f"u1d_{name}_{T}.so"
+    if not so.exists():
+        if is_channelwise(t):
+            _, paths = t.operation(0)
+            st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
+            tb = t.backward((True, True, True))
+            src = cw.emit_unit(st, T, name, key, tb.content_hash(code), **_tuning(st, T))
+            what = f"{st.num_paths} paths, extent {st.extent}"
+        else:
+            st = sc.analyze(polynomial)
+            bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
+            src = sc.emit_unit(st, T, name, key, bwd)
+            what = f"symmetric contraction, {len(st.terms)} folded terms, extent {st.extent}"
+        hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+        with tempfile.TemporaryDirectory(dir=so.parent) as tmp:
+            hip = Path(tmp) / f"u1d_{name}_{T}.hip"
+            hip.write_text(src)
+            out = Path(tmp) / so.name
+            cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Xclang", "-target-feature", "-Xclang",
+                   "-packed-fp32-ops", "-Wno-unused-command-line-argument", f"-I{INCLUDE}", f"-I{CSRC}", str(hip), "-o", str(out),
+                   f"-L{_lib.LIB_PATH.parent}", f"-l:{_lib.LIB_PATH.name}", f"-Wl,-rpath,{_lib.LIB_PATH.parent}"]
+            print(f"[cueq_amd.jit] compiling kernels for descriptor {key:016x} ({T}, {what}) ...", file=sys.stderr, flush=True)
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError(f"hipcc failed:\n{r.stderr[-2000:]}")
+            os.replace(out, so)  # atomic: another process may be compiling the same descriptor
+    _lib.load()  # the library the object links against is already in the process
+    return C.CDLL(str(so))
