@@ -17,6 +17,7 @@ those kernels refuse go through ``cueq_seg_gemm`` / ``cueq_seg_outer`` / ``cueq_
 from __future__ import annotations
 
 import ctypes as C
+import itertools
 import threading
 import weakref
 from typing import Dict, List, Optional
@@ -637,6 +638,7 @@ class _IndexedDenseFunction(torch.autograd.Function):
 # Forward and backward of the two shared-weight functions as opaque operators.  They call the static methods above with
 # a plain object in place of the autograd context; the module travels as a small integer.
 _traced_modules: dict = {}
+_traced_ids = itertools.count()
 _traced_lock = threading.Lock()
 _FUNCTIONS = (_DenseFunction, _FcFunction)
 
@@ -743,7 +745,7 @@ class SegmentedPolynomialDense(nn.Module):
         self.fc_plan = _FcPlan(self.paths, self.input_sizes[2]) if self.has_x2 else None
         self._merged: dict = {}
         with _traced_lock:  # the integer under which a traced graph names this module
-            self.traced_id = len(_traced_modules)
+            self.traced_id = next(_traced_ids)
             _traced_modules[self.traced_id] = weakref.ref(self)
 
     def tiled(self, dtype, A: torch.Tensor, Cout: torch.Tensor) -> bool:

@@ -18,6 +18,7 @@ Everything executes through the C ABI in ``libcueq_amd.so``; CPU tensors are rej
 from __future__ import annotations
 
 import ctypes as C
+import itertools
 import threading
 import warnings
 import weakref
@@ -49,6 +50,7 @@ _DTYPE_CODE = {
 
 
 _traced_plans: dict = {}
+_traced_ids = itertools.count()
 _PLAIN_TENSORS = (torch.Tensor, torch.nn.Parameter)
 _traced_lock = threading.Lock()
 
@@ -76,7 +78,7 @@ class Uniform1dPlan:
         self._lock = threading.Lock()
         # small integer under which a traced graph (torch.compile / export) names this plan
         with _traced_lock:
-            self.traced_id = len(_traced_plans)
+            self.traced_id = next(_traced_ids)  # (never reused: entries of plans that are gone are dropped)
             _traced_plans[self.traced_id] = weakref.ref(self)
 
     def __getattr__(self, item):
