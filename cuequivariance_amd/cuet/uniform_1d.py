@@ -73,6 +73,7 @@ class Uniform1dPlan:
         self.math_dtype = math_dtype
         self._handles: dict[int, int] = {}
         self._backward: dict[tuple, "Uniform1dPlan"] = {}
+        self._choice: dict = {}
         self.jit_root = None  # for a backward plan: the forward plan, whose translation unit holds its kernels
         self.polynomial = None  # the flattened polynomial the tables came from, when the caller has it
         self._lock = threading.Lock()
@@ -150,6 +151,24 @@ class Uniform1dPlan:
             plan.jit_root = self if self.jit_root is None else None
             self._backward[needs_grad] = plan
         return plan
+
+
+def _backward_choice(plan: Uniform1dPlan, needs: tuple, device: torch.device) -> tuple:
+    """The gradient plan to run for ``needs``: the exact one when it has specialised kernels (or nothing better exists),
+    else the plan for all inputs when that one has them - computing a gradient nobody asked for costs far less than
+    leaving the specialised kernels.  Returns ``(plan, needs it computes)``; remembered per plan."""
+    key = (needs, device.index)
+    hit = plan._choice.get(key)
+    if hit is None:
+        exact = plan.backward_plan(needs)
+        hit = (exact, needs)
+        if not all(needs) and device.type == "cuda" and not exact.specialised(device):
+            everything = (True,) * len(needs)
+            full = plan.backward_plan(everything)
+            if full.specialised(device):
+                hit = (full, everything)
+        plan._choice[key] = hit
+    return hit
 
 
 _plan_cache: "OrderedDict[tuple, Uniform1dPlan]" = OrderedDict()
@@ -310,7 +329,7 @@ class _Uniform1dFunction(torch.autograd.Function):
         needs = tuple(ctx.needs_input_grad[3: 3 + nin])
         if not any(needs):
             return (None,) * (3 + len(tensors))
-        bplan = plan.backward_plan(needs)
+        bplan, computed = _backward_choice(plan, needs, inputs[0].device)
         cots = []
         for o, g in enumerate(grad_outputs):
             b = nin + o
@@ -319,7 +338,7 @@ class _Uniform1dFunction(torch.autograd.Function):
                 g = torch.zeros((cfg.rows[b], plan.width(b)), device=inputs[0].device,
                                 dtype=plan.math_dtype if src < 0 else inputs[src].dtype)
             cots.append(g)
-        flagged = [i for i, n in enumerate(needs) if n]
+        flagged = [i for i, n in enumerate(computed) if n]
         modes = list(cfg.modes) + [cfg.modes[i] for i in flagged]
         index_of = list(cfg.index_of) + [cfg.index_of[i] for i in flagged]
         rows = list(cfg.rows) + [cfg.rows[i] for i in flagged]
@@ -327,7 +346,8 @@ class _Uniform1dFunction(torch.autograd.Function):
         grads = _Uniform1dFunction.apply(bplan, bcfg, num_index, *inputs, *cots, *indices)
         out = [None, None, None] + [None] * len(tensors)
         for g, i in zip(grads, flagged):
-            out[3 + i] = g
+            if needs[i]:
+                out[3 + i] = g
         return tuple(out)
 
 
@@ -372,7 +392,7 @@ def _u1d_backward(ctx, grad_outputs):
     needs = tuple(bool(f) for f in flags[:nin])
     grads: List[Optional[torch.Tensor]] = [None] * len(tensors)
     if any(needs):
-        bplan = plan.backward_plan(needs)
+        bplan, computed = _backward_choice(plan, needs, inputs[0].device)
         cots = []
         for o, g in enumerate(grad_outputs):
             if g is None:
@@ -380,11 +400,12 @@ def _u1d_backward(ctx, grad_outputs):
                 g = torch.zeros((rows[nin + o], plan.width(nin + o)), device=inputs[0].device,
                                 dtype=plan.math_dtype if src < 0 else inputs[src].dtype)
             cots.append(g)
-        flagged = [i for i, n in enumerate(needs) if n]
+        flagged = [i for i, n in enumerate(computed) if n]
         got = _u1d_launch_op(bplan.traced_id, list(modes) + [modes[i] for i in flagged], list(index_of) + [index_of[i] for i in flagged],
                              list(rows) + [rows[i] for i in flagged], batch, [*inputs, *cots, *indices])
         for g, i in zip(got, flagged):
-            grads[i] = g
+            if needs[i]:
+                grads[i] = g
     return None, None, None, None, None, grads
 
 

@@ -425,3 +425,34 @@ def test_spherical_harmonics_module(device, dtype):
         (grad,) = torch.autograd.grad(out, [b], cot.to(device))
         assert_close(out, ref, TOL[dtype], "Y")
         assert_close(grad, ref_grad, 4 * TOL[dtype], "dY/dx")
+
+
+@pytest.mark.gpu
+def test_gradient_subset_runs_on_the_specialised_full_backward(device):
+    """Only x1 and x2 ask for gradients (weights fixed, as in inference with forces): there are no specialised kernels for
+    that subset, so the specialised kernels for all three gradients run and the unwanted one is dropped; against the
+    oracle."""
+    from cuequivariance_amd.cuet.uniform_1d import _backward_choice
+
+    m = cw_module("32x0e+32x1o+32x2e", "0e+1o+2e", ["0e", "1o", "2e"])
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+    g = torch.Generator().manual_seed(77)
+    N, Z = 40, 600
+    x1 = torch.randn(N, m.irreps_in1.dim, generator=g)
+    x2 = torch.randn(Z, m.irreps_in2.dim, generator=g)
+    w = torch.randn(Z, m.weight_numel, generator=g)
+    snd = torch.randint(0, N, (Z,), generator=g, dtype=torch.int32)
+    rcv = torch.sort(torch.randint(0, N, (Z,), generator=g, dtype=torch.int32))[0]
+    cot = torch.randn(N, m.irreps_out.dim, generator=g)
+    a = [w.clone(), x1.clone().requires_grad_(True), x2.clone().requires_grad_(True)]
+    ref = naive_segmented_polynomial(spec, a, {1: snd}, {0: N}, {0: rcv})[0]
+    ref_grads = torch.autograd.grad(ref, a[1:], cot)
+    b = [w.to(device), x1.to(device).requires_grad_(True), x2.to(device).requires_grad_(True)]
+    out = m(b[1], b[2], b[0], indices_1=snd.to(device), indices_out=rcv.to(device), size_out=N)
+    grads = torch.autograd.grad(out, b[1:], cot.to(device))
+    for name, p, q in zip(("dx1", "dx2"), ref_grads, grads):
+        assert_close(q, p, 1e-5, name)
+    plan = m.f.m._plan(torch.float32)
+    chosen, computed = _backward_choice(plan, (False, True, True), device)
+    assert computed == (True, True, True) and chosen.specialised(device)
+    assert not plan.backward_plan((False, True, True)).specialised(device)
