@@ -113,7 +113,7 @@ class Uniform1dPlan:
             lib = _lib.load()
             if _jit.enabled():  # kernels generated for this descriptor at first use (off by default)
                 root = self.jit_root or self
-                _jit.ensure_specialised(root.tables, _DTYPE_CODE[self.math_dtype], root.polynomial)
+                _jit.ensure_plan(self.tables, _DTYPE_CODE[self.math_dtype], root.tables, root.polynomial)
             desc, keep = _lib.make_desc(self.tables, _DTYPE_CODE[self.math_dtype])
             out = C.c_void_p()
             with torch.cuda.device(idx):

@@ -30,7 +30,7 @@ from typing import Optional
 from . import _lib
 from .tables import U1dTables
 
-__all__ = ["enable", "enabled", "ensure_specialised", "is_channelwise", "cache_dir"]
+__all__ = ["enable", "enabled", "ensure_plan", "ensure_specialised", "is_channelwise", "is_symmetric_contraction", "cache_dir"]
 
 _enabled: Optional[bool] = None
 _lock = threading.Lock()
@@ -105,13 +105,32 @@ def is_symmetric_contraction(poly) -> bool:
     return True
 
 
-def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None) -> bool:
-    """Make sure specialised kernels for ``tables`` (forward) and for its backward are registered with the library,
-    compiling them if this module is enabled and the descriptor is a channel-wise product or (given the flattened
-    ``polynomial`` the tables came from) a symmetric contraction.  Returns whether they are."""
+def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTables] = None, root_polynomial=None) -> bool:
+    """Kernels for one plan: first the family unit of its root (the forward plan of a channel-wise product or symmetric
+    contraction holds the kernels of its backward plans too), then, if the plan still has none, a unit of its own from
+    the general generator (``codegen/general.py``: second derivatives, harmonics, flattened dense products, ...)."""
     if _has_spec(tables, math_code):
         return True
-    if not enabled() or not (is_channelwise(tables) or is_symmetric_contraction(polynomial)):
+    if not enabled():
+        return False
+    if root_tables is not None and (is_channelwise(root_tables) or is_symmetric_contraction(root_polynomial)):
+        ensure_specialised(root_tables, math_code, root_polynomial)
+        if _has_spec(tables, math_code):
+            return True
+    return ensure_specialised(tables, math_code, None, general=True)
+
+
+def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, general: bool = False) -> bool:
+    """Make sure specialised kernels for ``tables`` (forward) and for its backward are registered with the library,
+    compiling them if this module is enabled and the descriptor is a channel-wise product or (given the flattened
+    ``polynomial`` the tables came from) a symmetric contraction - or, with ``general``, anything the general generator
+    covers.  Returns whether they are."""
+    from .codegen import general as gen
+
+    if _has_spec(tables, math_code):
+        return True
+    family = is_channelwise(tables) or is_symmetric_contraction(polynomial)
+    if not enabled() or not (family or (general and gen.supported(tables))):
         return False
     key = tables.content_hash(math_code)
     with _lock:
@@ -136,7 +155,12 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None):
     name = f"jit_{key:016x}"
     so = cache_dir() / f"u1d_{name}_{T}.so"
     if not so.exists():
-        if is_channelwise(t):
+        if not (is_channelwise(t) or is_symmetric_contraction(polynomial)):
+            from .codegen import general as gen
+
+            src = gen.emit_unit(t, T, name, key)
+            what = f"general plan, {sum(t.num_paths)} paths, extent {t.operand_extent}"
+        elif is_channelwise(t):
             _, paths = t.operation(0)
             st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
             tb = t.backward((True, True, True))

@@ -453,6 +453,10 @@ def test_gradient_subset_runs_on_the_specialised_full_backward(device):
     for name, p, q in zip(("dx1", "dx2"), ref_grads, grads):
         assert_close(q, p, 1e-5, name)
     plan = m.f.m._plan(torch.float32)
+    from cuequivariance_amd import jit
+
     chosen, computed = _backward_choice(plan, (False, True, True), device)
-    assert computed == (True, True, True) and chosen.specialised(device)
-    assert not plan.backward_plan((False, True, True)).specialised(device)
+    assert chosen.specialised(device)
+    if not jit.enabled():  # (with kernels compiled at first use the subset gets a unit of its own)
+        assert computed == (True, True, True)
+        assert not plan.backward_plan((False, True, True)).specialised(device)

@@ -102,3 +102,53 @@ def test_jit_symmetric_contraction_matches_generic(device, jit_on, monkeypatch):
     want = step()
     for name, u, v in zip(("out", "dw", "dx"), got, want):
         assert (u - v).abs().max().item() <= 1e-5 * v.abs().max().item(), name
+
+
+@pytest.mark.gpu
+def test_general_generator_second_derivative_and_harmonics(device, jit_on):
+    """Plans outside the two generated families get a unit of their own from the general generator: the backward of the
+    backward of a channel-wise product (double backward against the CPU oracle's autograd) and spherical harmonics (a plan
+    without channel mode: a lane per row)."""
+    from cuequivariance_amd import cuet
+
+    i1, i2 = cue.Irreps("O3", "24x0e+24x1o"), cue.Irreps("O3", "0e+1o")
+    m = cuet.ChannelWiseTensorProduct(i1, i2, ["0e", "1o"], layout=cue.ir_mul, shared_weights=False, internal_weights=False,
+                                      device=device, dtype=torch.float64)
+    g = torch.Generator().manual_seed(9)
+    N, Z = 13, 90
+    x1 = torch.randn(N, i1.dim, generator=g, dtype=torch.float64)
+    x2 = torch.randn(Z, i2.dim, generator=g, dtype=torch.float64)
+    w = torch.randn(Z, m.weight_numel, generator=g, dtype=torch.float64)
+    snd = torch.randint(0, N, (Z,), generator=g, dtype=torch.int32)
+    rcv = torch.sort(torch.randint(0, N, (Z,), generator=g, dtype=torch.int32))[0]
+    cot = torch.randn(N, m.irreps_out.dim, generator=g, dtype=torch.float64)
+    v = torch.randn(Z, i2.dim, generator=g, dtype=torch.float64)
+
+    def second(w_, x1_, x2_, fwd):
+        out = fwd(w_, x1_, x2_)
+        (gx2,) = torch.autograd.grad(out, [x2_], cot.to(out.device), create_graph=True)
+        return torch.autograd.grad((gx2 * v.to(out.device)).sum(), [w_, x1_, x2_], allow_unused=True)
+
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+    a = [t.clone().requires_grad_(True) for t in (w, x1, x2)]
+    want = second(*a, lambda w_, x1_, x2_: naive_segmented_polynomial(spec, [w_, x1_, x2_], {1: snd}, {0: N}, {0: rcv})[0])
+    b = [t.clone().to(device).requires_grad_(True) for t in (w, x1, x2)]
+    got = second(*b, lambda w_, x1_, x2_: m(x1_, x2_, w_, indices_1=snd.to(device), indices_out=rcv.to(device), size_out=N))
+    for p, q in zip(want, got):
+        if p is None:
+            assert q is None or q.abs().max().item() == 0
+        else:
+            assert (q.cpu() - p).abs().max().item() <= 1e-12 * max(p.abs().max().item(), 1e-30)
+    plan = m.f.m._plan(torch.float64)
+    assert plan.specialised(device)
+
+    sh = cuet.SphericalHarmonics([0, 1, 2, 3], normalize=False, device=device)
+    vec = torch.randn(1000, 3, generator=g, dtype=torch.float64)
+    y = sh(vec.to(device))
+    assert sh.f.m._plan(torch.float64).specialised(device)
+    # closed forms: Y_0 = 1, Y_1 = sqrt(3) x, and sum_m Y_lm^2 = (2 l + 1) |x|^(2 l) (component normalisation)
+    r2 = (vec * vec).sum(1)
+    assert torch.allclose(y[:, 0].cpu(), torch.ones(1000, dtype=torch.float64), atol=1e-12)
+    assert torch.allclose(y[:, 1:4].cpu(), 3 ** 0.5 * vec, atol=1e-12)
+    for l, lo in ((2, 4), (3, 9)):
+        assert torch.allclose((y[:, lo:lo + 2 * l + 1].cpu() ** 2).sum(1), (2 * l + 1) * r2 ** l, rtol=1e-11)
