@@ -1,17 +1,19 @@
 """Descriptor-specialised kernels at first use.
 
 The library ships straight-line kernels for the descriptors listed in ``codegen/registry.py``; every other descriptor
-runs on the table-driven kernels, which are two to three orders of magnitude slower for channel-wise products.  With
-this module enabled (``CUEQ_AMD_JIT=1`` in the environment, or :func:`enable`), the first plan of a channel-wise
-descriptor that has no specialised kernels yet generates the same kind of translation unit the build generates
-(``codegen/channelwise.py``), compiles it with ``hipcc`` for gfx950 into a small shared object next to a cache key, and
-loads it: its static initialiser registers the kernels with the library (``cueq::register_u1d_spec``), and the plan that
+would run on the table-driven kernels, which are two orders of magnitude slower.  Unless this module is switched off
+(``CUEQ_AMD_JIT=0`` in the environment, or ``enable(False)``), the first plan of a descriptor that has no specialised
+kernels yet generates a translation unit - the same kind the build generates for channel-wise products
+(``codegen/channelwise.py``) and symmetric contractions (``codegen/symmetric.py``), a general straight-line one
+(``codegen/general.py``) for anything else -, compiles it with ``hipcc`` for gfx950 into a small shared object next to a
+cache key, and loads it: its static initialiser registers the kernels with the library (``cueq::register_u1d_spec``), and the plan that
 is created right afterwards finds them.  The reference's uniform-1d operator is compiled at first use as well
 (``SegmentedPolynomialFromUniform1dJit``, ``cuequivariance_torch/primitives/segmented_polynomial_uniform_1d.py:82``).
 
 Compiling takes a few seconds per descriptor and math type (tens for the largest), once per machine: shared objects are kept under
 ``CUEQ_AMD_JIT_CACHE`` (default ``~/.cache/cuequivariance_amd``), keyed by the table hash and the library build.
-Off by default, so that a test suite that touches dozens of small descriptors does not compile each of them.
+When ``hipcc`` is missing or the cache cannot be written the plan runs on the table-driven kernels and says so once.
+(The test suite switches it off except where it is the subject: dozens of small descriptors would each be compiled.)
 """
 
 from __future__ import annotations
@@ -51,7 +53,7 @@ def enable(on: bool = True) -> None:
 def enabled() -> bool:
     if _enabled is not None:
         return _enabled
-    return os.environ.get("CUEQ_AMD_JIT", "0") not in ("", "0", "false", "False")
+    return os.environ.get("CUEQ_AMD_JIT", "1") not in ("", "0", "false", "False")
 
 
 def cache_dir() -> Path:

@@ -19,3 +19,14 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True, scope="session")
+def _kernels_at_first_use_off():
+    """Compilation at first use is on for users; the suite keeps it off (the table-driven kernels stay covered and dozens
+    of small descriptors are not compiled), ``tests/test_jit.py`` switches it on for its cases."""
+    from cuequivariance_amd import jit
+
+    jit.enable(False)
+    yield
+
