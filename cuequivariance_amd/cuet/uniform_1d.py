@@ -162,10 +162,15 @@ def _backward_choice(plan: Uniform1dPlan, needs: tuple, device: torch.device) ->
     if hit is None:
         exact = plan.backward_plan(needs)
         hit = (exact, needs)
-        if not all(needs) and device.type == "cuda" and not exact.specialised(device):
+        if not all(needs) and device.type == "cuda":
             everything = (True,) * len(needs)
             full = plan.backward_plan(everything)
-            if full.specialised(device):
+            if _jit.is_channelwise(plan.tables):
+                # the fused backward of the family reads every operand once for all three gradients: preferred over a
+                # unit per gradient from the general generator
+                if full.specialised(device):
+                    hit = (full, everything)
+            elif not exact.specialised(device) and full.specialised(device):
                 hit = (full, everything)
         plan._choice[key] = hit
     return hit
