@@ -267,7 +267,8 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
-              "the path shards over receiver ranges without exchange in forward, see DESIGN.md", file=sys.stderr)
+              "the path would shard over receiver ranges (no exchange in the forward, one reduce-scatter of the node gradient in the backward)",
+              file=sys.stderr)
         return 2
     if args.deterministic:
         os.environ["CUEQ_DETERMINISTIC"] = "1"
