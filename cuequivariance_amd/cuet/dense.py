@@ -479,6 +479,14 @@ class _FcFunction(torch.autograd.Function):
             with torch.cuda.device(dev):
                 stream = torch.cuda.current_stream(dev).cuda_stream
                 code, es = _DTYPE_CODE[dtype], x1d.element_size()
+                unit = mod.fused_unit(dtype, x1d, out)
+                if unit is not None:
+                    if unit.fcj_fwd(Z, wd.data_ptr(), x1d.data_ptr(), x1d.stride(0), x2d.data_ptr(), x2d.stride(0), out.data_ptr(),
+                                    out.stride(0), stream) != 0:
+                        raise RuntimeError("fused fully connected forward: launch failed")
+                    ctx.mod = mod
+                    ctx.save_for_backward(w, x1, x2)
+                    return out
                 T = torch.empty(Z, plan.t_cols, dtype=torch.float32, device=dev)
                 tables = plan.device(dev)
                 for (K, N), tab in tables["t"].items():
@@ -511,7 +519,15 @@ class _FcFunction(torch.autograd.Function):
                 gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
             if need_x2:
                 gx2 = torch.zeros_like(x2d)
-            if (need_x1 or need_x2) and Z > 0:
+            unit = mod.fused_unit(dtype, x1d, g) if Z > 0 and (need_x1 or need_x2) else None
+            if unit is not None:
+                if need_x1 and unit.fcj_dx1(Z, wd.data_ptr(), g.data_ptr(), g.stride(0), x2d.data_ptr(), x2d.stride(0), gx1.data_ptr(),
+                                            gx1.stride(0), stream) != 0:
+                    raise RuntimeError("fused fully connected gradient (first operand): launch failed")
+                if need_x2 and unit.fcj_dx2(Z, wd.data_ptr(), x1d.data_ptr(), x1d.stride(0), x2d.data_ptr(), x2d.stride(0), g.data_ptr(),
+                                            g.stride(0), gx2.data_ptr(), gx2.stride(0), stream) != 0:
+                    raise RuntimeError("fused fully connected gradient (second operand): launch failed")
+            elif (need_x1 or need_x2) and Z > 0:
                 G = torch.empty(Z, plan.g_cols, dtype=torch.float32, device=dev)
                 for (K, N), tab in tables["g"].items():
                     # G[:, gq : + K] = g[:, c_off : + N] @ W_p^T for every row (c_off, w_off, gq); W_p (K x N) is
@@ -744,9 +760,25 @@ class SegmentedPolynomialDense(nn.Module):
         self.weight_blocks = sorted({(p.w_off, p.K, p.N) for p in self.paths})
         self.fc_plan = _FcPlan(self.paths, self.input_sizes[2]) if self.has_x2 else None
         self._merged: dict = {}
+        self._fused: dict = {}
         with _traced_lock:  # the integer under which a traced graph names this module
             self.traced_id = next(_traced_ids)
             _traced_modules[self.traced_id] = weakref.ref(self)
+
+    def fused_unit(self, dtype, *row_tensors):
+        """The kernels generated for this product (``codegen/fullyconnected.py``; compiled at first use), or ``None``:
+        then the table-driven GEMMs run.  Rows are read and written in 16-byte pieces."""
+        if dtype not in (torch.float32, torch.bfloat16) or not self.has_x2:
+            return None
+        if any(t.data_ptr() % 16 or (t.stride(0) * t.element_size()) % 16 or t.stride(1) != 1 for t in row_tensors):
+            return None
+        from .. import jit
+
+        key = (dtype, jit.enabled())
+        if key not in self._fused:
+            self._fused[key] = jit.fully_connected_unit(self.paths, self.input_sizes[2], self.input_sizes[1], self.out_size,
+                                                          "float" if dtype == torch.float32 else "uint16_t")
+        return self._fused[key]
 
     def tiled(self, dtype, A: torch.Tensor, Cout: torch.Tensor) -> bool:
         """The tiled kernel serves fp32 / bf16 contractions without a per-row scale."""

@@ -32,7 +32,7 @@ from typing import Optional
 from . import _lib
 from .tables import U1dTables
 
-__all__ = ["enable", "enabled", "ensure_plan", "ensure_specialised", "is_channelwise", "is_symmetric_contraction", "cache_dir"]
+__all__ = ["enable", "enabled", "ensure_plan", "ensure_specialised", "fully_connected_unit", "is_channelwise", "is_symmetric_contraction", "cache_dir"]
 
 _enabled: Optional[bool] = None
 _lock = threading.Lock()
@@ -173,18 +173,58 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None):
             bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
             src = sc.emit_unit(st, T, name, key, bwd)
             what = f"symmetric contraction, {len(st.terms)} folded terms, extent {st.extent}"
-        hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-        with tempfile.TemporaryDirectory(dir=so.parent) as tmp:
-            hip = Path(tmp) / f"u1d_{name}_{T}.hip"
-            hip.write_text(src)
-            out = Path(tmp) / so.name
-            cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Xclang", "-target-feature", "-Xclang",
-                   "-packed-fp32-ops", "-Wno-unused-command-line-argument", f"-I{INCLUDE}", f"-I{CSRC}", str(hip), "-o", str(out),
-                   f"-L{_lib.LIB_PATH.parent}", f"-l:{_lib.LIB_PATH.name}", f"-Wl,-rpath,{_lib.LIB_PATH.parent}"]
-            print(f"[cueq_amd.jit] compiling kernels for descriptor {key:016x} ({T}, {what}) ...", file=sys.stderr, flush=True)
-            r = subprocess.run(cmd, capture_output=True, text=True)
-            if r.returncode != 0:
-                raise RuntimeError(f"hipcc failed:\n{r.stderr[-2000:]}")
-            os.replace(out, so)  # atomic: another process may be compiling the same descriptor
+        _compile(src, so, f"descriptor {key:016x} ({T}, {what})")
     _lib.load()  # the library the object links against is already in the process
     return C.CDLL(str(so))
+
+
+def _compile(src: str, so: Path, what: str, link_library: bool = True) -> None:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    with tempfile.TemporaryDirectory(dir=so.parent) as tmp:
+        hip = Path(tmp) / (so.stem + ".hip")
+        hip.write_text(src)
+        out = Path(tmp) / so.name
+        cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Xclang", "-target-feature", "-Xclang",
+               "-packed-fp32-ops", "-Wno-unused-command-line-argument", f"-I{INCLUDE}", f"-I{CSRC}", str(hip), "-o", str(out)]
+        if link_library:
+            cmd += [f"-L{_lib.LIB_PATH.parent}", f"-l:{_lib.LIB_PATH.name}", f"-Wl,-rpath,{_lib.LIB_PATH.parent}"]
+        print(f"[cueq_amd.jit] compiling kernels for {what} ...", file=sys.stderr, flush=True)
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed:\n{r.stderr[-2000:]}")
+        os.replace(out, so)  # atomic: another process may be compiling the same descriptor
+
+
+def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str):
+    """The fused kernels of ``codegen/fullyconnected.py`` for one fully connected product and element type (``float`` or
+    ``uint16_t`` for bfloat16), compiled at first use and loaded: a ``ctypes`` handle with ``fcj_fwd``, ``fcj_dx1`` and
+    ``fcj_dx2``, or ``None`` when this module is off, the product is outside what the generator covers, or the compiler
+    failed (the caller then runs the table-driven GEMMs)."""
+    from .codegen import fullyconnected as fc
+
+    if not enabled() or not fc.supported(paths, n2, width_in, width_out, 4 if T == "float" else 2):
+        return None
+    src = fc.emit_unit(paths, n2, width_in, width_out, T)
+    key = "fc_" + hashlib.sha1(src.encode()).hexdigest()[:16]
+    with _lock:
+        if key in _loaded:
+            return _loaded[key]
+        if key in _failed:
+            return None
+        try:
+            so = cache_dir() / f"{key}_{T}.so"
+            if not so.exists():
+                _compile(src, so, f"a fully connected product ({T}, {len(paths)} paths, {width_in} x {n2} -> {width_out})", link_library=False)
+            h = C.CDLL(str(so))
+            i64, vp = C.c_int64, C.c_void_p
+            h.fcj_fwd.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp]
+            h.fcj_dx1.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp]
+            h.fcj_dx2.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp]
+            for f in (h.fcj_fwd, h.fcj_dx1, h.fcj_dx2):
+                f.restype = C.c_int
+            _loaded[key] = h
+            return h
+        except Exception as e:
+            _failed.add(key)
+            print(f"[cueq_amd.jit] fused fully connected kernels not built: {e}", file=sys.stderr, flush=True)
+            return None

@@ -152,3 +152,72 @@ def test_general_generator_second_derivative_and_harmonics(device, jit_on):
     assert torch.allclose(y[:, 1:4].cpu(), 3 ** 0.5 * vec, atol=1e-12)
     for l, lo in ((2, 4), (3, 9)):
         assert torch.allclose((y[:, lo:lo + 2 * l + 1].cpu() ** 2).sum(1), (2 * l + 1) * r2 ** l, rtol=1e-11)
+
+
+def _dense_of(module):
+    return next(x for x in module.modules() if type(x).__name__ == "SegmentedPolynomialDense")
+
+
+def test_fully_connected_generator_limits():
+    """What the fused fully connected generator takes: multiplicities that are multiples of 32 up to 128, rows of at most
+    256 columns; the source it emits holds the three kernels and their C entry points."""
+    from cuequivariance_amd import cuet
+    from cuequivariance_amd.codegen import fullyconnected as fc
+
+    def dense(i1, i2, i3):
+        return _dense_of(cuet.FullyConnectedTensorProduct(cue.Irreps("O3", i1), cue.Irreps("O3", i2), cue.Irreps("O3", i3),
+                                                          layout=cue.ir_mul, internal_weights=False))
+
+    d = dense("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o")
+    assert fc.supported(d.paths, 9, 256, 256, 4) and fc.supported(d.paths, 9, 256, 256, 2)
+    src = fc.emit_unit(d.paths, 9, 256, 256, "float")
+    for name in ("fwd_kernel", "dx1_kernel", "dx2_kernel", 'extern "C" int fcj_fwd', 'extern "C" int fcj_dx1', 'extern "C" int fcj_dx2'):
+        assert name in src
+    d = dense("8x0e+3x1o", "0e+1o", "5x0e+7x1o")
+    assert not fc.supported(d.paths, 4, d.input_sizes[1], d.out_size, 4)
+    d = dense("128x0e+128x1o", "0e+1o", "128x0e+128x1o")  # 512 columns a row
+    assert not fc.supported(d.paths, 4, d.input_sizes[1], d.out_size, 4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("i1,i2,i3,Z", [
+    ("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o", 777),   # ragged: the last 32-row tile holds 9 rows
+    ("32x0e+64x1o", "0e+1o", "96x0e+32x1o", 2500),     # mixed block shapes, a wavefront walks more than one tile on few CUs
+    ("32x0e", "0e+1o", "32x1o", 1),
+])
+def test_fused_fully_connected_matches_oracle_and_tables(device, dtype, i1, i2, i3, Z, jit_on):
+    """The generated fully connected kernels (weights resident in LDS, products scaled in registers) against the CPU
+    oracle, and against the table-driven GEMM path of the same module at the same tolerance."""
+    from cuequivariance_amd import cuet
+
+    m = cuet.FullyConnectedTensorProduct(cue.Irreps("O3", i1), cue.Irreps("O3", i2), cue.Irreps("O3", i3), layout=cue.ir_mul,
+                                         internal_weights=False)
+    g = torch.Generator().manual_seed(Z)
+    ins = [torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g),
+           torch.randn(Z, m.irreps_in1.dim, dtype=torch.float64, generator=g),
+           torch.randn(Z, m.irreps_in2.dim, dtype=torch.float64, generator=g)]
+    rounded = [t.to(dtype).double() for t in ins]
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+    a = [t.clone().requires_grad_(True) for t in rounded]
+    ref = naive_segmented_polynomial(spec, a)[0]
+    cot = torch.randn(ref.shape, dtype=torch.float64, generator=g).to(dtype).double()
+    want = (ref,) + torch.autograd.grad(ref, a, cot)
+
+    def run():
+        b = [t.to(dtype).to(device).requires_grad_(True) for t in rounded]
+        out = m.f(b)[0]
+        return (out,) + torch.autograd.grad(out, b, cot.to(dtype).to(device))
+
+    got = run()
+    d = _dense_of(m)
+    assert d._fused.get((dtype, True)) is not None, "the generated kernels were not built"
+    jit.enable(False)
+    tables = run()
+    assert d._fused.get((dtype, False)) is None
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    for name, u, v, t in zip(("out", "dw", "dx1", "dx2"), got, want, tables):
+        assert u.dtype == dtype and u.shape == v.shape
+        scale = max(v.abs().max().item(), 1e-30)
+        assert (u.double().cpu() - v).abs().max().item() <= tol * scale, name
+        assert (u.double() - t.double()).abs().max().item() <= 2 * tol * scale, name + " vs tables"
