@@ -153,16 +153,28 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
     by_seg = OrderedDict()
     for (w_off, K, N, in_off), uses in prods.items():
         by_seg.setdefault(in_off, []).append((w_off, K, N, uses))
-    for in_off, plist in by_seg.items():
-        C = (plist[0][1] if transposed else plist[0][2])
-        assert all((p[1] if transposed else p[2]) == C for p in plist), "one operand segment, one contraction length"
-        ns = C * es // 64
-        A("    {")
-        A(f"      uint4 xf[{ns}][2];")
-        A(f"      const {T}* xp = IN + z * ldi + {in_off};")
-        for s2 in range(ns):
+    # the fragments of the next operand segment are requested before the products of the current one are worked on
+    segs = list(by_seg.items())
+    contraction = [(pl[0][1] if transposed else pl[0][2]) for _, pl in segs]
+    for (in_off, pl), C in zip(segs, contraction):
+        assert all((p[1] if transposed else p[2]) == C for p in pl), "one operand segment, one contraction length"
+    nsmax = max(contraction) * es // 64
+    A(f"    uint4 xfa[{nsmax}][2], xfb[{nsmax}][2];")
+
+    def request(i):
+        in_off, C = segs[i][0], contraction[i]
+        name = "xfa" if i % 2 == 0 else "xfb"
+        for s2 in range(C * es // 64):
             for q in range(2):
-                A(f"      xf[{s2}][{q}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(xp) + {s2 * 64} + h * 32 + {q * 16});")
+                A(f"    {name}[{s2}][{q}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {in_off}) + {s2 * 64} + h * 32 + {q * 16});")
+
+    request(0)
+    for i, (in_off, plist) in enumerate(segs):
+        ns = contraction[i] * es // 64
+        xf = "xfa" if i % 2 == 0 else "xfb"
+        if i + 1 < len(segs):
+            request(i + 1)
+        A("    {")
         for w_off, K, N, uses in plist:
             o, R, Cc, RS = lds_off[w_off]
             for t in range(R // 32):
@@ -171,7 +183,7 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
                 A(f"        const char* wr = smem + {o} + ({32 * t} + c) * {RS} + h * 32;")
                 for s2 in range(ns):
                     for q in range(2):
-                        A(f"        mma_step<{T}>(T, *reinterpret_cast<const uint4*>(wr + {s2 * 64 + q * 16}), xf[{s2}][{q}]);")
+                        A(f"        mma_step<{T}>(T, *reinterpret_cast<const uint4*>(wr + {s2 * 64 + q * 16}), {xf}[{s2}][{q}]);")
                 for j, coeff, res_off in uses:
                     if rowdot:
                         A("        {")
@@ -211,6 +223,128 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
     A("")
 
 
+DW_ROWS = 16  # batch rows per staged tile of the weight-gradient kernel
+
+
+def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
+    """Weight gradient ``dW_b[k, n] = sum_z x1[z, a_off + k] H[z, n]`` with ``H = sum over the uses of (b, a_off) of
+    c x2[z, j] g[z, c_off + n]`` formed in registers.  The batch is the contraction: a lane feeds the 32x32x2 MFMA one
+    element of ``x1`` (row ``z0 + lane / 32``, column ``a_off + k``) and one of ``H``, no transposition.  A block owns a
+    range of rows and stages them 16 at a time through LDS as floats (16-byte global loads issued one tile ahead, two
+    LDS buffers, one barrier per tile); its wavefronts own disjoint sets of accumulator tiles (units ``(block, 32 columns
+    n)`` dealt out by weight) and read their operands from LDS.  The per-block sums go to ``PART[block]`` for a row sum."""
+    es = 4 if T == "float" else 2
+    per = 16 // es  # elements per 16-byte load
+    R, WX, WG, WS = DW_ROWS, width_in, width_out, 16
+    prods = _products(paths, True)  # (w_off, K, N, a_off) -> [(j, coeff, c_off)]
+    units = {}  # (w_off, K, N, nt) -> [(a_off, uses)]
+    for (w_off, K, N, a_off), uses in prods.items():
+        for nt in range(N // 32):
+            units.setdefault((w_off, K, N, nt), []).append((a_off, uses))
+    weight = lambda u: len(units[u]) * (u[1] // 32)
+    waves = [[] for _ in range(8)]
+    load = [0] * 8
+    for u in sorted(units, key=lambda u: (-weight(u), u)):
+        w = min(range(8), key=lambda i: (load[i], i))
+        waves[w].append(u)
+        load[w] += weight(u)
+    # wavefront i runs on SIMD i mod 4: pair the heaviest with the lightest
+    order = sorted(range(8), key=lambda i: -load[i])
+    slots = [order[0], order[1], order[2], order[3], order[7], order[6], order[5], order[4]]
+    tiles_of = [[(w_off, K, N, nt, kt) for (w_off, K, N, nt) in waves[wi] for kt in range(K // 32)] for wi in slots]
+    nacc = max(len(t) for t in tiles_of)
+    nx, ng = -(-(R * WX // per) // 512), -(-(R * WG // per) // 512)
+    stride = R * (WX + WG + WS)
+    A(f"// dw: {len(units)} units over 8 wavefronts, MFMAs per pair of rows: {[load[i] for i in slots]}")
+    A(f"constexpr int kdwLds = {2 * stride * 4};")
+    A("__device__ __forceinline__ void stage(float* dst, const uint4& v, const float*) { *reinterpret_cast<uint4*>(dst) = v; }")
+    A("__device__ __forceinline__ void stage(float* dst, const uint4& v, const uint16_t*) {")
+    A("  *reinterpret_cast<float4*>(dst) = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));")
+    A("  *reinterpret_cast<float4*>(dst + 4) = make_float4(__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xffff0000u), __uint_as_float(v.w << 16), __uint_as_float(v.w & 0xffff0000u));")
+    A("}")
+    A(f"__global__ void __launch_bounds__(64 * kWaves, 1) dw_kernel(const {T}* __restrict__ X, int64_t ldx, const {T}* __restrict__ S, int64_t lds_, "
+      f"const {T}* __restrict__ G, int64_t ldg, float* __restrict__ PART, int64_t numel, int Z, int chunk) {{")
+    A("  extern __shared__ __align__(16) char smem[];")
+    A("  float* const lds = reinterpret_cast<float*>(smem);")
+    A("  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c = lane & 31, h = lane >> 5;")
+    A("  const int z_begin = blockIdx.x * chunk, z_end = min(Z, z_begin + chunk);")
+    A("  if (z_begin >= z_end) return;")
+    A("  float* __restrict__ part = PART + static_cast<int64_t>(blockIdx.x) * numel;")
+    for a in range(nacc):
+        A(f"  floatx16 acc{a} = floatx16{{0}};")
+    A(f"  uint4 xr[{nx}], gr[{ng}]; float sr = 0.f;")
+    A("  auto fetch = [&](int z0) {  // this thread's pieces of the 16 rows from z0 on (zeros past the range)")
+    for name, W, n, src, ld in (("xr", WX, nx, "X", "ldx"), ("gr", WG, ng, "G", "ldg")):
+        for i in range(n):
+            A(f"    {{ const int s = tid + {512 * i}, row = s / {W // per}, q = s % {W // per}; {name}[{i}] = make_uint4(0, 0, 0, 0);")
+            A(f"      if (s < {R * W // per} && z0 + row < z_end) {name}[{i}] = *reinterpret_cast<const uint4*>({src} + static_cast<int64_t>(z0 + row) * {ld} + q * {per}); }}")
+    A(f"    {{ const int row = tid / {n2}, j = tid % {n2}; sr = (tid < {R * n2} && z0 + row < z_end) ? to_f(S[static_cast<int64_t>(z0 + row) * lds_ + j]) : 0.f; }}")
+    A("  };")
+    A("  auto commit = [&](float* buf) {")
+    for name, W, n, base in (("xr", WX, nx, 0), ("gr", WG, ng, R * WX)):
+        for i in range(n):
+            A(f"    {{ const int s = tid + {512 * i}, row = s / {W // per}, q = s % {W // per}; "
+              f"if (s < {R * W // per}) stage(buf + {base} + row * {W} + q * {per}, {name}[{i}], static_cast<const {T}*>(nullptr)); }}")
+    A(f"    if (tid < {R * n2}) buf[{R * (WX + WG)} + (tid / {n2}) * {WS} + tid % {n2}] = sr;")
+    A("  };")
+    A("  fetch(z_begin);")
+    A("  int which = 0;")
+    A(f"  for (int z0 = z_begin; z0 < z_end; z0 += {R}, which ^= 1) {{")
+    A(f"    float* const buf = lds + which * {stride};")
+    A("    commit(buf);")
+    A("    __syncthreads();  // (the other buffer is written next time round: everyone has left it by then)")
+    A(f"    if (z0 + {R} < z_end) fetch(z0 + {R});")
+    A("    switch (wave) {")
+    for slot in range(8):
+        tl = tiles_of[slot]
+        if not tl:
+            continue
+        acc_of = {t: i for i, t in enumerate(tl)}
+        us = waves[slots[slot]]
+        js = sorted({j for u in us for _, uses in units[u] for j, _, _ in uses})
+        xcols = sorted({a_off + 32 * kt for u in us for a_off, _ in units[u] for kt in range(u[1] // 32)})
+        gcols = sorted({c_off + 32 * u[3] for u in us for _, uses in units[u] for _, _, c_off in uses})
+        A(f"      case {slot}: {{")
+        A("#pragma unroll 4")
+        A(f"        for (int p = 0; p < {R // 2}; ++p) {{")
+        A(f"          const float* xs = buf + (2 * p + h) * {WX} + c;")
+        A(f"          const float* gs = buf + {R * WX} + (2 * p + h) * {WG} + c;")
+        A(f"          const float* ss = buf + {R * (WX + WG)} + (2 * p + h) * {WS};")
+        for j in js:
+            A(f"          const float s{j} = ss[{j}];")
+        for col in xcols:
+            A(f"          const float x{col} = xs[{col}];")
+        for col in gcols:
+            A(f"          const float g{col} = gs[{col}];")
+        for (w_off, K, N, nt) in us:
+            for a_off, uses in units[(w_off, K, N, nt)]:
+                terms = " + ".join(f"({coeff!r}f * s{j}) * g{c_off + 32 * nt}" for j, coeff, c_off in uses)
+                A(f"          {{ const float hv = {terms};")
+                for kt in range(K // 32):
+                    a = acc_of[(w_off, K, N, nt, kt)]
+                    A(f"            acc{a} = __builtin_amdgcn_mfma_f32_32x32x2f32(x{a_off + 32 * kt}, hv, acc{a}, 0, 0, 0);")
+                A("          }")
+        A("        }")
+        A("      } break;")
+    A("      default: break;")
+    A("    }")
+    A("  }")
+    A("  switch (wave) {")
+    for slot in range(8):
+        tl = tiles_of[slot]
+        if not tl:
+            continue
+        A(f"    case {slot}:")
+        for a, (w_off, K, N, nt, kt) in enumerate(tl):
+            A("#pragma unroll")
+            A(f"      for (int v = 0; v < 16; ++v) part[{w_off + 32 * kt * N + 32 * nt} + (8 * (v >> 2) + 4 * h + (v & 3)) * {N} + c] = acc{a}[v];")
+        A("      break;")
+    A("    default: break;")
+    A("  }")
+    A("}")
+    A("")
+
+
 def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str) -> str:
     """``paths``: objects with ``w_off, a_off, j, c_off, K, N, coeff``; ``T``: ``float`` or ``uint16_t`` (bfloat16 bits)."""
     L = []
@@ -220,36 +354,68 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str) -> str:
     _emit_kernel(A, "fwd", T, paths, True, False, width_out, n2)
     _emit_kernel(A, "dx1", T, paths, False, False, width_in, n2)
     _emit_kernel(A, "dx2", T, paths, True, True, width_out, n2)
+    _emit_dw_kernel(A, T, paths, n2, width_in, width_out)
+    A("// compute units of the current device (asked once per device: the query is slow)")
     A("int grid_for(int64_t Z) {")
-    A("  int dev = 0, cus = 256; hipDeviceProp_t p;")
-    A("  if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) cus = p.multiProcessorCount;")
+    A("  static int cus_of[64] = {0};")
+    A("  int dev = 0;")
+    A("  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;")
+    A("  int cus = __atomic_load_n(&cus_of[dev], __ATOMIC_RELAXED);")
+    A("  if (cus == 0) {")
+    A("    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;")
+    A("    __atomic_store_n(&cus_of[dev], cus, __ATOMIC_RELAXED);")
+    A("  }")
     A("  const int64_t need = (Z + 31) / 32;")
     A("  return static_cast<int>(need < cus ? (need < 1 ? 1 : need) : cus);")
     A("}")
-    A("template <typename F> int prepare(F fn, int lds) {")
-    A("  return hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess ? 0 : -1;")
+    A("// the LDS limit of a kernel is raised once per device")
+    A("template <typename F> int prepare(F fn, int lds, int* done) {")
+    A("  int dev = 0;")
+    A("  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;")
+    A("  if (__atomic_load_n(&done[dev], __ATOMIC_ACQUIRE)) return 0;")
+    A("  if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -1;")
+    A("  __atomic_store_n(&done[dev], 1, __ATOMIC_RELEASE);")
+    A("  return 0;")
     A("}")
+    A("int done_fwd[64], done_dx1[64], done_dx2[64], done_dw[64];")
     A("}  // namespace")
     A("")
     A(f'extern "C" int fcj_fwd(int64_t Z, const void* W, const void* X, int64_t ldx, const void* S, int64_t lds_, void* OUT, int64_t ldo, void* stream) {{')
     A("  if (Z <= 0) return 0;")
-    A("  if (prepare(fwd_kernel, kfwdLds)) return -1;")
+    A("  if (prepare(fwd_kernel, kfwdLds, done_fwd)) return -1;")
     A(f"  hipLaunchKernelGGL(fwd_kernel, dim3(grid_for(Z)), dim3(64 * kWaves), kfwdLds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(W), "
       f"static_cast<const {T}*>(X), ldx, static_cast<const {T}*>(S), lds_, static_cast<{T}*>(OUT), ldo, static_cast<int>(Z));")
     A("  return hipGetLastError() == hipSuccess ? 0 : -1;")
     A("}")
     A(f'extern "C" int fcj_dx1(int64_t Z, const void* W, const void* G, int64_t ldg, const void* S, int64_t lds_, void* DX1, int64_t ldd, void* stream) {{')
     A("  if (Z <= 0) return 0;")
-    A("  if (prepare(dx1_kernel, kdx1Lds)) return -1;")
+    A("  if (prepare(dx1_kernel, kdx1Lds, done_dx1)) return -1;")
     A(f"  hipLaunchKernelGGL(dx1_kernel, dim3(grid_for(Z)), dim3(64 * kWaves), kdx1Lds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(W), "
       f"static_cast<const {T}*>(G), ldg, static_cast<const {T}*>(S), lds_, static_cast<{T}*>(DX1), ldd, static_cast<int>(Z));")
     A("  return hipGetLastError() == hipSuccess ? 0 : -1;")
     A("}")
     A(f'extern "C" int fcj_dx2(int64_t Z, const void* W, const void* X, int64_t ldx, const void* S, int64_t lds_, const void* G, int64_t ldg, void* DX2, int64_t ld2, void* stream) {{')
     A("  if (Z <= 0) return 0;")
-    A("  if (prepare(dx2_kernel, kdx2Lds)) return -1;")
+    A("  if (prepare(dx2_kernel, kdx2Lds, done_dx2)) return -1;")
     A(f"  hipLaunchKernelGGL(dx2_kernel, dim3(grid_for(Z)), dim3(64 * kWaves), kdx2Lds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(W), "
       f"static_cast<const {T}*>(X), ldx, static_cast<const {T}*>(S), lds_, static_cast<const {T}*>(G), ldg, static_cast<{T}*>(DX2), ld2, static_cast<int>(Z));")
+    A("  return hipGetLastError() == hipSuccess ? 0 : -1;")
+    A("}")
+    A("// number of per-block partial sums fcj_dw writes for a batch of Z rows (the caller sizes PART with it)")
+    A('extern "C" int fcj_dw_blocks(int64_t Z) {')
+    A("  if (Z <= 0) return 0;")
+    A("  const int g = grid_for(Z);")
+    A(f"  const int64_t chunk = ((Z + g - 1) / g + {DW_ROWS - 1}) / {DW_ROWS} * {DW_ROWS};")
+    A("  return static_cast<int>((Z + chunk - 1) / chunk);")
+    A("}")
+    A(f'extern "C" int fcj_dw(int64_t Z, const void* X, int64_t ldx, const void* S, int64_t lds_, const void* G, int64_t ldg, float* PART, int64_t numel, void* stream) {{')
+    A("  if (Z <= 0) return 0;")
+    A("  const int g = grid_for(Z);")
+    A(f"  const int64_t chunk = ((Z + g - 1) / g + {DW_ROWS - 1}) / {DW_ROWS} * {DW_ROWS};")
+    A("  const int blocks = static_cast<int>((Z + chunk - 1) / chunk);")
+    A("  if (prepare(dw_kernel, kdwLds, done_dw)) return -1;")
+    A(f"  hipLaunchKernelGGL(dw_kernel, dim3(blocks), dim3(64 * kWaves), kdwLds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(X), ldx, "
+      f"static_cast<const {T}*>(S), lds_, static_cast<const {T}*>(G), ldg, PART, numel, static_cast<int>(Z), static_cast<int>(chunk));")
     A("  return hipGetLastError() == hipSuccess ? 0 : -1;")
     A("}")
     return "\n".join(L) + "\n"

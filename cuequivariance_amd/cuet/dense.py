@@ -542,7 +542,22 @@ class _FcFunction(torch.autograd.Function):
                     _lib.check(lib.cueq_fc_rowdot(code, _lib.F32, Z, x1d.data_ptr(), x1d.stride(0), G.data_ptr(), plan.g_cols,
                                                   gx2.data_ptr(), gx2.stride(0), plan.n2, uses.data_ptr(), nuses,
                                                   1 if plan.dx2_vec else 0, stream), "cueq_fc_rowdot")
-            if need_w:
+            unit_w = mod.fused_unit(dtype, x1d, g) if Z > 0 and need_w else None
+            if unit_w is not None:
+                # per-block partial sums of the generated kernel (x1^T H with H formed in registers), then a row sum
+                nblocks, numel = unit_w.fcj_dw_blocks(Z), wd.numel()
+                covered = sum(K * N for _, K, N in mod.weight_blocks) == numel
+                part = (torch.empty if covered else torch.zeros)(nblocks, numel, dtype=torch.float32, device=dev)
+                if unit_w.fcj_dw(Z, x1d.data_ptr(), x1d.stride(0), x2d.data_ptr(), x2d.stride(0), g.data_ptr(), g.stride(0),
+                                 part.data_ptr(), numel, stream) != 0:
+                    raise RuntimeError("fused fully connected weight gradient: launch failed")
+                gw32 = torch.empty(numel, dtype=torch.float32, device=dev)
+                ws_bytes = lib.cueq_sum_rows_workspace(nblocks, numel)
+                ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+                _lib.check(lib.cueq_sum_rows(_lib.F32, nblocks, numel, part.data_ptr(), gw32.data_ptr(), ws.data_ptr(), ws_bytes, stream),
+                           "cueq_sum_rows")
+                gw = gw32.to(w.dtype).reshape(w.shape)
+            elif need_w:
                 gwd = torch.zeros_like(wd)
                 if Z > 0:
                     # H[:, t] = sum over the uses of T-block t of coeff * x2[:, j] * g[:, k_seg]; then dW_p = sum_i x1[:, i_seg]^T H[:, t_i]

@@ -197,8 +197,8 @@ def _compile(src: str, so: Path, what: str, link_library: bool = True) -> None:
 
 def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str):
     """The fused kernels of ``codegen/fullyconnected.py`` for one fully connected product and element type (``float`` or
-    ``uint16_t`` for bfloat16), compiled at first use and loaded: a ``ctypes`` handle with ``fcj_fwd``, ``fcj_dx1`` and
-    ``fcj_dx2``, or ``None`` when this module is off, the product is outside what the generator covers, or the compiler
+    ``uint16_t`` for bfloat16), compiled at first use and loaded: a ``ctypes`` handle with ``fcj_fwd``, ``fcj_dx1``,
+    ``fcj_dx2`` and ``fcj_dw``, or ``None`` when this module is off, the product is outside what the generator covers, or the compiler
     failed (the caller then runs the table-driven GEMMs)."""
     from .codegen import fullyconnected as fc
 
@@ -220,7 +220,9 @@ def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str):
             h.fcj_fwd.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp]
             h.fcj_dx1.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp]
             h.fcj_dx2.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp]
-            for f in (h.fcj_fwd, h.fcj_dx1, h.fcj_dx2):
+            h.fcj_dw_blocks.argtypes = [i64]
+            h.fcj_dw.argtypes = [i64, vp, i64, vp, i64, vp, i64, vp, i64, vp]
+            for f in (h.fcj_fwd, h.fcj_dx1, h.fcj_dx2, h.fcj_dw_blocks, h.fcj_dw):
                 f.restype = C.c_int
             _loaded[key] = h
             return h
