@@ -172,8 +172,14 @@ def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
         unit, units, dt = "rows/s", Z, "bf16" if dtype == torch.bfloat16 else "f32"
         es = 2 if dtype == torch.bfloat16 else 4
         # every distinct element once: fwd reads x1, x2 and writes out; bwd reads x1, x2, g and writes dx1, dx2 (weights 20480 negligible)
-        alg = {"fwd": Z * (256 + 9 + 256) * es, "bwd": Z * (256 + 9 + 256 + 256 + 9) * es}
-        bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
+        if dtype == torch.float32:
+            # 11 distinct (weight block, x1 component) products of 64 x 64 per row; forward, dx1, dx2 and dw contract each once
+            f = 2 * Z * 64 * 64 * 11
+            alg = {"fwd": f, "bwd": 3 * f}
+            bound, peak, pu = "mfma", 157.3, "TFLOP/s"
+        else:
+            alg = {"fwd": Z * (256 + 9 + 256) * es, "bwd": Z * (256 + 9 + 256 + 256 + 9) * es}
+            bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
         desc = ("configs[3]: FullyConnectedTensorProduct 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, batch 50000, shared weights, "
                 "fwd + bwd (dw, dx1, dx2)")
     else:
