@@ -24,9 +24,12 @@ def device():
 @pytest.fixture(autouse=True, scope="session")
 def _kernels_at_first_use_off():
     """Compilation at first use is on for users; the suite keeps it off (the table-driven kernels stay covered and dozens
-    of small descriptors are not compiled), ``tests/test_jit.py`` switches it on for its cases."""
+    of small descriptors are not compiled), ``tests/test_jit.py`` switches it on for its cases; ``CUEQ_AMD_TEST_JIT=1`` leaves it on for the whole run."""
     from cuequivariance_amd import jit
 
+    if os.environ.get("CUEQ_AMD_TEST_JIT", "0") == "1":  # the whole suite on the kernels compiled at first use
+        yield
+        return
     jit.enable(False)
     yield
 
