@@ -515,11 +515,11 @@ class _FcFunction(torch.autograd.Function):
             stream = torch.cuda.current_stream(dev).cuda_stream
             code, es = _DTYPE_CODE[dtype], x1d.element_size()
             tables = plan.device(dev)
-            if need_x1:
-                gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
+            unit = unit_w = mod.fused_unit(dtype, x1d, g) if Z > 0 else None
+            if need_x1:  # (the generated kernels write every column)
+                gx1 = (torch.empty_like if mod.dx1_covers_input or unit is not None else torch.zeros_like)(x1d)
             if need_x2:
-                gx2 = torch.zeros_like(x2d)
-            unit = mod.fused_unit(dtype, x1d, g) if Z > 0 and (need_x1 or need_x2) else None
+                gx2 = (torch.empty_like if unit is not None else torch.zeros_like)(x2d)
             if unit is not None:
                 if need_x1 and unit.fcj_dx1(Z, wd.data_ptr(), g.data_ptr(), g.stride(0), x2d.data_ptr(), x2d.stride(0), gx1.data_ptr(),
                                             gx1.stride(0), stream) != 0:
@@ -542,8 +542,7 @@ class _FcFunction(torch.autograd.Function):
                     _lib.check(lib.cueq_fc_rowdot(code, _lib.F32, Z, x1d.data_ptr(), x1d.stride(0), G.data_ptr(), plan.g_cols,
                                                   gx2.data_ptr(), gx2.stride(0), plan.n2, uses.data_ptr(), nuses,
                                                   1 if plan.dx2_vec else 0, stream), "cueq_fc_rowdot")
-            unit_w = mod.fused_unit(dtype, x1d, g) if Z > 0 and need_w else None
-            if unit_w is not None:
+            if unit_w is not None and need_w:
                 # per-block partial sums of the generated kernel (x1^T H with H formed in registers), then a row sum
                 nblocks, numel = unit_w.fcj_dw_blocks(Z), wd.numel()
                 covered = sum(K * N for _, K, N in mod.weight_blocks) == numel
