@@ -171,8 +171,19 @@ def test_fully_connected_generator_limits():
     d = dense("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o")
     assert fc.supported(d.paths, 9, 256, 256, 4) and fc.supported(d.paths, 9, 256, 256, 2)
     src = fc.emit_unit(d.paths, 9, 256, 256, "float")
-    for name in ("fwd_kernel", "dx1_kernel", "dx2_kernel", 'extern "C" int fcj_fwd', 'extern "C" int fcj_dx1', 'extern "C" int fcj_dx2'):
+    for name in ("fwd_kernel", "dx1_kernel", "dx2_kernel", "dw_kernel"):
         assert name in src
+    # every entry point the header of the generated objects declares is defined, with the declared number of arguments
+    import pathlib
+    import re
+
+    header = (pathlib.Path(__file__).resolve().parent.parent / "include" / "cueq_amd_generated.h").read_text()
+    declared = re.findall(r"^int (fcj_\w+)\(([^;]*)\);", header, flags=re.M | re.S)
+    assert {n for n, _ in declared} == {"fcj_fwd", "fcj_dx1", "fcj_dx2", "fcj_dw_blocks", "fcj_dw"}
+    for name, args in declared:
+        m = re.search(r'extern "C" int %s\(([^)]*)\)' % name, src)
+        assert m, name
+        assert len(m.group(1).split(",")) == len(args.split(",")), name
     d = dense("8x0e+3x1o", "0e+1o", "5x0e+7x1o")
     assert not fc.supported(d.paths, 4, d.input_sizes[1], d.out_size, 4)
     d = dense("128x0e+128x1o", "0e+1o", "128x0e+128x1o")  # 512 columns a row
