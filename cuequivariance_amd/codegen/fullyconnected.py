@@ -47,6 +47,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
 
 template <typename TI>
 __device__ __forceinline__ void mma_step(floatx16& acc, const uint4& a, const uint4& b) {
@@ -254,7 +255,13 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
     tiles_of = [[(w_off, K, N, nt, kt) for (w_off, K, N, nt) in waves[wi] for kt in range(K // 32)] for wi in slots]
     nacc = max(len(t) for t in tiles_of)
     nx, ng = -(-(R * WX // per) // 512), -(-(R * WG // per) // 512)
-    stride = R * (WX + WG + WS)
+    # 2-byte elements: x1 stays as it is (rows of WX elements + 64 bytes, read back with the transposing LDS read as
+    # bf16 MFMA operands: 16 rows are one 32x32x16 step), g and x2 become floats, x2 column-major (8 rows per read)
+    fast16 = es == 2
+    XSTR = WX * 2 + 64
+    XB = R * XSTR if fast16 else R * WX * 4          # bytes of the x1 region
+    SB = XB + R * WG * 4                             # byte offset of the x2 region
+    stride = (SB + R * WS * 4) // 4                  # floats per buffer
     A(f"// dw: {len(units)} units over 8 wavefronts, MFMAs per pair of rows: {[load[i] for i in slots]}")
     A(f"constexpr int kdwLds = {2 * stride * 4};")
     A("__device__ __forceinline__ void stage(float* dst, const uint4& v, const float*) { *reinterpret_cast<uint4*>(dst) = v; }")
@@ -281,11 +288,18 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
     A(f"    {{ const int row = tid / {n2}, j = tid % {n2}; sr = (tid < {R * n2} && z0 + row < z_end) ? to_f(S[static_cast<int64_t>(z0 + row) * lds_ + j]) : 0.f; }}")
     A("  };")
     A("  auto commit = [&](float* buf) {")
-    for name, W, n, base in (("xr", WX, nx, 0), ("gr", WG, ng, R * WX)):
+    for name, W, n, base in (("xr", WX, nx, 0), ("gr", WG, ng, XB // 4)):
         for i in range(n):
-            A(f"    {{ const int s = tid + {512 * i}, row = s / {W // per}, q = s % {W // per}; "
-              f"if (s < {R * W // per}) stage(buf + {base} + row * {W} + q * {per}, {name}[{i}], static_cast<const {T}*>(nullptr)); }}")
-    A(f"    if (tid < {R * n2}) buf[{R * (WX + WG)} + (tid / {n2}) * {WS} + tid % {n2}] = sr;")
+            if fast16 and name == "xr":
+                A(f"    {{ const int s = tid + {512 * i}, row = s / {W // per}, q = s % {W // per}; "
+                  f"if (s < {R * W // per}) *reinterpret_cast<uint4*>(reinterpret_cast<char*>(buf) + row * {XSTR} + q * 16) = xr[{i}]; }}")
+            else:
+                A(f"    {{ const int s = tid + {512 * i}, row = s / {W // per}, q = s % {W // per}; "
+                  f"if (s < {R * W // per}) stage(buf + {base} + row * {W} + q * {per}, {name}[{i}], static_cast<const {T}*>(nullptr)); }}")
+    if fast16:
+        A(f"    if (tid < {R * n2}) buf[{SB // 4} + (tid % {n2}) * {R} + tid / {n2}] = sr;")
+    else:
+        A(f"    if (tid < {R * n2}) buf[{SB // 4} + (tid / {n2}) * {WS} + tid % {n2}] = sr;")
     A("  };")
     A("  fetch(z_begin);")
     A("  int which = 0;")
@@ -305,11 +319,41 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
         xcols = sorted({a_off + 32 * kt for u in us for a_off, _ in units[u] for kt in range(u[1] // 32)})
         gcols = sorted({c_off + 32 * u[3] for u in us for _, uses in units[u] for _, _, c_off in uses})
         A(f"      case {slot}: {{")
+        if fast16:
+            A("        typedef shortx4_t __attribute__((address_space(3))) * lptr;")
+            A("        const int s16 = lane & 15, g16 = (lane >> 4) & 1;")
+            A(f"        const char* xp = reinterpret_cast<const char*>(buf) + (8 * h + (s16 >> 2)) * {XSTR} + (16 * g16 + 4 * (s16 & 3)) * 2;")
+            A(f"        const float* gs = buf + {XB // 4} + (8 * h) * {WG} + c;")
+            A(f"        const float* st = buf + {SB // 4} + 8 * h;")
+            for j in js:
+                A(f"        float s{j}[8]; {{ const float4 lo = *reinterpret_cast<const float4*>(st + {j * R}), hi = *reinterpret_cast<const float4*>(st + {j * R + 4}); "
+                  f"s{j}[0] = lo.x; s{j}[1] = lo.y; s{j}[2] = lo.z; s{j}[3] = lo.w; s{j}[4] = hi.x; s{j}[5] = hi.y; s{j}[6] = hi.z; s{j}[7] = hi.w; }}")
+            for col in gcols:
+                A(f"        float g{col}[8];")
+                A("#pragma unroll")
+                A(f"        for (int e = 0; e < 8; ++e) g{col}[e] = gs[e * {WG} + {col}];")
+            for col in xcols:
+                A(f"        uint4 x{col}; {{ const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(xp + {col * 2}))), "
+                  f"hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(xp + {col * 2 + 4 * XSTR}))); x{col} = make_uint4(lo.x, lo.y, hi.x, hi.y); }}")
+            for (w_off, K, N, nt) in us:
+                for a_off, uses in units[(w_off, K, N, nt)]:
+                    A("        {")
+                    A("          float hv[8];")
+                    A("#pragma unroll")
+                    terms = " + ".join(f"({coeff!r}f * s{j}[e]) * g{c_off + 32 * nt}[e]" for j, coeff, c_off in uses)
+                    A(f"          for (int e = 0; e < 8; ++e) hv[e] = {terms};")
+                    A("          const uint4 hb = make_uint4(pack_bf16(hv[0], hv[1]), pack_bf16(hv[2], hv[3]), pack_bf16(hv[4], hv[5]), pack_bf16(hv[6], hv[7]));")
+                    for kt in range(K // 32):
+                        a = acc_of[(w_off, K, N, nt, kt)]
+                        A(f"          mma_step<uint16_t>(acc{a}, x{a_off + 32 * kt}, hb);")
+                    A("        }")
+            A("      } break;")
+            continue
         A("#pragma unroll 4")
         A(f"        for (int p = 0; p < {R // 2}; ++p) {{")
         A(f"          const float* xs = buf + (2 * p + h) * {WX} + c;")
-        A(f"          const float* gs = buf + {R * WX} + (2 * p + h) * {WG} + c;")
-        A(f"          const float* ss = buf + {R * (WX + WG)} + (2 * p + h) * {WS};")
+        A(f"          const float* gs = buf + {XB // 4} + (2 * p + h) * {WG} + c;")
+        A(f"          const float* ss = buf + {SB // 4} + (2 * p + h) * {WS};")
         for j in js:
             A(f"          const float s{j} = ss[{j}];")
         for col in xcols:
