@@ -458,6 +458,13 @@ class _FcPlan:
         return d
 
 
+def _aligned(t: torch.Tensor) -> torch.Tensor:
+    """``t`` contiguous and starting on a 16-byte boundary (a copy when a view starts elsewhere): the fully connected
+    kernels move rows in 16-byte pieces."""
+    t = t.contiguous()
+    return t.clone() if t.data_ptr() % 16 else t
+
+
 def _fc_combine(lib, code, t_code, Z, S, T, O, table, stream):
     blocks, uses, nblocks, max_n, vec = table
     _lib.check(lib.cueq_fc_combine(code, t_code, Z, S.data_ptr(), S.stride(0), T.data_ptr(), T.stride(0), O.data_ptr(), O.stride(0),
@@ -475,7 +482,7 @@ class _FcFunction(torch.autograd.Function):
         plan, lib = mod.fc_plan, _lib.load()
         out = (torch.empty if mod.fwd_covers_output else torch.zeros)((Z, mod.out_size), dtype=dtype, device=dev)
         if Z > 0:
-            wd, x1d, x2d = w.detach().to(dtype).contiguous(), x1.detach().contiguous(), x2.detach().contiguous()
+            wd, x1d, x2d = _aligned(w.detach().to(dtype)), _aligned(x1.detach()), x2.detach().contiguous()
             with torch.cuda.device(dev):
                 stream = torch.cuda.current_stream(dev).cuda_stream
                 code, es = _DTYPE_CODE[dtype], x1d.element_size()
@@ -507,8 +514,8 @@ class _FcFunction(torch.autograd.Function):
         dtype, dev = x1.dtype, x1.device
         Z = x1.shape[0]
         plan, lib = mod.fc_plan, _lib.load()
-        g = g.contiguous()
-        wd, x1d, x2d = w.detach().to(dtype).contiguous(), x1.detach().contiguous(), x2.detach().contiguous()
+        g = _aligned(g)
+        wd, x1d, x2d = _aligned(w.detach().to(dtype)), _aligned(x1.detach()), x2.detach().contiguous()
         gw = gx1 = gx2 = None
         need_w, need_x1, need_x2 = ctx.needs_input_grad[1], ctx.needs_input_grad[2], ctx.needs_input_grad[3]
         with torch.cuda.device(dev):

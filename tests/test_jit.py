@@ -232,3 +232,37 @@ def test_fused_fully_connected_matches_oracle_and_tables(device, dtype, i1, i2, 
         scale = max(v.abs().max().item(), 1e-30)
         assert (u.double().cpu() - v).abs().max().item() <= tol * scale, name
         assert (u.double() - t.double()).abs().max().item() <= 2 * tol * scale, name + " vs tables"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("on", [True, False])
+def test_fully_connected_unaligned_rows(device, jit_on, on):
+    """The fully connected kernels (generated and table-driven) move rows in 16-byte pieces; an operand view that starts
+    4 bytes off such a boundary is copied to aligned storage first and gives what an aligned copy gives."""
+    from cuequivariance_amd import cuet
+
+    jit.enable(on)
+    m = cuet.FullyConnectedTensorProduct(cue.Irreps("O3", "32x0e+32x1o"), cue.Irreps("O3", "0e+1o"), cue.Irreps("O3", "32x0e+32x1o"),
+                                         layout=cue.ir_mul, internal_weights=False)
+    g = torch.Generator().manual_seed(3)
+    Z = 100
+    w = torch.randn(1, m.weight_numel, generator=g).to(device)
+    x2 = torch.randn(Z, 4, generator=g).to(device)
+    flat = torch.randn(1 + Z * 128, generator=g).to(device)
+    x1_off = flat[1:].view(Z, 128)            # contiguous rows, first element 4 bytes past a 16-byte boundary
+    x1_al = x1_off.clone()
+    cot_off = torch.randn(1 + Z * 128, generator=g).to(device)[1:].view(Z, 128)
+    assert x1_off.data_ptr() % 16 == 4 and x1_al.data_ptr() % 16 == 0 and cot_off.data_ptr() % 16 == 4
+    d = _dense_of(m)
+    assert d.fused_unit(torch.float32, x1_off) is None
+
+    def run(x1, cot):
+        a = [w.clone().requires_grad_(True), x1.detach().requires_grad_(True), x2.clone().requires_grad_(True)]
+        out = m.f(a)[0]
+        return (out,) + torch.autograd.grad(out, a, cot)
+
+    want = run(x1_al, cot_off.clone())
+    got = run(x1_off, cot_off)
+    assert (d._fused.get((torch.float32, True)) is not None) == on
+    for u, v in zip(got, want):
+        assert torch.equal(u, v)
