@@ -1,0 +1,123 @@
+"""Element offsets beyond 2^31: one call over a batch whose largest operand holds more than 2^31 elements against the
+same work done in two halves (each below 2^31).  Size-independent properties only - the oracle would take hours here:
+batched outputs and per-row gradients of the halves concatenate, indexed outputs and shared gradients add."""
+
+import gc
+
+import pytest
+import torch
+
+from cuequivariance_amd import cue
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, want, name):
+    scale = want.abs().max().item()
+    err = (got - want).abs().max().item()
+    assert err <= 1e-5 * scale, (name, err, scale)
+
+
+@pytest.fixture(autouse=True)
+def _release():
+    yield
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def test_channelwise_indexed_weights_beyond_2g_elements(device):
+    """128 channels, l <= 3, 2 000 nodes, 800 000 edges: the per-edge weights hold 2.36e9 elements."""
+    from cuequivariance_amd import cuet
+
+    i1 = cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o")
+    i2 = cue.Irreps("O3", "0e+1o+2e+3o")
+    m = cuet.ChannelWiseTensorProduct(i1, i2, "0e+1o+2e+3o", layout=cue.ir_mul, shared_weights=False)
+    N, E = 2000, 800_000
+    assert E * m.weight_numel > 2 ** 31
+    g = torch.Generator(device=device).manual_seed(0)
+    x1 = torch.randn(N, i1.dim, device=device, generator=g)
+    x2 = torch.randn(E, i2.dim, device=device, generator=g)
+    w = torch.randn(E, m.weight_numel, device=device, generator=g)
+    snd = torch.randint(0, N, (E,), device=device, generator=g, dtype=torch.int32)
+    rcv = torch.sort(torch.randint(0, N, (E,), device=device, generator=g, dtype=torch.int32))[0]
+    cot = torch.randn(N, m.irreps_out.dim, device=device, generator=g)
+
+    def run(lo, hi):
+        a = [x1.clone().requires_grad_(True), x2[lo:hi].requires_grad_(True), w[lo:hi].requires_grad_(True)]
+        out = m(a[0], a[1], a[2], indices_1=snd[lo:hi], indices_out=rcv[lo:hi], size_out=N)
+        return (out.detach(),) + torch.autograd.grad(out, a, cot)
+
+    out, dx1, dx2, dw = run(0, E)
+    h = E // 2
+    out_a, dx1_a, dx2_a, dw_a = run(0, h)
+    _close(dw[:h], dw_a, "dw, first half")
+    _close(dx2[:h], dx2_a, "dx2, first half")
+    del dw_a, dx2_a
+    out_b, dx1_b, dx2_b, dw_b = run(h, E)
+    _close(dw[h:], dw_b, "dw, second half")  # rows whose element offset exceeds 2^31
+    _close(dx2[h:], dx2_b, "dx2, second half")
+    _close(out, out_a + out_b, "out")
+    _close(dx1, dx1_a + dx1_b, "dx1")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_rows_beyond_2g_elements(device, dtype):
+    """Linear on 128x0e+128x1o+128x2e (1152 columns), 2 000 000 rows: 2.3e9 elements per operand."""
+    from cuequivariance_amd import cuet
+
+    irreps = cue.Irreps("O3", "128x0e+128x1o+128x2e")
+    m = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=False, method="fused_tp")
+    Z = 2_000_000
+    assert Z * irreps.dim > 2 ** 31
+    g = torch.Generator(device=device).manual_seed(1)
+    x = torch.randn(Z, irreps.dim, device=device, generator=g).to(dtype)
+    w = torch.randn(1, m.weight_numel, device=device, generator=g).to(dtype)
+    cot = torch.randn(Z, irreps.dim, device=device, generator=g).to(dtype)
+
+    def run(lo, hi):
+        a = [x[lo:hi].requires_grad_(True), w.clone().requires_grad_(True)]
+        out = m(a[0], a[1])
+        return (out.detach(),) + torch.autograd.grad(out, a, cot[lo:hi])
+
+    out, dx, dw = run(0, Z)
+    h = Z // 2
+    out_a, dx_a, dw_a = run(0, h)
+    out_b, dx_b, dw_b = run(h, Z)
+    # per-row results do not depend on the batch they are computed in
+    assert torch.equal(out[:h], out_a) and torch.equal(out[h:], out_b)
+    assert torch.equal(dx[:h], dx_a) and torch.equal(dx[h:], dx_b)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    want = dw_a.double() + dw_b.double()
+    assert (dw.double() - want).abs().max().item() <= tol * want.abs().max().item()
+
+
+def test_symmetric_contraction_rows_beyond_2g_elements(device):
+    """Degree-3 contraction of 128x(0e+1o+2e+3o) (2048 columns) on 1 100 000 nodes: 2.25e9 input elements."""
+    from cuequivariance_amd import cuet
+
+    irreps_in = cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o")
+    irreps_out = cue.Irreps("O3", "128x0e+128x1o")
+    m = cuet.SymmetricContraction(irreps_in, irreps_out, 3, 10, layout_in=cue.ir_mul, layout_out=cue.ir_mul,
+                                  dtype=torch.float32, device=device)
+    Z = 1_100_000
+    assert Z * irreps_in.dim > 2 ** 31
+    g = torch.Generator(device=device).manual_seed(2)
+    x = torch.randn(Z, irreps_in.dim, device=device, generator=g) * 0.5
+    idx = torch.randint(0, 10, (Z,), device=device, generator=g, dtype=torch.int32)
+    cot = torch.randn(Z, irreps_out.dim, device=device, generator=g)
+
+    def run(lo, hi):
+        a = x[lo:hi].requires_grad_(True)
+        out = m(a, idx[lo:hi])
+        dx, dw = torch.autograd.grad(out, [a, m.weight], cot[lo:hi])
+        return out.detach(), dx, dw
+
+    out, dx, dw = run(0, Z)
+    h = Z // 2
+    out_a, dx_a, dw_a = run(0, h)
+    out_b, dx_b, dw_b = run(h, Z)
+    _close(out[:h], out_a, "out, first half")
+    _close(out[h:], out_b, "out, second half")
+    _close(dx[:h], dx_a, "dx, first half")
+    _close(dx[h:], dx_b, "dx, second half")
+    _close(dw, dw_a + dw_b, "dw")
