@@ -266,3 +266,41 @@ def test_fully_connected_unaligned_rows(device, jit_on, on):
     assert (d._fused.get((torch.float32, True)) is not None) == on
     for u, v in zip(got, want):
         assert torch.equal(u, v)
+
+
+@pytest.mark.gpu
+def test_fused_fully_connected_rows_beyond_2g_elements(device, jit_on):
+    """9 000 000 rows of 256 columns (2.3e9 elements per operand) through the generated kernels: one call against the
+    same rows in two halves (per-row results do not depend on the batch they are computed in; weight gradients add)."""
+    import gc
+
+    from cuequivariance_amd import cuet
+
+    i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e")
+    m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, internal_weights=False)
+    Z = 9_000_000
+    assert Z * i1.dim > 2 ** 31
+    g = torch.Generator(device=device).manual_seed(4)
+    x1 = torch.randn(Z, i1.dim, device=device, generator=g)
+    x2 = torch.randn(Z, i2.dim, device=device, generator=g)
+    w = torch.randn(1, m.weight_numel, device=device, generator=g)
+    cot = torch.randn(Z, i1.dim, device=device, generator=g)
+
+    def run(lo, hi):
+        a = [x1[lo:hi].requires_grad_(True), x2[lo:hi].requires_grad_(True), w.clone().requires_grad_(True)]
+        out = m(a[0], a[1], a[2])
+        return (out.detach(),) + torch.autograd.grad(out, a, cot[lo:hi])
+
+    out, dx1, dx2, dw = run(0, Z)
+    assert _dense_of(m)._fused.get((torch.float32, True)) is not None
+    h = Z // 2
+    halves = torch.zeros_like(dw, dtype=torch.float64)
+    for lo, hi in ((0, h), (h, Z)):
+        o, d1, d2, dwh = run(lo, hi)
+        assert torch.equal(out[lo:hi], o) and torch.equal(dx1[lo:hi], d1) and torch.equal(dx2[lo:hi], d2)
+        halves += dwh.double()
+        del o, d1, d2, dwh
+    assert (dw.double() - halves).abs().max().item() <= 1e-5 * halves.abs().max().item()  # (the halves sum in another order)
+    del out, dx1, dx2, x1, x2, cot
+    gc.collect()
+    torch.cuda.empty_cache()
