@@ -1308,11 +1308,12 @@ __global__ void __launch_bounds__(256) gemm_simple(const TI* __restrict__ A, int
 // batched transpose  out[b][c][r] = in[b][r][c]  (32 x 32 tiles through LDS)
 // ------------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ in, T* __restrict__ out, int R, int Ccols) {
+__global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ in, T* __restrict__ out, int R, int Ccols, int rows_on_x) {
   __shared__ T tile[32][33];
   const int64_t base = static_cast<int64_t>(blockIdx.z) * R * Ccols;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
-  const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+  // (grid.y holds at most 65535 tiles: the host puts the row tiles on grid.x when there are more)
+  const int r0 = (rows_on_x ? blockIdx.x : blockIdx.y) * 32, c0 = (rows_on_x ? blockIdx.y : blockIdx.x) * 32;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int r = r0 + ty + q * 8, cc = c0 + tx;
@@ -1327,11 +1328,11 @@ __global__ void __launch_bounds__(256) transpose_kernel(const T* __restrict__ in
 }
 
 // 2-byte elements, even extents: 64 x 64 tiles moved as pairs (4-byte accesses on both sides)
-__global__ void __launch_bounds__(256) transpose16_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, int R, int Ccols) {
+__global__ void __launch_bounds__(256) transpose16_kernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, int R, int Ccols, int rows_on_x) {
   __shared__ uint16_t tile[64][66];
   const int64_t base = static_cast<int64_t>(blockIdx.z) * R * Ccols;
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 pairs x 8
-  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int r0 = (rows_on_x ? blockIdx.x : blockIdx.y) * 64, c0 = (rows_on_x ? blockIdx.y : blockIdx.x) * 64;
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
     const int r = r0 + ty + q * 8, cc = c0 + 2 * tx;
@@ -1923,6 +1924,8 @@ __global__ void __launch_bounds__(256) fold_partials_kernel(const float* __restr
 }
 
 static bool is_io(int dt) { return dt == CUEQ_F32 || dt == CUEQ_BF16; }
+// rows one launch takes when its row tiles sit on grid.y (65535 tiles of 128; a multiple of every tile height used)
+constexpr int64_t kRowSlab = 65280ll * 128;
 
 }  // namespace cueq
 
@@ -1941,6 +1944,16 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
   CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, CUEQ_ERR_INVALID, "gemm: negative extent");
   if (M == 0 || N == 0 || batch == 0) return CUEQ_OK;
   CUEQ_REQUIRE(A && B && C, CUEQ_ERR_INVALID, "gemm: null operand");
+  if (M > kRowSlab) {  // grid.y holds at most 65535 row tiles: more rows go in slabs, which are independent
+    const int64_t es_in = in_dtype == CUEQ_F32 ? 4 : 2, es_out = out_dtype == CUEQ_F32 ? 4 : 2;
+    for (int64_t r0 = 0; r0 < M; r0 += kRowSlab) {
+      const int64_t mm = M - r0 < kRowSlab ? M - r0 : kRowSlab;
+      const int rc = cueq_gemm(in_dtype, out_dtype, trans_a, trans_b, mm, N, K, static_cast<const char*>(A) + (trans_a ? r0 : r0 * lda) * es_in, lda,
+                               stride_a, B, ldb, stride_b, static_cast<char*>(C) + r0 * ldc * es_out, ldc, stride_c, batch, alpha, accumulate, stream_);
+      if (rc != CUEQ_OK) return rc;
+    }
+    return CUEQ_OK;
+  }
   CUEQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch < 65536, CUEQ_ERR_TOO_LARGE, "gemm: extent too large");
   const int epv = in_dtype == CUEQ_F32 ? 4 : 8;
   // vectors run along k for a contraction-contiguous operand, along its other extent for a contraction-major one
@@ -2006,6 +2019,16 @@ extern "C" int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t tran
   CUEQ_REQUIRE(A && B && C && table, CUEQ_ERR_INVALID, "gemm_table: null operand");
   CUEQ_REQUIRE(k_chunks == 1 || (trans_a && trans_b), CUEQ_ERR_UNSUPPORTED, "gemm_table: the contraction is cut only for contraction-major operands");
   CUEQ_REQUIRE(!(trans_a && !trans_b), CUEQ_ERR_UNSUPPORTED, "gemm_table: A contraction-major with B contraction-contiguous is not built");
+  if (M > kRowSlab) {
+    const int64_t es_in = in_dtype == CUEQ_F32 ? 4 : 2, es_out = out_dtype == CUEQ_F32 ? 4 : 2;
+    for (int64_t r0 = 0; r0 < M; r0 += kRowSlab) {
+      const int64_t mm = M - r0 < kRowSlab ? M - r0 : kRowSlab;
+      const int rc = cueq_gemm_table(in_dtype, out_dtype, trans_a, trans_b, mm, N, K, static_cast<const char*>(A) + (trans_a ? r0 : r0 * lda) * es_in, lda, B,
+                                     ldb, static_cast<char*>(C) + r0 * ldc * es_out, ldc, table, nparts, k_chunks, chunk_stride_c, alpha, accumulate, stream_);
+      if (rc != CUEQ_OK) return rc;
+    }
+    return CUEQ_OK;
+  }
   CUEQ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && nparts * k_chunks < 65536, CUEQ_ERR_TOO_LARGE, "gemm_table: extent too large");
   const int epv = in_dtype == CUEQ_F32 ? 4 : 8;
   // the table's offsets must keep the 16-byte alignment too: the caller builds it from segment offsets (checked there)
@@ -2097,6 +2120,19 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
   const bool aligned = K % epv == 0 && lda % epv == 0 && ldb % epv == 0 &&
                        ((reinterpret_cast<uintptr_t>(A1) | reinterpret_cast<uintptr_t>(A2) | reinterpret_cast<uintptr_t>(B1) | reinterpret_cast<uintptr_t>(B2)) & 15) == 0;
   CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "dual_gate: K, row strides and pointers must be multiples of 16 bytes");
+  if (M > kRowSlab) {
+    const int64_t es = dtype == CUEQ_F32 ? 4 : 2;
+    auto rows = [&](const void* p, int64_t ld, int64_t r0) { return p ? static_cast<const void*>(static_cast<const char*>(p) + r0 * ld * es) : nullptr; };
+    for (int64_t r0 = 0; r0 < M; r0 += kRowSlab) {
+      const int64_t mm = M - r0 < kRowSlab ? M - r0 : kRowSlab;
+      const int rc = cueq_dual_gate(dtype, backward, mm, N, K, rows(A1, lda, r0), rows(A2, lda, r0), lda, B1, B2, ldb,
+                                    bias_axis == 0 ? rows(bias1, 1, r0) : bias1, bias_axis == 0 ? rows(bias2, 1, r0) : bias2, bias_axis,
+                                    mask_axis == 0 ? rows(mask, 1, r0) : mask, mask_axis, rows(dC, ldc, r0), const_cast<void*>(rows(out1, ldc, r0)),
+                                    const_cast<void*>(rows(out2, ldc, r0)), ldc, stream_);
+      if (rc != CUEQ_OK) return rc;
+    }
+    return CUEQ_OK;
+  }
   const int64_t gy = (M + kTile - 1) / kTile, gx = (N + kTile - 1) / kTile;
   CUEQ_REQUIRE(gy < 65536 && gx < (1ll << 31) && M < (1ll << 31) && N < (1ll << 31), CUEQ_ERR_TOO_LARGE, "dual_gate: extent too large");
   const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy));
@@ -2155,6 +2191,20 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
   CUEQ_REQUIRE(aligned, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: row strides and pointers must be multiples of 16 bytes");
   CUEQ_REQUIRE(split == !dc_by_row, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: built for one input with dC by rows (C x M) and two inputs with dC by columns (M x C)");
   const int64_t es = bf ? 2 : 4;
+  if (!dc_by_row && ldc > 0 && (M * ldc + 8) * es >= (1ll << 32)) {
+    // dC (M x C) is addressed with 32-bit byte offsets from a uniform base: more rows go in slabs (rows are independent)
+    const int64_t slab = (((1ll << 32) / es - 8) / ldc) & ~int64_t(255);
+    CUEQ_REQUIRE(slab > 0, CUEQ_ERR_TOO_LARGE, "gate_bwd_input: row stride of dC too large");
+    auto rows = [&](const void* p, int64_t ld, int64_t r0) { return p ? static_cast<const void*>(static_cast<const char*>(p) + r0 * ld * es) : nullptr; };
+    for (int64_t r0 = 0; r0 < M; r0 += slab) {
+      const int64_t mm = M - r0 < slab ? M - r0 : slab;
+      const int rc = cueq_gate_bwd_input(dtype, C, mm, K, W1, W2, ldw, rows(X1, ldx, r0), rows(X2, ldx, r0), ldx, bias1, bias2, rows(mask, 1, r0),
+                                         rows(dC, ldc, r0), ldc, 0, const_cast<void*>(rows(dX1, lddx, r0)), const_cast<void*>(rows(dX2, lddx, r0)), lddx,
+                                         accumulate, const_cast<void*>(rows(dU, ldc, r0)), const_cast<void*>(rows(dV, ldc, r0)), stream_);
+      if (rc != CUEQ_OK) return rc;
+    }
+    return CUEQ_OK;
+  }
   CUEQ_REQUIRE(ldc >= 0 && ldw >= 0 && 32 * ldw * es < (1ll << 31) &&
                    (dc_by_row ? (4 * ldc + M) : (M * ldc + 8)) * es < (1ll << 32),
                CUEQ_ERR_TOO_LARGE, "gate_bwd_input: strides too large for 32-bit lane offsets");
@@ -2240,21 +2290,25 @@ extern "C" int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_
   CUEQ_REQUIRE(in && out, CUEQ_ERR_INVALID, "transpose: null operand");
   CUEQ_REQUIRE(rows < (1ll << 31) && cols < (1ll << 31), CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
   if (dtype == CUEQ_BF16 && rows % 2 == 0 && cols % 2 == 0 && reinterpret_cast<uintptr_t>(in) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0) {
-    const int64_t gy2 = (rows + 63) / 64, gx2 = (cols + 63) / 64;
-    CUEQ_REQUIRE(gy2 < 65536 && batch < 65536, CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
+    int64_t gy2 = (rows + 63) / 64, gx2 = (cols + 63) / 64;
+    const int rows_on_x = gy2 >= 65536 ? 1 : 0;
+    if (rows_on_x) { const int64_t t = gx2; gx2 = gy2; gy2 = t; }
+    CUEQ_REQUIRE(gy2 < 65536 && gx2 < (1ll << 31) && batch < 65536, CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
     KernelTimer timer("transpose", stream);
     hipLaunchKernelGGL(transpose16_kernel, dim3(static_cast<unsigned>(gx2), static_cast<unsigned>(gy2), static_cast<unsigned>(batch)), dim3(256), 0, stream,
-                       static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols));
+                       static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols), rows_on_x);
     CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }
-  const int64_t gy = (rows + 31) / 32, gx = (cols + 31) / 32;
+  int64_t gy = (rows + 31) / 32, gx = (cols + 31) / 32;
+  const int rows_on_x = gy >= 65536 ? 1 : 0;
+  if (rows_on_x) { const int64_t t = gx; gx = gy; gy = t; }
   CUEQ_REQUIRE(gy < 65536 && batch < 65536 && gx < (1ll << 31), CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
   const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy), static_cast<unsigned>(batch));
   KernelTimer timer("transpose", stream);
   TRI_DISPATCH(dtype,
-               hipLaunchKernelGGL(transpose_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), static_cast<float*>(out), static_cast<int>(rows), static_cast<int>(cols)),
-               hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols)));
+               hipLaunchKernelGGL(transpose_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), static_cast<float*>(out), static_cast<int>(rows), static_cast<int>(cols), rows_on_x),
+               hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols), rows_on_x));
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }

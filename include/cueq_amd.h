@@ -207,7 +207,9 @@ int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int6
 /* cueq_gemm_nt with a choice of operand order: trans_a != 0 takes A as K x M (row stride lda, batch stride stride_a)
  * instead of M x K, trans_b != 0 takes B as K x N.  Serves the gradients of the triangular contraction
  * (da = dt b, db = dt^T a; _triangle_multiplicative_update.py:393-397) and its "incoming" form without transposed
- * copies.  Mixed input / output types are supported for trans_a == trans_b == 0 only. */
+ * copies.  Mixed input / output types are supported for trans_a == trans_b == 0 only.
+ * Sizes: M, N, K below 2^31, batch below 65536; one launch takes 8 355 840 rows (its row tiles sit on grid.y), more rows
+ * run as consecutive launches over slabs of rows (the same holds for cueq_gemm_table and cueq_dual_gate). */
 int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
               const void* A, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc,
               int64_t stride_c, int64_t batch, double alpha, int32_t accumulate, void* stream);
@@ -253,7 +255,8 @@ int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_
  * dC (and dU, dV when not NULL: the gate gradients for the weight / bias gradients) are C x M with row stride ldc when
  * dc_by_row != 0, M x C otherwise (built for one input with dC by rows and for two inputs with dC by columns).
  * K must be 32, 64, 96 or 128 and C a multiple of 32; strides and pointers multiples of 16 bytes, else
- * CUEQ_ERR_UNSUPPORTED (compose cueq_dual_gate and cueq_gemm_nt instead). */
+ * CUEQ_ERR_UNSUPPORTED (compose cueq_dual_gate and cueq_gemm_nt instead).  dC by columns is addressed with 32-bit byte
+ * offsets inside a launch: beyond 4 GiB of dC the rows run as consecutive launches over slabs of rows. */
 int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
                         const void* X1, const void* X2, int64_t ldx,
                         const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
@@ -270,7 +273,8 @@ int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows, const voi
                  const void* B, int64_t ldb, int64_t stride_b, int32_t nparts, float* partials, double alpha, void* stream);
 
 /* out[b][c][r] = in[b][r][c] (layout changes "bijd<->dbij" of _layer_norm_transpose.py:162-227 and operand
- * re-orientation for the incoming direction and the backward contractions). */
+ * re-orientation for the incoming direction and the backward contractions).  rows, cols below 2^31, batch below 65536,
+ * and at most one of rows / cols beyond 4 194 240 (2 097 120 for 4-byte or odd-sized inputs): the longer one goes to grid.x. */
 int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_t cols, const void* in, void* out, void* stream);
 
 /* Per-segment (u, v) -> (v, u) transposition of every row, one pass: out[r][o] = in[r][src_index[o]] with the row

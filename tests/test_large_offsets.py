@@ -121,3 +121,94 @@ def test_symmetric_contraction_rows_beyond_2g_elements(device):
     _close(dx[:h], dx_a, "dx, first half")
     _close(dx[h:], dx_b, "dx, second half")
     _close(dw, dw_a + dw_b, "dw")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_transpose_more_row_tiles_than_grid_y_holds(device, dtype):
+    """4 194 368 rows of 8 and of 6 columns (one more 64-row tile than grid.y can index, even and odd column pairs):
+    bit-exact against a strided copy, both ways."""
+    from cuequivariance_amd.cuet import triangle as T
+
+    for cols in (8, 6, 5):
+        rows = 65536 * 64 + 64
+        x = torch.randn(rows, cols, device=device).to(dtype)
+        y = T.transpose(x)
+        assert torch.equal(y, x.t().contiguous())
+        assert torch.equal(T.transpose(y), x)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_triangle_update_more_pair_rows_than_one_launch_takes(device, dtype):
+    """Two pair tensors of 2048 x 2048 x 128 in one call: 8 388 608 pair rows, more than the projections' launches take
+    at once (their row tiles sit on grid.y), so they run in slabs of rows.  Batch elements are independent: each half of the output and of
+    the input gradient must be what a call on that batch element alone gives; weight gradients add."""
+    from cuequivariance_amd.cuet import triangle_multiplicative_update as tmu
+
+    B, N, D = 2, 2048, 128
+    g = torch.Generator(device=device).manual_seed(5)
+    ws = {k: (torch.randn(*shape, device=device, generator=g) * 0.09).to(dtype)
+          for k, shape in (("p_in_weight", (2 * D, D)), ("g_in_weight", (2 * D, D)), ("p_out_weight", (D, D)), ("g_out_weight", (D, D)))}
+    x = torch.randn(B, N, N, D, device=device, generator=g).to(dtype)
+    mask = (torch.rand(B, N, N, device=device, generator=g) > 0.1).to(dtype)
+    cot = torch.randn(B, N, N, D, device=device, generator=g).to(dtype)
+
+    def run(lo, hi):
+        a = x[lo:hi].requires_grad_(True)
+        w = {k: v.clone().requires_grad_(True) for k, v in ws.items()}
+        out = tmu(a, "outgoing", mask=mask[lo:hi], **w)
+        grads = torch.autograd.grad(out, [a] + list(w.values()), cot[lo:hi])
+        return out.detach(), grads[0], [t.float() for t in grads[1:]]
+
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    out, dx, dws = run(0, B)
+    sums = [torch.zeros_like(t) for t in dws]
+    for b in range(B):
+        o, d, dw = run(b, b + 1)
+        for name, u, v in (("out", out[b:b + 1], o), ("dx", dx[b:b + 1], d)):
+            err = (u.float() - v.float()).abs().max().item()
+            assert err <= tol * v.float().abs().max().item(), (name, b, err)
+        for s_, t in zip(sums, dw):
+            s_ += t
+        del o, d, dw
+    for name, u, v in zip(ws, dws, sums):
+        assert (u - v).abs().max().item() <= tol * v.abs().max().item(), name
+
+
+@pytest.mark.parametrize("kind", ["linear", "fully_connected"])
+def test_dense_more_rows_than_one_launch_takes(device, kind):
+    """9 000 000 rows through the table-driven GEMM launches of the dense executor (row tiles on grid.y: 8 355 840 rows a
+    launch, the rest in a second slab): per-row results equal those of the two halves, weight gradients add."""
+    from cuequivariance_amd import cuet
+
+    Z = 9_000_000
+    g = torch.Generator(device=device).manual_seed(6)
+    if kind == "linear":
+        irreps = cue.Irreps("O3", "32x0e+32x1o")
+        m = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=False, method="fused_tp")
+        ins = [torch.randn(Z, irreps.dim, device=device, generator=g)]
+        call = lambda a, w: m(a[0], w)
+    else:
+        i1, i2 = cue.Irreps("O3", "8x0e+8x1o"), cue.Irreps("O3", "0e+1o")
+        m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, internal_weights=False)
+        ins = [torch.randn(Z, i1.dim, device=device, generator=g), torch.randn(Z, i2.dim, device=device, generator=g)]
+        call = lambda a, w: m(a[0], a[1], w)
+    w0 = torch.randn(1, m.weight_numel, device=device, generator=g)
+    cot = torch.randn(Z, m.irreps_out.dim, device=device, generator=g)
+
+    def run(lo, hi):
+        a = [t[lo:hi].requires_grad_(True) for t in ins]
+        w = w0.clone().requires_grad_(True)
+        out = call(a, w)
+        grads = torch.autograd.grad(out, a + [w], cot[lo:hi])
+        return [out.detach()] + list(grads[:-1]), grads[-1]
+
+    rows, dw = run(0, Z)
+    h = Z // 2
+    total = torch.zeros_like(dw, dtype=torch.float64)
+    for lo, hi in ((0, h), (h, Z)):
+        r, d = run(lo, hi)
+        for u, v in zip(rows, r):
+            assert torch.equal(u[lo:hi], v)
+        total += d.double()
+        del r, d
+    assert (dw.double() - total).abs().max().item() <= 1e-5 * total.abs().max().item()
