@@ -1944,6 +1944,17 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
   CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, CUEQ_ERR_INVALID, "gemm: negative extent");
   if (M == 0 || N == 0 || batch == 0) return CUEQ_OK;
   CUEQ_REQUIRE(A && B && C, CUEQ_ERR_INVALID, "gemm: null operand");
+  if (batch > 65535) {  // grid.z holds at most 65535 batch items
+    const int64_t es_in = in_dtype == CUEQ_F32 ? 4 : 2, es_out = out_dtype == CUEQ_F32 ? 4 : 2;
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+      const int64_t bb = batch - b0 < 65535 ? batch - b0 : 65535;
+      const int rc = cueq_gemm(in_dtype, out_dtype, trans_a, trans_b, M, N, K, static_cast<const char*>(A) + b0 * stride_a * es_in, lda, stride_a,
+                               static_cast<const char*>(B) + b0 * stride_b * es_in, ldb, stride_b, static_cast<char*>(C) + b0 * stride_c * es_out, ldc,
+                               stride_c, bb, alpha, accumulate, stream_);
+      if (rc != CUEQ_OK) return rc;
+    }
+    return CUEQ_OK;
+  }
   if (M > kRowSlab) {  // grid.y holds at most 65535 row tiles: more rows go in slabs, which are independent
     const int64_t es_in = in_dtype == CUEQ_F32 ? 4 : 2, es_out = out_dtype == CUEQ_F32 ? 4 : 2;
     for (int64_t r0 = 0; r0 < M; r0 += kRowSlab) {

@@ -208,8 +208,9 @@ int cueq_gemm_nt(int32_t in_dtype, int32_t out_dtype, int64_t M, int64_t N, int6
  * instead of M x K, trans_b != 0 takes B as K x N.  Serves the gradients of the triangular contraction
  * (da = dt b, db = dt^T a; _triangle_multiplicative_update.py:393-397) and its "incoming" form without transposed
  * copies.  Mixed input / output types are supported for trans_a == trans_b == 0 only.
- * Sizes: M, N, K below 2^31, batch below 65536; one launch takes 8 355 840 rows (its row tiles sit on grid.y), more rows
- * run as consecutive launches over slabs of rows (the same holds for cueq_gemm_table and cueq_dual_gate). */
+ * Sizes: M, N, K below 2^31; one launch takes 8 355 840 rows (its row tiles sit on grid.y) and 65 535 batch items
+ * (grid.z): more run as consecutive launches over slabs of rows / batch items (rows also in cueq_gemm_table and
+ * cueq_dual_gate). */
 int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
               const void* A, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C, int64_t ldc,
               int64_t stride_c, int64_t batch, double alpha, int32_t accumulate, void* stream);

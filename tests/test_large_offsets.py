@@ -212,3 +212,27 @@ def test_dense_more_rows_than_one_launch_takes(device, kind):
         total += d.double()
         del r, d
     assert (dw.double() - total).abs().max().item() <= 1e-5 * total.abs().max().item()
+
+
+def test_triangle_update_more_batch_items_than_grid_z_holds(device):
+    """600 pair tensors of 32 x 32 x 128: the triangular contraction is a batched product over 128 * 600 = 76 800
+    (channel, batch) items, more than grid.z indexes - it runs as two launches.  Every batch element must come out as in
+    a call of its own."""
+    from cuequivariance_amd.cuet import triangle_multiplicative_update as tmu
+
+    B, N, D = 600, 32, 128
+    dtype = torch.bfloat16
+    g = torch.Generator(device=device).manual_seed(7)
+    ws = {k: (torch.randn(*shape, device=device, generator=g) * 0.09).to(dtype)
+          for k, shape in (("p_in_weight", (2 * D, D)), ("g_in_weight", (2 * D, D)), ("p_out_weight", (D, D)), ("g_out_weight", (D, D)))}
+    x = torch.randn(B, N, N, D, device=device, generator=g).to(dtype).requires_grad_(True)
+    mask = (torch.rand(B, N, N, device=device, generator=g) > 0.1).to(dtype)
+    cot = torch.randn(B, N, N, D, device=device, generator=g).to(dtype)
+    for direction in ("outgoing", "incoming"):
+        out = tmu(x, direction, mask=mask, **ws)
+        (dx,) = torch.autograd.grad(out, [x], cot)
+        for b in (0, 511, 512, 599):  # 65 535 = 128 * 511 + 127: element 511 straddles the two launches
+            xb = x[b:b + 1].detach().requires_grad_(True)
+            ob = tmu(xb, direction, mask=mask[b:b + 1], **ws)
+            (db,) = torch.autograd.grad(ob, [xb], cot[b:b + 1])
+            assert torch.equal(out[b:b + 1], ob) and torch.equal(dx[b:b + 1], db), (direction, b)
