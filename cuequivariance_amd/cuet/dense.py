@@ -596,6 +596,16 @@ class _FcFunction(torch.autograd.Function):
         return None, gw, gx1, gx2
 
 
+def _row_ranges(Z: int, Cn: int, offsets: torch.Tensor):
+    """Row ranges for the rows-grouped launches (``cueq_gemm_grouped`` mode 1 keeps its row tiles, one extra per class,
+    on grid.y: 65 535 of them), each with the class offsets relative to the range - computed on the device, no
+    synchronisation."""
+    cap = (65535 - Cn - 1) * 128
+    if Z <= cap:
+        return [(0, Z, offsets)]
+    return [(lo, min(Z, lo + cap), (offsets - lo).clamp_(0, min(Z, lo + cap) - lo)) for lo in range(0, Z, cap)]
+
+
 class _IndexedDenseFunction(torch.autograd.Function):
     """Linear with one weight row per class and the batch rows sorted by class (``offsets[c] .. offsets[c+1]`` are the rows
     of class ``c``): grouped GEMMs on the tiled MFMA kernel (``cueq_gemm_grouped``), no host synchronisation."""
@@ -613,17 +623,20 @@ class _IndexedDenseFunction(torch.autograd.Function):
                 stream = torch.cuda.current_stream(x1.device).cuda_stream
                 code, es = _DTYPE_CODE[dtype], x1d.element_size()
                 written = set()
+                ranges = _row_ranges(Z, Cn, offsets)
                 for p, count, da, dc in mod.fwd_groups:
                     cols = tuple(p.c_off + t * dc for t in range(count))
                     acc = 1 if any(c in written for c in cols) else 0
                     written.update(cols)
                     # out[z, k_seg] (+)= c * x1[z, i_seg] @ W_p[class(z)]; the K x N block is contraction-major as it lies
-                    _lib.check(
-                        lib.cueq_gemm_grouped(code, code, 1, Z, p.N, p.K, x1d.data_ptr() + p.a_off * es, x1d.stride(0), da,
-                                              wd.data_ptr() + p.w_off * es, p.N, 0, out.data_ptr() + p.c_off * es, out.stride(0), dc,
-                                              count, offsets.data_ptr(), Cn, 1, W, p.coeff, acc, stream),
-                        "cueq_gemm_grouped",
-                    )
+                    for lo, hi, offs in ranges:
+                        _lib.check(
+                            lib.cueq_gemm_grouped(code, code, 1, hi - lo, p.N, p.K, x1d.data_ptr() + (lo * x1d.stride(0) + p.a_off) * es,
+                                                  x1d.stride(0), da, wd.data_ptr() + p.w_off * es, p.N, 0,
+                                                  out.data_ptr() + (lo * out.stride(0) + p.c_off) * es, out.stride(0), dc,
+                                                  count, offs.data_ptr(), Cn, 1, W, p.coeff, acc, stream),
+                            "cueq_gemm_grouped",
+                        )
         ctx.mod = mod
         ctx.save_for_backward(w, x1, offsets)
         return out
@@ -645,17 +658,19 @@ class _IndexedDenseFunction(torch.autograd.Function):
             if ctx.needs_input_grad[2]:
                 gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
                 written = set()
+                ranges = _row_ranges(Z, Cn, offsets)
                 for p, count, dc, da in mod.dx1_groups if Z > 0 else []:
                     cols = tuple(p.a_off + t * da for t in range(count))
                     acc = 1 if any(c in written for c in cols) else 0
                     written.update(cols)
                     # dx1[z, i_seg] (+)= c * g[z, k_seg] @ W_p[class(z)]^T: the K x N block is "N' x K'" for this product
-                    _lib.check(
-                        lib.cueq_gemm_grouped(code, code, 1, Z, p.K, p.N, g.data_ptr() + p.c_off * es, g.stride(0), dc,
-                                              wd.data_ptr() + p.w_off * es, p.N, 0, gx1.data_ptr() + p.a_off * es, gx1.stride(0), da,
-                                              count, offsets.data_ptr(), Cn, 0, W, p.coeff, acc, stream),
-                        "cueq_gemm_grouped",
-                    )
+                    for lo, hi, offs in ranges:
+                        _lib.check(
+                            lib.cueq_gemm_grouped(code, code, 1, hi - lo, p.K, p.N, g.data_ptr() + (lo * g.stride(0) + p.c_off) * es, g.stride(0), dc,
+                                                  wd.data_ptr() + p.w_off * es, p.N, 0, gx1.data_ptr() + (lo * gx1.stride(0) + p.a_off) * es,
+                                                  gx1.stride(0), da, count, offs.data_ptr(), Cn, 0, W, p.coeff, acc, stream),
+                            "cueq_gemm_grouped",
+                        )
             if ctx.needs_input_grad[1]:
                 # dW_p[c] += coeff * sum over the rows z of class c of x1[z, i_seg]^T g[z, k_seg]: float32 accumulation
                 gw32 = torch.zeros(Cn, W, dtype=torch.float32, device=x1.device)

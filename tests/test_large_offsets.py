@@ -236,3 +236,32 @@ def test_triangle_update_more_batch_items_than_grid_z_holds(device):
             ob = tmu(xb, direction, mask=mask[b:b + 1], **ws)
             (db,) = torch.autograd.grad(ob, [xb], cot[b:b + 1])
             assert torch.equal(out[b:b + 1], ob) and torch.equal(dx[b:b + 1], db), (direction, b)
+
+
+def test_indexed_linear_more_rows_than_one_launch_takes(device):
+    """9 500 000 rows in three weight classes (one of them empty, one of 9 499 900 rows): the rows-grouped launches take
+    8.4 M rows each, so the batch runs as two row ranges with class offsets relative to each.  Against the plain Linear
+    applied per class."""
+    from cuequivariance_amd import cuet
+
+    irreps = cue.Irreps("O3", "32x0e+32x1o")
+    m = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=False, weight_classes=3, method="indexed_linear")
+    plain = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=False, method="fused_tp")
+    Z = 9_500_000
+    g = torch.Generator(device=device).manual_seed(8)
+    x = torch.randn(Z, irreps.dim, device=device, generator=g)
+    w = torch.randn(3, m.weight_numel, device=device, generator=g)
+    cot = torch.randn(Z, irreps.dim, device=device, generator=g)
+    idx = torch.zeros(Z, dtype=torch.int32, device=device)
+    idx[-100:] = 2
+    a, b = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    out = m(a, b, weight_indices=idx)
+    dx, dw = torch.autograd.grad(out, [a, b], cot)
+    assert dw[1].abs().max().item() == 0
+    for c, (lo, hi) in ((0, (0, Z - 100)), (2, (Z - 100, Z))):
+        a2, b2 = x[lo:hi].clone().requires_grad_(True), w[c:c + 1].clone().requires_grad_(True)
+        o2 = plain(a2, b2)
+        dx2, dw2 = torch.autograd.grad(o2, [a2, b2], cot[lo:hi])
+        # (both weight gradients are float32 sums over 9.5 million rows, accumulated in different orders)
+        for name, u, v, tol in (("out", out[lo:hi], o2, 1e-5), ("dx", dx[lo:hi], dx2, 1e-5), ("dw", dw[c:c + 1], dw2, 3e-4)):
+            assert (u - v).abs().max().item() <= tol * v.abs().max().item(), (name, c)
