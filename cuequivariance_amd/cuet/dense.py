@@ -262,6 +262,19 @@ class _DenseFunction(torch.autograd.Function):
     def backward(ctx, g):
         mod = ctx.mod
         w, x1, x2 = ctx.saved_tensors
+        if not ctx.has_x2:
+            # the two gradients are functions of their own, each differentiable in terms of the other two:
+            # derivatives of any order (forces and their training) stay on these kernels
+            gx1 = _LinearDx.apply(mod, g, w, x1.dtype) if ctx.needs_input_grad[2] else None
+            gw = _LinearDw.apply(mod, x1, g, w) if ctx.needs_input_grad[1] else None
+            return None, gw, gx1, None
+        _first_order_only()
+        return _DenseFunction._backward_impl(ctx, g, ctx.needs_input_grad)
+
+    @staticmethod
+    def _backward_impl(ctx, g, needs_input_grad):
+        mod = ctx.mod
+        w, x1, x2 = ctx.saved_tensors
         x2 = x2 if ctx.has_x2 else None
         dtype = x1.dtype
         lib = _lib.load()
@@ -274,7 +287,7 @@ class _DenseFunction(torch.autograd.Function):
         with torch.cuda.device(x1.device):
             tables = mod.tables(x1.device)
             stream = torch.cuda.current_stream(x1.device).cuda_stream
-            if ctx.needs_input_grad[2]:
+            if needs_input_grad[2]:
                 # dx1[:, i_seg] += c * x2[:, j] * g[:, k_seg] @ W_p^T
                 gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
                 if Z > 0:
@@ -288,7 +301,7 @@ class _DenseFunction(torch.autograd.Function):
                                    mod.dx1_groups, lambda p: p.N, lambda p: p.K)
                     else:
                         _run_gemms(dtype, g, wd, x2d, gx1, tables.dx1)
-            if ctx.needs_input_grad[1]:
+            if needs_input_grad[1]:
                 gwd = None
                 if Z > 0 and mod.tiled(dtype, x1d, g):
                     # dW_p[k][n] += c * sum_z x1[z, i_seg + k] g[z, k_seg + n]: chunked partial products, ordered sum
@@ -331,7 +344,7 @@ class _DenseFunction(torch.autograd.Function):
                 if gwd is None:
                     gwd = torch.zeros_like(wd)
                 gw = gwd.to(w.dtype).reshape(w.shape)
-            if x2 is not None and ctx.needs_input_grad[3]:
+            if x2 is not None and needs_input_grad[3]:
                 gx2 = torch.zeros_like(x2d)
                 touched = set()
                 for p in mod.paths:
@@ -347,6 +360,52 @@ class _DenseFunction(torch.autograd.Function):
                         "cueq_seg_rowdot",
                     )
         return None, gw, gx1, gx2
+
+
+class _GradContext:
+    """What ``_DenseFunction._backward_impl`` reads from an autograd context."""
+
+    def __init__(self, mod, w, x1):
+        self.mod, self.saved_tensors, self.has_x2 = mod, (w, x1, torch.empty(0)), False
+
+
+class _LinearDx(torch.autograd.Function):
+    """``dx = g W^T`` of the 3-operand form as a function of ``(g, w)``: linear in both, so its own gradients are the
+    forward product (with respect to ``g``) and the weight-gradient product (with respect to ``w``)."""
+
+    @staticmethod
+    def forward(ctx, mod, g, w, x_dtype):
+        x_like = torch.empty(g.shape[0], mod.input_sizes[1], dtype=x_dtype, device=g.device)
+        gx1 = _DenseFunction._backward_impl(_GradContext(mod, w, x_like), g.to(x_dtype), (False, False, True, False))[2]
+        ctx.mod = mod
+        ctx.save_for_backward(g, w)
+        return gx1
+
+    @staticmethod
+    def backward(ctx, c):
+        g, w = ctx.saved_tensors
+        dg = _DenseFunction.apply(ctx.mod, w, c, None).to(g.dtype) if ctx.needs_input_grad[1] else None
+        dw = _LinearDw.apply(ctx.mod, c, g, w) if ctx.needs_input_grad[2] else None
+        return None, dg, dw, None
+
+
+class _LinearDw(torch.autograd.Function):
+    """``dW = x^T g`` (per weight block, with the path coefficients) as a function of ``(x, g)``; ``w`` only gives the
+    shape and dtype of the result."""
+
+    @staticmethod
+    def forward(ctx, mod, x1, g, w):
+        gw = _DenseFunction._backward_impl(_GradContext(mod, w, x1), g.to(x1.dtype), (False, True, False, False))[1]
+        ctx.mod = mod
+        ctx.save_for_backward(x1, g)
+        return gw
+
+    @staticmethod
+    def backward(ctx, c):
+        x1, g = ctx.saved_tensors
+        dx = _LinearDx.apply(ctx.mod, g, c, x1.dtype) if ctx.needs_input_grad[1] else None
+        dg = _DenseFunction.apply(ctx.mod, c, x1, None).to(g.dtype) if ctx.needs_input_grad[2] else None
+        return None, dx, dg, None
 
 
 def _progressions(items, key_a, key_c):
@@ -458,6 +517,16 @@ class _FcPlan:
         return d
 
 
+def _first_order_only() -> None:
+    """Called at the top of a backward that is not itself differentiable: under ``create_graph=True`` the gradients would
+    come out detached and a second derivative through them would silently be zero."""
+    if torch.is_grad_enabled():
+        raise NotImplementedError(
+            "fused_tp / indexed_linear: second derivatives (create_graph=True) are built for the 3-operand form with shared "
+            "weights only; the uniform-1d executor (per-sample weights, or method='uniform_1d' on a flattened descriptor) is "
+            "differentiable to any order")
+
+
 def _aligned(t: torch.Tensor) -> torch.Tensor:
     """``t`` contiguous and starting on a 16-byte boundary (a copy when a view starts elsewhere): the fully connected
     kernels move rows in 16-byte pieces."""
@@ -509,6 +578,7 @@ class _FcFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g):
+        _first_order_only()
         mod = ctx.mod
         w, x1, x2 = ctx.saved_tensors
         dtype, dev = x1.dtype, x1.device
@@ -643,6 +713,7 @@ class _IndexedDenseFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g):
+        _first_order_only()
         mod = ctx.mod
         w, x1, offsets = ctx.saved_tensors
         dtype = x1.dtype
@@ -724,7 +795,10 @@ def _dense_bwd_op(mod_id: int, kind: int, w: torch.Tensor, x1: torch.Tensor, x2:
     ctx.mod, ctx.has_x2 = _module_by_id(mod_id), x2 is not None
     ctx.saved_tensors = (w, x1, x2 if (x2 is not None or kind == 1) else torch.empty(0))
     ctx.needs_input_grad = (False, *need)
-    grads = _FUNCTIONS[kind].backward(ctx, g)[1:4]
+    if kind == 0:
+        grads = _DenseFunction._backward_impl(ctx, g, ctx.needs_input_grad)[1:4]
+    else:
+        grads = _FcFunction.backward(ctx, g)[1:4]
     return [x1.new_empty(0) if (t is None or not n) else t.contiguous() for t, n in zip(grads, need)]
 
 

@@ -221,3 +221,49 @@ def test_weights_per_sample_and_unsorted_classes(device, dtype):
     wz = torch.randn(Z, lin2.weight_numel, generator=g, dtype=torch.float64).to(dtype)
     ref = naive_segmented_polynomial(spec, [wz, x1])[0]
     assert rel_err(lin2(x1.to(device), wz.to(device)), ref) <= tol, "linear per-sample weights"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_linear_second_derivatives_match_oracle(device, dtype):
+    """Force training differentiates a gradient again: the gradients of the 3-operand form are functions of their own
+    (each differentiable in terms of the other two), so ``create_graph=True`` stays on the MFMA kernels.  Against
+    autograd through the CPU oracle, all second derivatives of a scalar built from the input gradient."""
+    m = linear_module("32x0e+32x1o+16x2e", "16x0e+32x1o+32x2e")
+    g = torch.Generator().manual_seed(11)
+    Z = 70
+    w = torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g).to(dtype).double()
+    x = torch.randn(Z, m.irreps_in.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    cot = torch.randn(Z, m.irreps_out.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    v = torch.randn(Z, m.irreps_in.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    u = torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g).to(dtype).double()
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+
+    def second(fwd, w_, x_, dev_, dt):
+        out = fwd(w_, x_)
+        gw, gx = torch.autograd.grad(out, [w_, x_], cot.to(dt).to(dev_), create_graph=True)
+        s = (gx * v.to(dt).to(dev_)).sum() + (gw * u.to(dt).to(dev_)).sum() + (gx * gx).sum()
+        return torch.autograd.grad(s, [w_, x_])
+
+    a = [w.clone().requires_grad_(True), x.clone().requires_grad_(True)]
+    want = second(lambda w_, x_: naive_segmented_polynomial(spec, [w_, x_])[0], *a, torch.device("cpu"), torch.float64)
+    b = [w.to(dtype).to(device).requires_grad_(True), x.to(dtype).to(device).requires_grad_(True)]
+    got = second(lambda w_, x_: m.f([w_, x_])[0], *b, device, dtype)
+    tol = 1e-12 if dtype == torch.float64 else 2e-5
+    for name, p, q in zip(("d/dw", "d/dx"), got, want):
+        assert rel_err(p, q) <= tol, (name, rel_err(p, q))
+
+
+def test_fully_connected_second_derivative_raises(device):
+    """The 4-operand form is differentiable once; a backward under ``create_graph=True`` says so instead of returning
+    detached gradients (a second derivative through them would silently be zero)."""
+    from cuequivariance_amd import cuet
+
+    ir = cue.Irreps("O3", "8x0e+8x1o")
+    m = cuet.FullyConnectedTensorProduct(ir, cue.Irreps("O3", "0e+1o"), ir, layout=cue.ir_mul, internal_weights=False)
+    x1 = torch.randn(10, ir.dim, device=device, requires_grad=True)
+    x2 = torch.randn(10, 4, device=device, requires_grad=True)
+    w = torch.randn(1, m.weight_numel, device=device, requires_grad=True)
+    with pytest.raises(NotImplementedError, match="second derivatives"):
+        torch.autograd.grad(m(x1, x2, w).sum(), [x1], create_graph=True)
+    (gx,) = torch.autograd.grad(m(x1, x2, w).sum(), [x1])  # (first order is unaffected)
+    assert gx.shape == x1.shape
