@@ -522,8 +522,8 @@ def _first_order_only() -> None:
     come out detached and a second derivative through them would silently be zero."""
     if torch.is_grad_enabled():
         raise NotImplementedError(
-            "fused_tp / indexed_linear: second derivatives (create_graph=True) are built for the 3-operand form with shared "
-            "weights only; the uniform-1d executor (per-sample weights, or method='uniform_1d' on a flattened descriptor) is "
+            "fused_tp / indexed_linear: second derivatives (create_graph=True) are built for shared weights in float32 / "
+            "bfloat16 (3- and 4-operand forms) only; the uniform-1d executor (per-sample weights, or method='uniform_1d' on a flattened descriptor) is "
             "differentiable to any order")
 
 
@@ -578,16 +578,24 @@ class _FcFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g):
-        _first_order_only()
+        # each gradient is a function of its own, trilinear like the product and differentiable in terms of the other
+        # three: derivatives of any order stay on these kernels
         mod = ctx.mod
         w, x1, x2 = ctx.saved_tensors
+        gw = _FcDw.apply(mod, x1, x2, g, w) if ctx.needs_input_grad[1] else None
+        gx1 = _FcDx1.apply(mod, w, g, x2, x1) if ctx.needs_input_grad[2] else None
+        gx2 = _FcDx2.apply(mod, w, x1, g, x2) if ctx.needs_input_grad[3] else None
+        return None, gw, gx1, gx2
+
+    @staticmethod
+    def grads(mod, w, x1, x2, g, need_w, need_x1, need_x2):
+        """``(dw, dx1, dx2)`` (``None`` where not asked for) of the product for the cotangent ``g``."""
         dtype, dev = x1.dtype, x1.device
         Z = x1.shape[0]
         plan, lib = mod.fc_plan, _lib.load()
-        g = _aligned(g)
-        wd, x1d, x2d = _aligned(w.detach().to(dtype)), _aligned(x1.detach()), x2.detach().contiguous()
+        g = _aligned(g.detach().to(dtype))
+        wd, x1d, x2d = _aligned(w.detach().to(dtype)), _aligned(x1.detach()), x2.detach().to(dtype).contiguous()
         gw = gx1 = gx2 = None
-        need_w, need_x1, need_x2 = ctx.needs_input_grad[1], ctx.needs_input_grad[2], ctx.needs_input_grad[3]
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             code, es = _DTYPE_CODE[dtype], x1d.element_size()
@@ -663,7 +671,67 @@ class _FcFunction(torch.autograd.Function):
                 gw = gwd.to(w.dtype).reshape(w.shape)
             if gx2 is not None and x2.shape[0] == 1 and Z != 1:
                 gx2 = gx2.sum(0, keepdim=True)
-        return None, gw, gx1, gx2
+        return gw, gx1, gx2
+
+
+class _FcDw(torch.autograd.Function):
+    """``dW(x1, x2, g)``; ``w`` gives the shape and dtype of the result."""
+
+    @staticmethod
+    def forward(ctx, mod, x1, x2, g, w):
+        ctx.mod = mod
+        ctx.save_for_backward(x1, x2, g)
+        return _FcFunction.grads(mod, w, x1, x2, g, True, False, False)[0]
+
+    @staticmethod
+    def backward(ctx, c):  # c: shaped like the weights
+        x1, x2, g = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        return (None,
+                _FcDx1.apply(ctx.mod, c, g, x2, x1) if need[1] else None,
+                _FcDx2.apply(ctx.mod, c, x1, g, x2) if need[2] else None,
+                _FcFunction.apply(ctx.mod, c, x1, x2).to(g.dtype) if need[3] else None,
+                None)
+
+
+class _FcDx1(torch.autograd.Function):
+    """``dx1(w, g, x2)``; ``x1`` gives the dtype of the result."""
+
+    @staticmethod
+    def forward(ctx, mod, w, g, x2, x1):
+        ctx.mod = mod
+        ctx.save_for_backward(w, g, x2)
+        return _FcFunction.grads(mod, w, x1, x2, g, False, True, False)[1]
+
+    @staticmethod
+    def backward(ctx, c):  # c: shaped like x1
+        w, g, x2 = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        return (None,
+                _FcDw.apply(ctx.mod, c, x2, g, w) if need[1] else None,
+                _FcFunction.apply(ctx.mod, w, c, x2).to(g.dtype) if need[2] else None,
+                _FcDx2.apply(ctx.mod, w, c, g, x2) if need[3] else None,
+                None)
+
+
+class _FcDx2(torch.autograd.Function):
+    """``dx2(w, x1, g)``; ``x2`` gives the shape and dtype of the result."""
+
+    @staticmethod
+    def forward(ctx, mod, w, x1, g, x2):
+        ctx.mod = mod
+        ctx.save_for_backward(w, x1, g)
+        return _FcFunction.grads(mod, w, x1, x2, g, False, False, True)[2]
+
+    @staticmethod
+    def backward(ctx, c):  # c: shaped like x2
+        w, x1, g = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        return (None,
+                _FcDw.apply(ctx.mod, x1, c, g, w) if need[1] else None,
+                _FcDx1.apply(ctx.mod, w, g, c, x1) if need[2] else None,
+                _FcFunction.apply(ctx.mod, w, x1, c).to(g.dtype) if need[3] else None,
+                None)
 
 
 def _row_ranges(Z: int, Cn: int, offsets: torch.Tensor):
@@ -798,7 +866,7 @@ def _dense_bwd_op(mod_id: int, kind: int, w: torch.Tensor, x1: torch.Tensor, x2:
     if kind == 0:
         grads = _DenseFunction._backward_impl(ctx, g, ctx.needs_input_grad)[1:4]
     else:
-        grads = _FcFunction.backward(ctx, g)[1:4]
+        grads = _FcFunction.grads(ctx.mod, w, x1, x2, g, *ctx.needs_input_grad[1:4])
     return [x1.new_empty(0) if (t is None or not n) else t.contiguous() for t, n in zip(grads, need)]
 
 

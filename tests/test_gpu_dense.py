@@ -253,17 +253,41 @@ def test_linear_second_derivatives_match_oracle(device, dtype):
         assert rel_err(p, q) <= tol, (name, rel_err(p, q))
 
 
-def test_fully_connected_second_derivative_raises(device):
-    """The 4-operand form is differentiable once; a backward under ``create_graph=True`` says so instead of returning
-    detached gradients (a second derivative through them would silently be zero)."""
+def fc_second_derivatives(device, dtype, irreps, Z=60):
+    """All second derivatives of a scalar built from the three first gradients of a fully connected product: GPU module
+    against autograd through the CPU oracle.  Returns the largest relative error."""
     from cuequivariance_amd import cuet
 
-    ir = cue.Irreps("O3", "8x0e+8x1o")
+    ir = cue.Irreps("O3", irreps)
     m = cuet.FullyConnectedTensorProduct(ir, cue.Irreps("O3", "0e+1o"), ir, layout=cue.ir_mul, internal_weights=False)
-    x1 = torch.randn(10, ir.dim, device=device, requires_grad=True)
-    x2 = torch.randn(10, 4, device=device, requires_grad=True)
-    w = torch.randn(1, m.weight_numel, device=device, requires_grad=True)
+    g = torch.Generator().manual_seed(12)
+    ins = [torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g), torch.randn(Z, ir.dim, dtype=torch.float64, generator=g),
+           torch.randn(Z, 4, dtype=torch.float64, generator=g)]
+    ins = [t.to(dtype).double() for t in ins]
+    cot = torch.randn(Z, ir.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    probes = [torch.randn(t.shape, dtype=torch.float64, generator=g).to(dtype).double() for t in ins]
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+
+    def second(fwd, a, dev_, dt):
+        out = fwd(a)
+        grads = torch.autograd.grad(out, a, cot.to(dt).to(dev_), create_graph=True)
+        s = sum((gr * p.to(dt).to(dev_)).sum() for gr, p in zip(grads, probes)) + (grads[1] * grads[1]).sum()
+        return torch.autograd.grad(s, a)
+
+    want = second(lambda a: naive_segmented_polynomial(spec, a)[0], [t.clone().requires_grad_(True) for t in ins], torch.device("cpu"), torch.float64)
+    got = second(lambda a: m.f(a)[0], [t.to(dtype).to(device).requires_grad_(True) for t in ins], device, dtype)
+    return max(rel_err(p, q) for p, q in zip(got, want)), m
+
+
+def test_fully_connected_second_derivatives_match_oracle(device):
+    """The four trilinear forms (product and its three gradients) are closed under differentiation: ``create_graph=True``
+    stays on the fully connected kernels (here the table-driven ones; ``tests/test_jit.py`` covers the generated ones)."""
+    err, _ = fc_second_derivatives(device, torch.float32, "32x0e+32x1o")
+    assert err <= 2e-5, err
+
+
+def test_fully_connected_float64_second_derivative_raises(device):
+    """float64 runs the per-path kernels, differentiable once: a backward under ``create_graph=True`` says so instead of
+    returning detached gradients (a second derivative through them would silently be zero)."""
     with pytest.raises(NotImplementedError, match="second derivatives"):
-        torch.autograd.grad(m(x1, x2, w).sum(), [x1], create_graph=True)
-    (gx,) = torch.autograd.grad(m(x1, x2, w).sum(), [x1])  # (first order is unaffected)
-    assert gx.shape == x1.shape
+        fc_second_derivatives(device, torch.float64, "8x0e+8x1o")

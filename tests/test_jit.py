@@ -304,3 +304,13 @@ def test_fused_fully_connected_rows_beyond_2g_elements(device, jit_on):
     del out, dx1, dx2, x1, x2, cot
     gc.collect()
     torch.cuda.empty_cache()
+
+
+@pytest.mark.gpu
+def test_fused_fully_connected_second_derivatives(device, jit_on):
+    """Second derivatives through the generated fully connected kernels (each gradient is one of them again)."""
+    from tests.test_gpu_dense import fc_second_derivatives
+
+    err, m = fc_second_derivatives(device, torch.float32, "32x0e+32x1o")
+    assert _dense_of(m)._fused.get((torch.float32, True)) is not None
+    assert err <= 2e-5, err
