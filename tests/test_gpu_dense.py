@@ -291,3 +291,50 @@ def test_fully_connected_float64_second_derivative_raises(device):
     returning detached gradients (a second derivative through them would silently be zero)."""
     with pytest.raises(NotImplementedError, match="second derivatives"):
         fc_second_derivatives(device, torch.float64, "8x0e+8x1o")
+
+
+@pytest.mark.parametrize("layout", [cue.ir_mul, cue.mul_ir])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_fully_connected_with_scalar_attributes_matches_oracle(device, dtype, layout):
+    """A second operand of several invariant scalars (node attributes, ``5x0e``) is outside the 4-operand dense form; the
+    module evaluates it as the Linear map of the features ``x1[i, u] x2[v]`` with the same weights.  Forward, gradients
+    and second derivatives against the CPU oracle on the fully connected descriptor itself."""
+    from cuequivariance_amd import cuet
+
+    i1, i2, i3 = cue.Irreps("O3", "16x0e+16x1o+8x0e"), cue.Irreps("O3", "5x0e"), cue.Irreps("O3", "16x0e+8x1o")
+    m = cuet.FullyConnectedTensorProduct(i1, i2, i3, layout=layout, internal_weights=False)
+    assert m.f is None and m.f_outer is not None
+    g = torch.Generator().manual_seed(13)
+    Z = 45
+    ins = [torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g), torch.randn(Z, i1.dim, dtype=torch.float64, generator=g),
+           torch.randn(Z, i2.dim, dtype=torch.float64, generator=g)]
+    ins = [t.to(dtype).double() for t in ins]
+    cot = torch.randn(Z, i3.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    ref_mod = cuet.FullyConnectedTensorProduct(i1, i2, i3, layout=cue.ir_mul, internal_weights=False)
+    spec = spec_from_polynomial(ref_mod.f_per_sample._polynomial)
+
+    def columns(irreps):  # index of every ir_mul column in a row of the tested layout
+        idx, off = [], 0
+        for mul, ir in irreps:
+            d = ir.dim
+            idx += [off + (u * d + i if layout == cue.mul_ir else i * mul + u) for i in range(d) for u in range(mul)]
+            off += mul * d
+        return torch.tensor(idx)
+
+    c1, c2, c3 = columns(i1), columns(i2), columns(i3)
+
+    def oracle(a):  # the oracle works on ir_mul rows; the layout changes are permutations of columns
+        out = naive_segmented_polynomial(spec, [a[0], a[1][:, c1], a[2][:, c2]])[0]
+        return out[:, torch.argsort(c3)]
+
+    def run(fwd, a, dev_, dt):
+        out = fwd(a)
+        grads = torch.autograd.grad(out, a, cot.to(dt).to(dev_), create_graph=True)
+        second = torch.autograd.grad((grads[1] * grads[1]).sum() + (grads[0] * grads[0]).sum(), a)
+        return (out,) + grads + second
+
+    want = run(oracle, [t.clone().requires_grad_(True) for t in ins], torch.device("cpu"), torch.float64)
+    got = run(lambda a: m(a[1], a[2], a[0]), [t.to(dtype).to(device).requires_grad_(True) for t in ins], device, dtype)
+    tol = 1e-12 if dtype == torch.float64 else 2e-5
+    for i, (p, q) in enumerate(zip(got, want)):
+        assert rel_err(p, q) <= tol, (i, rel_err(p, q))
