@@ -522,8 +522,8 @@ def _first_order_only() -> None:
     come out detached and a second derivative through them would silently be zero."""
     if torch.is_grad_enabled():
         raise NotImplementedError(
-            "fused_tp / indexed_linear: second derivatives (create_graph=True) are built for shared weights in float32 / "
-            "bfloat16 (3- and 4-operand forms) only; the uniform-1d executor (per-sample weights, or method='uniform_1d' on a flattened descriptor) is "
+            "fused_tp: second derivatives (create_graph=True) of the 4-operand form are built for float32 / bfloat16 with the "
+            "second operand of multiplicity one; the uniform-1d executor (per-sample weights, or method='uniform_1d' on a flattened descriptor) is "
             "differentiable to any order")
 
 
@@ -781,20 +781,26 @@ class _IndexedDenseFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g):
-        _first_order_only()
+        # as for the shared-weight form: the two gradients are differentiable functions of their own
         mod = ctx.mod
         w, x1, offsets = ctx.saved_tensors
+        gw = _IndexedDw.apply(mod, x1, g, w, offsets) if ctx.needs_input_grad[1] else None
+        gx1 = _IndexedDx.apply(mod, g, w, offsets, x1) if ctx.needs_input_grad[2] else None
+        return None, gw, gx1, None
+
+    @staticmethod
+    def grads(mod, w, x1, offsets, g, need_w, need_x1):
         dtype = x1.dtype
         Z, Cn, W = x1.shape[0], w.shape[0], w.shape[1]
         lib = _lib.load()
-        g = g.contiguous()
+        g = g.detach().to(dtype).contiguous()
         wd = w.detach().to(dtype).contiguous()
         x1d = x1.detach().contiguous()
         gw = gx1 = None
         with torch.cuda.device(x1.device):
             stream = torch.cuda.current_stream(x1.device).cuda_stream
             code, es = _DTYPE_CODE[dtype], x1d.element_size()
-            if ctx.needs_input_grad[2]:
+            if need_x1:
                 gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
                 written = set()
                 ranges = _row_ranges(Z, Cn, offsets)
@@ -810,7 +816,7 @@ class _IndexedDenseFunction(torch.autograd.Function):
                                                   gx1.stride(0), da, count, offs.data_ptr(), Cn, 0, W, p.coeff, acc, stream),
                             "cueq_gemm_grouped",
                         )
-            if ctx.needs_input_grad[1]:
+            if need_w:
                 # dW_p[c] += coeff * sum over the rows z of class c of x1[z, i_seg]^T g[z, k_seg]: float32 accumulation
                 gw32 = torch.zeros(Cn, W, dtype=torch.float32, device=x1.device)
                 for p, count, da, dc in mod.fwd_groups if Z > 0 else []:
@@ -822,7 +828,41 @@ class _IndexedDenseFunction(torch.autograd.Function):
                             "cueq_gemm_grouped",
                         )
                 gw = gw32.to(w.dtype)
-        return None, gw, gx1, None
+        return gw, gx1
+
+
+class _IndexedDx(torch.autograd.Function):
+    """``dx`` of the indexed Linear as a function of ``(g, w)``; ``x1`` gives the dtype of the result."""
+
+    @staticmethod
+    def forward(ctx, mod, g, w, offsets, x1):
+        ctx.mod = mod
+        ctx.save_for_backward(g, w, offsets)
+        return _IndexedDenseFunction.grads(mod, w, x1, offsets, g, False, True)[1]
+
+    @staticmethod
+    def backward(ctx, c):
+        g, w, offsets = ctx.saved_tensors
+        dg = _IndexedDenseFunction.apply(ctx.mod, w, c, offsets).to(g.dtype) if ctx.needs_input_grad[1] else None
+        dw = _IndexedDw.apply(ctx.mod, c, g, w, offsets) if ctx.needs_input_grad[2] else None
+        return None, dg, dw, None, None
+
+
+class _IndexedDw(torch.autograd.Function):
+    """``dW`` (one row per class) of the indexed Linear as a function of ``(x1, g)``; ``w`` gives shape and dtype."""
+
+    @staticmethod
+    def forward(ctx, mod, x1, g, w, offsets):
+        ctx.mod = mod
+        ctx.save_for_backward(x1, g, offsets)
+        return _IndexedDenseFunction.grads(mod, w, x1, offsets, g, True, False)[0]
+
+    @staticmethod
+    def backward(ctx, c):
+        x1, g, offsets = ctx.saved_tensors
+        dx = _IndexedDx.apply(ctx.mod, g, c, offsets, x1) if ctx.needs_input_grad[1] else None
+        dg = _IndexedDenseFunction.apply(ctx.mod, c, x1, offsets).to(g.dtype) if ctx.needs_input_grad[2] else None
+        return None, dx, dg, None, None
 
 
 # ---------------------------------------------------------------------- traced execution (torch.compile / export)

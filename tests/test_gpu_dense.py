@@ -338,3 +338,31 @@ def test_fully_connected_with_scalar_attributes_matches_oracle(device, dtype, la
     tol = 1e-12 if dtype == torch.float64 else 2e-5
     for i, (p, q) in enumerate(zip(got, want)):
         assert rel_err(p, q) <= tol, (i, rel_err(p, q))
+
+
+def test_indexed_linear_second_derivatives_match_oracle(device):
+    """The indexed Linear under ``create_graph=True``: second derivatives against autograd through the oracle's
+    gather-then-contract evaluation."""
+    from cuequivariance_amd import cuet
+
+    irreps = cue.Irreps("O3", "16x0e+16x1o")
+    m = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=False, weight_classes=3, method="indexed_linear")
+    g = torch.Generator().manual_seed(14)
+    Z = 50
+    x = torch.randn(Z, irreps.dim, dtype=torch.float64, generator=g).float().double()
+    w = torch.randn(3, m.weight_numel, dtype=torch.float64, generator=g).float().double()
+    cot = torch.randn(Z, irreps.dim, dtype=torch.float64, generator=g).float().double()
+    idx = torch.sort(torch.randint(0, 3, (Z,), generator=g, dtype=torch.int32))[0]
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+
+    def second(fwd, a, dev_, dt):
+        out = fwd(a)
+        gw, gx = torch.autograd.grad(out, a, cot.to(dt).to(dev_), create_graph=True)
+        return torch.autograd.grad((gx * gx).sum() + (gw * gw).sum(), a)
+
+    want = second(lambda a: naive_segmented_polynomial(spec, [a[0], a[1]], {0: idx}, {}, {})[0],
+                  [w.clone().requires_grad_(True), x.clone().requires_grad_(True)], torch.device("cpu"), torch.float64)
+    got = second(lambda a: m(a[1], a[0], weight_indices=idx.to(device)),
+                 [w.float().to(device).requires_grad_(True), x.float().to(device).requires_grad_(True)], device, torch.float32)
+    for name, p, q in zip(("d/dw", "d/dx"), got, want):
+        assert rel_err(p, q) <= 2e-5, (name, rel_err(p, q))
