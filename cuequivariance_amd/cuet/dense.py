@@ -268,8 +268,10 @@ class _DenseFunction(torch.autograd.Function):
             gx1 = _LinearDx.apply(mod, g, w, x1.dtype) if ctx.needs_input_grad[2] else None
             gw = _LinearDw.apply(mod, x1, g, w) if ctx.needs_input_grad[1] else None
             return None, gw, gx1, None
-        _first_order_only()
-        return _DenseFunction._backward_impl(ctx, g, ctx.needs_input_grad)
+        gw = _FcDw.apply(mod, x1, x2, g, w, 0) if ctx.needs_input_grad[1] else None
+        gx1 = _FcDx1.apply(mod, w, g, x2, x1, 0) if ctx.needs_input_grad[2] else None
+        gx2 = _FcDx2.apply(mod, w, x1, g, x2, 0) if ctx.needs_input_grad[3] else None
+        return None, gw, gx1, gx2
 
     @staticmethod
     def _backward_impl(ctx, g, needs_input_grad):
@@ -517,16 +519,6 @@ class _FcPlan:
         return d
 
 
-def _first_order_only() -> None:
-    """Called at the top of a backward that is not itself differentiable: under ``create_graph=True`` the gradients would
-    come out detached and a second derivative through them would silently be zero."""
-    if torch.is_grad_enabled():
-        raise NotImplementedError(
-            "fused_tp: second derivatives (create_graph=True) of the 4-operand form are built for float32 / bfloat16 with the "
-            "second operand of multiplicity one; the uniform-1d executor (per-sample weights, or method='uniform_1d' on a flattened descriptor) is "
-            "differentiable to any order")
-
-
 def _aligned(t: torch.Tensor) -> torch.Tensor:
     """``t`` contiguous and starting on a 16-byte boundary (a copy when a view starts elsewhere): the fully connected
     kernels move rows in 16-byte pieces."""
@@ -582,9 +574,9 @@ class _FcFunction(torch.autograd.Function):
         # three: derivatives of any order stay on these kernels
         mod = ctx.mod
         w, x1, x2 = ctx.saved_tensors
-        gw = _FcDw.apply(mod, x1, x2, g, w) if ctx.needs_input_grad[1] else None
-        gx1 = _FcDx1.apply(mod, w, g, x2, x1) if ctx.needs_input_grad[2] else None
-        gx2 = _FcDx2.apply(mod, w, x1, g, x2) if ctx.needs_input_grad[3] else None
+        gw = _FcDw.apply(mod, x1, x2, g, w, 1) if ctx.needs_input_grad[1] else None
+        gx1 = _FcDx1.apply(mod, w, g, x2, x1, 1) if ctx.needs_input_grad[2] else None
+        gx2 = _FcDx2.apply(mod, w, x1, g, x2, 1) if ctx.needs_input_grad[3] else None
         return None, gw, gx1, gx2
 
     @staticmethod
@@ -674,64 +666,74 @@ class _FcFunction(torch.autograd.Function):
         return gw, gx1, gx2
 
 
+def _fc_grads(kind, mod, w, x1, x2, g, need_w, need_x1, need_x2):
+    """``(dw, dx1, dx2)`` of the 4-operand product: ``kind`` 1 on the fully connected kernels (float32 / bfloat16), 0 on
+    the per-path kernels (float64, shapes the others do not take)."""
+    if kind == 1:
+        return _FcFunction.grads(mod, w, x1, x2, g, need_w, need_x1, need_x2)
+    ctx = _GradContext(mod, w, x1)
+    ctx.saved_tensors, ctx.has_x2 = (w, x1, x2), True
+    return _DenseFunction._backward_impl(ctx, g.detach().to(x1.dtype), (False, need_w, need_x1, need_x2))[1:4]
+
+
 class _FcDw(torch.autograd.Function):
     """``dW(x1, x2, g)``; ``w`` gives the shape and dtype of the result."""
 
     @staticmethod
-    def forward(ctx, mod, x1, x2, g, w):
-        ctx.mod = mod
+    def forward(ctx, mod, x1, x2, g, w, kind):
+        ctx.mod, ctx.kind = mod, kind
         ctx.save_for_backward(x1, x2, g)
-        return _FcFunction.grads(mod, w, x1, x2, g, True, False, False)[0]
+        return _fc_grads(kind, mod, w, x1, x2, g, True, False, False)[0]
 
     @staticmethod
     def backward(ctx, c):  # c: shaped like the weights
         x1, x2, g = ctx.saved_tensors
         need = ctx.needs_input_grad
         return (None,
-                _FcDx1.apply(ctx.mod, c, g, x2, x1) if need[1] else None,
-                _FcDx2.apply(ctx.mod, c, x1, g, x2) if need[2] else None,
-                _FcFunction.apply(ctx.mod, c, x1, x2).to(g.dtype) if need[3] else None,
-                None)
+                _FcDx1.apply(ctx.mod, c, g, x2, x1, ctx.kind) if need[1] else None,
+                _FcDx2.apply(ctx.mod, c, x1, g, x2, ctx.kind) if need[2] else None,
+                _FUNCTIONS[ctx.kind].apply(ctx.mod, c, x1, x2).to(g.dtype) if need[3] else None,
+                None, None)
 
 
 class _FcDx1(torch.autograd.Function):
     """``dx1(w, g, x2)``; ``x1`` gives the dtype of the result."""
 
     @staticmethod
-    def forward(ctx, mod, w, g, x2, x1):
-        ctx.mod = mod
+    def forward(ctx, mod, w, g, x2, x1, kind):
+        ctx.mod, ctx.kind = mod, kind
         ctx.save_for_backward(w, g, x2)
-        return _FcFunction.grads(mod, w, x1, x2, g, False, True, False)[1]
+        return _fc_grads(kind, mod, w, x1, x2, g, False, True, False)[1]
 
     @staticmethod
     def backward(ctx, c):  # c: shaped like x1
         w, g, x2 = ctx.saved_tensors
         need = ctx.needs_input_grad
         return (None,
-                _FcDw.apply(ctx.mod, c, x2, g, w) if need[1] else None,
-                _FcFunction.apply(ctx.mod, w, c, x2).to(g.dtype) if need[2] else None,
-                _FcDx2.apply(ctx.mod, w, c, g, x2) if need[3] else None,
-                None)
+                _FcDw.apply(ctx.mod, c, x2, g, w, ctx.kind) if need[1] else None,
+                _FUNCTIONS[ctx.kind].apply(ctx.mod, w, c, x2).to(g.dtype) if need[2] else None,
+                _FcDx2.apply(ctx.mod, w, c, g, x2, ctx.kind) if need[3] else None,
+                None, None)
 
 
 class _FcDx2(torch.autograd.Function):
     """``dx2(w, x1, g)``; ``x2`` gives the shape and dtype of the result."""
 
     @staticmethod
-    def forward(ctx, mod, w, x1, g, x2):
-        ctx.mod = mod
+    def forward(ctx, mod, w, x1, g, x2, kind):
+        ctx.mod, ctx.kind = mod, kind
         ctx.save_for_backward(w, x1, g)
-        return _FcFunction.grads(mod, w, x1, x2, g, False, False, True)[2]
+        return _fc_grads(kind, mod, w, x1, x2, g, False, False, True)[2]
 
     @staticmethod
     def backward(ctx, c):  # c: shaped like x2
         w, x1, g = ctx.saved_tensors
         need = ctx.needs_input_grad
         return (None,
-                _FcDw.apply(ctx.mod, x1, c, g, w) if need[1] else None,
-                _FcDx1.apply(ctx.mod, w, g, c, x1) if need[2] else None,
-                _FcFunction.apply(ctx.mod, w, x1, c).to(g.dtype) if need[3] else None,
-                None)
+                _FcDw.apply(ctx.mod, x1, c, g, w, ctx.kind) if need[1] else None,
+                _FcDx1.apply(ctx.mod, w, g, c, x1, ctx.kind) if need[2] else None,
+                _FUNCTIONS[ctx.kind].apply(ctx.mod, w, x1, c).to(g.dtype) if need[3] else None,
+                None, None)
 
 
 def _row_ranges(Z: int, Cn: int, offsets: torch.Tensor):

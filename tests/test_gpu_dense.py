@@ -286,11 +286,10 @@ def test_fully_connected_second_derivatives_match_oracle(device):
     assert err <= 2e-5, err
 
 
-def test_fully_connected_float64_second_derivative_raises(device):
-    """float64 runs the per-path kernels, differentiable once: a backward under ``create_graph=True`` says so instead of
-    returning detached gradients (a second derivative through them would silently be zero)."""
-    with pytest.raises(NotImplementedError, match="second derivatives"):
-        fc_second_derivatives(device, torch.float64, "8x0e+8x1o")
+def test_fully_connected_float64_second_derivatives_match_oracle(device):
+    """float64 runs the per-path kernels; the same closure of four forms makes them differentiable to any order."""
+    err, _ = fc_second_derivatives(device, torch.float64, "8x0e+8x1o")
+    assert err <= 1e-12, err
 
 
 @pytest.mark.parametrize("layout", [cue.ir_mul, cue.mul_ir])
