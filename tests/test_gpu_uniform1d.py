@@ -115,7 +115,10 @@ def test_channelwise_non_registered_descriptor_uses_table_driven_kernels(device)
     m = cw_module("48x0e+48x1o+48x1e", "0e+1o+2e", "0e+1o+1e+2o")
     run_cw_case(device, m, N=40, Z=333, dtype=torch.float64, seed=3)
     run_cw_case(device, m, N=40, Z=333, dtype=torch.float32, seed=3)
-    assert not m.f.m._plan(torch.float32).specialised(device)
+    from cuequivariance_amd import jit
+
+    if not jit.enabled():  # (with compilation at first use left on, the descriptor gets kernels of its own)
+        assert not m.f.m._plan(torch.float32).specialised(device)
 
 
 def test_channelwise_mul_ir_layout_and_shared_internal_weights(device):
