@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "cueq_u1d_run",
     "cueq_segment_csr_workspace",
     "cueq_segment_csr_build",
+    "cueq_segment_csr_build_async",
     "cueq_seg_gemm",
     "cueq_seg_outer_workspace",
     "cueq_seg_outer",
@@ -158,6 +159,8 @@ def load() -> C.CDLL:
             C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
         ]
         lib.cueq_segment_csr_build.restype = C.c_int
+        lib.cueq_segment_csr_build_async.argtypes = lib.cueq_segment_csr_build.argtypes
+        lib.cueq_segment_csr_build_async.restype = C.c_int
         lib.cueq_seg_gemm.argtypes = [
             C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
             C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p,

@@ -42,6 +42,22 @@ __global__ void __launch_bounds__(256) csr_widen(const uint32_t* src, int64_t n,
   if (i < n) dst[i] = src[i];
 }
 
+// Capture-safe variant of csr_load_keys: nothing is reported to the host; ids outside [0, nrows) get the key nrows, so
+// they sort behind every row and no row's range includes them.
+__global__ void __launch_bounds__(256) csr_load_keys_clamped(const void* index, int is64, int64_t n, int64_t nrows,
+                                                             uint32_t* keys, uint32_t* iota) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int64_t v = load_index(index, is64, i);
+  keys[i] = static_cast<uint32_t>((v < 0 || v >= nrows) ? nrows : v);
+  iota[i] = static_cast<uint32_t>(i);
+}
+
+__global__ void __launch_bounds__(256) csr_zero_offsets(int64_t* offsets, int64_t count) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) offsets[i] = 0;
+}
+
 static size_t sort_temp_bytes(int64_t n) {
   size_t bytes = 0;
   hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, static_cast<const uint32_t*>(nullptr),
@@ -71,7 +87,8 @@ extern "C" int cueq_segment_csr_build(const void* index, int32_t index_is_64, in
   CUEQ_REQUIRE(n < (int64_t(1) << 31) && nrows < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE,
                "at most 2^31-1 ids / rows are supported");
   if (n == 0) {
-    CUEQ_CHECK_HIP(hipMemsetAsync(offsets, 0, (nrows + 1) * sizeof(int64_t), stream));
+    hipLaunchKernelGGL(csr_zero_offsets, dim3(static_cast<unsigned>((nrows + 1 + 255) / 256)), dim3(256), 0, stream, offsets, nrows + 1);
+    CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }
   CUEQ_REQUIRE(index && perm && workspace, CUEQ_ERR_INVALID, "null pointer");
@@ -87,7 +104,8 @@ extern "C" int cueq_segment_csr_build(const void* index, int32_t index_is_64, in
   size_t temp_bytes = sort_temp_bytes(n);
 
   const unsigned nb = static_cast<unsigned>((n + 255) / 256);
-  CUEQ_CHECK_HIP(hipMemsetAsync(flags, 0, 2 * sizeof(int), stream));
+  hipLaunchKernelGGL(csr_zero_offsets, dim3(1), dim3(256), 0, stream, reinterpret_cast<int64_t*>(flags), 1);  // both flags
+  CUEQ_CHECK_HIP(hipGetLastError());
   hipLaunchKernelGGL(csr_load_keys, dim3(nb), dim3(256), 0, stream, index, index_is_64, n, nrows, keys, iota, flags);
   CUEQ_CHECK_HIP(hipGetLastError());
   int h_flags[2] = {0, 0};
@@ -108,6 +126,46 @@ extern "C" int cueq_segment_csr_build(const void* index, int32_t index_is_64, in
   hipLaunchKernelGGL(csr_offsets, dim3(nbr), dim3(256), 0, stream, final_keys, n, nrows, offsets);
   CUEQ_CHECK_HIP(hipGetLastError());
   hipLaunchKernelGGL(csr_widen, dim3(nb), dim3(256), 0, stream, final_perm, n, perm);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
+// The same grouping with device-side work only: no host read of the "sorted" / "in range" flags, no memset node, so the
+// call may be recorded into a HIP graph and regroups from the live index buffer on every replay.  Always sorts
+// (stable radix sort, so already-sorted ids come out unchanged).  Ids outside [0, nrows) cannot be reported from
+// here: they are left out of every row's range.
+extern "C" int cueq_segment_csr_build_async(const void* index, int32_t index_is_64, int64_t n, int64_t nrows,
+                                            int64_t* offsets, int64_t* perm, void* workspace, int64_t workspace_bytes,
+                                            void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(n >= 0 && nrows >= 0 && offsets, CUEQ_ERR_INVALID, "bad arguments");
+  CUEQ_REQUIRE(n < (int64_t(1) << 31) && nrows < (int64_t(1) << 31) - 1, CUEQ_ERR_TOO_LARGE,
+               "at most 2^31-1 ids / 2^31-2 rows are supported");
+  if (n == 0) {
+    hipLaunchKernelGGL(csr_zero_offsets, dim3(static_cast<unsigned>((nrows + 1 + 255) / 256)), dim3(256), 0, stream, offsets, nrows + 1);
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
+  CUEQ_REQUIRE(index && perm && workspace, CUEQ_ERR_INVALID, "null pointer");
+  CUEQ_REQUIRE(workspace_bytes >= cueq_segment_csr_workspace(n, nrows), CUEQ_ERR_INVALID, "workspace too small");
+  char* w = static_cast<char*>(workspace);
+  const size_t a = align256(n * sizeof(uint32_t));
+  auto* keys = reinterpret_cast<uint32_t*>(w);
+  auto* iota = reinterpret_cast<uint32_t*>(w + a);
+  auto* skeys = reinterpret_cast<uint32_t*>(w + 2 * a);
+  auto* siota = reinterpret_cast<uint32_t*>(w + 3 * a);
+  void* temp = w + 4 * a + 256;
+  size_t temp_bytes = sort_temp_bytes(n);
+  const unsigned nb = static_cast<unsigned>((n + 255) / 256);
+  hipLaunchKernelGGL(csr_load_keys_clamped, dim3(nb), dim3(256), 0, stream, index, index_is_64, n, nrows, keys, iota);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  int end_bit = 1;
+  while ((int64_t(1) << end_bit) <= nrows && end_bit < 32) ++end_bit;  // keys reach nrows (the out-of-range key)
+  CUEQ_CHECK_HIP(hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys, skeys, iota, siota, static_cast<int>(n), 0, end_bit, stream));
+  const unsigned nbr = static_cast<unsigned>((nrows + 1 + 255) / 256);
+  hipLaunchKernelGGL(csr_offsets, dim3(nbr), dim3(256), 0, stream, skeys, n, nrows, offsets);
+  CUEQ_CHECK_HIP(hipGetLastError());
+  hipLaunchKernelGGL(csr_widen, dim3(nb), dim3(256), 0, stream, siota, n, perm);
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }

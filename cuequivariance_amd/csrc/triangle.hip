@@ -1978,11 +1978,12 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
   if (aligned && mixed_ok) {
     const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(batch));
     CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm: too many row tiles (M <= 8388480)");
-    KernelTimer timer(in_dtype == CUEQ_F32 ? "gemm_nt_f32" : "gemm_nt_bf16", stream);
     const int64_t out_es = out_dtype == CUEQ_F32 ? 4 : 2;
     const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
     // 256 x 256 tiles when both extents are multiples of 256 and there are enough of them to fill the chip
     const bool big = !mixed && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) * batch >= 2 * static_cast<int64_t>(device_cus());
+    // (the timing label names the tile size, so a test can tell which kernel a shape ran on)
+    KernelTimer timer(in_dtype == CUEQ_F32 ? (big ? "gemm_nt_f32_256" : "gemm_nt_f32") : (big ? "gemm_nt_bf16_256" : "gemm_nt_bf16"), stream);
     const dim3 grid_big(static_cast<unsigned>(N / 256), static_cast<unsigned>(M / 256), static_cast<unsigned>(batch));
 #define GEMM_ARGS(TI, TO) static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0, nullptr, 0, 0, 0, 0
 #define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, GEMM_ARGS(TI, TO))

@@ -198,30 +198,39 @@ _csr_cache: "OrderedDict[tuple, tuple]" = OrderedDict()
 
 
 def _segment_csr(index: torch.Tensor, nrows: int):
-    """(offsets[nrows+1], perm[n]) grouping batch ids by output row; cached per index tensor."""
-    key = (index.data_ptr(), index._version, index.numel(), int(nrows), index.dtype, index.device)
-    hit = _csr_cache.get(key)
-    if hit is not None:
-        _csr_cache.move_to_end(key)
-        return hit[1], hit[2]
+    """(offsets[nrows+1], perm[n]) grouping batch ids by output row.
+
+    Eager mode: built once per index tensor and cached (the build checks on the host that the ids are in range and
+    skips the sort when they are sorted already).  While the current stream is being captured into a HIP graph the
+    grouping is recorded into the graph instead (device-side work only, nothing cached), so every replay regroups from
+    whatever the index buffer holds then.  Index tensors made under ``torch.inference_mode()`` carry no version counter
+    and are not cached either."""
     lib = _lib.load()
     n = index.numel()
+    capturing = torch.cuda.is_current_stream_capturing()
+    cacheable = not capturing and not index.is_inference()
+    if cacheable:
+        key = (index.data_ptr(), index._version, n, int(nrows), index.dtype, index.device)
+        hit = _csr_cache.get(key)
+        if hit is not None:
+            _csr_cache.move_to_end(key)
+            return hit[1], hit[2]
     offsets = torch.empty(nrows + 1, dtype=torch.int64, device=index.device)
     perm = torch.empty(max(n, 1), dtype=torch.int64, device=index.device)
     ws_bytes = lib.cueq_segment_csr_workspace(n, nrows)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=index.device)
     stream = torch.cuda.current_stream(index.device).cuda_stream
+    build = lib.cueq_segment_csr_build_async if capturing else lib.cueq_segment_csr_build
     _lib.check(
-        lib.cueq_segment_csr_build(
-            index.data_ptr(), 1 if index.dtype == torch.int64 else 0, n, nrows,
-            offsets.data_ptr(), perm.data_ptr(), ws.data_ptr(), ws_bytes, stream,
-        ),
+        build(index.data_ptr(), 1 if index.dtype == torch.int64 else 0, n, nrows,
+              offsets.data_ptr(), perm.data_ptr(), ws.data_ptr(), ws_bytes, stream),
         "cueq_segment_csr_build",
     )
-    # the index tensor is kept alive with the entry so its address cannot be reused meanwhile
-    _csr_cache[key] = (index, offsets, perm)
-    while len(_csr_cache) > 32:
-        _csr_cache.popitem(last=False)
+    if cacheable:
+        # the index tensor is kept alive with the entry so its address cannot be reused meanwhile
+        _csr_cache[key] = (index, offsets, perm)
+        while len(_csr_cache) > 32:
+            _csr_cache.popitem(last=False)
     return offsets, perm
 
 

@@ -89,6 +89,9 @@ _transpose_by_address: dict = {}
 def _tables_for_info(info: torch.Tensor, device: torch.device):
     # the frontend passes the same registered buffer on every call: recognise it by address and version, so that only
     # the first call reads the table back to the host
+    # (tensors made under torch.inference_mode() have no version counter: they are read back on every call)
+    if info.is_inference():
+        return _tables_for_rows(tuple(map(tuple, info.cpu().to(torch.int64).tolist())), device)
     fast = (info.data_ptr(), info._version, tuple(info.shape), device.type, device.index)
     entry = _transpose_by_address.get(fast)
     if entry is not None and entry[0]() is info:

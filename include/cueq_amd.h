@@ -126,6 +126,12 @@ int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int6
 int64_t cueq_segment_csr_workspace(int64_t n, int64_t nrows);
 int cueq_segment_csr_build(const void* index, int32_t index_is_64, int64_t n, int64_t nrows,
                            int64_t* offsets, int64_t* perm, void* workspace, int64_t workspace_bytes, void* stream);
+/* Same grouping with device-side work only (always sorts; no host synchronisation, no memset node), so it can be
+ * recorded into a HIP graph and regroups from the live index buffer at every replay.  cueq_segment_csr_build reads two
+ * flags on the host (ids sorted already? in range?) and therefore cannot be captured.  Ids outside [0, nrows) cannot
+ * be reported here: they are left out of every row.  Same workspace size. */
+int cueq_segment_csr_build_async(const void* index, int32_t index_is_64, int64_t n, int64_t nrows,
+                                 int64_t* offsets, int64_t* perm, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* dense segmented contractions (matrix cores)                                */

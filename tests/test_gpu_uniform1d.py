@@ -200,6 +200,46 @@ def test_cfg2_full_size_properties(device, monkeypatch):
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), (out_s.double().abs() * cot.double().abs()).sum().item())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("deterministic", ["0", "1"])
+def test_cfg2_full_size_block_of_receivers_against_oracle(device, dtype, deterministic, monkeypatch):
+    """The benchmark's own problem (5 000 nodes, 100 000 edges, 128 channels, l <= 3) against the oracle on 200 contiguous
+    receiver rows: the output rows of the block depend only on the block's edges (all senders), and with a cotangent
+    that is zero outside the block so do all three gradients - dw and dx2 on the block's edges (exactly zero elsewhere)
+    and dx1 on every node.  The oracle evaluates just those edges; the GPU runs the whole problem in one call."""
+    monkeypatch.setenv("CUEQ_DETERMINISTIC", deterministic)
+    m = cw_module("128x0e+128x1o+128x2e+128x3o", "0e+1o+2e+3o", "0e+1o+2e+3o")
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+    g = torch.Generator().manual_seed(11)
+    N, E, r0, r1 = 5000, 100_000, 2417, 2617
+    x1 = torch.randn(N, 2048, generator=g).to(dtype)
+    x2 = torch.randn(E, 16, generator=g).to(dtype)
+    w = torch.randn(E, 2944, generator=g).to(dtype)
+    snd = torch.randint(0, N, (E,), generator=g, dtype=torch.int32)
+    rcv = torch.sort(torch.randint(0, N, (E,), generator=g, dtype=torch.int32))[0]
+    cot = torch.zeros(N, 12672, dtype=dtype)
+    cot[r0:r1] = torch.randn(r1 - r0, 12672, generator=g).to(dtype)
+    sel = ((rcv >= r0) & (rcv < r1)).nonzero().squeeze(1)
+    assert 3000 < sel.numel() < 5000 and torch.equal(sel, torch.arange(sel[0], sel[-1] + 1))
+    # oracle: the block's edges only, receivers renumbered to [0, 200)
+    a = [w[sel].clone().requires_grad_(True), x1.clone().requires_grad_(True), x2[sel].clone().requires_grad_(True)]
+    ref = naive_segmented_polynomial(spec, a, {1: snd[sel]}, {0: r1 - r0}, {0: rcv[sel] - r0})[0]
+    ref_dw, ref_dx1, ref_dx2 = torch.autograd.grad(ref, a, cot[r0:r1])
+    # GPU: the whole problem
+    b = [t.clone().to(device).requires_grad_(True) for t in (w, x1, x2)]
+    out = m(b[1], b[2], b[0], indices_1=snd.to(device), indices_out=rcv.to(device), size_out=N)
+    dw, dx1, dx2 = torch.autograd.grad(out, b, cot.to(device))
+    assert m.f.m._plan(dtype).specialised(device)
+    tol = TOL[dtype]
+    assert_close(out[r0:r1], ref, tol, "out rows of the block")
+    assert_close(dw[sel.to(device)], ref_dw, tol, "dw of the block's edges")
+    assert_close(dx2[sel.to(device)], ref_dx2, tol, "dx2 of the block's edges")
+    assert_close(dx1, ref_dx1, tol, "dx1 (all nodes)")
+    outside = torch.ones(E, dtype=torch.bool)
+    outside[sel] = False
+    assert dw[outside.to(device)].abs().max().item() == 0 and dx2[outside.to(device)].abs().max().item() == 0
+
+
 # --------------------------------------------------------------------------- indexing matrix (table-driven kernels)
 def small_poly():
     e = cue.descriptors.channelwise_tensor_product(

@@ -110,21 +110,33 @@ def test_hip_path_matches_oracle(device, dtype, direction, shape):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21), (160, 512, 256, 96)])
+@pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21), (160, 512, 256, 96),
+                                  (128, 512, 512, 512)])
 def test_gemm_operand_orders(device, dtype, trans_a, trans_b, dims):
     """cueq_gemm against torch.matmul in float64 for the four operand orders: tiled MFMA path (aligned extents,
-    partial tiles included), the 256 x 256 tiles (both extents multiples of 256, many tiles) and the element-wise
-    path (odd extents)."""
+    partial tiles included), the 256 x 256 tiles (both extents multiples of 256 and at least two tiles per compute
+    unit: the last case, which is the contraction of the N = 512, D = 128 update and of its two gradients) and the
+    element-wise path (odd extents).  The kernel each case ran on is read back from the library's timing labels."""
+    from cuequivariance_amd import _lib
     from cuequivariance_amd.cuet import triangle as tri
 
     batch, M, N, K = dims
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    aligned = all(v % 8 == 0 for v in (M, N, K))
+    big = M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) * batch >= 2 * cus
+    if dims == (128, 512, 512, 512):
+        assert big or cus > 256, "the benchmark's contraction shape must run on the 256 x 256 tiles"
+    label = ("gemm_nt_f32" if dtype == torch.float32 else "gemm_nt_bf16") + ("_256" if big else "") if aligned else "gemm_nt_simple"
     g = torch.Generator().manual_seed(M * 7 + N)
     A = torch.randn((batch, K, M) if trans_a else (batch, M, K), generator=g).to(dtype)
     B = torch.randn((batch, K, N) if trans_b else (batch, N, K), generator=g).to(dtype)
     A64 = A.double().transpose(1, 2) if trans_a else A.double()
     B64 = B.double() if trans_b else B.double().transpose(1, 2)
     ref = 0.5 * A64 @ B64
+    _lib.timing_begin()
     got = tri.gemm_nt(A.to(device), B.to(device), dtype, alpha=0.5, trans_a=trans_a, trans_b=trans_b)
+    ran = _lib.timing_end()
+    assert list(ran) == [label], (ran, label)
     assert rel_err(got, ref) <= TOL[dtype], rel_err(got, ref)
     prev = torch.randn(batch, M, N, generator=g).to(dtype)
     got2 = tri.gemm_nt(A.to(device), B.to(device), dtype, out=prev.to(device).clone(), accumulate=True, trans_a=trans_a, trans_b=trans_b)
@@ -173,6 +185,32 @@ def test_defaults_shapes_and_errors(device):
     with pytest.raises(ValueError):
         cuet.triangle_multiplicative_update(x.detach().cpu())
     assert int(cuet.TriMulPrecision.IEEE) == 3 and int(cuet.TriMulPrecision.NONE) == -1
+
+
+@pytest.mark.gpu
+def test_benchmark_size_against_oracle(device):
+    """The benchmarked case itself (one 512 x 512 pair tensor, 128 channels, bfloat16, outgoing, Bernoulli(0.9) mask):
+    forward and the gradient with respect to the pair tensor against the float64 oracle evaluated on the
+    bfloat16-rounded inputs, 2e-2 * max|ref|.  This is the only size at which the 256 x 256 contraction tiles, the
+    LDS-resident gate backward on 262 144 rows and the LayerNorm with layout change run inside the composed update."""
+    from cuequivariance_amd import _lib, cuet
+
+    p, cot = make_case(1, 512, 128, torch.bfloat16, 7)
+    pr = {k: v.clone() for k, v in p.items()}
+    pr["x"].requires_grad_(True)
+    ref = oracle_trimul(direction="outgoing", **pr)
+    (want,) = torch.autograd.grad(ref, [pr["x"]], cot)
+    ref = ref.detach()
+    pg = {k: v.to(torch.bfloat16).to(device) for k, v in p.items()}
+    pg["x"].requires_grad_(True)
+    _lib.timing_begin()
+    out = cuet.triangle_multiplicative_update(direction="outgoing", **pg)
+    (got,) = torch.autograd.grad(out, [pg["x"]], cot.to(torch.bfloat16).to(device))
+    ran = _lib.timing_end()
+    if torch.cuda.get_device_properties(device).multi_processor_count <= 256:
+        assert ran.get("gemm_nt_bf16_256", (0, 0))[0] == 3, ran  # the contraction and its two gradients
+    assert rel_err(out, ref) <= 2e-2, ("out", rel_err(out, ref))
+    assert rel_err(got, want) <= 2e-2, ("dx", rel_err(got, want))
 
 
 @pytest.mark.gpu
