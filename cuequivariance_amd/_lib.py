@@ -31,6 +31,8 @@ EXPORTED_SYMBOLS = (
     "cueq_u1d_desc_info",
     "cueq_u1d_workspace_size",
     "cueq_u1d_run",
+    "cueq_u1d_static_scratch_bytes",
+    "cueq_u1d_run_static",
     "cueq_segment_csr_workspace",
     "cueq_segment_csr_build",
     "cueq_segment_csr_build_async",
@@ -153,6 +155,10 @@ def load() -> C.CDLL:
         lib.cueq_u1d_workspace_size.restype = C.c_int64
         lib.cueq_u1d_run.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]
         lib.cueq_u1d_run.restype = C.c_int
+        lib.cueq_u1d_static_scratch_bytes.argtypes = []
+        lib.cueq_u1d_static_scratch_bytes.restype = C.c_int64
+        lib.cueq_u1d_run_static.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64, C.c_void_p]
+        lib.cueq_u1d_run_static.restype = C.c_int
         lib.cueq_segment_csr_workspace.argtypes = [C.c_int64, C.c_int64]
         lib.cueq_segment_csr_workspace.restype = C.c_int64
         lib.cueq_segment_csr_build.argtypes = [

@@ -545,3 +545,52 @@ extern "C" int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* bu
   if (plan->math_dtype == CUEQ_F64) return run_typed<double>(plan, buffers, batch, workspace, workspace_bytes, s);
   return run_typed<float>(plan, buffers, batch, workspace, workspace_bytes, s);
 }
+
+// ---- cueq_u1d_run for callers that cannot allocate -------------------------------------------------
+// The workspace of cueq_u1d_run (per-chunk partial rows of a batch-reduced output, per-channel-half partials of the
+// fused backward) lives in a file-scope device array instead of a caller-supplied buffer.  Every device that loads
+// this library holds its own copy of the array until the process ends.  The array's name is only a host-side handle:
+// the address a kernel may use is asked for once per device with hipGetSymbolAddress and kept.
+namespace cueq {
+constexpr int64_t kStaticScratchBytes = int64_t(32) << 20;  // 32 MiB
+constexpr int kMaxScratchDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kMaxScratchDevices] = {};
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up on the first call on that device).
+static int static_scratch(void** out) {
+  int dev = 0;
+  CUEQ_CHECK_HIP(hipGetDevice(&dev));
+  CUEQ_REQUIRE(dev >= 0 && dev < kMaxScratchDevices, CUEQ_ERR_UNSUPPORTED, "device %d beyond the %d this entry point serves", dev,
+               kMaxScratchDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    CUEQ_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    CUEQ_REQUIRE(p != nullptr, CUEQ_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return CUEQ_OK;
+}
+}  // namespace cueq
+
+extern "C" int64_t cueq_u1d_static_scratch_bytes(void) { return cueq::kStaticScratchBytes; }
+
+extern "C" int cueq_u1d_run_static(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch, void* stream) {
+  CUEQ_REQUIRE(plan && buffers, CUEQ_ERR_INVALID, "null argument");
+  CUEQ_REQUIRE(batch >= 0, CUEQ_ERR_INVALID, "negative batch size");
+  const int64_t need = cueq_u1d_workspace_size(plan, buffers, batch);
+  CUEQ_REQUIRE(need <= cueq::kStaticScratchBytes, CUEQ_ERR_TOO_LARGE,
+               "this call needs %lld bytes of scratch, the static array holds %lld: use cueq_u1d_run with a workspace",
+               (long long)need, (long long)cueq::kStaticScratchBytes);
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = cueq::static_scratch(&ws);
+    if (rc != CUEQ_OK) return rc;
+  }
+  // Every kernel that uses the workspace writes each element it later reads (partial rows are stored, not
+  // accumulated), so nothing has to be cleared between calls.
+  return cueq_u1d_run(plan, buffers, batch, ws, need > 0 ? cueq::kStaticScratchBytes : 0, stream);
+}

@@ -121,6 +121,15 @@ int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer
 int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size,
                  void* workspace, int64_t workspace_bytes, void* stream);
 
+/* cueq_u1d_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as cueq_u1d_run,
+ * but the workspace is a static device array of cueq_u1d_static_scratch_bytes() (32 MiB) that every device running
+ * the library holds until the process ends; the call allocates nothing.  A call shape whose
+ * cueq_u1d_workspace_size exceeds that returns CUEQ_ERR_TOO_LARGE.  All calls on one device share the array:
+ * calls that overlap on one device (different streams or threads) race; calls on one stream do not. */
+int64_t cueq_u1d_static_scratch_bytes(void);
+int cueq_u1d_run_static(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size, void* stream);
+
 /* Stable grouping of n row ids (values in [0, nrows)) by value: offsets[nrows+1], perm[n].
  * Deterministic (no atomics decide the order).  workspace: cueq_segment_csr_workspace(n, nrows) bytes. */
 int64_t cueq_segment_csr_workspace(int64_t n, int64_t nrows);
