@@ -26,14 +26,26 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# published dense peaks, TFLOP/s: matrix cores per input type, and the fp32 vector units
+MFMA_PEAK = {"bf16": 2500.0, "f32": 157.3}
+VALU_PEAK_F32 = 157.3
 
 # Bytes that left the L2 per launch at the default workload (5000 nodes, 100000 edges, fp32), from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE; KiB per dispatch) scaled by what the same
-# counters read for a 1 GiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Summary and commands:
-# profiles/channelwise_c128_l3_fp32_cfg2_hbm_traffic.txt.  Not measurable from inside this process.
+# counters read for a 1 GiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Not measurable from inside this
+# process: the figures are those of the profile named in TRAFFIC_SOURCE, taken with these kernels.
+TRAFFIC_SOURCE = "profiles/channelwise_c128_l3_fp32_cfg2_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, not of this run)"
 MEASURED_TRAFFIC_BYTES = {
     ("c128_l3_bwd_float", 5000, 100_000): 4.270e9,
     ("c128_l3_fwd_float", 5000, 100_000): 2.135e9,
+}
+
+# Vector instructions executed per batch element (edge, node) by the generated kernels, forward + backward, counted by
+# rocprofv3 --pmc SQ_INSTS_VALU over one launch each (profiles/*_valu_counters.txt).  One wave64 instruction is at
+# most 64 fused multiply-adds = 128 flops; the published fp32 vector peak counts 256 flops per compute unit and clock.
+VALU_INSTS_PER_ELEMENT = {
+    # workload: (wave64 instructions per batch element: forward, backward; source)
+    "cfg2": (2 * 510, 2 * 1255, "profiles/channelwise_c128_l3_fp32_cfg2_valu_counters.txt"),
 }
 
 
@@ -93,9 +105,20 @@ def cpu_baseline(torch, cue, module, host, sample_edges: int, sample_nodes: int,
     }
 
 
-def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
-    """Secondary workloads (BASELINE.json configs[2..4]); same timing discipline as the headline line."""
-    wl = args.workload
+def _roofs(bytes_, flops, seconds, flop_peak_tflops, flop_roof: str) -> dict:
+    """Position of a measured time against both roofs; the binding roof is the one whose minimum time is longer."""
+    hbm = bytes_ / seconds / 1e9 / HBM_PEAK_GBS
+    cmp_ = flops / seconds / 1e12 / flop_peak_tflops if flops else 0.0
+    t_hbm, t_cmp = bytes_ / (HBM_PEAK_GBS * 1e9), (flops / (flop_peak_tflops * 1e12) if flops else 0.0)
+    bound = "hbm" if t_hbm >= t_cmp else flop_roof
+    return {"hbm_frac": hbm, f"{flop_roof}_frac": cmp_, "bound": bound, "frac": hbm if bound == "hbm" else cmp_,
+            "algorithmic_bytes": bytes_, "flops": flops}
+
+
+def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warmup: int, graph: bool = False) -> dict:
+    """One secondary workload (BASELINE.json configs[0], [2], [3], [4]); same timing discipline as the headline line.
+    Both roofs are reported: algorithmic bytes against 8 TB/s and flops against the matrix-core peak of the input type
+    (dense workloads) or the fp32 vector peak (path-table workloads)."""
     if wl == "cfg1":
         Z = 4096
         i1, i2 = cue.Irreps("O3", "32x0e+32x1o+32x2e"), cue.Irreps("O3", "0e+1o+2e")
@@ -113,7 +136,10 @@ def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
         unit, units, dt = "samples/s", Z, "f32"
         d1, d2, dw, do = i1.dim, i2.dim, m.weight_numel, m.irreps_out.dim
         alg = {"fwd": Z * (d1 + d2 + dw + do) * 4, "bwd": Z * (2 * (d1 + d2 + dw) + do) * 4}
-        bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
+        # 83 flattened paths x 32 channels; per path and operation: 2 multiplies between the 3 inputs, 1 by the coefficient,
+        # 1 accumulate; forward = 1 operation, backward = 3
+        flops = {"fwd": Z * 83 * 32 * 4, "bwd": 3 * Z * 83 * 32 * 4}
+        flop_roof, flop_peak = "valu", VALU_PEAK_F32
         desc = ("configs[0]: channel-wise TP 32x0e+32x1o+32x2e (x) 0e+1o+2e, outputs up to l = 2, batch 4096, per-sample weights, "
                 "fwd + bwd (dx1, dx2, dw); 69 MB of traffic: launch-latency regime")
     elif wl == "cfg3":
@@ -133,12 +159,21 @@ def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
         unit, units, dt = "nodes/s", Z, "f32"
         # every distinct element once: fwd reads x and writes out; bwd reads x, g and writes dx (weights 10 x 3712 negligible)
         alg = {"fwd": Z * (2048 + 512) * 4, "bwd": Z * (2048 + 512 + 2048) * 4}
-        bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
+        # flops of the folded path table the kernels evaluate (4 + 51 + 425 terms of degree 1, 2, 3 after folding the
+        # 4 + 86 + 1949 paths onto sorted index tuples): a term of degree d costs d + 2 flops per channel and operation
+        # (d multiplies between its d + 1 inputs, one by the coefficient, one accumulate); the forward is one
+        # operation, the backward d + 1 (one per differentiated input)
+        terms = {1: 4, 2: 51, 3: 425}
+        fwd_f = sum(n * (d + 2) for d, n in terms.items())
+        bwd_f = sum(n * (d + 2) * (d + 1) for d, n in terms.items())
+        flops = {"fwd": Z * 128 * fwd_f, "bwd": Z * 128 * bwd_f}
+        flop_roof, flop_peak = "valu", VALU_PEAK_F32
         desc = ("configs[2]: symmetric contraction 128x(0e+1o+2e+3o) -> 128x(0e+1o), degree 3, 10 element types, "
-                "50000 nodes, int32 element index, fwd + bwd (dw, dx)")
+                "50000 nodes, int32 element index, fwd + bwd (dw, dx); flops are those of the folded path table "
+                "(the kernels share pair products between terms and execute fewer)")
     elif wl == "cfg4":
         Z = 200_000
-        dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+        dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
         irreps = cue.Irreps("O3", "128x0e+128x1o+128x2e")
         m = cuet.Linear(irreps, irreps, layout=cue.ir_mul, internal_weights=False, method="fused_tp")
         g = torch.Generator(device=dev).manual_seed(0)
@@ -150,14 +185,16 @@ def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
             return torch.autograd.grad(m(x, w), [w, x], cot)
 
         unit, units, dt = "rows/s", Z, "bf16" if dtype == torch.bfloat16 else "f32"
+        es = 2 if dtype == torch.bfloat16 else 4
         f = 2 * Z * 128 * 128 * 9
-        alg = {"fwd": f, "bwd": 2 * f}
-        bound, pu = "mfma", "TFLOP/s"
-        peak = 2500.0 if dtype == torch.bfloat16 else 157.3
+        flops = {"fwd": f, "bwd": 2 * f}
+        # fwd reads x, writes out; bwd reads x and g, writes dx (weights 49152 elements negligible)
+        alg = {"fwd": 2 * Z * 1152 * es, "bwd": 3 * Z * 1152 * es}
+        flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = "configs[3]: Linear 128x0e+128x1o+128x2e -> same, batch 200000, shared weights, fwd + bwd (dw, dx)"
     elif wl == "cfg4fc":
         Z = 50_000
-        dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+        dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
         i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e")
         m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, internal_weights=False)
         g = torch.Generator(device=dev).manual_seed(0)
@@ -172,18 +209,15 @@ def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
         unit, units, dt = "rows/s", Z, "bf16" if dtype == torch.bfloat16 else "f32"
         es = 2 if dtype == torch.bfloat16 else 4
         # every distinct element once: fwd reads x1, x2 and writes out; bwd reads x1, x2, g and writes dx1, dx2 (weights 20480 negligible)
-        if dtype == torch.float32:
-            # 11 distinct (weight block, x1 component) products of 64 x 64 per row; forward, dx1, dx2 and dw contract each once
-            f = 2 * Z * 64 * 64 * 11
-            alg = {"fwd": f, "bwd": 3 * f}
-            bound, peak, pu = "mfma", 157.3, "TFLOP/s"
-        else:
-            alg = {"fwd": Z * (256 + 9 + 256) * es, "bwd": Z * (256 + 9 + 256 + 256 + 9) * es}
-            bound, peak, pu = "hbm", HBM_PEAK_GBS, "GB/s"
+        alg = {"fwd": Z * (256 + 9 + 256) * es, "bwd": Z * (256 + 9 + 256 + 256 + 9) * es}
+        # 11 distinct (weight block, x1 component) products of 64 x 64 per row; forward, dx1, dx2 and dw contract each once
+        f = 2 * Z * 64 * 64 * 11
+        flops = {"fwd": f, "bwd": 3 * f}
+        flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = ("configs[3]: FullyConnectedTensorProduct 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, batch 50000, shared weights, "
                 "fwd + bwd (dw, dx1, dx2)")
-    else:
-        dtype = torch.float32 if args.dtype == "fp32" else torch.bfloat16
+    elif wl == "cfg5":
+        dtype = torch.float32 if dtype_name == "fp32" else torch.bfloat16
         n, D = 512, 128
         g = torch.Generator(device=dev).manual_seed(0)
 
@@ -202,50 +236,211 @@ def secondary(torch, cue, cuet, _lib, dev, args) -> dict:
             return torch.autograd.grad(cuet.triangle_multiplicative_update(x, "outgoing", **kw), [x], cot)
 
         unit, units, dt = "pair rows/s", n * n, "bf16" if dtype == torch.bfloat16 else "f32"
+        es = 2 if dtype == torch.bfloat16 else 4
         f = 2 * n * n * D * 4 * D + 2 * D * n ** 3 + 2 * n * n * D * 2 * D  # projections in, contraction, projections out
-        alg = {"fwd": f, "bwd": 2 * f}
-        bound, pu = "mfma", "TFLOP/s"
-        peak = 2500.0 if dtype == torch.bfloat16 else 157.3
+        flops = {"fwd": f, "bwd": 2 * f}
+        # fwd reads z and the mask, writes the update; bwd reads z, the mask and the cotangent, writes dz
+        alg = {"fwd": (2 * n * n * D + n * n) * es, "bwd": (3 * n * n * D + n * n) * es}
+        flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = "configs[4]: triangle multiplicative update, outgoing, z [1,512,512,128], mask Bernoulli(0.9), fwd + bwd w.r.t. z"
-    if args.graph:
+    else:
+        raise ValueError(wl)
+    if graph:
         # the step as one HIP graph: same kernels, no launch gaps (per-kernel events cannot be recorded inside a graph)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            for _ in range(max(args.warmup, 3)):
+            for _ in range(max(warmup, 3)):
                 step()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        cuda_graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(cuda_graph):
             step()
-        run = graph.replay
+        run = cuda_graph.replay
     else:
         run = step
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         run()
     torch.cuda.synchronize()
-    if not args.graph:
+    if not graph:
         _lib.timing_begin()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         run()
     torch.cuda.synchronize()
-    elapsed = (time.perf_counter() - t0) / args.steps
-    kernels = {} if args.graph else {
-        n_: {"launches": l, "avg_ms": t / max(l, 1), "ms_per_step": t / args.steps} for n_, (l, t) in _lib.timing_end().items()}
-    if args.graph:
+    elapsed = (time.perf_counter() - t0) / steps
+    kernels = {} if graph else {
+        n_: {"launches": l, "avg_ms": t / max(l, 1), "ms_per_step": t / steps} for n_, (l, t) in _lib.timing_end().items()}
+    if graph:
         desc += "; the step replayed as one HIP graph"
-    total = alg["fwd"] + alg["bwd"]
-    achieved = total / elapsed / (1e9 if bound == "hbm" else 1e12)
+    roofs = _roofs(alg["fwd"] + alg["bwd"], flops["fwd"] + flops["bwd"], elapsed, flop_peak, flop_roof)
+    achieved = ((alg["fwd"] + alg["bwd"]) / elapsed / 1e9) if roofs["bound"] == "hbm" else ((flops["fwd"] + flops["bwd"]) / elapsed / 1e12)
     return {
         "metric": f"{unit.split('/')[0]}/sec, {wl} fwd+bwd (secondary workload)", "value": units / elapsed, "unit": unit, "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": elapsed * 1e3, "higher_is_better": True, "scaling": "weak",
+        "steps": steps, "warmup": warmup, "ms_per_step": elapsed * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dt, "data": "synthetic", "config": {"workload": desc},
-        "roofline": {"bound": bound, "achieved": achieved, "peak": peak, "unit": pu, "frac": achieved / peak, "traffic": None,
-                     "scope": "whole step: algorithmic bytes or flops of forward + backward over the step time"},
+        "roofline": {"bound": roofs["bound"], "achieved": achieved, "peak": HBM_PEAK_GBS if roofs["bound"] == "hbm" else flop_peak,
+                     "unit": "GB/s" if roofs["bound"] == "hbm" else "TFLOP/s", "frac": roofs["frac"], "traffic": None,
+                     "hbm_frac": roofs["hbm_frac"], f"{flop_roof}_frac": roofs[f"{flop_roof}_frac"],
+                     "algorithmic_bytes": roofs["algorithmic_bytes"], "flops": roofs["flops"],
+                     "scope": "whole step: algorithmic bytes and flops of forward + backward over the step time, against 8 TB/s and the "
+                              f"{flop_roof} peak ({flop_peak} TFLOP/s); bound = the roof with the longer minimum time"},
         "kernels": kernels,
     }
+
+
+def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, warmup: int, deterministic: bool):
+    """The headline workload once; returns (JSON line, module, host inputs)."""
+    prev = os.environ.get("CUEQ_DETERMINISTIC")
+    os.environ["CUEQ_DETERMINISTIC"] = "1" if deterministic else "0"
+    try:
+        m = cuet.ChannelWiseTensorProduct(
+            cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "0e+1o+2e+3o"), "0e+1o+2e+3o",
+            layout=cue.ir_mul, shared_weights=False,
+        )
+        host = make_inputs(torch, cue, N, E, dtype)
+        node, sh, w, senders, receivers, cot = (t.to(dev) for t in host)
+        node.requires_grad_(True), sh.requires_grad_(True), w.requires_grad_(True)
+
+        def step():
+            out = m(node, sh, w, indices_1=senders, indices_out=receivers, size_out=N)
+            return torch.autograd.grad(out, [w, node, sh], cot)
+
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        _lib.timing_begin()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        kernels = _lib.timing_end()
+    finally:
+        if prev is None:
+            os.environ.pop("CUEQ_DETERMINISTIC", None)
+        else:
+            os.environ["CUEQ_DETERMINISTIC"] = prev
+    ms_per_step = elapsed / steps * 1e3
+    value = E / (elapsed / steps)
+
+    plan = m.f.m._plan(dtype)
+    specialised = bool(plan.specialised(dev) and plan.backward_plan((True, True, True)).specialised(dev))
+    s = 4 if dtype == torch.float32 else 8
+    alg = algorithmic_bytes(E, N, 2944, 2048, 16, 12672, s)
+    per_kernel = {}
+    for name, (launches, total_ms) in kernels.items():
+        kind = "fwd" if "_fwd_" in name else "bwd"
+        avg_ms = total_ms / max(launches, 1)
+        per_kernel[name] = {
+            "launches": launches, "avg_ms": avg_ms, "algorithmic_bytes": alg[kind],
+            "achieved_GBps": alg[kind] / (avg_ms * 1e-3) / 1e9,
+        }
+    dominant = max(per_kernel.items(), key=lambda kv: kv[1]["avg_ms"]) if per_kernel else None
+    roofline = None
+    if dominant is not None:
+        a = dominant[1]["achieved_GBps"]
+        traffic = MEASURED_TRAFFIC_BYTES.get((dominant[0], N, E)) if not deterministic else None
+        roofline = {
+            "bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
+            "traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic else None,
+            "kernel": dominant[0], "avg_ms": dominant[1]["avg_ms"],
+            "algorithmic_bytes_per_launch": dominant[1]["algorithmic_bytes"],
+        }
+    total_alg = alg["fwd"] + alg["bwd"]
+    # 353 flattened paths x 128 channels, 4 flops per path and operation (SURVEY formula), forward 1 operation, backward 3
+    nominal_flops = 4 * E * 353 * 128 * 4
+    line = {
+        "metric": "edges/sec, indexed channelwise TP fwd+bwd (128ch, lmax=3); % HBM roofline",
+        "value": value,
+        "unit": "edges/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if dtype == torch.float32 else "f64",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: MACE-style indexed channel-wise TP, 5000 nodes x 128x0e+128x1o+128x2e+128x3o, "
+                        "100000 edges x SH 0e+1o+2e+3o, per-edge weights [E,2944], int32 sender/receiver (receivers "
+                        "sorted), scatter-sum onto 5000 nodes, fwd + bwd (dw, dx1, dx2)",
+            "nodes": N, "edges": E, "specialised_kernels": specialised,
+            "dx1_scatter": "ordered" if deterministic else "fp-atomics",
+        },
+        "roofline": roofline,
+        "step_roofline_frac": (total_alg / (elapsed / steps)) / 1e9 / HBM_PEAK_GBS,
+        "step_valu_frac": nominal_flops / (elapsed / steps) / 1e12 / (VALU_PEAK_F32 if dtype == torch.float32 else 78.6),
+        "kernels": per_kernel,
+    }
+    return line, m, host
+
+
+def cpu_baseline_dense(torch, cue, wl: str, threads: int) -> dict:
+    """CPU baselines of the dense workloads: the oracle (plain torch on the host) on a bounded sample, fwd + bwd."""
+    import statistics as st
+
+    cores = threads if threads > 0 else min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    if wl == "cfg5":
+        from oracle.triangle import triangle_multiplicative_update as oracle_trimul
+
+        n, D = 192, 128
+
+        def r(*shape, scale=1.0):
+            return torch.randn(*shape, generator=g) * scale
+
+        x = r(1, n, n, D).requires_grad_(True)
+        kw = dict(mask=(torch.rand(1, n, n, generator=g) < 0.9).float(), norm_in_weight=torch.ones(D), norm_in_bias=torch.zeros(D),
+                  p_in_weight=r(2 * D, D, scale=D ** -0.5), g_in_weight=r(2 * D, D, scale=D ** -0.5),
+                  norm_out_weight=torch.ones(D), norm_out_bias=torch.zeros(D),
+                  p_out_weight=r(D, D, scale=D ** -0.5), g_out_weight=r(D, D, scale=D ** -0.5))
+        cot = r(1, n, n, D)
+
+        def once():
+            t0 = time.perf_counter()
+            torch.autograd.grad(oracle_trimul(x, "outgoing", **kw), [x], cot)
+            return time.perf_counter() - t0
+
+        units, unit = n * n, "pair rows/s"
+        sample = f"one {n} x {n} x {D} pair tensor (the workload has 512 x 512; the contraction grows with the cube), float32"
+    else:  # cfg4 Linear: three 128 x 128 blocks per irrep component on ir_mul slices = the oracle's per-path einsum
+        from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
+
+        Z = 20_000
+        irreps = cue.Irreps("O3", "128x0e+128x1o+128x2e")
+        e = cue.descriptors.linear(irreps, irreps)
+        spec = spec_from_polynomial(e.polynomial)
+        x = torch.randn(Z, 1152, generator=g).requires_grad_(True)
+        w = torch.randn(1, e.polynomial.inputs[0].size, generator=g).requires_grad_(True)
+        cot = torch.randn(Z, 1152, generator=g)
+
+        def once():
+            t0 = time.perf_counter()
+            out = naive_segmented_polynomial(spec, [w, x])[0]
+            torch.autograd.grad(out, [w, x], cot)
+            return time.perf_counter() - t0
+
+        units, unit = Z, "rows/s"
+        sample = f"{Z} of the 200000 rows, float32"
+    once()
+    t = st.median([once() for _ in range(3)])
+    return {"value": units / t, "unit": unit, "cores": cores, "kind": "port",
+            "sample": f"{sample}, fwd+bwd, median of 3 after 1 warm-up ({t:.2f} s each)"}
+
+
+def _compact(line: dict) -> dict:
+    r = line["roofline"]
+    out = {"ms_per_step": line["ms_per_step"], "value": line["value"], "unit": line["unit"], "dtype": line["dtype"],
+           "bound": r["bound"], "frac": r["frac"], "workload": line["config"]["workload"]}
+    for k in ("hbm_frac", "mfma_frac", "valu_frac"):
+        if k in r:
+            out[k] = r[k]
+    return out
 
 
 def main() -> int:
@@ -259,6 +454,7 @@ def main() -> int:
     ap.add_argument("--edges", type=int, default=100_000)
     ap.add_argument("--cpu-sample-edges", type=int, default=12000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true", help="headline line only (no 'secondary' object)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (default: the box's share, at most 16)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
@@ -266,18 +462,17 @@ def main() -> int:
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
     ap.add_argument("--graph", action="store_true",
                     help="secondary workloads only: capture the step into a HIP graph and time its replays")
-    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4fc", "cfg5"], default="cfg2",
-                    help="cfg2 (default) is the headline metric; the others print a secondary line for the same "
-                         "library: cfg1 the reference's CPU-sized channel-wise case, cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected product, "
-                         "cfg5 triangle update")
+    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4fc", "cfg5"], default=None,
+                    help="default: the headline metric (cfg2, fp32) with every other configuration in a 'secondary' object.  "
+                         "Naming a workload prints one line for it alone: cfg2 the headline, cfg1 the reference's CPU-sized "
+                         "channel-wise case, cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected "
+                         "product, cfg5 triangle update")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU only (got --gpus {args.gpus}); "
               "the path would shard over receiver ranges (no exchange in the forward, one reduce-scatter of the node gradient in the backward)",
               file=sys.stderr)
         return 2
-    if args.deterministic:
-        os.environ["CUEQ_DETERMINISTIC"] = "1"
 
     import torch
 
@@ -296,90 +491,58 @@ def main() -> int:
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "copy", "bytes_read": n * 4, "bytes_written": n * 4, "launches": 5}))
         return 0
-    if args.workload != "cfg2":
-        print(json.dumps(secondary(torch, cue, cuet, _lib, dev, args)))
+    if args.workload not in (None, "cfg2"):
+        print(json.dumps(secondary(torch, cue, cuet, _lib, dev, args.workload, args.dtype, args.steps, args.warmup, args.graph)))
         return 0
     if args.dtype == "bf16":
         print("bench.py: cfg2 is measured in fp32 or fp64 (the uniform-1d math types)", file=sys.stderr)
         return 2
     dtype = torch.float64 if args.dtype == "fp64" else torch.float32
     N, E = args.nodes, args.edges
-
-    m = cuet.ChannelWiseTensorProduct(
-        cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "0e+1o+2e+3o"), "0e+1o+2e+3o",
-        layout=cue.ir_mul, shared_weights=False,
-    )
-    host = make_inputs(torch, cue, N, E, dtype)
-    node, sh, w, senders, receivers, cot = (t.to(dev) for t in host)
-    node.requires_grad_(True), sh.requires_grad_(True), w.requires_grad_(True)
-
-    def step():
-        out = m(node, sh, w, indices_1=senders, indices_out=receivers, size_out=N)
-        return torch.autograd.grad(out, [w, node, sh], cot)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    _lib.timing_begin()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    kernels = _lib.timing_end()
-    ms_per_step = elapsed / args.steps * 1e3
-    value = E / (elapsed / args.steps)
-
-    plan = m.f.m._plan(dtype)
-    specialised = bool(plan.specialised(dev) and plan.backward_plan((True, True, True)).specialised(dev))
-    s = 4 if dtype == torch.float32 else 8
-    alg = algorithmic_bytes(E, N, 2944, 2048, 16, 12672, s)
-    per_kernel = {}
-    for name, (launches, total_ms) in kernels.items():
-        kind = "fwd" if "_fwd_" in name else "bwd"
-        avg_ms = total_ms / max(launches, 1)
-        per_kernel[name] = {
-            "launches": launches, "avg_ms": avg_ms, "algorithmic_bytes": alg[kind],
-            "achieved_GBps": alg[kind] / (avg_ms * 1e-3) / 1e9,
-        }
-    dominant = max(per_kernel.items(), key=lambda kv: kv[1]["avg_ms"]) if per_kernel else None
-    roofline = None
-    if dominant is not None:
-        a = dominant[1]["achieved_GBps"]
-        roofline = {
-            "bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((dominant[0], N, E)), "kernel": dominant[0], "avg_ms": dominant[1]["avg_ms"],
-            "algorithmic_bytes_per_launch": dominant[1]["algorithmic_bytes"],
-        }
-    total_alg = alg["fwd"] + alg["bwd"]
-    line = {
-        "metric": "edges/sec, indexed channelwise TP fwd+bwd (128ch, lmax=3); % HBM roofline",
-        "value": value,
-        "unit": "edges/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32" if dtype == torch.float32 else "f64",
-        "data": "synthetic",
-        "config": {
-            "workload": "configs[1]: MACE-style indexed channel-wise TP, 5000 nodes x 128x0e+128x1o+128x2e+128x3o, "
-                        "100000 edges x SH 0e+1o+2e+3o, per-edge weights [E,2944], int32 sender/receiver (receivers "
-                        "sorted), scatter-sum onto 5000 nodes, fwd + bwd (dw, dx1, dx2)",
-            "nodes": N, "edges": E, "specialised_kernels": specialised,
-            "dx1_scatter": "ordered" if os.environ.get("CUEQ_DETERMINISTIC") == "1" else "fp-atomics",
-        },
-        "roofline": roofline,
-        "step_roofline_frac": (total_alg / (elapsed / args.steps)) / 1e9 / HBM_PEAK_GBS,
-        "kernels": per_kernel,
-    }
+    line, m, host = run_cfg2(torch, cue, cuet, _lib, dev, dtype, N, E, args.steps, args.warmup, args.deterministic)
+    full = args.workload is None and not args.no_secondary
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(torch, cue, m, host, min(args.cpu_sample_edges, E), min(200, N), args.cpu_threads)
+    if full:
+        # every other configuration in the same run: fewer steps each, same discipline (warm-up, synchronise, wall clock)
+        del m, host
+        sec = {}
+        ssteps, swarm = 20, 5
+
+        def add(key, fn):
+            torch.cuda.empty_cache()
+            try:
+                sec[key] = fn()
+            except Exception as e:  # a secondary workload must not take the headline down with it
+                sec[key] = {"error": f"{type(e).__name__}: {e}"}
+
+        add("cfg2_fp32_ordered_dx1", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float32, N, E, ssteps, swarm, True)[0]))
+        add("cfg2_fp64", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float64, N, E, ssteps, swarm, False)[0]))
+        for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg4_linear_fp32", "cfg4", "fp32"),
+                            ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"),
+                            ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp32", "cfg5", "fp32")):
+            add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))
+        if not args.no_cpu_baseline:
+            # more CPU baselines (the oracle on this box's host cores, bounded samples): the headline workload on one
+            # thread, the dense workloads on the box's share of cores
+            h1 = make_inputs(torch, cue, N, E, torch.float32)
+            m1 = cuet.ChannelWiseTensorProduct(cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "0e+1o+2e+3o"),
+                                               "0e+1o+2e+3o", layout=cue.ir_mul, shared_weights=False)
+            sec["cpu_baselines"] = {
+                "cfg2_fp32_1_thread": cpu_baseline(torch, cue, m1, h1, 2000, 200, 1),
+                "cfg4_linear_fp32": cpu_baseline_dense(torch, cue, "cfg4", args.cpu_threads),
+                "cfg5_fp32": cpu_baseline_dense(torch, cue, "cfg5", args.cpu_threads),
+            }
+        line["secondary"] = sec
     print(json.dumps(line))
     return 0
+
+
+def _cfg2_compact(line: dict) -> dict:
+    return {"ms_per_step": line["ms_per_step"], "value": line["value"], "unit": line["unit"], "dtype": line["dtype"],
+            "bound": "hbm", "frac": line["step_roofline_frac"], "hbm_frac": line["step_roofline_frac"],
+            "valu_frac": line["step_valu_frac"], "dx1_scatter": line["config"]["dx1_scatter"],
+            "kernels_avg_ms": {k: v["avg_ms"] for k, v in line["kernels"].items()}, "workload": line["config"]["workload"]}
 
 
 if __name__ == "__main__":

@@ -23,6 +23,8 @@ BATCH_DIM_AUTO, BATCH_DIM_SHARED, BATCH_DIM_BATCHED, BATCH_DIM_INDEXED = -1, 0, 
 EXPORTED_SYMBOLS = (
     "cueq_last_error",
     "cueq_version",
+    "cueq_set_option",
+    "cueq_get_option",
     "cueq_timing_begin",
     "cueq_timing_end",
     "cueq_u1d_plan_create",
@@ -141,6 +143,10 @@ def load() -> C.CDLL:
         lib.cueq_last_error.restype = C.c_char_p
         lib.cueq_version.restype = C.c_char_p
         lib.cueq_timing_begin.restype = C.c_int
+        lib.cueq_set_option.argtypes = [C.c_char_p, C.c_int32]
+        lib.cueq_set_option.restype = C.c_int
+        lib.cueq_get_option.argtypes = [C.c_char_p]
+        lib.cueq_get_option.restype = C.c_int
         lib.cueq_timing_end.argtypes = [C.POINTER(TimingEntry), C.c_int]
         lib.cueq_timing_end.restype = C.c_int
         lib.cueq_u1d_plan_create.argtypes = [C.POINTER(U1dDesc), C.POINTER(C.c_void_p)]
@@ -236,6 +242,21 @@ def load() -> C.CDLL:
         lib.cueq_sum_rows.restype = C.c_int
         _lib = lib
     return _lib
+
+
+_ENV_OPTIONS = (("CUEQ_DETERMINISTIC", b"deterministic"), ("CUEQ_FORCE_GENERIC", b"force_generic"))
+_env_seen: dict = {}
+
+
+def sync_options_from_env() -> None:
+    """The library reads CUEQ_DETERMINISTIC / CUEQ_FORCE_GENERIC once; a process that changes them afterwards
+    (``os.environ[...] = "1"``) is followed here: called by the Python launch paths, two dictionary lookups when
+    nothing changed."""
+    for env, name in _ENV_OPTIONS:
+        v = os.environ.get(env)
+        if env not in _env_seen or _env_seen[env] != v:
+            _env_seen[env] = v
+            load().cueq_set_option(name, 1 if (v and v[0] == "1") else 0)
 
 
 def check(status: int, what: str) -> None:

@@ -123,14 +123,40 @@ def _lit(c: float, T: str) -> str:
 # ---------------------------------------------------------------------------------------------
 # forward
 # ---------------------------------------------------------------------------------------------
+def _block_cost(blk: Block) -> int:
+    return len(blk.entries) + 2 * len(blk.k_list)
+
+
 def _split_blocks(st: ChannelwiseStructure, nsplit: int) -> list[list[Block]]:
-    """Greedy balance of blocks over ``nsplit`` groups by path count, keeping the sorted order inside groups."""
+    """Blocks dealt out to ``nsplit`` groups (one wavefront each) so that no two groups read the same x1 segment: every
+    output segment belongs to one block, so groups then share nothing but x2 - each loads its own x1 segments and
+    weights, keeps its own accumulators (forward) or cotangent registers (backward) and owns the x1 gradient of its
+    segments.  Blocks are first joined into components that share x1 segments (for a channel-wise product: one per
+    irrep of the first operand), the components are balanced greedily by path count.  Fewer groups come back when
+    there are fewer components."""
+    parent = {}
+
+    def find(a):
+        while parent.setdefault(a, a) != a:
+            parent[a] = parent[parent[a]]
+            a = parent[a]
+        return a
+
+    for blk in st.blocks:
+        first = blk.i_list[0]
+        for i in blk.i_list[1:]:
+            parent[find(i)] = find(first)
+    comps = defaultdict(list)
+    for blk in st.blocks:
+        comps[find(blk.i_list[0])].append(blk)
+    comps = sorted(comps.values(), key=lambda c: -sum(_block_cost(b) for b in c))
+    nsplit = max(1, min(nsplit, len(comps)))
     groups = [[] for _ in range(nsplit)]
     load = [0] * nsplit
-    for blk in sorted(st.blocks, key=lambda b: -len(b.entries)):
+    for comp in comps:
         g = load.index(min(load))
-        groups[g].append(blk)
-        load[g] += len(blk.entries) + 2 * len(blk.k_list)
+        groups[g] += comp
+        load[g] += sum(_block_cost(b) for b in comp)
     for g in groups:
         g.sort(key=lambda blk: (blk.i_list, blk.j_list, blk.b))
     return groups
@@ -167,6 +193,7 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
     fp = T
     dpp = "v_fmac_f32_dpp" if T == "float" else "v_fmac_f64_dpp"
     groups = _split_blocks(st, nsplit)
+    nsplit = len(groups)
     L = []
     A = L.append
     A(f"// forward: {st.num_paths} paths, {len(st.blocks)} blocks, split over {nsplit} wave group(s)")
@@ -235,24 +262,24 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
             A(f"  {fp} " + ", ".join([f"{S}_yv{m} = 0" for m in ms] + [f"{S}_xv{i} = 0" for i in i_used]
                                       + [f"{S}_wv{blk.b} = 0" for blk in blocks]) + ";")
         if prefetch:
+            # The rows of the next batch element are requested before the arithmetic of the current one.  The requests
+            # are unconditional (past the end the last element is fetched again): after a conditional request the
+            # number of outstanding loads is unknown and the wait before the arithmetic becomes "all of them",
+            # the ones just issued included.
             A("  if (z0 < z1) {")
             load("a", "z0", "    ")
-            A("  }")
-            A("  for (int64_t zz = z0; zz < z1; zz += 2) {")
-            A("    if (zz + 1 < z1) {")
-            load("b", "zz + 1", "      ")
-            A("    }")
-            A("    __builtin_amdgcn_sched_barrier(0);")
-            A("    {")
-            body("a", "      ")
-            A("    }")
-            A("    if (zz + 1 >= z1) break;")
-            A("    if (zz + 2 < z1) {")
-            load("a", "zz + 2", "      ")
-            A("    }")
-            A("    __builtin_amdgcn_sched_barrier(0);")
-            A("    {")
-            body("b", "      ")
+            A("    for (int64_t zz = z0; zz < z1; zz += 2) {")
+            load("b", "(zz + 1 < z1 ? zz + 1 : z1 - 1)", "      ")
+            A("      __builtin_amdgcn_sched_barrier(0);")
+            A("      {")
+            body("a", "        ")
+            A("      }")
+            A("      if (zz + 1 >= z1) break;")
+            load("a", "(zz + 2 < z1 ? zz + 2 : z1 - 1)", "      ")
+            A("      __builtin_amdgcn_sched_barrier(0);")
+            A("      {")
+            body("b", "        ")
+            A("      }")
             A("    }")
             A("  }")
         else:
@@ -295,149 +322,179 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
 # ---------------------------------------------------------------------------------------------
 # backward
 # ---------------------------------------------------------------------------------------------
-def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: int, prefetch: bool = False) -> str:
-    """HIP source of the fused backward kernel (dw, dx1, dx2 in one pass).  With ``prefetch`` the operands of the next
-    batch row (x1 row, weight row, x2 row, indices) are fetched into a second register set while the current row is
-    processed.  Measured on the 128-channel l <= 3 case: 219 instead of 178 registers, no spills, same time
-    (0.759 vs 0.757 ms): the loop does not wait on these loads, so the option is off."""
+def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: int, prefetch: bool = False, nsplit: int = 1) -> str:
+    """HIP source of the fused backward kernel (dw, dx1, dx2 in one pass).
+
+    ``nsplit`` > 1 deals the blocks out to that many wavefronts per (range of batch rows, 64 channels) with disjoint x1
+    segments (``_split_blocks``): each holds only the cotangent segments of its own blocks in registers, loads its
+    own x1 segments and weights, stores its own weight gradients and owns the x1 gradient of its segments; only the x2
+    gradient is shared, as one more partial row per wavefront for the fold that already sums the channel chunks.
+    Fewer registers per wavefront, more wavefronts per SIMD.
+
+    With ``prefetch`` the operands of the next batch row (x1 row, weight row, x2 row, indices) are fetched into a second
+    register set while the current row is processed."""
     fp = T
     L = []
     A = L.append
-    A("// backward: fused dw / dx1 / dx2; every wavefront owns one contiguous, equally sized range of batch rows")
+    nch = (st.extent + 63) // 64
+    groups = _split_blocks(st, nsplit)
+    nsplit = len(groups)
+    nparts = nch * nsplit
+    i_all = sorted({i for blk in st.blocks for i in blk.i_list})
+    w_all = sorted({blk.b for blk in st.blocks})
+    A(f"// backward: fused dw / dx1 / dx2; every wavefront owns one contiguous, equally sized range of batch rows; the blocks are")
+    A(f"// dealt out to {nsplit} wavefront(s) per range and channel chunk")
+    for q, blocks in enumerate(groups):
+        ks = sorted({k for blk in blocks for k in blk.k_list})
+        i_used = sorted({i for blk in blocks for i in blk.i_list})
+        j_used = sorted({j for blk in blocks for j in blk.j_list})
+        # segments nobody computes (all coefficients zero) are zero-filled by the first wavefront
+        i_zero = [i for i in range(st.nseg_x1) if i not in i_all] if q == 0 else []
+        w_zero = [b for b in range(st.nseg_w) if b not in w_all] if q == 0 else []
+
+        def load(S: str, zz: str, ind: str):
+            A(f"{ind}{{")
+            A(f"{ind}  const int64_t z = {zz};")
+            A(f"{ind}  {S}_grow = z;")
+            A(f"{ind}  if (G_IDX) {S}_grow = g_idx64 ? static_cast<const int64_t*>(g_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(g_index)[z]);")
+            A(f"{ind}  {S}_srow = z;")
+            A(f"{ind}  if (X1_IDX) {S}_srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
+            A(f"{ind}  const {fp}* __restrict__ x1p = x1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
+            A(f"{ind}  const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
+            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
+            for i in i_used:
+                A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
+            for blk in blocks:
+                A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
+            for j in j_used:
+                A(f"{ind}  {S}_yv{j} = x2p[{j}];")
+            A(f"{ind}}}")
+
+        def body(S: str, zz: str, ind: str):
+            A(f"{ind}const int64_t z = {zz};")
+            A(f"{ind}if ({S}_grow != grow_cur) {{")
+            A(f"{ind}  grow_cur = {S}_grow;")
+            A(f"{ind}  const {fp}* __restrict__ gp = g + grow_cur * {st.nseg_out * st.extent}ll;")
+            for k in ks:
+                A(f"{ind}  gr{k} = STREAM_LOAD(gp + {k * st.extent} + uu);")
+            A(f"{ind}}}")
+            A(f"{ind}{fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
+            for i in i_used:
+                A(f"{ind}{fp} dxa{i} = 0;")
+            for j in j_used:
+                A(f"{ind}{fp} pj{j} = 0;")
+            for blk in blocks:
+                A(f"{ind}{{  // block w[{blk.b}]")
+                A(f"{ind}  const {fp} wb = {S}_wv{blk.b};")
+                gij = defaultdict(list)
+                for i, j, k, c in blk.entries:
+                    gij[(i, j)].append((k, c))
+                A(f"{ind}  {fp} dwb = 0;")
+                for j in blk.j_list:
+                    A(f"{ind}  {fp} F{j} = 0;")
+                # per x1 component: G = sum_k c g_k is a temporary feeding both D (with x2) and F (with x1)
+                for i in blk.i_list:
+                    A(f"{ind}  {{")
+                    A(f"{ind}    {fp} D = 0;")
+                    for j in blk.j_list:
+                        if (i, j) not in gij:
+                            continue
+                        expr = None
+                        for k, c in gij[(i, j)]:
+                            expr = f"{_lit(c, T)} * gr{k}" if expr is None else f"fma({_lit(c, T)}, gr{k}, {expr})"
+                        A(f"{ind}    {{ const {fp} G = {expr}; D = fma(G, {S}_yv{j}, D); F{j} = fma(G, {S}_xv{i}, F{j}); }}")
+                    A(f"{ind}    dwb = fma({S}_xv{i}, D, dwb); dxa{i} = fma(wb, D, dxa{i});")
+                    A(f"{ind}  }}")
+                A(f"{ind}  if (active) STREAM_STORE(dwb, dwp + {blk.b * st.extent} + uu);")
+                for j in blk.j_list:
+                    A(f"{ind}  pj{j} = fma(wb, F{j}, pj{j});")
+                A(f"{ind}}}")
+                A(f"{ind}__builtin_amdgcn_sched_barrier(0);")
+            for b_ in w_zero:
+                A(f"{ind}if (active) STREAM_STORE({fp}(0), dwp + {b_ * st.extent} + uu);")
+            # dx1: scatter
+            A(f"{ind}if (active) {{")
+            A(f"{ind}  if (ATOMIC_DX1) {{")
+            A(f"{ind}    {fp}* dp = dx1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
+            for i in i_used:
+                A(f"{ind}    unsafeAtomicAdd(dp + ({i * st.extent} + uu), dxa{i});")
+            A(f"{ind}  }} else {{")
+            A(f"{ind}    {fp}* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
+            for i in sorted(i_used + i_zero):
+                A(f"{ind}    dp[{i * st.extent} + uu] = " + (f"dxa{i};" if i in i_used else "0;"))
+            A(f"{ind}  }}")
+            A(f"{ind}}}")
+            # dx2: reduce over the 64 lanes; channel chunks and wavefronts of one batch row are folded afterwards
+            A(f"{ind}if (!active) {{" + " ".join(f"pj{j} = 0;" for j in j_used) + "}")
+            for j in j_used:
+                A(f"{ind}pj{j} = wave_sum(pj{j});")
+            A(f"{ind}if (lane == 0) {{")
+            if nparts == 1:
+                A(f"{ind}  {fp}* __restrict__ d2 = dx2 + z * {st.nseg_x2}ll;")
+            else:
+                A(f"{ind}  {fp}* __restrict__ d2 = dx2_partial + (z * {nparts} + ch * {nsplit} + {q}) * {st.nseg_x2}ll;")
+            for j in range(st.nseg_x2):
+                A(f"{ind}  d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+            A(f"{ind}}}")
+
+        A("template <bool X1_IDX, bool G_IDX, bool ATOMIC_DX1>")
+        A(f"__device__ __forceinline__ void bwd_group{q}(BWD_PARAMS, int64_t z0, int64_t z1, int lane, int uu, bool active, int ch) {{")
+        for k in ks:
+            A(f"  {fp} gr{k} = 0;")
+        A("  int64_t grow_cur = -1;")
+        sets = ("a", "b") if prefetch else ("a",)
+        for S in sets:
+            A(f"  int64_t {S}_grow = -1, {S}_srow = 0;")
+            A(f"  {fp} " + ", ".join([f"{S}_xv{i} = 0" for i in i_used] + [f"{S}_wv{blk.b} = 0" for blk in blocks]
+                                      + [f"{S}_yv{j} = 0" for j in j_used]) + ";")
+        if prefetch:
+            # one copy of the body (two copies drive the register allocator into hundreds of spills): set "a" is the row in
+            # work, set "b" the row being fetched; "a = b" at the end of the iteration
+            A("  if (z0 < z1) {")
+            load("a", "z0", "    ")
+            A("  }")
+            A("  for (int64_t zz = z0; zz < z1; ++zz) {")
+            A("    {")
+            load("b", "(zz + 1 < z1 ? zz + 1 : zz)", "      ")
+            A("    }")
+            A("    __builtin_amdgcn_sched_barrier(0);")
+            A("    {")
+            body("a", "zz", "      ")
+            A("    }")
+            A("    a_grow = b_grow; a_srow = b_srow;")
+            A("    " + " ".join([f"a_xv{i} = b_xv{i};" for i in i_used] + [f"a_wv{blk.b} = b_wv{blk.b};" for blk in blocks]
+                                 + [f"a_yv{j} = b_yv{j};" for j in j_used]))
+            A("  }")
+        else:
+            A("  for (int64_t zz = z0; zz < z1; ++zz) {")
+            load("a", "zz", "    ")
+            A("    {")
+            body("a", "zz", "      ")
+            A("    }")
+            A("  }")
+        A("}")
+        A("")
     A("template <bool X1_IDX, bool G_IDX, bool ATOMIC_DX1>")
     A(f"__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu({waves_per_eu}))) bwd_kernel(BWD_PARAMS) {{")
-    nch = (st.extent + 63) // 64
     A("  const int lane = threadIdx.x;")
     A("  int64_t wid = blockIdx.x;")
+    A(f"  const int q = static_cast<int>(wid % {nsplit}); wid /= {nsplit};")
     A(f"  const int ch = static_cast<int>(wid % {nch}); const int64_t cid = wid / {nch};")
     if st.extent % 64 == 0:
         A("  const int uu = ch * 64 + lane; constexpr bool active = true;")
     else:
         A(f"  const int u = ch * 64 + lane; const bool active = u < {st.extent}; const int uu = active ? u : 0;")
-    A(f"  const int64_t nranges = gridDim.x / {nch};")
+    A(f"  const int64_t nranges = gridDim.x / {nparts};")
     A("  const int64_t z0 = cid * batch / nranges, z1 = (cid + 1) * batch / nranges;")
-    for k in range(st.nseg_out):
-        A(f"  {fp} gr{k} = 0;")
-    A("  int64_t grow_cur = -1;")
-    i_used = sorted({i for blk in st.blocks for i in blk.i_list})
-    j_used = sorted({j for blk in st.blocks for j in blk.j_list})
-
-    def load(S: str, zz: str, ind: str):
-        A(f"{ind}{{")
-        A(f"{ind}  const int64_t z = {zz};")
-        A(f"{ind}  {S}_grow = z;")
-        A(f"{ind}  if (G_IDX) {S}_grow = g_idx64 ? static_cast<const int64_t*>(g_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(g_index)[z]);")
-        A(f"{ind}  {S}_srow = z;")
-        A(f"{ind}  if (X1_IDX) {S}_srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
-        A(f"{ind}  const {fp}* __restrict__ x1p = x1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
-        A(f"{ind}  const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
-        A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
-        for i in i_used:
-            A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
-        for blk in st.blocks:
-            A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
-        for j in j_used:
-            A(f"{ind}  {S}_yv{j} = x2p[{j}];")
-        A(f"{ind}}}")
-
-    def body(S: str, zz: str, ind: str):
-        A(f"{ind}const int64_t z = {zz};")
-        A(f"{ind}if ({S}_grow != grow_cur) {{")
-        A(f"{ind}  grow_cur = {S}_grow;")
-        A(f"{ind}  const {fp}* __restrict__ gp = g + grow_cur * {st.nseg_out * st.extent}ll;")
-        for k in range(st.nseg_out):
-            A(f"{ind}  gr{k} = STREAM_LOAD(gp + {k * st.extent} + uu);")
-        A(f"{ind}}}")
-        A(f"{ind}{fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
-        for i in i_used:
-            A(f"{ind}{fp} dxa{i} = 0;")
-        for j in j_used:
-            A(f"{ind}{fp} pj{j} = 0;")
-        for blk in st.blocks:
-            A(f"{ind}{{  // block w[{blk.b}]")
-            A(f"{ind}  const {fp} wb = {S}_wv{blk.b};")
-            gij = defaultdict(list)
-            for i, j, k, c in blk.entries:
-                gij[(i, j)].append((k, c))
-            A(f"{ind}  {fp} dwb = 0;")
-            for j in blk.j_list:
-                A(f"{ind}  {fp} F{j} = 0;")
-            # per x1 component: G = sum_k c g_k is a temporary feeding both D (with x2) and F (with x1)
-            for i in blk.i_list:
-                A(f"{ind}  {{")
-                A(f"{ind}    {fp} D = 0;")
-                for j in blk.j_list:
-                    if (i, j) not in gij:
-                        continue
-                    expr = None
-                    for k, c in gij[(i, j)]:
-                        expr = f"{_lit(c, T)} * gr{k}" if expr is None else f"fma({_lit(c, T)}, gr{k}, {expr})"
-                    A(f"{ind}    {{ const {fp} G = {expr}; D = fma(G, {S}_yv{j}, D); F{j} = fma(G, {S}_xv{i}, F{j}); }}")
-                A(f"{ind}    dwb = fma({S}_xv{i}, D, dwb); dxa{i} = fma(wb, D, dxa{i});")
-                A(f"{ind}  }}")
-            A(f"{ind}  if (active) STREAM_STORE(dwb, dwp + {blk.b * st.extent} + uu);")
-            for j in blk.j_list:
-                A(f"{ind}  pj{j} = fma(wb, F{j}, pj{j});")
-            A(f"{ind}}}")
-            A(f"{ind}__builtin_amdgcn_sched_barrier(0);")
-        # dx1: scatter
-        A(f"{ind}if (active) {{")
-        A(f"{ind}  if (ATOMIC_DX1) {{")
-        A(f"{ind}    {fp}* dp = dx1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
-        for i in i_used:
-            A(f"{ind}    unsafeAtomicAdd(dp + ({i * st.extent} + uu), dxa{i});")
-        A(f"{ind}  }} else {{")
-        A(f"{ind}    {fp}* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
-        for i in range(st.nseg_x1):
-            A(f"{ind}    dp[{i * st.extent} + uu] = " + (f"dxa{i};" if i in i_used else "0;"))
-        A(f"{ind}  }}")
-        A(f"{ind}}}")
-        # dx2: reduce over the 64 lanes, then combine channel chunks
-        A(f"{ind}if (!active) {{" + " ".join(f"pj{j} = 0;" for j in j_used) + "}")
-        for j in j_used:
-            A(f"{ind}pj{j} = wave_sum(pj{j});")
-        A(f"{ind}if (lane == 0) {{")
-        if nch == 1:
-            A(f"{ind}  {fp}* __restrict__ d2 = dx2 + z * {st.nseg_x2}ll;")
-        else:
-            A(f"{ind}  {fp}* __restrict__ d2 = dx2_partial + (z * {nch} + ch) * {st.nseg_x2}ll;")
-        for j in range(st.nseg_x2):
-            A(f"{ind}  d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
-        A(f"{ind}}}")
-
-    sets = ("a", "b") if prefetch else ("a",)
-    for S in sets:
-        A(f"  int64_t {S}_grow = -1, {S}_srow = 0;")
-        A(f"  {fp} " + ", ".join([f"{S}_xv{i} = 0" for i in i_used] + [f"{S}_wv{blk.b} = 0" for blk in st.blocks]
-                                  + [f"{S}_yv{j} = 0" for j in j_used]) + ";")
-    if prefetch:
-        # one copy of the body (two copies drive the register allocator into hundreds of spills): set "a" is the row in
-        # work, set "b" the row being fetched; "a = b" at the end of the iteration
-        A("  if (z0 < z1) {")
-        load("a", "z0", "    ")
-        A("  }")
-        A("  for (int64_t zz = z0; zz < z1; ++zz) {")
-        A("    {")
-        load("b", "(zz + 1 < z1 ? zz + 1 : zz)", "      ")
-        A("    }")
-        A("    __builtin_amdgcn_sched_barrier(0);")
-        A("    {")
-        body("a", "zz", "      ")
-        A("    }")
-        A("    a_grow = b_grow; a_srow = b_srow;")
-        A("    " + " ".join([f"a_xv{i} = b_xv{i};" for i in i_used] + [f"a_wv{blk.b} = b_wv{blk.b};" for blk in st.blocks]
-                             + [f"a_yv{j} = b_yv{j};" for j in j_used]))
-        A("  }")
-    else:
-        A("  for (int64_t zz = z0; zz < z1; ++zz) {")
-        load("a", "zz", "    ")
-        A("    {")
-        body("a", "zz", "      ")
-        A("    }")
-        A("  }")
+    A("  switch (q) {")
+    for q in range(nsplit):
+        A(f"    case {q}: bwd_group{q}<X1_IDX, G_IDX, ATOMIC_DX1>(BWD_ARGS, z0, z1, lane, uu, active, ch); break;")
+    A("  }")
     A("}")
     A(f"constexpr int kBwdMinRange = {chunk};   // fewest batch rows worth a wavefront of their own")
     A(f"constexpr int kBwdWaves = {waves_per_eu};")
+    A(f"constexpr int kBwdSplit = {nsplit};")
+    A(f"constexpr int kBwdParts = {nparts};     // partial rows of the x2 gradient per batch row")
     return "\n".join(L)
 
 
@@ -449,6 +506,7 @@ FWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}*
               "const void* __restrict__ x1_index, int x1_idx64, const int64_t* __restrict__ csr_offsets, "
               "const int64_t* __restrict__ csr_perm")
 FWD_ARGS = "w, x1, x2, out, x1_index, x1_idx64, csr_offsets, csr_perm"
+BWD_ARGS = "w, x1, x2, g, dw, dx1, dx1_partial, dx2, dx2_partial, x1_index, x1_idx64, g_index, g_idx64, batch"
 BWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}* __restrict__ x2, const {T}* __restrict__ g, "
               "{T}* __restrict__ dw, {T}* dx1, {T}* __restrict__ dx1_partial, {T}* __restrict__ dx2, "
               "{T}* __restrict__ dx2_partial, const void* __restrict__ x1_index, int x1_idx64, "
@@ -457,7 +515,7 @@ BWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}*
 
 def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_hash: int, *, fwd_split: int = 1,
               fwd_waves: int = 2, fwd_prefetch: bool = True, bwd_waves: int = 2, bwd_chunk: int = 16,
-              bwd_prefetch: bool = False) -> str:
+              bwd_prefetch: bool = False, bwd_split: int = 1) -> str:
     """Complete .hip translation unit: kernels, host launchers, registration under both table hashes."""
     ns = f"cw_{name}"
     nch = (st.extent + 63) // 64
@@ -483,10 +541,11 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     A(f"#define FWD_PARAMS {FWD_PARAMS.format(T=T)}")
     A(f"#define FWD_ARGS {FWD_ARGS}")
     A(f"#define BWD_PARAMS {BWD_PARAMS.format(T=T)}")
+    A(f"#define BWD_ARGS {BWD_ARGS}")
     A("")
     A(emit_forward(st, T, fwd_split, fwd_waves, ns, fwd_prefetch))
     A("")
-    A(emit_backward(st, T, bwd_waves, bwd_chunk, bwd_prefetch))
+    A(emit_backward(st, T, bwd_waves, bwd_chunk, bwd_prefetch, bwd_split))
     A("")
     code = f"dtype_code<{T}>::value"
     A(f"""
@@ -530,7 +589,7 @@ static int run_fwd(const SpecCall& c) {{
 // buffers: w, x1, x2, g | dw, dx1, dx2
 static int64_t bwd_workspace(const cueq_u1d_buffer* b, int64_t batch) {{
   int64_t need = 0;
-  if ({nch} > 1) need += batch * {nch} * {W2}ll * sizeof({T});
+  if (kBwdParts > 1) need += batch * kBwdParts * {W2}ll * sizeof({T});
   need = (need + 255) & ~int64_t(255);
   if (b[1].batch_dim == CUEQ_BATCH_INDEXED && deterministic_scatter()) need += batch * {W1}ll * sizeof({T});
   return need;
@@ -560,7 +619,7 @@ static int run_bwd(const SpecCall& c) {{
   char* ws = static_cast<char*>(c.workspace);
   {T}* dx2_partial = nullptr;
   int64_t off = 0;
-  if ({nch} > 1) {{ dx2_partial = reinterpret_cast<{T}*>(ws); off = (batch * {nch} * {W2}ll * sizeof({T}) + 255) & ~int64_t(255); }}
+  if (kBwdParts > 1) {{ dx2_partial = reinterpret_cast<{T}*>(ws); off = (batch * kBwdParts * {W2}ll * sizeof({T}) + 255) & ~int64_t(255); }}
   {T}* dx1_partial = nullptr;
   bool atomic = false;
   if (!x1_idx) dx1_partial = dx1;  // one row per batch element: plain stores
@@ -573,11 +632,11 @@ static int run_bwd(const SpecCall& c) {{
   }}
   if (batch > 0) {{
     // one launch round of resident wavefronts; short batches get fewer, not shorter than kBwdMinRange rows
-    int64_t nranges = wave_slots(kBwdWaves) / {nch};
+    int64_t nranges = wave_slots(kBwdWaves) / kBwdParts;
     const int64_t most = (batch + kBwdMinRange - 1) / kBwdMinRange;
     if (nranges > most) nranges = most;
     if (nranges < 1) nranges = 1;
-    const int64_t grid = nranges * {nch};
+    const int64_t grid = nranges * kBwdParts;
     const dim3 gd(static_cast<unsigned>(grid)), t(64);
     {{
     KernelTimer timer("{name}_bwd_{T}", c.stream);
@@ -591,8 +650,8 @@ static int run_bwd(const SpecCall& c) {{
 #undef LAUNCH_BWD
     }}
     CUEQ_CHECK_HIP(hipGetLastError());
-    if ({nch} > 1) {{
-      hipLaunchKernelGGL(fold_parts<{T}>, dim3(blocks_for(batch * {W2}ll)), dim3(256), 0, c.stream, dx2_partial, batch, {nch}, {W2}, dx2);
+    if (kBwdParts > 1) {{
+      hipLaunchKernelGGL(fold_parts<{T}>, dim3(blocks_for(batch * {W2}ll)), dim3(256), 0, c.stream, dx2_partial, batch, kBwdParts, {W2}, dx2);
       CUEQ_CHECK_HIP(hipGetLastError());
     }}
   }}

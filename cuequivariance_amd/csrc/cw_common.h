@@ -101,10 +101,8 @@ inline unsigned blocks_for(int64_t n, int per_block = 256) { return static_cast<
 // Scatter policy of the fused backward for the gradient of a gathered operand:
 // hardware floating-point atomics (fast, summation order varies) or per-row partials
 // followed by a gather-sum in index order (bit-reproducible, one extra pass over batch x row).
-inline bool deterministic_scatter() {
-  const char* e = getenv("CUEQ_DETERMINISTIC");
-  return e && e[0] == '1';
-}
+// A process-wide option (cueq_set_option("deterministic", ...); initial value from CUEQ_DETERMINISTIC, read once).
+bool deterministic_scatter();
 
 template <typename T> struct dtype_code;
 template <> struct dtype_code<float> { static constexpr int value = CUEQ_F32; };

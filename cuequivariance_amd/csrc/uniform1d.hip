@@ -1,10 +1,12 @@
 // uniform-1d executor: plan creation and the table-driven kernels.
 //
 // A plan regroups the descriptor's paths by (output buffer, output segment) and uploads
-// them once.  Every output element is owned by one thread (or one wavefront when a
-// scalar output contracts the channel mode), which walks the batch rows that
-// contribute to it and the paths of its segment in a fixed order: no atomics, results
-// are bit-reproducible from run to run.
+// them once.  In the table-driven kernels of this file every output element is owned by one
+// thread (or one wavefront when a scalar output contracts the channel mode), which walks the
+// batch rows that contribute to it and the paths of its segment in a fixed order: no atomics,
+// results are bit-reproducible from run to run.  (The generated channel-wise backward scatters
+// the gradient of a gathered operand with floating-point atomics unless the "deterministic"
+// option is set; everything else there is bit-reproducible too.)
 //
 // Semantics follow the reference's PyTorch executor,
 // cuequivariance_torch/cuequivariance_torch/primitives/segmented_polynomial_naive.py:61-160
@@ -13,6 +15,7 @@
 // for a one-row output).
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -47,6 +50,21 @@ const U1dSpec* find_u1d_spec(uint64_t hash) {
     if (s->hash == hash) return s;
   return nullptr;
 }
+
+// ---- process-wide options: the environment is read once, cueq_set_option changes them afterwards ----
+static int env_flag(const char* name) {
+  const char* e = getenv(name);
+  return (e && e[0] == '1') ? 1 : 0;
+}
+static std::atomic<int>& opt_deterministic() {
+  static std::atomic<int> v{env_flag("CUEQ_DETERMINISTIC")};
+  return v;
+}
+static std::atomic<int>& opt_force_generic() {
+  static std::atomic<int> v{env_flag("CUEQ_FORCE_GENERIC")};
+  return v;
+}
+bool deterministic_scatter() { return opt_deterministic().load(std::memory_order_relaxed) != 0; }
 
 uint64_t hash_u1d_desc(const cueq_u1d_desc* d) {
   Fnv64 f;
@@ -208,8 +226,16 @@ __global__ void __launch_bounds__(256) u1d_generic_wave(KernelArgs a) {
   M acc = 0;
   for (int64_t zz = z0; zz < z1; ++zz) {
     const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
-    for (int p = p0; p < p1; ++p)
-      for (int u = lane; u < a.extent; u += 64) acc += path_product<M>(a, p, z, u);
+    for (int p = p0; p < p1; ++p) {
+      // a path sums over the channel mode only when one of its inputs carries it; a path of scalars contributes once
+      bool has_channel = false;
+      for (int k = 0; k < a.nin[p]; ++k) has_channel |= a.buf[a.in[p * kMaxInOperands + k] >> 24].dim != 0;
+      if (has_channel) {
+        for (int u = lane; u < a.extent; u += 64) acc += path_product<M>(a, p, z, u);
+      } else if (lane == 0) {
+        acc += path_product<M>(a, p, z, 0);
+      }
+    }
   }
   for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 64);
   if (lane == 0) store_as<M>(a.out, a.out_dtype, wid, acc);
@@ -283,6 +309,19 @@ extern "C" int cueq_timing_end(cueq_timing_entry* out, int max_entries) {
   return n;
 }
 extern "C" const char* cueq_version(void) { return "cueq_amd 0.1 (gfx950)"; }
+
+extern "C" int cueq_set_option(const char* name, int32_t value) {
+  CUEQ_REQUIRE(name, CUEQ_ERR_INVALID, "null option name");
+  if (std::strcmp(name, "deterministic") == 0) opt_deterministic().store(value ? 1 : 0);
+  else if (std::strcmp(name, "force_generic") == 0) opt_force_generic().store(value ? 1 : 0);
+  else CUEQ_REQUIRE(false, CUEQ_ERR_INVALID, "unknown option '%s' (deterministic, force_generic)", name);
+  return CUEQ_OK;
+}
+extern "C" int cueq_get_option(const char* name) {
+  if (name && std::strcmp(name, "deterministic") == 0) return opt_deterministic().load();
+  if (name && std::strcmp(name, "force_generic") == 0) return opt_force_generic().load();
+  return -1;
+}
 
 extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_plan) {
   CUEQ_REQUIRE(d && out_plan, CUEQ_ERR_INVALID, "null argument");
@@ -537,7 +576,7 @@ extern "C" int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* bu
   CUEQ_REQUIRE(plan && buffers, CUEQ_ERR_INVALID, "null argument");
   CUEQ_REQUIRE(batch >= 0, CUEQ_ERR_INVALID, "negative batch size");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (plan->spec && !getenv("CUEQ_FORCE_GENERIC")) {
+  if (plan->spec && !opt_force_generic().load(std::memory_order_relaxed)) {
     SpecCall call{buffers, batch, workspace, workspace_bytes, s};
     const int rc = plan->spec->run(call);
     if (rc != CUEQ_ERR_UNSUPPORTED) return rc;

@@ -96,7 +96,11 @@ class ChannelWiseTensorProduct(torch.nn.Module):
 
     ``forward(x1, x2, weight=None, indices_1=None, indices_2=None, indices_out=None, size_out=None)``:
     ``indices_1`` / ``indices_2`` gather rows of ``x1`` / ``x2`` per batch element, ``indices_out`` scatter-adds
-    the batch elements into ``size_out`` output rows (deterministically).
+    the batch elements into ``size_out`` output rows.  The forward sums each output row's batch elements in batch
+    order (bit-reproducible).  In the backward, the gradient of a gathered operand (``x1`` with ``indices_1``) is
+    scattered with floating-point atomics by default - summation order, hence the last bits, vary from run to run; set
+    ``CUEQ_DETERMINISTIC=1`` (or ``cueq_set_option("deterministic", 1)``) for an ordered, bit-reproducible sum at the
+    price of one more pass.  The other gradients are bit-reproducible in both modes.
     """
 
     def __init__(

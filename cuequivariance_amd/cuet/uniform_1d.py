@@ -272,6 +272,7 @@ def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor
     if device.type != "cuda":
         raise RuntimeError("uniform_1d runs on the GPU only; got tensors on " + str(device))
     lib = _lib.load()
+    _lib.sync_options_from_env()
     with _on_device(device):
         handle = plan.handle(device)
         bufs = (_lib.U1dBuffer * (nin + nout))()

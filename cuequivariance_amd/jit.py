@@ -72,19 +72,43 @@ def is_channelwise(t: U1dTables) -> bool:
 
 
 def _tuning(st, T: str) -> dict:
-    """Wavefronts per SIMD and prefetching from a register estimate (accumulators + operand sets; doubles take two)."""
+    """Wavefronts per SIMD, prefetching and the number of wavefronts the blocks are dealt out to, from a register
+    estimate (accumulators + operand sets; doubles take two registers).  A descriptor whose kernels would be left with
+    one wavefront per SIMD is split over two or four wavefronts with disjoint x1 segments when it has that many."""
+    from .codegen import channelwise as cw
+
     per = 2 if T == "double" else 1
-    operands = st.nseg_x1 + st.nseg_w + 4
-    fwd_two_sets = (st.nseg_out + 2 * operands + 30) * per
-    fwd_one_set = (st.nseg_out + operands + 30) * per
-    if fwd_two_sets <= 250:
-        fwd = dict(fwd_waves=2, fwd_prefetch=True)
-    elif fwd_one_set <= 250:
-        fwd = dict(fwd_waves=2, fwd_prefetch=False)
-    else:
-        fwd = dict(fwd_waves=1, fwd_prefetch=fwd_two_sets <= 500)
-    bwd_regs = (st.nseg_out + 2 * st.nseg_x1 + st.nseg_w + st.nseg_x2 + 30) * per
-    return dict(fwd, bwd_waves=2 if bwd_regs <= 250 else 1)
+    most = len(cw._split_blocks(st, 4))
+
+    def part(n, ns):
+        return -(-n // ns)
+
+    def fwd_regs(ns, sets):
+        return (part(st.nseg_out, ns) + sets * (part(st.nseg_x1 + st.nseg_w, ns) + 4) + 30) * per
+
+    def bwd_regs(ns):
+        return (part(st.nseg_out, ns) + part(2 * st.nseg_x1 + st.nseg_w, ns) + st.nseg_x2 + 30) * per
+
+    fwd = None
+    for ns in (1, 2, 4):
+        if ns > most:
+            break
+        if fwd_regs(ns, 2) <= 250:
+            fwd = dict(fwd_split=ns, fwd_waves=2, fwd_prefetch=True)
+        elif fwd_regs(ns, 1) <= 250:
+            fwd = dict(fwd_split=ns, fwd_waves=2, fwd_prefetch=False)
+        if fwd:
+            break
+    if fwd is None:
+        fwd = dict(fwd_split=1, fwd_waves=1, fwd_prefetch=fwd_regs(1, 2) <= 500)
+    bwd = dict(bwd_split=1, bwd_waves=1)
+    for ns in (1, 2, 4):
+        if ns > most:
+            break
+        if bwd_regs(ns) <= 250:
+            bwd = dict(bwd_split=ns, bwd_waves=2)
+            break
+    return dict(fwd, **bwd)
 
 
 def _has_spec(t: U1dTables, code: int) -> bool:
@@ -155,24 +179,25 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None):
 
     T = "float" if code == _lib.F32 else "double"
     name = f"jit_{key:016x}"
-    so = cache_dir() / f"u1d_{name}_{T}.so"
-    if not so.exists():
-        if not (is_channelwise(t) or is_symmetric_contraction(polynomial)):
-            from .codegen import general as gen
+    # the object's name carries a hash of the emitted source, so a changed generator (or tuning) never meets a stale object
+    if not (is_channelwise(t) or is_symmetric_contraction(polynomial)):
+        from .codegen import general as gen
 
-            src = gen.emit_unit(t, T, name, key)
-            what = f"general plan, {sum(t.num_paths)} paths, extent {t.operand_extent}"
-        elif is_channelwise(t):
-            _, paths = t.operation(0)
-            st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
-            tb = t.backward((True, True, True))
-            src = cw.emit_unit(st, T, name, key, tb.content_hash(code), **_tuning(st, T))
-            what = f"{st.num_paths} paths, extent {st.extent}"
-        else:
-            st = sc.analyze(polynomial)
-            bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
-            src = sc.emit_unit(st, T, name, key, bwd)
-            what = f"symmetric contraction, {len(st.terms)} folded terms, extent {st.extent}"
+        src = gen.emit_unit(t, T, name, key)
+        what = f"general plan, {sum(t.num_paths)} paths, extent {t.operand_extent}"
+    elif is_channelwise(t):
+        _, paths = t.operation(0)
+        st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
+        tb = t.backward((True, True, True))
+        src = cw.emit_unit(st, T, name, key, tb.content_hash(code), **_tuning(st, T))
+        what = f"{st.num_paths} paths, extent {st.extent}"
+    else:
+        st = sc.analyze(polynomial)
+        bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
+        src = sc.emit_unit(st, T, name, key, bwd)
+        what = f"symmetric contraction, {len(st.terms)} folded terms, extent {st.extent}"
+    so = cache_dir() / f"u1d_{name}_{T}_{hashlib.sha1(src.encode()).hexdigest()[:10]}.so"
+    if not so.exists():
         _compile(src, so, f"descriptor {key:016x} ({T}, {what})")
     _lib.load()  # the library the object links against is already in the process
     return C.CDLL(str(so))

@@ -39,6 +39,14 @@ enum cueq_status {
 const char* cueq_last_error(void);
 const char* cueq_version(void);
 
+/* Process-wide options (no counterpart in the reference).  "deterministic": 1 makes the fused channel-wise backward
+ * sum the gradient of a gathered operand in index order (bit-reproducible, one more pass) instead of scattering it
+ * with floating-point atomics; "force_generic": 1 runs the table-driven kernels even where generated ones exist.
+ * Initial values come from the environment variables CUEQ_DETERMINISTIC / CUEQ_FORCE_GENERIC ("1"), read once when
+ * first needed.  cueq_get_option returns the value, or -1 for an unknown name. */
+int cueq_set_option(const char* name, int32_t value);
+int cueq_get_option(const char* name);
+
 /* Per-kernel timing with HIP events recorded on the stream each kernel is launched on.
  * Between cueq_timing_begin() and cueq_timing_end() the main kernel of every call is bracketed by a
  * pair of events; cueq_timing_end waits for them and returns, per kernel name, the number of launches

@@ -21,8 +21,8 @@ not depend on the descriptor classes of the package under test.
 
 Pinned by ``tests/test_oracle.py``: brute-force loops on tiny descriptors, matmul identities
 (the reference's ``evaluate_test.py:20-104``), gather/scatter identity
-(``cuequivariance_torch/tests/operations/channel_wise_test.py:231-305``), and the closed-form
-channel-wise product of :mod:`oracle.closed_forms`.
+(``cuequivariance_torch/tests/operations/channel_wise_test.py:231-305``), and a closed-form
+channel-wise product written out in that test file.
 """
 
 from __future__ import annotations

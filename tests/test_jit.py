@@ -34,12 +34,42 @@ def test_compile_load_and_register(jit_on):
     assert not jit.ensure_specialised(U1dTables.from_polynomial(lin), 0)
 
 
+def test_tuning_splits_descriptors_that_would_run_one_wavefront_per_simd():
+    """Register estimate: the 40-channel l <= 2 product fits as it is; the l <= 3 product in float64 would be left with
+    one wavefront per SIMD and is dealt out to two wavefronts with disjoint x1 segments (forward and backward)."""
+    from cuequivariance_amd import jit
+    from cuequivariance_amd.codegen import channelwise as cw
+    from cuequivariance_amd.codegen.registry import channelwise_tables
+
+    def structure(i1, i2, filt):
+        t = channelwise_tables(i1, i2, filt)
+        _, paths = t.operation(0)
+        return cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
+
+    small = structure("40x0e+40x1o+40x2e", "0e+1o+2e", "0e+1o+2e")
+    assert jit._tuning(small, "double")["fwd_split"] == 1 and jit._tuning(small, "double")["bwd_split"] == 1
+    big = structure("24x0e+24x1o+24x2e+24x3o", "0e+1o+2e+3o", "0e+1o+2e+3o")
+    assert jit._tuning(big, "float")["fwd_split"] == 1
+    tune = jit._tuning(big, "double")
+    assert tune["fwd_split"] == 2 and tune["bwd_split"] == 2 and tune["fwd_waves"] == 2 and tune["bwd_waves"] == 2
+    groups = cw._split_blocks(big, 2)
+    seg = [{i for blk in g for i in blk.i_list} for g in groups]
+    assert len(groups) == 2 and not (seg[0] & seg[1]) and seg[0] | seg[1] == set(range(16))
+    assert sorted(blk.b for g in groups for blk in g) == list(range(23))
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-def test_jit_kernels_match_oracle_and_generic(device, dtype, jit_on):
+@pytest.mark.parametrize("dtype,irreps", [(torch.float32, "40x0e+40x1o+40x2e"), (torch.float64, "40x0e+40x1o+40x2e"),
+                                          (torch.float64, "24x0e+24x1o+24x2e+24x3o")])
+def test_jit_kernels_match_oracle_and_generic(device, dtype, irreps, jit_on):
+    """Kernels compiled at first use against the oracle; the last case is dealt out to two wavefronts per batch row
+    (see the tuning test above), the others run one."""
     from cuequivariance_amd import cuet
 
-    i1, i2, filt = cue.Irreps("O3", "40x0e+40x1o+40x2e"), cue.Irreps("O3", "0e+1o+2e"), ["0e", "1o", "2e"]
+    i1 = cue.Irreps("O3", irreps)
+    lmax = 3 if "3o" in irreps else 2
+    i2 = cue.Irreps("O3", "0e+1o+2e+3o" if lmax == 3 else "0e+1o+2e")
+    filt = ["0e", "1o", "2e", "3o"][: lmax + 1]
     g = torch.Generator().manual_seed(41)
     N, Z = 31, 500
 
@@ -314,3 +344,46 @@ def test_fused_fully_connected_second_derivatives(device, jit_on):
     err, m = fc_second_derivatives(device, torch.float32, "32x0e+32x1o")
     assert _dense_of(m)._fused.get((torch.float32, True)) is not None
     assert err <= 2e-5, err
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("on", [False, True])
+def test_scalar_output_mixing_contracting_and_scalar_paths(device, jit_on, on):
+    """One scalar output fed by a path that contracts the channel mode (x[u] gy[u] -> dw[]) and by a path of scalars only
+    (s[] gt[] -> dw[]) - what the weight gradient of ``w[] x[u] -> y[u]`` plus ``w[] s[] -> t[]`` looks like.  The scalar
+    path must be counted once, not once per channel.  Table-driven kernels (``on`` False) and the general generator
+    (True) against the oracle and against the closed form."""
+    import numpy as np
+
+    from cuequivariance_amd.cuet.uniform_1d import Uniform1dPlan, run_plan
+    from cuequivariance_amd import _lib
+
+    jit.enable(on)
+    E, Z = 48, 37
+    # buffers: 0 x[u] (2 segments), 1 gy[u] (2), 2 s[] (2), 3 gt[] (2) | 4 dw[] (2 scalar segments)
+    tables = U1dTables.make(
+        E, 4, 1, [1, 1, 0, 0, 0], [2, 2, 2, 2, 2], [0, 1, 2, 3, -1], [3, 3], [0, 1, 4, 2, 3, 4], [3, 2], [0, 9], [0, 3],
+        [0, 0, 0, 1, 1, 1, 0, 1, 1,  0, 0, 0, 1, 0, 1], [2.0, -1.5, 0.5, 3.0, 0.25])
+    spec = dict(
+        num_inputs=4, num_outputs=1, sizes=[2 * E, 2 * E, 2, 2, 2],
+        operations=[
+            dict(buffers=[0, 1, 4], operand_subscripts=["u", "u", ""], coefficient_subscripts="",
+                 segments=[[(E,), (E,)], [(E,), (E,)], [(), ()]], path_indices=[(0, 0, 0), (1, 1, 1), (0, 1, 1)],
+                 path_coefficients=[np.array(2.0), np.array(-1.5), np.array(0.5)]),
+            dict(buffers=[2, 3, 4], operand_subscripts=["", "", ""], coefficient_subscripts="",
+                 segments=[[(), ()], [(), ()], [(), ()]], path_indices=[(0, 0, 0), (1, 0, 1)],
+                 path_coefficients=[np.array(3.0), np.array(0.25)]),
+        ])
+    g = torch.Generator().manual_seed(3)
+    x, gy = (torch.randn(Z, 2 * E, generator=g, dtype=torch.float64) for _ in range(2))
+    sc, gt = (torch.randn(Z, 2, generator=g, dtype=torch.float64) for _ in range(2))
+    want = naive_segmented_polynomial(spec, [x, gy, sc, gt])[0]
+    closed = torch.stack([
+        2.0 * (x[:, :E] * gy[:, :E]).sum(1) + 3.0 * sc[:, 0] * gt[:, 0],
+        -1.5 * (x[:, E:] * gy[:, E:]).sum(1) + 0.5 * (x[:, :E] * gy[:, E:]).sum(1) + 0.25 * sc[:, 1] * gt[:, 0]], 1)
+    assert (want - closed).abs().max().item() <= 1e-12 * closed.abs().max().item()
+    plan = Uniform1dPlan(tables, torch.float64, name="mixed_scalar_output")
+    B = _lib.BATCH_DIM_BATCHED
+    got = run_plan(plan, [B] * 5, [-1] * 5, Z, 0, [v.to(device) for v in (x, gy, sc, gt)])[0]
+    assert plan.specialised(device) == on
+    assert (got.cpu() - want).abs().max().item() <= 1e-12 * want.abs().max().item()
