@@ -9,7 +9,13 @@ forward pass plus the backward pass for the gradients of node features, edge att
 
 Prints ONE JSON line: whole-job edges/s with inputs resident in HBM, the roofline position of the
 dominant kernel (fused backward) from HIP-event timings taken inside the timed region, and the CPU
-oracle timed on a bounded sample of the same workload on this box's host cores.
+oracle timed on a bounded sample of the same workload on this box's host cores.  Run without
+``--workload`` the line also carries a ``secondary`` object: the same workload in float64 and with the
+ordered (bit-reproducible) node-gradient sum, and every other BASELINE.json configuration (channel-wise
+batch 4096, symmetric contraction, Linear and fully connected product in fp32 / bf16, triangle update in
+bf16 / fp32), each with its step time, throughput, both roofline fractions (algorithmic bytes against
+8 TB/s; flops against the matrix-core or vector peak) and the binding roof, plus CPU baselines of the
+dense workloads and the one-thread figure of the headline workload.
 """
 
 from __future__ import annotations
@@ -40,13 +46,13 @@ MEASURED_TRAFFIC_BYTES = {
     ("c128_l3_fwd_float", 5000, 100_000): 2.135e9,
 }
 
-# Vector instructions executed per batch element (edge, node) by the generated kernels, forward + backward, counted by
-# rocprofv3 --pmc SQ_INSTS_VALU over one launch each (profiles/*_valu_counters.txt).  One wave64 instruction is at
-# most 64 fused multiply-adds = 128 flops; the published fp32 vector peak counts 256 flops per compute unit and clock.
-VALU_INSTS_PER_ELEMENT = {
-    # workload: (wave64 instructions per batch element: forward, backward; source)
-    "cfg2": (2 * 510, 2 * 1255, "profiles/channelwise_c128_l3_fp32_cfg2_valu_counters.txt"),
-}
+# Vector (wave64) instructions the generated kernels execute per batch element (sample, edge, node), forward and backward,
+# counted with rocprofv3 --pmc SQ_INSTS_VALU over one launch each and divided by the batch size (summary and command:
+# profiles/uniform1d_fp32_valu_instruction_counts.txt).  A wave64 instruction is at most 64 fused multiply-adds =
+# 128 flops, and the published fp32 vector peak (157.3 TFLOP/s) is one such instruction per SIMD every two clocks, so
+# instructions x 128 / time against that peak is the issue utilisation of the vector units.
+VALU_INSTS_PER_ELEMENT = {"cfg1": (242, 376), "cfg2": (1020, 2510), "cfg3": (1734, 4180)}
+VALU_SOURCE = "profiles/uniform1d_fp32_valu_instruction_counts.txt (rocprofv3 --pmc SQ_INSTS_VALU of an earlier run of these kernels)"
 
 
 def algorithmic_bytes(E: int, N: int, W: int, D1: int, D2: int, D3: int, s: int) -> dict:
@@ -136,9 +142,7 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         unit, units, dt = "samples/s", Z, "f32"
         d1, d2, dw, do = i1.dim, i2.dim, m.weight_numel, m.irreps_out.dim
         alg = {"fwd": Z * (d1 + d2 + dw + do) * 4, "bwd": Z * (2 * (d1 + d2 + dw) + do) * 4}
-        # 83 flattened paths x 32 channels; per path and operation: 2 multiplies between the 3 inputs, 1 by the coefficient,
-        # 1 accumulate; forward = 1 operation, backward = 3
-        flops = {"fwd": Z * 83 * 32 * 4, "bwd": 3 * Z * 83 * 32 * 4}
+        flops = {k: Z * n * 128 for k, n in zip(("fwd", "bwd"), VALU_INSTS_PER_ELEMENT["cfg1"])}  # executed vector instructions x 128
         flop_roof, flop_peak = "valu", VALU_PEAK_F32
         desc = ("configs[0]: channel-wise TP 32x0e+32x1o+32x2e (x) 0e+1o+2e, outputs up to l = 2, batch 4096, per-sample weights, "
                 "fwd + bwd (dx1, dx2, dw); 69 MB of traffic: launch-latency regime")
@@ -159,18 +163,10 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         unit, units, dt = "nodes/s", Z, "f32"
         # every distinct element once: fwd reads x and writes out; bwd reads x, g and writes dx (weights 10 x 3712 negligible)
         alg = {"fwd": Z * (2048 + 512) * 4, "bwd": Z * (2048 + 512 + 2048) * 4}
-        # flops of the folded path table the kernels evaluate (4 + 51 + 425 terms of degree 1, 2, 3 after folding the
-        # 4 + 86 + 1949 paths onto sorted index tuples): a term of degree d costs d + 2 flops per channel and operation
-        # (d multiplies between its d + 1 inputs, one by the coefficient, one accumulate); the forward is one
-        # operation, the backward d + 1 (one per differentiated input)
-        terms = {1: 4, 2: 51, 3: 425}
-        fwd_f = sum(n * (d + 2) for d, n in terms.items())
-        bwd_f = sum(n * (d + 2) * (d + 1) for d, n in terms.items())
-        flops = {"fwd": Z * 128 * fwd_f, "bwd": Z * 128 * bwd_f}
+        flops = {k: Z * n * 128 for k, n in zip(("fwd", "bwd"), VALU_INSTS_PER_ELEMENT["cfg3"])}  # executed vector instructions x 128
         flop_roof, flop_peak = "valu", VALU_PEAK_F32
         desc = ("configs[2]: symmetric contraction 128x(0e+1o+2e+3o) -> 128x(0e+1o), degree 3, 10 element types, "
-                "50000 nodes, int32 element index, fwd + bwd (dw, dx); flops are those of the folded path table "
-                "(the kernels share pair products between terms and execute fewer)")
+                "50000 nodes, int32 element index, fwd + bwd (dw, dx)")
     elif wl == "cfg4":
         Z = 200_000
         dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
@@ -285,7 +281,8 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
                      "hbm_frac": roofs["hbm_frac"], f"{flop_roof}_frac": roofs[f"{flop_roof}_frac"],
                      "algorithmic_bytes": roofs["algorithmic_bytes"], "flops": roofs["flops"],
                      "scope": "whole step: algorithmic bytes and flops of forward + backward over the step time, against 8 TB/s and the "
-                              f"{flop_roof} peak ({flop_peak} TFLOP/s); bound = the roof with the longer minimum time"},
+                              f"{flop_roof} peak ({flop_peak} TFLOP/s); bound = the roof with the longer minimum time"
+                              + ("; flops = executed vector instructions x 128, " + VALU_SOURCE if flop_roof == "valu" else "")},
         "kernels": kernels,
     }
 
@@ -349,8 +346,7 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
             "algorithmic_bytes_per_launch": dominant[1]["algorithmic_bytes"],
         }
     total_alg = alg["fwd"] + alg["bwd"]
-    # 353 flattened paths x 128 channels, 4 flops per path and operation (SURVEY formula), forward 1 operation, backward 3
-    nominal_flops = 4 * E * 353 * 128 * 4
+    valu_flops = E * sum(VALU_INSTS_PER_ELEMENT["cfg2"]) * 128  # executed vector instructions x 128 flops
     line = {
         "metric": "edges/sec, indexed channelwise TP fwd+bwd (128ch, lmax=3); % HBM roofline",
         "value": value,
@@ -373,7 +369,8 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
         },
         "roofline": roofline,
         "step_roofline_frac": (total_alg / (elapsed / steps)) / 1e9 / HBM_PEAK_GBS,
-        "step_valu_frac": nominal_flops / (elapsed / steps) / 1e12 / (VALU_PEAK_F32 if dtype == torch.float32 else 78.6),
+        "step_valu_frac": valu_flops / (elapsed / steps) / 1e12 / (VALU_PEAK_F32 if dtype == torch.float32 else 78.6),
+        "valu_source": VALU_SOURCE,
         "kernels": per_kernel,
     }
     return line, m, host
@@ -389,7 +386,7 @@ def cpu_baseline_dense(torch, cue, wl: str, threads: int) -> dict:
     if wl == "cfg5":
         from oracle.triangle import triangle_multiplicative_update as oracle_trimul
 
-        n, D = 192, 128
+        n, D = 384, 128
 
         def r(*shape, scale=1.0):
             return torch.randn(*shape, generator=g) * scale
@@ -411,7 +408,7 @@ def cpu_baseline_dense(torch, cue, wl: str, threads: int) -> dict:
     else:  # cfg4 Linear: three 128 x 128 blocks per irrep component on ir_mul slices = the oracle's per-path einsum
         from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
 
-        Z = 20_000
+        Z = 200_000
         irreps = cue.Irreps("O3", "128x0e+128x1o+128x2e")
         e = cue.descriptors.linear(irreps, irreps)
         spec = spec_from_polynomial(e.polynomial)
@@ -426,7 +423,7 @@ def cpu_baseline_dense(torch, cue, wl: str, threads: int) -> dict:
             return time.perf_counter() - t0
 
         units, unit = Z, "rows/s"
-        sample = f"{Z} of the 200000 rows, float32"
+        sample = f"all {Z} rows, float32"
     once()
     t = st.median([once() for _ in range(3)])
     return {"value": units / t, "unit": unit, "cores": cores, "kind": "port",
