@@ -77,6 +77,10 @@ def build_library(force: bool = False, jobs: int | None = None, verbose: bool = 
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    # fused kernels of the registered fully connected products: separate small objects next to the library
+    from cuequivariance_amd import jit as _jit
+
+    _jit.prebuild_fully_connected(force)
     return LIB
 
 

@@ -28,6 +28,12 @@ SYMMETRIC = [
     ("s32_l2", "32x0e+32x1o+32x2e", "32x0e+32x1o", 3),
 ]
 
+# Fully connected products (shared weights) whose fused kernels are compiled when the library is built, into
+# cuequivariance_amd/prebuilt/: (irreps_in1, irreps_in2, irreps_out), float and bfloat16.  Others are compiled at first use.
+FULLY_CONNECTED = [
+    ("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o"),
+]
+
 MATH = (("float", 0), ("double", 1))
 
 

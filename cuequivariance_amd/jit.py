@@ -220,6 +220,35 @@ def _compile(src: str, so: Path, what: str, link_library: bool = True) -> None:
         os.replace(out, so)  # atomic: another process may be compiling the same descriptor
 
 
+PREBUILT = Path(__file__).resolve().parent / "prebuilt"
+
+
+def prebuild_fully_connected(force: bool = False) -> list:
+    """Compile the fused kernels of the fully connected products listed in ``codegen/registry.py`` into
+    ``cuequivariance_amd/prebuilt/`` (called when the library is built; the objects are named by the hash of their
+    source, so a changed generator never meets a stale object).  Returns the objects."""
+    from . import cue, cuet
+    from .codegen import fullyconnected as fc
+    from .codegen import registry
+
+    PREBUILT.mkdir(exist_ok=True)
+    wanted = []
+    for i1, i2, i3 in registry.FULLY_CONNECTED:
+        m = cuet.FullyConnectedTensorProduct(cue.Irreps("O3", i1), cue.Irreps("O3", i2), cue.Irreps("O3", i3), layout=cue.ir_mul,
+                                             internal_weights=False)
+        dense = next(x for x in m.modules() if type(x).__name__ == "SegmentedPolynomialDense")
+        for T in ("float", "uint16_t"):
+            src = fc.emit_unit(dense.paths, dense.input_sizes[2], dense.input_sizes[1], dense.out_size, T)
+            so = PREBUILT / f"fc_{hashlib.sha1(src.encode()).hexdigest()[:16]}_{T}.so"
+            if force or not so.exists():
+                _compile(src, so, f"the fully connected product {i1} (x) {i2} -> {i3} ({T})", link_library=False)
+            wanted.append(so)
+    for old in PREBUILT.glob("fc_*.so"):
+        if old not in wanted:
+            old.unlink()
+    return wanted
+
+
 def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str):
     """The fused kernels of ``codegen/fullyconnected.py`` for one fully connected product and element type (``float`` or
     ``uint16_t`` for bfloat16), compiled at first use and loaded: a ``ctypes`` handle with ``fcj_fwd``, ``fcj_dx1``,
@@ -237,7 +266,9 @@ def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str):
         if key in _failed:
             return None
         try:
-            so = cache_dir() / f"{key}_{T}.so"
+            so = PREBUILT / f"{key}_{T}.so"  # compiled with the library for the registered products
+            if not so.exists():
+                so = cache_dir() / f"{key}_{T}.so"
             if not so.exists():
                 _compile(src, so, f"a fully connected product ({T}, {len(paths)} paths, {width_in} x {n2} -> {width_out})", link_library=False)
             h = C.CDLL(str(so))
