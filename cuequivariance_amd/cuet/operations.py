@@ -247,11 +247,10 @@ class FullyConnectedTensorProduct(torch.nn.Module):
         )
         self.method = _method_from_fallback(method, use_fallback, "fused_tp")
         self.f_per_sample = _FlattenedUniform(e.polynomial, math_dtype)  # weights of shape (batch, weight_numel)
-        try:
-            self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
-        except NotImplementedError:
-            # the dense executor takes a second operand of multiplicity one; others run on the uniform-1d kernels of the
-            # flattened descriptor, with the weight row shared by the batch
+        self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+        if getattr(self.f.m, "dense", True) is None:
+            # the matrix-core executor takes a second operand of multiplicity one; others run on the uniform-1d kernels of
+            # the flattened descriptor, with the weight row shared by the batch
             self.f = None
         # A second operand of V invariant scalars ("10x0e" node attributes): the product is the Linear map of the
         # features x1[i, u] * x2[v] (multiplicity u * V) with the very same weights - same paths, same weight layout

@@ -215,9 +215,9 @@ class SegmentedPolynomial(nn.Module):
         if method == "uniform_1d":
             self.m = SegmentedPolynomialFromUniform1d(polynomial, math_dtype, output_dtype_map, name, self.options)
         elif method == "fused_tp":
-            from .dense import SegmentedPolynomialDense
+            from .fused_tp import SegmentedPolynomialFusedTP
 
-            self.m = SegmentedPolynomialDense(polynomial, math_dtype, output_dtype_map, name)
+            self.m = SegmentedPolynomialFusedTP(polynomial, math_dtype, output_dtype_map, name)
         elif method == "naive":
             raise ValueError(
                 "method='naive' (the PyTorch executor) is not part of this engine: every method runs HIP kernels. "
