@@ -657,7 +657,13 @@ static int run_bwd(const SpecCall& c) {{
   }}
   if (x1_idx && det && b[5].rows > 0) {{
     const int64_t n = b[5].rows * {W1}ll;
-    hipLaunchKernelGGL(segment_sum_rows<{T}>, dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1_partial, b[5].csr_offsets, b[5].csr_perm, b[5].rows, {W1}, dx1);
+    if ({W1} % 4 == 0 && reinterpret_cast<uintptr_t>(dx1) % (4 * sizeof({T})) == 0 && reinterpret_cast<uintptr_t>(dx1_partial) % (4 * sizeof({T})) == 0 &&
+        b[5].rows < 65536) {{
+      hipLaunchKernelGGL(segment_sum_rows_vec<{T}>, dim3(({W1} / 4 + 255) / 256, static_cast<unsigned>(b[5].rows)), dim3(256), 0, c.stream,
+                         dx1_partial, b[5].csr_offsets, b[5].csr_perm, {W1}, dx1);
+    }} else {{
+      hipLaunchKernelGGL(segment_sum_rows<{T}>, dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1_partial, b[5].csr_offsets, b[5].csr_perm, b[5].rows, {W1}, dx1);
+    }}
     CUEQ_CHECK_HIP(hipGetLastError());
   }}
   return CUEQ_OK;
