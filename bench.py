@@ -43,7 +43,7 @@ VALU_PEAK_F32 = 157.3
 TRAFFIC_SOURCE = "profiles/channelwise_c128_l3_fp32_cfg2_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, not of this run)"
 MEASURED_TRAFFIC_BYTES = {
     ("c128_l3_bwd_float", 5000, 100_000): 4.270e9,
-    ("c128_l3_fwd_float", 5000, 100_000): 2.135e9,
+    ("c128_l3_fwd_float", 5000, 100_000): 2.143e9,
 }
 
 # Vector (wave64) instructions the generated kernels execute per batch element (sample, edge, node), forward and backward,
@@ -455,6 +455,9 @@ def main() -> int:
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (default: the box's share, at most 16)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="only measure what the memory system delivers to streaming kernels of this library's shape: read, write, "
+                         "copy and float atomic-add rates over 1 GiB")
     ap.add_argument("--deterministic", action="store_true",
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
     ap.add_argument("--graph", action="store_true",
@@ -479,6 +482,26 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
     dev = torch.device("cuda:0")
+    if args.calibrate:
+        # what the memory system delivers to kernels shaped like the path-table kernels (cueq_calibrate): 1 GiB per launch
+        n = 1 << 30
+        a = torch.zeros(n // 4, dtype=torch.float32, device=dev)
+        b = torch.zeros(n // 4, dtype=torch.float32, device=dev)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        out = {"calibration": "cueq_calibrate, 1 GiB per launch, 64-thread workgroups, one dword per lane and instruction, 8 wavefronts per CU",
+               "published_hbm_TBps": HBM_PEAK_GBS / 1e3}
+        for kind, name, moved in ((0, "read", n), (1, "write", n), (3, "copy", 2 * n), (2, "atomic_add_f32", n)):
+            for _ in range(2):
+                _lib.check(_lib.load().cueq_calibrate(kind, a.data_ptr(), b.data_ptr(), n, stream), "cueq_calibrate")
+            torch.cuda.synchronize()
+            _lib.timing_begin()
+            for _ in range(5):
+                _lib.check(_lib.load().cueq_calibrate(kind, a.data_ptr(), b.data_ptr(), n, stream), "cueq_calibrate")
+            torch.cuda.synchronize()
+            (launches, total_ms), = _lib.timing_end().values()
+            out[name + "_TBps"] = moved / (total_ms / launches * 1e-3) / 1e12
+        print(json.dumps(out))
+        return 0
     if args.calibration_copy:
         n = 1 << 28  # 2^28 floats = 1 GiB read and 1 GiB written per copy
         a = torch.ones(n, dtype=torch.float32, device=dev)

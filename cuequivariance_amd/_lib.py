@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "cueq_get_option",
     "cueq_timing_begin",
     "cueq_timing_end",
+    "cueq_calibrate",
     "cueq_u1d_plan_create",
     "cueq_u1d_plan_destroy",
     "cueq_u1d_plan_info",
@@ -149,6 +150,8 @@ def load() -> C.CDLL:
         lib.cueq_get_option.restype = C.c_int
         lib.cueq_timing_end.argtypes = [C.POINTER(TimingEntry), C.c_int]
         lib.cueq_timing_end.restype = C.c_int
+        lib.cueq_calibrate.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+        lib.cueq_calibrate.restype = C.c_int
         lib.cueq_u1d_plan_create.argtypes = [C.POINTER(U1dDesc), C.POINTER(C.c_void_p)]
         lib.cueq_u1d_plan_create.restype = C.c_int
         lib.cueq_u1d_plan_destroy.argtypes = [C.c_void_p]

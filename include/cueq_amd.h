@@ -53,6 +53,12 @@ int cueq_get_option(const char* name);
  * and their summed duration.  Same purpose as the reference's event-based helper
  * cuequivariance_torch/cuequivariance_torch/benchmarking.py:24-158; unlike it, the events sit directly
  * around the kernel inside the library, so host-side launch work is excluded. */
+/* Memory-system calibration (no counterpart in the reference): one launch of a streaming kernel shaped like the
+ * path-table kernels (64-thread workgroups, a dword per lane and instruction, 8 wavefronts per compute unit) over
+ * `bytes` of the two device buffers; kind 0 reads `in`, 1 writes `out`, 2 adds to `out` with float atomics, 3 copies.
+ * Time it with cueq_timing_begin / cueq_timing_end (labels calibrate_read / _write / _atomic / _copy). */
+int cueq_calibrate(int32_t kind, const void* in, void* out, int64_t bytes, void* stream);
+
 typedef struct {
   char name[64];
   int64_t launches;
