@@ -98,8 +98,12 @@ def _poly_expr(terms, T: str) -> list[str]:
 
 
 def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hashes: dict, *, fwd_waves: int = 4,
-              bwd_waves: int = 2) -> str:
+              bwd_waves: int = 2, fwd_prefetch: bool = None) -> str:
     """Complete translation unit.  ``bwd_hashes``: {(need_dw, need_dx): table hash}."""
+    if fwd_prefetch is None:
+        # float: 96 -> 119 registers, still 4 wavefronts per SIMD; double: the pair products alone exceed the register file
+        # (the kernel spills either way), a second set of x rows only adds to that
+        fwd_prefetch = T == "float"
     ns = f"sc_{name}"
     E, W, X, O = st.extent, st.nseg_w * st.extent, st.nseg_x * st.extent, st.nseg_out * st.extent
     nch = (E + 63) // 64
@@ -131,15 +135,44 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A(f"  const int ch = blockIdx.x % {nch}; const int64_t slot = blockIdx.x / {nch}; const int64_t nslots = gridDim.x / {nch};")
     A(lane_setup)
     A("  const int64_t z0 = slot * batch / nslots, z1 = (slot + 1) * batch / nslots;")
-    A("  for (int64_t z = z0; z < z1; ++z) {")
-    A("    int64_t wrow = W_MODE == 0 ? z : 0;")
-    A("    if (W_MODE == 1) wrow = load_index(w_index, idx64, z);")
-    A(f"    const {T}* __restrict__ xp = x + z * {X}ll;")
-    A(f"    const {T}* __restrict__ wp = w + wrow * {W}ll;")
-    for a in x_used:
-        A(f"    const {T} xv{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
-    for s in w_used:
-        A(f"    const {T} wv{s} = wp[{s * E} + uu];")
+    if fwd_prefetch:
+        # the x row (and the weight index) of the next batch row are requested before the arithmetic of the current one; the
+        # request is unconditional (the last row is fetched again) so that the waits can count outstanding loads
+        A("  if (z0 >= z1) return;")
+        A("  int64_t wrow_n = W_MODE == 0 ? z0 : 0;")
+        A("  if (W_MODE == 1) wrow_n = load_index(w_index, idx64, z0);")
+        A(f"  {T} " + ", ".join(f"xn{a}" for a in x_used) + ";")
+        A("  {")
+        A(f"    const {T}* __restrict__ xp = x + z0 * {X}ll;")
+        for a in x_used:
+            A(f"    xn{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
+        A("  }")
+        A("  for (int64_t z = z0; z < z1; ++z) {")
+        A("    const int64_t wrow = wrow_n;")
+        A(f"    const {T}* __restrict__ wp = w + wrow * {W}ll;")
+        for s in w_used:
+            A(f"    const {T} wv{s} = wp[{s * E} + uu];")
+        for a in x_used:
+            A(f"    const {T} xv{a} = xn{a};")
+        A("    {")
+        A("      const int64_t zn = z + 1 < z1 ? z + 1 : z;")
+        A("      wrow_n = W_MODE == 0 ? zn : 0;")
+        A("      if (W_MODE == 1) wrow_n = load_index(w_index, idx64, zn);")
+        A(f"      const {T}* __restrict__ xp = x + zn * {X}ll;")
+        for a in x_used:
+            A(f"      xn{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
+        A("    }")
+        A("    __builtin_amdgcn_sched_barrier(0);")
+    else:
+        A("  for (int64_t z = z0; z < z1; ++z) {")
+        A("    int64_t wrow = W_MODE == 0 ? z : 0;")
+        A("    if (W_MODE == 1) wrow = load_index(w_index, idx64, z);")
+        A(f"    const {T}* __restrict__ xp = x + z * {X}ll;")
+        A(f"    const {T}* __restrict__ wp = w + wrow * {W}ll;")
+        for a in x_used:
+            A(f"    const {T} xv{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
+        for s in w_used:
+            A(f"    const {T} wv{s} = wp[{s * E} + uu];")
     for a, b in pairs:
         A(f"    const {T} pp_{a}_{b} = xv{a} * xv{b};")
     for k in range(st.nseg_out):
