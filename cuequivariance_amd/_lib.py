@@ -87,6 +87,8 @@ class U1dDesc(C.Structure):
         ("path_indices_len", C.c_int64),
         ("path_coefficients", C.POINTER(C.c_double)),
         ("path_coefficients_len", C.c_int64),
+        ("layout_num_groups", C.POINTER(C.c_int32)),
+        ("layout_group_dims", C.POINTER(C.c_int32)),
     ]
 
 
@@ -293,6 +295,10 @@ def make_desc(tables, math_code: int):
         pi=int32_array(tables.path_indices),
         pc=double_array(tables.path_coefficients),
     )
+    layouts = getattr(tables, "layouts", ())
+    if layouts:
+        keep["lay_n"] = int32_array([len(lay) for lay in layouts])
+        keep["lay_d"] = int32_array([d for lay in layouts for d in lay])
     desc = U1dDesc(
         math_dtype=math_code,
         operand_extent=tables.operand_extent,
@@ -311,6 +317,9 @@ def make_desc(tables, math_code: int):
         path_coefficients=keep["pc"],
         path_coefficients_len=len(tables.path_coefficients),
     )
+    if layouts:
+        desc.layout_num_groups = keep["lay_n"]
+        desc.layout_group_dims = keep["lay_d"]
     return desc, keep
 
 

@@ -94,13 +94,35 @@ class ChannelwiseStructure:
     nseg_x2: int
     nseg_out: int
     blocks: list
+    # row layouts of x1 (also of its gradient) and of the output (also of its cotangent): () = segment s, channel u at
+    # s * extent + u; group sizes (d_0, d_1, ...) = groups of consecutive segments stored channel-major ("mul_ir")
+    layout_x1: tuple = ()
+    layout_out: tuple = ()
 
     @property
     def num_paths(self):
         return sum(len(b.entries) for b in self.blocks)
 
+    def _at(self, layout, seg: int) -> str:
+        """Element offset of (segment, this lane's channel ``uu``) inside a row, as a C expression."""
+        if not layout:
+            return f"{seg * self.extent} + uu"
+        off = 0
+        for d in layout:
+            if seg < d:
+                return f"{off + seg} + uu" if d == 1 else f"{off + seg} + uu * {d}"
+            seg -= d
+            off += d * self.extent
+        raise IndexError(seg)
 
-def analyze(extent: int, nseg: Sequence[int], paths: Sequence[tuple]) -> ChannelwiseStructure:
+    def x1_at(self, i: int) -> str:
+        return self._at(self.layout_x1, i)
+
+    def out_at(self, k: int) -> str:
+        return self._at(self.layout_out, k)
+
+
+def analyze(extent: int, nseg: Sequence[int], paths: Sequence[tuple], layout_x1: tuple = (), layout_out: tuple = ()) -> ChannelwiseStructure:
     """``paths``: (w_seg, x1_seg, x2_seg, out_seg, coefficient)."""
     blocks: dict[int, Block] = {}
     for b, i, j, k, c in paths:
@@ -110,7 +132,7 @@ def analyze(extent: int, nseg: Sequence[int], paths: Sequence[tuple]) -> Channel
     out = [blocks[b] for b in sorted(blocks)]
     # Order blocks so that blocks reading the same x1 segments are neighbours (register reuse).
     out.sort(key=lambda blk: (blk.i_list, blk.j_list, blk.b))
-    return ChannelwiseStructure(extent, nseg[0], nseg[1], nseg[2], nseg[3], out)
+    return ChannelwiseStructure(extent, nseg[0], nseg[1], nseg[2], nseg[3], out, tuple(layout_x1), tuple(layout_out))
 
 
 def _lit(c: float, T: str) -> str:
@@ -228,7 +250,7 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
                 nvalid = min(16, st.nseg_x2 - 16 * m)
                 A(f"{ind}  {S}_yv{m} = x2p[{16 * m} + (n16 < {nvalid} ? n16 : 0)];")
             for i in i_used:
-                A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
+                A(f"{ind}  {S}_xv{i} = x1p[{st.x1_at(i)}];")
             for blk in blocks:
                 A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
             A(f"{ind}}}")
@@ -290,7 +312,7 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
         A("  if (active) {")
         A(f"    {fp}* __restrict__ op = out + r * {st.nseg_out * st.extent}ll;")
         for k in ks:
-            A(f"    STREAM_STORE(acc{k}, op + {k * st.extent} + uu);")
+            A(f"    STREAM_STORE(acc{k}, op + {st.out_at(k)});")
         A("  }")
         A("}")
         A("")
@@ -352,6 +374,14 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
         i_zero = [i for i in range(st.nseg_x1) if i not in i_all] if q == 0 else []
         w_zero = [b for b in range(st.nseg_w) if b not in w_all] if q == 0 else []
 
+        # channel-major groups of x1 this wavefront owns whole: (first segment, size); their gradient is staged through LDS
+        staged, first = [], 0
+        for d in st.layout_x1:
+            if d > 1 and all(i in i_used for i in range(first, first + d)):
+                staged.append((first, d))
+            first += d
+        staged_segments = {i for i0, d in staged for i in range(i0, i0 + d)}
+
         def load(S: str, zz: str, ind: str):
             A(f"{ind}{{")
             A(f"{ind}  const int64_t z = {zz};")
@@ -363,7 +393,7 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
             A(f"{ind}  const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
             A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
             for i in i_used:
-                A(f"{ind}  {S}_xv{i} = x1p[{i * st.extent} + uu];")
+                A(f"{ind}  {S}_xv{i} = x1p[{st.x1_at(i)}];")
             for blk in blocks:
                 A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
             for j in j_used:
@@ -376,7 +406,7 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
             A(f"{ind}  grow_cur = {S}_grow;")
             A(f"{ind}  const {fp}* __restrict__ gp = g + grow_cur * {st.nseg_out * st.extent}ll;")
             for k in ks:
-                A(f"{ind}  gr{k} = STREAM_LOAD(gp + {k * st.extent} + uu);")
+                A(f"{ind}  gr{k} = STREAM_LOAD(gp + {st.out_at(k)});")
             A(f"{ind}}}")
             A(f"{ind}{fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
             for i in i_used:
@@ -412,16 +442,30 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
                 A(f"{ind}__builtin_amdgcn_sched_barrier(0);")
             for b_ in w_zero:
                 A(f"{ind}if (active) STREAM_STORE({fp}(0), dwp + {b_ * st.extent} + uu);")
-            # dx1: scatter
+            # dx1: scatter.  Atomic adds are served per touched 32-byte sector, not per element: the components of a
+            # channel-major group (a stride of d elements between lanes) go through LDS first, so that every atomic
+            # instruction of the wavefront covers 64 consecutive elements as it does in the default layout.
+            for i0, d in staged:
+                A(f"{ind}if (ATOMIC_DX1) {{")
+                A(f"{ind}  {fp}* dp = dx1 + {S}_srow * {st.nseg_x1 * st.extent}ll + {st.extent * i0} + ch * {64 * d};")
+                A(f"{ind}  __builtin_amdgcn_wave_barrier();")
+                for c in range(d):
+                    A(f"{ind}  dxs[lane * {d} + {c}] = dxa{i0 + c};")
+                A(f"{ind}  __builtin_amdgcn_wave_barrier();")
+                for k in range(d):
+                    guard = "" if st.extent % 64 == 0 else f"if (ch * {64 * d} + {k * 64} + lane < {st.extent * d}) "
+                    A(f"{ind}  {guard}unsafeAtomicAdd(dp + {k * 64} + lane, dxs[{k * 64} + lane]);")
+                A(f"{ind}}}")
             A(f"{ind}if (active) {{")
             A(f"{ind}  if (ATOMIC_DX1) {{")
             A(f"{ind}    {fp}* dp = dx1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
             for i in i_used:
-                A(f"{ind}    unsafeAtomicAdd(dp + ({i * st.extent} + uu), dxa{i});")
+                if i not in staged_segments:
+                    A(f"{ind}    unsafeAtomicAdd(dp + ({st.x1_at(i)}), dxa{i});")
             A(f"{ind}  }} else {{")
             A(f"{ind}    {fp}* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
             for i in sorted(i_used + i_zero):
-                A(f"{ind}    dp[{i * st.extent} + uu] = " + (f"dxa{i};" if i in i_used else "0;"))
+                A(f"{ind}    dp[{st.x1_at(i)}] = " + (f"dxa{i};" if i in i_used else "0;"))
             A(f"{ind}  }}")
             A(f"{ind}}}")
             # dx2: reduce over the 64 lanes; channel chunks and wavefronts of one batch row are folded afterwards
@@ -439,6 +483,8 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
 
         A("template <bool X1_IDX, bool G_IDX, bool ATOMIC_DX1>")
         A(f"__device__ __forceinline__ void bwd_group{q}(BWD_PARAMS, int64_t z0, int64_t z1, int lane, int uu, bool active, int ch) {{")
+        if staged:
+            A(f"  __shared__ {fp} dxs[{64 * max(d for _, d in staged)}];")
         for k in ks:
             A(f"  {fp} gr{k} = 0;")
         A("  int64_t grow_cur = -1;")
@@ -524,7 +570,8 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     A = out.append
     A("// GENERATED by cuequivariance_amd/codegen/channelwise.py - do not edit.")
     A(f"// channel-wise tensor product '{name}': extent {st.extent}, segments w/x1/x2/out = "
-      f"{st.nseg_w}/{st.nseg_x1}/{st.nseg_x2}/{st.nseg_out}, {st.num_paths} paths, math {T}")
+      f"{st.nseg_w}/{st.nseg_x1}/{st.nseg_x2}/{st.nseg_out}, {st.num_paths} paths, math {T}"
+      + (f", x1 rows in groups {list(st.layout_x1)}" if st.layout_x1 else "") + (f", output rows in groups {list(st.layout_out)}" if st.layout_out else ""))
     A('#include "cw_common.h"')
     A("// operands that are read or written exactly once per launch (weights, weight gradients, the output rows) are")
     A("// marked non-temporal so that they do not displace the gathered rows in the caches")

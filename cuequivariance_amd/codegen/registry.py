@@ -22,6 +22,10 @@ CHANNELWISE = [
     ("c32_l2", "32x0e+32x1o+32x2e", "0e+1o+2e", "0e+1o+2e", {}),
 ]
 
+# Channel-wise entries that are also generated for operands in the mul_ir layout (x1, the output and their gradients
+# addressed channel-major inside every irrep block: no transposition pass before or after the kernels); unit "<name>_mulir".
+CHANNELWISE_MUL_IR = ["c128_l3", "c32_l2"]
+
 # (name, irreps_in, irreps_out, contraction degree)
 SYMMETRIC = [
     ("s128_l3", "128x0e+128x1o+128x2e+128x3o", "128x0e+128x1o", 3),
@@ -40,6 +44,13 @@ MATH = (("float", 0), ("double", 1))
 def channelwise_tables(irreps1: str, irreps2: str, filt) -> U1dTables:
     e = cue.descriptors.channelwise_tensor_product(cue.Irreps("O3", irreps1), cue.Irreps("O3", irreps2), filt)
     return U1dTables.from_polynomial(e.polynomial.flatten_coefficient_modes().squeeze_modes())
+
+
+def channelwise_mul_ir_groups(irreps1: str, irreps2: str, filt):
+    """{buffer: group sizes} of the flattened channel-wise tables when x1 (buffer 1) and the output (buffer 3) are stored
+    mul_ir: one group of ``ir.dim`` segments per ``(mul, ir)`` block."""
+    e = cue.descriptors.channelwise_tensor_product(cue.Irreps("O3", irreps1), cue.Irreps("O3", irreps2), filt)
+    return {1: [ir.dim for _, ir in e.inputs[1].irreps], 3: [ir.dim for _, ir in e.outputs[0].irreps]}
 
 
 def symmetric_polynomial(irreps_in: str, irreps_out: str, degree: int):
@@ -71,14 +82,20 @@ def generate(verbose: bool = False) -> list[Path]:
         _, paths = t.operation(0)
         st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
         tb = t.backward((True, True, True))
-        for T, code in MATH:
-            src = cw.emit_unit(st, T, name, t.content_hash(code), tb.content_hash(code), **tuning.get(T, {}))
-            path = GENERATED_DIR / f"cw_{name}_{T}.hip"
-            if not path.exists() or path.read_text() != src:
-                path.write_text(src)
-            written.append(path)
-            if verbose:
-                print(f"generated {path.name}: {st.num_paths} paths")
+        variants = [(name, st, t, tb)]
+        if name in CHANNELWISE_MUL_IR:
+            tl = t.with_layouts(channelwise_mul_ir_groups(ir1, ir2, filt))
+            stl = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths], tl.layout(1), tl.layout(3))
+            variants.append((name + "_mulir", stl, tl, tl.backward((True, True, True))))
+        for vname, vst, vt, vtb in variants:
+            for T, code in MATH:
+                src = cw.emit_unit(vst, T, vname, vt.content_hash(code), vtb.content_hash(code), **tuning.get(T, {}))
+                path = GENERATED_DIR / f"cw_{vname}_{T}.hip"
+                if not path.exists() or path.read_text() != src:
+                    path.write_text(src)
+                written.append(path)
+                if verbose:
+                    print(f"generated {path.name}: {vst.num_paths} paths")
     return written
 
 

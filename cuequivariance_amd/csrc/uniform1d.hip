@@ -92,6 +92,20 @@ uint64_t hash_u1d_desc(const cueq_u1d_desc* d) {
       f.word(bits);
     }
   }
+  // row layouts (descriptors without any hash as they always did)
+  bool any_layout = false;
+  if (d->layout_num_groups)
+    for (int b = 0; b < nbuf; ++b) any_layout |= d->layout_num_groups[b] > 0;
+  if (any_layout) {
+    f.word(0x6C61796F757473ull);
+    int64_t g0 = 0;
+    for (int b = 0; b < nbuf; ++b) {
+      const int ng = d->layout_num_groups[b];
+      f.word(static_cast<uint64_t>(ng));
+      for (int g = 0; g < ng; ++g) f.word(static_cast<uint64_t>(d->layout_group_dims[g0 + g]));
+      g0 += ng;
+    }
+  }
   return f.h;
 }
 
@@ -143,6 +157,9 @@ struct DevBuffer {
   int32_t dim;
   int32_t nseg;
   int32_t pad;
+  // row layout other than "segment s, channel u at s * extent + u": element offset of (s, u) = seg_base[s] + u * seg_stride[s]
+  const int32_t* seg_base;
+  const int32_t* seg_stride;
 };
 
 struct KernelArgs {
@@ -163,6 +180,8 @@ struct KernelArgs {
   int32_t out_nseg;
   int32_t extent;
   int32_t chunk;
+  const int32_t* out_seg_base;  // layout of the output rows (null: default)
+  const int32_t* out_seg_stride;
 };
 
 template <typename M>
@@ -177,7 +196,9 @@ __device__ __forceinline__ M path_product(const KernelArgs& a, int p, int64_t z,
     if (b.mode == CUEQ_BATCH_BATCHED) row = z;
     else if (b.mode == CUEQ_BATCH_INDEXED) row = load_index(b.index, b.index_is_64, z);
     const int64_t width = b.dim ? static_cast<int64_t>(b.nseg) * a.extent : b.nseg;
-    const int64_t off = row * width + (b.dim ? static_cast<int64_t>(seg) * a.extent + u : seg);
+    const int64_t off = row * width + (b.dim ? (b.seg_base ? static_cast<int64_t>(b.seg_base[seg]) + static_cast<int64_t>(u) * b.seg_stride[seg]
+                                                              : static_cast<int64_t>(seg) * a.extent + u)
+                                            : seg);
     prod *= load_as<M>(b.data, b.dtype, off);
   }
   return prod;
@@ -208,7 +229,8 @@ __global__ void __launch_bounds__(256) u1d_generic_elem(KernelArgs a) {
     const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
     for (int p = p0; p < p1; ++p) acc += path_product<M>(a, p, z, u);
   }
-  store_as<M>(a.out, a.out_dtype, tid, acc);
+  const int64_t where = a.out_seg_base ? r * per_row + a.out_seg_base[s] + static_cast<int64_t>(u) * a.out_seg_stride[s] : tid;
+  store_as<M>(a.out, a.out_dtype, where, acc);
 }
 
 // One wavefront per scalar output element (row, segment): lanes stride over the channel
@@ -271,6 +293,7 @@ struct cueq_u1d_plan {
   int32_t num_inputs, num_outputs;
   std::vector<int32_t> buffer_dim, buffer_nseg;
   std::vector<OutTables> out;  // one per output buffer
+  std::vector<const int32_t*> seg_base, seg_stride;  // per buffer, device pointers (null: default layout)
   const cueq::U1dSpec* spec = nullptr;  // descriptor-specialised kernels, if any were built
   uint64_t hash = 0;
   void* device_blob = nullptr;
@@ -404,7 +427,39 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
     offs[ob].in = reserve(v.size() * kMaxInOperands * sizeof(int32_t));
     offs[ob].seg = reserve((nseg + 1) * sizeof(int32_t));
   }
+  // row layouts: per buffer the base offset and channel stride of every segment
+  std::vector<size_t> lay_off(nbuf, SIZE_MAX);
+  std::vector<std::vector<int32_t>> lay_tab(nbuf);
+  if (d->layout_num_groups) {
+    int64_t g0 = 0;
+    for (int b = 0; b < nbuf; ++b) {
+      const int ng = d->layout_num_groups[b];
+      if (ng < 0) { delete plan; CUEQ_REQUIRE(false, CUEQ_ERR_INVALID, "negative group count for buffer %d", b); }
+      if (ng > 0) {
+        const int nseg = d->buffer_num_segments[b];
+        std::vector<int32_t>& t = lay_tab[b];
+        t.assign(2 * static_cast<size_t>(nseg), 0);
+        int64_t seg = 0, off = 0;
+        bool ok = d->buffer_dim[b] == 1 && d->layout_group_dims != nullptr;
+        for (int g = 0; ok && g < ng; ++g) {
+          const int dim = d->layout_group_dims[g0 + g];
+          if (dim < 1 || seg + dim > nseg) { ok = false; break; }
+          for (int c = 0; c < dim; ++c) { t[seg + c] = static_cast<int32_t>(off + c); t[nseg + seg + c] = dim; }
+          seg += dim;
+          off += static_cast<int64_t>(dim) * d->operand_extent;
+        }
+        if (!ok || seg != nseg || off >= (int64_t(1) << 31)) {
+          delete plan;
+          CUEQ_REQUIRE(false, CUEQ_ERR_INVALID, "layout groups of buffer %d do not partition its %d channel segments", b, nseg);
+        }
+        lay_off[b] = reserve(t.size() * sizeof(int32_t));
+      }
+      g0 += ng;
+    }
+  }
   std::vector<char> host(total ? total : 16, 0);
+  for (int b = 0; b < nbuf; ++b)
+    if (lay_off[b] != SIZE_MAX) std::memcpy(host.data() + lay_off[b], lay_tab[b].data(), lay_tab[b].size() * sizeof(int32_t));
   for (int ob = 0; ob < d->num_outputs; ++ob) {
     auto& v = per_out[ob];
     const int nseg = d->buffer_num_segments[d->num_inputs + ob];
@@ -440,6 +495,13 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
     t.seg_start = reinterpret_cast<int32_t*>(base + offs[ob].seg);
     t.contracts_channel = contracts[ob];
   }
+  plan->seg_base.assign(nbuf, nullptr);
+  plan->seg_stride.assign(nbuf, nullptr);
+  for (int b = 0; b < nbuf; ++b)
+    if (lay_off[b] != SIZE_MAX) {
+      plan->seg_base[b] = reinterpret_cast<const int32_t*>(base + lay_off[b]);
+      plan->seg_stride[b] = plan->seg_base[b] + d->buffer_num_segments[b];
+    }
   plan->hash = hash_u1d_desc(d);
   plan->spec = find_u1d_spec(plan->hash);
   *out_plan = plan;
@@ -516,6 +578,8 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
     dbuf.index_is_64 = s.index_is_64;
     dbuf.dim = plan->buffer_dim[b];
     dbuf.nseg = plan->buffer_nseg[b];
+    dbuf.seg_base = plan->seg_base[b];
+    dbuf.seg_stride = plan->seg_stride[b];
   }
   a.batch = batch;
   a.extent = plan->extent;
@@ -540,6 +604,8 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
     a.out = o.data;
     a.out_dtype = o.dtype;
     a.out_rows = o.rows;
+    a.out_seg_base = plan->seg_base[b];
+    a.out_seg_stride = plan->seg_stride[b];
     int64_t nchunks = 0;
     if (o.batch_dim == CUEQ_BATCH_SHARED) {
       nchunks = share_chunks(batch);

@@ -47,6 +47,11 @@ def _assert_same_group(*irreps_list):
             raise ValueError("The provided irreps are not of the same group.")
 
 
+def _transposition_moves(irreps) -> bool:
+    """Whether mul_ir and ir_mul differ for these irreps (some block has both a multiplicity and a dimension above one)."""
+    return any(mul > 1 and ir.dim > 1 for mul, ir in irreps)
+
+
 def _default_layout(layout) -> cue.IrrepsLayout:
     if layout is None:
         warnings.warn("layout is not specified, defaulting to cue.mul_ir (the e3nn layout)")
@@ -141,22 +146,32 @@ class ChannelWiseTensorProduct(torch.nn.Module):
             self.weight = torch.nn.Parameter(torch.randn(1, self.weight_numel, device=device, dtype=dtype))
         else:
             self.weight = None
-        self.transpose_in1 = TransposeIrrepsLayout(
-            e.inputs[1].irreps, source=_default_layout(layout_in1 or layout), target=e.inputs[1].layout, device=device
-        )
-        self.transpose_in2 = TransposeIrrepsLayout(
-            e.inputs[2].irreps, source=_default_layout(layout_in2 or layout), target=e.inputs[2].layout, device=device
-        )
-        self.transpose_out = TransposeIrrepsLayout(
-            e.outputs[0].irreps, source=e.outputs[0].layout, target=_default_layout(layout_out or layout), device=device
-        )
         self.method = _method_from_fallback(method, use_fallback, "uniform_1d")
         if self.method == "uniform_1d" and not u1d_compatible:
             raise ValueError(
                 "`uniform_1d` method requires segments to be the same shape\n"
                 "You can consider making the segments uniform in the descriptor."
             )
-        self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+        source_in1, target_out = _default_layout(layout_in1 or layout), _default_layout(layout_out or layout)
+        # x1 and the output in the mul_ir layout are addressed as they lie by the uniform-1d kernels (the flattened
+        # descriptor has one segment per component of a block: a group of ir.dim segments stored channel-major), which
+        # saves the transposition pass before and after the product, and their counterparts in the backward
+        groups = {}
+        if self.method == "uniform_1d":
+            if source_in1 == cue.mul_ir and e.inputs[1].layout == cue.ir_mul and _transposition_moves(e.inputs[1].irreps):
+                groups[1] = [ir.dim for _, ir in e.inputs[1].irreps]
+                source_in1 = cue.ir_mul
+            if target_out == cue.mul_ir and e.outputs[0].layout == cue.ir_mul and _transposition_moves(irreps_out):
+                groups[3] = [ir.dim for _, ir in irreps_out]
+                target_out = cue.ir_mul
+        self.transpose_in1 = TransposeIrrepsLayout(e.inputs[1].irreps, source=source_in1, target=e.inputs[1].layout, device=device)
+        self.transpose_in2 = TransposeIrrepsLayout(
+            e.inputs[2].irreps, source=_default_layout(layout_in2 or layout), target=e.inputs[2].layout, device=device
+        )
+        self.transpose_out = TransposeIrrepsLayout(irreps_out, source=e.outputs[0].layout, target=target_out, device=device)
+        self.f = SegmentedPolynomial(
+            e.polynomial, method=self.method, math_dtype=math_dtype, options={"segment_groups": groups} if groups else None
+        )
 
     def extra_repr(self) -> str:
         return (

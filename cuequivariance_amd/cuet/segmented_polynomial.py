@@ -82,6 +82,15 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
             tables = U1dTables.from_polynomial(polynomial, output_dtype_map)
         except ValueError as e:
             raise ValueError(f"For method 'uniform_1d': {e}") from e
+        groups = (options or {}).get("segment_groups")
+        if groups:
+            # {operand: sizes of consecutive groups of its segments}: the rows of that operand are stored channel-major
+            # inside every group (an irreps operand in the mul_ir layout, one group per block), and the kernels address
+            # them so - no transposition pass around the call.  Not part of the reference's options.
+            try:
+                tables = tables.with_layouts({int(b): [int(d) for d in dims] for b, dims in groups.items()})
+            except ValueError as e:
+                raise ValueError(f"For method 'uniform_1d', option 'segment_groups': {e}") from e
         self.tables = tables
         self.num_inputs = polynomial.num_inputs
         self.num_outputs = polynomial.num_outputs

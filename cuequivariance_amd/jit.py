@@ -131,6 +131,16 @@ def is_symmetric_contraction(poly) -> bool:
     return True
 
 
+def _family(t: U1dTables, polynomial=None) -> Optional[str]:
+    """The family generator that serves these tables: "channelwise" (which addresses x1 and the output through their
+    layouts), "symmetric" (default layouts only) or None."""
+    if is_channelwise(t) and not t.layout(0) and not t.layout(2):
+        return "channelwise"
+    if not t.layouts and is_symmetric_contraction(polynomial):
+        return "symmetric"
+    return None
+
+
 def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTables] = None, root_polynomial=None) -> bool:
     """Kernels for one plan: first the family unit of its root (the forward plan of a channel-wise product or symmetric
     contraction holds the kernels of its backward plans too), then, if the plan still has none, a unit of its own from
@@ -139,7 +149,7 @@ def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTabl
         return True
     if not enabled():
         return False
-    if root_tables is not None and (is_channelwise(root_tables) or is_symmetric_contraction(root_polynomial)):
+    if root_tables is not None and _family(root_tables, root_polynomial):
         ensure_specialised(root_tables, math_code, root_polynomial)
         if _has_spec(tables, math_code):
             return True
@@ -155,7 +165,7 @@ def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, gener
 
     if _has_spec(tables, math_code):
         return True
-    family = is_channelwise(tables) or is_symmetric_contraction(polynomial)
+    family = _family(tables, polynomial)
     if not enabled() or not (family or (general and gen.supported(tables))):
         return False
     key = tables.content_hash(math_code)
@@ -180,14 +190,15 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None):
     T = "float" if code == _lib.F32 else "double"
     name = f"jit_{key:016x}"
     # the object's name carries a hash of the emitted source, so a changed generator (or tuning) never meets a stale object
-    if not (is_channelwise(t) or is_symmetric_contraction(polynomial)):
+    family = _family(t, polynomial)
+    if family is None:
         from .codegen import general as gen
 
         src = gen.emit_unit(t, T, name, key)
         what = f"general plan, {sum(t.num_paths)} paths, extent {t.operand_extent}"
-    elif is_channelwise(t):
+    elif family == "channelwise":
         _, paths = t.operation(0)
-        st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths])
+        st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths], t.layout(1), t.layout(3))
         tb = t.backward((True, True, True))
         src = cw.emit_unit(st, T, name, key, tb.content_hash(code), **_tuning(st, T))
         what = f"{st.num_paths} paths, extent {st.extent}"

@@ -29,6 +29,11 @@ class U1dTables:
     path_coefficients_start: tuple
     path_indices: tuple
     path_coefficients: tuple
+    # Optional layout of the rows of channel-carrying buffers: per buffer either () - segment s, channel u at
+    # s * extent + u ("ir_mul": channels contiguous) - or the sizes (d_0, d_1, ...) of groups of consecutive segments whose
+    # rows are stored channel-major inside the group ("mul_ir": segment c of group g, channel u at
+    # extent * (d_0 + ... + d_{g-1}) + u * d_g + c).  () for the whole field: every buffer in the default layout.
+    layouts: tuple = ()
 
     @classmethod
     def make(cls, operand_extent, num_inputs, num_outputs, buffer_dim, buffer_num_segments, dtypes, num_operands,
@@ -89,6 +94,35 @@ class U1dTables:
     def width(self, b: int) -> int:
         return self.buffer_num_segments[b] * (self.operand_extent if self.buffer_dim[b] else 1)
 
+    def layout(self, b: int) -> tuple:
+        return self.layouts[b] if self.layouts else ()
+
+    def with_layouts(self, groups: dict) -> "U1dTables":
+        """The same tables with the rows of the buffers in ``groups`` ({buffer: group sizes}) stored group by group,
+        channel-major inside a group (the ``mul_ir`` layout of an irreps operand: one group per ``(mul, ir)`` block)."""
+        from dataclasses import replace
+
+        nbuf = self.num_inputs + self.num_outputs
+        lay = [tuple(self.layout(b)) for b in range(nbuf)]
+        for b, dims in groups.items():
+            dims = tuple(int(d) for d in dims)
+            if not self.buffer_dim[b] or sum(dims) != self.buffer_num_segments[b] or any(d < 1 for d in dims):
+                raise ValueError(f"uniform_1d: groups {dims} do not partition the {self.buffer_num_segments[b]} channel segments of buffer {b}")
+            lay[b] = () if all(d == 1 for d in dims) else dims  # groups of one segment are the default layout
+        return replace(self, layouts=tuple(lay) if any(lay) else ())
+
+    def segment_addressing(self, b: int):
+        """(base offset, channel stride) of every segment of buffer ``b`` under its layout."""
+        E = self.operand_extent if self.buffer_dim[b] else 1
+        dims = self.layout(b)
+        if not dims:
+            return [(seg * E, 1) for seg in range(self.buffer_num_segments[b])]
+        out, off = [], 0
+        for d in dims:
+            out += [(off + c, d) for c in range(d)]
+            off += d * E
+        return out
+
     def operation(self, o: int):
         """(buffers, [(indices..., coefficient)]) of operation ``o``."""
         off = sum(self.num_operands[:o])
@@ -137,10 +171,15 @@ class U1dTables:
                 num_paths.append(self.num_paths[o])
                 pis.append(self.path_indices_start[o])
                 pcs.append(self.path_coefficients_start[o])
-        return U1dTables.make(
+        out = U1dTables.make(
             self.operand_extent, nin + nout, len(grad_buf), buf_dim, buf_nseg, dtypes, num_operands, operations,
             num_paths, pis, pcs, self.path_indices, self.path_coefficients,
         )
+        if self.layouts:  # cotangents keep the layout of their output, gradients that of their input
+            lay = {b: self.layout(b) for b in range(nin + nout) if self.layout(b)}
+            lay.update({g: self.layout(i) for i, g in grad_buf.items() if self.layout(i)})
+            out = out.with_layouts(lay)
+        return out
 
     def content_hash(self, math_code: int) -> int:
         """FNV-1a 64 over the table contents; equals ``cueq::hash_u1d_desc`` of the C library."""
@@ -156,6 +195,11 @@ class U1dTables:
             words += list(self.path_indices[pi0: pi0 + self.num_paths[o] * nop])
             for p in range(self.num_paths[o]):
                 words.append(struct.unpack("<Q", struct.pack("<d", self.path_coefficients[pc0 + p]))[0])
+        if self.layouts:  # (tables without layouts hash as they always did)
+            words.append(0x6C61796F757473)
+            for lay in self.layouts:
+                words.append(len(lay))
+                words += list(lay)
         h = 1469598103934665603
         for w in words:
             w &= _MASK64

@@ -93,6 +93,13 @@ typedef struct {
   int64_t path_indices_len;
   const double* path_coefficients;
   int64_t path_coefficients_len;
+  /* Optional row layouts (no counterpart in the reference's tables, where a transposition module sits in front of the op:
+   * cuequivariance_torch/cuequivariance_torch/primitives/transpose.py:83-183).  Default (both NULL, or 0 groups for a
+   * buffer): segment s, channel u at s * extent + u ("ir_mul").  With groups (d_0, d_1, ...) partitioning the segments of
+   * a channel-carrying buffer, the rows are stored group by group, channel-major inside a group ("mul_ir"): segment c of
+   * group g, channel u at extent * (d_0 + ... + d_{g-1}) + u * d_g + c.  The kernels address such rows directly. */
+  const int32_t* layout_num_groups;    /* [num_inputs+num_outputs] or NULL                          */
+  const int32_t* layout_group_dims;    /* the group sizes of all buffers, concatenated              */
 } cueq_u1d_desc;
 
 /* One tensor at the boundary. */
