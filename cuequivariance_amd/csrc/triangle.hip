@@ -121,37 +121,39 @@ typedef short shortx4_t __attribute__((ext_vector_type(4)));
 // bytes between the k rows of a contraction-major tile of EXT columns: the row plus 64 (2-byte) / 128 (4-byte) bytes
 template <typename TI, int EXT>
 constexpr int trans_stride() { return EXT * static_cast<int>(sizeof(TI)) + (sizeof(TI) == 2 ? 64 : 128); }
-// LDS bytes of one operand tile of EXT rows (either layout)
-template <typename TI, int EXT>
+// LDS bytes of one operand tile of EXT rows (either layout); KB = bytes of k per row and step (64 or 128), rows of a
+// contraction-contiguous tile are KB + 16 bytes apart (conflict-free 16-byte reads by 16 consecutive rows for both)
+template <typename TI, int EXT, int KB = 64>
 constexpr int gemm_tile_bytes() {
-  constexpr int a = EXT * kRowBytes, b = (64 / static_cast<int>(sizeof(TI))) * trans_stride<TI, EXT>();
+  constexpr int a = EXT * (KB + 16), b = (KB / static_cast<int>(sizeof(TI))) * trans_stride<TI, EXT>();
   return a > b ? a : b;
 }
 
-template <typename TI, bool TR, int EXT>
+template <typename TI, bool TR, int EXT, int KB = 64>
 __device__ __forceinline__ void gemm_stage_offsets(int e, int& row, int& part) {
   constexpr int VPRN = EXT * sizeof(TI) / 16;  // vectors per k row of a contraction-major tile
   if constexpr (TR) { row = e / VPRN; part = e % VPRN; }
-  else { row = e >> 2; part = e & 3; }
+  else { row = e / (KB / 16); part = e % (KB / 16); }
 }
 
-// fragment of subtile rows [base, base + 32) for MFMA step half q: 16 bytes of k per lane
-template <typename TI, bool TR, int EXT>
+// fragment of subtile rows [base, base + 32) for MFMA slice q of the step (KB / 32 slices): 16 bytes of k per lane
+template <typename TI, bool TR, int EXT, int KB = 64>
 __device__ __forceinline__ uint4 gemm_fragment(const char* tile, int base, int q, int lane) {
   constexpr int kTransStride16 = trans_stride<uint16_t, EXT>(), kTransStride32 = trans_stride<float, EXT>();
+  constexpr int HK = KB / 2 / static_cast<int>(sizeof(TI));  // k rows of a contraction-major tile per half wavefront
   const int c = lane & 31, h = lane >> 5;
   if constexpr (!TR) {
-    return *reinterpret_cast<const uint4*>(tile + (base + c) * kRowBytes + h * 32 + q * 16);
+    return *reinterpret_cast<const uint4*>(tile + (base + c) * (KB + 16) + h * (KB / 2) + q * 16);
   } else if constexpr (sizeof(TI) == 2) {
     const int s = lane & 15, g16 = (lane >> 4) & 1;
-    const char* p = tile + (16 * h + 8 * q + (s >> 2)) * kTransStride16 + (base + 16 * g16 + 4 * (s & 3)) * 2;  // k as in the other layout
+    const char* p = tile + (HK * h + 8 * q + (s >> 2)) * kTransStride16 + (base + 16 * g16 + 4 * (s & 3)) * 2;  // k as in the other layout
     typedef shortx4_t __attribute__((address_space(3))) * lptr;
     const shortx4_t r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p));
     const shortx4_t r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(p + 4 * kTransStride16));
     const uint2 a = __builtin_bit_cast(uint2, r0), b = __builtin_bit_cast(uint2, r1);
     return make_uint4(a.x, a.y, b.x, b.y);
   } else {
-    const char* p = tile + (8 * h + 4 * q) * kTransStride32 + (base + c) * 4;
+    const char* p = tile + (HK * h + 4 * q) * kTransStride32 + (base + c) * 4;
     return make_uint4(*reinterpret_cast<const uint32_t*>(p), *reinterpret_cast<const uint32_t*>(p + kTransStride32),
                       *reinterpret_cast<const uint32_t*>(p + 2 * kTransStride32), *reinterpret_cast<const uint32_t*>(p + 3 * kTransStride32));
   }
@@ -159,7 +161,9 @@ __device__ __forceinline__ uint4 gemm_fragment(const char* tile, int base, int q
 
 // WM x WN wavefronts of 64 x 64 per block: 2 x 2 (a 128 x 128 tile) by default; 4 x 4 (256 x 256, 16 wavefronts) halves
 // the operand traffic between L2 and the CUs for products whose both extents are large.
-template <typename TI, typename TO, bool TA, bool TB, int WM = 2, int WN = 2>
+// KB: bytes of k per row and step; 128 makes every request of a contraction-contiguous operand a whole 128-byte line (with
+// 64 a line is fetched in two halves one step apart, and a 256 x 256 step turns over the whole L1 in between).
+template <typename TI, typename TO, bool TA, bool TB, int WM = 2, int WN = 2, int KB = 64>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA,
                                                    const TI* __restrict__ B, int64_t ldb, int64_t sB,
                                                    TO* __restrict__ C, int64_t ldc, int64_t sC, int Mfull, int N, int Kfull,
@@ -167,11 +171,13 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
                                                    int64_t pB, int64_t pC, const int64_t* __restrict__ goff, int ngroups, int gmode,
                                                    int64_t gsB, int64_t gsC) {
   constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
-  constexpr int BK = 64 / sizeof(TI);   // k extent of one step
+  constexpr int BK = KB / sizeof(TI);   // k extent of one step
+  constexpr int RB = KB + 16;           // bytes between the rows of a contraction-contiguous tile
+  constexpr int NQ = KB / 32;           // 16-byte slices of k per half wavefront and step
   constexpr int TMR = 64 * WM, TNC = 64 * WN, NTH = 64 * WM * WN;  // tile rows, tile columns, threads
   constexpr int TSA = trans_stride<TI, TMR>(), TSB = trans_stride<TI, TNC>();
-  constexpr int ABYTES = gemm_tile_bytes<TI, TMR>(), BBYTES = gemm_tile_bytes<TI, TNC>();
-  constexpr int NVA = TMR * 4 / NTH, NVB = TNC * 4 / NTH;  // 16-byte vectors per thread and step
+  constexpr int ABYTES = gemm_tile_bytes<TI, TMR, KB>(), BBYTES = gemm_tile_bytes<TI, TNC, KB>();
+  constexpr int NVA = TMR * (KB / 16) / NTH, NVB = TNC * (KB / 16) / NTH;  // 16-byte vectors per thread and step
   __shared__ __align__(16) char smem[2][ABYTES + BBYTES];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
@@ -222,9 +228,9 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
   uint4 stA[NVA], stB[NVB];
   int arow[NVA], apart[NVA], brow[NVB], bpart[NVB];
 #pragma unroll
-  for (int q = 0; q < NVA; ++q) gemm_stage_offsets<TI, TA, TMR>(tid + q * NTH, arow[q], apart[q]);
+  for (int q = 0; q < NVA; ++q) gemm_stage_offsets<TI, TA, TMR, KB>(tid + q * NTH, arow[q], apart[q]);
 #pragma unroll
-  for (int q = 0; q < NVB; ++q) gemm_stage_offsets<TI, TB, TNC>(tid + q * NTH, brow[q], bpart[q]);
+  for (int q = 0; q < NVB; ++q) gemm_stage_offsets<TI, TB, TNC, KB>(tid + q * NTH, brow[q], bpart[q]);
   auto load_one = [&](const TI* __restrict__ P, int64_t ld, bool tr, int row, int part, int x0, int X, int ks) -> uint4 {
     if (tr) {  // row = k within the step, part = vector along the tile's columns (extent X is a multiple of EPV)
       const int k = ks * BK + row, x = x0 + part * EPV;
@@ -245,10 +251,10 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
   };
   auto store_step = [&](int buf) {
 #pragma unroll
-    for (int q = 0; q < NVA; ++q) *reinterpret_cast<uint4*>(&smem[buf][arow[q] * (TA ? TSA : kRowBytes) + apart[q] * 16]) = stA[q];
+    for (int q = 0; q < NVA; ++q) *reinterpret_cast<uint4*>(&smem[buf][arow[q] * (TA ? TSA : RB) + apart[q] * 16]) = stA[q];
 #pragma unroll
     for (int q = 0; q < NVB; ++q)
-      *reinterpret_cast<uint4*>(&smem[buf][ABYTES + brow[q] * (TB ? TSB : kRowBytes) + bpart[q] * 16]) = stB[q];
+      *reinterpret_cast<uint4*>(&smem[buf][ABYTES + brow[q] * (TB ? TSB : RB) + bpart[q] * 16]) = stB[q];
   };
 
   floatx16 acc[2][2];
@@ -264,17 +270,17 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
     store_step(buf);
     __syncthreads();
     if (ks + 1 < nsteps) load_step(ks + 1);
-    uint4 fa[2][2], fb[2][2];
+    uint4 fa[2][NQ], fb[2][NQ];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        fa[t][q] = gemm_fragment<TI, TA, TMR>(&smem[buf][0], wm * 64 + t * 32, q, lane);
-        fb[t][q] = gemm_fragment<TI, TB, TNC>(&smem[buf][ABYTES], wn * 64 + t * 32, q, lane);
+      for (int q = 0; q < NQ; ++q) {
+        fa[t][q] = gemm_fragment<TI, TA, TMR, KB>(&smem[buf][0], wm * 64 + t * 32, q, lane);
+        fb[t][q] = gemm_fragment<TI, TB, TNC, KB>(&smem[buf][ABYTES], wn * 64 + t * 32, q, lane);
       }
     // consecutive MFMAs go to different accumulators: a dependent one would wait for its predecessor to drain
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < NQ; ++q) {
       if constexpr (sizeof(TI) == 2) {
 #pragma unroll
         for (int i = 0; i < 2; ++i)
@@ -1987,7 +1993,7 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
     const dim3 grid_big(static_cast<unsigned>(N / 256), static_cast<unsigned>(M / 256), static_cast<unsigned>(batch));
 #define GEMM_ARGS(TI, TO) static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0, nullptr, 0, 0, 0, 0
 #define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, GEMM_ARGS(TI, TO))
-#define GEMM_SZ(TI, TA, TB) do { if (big) hipLaunchKernelGGL((gemm_kernel<TI, TI, TA, TB, 4, 4>), grid_big, dim3(1024), 0, stream, GEMM_ARGS(TI, TI)); else GEMM_LAUNCH(TI, TI, TA, TB); } while (0)
+#define GEMM_SZ(TI, TA, TB) do { if (big) hipLaunchKernelGGL((gemm_kernel<TI, TI, TA, TB, 4, 4, (sizeof(TI) == 2 ? 128 : 64)>), grid_big, dim3(1024), 0, stream, GEMM_ARGS(TI, TI)); else GEMM_LAUNCH(TI, TI, TA, TB); } while (0)
 #define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_SZ(TI, true, true); else if (trans_a) GEMM_SZ(TI, true, false); else if (trans_b) GEMM_SZ(TI, false, true); else GEMM_SZ(TI, false, false); } while (0)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_TR(float);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t, false, false);
