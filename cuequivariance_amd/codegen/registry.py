@@ -11,6 +11,7 @@ from pathlib import Path
 from .. import cue
 from ..tables import U1dTables
 from . import channelwise as cw
+from . import fullyconnected_rows as fcr
 from . import symmetric as sc
 
 GENERATED_DIR = Path(__file__).resolve().parent.parent / "csrc" / "generated"
@@ -58,6 +59,15 @@ def symmetric_polynomial(irreps_in: str, irreps_out: str, degree: int):
     return e.polynomial.flatten_coefficient_modes().squeeze_modes()
 
 
+def flattened_fully_connected_tables(polynomial) -> U1dTables:
+    """The uniform-1d tables of a fully connected product with a weight row per batch row: every mode but the output's
+    multiplicity flattened away (what ``cuet.operations._FlattenedUniform`` builds at first use)."""
+    q = polynomial.flatten_coefficient_modes()
+    stp = q.operations[0][1]
+    keep = stp.subscripts.operands[-1][-1]
+    return U1dTables.from_polynomial(q.flatten_modes([m for m in stp.subscripts.modes() if m != keep]))
+
+
 def _write(path: Path, src: str, written: list) -> None:
     if not path.exists() or path.read_text() != src:
         path.write_text(src)
@@ -76,6 +86,20 @@ def generate(verbose: bool = False) -> list[Path]:
             _write(GENERATED_DIR / f"sc_{name}_{T}.hip", sc.emit_unit(st, T, name, t.content_hash(code), bwd), written)
             if verbose:
                 print(f"generated sc_{name}_{T}.hip: {len(st.terms)} folded terms")
+    for ir1, ir2, ir3 in FULLY_CONNECTED:
+        # the same products with a weight row per batch row (the convolution layer's per-edge weights)
+        poly = cue.descriptors.fully_connected_tensor_product(cue.Irreps("O3", ir1), cue.Irreps("O3", ir2), cue.Irreps("O3", ir3)).polynomial
+        st = fcr.analyze(poly)
+        if st is None:
+            continue
+        t = flattened_fully_connected_tables(poly)
+        lmax = [max(ir.l for _, ir in cue.Irreps("O3", x)) for x in (ir1, ir2, ir3)]
+        name = f"fcr_{st.U}l{lmax[0]}_l{lmax[1]}_{st.Wd}l{lmax[2]}"
+        for T, code in MATH:
+            _write(GENERATED_DIR / f"{name}_{T}.hip",
+                   fcr.emit_unit(st, T, name, t.content_hash(code), t.backward((True, True, True)).content_hash(code)), written)
+            if verbose:
+                print(f"generated {name}_{T}.hip: {len(st.blocks)} blocks")
     for name, ir1, ir2, filt, tuning in CHANNELWISE:
         t = channelwise_tables(ir1, ir2, filt)
         assert t.operations == (0, 1, 2, 3) and t.buffer_dim == (1, 1, 0, 1)

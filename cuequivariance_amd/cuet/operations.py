@@ -91,7 +91,7 @@ class _FlattenedUniform(torch.nn.Module):
             extents = sorted(q.operations[0][1].get_dims(keep))
             if len(extents) > 1:
                 q = q.split_mode(keep, math.gcd(*extents))
-            self.f = SegmentedPolynomial(q, method="uniform_1d", math_dtype=self._math_dtype)
+            self.f = SegmentedPolynomial(q, method="uniform_1d", math_dtype=self._math_dtype, options={"origin": self._polynomial})
         return self.f(inputs, input_indices=input_indices or {}, output_shapes=output_shapes or {},
                       output_indices=output_indices or {})
 

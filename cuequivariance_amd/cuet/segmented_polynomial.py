@@ -119,6 +119,7 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
         self._plans: dict = {dt: u1d.Uniform1dPlan(self.tables, dt, name=self.name) for dt in (torch.float32, torch.float64)}
         for plan in self._plans.values():
             plan.polynomial = polynomial  # (lets kernels for symmetric contractions be generated at first use)
+            plan.origin = (options or {}).get("origin")  # (the descriptor a flattened fully connected product came from)
 
     def __reduce__(self):
         return (

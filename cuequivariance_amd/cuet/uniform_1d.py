@@ -76,6 +76,7 @@ class Uniform1dPlan:
         self._choice: dict = {}
         self.jit_root = None  # for a backward plan: the forward plan, whose translation unit holds its kernels
         self.polynomial = None  # the flattened polynomial the tables came from, when the caller has it
+        self.origin = None      # the polynomial that one was flattened from (a fully connected product's descriptor)
         self._lock = threading.Lock()
         # small integer under which a traced graph (torch.compile / export) names this plan
         with _traced_lock:
@@ -113,7 +114,7 @@ class Uniform1dPlan:
             lib = _lib.load()
             if _jit.enabled():  # kernels generated for this descriptor at first use (off by default)
                 root = self.jit_root or self
-                _jit.ensure_plan(self.tables, _DTYPE_CODE[self.math_dtype], root.tables, root.polynomial)
+                _jit.ensure_plan(self.tables, _DTYPE_CODE[self.math_dtype], root.tables, root.polynomial, root.origin)
             desc, keep = _lib.make_desc(self.tables, _DTYPE_CODE[self.math_dtype])
             out = C.c_void_p()
             with torch.cuda.device(idx):
@@ -165,7 +166,7 @@ def _backward_choice(plan: Uniform1dPlan, needs: tuple, device: torch.device) ->
         if not all(needs) and device.type == "cuda":
             everything = (True,) * len(needs)
             full = plan.backward_plan(everything)
-            if _jit.is_channelwise(plan.tables):
+            if _jit.has_fused_backward(plan.tables, plan.polynomial, plan.origin):
                 # the fused backward of the family reads every operand once for all three gradients: preferred over a
                 # unit per gradient from the general generator
                 if full.specialised(device):

@@ -131,17 +131,39 @@ def is_symmetric_contraction(poly) -> bool:
     return True
 
 
-def _family(t: U1dTables, polynomial=None) -> Optional[str]:
+def is_row_weight_fully_connected(t: U1dTables, origin) -> bool:
+    """Tables flattened from a fully connected product ``origin`` (``uvw,iu,jv,kw+ijk``, second operand of multiplicity one,
+    one multiplicity per operand) - the form ``codegen/fullyconnected_rows.py`` generates kernels for when every batch row
+    brings its own weights."""
+    from .codegen import fullyconnected_rows as fcr
+
+    if origin is None or t.layouts or t.num_inputs != 3 or t.num_outputs != 1 or tuple(t.buffer_dim) != (1, 0, 0, 1):
+        return False
+    st = fcr.analyze(origin)
+    return (st is not None and t.operand_extent == st.Wd and
+            list(t.buffer_num_segments) == [st.width_w // st.Wd, st.width_x1, st.width_x2, st.width_out // st.Wd])
+
+
+def _family(t: U1dTables, polynomial=None, origin=None) -> Optional[str]:
     """The family generator that serves these tables: "channelwise" (which addresses x1 and the output through their
-    layouts), "symmetric" (default layouts only) or None."""
+    layouts), "symmetric" (default layouts only), "fc_rows" (a fully connected product with a weight row per batch row;
+    ``origin`` is the polynomial the tables were flattened from) or None."""
     if is_channelwise(t) and not t.layout(0) and not t.layout(2):
         return "channelwise"
     if not t.layouts and is_symmetric_contraction(polynomial):
         return "symmetric"
+    if is_row_weight_fully_connected(t, origin):
+        return "fc_rows"
     return None
 
 
-def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTables] = None, root_polynomial=None) -> bool:
+def has_fused_backward(t: U1dTables, polynomial=None, origin=None) -> bool:
+    """Families whose unit computes every gradient in one pass over the operands (preferred over a kernel per gradient)."""
+    return _family(t, polynomial, origin) in ("channelwise", "fc_rows")
+
+
+def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTables] = None, root_polynomial=None,
+                root_origin=None) -> bool:
     """Kernels for one plan: first the family unit of its root (the forward plan of a channel-wise product or symmetric
     contraction holds the kernels of its backward plans too), then, if the plan still has none, a unit of its own from
     the general generator (``codegen/general.py``: second derivatives, harmonics, flattened dense products, ...)."""
@@ -149,14 +171,14 @@ def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTabl
         return True
     if not enabled():
         return False
-    if root_tables is not None and _family(root_tables, root_polynomial):
-        ensure_specialised(root_tables, math_code, root_polynomial)
+    if root_tables is not None and _family(root_tables, root_polynomial, root_origin):
+        ensure_specialised(root_tables, math_code, root_polynomial, origin=root_origin)
         if _has_spec(tables, math_code):
             return True
     return ensure_specialised(tables, math_code, None, general=True)
 
 
-def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, general: bool = False) -> bool:
+def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, general: bool = False, origin=None) -> bool:
     """Make sure specialised kernels for ``tables`` (forward) and for its backward are registered with the library,
     compiling them if this module is enabled and the descriptor is a channel-wise product or (given the flattened
     ``polynomial`` the tables came from) a symmetric contraction - or, with ``general``, anything the general generator
@@ -165,7 +187,7 @@ def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, gener
 
     if _has_spec(tables, math_code):
         return True
-    family = _family(tables, polynomial)
+    family = _family(tables, polynomial, origin)
     if not enabled() or not (family or (general and gen.supported(tables))):
         return False
     key = tables.content_hash(math_code)
@@ -175,7 +197,7 @@ def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, gener
         if key in _failed:
             return False
         try:
-            _loaded[key] = _build_and_load(tables, math_code, key, polynomial)
+            _loaded[key] = _build_and_load(tables, math_code, key, polynomial, origin)
         except Exception as e:  # compilation is an optimisation: the table-driven kernels still serve the plan
             _failed.add(key)
             print(f"[cueq_amd.jit] specialised kernels for descriptor {key:016x} not built: {e}", file=sys.stderr, flush=True)
@@ -183,14 +205,14 @@ def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, gener
     return _has_spec(tables, math_code)
 
 
-def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None):
+def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None, origin=None):
     from .codegen import channelwise as cw
     from .codegen import symmetric as sc
 
     T = "float" if code == _lib.F32 else "double"
     name = f"jit_{key:016x}"
     # the object's name carries a hash of the emitted source, so a changed generator (or tuning) never meets a stale object
-    family = _family(t, polynomial)
+    family = _family(t, polynomial, origin)
     if family is None:
         from .codegen import general as gen
 
@@ -202,6 +224,12 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None):
         tb = t.backward((True, True, True))
         src = cw.emit_unit(st, T, name, key, tb.content_hash(code), **_tuning(st, T))
         what = f"{st.num_paths} paths, extent {st.extent}"
+    elif family == "fc_rows":
+        from .codegen import fullyconnected_rows as fcr
+
+        st = fcr.analyze(origin)
+        src = fcr.emit_unit(st, T, name, key, t.backward((True, True, True)).content_hash(code))
+        what = f"fully connected, weights per row, {len(st.blocks)} blocks, U = {st.U}, W = {st.Wd}"
     else:
         st = sc.analyze(polynomial)
         bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
