@@ -212,6 +212,34 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = ("configs[3]: FullyConnectedTensorProduct 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, batch 50000, shared weights, "
                 "fwd + bwd (dw, dx1, dx2)")
+    elif wl == "fcconv":
+        # the product inside FullyConnectedTensorProductConv: a weight row per edge, x1 gathered by source, output summed by
+        # destination (no BASELINE config; sizes chosen here)
+        E, N = 20_000, 2_000
+        i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e")
+        m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, shared_weights=False, internal_weights=False,
+                                             device=dev, dtype=torch.float32)
+        g = torch.Generator(device=dev).manual_seed(0)
+        x1 = torch.randn(N, i1.dim, device=dev, generator=g, requires_grad=True)
+        x2 = torch.randn(E, i2.dim, device=dev, generator=g, requires_grad=True)
+        w = torch.randn(E, m.weight_numel, device=dev, generator=g, requires_grad=True)
+        snd = torch.randint(0, N, (E,), device=dev, generator=g, dtype=torch.int32)
+        rcv = torch.sort(torch.randint(0, N, (E,), device=dev, generator=g, dtype=torch.int32))[0]
+        cot = torch.randn(N, i1.dim, device=dev, generator=g)
+
+        def step():
+            return torch.autograd.grad(m(x1, x2, w, indices_1=snd, indices_out=rcv, size_out=N), [x1, x2, w], cot)
+
+        unit, units, dt = "edges/s", E, "f32"
+        W = m.weight_numel
+        # every distinct element once: fwd reads w, x2, x1, two index arrays and writes out; bwd reads w, x2, x1, g and writes dw, dx2, dx1
+        alg = {"fwd": (E * (W + 9) + 2 * N * 256) * 4 + 2 * E * 4, "bwd": (2 * E * (W + 9) + 3 * N * 256) * 4 + 2 * E * 4}
+        # per weight: forward 2 (2 l3 + 1) / block flops, backward twice that (weight gradient and R)
+        f = 2 * E * 64 * 64 * 11
+        flops = {"fwd": f, "bwd": 2 * f}
+        flop_roof, flop_peak = "valu", VALU_PEAK_F32
+        desc = ("next row (FullyConnectedTensorProductConv's product): 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, a weight row per edge, "
+                "20000 edges, 2000 nodes, x1 gathered by source, output summed by destination, fwd + bwd (dw, dx1, dx2)")
     elif wl == "cfg5":
         dtype = torch.float32 if dtype_name == "fp32" else torch.bfloat16
         n, D = 512, 128
@@ -282,7 +310,8 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
                      "algorithmic_bytes": roofs["algorithmic_bytes"], "flops": roofs["flops"],
                      "scope": "whole step: algorithmic bytes and flops of forward + backward over the step time, against 8 TB/s and the "
                               f"{flop_roof} peak ({flop_peak} TFLOP/s); bound = the roof with the longer minimum time"
-                              + ("; flops = executed vector instructions x 128, " + VALU_SOURCE if flop_roof == "valu" else "")},
+                              + ("; flops = 2 (2 l3 + 1) per weight, forward once and backward twice (algorithmic)" if wl == "fcconv" else
+                                 "; flops = executed vector instructions x 128, " + VALU_SOURCE if flop_roof == "valu" else "")},
         "kernels": kernels,
     }
 
@@ -462,7 +491,7 @@ def main() -> int:
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
     ap.add_argument("--graph", action="store_true",
                     help="secondary workloads only: capture the step into a HIP graph and time its replays")
-    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4fc", "cfg5"], default=None,
+    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4fc", "fcconv", "cfg5"], default=None,
                     help="default: the headline metric (cfg2, fp32) with every other configuration in a 'secondary' object.  "
                          "Naming a workload prints one line for it alone: cfg2 the headline, cfg1 the reference's CPU-sized "
                          "channel-wise case, cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected "
@@ -539,7 +568,7 @@ def main() -> int:
         add("cfg2_fp32_ordered_dx1", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float32, N, E, ssteps, swarm, True)[0]))
         add("cfg2_fp64", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float64, N, E, ssteps, swarm, False)[0]))
         for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg4_linear_fp32", "cfg4", "fp32"),
-                            ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"),
+                            ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"),
                             ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp32", "cfg5", "fp32")):
             add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))
         if not args.no_cpu_baseline:

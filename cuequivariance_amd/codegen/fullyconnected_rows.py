@@ -25,6 +25,9 @@ from dataclasses import dataclass, field
 from typing import List, Optional, Tuple
 
 
+MAX_GROUP = 16
+
+
 @dataclass
 class Block:
     w_off: int          # element offset of the (U x Wd) weight block in a weight row
@@ -114,7 +117,7 @@ def emit_unit(st: RowWeightStructure, T: str, name: str, fwd_hash: int, bwd_hash
     nout = st.width_out // Wd       # output components (each a vector over w)
     n2 = st.width_x2
     TS = 65                         # row stride of the LDS tile in elements: column reads touch every bank once
-    G = next(n for n in (16, 8, 4, 2, 1) if U % n == 0)  # weight rows requested together, one group ahead of their use
+    G = next(n for n in (32, 16, 8, 4, 2, 1) if n <= MAX_GROUP and U % n == 0)  # weight rows requested together, one group ahead of their use
     waves = 2 if T == "float" else 1
     L: List[str] = []
     A = L.append
@@ -139,19 +142,22 @@ def emit_unit(st: RowWeightStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("")
 
     # ------------------------------------------------------------------ forward
-    A("// forward: one wavefront per output row; its batch rows are summed in list order")
+    A("// forward: `parts` wavefronts per output row, each sums a contiguous piece of the row's batch rows in list order (one")
+    A("// wavefront per row when there are enough rows to fill the chip; else the pieces go to partial rows, folded in order)")
     A("template <bool X1_IDX>")
     A(f"__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu({waves}))) fwd_kernel(")
     A(f"    const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}* __restrict__ x2, {T}* __restrict__ out,")
-    A("    const void* __restrict__ x1_index, int x1_idx64, const int64_t* __restrict__ csr_offsets, const int64_t* __restrict__ csr_perm) {")
+    A("    const void* __restrict__ x1_index, int x1_idx64, const int64_t* __restrict__ csr_offsets, const int64_t* __restrict__ csr_perm, int parts) {")
     A("  const int lane = threadIdx.x;")
-    A("  const int64_t r = blockIdx.x;")
+    A("  const int64_t r = blockIdx.x / parts;")
+    A("  const int part = static_cast<int>(blockIdx.x - r * parts);")
     A(f"  const bool act_u = lane < {U}, act_w = lane < {Wd};")
     A(f"  const int lu = act_u ? lane : 0, lw = act_w ? lane : 0;")
     for k in range(nout):
         A(f"  {T} acc{k} = 0;")
     A("  int64_t z0, z1;")
     A("  if (csr_offsets) { z0 = csr_offsets[r]; z1 = csr_offsets[r + 1]; } else { z0 = r; z1 = r + 1; }")
+    A("  { const int64_t n = z1 - z0; z1 = z0 + n * (part + 1) / parts; z0 = z0 + n * part / parts; }")
     A("  for (int64_t zz = z0; zz < z1; ++zz) {")
     A("    const int64_t z = csr_perm ? csr_perm[zz] : zz;")
     A("    int64_t srow = z;")
@@ -184,7 +190,7 @@ def emit_unit(st: RowWeightStructure, T: str, name: str, fwd_hash: int, bwd_hash
             for k in sorted(S):
                 A(f"    acc{blk.c_off // Wd + k} = fma(wq{gi & 1}_{r}, lane_value(S{b}_{k}, {g0 + r}), acc{blk.c_off // Wd + k});")
     A("  }")
-    A(f"  {T}* __restrict__ op = out + r * {st.width_out}ll + lw;")
+    A(f"  {T}* __restrict__ op = out + static_cast<int64_t>(blockIdx.x) * {st.width_out}ll + lw;  // (out = the partial rows when parts > 1)")
     A("  if (act_w) {")
     for k in range(nout):
         A(f"    STREAM_STORE(acc{k}, op + {k * Wd});")
@@ -300,6 +306,20 @@ static bool all_dtype(const cueq_u1d_buffer* b, int n) {{
 }}
 
 // buffers: w, x1, x2 | out
+// wavefronts per output row: one when the rows fill the chip about three times over, else up to 8 pieces per row - but
+// no more pieces than a row has batch rows on average
+static int fwd_parts(const cueq_u1d_buffer* b, int64_t batch) {{
+  if (b[3].batch_dim != CUEQ_BATCH_INDEXED || b[3].rows <= 0) return 1;
+  const int64_t want = (3 * wave_slots({waves}) + b[3].rows - 1) / b[3].rows, mean = batch / b[3].rows;
+  int64_t p = want < mean ? want : mean;
+  if (p > 8) p = 8;
+  return p < 1 ? 1 : static_cast<int>(p);
+}}
+static int64_t fwd_workspace(const cueq_u1d_buffer* b, int64_t batch) {{
+  const int parts = fwd_parts(b, batch);
+  return parts > 1 ? b[3].rows * parts * {st.width_out}ll * sizeof({T}) : 0;
+}}
+
 static int run_fwd(const SpecCall& c) {{
   const cueq_u1d_buffer* b = c.buffers;
   if (!all_dtype(b, 4)) return CUEQ_ERR_UNSUPPORTED;
@@ -309,18 +329,28 @@ static int run_fwd(const SpecCall& c) {{
   if (out_idx && (!b[3].csr_offsets || (!b[3].csr_perm && c.batch > 0))) return CUEQ_ERR_UNSUPPORTED;
   const int64_t rows = b[3].rows;
   if (rows == 0) return CUEQ_OK;
-  CUEQ_REQUIRE(rows < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "too many output rows for one launch");
+  const int parts = fwd_parts(b, c.batch);
+  CUEQ_REQUIRE(rows * parts < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "too many output rows for one launch");
+  const int64_t need = fwd_workspace(b, c.batch);
+  CUEQ_REQUIRE(need == 0 || (c.workspace && c.workspace_bytes >= need), CUEQ_ERR_INVALID, "workspace too small: need %lld bytes", (long long)need);
   const {T}* w = static_cast<const {T}*>(b[0].data);
   const {T}* x1 = static_cast<const {T}*>(b[1].data);
   const {T}* x2 = static_cast<const {T}*>(b[2].data);
   {T}* o = static_cast<{T}*>(b[3].data);
   const int64_t* offs = out_idx ? b[3].csr_offsets : nullptr;
   const int64_t* perm = out_idx ? b[3].csr_perm : nullptr;
-  const dim3 g(static_cast<unsigned>(rows)), t(64);
-  KernelTimer timer("{name}_fwd_{T}", c.stream);
-  if (x1_idx) hipLaunchKernelGGL((fwd_kernel<true>), g, t, 0, c.stream, w, x1, x2, o, b[1].index, b[1].index_is_64, offs, perm);
-  else hipLaunchKernelGGL((fwd_kernel<false>), g, t, 0, c.stream, w, x1, x2, o, b[1].index, b[1].index_is_64, offs, perm);
+  const dim3 g(static_cast<unsigned>(rows * parts)), t(64);
+  {T}* dst = parts > 1 ? static_cast<{T}*>(c.workspace) : o;
+  {{
+    KernelTimer timer("{name}_fwd_{T}", c.stream);
+    if (x1_idx) hipLaunchKernelGGL((fwd_kernel<true>), g, t, 0, c.stream, w, x1, x2, dst, b[1].index, b[1].index_is_64, offs, perm, parts);
+    else hipLaunchKernelGGL((fwd_kernel<false>), g, t, 0, c.stream, w, x1, x2, dst, b[1].index, b[1].index_is_64, offs, perm, parts);
+  }}
   CUEQ_CHECK_HIP(hipGetLastError());
+  if (parts > 1) {{
+    hipLaunchKernelGGL(fold_parts<{T}>, dim3(blocks_for(rows * {st.width_out}ll)), dim3(256), 0, c.stream, dst, rows, parts, {st.width_out}, o);
+    CUEQ_CHECK_HIP(hipGetLastError());
+  }}
   return CUEQ_OK;
 }}
 
@@ -391,7 +421,7 @@ static int run_bwd(const SpecCall& c) {{
   return CUEQ_OK;
 }}
 
-static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{T}", run_fwd, nullptr}};
+static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{T}", run_fwd, fwd_workspace}};
 static const U1dSpec spec_bwd = {{0x{bwd_hash:016x}ull, "{name}_bwd_{T}", run_bwd, bwd_workspace}};
 static SpecRegistrar reg_fwd(&spec_fwd);
 static SpecRegistrar reg_bwd(&spec_bwd);
