@@ -33,6 +33,9 @@ SYMMETRIC = [
     ("s32_l2", "32x0e+32x1o+32x2e", "32x0e+32x1o", 3),
 ]
 
+# Symmetric contractions also generated for x and the output in the mul_ir layout; unit "<name>_mulir".
+SYMMETRIC_MUL_IR = ["s128_l3"]
+
 # Fully connected products (shared weights) whose fused kernels are compiled when the library is built, into
 # cuequivariance_amd/prebuilt/: (irreps_in1, irreps_in2, irreps_out), float and bfloat16.  Others are compiled at first use.
 FULLY_CONNECTED = [
@@ -79,13 +82,17 @@ def generate(verbose: bool = False) -> list[Path]:
     written = []
     for name, irreps_in, irreps_out, degree in SYMMETRIC:
         poly = symmetric_polynomial(irreps_in, irreps_out, degree)
-        t = U1dTables.from_polynomial(poly)
-        st = sc.analyze(poly)
-        for T, code in MATH:
-            bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
-            _write(GENERATED_DIR / f"sc_{name}_{T}.hip", sc.emit_unit(st, T, name, t.content_hash(code), bwd), written)
-            if verbose:
-                print(f"generated sc_{name}_{T}.hip: {len(st.terms)} folded terms")
+        variants = [(name, U1dTables.from_polynomial(poly))]
+        if name in SYMMETRIC_MUL_IR:  # buffers: w, x | out
+            groups = {1: [ir.dim for _, ir in cue.Irreps("O3", irreps_in)], 2: [ir.dim for _, ir in cue.Irreps("O3", irreps_out)]}
+            variants.append((name + "_mulir", variants[0][1].with_layouts(groups)))
+        for vname, t in variants:
+            st = sc.analyze(poly, t.layout(1), t.layout(2))
+            for T, code in MATH:
+                bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
+                _write(GENERATED_DIR / f"sc_{vname}_{T}.hip", sc.emit_unit(st, T, vname, t.content_hash(code), bwd), written)
+                if verbose:
+                    print(f"generated sc_{vname}_{T}.hip: {len(st.terms)} folded terms")
     for ir1, ir2, ir3 in FULLY_CONNECTED:
         # the same products with a weight row per batch row (the convolution layer's per-edge weights)
         poly = cue.descriptors.fully_connected_tensor_product(cue.Irreps("O3", ir1), cue.Irreps("O3", ir2), cue.Irreps("O3", ir3)).polynomial

@@ -34,14 +34,45 @@ class SymmetricStructure:
     nseg_x: int
     nseg_out: int
     terms: list  # (weight segment, tuple of sorted x segments, output segment, coefficient)
+    layout_x: tuple = ()    # groups of x segments stored channel-major (``U1dTables.layouts``), () = segment-major rows
+    layout_out: tuple = ()  # the same for the output rows
+
+    def _at(self, layout: tuple, seg: int) -> str:
+        """Element (segment ``seg``, channel ``uu``) of a row under ``layout``, as a C expression."""
+        if not layout:
+            return f"{seg * self.extent} + uu"
+        first = 0
+        for d in layout:
+            if seg < first + d:
+                return f"{first * self.extent + (seg - first)} + uu" + (f" * {d}" if d > 1 else "")
+            first += d
+        raise ValueError(f"segment {seg} outside the layout {layout}")
+
+    def x_at(self, a: int) -> str:
+        return self._at(self.layout_x, a)
+
+    @staticmethod
+    def _staged(layout: tuple) -> dict:
+        """{segment: (first segment of its group, group size, position in the group)} for groups of more than one segment."""
+        out, first = {}, 0
+        for d in layout:
+            if d > 1:
+                for c in range(d):
+                    out[first + c] = (first, d, c)
+            first += d
+        return out
+
+    def out_at(self, k: int) -> str:
+        return self._at(self.layout_out, k)
 
     @property
     def degree(self) -> int:
         return max(len(t[1]) for t in self.terms)
 
 
-def analyze(poly) -> SymmetricStructure:
-    """``poly``: the SegmentedPolynomial of a symmetric contraction (modes flattened, ``u`` uniform)."""
+def analyze(poly, layout_x: tuple = (), layout_out: tuple = ()) -> SymmetricStructure:
+    """``poly``: the SegmentedPolynomial of a symmetric contraction (modes flattened, ``u`` uniform); the layouts are those
+    of the x and output buffers of its tables."""
     assert poly.num_inputs == 2 and poly.num_outputs == 1
     folded = poly.unsymmetrize_for_identical_operands()
     w, x = folded.inputs
@@ -56,7 +87,7 @@ def analyze(poly) -> SymmetricStructure:
             c = float(path.coefficients)
             if c != 0.0:
                 terms.append((path.indices[0], tuple(sorted(path.indices[1:-1])), path.indices[-1], c))
-    return SymmetricStructure(extent, w.num_segments, x.num_segments, out.num_segments, terms)
+    return SymmetricStructure(extent, w.num_segments, x.num_segments, out.num_segments, terms, tuple(layout_x), tuple(layout_out))
 
 
 def _groups(st: SymmetricStructure):
@@ -97,6 +128,85 @@ def _poly_expr(terms, T: str) -> list[str]:
     return lines
 
 
+# A channel-major group of d segments is a contiguous piece of 64 d elements per wavefront.  Lanes that each walk their own
+# d elements make every load or store instruction touch d times the cache lines it uses, which the address units pay for in
+# full; so the piece moves as d unit-stride instructions and crosses the lanes through LDS (lane * d + c <-> k * 64 + lane:
+# conflict-free for odd d).  `stage` is private to the wavefront, whose LDS operations execute in program order.
+def _piece(st: SymmetricStructure, first: int, d: int, k: int) -> str:
+    return f"{first * st.extent} + ch * {64 * d} + {k * 64} + lane"
+
+
+def _piece_ok(st: SymmetricStructure, d: int, k: int) -> str:
+    return "" if st.extent % 64 == 0 else f"(ch * {64 * d} + {k * 64} + lane < {st.extent * d})"
+
+
+def _row_request(A, ind: str, st: SymmetricStructure, T: str, layout: tuple, segs, ptr: str, dst: str, declare: bool):
+    """Loads of the segments `segs` of a row into `dst<seg>`: the value itself for unit-stride segments, for a segment of a
+    channel-major group the k-th unit-stride piece of its group (to be unpacked by `_row_unpack`)."""
+    staged = st._staged(layout)
+    decl = f"const {T} " if declare else ""
+    for a in segs:
+        if a in staged:
+            first, d, k = staged[a]
+            ok = _piece_ok(st, d, k)
+            load = f"__builtin_nontemporal_load({ptr} + {_piece(st, first, d, k)})"
+            A(f"{ind}{decl}{dst}{a} = " + (f"{ok} ? {load} : {T}(0);" if ok else f"{load};"))
+        else:
+            A(f"{ind}{decl}{dst}{a} = __builtin_nontemporal_load({ptr} + {a * st.extent} + uu);")
+
+
+def _row_unpack(A, ind: str, st: SymmetricStructure, T: str, layout: tuple, segs, src: str, dst: str):
+    """`dst<seg>` = the value of segment `seg` for this lane's channel, from what `_row_request` loaded into `src<seg>`."""
+    staged = st._staged(layout)
+    done = set()
+    for a in segs:
+        if a not in staged:
+            A(f"{ind}const {T} {dst}{a} = {src}{a};")
+            continue
+        first, d, _ = staged[a]
+        if first in done:
+            continue
+        done.add(first)
+        for k in range(d):
+            A(f"{ind}stage[{k * 64} + lane] = {src}{first + k};")
+        A(f"{ind}__builtin_amdgcn_wave_barrier();")
+        for c in range(d):
+            A(f"{ind}const {T} {dst}{first + c} = stage[lane * {d} + {c}];")
+        A(f"{ind}__builtin_amdgcn_wave_barrier();")
+
+
+def _row_store(A, ind: str, st: SymmetricStructure, T: str, layout: tuple, nseg: int, ptr: str, value):
+    """Stores of a whole row; `value(seg)` is the expression of this lane's element of segment `seg`."""
+    staged = st._staged(layout)
+    done = set()
+    for a in range(nseg):
+        if a not in staged:
+            A(f"{ind}if (active) __builtin_nontemporal_store({value(a)}, {ptr} + {a * st.extent} + uu);")
+            continue
+        first, d, _ = staged[a]
+        if first in done:
+            continue
+        done.add(first)
+        for c in range(d):
+            A(f"{ind}stage[lane * {d} + {c}] = {value(first + c)};")
+        A(f"{ind}__builtin_amdgcn_wave_barrier();")
+        for k in range(d):
+            ok = _piece_ok(st, d, k)
+            A(f"{ind}" + (f"if {ok} " if ok else "") + f"__builtin_nontemporal_store(stage[{k * 64} + lane], {ptr} + {_piece(st, first, d, k)});")
+        A(f"{ind}__builtin_amdgcn_wave_barrier();")
+
+
+def _whole_groups(layout: tuple, segs, nseg: int):
+    """`segs` widened so that every channel-major group it meets is complete."""
+    staged = SymmetricStructure._staged(layout)
+    out = set(segs)
+    for a in segs:
+        if a in staged:
+            first, d, _ = staged[a]
+            out.update(range(first, first + d))
+    return sorted(out)
+
+
 def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hashes: dict, *, fwd_waves: int = 4,
               bwd_waves: int = 2, fwd_prefetch: bool = None) -> str:
     """Complete translation unit.  ``bwd_hashes``: {(need_dw, need_dx): table hash}."""
@@ -110,12 +220,16 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     groups = _groups(st)
     pairs = _pairs(st)
     x_used = sorted({a for _, xs, _, _ in st.terms for a in xs})
+    x_read = _whole_groups(st.layout_x, x_used, st.nseg_x)   # (a group is loaded whole, as its unit-stride pieces)
     w_used = sorted({s for s, _, _, _ in st.terms})
+    dmax = max([d for d in tuple(st.layout_x) + tuple(st.layout_out) if d > 1], default=0)
+    stage_decl = f"  __shared__ {T} stage[{64 * dmax}];" if dmax else None
     L = []
     A = L.append
     A("// GENERATED by cuequivariance_amd/codegen/symmetric.py - do not edit.")
     A(f"// symmetric contraction '{name}': extent {E}, segments w/x/out = {st.nseg_w}/{st.nseg_x}/{st.nseg_out}, "
-      f"{len(st.terms)} folded terms in {len(groups)} (weight, output) groups, math {T}")
+      f"{len(st.terms)} folded terms in {len(groups)} (weight, output) groups, math {T}"
+      + (f", x rows in groups {list(st.layout_x)}" if st.layout_x else "") + (f", output rows in groups {list(st.layout_out)}" if st.layout_out else ""))
     A('#include "cw_common.h"')
     A("")
     A("namespace cueq {")
@@ -134,6 +248,8 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("  const int lane = threadIdx.x;")
     A(f"  const int ch = blockIdx.x % {nch}; const int64_t slot = blockIdx.x / {nch}; const int64_t nslots = gridDim.x / {nch};")
     A(lane_setup)
+    if stage_decl:
+        A(stage_decl)
     A("  const int64_t z0 = slot * batch / nslots, z1 = (slot + 1) * batch / nslots;")
     if fwd_prefetch:
         # the x row (and the weight index) of the next batch row are requested before the arithmetic of the current one; the
@@ -141,26 +257,23 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
         A("  if (z0 >= z1) return;")
         A("  int64_t wrow_n = W_MODE == 0 ? z0 : 0;")
         A("  if (W_MODE == 1) wrow_n = load_index(w_index, idx64, z0);")
-        A(f"  {T} " + ", ".join(f"xn{a}" for a in x_used) + ";")
+        A(f"  {T} " + ", ".join(f"xn{a}" for a in x_read) + ";")
         A("  {")
         A(f"    const {T}* __restrict__ xp = x + z0 * {X}ll;")
-        for a in x_used:
-            A(f"    xn{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
+        _row_request(A, "    ", st, T, st.layout_x, x_read, "xp", "xn", False)
         A("  }")
         A("  for (int64_t z = z0; z < z1; ++z) {")
         A("    const int64_t wrow = wrow_n;")
         A(f"    const {T}* __restrict__ wp = w + wrow * {W}ll;")
         for s in w_used:
             A(f"    const {T} wv{s} = wp[{s * E} + uu];")
-        for a in x_used:
-            A(f"    const {T} xv{a} = xn{a};")
+        _row_unpack(A, "    ", st, T, st.layout_x, x_read, "xn", "xv")
         A("    {")
         A("      const int64_t zn = z + 1 < z1 ? z + 1 : z;")
         A("      wrow_n = W_MODE == 0 ? zn : 0;")
         A("      if (W_MODE == 1) wrow_n = load_index(w_index, idx64, zn);")
         A(f"      const {T}* __restrict__ xp = x + zn * {X}ll;")
-        for a in x_used:
-            A(f"      xn{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
+        _row_request(A, "      ", st, T, st.layout_x, x_read, "xp", "xn", False)
         A("    }")
         A("    __builtin_amdgcn_sched_barrier(0);")
     else:
@@ -169,10 +282,10 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
         A("    if (W_MODE == 1) wrow = load_index(w_index, idx64, z);")
         A(f"    const {T}* __restrict__ xp = x + z * {X}ll;")
         A(f"    const {T}* __restrict__ wp = w + wrow * {W}ll;")
-        for a in x_used:
-            A(f"    const {T} xv{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
+        _row_request(A, "    ", st, T, st.layout_x, x_read, "xp", "xr", True)
         for s in w_used:
             A(f"    const {T} wv{s} = wp[{s * E} + uu];")
+        _row_unpack(A, "    ", st, T, st.layout_x, x_read, "xr", "xv")
     for a, b in pairs:
         A(f"    const {T} pp_{a}_{b} = xv{a} * xv{b};")
     for k in range(st.nseg_out):
@@ -183,10 +296,9 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
             A("      " + ln)
         A(f"      acc{k} = fma(wv{s}, P, acc{k});")
         A("    }")
-    A("    if (active) {")
+    A("    {")
     A(f"      {T}* __restrict__ op = out + z * {O}ll;")
-    for k in range(st.nseg_out):
-        A(f"      __builtin_nontemporal_store(acc{k}, op + {k * E} + uu);")
+    _row_store(A, "      ", st, T, st.layout_out, st.nseg_out, "op", lambda k: f"acc{k}")
     A("    }")
     A("  }")
     A("}")
@@ -201,6 +313,8 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("  const int lane = threadIdx.x;")
     A(f"  const int ch = blockIdx.x % {nch}; const int64_t slot = blockIdx.x / {nch}; const int64_t nslots = gridDim.x / {nch};")
     A(lane_setup)
+    if stage_decl:
+        A(stage_decl)
     A("  const int64_t p0 = slot * batch / nslots, p1 = (slot + 1) * batch / nslots;")
     A("  if (p0 >= p1) return;")
     for s in w_used:
@@ -231,10 +345,10 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("    }")
     A(f"    const {T}* __restrict__ xp = x + z * {X}ll;")
     A(f"    const {T}* __restrict__ gp = g + z * {O}ll;")
-    for a in x_used:
-        A(f"    const {T} xv{a} = __builtin_nontemporal_load(xp + {a * E} + uu);")
-    for k in range(st.nseg_out):
-        A(f"    const {T} gv{k} = __builtin_nontemporal_load(gp + {k * E} + uu);")
+    _row_request(A, "    ", st, T, st.layout_x, x_read, "xp", "xr", True)
+    _row_request(A, "    ", st, T, st.layout_out, range(st.nseg_out), "gp", "gr", True)
+    _row_unpack(A, "    ", st, T, st.layout_x, x_read, "xr", "xv")
+    _row_unpack(A, "    ", st, T, st.layout_out, range(st.nseg_out), "gr", "gv")
     for a, b in pairs:
         A(f"    const {T} pp_{a}_{b} = xv{a} * xv{b};")
     for a in x_used:
@@ -269,10 +383,9 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
             A(f"        dxa{v} = fma(wg, {expr}, dxa{v});")
         A("      }")
         A("    }")
-    A("    if (NEED_DX && active) {")
+    A("    if (NEED_DX) {")
     A(f"      {T}* __restrict__ dp = dx + z * {X}ll;")
-    for a in range(st.nseg_x):
-        A(f"      __builtin_nontemporal_store(" + (f"dxa{a}" if a in x_used else f"{T}(0)") + f", dp + {a * E} + uu);")
+    _row_store(A, "      ", st, T, st.layout_x, st.nseg_x, "dp", lambda a: f"dxa{a}" if a in x_used else f"{T}(0)")
     A("    }")
     A("  }")
     A("  flush(true);")

@@ -442,18 +442,27 @@ class SymmetricContraction(torch.nn.Module):
             self.weight_shape = (self.etp.inputs[0].dim // mul, mul)
         self.num_elements = num_elements
         self.weight = torch.nn.Parameter(torch.randn(num_elements, *self.weight_shape, device=device, dtype=dtype))
-        self.transpose_in = TransposeIrrepsLayout(
-            self.etp.inputs[1].irreps, source=_default_layout(layout_in or layout), target=self.etp.inputs[1].layout,
-            device=device,
-        )
-        self.transpose_out = TransposeIrrepsLayout(
-            self.etp.outputs[0].irreps, source=self.etp.outputs[0].layout,
-            target=_default_layout(layout_out or layout), device=device,
-        )
         if method == "uniform_1d" and not self.etp.polynomial.all_same_segment_shape():
             raise ValueError("`uniform_1d` method requires segments to be the same shape")
         self.method = _method_from_fallback(method, use_fallback, "uniform_1d")
-        self.f = SegmentedPolynomial(self.etp.polynomial, method=self.method, math_dtype=math_dtype)
+        source_in, target_out = _default_layout(layout_in or layout), _default_layout(layout_out or layout)
+        # mul_ir rows of x and of the output are addressed as they lie by the uniform-1d kernels (see ChannelWiseTensorProduct)
+        groups = {}
+        if self.method == "uniform_1d":
+            if source_in == cue.mul_ir and self.etp.inputs[1].layout == cue.ir_mul and _transposition_moves(self.etp.inputs[1].irreps):
+                groups[1] = [ir.dim for _, ir in self.etp.inputs[1].irreps]
+                source_in = cue.ir_mul
+            if target_out == cue.mul_ir and self.etp.outputs[0].layout == cue.ir_mul and _transposition_moves(self.etp.outputs[0].irreps):
+                groups[2] = [ir.dim for _, ir in self.etp.outputs[0].irreps]
+                target_out = cue.ir_mul
+        self.transpose_in = TransposeIrrepsLayout(
+            self.etp.inputs[1].irreps, source=source_in, target=self.etp.inputs[1].layout, device=device,
+        )
+        self.transpose_out = TransposeIrrepsLayout(
+            self.etp.outputs[0].irreps, source=self.etp.outputs[0].layout, target=target_out, device=device,
+        )
+        self.f = SegmentedPolynomial(self.etp.polynomial, method=self.method, math_dtype=math_dtype,
+                                     options={"segment_groups": groups} if groups else None)
 
     def extra_repr(self) -> str:
         return f"contraction_degree={self.contraction_degree}, weight_shape={self.weight_shape}"

@@ -146,11 +146,11 @@ def is_row_weight_fully_connected(t: U1dTables, origin) -> bool:
 
 def _family(t: U1dTables, polynomial=None, origin=None) -> Optional[str]:
     """The family generator that serves these tables: "channelwise" (which addresses x1 and the output through their
-    layouts), "symmetric" (default layouts only), "fc_rows" (a fully connected product with a weight row per batch row;
+    layouts), "symmetric" (likewise for x and the output), "fc_rows" (a fully connected product with a weight row per batch row;
     ``origin`` is the polynomial the tables were flattened from) or None."""
     if is_channelwise(t) and not t.layout(0) and not t.layout(2):
         return "channelwise"
-    if not t.layouts and is_symmetric_contraction(polynomial):
+    if not t.layout(0) and is_symmetric_contraction(polynomial):
         return "symmetric"
     if is_row_weight_fully_connected(t, origin):
         return "fc_rows"
@@ -231,7 +231,7 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None, origin=N
         src = fcr.emit_unit(st, T, name, key, t.backward((True, True, True)).content_hash(code))
         what = f"fully connected, weights per row, {len(st.blocks)} blocks, U = {st.U}, W = {st.Wd}"
     else:
-        st = sc.analyze(polynomial)
+        st = sc.analyze(polynomial, t.layout(1), t.layout(2))
         bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
         src = sc.emit_unit(st, T, name, key, bwd)
         what = f"symmetric contraction, {len(st.terms)} folded terms, extent {st.extent}"

@@ -252,3 +252,56 @@ def test_first_use_kernels_mul_ir(device, dtype, ir1, lmax, jit_on):
 def test_first_use_general_units_mul_ir(device, jit_on):
     """Second derivatives with compilation at first use on: units of the general generator on tables with layouts."""
     test_second_derivative_mul_ir(device)
+
+
+# --------------------------------------------------------------------------- symmetric contraction
+def run_symmetric_case(device, irreps_in, irreps_out, degree, nel, Z, dtype, seed):
+    """``SymmetricContraction(layout=mul_ir)`` (x and the output addressed in place) against the oracle in ir_mul."""
+    from cuequivariance_amd import cuet
+    from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
+
+    m = cuet.SymmetricContraction(cue.Irreps("O3", irreps_in), cue.Irreps("O3", irreps_out), degree, nel, layout=cue.mul_ir,
+                                  dtype=dtype, device=device)
+    assert isinstance(m.transpose_in.f, torch.nn.Identity) and isinstance(m.transpose_out.f, torch.nn.Identity)
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(Z, m.irreps_in.dim, dtype=torch.float64, generator=gen).to(dtype)
+    idx = torch.randint(0, nel, (Z,), generator=gen, dtype=torch.int32)
+    w = m.weight.detach().cpu().clone()
+    a = [w.flatten(1).double().requires_grad_(True), x.double().requires_grad_(True)]
+    ref = naive_segmented_polynomial(spec_from_polynomial(m.etp.polynomial), a, {0: idx})[0]
+    cot = torch.randn(ref.shape, dtype=torch.float64, generator=gen).to(dtype)
+    ref_dw, ref_dx = torch.autograd.grad(ref, a, cot.double())
+    xg = to_mul_ir(x, m.irreps_in).to(device).requires_grad_(True)
+    out = m(xg, idx.to(device))
+    dw, dx = torch.autograd.grad(out, [m.weight, xg], to_mul_ir(cot, m.irreps_out).to(device))
+    tol = TOL[dtype]
+    assert_close(out, to_mul_ir(ref, m.irreps_out), tol, "out")
+    assert_close(dw.flatten(1), ref_dw, tol, "dw")
+    assert_close(dx, to_mul_ir(ref_dx, m.irreps_in), tol, "dx")
+    return m
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_symmetric_contraction_cfg3_descriptor_mul_ir(device, dtype):
+    """128 channels, 0e+1o+2e+3o -> 0e+1o, degree 3, 10 element types, 40 nodes: the build's mul_ir unit."""
+    m = run_symmetric_case(device, "128x0e+128x1o+128x2e+128x3o", "128x0e+128x1o", 3, 10, 40, dtype, seed=31)
+    plan = m.f.m._plan(dtype)
+    assert plan.specialised(device) and plan.backward_plan((True, True)).specialised(device)
+    assert tuple(plan.tables.layout(1)) == (1, 3, 5, 7) and tuple(plan.tables.layout(2)) == (1, 3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("first_use", [False, True])
+def test_symmetric_contraction_other_descriptor_mul_ir(device, first_use, tmp_path, monkeypatch):
+    """48 channels, degree 2: the table-driven kernels, and a unit compiled at first use."""
+    from cuequivariance_amd import jit
+
+    if first_use:
+        monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
+        jit.enable(True)
+    try:
+        m = run_symmetric_case(device, "48x0e+48x1o+48x2e", "48x0e+48x1o", 2, 3, 77, torch.float64, seed=32)
+        assert m.f.m._plan(torch.float64).specialised(device) == first_use
+    finally:
+        jit.enable(False)
