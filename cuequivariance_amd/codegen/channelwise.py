@@ -98,6 +98,19 @@ class ChannelwiseStructure:
     # s * extent + u; group sizes (d_0, d_1, ...) = groups of consecutive segments stored channel-major ("mul_ir")
     layout_x1: tuple = ()
     layout_out: tuple = ()
+    # x2 = spherical harmonics of a 3-vector, evaluated in the kernels: per x2 segment its terms
+    # ((sorted indices into the vector, coefficient), ...); () = x2 is read from memory
+    harmonics: tuple = ()
+
+    @property
+    def x2_width(self) -> int:
+        """Elements of a row of the second operand (and of its gradient) in memory."""
+        return 3 if self.harmonics else self.nseg_x2
+
+    @property
+    def monomials(self) -> list:
+        """The distinct monomials (sorted index tuples, the constant first) of the harmonics."""
+        return sorted({vi for terms in self.harmonics for vi, _ in terms}, key=lambda t: (len(t), t))
 
     @property
     def num_paths(self):
@@ -122,7 +135,8 @@ class ChannelwiseStructure:
         return self._at(self.layout_out, k)
 
 
-def analyze(extent: int, nseg: Sequence[int], paths: Sequence[tuple], layout_x1: tuple = (), layout_out: tuple = ()) -> ChannelwiseStructure:
+def analyze(extent: int, nseg: Sequence[int], paths: Sequence[tuple], layout_x1: tuple = (), layout_out: tuple = (),
+            harmonics: tuple = ()) -> ChannelwiseStructure:
     """``paths``: (w_seg, x1_seg, x2_seg, out_seg, coefficient)."""
     blocks: dict[int, Block] = {}
     for b, i, j, k, c in paths:
@@ -132,7 +146,8 @@ def analyze(extent: int, nseg: Sequence[int], paths: Sequence[tuple], layout_x1:
     out = [blocks[b] for b in sorted(blocks)]
     # Order blocks so that blocks reading the same x1 segments are neighbours (register reuse).
     out.sort(key=lambda blk: (blk.i_list, blk.j_list, blk.b))
-    return ChannelwiseStructure(extent, nseg[0], nseg[1], nseg[2], nseg[3], out, tuple(layout_x1), tuple(layout_out))
+    assert not harmonics or len(harmonics) == nseg[2]
+    return ChannelwiseStructure(extent, nseg[0], nseg[1], nseg[2], nseg[3], out, tuple(layout_x1), tuple(layout_out), tuple(harmonics))
 
 
 def _lit(c: float, T: str) -> str:
@@ -140,6 +155,34 @@ def _lit(c: float, T: str) -> str:
     if "e" not in s and "." not in s and "inf" not in s and "nan" not in s:
         s += ".0"
     return s + ("f" if T == "float" else "")
+
+
+def _mono_name(vi: tuple) -> str:
+    return "mo_" + "".join(str(i) for i in vi) if vi else "mo_one"
+
+
+def _emit_monomials(A, ind: str, T: str, monos: Sequence[tuple], v: Sequence[str]):
+    """``const T mo_<indices>`` for every monomial, each from a lower one by one multiplication."""
+    done = set()
+    for vi in sorted(monos, key=lambda t: (len(t), t)):
+        if not vi:
+            A(f"{ind}const {T} mo_one = 1;")
+        elif len(vi) == 1:
+            A(f"{ind}const {T} {_mono_name(vi)} = {v[vi[0]]};")
+        else:
+            if vi[:-1] not in done:  # (a prefix nobody asked for)
+                _emit_monomials(A, ind, T, [vi[:-1]], v)
+                done.add(vi[:-1])
+            A(f"{ind}const {T} {_mono_name(vi)} = {_mono_name(vi[:-1])} * {v[vi[-1]]};")
+        done.add(vi)
+
+
+def _with_prefixes(monos) -> list:
+    out = set()
+    for vi in monos:
+        for n in range(len(vi) + 1):
+            out.add(tuple(vi[:n]))
+    return sorted(out, key=lambda t: (len(t), t))
 
 
 # ---------------------------------------------------------------------------------------------
@@ -230,6 +273,16 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
         A("  " + ", ".join(_lit(c, T) for c in row) + ",")
     A("};")
     A(f"constexpr int kFwdTables = {len(all_tables)};")
+    monos = st.monomials
+    NM = len(monos)
+    if st.harmonics:
+        # lane n16 evaluates Y_(16 m + n16): its coefficients come from LDS, the monomials of the vector are the same in all lanes
+        npad = 16 * ((st.nseg_x2 + 15) // 16)
+        A(f"__device__ const {fp} fwd_shtab[{npad * NM}] = {{")
+        for j in range(npad):
+            row = dict(st.harmonics[j]) if j < st.nseg_x2 else {}
+            A("  " + ", ".join(_lit(row.get(vi, 0.0), T) for vi in monos) + ",")
+        A("};")
     A("")
     for q, blocks in enumerate(groups):
         slots, tbase, ntab = group_meta[q]
@@ -245,8 +298,11 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
             A(f"{ind}  if (X1_IDX) srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
             A(f"{ind}  const {fp}* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
             A(f"{ind}  const {fp}* __restrict__ wp = w + (W_SHARED ? 0 : z * {st.nseg_w * st.extent}ll);")
-            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
-            for m in ms:
+            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.x2_width}ll;")
+            if st.harmonics:
+                for a in range(3):
+                    A(f"{ind}  {S}_v{a} = x2p[{a}];")
+            for m in ([] if st.harmonics else ms):
                 nvalid = min(16, st.nseg_x2 - 16 * m)
                 A(f"{ind}  {S}_yv{m} = x2p[{16 * m} + (n16 < {nvalid} ? n16 : 0)];")
             for i in i_used:
@@ -256,6 +312,14 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
             A(f"{ind}}}")
 
         def body(S: str, ind: str):
+            if st.harmonics:
+                _emit_monomials(A, ind, fp, _with_prefixes(monos), [f"{S}_v0", f"{S}_v1", f"{S}_v2"])
+                for m in ms:
+                    expr = None
+                    for q_, vi in enumerate(monos):
+                        term = f"s_sh[({16 * m} + n16) * {NM} + {q_}]"
+                        expr = f"{term} * {_mono_name(vi)}" if expr is None else f"fma({term}, {_mono_name(vi)}, {expr})"
+                    A(f"{ind}const {fp} {S}_yv{m} = {expr};")
             for t, (m, _row) in enumerate(tables):
                 A(f"{ind}{fp} t{t} = s_c[{(tbase + t) * 16} + n16] * {S}_yv{m};")
             # fence: table registers are produced by VALU and consumed through DPP
@@ -273,7 +337,7 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
                 A(f"{ind}}}")
 
         A(f"template <bool X1_IDX, bool W_SHARED>")
-        A(f"__device__ __forceinline__ void fwd_group{q}(FWD_PARAMS, const {fp}* s_c, int64_t r, int lane, int uu, bool active) {{")
+        A(f"__device__ __forceinline__ void fwd_group{q}(FWD_PARAMS, const {fp}* s_c, const {fp}* s_sh, int64_t r, int lane, int uu, bool active) {{")
         for k in ks:
             A(f"  {fp} acc{k} = 0;")
         A("  int64_t z0, z1;")
@@ -281,7 +345,8 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
         A("  const int n16 = lane & 15;")
         sets = ("a", "b") if prefetch else ("a",)
         for S in sets:
-            A(f"  {fp} " + ", ".join([f"{S}_yv{m} = 0" for m in ms] + [f"{S}_xv{i} = 0" for i in i_used]
+            second = [f"{S}_v{a} = 0" for a in range(3)] if st.harmonics else [f"{S}_yv{m} = 0" for m in ms]
+            A(f"  {fp} " + ", ".join(second + [f"{S}_xv{i} = 0" for i in i_used]
                                       + [f"{S}_wv{blk.b} = 0" for blk in blocks]) + ";")
         if prefetch:
             # The rows of the next batch element are requested before the arithmetic of the current one.  The requests
@@ -323,6 +388,11 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
     A(f"  __shared__ {fp} s_c[{max(1, len(all_tables)) * 16}];")
     A("  const int lane = threadIdx.x;")
     A(f"  for (int i = lane; i < {len(all_tables) * 16}; i += 64) s_c[i] = fwd_ctab[i];")
+    if st.harmonics:
+        A(f"  __shared__ {fp} s_sh[{npad * NM}];")
+        A(f"  for (int i = lane; i < {npad * NM}; i += 64) s_sh[i] = fwd_shtab[i];")
+    else:
+        A(f"  const {fp}* s_sh = nullptr;")
     A("  __syncthreads();")
     A("  int64_t wid = blockIdx.x;")
     A(f"  const int q = static_cast<int>(wid % {nsplit}); wid /= {nsplit};")
@@ -333,7 +403,7 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
         A(f"  const int u = ch * 64 + lane; const bool active = u < {st.extent}; const int uu = active ? u : 0;")
     A("  switch (q) {")
     for q in range(nsplit):
-        A(f"    case {q}: fwd_group{q}<X1_IDX, W_SHARED>(FWD_ARGS, s_c, r, lane, uu, active); break;")
+        A(f"    case {q}: fwd_group{q}<X1_IDX, W_SHARED>(FWD_ARGS, s_c, s_sh, r, lane, uu, active); break;")
     A("  }")
     A("}")
     A(f"constexpr int kFwdSplit = {nsplit};")
@@ -391,12 +461,25 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
             A(f"{ind}  if (X1_IDX) {S}_srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
             A(f"{ind}  const {fp}* __restrict__ x1p = x1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
             A(f"{ind}  const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
-            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.nseg_x2}ll;")
+            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.x2_width}ll;")
+            if st.harmonics:  # (requested first: the harmonics below wait for these three only)
+                for a in range(3):
+                    A(f"{ind}  {S}_v{a} = x2p[{a}];")
             for i in i_used:
                 A(f"{ind}  {S}_xv{i} = x1p[{st.x1_at(i)}];")
             for blk in blocks:
                 A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
-            for j in j_used:
+            if st.harmonics:
+                A(f"{ind}  {{")
+                need = sorted({vi for j in j_used for vi, _ in st.harmonics[j]}, key=lambda t: (len(t), t))
+                _emit_monomials(A, ind + "    ", fp, _with_prefixes(need), [f"{S}_v0", f"{S}_v1", f"{S}_v2"])
+                for j in j_used:
+                    expr = None
+                    for vi, c in st.harmonics[j]:
+                        expr = f"{_lit(c, T)} * {_mono_name(vi)}" if expr is None else f"fma({_lit(c, T)}, {_mono_name(vi)}, {expr})"
+                    A(f"{ind}    {S}_yv{j} = {expr if expr is not None else '0'};")
+                A(f"{ind}  }}")
+            for j in ([] if st.harmonics else j_used):
                 A(f"{ind}  {S}_yv{j} = x2p[{j}];")
             A(f"{ind}}}")
 
@@ -472,13 +555,36 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
             A(f"{ind}if (!active) {{" + " ".join(f"pj{j} = 0;" for j in j_used) + "}")
             for j in j_used:
                 A(f"{ind}pj{j} = wave_sum(pj{j});")
+            if st.harmonics:
+                # dv[a] = sum_j pj[j] dY_j/dv[a] (this wavefront's share: the sum over its channels and blocks is linear)
+                rests = set()
+                for j in j_used:
+                    for vi, _ in st.harmonics[j]:
+                        for a in sorted(set(vi)):
+                            rest = list(vi)
+                            rest.remove(a)
+                            rests.add(tuple(rest))
+                A(f"{ind}{fp} dv0 = 0, dv1 = 0, dv2 = 0;")
+                A(f"{ind}{{")
+                _emit_monomials(A, ind + "  ", fp, _with_prefixes(rests), [f"{S}_v0", f"{S}_v1", f"{S}_v2"])
+                for j in j_used:
+                    for vi, c in st.harmonics[j]:
+                        for a in sorted(set(vi)):
+                            rest = list(vi)
+                            rest.remove(a)
+                            A(f"{ind}  dv{a} = fma({_lit(c * vi.count(a), T)} * pj{j}, {_mono_name(tuple(rest))}, dv{a});")
+                A(f"{ind}}}")
             A(f"{ind}if (lane == 0) {{")
             if nparts == 1:
-                A(f"{ind}  {fp}* __restrict__ d2 = dx2 + z * {st.nseg_x2}ll;")
+                A(f"{ind}  {fp}* __restrict__ d2 = dx2 + z * {st.x2_width}ll;")
             else:
-                A(f"{ind}  {fp}* __restrict__ d2 = dx2_partial + (z * {nparts} + ch * {nsplit} + {q}) * {st.nseg_x2}ll;")
-            for j in range(st.nseg_x2):
-                A(f"{ind}  d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+                A(f"{ind}  {fp}* __restrict__ d2 = dx2_partial + (z * {nparts} + ch * {nsplit} + {q}) * {st.x2_width}ll;")
+            if st.harmonics:
+                for a in range(3):
+                    A(f"{ind}  d2[{a}] = dv{a};")
+            else:
+                for j in range(st.nseg_x2):
+                    A(f"{ind}  d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
             A(f"{ind}}}")
 
         A("template <bool X1_IDX, bool G_IDX, bool ATOMIC_DX1>")
@@ -492,7 +598,8 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
         for S in sets:
             A(f"  int64_t {S}_grow = -1, {S}_srow = 0;")
             A(f"  {fp} " + ", ".join([f"{S}_xv{i} = 0" for i in i_used] + [f"{S}_wv{blk.b} = 0" for blk in blocks]
-                                      + [f"{S}_yv{j} = 0" for j in j_used]) + ";")
+                                      + [f"{S}_yv{j} = 0" for j in j_used]
+                                      + ([f"{S}_v{a} = 0" for a in range(3)] if st.harmonics else [])) + ";")
         if prefetch:
             # one copy of the body (two copies drive the register allocator into hundreds of spills): set "a" is the row in
             # work, set "b" the row being fetched; "a = b" at the end of the iteration
@@ -509,7 +616,8 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
             A("    }")
             A("    a_grow = b_grow; a_srow = b_srow;")
             A("    " + " ".join([f"a_xv{i} = b_xv{i};" for i in i_used] + [f"a_wv{blk.b} = b_wv{blk.b};" for blk in blocks]
-                                 + [f"a_yv{j} = b_yv{j};" for j in j_used]))
+                                 + [f"a_yv{j} = b_yv{j};" for j in j_used]
+                                 + ([f"a_v{a} = b_v{a};" for a in range(3)] if st.harmonics else [])))
             A("  }")
         else:
             A("  for (int64_t zz = z0; zz < z1; ++zz) {")
@@ -565,13 +673,14 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     """Complete .hip translation unit: kernels, host launchers, registration under both table hashes."""
     ns = f"cw_{name}"
     nch = (st.extent + 63) // 64
-    W1, WW, W2, WO = st.nseg_x1 * st.extent, st.nseg_w * st.extent, st.nseg_x2, st.nseg_out * st.extent
+    W1, WW, W2, WO = st.nseg_x1 * st.extent, st.nseg_w * st.extent, st.x2_width, st.nseg_out * st.extent
     out = []
     A = out.append
     A("// GENERATED by cuequivariance_amd/codegen/channelwise.py - do not edit.")
     A(f"// channel-wise tensor product '{name}': extent {st.extent}, segments w/x1/x2/out = "
       f"{st.nseg_w}/{st.nseg_x1}/{st.nseg_x2}/{st.nseg_out}, {st.num_paths} paths, math {T}"
-      + (f", x1 rows in groups {list(st.layout_x1)}" if st.layout_x1 else "") + (f", output rows in groups {list(st.layout_out)}" if st.layout_out else ""))
+      + (f", x1 rows in groups {list(st.layout_x1)}" if st.layout_x1 else "") + (f", output rows in groups {list(st.layout_out)}" if st.layout_out else "")
+      + (", x2 = spherical harmonics of a 3-vector evaluated in the kernels" if st.harmonics else ""))
     A('#include "cw_common.h"')
     A("// operands that are read or written exactly once per launch (weights, weight gradients, the output rows) are")
     A("// marked non-temporal so that they do not displace the gathered rows in the caches")

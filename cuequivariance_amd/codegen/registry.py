@@ -27,6 +27,10 @@ CHANNELWISE = [
 # addressed channel-major inside every irrep block: no transposition pass before or after the kernels); unit "<name>_mulir".
 CHANNELWISE_MUL_IR = ["c128_l3", "c32_l2"]
 
+# Channel-wise entries also generated with the second operand computed in the kernels as the spherical harmonics of a
+# 3-vector (the degrees of the entry's second irreps); unit "<name>_sh".
+CHANNELWISE_HARMONICS = ["c128_l3"]
+
 # (name, irreps_in, irreps_out, contraction degree)
 SYMMETRIC = [
     ("s128_l3", "128x0e+128x1o+128x2e+128x3o", "128x0e+128x1o", 3),
@@ -118,6 +122,14 @@ def generate(verbose: bool = False) -> list[Path]:
             tl = t.with_layouts(channelwise_mul_ir_groups(ir1, ir2, filt))
             stl = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths], tl.layout(1), tl.layout(3))
             variants.append((name + "_mulir", stl, tl, tl.backward((True, True, True))))
+        if name in CHANNELWISE_HARMONICS:
+            from ..cue import fused
+
+            ls = [ir.l for _, ir in cue.Irreps("O3", ir2)]
+            poly, info, _ = fused.channelwise_spherical(cue.Irreps("O3", ir1), ls, filt)
+            tf = U1dTables.from_polynomial(poly)
+            sth = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths], harmonics=info.terms)
+            variants.append((name + "_sh", sth, tf, tf.backward((True, True, True))))
         for vname, vst, vt, vtb in variants:
             for T, code in MATH:
                 src = cw.emit_unit(vst, T, vname, vt.content_hash(code), vtb.content_hash(code), **tuning.get(T, {}))

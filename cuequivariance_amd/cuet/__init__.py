@@ -2,7 +2,7 @@
 
 from .transpose import TransposeSegments, TransposeIrrepsLayout
 from .segmented_polynomial import SegmentedPolynomial
-from .operations import ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction, SphericalHarmonics
+from .operations import ChannelWiseSphericalTensorProduct, ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction, SphericalHarmonics
 from .uniform_1d import uniform_1d
 from .triangle import triangle_multiplicative_update, TriMulPrecision
 from . import layers
@@ -11,6 +11,7 @@ __all__ = [
     "TransposeSegments",
     "TransposeIrrepsLayout",
     "SegmentedPolynomial",
+    "ChannelWiseSphericalTensorProduct",
     "ChannelWiseTensorProduct",
     "FullyConnectedTensorProduct",
     "Linear",

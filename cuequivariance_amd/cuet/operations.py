@@ -213,6 +213,101 @@ class ChannelWiseTensorProduct(torch.nn.Module):
         return self.transpose_out(out[0])
 
 
+class ChannelWiseSphericalTensorProduct(torch.nn.Module):
+    """``ChannelWiseTensorProduct(irreps_in1, Y_ls, filter)(x1, SphericalHarmonics(ls, normalize)(vectors), weight, ...)`` as one
+    polynomial of ``(weight, x1, vectors)``: the harmonics of the edge vectors are evaluated in registers inside the edge
+    kernels - they are neither written nor read back - and the backward returns the gradient with respect to the vectors.
+    An extension over the reference, which runs the two modules one after the other
+    (``cuequivariance_torch/operations/spherical_harmonics.py:26-93``, ``tp_channel_wise.py:30-258``).
+
+    ``forward(x1, vectors (batch, 3), weight=None, indices_1=None, indices_out=None, size_out=None)``; weights, irreps of the
+    output, layouts and indices as for ``ChannelWiseTensorProduct``; component normalisation of the harmonics,
+    ``normalize=True`` divides the vectors by their norm first (as ``SphericalHarmonics`` does).
+    """
+
+    def __init__(
+        self,
+        irreps_in1: cue.Irreps,
+        ls: Sequence[int],
+        filter_irreps_out: Sequence[cue.Irrep] = None,
+        *,
+        normalize: bool = True,
+        layout: Optional[cue.IrrepsLayout] = None,
+        layout_in1: Optional[cue.IrrepsLayout] = None,
+        layout_out: Optional[cue.IrrepsLayout] = None,
+        shared_weights: bool = True,
+        internal_weights: bool = None,
+        device: Optional[torch.device] = None,
+        dtype: Optional[torch.dtype] = None,
+        math_dtype=None,
+    ):
+        super().__init__()
+        from ..cue import fused
+
+        ls = list(ls)
+        if ls != sorted(set(ls)) or not ls:
+            raise ValueError(f"ls must be ascending and unique, got {ls}")
+        self.ls, self.normalize = ls, normalize
+        polynomial, info, irreps_out = fused.channelwise_spherical(irreps_in1, ls, filter_irreps_out)
+        self.irreps_in1, self.irreps_out = irreps_in1, irreps_out
+        self.weight_numel = polynomial.inputs[0].size
+        self.shared_weights = shared_weights
+        self.internal_weights = internal_weights if internal_weights is not None else shared_weights
+        if self.internal_weights:
+            if not self.shared_weights:
+                raise ValueError("Internal weights should be shared")
+            self.weight = torch.nn.Parameter(torch.randn(1, self.weight_numel, device=device, dtype=dtype))
+        else:
+            self.weight = None
+        source_in1, target_out = _default_layout(layout_in1 or layout), _default_layout(layout_out or layout)
+        groups = {}
+        if source_in1 == cue.mul_ir and _transposition_moves(irreps_in1):
+            groups[1] = [ir.dim for _, ir in irreps_in1]
+            source_in1 = cue.ir_mul
+        if target_out == cue.mul_ir and _transposition_moves(irreps_out):
+            groups[3] = [ir.dim for _, ir in irreps_out]
+            target_out = cue.ir_mul
+        self.transpose_in1 = TransposeIrrepsLayout(irreps_in1, source=source_in1, target=cue.ir_mul, device=device)
+        self.transpose_out = TransposeIrrepsLayout(irreps_out, source=cue.ir_mul, target=target_out, device=device)
+        options = {"origin": info}
+        if groups:
+            options["segment_groups"] = groups
+        self.f = SegmentedPolynomial(polynomial, method="uniform_1d", math_dtype=math_dtype, options=options)
+
+    def extra_repr(self) -> str:
+        return f"ls={self.ls}, normalize={self.normalize}, shared_weights={self.shared_weights}, weight_numel={self.weight_numel}"
+
+    def forward(
+        self,
+        x1: torch.Tensor,
+        vectors: torch.Tensor,
+        weight: Optional[torch.Tensor] = None,
+        indices_1: Optional[torch.Tensor] = None,
+        indices_out: Optional[torch.Tensor] = None,
+        size_out: Optional[int] = None,
+    ) -> torch.Tensor:
+        torch._assert(vectors.ndim == 2 and vectors.shape[1] == 3, f"vectors must have shape (batch, 3) - got {vectors.shape}")
+        if self.normalize:
+            vectors = torch.nn.functional.normalize(vectors, dim=1)
+        x1 = self.transpose_in1(x1)
+        indices_in: Dict[int, torch.Tensor] = {} if indices_1 is None else {1: indices_1}
+        indices_o: Dict[int, torch.Tensor] = {}
+        sizes_out: Dict[int, torch.Tensor] = {}
+        if indices_out is not None:
+            if size_out is None:
+                raise ValueError("size_out should be provided if indices_out is provided")
+            indices_o = {0: indices_out}
+            sizes_out = {0: torch.empty(size_out, 1, device="meta")}  # only .shape[0] is read
+        if self.weight is not None:
+            if weight is not None:
+                raise ValueError("Internal weights are used, weight should be None")
+            weight = self.weight
+        elif weight is None:
+            raise ValueError("Internal weights are not used, weight should not be None")
+        out = self.f([weight, x1, vectors], input_indices=indices_in, output_shapes=sizes_out, output_indices=indices_o)
+        return self.transpose_out(out[0])
+
+
 class FullyConnectedTensorProduct(torch.nn.Module):
     """``out[k w] = sum_{u v i j} w[u v w] C[i j k] x1[i u] x2[j v]`` over every allowed irrep triple."""
 

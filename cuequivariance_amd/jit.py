@@ -144,10 +144,21 @@ def is_row_weight_fully_connected(t: U1dTables, origin) -> bool:
             list(t.buffer_num_segments) == [st.width_w // st.Wd, st.width_x1, st.width_x2, st.width_out // st.Wd])
 
 
+def is_channelwise_with_harmonics(t: U1dTables, origin) -> bool:
+    """Tables of ``cue.fused.channelwise_spherical`` (``origin``: its ``FusedHarmonics``): a channel-wise product whose second
+    operand is the spherical harmonics of the 3-vector in buffer 2."""
+    from .cue.fused import FusedHarmonics
+
+    return (isinstance(origin, FusedHarmonics) and t.num_inputs == 3 and t.num_outputs == 1 and tuple(t.buffer_dim) == (1, 1, 0, 1)
+            and t.buffer_num_segments[2] == 3 and not t.layout(0) and not t.layout(2))
+
+
 def _family(t: U1dTables, polynomial=None, origin=None) -> Optional[str]:
     """The family generator that serves these tables: "channelwise" (which addresses x1 and the output through their
     layouts), "symmetric" (likewise for x and the output), "fc_rows" (a fully connected product with a weight row per batch row;
     ``origin`` is the polynomial the tables were flattened from) or None."""
+    if is_channelwise_with_harmonics(t, origin):
+        return "channelwise_sh"
     if is_channelwise(t) and not t.layout(0) and not t.layout(2):
         return "channelwise"
     if not t.layout(0) and is_symmetric_contraction(polynomial):
@@ -159,7 +170,7 @@ def _family(t: U1dTables, polynomial=None, origin=None) -> Optional[str]:
 
 def has_fused_backward(t: U1dTables, polynomial=None, origin=None) -> bool:
     """Families whose unit computes every gradient in one pass over the operands (preferred over a kernel per gradient)."""
-    return _family(t, polynomial, origin) in ("channelwise", "fc_rows")
+    return _family(t, polynomial, origin) in ("channelwise", "channelwise_sh", "fc_rows")
 
 
 def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTables] = None, root_polynomial=None,
@@ -224,6 +235,12 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None, origin=N
         tb = t.backward((True, True, True))
         src = cw.emit_unit(st, T, name, key, tb.content_hash(code), **_tuning(st, T))
         what = f"{st.num_paths} paths, extent {st.extent}"
+    elif family == "channelwise_sh":
+        tp = U1dTables.from_polynomial(origin.product)
+        _, paths = tp.operation(0)
+        st = cw.analyze(tp.operand_extent, tp.buffer_num_segments, [(*idx, c) for idx, c in paths], t.layout(1), t.layout(3), origin.terms)
+        src = cw.emit_unit(st, T, name, key, t.backward((True, True, True)).content_hash(code), **_tuning(st, T))
+        what = f"{st.num_paths} paths, extent {st.extent}, spherical harmonics of degrees {list(origin.ls)} in the kernels"
     elif family == "fc_rows":
         from .codegen import fullyconnected_rows as fcr
 
