@@ -268,6 +268,8 @@ class _DenseFunction(torch.autograd.Function):
             gx1 = _LinearDx.apply(mod, g, w, x1.dtype) if ctx.needs_input_grad[2] else None
             gw = _LinearDw.apply(mod, x1, g, w) if ctx.needs_input_grad[1] else None
             return None, gw, gx1, None
+        if not torch.is_grad_enabled():  # (a plain backward: one call for the three gradients)
+            return (None, *_fc_grads(0, mod, w, x1, x2, g, *ctx.needs_input_grad[1:4]))
         gw = _FcDw.apply(mod, x1, x2, g, w, 0) if ctx.needs_input_grad[1] else None
         gx1 = _FcDx1.apply(mod, w, g, x2, x1, 0) if ctx.needs_input_grad[2] else None
         gx2 = _FcDx2.apply(mod, w, x1, g, x2, 0) if ctx.needs_input_grad[3] else None
@@ -574,6 +576,10 @@ class _FcFunction(torch.autograd.Function):
         # three: derivatives of any order stay on these kernels
         mod = ctx.mod
         w, x1, x2 = ctx.saved_tensors
+        if not torch.is_grad_enabled():
+            # a plain backward (no graph of the gradients asked for): the three gradients in one call, their operands
+            # prepared once
+            return (None, *_fc_grads(1, mod, w, x1, x2, g, *ctx.needs_input_grad[1:4]))
         gw = _FcDw.apply(mod, x1, x2, g, w, 1) if ctx.needs_input_grad[1] else None
         gx1 = _FcDx1.apply(mod, w, g, x2, x1, 1) if ctx.needs_input_grad[2] else None
         gx2 = _FcDx2.apply(mod, w, x1, g, x2, 1) if ctx.needs_input_grad[3] else None
