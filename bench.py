@@ -212,6 +212,31 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = ("configs[3]: FullyConnectedTensorProduct 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, batch 50000, shared weights, "
                 "fwd + bwd (dw, dx1, dx2)")
+    elif wl == "cfg2sh":
+        # configs[1] with the spherical harmonics of the edge vectors evaluated inside the edge kernels (the step before the
+        # product in a MACE interaction block): inputs are the raw edge vectors, gradients also with respect to them
+        N, E = 5_000, 100_000
+        i1 = cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o")
+        m = cuet.ChannelWiseSphericalTensorProduct(i1, [0, 1, 2, 3], "0e+1o+2e+3o", layout=cue.ir_mul, shared_weights=False,
+                                                   internal_weights=False, device=dev, dtype=torch.float32)
+        g = torch.Generator(device=dev).manual_seed(0)
+        x1 = torch.randn(N, i1.dim, device=dev, generator=g, requires_grad=True)
+        vec = torch.randn(E, 3, device=dev, generator=g, requires_grad=True)
+        w = torch.randn(E, m.weight_numel, device=dev, generator=g, requires_grad=True)
+        snd = torch.randint(0, N, (E,), device=dev, generator=g, dtype=torch.int32)
+        rcv = torch.sort(torch.randint(0, N, (E,), device=dev, generator=g, dtype=torch.int32))[0]
+        cot = torch.randn(N, m.irreps_out.dim, device=dev, generator=g)
+
+        def step():
+            return torch.autograd.grad(m(x1, vec, w, indices_1=snd, indices_out=rcv, size_out=N), [w, x1, vec], cot)
+
+        unit, units, dt = "edges/s", E, "f32"
+        alg = {"fwd": (E * (2944 + 3) + N * (2048 + 12672)) * 4 + 2 * E * 4,
+               "bwd": (2 * E * (2944 + 3) + N * (2 * 2048 + 12672)) * 4 + 2 * E * 4}
+        flops = {k: E * n_ * 128 for k, n_ in zip(("fwd", "bwd"), VALU_INSTS_PER_ELEMENT["cfg2"])}
+        flop_roof, flop_peak = "valu", VALU_PEAK_F32
+        desc = ("configs[1] with the spherical harmonics (l <= 3, normalised vectors) evaluated inside the edge kernels: 5000 nodes, "
+                "100000 edges, inputs node features / edge vectors / per-edge weights, fwd + bwd (dw, dx1, d vectors)")
     elif wl == "fcconv":
         # the product inside FullyConnectedTensorProductConv: a weight row per edge, x1 gathered by source, output summed by
         # destination (no BASELINE config; sizes chosen here)
@@ -497,7 +522,7 @@ def main() -> int:
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
     ap.add_argument("--graph", action="store_true",
                     help="secondary workloads only: capture the step into a HIP graph and time its replays")
-    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg4fc", "fcconv", "cfg5"], default=None,
+    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg2sh", "cfg3", "cfg4", "cfg4fc", "fcconv", "cfg5"], default=None,
                     help="default: the headline metric (cfg2, fp32) with every other configuration in a 'secondary' object.  "
                          "Naming a workload prints one line for it alone: cfg2 the headline, cfg1 the reference's CPU-sized "
                          "channel-wise case, cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected "
@@ -574,7 +599,7 @@ def main() -> int:
         add("cfg2_fp32_ordered_dx1", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float32, N, E, ssteps, swarm, True)[0]))
         add("cfg2_fp64", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float64, N, E, ssteps, swarm, False)[0]))
         for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg4_linear_fp32", "cfg4", "fp32"),
-                            ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"),
+                            ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
                             ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp32", "cfg5", "fp32")):
             add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))
         if not args.no_cpu_baseline:

@@ -162,19 +162,16 @@ def _mono_name(vi: tuple) -> str:
 
 
 def _emit_monomials(A, ind: str, T: str, monos: Sequence[tuple], v: Sequence[str]):
-    """``const T mo_<indices>`` for every monomial, each from a lower one by one multiplication."""
-    done = set()
+    """``const T mo_<indices>`` for every monomial of ``monos`` (closed under prefixes, see ``_with_prefixes``), each from its
+    prefix by one multiplication."""
     for vi in sorted(monos, key=lambda t: (len(t), t)):
         if not vi:
             A(f"{ind}const {T} mo_one = 1;")
         elif len(vi) == 1:
             A(f"{ind}const {T} {_mono_name(vi)} = {v[vi[0]]};")
         else:
-            if vi[:-1] not in done:  # (a prefix nobody asked for)
-                _emit_monomials(A, ind, T, [vi[:-1]], v)
-                done.add(vi[:-1])
+            assert vi[:-1] in monos, (vi, monos)
             A(f"{ind}const {T} {_mono_name(vi)} = {_mono_name(vi[:-1])} * {v[vi[-1]]};")
-        done.add(vi)
 
 
 def _with_prefixes(monos) -> list:
