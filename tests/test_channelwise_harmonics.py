@@ -152,3 +152,20 @@ def test_harmonics_with_mul_ir_rows(device, tmp_path, monkeypatch):
         assert b.f.m._plan(torch.float64).specialised(device)
     finally:
         jit.enable(False)
+
+
+@pytest.mark.gpu
+def test_harmonics_without_edges(device):
+    from cuequivariance_amd import cuet
+
+    i1 = cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o")
+    m = cuet.ChannelWiseSphericalTensorProduct(i1, [0, 1, 2, 3], ["0e", "1o", "2e", "3o"], layout=cue.ir_mul, shared_weights=False,
+                                               device=device, dtype=torch.float32)
+    x1 = torch.randn(6, i1.dim, device=device, requires_grad=True)
+    v = torch.randn(0, 3, device=device, requires_grad=True)
+    w = torch.randn(0, m.weight_numel, device=device, requires_grad=True)
+    idx = torch.zeros(0, dtype=torch.int32, device=device)
+    out = m(x1, v, w, indices_1=idx, indices_out=idx, size_out=6)
+    assert out.shape == (6, m.irreps_out.dim) and float(out.detach().abs().sum()) == 0.0
+    g1, gv, gw = torch.autograd.grad(out, [x1, v, w], torch.ones_like(out))
+    assert g1.shape == x1.shape and float(g1.abs().sum()) == 0.0 and gv.shape == (0, 3) and gw.shape == w.shape

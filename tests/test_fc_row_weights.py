@@ -116,3 +116,22 @@ def test_row_weights_multiplicities_below_the_wavefront(device, dtype, jit_on):
     """24 input and 40 output channels (lanes beyond them idle), outputs up to l = 2."""
     m = run_case(device, "24x0e+24x1o+24x2e", "0e+1o", "40x0e+40x1o+40x2e", 37, 333, dtype, seed=24, indexed=True)
     assert m.f_per_sample.f.m._plan(dtype).specialised(device)
+
+
+@pytest.mark.gpu
+def test_row_weights_without_batch_rows(device):
+    """No edges at all: the output rows are zeros, the gradients have their shapes (the build's unit, no compilation)."""
+    from cuequivariance_amd import cuet
+
+    i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e")
+    m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, shared_weights=False, internal_weights=False,
+                                         device=device, dtype=torch.float32)
+    x1 = torch.randn(5, i1.dim, device=device, requires_grad=True)
+    x2 = torch.randn(0, i2.dim, device=device, requires_grad=True)
+    w = torch.randn(0, m.weight_numel, device=device, requires_grad=True)
+    idx = torch.zeros(0, dtype=torch.int32, device=device)
+    out = m(x1, x2, w, indices_1=idx, indices_out=idx, size_out=5)
+    assert out.shape == (5, i1.dim) and float(out.detach().abs().sum()) == 0.0
+    g1, g2, gw = torch.autograd.grad(out, [x1, x2, w], torch.ones_like(out))
+    assert g1.shape == x1.shape and float(g1.abs().sum()) == 0.0 and g2.shape == x2.shape and gw.shape == w.shape
+    assert m.f_per_sample.f.m._plan(torch.float32).specialised(device)
