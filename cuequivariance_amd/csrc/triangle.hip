@@ -378,7 +378,7 @@ __global__ void __launch_bounds__(256) gemm_tn_kernel(const TI* __restrict__ A, 
   const int part = static_cast<int>(item - chunk * nparts);
   A += part * sA;
   B += part * sB;
-  P += item * static_cast<int64_t>(M) * N;
+  P += (part * (static_cast<int64_t>(gridDim.z) / nparts) + chunk) * static_cast<int64_t>(M) * N;  // part-major
   const int64_t z_begin = chunk * rows_per_chunk;
   const int64_t z_end = min(z_begin + rows_per_chunk, rows);
 
@@ -2261,7 +2261,7 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
 
 extern "C" int64_t cueq_gemm_tn_items(int64_t rows, int32_t nparts) {
   if (nparts < 1) nparts = 1;
-  int64_t chunks = (static_cast<int64_t>(device_cus()) * 2 + nparts - 1) / nparts;
+  int64_t chunks = static_cast<int64_t>(device_cus()) * 2 / nparts;  // at most two blocks per CU: no tail round
   const int64_t most = (rows + 4 * kTnRows - 1) / (4 * kTnRows);  // at least 64 rows per chunk
   if (chunks > most) chunks = most;
   if (chunks < 1) chunks = 1;
@@ -2287,9 +2287,9 @@ extern "C" int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows
     // 2-byte inputs: bf16 MFMA on contraction-major tiles (transposing LDS reads); batch items = (row chunk, part)
     const int64_t rpc32 = (((rows + chunks - 1) / chunks + 31) / 32) * 32;
     hipLaunchKernelGGL((gemm_kernel<uint16_t, float, true, true>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(A), lda,
-                       rpc32 * lda, static_cast<const uint16_t*>(B), ldb, rpc32 * ldb, partials, N, static_cast<int64_t>(nparts) * M * N,
+                       rpc32 * lda, static_cast<const uint16_t*>(B), ldb, rpc32 * ldb, partials, N, static_cast<int64_t>(M) * N,
                        static_cast<int>(M), static_cast<int>(N), static_cast<int>(rpc32), static_cast<float>(alpha), 0, 0, rows, nparts,
-                       stride_a, stride_b, static_cast<int64_t>(M) * N, nullptr, 0, 0, 0, 0);
+                       stride_a, stride_b, chunks * static_cast<int64_t>(M) * N, nullptr, 0, 0, 0, 0);
     CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }

@@ -160,6 +160,33 @@ def _batched_groups(paths, a_key, c_key):
     return groups
 
 
+def _merged_weight_gradient(mod: "SegmentedPolynomialDense"):
+    """``(K, N, coeff, a0, c0, da, dc, [(w_off, components)])`` when the weight gradients of all blocks of the 3-operand form
+    can come from one launch: one block shape and scale, every weight block used by one run of components, and the
+    components of all blocks at constant strides in the input and in the cotangent (a Linear layer over ``ir_mul`` rows:
+    the components of all irreps one after the other).  ``None`` otherwise (one launch per block then)."""
+    hit = getattr(mod, "_dw_merged", False)
+    if hit is not False:
+        return hit
+    out = None
+    comps = sorted(((p.a_off + i * da, p.c_off + i * dc, p.w_off, p.K, p.N, p.coeff) for p, count, da, dc in mod.fwd_groups
+                    for i in range(count)))
+    if len(comps) > 1 and len({c[3:] for c in comps}) == 1:
+        K, N, coeff = comps[0][3:]
+        da, dc = comps[1][0] - comps[0][0], comps[1][1] - comps[0][1]
+        regular = da > 0 and dc > 0 and all(b[0] - a[0] == da and b[1] - a[1] == dc for a, b in zip(comps, comps[1:]))
+        runs = []
+        for c in comps:
+            if runs and runs[-1][0] == c[2]:
+                runs[-1][1] += 1
+            else:
+                runs.append([c[2], 1])
+        if regular and len({w for w, _ in runs}) == len(runs) and len(comps) <= 64:
+            out = (K, N, coeff, comps[0][0], comps[0][1], da, dc, [(w, n) for w, n in runs])
+    mod._dw_merged = out
+    return out
+
+
 def _merged_tables(mod: "SegmentedPolynomialDense", device: torch.device):
     """For the 3-operand form: the column blocks of all paths as parts of table-driven launches, one launch per distinct
     (K, N, coefficient).  ``fwd``: rows (x offset, weight offset, out offset); ``dx``: rows (g offset, weight offset, dx
@@ -313,7 +340,27 @@ class _DenseFunction(torch.autograd.Function):
                     code, es = _DTYPE_CODE[dtype], x1d.element_size()
                     gw32 = torch.zeros(wd.numel(), dtype=torch.float32, device=x1.device)
                     written = set()
-                    for p, count, da, dc in mod.fwd_groups:
+                    merged = _merged_weight_gradient(mod)
+                    if merged is not None:
+                        # every component of every block in one launch (the partial products of a block's components are
+                        # consecutive rows of `part`), then one ordered row sum per block
+                        K, N, coeff, a0, c0, da, dc, runs = merged
+                        nparts = sum(n for _, n in runs)
+                        items = lib.cueq_gemm_tn_items(Z, nparts)
+                        chunks = items // nparts
+                        part = torch.empty(items, K * N, dtype=torch.float32, device=x1.device)
+                        _lib.check(
+                            lib.cueq_gemm_tn(code, K, N, Z, x1d.data_ptr() + a0 * es, x1d.stride(0), da, g.data_ptr() + c0 * es,
+                                             g.stride(0), dc, nparts, part.data_ptr(), coeff, stream), "cueq_gemm_tn")
+                        first_part = 0
+                        for w_off, n in runs:
+                            rows = part[first_part * chunks: (first_part + n) * chunks]
+                            ws_bytes = lib.cueq_sum_rows_workspace(n * chunks, K * N)
+                            ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x1.device)
+                            _lib.check(lib.cueq_sum_rows(_lib.F32, n * chunks, K * N, rows.data_ptr(), gw32[w_off: w_off + K * N].data_ptr(),
+                                                         ws.data_ptr(), ws_bytes, stream), "cueq_sum_rows")
+                            first_part += n
+                    for p, count, da, dc in (mod.fwd_groups if merged is None else []):
                         items = lib.cueq_gemm_tn_items(Z, count)
                         part = torch.empty(items, p.K * p.N, dtype=torch.float32, device=x1.device)
                         _lib.check(

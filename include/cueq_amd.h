@@ -301,9 +301,10 @@ int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const vo
                         void* stream);
 
 /* Weight-gradient shaped product C (M x N) = sum over rows z and parts p of A[z, p*stride_a : +M]^T B[z, p*stride_b : +N]
- * (both operands row-major with the long index z as rows).  The rows are cut into chunks; item (chunk, part) writes
- * alpha * its partial product to partials[item] (float32, M x N); the caller adds the cueq_gemm_tn_items(rows, nparts)
- * items in order (e.g. cueq_sum_rows over an items x (M*N) view): no atomics.  Serves the weight gradients of the dense
+ * (both operands row-major with the long index z as rows).  The rows are cut into chunks = items / nparts pieces; item
+ * (part, chunk) writes alpha * its partial product to partials[part * chunks + chunk] (float32, M x N): the partials of one
+ * part are consecutive, so the caller adds all cueq_gemm_tn_items(rows, nparts) items in order (cueq_sum_rows over an
+ * items x (M*N) view) or, for parts that belong to different results, each run of parts on its own: no atomics.  Serves the weight gradients of the dense
  * layers (reference: the backward of FusedTensorProductOp3, primitives/segmented_polynomial_fused_tp.py:32-48). */
 int64_t cueq_gemm_tn_items(int64_t rows, int32_t nparts);
 int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows, const void* A, int64_t lda, int64_t stride_a,
