@@ -46,6 +46,7 @@ EXPORTED_SYMBOLS = (
     "cueq_gemm_nt",
     "cueq_gemm",
     "cueq_gemm_table",
+    "cueq_linear_rows",
     "cueq_fc_combine",
     "cueq_fc_rowdot",
     "cueq_gemm_grouped",
@@ -206,6 +207,8 @@ def load() -> C.CDLL:
         lib.cueq_gemm_grouped.restype = C.c_int
         lib.cueq_gemm_table.argtypes = [i32, i32, i32, i32, i64, i64, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i64, i64, i64, f64, i32, ptr]
         lib.cueq_gemm_table.restype = C.c_int
+        lib.cueq_linear_rows.argtypes = [i32, i32, i64, i64, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i64, f64, ptr]
+        lib.cueq_linear_rows.restype = C.c_int
         lib.cueq_fc_combine.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i32, ptr, i32, i32, ptr]
         lib.cueq_fc_combine.restype = C.c_int
         lib.cueq_fc_rowdot.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, i32, ptr, i32, i32, ptr]

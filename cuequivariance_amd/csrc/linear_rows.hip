@@ -1,0 +1,289 @@
+// Row-streaming product for Linear-like operations in a 2-byte type:
+//   C[z, c_p : c_p + N] = alpha * A[z, a_p : a_p + K] * W_s(p)      for every part p of a host table, all rows z,
+// with every distinct weight block W_s resident in LDS for the whole launch.  One persistent block per compute unit;
+// each wavefront walks units (32 rows, part) on its own: the rows of A are requested three units ahead as they lie in
+// memory (every load instruction covers whole 128-byte pieces of rows), pass through a staging tile private to the
+// wavefront to become MFMA operands, the weight fragments come from LDS, and the 32 x N result leaves through the same
+// staging tile as whole 128-byte row pieces.  No barrier after the weights are in place, so the loads, arithmetic and
+// stores of the wavefronts of a compute unit overlap freely: the kernel is meant to run at the rate of a copy of A to C.
+// A and C are marked as streams (every byte is touched once); measured, that also leaves the last-level cache to the
+// kernel that reads A next.
+//
+// Serves the forward and the input gradient of the reference's Linear (descriptor `uv,iu,iv` per irrep,
+// cuequivariance/group_theory/descriptors/irreps_tp.py:524-547; executed there through FusedTensorProductOp3,
+// cuequivariance_torch/primitives/segmented_polynomial_fused_tp.py:40-48).
+
+#include "common.h"
+#include "cw_common.h"
+#include "u1d_spec.h"
+
+namespace cueq {
+
+namespace {
+
+typedef float lr_floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 lr_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float lr_floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 lr_bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t lr_u32x4 __attribute__((ext_vector_type(4)));
+
+// 16-byte accesses marked as streams: every byte of A and C is touched once
+__device__ __forceinline__ uint4 lr_stream_load(const char* p) {
+  const lr_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const lr_u32x4*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void lr_stream_store(uint4 v, void* p) {
+  const lr_u32x4 w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<lr_u32x4*>(p));
+}
+
+constexpr int kLrWaves = 8;
+constexpr int kLrMaxParts = 48;
+constexpr int kLrMaxSlots = 8;
+
+struct LrPart {
+  int32_t a_off, c_off, slot;
+};
+struct LrParts {
+  LrPart part[kLrMaxParts];
+  int64_t w_off[kLrMaxSlots];
+};
+
+__device__ __forceinline__ uint32_t lr_pack(float lo, float hi) {
+  const lr_floatx2 f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lr_bf16x2));
+}
+
+constexpr int kLrStageStride = 144;                   // bytes between the rows of a wavefront's staging tile: 128 of data + 16
+constexpr int kLrStageBytes = 32 * kLrStageStride;    // 32 rows
+
+// The rows of a unit are requested as they lie in memory - every load instruction covers whole 128-byte (or 64-byte) row
+// pieces, 8 (16) rows at a time - in passes of at most 128 bytes of k.  Vector i of pass ps: row i * rpi + lane / lpr,
+// bytes 128 ps + 16 (lane % lpr), with lpr = 8 lanes per 128-byte piece (4 per 64-byte piece), rpi = 64 / lpr.
+// A load that touches a line only in part leaves the rest to a later instruction; marked as a stream, that line would be
+// fetched again.
+template <int KT>
+__device__ __forceinline__ void lr_request(uint4 (&xs)[2 * KT], const char* base, int64_t row_bytes, int last_row, int lane) {
+#pragma unroll
+  for (int ps = 0; ps < (KT + 1) / 2; ++ps) {
+    const int w = 64 * KT - 128 * ps >= 128 ? 128 : 64, lpr = w / 16, rpi = 64 / lpr;
+#pragma unroll
+    for (int i = 0; i < 32 / rpi; ++i) {
+      int r = i * rpi + lane / lpr;
+      r = r < last_row ? r : last_row;  // rows past the end repeat the last one
+      xs[4 * ps + i] = lr_stream_load(base + r * row_bytes + 128 * ps + 16 * (lane % lpr));
+    }
+  }
+}
+
+// One unit: 32 rows (tile) of one part.  xs holds the rows as requested; they pass through the staging tile to become MFMA
+// operands (lane (c, h): row c, bytes 32 h .. + 32 of every 64 bytes of k); after that `requested()` may refill xs.
+// FULL: all 32 rows exist (stores without conditions, so that the number of outstanding memory operations at every wait
+// is known at compile time and a wait for loads does not also wait for the stores issued after them).
+template <int KT, int NT, bool FULL, typename Refill>
+__device__ __forceinline__ void lr_unit(uint4 (&xs)[2 * KT], const char* wl, char* stage, uint16_t* crow, int64_t ldc, int rows, float alpha, int lane,
+                                        Refill&& refill) {
+  constexpr int K = 32 * KT;
+  constexpr int WRS = 2 * K + 16;
+  constexpr int SC = NT >= 2 ? 64 : 32;
+  constexpr int SRS = kLrStageStride;
+  const int c = lane & 31, h = lane >> 5;
+  uint4 xf[KT][2];
+#pragma unroll
+  for (int ps = 0; ps < (KT + 1) / 2; ++ps) {
+    const int w = 64 * KT - 128 * ps >= 128 ? 128 : 64, lpr = w / 16, rpi = 64 / lpr;
+#pragma unroll
+    for (int i = 0; i < 32 / rpi; ++i) *reinterpret_cast<uint4*>(stage + (i * rpi + lane / lpr) * SRS + 16 * (lane % lpr)) = xs[4 * ps + i];
+#pragma unroll
+    for (int s2 = 0; s2 < w / 64; ++s2) {
+      xf[2 * ps + s2][0] = *reinterpret_cast<const uint4*>(stage + c * SRS + s2 * 64 + h * 32);
+      xf[2 * ps + s2][1] = *reinterpret_cast<const uint4*>(stage + c * SRS + s2 * 64 + h * 32 + 16);
+    }
+  }
+  refill();
+  uint4 af[2][2 * KT];  // weight fragments of the current and the next 32 result columns
+#pragma unroll
+  for (int s = 0; s < 2 * KT; ++s) af[0][s] = *reinterpret_cast<const uint4*>(wl + (s >> 1) * 64 + (s & 1) * 16);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (t + 1 < NT) {
+#pragma unroll
+      for (int s = 0; s < 2 * KT; ++s) af[(t + 1) & 1][s] = *reinterpret_cast<const uint4*>(wl + (t + 1) * 32 * WRS + (s >> 1) * 64 + (s & 1) * 16);
+    }
+    lr_floatx16 acc = lr_floatx16{0};
+#pragma unroll
+    for (int s = 0; s < 2 * KT; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(lr_bf16x8, af[t & 1][s]), __builtin_bit_cast(lr_bf16x8, xf[s >> 1][s & 1]), acc, 0, 0, 0);
+    // lane (c, h) holds row z = c of the result, columns 32 t + 8 a + 4 h + (0..3)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const uint2 v = make_uint2(lr_pack(alpha * acc[4 * a], alpha * acc[4 * a + 1]), lr_pack(alpha * acc[4 * a + 2], alpha * acc[4 * a + 3]));
+      *reinterpret_cast<uint2*>(stage + c * SRS + ((t * 32) % SC + 8 * a + 4 * h) * 2) = v;
+    }
+    if ((t * 32) % SC + 32 == SC || t == NT - 1) {
+      const int cols = (t * 32) % SC + 32;  // staged columns of this pass
+      const int col0 = t * 32 + 32 - cols;  // first result column of the pass
+      const int vpr = cols / 8;             // 16-byte vectors per row
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j < vpr / 2) {
+          const int idx = lane + 64 * j;
+          const int r = idx / vpr, cv = idx % vpr;
+          if (FULL || r < rows) {
+            const uint4 v = *reinterpret_cast<const uint4*>(stage + r * SRS + cv * 16);
+            lr_stream_store(v, crow + static_cast<int64_t>(r) * ldc + col0 + cv * 8);
+          }
+        }
+      }
+    }
+  }
+}
+
+// KT, NT: contraction length and result columns in units of 32
+template <int KT, int NT>
+__global__ void __launch_bounds__(64 * kLrWaves, 1)
+    linear_rows_kernel(const uint16_t* __restrict__ A, int64_t lda, const uint16_t* __restrict__ W, LrParts parts, int nslots, int nparts,
+                       int w_contraction_major, uint16_t* __restrict__ C, int64_t ldc, int M, float alpha) {
+  constexpr int K = 32 * KT, N = 32 * NT;
+  constexpr int WRS = 2 * K + 16;        // bytes between weight rows (one row per result column) in LDS
+  extern __shared__ __align__(16) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  for (int s = 0; s < nslots; ++s) {
+    const uint16_t* w = W + parts.w_off[s];
+    char* dst = smem + s * (N * WRS);
+    if (w_contraction_major) {  // K x N as it lies: element (k, n) becomes column k of row n
+      for (int e = tid; e < K * N; e += 64 * kLrWaves) {
+        const int k = e / N, n = e % N;
+        *reinterpret_cast<uint16_t*>(dst + n * WRS + 2 * k) = w[e];
+      }
+    } else {  // N x K as it lies
+      for (int e = tid; e < N * (K / 8); e += 64 * kLrWaves) {
+        const int n = e / (K / 8), v = e % (K / 8);
+        *reinterpret_cast<uint4*>(dst + n * WRS + 16 * v) = *reinterpret_cast<const uint4*>(w + n * K + 8 * v);
+      }
+    }
+  }
+  __syncthreads();
+
+  char* stage = smem + nslots * (N * WRS) + wave * kLrStageBytes;
+  const char* wlane = smem + c * WRS + h * 32;
+  const int nfull = M / 32;  // tiles of 32 existing rows
+  const int wslot = blockIdx.x * kLrWaves + wave, nw = gridDim.x * kLrWaves;
+  // unit = tile * nparts + part; this wavefront takes the units wslot, wslot + nw, ... - walked as (tile, part) pairs
+  const int step_t = nw / nparts, step_p = nw % nparts;
+  auto advance = [&](int& t, int& p) {
+    t += step_t;
+    p += step_p;
+    if (p >= nparts) { p -= nparts; ++t; }
+  };
+  auto source = [&](int t, int p) {
+    const int tt = t < nfull ? t : nfull - 1;  // past the end: a tile that exists (the values are not used)
+    return reinterpret_cast<const char*>(A + static_cast<int64_t>(tt) * 32 * lda + parts.part[p].a_off);
+  };
+  const int64_t row_bytes = lda * 2;
+  const int64_t total_full = static_cast<int64_t>(nfull) * nparts;
+  if (wslot < total_full) {
+    // Three operand sets in rotation: the rows of unit i + 3 are requested as soon as the products of unit i have read
+    // theirs.  The loop body is three units without a branch in between (one basic block: the requests stay where they
+    // are written); the one or two units left over follow it.
+    const int mine = static_cast<int>((total_full - wslot + nw - 1) / nw);  // units of this wavefront
+    uint4 x0[2 * KT], x1[2 * KT], x2[2 * KT];
+    int t = wslot / nparts, p = wslot % nparts;  // the unit worked on
+    int rt = t, rp = p;                          // the unit requested
+    lr_request<KT>(x0, source(rt, rp), row_bytes, 31, lane);
+    advance(rt, rp);
+    lr_request<KT>(x1, source(rt, rp), row_bytes, 31, lane);
+    advance(rt, rp);
+    lr_request<KT>(x2, source(rt, rp), row_bytes, 31, lane);
+    advance(rt, rp);
+#define LR_PHASE(XS, AFTER)                                                                                                              \
+    {                                                                                                                                     \
+      const char* src = source(rt, rp);                                                                                                   \
+      lr_unit<KT, NT, true>(XS, wlane + parts.part[p].slot * (N * WRS), stage, C + static_cast<int64_t>(t) * 32 * ldc + parts.part[p].c_off, \
+                            ldc, 32, alpha, lane, AFTER);                                                                                 \
+      advance(rt, rp);                                                                                                                    \
+      advance(t, p);                                                                                                                      \
+    }
+#define LR_NEXT(XS) [&]() { lr_request<KT>(XS, src, row_bytes, 31, lane); __builtin_amdgcn_sched_barrier(0); }
+    for (int it = 0; it < mine / 3; ++it) {
+      LR_PHASE(x0, LR_NEXT(x0))
+      LR_PHASE(x1, LR_NEXT(x1))
+      LR_PHASE(x2, LR_NEXT(x2))
+    }
+    if (mine % 3 >= 1) LR_PHASE(x0, [&]() { (void)src; })
+    if (mine % 3 == 2) LR_PHASE(x1, [&]() { (void)src; })
+#undef LR_NEXT
+#undef LR_PHASE
+  }
+  if (M % 32 != 0) {  // the units of the last, partial tile
+    for (int p = wslot; p < nparts; p += nw) {
+      uint4 xs[2 * KT];
+      lr_request<KT>(xs, reinterpret_cast<const char*>(A + static_cast<int64_t>(nfull) * 32 * lda + parts.part[p].a_off), row_bytes, M - nfull * 32 - 1, lane);
+      lr_unit<KT, NT, false>(xs, wlane + parts.part[p].slot * (N * WRS), stage, C + static_cast<int64_t>(nfull) * 32 * ldc + parts.part[p].c_off, ldc,
+                             M - nfull * 32, alpha, lane, []() {});
+    }
+  }
+}
+
+}  // namespace
+
+}  // namespace cueq
+
+// table: host memory, nparts rows of (a_off, w_off, c_off) in elements
+extern "C" int cueq_linear_rows(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                                const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts, double alpha, void* stream_) {
+  using namespace cueq;
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(dtype == CUEQ_BF16, CUEQ_ERR_UNSUPPORTED, "linear_rows: bfloat16 only");
+  CUEQ_REQUIRE(M >= 0 && N > 0 && K > 0 && nparts >= 0, CUEQ_ERR_INVALID, "linear_rows: bad extents");
+  CUEQ_REQUIRE(N % 32 == 0 && K % 32 == 0 && N <= 128 && K <= 128, CUEQ_ERR_UNSUPPORTED, "linear_rows: K and N must be 32, 64, 96 or 128");
+  CUEQ_REQUIRE(nparts <= kLrMaxParts, CUEQ_ERR_TOO_LARGE, "linear_rows: at most %d parts per launch", kLrMaxParts);
+  if (M == 0 || nparts == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(A && W && C && table, CUEQ_ERR_INVALID, "linear_rows: null operand");
+  CUEQ_REQUIRE(M <= (1ll << 31) - 64, CUEQ_ERR_TOO_LARGE, "linear_rows: too many rows");
+  CUEQ_REQUIRE(lda % 8 == 0 && ldc % 8 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(C) % 16 == 0,
+               CUEQ_ERR_UNSUPPORTED, "linear_rows: row strides and pointers must be multiples of 16 bytes");
+  LrParts parts;
+  int nslots = 0;
+  for (int64_t p = 0; p < nparts; ++p) {
+    const int64_t a_off = table[3 * p], w_off = table[3 * p + 1], c_off = table[3 * p + 2];
+    CUEQ_REQUIRE(a_off >= 0 && a_off + K <= lda && c_off >= 0 && c_off + N <= ldc && w_off >= 0 && w_off + K * N <= w_numel && a_off % 8 == 0 && c_off % 8 == 0 && w_off % 8 == 0,
+                 CUEQ_ERR_INVALID, "linear_rows: part %lld: offsets must lie inside a row / the weights and be multiples of 8 elements", static_cast<long long>(p));
+    int s = 0;
+    while (s < nslots && parts.w_off[s] != w_off) ++s;
+    if (s == nslots) {
+      CUEQ_REQUIRE(nslots < kLrMaxSlots, CUEQ_ERR_TOO_LARGE, "linear_rows: at most %d distinct weight blocks per launch", kLrMaxSlots);
+      parts.w_off[nslots++] = w_off;
+    }
+    parts.part[p] = LrPart{static_cast<int32_t>(a_off), static_cast<int32_t>(c_off), s};
+  }
+  const size_t lds = static_cast<size_t>(nslots) * N * (2 * K + 16) + static_cast<size_t>(kLrWaves) * kLrStageBytes;
+  CUEQ_REQUIRE(lds <= 160 * 1024, CUEQ_ERR_TOO_LARGE, "linear_rows: the weight blocks of one launch do not fit the local data share");
+  const int64_t total = ((M + 31) / 32) * nparts;
+  int64_t gx = (total + kLrWaves - 1) / kLrWaves;
+  if (gx > device_cus()) gx = device_cus();
+  KernelTimer timer("linear_rows", stream);
+#define LR(KT_, NT_)                                                                                                                          \
+  do {                                                                                                                                        \
+    auto kfn = linear_rows_kernel<KT_, NT_>;                                                                                                  \
+    CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(64 * kLrWaves), lds, stream, static_cast<const uint16_t*>(A), lda,          \
+                       static_cast<const uint16_t*>(W), parts, nslots, static_cast<int>(nparts), w_contraction_major,                         \
+                       static_cast<uint16_t*>(C), ldc, static_cast<int>(M), static_cast<float>(alpha));                                       \
+  } while (0)
+#define LR_N(KT_)                                                                        \
+  switch (N / 32) { case 1: LR(KT_, 1); break; case 2: LR(KT_, 2); break; case 3: LR(KT_, 3); break; default: LR(KT_, 4); break; }
+  switch (K / 32) {
+    case 1: LR_N(1); break;
+    case 2: LR_N(2); break;
+    case 3: LR_N(3); break;
+    default: LR_N(4); break;
+  }
+#undef LR_N
+#undef LR
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}

@@ -207,11 +207,28 @@ def _merged_tables(mod: "SegmentedPolynomialDense", device: torch.device):
         if ok:
             hit = [(K, N, coeff,
                     torch.tensor([(p.a_off, p.w_off, p.c_off) for p in plist], dtype=torch.int64, device=device),
-                    torch.tensor([(p.c_off, p.w_off, p.a_off) for p in plist], dtype=torch.int64, device=device))
+                    torch.tensor([(p.c_off, p.w_off, p.a_off) for p in plist], dtype=torch.int64, device=device),
+                    _rows_tables(K, N, plist))
                    for (K, N, coeff), plist in by.items()]
         mod._merged[key] = hit if hit is not None else False
         return hit
     return hit or None
+
+
+def _rows_tables(K: int, N: int, plist):
+    """Host tables ``(forward, input gradient)`` for the row-streaming launch (``cueq_linear_rows``: every distinct weight
+    block of the launch resident in the local data share), or ``None`` where its limits do not hold."""
+    slots = len({p.w_off for p in plist})
+    if K not in (32, 64, 96, 128) or N not in (32, 64, 96, 128) or len(plist) > 48 or slots > 8:
+        return None
+
+    def fits(cols, contraction):
+        return slots * cols * (2 * contraction + 16) + 8 * 32 * (2 * min(cols, 64) + 16) <= 160 * 1024
+
+    if not (fits(N, K) and fits(K, N)):
+        return None
+    flat = lambda rows: (C.c_int64 * (3 * len(rows)))(*[v for r in rows for v in r])
+    return flat([(p.a_off, p.w_off, p.c_off) for p in plist]), flat([(p.c_off, p.w_off, p.a_off) for p in plist])
 
 
 def _vector_rows(*tensors) -> bool:
@@ -224,8 +241,15 @@ def _run_merged(dtype, A, B, Cout, launches, forward: bool):
     lib = _lib.load()
     stream = torch.cuda.current_stream(A.device).cuda_stream
     code = _DTYPE_CODE[dtype]
-    for K, N, coeff, fwd_tab, dx_tab in launches:
-        if forward:
+    for K, N, coeff, fwd_tab, dx_tab, rows in launches:
+        if rows is not None and dtype == torch.bfloat16:
+            if forward:
+                _lib.check(lib.cueq_linear_rows(code, 1, A.shape[0], N, K, A.data_ptr(), A.stride(0), B.data_ptr(), B.numel(), Cout.data_ptr(),
+                                                Cout.stride(0), rows[0], fwd_tab.shape[0], coeff, stream), "cueq_linear_rows")
+            else:
+                _lib.check(lib.cueq_linear_rows(code, 0, A.shape[0], K, N, A.data_ptr(), A.stride(0), B.data_ptr(), B.numel(), Cout.data_ptr(),
+                                                Cout.stride(0), rows[1], dx_tab.shape[0], coeff, stream), "cueq_linear_rows")
+        elif forward:
             _lib.check(lib.cueq_gemm_table(code, code, 0, 1, A.shape[0], N, K, A.data_ptr(), A.stride(0), B.data_ptr(), N,
                                            Cout.data_ptr(), Cout.stride(0), fwd_tab.data_ptr(), fwd_tab.shape[0], 1, 0, coeff, 0, stream),
                        "cueq_gemm_table")
