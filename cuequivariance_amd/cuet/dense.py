@@ -216,19 +216,35 @@ def _merged_tables(mod: "SegmentedPolynomialDense", device: torch.device):
 
 
 def _rows_tables(K: int, N: int, plist):
-    """Host tables ``(forward, input gradient)`` for the row-streaming launch (``cueq_linear_rows``: every distinct weight
-    block of the launch resident in the local data share), or ``None`` where its limits do not hold."""
-    slots = len({p.w_off for p in plist})
-    if K not in (32, 64, 96, 128) or N not in (32, 64, 96, 128) or len(plist) > 48 or slots > 8:
-        return None
-
-    def fits(cols, contraction):
-        return slots * cols * (2 * contraction + 16) + 8 * 32 * (2 * min(cols, 64) + 16) <= 160 * 1024
-
-    if not (fits(N, K) and fits(K, N)):
+    """Host tables for the row-streaming launch (``cueq_linear_rows``: every distinct weight block of a launch resident in
+    the local data share): per element size a list of launches ``(forward table, input-gradient table, parts)``, the parts
+    dealt out so that the weight blocks of one launch fit - or ``None`` where the launch's limits do not hold."""
+    if K not in (32, 64, 96, 128) or N not in (32, 64, 96, 128):
         return None
     flat = lambda rows: (C.c_int64 * (3 * len(rows)))(*[v for r in rows for v in r])
-    return flat([(p.a_off, p.w_off, p.c_off) for p in plist]), flat([(p.c_off, p.w_off, p.a_off) for p in plist])
+    out = {}
+    for es in (2, 4):
+        room = 160 * 1024 - 8 * 32 * 144  # what the staging tiles of the eight wavefronts leave
+        per_block = max(N * (es * K + 16), K * (es * N + 16))  # forward / input gradient
+        cap = min(8, room // per_block)
+        if cap < 1:
+            return None
+        groups, blocks = [], {}
+        for p in plist:  # parts of one weight block stay together
+            blocks.setdefault(p.w_off, []).append(p)
+        cur = []
+        for w_off, ps in blocks.items():
+            if cur and (len({q.w_off for q in cur}) + 1 > cap or len(cur) + len(ps) > 48):
+                groups.append(cur)
+                cur = []
+            cur = cur + ps
+            while len(cur) > 48:
+                groups.append(cur[:48])
+                cur = cur[48:]
+        if cur:
+            groups.append(cur)
+        out[es] = [(flat([(p.a_off, p.w_off, p.c_off) for p in g]), flat([(p.c_off, p.w_off, p.a_off) for p in g]), len(g)) for g in groups]
+    return out
 
 
 def _vector_rows(*tensors) -> bool:
@@ -242,13 +258,14 @@ def _run_merged(dtype, A, B, Cout, launches, forward: bool):
     stream = torch.cuda.current_stream(A.device).cuda_stream
     code = _DTYPE_CODE[dtype]
     for K, N, coeff, fwd_tab, dx_tab, rows in launches:
-        if rows is not None and dtype == torch.bfloat16:
-            if forward:
-                _lib.check(lib.cueq_linear_rows(code, 1, A.shape[0], N, K, A.data_ptr(), A.stride(0), B.data_ptr(), B.numel(), Cout.data_ptr(),
-                                                Cout.stride(0), rows[0], fwd_tab.shape[0], coeff, stream), "cueq_linear_rows")
-            else:
-                _lib.check(lib.cueq_linear_rows(code, 0, A.shape[0], K, N, A.data_ptr(), A.stride(0), B.data_ptr(), B.numel(), Cout.data_ptr(),
-                                                Cout.stride(0), rows[1], dx_tab.shape[0], coeff, stream), "cueq_linear_rows")
+        if rows is not None and dtype in (torch.bfloat16, torch.float32):
+            for fwd_host, dx_host, nparts in rows[A.element_size()]:
+                if forward:
+                    _lib.check(lib.cueq_linear_rows(code, 1, A.shape[0], N, K, A.data_ptr(), A.stride(0), B.data_ptr(), B.numel(), Cout.data_ptr(),
+                                                    Cout.stride(0), fwd_host, nparts, coeff, stream), "cueq_linear_rows")
+                else:
+                    _lib.check(lib.cueq_linear_rows(code, 0, A.shape[0], K, N, A.data_ptr(), A.stride(0), B.data_ptr(), B.numel(), Cout.data_ptr(),
+                                                    Cout.stride(0), dx_host, nparts, coeff, stream), "cueq_linear_rows")
         elif forward:
             _lib.check(lib.cueq_gemm_table(code, code, 0, 1, A.shape[0], N, K, A.data_ptr(), A.stride(0), B.data_ptr(), N,
                                            Cout.data_ptr(), Cout.stride(0), fwd_tab.data_ptr(), fwd_tab.shape[0], 1, 0, coeff, 0, stream),

@@ -261,15 +261,15 @@ int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_
                     const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc, const int64_t* table,
                     int64_t nparts, int64_t k_chunks, int64_t chunk_stride_c, double alpha, int32_t accumulate, void* stream);
 
-/* Row-streaming form of the same product for a 2-byte type, meant for the forward and the input gradient of Linear
+/* Row-streaming form of the same product, meant for the forward and the input gradient of Linear
  * (descriptor uv,iu,iv per irrep; FusedTensorProductOp3, primitives/segmented_polynomial_fused_tp.py:40-48):
  *   C[z, c_p : c_p + N] = alpha * A[z, a_p : a_p + K] . W_p      for all rows z < M and the parts p of the table,
  * where W_p = W + w_p is K x N as it lies (w_contraction_major != 0) or N x K (w_contraction_major == 0).  table: HOST
- * memory, nparts rows of (a_p, w_p, c_p) in elements, multiples of 8, inside a row resp. the w_numel elements of W; the parts
- * must write disjoint columns.
+ * memory, nparts rows of (a_p, w_p, c_p) in elements, multiples of 16 bytes, inside a row resp. the w_numel elements of W;
+ * the parts must write disjoint columns.  dtype: bfloat16 or float32 (A, W and C alike; float32 accumulation).
  * All distinct weight blocks of the launch stay in the local data share: K, N in {32, 64, 96, 128}, at most 8 distinct
- * blocks and 48 parts, (blocks * N * (2 K + 16) + 8 * 32 * (2 * min(N, 64) + 16)) bytes <= 160 KiB, else
- * CUEQ_ERR_TOO_LARGE / CUEQ_ERR_UNSUPPORTED (the caller then takes cueq_gemm_table).  bfloat16 only. */
+ * blocks and 48 parts, (blocks * N * (K * element size + 16) + 36 864) bytes <= 160 KiB, else CUEQ_ERR_TOO_LARGE /
+ * CUEQ_ERR_UNSUPPORTED (the caller then splits the parts over several launches or takes cueq_gemm_table). */
 int cueq_linear_rows(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
                      const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts, double alpha, void* stream);
 
