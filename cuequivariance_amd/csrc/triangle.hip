@@ -1823,6 +1823,249 @@ __global__ void __launch_bounds__(256) ln_t_bwd_kernel(const T* __restrict__ dy,
 }
 
 // ------------------------------------------------------------------------------------------------
+// The same two kernels for 2-byte types and D = 64 or 128 without a block-wide step: a wavefront takes 64 consecutive
+// m (128-byte pieces of the rows of x_t); lane (cp, dh) owns the column pair (2 cp, 2 cp + 1) for the half dh of d and
+// reads x_t as one dword per d (two whole lines per instruction, addressed as a base that is the same for all lanes +
+// a 32-bit lane offset that also carries the distance between the halves).  The statistics are sums over a lane's own
+// registers completed by one exchange between the lane halves.  Rows of y (forward) and of dy (backward) pass through a
+// staging tile private to the wavefront, so global memory sees whole 256-byte rows; dx_t leaves as dwords, 128
+// contiguous bytes per d.  Staging rows are stored pair-member-major (row 32 j + cp for column 2 cp + j): 16-byte
+// accesses of consecutive lanes fall into distinct banks.  The forward keeps a second tile in flight.  The backward
+// here computes the gradient of the tensor only; with the affine gradients asked for the kernel above runs.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float lo_bf16(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float hi_bf16(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+// The value again, as far as the compiler can tell a new one: the two floats of a packed pair are then unpacked where they
+// are used instead of being kept, one register each, from the first pass over the data to the last.
+__device__ __forceinline__ uint32_t again(uint32_t w) {
+  asm volatile("" : "+v"(w));
+  return w;
+}
+template <typename V>
+__device__ __forceinline__ void store_global(char* uniform_base, uint32_t lane_offset, V value) {
+  typedef __attribute__((address_space(1))) V* gptr;
+  *reinterpret_cast<gptr>(reinterpret_cast<uint64_t>(uniform_base) + lane_offset) = value;
+}
+
+template <typename V>
+__device__ __forceinline__ V load_global_stream(const char* uniform_base, uint32_t lane_offset) {
+  typedef const __attribute__((address_space(1))) V* gptr;
+  return __builtin_nontemporal_load(reinterpret_cast<gptr>(reinterpret_cast<uint64_t>(uniform_base) + lane_offset));
+}
+
+template <int D>
+struct LnCols {
+  static constexpr int H = D / 2;           // values of d per lane
+  static constexpr int RS = 2 * D + 16;     // bytes between staged rows
+  static constexpr int WAVE_LDS = 64 * RS;  // 64 rows (columns m of the tile)
+};
+
+// the H dwords of lane (cp, dh) for the tile at column m0 (which every lane of the wavefront shares); LAST: nothing reads
+// x_t after this kernel (the backward: marked as a stream 45 instead of 47 us; in the forward, which reads what the
+// contraction has just written, the mark costs 9 us)
+template <int D, bool LAST = false>
+__device__ __forceinline__ void lncols_request(uint32_t (&xv)[D / 2], const uint16_t* xt, int64_t m0, int64_t row_bytes, uint32_t voff) {
+  // (one scalar base that walks down the rows; the scheduling barriers keep every address next to its load - computed
+  // all at once, the D / 2 bases would not fit the scalar registers)
+  const char* src = uniform_ptr(xt + m0);
+#pragma unroll
+  for (int i = 0; i < D / 2; ++i) {
+    xv[i] = LAST ? load_global_stream<uint32_t>(src, voff) : load_global<uint32_t>(src, voff);
+    src += row_bytes;
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+template <int D>
+__global__ void __launch_bounds__(256, 2) ln_t_fwd_cols_kernel(const uint16_t* __restrict__ xt, const uint16_t* __restrict__ gamma,
+                                                               const uint16_t* __restrict__ beta, uint16_t* __restrict__ y, float* __restrict__ mean,
+                                                               float* __restrict__ rstd, int64_t M, float eps) {
+  using L = LnCols<D>;
+  constexpr int H = L::H, RS = L::RS;
+  extern __shared__ __align__(16) char lntc_dyn[];  // 4 wavefronts x WAVE_LDS
+  __shared__ __align__(16) float sgam[D], sbet[D];
+  const int tid = threadIdx.x, lane = tid & 63, cp = lane & 31, dh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (tid < D) {
+    sgam[tid] = gamma ? tri_load(gamma, tid) : 1.0f;
+    sbet[tid] = beta ? tri_load(beta, tid) : 0.0f;
+  }
+  __syncthreads();
+  char* stage = lntc_dyn + wave * L::WAVE_LDS;
+  const int64_t ntiles = (M + 63) / 64;
+  const int64_t nw = static_cast<int64_t>(gridDim.x) * 4;
+  const int64_t row_bytes = 2 * M;
+  const float* gam = sgam + dh * H;
+  const float* bet = sbet + dh * H;
+  // columns past M (only in the last tile; M is even, so a pair is in or out as a whole) read the tile's first pair
+  auto lane_offset = [&](int64_t tile) -> uint32_t {
+    return static_cast<uint32_t>(dh * (H * row_bytes)) + (tile * 64 + 2 * cp < M ? 4u * cp : 0u);
+  };
+  auto work = [&](const uint32_t (&xv)[H], int64_t tile) {
+    asm volatile("" ::: "memory");  // gamma / beta are read from LDS again for every tile, not kept in 2 D registers
+    const int64_t m0 = tile * 64;
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < H; ++i) { s0 += lo_bf16(xv[i]); s1 += hi_bf16(xv[i]); }
+    s0 += __shfl_xor(s0, 32, 64);
+    s1 += __shfl_xor(s1, 32, 64);
+    const float mu0 = s0 * (1.0f / D), mu1 = s1 * (1.0f / D);
+    float q0 = 0.f, q1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < H; ++i) {
+      const uint32_t w = again(xv[i]);
+      const float c0 = lo_bf16(w) - mu0, c1 = hi_bf16(w) - mu1;
+      q0 = fmaf(c0, c0, q0);
+      q1 = fmaf(c1, c1, q1);
+    }
+    q0 += __shfl_xor(q0, 32, 64);
+    q1 += __shfl_xor(q1, 32, 64);
+    const float r0 = rsqrtf(q0 * (1.0f / D) + eps), r1 = rsqrtf(q1 * (1.0f / D) + eps);
+    if (dh == 0 && m0 + 2 * cp < M) {
+      *reinterpret_cast<float2*>(mean + m0 + 2 * cp) = make_float2(mu0, mu1);
+      *reinterpret_cast<float2*>(rstd + m0 + 2 * cp) = make_float2(r0, r1);
+    }
+#pragma unroll
+    for (int p = 0; p < H / 8; ++p) {
+      uint32_t w0[4], w1[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = p * 8 + 2 * e;
+        const float ga = gam[i], gb = gam[i + 1], ba = bet[i], bb = bet[i + 1];
+        const uint32_t xa_ = again(xv[i]), xb_ = again(xv[i + 1]);
+        w0[e] = pack_bf16((lo_bf16(xa_) - mu0) * r0 * ga + ba, (lo_bf16(xb_) - mu0) * r0 * gb + bb);
+        w1[e] = pack_bf16((hi_bf16(xa_) - mu1) * r1 * ga + ba, (hi_bf16(xb_) - mu1) * r1 * gb + bb);
+      }
+      *reinterpret_cast<uint4*>(stage + cp * RS + dh * D + p * 16) = make_uint4(w0[0], w0[1], w0[2], w0[3]);
+      *reinterpret_cast<uint4*>(stage + (32 + cp) * RS + dh * D + p * 16) = make_uint4(w1[0], w1[1], w1[2], w1[3]);
+      __builtin_amdgcn_sched_barrier(0);  // one group of eight d at a time: its gamma / beta values die here
+    }
+    char* dst = const_cast<char*>(uniform_ptr(y + m0 * D));
+#pragma unroll
+    for (int i = 0; i < D / 8; ++i) {  // 64 rows of D / 8 vectors
+      const int idx = lane + 64 * i;
+      const int r = idx / (D / 8), v = idx % (D / 8);
+      const int mm = 2 * (r & 31) + (r >> 5);
+      if (m0 + mm < M) {
+        const uint4 val = *reinterpret_cast<const uint4*>(stage + r * RS + v * 16);
+        store_global<u32x4_t>(dst, static_cast<uint32_t>(mm * (2 * D) + v * 16), u32x4_t{val.x, val.y, val.z, val.w});
+      }
+    }
+  };
+  // two register sets: while one tile is worked on, the next one's rows are in flight (the loop body is two tiles
+  // without a branch in between)
+  int64_t tile = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+  if (tile >= ntiles) return;
+  const int64_t mine = (ntiles - tile + nw - 1) / nw;
+  uint32_t xa[H], xb[H];
+  auto clamp = [&](int64_t t) { return t < ntiles ? t : ntiles - 1; };  // past the end: the last tile again, not used
+  lncols_request<D>(xa, xt, clamp(tile) * 64, row_bytes, lane_offset(clamp(tile)));
+  lncols_request<D>(xb, xt, clamp(tile + nw) * 64, row_bytes, lane_offset(clamp(tile + nw)));
+  for (int64_t it = 0; it < mine / 2; ++it) {
+    work(xa, tile);
+    lncols_request<D>(xa, xt, clamp(tile + 2 * nw) * 64, row_bytes, lane_offset(clamp(tile + 2 * nw)));
+    __builtin_amdgcn_sched_barrier(0);
+    work(xb, tile + nw);
+    lncols_request<D>(xb, xt, clamp(tile + 3 * nw) * 64, row_bytes, lane_offset(clamp(tile + 3 * nw)));
+    __builtin_amdgcn_sched_barrier(0);
+    tile += 2 * nw;
+  }
+  if (mine % 2) work(xa, tile);
+}
+
+template <int D>
+__global__ void __launch_bounds__(256, 2) ln_t_bwd_cols_kernel(const uint16_t* __restrict__ dy, const uint16_t* __restrict__ xt,
+                                                               const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                               const uint16_t* __restrict__ gamma, uint16_t* __restrict__ dxt, int64_t M) {
+  using L = LnCols<D>;
+  constexpr int H = L::H, RS = L::RS;
+  extern __shared__ __align__(16) char lntc_dyn[];  // 4 wavefronts x WAVE_LDS
+  __shared__ __align__(16) float sgam[D];
+  const int tid = threadIdx.x, lane = tid & 63, cp = lane & 31, dh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (tid < D) sgam[tid] = gamma ? tri_load(gamma, tid) : 1.0f;
+  __syncthreads();
+  char* stage = lntc_dyn + wave * L::WAVE_LDS;
+  const int64_t ntiles = (M + 63) / 64;
+  const int64_t nw = static_cast<int64_t>(gridDim.x) * 4;
+  const int64_t row_bytes = 2 * M;
+  const float* gam = sgam + dh * H;
+  for (int64_t tile = static_cast<int64_t>(blockIdx.x) * 4 + wave; tile < ntiles; tile += nw) {
+    asm volatile("" ::: "memory");  // gamma is read from LDS again for every tile, not kept in D registers
+    const int64_t m0 = tile * 64;
+    const bool ok = m0 + 2 * cp < M;
+    const uint32_t voff = static_cast<uint32_t>(dh * (H * row_bytes)) + (ok ? 4u * cp : 0u);
+    uint32_t xv[H];
+    lncols_request<D, true>(xv, xt, m0, row_bytes, voff);
+    // the 64 rows of dy as they lie (D / 8 lanes per row) into the staging tile
+    {
+      const char* src = uniform_ptr(dy + m0 * D);
+      uint4 raw[D / 8];
+#pragma unroll
+      for (int i = 0; i < D / 8; ++i) {
+        const int idx = lane + 64 * i;
+        const int r = idx / (D / 8), v = idx % (D / 8);
+        const int rr = m0 + r < M ? r : 0;  // rows past the end: the tile's first row again, not used
+        raw[i] = load_global<uint4>(src, static_cast<uint32_t>(rr * (2 * D) + v * 16));
+      }
+      __builtin_amdgcn_sched_barrier(0);  // all requests first
+#pragma unroll
+      for (int i = 0; i < D / 8; ++i) {
+        const int idx = lane + 64 * i;
+        const int r = idx / (D / 8), v = idx % (D / 8);
+        *reinterpret_cast<uint4*>(stage + ((r & 1) * 32 + (r >> 1)) * RS + v * 16) = raw[i];
+      }
+    }
+    const float2 mu = ok ? *reinterpret_cast<const float2*>(mean + m0 + 2 * cp) : make_float2(0.f, 0.f);
+    const float2 rs = ok ? *reinterpret_cast<const float2*>(rstd + m0 + 2 * cp) : make_float2(0.f, 0.f);
+    uint4 dv[2][H / 8];  // this lane's half of its two dy rows, packed along d
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int p = 0; p < H / 8; ++p) dv[j][p] = *reinterpret_cast<const uint4*>(stage + (j * 32 + cp) * RS + dh * D + p * 16);
+    auto dy_at = [&](int j, int i) -> float {  // value i of the lane's half
+      const uint4 q = dv[j][i >> 3];
+      const uint32_t w = ((i >> 1) & 3) == 0 ? q.x : ((i >> 1) & 3) == 1 ? q.y : ((i >> 1) & 3) == 2 ? q.z : q.w;
+      return (i & 1) ? hi_bf16(w) : lo_bf16(w);
+    };
+    auto dy_at2 = [&](int j, int i) -> float {  // the same for the second pass
+      const uint4 q = dv[j][i >> 3];
+      const uint32_t w = again(((i >> 1) & 3) == 0 ? q.x : ((i >> 1) & 3) == 1 ? q.y : ((i >> 1) & 3) == 2 ? q.z : q.w);
+      return (i & 1) ? hi_bf16(w) : lo_bf16(w);
+    };
+    float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < H; ++i) {
+      const float g = gam[i];
+      const float g0 = dy_at(0, i) * g, g1 = dy_at(1, i) * g;
+      a0 += g0;
+      a1 += g1;
+      b0 = fmaf(g0, (lo_bf16(xv[i]) - mu.x) * rs.x, b0);
+      b1 = fmaf(g1, (hi_bf16(xv[i]) - mu.y) * rs.y, b1);
+      if (i % 8 == 7) __builtin_amdgcn_sched_barrier(0);
+    }
+    a0 += __shfl_xor(a0, 32, 64);
+    a1 += __shfl_xor(a1, 32, 64);
+    b0 += __shfl_xor(b0, 32, 64);
+    b1 += __shfl_xor(b1, 32, 64);
+    const float k10 = a0 * (1.0f / D), k11 = a1 * (1.0f / D), k20 = b0 * (1.0f / D), k21 = b1 * (1.0f / D);
+    if (ok) {
+      char* dst = const_cast<char*>(uniform_ptr(dxt + m0));
+#pragma unroll
+      for (int i = 0; i < H; ++i) {
+        const float g = gam[i];
+        const uint32_t w = again(xv[i]);
+        const float xh0 = (lo_bf16(w) - mu.x) * rs.x, xh1 = (hi_bf16(w) - mu.y) * rs.y;
+        const float o0 = rs.x * (dy_at2(0, i) * g - k10 - xh0 * k20), o1 = rs.y * (dy_at2(1, i) * g - k11 - xh1 * k21);
+        store_global<uint32_t>(dst, voff, pack_bf16(o0, o1));
+        dst += row_bytes;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // gate: out[r][c] = sigmoid(u + bu) * (v + bv) * mask;  biases and mask are indexed by row (axis 0) or column (axis 1)
 // ------------------------------------------------------------------------------------------------
 template <typename T>
@@ -2438,6 +2681,25 @@ extern "C" int cueq_layer_norm_t_fwd(int32_t dtype, int64_t M, int64_t D, const 
   CUEQ_REQUIRE(ntiles < (1ll << 31), CUEQ_ERR_TOO_LARGE, "layer_norm_t: too many rows");
   const size_t fwd_lds = static_cast<size_t>(D) * 132;
   KernelTimer timer("layer_norm_t_fwd", stream);
+  if (dtype == CUEQ_BF16 && (D == 64 || D == 128) && D * M + 256 < (1ll << 32) &&
+      ((reinterpret_cast<uintptr_t>(mean) | reinterpret_cast<uintptr_t>(rstd)) & 7) == 0) {
+    // one lane per column pair and half of d, 64 columns per wavefront, four wavefronts per block, two blocks per CU
+    int64_t nb = (ntiles + 3) / 4;
+    if (nb > 2 * device_cus()) nb = 2 * device_cus();
+    const size_t lds = static_cast<size_t>(4 * 64) * (2 * D + 16);
+#define LNTC(DD)                                                                                                                             \
+  do {                                                                                                                                       \
+    auto kfn = ln_t_fwd_cols_kernel<DD>;                                                                                                     \
+    CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(nb)), dim3(256), lds, stream, static_cast<const uint16_t*>(x_t),                       \
+                       static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, M,    \
+                       static_cast<float>(eps));                                                                                             \
+  } while (0)
+    if (D == 64) LNTC(64); else LNTC(128);
+#undef LNTC
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
   TRI_DISPATCH(dtype,
                hipLaunchKernelGGL(ln_t_fwd_kernel<float>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const float*>(x_t), static_cast<const float*>(gamma), static_cast<const float*>(beta), static_cast<float*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)),
                hipLaunchKernelGGL(ln_t_fwd_kernel<uint16_t>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const uint16_t*>(x_t), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)));
@@ -2477,6 +2739,25 @@ extern "C" int cueq_layer_norm_t_bwd(int32_t dtype, int64_t M, int64_t D, const 
   const int64_t nb = ln_t_bwd_blocks(dtype, M);
   float* part = static_cast<float*>(workspace);
   const int64_t es = dtype == CUEQ_F32 ? 4 : 2;
+  if (dtype == CUEQ_BF16 && !need_affine && (D == 64 || D == 128) && D * M + 256 < (1ll << 32) &&
+      ((reinterpret_cast<uintptr_t>(mean) | reinterpret_cast<uintptr_t>(rstd)) & 7) == 0) {
+    // one lane per column pair and half of d, 64 columns per wavefront, four wavefronts per block, two blocks per CU
+    int64_t nbc = (ntiles + 3) / 4;
+    if (nbc > 2 * device_cus()) nbc = 2 * device_cus();
+    const size_t lds = static_cast<size_t>(4 * 64) * (2 * D + 16);
+    KernelTimer timer("layer_norm_t_bwd", stream);
+#define LNTC(DD)                                                                                                                             \
+  do {                                                                                                                                       \
+    auto kfn = ln_t_bwd_cols_kernel<DD>;                                                                                                     \
+    CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(nbc)), dim3(256), lds, stream, static_cast<const uint16_t*>(dy),                       \
+                       static_cast<const uint16_t*>(x_t), mean, rstd, static_cast<const uint16_t*>(gamma), static_cast<uint16_t*>(dx_t), M); \
+  } while (0)
+    if (D == 64) LNTC(64); else LNTC(128);
+#undef LNTC
+    CUEQ_CHECK_HIP(hipGetLastError());
+    return CUEQ_OK;
+  }
   const size_t bwd_lds = static_cast<size_t>(((D * 132 + 15) & ~15ll) + mt * (D * es + 4));
   {
     KernelTimer timer("layer_norm_t_bwd", stream);

@@ -108,6 +108,36 @@ def test_hip_path_matches_oracle(device, dtype, direction, shape):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("need_affine", [False, True])
+@pytest.mark.parametrize("D,M", [(128, 64), (128, 72), (64, 8), (128, 8 * 1001), (64, 64 * 2048 * 2 + 64 * 700 + 24), (128, 64 * 2048 * 3 + 8),
+                                 (96, 4104)])
+def test_layer_norm_with_layout_change_against_torch(device, D, M, need_affine):
+    """``cueq_layer_norm_t_fwd / _bwd`` in bfloat16 on their own (the kernels with one lane per column pair for D = 64 / 128 and
+    the tile kernel for other D and for the affine gradients): ragged last tiles, one to three tiles per wavefront, against
+    ``F.layer_norm`` in float64 on the same bfloat16 values.  Tolerance 2^-7 of ``max|ref|`` (one rounding of the result)."""
+    from cuequivariance_amd.cuet import triangle as tri
+
+    g = torch.Generator(device=device).manual_seed(D + M)
+    xt = (torch.randn(D, M, device=device, generator=g) * 1.7 + 0.3).bfloat16()
+    gamma = (torch.randn(D, device=device, generator=g) * 0.5 + 1.0).bfloat16()
+    beta = torch.randn(D, device=device, generator=g).bfloat16()
+    dy = torch.randn(M, D, device=device, generator=g).bfloat16()
+    y, mean, rstd = tri.layer_norm_t_fwd(xt, gamma, beta, 1e-5)
+    dxt, dgamma, dbeta = tri.layer_norm_t_bwd(dy, xt, mean, rstd, gamma, need_affine)
+    x64 = xt.double().t().contiguous().requires_grad_(True)
+    g64, b64 = gamma.double().requires_grad_(True), beta.double().requires_grad_(True)
+    ref = F.layer_norm(x64, (D,), g64, b64, 1e-5)
+    rx, rg, rb = torch.autograd.grad(ref, [x64, g64, b64], dy.double())
+    tol = 2.0 ** -7
+    assert (y.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
+    assert (mean.double() - x64.mean(1)).abs().max().item() <= 1e-5
+    assert (dxt.double().t() - rx).abs().max().item() <= tol * rx.abs().max().item()
+    if need_affine:
+        assert (dgamma.double() - rg).abs().max().item() <= 1e-3 * rg.abs().max().item()
+        assert (dbeta.double() - rb).abs().max().item() <= 1e-3 * rb.abs().max().item()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21), (160, 512, 256, 96),
