@@ -191,18 +191,33 @@ __global__ void __launch_bounds__(64 * kLrWaves, 1)
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
+  // the weight blocks into LDS, 16-byte vectors requested in batches of four before the first is stored (one wait per
+  // batch instead of one per vector)
+  constexpr int NTH = 64 * kLrWaves;
   for (int s = 0; s < nslots; ++s) {
     const TI* w = W + parts.w_off[s];
     char* dst = smem + s * (N * WRS);
-    if (w_contraction_major) {  // K x N as it lies: element (k, n) becomes column k of row n
-      for (int e = tid; e < K * N; e += 64 * kLrWaves) {
-        const int k = e / N, n = e % N;
-        *reinterpret_cast<TI*>(dst + n * WRS + ES * k) = w[e];
-      }
-    } else {  // N x K as it lies
-      for (int e = tid; e < N * (K / EPV); e += 64 * kLrWaves) {
-        const int n = e / (K / EPV), v = e % (K / EPV);
-        *reinterpret_cast<uint4*>(dst + n * WRS + 16 * v) = *reinterpret_cast<const uint4*>(w + n * K + EPV * v);
+    constexpr int NVEC = K * N / EPV;  // vectors of the block
+    for (int e0 = tid; e0 < NVEC; e0 += 4 * NTH) {
+      uint4 v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const uint4*>(w + static_cast<int64_t>(e0 + j * NTH < NVEC ? e0 + j * NTH : e0) * EPV);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int e = e0 + j * NTH;
+        if (e >= NVEC) continue;
+        if (w_contraction_major) {  // K x N as it lies: the vector holds (k, n .. n + EPV - 1), which become column k of EPV rows
+          const int k = e / (N / EPV), n = (e % (N / EPV)) * EPV;
+          const uint32_t q[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+          for (int i = 0; i < EPV; ++i) {
+            if constexpr (ES == 4) *reinterpret_cast<uint32_t*>(dst + (n + i) * WRS + 4 * k) = q[i];
+            else *reinterpret_cast<uint16_t*>(dst + (n + i) * WRS + 2 * k) = static_cast<uint16_t>(q[i >> 1] >> (16 * (i & 1)));
+          }
+        } else {  // N x K as it lies
+          const int n = e / (K / EPV), vv = e % (K / EPV);
+          *reinterpret_cast<uint4*>(dst + n * WRS + 16 * vv) = v[j];
+        }
       }
     }
   }
