@@ -67,6 +67,8 @@ def _reference(A, W, parts, K, N, contraction_major, alpha, ldc):
         (65, 96, 64, 3, 4),
         (50_000, 128, 32, 2, 6),
         (1, 32, 128, 1, 2),
+        (200, 64, 64, 2, 40),  # more parts than a block has wavefronts
+        (40, 128, 128, 3, 48),  # the most parts a launch takes, fewer units than wavefronts
     ],
 )
 def test_linear_rows_against_float64_product(device, dtype, contraction_major, M, K, N, nblocks, nparts):
@@ -78,7 +80,7 @@ def test_linear_rows_against_float64_product(device, dtype, contraction_major, M
     A = torch.randn(M, lda, device=device, generator=g).to(dtype)
     W = torch.randn(nblocks * K * N + 8, device=device, generator=g).to(dtype)
     # parts in scrambled column order, weight blocks shared between parts
-    parts = [(((3 * p + 1) % nparts) * K, (p % nblocks) * K * N, ((5 * p + 2) % nparts) * N + 16) for p in range(nparts)]
+    parts = [(((p + 1) % nparts) * K, (p % nblocks) * K * N, (nparts - 1 - p) * N + 16) for p in range(nparts)]
     assert len({p[2] for p in parts}) == nparts
     out = torch.full((M, ldc), 7.0, device=device).to(dtype)
     alpha = 0.37
