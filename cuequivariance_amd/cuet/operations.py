@@ -24,7 +24,7 @@ import torch
 from .. import cue
 from ..cue import descriptors
 from .segmented_polynomial import SegmentedPolynomial
-from .transpose import TransposeIrrepsLayout
+from .transpose import TransposeIrrepsLayout, apply_layout
 
 __all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear", "SymmetricContraction", "SphericalHarmonics"]
 
@@ -189,8 +189,8 @@ class ChannelWiseTensorProduct(torch.nn.Module):
         indices_out: Optional[torch.Tensor] = None,
         size_out: Optional[int] = None,
     ) -> torch.Tensor:
-        x1 = self.transpose_in1(x1)
-        x2 = self.transpose_in2(x2)
+        x1 = apply_layout(self.transpose_in1, x1)
+        x2 = apply_layout(self.transpose_in2, x2)
         indices_in: Dict[int, torch.Tensor] = {}
         if indices_1 is not None:
             indices_in[1] = indices_1
@@ -210,7 +210,7 @@ class ChannelWiseTensorProduct(torch.nn.Module):
         elif weight is None:
             raise ValueError("Internal weights are not used, weight should not be None")
         out = self.f([weight, x1, x2], input_indices=indices_in, output_shapes=sizes_out, output_indices=indices_o)
-        return self.transpose_out(out[0])
+        return apply_layout(self.transpose_out, out[0])
 
 
 class ChannelWiseSphericalTensorProduct(torch.nn.Module):
@@ -289,7 +289,7 @@ class ChannelWiseSphericalTensorProduct(torch.nn.Module):
         torch._assert(vectors.ndim == 2 and vectors.shape[1] == 3, f"vectors must have shape (batch, 3) - got {vectors.shape}")
         if self.normalize:
             vectors = torch.nn.functional.normalize(vectors, dim=1)
-        x1 = self.transpose_in1(x1)
+        x1 = apply_layout(self.transpose_in1, x1)
         indices_in: Dict[int, torch.Tensor] = {} if indices_1 is None else {1: indices_1}
         indices_o: Dict[int, torch.Tensor] = {}
         sizes_out: Dict[int, torch.Tensor] = {}
@@ -305,7 +305,7 @@ class ChannelWiseSphericalTensorProduct(torch.nn.Module):
         elif weight is None:
             raise ValueError("Internal weights are not used, weight should not be None")
         out = self.f([weight, x1, vectors], input_indices=indices_in, output_shapes=sizes_out, output_indices=indices_o)
-        return self.transpose_out(out[0])
+        return apply_layout(self.transpose_out, out[0])
 
 
 class FullyConnectedTensorProduct(torch.nn.Module):
@@ -385,8 +385,8 @@ class FullyConnectedTensorProduct(torch.nn.Module):
                 size_out: Optional[int] = None) -> torch.Tensor:
         """``indices_1`` (rows of ``x1`` per batch element) and ``indices_out`` / ``size_out`` (output row per batch
         element, summed) are extensions over the reference's signature: gather and scatter-sum inside the kernel."""
-        x1 = self.transpose_in1(x1)
-        x2 = self.transpose_in2(x2)
+        x1 = apply_layout(self.transpose_in1, x1)
+        x2 = apply_layout(self.transpose_in2, x2)
         if self.weight is not None:
             if weight is not None:
                 raise ValueError("Internal weights are used, weight should be None")
@@ -400,16 +400,16 @@ class FullyConnectedTensorProduct(torch.nn.Module):
                 [weight, x1, x2], {} if indices_1 is None else {1: indices_1},
                 {} if indices_out is None else {0: torch.empty(size_out, 1, device="meta")},
                 {} if indices_out is None else {0: indices_out})
-            return self.transpose_out(out[0])
+            return apply_layout(self.transpose_out, out[0])
         if self.f_outer is not None and weight.shape[0] == 1:
             Z, off, parts = x1.shape[0], 0, []
             for d, u in self._outer_segments:  # ir_mul rows: (component, channel) -> (component, channel * V + v)
                 parts.append((x1[:, off:off + d * u].reshape(Z, d, u, 1) * x2.reshape(x2.shape[0], 1, 1, -1)).reshape(Z, -1))
                 off += d * u
-            return self.transpose_out(self.f_outer([weight, torch.cat(parts, 1)])[0])
+            return apply_layout(self.transpose_out, self.f_outer([weight, torch.cat(parts, 1)])[0])
         if weight.shape[0] != 1 or self.f is None:
-            return self.transpose_out(self.f_per_sample([weight, x1, x2])[0])
-        return self.transpose_out(self.f([weight, x1, x2])[0])
+            return apply_layout(self.transpose_out, self.f_per_sample([weight, x1, x2])[0])
+        return apply_layout(self.transpose_out, self.f([weight, x1, x2])[0])
 
 
 class Linear(torch.nn.Module):
@@ -486,10 +486,10 @@ class Linear(torch.nn.Module):
         if weight is None:
             raise ValueError("Weights should not be None")
         if self.method != "indexed_linear" and (input_indices or weight.shape[0] != 1):
-            out = self.f_per_sample([weight, self.transpose_in(x)], input_indices)
+            out = self.f_per_sample([weight, apply_layout(self.transpose_in, x)], input_indices)
         else:
-            out = self.f([weight, self.transpose_in(x)], input_indices=input_indices)
-        return self.transpose_out(out[0])
+            out = self.f([weight, apply_layout(self.transpose_in, x)], input_indices=input_indices)
+        return apply_layout(self.transpose_out, out[0])
 
 
 class SymmetricContraction(torch.nn.Module):
@@ -568,8 +568,8 @@ class SymmetricContraction(torch.nn.Module):
             weight = torch.einsum("zau,ab->zbu", self.weight, self.projection)
         else:
             weight = self.weight
-        out = self.f([weight.flatten(1), self.transpose_in(x)], input_indices={0: indices})
-        return self.transpose_out(out[0])
+        out = self.f([weight.flatten(1), apply_layout(self.transpose_in, x)], input_indices={0: indices})
+        return apply_layout(self.transpose_out, out[0])
 
 
 class SphericalHarmonics(torch.nn.Module):
