@@ -933,7 +933,7 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
 // The same computation for 2-byte types with the weights resident in LDS: one block per CU loads W1, W2 (C rows)
 // and the biases once, then its wavefronts walk 32-column tiles of m independently - no barrier and no weight
 // traffic inside the loop, and wavefronts of one SIMD drift into different phases (MFMA / gate math / memory).
-// LDS: 2 C (2 K + 16) bytes of weights + 8 C bytes of biases + a wave-private 8-row staging tile for the results.
+// LDS: 2 C (2 K + 16) bytes of weights + 8 C bytes of biases (+ with two inputs a wave-private 8-row staging tile for the results).
 // ------------------------------------------------------------------------------------------------
 template <int KT, bool SPLIT, bool DC_BY_ROW>
 __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
@@ -957,8 +957,9 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   char* sw2 = gbi_dsm + C * WSTR;
   float* sb = reinterpret_cast<float*>(gbi_dsm + 2 * C * WSTR);  // bias1[C], bias2[C]
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
-  char* stage = reinterpret_cast<char*>(sb + 2 * C) + wave * (8 * SSTR);
+  // (the wavefront's number as a scalar: tile indices and row bases derived from it stay in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c = lane & 31, h = lane >> 5;
+  char* stage = reinterpret_cast<char*>(sb + 2 * C) + wave * (8 * SSTR);  // (two inputs only)
 
   for (int e = tid; e < C * VPR; e += NTH) {
     const int r = e / VPR, part = e % VPR;
@@ -1017,29 +1018,30 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
     const uint32_t w = dcr[v >> 1];
     return (v & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
   };
-  // the rows of X of a tile, one row per lane, and its mask value; those of the next tile are requested a tile ahead
-  uint4 xf1[NS][2], xf2[SPLIT ? NS : 1][2], xn1[NS][2], xn2[SPLIT ? NS : 1][2];
-  float mk = 1.0f, mkn = 1.0f;
-  auto request_x = [&](int mld, uint4 (&x1)[NS][2], uint4 (&x2)[SPLIT ? NS : 1][2], float& m) {
+  // the rows of X of a tile, one row per lane, and its mask value (as stored: converted where it is used, so that the
+  // request is not followed by a wait).  The registers are free once the last chunk's first product has read them:
+  // the rows of the wavefront's next tile are requested then, and arrive while the results of this one leave.
+  uint4 xf1[NS][2], xf2[SPLIT ? NS : 1][2];
+  uint32_t mraw = 0;
+  auto request_x = [&](int mld) {
 #pragma unroll
     for (int s2 = 0; s2 < NS; ++s2)
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const int64_t o = static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES;
-        x1[s2][q] = *reinterpret_cast<const uint4*>(X1 + o);
-        if constexpr (SPLIT) x2[s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
+        xf1[s2][q] = *reinterpret_cast<const uint4*>(X1 + o);
+        if constexpr (SPLIT) xf2[s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
       }
-    if (mask) m = tri_load(mask, mld);
+    if (mask) mraw = mask[mld];
   };
   int64_t tile = ptile;
-  if (tile < ntiles) request_x(tile_row(tile), xf1, xf2, mk);
+  if (tile < ntiles) request_x(tile_row(tile));
   request_dc(dcn);
 
   for (; tile < ntiles; tile += tstep) {
     const int mrow0 = static_cast<int>(tile * 32);
     const int mcol = mrow0 + c;
-    const bool more = tile + tstep < ntiles;
-    if (more) request_x(tile_row(tile + tstep), xn1, xn2, mkn);
+    const float mk = mask ? __uint_as_float(mraw << 16) : 1.0f;
     floatx16 ax1[KT], ax2[SPLIT ? KT : 1];
 #pragma unroll
     for (int t = 0; t < KT; ++t) ax1[t] = floatx16{0};
@@ -1137,46 +1139,85 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
             const uint2 h1 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw1 + o8)));
             const uint2 l2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw2 + o)));
             const uint2 h2 = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lptr)(sw2 + o8)));
-            mma_step<TI>(ax1[ds], make_uint4(pu[4 * t], pu[4 * t + 1], pu[4 * t + 2], pu[4 * t + 3]), make_uint4(l1.x, l1.y, h1.x, h1.y));
-            mma_step<TI>(SPLIT ? ax2[ds] : ax1[ds], make_uint4(pv[4 * t], pv[4 * t + 1], pv[4 * t + 2], pv[4 * t + 3]),
-                         make_uint4(l2.x, l2.y, h2.x, h2.y));
+            const uint4 w1f = make_uint4(l1.x, l1.y, h1.x, h1.y), w2f = make_uint4(l2.x, l2.y, h2.x, h2.y);
+            const uint4 duf = make_uint4(pu[4 * t], pu[4 * t + 1], pu[4 * t + 2], pu[4 * t + 3]);
+            const uint4 dvf = make_uint4(pv[4 * t], pv[4 * t + 1], pv[4 * t + 2], pv[4 * t + 3]);
+            if constexpr (SPLIT) {  // a lane of the result holds one k and 16 values of m
+              mma_step<TI>(ax1[ds], duf, w1f);
+              mma_step<TI>(ax2[ds], dvf, w2f);
+            } else {  // the weight columns are the rows of the product: a lane holds its own m and 16 values of k
+              mma_step<TI>(ax1[ds], w1f, duf);
+              mma_step<TI>(ax1[ds], w2f, dvf);
+            }
           }
       }
     }
 
-    // results: 8 rows (one value group a) at a time through the wave-private staging tile, 16-byte row vectors out
+    // the rows of the next tile (past the end: the last tile again, so that the request is unconditional)
+    request_x(tile_row(min(tile + tstep, ntiles - 1)));
+    if constexpr (SPLIT) {
+      // Results of the two-input form (one wavefront per SIMD, nothing to add to): 8 rows (one value group a) at a time
+      // through the wave-private staging tile, whole rows out as 16-byte vectors.  (The stores from registers of the
+      // other form, 32 bytes per row and instruction, measure 5 % slower here.)
 #pragma unroll
-    for (int which = 0; which < (SPLIT ? 2 : 1); ++which) {
-      uint16_t* dst = which == 0 ? dX1 : dX2;
+      for (int which = 0; which < 2; ++which) {
+        uint16_t* dst = which == 0 ? dX1 : dX2;
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        __builtin_amdgcn_wave_barrier();
+        for (int a = 0; a < 4; ++a) {
+          __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int ds = 0; ds < KT; ++ds) {
-          const floatx16& acc = (which == 0) ? ax1[ds] : ax2[SPLIT ? ds : 0];
-          const uint32_t w01 = pack_bf16(acc[4 * a], acc[4 * a + 1]), w23 = pack_bf16(acc[4 * a + 2], acc[4 * a + 3]);
-          char* p = stage + (4 * h) * SSTR + (ds * 32 + c) * 2;
-          *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(w01 & 0xffffu);
-          *reinterpret_cast<uint16_t*>(p + SSTR) = static_cast<uint16_t>(w01 >> 16);
-          *reinterpret_cast<uint16_t*>(p + 2 * SSTR) = static_cast<uint16_t>(w23 & 0xffffu);
-          *reinterpret_cast<uint16_t*>(p + 3 * SSTR) = static_cast<uint16_t>(w23 >> 16);
+          for (int ds = 0; ds < KT; ++ds) {
+            const floatx16& acc = (which == 0) ? ax1[ds] : ax2[ds];
+            const uint32_t w01 = pack_bf16(acc[4 * a], acc[4 * a + 1]), w23 = pack_bf16(acc[4 * a + 2], acc[4 * a + 3]);
+            char* p = stage + (4 * h) * SSTR + (ds * 32 + c) * 2;
+            *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(w01 & 0xffffu);
+            *reinterpret_cast<uint16_t*>(p + SSTR) = static_cast<uint16_t>(w01 >> 16);
+            *reinterpret_cast<uint16_t*>(p + 2 * SSTR) = static_cast<uint16_t>(w23 & 0xffffu);
+            *reinterpret_cast<uint16_t*>(p + 3 * SSTR) = static_cast<uint16_t>(w23 >> 16);
+          }
+          __builtin_amdgcn_wave_barrier();
+          const int r0 = mrow0 + 8 * a;
+          const int rows = min(8, M - r0);
+          if (rows > 0) stage_flush<TI, K>(stage, SSTR, rows, dst + static_cast<int64_t>(r0) * lddx, lddx, lane, 64, false);
         }
-        __builtin_amdgcn_wave_barrier();
-        const int r0 = mrow0 + 8 * a;
-        const int rows = min(8, M - r0);
-        if (rows > 0)
-          stage_flush<TI, K>(stage, SSTR, rows, dst + static_cast<int64_t>(r0) * lddx, lddx, lane, 64, which == 0 && accumulate != 0);
       }
-    }
-    if (more) {
+    } else {
+      // Results of the one-input form.  A lane holds row m = mrow0 + c and, per 32 columns, k = 8 (v >> 2) + 4 h + (v & 3):
+      // the lane halves swap register pairs (v_permlane32_swap: lanes 32-63 of the first register with lanes 0-31 of the
+      // second), after which the lower half has k 0-7 and the upper half k 8-15 of every 16 columns - 16 contiguous bytes
+      // per lane, 32 per row and instruction, straight from the registers.  What the results are added to is requested
+      // first, in the same shape, all of it at once.  All vectors are formed before the first of them is stored.
+      const int mrow = mrow0 + c;
+      const int64_t orow = static_cast<int64_t>(min(mrow, M - 1)) * lddx + (h * 16) / ES;
+      uint4 old[KT][2];
+      if (accumulate) {
 #pragma unroll
-      for (int s2 = 0; s2 < NS; ++s2)
+        for (int ds = 0; ds < KT; ++ds)
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          xf1[s2][q] = xn1[s2][q];
-          if constexpr (SPLIT) xf2[s2][q] = xn2[s2][q];
+          for (int j = 0; j < 2; ++j) old[ds][j] = *reinterpret_cast<const uint4*>(dX1 + orow + (ds * 64 + j * 32) / ES);
+      }
+      uint4 val[KT][2];
+#pragma unroll
+      for (int ds = 0; ds < KT; ++ds) {
+        const floatx16& acc = ax1[ds];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const uint32_t p0 = pack_bf16(acc[8 * j], acc[8 * j + 1]), p1 = pack_bf16(acc[8 * j + 2], acc[8 * j + 3]);
+          const uint32_t p2 = pack_bf16(acc[8 * j + 4], acc[8 * j + 5]), p3 = pack_bf16(acc[8 * j + 6], acc[8 * j + 7]);
+          const auto s0 = __builtin_amdgcn_permlane32_swap(p0, p2, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(p1, p3, false, false);
+          val[ds][j] = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+          if (accumulate) val[ds][j] = add_vec<TI>(val[ds][j], old[ds][j]);
         }
-      mk = mkn;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (mrow < M) {
+#pragma unroll
+        for (int ds = 0; ds < KT; ++ds)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) *reinterpret_cast<uint4*>(dX1 + orow + (ds * 64 + j * 32) / ES) = val[ds][j];
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
@@ -1205,7 +1246,8 @@ __global__ void __launch_bounds__(512, 2)
   char* sw2 = dgr_dsm + C * WSTR;
   float* sb = reinterpret_cast<float*>(dgr_dsm + 2 * C * WSTR);  // bias1[C], bias2[C]
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+  // (the wavefront's number as a scalar: tile indices and row bases derived from it stay in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c = lane & 31, h = lane >> 5;
 
   for (int e = tid; e < C * VPR; e += NTH) {
     const int r = e / VPR, part = e % VPR;
@@ -2471,9 +2513,9 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
                CUEQ_ERR_TOO_LARGE, "gate_bwd_input: strides too large for 32-bit lane offsets");
   KernelTimer timer("gate_bwd_input", stream);
   if (bf) {
-    // weights resident in LDS when they fit (2 C rows of 2 K + 16 bytes, biases, staging tiles)
+    // weights resident in LDS when they fit (2 C rows of 2 K + 16 bytes, biases, with two inputs the staging tiles)
     const int nwaves = split ? 4 : 8;
-    const size_t lds = static_cast<size_t>(2 * C * (K == 128 ? 2 * K : 2 * K + 16) + 8 * C + nwaves * 8 * (2 * K + 16));
+    const size_t lds = static_cast<size_t>(2 * C * (K == 128 ? 2 * K : 2 * K + 16) + 8 * C + (split ? nwaves * 8 * (2 * K + 16) : 0));
     // (dC by rows is read, and the gate gradients written, as 4-byte column pairs)
     const bool pairs_ok = !dc_by_row || (M % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(dC) % 4 == 0);
     if (lds <= 160 * 1024 && pairs_ok) {
