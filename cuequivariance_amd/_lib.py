@@ -55,6 +55,7 @@ EXPORTED_SYMBOLS = (
     "cueq_layer_norm_t_bwd_workspace",
     "cueq_layer_norm_t_bwd",
     "cueq_dual_gate",
+    "cueq_ln_dual_gate",
     "cueq_gate_bwd_input",
     "cueq_gemm_tn_items",
     "cueq_gemm_tn",
@@ -223,6 +224,8 @@ def load() -> C.CDLL:
         lib.cueq_layer_norm_t_bwd.restype = C.c_int
         lib.cueq_dual_gate.argtypes = [i32, i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, i32, ptr, i32, ptr, ptr, ptr, i64, ptr]
         lib.cueq_dual_gate.restype = C.c_int
+        lib.cueq_ln_dual_gate.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, i64, ptr, ptr, C.c_double, ptr, ptr, ptr, ptr, i64, ptr, i64, ptr, ptr, ptr]
+        lib.cueq_ln_dual_gate.restype = C.c_int
         lib.cueq_gate_bwd_input.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, ptr, ptr, i64,
                                             i32, ptr, ptr, i64, i32, ptr, ptr, ptr]
         lib.cueq_gate_bwd_input.restype = C.c_int

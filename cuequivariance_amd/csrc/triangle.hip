@@ -66,6 +66,36 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {  // round to
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 
+// The value again, as far as the compiler can tell a new one: the two floats of a packed pair are then unpacked where they
+// are used instead of being kept, one register each, from the first pass over the data to the last.
+__device__ __forceinline__ uint32_t again(uint32_t w) {
+  asm volatile("" : "+v"(w));
+  return w;
+}
+// The arithmetic of the LayerNorm statistics over groups of eight elements, spelled out operation by operation (no
+// contraction left to the compiler) because two kernels share it and must give the same bits: the row kernel
+// ln_fwd_rows8 and the LayerNorm inside dual_gate_res_kernel.
+__device__ __forceinline__ float ln_sum8(const float* v) {
+  float s = v[0];
+#pragma unroll
+  for (int e = 1; e < 8; ++e) s = __fadd_rn(s, v[e]);
+  return s;
+}
+__device__ __forceinline__ float ln_center_sq8(float* v, float mu) {  // v -= mu, returns the sum of squares
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = __fsub_rn(v[e], mu);
+  float ss = __fmul_rn(v[0], v[0]);
+#pragma unroll
+  for (int e = 1; e < 8; ++e) ss = fmaf(v[e], v[e], ss);
+  return ss;
+}
+__device__ __forceinline__ float ln_rstd(float sumsq, float inv_d, float eps) { return 1.0f / sqrtf(fmaf(sumsq, inv_d, eps)); }
+__device__ __forceinline__ float ln_affine(float centered, float rs, float gm, float bt) {
+  return __fadd_rn(__fmul_rn(__fmul_rn(centered, rs), gm), bt);
+}
+__device__ __forceinline__ float lo_bf16(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float hi_bf16(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
 template <typename TO>
 __device__ __forceinline__ void stage_put(char* tile, int row_stride, int col, int h, const floatx16& acc, float alpha) {
 #pragma unroll
@@ -1228,12 +1258,19 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
 // block per CU, every wavefront walks tiles of 64 columns m on its own (two 32-column MFMA tiles sharing each weight
 // fragment).  Results leave as 4-byte column pairs: neighbouring lanes swap halves (even lane: row 2 j for columns
 // m, m + 1; odd lane: row 2 j + 1 for m - 1, m), so N and ldc must be even.
+//
+// LN: X holds the rows before their LayerNorm.  A lane has half of its row in registers (the other half is in the lane
+// 32 further), so the statistics are sums over the lane's own values completed by one exchange; the rows are
+// normalised in the registers, rounded to the 2-byte type - the operand of the products, exactly what a separate
+// LayerNorm launch would have written - and stored with their mean and 1 / std for the later stages.
 // ------------------------------------------------------------------------------------------------
-template <int KT>
+template <int KT, bool LN>
 __global__ void __launch_bounds__(512, 2)
     dual_gate_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X, int64_t ldx,
                          const uint16_t* __restrict__ bias1, const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask,
-                         uint16_t* __restrict__ out, int64_t ldc, int C, int M) {
+                         uint16_t* __restrict__ out, int64_t ldc, int C, int M, const uint16_t* __restrict__ gamma,
+                         const uint16_t* __restrict__ beta, float eps, uint16_t* __restrict__ xhat, int64_t ldxh, float* __restrict__ mean,
+                         float* __restrict__ rstd) {
   using TI = uint16_t;
   constexpr int ES = 2, EPV = 8;
   constexpr int K = 32 * KT, ROWB = K * ES, NS = ROWB / 64, VPR = ROWB / 16;
@@ -1245,6 +1282,7 @@ __global__ void __launch_bounds__(512, 2)
   char* sw1 = dgr_dsm;
   char* sw2 = dgr_dsm + C * WSTR;
   float* sb = reinterpret_cast<float*>(dgr_dsm + 2 * C * WSTR);  // bias1[C], bias2[C]
+  float* sg = sb + 2 * C;                                           // LN: gamma[K], beta[K]
   const int tid = threadIdx.x;
   // (the wavefront's number as a scalar: tile indices and row bases derived from it stay in scalar registers)
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c = lane & 31, h = lane >> 5;
@@ -1259,26 +1297,112 @@ __global__ void __launch_bounds__(512, 2)
     sb[i] = bias1 ? tri_load(bias1, i) : 0.f;
     sb[C + i] = bias2 ? tri_load(bias2, i) : 0.f;
   }
+  if constexpr (LN) {
+    for (int i = tid; i < K; i += NTH) {
+      sg[i] = gamma ? tri_load(gamma, i) : 1.f;
+      sg[K + i] = beta ? tri_load(beta, i) : 0.f;
+    }
+  }
   __syncthreads();
 
   const int nchunks = C / 32;
   const int64_t ntiles = (static_cast<int64_t>(M) + 63) / 64;
   const int64_t tstep = static_cast<int64_t>(gridDim.x) * NWAVES;
   const uint32_t pair_sel = (lane & 1) ? 0x03020706u : 0x05040100u;
-  for (int64_t tile = static_cast<int64_t>(blockIdx.x) * NWAVES + wave; tile < ntiles; tile += tstep) {
+  // the rows of a tile, one row per lane (and the lane 32 further), with their mask values as stored; those of the
+  // wavefront's next tile are requested while the current one is worked on
+  uint4 xn[2][NS][2];
+  uint32_t mraw[2] = {0, 0};
+  auto request_x = [&](int64_t tl) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int mld = static_cast<int>(min(tl * 64 + 32 * t + c, static_cast<int64_t>(M) - 1));
+#pragma unroll
+      for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+          xn[t][s2][q] = *reinterpret_cast<const uint4*>(X + static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES);
+      if (mask) mraw[t] = mask[mld];
+    }
+  };
+  const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * NWAVES + wave;
+  if (tile0 < ntiles) request_x(tile0);
+  for (int64_t tile = tile0; tile < ntiles; tile += tstep) {
     uint4 xf[2][NS][2];
     float mk[2];
     int mcol[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       mcol[t] = static_cast<int>(tile * 64) + 32 * t + c;
-      const int mld = min(mcol[t], M - 1);
 #pragma unroll
       for (int s2 = 0; s2 < NS; ++s2)
 #pragma unroll
-        for (int q = 0; q < 2; ++q)
-          xf[t][s2][q] = *reinterpret_cast<const uint4*>(X + static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES);
-      mk[t] = mask ? tri_load(mask, mld) : 1.0f;
+        for (int q = 0; q < 2; ++q) xf[t][s2][q] = xn[t][s2][q];
+      mk[t] = mask ? __uint_as_float(mraw[t] << 16) : 1.0f;
+    }
+    request_x(min(tile + tstep, ntiles - 1));  // (past the end: the last tile again, so that the request is unconditional)
+    if constexpr (LN) {
+      // The sums are formed in the order of the row kernel ln_fwd_rows8 - groups of eight elements summed in sequence,
+      // then pairs, fours, eights of groups - so that both give the same bits: a group pair lives in one lane, the
+      // neighbouring pair in the lane 32 further.
+      auto tree = [&](const float (&gs)[NS][2]) -> float {
+        float quad[NS];
+#pragma unroll
+        for (int s2 = 0; s2 < NS; ++s2) {
+          const float pair = gs[s2][0] + gs[s2][1];
+          quad[s2] = pair + __shfl_xor(pair, 32, 64);
+        }
+        if constexpr (NS == 1) return quad[0];
+        else if constexpr (NS == 2) return quad[0] + quad[1];
+        else if constexpr (NS == 3) return (quad[0] + quad[1]) + quad[2];
+        else return (quad[0] + quad[1]) + (quad[2] + quad[3]);
+      };
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        float gs[NS][2];
+#pragma unroll
+        for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const uint32_t w[4] = {xf[t][s2][q].x, xf[t][s2][q].y, xf[t][s2][q].z, xf[t][s2][q].w};
+            const float v[8] = {lo_bf16(w[0]), hi_bf16(w[0]), lo_bf16(w[1]), hi_bf16(w[1]), lo_bf16(w[2]), hi_bf16(w[2]), lo_bf16(w[3]), hi_bf16(w[3])};
+            gs[s2][q] = ln_sum8(v);
+          }
+        const float mu = __fmul_rn(tree(gs), 1.0f / K);
+#pragma unroll
+        for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const uint32_t w[4] = {again(xf[t][s2][q].x), again(xf[t][s2][q].y), again(xf[t][s2][q].z), again(xf[t][s2][q].w)};
+            float v[8] = {lo_bf16(w[0]), hi_bf16(w[0]), lo_bf16(w[1]), hi_bf16(w[1]), lo_bf16(w[2]), hi_bf16(w[2]), lo_bf16(w[3]), hi_bf16(w[3])};
+            gs[s2][q] = ln_center_sq8(v, mu);
+          }
+        const float rs = ln_rstd(tree(gs), 1.0f / K, eps);
+        const int mld = min(mcol[t], M - 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < NS; ++s2)
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const int k0 = s2 * 32 + h * 16 + q * 8;
+            const float4 g0 = *reinterpret_cast<const float4*>(sg + k0), g1 = *reinterpret_cast<const float4*>(sg + k0 + 4);
+            const float4 b0 = *reinterpret_cast<const float4*>(sg + K + k0), b1 = *reinterpret_cast<const float4*>(sg + K + k0 + 4);
+            const float gm[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w}, bt[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+            const uint32_t w[4] = {again(xf[t][s2][q].x), again(xf[t][s2][q].y), again(xf[t][s2][q].z), again(xf[t][s2][q].w)};
+            uint32_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              o[e] = pack_bf16(ln_affine(__fsub_rn(lo_bf16(w[e]), mu), rs, gm[2 * e], bt[2 * e]),
+                               ln_affine(__fsub_rn(hi_bf16(w[e]), mu), rs, gm[2 * e + 1], bt[2 * e + 1]));
+            xf[t][s2][q] = make_uint4(o[0], o[1], o[2], o[3]);
+            if (mcol[t] < M) *reinterpret_cast<uint4*>(xhat + static_cast<int64_t>(mld) * ldxh + (s2 * 64 + h * 32 + q * 16) / ES) = xf[t][s2][q];
+            __builtin_amdgcn_sched_barrier(0);  // one piece at a time: its gamma / beta values die here
+          }
+        if (h == 0 && mcol[t] < M) {
+          mean[mld] = mu;
+          rstd[mld] = rs;
+        }
+      }
     }
     for (int ci = 0; ci < nchunks; ++ci) {
       const int c0 = ci * 32;
@@ -1548,25 +1672,14 @@ __global__ void __launch_bounds__(256) ln_fwd_rows8(const T* __restrict__ x, con
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = 0.f;
   }
-  float s = 0;
+  const float mu = __fmul_rn(group_sum<L>(ln_sum8(v)), 1.0f / D);
+  const float rs = ln_rstd(group_sum<L>(ln_center_sq8(v, mu)), 1.0f / D, eps);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) s += v[e];
-  const float mu = group_sum<L>(s) * (1.0f / D);
-  float ss = 0;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    v[e] -= mu;
-    ss += v[e] * v[e];
-  }
-  const float rs = 1.0f / sqrtf(group_sum<L>(ss) * (1.0f / D) + eps);
+  for (int e = 0; e < 8; ++e) gm[e] = 1.f, bt[e] = 0.f;
   if (gamma) tn_load8(gamma + col, gm);
   if (beta) tn_load8(beta + col, bt);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    v[e] *= rs;
-    if (gamma) v[e] *= gm[e];
-    if (beta) v[e] += bt[e];
-  }
+  for (int e = 0; e < 8; ++e) v[e] = ln_affine(v[e], rs, gm[e], bt[e]);
   if (ok) {
     ln_store8(y + row * D + col, v);
     if (lane % L == 0) {
@@ -1875,14 +1988,6 @@ __global__ void __launch_bounds__(256) ln_t_bwd_kernel(const T* __restrict__ dy,
 // accesses of consecutive lanes fall into distinct banks.  The forward keeps a second tile in flight.  The backward
 // here computes the gradient of the tensor only; with the affine gradients asked for the kernel above runs.
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ float lo_bf16(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float hi_bf16(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
-// The value again, as far as the compiler can tell a new one: the two floats of a packed pair are then unpacked where they
-// are used instead of being kept, one register each, from the first pass over the data to the last.
-__device__ __forceinline__ uint32_t again(uint32_t w) {
-  asm volatile("" : "+v"(w));
-  return w;
-}
 template <typename V>
 __device__ __forceinline__ void store_global(char* uniform_base, uint32_t lane_offset, V value) {
   typedef __attribute__((address_space(1))) V* gptr;
@@ -2411,6 +2516,32 @@ extern "C" int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mo
   return CUEQ_OK;
 }
 
+// the resident-weights forward kernel: C weight rows (a multiple of 32) of K = 32, 64, 96 or 128 elements, 2-byte type
+static size_t dual_gate_res_lds(int64_t C, int64_t K, bool ln) {
+  return static_cast<size_t>(2 * C * (K == 128 ? 2 * K : 2 * K + 16) + 8 * C + (ln ? 8 * K : 0));
+}
+static bool dual_gate_res_fits(int64_t C, int64_t M, int64_t K, const void* out, int64_t ldc, bool ln) {
+  return K % 32 == 0 && K <= 128 && C % 32 == 0 && M % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0 && M >= 4096 &&
+         dual_gate_res_lds(C, K, ln) <= 160 * 1024;
+}
+static int launch_dual_gate_res(int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X, int64_t ldx,
+                                const void* bias1, const void* bias2, const void* mask, void* out, int64_t ldc, const void* gamma,
+                                const void* beta, float eps, void* xhat, int64_t ldxh, float* mean, float* rstd, hipStream_t stream) {
+  const size_t lds = dual_gate_res_lds(C, K, xhat != nullptr);
+  const int64_t ntiles = (M + 63) / 64;
+  int64_t gx = (ntiles + 7) / 8;
+  if (gx > device_cus()) gx = device_cus();
+#define DGR(KT, LN) do { auto kfn = dual_gate_res_kernel<KT, LN>; \
+    CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<uint16_t*>(out), ldc, static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), eps, static_cast<uint16_t*>(xhat), ldxh, mean, rstd); } while (0)
+#define DGR_K(LN) do { switch (K / 32) { case 1: DGR(1, LN); break; case 2: DGR(2, LN); break; case 3: DGR(3, LN); break; default: DGR(4, LN); break; } } while (0)
+  if (xhat) DGR_K(true); else DGR_K(false);
+#undef DGR_K
+#undef DGR
+  CUEQ_CHECK_HIP(hipGetLastError());
+  return CUEQ_OK;
+}
+
 extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_t K, const void* A1, const void* A2, int64_t lda,
                               const void* B1, const void* B2, int64_t ldb, const void* bias1, const void* bias2, int32_t bias_axis,
                               const void* mask, int32_t mask_axis, const void* dC, void* out1, void* out2, int64_t ldc, void* stream_) {
@@ -2444,21 +2575,9 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
   KernelTimer timer(backward ? "dual_gate_bwd" : "dual_gate_fwd", stream);
   // forward with one shared right operand, biases along the rows and the mask along the columns, in a 2-byte type:
   // the left operands (the weights, M rows) stay resident in LDS when they fit
-  if (dtype == CUEQ_BF16 && !backward && share && (!(bias1 || bias2) || bias_axis == 0) && (!mask || mask_axis == 1) && K % 32 == 0 && K <= 128 &&
-      M % 32 == 0 && N % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(out1) % 4 == 0 && N >= 4096) {
-    const size_t lds = static_cast<size_t>(2 * M * (K == 128 ? 2 * K : 2 * K + 16) + 8 * M);
-    if (lds <= 160 * 1024) {
-      const int64_t ntiles = (N + 63) / 64;
-      int64_t gx2 = (ntiles + 7) / 8;
-      if (gx2 > device_cus()) gx2 = device_cus();
-#define DGR(KT) do { auto kfn = dual_gate_res_kernel<KT>; \
-        CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx2)), dim3(512), lds, stream, static_cast<const uint16_t*>(A1), static_cast<const uint16_t*>(A2), lda, static_cast<const uint16_t*>(B1), ldb, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<uint16_t*>(out1), ldc, static_cast<int>(M), static_cast<int>(N)); } while (0)
-      switch (K / 32) { case 1: DGR(1); break; case 2: DGR(2); break; case 3: DGR(3); break; default: DGR(4); break; }
-#undef DGR
-      CUEQ_CHECK_HIP(hipGetLastError());
-      return CUEQ_OK;
-    }
+  if (dtype == CUEQ_BF16 && !backward && share && (!(bias1 || bias2) || bias_axis == 0) && (!mask || mask_axis == 1) &&
+      dual_gate_res_fits(M, N, K, out1, ldc, false)) {
+    return launch_dual_gate_res(M, N, K, A1, A2, lda, B1, ldb, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, stream);
   }
 #define DG(TI, BW, SH) hipLaunchKernelGGL((dual_gate_kernel<TI, BW, SH>), grid, dim3(512), 0, stream, static_cast<const TI*>(A1), static_cast<const TI*>(A2), lda, static_cast<const TI*>(B1), static_cast<const TI*>(B2), ldb, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), bias_axis, static_cast<const TI*>(mask), mask_axis, static_cast<const TI*>(dC), static_cast<TI*>(out1), static_cast<TI*>(out2), ldc, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), vec_out)
 #define DG_T(TI) do { if (backward) { if (share) DG(TI, true, true); else DG(TI, true, false); } else { if (share) DG(TI, false, true); else DG(TI, false, false); } } while (0)
@@ -2467,6 +2586,24 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
 #undef DG
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
+}
+
+extern "C" int cueq_ln_dual_gate(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X,
+                                 int64_t ldx, const void* gamma, const void* beta, double eps, const void* bias1, const void* bias2,
+                                 const void* mask, void* out, int64_t ldc, void* xhat, int64_t ldxh, float* mean, float* rstd, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  CUEQ_REQUIRE(dtype == CUEQ_BF16, CUEQ_ERR_UNSUPPORTED, "ln_dual_gate: built for bfloat16 (compose cueq_layer_norm_fwd and cueq_dual_gate otherwise)");
+  CUEQ_REQUIRE(C > 0 && M >= 0 && K > 0, CUEQ_ERR_INVALID, "ln_dual_gate: bad extents");
+  if (M == 0) return CUEQ_OK;
+  CUEQ_REQUIRE(W1 && W2 && X && out && xhat && mean && rstd, CUEQ_ERR_INVALID, "ln_dual_gate: null operand");
+  const uintptr_t ptrs = reinterpret_cast<uintptr_t>(W1) | reinterpret_cast<uintptr_t>(W2) | reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(xhat);
+  CUEQ_REQUIRE((ptrs & 15) == 0 && ldw % 8 == 0 && ldx % 8 == 0 && ldxh % 8 == 0 && ldw >= K && ldx >= K && ldxh >= K, CUEQ_ERR_UNSUPPORTED,
+               "ln_dual_gate: row strides and pointers must be multiples of 16 bytes");
+  CUEQ_REQUIRE(M <= kRowSlab && C < (1ll << 31) && ldc >= M, CUEQ_ERR_TOO_LARGE, "ln_dual_gate: extent too large");
+  CUEQ_REQUIRE(dual_gate_res_fits(C, M, K, out, ldc, true), CUEQ_ERR_UNSUPPORTED,
+               "ln_dual_gate: needs K = 32, 64, 96 or 128, C a multiple of 32 that fits the local data share, an even M of at least 4096 and an even ldc");
+  KernelTimer timer("ln_dual_gate_fwd", stream);
+  return launch_dual_gate_res(C, M, K, W1, W2, ldw, X, ldx, bias1, bias2, mask, out, ldc, gamma, beta, static_cast<float>(eps), xhat, ldxh, mean, rstd, stream);
 }
 
 extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,

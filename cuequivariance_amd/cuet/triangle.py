@@ -213,6 +213,29 @@ def dual_gate_fwd(A1, A2, B1, B2, bias1, bias2, bias_axis: int, mask, mask_axis:
     return gate_fwd(u, v, bias1, bias2, bias_axis, mask, mask_axis, T)
 
 
+def ln_dual_gate_fwd(x, gamma, beta, eps: float, W1, W2, bias1, bias2, mask):
+    """``LayerNorm`` of the rows of ``x (M, K)`` and ``sigmoid(W1 xh^T + bias1) * (W2 xh^T + bias2) * mask`` in one kernel
+    (``cueq_ln_dual_gate``).  Returns ``(out (C, M), xh, mean, rstd)``, or ``None`` when the shapes do not allow it
+    (then :func:`layer_norm_fwd` and :func:`dual_gate_fwd` do the same in two launches)."""
+    M, K = x.shape
+    Cn = W1.shape[0]
+    if x.dtype != torch.bfloat16 or K % 32 or K > 128 or Cn % 32 or M % 2 or M < 4096 or M > 65280 * 128:
+        return None
+    if 2 * Cn * (2 * K if K == 128 else 2 * K + 16) + 8 * Cn + 8 * K > 160 * 1024 or not _fusable(x, W1, W2):
+        return None
+    out = torch.empty(Cn, M, dtype=x.dtype, device=x.device)
+    xh = torch.empty(M, K, dtype=x.dtype, device=x.device)
+    mean = torch.empty(M, dtype=torch.float32, device=x.device)
+    rstd = torch.empty(M, dtype=torch.float32, device=x.device)
+    _lib.check(
+        _lib.load().cueq_ln_dual_gate(_CODE[x.dtype], Cn, M, K, W1.data_ptr(), W2.data_ptr(), W1.stride(0), x.data_ptr(), x.stride(0),
+                                      _ptr(gamma), _ptr(beta), float(eps), _ptr(bias1), _ptr(bias2), _ptr(mask), out.data_ptr(), M,
+                                      xh.data_ptr(), K, mean.data_ptr(), rstd.data_ptr(), _stream(x)),
+        "cueq_ln_dual_gate",
+    )
+    return out, xh, mean, rstd
+
+
 def dual_gate_bwd(dout, A1, A2, B1, B2, bias1, bias2, bias_axis: int, mask, mask_axis: int):
     """Gradients of the two products of :func:`dual_gate_fwd` (they are recomputed, not read back)."""
     M, K = A1.shape
@@ -312,10 +335,14 @@ def _trimul_fwd(x, mask, nin_w, nin_b, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, n
         M = Bsz * N * N
         Do = p_out_w.shape[0]
         x2 = x.reshape(M, D)
-        xh, mean1, rstd1 = layer_norm_fwd(x2, nin_w, nin_b, eps)
         mflat = None if mask is None else mask.reshape(M)
         # (2D, M) == (2D, B, N, N): the "transposed output" of the reference comes for free with the weights as rows
-        ab = dual_gate_fwd(g_in_w, p_in_w, xh, None, g_in_b, p_in_b, 0, mflat, 1)
+        fused = ln_dual_gate_fwd(x2, nin_w, nin_b, eps, g_in_w, p_in_w, g_in_b, p_in_b, mflat)
+        if fused is not None:
+            ab, xh, mean1, rstd1 = fused
+        else:
+            xh, mean1, rstd1 = layer_norm_fwd(x2, nin_w, nin_b, eps)
+            ab = dual_gate_fwd(g_in_w, p_in_w, xh, None, g_in_b, p_in_b, 0, mflat, 1)
         a = ab[:D].view(D * Bsz, N, N)
         b = ab[D:].view(D * Bsz, N, N)
         if outgoing:

@@ -296,6 +296,19 @@ int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_t N, int64_
                    const void* B1, const void* B2, int64_t ldb, const void* bias1, const void* bias2, int32_t bias_axis,
                    const void* mask, int32_t mask_axis, const void* dC, void* out1, void* out2, int64_t ldc, void* stream);
 
+/* LayerNorm of the rows of X followed by the gated dual projection with the weights as rows, in one kernel - the first two
+ * stages of the triangle update (cuequivariance_jax/cuequivariance_jax/triangle/_triangle_multiplicative_update.py:371-400:
+ * x_hat = LN(x), then sigmoid(x_hat G^T + b) * (x_hat P^T + b) * mask written "transposed"):
+ *   xhat[m, :] = (X[m, :] - mean[m]) * rstd[m] * gamma + beta   (biased variance, rstd = 1 / sqrt(var + eps); gamma / beta may be NULL)
+ *   out[c, m]  = sigmoid(W1[c, :] . xhat[m, :] + bias1[c]) * (W2[c, :] . xhat[m, :] + bias2[c]) * mask[m]
+ * with xhat rounded to bfloat16 before the products, as a separate cueq_layer_norm_fwd would have stored it; xhat (M x K, row
+ * stride ldxh), mean and rstd (M floats each) are written for the later stages.  bfloat16 only, K = 32, 64, 96 or 128, C a
+ * multiple of 32 with both weight matrices fitting the local data share, M even and at least 4096, ldc even; other shapes
+ * return CUEQ_ERR_UNSUPPORTED (compose cueq_layer_norm_fwd and cueq_dual_gate instead). */
+int cueq_ln_dual_gate(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X,
+                      int64_t ldx, const void* gamma, const void* beta, double eps, const void* bias1, const void* bias2,
+                      const void* mask, void* out, int64_t ldc, void* xhat, int64_t ldxh, float* mean, float* rstd, void* stream);
+
 /* Backward of the gated dual projection down to the projection inputs (_sigmoid_gated_dual_gemm.py:153-218), one kernel:
  *   u[c][m] = W1[c,:] . X1[m,:],  v[c][m] = W2[c,:] . X2[m,:]   (W* C x K row-major with row stride ldw, X* M x K; recomputed)
  *   s = sigmoid(u + bias1[c]),  d = dC * mask[m],  du = d (v + bias2[c]) s (1 - s),  dv = d s

@@ -138,6 +138,51 @@ def test_layer_norm_with_layout_change_against_torch(device, D, M, need_affine):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("affine,bias,masked", [(True, True, True), (False, False, False), (True, False, True)])
+@pytest.mark.parametrize("M,K,C", [(4096, 128, 256), (4098, 64, 64), (5000, 96, 96), (8192 + 70, 32, 32), (262144, 128, 256)])
+def test_layer_norm_fused_into_the_gated_projection(device, M, K, C, affine, bias, masked):
+    """``cueq_ln_dual_gate`` (bfloat16): the normalised rows, their statistics and the gated projection against ``F.layer_norm``
+    + the two products in float64 on the same bfloat16 values, and against the two separate launches it replaces.  Row counts
+    that end inside a 64-row tile, every K the kernel takes, with and without affine weights, biases and mask.  Tolerances
+    relative to ``max|ref|``: 2^-7 for the normalised rows (one rounding), 2^-6 for the projection (computed from the rounded
+    rows)."""
+    from cuequivariance_amd.cuet import triangle as tri
+
+    g = torch.Generator(device=device).manual_seed(M + K + C)
+    rn = lambda *shape: torch.randn(*shape, device=device, generator=g)
+    x = (rn(M, K) * 1.3 + 0.2).bfloat16()
+    gamma = (rn(K) * 0.5 + 1.0).bfloat16() if affine else None
+    beta = rn(K).bfloat16() if affine else None
+    W1, W2 = (rn(C, K) / K ** 0.5).bfloat16(), (rn(C, K) / K ** 0.5).bfloat16()
+    b1, b2 = (rn(C).bfloat16(), rn(C).bfloat16()) if bias else (None, None)
+    mask = (torch.rand(M, device=device, generator=g) < 0.8).bfloat16() if masked else None
+    fused = tri.ln_dual_gate_fwd(x, gamma, beta, 1e-5, W1, W2, b1, b2, mask)
+    assert fused is not None
+    out, xh, mean, rstd = fused
+    # float64 on the same values; the products take the rounded rows, as the kernels do
+    x64 = x.double()
+    ref_xh = F.layer_norm(x64, (K,), None if gamma is None else gamma.double(), None if beta is None else beta.double(), 1e-5)
+    assert (xh.double() - ref_xh).abs().max().item() <= 2.0 ** -7 * ref_xh.abs().max().item()
+    assert (mean.double() - x64.mean(1)).abs().max().item() <= 1e-5
+    assert (rstd.double() * torch.sqrt(x64.var(1, unbiased=False) + 1e-5) - 1).abs().max().item() <= 1e-5
+    u = xh.double() @ W1.double().t() + (0 if b1 is None else b1.double())
+    v = xh.double() @ W2.double().t() + (0 if b2 is None else b2.double())
+    ref = torch.sigmoid(u) * v * (1 if mask is None else mask.double()[:, None])
+    assert (out.double().t() - ref).abs().max().item() <= 2.0 ** -6 * ref.abs().max().item()
+    # the two launches it replaces: for the row lengths that the row kernel sums as a tree of 8-element groups (32, 64, 128) the
+    # fused kernel forms its sums in the same order and every bit agrees - a batch that takes the fused launch and a small one
+    # that does not give the same rows; for 96 the orders differ
+    xh2, mean2, rstd2 = tri.layer_norm_fwd(x, gamma, beta, 1e-5)
+    out2 = tri.dual_gate_fwd(W1, W2, xh2, None, b1, b2, 0, mask, 1)
+    if K != 96:
+        assert torch.equal(mean, mean2) and torch.equal(rstd, rstd2) and torch.equal(xh, xh2) and torch.equal(out, out2)
+    else:
+        assert (mean - mean2).abs().max().item() <= 1e-6 and (rstd / rstd2 - 1).abs().max().item() <= 1e-6
+        assert (xh != xh2).float().mean().item() <= 1e-3
+        assert (out.float() - out2.float()).abs().max().item() <= 2.0 ** -6 * out2.float().abs().max().item()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21), (160, 512, 256, 96),
