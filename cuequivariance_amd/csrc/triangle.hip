@@ -1259,15 +1259,17 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
 // fragment).  Results leave as 4-byte column pairs: neighbouring lanes swap halves (even lane: row 2 j for columns
 // m, m + 1; odd lane: row 2 j + 1 for m - 1, m), so N and ldc must be even.
 //
+// ROWS: two inputs (W1 meets X, W2 meets X2) and the result by rows, M x C - the output stage of the triangle update.
+//
 // LN: X holds the rows before their LayerNorm.  A lane has half of its row in registers (the other half is in the lane
 // 32 further), so the statistics are sums over the lane's own values completed by one exchange; the rows are
 // normalised in the registers, rounded to the 2-byte type - the operand of the products, exactly what a separate
 // LayerNorm launch would have written - and stored with their mean and 1 / std for the later stages.
 // ------------------------------------------------------------------------------------------------
-template <int KT, bool LN>
+template <int KT, bool LN, bool ROWS>
 __global__ void __launch_bounds__(512, 2)
-    dual_gate_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X, int64_t ldx,
-                         const uint16_t* __restrict__ bias1, const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask,
+    dual_gate_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X,
+                         const uint16_t* __restrict__ X2, int64_t ldx, const uint16_t* __restrict__ bias1, const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask,
                          uint16_t* __restrict__ out, int64_t ldc, int C, int M, const uint16_t* __restrict__ gamma,
                          const uint16_t* __restrict__ beta, float eps, uint16_t* __restrict__ xhat, int64_t ldxh, float* __restrict__ mean,
                          float* __restrict__ rstd) {
@@ -1277,6 +1279,8 @@ __global__ void __launch_bounds__(512, 2)
   constexpr bool SWZ = KT == 4;  // (same layout of the weight rows as gate_bwd_input_res_kernel)
   constexpr int WSTR = SWZ ? ROWB : ROWB + 16;
   constexpr int NTH = 512, NWAVES = NTH / 64;
+  constexpr int NT = ROWS ? 1 : 2;  // 32-row MFMA tiles per step of a wavefront (two inputs: one, their rows take the registers)
+  static_assert(!(LN && ROWS), "the LayerNorm variant has one input");
   auto swz = [](int row) -> int { return SWZ ? (((row & 3) << 2) | ((row >> 2) & 3)) : 0; };
   extern __shared__ __align__(16) char dgr_dsm[];
   char* sw1 = dgr_dsm;
@@ -1306,38 +1310,44 @@ __global__ void __launch_bounds__(512, 2)
   __syncthreads();
 
   const int nchunks = C / 32;
-  const int64_t ntiles = (static_cast<int64_t>(M) + 63) / 64;
+  const int64_t ntiles = (static_cast<int64_t>(M) + 32 * NT - 1) / (32 * NT);
   const int64_t tstep = static_cast<int64_t>(gridDim.x) * NWAVES;
   const uint32_t pair_sel = (lane & 1) ? 0x03020706u : 0x05040100u;
   // the rows of a tile, one row per lane (and the lane 32 further), with their mask values as stored; those of the
   // wavefront's next tile are requested while the current one is worked on
-  uint4 xn[2][NS][2];
-  uint32_t mraw[2] = {0, 0};
+  uint4 xn[NT][NS][2], xn2[1][NS][2];
+  uint32_t mraw[NT] = {};
   auto request_x = [&](int64_t tl) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int mld = static_cast<int>(min(tl * 64 + 32 * t + c, static_cast<int64_t>(M) - 1));
+    for (int t = 0; t < NT; ++t) {
+      const int mld = static_cast<int>(min(tl * (32 * NT) + 32 * t + c, static_cast<int64_t>(M) - 1));
 #pragma unroll
       for (int s2 = 0; s2 < NS; ++s2)
 #pragma unroll
-        for (int q = 0; q < 2; ++q)
-          xn[t][s2][q] = *reinterpret_cast<const uint4*>(X + static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES);
+        for (int q = 0; q < 2; ++q) {
+          const int64_t o = static_cast<int64_t>(mld) * ldx + (s2 * 64 + h * 32 + q * 16) / ES;
+          xn[t][s2][q] = *reinterpret_cast<const uint4*>(X + o);
+          if constexpr (ROWS) xn2[t][s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
+        }
       if (mask) mraw[t] = mask[mld];
     }
   };
   const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * NWAVES + wave;
   if (tile0 < ntiles) request_x(tile0);
   for (int64_t tile = tile0; tile < ntiles; tile += tstep) {
-    uint4 xf[2][NS][2];
-    float mk[2];
-    int mcol[2];
+    uint4 xf[NT][NS][2], xf2[1][NS][2];
+    float mk[NT];
+    int mcol[NT];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      mcol[t] = static_cast<int>(tile * 64) + 32 * t + c;
+    for (int t = 0; t < NT; ++t) {
+      mcol[t] = static_cast<int>(tile * (32 * NT)) + 32 * t + c;
 #pragma unroll
       for (int s2 = 0; s2 < NS; ++s2)
 #pragma unroll
-        for (int q = 0; q < 2; ++q) xf[t][s2][q] = xn[t][s2][q];
+        for (int q = 0; q < 2; ++q) {
+          xf[t][s2][q] = xn[t][s2][q];
+          if constexpr (ROWS) xf2[t][s2][q] = xn2[t][s2][q];
+        }
       mk[t] = mask ? __uint_as_float(mraw[t] << 16) : 1.0f;
     }
     request_x(min(tile + tstep, ntiles - 1));  // (past the end: the last tile again, so that the request is unconditional)
@@ -1358,7 +1368,7 @@ __global__ void __launch_bounds__(512, 2)
         else return (quad[0] + quad[1]) + (quad[2] + quad[3]);
       };
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < NT; ++t) {
         float gs[NS][2];
 #pragma unroll
         for (int s2 = 0; s2 < NS; ++s2)
@@ -1406,13 +1416,13 @@ __global__ void __launch_bounds__(512, 2)
     }
     for (int ci = 0; ci < nchunks; ++ci) {
       const int c0 = ci * 32;
-      floatx16 au[2], av[2];
+      floatx16 au[NT], av[NT];
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
         const float4 b1 = *reinterpret_cast<const float4*>(sb + c0 + 8 * a + 4 * h);
         const float4 b2 = *reinterpret_cast<const float4*>(sb + C + c0 + 8 * a + 4 * h);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < NT; ++t) {
           au[t][4 * a] = b1.x; au[t][4 * a + 1] = b1.y; au[t][4 * a + 2] = b1.z; au[t][4 * a + 3] = b1.w;
           av[t][4 * a] = b2.x; av[t][4 * a + 1] = b2.y; av[t][4 * a + 2] = b2.z; av[t][4 * a + 3] = b2.w;
         }
@@ -1426,13 +1436,36 @@ __global__ void __launch_bounds__(512, 2)
           const uint4 a1 = *reinterpret_cast<const uint4*>(sw1 + wo);
           const uint4 a2 = *reinterpret_cast<const uint4*>(sw2 + wo);
 #pragma unroll
-          for (int t = 0; t < 2; ++t) {
+          for (int t = 0; t < NT; ++t) {
             mma_step<TI>(au[t], a1, xf[t][s2][q]);
-            mma_step<TI>(av[t], a2, xf[t][s2][q]);
+            mma_step<TI>(av[t], a2, ROWS ? xf2[t][s2][q] : xf[t][s2][q]);
           }
         }
+      if constexpr (ROWS) {
+        // result by rows (M x C): the lane holds its own row m and, of this chunk, c = 8 (v >> 2) + 4 h + (v & 3); the lane
+        // halves swap register pairs (v_permlane32_swap), after which each stores 16 contiguous bytes of its row
+        uint32_t pk[8];
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int a = 0; a < 4; ++a) {
+          float g[4];
+#pragma unroll
+          for (int b = 0; b < 4; ++b) {
+            const int v = 4 * a + b;
+            g[b] = __builtin_amdgcn_rcpf(1.0f + __expf(-au[0][v])) * av[0][v] * mk[0];
+          }
+          pk[2 * a] = pack_bf16(g[0], g[1]);
+          pk[2 * a + 1] = pack_bf16(g[2], g[3]);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const auto s0 = __builtin_amdgcn_permlane32_swap(pk[4 * j], pk[4 * j + 2], false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(pk[4 * j + 1], pk[4 * j + 3], false, false);
+          if (mcol[0] < M)
+            *reinterpret_cast<uint4*>(out + static_cast<int64_t>(mcol[0]) * ldc + c0 + 16 * j + 8 * h) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+        }
+      } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
           float g[4];
@@ -1452,6 +1485,7 @@ __global__ void __launch_bounds__(512, 2)
             }
           }
         }
+      }
     }
   }
 }
@@ -2520,22 +2554,24 @@ extern "C" int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mo
 static size_t dual_gate_res_lds(int64_t C, int64_t K, bool ln) {
   return static_cast<size_t>(2 * C * (K == 128 ? 2 * K : 2 * K + 16) + 8 * C + (ln ? 8 * K : 0));
 }
-static bool dual_gate_res_fits(int64_t C, int64_t M, int64_t K, const void* out, int64_t ldc, bool ln) {
-  return K % 32 == 0 && K <= 128 && C % 32 == 0 && M % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0 && M >= 4096 &&
-         dual_gate_res_lds(C, K, ln) <= 160 * 1024;
+// by_rows: two inputs and the result M x C (16-byte row pieces); otherwise one input and the result C x M (4-byte column pairs)
+static bool dual_gate_res_fits(int64_t C, int64_t M, int64_t K, const void* out, int64_t ldc, bool ln, bool by_rows) {
+  const bool stores_ok = by_rows ? (ldc % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) : (M % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0);
+  return K % 32 == 0 && K <= 128 && C % 32 == 0 && stores_ok && M >= 4096 && dual_gate_res_lds(C, K, ln) <= 160 * 1024;
 }
-static int launch_dual_gate_res(int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X, int64_t ldx,
-                                const void* bias1, const void* bias2, const void* mask, void* out, int64_t ldc, const void* gamma,
+static int launch_dual_gate_res(int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X, const void* X2,
+                                int64_t ldx, const void* bias1, const void* bias2, const void* mask, void* out, int64_t ldc, const void* gamma,
                                 const void* beta, float eps, void* xhat, int64_t ldxh, float* mean, float* rstd, hipStream_t stream) {
+  const bool by_rows = X2 != nullptr;
   const size_t lds = dual_gate_res_lds(C, K, xhat != nullptr);
-  const int64_t ntiles = (M + 63) / 64;
+  const int64_t ntiles = (M + (by_rows ? 31 : 63)) / (by_rows ? 32 : 64);
   int64_t gx = (ntiles + 7) / 8;
   if (gx > device_cus()) gx = device_cus();
-#define DGR(KT, LN) do { auto kfn = dual_gate_res_kernel<KT, LN>; \
+#define DGR(KT, LN, RW) do { auto kfn = dual_gate_res_kernel<KT, LN, RW>; \
     CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<uint16_t*>(out), ldc, static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), eps, static_cast<uint16_t*>(xhat), ldxh, mean, rstd); } while (0)
-#define DGR_K(LN) do { switch (K / 32) { case 1: DGR(1, LN); break; case 2: DGR(2, LN); break; case 3: DGR(3, LN); break; default: DGR(4, LN); break; } } while (0)
-  if (xhat) DGR_K(true); else DGR_K(false);
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<uint16_t*>(out), ldc, static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), eps, static_cast<uint16_t*>(xhat), ldxh, mean, rstd); } while (0)
+#define DGR_K(LN, RW) do { switch (K / 32) { case 1: DGR(1, LN, RW); break; case 2: DGR(2, LN, RW); break; case 3: DGR(3, LN, RW); break; default: DGR(4, LN, RW); break; } } while (0)
+  if (by_rows) DGR_K(false, true); else if (xhat) DGR_K(true, false); else DGR_K(false, false);
 #undef DGR_K
 #undef DGR
   CUEQ_CHECK_HIP(hipGetLastError());
@@ -2576,8 +2612,14 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
   // forward with one shared right operand, biases along the rows and the mask along the columns, in a 2-byte type:
   // the left operands (the weights, M rows) stay resident in LDS when they fit
   if (dtype == CUEQ_BF16 && !backward && share && (!(bias1 || bias2) || bias_axis == 0) && (!mask || mask_axis == 1) &&
-      dual_gate_res_fits(M, N, K, out1, ldc, false)) {
-    return launch_dual_gate_res(M, N, K, A1, A2, lda, B1, ldb, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, stream);
+      dual_gate_res_fits(M, N, K, out1, ldc, false, false)) {
+    return launch_dual_gate_res(M, N, K, A1, A2, lda, B1, nullptr, ldb, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, stream);
+  }
+  // the mirrored case - two left operands of many rows, the weights on the right, biases along the columns and the mask
+  // along the rows: the same kernel with the weights (N rows) resident, two inputs and the result by rows
+  if (dtype == CUEQ_BF16 && !backward && !share && A2 != A1 && (!(bias1 || bias2) || bias_axis == 1) && (!mask || mask_axis == 0) && M <= kRowSlab &&
+      dual_gate_res_fits(N, M, K, out1, ldc, false, true)) {
+    return launch_dual_gate_res(N, M, K, B1, B2, ldb, A1, A2, lda, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, stream);
   }
 #define DG(TI, BW, SH) hipLaunchKernelGGL((dual_gate_kernel<TI, BW, SH>), grid, dim3(512), 0, stream, static_cast<const TI*>(A1), static_cast<const TI*>(A2), lda, static_cast<const TI*>(B1), static_cast<const TI*>(B2), ldb, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), bias_axis, static_cast<const TI*>(mask), mask_axis, static_cast<const TI*>(dC), static_cast<TI*>(out1), static_cast<TI*>(out2), ldc, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), vec_out)
 #define DG_T(TI) do { if (backward) { if (share) DG(TI, true, true); else DG(TI, true, false); } else { if (share) DG(TI, false, true); else DG(TI, false, false); } } while (0)
@@ -2600,10 +2642,10 @@ extern "C" int cueq_ln_dual_gate(int32_t dtype, int64_t C, int64_t M, int64_t K,
   CUEQ_REQUIRE((ptrs & 15) == 0 && ldw % 8 == 0 && ldx % 8 == 0 && ldxh % 8 == 0 && ldw >= K && ldx >= K && ldxh >= K, CUEQ_ERR_UNSUPPORTED,
                "ln_dual_gate: row strides and pointers must be multiples of 16 bytes");
   CUEQ_REQUIRE(M <= kRowSlab && C < (1ll << 31) && ldc >= M, CUEQ_ERR_TOO_LARGE, "ln_dual_gate: extent too large");
-  CUEQ_REQUIRE(dual_gate_res_fits(C, M, K, out, ldc, true), CUEQ_ERR_UNSUPPORTED,
+  CUEQ_REQUIRE(dual_gate_res_fits(C, M, K, out, ldc, true, false), CUEQ_ERR_UNSUPPORTED,
                "ln_dual_gate: needs K = 32, 64, 96 or 128, C a multiple of 32 that fits the local data share, an even M of at least 4096 and an even ldc");
   KernelTimer timer("ln_dual_gate_fwd", stream);
-  return launch_dual_gate_res(C, M, K, W1, W2, ldw, X, ldx, bias1, bias2, mask, out, ldc, gamma, beta, static_cast<float>(eps), xhat, ldxh, mean, rstd, stream);
+  return launch_dual_gate_res(C, M, K, W1, W2, ldw, X, nullptr, ldx, bias1, bias2, mask, out, ldc, gamma, beta, static_cast<float>(eps), xhat, ldxh, mean, rstd, stream);
 }
 
 extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,

@@ -13,6 +13,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle.triangle import triangle_multiplicative_update as oracle_trimul
+from cuequivariance_amd import _lib
 
 TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
 
@@ -381,6 +382,38 @@ def test_dual_gate_many_column_tiles(device, dtype, N, with_bias):
     got = T.dual_gate_fwd(dev(W1), dev(W2), dev(X), None, dev(b1), dev(b2), 0, dev(mask), 1)
     assert got.shape == (C, N) and got.dtype == dtype
     assert rel_err(got, want) <= TOL[dtype], rel_err(got, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("with_bias,masked", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("M,K,C", [(4096, 128, 128), (32 * 2048 * 2 + 32 * 9 + 5, 64, 96), (5001, 96, 32), (4100, 32, 256)])
+def test_dual_gate_two_inputs_result_by_rows(device, M, K, C, with_bias, masked):
+    """The forward gate of the output stage in bfloat16 - two inputs of many rows, the weights on the right, biases by column,
+    mask by row: the kernel with the weights resident in the local data share (rows past a multiple of 32, more tiles than
+    wavefronts, every K) against torch in float64 on the rounded inputs, and bit for bit against the tiled kernel that the
+    same call takes for fewer than 4096 rows."""
+    from cuequivariance_amd.cuet import triangle as T
+
+    g = torch.Generator(device=device).manual_seed(M + K + C)
+    r = lambda *s: torch.randn(*s, device=device, generator=g)
+    X1, X2 = r(M, K).bfloat16(), r(M, K).bfloat16()
+    W1, W2 = (r(C, K) / K ** 0.5).bfloat16(), (r(C, K) / K ** 0.5).bfloat16()
+    b1, b2 = (r(C).bfloat16(), r(C).bfloat16()) if with_bias else (None, None)
+    mask = (torch.rand(M, device=device, generator=g) > 0.2).bfloat16() if masked else None
+    lib = _lib.load()
+    lib.cueq_timing_begin()
+    got = T.dual_gate_fwd(X1, X2, W1, W2, b1, b2, 1, mask, 0)
+    torch.cuda.synchronize()
+    assert dict(_lib.timing_end()).get("dual_gate_fwd", (0, 0))[0] == 1
+    d = lambda t: t.double()
+    U = d(X1) @ d(W1).T + (d(b1) if with_bias else 0)
+    V = d(X2) @ d(W2).T + (d(b2) if with_bias else 0)
+    want = torch.sigmoid(U) * V * (d(mask)[:, None] if masked else 1)
+    assert got.shape == (M, C) and rel_err(got, want.cpu()) <= TOL[torch.bfloat16], rel_err(got, want.cpu())
+    # the same rows in pieces of fewer than 4096: the tiled kernel
+    for r0 in (0, M - 3000):
+        part = T.dual_gate_fwd(X1[r0:r0 + 3000], X2[r0:r0 + 3000], W1, W2, b1, b2, 1, None if mask is None else mask[r0:r0 + 3000], 0)
+        assert torch.equal(part, got[r0:r0 + 3000])
 
 
 @pytest.mark.gpu
