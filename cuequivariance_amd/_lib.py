@@ -57,6 +57,7 @@ EXPORTED_SYMBOLS = (
     "cueq_dual_gate",
     "cueq_ln_dual_gate",
     "cueq_gate_bwd_input",
+    "cueq_gate_bwd_input_ln",
     "cueq_gemm_tn_items",
     "cueq_gemm_tn",
     "cueq_transpose",
@@ -229,6 +230,8 @@ def load() -> C.CDLL:
         lib.cueq_gate_bwd_input.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, ptr, i64, ptr, ptr, ptr, ptr, i64,
                                             i32, ptr, ptr, i64, i32, ptr, ptr, ptr]
         lib.cueq_gate_bwd_input.restype = C.c_int
+        lib.cueq_gate_bwd_input_ln.argtypes = [i32, i64, i64, i64, ptr, ptr, i64, ptr, i64, ptr, ptr, ptr, ptr, i64, ptr, i64, i32, ptr, i64, ptr, ptr, ptr, ptr]
+        lib.cueq_gate_bwd_input_ln.restype = C.c_int
         lib.cueq_gemm_tn_items.argtypes = [i64, i32]
         lib.cueq_gemm_tn_items.restype = i64
         lib.cueq_gemm_tn.argtypes = [i32, i64, i64, i64, ptr, i64, i64, ptr, i64, i64, i32, ptr, f64, ptr]

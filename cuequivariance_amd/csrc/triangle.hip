@@ -964,14 +964,21 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
 // and the biases once, then its wavefronts walk 32-column tiles of m independently - no barrier and no weight
 // traffic inside the loop, and wavefronts of one SIMD drift into different phases (MFMA / gate math / memory).
 // LDS: 2 C (2 K + 16) bytes of weights + 8 C bytes of biases (+ with two inputs a wave-private 8-row staging tile for the results).
+//
+// LNB (one-input form): X1 holds the rows of a LayerNorm whose input rows, mean and 1 / std are given, and the kernel
+// goes on to the gradient with respect to those input rows - the lane has half of the gradient row in registers, so the two
+// row sums of the LayerNorm backward are sums over its own values completed by one exchange - and writes that to dX1.
 // ------------------------------------------------------------------------------------------------
-template <int KT, bool SPLIT, bool DC_BY_ROW>
+template <int KT, bool SPLIT, bool DC_BY_ROW, bool LNB = false>
 __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
     gate_bwd_input_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X1,
                               const uint16_t* __restrict__ X2, int64_t ldx, const uint16_t* __restrict__ bias1,
                               const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask, const uint16_t* __restrict__ dC,
                               int64_t ldc, uint16_t* __restrict__ dX1, uint16_t* __restrict__ dX2, int64_t lddx, int accumulate,
-                              uint16_t* __restrict__ dU, uint16_t* __restrict__ dV, int C, int M) {
+                              uint16_t* __restrict__ dU, uint16_t* __restrict__ dV, int C, int M, const uint16_t* __restrict__ ln_x = nullptr,
+                              int64_t ldlx = 0, const float* __restrict__ ln_mean = nullptr, const float* __restrict__ ln_rstd = nullptr,
+                              const uint16_t* __restrict__ ln_gamma = nullptr) {
+  static_assert(!(LNB && SPLIT), "the LayerNorm backward goes with the one-input form");
   using TI = uint16_t;
   constexpr int ES = 2, EPV = 8;
   constexpr int K = 32 * KT, ROWB = K * ES, NS = ROWB / 64, VPR = ROWB / 16;
@@ -990,6 +997,7 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   // (the wavefront's number as a scalar: tile indices and row bases derived from it stay in scalar registers)
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c = lane & 31, h = lane >> 5;
   char* stage = reinterpret_cast<char*>(sb + 2 * C) + wave * (8 * SSTR);  // (two inputs only)
+  float* sg = sb + 2 * C;                                                   // (LNB only) gamma[K]
 
   for (int e = tid; e < C * VPR; e += NTH) {
     const int r = e / VPR, part = e % VPR;
@@ -1000,6 +1008,9 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   for (int i = tid; i < C; i += NTH) {
     sb[i] = bias1 ? tri_load(bias1, i) : 0.f;
     sb[C + i] = bias2 ? tri_load(bias2, i) : 0.f;
+  }
+  if constexpr (LNB) {
+    for (int i = tid; i < K; i += NTH) sg[i] = ln_gamma ? tri_load(ln_gamma, i) : 1.f;
   }
   __syncthreads();
 
@@ -1227,6 +1238,64 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
           for (int j = 0; j < 2; ++j) old[ds][j] = *reinterpret_cast<const uint4*>(dX1 + orow + (ds * 64 + j * 32) / ES);
       }
       uint4 val[KT][2];
+      if constexpr (LNB) {
+        // dx = rstd (g - mean(g) - xn mean(g xn)) with g = dy gamma, xn = (x - mean) rstd, over the K elements of the row.
+        // The float accumulators are swapped into row order (k = 16 j + 8 h + e per 32 columns), what is added to them
+        // and the LayerNorm's input rows arrive in the same order.
+        uint4 xr[KT][2];
+        const int64_t xrow = static_cast<int64_t>(min(mrow, M - 1)) * ldlx + (h * 16) / ES;
+#pragma unroll
+        for (int ds = 0; ds < KT; ++ds)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) xr[ds][j] = *reinterpret_cast<const uint4*>(ln_x + xrow + (ds * 64 + j * 32) / ES);
+        const float mu = ln_mean[min(mrow, M - 1)], rs = ln_rstd[min(mrow, M - 1)];
+        float s1 = 0, s2 = 0;
+#pragma unroll
+        for (int ds = 0; ds < KT; ++ds) {
+          floatx16& acc = ax1[ds];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[8 * j + i]), __float_as_uint(acc[8 * j + 4 + i]), false, false);
+              acc[8 * j + i] = __uint_as_float(sw[0]);
+              acc[8 * j + 4 + i] = __uint_as_float(sw[1]);
+            }
+            const int k0 = ds * 32 + j * 16 + h * 8;
+            const float4 g0 = *reinterpret_cast<const float4*>(sg + k0), g1 = *reinterpret_cast<const float4*>(sg + k0 + 4);
+            const float gm[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+            const uint32_t ow[4] = {old[ds][j].x, old[ds][j].y, old[ds][j].z, old[ds][j].w};
+            const uint32_t xw[4] = {xr[ds][j].x, xr[ds][j].y, xr[ds][j].z, xr[ds][j].w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              float d = acc[8 * j + e];
+              if (accumulate) d += (e & 1) ? hi_bf16(ow[e >> 1]) : lo_bf16(ow[e >> 1]);
+              const float g = d * gm[e];
+              const float xn = (((e & 1) ? hi_bf16(xw[e >> 1]) : lo_bf16(xw[e >> 1])) - mu) * rs;
+              s1 += g;
+              s2 = fmaf(g, xn, s2);
+              acc[8 * j + e] = g;
+            }
+          }
+        }
+        s1 = (s1 + __shfl_xor(s1, 32, 64)) * (1.0f / K);
+        s2 = (s2 + __shfl_xor(s2, 32, 64)) * (1.0f / K);
+#pragma unroll
+        for (int ds = 0; ds < KT; ++ds) {
+          const floatx16& acc = ax1[ds];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const uint32_t xw[4] = {again(xr[ds][j].x), again(xr[ds][j].y), again(xr[ds][j].z), again(xr[ds][j].w)};
+            uint32_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float x0 = (lo_bf16(xw[e]) - mu) * rs, x1 = (hi_bf16(xw[e]) - mu) * rs;
+              o[e] = pack_bf16(rs * (acc[8 * j + 2 * e] - s1 - x0 * s2), rs * (acc[8 * j + 2 * e + 1] - s1 - x1 * s2));
+            }
+            val[ds][j] = make_uint4(o[0], o[1], o[2], o[3]);
+          }
+        }
+      } else {
 #pragma unroll
       for (int ds = 0; ds < KT; ++ds) {
         const floatx16& acc = ax1[ds];
@@ -1239,6 +1308,7 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
           val[ds][j] = make_uint4(s0[0], s1[0], s0[1], s1[1]);
           if (accumulate) val[ds][j] = add_vec<TI>(val[ds][j], old[ds][j]);
         }
+      }
       }
       __builtin_amdgcn_sched_barrier(0);
       if (mrow < M) {
@@ -2648,11 +2718,12 @@ extern "C" int cueq_ln_dual_gate(int32_t dtype, int64_t C, int64_t M, int64_t K,
   return launch_dual_gate_res(C, M, K, W1, W2, ldw, X, nullptr, ldx, bias1, bias2, mask, out, ldc, gamma, beta, static_cast<float>(eps), xhat, ldxh, mean, rstd, stream);
 }
 
-extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
-                                   const void* X1, const void* X2, int64_t ldx,
-                                   const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
-                                   int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
-                                   void* stream_) {
+// ln_x != NULL: the LayerNorm backward in the same kernel (cueq_gate_bwd_input_ln)
+static int gate_bwd_input_impl(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
+                               const void* X1, const void* X2, int64_t ldx,
+                               const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
+                               int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
+                               const void* ln_x, int64_t ldlx, const float* ln_mean, const float* ln_rstd, const void* ln_gamma, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   CUEQ_REQUIRE(is_io(dtype), CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: dtype must be float32 or bfloat16");
   CUEQ_REQUIRE(C >= 0 && M >= 0 && K > 0, CUEQ_ERR_INVALID, "gate_bwd_input: bad extents");
@@ -2690,28 +2761,34 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
   CUEQ_REQUIRE(ldc >= 0 && ldw >= 0 && 32 * ldw * es < (1ll << 31) &&
                    (dc_by_row ? (4 * ldc + M) : (M * ldc + 8)) * es < (1ll << 32),
                CUEQ_ERR_TOO_LARGE, "gate_bwd_input: strides too large for 32-bit lane offsets");
-  KernelTimer timer("gate_bwd_input", stream);
+  KernelTimer timer(ln_x ? "gate_bwd_input_ln" : "gate_bwd_input", stream);
   if (bf) {
     // weights resident in LDS when they fit (2 C rows of 2 K + 16 bytes, biases, with two inputs the staging tiles)
     const int nwaves = split ? 4 : 8;
-    const size_t lds = static_cast<size_t>(2 * C * (K == 128 ? 2 * K : 2 * K + 16) + 8 * C + (split ? nwaves * 8 * (2 * K + 16) : 0));
+    const size_t lds = static_cast<size_t>(2 * C * (K == 128 ? 2 * K : 2 * K + 16) + 8 * C + (split ? nwaves * 8 * (2 * K + 16) : 0) + (ln_x ? 4 * K : 0));
     // (dC by rows is read, and the gate gradients written, as 4-byte column pairs)
     const bool pairs_ok = !dc_by_row || (M % 2 == 0 && ldc % 2 == 0 && reinterpret_cast<uintptr_t>(dC) % 4 == 0);
     if (lds <= 160 * 1024 && pairs_ok) {
       const int64_t ntiles = (M + 31) / 32;
       int64_t gx = (ntiles + nwaves - 1) / nwaves;
       if (gx > device_cus()) gx = device_cus();
-#define GBR(KT, SP) do { auto kfn = gate_bwd_input_res_kernel<KT, SP, !SP>; \
+#define GBR(KT, SP) do { auto kfn = gate_bwd_input_res_kernel<KT, SP, !SP, false>; \
         CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(SP ? 256 : 512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X1), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<const uint16_t*>(dC), ldc, static_cast<uint16_t*>(dX1), static_cast<uint16_t*>(dX2), lddx, accumulate, static_cast<uint16_t*>(dU), static_cast<uint16_t*>(dV), static_cast<int>(C), static_cast<int>(M)); } while (0)
+        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(SP ? 256 : 512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X1), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<const uint16_t*>(dC), ldc, static_cast<uint16_t*>(dX1), static_cast<uint16_t*>(dX2), lddx, accumulate, static_cast<uint16_t*>(dU), static_cast<uint16_t*>(dV), static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(nullptr), int64_t(0), static_cast<const float*>(nullptr), static_cast<const float*>(nullptr), static_cast<const uint16_t*>(nullptr)); } while (0)
 #define GBR_K(SP) do { switch (K / 32) { case 1: GBR(1, SP); break; case 2: GBR(2, SP); break; case 3: GBR(3, SP); break; default: GBR(4, SP); break; } } while (0)
-      if (split) GBR_K(true); else GBR_K(false);
+#define GBL(KT) do { auto kfn = gate_bwd_input_res_kernel<KT, false, true, true>; \
+        CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
+        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X1), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<const uint16_t*>(dC), ldc, static_cast<uint16_t*>(dX1), static_cast<uint16_t*>(dX2), lddx, accumulate, static_cast<uint16_t*>(dU), static_cast<uint16_t*>(dV), static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(ln_x), ldlx, ln_mean, ln_rstd, static_cast<const uint16_t*>(ln_gamma)); } while (0)
+      if (ln_x) { switch (K / 32) { case 1: GBL(1); break; case 2: GBL(2); break; case 3: GBL(3); break; default: GBL(4); break; } }
+      else if (split) GBR_K(true); else GBR_K(false);
+#undef GBL
 #undef GBR_K
 #undef GBR
       CUEQ_CHECK_HIP(hipGetLastError());
       return CUEQ_OK;
     }
   }
+  CUEQ_REQUIRE(!ln_x, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input_ln: needs bfloat16, the weights fitting the local data share, an even M and ldc (compose cueq_gate_bwd_input and cueq_layer_norm_bwd otherwise)");
 #define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP, !SP>), dim3(static_cast<unsigned>((M + gbi_threads<TI, SP>() / 2 - 1) / (gbi_threads<TI, SP>() / 2))), dim3(gbi_threads<TI, SP>()), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
 #define GBI_K(TI, SP) do { switch (K / 32) { case 1: GBI(TI, 1, SP); break; case 2: GBI(TI, 2, SP); break; case 3: GBI(TI, 3, SP); break; default: GBI(TI, 4, SP); break; } } while (0)
 #define GBI_T(TI) do { if (split) GBI_K(TI, true); else GBI_K(TI, false); } while (0)
@@ -2721,6 +2798,27 @@ extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t 
 #undef GBI
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
+}
+
+extern "C" int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw,
+                                   const void* X1, const void* X2, int64_t ldx,
+                                   const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
+                                   int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
+                                   void* stream_) {
+  return gate_bwd_input_impl(dtype, C, M, K, W1, W2, ldw, X1, X2, ldx, bias1, bias2, mask, dC, ldc, dc_by_row, dX1, dX2, lddx, accumulate, dU, dV,
+                             nullptr, 0, nullptr, nullptr, nullptr, stream_);
+}
+
+extern "C" int cueq_gate_bwd_input_ln(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X,
+                                      int64_t ldx, const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
+                                      void* dX, int64_t lddx, int32_t accumulate, const void* ln_x, int64_t ldlx, const float* ln_mean,
+                                      const float* ln_rstd, const void* ln_gamma, void* stream_) {
+  CUEQ_REQUIRE(dtype == CUEQ_BF16, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input_ln: built for bfloat16");
+  CUEQ_REQUIRE(ln_x && ln_mean && ln_rstd, CUEQ_ERR_INVALID, "gate_bwd_input_ln: null operand");
+  CUEQ_REQUIRE(reinterpret_cast<uintptr_t>(ln_x) % 16 == 0 && ldlx % 8 == 0 && ldlx >= K, CUEQ_ERR_UNSUPPORTED,
+               "gate_bwd_input_ln: the LayerNorm input rows must be 16-byte aligned");
+  return gate_bwd_input_impl(dtype, C, M, K, W1, W2, ldw, X, nullptr, ldx, bias1, bias2, mask, dC, ldc, 1, dX, nullptr, lddx, accumulate, nullptr, nullptr,
+                             ln_x, ldlx, ln_mean, ln_rstd, ln_gamma, stream_);
 }
 
 extern "C" int64_t cueq_gemm_tn_items(int64_t rows, int32_t nparts) {

@@ -282,6 +282,33 @@ def gate_bwd_input(dC, dc_by_row: bool, W1, W2, X1, X2, bias1, bias2, mask, dX1=
     return dX1, dX2, dU, dV
 
 
+def gate_bwd_input_ln(dC, W1, W2, X, bias1, bias2, mask, dX, ln_x, ln_mean, ln_rstd, ln_gamma):
+    """:func:`gate_bwd_input` in its one-input form (``dC`` is ``(C, M)``) continued through the LayerNorm that produced ``X``
+    from ``ln_x``, in one kernel (``cueq_gate_bwd_input_ln``): ``dX`` (the gradient that has already arrived at ``X``, or
+    ``None``) is replaced by the gradient with respect to ``ln_x``.  Returns it, or ``None`` when the shapes do not allow the
+    kernel (then :func:`gate_bwd_input` and :func:`layer_norm_bwd` do the same in two launches)."""
+    Cn, K = W1.shape
+    M = X.shape[0]
+    T = W1.dtype
+    if T != torch.bfloat16 or K % 32 or K > 128 or Cn % 32 or M % 2 or dC.stride(0) % 2 or dC.data_ptr() % 4:
+        return None
+    if 2 * Cn * (2 * K if K == 128 else 2 * K + 16) + 8 * Cn + 4 * K > 160 * 1024 or not _fusable(W1, W2, X, dX, ln_x):
+        return None
+    if (4 * dC.stride(0) + M) * 2 >= (1 << 32) or M >= (1 << 31) - 128:
+        return None
+    accumulate = dX is not None
+    if dX is None:
+        dX = torch.empty(M, K, dtype=T, device=W1.device)
+    _lib.check(
+        _lib.load().cueq_gate_bwd_input_ln(_CODE[T], Cn, M, K, W1.data_ptr(), W2.data_ptr(), W1.stride(0), X.data_ptr(), X.stride(0),
+                                           _ptr(bias1), _ptr(bias2), _ptr(mask), dC.data_ptr(), dC.stride(0), dX.data_ptr(), dX.stride(0),
+                                           int(accumulate), ln_x.data_ptr(), ln_x.stride(0), ln_mean.data_ptr(), ln_rstd.data_ptr(),
+                                           _ptr(ln_gamma), _stream(W1)),
+        "cueq_gate_bwd_input_ln",
+    )
+    return dX
+
+
 def sum_cols(x: torch.Tensor) -> torch.Tensor:
     rows, cols = x.shape
     out = torch.empty(rows, dtype=torch.float32, device=x.device)
@@ -361,6 +388,10 @@ def _trimul_fwd(x, mask, nin_w, nin_b, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, n
         return out.view(Bsz, N, N, Do), saved, (Bsz, N, D, Do), has
 
 
+def _cast(g, like, have):
+    return g.to(like.dtype) if (g is not None and have) else None
+
+
 def _trimul_bwd(saved, dims, has, outgoing: bool, need, dout):
     """Gradients for the 16 arguments of :func:`_trimul_fwd` (``need[k]``: whether argument ``k`` wants one)."""
     if True:
@@ -414,7 +445,14 @@ def _trimul_bwd(saved, dims, has, outgoing: bool, need, dout):
             gemm_nt(b, dt, T, out=da)  # da[k, i] = sum_j b[k, j] dt[i, j]
             gemm_nt(a, dt, T, out=db, trans_b=True)  # db[k, j] = sum_i a[k, i] dt[i, j]
 
-        # input gate and projections
+        # input gate and projections - and, when neither their weights nor the LayerNorm's ask for a gradient, the input
+        # LayerNorm in the same kernel
+        affine_in = (has[0] and need[2]) or (has[1] and need[3])
+        if not w_in and not affine_in and need[0]:
+            dx = gate_bwd_input_ln(dab, g_in_w, p_in_w, xh, g_in_b, p_in_b, mflat, dxh, x2, mean1, rstd1, nin_w)
+            if dx is not None:
+                return (dx.view(Bsz, N, N, D), None, None, None, None, None, None, None, _cast(d_nout_w, x2, has[2]), _cast(d_nout_b, x2, has[3]),
+                        d_p_out_w, d_p_out_b, d_g_out_w, d_g_out_b, None, None)
         fused = gate_bwd_input(dab, True, g_in_w, p_in_w, xh, None, g_in_b, p_in_b, mflat, dxh, w_in)
         if fused is not None:
             du1, dv1 = fused[2], fused[3]
@@ -433,15 +471,10 @@ def _trimul_bwd(saved, dims, has, outgoing: bool, need, dout):
             d_p_in_b = sum_cols(dv1).to(p_in_b.dtype)
 
         # input LayerNorm
-        affine_in = (has[0] and need[2]) or (has[1] and need[3])
         dx, d_nin_w, d_nin_b = layer_norm_bwd(dxh, x2, mean1, rstd1, nin_w, affine_in)
         dx = dx.view(Bsz, N, N, D) if need[0] else None
-
-        def cast(g, like, have):
-            return g.to(like.dtype) if (g is not None and have) else None
-
-        return (dx, None, cast(d_nin_w, x2, has[0]), cast(d_nin_b, x2, has[1]), d_p_in_w, d_p_in_b, d_g_in_w, d_g_in_b,
-                cast(d_nout_w, x2, has[2]), cast(d_nout_b, x2, has[3]), d_p_out_w, d_p_out_b, d_g_out_w, d_g_out_b, None, None)
+        return (dx, None, _cast(d_nin_w, x2, has[0]), _cast(d_nin_b, x2, has[1]), d_p_in_w, d_p_in_b, d_g_in_w, d_g_in_b,
+                _cast(d_nout_w, x2, has[2]), _cast(d_nout_b, x2, has[3]), d_p_out_w, d_p_out_b, d_g_out_w, d_g_out_b, None, None)
 
 
 class _TriMul(torch.autograd.Function):

@@ -325,6 +325,18 @@ int cueq_gate_bwd_input(int32_t dtype, int64_t C, int64_t M, int64_t K, const vo
                         int32_t dc_by_row, void* dX1, void* dX2, int64_t lddx, int32_t accumulate, void* dU, void* dV,
                         void* stream);
 
+/* cueq_gate_bwd_input in its one-input form with dC by rows, continued through the LayerNorm that produced X
+ * (cuequivariance_jax/cuequivariance_jax/triangle/_triangle_multiplicative_update.py:371-400 backwards: the gradient of the input
+ * projections and of x_hat = LN(x) in one kernel): with d = (dX if accumulate else 0) + sum_c du[c][m] W1[c,:] + dv[c][m] W2[c,:],
+ *   g = d * ln_gamma,  xn = (ln_x - ln_mean) * ln_rstd,  dX[m,:] = ln_rstd[m] * (g - mean_k(g) - xn * mean_k(g * xn))
+ * (ln_x: the M x K rows the LayerNorm took, row stride ldlx; ln_gamma may be NULL).  The gradients of gamma / beta and the gate
+ * gradients are not formed here.  bfloat16 only, same shape limits as the resident form of cueq_gate_bwd_input; otherwise
+ * CUEQ_ERR_UNSUPPORTED (compose cueq_gate_bwd_input and cueq_layer_norm_bwd instead). */
+int cueq_gate_bwd_input_ln(int32_t dtype, int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X,
+                           int64_t ldx, const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc, void* dX,
+                           int64_t lddx, int32_t accumulate, const void* ln_x, int64_t ldlx, const float* ln_mean, const float* ln_rstd,
+                           const void* ln_gamma, void* stream);
+
 /* Weight-gradient shaped product C (M x N) = sum over rows z and parts p of A[z, p*stride_a : +M]^T B[z, p*stride_b : +N]
  * (both operands row-major with the long index z as rows).  The rows are cut into chunks = items / nparts pieces; item
  * (part, chunk) writes alpha * its partial product to partials[part * chunks + chunk] (float32, M x N): the partials of one

@@ -359,6 +359,46 @@ def test_gate_bwd_input_many_tiles(device, dtype, split, M):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("with_prior,affine", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("M,K,C", [(2048 * 32 + 37 * 32 + 8, 128, 256), (3 * 32 + 8, 64, 64), (1000, 96, 32), (262144, 128, 256)])
+def test_gate_bwd_input_through_the_layer_norm(device, M, K, C, with_prior, affine):
+    """``cueq_gate_bwd_input_ln`` (bfloat16): the gradient of the input projections continued through the LayerNorm of their
+    input, against torch in float64 on the rounded inputs - d/dx of sum(dC * sigmoid(U) * V * mask) + sum(prior * xh) with
+    xh = LN(x), U = W1 xh^T + b1, V = W2 xh^T + b2, where xh enters the products as the kernel reads it (rounded to bfloat16)
+    and the LayerNorm backward takes the stored mean and 1 / std.  More tiles than wavefronts, a partial last tile, every K."""
+    from cuequivariance_amd.cuet import triangle as T
+
+    g = torch.Generator(device=device).manual_seed(M + K + C)
+    r = lambda *s: torch.randn(*s, device=device, generator=g)
+    x = (r(M, K) * 1.4 + 0.3).bfloat16()
+    gamma = (r(K) * 0.5 + 1.0).bfloat16() if affine else None
+    beta = r(K).bfloat16() if affine else None
+    xh, mean, rstd = T.layer_norm_fwd(x, gamma, beta, 1e-5)
+    W1, W2 = (r(C, K) / K ** 0.5).bfloat16(), (r(C, K) / K ** 0.5).bfloat16()
+    b1, b2 = r(C).bfloat16(), r(C).bfloat16()
+    mask = (torch.rand(M, device=device, generator=g) > 0.2).bfloat16()
+    dC = r(C, M).bfloat16()
+    prior = r(M, K).bfloat16() if with_prior else None
+    got = T.gate_bwd_input_ln(dC, W1, W2, xh, b1, b2, mask, None if prior is None else prior.clone(), x, mean, rstd, gamma)
+    assert got is not None and got.shape == (M, K) and got.dtype == torch.bfloat16
+    d = lambda t: t.double()
+    U = d(W1) @ d(xh).T + d(b1)[:, None]
+    V = d(W2) @ d(xh).T + d(b2)[:, None]
+    dCm = d(dC) * d(mask)[None, :]
+    sg = torch.sigmoid(U)
+    dxh = (dCm * V * sg * (1 - sg)).T @ d(W1) + (dCm * sg).T @ d(W2) + (d(prior) if with_prior else 0)
+    gg = dxh * (d(gamma) if affine else 1)
+    xn = (d(x) - d(mean)[:, None]) * d(rstd)[:, None]
+    want = d(rstd)[:, None] * (gg - gg.mean(1, keepdim=True) - xn * (gg * xn).mean(1, keepdim=True))
+    assert rel_err(got, want.cpu()) <= TOL[torch.bfloat16], rel_err(got, want.cpu())
+    # the two launches it replaces (they round the gradient of xh to bfloat16 in between)
+    two = T.gate_bwd_input(dC, True, W1, W2, xh, None, b1, b2, mask, None if prior is None else prior.clone(), False)[0]
+    two = T.layer_norm_bwd(two, x, mean, rstd, gamma, False)[0]
+    assert rel_err(two, want.cpu()) <= TOL[torch.bfloat16]
+    assert (got.float() - two.float()).abs().max().item() <= 2.0 ** -5 * want.abs().max().item()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("N", [64 * 2048 + 64 * 5 + 2, 4096 + 34])
 @pytest.mark.parametrize("with_bias", [True, False])
