@@ -84,3 +84,16 @@ def test_dense_entries_refuse_bad_arguments_before_any_launch():
     # fully-connected stages: block width, operand width
     assert lib.cueq_fc_combine(F32, F32, 4, p, 1, p, 1, p, 1, p, 1, p, 512, 0, None) == -1
     assert lib.cueq_fc_rowdot(F32, F32, 4, p, 1, p, 1, p, 1, 100, p, 1, 0, None) == -2
+    # LayerNorm fused into the gated projection: bfloat16 only, row count, weights that do not fit the local data share
+    ln = lambda dtype, C, M, K, ldc: lib.cueq_ln_dual_gate(dtype, C, M, K, p, p, K, p, K, None, None, 1e-5, None, None, None, p, ldc, p, K, p, p, None)
+    assert ln(F32, 256, 8192, 128, 8192) == -2 and b"bfloat16" in lib.cueq_last_error()
+    assert ln(BF16, 256, 2048, 128, 2048) == -2 and b"at least 4096" in lib.cueq_last_error()
+    assert ln(BF16, 256, 8192, 160, 8192) == -2
+    assert ln(BF16, 1024, 8192, 128, 8192) == -2  # 2 x 1024 x 256 bytes of weights
+    assert ln(BF16, 256, 8192, 128, 4096) == -4  # result rows shorter than M
+    assert ln(BF16, 256, 0, 128, 0) == 0
+    # gate backward continued through the LayerNorm: bfloat16 only, the LayerNorm's input rows given and aligned
+    lnb = lambda dtype, lx, ldlx: lib.cueq_gate_bwd_input_ln(dtype, 256, 8192, 128, p, p, 128, p, 128, None, None, None, p, 8192, p, 128, 0, lx, ldlx, p, p,
+                                                             None, None)
+    assert lnb(F32, p, 128) == -2 and lnb(BF16, None, 128) == -1 and lnb(BF16, p + 8, 128) == -2 and lnb(BF16, p, 100) == -2
+
