@@ -226,7 +226,9 @@ __global__ void __launch_bounds__(64 * kLrWaves, 1)
   char* stage = smem + nslots * (N * WRS) + wave * kLrStageBytes;
   const char* wlane = smem + c * WRS + h * (ES == 2 ? 32 : 16);
   const int nfull = M / 32;  // tiles of 32 existing rows
-  const int wslot = blockIdx.x * kLrWaves + wave, nw = gridDim.x * kLrWaves;
+  // (slots numbered wavefront-major: when the units do not divide evenly, the wavefronts with one unit more are spread over
+  // the CUs and their SIMDs instead of filling the first blocks)
+  const int wslot = wave * gridDim.x + blockIdx.x, nw = gridDim.x * kLrWaves;
   // unit = tile * nparts + part; this wavefront takes the units wslot, wslot + nw, ... - walked as (tile, part) pairs
   const int step_t = nw / nparts, step_p = nw % nparts;
   auto advance = [&](int& t, int& p) {
