@@ -254,6 +254,10 @@ def load() -> C.CDLL:
         lib.cueq_sum_rows_workspace.restype = i64
         lib.cueq_sum_rows.argtypes = [i32, i64, i64, ptr, ptr, ptr, i64, ptr]
         lib.cueq_sum_rows.restype = C.c_int
+        # the library has read the environment itself at this point: remember what it saw, so that the first launch does
+        # not push those values again over an option set by cueq_set_option in the meantime
+        for env, _ in _ENV_OPTIONS:
+            _env_seen[env] = os.environ.get(env)
         _lib = lib
     return _lib
 
@@ -263,14 +267,25 @@ _env_seen: dict = {}
 
 
 def sync_options_from_env() -> None:
-    """The library reads CUEQ_DETERMINISTIC / CUEQ_FORCE_GENERIC once; a process that changes them afterwards
-    (``os.environ[...] = "1"``) is followed here: called by the Python launch paths, two dictionary lookups when
-    nothing changed."""
+    """The library reads CUEQ_DETERMINISTIC / CUEQ_FORCE_GENERIC once, when it is loaded; a process that changes them
+    afterwards (``os.environ[...] = "1"``) is followed here: called by the Python launch paths, two dictionary lookups
+    when nothing changed.  Only a *change* of a variable is pushed, so an option set with ``set_option`` stays as set
+    until the variable of the same name is assigned a different value."""
+    lib = load()
     for env, name in _ENV_OPTIONS:
         v = os.environ.get(env)
-        if env not in _env_seen or _env_seen[env] != v:
+        if _env_seen.get(env) != v:
             _env_seen[env] = v
-            load().cueq_set_option(name, 1 if (v and v[0] == "1") else 0)
+            lib.cueq_set_option(name, 1 if (v and v[0] == "1") else 0)
+
+
+def set_option(name: str, value: int) -> None:
+    """``cueq_set_option`` ("deterministic", "force_generic"); raises for an unknown name."""
+    check(load().cueq_set_option(name.encode(), int(value)), f"cueq_set_option({name!r})")
+
+
+def get_option(name: str) -> int:
+    return int(load().cueq_get_option(name.encode()))
 
 
 def check(status: int, what: str) -> None:

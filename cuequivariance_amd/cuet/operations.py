@@ -104,7 +104,7 @@ class ChannelWiseTensorProduct(torch.nn.Module):
     the batch elements into ``size_out`` output rows.  The forward sums each output row's batch elements in batch
     order (bit-reproducible).  In the backward, the gradient of a gathered operand (``x1`` with ``indices_1``) is
     scattered with floating-point atomics by default - summation order, hence the last bits, vary from run to run; set
-    ``CUEQ_DETERMINISTIC=1`` (or ``cueq_set_option("deterministic", 1)``) for an ordered, bit-reproducible sum at the
+    ``CUEQ_DETERMINISTIC=1`` (or ``cuequivariance_amd._lib.set_option("deterministic", 1)``, the C entry point ``cueq_set_option``) for an ordered, bit-reproducible sum at the
     price of one more pass.  The other gradients are bit-reproducible in both modes.
     """
 

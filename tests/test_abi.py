@@ -97,3 +97,29 @@ def test_dense_entries_refuse_bad_arguments_before_any_launch():
                                                              None, None)
     assert lnb(F32, p, 128) == -2 and lnb(BF16, None, 128) == -1 and lnb(BF16, p + 8, 128) == -2 and lnb(BF16, p, 100) == -2
 
+
+
+def test_option_set_by_the_program_survives_the_environment_sync(monkeypatch):
+    """An option set with ``cueq_set_option`` stays as set when the launch path looks at the environment (only a change
+    of the variable is pushed); assigning the variable afterwards is followed."""
+    monkeypatch.delenv("CUEQ_DETERMINISTIC", raising=False)
+    lib = _lib.load()
+    _lib._env_seen["CUEQ_DETERMINISTIC"] = None  # what load() records when the variable is unset
+    try:
+        assert lib.cueq_set_option(b"deterministic", 1) == 0
+        _lib.sync_options_from_env()
+        assert lib.cueq_get_option(b"deterministic") == 1
+        _lib.set_option("deterministic", 0)
+        _lib.sync_options_from_env()
+        assert _lib.get_option("deterministic") == 0
+        monkeypatch.setenv("CUEQ_DETERMINISTIC", "1")
+        _lib.sync_options_from_env()
+        assert _lib.get_option("deterministic") == 1
+        monkeypatch.delenv("CUEQ_DETERMINISTIC")
+        _lib.sync_options_from_env()
+        assert _lib.get_option("deterministic") == 0
+        with pytest.raises(_lib.CueqError):
+            _lib.set_option("no_such_option", 1)
+    finally:
+        lib.cueq_set_option(b"deterministic", 0)
+        _lib._env_seen["CUEQ_DETERMINISTIC"] = None
