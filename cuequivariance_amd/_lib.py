@@ -47,6 +47,9 @@ EXPORTED_SYMBOLS = (
     "cueq_gemm",
     "cueq_gemm_table",
     "cueq_linear_rows",
+    "cueq_linear_rows_mul_ir",
+    "cueq_linear_dw_mul_ir_items",
+    "cueq_linear_dw_mul_ir",
     "cueq_fc_combine",
     "cueq_fc_rowdot",
     "cueq_gemm_grouped",
@@ -211,6 +214,12 @@ def load() -> C.CDLL:
         lib.cueq_gemm_table.restype = C.c_int
         lib.cueq_linear_rows.argtypes = [i32, i32, i64, i64, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i64, f64, ptr]
         lib.cueq_linear_rows.restype = C.c_int
+        lib.cueq_linear_rows_mul_ir.argtypes = [i32, i32, i64, i64, i64, i32, ptr, i64, ptr, i64, ptr, i64, ptr, i64, f64, ptr]
+        lib.cueq_linear_rows_mul_ir.restype = C.c_int
+        lib.cueq_linear_dw_mul_ir_items.argtypes = [i64, ptr, i32, ptr]
+        lib.cueq_linear_dw_mul_ir_items.restype = i64
+        lib.cueq_linear_dw_mul_ir.argtypes = [i32, i64, i64, i64, ptr, i64, ptr, i64, ptr, i32, ptr, f64, ptr]
+        lib.cueq_linear_dw_mul_ir.restype = C.c_int
         lib.cueq_fc_combine.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i32, ptr, i32, i32, ptr]
         lib.cueq_fc_combine.restype = C.c_int
         lib.cueq_fc_rowdot.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, i32, ptr, i32, i32, ptr]

@@ -17,43 +17,11 @@
 #include "common.h"
 #include "cw_common.h"
 #include "u1d_spec.h"
+#include "linear_rows_common.h"
 
 namespace cueq {
 
 namespace {
-
-typedef float lr_floatx16 __attribute__((ext_vector_type(16)));
-typedef __bf16 lr_bf16x8 __attribute__((ext_vector_type(8)));
-typedef float lr_floatx2 __attribute__((ext_vector_type(2)));
-typedef __bf16 lr_bf16x2 __attribute__((ext_vector_type(2)));
-typedef uint32_t lr_u32x4 __attribute__((ext_vector_type(4)));
-
-// 16-byte accesses marked as streams: every byte of A and C is touched once
-__device__ __forceinline__ uint4 lr_stream_load(const char* p) {
-  const lr_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const lr_u32x4*>(p));
-  return make_uint4(v.x, v.y, v.z, v.w);
-}
-__device__ __forceinline__ void lr_stream_store(uint4 v, void* p) {
-  const lr_u32x4 w = {v.x, v.y, v.z, v.w};
-  __builtin_nontemporal_store(w, reinterpret_cast<lr_u32x4*>(p));
-}
-
-constexpr int kLrWaves = 8;
-constexpr int kLrMaxParts = 48;
-constexpr int kLrMaxSlots = 8;
-
-struct LrPart {
-  int32_t a_off, c_off, slot;
-};
-struct LrParts {
-  LrPart part[kLrMaxParts];
-  int64_t w_off[kLrMaxSlots];
-};
-
-__device__ __forceinline__ uint32_t lr_pack(float lo, float hi) {
-  const lr_floatx2 f = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lr_bf16x2));
-}
 
 constexpr int kLrStageStride = 144;                 // bytes between the rows of a wavefront's staging tile: 128 of data + 16
 constexpr int kLrStageBytes = 32 * kLrStageStride;  // 32 rows
@@ -191,36 +159,7 @@ __global__ void __launch_bounds__(64 * kLrWaves, 1)
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  // the weight blocks into LDS, 16-byte vectors requested in batches of four before the first is stored (one wait per
-  // batch instead of one per vector)
-  constexpr int NTH = 64 * kLrWaves;
-  for (int s = 0; s < nslots; ++s) {
-    const TI* w = W + parts.w_off[s];
-    char* dst = smem + s * (N * WRS);
-    constexpr int NVEC = K * N / EPV;  // vectors of the block
-    for (int e0 = tid; e0 < NVEC; e0 += 4 * NTH) {
-      uint4 v[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const uint4*>(w + static_cast<int64_t>(e0 + j * NTH < NVEC ? e0 + j * NTH : e0) * EPV);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int e = e0 + j * NTH;
-        if (e >= NVEC) continue;
-        if (w_contraction_major) {  // K x N as it lies: the vector holds (k, n .. n + EPV - 1), which become column k of EPV rows
-          const int k = e / (N / EPV), n = (e % (N / EPV)) * EPV;
-          const uint32_t q[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-#pragma unroll
-          for (int i = 0; i < EPV; ++i) {
-            if constexpr (ES == 4) *reinterpret_cast<uint32_t*>(dst + (n + i) * WRS + 4 * k) = q[i];
-            else *reinterpret_cast<uint16_t*>(dst + (n + i) * WRS + 2 * k) = static_cast<uint16_t>(q[i >> 1] >> (16 * (i & 1)));
-          }
-        } else {  // N x K as it lies
-          const int n = e / (K / EPV), vv = e % (K / EPV);
-          *reinterpret_cast<uint4*>(dst + n * WRS + 16 * vv) = v[j];
-        }
-      }
-    }
-  }
+  lr_stage_weights<TI, 64 * kLrWaves>(W, parts, nslots, K, N, WRS, w_contraction_major, smem, tid);
   __syncthreads();
 
   char* stage = smem + nslots * (N * WRS) + wave * kLrStageBytes;

@@ -273,6 +273,32 @@ int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_
 int cueq_linear_rows(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
                      const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts, double alpha, void* stream);
 
+/* The same launch for rows that keep the irrep component contiguous (`mul_ir`: element (channel u, component i) of a block
+ * of D components at u * D + i).  The reference converts such rows to channel-contiguous ones in front of its dense
+ * kernels and back behind them (cuequivariance_torch/primitives/transpose.py:83-183, called from
+ * operations/linear.py:153-191); this entry point reads and writes them as they lie:
+ *   C[z, c_p + v * D + i] = alpha * sum_u A[z, a_p + u * D + i] * W_p[u, v]     for i < D, all rows z < M and parts p.
+ * A part reads K * D and writes N * D consecutive elements of a row.  D in {3, 5, 7} (a block of one component is the
+ * same in both layouts: cueq_linear_rows); N in {32, 64, 96, 128}; K a multiple of 64 (bfloat16) or 32 (float32) up to
+ * 128; other limits and the table as for cueq_linear_rows, with (blocks * N * (K * element size + 16) +
+ * waves * 16 * (128 * D + 16)) bytes <= 160 KiB, waves = 8 if D * N <= 384 else 4. */
+int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, int32_t D, const void* A,
+                            int64_t lda, const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts,
+                            double alpha, void* stream);
+
+/* Weight gradient of the same operation on `mul_ir` rows (the reference reaches it through autograd of its dense kernel
+ * after the transposition of cuequivariance_torch/primitives/transpose.py:83-183):
+ *   dW_p[u, v] = alpha * sum_{z < rows} sum_{i < D_p} A[z, a_p + u * D_p + i] * G[z, c_p + v * D_p + i]     (K x N, row-major)
+ * table: HOST memory, nparts (<= 32) rows of (a_p, c_p, D_p), D_p in {1, 3, 5, 7}, offsets multiples of 16 bytes; K, N in
+ * {32, 64, 96, 128}; bfloat16 or float32 inputs, float32 partial results.  Part p is cut into chunks of rows (counts in
+ * proportion to D_p); chunk c of part p writes its partial product to row first_item[p] + c of `partials` (K * N floats per
+ * row), and the caller adds the rows first_item[p] .. first_item[p + 1] - 1 in order (cueq_sum_rows): no atomics.
+ * cueq_linear_dw_mul_ir_items returns the number of rows `partials` needs for this call shape on the current device and
+ * fills first_item (nparts + 1 entries; may be NULL); -1 for a bad argument. */
+int64_t cueq_linear_dw_mul_ir_items(int64_t rows, const int64_t* table, int32_t nparts, int32_t* first_item);
+int cueq_linear_dw_mul_ir(int32_t dtype, int64_t K, int64_t N, int64_t rows, const void* A, int64_t lda, const void* G, int64_t ldg,
+                          const int64_t* table, int32_t nparts, float* partials, double alpha, void* stream);
+
 /* Grouped products on the tiled kernel, for a Linear whose weights are chosen per row by a sorted class index
  * (the closed indexed_linear op behind cuequivariance_torch/primitives/segmented_polynomial_indexed_linear.py:116-156):
  * offsets (device, int64, ngroups + 1) gives the row range [offsets[g], offsets[g+1]) of group g.
