@@ -5,12 +5,13 @@
 // product through autograd of its dense kernel after transposing the rows to channel-contiguous ones
 // (cuequivariance_torch/primitives/transpose.py:83-183, operations/linear.py:153-191); here the rows are read as they lie.
 //
-// A block of 256 threads owns one (part, chunk of rows).  Per step it takes 16 rows (8 of float): every thread loads one
-// run of 16 D bytes of A and one of G - 8 (4) channels with all their components - and scatters the elements into LDS
-// planes [component][channel][row] (rows contiguous, 48 bytes per channel), from which the lanes read MFMA operands with
-// the rows as contraction index: one 16-byte read per 32 x 32 tile side, component and step.  The four wavefronts split
+// A block of 256 threads owns one (part, chunk of rows).  Per step it takes 16 rows (8 of float): the rows are loaded as
+// they lie (whole 128-byte lines per instruction) and every element is scattered into LDS planes
+// [component][row half][channel][8 (4) rows = 16 bytes] - the slot addresses are D registers per operand plus immediate
+// offsets - from which the lanes read MFMA operands with the rows as contraction index: one 16-byte read per 32 x 32 tile
+// side, component and step, 512 contiguous bytes per half wavefront.  The four wavefronts split
 // the K x N result two by two.  Parts of different D run in one launch (the block branches once on its part's D), with
-// chunk counts in proportion to D so that all blocks carry about the same work.
+// chunk counts in proportion to D + 1 so that all blocks carry about the same work.
 
 #include "common.h"
 #include "cw_common.h"
@@ -24,7 +25,6 @@ typedef float dw_floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 dw_bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kDwMaxParts = 32;
-constexpr int kDwZS = 48;  // bytes between the channels of a plane: 32 bytes of rows + 16
 
 struct DwParts {
   int32_t a_off[kDwMaxParts], c_off[kDwMaxParts], d[kDwMaxParts];
@@ -35,50 +35,64 @@ template <typename TI, int D>
 __device__ __forceinline__ void dw_body(const TI* __restrict__ A, int64_t lda, const TI* __restrict__ G, int64_t ldg, float* __restrict__ P,
                                         int K, int N, int64_t z_begin, int64_t z_end, float alpha, char* smem) {
   constexpr int ES = sizeof(TI);
-  constexpr int EPG = 16 / ES;   // channels per run
-  constexpr int ZR = 2 * EPG;    // rows per step: 16 (2-byte type) or 8 (float)
+  constexpr int EPV = 16 / ES;    // elements per 16-byte vector
+  constexpr int ZR = 2 * EPV;     // rows per step: 16 (2-byte type) or 8 (float)
+  constexpr int ZH = ZR / 2;      // rows per 16-byte slot
+  constexpr int EPL = 128 / ES;   // elements per 128-byte line
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int KT = K / 32, NT = N / 32;
   const int TU = (KT + 1) / 2, TV = (NT + 1) / 2;  // tiles of a wavefront along u and v (at most 2 x 2)
-  const int PLX = K * kDwZS, PLG = N * kDwZS;      // bytes of a plane
+  // planes [component][row half][channel][16 bytes = ZH rows]; 16 bytes more per plane so that planes start on different banks
+  const int PLX = K * 32 + 16, PLG = N * 32 + 16;
   char* sx = smem;
   char* sg = smem + D * PLX;
 
-  // the thread's runs: row tid / (K / EPG), channels EPG * (tid % (K / EPG)) ... of A; the same with N for G
-  const int gx = K / EPG, gg = N / EPG;
-  const int xr = tid / gx, xq = tid - xr * gx;
-  const int gr = tid / gg, gq = tid - gr * gg;
-  const bool xon = xr < ZR, gon = gr < ZR;
-  const TI* xp = A + xq * (EPG * D);
-  const TI* gp = G + gq * (EPG * D);
-  char* xdst = sx + xq * EPG * kDwZS + xr * ES;
-  char* gdst = sg + gq * EPG * kDwZS + gr * ES;
+  // Loads: eight lanes per 128-byte line; instruction v of a thread takes line v * (32 / ZR) + gidx / ZR of row gidx % ZR
+  // (gidx = tid / 8), so every instruction covers whole lines and the row of a thread is the same for all v.
+  // Element j of that vector is element E = E0 + 128 v + j of the row piece, E0 = (gidx / ZR) * EPL + (tid % 8) * EPV, i.e.
+  // channel E / D, component E % D.  With r0 = E0 % D the slot of element (v, j) is  slot[(128 v + j) % D] + 16 * ((128 v + j) / D),
+  // where slot[k] is the address of (channel E0 / D + (r0 + k) / D, component (r0 + k) % D, the thread's row): D address
+  // registers per operand, everything else is an immediate offset.
+  const int gidx = tid >> 3, l8 = tid & 7;
+  const int row = gidx % ZR, line0 = gidx / ZR;
+  const int E0 = line0 * EPL + l8 * EPV, r0 = E0 % D, u0 = E0 / D;
+  const int VRX = K * D / EPV, VRG = N * D / EPV;  // 16-byte vectors per row piece
+  const TI* xp = A + row * lda + E0;
+  const TI* gp = G + row * ldg + E0;
+  char* xslot[D];
+  char* gslot[D];
+#pragma unroll
+  for (int k = 0; k < D; ++k) {
+    const int du = (r0 + k) / D, i = (r0 + k) % D;
+    xslot[k] = sx + i * PLX + (row / ZH) * (K * 16) + (u0 + du) * 16 + (row % ZH) * ES;
+    gslot[k] = sg + i * PLG + (row / ZH) * (N * 16) + (u0 + du) * 16 + (row % ZH) * ES;
+  }
 
   uint4 rx[D], rg[D];
   auto load_step = [&](int64_t z) {
-    const bool okx = xon && z + xr < z_end, okg = gon && z + gr < z_end;
+    const bool ok = z + row < z_end;
 #pragma unroll
     for (int v = 0; v < D; ++v) {
-      rx[v] = okx ? *reinterpret_cast<const uint4*>(xp + (z + xr) * lda + v * EPG) : make_uint4(0, 0, 0, 0);
-      rg[v] = okg ? *reinterpret_cast<const uint4*>(gp + (z + gr) * ldg + v * EPG) : make_uint4(0, 0, 0, 0);
+      const int vi = (v * (32 / ZR) + line0) * 8 + l8;  // the vector's place in the row piece
+      rx[v] = (ok && vi < VRX) ? *reinterpret_cast<const uint4*>(xp + z * lda + v * (32 / ZR) * EPL) : make_uint4(0, 0, 0, 0);
+      rg[v] = (ok && vi < VRG) ? *reinterpret_cast<const uint4*>(gp + z * ldg + v * (32 / ZR) * EPL) : make_uint4(0, 0, 0, 0);
     }
   };
-  // element j * D + i of a run (channel j, component i) -> plane i, channel j, the thread's row
-  auto scatter = [&](const uint4 (&r)[D], char* dst, int PL, bool on) {
-    if (!on) return;
-    uint32_t w[4 * D];
+  auto scatter = [&](const uint4 (&r)[D], char* const (&slot)[D], int VR) {
 #pragma unroll
-    for (int v = 0; v < D; ++v) { w[4 * v] = r[v].x; w[4 * v + 1] = r[v].y; w[4 * v + 2] = r[v].z; w[4 * v + 3] = r[v].w; }
+    for (int v = 0; v < D; ++v) {
+      if ((v * (32 / ZR) + line0) * 8 + l8 >= VR) continue;
+      const uint32_t w[4] = {r[v].x, r[v].y, r[v].z, r[v].w};
 #pragma unroll
-    for (int j = 0; j < EPG; ++j)
-#pragma unroll
-      for (int i = 0; i < D; ++i) {
-        const int e = j * D + i;
-        if constexpr (ES == 2) *reinterpret_cast<uint16_t*>(dst + i * PL + j * kDwZS) = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
-        else *reinterpret_cast<uint32_t*>(dst + i * PL + j * kDwZS) = w[e];
+      for (int j = 0; j < EPV; ++j) {
+        const int sidx = 128 * v + j;
+        char* dst = slot[sidx % D] + 16 * (sidx / D);
+        if constexpr (ES == 2) *reinterpret_cast<uint16_t*>(dst) = static_cast<uint16_t>(w[j >> 1] >> (16 * (j & 1)));
+        else *reinterpret_cast<uint32_t*>(dst) = w[j];
       }
+    }
   };
 
   dw_floatx16 acc[2][2];
@@ -90,8 +104,8 @@ __device__ __forceinline__ void dw_body(const TI* __restrict__ A, int64_t lda, c
   if (z_begin < z_end) load_step(z_begin);
   for (int64_t z = z_begin; z < z_end; z += ZR) {
     __syncthreads();  // the previous step's reads are done
-    scatter(rx, xdst, PLX, xon);
-    scatter(rg, gdst, PLG, gon);
+    scatter(rx, xslot, VRX);
+    scatter(rg, gslot, VRG);
     __syncthreads();
     if (z + ZR < z_end) load_step(z + ZR);
 #pragma unroll
@@ -100,9 +114,9 @@ __device__ __forceinline__ void dw_body(const TI* __restrict__ A, int64_t lda, c
 #pragma unroll
       for (int a = 0; a < 2; ++a) {
         const int tu = wm * TU + a;
-        if (a < TU && tu < KT) fa[a] = *reinterpret_cast<const uint4*>(sx + i * PLX + (32 * tu + c) * kDwZS + 16 * h);
+        if (a < TU && tu < KT) fa[a] = *reinterpret_cast<const uint4*>(sx + i * PLX + h * (K * 16) + (32 * tu + c) * 16);
         const int tv = wn * TV + a;
-        if (a < TV && tv < NT) fb[a] = *reinterpret_cast<const uint4*>(sg + i * PLG + (32 * tv + c) * kDwZS + 16 * h);
+        if (a < TV && tv < NT) fb[a] = *reinterpret_cast<const uint4*>(sg + i * PLG + h * (N * 16) + (32 * tv + c) * 16);
       }
 #pragma unroll
       for (int a = 0; a < 2; ++a)
@@ -160,15 +174,16 @@ __global__ void __launch_bounds__(256) linear_dw_mul_ir_kernel(const TI* __restr
   }
 }
 
-// chunk counts per part, in proportion to D, about two blocks per compute unit in all; every chunk at least 64 rows
+// chunk counts per part, in proportion to D + 1 (measured: a step costs about as much again as one of its D components),
+// about two blocks per compute unit in all; every chunk at least 64 rows
 int64_t dw_plan(int64_t rows, const int64_t* table, int nparts, int32_t* first) {
   int64_t dsum = 0;
-  for (int p = 0; p < nparts; ++p) dsum += table[3 * p + 2];
+  for (int p = 0; p < nparts; ++p) dsum += table[3 * p + 2] + 1;
   const int64_t budget = static_cast<int64_t>(device_cus()) * 2;
   const int64_t most = (rows + 63) / 64 > 0 ? (rows + 63) / 64 : 1;
   int64_t total = 0;
   for (int p = 0; p < nparts; ++p) {
-    int64_t n = budget * table[3 * p + 2] / (dsum > 0 ? dsum : 1);
+    int64_t n = budget * (table[3 * p + 2] + 1) / (dsum > 0 ? dsum : 1);
     if (n > most) n = most;
     if (n < 1) n = 1;
     first[p] = static_cast<int32_t>(total);
@@ -219,7 +234,7 @@ extern "C" int cueq_linear_dw_mul_ir(int32_t dtype, int64_t K, int64_t N, int64_
     if (d > dmax) dmax = static_cast<int>(d);
   }
   const int64_t items = dw_plan(rows, table, nparts, parts.first);
-  const size_t lds = static_cast<size_t>(dmax) * (K + N) * kDwZS;
+  const size_t lds = static_cast<size_t>(dmax) * ((K + N) * 32 + 32);
   CUEQ_REQUIRE(lds <= 160 * 1024, CUEQ_ERR_TOO_LARGE, "linear_dw_mul_ir: the planes do not fit the local data share");
   KernelTimer timer("linear_dw_mul_ir", stream);
 #define DW(TI_)                                                                                                                               \

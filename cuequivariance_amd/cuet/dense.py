@@ -247,6 +247,116 @@ def _rows_tables(K: int, N: int, plist):
     return out
 
 
+class _MulIrPlan:
+    """Host tables of the 3-operand form on rows that keep the irrep component contiguous (``mul_ir``): every block
+    ``(mul, ir)`` of the input is one part ``(a0, c0, w_off, K, N, d)`` - ``K * d`` consecutive elements of an input row,
+    element (channel u, component i) at ``u * d + i``, ``N * d`` of an output row - served by ``cueq_linear_rows`` (d = 1: the
+    block is the same in both layouts), ``cueq_linear_rows_mul_ir`` (d = 3, 5, 7) and ``cueq_linear_dw_mul_ir``.  ``None`` from
+    ``build`` when the blocks are not of that shape."""
+
+    def __init__(self, blocks):
+        self.blocks = blocks
+        self._tables: dict = {}
+
+    @staticmethod
+    def build(mod: "SegmentedPolynomialDense"):
+        if mod.has_x2 or not mod.fwd_covers_output or not mod.dx1_covers_input:
+            return None
+        blocks = []
+        for p, count, da, dc in mod.fwd_groups:  # the components of a block: `count` paths at strides (K, N)
+            if count > 1 and (da != p.K or dc != p.N):
+                return None
+            if count not in (1, 3, 5, 7) or p.K % 32 or p.N % 32 or not (32 <= p.K <= 128 and 32 <= p.N <= 128):
+                return None
+            blocks.append((p.a_off, p.c_off, p.w_off, p.K, p.N, count, p.coeff))
+        if len({b[2] for b in blocks}) != len(blocks) or not any(b[5] > 1 for b in blocks):
+            return None  # (a weight block met twice is summed by the other path; nothing to gain without d > 1)
+        if any(v % 8 for b in blocks for v in b[:3]):
+            return None
+        return _MulIrPlan(blocks)
+
+    def accepts(self, dtype) -> bool:
+        if dtype not in (torch.float32, torch.bfloat16):
+            return False
+        us = 64 if dtype == torch.bfloat16 else 32  # channels per slice of the row-streaming launch
+        return all(d == 1 or (K % us == 0 and N % us == 0) for _, _, _, K, N, d, _ in self.blocks)
+
+    def tables(self, es: int):
+        """``(forward launches, input-gradient launches, weight-gradient launches)`` for elements of ``es`` bytes.
+        forward / input gradient: ``(d, rows of the result, contraction, table, parts, coefficient)``;
+        weight gradient: ``(K, N, coefficient, table, parts, [weight offset per part])``."""
+        hit = self._tables.get(es)
+        if hit is not None:
+            return hit
+        flat = lambda rows: (C.c_int64 * (3 * len(rows)))(*[v for r in rows for v in r])
+
+        def launches(key, row):
+            by = {}
+            for b in self.blocks:
+                by.setdefault(key(b), []).append(b)
+            out = []
+            for (d, n_res, k_con, coeff), bl in by.items():
+                if d == 1:
+                    room = 160 * 1024 - 8 * 32 * 144
+                else:
+                    room = 160 * 1024 - (8 if d * n_res <= 384 else 4) * 16 * (128 * d + 16)
+                cap = max(1, min(8, room // (n_res * (es * k_con + 16))))
+                for i in range(0, len(bl), cap):
+                    part = bl[i: i + cap]
+                    out.append((d, n_res, k_con, flat([row(b) for b in part]), len(part), coeff))
+            return out
+
+        fwd = launches(lambda b: (b[5], b[4], b[3], b[6]), lambda b: (b[0], b[2], b[1]))
+        dx = launches(lambda b: (b[5], b[3], b[4], b[6]), lambda b: (b[1], b[2], b[0]))
+        by = {}
+        for b in self.blocks:
+            by.setdefault((b[3], b[4], b[6]), []).append(b)
+        dw = []
+        for (K, N, coeff), bl in by.items():
+            for i in range(0, len(bl), 32):
+                part = bl[i: i + 32]
+                dw.append((K, N, coeff, flat([(b[0], b[1], b[5]) for b in part]), len(part), [b[2] for b in part]))
+        self._tables[es] = (fwd, dx, dw)
+        return self._tables[es]
+
+
+def _run_mul_ir(dtype, A, W, Cout, launches, forward: bool):
+    """Forward (``W`` blocks ``K x N`` as they lie) or input gradient (the same blocks read as ``N x K``) of the ``mul_ir``
+    parts: ``Cout[z, c0 + v d + i] = coeff * sum_u A[z, a0 + u d + i] W[u, v]``."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(A.device).cuda_stream
+    code = _DTYPE_CODE[dtype]
+    for d, n_res, k_con, table, nparts, coeff in launches:
+        if d == 1:
+            _lib.check(lib.cueq_linear_rows(code, 1 if forward else 0, A.shape[0], n_res, k_con, A.data_ptr(), A.stride(0), W.data_ptr(), W.numel(),
+                                            Cout.data_ptr(), Cout.stride(0), table, nparts, coeff, stream), "cueq_linear_rows")
+        else:
+            _lib.check(lib.cueq_linear_rows_mul_ir(code, 1 if forward else 0, A.shape[0], n_res, k_con, d, A.data_ptr(), A.stride(0), W.data_ptr(),
+                                                   W.numel(), Cout.data_ptr(), Cout.stride(0), table, nparts, coeff, stream),
+                       "cueq_linear_rows_mul_ir")
+
+
+def _weight_gradient_mul_ir(dtype, x, g, numel, launches):
+    """``dW`` (float32, flat) of the ``mul_ir`` parts: chunked partial products, then one ordered row sum per block."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    code = _DTYPE_CODE[dtype]
+    gw32 = torch.zeros(numel, dtype=torch.float32, device=x.device)
+    for K, N, coeff, table, nparts, w_offs in launches:
+        first = (C.c_int32 * (nparts + 1))()
+        items = lib.cueq_linear_dw_mul_ir_items(x.shape[0], table, nparts, first)
+        part = torch.empty(items, K * N, dtype=torch.float32, device=x.device)
+        _lib.check(lib.cueq_linear_dw_mul_ir(code, K, N, x.shape[0], x.data_ptr(), x.stride(0), g.data_ptr(), g.stride(0), table, nparts,
+                                             part.data_ptr(), coeff, stream), "cueq_linear_dw_mul_ir")
+        ws_bytes = max(lib.cueq_sum_rows_workspace(first[p + 1] - first[p], K * N) for p in range(nparts))
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+        for p, w_off in enumerate(w_offs):
+            rows = part[first[p]: first[p + 1]]
+            _lib.check(lib.cueq_sum_rows(_lib.F32, rows.shape[0], K * N, rows.data_ptr(), gw32[w_off: w_off + K * N].data_ptr(), ws.data_ptr(),
+                                         ws_bytes, stream), "cueq_sum_rows")
+    return gw32
+
+
 def _vector_rows(*tensors) -> bool:
     return all(t.data_ptr() % 16 == 0 and (t.dim() < 2 or (t.stride(0) * t.element_size()) % 16 == 0) for t in tensors)
 
@@ -308,7 +418,11 @@ class _DenseFunction(torch.autograd.Function):
         wd = w.detach().to(dtype).contiguous()
         x1d = x1.detach().contiguous()
         x2d = x2.detach().contiguous() if x2 is not None else None
-        if Z > 0:
+        if Z > 0 and mod.rows_mul_ir:
+            x1d, wd = _aligned(x1d), _aligned(wd)
+            with torch.cuda.device(x1.device):
+                _run_mul_ir(dtype, x1d, wd, out, mod.mul_ir.tables(x1d.element_size())[0], True)
+        elif Z > 0:
             with torch.cuda.device(x1.device):
                 merged = _merged_tables(mod, x1.device) if (mod.tiled(dtype, x1d, out) and _vector_rows(x1d, wd, out)) else None
                 if merged is not None:
@@ -362,7 +476,9 @@ class _DenseFunction(torch.autograd.Function):
             if needs_input_grad[2]:
                 # dx1[:, i_seg] += c * x2[:, j] * g[:, k_seg] @ W_p^T
                 gx1 = (torch.empty_like if mod.dx1_covers_input else torch.zeros_like)(x1d)
-                if Z > 0:
+                if Z > 0 and mod.rows_mul_ir:
+                    _run_mul_ir(dtype, _aligned(g), _aligned(wd), gx1, mod.mul_ir.tables(g.element_size())[1], False)
+                elif Z > 0:
                     merged = _merged_tables(mod, x1.device) if (mod.tiled(dtype, g, gx1) and _vector_rows(g, wd, gx1)) else None
                     if merged is not None:
                         _run_merged(dtype, g, wd, gx1, merged, False)
@@ -375,7 +491,9 @@ class _DenseFunction(torch.autograd.Function):
                         _run_gemms(dtype, g, wd, x2d, gx1, tables.dx1)
             if needs_input_grad[1]:
                 gwd = None
-                if Z > 0 and mod.tiled(dtype, x1d, g):
+                if Z > 0 and mod.rows_mul_ir:
+                    gwd = _weight_gradient_mul_ir(dtype, _aligned(x1d), _aligned(g), wd.numel(), mod.mul_ir.tables(x1d.element_size())[2]).view(wd.shape)
+                elif Z > 0 and mod.tiled(dtype, x1d, g):
                     # dW_p[k][n] += c * sum_z x1[z, i_seg + k] g[z, k_seg + n]: chunked partial products, ordered sum
                     # straight into a float32 image of the weights (a block met a second time is added)
                     code, es = _DTYPE_CODE[dtype], x1d.element_size()
@@ -1040,9 +1158,10 @@ class SegmentedPolynomialDense(nn.Module):
     """Dense (MFMA) executor for Linear / fully-connected polynomials with weights shared over the batch."""
 
     def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype=None, output_dtype_map: List[int] = None,
-                 name: str = "segmented_polynomial", method: str = "fused_tp"):
+                 name: str = "segmented_polynomial", method: str = "fused_tp", rows: str = "ir_mul"):
         super().__init__()
         self._polynomial_orig = polynomial
+        self._rows_orig = rows
         self._output_dtype_map_orig = output_dtype_map
         self.name = name
         self.method = method
@@ -1075,6 +1194,14 @@ class SegmentedPolynomialDense(nn.Module):
         self.fc_plan = _FcPlan(self.paths, self.input_sizes[2]) if self.has_x2 else None
         self._merged: dict = {}
         self._fused: dict = {}
+        # rows="mul_ir": the irreps operands (input 1 and the output of the 3-operand form) keep the component index
+        # contiguous inside every block; the kernels address them so - no transposition pass around the call.  Not part of
+        # the reference's interface.  `mul_ir` is None when the blocks do not have the shape those kernels take.
+        self.mul_ir = _MulIrPlan.build(self) if rows == "mul_ir" else None
+        if rows == "mul_ir" and self.mul_ir is None:
+            raise NotImplementedError("fused_tp: rows='mul_ir' needs a Linear-like polynomial with blocks of 1, 3, 5 or 7 components and "
+                                      "multiplicities 32, 64, 96 or 128")
+        self.rows_mul_ir = self.mul_ir is not None
         with _traced_lock:  # the integer under which a traced graph names this module
             self.traced_id = next(_traced_ids)
             _traced_modules[self.traced_id] = weakref.ref(self)
@@ -1119,7 +1246,8 @@ class SegmentedPolynomialDense(nn.Module):
     def __reduce__(self):
         from .segmented_polynomial import SegmentedPolynomial
 
-        return (SegmentedPolynomial, (self._polynomial_orig, self.method, self.math_dtype, self._output_dtype_map_orig, self.name))
+        return (SegmentedPolynomial, (self._polynomial_orig, self.method, self.math_dtype, self._output_dtype_map_orig, self.name,
+                                      {"rows": self._rows_orig} if self._rows_orig != "ir_mul" else None))
 
     def _indexed(self, w: torch.Tensor, x1: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
         """One weight row per class, rows of ``x1`` sorted by class (reference
@@ -1161,6 +1289,8 @@ class SegmentedPolynomialDense(nn.Module):
             raise NotImplementedError("fused_tp: weights must be shared over the batch (one row)")
         if x1.dtype not in _DTYPE_CODE:
             raise ValueError(f"fused_tp: unsupported dtype {x1.dtype}")
+        if self.rows_mul_ir and not self.mul_ir.accepts(x1.dtype):
+            raise NotImplementedError(f"fused_tp: rows='mul_ir' does not take {x1.dtype} with these multiplicities")
         if self.math_dtype == torch.float32 and x1.dtype == torch.float64:
             raise ValueError("Fused TP does not support float32 math_dtype with float64 inputs.")
         if x2 is not None:

@@ -77,9 +77,11 @@ def _permute_inputs(polynomial: cue.SegmentedPolynomial, perm) -> cue.SegmentedP
 
 class SegmentedPolynomialFusedTP(nn.Module):
     def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype=None, output_dtype_map: Optional[List[int]] = None,
-                 name: str = "segmented_polynomial"):
+                 name: str = "segmented_polynomial", rows: str = "ir_mul"):
         super().__init__()
         from .dense import SegmentedPolynomialDense
+
+        self._rows_orig = rows
 
         self._polynomial_orig = polynomial
         self._output_dtype_map_orig = output_dtype_map
@@ -112,11 +114,13 @@ class SegmentedPolynomialFusedTP(nn.Module):
 
             for perm in itertools.permutations(range(polynomial.num_inputs)):
                 try:
-                    self.dense = SegmentedPolynomialDense(_permute_inputs(polynomial, perm), math_dtype, output_dtype_map, name)
+                    self.dense = SegmentedPolynomialDense(_permute_inputs(polynomial, perm), math_dtype, output_dtype_map, name, rows=rows)
                     self.dense_perm = perm
                     break
                 except NotImplementedError:
                     continue
+        if rows == "mul_ir" and self.dense is None:
+            raise NotImplementedError("fused_tp: rows='mul_ir' is served by the matrix-core executor only")
         # one flattened executor per operation: (module, input buffers it reads, output it adds to)
         self.ops = nn.ModuleList()
         self.op_inputs, self.op_output = [], []
@@ -133,7 +137,8 @@ class SegmentedPolynomialFusedTP(nn.Module):
     def __reduce__(self):
         from .segmented_polynomial import SegmentedPolynomial
 
-        return (SegmentedPolynomial, (self._polynomial_orig, "fused_tp", self.math_dtype, self._output_dtype_map_orig, self.name))
+        return (SegmentedPolynomial, (self._polynomial_orig, "fused_tp", self.math_dtype, self._output_dtype_map_orig, self.name,
+                                      {"rows": self._rows_orig} if self._rows_orig != "ir_mul" else None))
 
     def forward(self, inputs: List[torch.Tensor], input_indices: Dict[int, torch.Tensor],
                 output_shapes: Dict[int, torch.Tensor], output_indices: Dict[int, torch.Tensor]):
@@ -150,6 +155,8 @@ class SegmentedPolynomialFusedTP(nn.Module):
                 and inputs[self.dense_perm[0]].shape[0] == 1 and inputs[0].dtype in (torch.float32, torch.float64, torch.bfloat16)
                 and all(t.dtype == inputs[0].dtype for t in inputs)):
             return self.dense([inputs[i] for i in self.dense_perm], input_indices, output_shapes, output_indices)
+        if self._rows_orig == "mul_ir":
+            raise NotImplementedError("fused_tp: rows='mul_ir' takes shared weights, no index tensors and one dtype for all inputs")
         device = inputs[0].device
         outs: List[Optional[torch.Tensor]] = [None] * self.num_outputs
         for f, ins, o in zip(self.ops, self.op_inputs, self.op_output):

@@ -464,6 +464,16 @@ class Linear(torch.nn.Module):
         self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
         # weights per sample, or per class with an index in any order (sorted classes: method="indexed_linear")
         self.f_per_sample = _FlattenedUniform(e.polynomial, math_dtype)
+        # mul_ir rows on both sides: the dense kernels address them as they lie (no transposition pass) whenever the blocks
+        # have a shape those kernels take; other shapes, dtypes and per-sample / indexed weights keep the passes
+        self.f_rows = None
+        if (self.method == "fused_tp" and self.transpose_in.source == cue.mul_ir and self.transpose_out.target == cue.mul_ir
+                and e.inputs[1].layout == cue.ir_mul and e.outputs[0].layout == cue.ir_mul
+                and (_transposition_moves(e.inputs[1].irreps) or _transposition_moves(e.outputs[0].irreps))):
+            try:
+                self.f_rows = SegmentedPolynomial(e.polynomial, method="fused_tp", math_dtype=math_dtype, options={"rows": "mul_ir"})
+            except NotImplementedError:
+                self.f_rows = None
 
     def extra_repr(self) -> str:
         return (
@@ -485,6 +495,9 @@ class Linear(torch.nn.Module):
             input_indices[0] = weight_indices
         if weight is None:
             raise ValueError("Weights should not be None")
+        if (self.f_rows is not None and not input_indices and weight.shape[0] == 1 and x.is_cuda and x.dtype == weight.dtype
+                and self.f_rows.m.dense.mul_ir.accepts(x.dtype)):
+            return self.f_rows([weight, x])[0]
         if self.method != "indexed_linear" and (input_indices or weight.shape[0] != 1):
             out = self.f_per_sample([weight, apply_layout(self.transpose_in, x)], input_indices)
         else:

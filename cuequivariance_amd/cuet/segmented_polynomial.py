@@ -227,7 +227,9 @@ class SegmentedPolynomial(nn.Module):
         elif method == "fused_tp":
             from .fused_tp import SegmentedPolynomialFusedTP
 
-            self.m = SegmentedPolynomialFusedTP(polynomial, math_dtype, output_dtype_map, name)
+            # option "rows": "mul_ir" - the irreps operands of a Linear-like polynomial keep the component index contiguous
+            # inside every block and the dense kernels address them so (not part of the reference's options)
+            self.m = SegmentedPolynomialFusedTP(polynomial, math_dtype, output_dtype_map, name, rows=self.options.get("rows", "ir_mul"))
         elif method == "naive":
             raise ValueError(
                 "method='naive' (the PyTorch executor) is not part of this engine: every method runs HIP kernels. "
