@@ -291,7 +291,7 @@ int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_major, int64_t 
  *   dW_p[u, v] = alpha * sum_{z < rows} sum_{i < D_p} A[z, a_p + u * D_p + i] * G[z, c_p + v * D_p + i]     (K x N, row-major)
  * table: HOST memory, nparts (<= 32) rows of (a_p, c_p, D_p), D_p in {1, 3, 5, 7}, offsets multiples of 16 bytes; K, N in
  * {32, 64, 96, 128}; bfloat16 or float32 inputs, float32 partial results.  Part p is cut into chunks of rows (counts in
- * proportion to D_p + 1); chunk c of part p writes its partial product to row first_item[p] + c of `partials` (K * N floats per
+ * proportion to 2 D_p + 1); chunk c of part p writes its partial product to row first_item[p] + c of `partials` (K * N floats per
  * row), and the caller adds the rows first_item[p] .. first_item[p + 1] - 1 in order (cueq_sum_rows): no atomics.
  * cueq_linear_dw_mul_ir_items returns the number of rows `partials` needs for this call shape on the current device and
  * fills first_item (nparts + 1 entries; may be NULL); -1 for a bad argument. */
