@@ -214,7 +214,7 @@ def load() -> C.CDLL:
         lib.cueq_gemm_table.restype = C.c_int
         lib.cueq_linear_rows.argtypes = [i32, i32, i64, i64, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i64, f64, ptr]
         lib.cueq_linear_rows.restype = C.c_int
-        lib.cueq_linear_rows_mul_ir.argtypes = [i32, i32, i64, i64, i64, i32, ptr, i64, ptr, i64, ptr, i64, ptr, i64, f64, ptr]
+        lib.cueq_linear_rows_mul_ir.argtypes = [i32, i32, i64, i64, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i64, f64, ptr]
         lib.cueq_linear_rows_mul_ir.restype = C.c_int
         lib.cueq_linear_dw_mul_ir_items.argtypes = [i64, ptr, i32, ptr]
         lib.cueq_linear_dw_mul_ir_items.restype = i64

@@ -16,7 +16,11 @@
 //  * the products are 16 x 16 (weight columns x rows), so that the accumulators of all D components of a unit stay in
 //    registers: 4 * D * N / 16 per lane - a lane ends up with 4 channels x D components of its row, which are 4 * D
 //    contiguous elements of the result row and leave through the staging tile as whole lines.
-// D is 3, 5 or 7 (a block of one component is the same in both layouts and takes linear_rows.hip).
+// The parts of one launch may have different numbers of components D (1, 3, 5 or 7 - the irreps of one Linear).  The blocks of
+// the launch are dealt out to the values of D in proportion to the bytes their parts move, and every block walks all rows for
+// the parts of its D: the groups advance through the rows at the same pace, so what the chip reads and writes at one time are
+// whole rows.  That matters to the memory system: launches that touch only a column range of every row measured 5.0 TB/s where
+// whole rows reach 5.7.
 
 #include "common.h"
 #include "cw_common.h"
@@ -29,7 +33,12 @@ namespace {
 
 typedef float mi_floatx4 __attribute__((ext_vector_type(4)));
 
-template <typename TI, int D, int NT16>
+// WAVES: wavefronts per block, the same for all blocks of a launch (8 while the accumulators of its largest D leave room for
+// two wavefronts per SIMD, else 4).
+template <int DMAX, int NT16>
+struct MiLaunch { static constexpr int WAVES = 4 * DMAX * NT16 <= 96 ? 8 : 4; };
+
+template <typename TI, int D, int NT16, int WAVES_>
 struct MiShape {
   static constexpr int ES = sizeof(TI);
   static constexpr int US = 128 / ES;        // channels per slice
@@ -37,9 +46,11 @@ struct MiShape {
   static constexpr int RS = 128 * D + 16;    // bytes between the rows of the staging tile
   static constexpr int STAGE = 16 * RS;      // per wavefront
   static constexpr int ACC = 4 * D * NT16;   // accumulator registers per lane
-  static constexpr int WAVES = ACC <= 96 ? 8 : 4;  // two wavefronts per SIMD while the registers allow it
+  static constexpr int WAVES = WAVES_;
   static constexpr int TPP = 8 / ES;         // 16-column tiles of the result per pass through the staging tile
-  static constexpr int PF = 2;               // slices requested ahead (register sets of 8 D; a third set spills)
+  // slices requested ahead (register sets of 8 D registers): two where the registers are tight, more for the small D of a launch
+  // whose blocks run four wavefronts - about the same number of bytes in flight per wavefront either way
+  static constexpr int PF = WAVES == 8 ? (D == 1 ? 4 : 2) : (D == 1 ? 8 : D == 3 ? 3 : D == 5 ? 2 : 1);
 };
 
 // one dword made of two 2-byte halves: the low half from half `lh` of `lo`, the high half from half `hh` of `hi`
@@ -73,7 +84,7 @@ __device__ __forceinline__ void mi_request(uint4 (&xs)[2 * D], const char* base,
 // The state a wavefront keeps while it walks its units.
 template <typename TI, int D, int NT16>
 struct MiWork {
-  using S = MiShape<TI, D, NT16>;
+  using S = MiShape<TI, D, NT16, 8>;  // (what it reads does not depend on the number of wavefronts)
   mi_floatx4 acc[D][NT16];
 
   __device__ __forceinline__ void clear() {
@@ -210,25 +221,39 @@ struct MiWork {
   }
 };
 
-template <typename TI, int D, int NT16>
-__global__ void __launch_bounds__((64 * MiShape<TI, D, NT16>::WAVES), 1)
-    linear_rows_mul_ir_kernel(const TI* __restrict__ A, int64_t lda, const TI* __restrict__ W, LrParts parts, int nslots, int nparts,
-                              int w_contraction_major, TI* __restrict__ C, int64_t ldc, int M, int K, float alpha) {
-  using S = MiShape<TI, D, NT16>;
+struct MiParts {
+  int32_t a_off[kLrMaxParts], c_off[kLrMaxParts];
+  int8_t slot[kLrMaxParts];  // the part's weight block, counted within its group
+  int64_t w_off[kLrMaxSlots];
+  // group g holds the parts of D = 2 g + 1: parts [part_first[g], part_first[g + 1]), weight blocks [slot_first[g], ...),
+  // blocks of the launch [block_first[g], ...)
+  int16_t part_first[5], slot_first[5], block_first[5];
+};
+
+// The work of one block for the parts of one D: block `bid` of `nblocks`, parts `first_part ...` (nparts of them), weight
+// blocks `first_slot ...` (nslots of them).
+template <typename TI, int D, int NT16, int WAVES_>
+__device__ __forceinline__ void mi_run(const TI* __restrict__ A, int64_t lda, const TI* __restrict__ W, const MiParts& parts, int first_part,
+                                       int nparts, int first_slot, int nslots, int bid, int nblocks, int w_contraction_major,
+                                       TI* __restrict__ C, int64_t ldc, int M, int K, float alpha, char* smem) {
+  using S = MiShape<TI, D, NT16, WAVES_>;
   constexpr int ES = S::ES, US = S::US, NV = S::NV, WAVES = S::WAVES, N = 16 * NT16, PF = S::PF;
-  extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, h = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int WRS = K * ES + 16;  // bytes between weight rows (one row per result column) in LDS
   const int NS = K / US;        // slices per unit
 
-  lr_stage_weights<TI, 64 * WAVES>(W, parts, nslots, K, N, WRS, w_contraction_major, smem, tid);
+  {
+    LrParts wparts;  // (the weight staging reads the block offsets only)
+    for (int s = 0; s < nslots; ++s) wparts.w_off[s] = parts.w_off[first_slot + s];
+    lr_stage_weights<TI, 64 * WAVES>(W, wparts, nslots, K, N, WRS, w_contraction_major, smem, tid);
+  }
   __syncthreads();
 
   char* stage = smem + nslots * (N * WRS) + wave * S::STAGE;
   const char* wlane = smem + c * WRS + h * 32;  // the lane's channels of a slice start 32 h bytes into it (16 h or 8 h elements)
   const int nfull = M / 16;
-  const int wslot = wave * gridDim.x + blockIdx.x, nw = gridDim.x * WAVES;  // wavefront-major, as in linear_rows.hip
+  const int wslot = wave * nblocks + bid, nw = nblocks * WAVES;  // wavefront-major, as in linear_rows.hip
   const int step_t = nw / nparts, step_p = nw % nparts;
   const int row_bytes = static_cast<int>(lda * ES);
   const int64_t total_full = static_cast<int64_t>(nfull) * nparts;
@@ -251,7 +276,7 @@ __global__ void __launch_bounds__((64 * MiShape<TI, D, NT16>::WAVES), 1)
     };
     auto source = [&]() {
       const int tt = rt < nfull ? rt : nfull - 1;  // past the end: a tile that exists (the values are not used)
-      return reinterpret_cast<const char*>(A + static_cast<int64_t>(tt) * 16 * lda + parts.part[rp].a_off) + rs * (128 * D);
+      return reinterpret_cast<const char*>(A + static_cast<int64_t>(tt) * 16 * lda + parts.a_off[first_part + rp]) + rs * (128 * D);
     };
     // PF register sets in rotation: the slice PF steps ahead is requested as soon as the current one sits in the staging
     // tile.  The loop body is PF steps without a branch around them; the steps left over follow it.
@@ -264,11 +289,11 @@ __global__ void __launch_bounds__((64 * MiShape<TI, D, NT16>::WAVES), 1)
 #define MI_STEP(XS)                                                                                                                     \
     {                                                                                                                                    \
       const char* src = source();                                                                                                        \
-      work.slice(XS, wlane + parts.part[p].slot * (N * WRS) + s * 128, WRS, stage, lane,                                                 \
+      work.slice(XS, wlane + parts.slot[first_part + p] * (N * WRS) + s * 128, WRS, stage, lane,                                                 \
                  [&]() { mi_request<D, true>(XS, src, row_bytes, 15, lane); __builtin_amdgcn_sched_barrier(0); });                       \
       advance(rt, rp, rs);                                                                                                               \
       if (s == NS - 1) {                                                                                                                 \
-        work.template store<true>(stage, C + static_cast<int64_t>(t) * 16 * ldc + parts.part[p].c_off, ldc, 16, alpha, lane);            \
+        work.template store<true>(stage, C + static_cast<int64_t>(t) * 16 * ldc + parts.c_off[first_part + p], ldc, 16, alpha, lane);            \
         work.clear();                                                                                                                    \
       }                                                                                                                                  \
       advance(t, p, s);                                                                                                                  \
@@ -288,28 +313,46 @@ __global__ void __launch_bounds__((64 * MiShape<TI, D, NT16>::WAVES), 1)
       work.clear();
       for (int s = 0; s < NS; ++s) {
         uint4 xs[NV];
-        mi_request<D, false>(xs, reinterpret_cast<const char*>(A + static_cast<int64_t>(nfull) * 16 * lda + parts.part[p].a_off) + s * (128 * D), row_bytes,
+        mi_request<D, false>(xs, reinterpret_cast<const char*>(A + static_cast<int64_t>(nfull) * 16 * lda + parts.a_off[first_part + p]) + s * (128 * D), row_bytes,
                       rows - 1, lane);
-        work.slice(xs, wlane + parts.part[p].slot * (N * WRS) + s * 128, WRS, stage, lane, []() {});
+        work.slice(xs, wlane + parts.slot[first_part + p] * (N * WRS) + s * 128, WRS, stage, lane, []() {});
       }
-      work.template store<false>(stage, C + static_cast<int64_t>(nfull) * 16 * ldc + parts.part[p].c_off, ldc, rows, alpha, lane);
+      work.template store<false>(stage, C + static_cast<int64_t>(nfull) * 16 * ldc + parts.c_off[first_part + p], ldc, rows, alpha, lane);
     }
   }
+}
+
+
+// DMAX: the largest D of the launch (it sets the wavefronts per block and the registers of the kernel).
+template <typename TI, int DMAX, int NT16>
+__global__ void __launch_bounds__((64 * MiLaunch<DMAX, NT16>::WAVES), 1)
+    linear_rows_mul_ir_kernel(const TI* __restrict__ A, int64_t lda, const TI* __restrict__ W, MiParts parts, int w_contraction_major,
+                              TI* __restrict__ C, int64_t ldc, int M, int K, float alpha) {
+  constexpr int WAVES = MiLaunch<DMAX, NT16>::WAVES;
+  extern __shared__ __align__(16) char smem[];
+  const int b = blockIdx.x;
+  int g = 0;
+  while (g < 3 && b >= parts.block_first[g + 1]) ++g;
+  const int bid = b - parts.block_first[g], nblocks = parts.block_first[g + 1] - parts.block_first[g];
+  const int fp = parts.part_first[g], np = parts.part_first[g + 1] - fp, fs = parts.slot_first[g], ns = parts.slot_first[g + 1] - fs;
+  if (g == 0) mi_run<TI, 1, NT16, WAVES>(A, lda, W, parts, fp, np, fs, ns, bid, nblocks, w_contraction_major, C, ldc, M, K, alpha, smem);
+  if constexpr (DMAX >= 3) { if (g == 1) mi_run<TI, 3, NT16, WAVES>(A, lda, W, parts, fp, np, fs, ns, bid, nblocks, w_contraction_major, C, ldc, M, K, alpha, smem); }
+  if constexpr (DMAX >= 5) { if (g == 2) mi_run<TI, 5, NT16, WAVES>(A, lda, W, parts, fp, np, fs, ns, bid, nblocks, w_contraction_major, C, ldc, M, K, alpha, smem); }
+  if constexpr (DMAX >= 7) { if (g == 3) mi_run<TI, 7, NT16, WAVES>(A, lda, W, parts, fp, np, fs, ns, bid, nblocks, w_contraction_major, C, ldc, M, K, alpha, smem); }
 }
 
 }  // namespace
 
 }  // namespace cueq
 
-// table: host memory, nparts rows of (a_off, w_off, c_off) in elements; a part reads K * D and writes N * D elements per row
-extern "C" int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, int32_t D, const void* A,
-                                       int64_t lda, const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts,
-                                       double alpha, void* stream_) {
+// table: host memory, nparts rows of (a_off, w_off, c_off, D) in elements; a part reads K * D and writes N * D elements per row
+extern "C" int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                                       const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts, double alpha,
+                                       void* stream_) {
   using namespace cueq;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "linear_rows_mul_ir: bfloat16 or float32");
   CUEQ_REQUIRE(M >= 0 && N > 0 && K > 0 && nparts >= 0, CUEQ_ERR_INVALID, "linear_rows_mul_ir: bad extents");
-  CUEQ_REQUIRE(D == 3 || D == 5 || D == 7, CUEQ_ERR_UNSUPPORTED, "linear_rows_mul_ir: blocks of 3, 5 or 7 components");
   const int es = dtype == CUEQ_F32 ? 4 : 2, epv = 16 / es, us = 128 / es;
   CUEQ_REQUIRE(N % 32 == 0 && N <= 128 && K % us == 0 && K <= 128, CUEQ_ERR_UNSUPPORTED,
                "linear_rows_mul_ir: N must be 32, 64, 96 or 128 and K a multiple of %d up to 128", us);
@@ -321,41 +364,73 @@ extern "C" int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_majo
   CUEQ_REQUIRE(lda % epv == 0 && ldc % epv == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(C) % 16 == 0,
                CUEQ_ERR_UNSUPPORTED, "linear_rows_mul_ir: row strides and pointers must be multiples of 16 bytes");
-  LrParts parts;
-  int nslots = 0;
   for (int64_t p = 0; p < nparts; ++p) {
-    const int64_t a_off = table[3 * p], w_off = table[3 * p + 1], c_off = table[3 * p + 2];
-    CUEQ_REQUIRE(a_off >= 0 && a_off + K * D <= lda && c_off >= 0 && c_off + N * D <= ldc && w_off >= 0 && w_off + K * N <= w_numel &&
+    const int64_t a_off = table[4 * p], w_off = table[4 * p + 1], c_off = table[4 * p + 2], d = table[4 * p + 3];
+    CUEQ_REQUIRE(d == 1 || d == 3 || d == 5 || d == 7, CUEQ_ERR_UNSUPPORTED, "linear_rows_mul_ir: blocks of 1, 3, 5 or 7 components");
+    CUEQ_REQUIRE(a_off >= 0 && a_off + K * d <= lda && c_off >= 0 && c_off + N * d <= ldc && w_off >= 0 && w_off + K * N <= w_numel &&
                      a_off % epv == 0 && c_off % epv == 0 && w_off % epv == 0,
                  CUEQ_ERR_INVALID, "linear_rows_mul_ir: part %lld: offsets must lie inside a row / the weights and be multiples of 16 bytes",
                  static_cast<long long>(p));
-    int s = 0;
-    while (s < nslots && parts.w_off[s] != w_off) ++s;
-    if (s == nslots) {
-      CUEQ_REQUIRE(nslots < kLrMaxSlots, CUEQ_ERR_TOO_LARGE, "linear_rows_mul_ir: at most %d distinct weight blocks per launch", kLrMaxSlots);
-      parts.w_off[nslots++] = w_off;
-    }
-    parts.part[p] = LrPart{static_cast<int32_t>(a_off), static_cast<int32_t>(c_off), s};
   }
-  const int waves = 4 * D * (N / 16) <= 96 ? 8 : 4;
-  const size_t lds = static_cast<size_t>(nslots) * N * (es * K + 16) + static_cast<size_t>(waves) * 16 * (128 * D + 16);
+  // the parts grouped by D (group g: D = 2 g + 1), each group with its own list of weight blocks
+  MiParts parts;
+  int np = 0, nslots = 0, dmax = 1, max_slots = 0;
+  int64_t weight[4] = {0, 0, 0, 0};
+  for (int g = 0; g < 4; ++g) {
+    parts.part_first[g] = static_cast<int16_t>(np);
+    parts.slot_first[g] = static_cast<int16_t>(nslots);
+    for (int64_t p = 0; p < nparts; ++p) {
+      if (table[4 * p + 3] != 2 * g + 1) continue;
+      const int64_t w_off = table[4 * p + 1];
+      int s = parts.slot_first[g];
+      while (s < nslots && parts.w_off[s] != w_off) ++s;
+      if (s == nslots) {
+        CUEQ_REQUIRE(nslots < kLrMaxSlots, CUEQ_ERR_TOO_LARGE, "linear_rows_mul_ir: at most %d distinct weight blocks per launch", kLrMaxSlots);
+        parts.w_off[nslots++] = w_off;
+      }
+      parts.a_off[np] = static_cast<int32_t>(table[4 * p]);
+      parts.c_off[np] = static_cast<int32_t>(table[4 * p + 2]);
+      parts.slot[np] = static_cast<int8_t>(s - parts.slot_first[g]);
+      ++np;
+      weight[g] += 2 * g + 1;
+      dmax = 2 * g + 1;
+    }
+    if (nslots - parts.slot_first[g] > max_slots) max_slots = nslots - parts.slot_first[g];
+  }
+  parts.part_first[4] = static_cast<int16_t>(np);
+  parts.slot_first[4] = static_cast<int16_t>(nslots);
+  if (dmax == 1) dmax = 3;  // (parts of one component alone: cueq_linear_rows is the better launch, this one still serves them)
+  const int waves = 4 * dmax * (N / 16) <= 96 ? 8 : 4;
+  const size_t lds = static_cast<size_t>(max_slots) * N * (es * K + 16) + static_cast<size_t>(waves) * 16 * (128 * dmax + 16);
   CUEQ_REQUIRE(lds <= 160 * 1024, CUEQ_ERR_TOO_LARGE, "linear_rows_mul_ir: the weight blocks of one launch do not fit the local data share");
-  const int64_t total = ((M + 15) / 16) * nparts;
-  int64_t gx = (total + waves - 1) / waves;
-  if (gx > device_cus()) gx = device_cus();
+  // blocks per group in proportion to the bytes its parts move (sum of D), every group with parts at least one, none more
+  // than it has units for its wavefronts
+  const int64_t tiles = (M + 15) / 16;
+  int64_t budget = device_cus(), wsum = weight[0] + weight[1] + weight[2] + weight[3];
+  int64_t nb[4], total_blocks = 0;
+  for (int g = 0; g < 4; ++g) {
+    const int64_t gp = parts.part_first[g + 1] - parts.part_first[g];
+    nb[g] = gp == 0 ? 0 : (budget * weight[g] + wsum / 2) / wsum;
+    const int64_t most = (tiles * gp + waves - 1) / waves;
+    if (gp > 0 && nb[g] < 1) nb[g] = 1;
+    if (nb[g] > most) nb[g] = most;
+    parts.block_first[g] = static_cast<int16_t>(total_blocks);
+    total_blocks += nb[g];
+  }
+  parts.block_first[4] = static_cast<int16_t>(total_blocks);
   KernelTimer timer("linear_rows_mul_ir", stream);
 #define MI(TI_, D_, NT_)                                                                                                                      \
   do {                                                                                                                                        \
     auto kfn = linear_rows_mul_ir_kernel<TI_, D_, NT_>;                                                                                       \
     CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(64 * MiShape<TI_, D_, NT_>::WAVES), lds, stream, static_cast<const TI_*>(A), lda, \
-                       static_cast<const TI_*>(W), parts, nslots, static_cast<int>(nparts), w_contraction_major, static_cast<TI_*>(C), ldc,   \
-                       static_cast<int>(M), static_cast<int>(K), static_cast<float>(alpha));                                                  \
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(total_blocks)), dim3(64 * MiLaunch<D_, NT_>::WAVES), lds, stream, static_cast<const TI_*>(A), \
+                       lda, static_cast<const TI_*>(W), parts, w_contraction_major, static_cast<TI_*>(C), ldc, static_cast<int>(M),           \
+                       static_cast<int>(K), static_cast<float>(alpha));                                                                       \
   } while (0)
 #define MI_N(TI_, D_)                                                                                                                          \
   switch (N / 32) { case 1: MI(TI_, D_, 2); break; case 2: MI(TI_, D_, 4); break; case 3: MI(TI_, D_, 6); break; default: MI(TI_, D_, 8); break; }
 #define MI_D(TI_)                 \
-  switch (D) {                    \
+  switch (dmax) {                 \
     case 3: MI_N(TI_, 3); break;  \
     case 5: MI_N(TI_, 5); break;  \
     default: MI_N(TI_, 7); break; \

@@ -283,31 +283,48 @@ class _MulIrPlan:
 
     def tables(self, es: int):
         """``(forward launches, input-gradient launches, weight-gradient launches)`` for elements of ``es`` bytes.
-        forward / input gradient: ``(d, rows of the result, contraction, table, parts, coefficient)``;
+        forward / input gradient: ``(d, columns of the result block, contraction, table of (a, w, c[, d]), parts, coefficient)``;
         weight gradient: ``(K, N, coefficient, table, parts, [weight offset per part])``."""
         hit = self._tables.get(es)
         if hit is not None:
             return hit
-        flat = lambda rows: (C.c_int64 * (3 * len(rows)))(*[v for r in rows for v in r])
+        flat = lambda rows: (C.c_int64 * (len(rows[0]) * len(rows)))(*[v for r in rows for v in r])
+
+        def fits(part, n_res, k_con):
+            """What ``cueq_linear_rows_mul_ir`` checks: the weight blocks of the largest group of equal d and the staging
+            tiles of the wavefronts within 160 KiB, at most 8 distinct blocks and 48 parts."""
+            dmax = max(3, max(b[5] for b in part))
+            waves = 8 if dmax * n_res <= 384 else 4
+            slots = max(sum(1 for b in part if b[5] == d) for d in {b[5] for b in part})
+            return (len(part) <= 8 and slots * n_res * (es * k_con + 16) + waves * 16 * (128 * dmax + 16) <= 160 * 1024)
 
         def launches(key, row):
+            # One launch per number of components: the kernels are bound by what one compute unit keeps in flight, not
+            # by the memory system, so the blocks of different d gain nothing from sharing a launch (measured: the three
+            # blocks of 128x0e+128x1o+128x2e in one launch 265 us, in three 200 us) - and blocks of one component are the
+            # same in both layouts and take the launch with 32-row units.
             by = {}
             for b in self.blocks:
-                by.setdefault(key(b), []).append(b)
+                by.setdefault((b[5],) + key(b), []).append(b)
             out = []
             for (d, n_res, k_con, coeff), bl in by.items():
                 if d == 1:
-                    room = 160 * 1024 - 8 * 32 * 144
-                else:
-                    room = 160 * 1024 - (8 if d * n_res <= 384 else 4) * 16 * (128 * d + 16)
-                cap = max(1, min(8, room // (n_res * (es * k_con + 16))))
-                for i in range(0, len(bl), cap):
-                    part = bl[i: i + cap]
-                    out.append((d, n_res, k_con, flat([row(b) for b in part]), len(part), coeff))
+                    cap = max(1, min(8, (160 * 1024 - 8 * 32 * 144) // (n_res * (es * k_con + 16))))
+                    for i in range(0, len(bl), cap):
+                        part = bl[i: i + cap]
+                        out.append((1, n_res, k_con, flat([row(q)[:3] for q in part]), len(part), coeff))
+                    continue
+                cur = []
+                for b in bl:
+                    if cur and not fits(cur + [b], n_res, k_con):
+                        out.append((d, n_res, k_con, flat([row(q) for q in cur]), len(cur), coeff))
+                        cur = []
+                    cur.append(b)
+                out.append((d, n_res, k_con, flat([row(q) for q in cur]), len(cur), coeff))
             return out
 
-        fwd = launches(lambda b: (b[5], b[4], b[3], b[6]), lambda b: (b[0], b[2], b[1]))
-        dx = launches(lambda b: (b[5], b[3], b[4], b[6]), lambda b: (b[1], b[2], b[0]))
+        fwd = launches(lambda b: (b[4], b[3], b[6]), lambda b: (b[0], b[2], b[1], b[5]))
+        dx = launches(lambda b: (b[3], b[4], b[6]), lambda b: (b[1], b[2], b[0], b[5]))
         by = {}
         for b in self.blocks:
             by.setdefault((b[3], b[4], b[6]), []).append(b)
@@ -331,7 +348,7 @@ def _run_mul_ir(dtype, A, W, Cout, launches, forward: bool):
             _lib.check(lib.cueq_linear_rows(code, 1 if forward else 0, A.shape[0], n_res, k_con, A.data_ptr(), A.stride(0), W.data_ptr(), W.numel(),
                                             Cout.data_ptr(), Cout.stride(0), table, nparts, coeff, stream), "cueq_linear_rows")
         else:
-            _lib.check(lib.cueq_linear_rows_mul_ir(code, 1 if forward else 0, A.shape[0], n_res, k_con, d, A.data_ptr(), A.stride(0), W.data_ptr(),
+            _lib.check(lib.cueq_linear_rows_mul_ir(code, 1 if forward else 0, A.shape[0], n_res, k_con, A.data_ptr(), A.stride(0), W.data_ptr(),
                                                    W.numel(), Cout.data_ptr(), Cout.stride(0), table, nparts, coeff, stream),
                        "cueq_linear_rows_mul_ir")
 

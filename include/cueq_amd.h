@@ -277,14 +277,15 @@ int cueq_linear_rows(int32_t dtype, int32_t w_contraction_major, int64_t M, int6
  * of D components at u * D + i).  The reference converts such rows to channel-contiguous ones in front of its dense
  * kernels and back behind them (cuequivariance_torch/primitives/transpose.py:83-183, called from
  * operations/linear.py:153-191); this entry point reads and writes them as they lie:
- *   C[z, c_p + v * D + i] = alpha * sum_u A[z, a_p + u * D + i] * W_p[u, v]     for i < D, all rows z < M and parts p.
- * A part reads K * D and writes N * D consecutive elements of a row.  D in {3, 5, 7} (a block of one component is the
- * same in both layouts: cueq_linear_rows); N in {32, 64, 96, 128}; K a multiple of 64 (bfloat16) or 32 (float32) up to
- * 128; other limits and the table as for cueq_linear_rows, with (blocks * N * (K * element size + 16) +
- * waves * 16 * (128 * D + 16)) bytes <= 160 KiB, waves = 8 if D * N <= 384 else 4. */
-int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, int32_t D, const void* A,
-                            int64_t lda, const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts,
-                            double alpha, void* stream);
+ *   C[z, c_p + v * D_p + i] = alpha * sum_u A[z, a_p + u * D_p + i] * W_p[u, v]     for i < D_p, all rows z < M and parts p.
+ * table: HOST memory, nparts rows of (a_p, w_p, c_p, D_p); part p reads K * D_p and writes N * D_p consecutive elements of a
+ * row; D_p in {1, 3, 5, 7}, mixed freely in one launch (all blocks of a row in one launch is also what the memory system
+ * likes best).  N in {32, 64, 96, 128}; K a multiple of 64 (bfloat16) or 32 (float32) up to 128; other limits as for
+ * cueq_linear_rows, with (blocks * N * (K * element size + 16) + waves * 16 * (128 * Dmax + 16)) bytes <= 160 KiB,
+ * Dmax = max(3, largest D_p), waves = 8 if Dmax * N <= 384 else 4. */
+int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_major, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                            const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts, double alpha,
+                            void* stream);
 
 /* Weight gradient of the same operation on `mul_ir` rows (the reference reaches it through autograd of its dense kernel
  * after the transposition of cuequivariance_torch/primitives/transpose.py:83-183):

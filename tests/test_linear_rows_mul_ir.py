@@ -17,30 +17,32 @@ BF16, F32, F64 = 3, 0, 1
 
 
 def _table(rows):
-    return (C.c_int64 * (3 * len(rows)))(*[v for r in rows for v in r])
+    return (C.c_int64 * (len(rows[0]) * len(rows)))(*[v for r in rows for v in r])
 
 
 def test_argument_checks_without_a_device():
     lib = _lib.load()
     buf = (C.c_char * 4096)()
     ptr = C.addressof(buf) + (-C.addressof(buf)) % 16
-    one = _table([(0, 0, 0)])
-    call = lambda dtype, M, N, K, D, lda, ldc, table, nparts: lib.cueq_linear_rows_mul_ir(
-        dtype, 1, M, N, K, D, ptr, lda, ptr, 9 * 128 * 128, ptr, ldc, table, nparts, 1.0, None)
-    assert call(F64, 64, 128, 128, 3, 384, 384, one, 1) == -2  # float64: not built
-    assert call(BF16, 64, 128, 128, 1, 128, 128, one, 1) == -2  # one component: the other entry point
-    assert call(BF16, 64, 128, 128, 4, 512, 512, one, 1) == -2  # 4 components: not built
-    assert call(BF16, 64, 48, 128, 3, 384, 384, one, 1) == -2  # extent not a multiple of 32
-    assert call(BF16, 64, 128, 96, 3, 384, 384, one, 1) == -2  # bfloat16 contraction not a multiple of 64
-    assert call(BF16, 64, 128, 128, 3, 380, 384, one, 1) == -2  # row stride not a multiple of 16 bytes
-    assert call(BF16, 64, 128, 128, 3, 384, 384, _table([(8, 0, 0)]), 1) == -1  # part runs past the row
-    assert call(BF16, 64, 128, 128, 3, 384, 384, one, 49) == -4  # too many parts
-    assert call(BF16, 0, 128, 128, 3, 384, 384, one, 1) == 0  # nothing to do
+    call = lambda dtype, M, N, K, lda, ldc, rows, nparts=None: lib.cueq_linear_rows_mul_ir(
+        dtype, 1, M, N, K, ptr, lda, ptr, 9 * 128 * 128, ptr, ldc, _table(rows), len(rows) if nparts is None else nparts, 1.0, None)
+    one = [(0, 0, 0, 3)]
+    assert call(F64, 64, 128, 128, 384, 384, one) == -2  # float64: not built
+    assert call(BF16, 64, 128, 128, 512, 512, [(0, 0, 0, 4)]) == -2  # 4 components: not built
+    assert call(BF16, 64, 48, 128, 384, 384, one) == -2  # extent not a multiple of 32
+    assert call(BF16, 64, 128, 96, 384, 384, one) == -2  # bfloat16 contraction not a multiple of 64
+    assert call(BF16, 64, 128, 128, 380, 384, one) == -2  # row stride not a multiple of 16 bytes
+    assert call(BF16, 64, 128, 128, 384, 384, [(8, 0, 0, 3)]) == -1  # part runs past the row
+    assert call(BF16, 64, 128, 128, 384, 384, one * 49) == -4  # too many parts
+    five = [(0, 128 * 128 * s, 0, 3) for s in range(5)]
+    assert call(BF16, 64, 128, 128, 384, 384, five) == -4  # five blocks of one D: 5 x 34 KB + staging exceed 160 KB
+    assert b"local data share" in lib.cueq_last_error()
+    assert call(BF16, 0, 128, 128, 384, 384, one) == 0  # nothing to do
 
 
-def _reference(A, W, parts, K, N, D, contraction_major, alpha, ldc):
+def _reference(A, W, parts, K, N, contraction_major, alpha, ldc):
     out = torch.zeros(A.shape[0], ldc, dtype=torch.float64, device=A.device)
-    for a_off, w_off, c_off in parts:
+    for a_off, w_off, c_off, D in parts:
         blk = W[w_off: w_off + K * N].double()
         blk = blk.view(K, N) if contraction_major else blk.view(N, K).t()
         x = A[:, a_off: a_off + K * D].double().view(-1, K, D)
@@ -52,45 +54,48 @@ def _reference(A, W, parts, K, N, D, contraction_major, alpha, ldc):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("contraction_major", [1, 0])
 @pytest.mark.parametrize(
-    "M,K,N,D,nblocks,nparts",
+    "M,K,N,dims",
     [
-        (1000, 128, 128, 3, 2, 3),
-        (1000, 128, 128, 5, 1, 2),
-        (15, 128, 128, 7, 1, 1),
-        (4097, 64, 96, 3, 2, 3),
-        (333, 64, 32, 5, 3, 7),
-        (65, 128, 64, 7, 2, 4),
-        (20_000, 128, 32, 3, 2, 6),
-        (1, 64, 128, 5, 1, 2),
-        (200, 64, 64, 3, 2, 40),  # more parts than a block has wavefronts
-        (48, 128, 128, 3, 2, 48),  # the most parts a launch takes
-        (77, 32, 64, 3, 1, 2),  # (float32 only: a bfloat16 slice is 64 channels)
-        (130, 96, 96, 5, 1, 2),  # (float32 only)
+        (1000, 128, 128, [1, 3, 5]),  # the irreps of the benchmark's Linear
+        (1000, 128, 128, [5, 5]),  # two parts of one D sharing a weight block
+        (15, 128, 128, [7]),
+        (4097, 64, 96, [3, 1, 3]),
+        (333, 64, 32, [5, 3, 1, 7, 5, 3, 1]),
+        (65, 128, 64, [7, 7, 1, 1]),
+        (20_000, 128, 32, [3, 3, 3, 1, 1, 5]),
+        (1, 64, 128, [5, 1]),
+        (200, 64, 64, [3] * 20 + [1] * 20),  # more parts than a block has wavefronts
+        (48, 128, 128, [3] * 24 + [1] * 24),  # the most parts a launch takes
+        (77, 32, 64, [3, 1]),  # (float32 only: a bfloat16 slice is 64 channels)
+        (130, 96, 96, [5, 1, 3]),  # (float32 only)
+        (900, 128, 128, [1, 1]),  # parts of one component only
     ],
 )
-def test_against_float64_product(device, dtype, contraction_major, M, K, N, D, nblocks, nparts):
+def test_against_float64_product(device, dtype, contraction_major, M, K, N, dims):
     if dtype == torch.bfloat16 and K % 64:
         pytest.skip("a bfloat16 slice is 64 channels")
     lib = _lib.load()
-    g = torch.Generator(device=device).manual_seed(M + K + N + D)
-    lda, ldc = nparts * K * D + 8, nparts * N * D + 16
-    es = 2 if dtype == torch.bfloat16 else 4
-    waves = 8 if D * N <= 384 else 4
-    nblocks = max(1, min(nblocks, (160 * 1024 - waves * 16 * (128 * D + 16)) // (N * (es * K + 16))))
+    g = torch.Generator(device=device).manual_seed(M + K + N + sum(dims))
+    nparts = len(dims)
+    lda, ldc = sum(K * d for d in dims) + 8, sum(N * d for d in dims) + 16
+    # one weight block per distinct D (parts of equal D share it)
+    ds = sorted(set(dims))
     A = torch.randn(M, lda, device=device, generator=g).to(dtype)
-    W = torch.randn(nblocks * K * N + 8, device=device, generator=g).to(dtype)
-    # parts in scrambled column order, weight blocks shared between parts
-    parts = [(((p + 1) % nparts) * K * D, (p % nblocks) * K * N, (nparts - 1 - p) * N * D + 16) for p in range(nparts)]
+    W = torch.randn(len(ds) * K * N + 8, device=device, generator=g).to(dtype)
+    # input blocks in order, output blocks in reverse order
+    a_offs = [sum(K * d for d in dims[:p]) for p in range(nparts)]
+    c_offs = [16 + sum(N * d for d in dims[p + 1:]) for p in range(nparts)]
+    parts = [(a_offs[p], ds.index(dims[p]) * K * N, c_offs[p], dims[p]) for p in range(nparts)]
     out = torch.full((M, ldc), 7.0, device=device).to(dtype)
     alpha = 0.37
     stream = torch.cuda.current_stream(device).cuda_stream
     code = BF16 if dtype == torch.bfloat16 else F32
-    _lib.check(lib.cueq_linear_rows_mul_ir(code, contraction_major, M, N, K, D, A.data_ptr(), lda, W.data_ptr(), W.numel(), out.data_ptr(), ldc,
+    _lib.check(lib.cueq_linear_rows_mul_ir(code, contraction_major, M, N, K, A.data_ptr(), lda, W.data_ptr(), W.numel(), out.data_ptr(), ldc,
                                            _table(parts), nparts, alpha, stream), "cueq_linear_rows_mul_ir")
-    ref = _reference(A, W, parts, K, N, D, contraction_major, alpha, ldc)
+    ref = _reference(A, W, parts, K, N, contraction_major, alpha, ldc)
     written = torch.zeros(ldc, dtype=torch.bool, device=device)
-    for _, _, c_off in parts:
-        written[c_off: c_off + N * D] = True
+    for _, _, c_off, d in parts:
+        written[c_off: c_off + N * d] = True
     got = out.double()
     assert (got[:, ~written] == 7.0).all()  # columns of no part stay as they were
     err = (got[:, written] - ref[:, written]).abs().max().item()
