@@ -191,11 +191,12 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         desc = "configs[3]: Linear 128x0e+128x1o+128x2e -> same, batch 200000, shared weights, fwd + bwd (dw, dx)"
         if wl == "cfg4mi":
             desc += "; rows in mul_ir, addressed as they lie by the dense kernels (no transposition pass)"
-    elif wl == "cfg4fc":
+    elif wl in ("cfg4fc", "cfg4fcmi"):
         Z = 50_000
         dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
         i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e")
-        m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, internal_weights=False)
+        # cfg4fcmi: the same product on mul_ir rows (the module's default layout), taken as they lie by the fused kernels
+        m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.mul_ir if wl == "cfg4fcmi" else cue.ir_mul, internal_weights=False)
         g = torch.Generator(device=dev).manual_seed(0)
         x1 = torch.randn(Z, i1.dim, device=dev, generator=g).to(dtype).requires_grad_(True)
         x2 = torch.randn(Z, i2.dim, device=dev, generator=g).to(dtype).requires_grad_(True)
@@ -215,6 +216,8 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = ("configs[3]: FullyConnectedTensorProduct 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, batch 50000, shared weights, "
                 "fwd + bwd (dw, dx1, dx2)")
+        if wl == "cfg4fcmi":
+            desc += "; rows in mul_ir, taken as they lie by the fused kernels (no transposition pass)"
     elif wl == "cfg2sh":
         # configs[1] with the spherical harmonics of the edge vectors evaluated inside the edge kernels (the step before the
         # product in a MACE interaction block): inputs are the raw edge vectors, gradients also with respect to them
@@ -525,7 +528,7 @@ def main() -> int:
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
     ap.add_argument("--graph", action="store_true",
                     help="secondary workloads only: capture the step into a HIP graph and time its replays")
-    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg2sh", "cfg3", "cfg4", "cfg4mi", "cfg4fc", "fcconv", "cfg5"], default=None,
+    ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg2sh", "cfg3", "cfg4", "cfg4mi", "cfg4fc", "cfg4fcmi", "fcconv", "cfg5"], default=None,
                     help="default: the headline metric (cfg2, fp32) with every other configuration in a 'secondary' object.  "
                          "Naming a workload prints one line for it alone: cfg2 the headline, cfg1 the reference's CPU-sized "
                          "channel-wise case, cfg3 symmetric contraction, cfg4 Linear 128 channels l<=2, cfg4fc fully connected "
@@ -603,7 +606,8 @@ def main() -> int:
         add("cfg2_fp64", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float64, N, E, ssteps, swarm, False)[0]))
         for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg4_linear_fp32", "cfg4", "fp32"),
                             ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_linear_fp32_mul_ir", "cfg4mi", "fp32"),
-                            ("cfg4_linear_bf16_mul_ir", "cfg4mi", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
+                            ("cfg4_linear_bf16_mul_ir", "cfg4mi", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("cfg4_fc_fp32_mul_ir", "cfg4fcmi", "fp32"),
+                            ("cfg4_fc_bf16_mul_ir", "cfg4fcmi", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
                             ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp32", "cfg5", "fp32")):
             add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))
         if not args.no_cpu_baseline:

@@ -87,6 +87,23 @@ constexpr int kWaves = 8;
 '''
 
 
+def _mul_ir_blocks(blocks):
+    """``[(start, mul, d)]`` of the blocks of an operand whose rows keep the component index contiguous (``mul_ir``:
+    element (channel u, component i) of the block at ``start + u * d + i``; the kernels' own order is ``start + i * mul +
+    u``).  Blocks of one component or one channel are the same in both orders and are left out."""
+    return [(s0, mul, d) for s0, mul, d in (blocks or []) if d > 1 and mul > 1]
+
+
+def _block_at(col: int, blocks, segment_start: bool = True):
+    """The block ``(start, mul, d, component)`` that holds column ``col`` (in the kernels' own order), or None;
+    ``segment_start``: ``col`` is the first column of an operand segment."""
+    for s0, mul, d in blocks:
+        if s0 <= col < s0 + mul * d:
+            assert not segment_start or (col - s0) % mul == 0, "a path operand is one whole segment of a block"
+            return s0, mul, d, (col - s0) // mul
+    return None
+
+
 def _products(paths, transposed: bool):
     """Group the paths by product.  Forward orientation (``transposed``): product = (block, x1 segment), result rows n,
     contraction k, uses = (j, coeff, output offset).  Otherwise: product = (block, output segment), result rows k,
@@ -101,10 +118,13 @@ def _products(paths, transposed: bool):
     return prods
 
 
-def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, width_res: int, n2: int):
+def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, width_res: int, n2: int, in_blocks=None, res_blocks=None):
     """One kernel.  ``transposed``: the blocks sit in LDS as W^T (rows n, contraction k).  ``rowdot``: instead of
-    accumulating the scaled products into result columns, they are multiplied element-wise with G and summed per row."""
+    accumulating the scaled products into result columns, they are multiplied element-wise with G and summed per row.
+    ``in_blocks`` / ``res_blocks``: blocks of the row operand ``IN`` / of the result (``G`` for ``rowdot``) that lie in
+    ``mul_ir`` order in memory - see ``_mul_ir_blocks``; column numbers everywhere else are in the kernels' own order."""
     es = 4 if T == "float" else 2
+    in_blocks, res_blocks = _mul_ir_blocks(in_blocks), _mul_ir_blocks(res_blocks)
     blocks = sorted({(p.w_off, p.K, p.N) for p in paths})
     lds_off, off = {}, 0
     for w_off, K, N in blocks:
@@ -144,9 +164,31 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
         used_tiles = sorted({u[2] // 32 + t for (w_off, K, N, _), us in prods.items() for u in us for t in range((N if transposed else K) // 32)})
         for gt in used_tiles:
             A(f"    float g{gt}[16];")
-            A("#pragma unroll")
-            A(f"    for (int a = 0; a < 4; ++a) {{ float gv[4]; load4(G + z * ldg + {32 * gt} + 4 * h + 8 * a, gv); "
-              f"g{gt}[4 * a] = gv[0]; g{gt}[4 * a + 1] = gv[1]; g{gt}[4 * a + 2] = gv[2]; g{gt}[4 * a + 3] = gv[3]; }}")
+        done = set()
+        for gt in used_tiles:
+            blk = _block_at(32 * gt, res_blocks, False)
+            if blk is None:
+                A("#pragma unroll")
+                A(f"    for (int a = 0; a < 4; ++a) {{ float gv[4]; load4(G + z * ldg + {32 * gt} + 4 * h + 8 * a, gv); "
+                  f"g{gt}[4 * a] = gv[0]; g{gt}[4 * a + 1] = gv[1]; g{gt}[4 * a + 2] = gv[2]; g{gt}[4 * a + 3] = gv[3]; }}")
+                continue
+            # mul_ir block: the lane's columns 8 a + 4 h + r of tile t with all d components are 4 d consecutive elements
+            s0, mul, d, _ = blk
+            t = ((32 * gt - s0) % mul) // 32
+            if (s0, t) in done:
+                continue
+            done.add((s0, t))
+            for a in range(4):
+                A(f"    {{ float gv[{4 * d}];")
+                for m in range(d):
+                    A(f"      {{ float q4[4]; load4(G + z * ldg + {s0} + ({32 * t + 8 * a} + 4 * h) * {d} + {4 * m}, q4); "
+                      f"gv[{4 * m}] = q4[0]; gv[{4 * m + 1}] = q4[1]; gv[{4 * m + 2}] = q4[2]; gv[{4 * m + 3}] = q4[3]; }}")
+                for kc in range(d):
+                    tile = (s0 + kc * mul) // 32 + t
+                    if tile in used_tiles:
+                        for r in range(4):
+                            A(f"      g{tile}[{4 * a + r}] = gv[{r * d + kc}];")
+                A("    }")
     else:
         for t in range(ntiles):
             A(f"    floatx16 o{t} = floatx16{{0}};")
@@ -154,53 +196,96 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
     by_seg = OrderedDict()
     for (w_off, K, N, in_off), uses in prods.items():
         by_seg.setdefault(in_off, []).append((w_off, K, N, uses))
-    # the fragments of the next operand segment are requested before the products of the current one are worked on
     segs = list(by_seg.items())
-    contraction = [(pl[0][1] if transposed else pl[0][2]) for _, pl in segs]
-    for (in_off, pl), C in zip(segs, contraction):
-        assert all((p[1] if transposed else p[2]) == C for p in pl), "one operand segment, one contraction length"
-    nsmax = max(contraction) * es // 64
-    A(f"    uint4 xfa[{nsmax}][2], xfb[{nsmax}][2];")
+    if in_blocks:
+        segs.sort(key=lambda it: it[0])  # the segments of a block next to each other
+    contraction = {in_off: (pl[0][1] if transposed else pl[0][2]) for in_off, pl in segs}
+    for in_off, pl in segs:
+        assert all((p[1] if transposed else p[2]) == contraction[in_off] for p in pl), "one operand segment, one contraction length"
+    # Operand groups: a segment on its own, or the segments of one mul_ir block together - the lane's channels of such a
+    # block with all their components are one contiguous run of the row, loaded once and taken apart in registers.
+    groups = []
+    for in_off, pl in segs:
+        blk = _block_at(in_off, in_blocks)
+        if blk is not None and groups and groups[-1][0] is not None and groups[-1][0][:3] == blk[:3]:
+            groups[-1][1].append((in_off, pl, blk[3]))
+        else:
+            groups.append((blk, [(in_off, pl, blk[3] if blk else 0)]))
+    def nraw(g):  # 16-byte vectors a lane holds for the group
+        blk, members = g
+        C = contraction[members[0][0]]
+        return (C * es // 64) * 2 * (blk[2] if blk else 1)
+    A(f"    uint4 rawa[{max(nraw(g) for g in groups[0::2])}], rawb[{max([nraw(g) for g in groups[1::2]] or [1])}];")
 
-    def request(i):
-        in_off, C = segs[i][0], contraction[i]
-        name = "xfa" if i % 2 == 0 else "xfb"
-        for s2 in range(C * es // 64):
-            for q in range(2):
-                A(f"    {name}[{s2}][{q}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {in_off}) + {s2 * 64} + h * 32 + {q * 16});")
+    def request(gi):
+        blk, members = groups[gi]
+        C = contraction[members[0][0]]
+        name = "rawa" if gi % 2 == 0 else "rawb"
+        if blk is None:
+            in_off = members[0][0]
+            for s2 in range(C * es // 64):
+                for q in range(2):
+                    A(f"    {name}[{2 * s2 + q}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {in_off}) + {s2 * 64} + h * 32 + {q * 16});")
+        else:
+            s0, mul, d, _ = blk
+            for s2 in range(C * es // 64):
+                for m in range(2 * d):
+                    A(f"    {name}[{2 * d * s2 + m}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {s0}) + ({s2 * 64} + h * 32) * {d} + {16 * m});")
+
+    def fragment(gi, comp, s2, q):
+        """Expression of the MFMA operand (s2, q) of component ``comp`` of group ``gi``: 16 bytes of consecutive channels."""
+        blk, members = groups[gi]
+        name = "rawa" if gi % 2 == 0 else "rawb"
+        if blk is None:
+            return f"{name}[{2 * s2 + q}]"
+        d = blk[2]
+        word = lambda e: f"{name}[{2 * d * s2 + (e // (4 if es == 4 else 8))}].{'xyzw'[(e // (1 if es == 4 else 2)) % 4]}"
+        if es == 4:  # elements (4 q + e) * d + comp of the run, e < 4
+            return "make_uint4(" + ", ".join(word((4 * q + e) * d + comp) for e in range(4)) + ")"
+        parts = []
+        for j in range(4):  # dword j: elements (8 q + 2 j) * d + comp (low half) and the next channel's (high half)
+            e0 = (8 * q + 2 * j) * d + comp
+            e1 = e0 + d
+            sel = (0x0302 if e0 & 1 else 0x0100) | ((0x0706 if e1 & 1 else 0x0504) << 16)
+            parts.append(f"__builtin_amdgcn_perm({word(e1)}, {word(e0)}, 0x{sel:08x}u)")
+        return "make_uint4(" + ", ".join(parts) + ")"
 
     request(0)
-    for i, (in_off, plist) in enumerate(segs):
-        ns = contraction[i] * es // 64
-        xf = "xfa" if i % 2 == 0 else "xfb"
-        if i + 1 < len(segs):
-            request(i + 1)
-        A("    {")
-        for w_off, K, N, uses in plist:
-            o, R, Cc, RS = lds_off[w_off]
-            for t in range(R // 32):
-                A("      {")
-                A("        floatx16 T = floatx16{0};")
-                A(f"        const char* wr = smem + {o} + ({32 * t} + c) * {RS} + h * 32;")
-                for s2 in range(ns):
-                    for q in range(2):
-                        A(f"        mma_step<{T}>(T, *reinterpret_cast<const uint4*>(wr + {s2 * 64 + q * 16}), {xf}[{s2}][{q}]);")
-                for j, coeff, res_off in uses:
-                    if rowdot:
-                        A("        {")
-                        A("          float p = 0.f;")
-                        A("#pragma unroll")
-                        A(f"          for (int v = 0; v < 16; ++v) p = fmaf(T[v], g{res_off // 32 + t}[v], p);")
-                        A(f"          d{j} = fmaf({coeff!r}f, p, d{j});")
-                        A(f'          asm volatile("" : "+v"(d{j}));  // finish this use here: a product\'s result is not kept for later')
-                        A("        }")
-                    else:
-                        A(f"        {{ const float sc = {coeff!r}f * s{j};")
-                        A("#pragma unroll")
-                        A(f"          for (int v = 0; v < 16; ++v) o{res_off // 32 + t}[v] = fmaf(sc, T[v], o{res_off // 32 + t}[v]); }}")
-                A("      }")
-                A("      __builtin_amdgcn_sched_barrier(0);  // keep the loads of later products from piling up ahead of this one")
-        A("    }")
+    for gi, (blk, members) in enumerate(groups):
+        # the operands of the next group are requested before the products of the current one are worked on
+        if gi + 1 < len(groups):
+            request(gi + 1)
+        for in_off, plist, comp in members:
+            ns = contraction[in_off] * es // 64
+            A("    {")
+            for s2 in range(ns):
+                for q in range(2):
+                    A(f"      const uint4 xf_{s2}_{q} = {fragment(gi, comp, s2, q)};")
+            for w_off, K, N, uses in plist:
+                o, R, Cc, RS = lds_off[w_off]
+                for t in range(R // 32):
+                    A("      {")
+                    A("        floatx16 T = floatx16{0};")
+                    A(f"        const char* wr = smem + {o} + ({32 * t} + c) * {RS} + h * 32;")
+                    for s2 in range(ns):
+                        for q in range(2):
+                            A(f"        mma_step<{T}>(T, *reinterpret_cast<const uint4*>(wr + {s2 * 64 + q * 16}), xf_{s2}_{q});")
+                    for j, coeff, res_off in uses:
+                        if rowdot:
+                            A("        {")
+                            A("          float p = 0.f;")
+                            A("#pragma unroll")
+                            A(f"          for (int v = 0; v < 16; ++v) p = fmaf(T[v], g{res_off // 32 + t}[v], p);")
+                            A(f"          d{j} = fmaf({coeff!r}f, p, d{j});")
+                            A(f'          asm volatile("" : "+v"(d{j}));  // finish this use here: a product\'s result is not kept for later')
+                            A("        }")
+                        else:
+                            A(f"        {{ const float sc = {coeff!r}f * s{j};")
+                            A("#pragma unroll")
+                            A(f"          for (int v = 0; v < 16; ++v) o{res_off // 32 + t}[v] = fmaf(sc, T[v], o{res_off // 32 + t}[v]); }}")
+                    A("      }")
+                    A("      __builtin_amdgcn_sched_barrier(0);  // keep the loads of later products from piling up ahead of this one")
+            A("    }")
     # rows past the end were clamped to the last row: those lanes hold its values and store them again (the same
     # bits to the same place) - a store under a condition would let the compiler sink every use of a product down
     # to it, past all the other products, and keep their results alive in scratch memory
@@ -215,9 +300,24 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
     else:
         A("    {")
         A(f"      {T}* op = OUT + z * ldo + 4 * h;")
+        done = set()
         for t in range(ntiles):
-            A("#pragma unroll")
-            A(f"      for (int a = 0; a < 4; ++a) store4(op + {32 * t} + 8 * a, o{t}[4 * a], o{t}[4 * a + 1], o{t}[4 * a + 2], o{t}[4 * a + 3]);")
+            blk = _block_at(32 * t, res_blocks, False)
+            if blk is None:
+                A("#pragma unroll")
+                A(f"      for (int a = 0; a < 4; ++a) store4(op + {32 * t} + 8 * a, o{t}[4 * a], o{t}[4 * a + 1], o{t}[4 * a + 2], o{t}[4 * a + 3]);")
+                continue
+            # mul_ir block: the lane's channels 8 a + 4 h + r of tile tb with their d components are 4 d consecutive elements
+            s0, mul, d, _ = blk
+            tb = ((32 * t - s0) % mul) // 32
+            if (s0, tb) in done:
+                continue
+            done.add((s0, tb))
+            val = lambda a, m: f"o{(s0 + (m % d) * mul) // 32 + tb}[{4 * a + m // d}]"
+            for a in range(4):
+                for m4 in range(d):
+                    A(f"      store4(OUT + z * ldo + {s0} + ({32 * tb + 8 * a} + 4 * h) * {d} + {4 * m4}, "
+                      + ", ".join(val(a, 4 * m4 + e) for e in range(4)) + ");")
         A("    }")
     A("  }")
     A("}")
@@ -227,7 +327,16 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
 DW_ROWS = 16  # batch rows per staged tile of the weight-gradient kernel
 
 
-def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
+def _emit_colmap(A, name: str, blocks):
+    """``int name(int p)``: the column in the kernels' own order of the element at column ``p`` of a row in memory."""
+    A(f"__device__ __forceinline__ int {name}(int p) {{")
+    for s0, mul, d in blocks:
+        A(f"  if (p >= {s0} && p < {s0 + mul * d}) {{ const int r = p - {s0}; return {s0} + (r % {d}) * {mul} + r / {d}; }}")
+    A("  return p;")
+    A("}")
+
+
+def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int, x_blocks=None, g_blocks=None):
     """Weight gradient ``dW_b[k, n] = sum_z x1[z, a_off + k] H[z, n]`` with ``H = sum over the uses of (b, a_off) of
     c x2[z, j] g[z, c_off + n]`` formed in registers.  The batch is the contraction: a lane feeds the 32x32x2 MFMA one
     element of ``x1`` (row ``z0 + lane / 32``, column ``a_off + k``) and one of ``H``, no transposition.  A block owns a
@@ -237,6 +346,13 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
     es = 4 if T == "float" else 2
     per = 16 // es  # elements per 16-byte load
     R, WX, WG, WS = DW_ROWS, width_in, width_out, 16
+    # rows in mul_ir order are put into the kernels' own order while they are staged in LDS (element by element: a tile is
+    # 16 rows), everything behind the staging is the same
+    x_blocks, g_blocks = _mul_ir_blocks(x_blocks), _mul_ir_blocks(g_blocks)
+    if x_blocks:
+        _emit_colmap(A, "dw_xcol", x_blocks)
+    if g_blocks:
+        _emit_colmap(A, "dw_gcol", g_blocks)
     prods = _products(paths, True)  # (w_off, K, N, a_off) -> [(j, coeff, c_off)]
     units = {}  # (w_off, K, N, nt) -> [(a_off, uses)]
     for (w_off, K, N, a_off), uses in prods.items():
@@ -290,6 +406,24 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
     A("  auto commit = [&](float* buf) {")
     for name, W, n, base in (("xr", WX, nx, 0), ("gr", WG, ng, XB // 4)):
         for i in range(n):
+            blocks, cmap = (x_blocks, "dw_xcol") if name == "xr" else (g_blocks, "dw_gcol")
+            if blocks:
+                A(f"    {{ const int s = tid + {512 * i}, row = s / {W // per}, q = s % {W // per};")
+                A(f"      if (s < {R * W // per}) {{")
+                A(f"        const uint32_t w4[4] = {{{name}[{i}].x, {name}[{i}].y, {name}[{i}].z, {name}[{i}].w}};")
+                A("#pragma unroll")
+                A(f"        for (int e = 0; e < {per}; ++e) {{")
+                A(f"          const int col = {cmap}(q * {per} + e);")
+                if es == 4:
+                    A(f"          buf[{base} + row * {W} + col] = __uint_as_float(w4[e]);")
+                elif fast16 and name == "xr":
+                    A(f"          *reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(buf) + row * {XSTR} + col * 2) = static_cast<uint16_t>(w4[e >> 1] >> (16 * (e & 1)));")
+                else:
+                    A(f"          buf[{base} + row * {W} + col] = __uint_as_float((w4[e >> 1] >> (16 * (e & 1))) << 16);")
+                A("        }")
+                A("      }")
+                A("    }")
+                continue
             if fast16 and name == "xr":
                 A(f"    {{ const int s = tid + {512 * i}, row = s / {W // per}, q = s % {W // per}; "
                   f"if (s < {R * W // per}) *reinterpret_cast<uint4*>(reinterpret_cast<char*>(buf) + row * {XSTR} + q * 16) = xr[{i}]; }}")
@@ -389,16 +523,19 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int):
     A("")
 
 
-def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str) -> str:
-    """``paths``: objects with ``w_off, a_off, j, c_off, K, N, coeff``; ``T``: ``float`` or ``uint16_t`` (bfloat16 bits)."""
+def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=None, out_blocks=None) -> str:
+    """``paths``: objects with ``w_off, a_off, j, c_off, K, N, coeff``; ``T``: ``float`` or ``uint16_t`` (bfloat16 bits).
+    ``in_blocks`` / ``out_blocks``: ``[(start, mul, d)]`` of the first operand / the output when their rows lie in ``mul_ir``
+    order in memory (the reference transposes such rows in front of and behind its kernel,
+    ``cuequivariance_torch/operations/tp_fully_connected.py:118-150``); ``None``: ``ir_mul``, the kernels' own order."""
     L = []
     A = L.append
     A("// GENERATED by cuequivariance_amd/codegen/fullyconnected.py - do not edit.")
     A(PRELUDE)
-    _emit_kernel(A, "fwd", T, paths, True, False, width_out, n2)
-    _emit_kernel(A, "dx1", T, paths, False, False, width_in, n2)
-    _emit_kernel(A, "dx2", T, paths, True, True, width_out, n2)
-    _emit_dw_kernel(A, T, paths, n2, width_in, width_out)
+    _emit_kernel(A, "fwd", T, paths, True, False, width_out, n2, in_blocks, out_blocks)
+    _emit_kernel(A, "dx1", T, paths, False, False, width_in, n2, out_blocks, in_blocks)
+    _emit_kernel(A, "dx2", T, paths, True, True, width_out, n2, in_blocks, out_blocks)
+    _emit_dw_kernel(A, T, paths, n2, width_in, width_out, in_blocks, out_blocks)
     A("// compute units of the current device (asked once per device: the query is slow)")
     A("int grid_for(int64_t Z) {")
     A("  static int cus_of[64] = {0};")

@@ -773,6 +773,8 @@ class _FcFunction(torch.autograd.Function):
                 stream = torch.cuda.current_stream(dev).cuda_stream
                 code, es = _DTYPE_CODE[dtype], x1d.element_size()
                 unit = mod.fused_unit(dtype, x1d, out)
+                if unit is None and mod.rows_mul_ir:
+                    raise NotImplementedError("fused_tp: rows='mul_ir' needs the generated fused kernels")
                 if unit is not None:
                     if unit.fcj_fwd(Z, wd.data_ptr(), x1d.data_ptr(), x1d.stride(0), x2d.data_ptr(), x2d.stride(0), out.data_ptr(),
                                     out.stride(0), stream) != 0:
@@ -822,6 +824,8 @@ class _FcFunction(torch.autograd.Function):
             code, es = _DTYPE_CODE[dtype], x1d.element_size()
             tables = plan.device(dev)
             unit = unit_w = mod.fused_unit(dtype, x1d, g) if Z > 0 else None
+            if unit is None and mod.rows_mul_ir and Z > 0:
+                raise NotImplementedError("fused_tp: rows='mul_ir' needs the generated fused kernels")
             if need_x1:  # (the generated kernels write every column)
                 gx1 = (torch.empty_like if mod.dx1_covers_input or unit is not None else torch.zeros_like)(x1d)
             if need_x2:
@@ -1175,10 +1179,11 @@ class SegmentedPolynomialDense(nn.Module):
     """Dense (MFMA) executor for Linear / fully-connected polynomials with weights shared over the batch."""
 
     def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype=None, output_dtype_map: List[int] = None,
-                 name: str = "segmented_polynomial", method: str = "fused_tp", rows: str = "ir_mul"):
+                 name: str = "segmented_polynomial", method: str = "fused_tp", rows: str = "ir_mul", row_blocks=None):
         super().__init__()
         self._polynomial_orig = polynomial
         self._rows_orig = rows
+        self._row_blocks_orig = row_blocks
         self._output_dtype_map_orig = output_dtype_map
         self.name = name
         self.method = method
@@ -1214,11 +1219,28 @@ class SegmentedPolynomialDense(nn.Module):
         # rows="mul_ir": the irreps operands (input 1 and the output of the 3-operand form) keep the component index
         # contiguous inside every block; the kernels address them so - no transposition pass around the call.  Not part of
         # the reference's interface.  `mul_ir` is None when the blocks do not have the shape those kernels take.
-        self.mul_ir = _MulIrPlan.build(self) if rows == "mul_ir" else None
-        if rows == "mul_ir" and self.mul_ir is None:
-            raise NotImplementedError("fused_tp: rows='mul_ir' needs a Linear-like polynomial with blocks of 1, 3, 5 or 7 components and "
-                                      "multiplicities 32, 64, 96 or 128")
-        self.rows_mul_ir = self.mul_ir is not None
+        # 4-operand form: `row_blocks` = ([(mul, d)] of the first operand, [(mul, d)] of the output); the generated fused kernels
+        # take such rows apart / put them together in registers, other executors of this module do not take them.
+        self.mul_ir, self.fc_blocks = None, None
+        if rows == "mul_ir" and not self.has_x2:
+            self.mul_ir = _MulIrPlan.build(self)
+            if self.mul_ir is None:
+                raise NotImplementedError("fused_tp: rows='mul_ir' needs a Linear-like polynomial with blocks of 1, 3, 5 or 7 components "
+                                          "and multiplicities 32, 64, 96 or 128")
+        elif rows == "mul_ir":
+            def starts(blocks, size):
+                out, off = [], 0
+                for mul, d in blocks:
+                    out.append((off, int(mul), int(d)))
+                    off += mul * d
+                if off != size:
+                    raise ValueError("fused_tp: row_blocks do not cover the operand")
+                return out
+
+            if row_blocks is None:
+                raise NotImplementedError("fused_tp: rows='mul_ir' of a 4-operand contraction needs row_blocks")
+            self.fc_blocks = (starts(row_blocks[0], self.input_sizes[1]), starts(row_blocks[1], self.out_size))
+        self.rows_mul_ir = rows == "mul_ir"
         with _traced_lock:  # the integer under which a traced graph names this module
             self.traced_id = next(_traced_ids)
             _traced_modules[self.traced_id] = weakref.ref(self)
@@ -1234,9 +1256,26 @@ class SegmentedPolynomialDense(nn.Module):
 
         key = (dtype, jit.enabled())
         if key not in self._fused:
+            blocks = self.fc_blocks or (None, None)
             self._fused[key] = jit.fully_connected_unit(self.paths, self.input_sizes[2], self.input_sizes[1], self.out_size,
-                                                          "float" if dtype == torch.float32 else "uint16_t")
+                                                          "float" if dtype == torch.float32 else "uint16_t", blocks[0], blocks[1])
         return self._fused[key]
+
+    def mul_ir_ready(self, dtype) -> bool:
+        """Whether rows in ``mul_ir`` can be taken as they lie for this dtype."""
+        if not self.rows_mul_ir:
+            return False
+        if self.mul_ir is not None:
+            return self.mul_ir.accepts(dtype)
+        if dtype not in (torch.float32, torch.bfloat16) or not self.fc_plan.ok:
+            return False
+        from .. import jit
+
+        key = (dtype, jit.enabled())
+        if key not in self._fused:
+            self._fused[key] = jit.fully_connected_unit(self.paths, self.input_sizes[2], self.input_sizes[1], self.out_size,
+                                                          "float" if dtype == torch.float32 else "uint16_t", *self.fc_blocks)
+        return self._fused[key] is not None
 
     def tiled(self, dtype, A: torch.Tensor, Cout: torch.Tensor) -> bool:
         """The tiled kernel serves fp32 / bf16 contractions without a per-row scale."""
@@ -1264,7 +1303,7 @@ class SegmentedPolynomialDense(nn.Module):
         from .segmented_polynomial import SegmentedPolynomial
 
         return (SegmentedPolynomial, (self._polynomial_orig, self.method, self.math_dtype, self._output_dtype_map_orig, self.name,
-                                      {"rows": self._rows_orig} if self._rows_orig != "ir_mul" else None))
+                                      {"rows": self._rows_orig, "row_blocks": self._row_blocks_orig} if self._rows_orig != "ir_mul" else None))
 
     def _indexed(self, w: torch.Tensor, x1: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
         """One weight row per class, rows of ``x1`` sorted by class (reference
@@ -1306,8 +1345,11 @@ class SegmentedPolynomialDense(nn.Module):
             raise NotImplementedError("fused_tp: weights must be shared over the batch (one row)")
         if x1.dtype not in _DTYPE_CODE:
             raise ValueError(f"fused_tp: unsupported dtype {x1.dtype}")
-        if self.rows_mul_ir and not self.mul_ir.accepts(x1.dtype):
+        if self.rows_mul_ir and self.mul_ir is not None and not self.mul_ir.accepts(x1.dtype):
             raise NotImplementedError(f"fused_tp: rows='mul_ir' does not take {x1.dtype} with these multiplicities")
+        if self.rows_mul_ir and self.fc_blocks is not None and not self.mul_ir_ready(x1.dtype):
+            raise NotImplementedError("fused_tp: rows='mul_ir' of a fully connected product runs on the generated fused kernels only "
+                                      "(float32 / bfloat16, compilation at first use switched on or the product prebuilt)")
         if self.math_dtype == torch.float32 and x1.dtype == torch.float64:
             raise ValueError("Fused TP does not support float32 math_dtype with float64 inputs.")
         if x2 is not None:

@@ -77,11 +77,11 @@ def _permute_inputs(polynomial: cue.SegmentedPolynomial, perm) -> cue.SegmentedP
 
 class SegmentedPolynomialFusedTP(nn.Module):
     def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype=None, output_dtype_map: Optional[List[int]] = None,
-                 name: str = "segmented_polynomial", rows: str = "ir_mul"):
+                 name: str = "segmented_polynomial", rows: str = "ir_mul", row_blocks=None):
         super().__init__()
         from .dense import SegmentedPolynomialDense
 
-        self._rows_orig = rows
+        self._rows_orig, self._row_blocks_orig = rows, row_blocks
 
         self._polynomial_orig = polynomial
         self._output_dtype_map_orig = output_dtype_map
@@ -114,7 +114,10 @@ class SegmentedPolynomialFusedTP(nn.Module):
 
             for perm in itertools.permutations(range(polynomial.num_inputs)):
                 try:
-                    self.dense = SegmentedPolynomialDense(_permute_inputs(polynomial, perm), math_dtype, output_dtype_map, name, rows=rows)
+                    if rows == "mul_ir" and perm != tuple(range(polynomial.num_inputs)):
+                        continue  # (row_blocks name the operands in the given order)
+                    self.dense = SegmentedPolynomialDense(_permute_inputs(polynomial, perm), math_dtype, output_dtype_map, name, rows=rows,
+                                                          row_blocks=row_blocks)
                     self.dense_perm = perm
                     break
                 except NotImplementedError:
@@ -138,7 +141,7 @@ class SegmentedPolynomialFusedTP(nn.Module):
         from .segmented_polynomial import SegmentedPolynomial
 
         return (SegmentedPolynomial, (self._polynomial_orig, "fused_tp", self.math_dtype, self._output_dtype_map_orig, self.name,
-                                      {"rows": self._rows_orig} if self._rows_orig != "ir_mul" else None))
+                                      {"rows": self._rows_orig, "row_blocks": self._row_blocks_orig} if self._rows_orig != "ir_mul" else None))
 
     def forward(self, inputs: List[torch.Tensor], input_indices: Dict[int, torch.Tensor],
                 output_shapes: Dict[int, torch.Tensor], output_indices: Dict[int, torch.Tensor]):

@@ -362,6 +362,19 @@ class FullyConnectedTensorProduct(torch.nn.Module):
             # the matrix-core executor takes a second operand of multiplicity one; others run on the uniform-1d kernels of
             # the flattened descriptor, with the weight row shared by the batch
             self.f = None
+        # mul_ir rows of the first operand and of the output taken as they lie by the generated fused kernels (no
+        # transposition pass) when those kernels serve the call; everything else keeps the passes
+        self.f_rows = None
+        if (self.f is not None and self.method == "fused_tp" and self.transpose_in1.source == cue.mul_ir
+                and self.transpose_out.target == cue.mul_ir and e.inputs[1].layout == cue.ir_mul and e.outputs[0].layout == cue.ir_mul
+                and (_transposition_moves(e.inputs[1].irreps) or _transposition_moves(e.outputs[0].irreps))):
+            try:
+                self.f_rows = SegmentedPolynomial(
+                    e.polynomial, method="fused_tp", math_dtype=math_dtype,
+                    options={"rows": "mul_ir", "row_blocks": ([(mul, ir.dim) for mul, ir in e.inputs[1].irreps],
+                                                               [(mul, ir.dim) for mul, ir in e.outputs[0].irreps])})
+            except (NotImplementedError, ValueError):
+                self.f_rows = None
         # A second operand of V invariant scalars ("10x0e" node attributes): the product is the Linear map of the
         # features x1[i, u] * x2[v] (multiplicity u * V) with the very same weights - same paths, same weight layout
         # (u, v, w) = (u * V + v, w), same coefficients - and runs on the dense 3-operand kernels.
@@ -385,14 +398,16 @@ class FullyConnectedTensorProduct(torch.nn.Module):
                 size_out: Optional[int] = None) -> torch.Tensor:
         """``indices_1`` (rows of ``x1`` per batch element) and ``indices_out`` / ``size_out`` (output row per batch
         element, summed) are extensions over the reference's signature: gather and scatter-sum inside the kernel."""
-        x1 = apply_layout(self.transpose_in1, x1)
-        x2 = apply_layout(self.transpose_in2, x2)
         if self.weight is not None:
             if weight is not None:
                 raise ValueError("Internal weights are used, weight should be None")
             weight = self.weight
         elif weight is None:
             raise ValueError("Internal weights are not used, weight should not be None")
+        if indices_1 is None and indices_out is None and self._rows_ready(x1, x2, weight):
+            return self.f_rows([weight, x1, apply_layout(self.transpose_in2, x2)])[0]
+        x1 = apply_layout(self.transpose_in1, x1)
+        x2 = apply_layout(self.transpose_in2, x2)
         if indices_1 is not None or indices_out is not None:
             if indices_out is not None and size_out is None:
                 raise ValueError("size_out should be provided if indices_out is provided")
@@ -410,6 +425,11 @@ class FullyConnectedTensorProduct(torch.nn.Module):
         if weight.shape[0] != 1 or self.f is None:
             return apply_layout(self.transpose_out, self.f_per_sample([weight, x1, x2])[0])
         return apply_layout(self.transpose_out, self.f([weight, x1, x2])[0])
+
+    def _rows_ready(self, x1, x2, weight) -> bool:
+        dense = self.f_rows.m.dense if self.f_rows is not None else None
+        return (dense is not None and weight is not None and weight.shape[0] == 1 and x1.is_cuda and x1.dtype == x2.dtype == weight.dtype
+                and x1.shape[0] == x2.shape[0] and dense.mul_ir_ready(x1.dtype))
 
 
 class Linear(torch.nn.Module):

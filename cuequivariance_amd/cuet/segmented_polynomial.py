@@ -229,7 +229,8 @@ class SegmentedPolynomial(nn.Module):
 
             # option "rows": "mul_ir" - the irreps operands of a Linear-like polynomial keep the component index contiguous
             # inside every block and the dense kernels address them so (not part of the reference's options)
-            self.m = SegmentedPolynomialFusedTP(polynomial, math_dtype, output_dtype_map, name, rows=self.options.get("rows", "ir_mul"))
+            self.m = SegmentedPolynomialFusedTP(polynomial, math_dtype, output_dtype_map, name, rows=self.options.get("rows", "ir_mul"),
+                                                row_blocks=self.options.get("row_blocks"))
         elif method == "naive":
             raise ValueError(
                 "method='naive' (the PyTorch executor) is not part of this engine: every method runs HIP kernels. "

@@ -279,6 +279,14 @@ def _compile(src: str, so: Path, what: str, link_library: bool = True) -> None:
 PREBUILT = Path(__file__).resolve().parent / "prebuilt"
 
 
+def _starts(irreps) -> list:
+    out, off = [], 0
+    for mul, ir in irreps:
+        out.append(off)
+        off += mul * ir.dim
+    return out
+
+
 def prebuild_fully_connected(force: bool = False) -> list:
     """Compile the fused kernels of the fully connected products listed in ``codegen/registry.py`` into
     ``cuequivariance_amd/prebuilt/`` (called when the library is built; the objects are named by the hash of their
@@ -293,19 +301,23 @@ def prebuild_fully_connected(force: bool = False) -> list:
         m = cuet.FullyConnectedTensorProduct(cue.Irreps("O3", i1), cue.Irreps("O3", i2), cue.Irreps("O3", i3), layout=cue.ir_mul,
                                              internal_weights=False)
         dense = next(x for x in m.modules() if type(x).__name__ == "SegmentedPolynomialDense")
+        # both row orders of the first operand and the output: ir_mul (the kernels' own) and mul_ir (the modules' default)
+        mul_ir = ([(o, mul, ir.dim) for o, (mul, ir) in zip(_starts(m.irreps_in1), m.irreps_in1)],
+                  [(o, mul, ir.dim) for o, (mul, ir) in zip(_starts(m.irreps_out), m.irreps_out)])
         for T in ("float", "uint16_t"):
-            src = fc.emit_unit(dense.paths, dense.input_sizes[2], dense.input_sizes[1], dense.out_size, T)
-            so = PREBUILT / f"fc_{hashlib.sha1(src.encode()).hexdigest()[:16]}_{T}.so"
-            if force or not so.exists():
-                _compile(src, so, f"the fully connected product {i1} (x) {i2} -> {i3} ({T})", link_library=False)
-            wanted.append(so)
+            for blocks, tag in (((None, None), ""), (mul_ir, ", mul_ir rows")):
+                src = fc.emit_unit(dense.paths, dense.input_sizes[2], dense.input_sizes[1], dense.out_size, T, *blocks)
+                so = PREBUILT / f"fc_{hashlib.sha1(src.encode()).hexdigest()[:16]}_{T}.so"
+                if force or not so.exists():
+                    _compile(src, so, f"the fully connected product {i1} (x) {i2} -> {i3} ({T}{tag})", link_library=False)
+                wanted.append(so)
     for old in PREBUILT.glob("fc_*.so"):
         if old not in wanted:
             old.unlink()
     return wanted
 
 
-def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str):
+def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=None, out_blocks=None):
     """The fused kernels of ``codegen/fullyconnected.py`` for one fully connected product and element type (``float`` or
     ``uint16_t`` for bfloat16), compiled at first use and loaded: a ``ctypes`` handle with ``fcj_fwd``, ``fcj_dx1``,
     ``fcj_dx2`` and ``fcj_dw``, or ``None`` when this module is off, the product is outside what the generator covers, or the compiler
@@ -314,7 +326,7 @@ def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str):
 
     if not enabled() or not fc.supported(paths, n2, width_in, width_out, 4 if T == "float" else 2):
         return None
-    src = fc.emit_unit(paths, n2, width_in, width_out, T)
+    src = fc.emit_unit(paths, n2, width_in, width_out, T, in_blocks, out_blocks)
     key = "fc_" + hashlib.sha1(src.encode()).hexdigest()[:16]
     with _lock:
         if key in _loaded:

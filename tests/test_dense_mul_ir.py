@@ -133,3 +133,52 @@ def test_linear_mul_ir_second_derivatives(device):
     got_g = torch.autograd.grad(got, b)
     for gg, rr in zip(got_g, ref_g):
         assert rel_err(gg, rr) <= 2e-5
+
+
+@pytest.fixture
+def kernels_at_first_use():
+    from cuequivariance_amd import jit
+
+    on = jit.enabled()
+    jit.enable(True)
+    yield
+    jit.enable(on)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(
+    "irreps_in1,irreps_in2,irreps_out,Z",
+    [
+        ("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o", 2500),  # the benchmark's product
+        ("32x0e+64x1o", "0e+1o", "64x0e+32x1o", 333),  # mixed multiplicities, ragged rows
+        ("32x0e+32x2e", "0e+2e", "64x0e+32x2e", 77),  # blocks of 5 components
+    ],
+)
+def test_fully_connected_mul_ir_matches_oracle_without_transposition(device, kernels_at_first_use, dtype, irreps_in1, irreps_in2, irreps_out, Z):
+    """The generated fused kernels take mul_ir rows of the first operand and of the output as they lie
+    (reference: transposition passes around the kernel, ``cuequivariance_torch/operations/tp_fully_connected.py:118-150``)."""
+    i1, i2, i3 = (cue.Irreps("O3", s) for s in (irreps_in1, irreps_in2, irreps_out))
+    m = cuet.FullyConnectedTensorProduct(i1, i2, i3, layout=cue.mul_ir, internal_weights=False)
+    assert m.f_rows is not None
+    g = torch.Generator().manual_seed(Z)
+    w = torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g).to(dtype).double()
+    x1 = torch.randn(Z, i1.dim, dtype=torch.float64, generator=g).to(dtype).double()  # mul_ir rows
+    x2 = torch.randn(Z, i2.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    cot = torch.randn(Z, i3.dim, dtype=torch.float64, generator=g).to(dtype).double()
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+    a = [t.clone().requires_grad_(True) for t in (w, to_ir_mul(x1, i1), x2)]
+    ref = naive_segmented_polynomial(spec, a)[0]
+    ref_gw, ref_gx1, ref_gx2 = torch.autograd.grad(ref, a, to_ir_mul(cot, i3))
+    b = [t.to(dtype).to(device).requires_grad_(True) for t in (w, x1, x2)]
+
+    def step():
+        out = m(b[1], b[2], b[0])
+        return (out, *torch.autograd.grad(out, b, cot.to(dtype).to(device)))
+
+    (out, gw, gx1, gx2), names = kernel_names(step)
+    assert "segmented_transpose" not in names, names
+    tol = TOL[dtype]
+    assert rel_err(out, to_mul_ir(ref, i3)) <= tol
+    assert rel_err(gx1, to_mul_ir(ref_gx1, i1)) <= tol
+    assert rel_err(gx2, ref_gx2) <= tol
+    assert rel_err(gw, ref_gw) <= tol
