@@ -71,6 +71,8 @@ class Uniform1dPlan:
         self.tables = tables
         self.name = name
         self.math_dtype = math_dtype
+        self.widths = tuple(tables.width(b) for b in range(tables.num_inputs + tables.num_outputs))
+        self._configs: dict = {}  # resolved call configurations by call shape
         self._handles: dict[int, int] = {}
         self._backward: dict[tuple, "Uniform1dPlan"] = {}
         self._choice: dict = {}
@@ -237,15 +239,57 @@ def _segment_csr(index: torch.Tensor, nrows: int):
 
 # ---------------------------------------------------------------------- execution
 class _CallConfig:
-    """Resolved batching of one call: per buffer the mode, the index tensor slot and the row count."""
+    """Resolved batching of one call: per buffer the mode, the index tensor slot and the row count.  Also holds what the
+    launches of this call shape reuse: prepared argument records (by dtype signature) and the configurations of its
+    backward calls."""
 
-    __slots__ = ("modes", "index_of", "rows", "batch")
+    __slots__ = ("modes", "index_of", "rows", "batch", "records", "backward")
 
     def __init__(self, modes, index_of, rows, batch):
         self.modes = tuple(modes)
         self.index_of = tuple(index_of)
         self.rows = tuple(rows)
         self.batch = int(batch)
+        self.records: dict = {}
+        self.backward: dict = {}
+
+    def backward_config(self, computed: tuple) -> "_CallConfig":
+        """The configuration of the gradient call for the inputs flagged in ``computed`` (its outputs are their gradients)."""
+        hit = self.backward.get(computed)
+        if hit is None:
+            flagged = [i for i, n in enumerate(computed) if n]
+            hit = self.backward[computed] = _CallConfig(
+                list(self.modes) + [self.modes[i] for i in flagged], list(self.index_of) + [self.index_of[i] for i in flagged],
+                list(self.rows) + [self.rows[i] for i in flagged], self.batch)
+        return hit
+
+
+class _LaunchRecord:
+    """The argument array of ``cueq_u1d_run`` for one call shape and dtype signature, with every field that does not change
+    from call to call filled in once; a launch writes the data / index / grouping pointers only."""
+
+    __slots__ = ("bufs", "proxies", "out_dtypes")
+
+    def __init__(self, plan: "Uniform1dPlan", cfg: _CallConfig, in_dtypes, idx_dtypes):
+        nin, nout = plan.num_inputs, plan.num_outputs
+        self.bufs = (_lib.U1dBuffer * (nin + nout))()
+        self.proxies = [self.bufs[b] for b in range(nin + nout)]  # (one ctypes proxy per buffer, made once)
+        self.out_dtypes = []
+        for b in range(nin + nout):
+            bb = self.proxies[b]
+            if b < nin:
+                dtype = in_dtypes[b]
+                if dtype not in _DTYPE_CODE:
+                    raise ValueError(f"uniform_1d: unsupported dtype {dtype} for input {b}")
+            else:
+                src = plan.dtypes[b]
+                dtype = plan.math_dtype if src < 0 else in_dtypes[src]
+                self.out_dtypes.append(dtype)
+            bb.rows = cfg.rows[b]
+            bb.dtype = _DTYPE_CODE[dtype]
+            bb.batch_dim = cfg.modes[b]
+            if cfg.modes[b] == BATCH_DIM_INDEXED:
+                bb.index_is_64 = 1 if idx_dtypes[cfg.index_of[b]] == torch.int64 else 0
 
 
 class _NoSwitch:
@@ -274,55 +318,53 @@ def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor
         raise RuntimeError("uniform_1d runs on the GPU only; got tensors on " + str(device))
     lib = _lib.load()
     _lib.sync_options_from_env()
+    sig = (tuple([t.dtype for t in inputs]), tuple([i.dtype for i in indices]))
+    pool = cfg.records.get(sig)
+    if pool is None:
+        pool = cfg.records[sig] = []
+    try:
+        rec = pool.pop()  # (a record is used by one launch at a time: list.pop / append are atomic)
+    except IndexError:
+        rec = _LaunchRecord(plan, cfg, sig[0], sig[1])
+    modes, widths = cfg.modes, plan.widths
     with _on_device(device):
-        handle = plan.handle(device)
-        bufs = (_lib.U1dBuffer * (nin + nout))()
+        handle = plan._handles.get(device.index)
+        if handle is None:
+            handle = plan.handle(device)
+        proxies = rec.proxies
         keep = []
         for b in range(nin):
             t = inputs[b]
-            if t.dtype not in _DTYPE_CODE:
-                raise ValueError(f"uniform_1d: unsupported dtype {t.dtype} for input {b}")
-            if t.dim() != 2 or t.shape[1] != plan.width(b):
-                raise ValueError(f"uniform_1d: input {b} has shape {tuple(t.shape)}, expected (rows, {plan.width(b)})")
+            if t.dim() != 2 or t.shape[1] != widths[b]:
+                raise ValueError(f"uniform_1d: input {b} has shape {tuple(t.shape)}, expected (rows, {widths[b]})")
             if not t.is_contiguous():
                 t = t.contiguous()
-            keep.append(t)
-            bb = bufs[b]  # (one ctypes proxy per buffer, not one per field)
+                keep.append(t)
+            bb = proxies[b]
             bb.data = t.data_ptr()
-            bb.rows = t.shape[0]
-            bb.dtype = _DTYPE_CODE[t.dtype]
-            bb.batch_dim = cfg.modes[b]
-            if cfg.modes[b] == BATCH_DIM_INDEXED:
-                idx = indices[cfg.index_of[b]]
-                bb.index = idx.data_ptr()
-                bb.index_is_64 = 1 if idx.dtype == torch.int64 else 0
+            if modes[b] == BATCH_DIM_INDEXED:
+                bb.index = indices[cfg.index_of[b]].data_ptr()
         outputs = []
         for o in range(nout):
             b = nin + o
-            src = plan.dtypes[b]
-            dtype = plan.math_dtype if src < 0 else inputs[src].dtype
-            out = torch.empty((cfg.rows[b], plan.width(b)), dtype=dtype, device=device)
+            out = torch.empty((cfg.rows[b], widths[b]), dtype=rec.out_dtypes[o], device=device)
             outputs.append(out)
-            bb = bufs[b]
+            bb = proxies[b]
             bb.data = out.data_ptr()
-            bb.rows = out.shape[0]
-            bb.dtype = _DTYPE_CODE[dtype]
-            bb.batch_dim = cfg.modes[b]
-            if cfg.modes[b] == BATCH_DIM_INDEXED:
+            if modes[b] == BATCH_DIM_INDEXED:
                 idx = indices[cfg.index_of[b]]
                 bb.index = idx.data_ptr()
-                bb.index_is_64 = 1 if idx.dtype == torch.int64 else 0
                 offsets, perm = _segment_csr(idx, cfg.rows[b])
                 keep += [offsets, perm]
                 bb.csr_offsets = offsets.data_ptr()
                 bb.csr_perm = perm.data_ptr()
-        ws_bytes = lib.cueq_u1d_workspace_size(handle, bufs, cfg.batch)
+        ws_bytes = lib.cueq_u1d_workspace_size(handle, rec.bufs, cfg.batch)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=device) if ws_bytes > 0 else None
         stream = torch._C._cuda_getCurrentRawStream(device.index if device.index is not None else torch.cuda.current_device())
-        _lib.check(
-            lib.cueq_u1d_run(handle, bufs, cfg.batch, ws.data_ptr() if ws is not None else None, ws_bytes, stream),
-            f"cueq_u1d_run[{plan.name}]",
-        )
+        status = lib.cueq_u1d_run(handle, rec.bufs, cfg.batch, ws.data_ptr() if ws is not None else None, ws_bytes, stream)
+        if status != 0:
+            _lib.check(status, f"cueq_u1d_run[{plan.name}]")
+    pool.append(rec)
     return outputs
 
 
@@ -355,11 +397,11 @@ class _Uniform1dFunction(torch.autograd.Function):
                                 dtype=plan.math_dtype if src < 0 else inputs[src].dtype)
             cots.append(g)
         flagged = [i for i, n in enumerate(computed) if n]
-        modes = list(cfg.modes) + [cfg.modes[i] for i in flagged]
-        index_of = list(cfg.index_of) + [cfg.index_of[i] for i in flagged]
-        rows = list(cfg.rows) + [cfg.rows[i] for i in flagged]
-        bcfg = _CallConfig(modes, index_of, rows, cfg.batch)
-        grads = _Uniform1dFunction.apply(bplan, bcfg, num_index, *inputs, *cots, *indices)
+        bcfg = cfg.backward_config(computed)
+        if torch.is_grad_enabled():  # (create_graph: the gradient call is recorded, derivatives of any order)
+            grads = _Uniform1dFunction.apply(bplan, bcfg, num_index, *inputs, *cots, *indices)
+        else:
+            grads = _launch(bplan, bcfg, [t.detach() for t in inputs] + cots, indices)
         out = [None, None, None] + [None] * len(tensors)
         for g, i in zip(grads, flagged):
             if needs[i]:
@@ -438,7 +480,13 @@ def run_plan(plan: Uniform1dPlan, batch_dim: Sequence[int], index_buffer: Sequen
     for k, idx in enumerate(indices):
         if idx.dtype not in (torch.int32, torch.int64) or idx.dim() != 1:
             raise ValueError(f"uniform_1d: index tensor {k} must be a 1-D int32/int64 tensor")
-        indices[k] = idx.contiguous()
+        if not idx.is_contiguous():
+            indices[k] = idx.contiguous()
+    # the resolution below depends on these numbers only: resolved once per call shape
+    key = (tuple(batch_dim), tuple(index_buffer), batch_size, tuple([t.shape[0] for t in inputs]), tuple([i.shape[0] for i in indices]))
+    cfg = plan._configs.get(key) if not torch.compiler.is_compiling() else None
+    if cfg is not None and inputs and type(inputs[0]) in _PLAIN_TENSORS:
+        return list(_Uniform1dFunction.apply(plan, cfg, num_index, *inputs, *indices))
     modes = list(batch_dim)
     batch = batch_size
     # batch size: the common length of index tensors and of batched (multi-row) inputs
@@ -476,6 +524,9 @@ def run_plan(plan: Uniform1dPlan, batch_dim: Sequence[int], index_buffer: Sequen
     if torch.compiler.is_compiling() or (inputs and type(inputs[0]) not in _PLAIN_TENSORS):
         return list(_u1d_launch_op(plan.traced_id, modes, list(index_buffer[: nin + nout]), rows, batch, [*inputs, *indices]))
     cfg = _CallConfig(modes, list(index_buffer[: nin + nout]), rows, batch)
+    if len(plan._configs) >= 64:  # (call shapes of a module are few; a stream of ever new batch sizes starts over)
+        plan._configs.clear()
+    plan._configs[key] = cfg
     outs = _Uniform1dFunction.apply(plan, cfg, num_index, *inputs, *indices)
     return list(outs)
 
