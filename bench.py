@@ -353,7 +353,7 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
     }
 
 
-def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, warmup: int, deterministic: bool):
+def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, warmup: int, deterministic: bool, fresh_indices: bool = False):
     """The headline workload once; returns (JSON line, module, host inputs)."""
     prev = os.environ.get("CUEQ_DETERMINISTIC")
     os.environ["CUEQ_DETERMINISTIC"] = "1" if deterministic else "0"
@@ -367,7 +367,10 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
         node.requires_grad_(True), sh.requires_grad_(True), w.requires_grad_(True)
 
         def step():
-            out = m(node, sh, w, indices_1=senders, indices_out=receivers, size_out=N)
+            # fresh_indices: a new receiver tensor every step (a neighbour list that changes with every MD step): the grouping
+            # of edges by receiver is built again instead of taken from the cache
+            rcv = receivers.clone() if fresh_indices else receivers
+            out = m(node, sh, w, indices_1=senders, indices_out=rcv, size_out=N)
             return torch.autograd.grad(out, [w, node, sh], cot)
 
         for _ in range(warmup):
@@ -440,6 +443,69 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
         "kernels": per_kernel,
     }
     return line, m, host
+
+
+def setup_costs(torch, cue, cuet, _lib, dev, N: int, E: int, compile_probe: bool) -> dict:
+    """What a user pays before / around the timed steps of the headline workload: building the module (descriptor and
+    path tables, on the host), creating the device plans of forward and backward, grouping the edges by receiver (built once
+    per index tensor in eager mode and cached; measured for sorted and for shuffled receivers), and - for a descriptor the
+    library was not built for - compiling its kernels at first use."""
+    import tempfile
+
+    out = {}
+    t0 = time.perf_counter()
+    m = cuet.ChannelWiseTensorProduct(cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "0e+1o+2e+3o"), "0e+1o+2e+3o",
+                                      layout=cue.ir_mul, shared_weights=False)
+    out["module_build_ms"] = (time.perf_counter() - t0) * 1e3
+    plan = m.f.m._plan(torch.float32)
+    t0 = time.perf_counter()
+    plan.handle(dev)
+    plan.backward_plan((True, True, True)).handle(dev)
+    torch.cuda.synchronize()
+    out["plan_create_ms"] = (time.perf_counter() - t0) * 1e3
+    import importlib
+
+    u1d = importlib.import_module("cuequivariance_amd.cuet.uniform_1d")  # (the package also exports a function of this name)
+
+    g = torch.Generator().manual_seed(1)
+    sorted_ids = torch.sort(torch.randint(0, N, (E,), generator=g, dtype=torch.int32))[0].to(dev)
+    shuffled = sorted_ids[torch.randperm(E, generator=g).to(dev)].contiguous()
+    for name, ids in (("csr_build_ms_sorted_receivers", sorted_ids), ("csr_build_ms_unsorted_receivers", shuffled)):
+        times = []
+        for _ in range(5):
+            fresh = ids.clone()  # (a new tensor: the cache of groupings misses)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            u1d._segment_csr(fresh, N)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        out[name] = sorted(times)[len(times) // 2]
+    if compile_probe:
+        # a channel-wise product the library holds no kernels for (64 channels, l <= 3), compiled into an empty cache
+        from cuequivariance_amd import jit
+
+        prev = os.environ.get("CUEQ_AMD_JIT_CACHE")
+        try:
+            with tempfile.TemporaryDirectory() as tmp:
+                os.environ["CUEQ_AMD_JIT_CACHE"] = tmp
+                if jit.enabled():
+                    mm = cuet.ChannelWiseTensorProduct(cue.Irreps("O3", "64x0e+64x1o+64x2e+64x3o"), cue.Irreps("O3", "0e+1o+2e+3o"),
+                                                       "0e+1o+2e+3o", layout=cue.ir_mul, shared_weights=False)
+                    t0 = time.perf_counter()
+                    p2 = mm.f.m._plan(torch.float32)
+                    p2.handle(dev)
+                    p2.backward_plan((True, True, True)).handle(dev)
+                    out["first_use_compile_s"] = time.perf_counter() - t0
+                    out["first_use_compile_descriptor"] = "channel-wise 64x(0e+1o+2e+3o) x (0e+1o+2e+3o), forward + backward unit, hipcc -O3 for gfx950"
+        except Exception as e:  # (no compiler on the box, cache not writable: the table-driven kernels would run)
+            out["first_use_compile_s"] = None
+            out["first_use_compile_error"] = f"{type(e).__name__}: {e}"
+        finally:
+            if prev is None:
+                os.environ.pop("CUEQ_AMD_JIT_CACHE", None)
+            else:
+                os.environ["CUEQ_AMD_JIT_CACHE"] = prev
+    return out
 
 
 def cpu_baseline_dense(torch, cue, wl: str, threads: int) -> dict:
@@ -518,6 +584,7 @@ def main() -> int:
     ap.add_argument("--cpu-sample-edges", type=int, default=12000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="headline line only (no 'secondary' object)")
+    ap.add_argument("--no-setup-costs", action="store_true", help="leave out the 'setup' object (module build, plan creation, edge grouping, first-use compilation)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (default: the box's share, at most 16)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy a few times (to scale rocprofv3 FETCH_SIZE/WRITE_SIZE)")
@@ -604,12 +671,21 @@ def main() -> int:
 
         add("cfg2_fp32_ordered_dx1", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float32, N, E, ssteps, swarm, True)[0]))
         add("cfg2_fp64", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float64, N, E, ssteps, swarm, False)[0]))
+        add("cfg2_fp32_grouping_rebuilt_every_step",
+            lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float32, N, E, ssteps, swarm, False, fresh_indices=True)[0]))
         for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg4_linear_fp32", "cfg4", "fp32"),
                             ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_linear_fp32_mul_ir", "cfg4mi", "fp32"),
                             ("cfg4_linear_bf16_mul_ir", "cfg4mi", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("cfg4_fc_fp32_mul_ir", "cfg4fcmi", "fp32"),
                             ("cfg4_fc_bf16_mul_ir", "cfg4fcmi", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
                             ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp32", "cfg5", "fp32")):
             add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))
+            if key in ("cfg1_fp32", "cfg4_fc_bf16", "cfg4_fc_bf16_mul_ir") and "error" not in sec[key]:
+                # workloads whose eager step is bound by the host's launch path: the same step replayed as one HIP graph
+                try:
+                    sec[key]["graph_ms_per_step"] = secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm, graph=True)["ms_per_step"]
+                except Exception as e:
+                    sec[key]["graph_ms_per_step"] = None
+                    sec[key]["graph_error"] = f"{type(e).__name__}: {e}"
         if not args.no_cpu_baseline:
             # more CPU baselines (the oracle on this box's host cores, bounded samples): the headline workload on one
             # thread, the dense workloads on the box's share of cores
@@ -622,6 +698,11 @@ def main() -> int:
                 "cfg5_fp32": cpu_baseline_dense(torch, cue, "cfg5", args.cpu_threads),
             }
         line["secondary"] = sec
+    if args.workload is None and not args.no_setup_costs:
+        try:
+            line["setup"] = setup_costs(torch, cue, cuet, _lib, dev, N, E, compile_probe=full)
+        except Exception as e:
+            line["setup"] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line))
     return 0
 

@@ -822,8 +822,8 @@ class _FcFunction(torch.autograd.Function):
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             code, es = _DTYPE_CODE[dtype], x1d.element_size()
-            tables = plan.device(dev)
             unit = unit_w = mod.fused_unit(dtype, x1d, g) if Z > 0 else None
+            tables = plan.device(dev) if unit is None else None  # (the fused kernels carry their tables in their code)
             if unit is None and mod.rows_mul_ir and Z > 0:
                 raise NotImplementedError("fused_tp: rows='mul_ir' needs the generated fused kernels")
             if need_x1:  # (the generated kernels write every column)
@@ -854,14 +854,20 @@ class _FcFunction(torch.autograd.Function):
                                                   1 if plan.dx2_vec else 0, stream), "cueq_fc_rowdot")
             if unit_w is not None and need_w:
                 # per-block partial sums of the generated kernel (x1^T H with H formed in registers), then a row sum
-                nblocks, numel = unit_w.fcj_dw_blocks(Z), wd.numel()
-                covered = sum(K * N for _, K, N in mod.weight_blocks) == numel
+                numel = wd.numel()
+                shape = mod._dw_shapes.get((Z, dtype))  # (chunk count and row-sum workspace: two library calls per batch size)
+                if shape is None:
+                    nb = unit_w.fcj_dw_blocks(Z)
+                    if len(mod._dw_shapes) >= 64:
+                        mod._dw_shapes.clear()
+                    shape = mod._dw_shapes[(Z, dtype)] = (nb, lib.cueq_sum_rows_workspace(nb, numel),
+                                                          sum(K * N for _, K, N in mod.weight_blocks) == numel)
+                nblocks, ws_bytes, covered = shape
                 part = (torch.empty if covered else torch.zeros)(nblocks, numel, dtype=torch.float32, device=dev)
                 if unit_w.fcj_dw(Z, x1d.data_ptr(), x1d.stride(0), x2d.data_ptr(), x2d.stride(0), g.data_ptr(), g.stride(0),
                                  part.data_ptr(), numel, stream) != 0:
                     raise RuntimeError("fused fully connected weight gradient: launch failed")
                 gw32 = torch.empty(numel, dtype=torch.float32, device=dev)
-                ws_bytes = lib.cueq_sum_rows_workspace(nblocks, numel)
                 ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
                 _lib.check(lib.cueq_sum_rows(_lib.F32, nblocks, numel, part.data_ptr(), gw32.data_ptr(), ws.data_ptr(), ws_bytes, stream),
                            "cueq_sum_rows")
@@ -1216,6 +1222,7 @@ class SegmentedPolynomialDense(nn.Module):
         self.fc_plan = _FcPlan(self.paths, self.input_sizes[2]) if self.has_x2 else None
         self._merged: dict = {}
         self._fused: dict = {}
+        self._dw_shapes: dict = {}
         # rows="mul_ir": the irreps operands (input 1 and the output of the 3-operand form) keep the component index
         # contiguous inside every block; the kernels address them so - no transposition pass around the call.  Not part of
         # the reference's interface.  `mul_ir` is None when the blocks do not have the shape those kernels take.

@@ -85,6 +85,64 @@ def test_fully_connected_matches_oracle(device, dtype):
     check_against_oracle(device, m, [w, x1, x2], dtype)
 
 
+@pytest.mark.parametrize("layout", [cue.ir_mul, cue.mul_ir])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fully_connected_benchmark_size(device, dtype, layout):
+    """At the benchmark's size (50 000 rows, 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o): rows drawn from all over the batch
+    (the first, the last and those of the last, partly filled tile among them) against the float64 oracle, outputs and
+    gradients of the row operands; the weight gradient and the sums over the whole batch through the identities
+    <dy, y> = <dL/dw, w> = <dL/dx1, x1> = <dL/dx2, x2> that a product linear in each operand obeys."""
+    from cuequivariance_amd import cuet
+
+    m = cuet.FullyConnectedTensorProduct(
+        cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e"), cue.Irreps("O3", "64x0e+64x1o"),
+        layout=layout, internal_weights=False,
+    )
+    Z = 50_000
+    g = torch.Generator().manual_seed(11)
+    w = (0.2 * torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g)).to(dtype)
+    x1 = torch.randn(Z, 256, dtype=torch.float64, generator=g).to(dtype)
+    x2 = torch.randn(Z, 9, dtype=torch.float64, generator=g).to(dtype)
+    cot = torch.randn(Z, 256, dtype=torch.float64, generator=g).to(dtype)
+    a = [t.to(device).requires_grad_(True) for t in (w, x1, x2)]
+    y = m(a[1], a[2], a[0])
+    assert y.dtype == dtype and y.shape == (Z, 256)
+    gw, g1, g2 = torch.autograd.grad(y, a, cot.to(device))
+    rows = torch.cat([torch.arange(0, 40), torch.randint(0, Z, (200,), generator=g), torch.arange(Z - 40, Z)])
+    b = [w.double().requires_grad_(True), x1[rows].double().requires_grad_(True), x2[rows].double().requires_grad_(True)]
+    spec = spec_from_polynomial(m.f._polynomial_orig)
+    if layout == cue.mul_ir:  # the oracle's polynomial is written for ir_mul rows: turn the sampled rows
+        def to_ir_mul(t, irreps):
+            return torch.cat([t[:, o:o + mul * ir.dim].reshape(-1, mul, ir.dim).transpose(1, 2).reshape(len(t), -1)
+                              for o, (mul, ir) in zip(_starts(irreps), irreps)], 1)
+
+        def to_mul_ir(t, irreps):
+            return torch.cat([t[:, o:o + mul * ir.dim].reshape(-1, ir.dim, mul).transpose(1, 2).reshape(len(t), -1)
+                              for o, (mul, ir) in zip(_starts(irreps), irreps)], 1)
+    else:
+        to_ir_mul = to_mul_ir = lambda t, irreps: t
+    ref = naive_segmented_polynomial(spec, [b[0], to_ir_mul(b[1], m.irreps_in1), b[2]])[0]
+    ref_rows = to_mul_ir(ref, m.irreps_out)
+    r1, r2 = torch.autograd.grad(ref_rows, b[1:], cot[rows].double())
+    tol = TOL[dtype]
+    assert rel_err(y[rows.to(device)], ref_rows) <= tol
+    assert rel_err(g1[rows.to(device)], r1) <= tol
+    assert rel_err(g2[rows.to(device)], r2) <= tol
+    lhs = (cot.double().to(device) * y.detach().double()).sum().item()
+    scale = (cot.double().to(device) * y.detach().double()).abs().sum().item()
+    slack = (3e-6 if dtype == torch.float32 else 2e-3) * scale / Z ** 0.5 * 30
+    for grad, operand in zip((gw, g1, g2), a):
+        assert abs((grad.double() * operand.detach().double()).sum().item() - lhs) <= slack, (grad.shape, lhs, slack)
+
+
+def _starts(irreps):
+    out, off = [], 0
+    for mul, ir in irreps:
+        out.append(off)
+        off += mul * ir.dim
+    return out
+
+
 def test_linear_module_call_and_internal_weights(device):
     """The module call path (x, weight) and internal weights give what the functional core gives."""
     from cuequivariance_amd import cuet
