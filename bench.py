@@ -148,25 +148,27 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
                 "fwd + bwd (dx1, dx2, dw); 69 MB of traffic: launch-latency regime")
     elif wl == "cfg3":
         Z = 50_000
+        dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32  # (bf16: the buffers; the arithmetic stays float32)
         m = cuet.SymmetricContraction(cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "128x0e+128x1o"),
-                                      3, 10, layout=cue.ir_mul, dtype=torch.float32, device=dev)
+                                      3, 10, layout=cue.ir_mul, dtype=dtype, device=dev)
         g = torch.Generator(device=dev).manual_seed(0)
-        x = torch.randn(Z, 2048, device=dev, generator=g, requires_grad=True)
+        x = torch.randn(Z, 2048, device=dev, generator=g).to(dtype).requires_grad_(True)
         idx = torch.randint(0, 10, (Z,), device=dev, generator=g, dtype=torch.int32)
         with torch.no_grad():
             m.weight.mul_(1.0 / m.weight.shape[1] ** 0.5)
-        cot = torch.randn(Z, 512, device=dev, generator=g)
+        cot = torch.randn(Z, 512, device=dev, generator=g).to(dtype)
 
         def step():
             return torch.autograd.grad(m(x, idx), [m.weight, x], cot)
 
         unit, units, dt = "nodes/s", Z, "f32"
         # every distinct element once: fwd reads x and writes out; bwd reads x, g and writes dx (weights 10 x 3712 negligible)
-        alg = {"fwd": Z * (2048 + 512) * 4, "bwd": Z * (2048 + 512 + 2048) * 4}
+        es = x.element_size()
+        alg = {"fwd": Z * (2048 + 512) * es, "bwd": Z * (2048 + 512 + 2048) * es}
         flops = {k: Z * n * 128 for k, n in zip(("fwd", "bwd"), VALU_INSTS_PER_ELEMENT["cfg3"])}  # executed vector instructions x 128
         flop_roof, flop_peak = "valu", VALU_PEAK_F32
         desc = ("configs[2]: symmetric contraction 128x(0e+1o+2e+3o) -> 128x(0e+1o), degree 3, 10 element types, "
-                "50000 nodes, int32 element index, fwd + bwd (dw, dx)")
+                "50000 nodes, int32 element index, fwd + bwd (dw, dx)" + ("; buffers of bfloat16, arithmetic in float32" if es == 2 else ""))
     elif wl in ("cfg4", "cfg4mi"):
         Z = 200_000
         dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
@@ -391,9 +393,9 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
     ms_per_step = elapsed / steps * 1e3
     value = E / (elapsed / steps)
 
-    plan = m.f.m._plan(dtype)
-    specialised = bool(plan.specialised(dev) and plan.backward_plan((True, True, True)).specialised(dev))
-    s = 4 if dtype == torch.float32 else 8
+    plan = m.f.m._plan(torch.float64 if dtype == torch.float64 else torch.float32)
+    specialised = bool(plan.serves(dtype) and plan.backward_plan((True, True, True)).serves(dtype))
+    s = {torch.float32: 4, torch.float64: 8, torch.bfloat16: 2}[dtype]
     alg = algorithmic_bytes(E, N, 2944, 2048, 16, 12672, s)
     per_kernel = {}
     for name, (launches, total_ms) in kernels.items():
@@ -427,18 +429,19 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if dtype == torch.float32 else "f64",
+        "dtype": "f64" if dtype == torch.float64 else "f32",
         "data": "synthetic",
         "config": {
             "workload": "configs[1]: MACE-style indexed channel-wise TP, 5000 nodes x 128x0e+128x1o+128x2e+128x3o, "
                         "100000 edges x SH 0e+1o+2e+3o, per-edge weights [E,2944], int32 sender/receiver (receivers "
                         "sorted), scatter-sum onto 5000 nodes, fwd + bwd (dw, dx1, dx2)",
             "nodes": N, "edges": E, "specialised_kernels": specialised,
+            "buffers": {torch.float32: "f32", torch.float64: "f64", torch.bfloat16: "bf16 (arithmetic in f32)"}[dtype],
             "dx1_scatter": "ordered" if deterministic else "fp-atomics",
         },
         "roofline": roofline,
         "step_roofline_frac": (total_alg / (elapsed / steps)) / 1e9 / HBM_PEAK_GBS,
-        "step_valu_frac": valu_flops / (elapsed / steps) / 1e12 / (VALU_PEAK_F32 if dtype == torch.float32 else 78.6),
+        "step_valu_frac": valu_flops / (elapsed / steps) / 1e12 / (78.6 if dtype == torch.float64 else VALU_PEAK_F32),
         "valu_source": VALU_SOURCE,
         "kernels": per_kernel,
     }
@@ -647,10 +650,8 @@ def main() -> int:
     if args.workload not in (None, "cfg2"):
         print(json.dumps(secondary(torch, cue, cuet, _lib, dev, args.workload, args.dtype, args.steps, args.warmup, args.graph)))
         return 0
-    if args.dtype == "bf16":
-        print("bench.py: cfg2 is measured in fp32 or fp64 (the uniform-1d math types)", file=sys.stderr)
-        return 2
-    dtype = torch.float64 if args.dtype == "fp64" else torch.float32
+    # (bf16: buffers of bfloat16, arithmetic in float32 - a secondary measurement, the headline is float32 throughout)
+    dtype = {"fp64": torch.float64, "bf16": torch.bfloat16}.get(args.dtype, torch.float32)
     N, E = args.nodes, args.edges
     line, m, host = run_cfg2(torch, cue, cuet, _lib, dev, dtype, N, E, args.steps, args.warmup, args.deterministic)
     full = args.workload is None and not args.no_secondary
@@ -671,9 +672,10 @@ def main() -> int:
 
         add("cfg2_fp32_ordered_dx1", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float32, N, E, ssteps, swarm, True)[0]))
         add("cfg2_fp64", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float64, N, E, ssteps, swarm, False)[0]))
+        add("cfg2_bf16_io", lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.bfloat16, N, E, ssteps, swarm, False)[0]))
         add("cfg2_fp32_grouping_rebuilt_every_step",
             lambda: _cfg2_compact(run_cfg2(torch, cue, cuet, _lib, dev, torch.float32, N, E, ssteps, swarm, False, fresh_indices=True)[0]))
-        for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg4_linear_fp32", "cfg4", "fp32"),
+        for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg3_bf16_io", "cfg3", "bf16"), ("cfg4_linear_fp32", "cfg4", "fp32"),
                             ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_linear_fp32_mul_ir", "cfg4mi", "fp32"),
                             ("cfg4_linear_bf16_mul_ir", "cfg4mi", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("cfg4_fc_fp32_mul_ir", "cfg4fcmi", "fp32"),
                             ("cfg4_fc_bf16_mul_ir", "cfg4fcmi", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
@@ -710,7 +712,8 @@ def main() -> int:
 def _cfg2_compact(line: dict) -> dict:
     return {"ms_per_step": line["ms_per_step"], "value": line["value"], "unit": line["unit"], "dtype": line["dtype"],
             "bound": "hbm", "frac": line["step_roofline_frac"], "hbm_frac": line["step_roofline_frac"],
-            "valu_frac": line["step_valu_frac"], "dx1_scatter": line["config"]["dx1_scatter"],
+            "valu_frac": line["step_valu_frac"], "dx1_scatter": line["config"]["dx1_scatter"], "buffers": line["config"]["buffers"],
+            "specialised_kernels": line["config"]["specialised_kernels"],
             "kernels_avg_ms": {k: v["avg_ms"] for k, v in line["kernels"].items()}, "workload": line["config"]["workload"]}
 
 

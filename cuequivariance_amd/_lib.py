@@ -32,6 +32,7 @@ EXPORTED_SYMBOLS = (
     "cueq_u1d_plan_destroy",
     "cueq_u1d_plan_info",
     "cueq_u1d_desc_info",
+    "cueq_u1d_desc_serves",
     "cueq_u1d_workspace_size",
     "cueq_u1d_run",
     "cueq_u1d_static_scratch_bytes",
@@ -168,6 +169,8 @@ def load() -> C.CDLL:
         lib.cueq_u1d_plan_info.restype = C.c_int
         lib.cueq_u1d_desc_info.argtypes = [C.POINTER(U1dDesc), C.POINTER(C.c_uint64)]
         lib.cueq_u1d_desc_info.restype = C.c_int
+        lib.cueq_u1d_desc_serves.argtypes = [C.POINTER(U1dDesc), C.c_int32]
+        lib.cueq_u1d_desc_serves.restype = C.c_int
         lib.cueq_u1d_workspace_size.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64]
         lib.cueq_u1d_workspace_size.restype = C.c_int64
         lib.cueq_u1d_run.argtypes = [C.c_void_p, C.POINTER(U1dBuffer), C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]

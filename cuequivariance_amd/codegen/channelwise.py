@@ -293,19 +293,19 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
             A(f"{ind}  const int64_t z = csr_perm ? csr_perm[{zz}] : ({zz});")
             A(f"{ind}  int64_t srow = z;")
             A(f"{ind}  if (X1_IDX) srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
-            A(f"{ind}  const {fp}* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
-            A(f"{ind}  const {fp}* __restrict__ wp = w + (W_SHARED ? 0 : z * {st.nseg_w * st.extent}ll);")
-            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.x2_width}ll;")
+            A(f"{ind}  const TI* __restrict__ x1p = x1 + srow * {st.nseg_x1 * st.extent}ll;")
+            A(f"{ind}  const TI* __restrict__ wp = w + (W_SHARED ? 0 : z * {st.nseg_w * st.extent}ll);")
+            A(f"{ind}  const TI* __restrict__ x2p = x2 + z * {st.x2_width}ll;")
             if st.harmonics:
                 for a in range(3):
-                    A(f"{ind}  {S}_v{a} = x2p[{a}];")
+                    A(f"{ind}  {S}_v{a} = io_ld(x2p + {a});")
             for m in ([] if st.harmonics else ms):
                 nvalid = min(16, st.nseg_x2 - 16 * m)
-                A(f"{ind}  {S}_yv{m} = x2p[{16 * m} + (n16 < {nvalid} ? n16 : 0)];")
+                A(f"{ind}  {S}_yv{m} = io_ld(x2p + {16 * m} + (n16 < {nvalid} ? n16 : 0));")
             for i in i_used:
-                A(f"{ind}  {S}_xv{i} = x1p[{st.x1_at(i)}];")
+                A(f"{ind}  {S}_xv{i} = io_ld(x1p + ({st.x1_at(i)}));")
             for blk in blocks:
-                A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
+                A(f"{ind}  {S}_wv{blk.b} = io_ldnt(wp + {blk.b * st.extent} + uu);")
             A(f"{ind}}}")
 
         def body(S: str, ind: str):
@@ -372,9 +372,9 @@ def emit_forward(st: ChannelwiseStructure, T: str, nsplit: int, waves_per_eu: in
             body("a", "    ")
             A("  }")
         A("  if (active) {")
-        A(f"    {fp}* __restrict__ op = out + r * {st.nseg_out * st.extent}ll;")
+        A(f"    TI* __restrict__ op = out + r * {st.nseg_out * st.extent}ll;")
         for k in ks:
-            A(f"    STREAM_STORE(acc{k}, op + {st.out_at(k)});")
+            A(f"    io_stnt(acc{k}, op + ({st.out_at(k)}));")
         A("  }")
         A("}")
         A("")
@@ -456,16 +456,16 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
             A(f"{ind}  if (G_IDX) {S}_grow = g_idx64 ? static_cast<const int64_t*>(g_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(g_index)[z]);")
             A(f"{ind}  {S}_srow = z;")
             A(f"{ind}  if (X1_IDX) {S}_srow = x1_idx64 ? static_cast<const int64_t*>(x1_index)[z] : static_cast<int64_t>(static_cast<const int32_t*>(x1_index)[z]);")
-            A(f"{ind}  const {fp}* __restrict__ x1p = x1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
-            A(f"{ind}  const {fp}* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
-            A(f"{ind}  const {fp}* __restrict__ x2p = x2 + z * {st.x2_width}ll;")
+            A(f"{ind}  const TI* __restrict__ x1p = x1 + {S}_srow * {st.nseg_x1 * st.extent}ll;")
+            A(f"{ind}  const TI* __restrict__ wp = w + z * {st.nseg_w * st.extent}ll;")
+            A(f"{ind}  const TI* __restrict__ x2p = x2 + z * {st.x2_width}ll;")
             if st.harmonics:  # (requested first: the harmonics below wait for these three only)
                 for a in range(3):
-                    A(f"{ind}  {S}_v{a} = x2p[{a}];")
+                    A(f"{ind}  {S}_v{a} = io_ld(x2p + {a});")
             for i in i_used:
-                A(f"{ind}  {S}_xv{i} = x1p[{st.x1_at(i)}];")
+                A(f"{ind}  {S}_xv{i} = io_ld(x1p + ({st.x1_at(i)}));")
             for blk in blocks:
-                A(f"{ind}  {S}_wv{blk.b} = STREAM_LOAD(wp + {blk.b * st.extent} + uu);")
+                A(f"{ind}  {S}_wv{blk.b} = io_ldnt(wp + {blk.b * st.extent} + uu);")
             if st.harmonics:
                 A(f"{ind}  {{")
                 need = sorted({vi for j in j_used for vi, _ in st.harmonics[j]}, key=lambda t: (len(t), t))
@@ -477,18 +477,18 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
                     A(f"{ind}    {S}_yv{j} = {expr if expr is not None else '0'};")
                 A(f"{ind}  }}")
             for j in ([] if st.harmonics else j_used):
-                A(f"{ind}  {S}_yv{j} = x2p[{j}];")
+                A(f"{ind}  {S}_yv{j} = io_ld(x2p + {j});")
             A(f"{ind}}}")
 
         def body(S: str, zz: str, ind: str):
             A(f"{ind}const int64_t z = {zz};")
             A(f"{ind}if ({S}_grow != grow_cur) {{")
             A(f"{ind}  grow_cur = {S}_grow;")
-            A(f"{ind}  const {fp}* __restrict__ gp = g + grow_cur * {st.nseg_out * st.extent}ll;")
+            A(f"{ind}  const TI* __restrict__ gp = g + grow_cur * {st.nseg_out * st.extent}ll;")
             for k in ks:
-                A(f"{ind}  gr{k} = STREAM_LOAD(gp + {st.out_at(k)});")
+                A(f"{ind}  gr{k} = io_ldnt(gp + ({st.out_at(k)}));")
             A(f"{ind}}}")
-            A(f"{ind}{fp}* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
+            A(f"{ind}TI* __restrict__ dwp = dw + z * {st.nseg_w * st.extent}ll;")
             for i in i_used:
                 A(f"{ind}{fp} dxa{i} = 0;")
             for j in j_used:
@@ -515,13 +515,13 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
                         A(f"{ind}    {{ const {fp} G = {expr}; D = fma(G, {S}_yv{j}, D); F{j} = fma(G, {S}_xv{i}, F{j}); }}")
                     A(f"{ind}    dwb = fma({S}_xv{i}, D, dwb); dxa{i} = fma(wb, D, dxa{i});")
                     A(f"{ind}  }}")
-                A(f"{ind}  if (active) STREAM_STORE(dwb, dwp + {blk.b * st.extent} + uu);")
+                A(f"{ind}  if (active) io_stnt(dwb, dwp + {blk.b * st.extent} + uu);")
                 for j in blk.j_list:
                     A(f"{ind}  pj{j} = fma(wb, F{j}, pj{j});")
                 A(f"{ind}}}")
                 A(f"{ind}__builtin_amdgcn_sched_barrier(0);")
             for b_ in w_zero:
-                A(f"{ind}if (active) STREAM_STORE({fp}(0), dwp + {b_ * st.extent} + uu);")
+                A(f"{ind}if (active) io_stnt({fp}(0), dwp + {b_ * st.extent} + uu);")
             # dx1: scatter.  Atomic adds are served per touched 32-byte sector, not per element: the components of a
             # channel-major group (a stride of d elements between lanes) go through LDS first, so that every atomic
             # instruction of the wavefront covers 64 consecutive elements as it does in the default layout.
@@ -543,9 +543,9 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
                 if i not in staged_segments:
                     A(f"{ind}    unsafeAtomicAdd(dp + ({st.x1_at(i)}), dxa{i});")
             A(f"{ind}  }} else {{")
-            A(f"{ind}    {fp}* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
+            A(f"{ind}    TI* __restrict__ dp = dx1_partial + z * {st.nseg_x1 * st.extent}ll;")
             for i in sorted(i_used + i_zero):
-                A(f"{ind}    dp[{st.x1_at(i)}] = " + (f"dxa{i};" if i in i_used else "0;"))
+                A(f"{ind}    io_st(" + (f"dxa{i}" if i in i_used else f"{fp}(0)") + f", dp + ({st.x1_at(i)}));")
             A(f"{ind}  }}")
             A(f"{ind}}}")
             # dx2: reduce over the 64 lanes; channel chunks and wavefronts of one batch row are folded afterwards
@@ -573,15 +573,15 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
                 A(f"{ind}}}")
             A(f"{ind}if (lane == 0) {{")
             if nparts == 1:
-                A(f"{ind}  {fp}* __restrict__ d2 = dx2 + z * {st.x2_width}ll;")
+                A(f"{ind}  TI* __restrict__ d2 = dx2 + z * {st.x2_width}ll;")
             else:
                 A(f"{ind}  {fp}* __restrict__ d2 = dx2_partial + (z * {nparts} + ch * {nsplit} + {q}) * {st.x2_width}ll;")
             if st.harmonics:
                 for a in range(3):
-                    A(f"{ind}  d2[{a}] = dv{a};")
+                    A(f"{ind}  io_st(dv{a}, d2 + {a});")
             else:
                 for j in range(st.nseg_x2):
-                    A(f"{ind}  d2[{j}] = " + (f"pj{j};" if j in j_used else "0;"))
+                    A(f"{ind}  io_st(" + (f"pj{j}" if j in j_used else f"{fp}(0)") + f", d2 + {j});")
             A(f"{ind}}}")
 
         A("template <bool X1_IDX, bool G_IDX, bool ATOMIC_DX1>")
@@ -653,22 +653,38 @@ def emit_backward(st: ChannelwiseStructure, T: str, waves_per_eu: int, chunk: in
 # ---------------------------------------------------------------------------------------------
 # translation unit
 # ---------------------------------------------------------------------------------------------
-FWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}* __restrict__ x2, {T}* __restrict__ out, "
+FWD_PARAMS = ("const TI* __restrict__ w, const TI* __restrict__ x1, const TI* __restrict__ x2, TI* __restrict__ out, "
               "const void* __restrict__ x1_index, int x1_idx64, const int64_t* __restrict__ csr_offsets, "
               "const int64_t* __restrict__ csr_perm")
 FWD_ARGS = "w, x1, x2, out, x1_index, x1_idx64, csr_offsets, csr_perm"
 BWD_ARGS = "w, x1, x2, g, dw, dx1, dx1_partial, dx2, dx2_partial, x1_index, x1_idx64, g_index, g_idx64, batch"
-BWD_PARAMS = ("const {T}* __restrict__ w, const {T}* __restrict__ x1, const {T}* __restrict__ x2, const {T}* __restrict__ g, "
-              "{T}* __restrict__ dw, {T}* dx1, {T}* __restrict__ dx1_partial, {T}* __restrict__ dx2, "
+# (dx1: sums by atomic additions, dx2_partial: partial rows - both in the arithmetic type; everything else holds TI)
+BWD_PARAMS = ("const TI* __restrict__ w, const TI* __restrict__ x1, const TI* __restrict__ x2, const TI* __restrict__ g, "
+              "TI* __restrict__ dw, {T}* dx1, TI* __restrict__ dx1_partial, TI* __restrict__ dx2, "
               "{T}* __restrict__ dx2_partial, const void* __restrict__ x1_index, int x1_idx64, "
               "const void* __restrict__ g_index, int g_idx64, int64_t batch")
 
 
+IO_TYPES = {"bf16": ("bf16_t", "CUEQ_BF16"), "f16": ("f16_t", "CUEQ_F16")}
+
+
+def io_type(T: str, io) -> tuple:
+    """(C++ element type of the buffers, its CUEQ_* code, tag for names) of a unit computing in ``T`` whose buffers hold
+    ``io`` (None: ``T`` itself; "bf16" / "f16": 16-bit elements, float arithmetic only)."""
+    if io is None:
+        return T, ("CUEQ_F32" if T == "float" else "CUEQ_F64"), T
+    if T != "float" or io not in IO_TYPES:
+        raise ValueError(f"buffers of {io} with {T} arithmetic are not generated")
+    return (*IO_TYPES[io], io)
+
+
 def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_hash: int, *, fwd_split: int = 1,
               fwd_waves: int = 2, fwd_prefetch: bool = True, bwd_waves: int = 2, bwd_chunk: int = 16,
-              bwd_prefetch: bool = False, bwd_split: int = 1) -> str:
-    """Complete .hip translation unit: kernels, host launchers, registration under both table hashes."""
-    ns = f"cw_{name}"
+              bwd_prefetch: bool = False, bwd_split: int = 1, io=None) -> str:
+    """Complete .hip translation unit: kernels, host launchers, registration under both table hashes.  ``io``: element type
+    of the buffers when it is not the arithmetic type ``T`` ("bf16" / "f16" with ``T`` = float)."""
+    TI, io_code, tag = io_type(T, io)
+    ns = f"cw_{name}" + (f"_{tag}" if io else "")
     nch = (st.extent + 63) // 64
     W1, WW, W2, WO = st.nseg_x1 * st.extent, st.nseg_w * st.extent, st.x2_width, st.nseg_out * st.extent
     out = []
@@ -676,21 +692,15 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     A("// GENERATED by cuequivariance_amd/codegen/channelwise.py - do not edit.")
     A(f"// channel-wise tensor product '{name}': extent {st.extent}, segments w/x1/x2/out = "
       f"{st.nseg_w}/{st.nseg_x1}/{st.nseg_x2}/{st.nseg_out}, {st.num_paths} paths, math {T}"
+      + (f", buffers of {tag}" if io else "")
       + (f", x1 rows in groups {list(st.layout_x1)}" if st.layout_x1 else "") + (f", output rows in groups {list(st.layout_out)}" if st.layout_out else "")
       + (", x2 = spherical harmonics of a 3-vector evaluated in the kernels" if st.harmonics else ""))
     A('#include "cw_common.h"')
-    A("// operands that are read or written exactly once per launch (weights, weight gradients, the output rows) are")
-    A("// marked non-temporal so that they do not displace the gathered rows in the caches")
-    A("#ifndef CUEQ_CW_NO_STREAM")
-    A("#define STREAM_LOAD(p) __builtin_nontemporal_load(p)")
-    A("#define STREAM_STORE(v, p) __builtin_nontemporal_store(v, p)")
-    A("#else")
-    A("#define STREAM_LOAD(p) (*(p))")
-    A("#define STREAM_STORE(v, p) (*(p) = (v))")
-    A("#endif")
     A("")
     A("namespace cueq {")
     A(f"namespace {ns} {{")
+    A(f"using TI = {TI};  // element type of the buffers; operands read or written exactly once per launch (weights, weight")
+    A("// gradients, output rows) go through io_ldnt / io_stnt so that they do not displace the gathered rows in the caches")
     A(f"#define FWD_PARAMS {FWD_PARAMS.format(T=T)}")
     A(f"#define FWD_ARGS {FWD_ARGS}")
     A(f"#define BWD_PARAMS {BWD_PARAMS.format(T=T)}")
@@ -700,17 +710,14 @@ def emit_unit(st: ChannelwiseStructure, T: str, name: str, fwd_hash: int, bwd_ha
     A("")
     A(emit_backward(st, T, bwd_waves, bwd_chunk, bwd_prefetch, bwd_split))
     A("")
-    code = f"dtype_code<{T}>::value"
+    same = "true" if io is None else "false"
     A(f"""
-static bool all_dtype(const cueq_u1d_buffer* b, int n) {{
-  for (int i = 0; i < n; ++i) if (b[i].dtype != {code}) return false;
-  return true;
-}}
+constexpr bool kSameType = {same};  // buffers hold the arithmetic type
 
 // buffers: w, x1, x2 | out
 static int run_fwd(const SpecCall& c) {{
   const cueq_u1d_buffer* b = c.buffers;
-  if (!all_dtype(b, 4)) return CUEQ_ERR_UNSUPPORTED;
+  if (common_dtype(b, 4) != {io_code}) return CUEQ_ERR_UNSUPPORTED;
   if (b[2].batch_dim != CUEQ_BATCH_BATCHED) return CUEQ_ERR_UNSUPPORTED;
   if (b[0].batch_dim == CUEQ_BATCH_INDEXED || b[1].batch_dim == CUEQ_BATCH_SHARED) return CUEQ_ERR_UNSUPPORTED;
   if (b[3].batch_dim == CUEQ_BATCH_SHARED) return CUEQ_ERR_UNSUPPORTED;
@@ -721,14 +728,14 @@ static int run_fwd(const SpecCall& c) {{
   if (rows == 0) return CUEQ_OK;
   const int64_t grid = rows * {nch} * kFwdSplit;
   CUEQ_REQUIRE(grid < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "too many output rows for one launch");
-  const {T}* w = static_cast<const {T}*>(b[0].data);
-  const {T}* x1 = static_cast<const {T}*>(b[1].data);
-  const {T}* x2 = static_cast<const {T}*>(b[2].data);
-  {T}* o = static_cast<{T}*>(b[3].data);
+  const TI* w = static_cast<const TI*>(b[0].data);
+  const TI* x1 = static_cast<const TI*>(b[1].data);
+  const TI* x2 = static_cast<const TI*>(b[2].data);
+  TI* o = static_cast<TI*>(b[3].data);
   const int64_t* offs = out_idx ? b[3].csr_offsets : nullptr;
   const int64_t* perm = out_idx ? b[3].csr_perm : nullptr;
   const dim3 g(static_cast<unsigned>(grid)), t(64);
-  KernelTimer timer("{name}_fwd_{T}", c.stream);
+  KernelTimer timer("{name}_fwd_{tag}", c.stream);
 #define LAUNCH_FWD(XI, WS) hipLaunchKernelGGL((fwd_kernel<XI, WS>), g, t, 0, c.stream, w, x1, x2, o, b[1].index, b[1].index_is_64, offs, perm)
   if (x1_idx && w_shared) LAUNCH_FWD(true, true);
   else if (x1_idx) LAUNCH_FWD(true, false);
@@ -740,17 +747,23 @@ static int run_fwd(const SpecCall& c) {{
 }}
 
 // buffers: w, x1, x2, g | dw, dx1, dx2
+// workspace: [partial rows of the x2 gradient, arithmetic type] [the x1 gradient of a gathered operand: one partial row per
+// batch row in TI (summed in index order afterwards), or - for 16-bit buffers and atomic sums - its rows in the arithmetic type]
 static int64_t bwd_workspace(const cueq_u1d_buffer* b, int64_t batch) {{
+  if (common_dtype(b, 7) != {io_code}) return 0;
   int64_t need = 0;
   if (kBwdParts > 1) need += batch * kBwdParts * {W2}ll * sizeof({T});
   need = (need + 255) & ~int64_t(255);
-  if (b[1].batch_dim == CUEQ_BATCH_INDEXED && deterministic_scatter()) need += batch * {W1}ll * sizeof({T});
+  if (b[1].batch_dim == CUEQ_BATCH_INDEXED) {{
+    if (deterministic_scatter()) need += batch * {W1}ll * sizeof(TI);
+    else if (!kSameType) need += b[5].rows * {W1}ll * sizeof({T});
+  }}
   return need;
 }}
 
 static int run_bwd(const SpecCall& c) {{
   const cueq_u1d_buffer* b = c.buffers;
-  if (!all_dtype(b, 7)) return CUEQ_ERR_UNSUPPORTED;
+  if (common_dtype(b, 7) != {io_code}) return CUEQ_ERR_UNSUPPORTED;
   if (b[0].batch_dim != CUEQ_BATCH_BATCHED || b[2].batch_dim != CUEQ_BATCH_BATCHED) return CUEQ_ERR_UNSUPPORTED;
   if (b[1].batch_dim == CUEQ_BATCH_SHARED || b[3].batch_dim == CUEQ_BATCH_SHARED) return CUEQ_ERR_UNSUPPORTED;
   if (b[4].batch_dim != CUEQ_BATCH_BATCHED || b[6].batch_dim != CUEQ_BATCH_BATCHED) return CUEQ_ERR_UNSUPPORTED;
@@ -760,27 +773,28 @@ static int run_bwd(const SpecCall& c) {{
   const bool det = deterministic_scatter();
   if (x1_idx && det && (!b[5].csr_offsets || (!b[5].csr_perm && c.batch > 0))) return CUEQ_ERR_UNSUPPORTED;
   const int64_t batch = c.batch;
-  const {T}* w = static_cast<const {T}*>(b[0].data);
-  const {T}* x1 = static_cast<const {T}*>(b[1].data);
-  const {T}* x2 = static_cast<const {T}*>(b[2].data);
-  const {T}* g = static_cast<const {T}*>(b[3].data);
-  {T}* dw = static_cast<{T}*>(b[4].data);
-  {T}* dx1 = static_cast<{T}*>(b[5].data);
-  {T}* dx2 = static_cast<{T}*>(b[6].data);
+  const TI* w = static_cast<const TI*>(b[0].data);
+  const TI* x1 = static_cast<const TI*>(b[1].data);
+  const TI* x2 = static_cast<const TI*>(b[2].data);
+  const TI* g = static_cast<const TI*>(b[3].data);
+  TI* dw = static_cast<TI*>(b[4].data);
+  TI* dx1 = static_cast<TI*>(b[5].data);
+  TI* dx2 = static_cast<TI*>(b[6].data);
   const int64_t need = bwd_workspace(b, batch);
   CUEQ_REQUIRE(need == 0 || (c.workspace && c.workspace_bytes >= need), CUEQ_ERR_INVALID, "workspace too small: need %lld bytes", (long long)need);
   char* ws = static_cast<char*>(c.workspace);
   {T}* dx2_partial = nullptr;
   int64_t off = 0;
   if (kBwdParts > 1) {{ dx2_partial = reinterpret_cast<{T}*>(ws); off = (batch * kBwdParts * {W2}ll * sizeof({T}) + 255) & ~int64_t(255); }}
-  {T}* dx1_partial = nullptr;
-  bool atomic = false;
+  TI* dx1_partial = nullptr;
+  {T}* dx1_sums = nullptr;  // target of the atomic additions
   if (!x1_idx) dx1_partial = dx1;  // one row per batch element: plain stores
-  else if (det) dx1_partial = reinterpret_cast<{T}*>(ws + off);
-  else atomic = true;
+  else if (det) dx1_partial = reinterpret_cast<TI*>(ws + off);
+  else dx1_sums = kSameType ? reinterpret_cast<{T}*>(dx1) : reinterpret_cast<{T}*>(ws + off);
+  const bool atomic = dx1_sums != nullptr;
   if (atomic && b[5].rows > 0) {{
     const int64_t n = b[5].rows * {W1}ll;
-    hipLaunchKernelGGL(fill_zero<{T}>, dim3(fill_blocks<{T}>(n)), dim3(256), 0, c.stream, dx1, n);
+    hipLaunchKernelGGL(fill_zero<{T}>, dim3(fill_blocks<{T}>(n)), dim3(256), 0, c.stream, dx1_sums, n);
     CUEQ_CHECK_HIP(hipGetLastError());
   }}
   if (batch > 0) {{
@@ -792,8 +806,8 @@ static int run_bwd(const SpecCall& c) {{
     const int64_t grid = nranges * kBwdParts;
     const dim3 gd(static_cast<unsigned>(grid)), t(64);
     {{
-    KernelTimer timer("{name}_bwd_{T}", c.stream);
-#define LAUNCH_BWD(XI, GI, AT) hipLaunchKernelGGL((bwd_kernel<XI, GI, AT>), gd, t, 0, c.stream, w, x1, x2, g, dw, dx1, dx1_partial, dx2, dx2_partial, b[1].index, b[1].index_is_64, b[3].index, b[3].index_is_64, batch)
+    KernelTimer timer("{name}_bwd_{tag}", c.stream);
+#define LAUNCH_BWD(XI, GI, AT) hipLaunchKernelGGL((bwd_kernel<XI, GI, AT>), gd, t, 0, c.stream, w, x1, x2, g, dw, dx1_sums, dx1_partial, dx2, dx2_partial, b[1].index, b[1].index_is_64, b[3].index, b[3].index_is_64, batch)
     if (x1_idx && g_idx && atomic) LAUNCH_BWD(true, true, true);
     else if (x1_idx && g_idx) LAUNCH_BWD(true, true, false);
     else if (x1_idx && atomic) LAUNCH_BWD(true, false, true);
@@ -804,26 +818,31 @@ static int run_bwd(const SpecCall& c) {{
     }}
     CUEQ_CHECK_HIP(hipGetLastError());
     if (kBwdParts > 1) {{
-      hipLaunchKernelGGL(fold_parts<{T}>, dim3(blocks_for(batch * {W2}ll)), dim3(256), 0, c.stream, dx2_partial, batch, kBwdParts, {W2}, dx2);
+      hipLaunchKernelGGL((fold_parts<{T}, TI>), dim3(blocks_for(batch * {W2}ll)), dim3(256), 0, c.stream, dx2_partial, batch, kBwdParts, {W2}, dx2);
       CUEQ_CHECK_HIP(hipGetLastError());
     }}
   }}
+  if (atomic && !kSameType && b[5].rows > 0) {{
+    const int64_t n = b[5].rows * {W1}ll;
+    hipLaunchKernelGGL((round_rows<{T}, TI>), dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1_sums, n, dx1);
+    CUEQ_CHECK_HIP(hipGetLastError());
+  }}
   if (x1_idx && det && b[5].rows > 0) {{
     const int64_t n = b[5].rows * {W1}ll;
-    if ({W1} % 4 == 0 && reinterpret_cast<uintptr_t>(dx1) % (4 * sizeof({T})) == 0 && reinterpret_cast<uintptr_t>(dx1_partial) % (4 * sizeof({T})) == 0 &&
+    if ({W1} % 4 == 0 && reinterpret_cast<uintptr_t>(dx1) % (4 * sizeof(TI)) == 0 && reinterpret_cast<uintptr_t>(dx1_partial) % (4 * sizeof(TI)) == 0 &&
         b[5].rows < 65536) {{
-      hipLaunchKernelGGL(segment_sum_rows_vec<{T}>, dim3(({W1} / 4 + 255) / 256, static_cast<unsigned>(b[5].rows)), dim3(256), 0, c.stream,
+      hipLaunchKernelGGL(segment_sum_rows_vec<TI>, dim3(({W1} / 4 + 255) / 256, static_cast<unsigned>(b[5].rows)), dim3(256), 0, c.stream,
                          dx1_partial, b[5].csr_offsets, b[5].csr_perm, {W1}, dx1);
     }} else {{
-      hipLaunchKernelGGL(segment_sum_rows<{T}>, dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1_partial, b[5].csr_offsets, b[5].csr_perm, b[5].rows, {W1}, dx1);
+      hipLaunchKernelGGL(segment_sum_rows<TI>, dim3(blocks_for(n)), dim3(256), 0, c.stream, dx1_partial, b[5].csr_offsets, b[5].csr_perm, b[5].rows, {W1}, dx1);
     }}
     CUEQ_CHECK_HIP(hipGetLastError());
   }}
   return CUEQ_OK;
 }}
 
-static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{T}", run_fwd, nullptr}};
-static const U1dSpec spec_bwd = {{0x{bwd_hash:016x}ull, "{name}_bwd_{T}", run_bwd, bwd_workspace}};
+static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{tag}", run_fwd, nullptr, {io_code}}};
+static const U1dSpec spec_bwd = {{0x{bwd_hash:016x}ull, "{name}_bwd_{tag}", run_bwd, bwd_workspace, {io_code}}};
 static SpecRegistrar reg_fwd(&spec_fwd);
 static SpecRegistrar reg_bwd(&spec_bwd);
 """)

@@ -421,8 +421,8 @@ static int run_bwd(const SpecCall& c) {{
   return CUEQ_OK;
 }}
 
-static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{T}", run_fwd, fwd_workspace}};
-static const U1dSpec spec_bwd = {{0x{bwd_hash:016x}ull, "{name}_bwd_{T}", run_bwd, bwd_workspace}};
+static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{T}", run_fwd, fwd_workspace, {code}}};
+static const U1dSpec spec_bwd = {{0x{bwd_hash:016x}ull, "{name}_bwd_{T}", run_bwd, bwd_workspace, {code}}};
 static SpecRegistrar reg_fwd(&spec_fwd);
 static SpecRegistrar reg_bwd(&spec_bwd);
 """)

@@ -48,6 +48,10 @@ FULLY_CONNECTED = [
 
 MATH = (("float", 0), ("double", 1))
 
+# Units (by name, the "_mulir" ones included) also generated for buffers of 16-bit elements with float arithmetic:
+# {unit name: ("bf16", ...)}.  Other units and element types are compiled at first use.
+IO_16BIT = {"c128_l3": ("bf16",), "c128_l3_mulir": ("bf16",), "s128_l3": ("bf16",), "s128_l3_mulir": ("bf16",)}
+
 
 def channelwise_tables(irreps1: str, irreps2: str, filt) -> U1dTables:
     e = cue.descriptors.channelwise_tensor_product(cue.Irreps("O3", irreps1), cue.Irreps("O3", irreps2), filt)
@@ -97,6 +101,8 @@ def generate(verbose: bool = False) -> list[Path]:
                 _write(GENERATED_DIR / f"sc_{vname}_{T}.hip", sc.emit_unit(st, T, vname, t.content_hash(code), bwd), written)
                 if verbose:
                     print(f"generated sc_{vname}_{T}.hip: {len(st.terms)} folded terms")
+                for io in (IO_16BIT.get(vname, ()) if T == "float" else ()):
+                    _write(GENERATED_DIR / f"sc_{vname}_{io}.hip", sc.emit_unit(st, T, vname, t.content_hash(code), bwd, io=io), written)
     for ir1, ir2, ir3 in FULLY_CONNECTED:
         # the same products with a weight row per batch row (the convolution layer's per-edge weights)
         poly = cue.descriptors.fully_connected_tensor_product(cue.Irreps("O3", ir1), cue.Irreps("O3", ir2), cue.Irreps("O3", ir3)).polynomial
@@ -133,12 +139,12 @@ def generate(verbose: bool = False) -> list[Path]:
         for vname, vst, vt, vtb in variants:
             for T, code in MATH:
                 src = cw.emit_unit(vst, T, vname, vt.content_hash(code), vtb.content_hash(code), **tuning.get(T, {}))
-                path = GENERATED_DIR / f"cw_{vname}_{T}.hip"
-                if not path.exists() or path.read_text() != src:
-                    path.write_text(src)
-                written.append(path)
+                _write(GENERATED_DIR / f"cw_{vname}_{T}.hip", src, written)
                 if verbose:
-                    print(f"generated {path.name}: {vst.num_paths} paths")
+                    print(f"generated cw_{vname}_{T}.hip: {vst.num_paths} paths")
+                for io in (IO_16BIT.get(vname, ()) if T == "float" else ()):
+                    _write(GENERATED_DIR / f"cw_{vname}_{io}.hip",
+                           cw.emit_unit(vst, T, vname, vt.content_hash(code), vtb.content_hash(code), io=io, **tuning.get(T, {})), written)
     return written
 
 

@@ -24,7 +24,7 @@ from __future__ import annotations
 from collections import defaultdict
 from dataclasses import dataclass
 
-from .channelwise import _lit
+from .channelwise import _lit, io_type
 
 
 @dataclass
@@ -149,10 +149,10 @@ def _row_request(A, ind: str, st: SymmetricStructure, T: str, layout: tuple, seg
         if a in staged:
             first, d, k = staged[a]
             ok = _piece_ok(st, d, k)
-            load = f"__builtin_nontemporal_load({ptr} + {_piece(st, first, d, k)})"
+            load = f"io_ldnt({ptr} + {_piece(st, first, d, k)})"
             A(f"{ind}{decl}{dst}{a} = " + (f"{ok} ? {load} : {T}(0);" if ok else f"{load};"))
         else:
-            A(f"{ind}{decl}{dst}{a} = __builtin_nontemporal_load({ptr} + {a * st.extent} + uu);")
+            A(f"{ind}{decl}{dst}{a} = io_ldnt({ptr} + {a * st.extent} + uu);")
 
 
 def _row_unpack(A, ind: str, st: SymmetricStructure, T: str, layout: tuple, segs, src: str, dst: str):
@@ -181,7 +181,7 @@ def _row_store(A, ind: str, st: SymmetricStructure, T: str, layout: tuple, nseg:
     done = set()
     for a in range(nseg):
         if a not in staged:
-            A(f"{ind}if (active) __builtin_nontemporal_store({value(a)}, {ptr} + {a * st.extent} + uu);")
+            A(f"{ind}if (active) io_stnt({value(a)}, {ptr} + {a * st.extent} + uu);")
             continue
         first, d, _ = staged[a]
         if first in done:
@@ -192,7 +192,7 @@ def _row_store(A, ind: str, st: SymmetricStructure, T: str, layout: tuple, nseg:
         A(f"{ind}__builtin_amdgcn_wave_barrier();")
         for k in range(d):
             ok = _piece_ok(st, d, k)
-            A(f"{ind}" + (f"if {ok} " if ok else "") + f"__builtin_nontemporal_store(stage[{k * 64} + lane], {ptr} + {_piece(st, first, d, k)});")
+            A(f"{ind}" + (f"if {ok} " if ok else "") + f"io_stnt(stage[{k * 64} + lane], {ptr} + {_piece(st, first, d, k)});")
         A(f"{ind}__builtin_amdgcn_wave_barrier();")
 
 
@@ -208,13 +208,15 @@ def _whole_groups(layout: tuple, segs, nseg: int):
 
 
 def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hashes: dict, *, fwd_waves: int = 4,
-              bwd_waves: int = 2, fwd_prefetch: bool = None) -> str:
-    """Complete translation unit.  ``bwd_hashes``: {(need_dw, need_dx): table hash}."""
+              bwd_waves: int = 2, fwd_prefetch: bool = None, io=None) -> str:
+    """Complete translation unit.  ``bwd_hashes``: {(need_dw, need_dx): table hash}.  ``io``: element type of the buffers when
+    it is not the arithmetic type ``T`` ("bf16" / "f16" with ``T`` = float)."""
+    TI, io_code, tag = io_type(T, io)
     if fwd_prefetch is None:
         # float: 96 -> 119 registers, still 4 wavefronts per SIMD; double: the pair products alone exceed the register file
         # (the kernel spills either way), a second set of x rows only adds to that
         fwd_prefetch = T == "float"
-    ns = f"sc_{name}"
+    ns = f"sc_{name}" + (f"_{tag}" if io else "")
     E, W, X, O = st.extent, st.nseg_w * st.extent, st.nseg_x * st.extent, st.nseg_out * st.extent
     nch = (E + 63) // 64
     groups = _groups(st)
@@ -228,12 +230,13 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A = L.append
     A("// GENERATED by cuequivariance_amd/codegen/symmetric.py - do not edit.")
     A(f"// symmetric contraction '{name}': extent {E}, segments w/x/out = {st.nseg_w}/{st.nseg_x}/{st.nseg_out}, "
-      f"{len(st.terms)} folded terms in {len(groups)} (weight, output) groups, math {T}"
+      f"{len(st.terms)} folded terms in {len(groups)} (weight, output) groups, math {T}" + (f", buffers of {tag}" if io else "")
       + (f", x rows in groups {list(st.layout_x)}" if st.layout_x else "") + (f", output rows in groups {list(st.layout_out)}" if st.layout_out else ""))
     A('#include "cw_common.h"')
     A("")
     A("namespace cueq {")
     A(f"namespace {ns} {{")
+    A(f"using TI = {TI};  // element type of the buffers")
     A("")
     if E % 64 == 0:
         lane_setup = "  const int uu = ch * 64 + lane; constexpr bool active = true;"
@@ -244,7 +247,7 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("// W_MODE: 0 one weight row per batch row, 1 weight row chosen by w_index, 2 a single shared weight row")
     A("template <int W_MODE>")
     A(f"__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu({fwd_waves}))) fwd_kernel(")
-    A(f"    const {T}* __restrict__ w, const {T}* __restrict__ x, {T}* __restrict__ out, const void* __restrict__ w_index, int idx64, int64_t batch) {{")
+    A(f"    const TI* __restrict__ w, const TI* __restrict__ x, TI* __restrict__ out, const void* __restrict__ w_index, int idx64, int64_t batch) {{")
     A("  const int lane = threadIdx.x;")
     A(f"  const int ch = blockIdx.x % {nch}; const int64_t slot = blockIdx.x / {nch}; const int64_t nslots = gridDim.x / {nch};")
     A(lane_setup)
@@ -259,20 +262,20 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
         A("  if (W_MODE == 1) wrow_n = load_index(w_index, idx64, z0);")
         A(f"  {T} " + ", ".join(f"xn{a}" for a in x_read) + ";")
         A("  {")
-        A(f"    const {T}* __restrict__ xp = x + z0 * {X}ll;")
+        A(f"    const TI* __restrict__ xp = x + z0 * {X}ll;")
         _row_request(A, "    ", st, T, st.layout_x, x_read, "xp", "xn", False)
         A("  }")
         A("  for (int64_t z = z0; z < z1; ++z) {")
         A("    const int64_t wrow = wrow_n;")
-        A(f"    const {T}* __restrict__ wp = w + wrow * {W}ll;")
+        A(f"    const TI* __restrict__ wp = w + wrow * {W}ll;")
         for s in w_used:
-            A(f"    const {T} wv{s} = wp[{s * E} + uu];")
+            A(f"    const {T} wv{s} = io_ld(wp + {s * E} + uu);")
         _row_unpack(A, "    ", st, T, st.layout_x, x_read, "xn", "xv")
         A("    {")
         A("      const int64_t zn = z + 1 < z1 ? z + 1 : z;")
         A("      wrow_n = W_MODE == 0 ? zn : 0;")
         A("      if (W_MODE == 1) wrow_n = load_index(w_index, idx64, zn);")
-        A(f"      const {T}* __restrict__ xp = x + zn * {X}ll;")
+        A(f"      const TI* __restrict__ xp = x + zn * {X}ll;")
         _row_request(A, "      ", st, T, st.layout_x, x_read, "xp", "xn", False)
         A("    }")
         A("    __builtin_amdgcn_sched_barrier(0);")
@@ -280,11 +283,11 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
         A("  for (int64_t z = z0; z < z1; ++z) {")
         A("    int64_t wrow = W_MODE == 0 ? z : 0;")
         A("    if (W_MODE == 1) wrow = load_index(w_index, idx64, z);")
-        A(f"    const {T}* __restrict__ xp = x + z * {X}ll;")
-        A(f"    const {T}* __restrict__ wp = w + wrow * {W}ll;")
+        A(f"    const TI* __restrict__ xp = x + z * {X}ll;")
+        A(f"    const TI* __restrict__ wp = w + wrow * {W}ll;")
         _row_request(A, "    ", st, T, st.layout_x, x_read, "xp", "xr", True)
         for s in w_used:
-            A(f"    const {T} wv{s} = wp[{s * E} + uu];")
+            A(f"    const {T} wv{s} = io_ld(wp + {s * E} + uu);")
         _row_unpack(A, "    ", st, T, st.layout_x, x_read, "xr", "xv")
     for a, b in pairs:
         A(f"    const {T} pp_{a}_{b} = xv{a} * xv{b};")
@@ -297,7 +300,7 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
         A(f"      acc{k} = fma(wv{s}, P, acc{k});")
         A("    }")
     A("    {")
-    A(f"      {T}* __restrict__ op = out + z * {O}ll;")
+    A(f"      TI* __restrict__ op = out + z * {O}ll;")
     _row_store(A, "      ", st, T, st.layout_out, st.nseg_out, "op", lambda k: f"acc{k}")
     A("    }")
     A("  }")
@@ -308,7 +311,7 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("// rows are visited in the order of the CSR grouping by weight index (csr_perm may be null: already grouped)")
     A("template <bool NEED_DW, bool NEED_DX>")
     A(f"__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu({bwd_waves}))) bwd_kernel(")
-    A(f"    const {T}* __restrict__ w, const {T}* __restrict__ x, const {T}* __restrict__ g, {T}* __restrict__ dw, {T}* __restrict__ dx,")
+    A(f"    const TI* __restrict__ w, const TI* __restrict__ x, const TI* __restrict__ g, TI* __restrict__ dw, TI* __restrict__ dx,")
     A(f"    {T}* __restrict__ part, const void* __restrict__ w_index, int idx64, const int64_t* __restrict__ csr_perm, int64_t batch) {{")
     A("  const int lane = threadIdx.x;")
     A(f"  const int ch = blockIdx.x % {nch}; const int64_t slot = blockIdx.x / {nch}; const int64_t nslots = gridDim.x / {nch};")
@@ -322,15 +325,16 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("  int64_t cur = -1, first = -1;")
     A("  auto flush = [&](bool last) {")
     A("    if (!NEED_DW || !active) return;")
-    A(f"    {T}* dst;")
-    A(f"    if (cur == first) dst = part + (slot * 2 + 0) * {W}ll;       // head: the group may have begun in an earlier slot")
-    A(f"    else if (last) dst = part + (slot * 2 + 1) * {W}ll;           // tail: the group may continue in the next slot")
-    A(f"    else dst = dw + cur * {W}ll;                                    // whole group inside this slot")
-    for s in w_used:
-        A(f"    dst[{s * E} + uu] = q{s};")
-    unused_w = [s for s in range(st.nseg_w) if s not in w_used]
-    for s in unused_w:
-        A(f"    dst[{s * E} + uu] = 0;")
+    A("    if (cur != first && !last) {                                     // whole group inside this slot")
+    A(f"      TI* dst = dw + cur * {W}ll;")
+    for s in range(st.nseg_w):
+        A(f"      io_st({f'q{s}' if s in w_used else f'{T}(0)'}, dst + {s * E} + uu);")
+    A("    } else {")
+    A("      // head (the group may have begun in an earlier slot) or tail (it may continue in the next one): a partial row")
+    A(f"      {T}* dst = part + (slot * 2 + (cur == first ? 0 : 1)) * {W}ll;")
+    for s in range(st.nseg_w):
+        A(f"      dst[{s * E} + uu] = {f'q{s}' if s in w_used else '0'};")
+    A("    }")
     A("  };")
     A("  for (int64_t p = p0; p < p1; ++p) {")
     A("    const int64_t z = csr_perm ? csr_perm[p] : p;")
@@ -339,12 +343,12 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("      if (cur >= 0) flush(false);")
     A("      if (first < 0) first = e;")
     A("      cur = e;")
-    A(f"      const {T}* __restrict__ wp = w + e * {W}ll;")
+    A(f"      const TI* __restrict__ wp = w + e * {W}ll;")
     for s in w_used:
-        A(f"      wv{s} = wp[{s * E} + uu]; q{s} = 0;")
+        A(f"      wv{s} = io_ld(wp + {s * E} + uu); q{s} = 0;")
     A("    }")
-    A(f"    const {T}* __restrict__ xp = x + z * {X}ll;")
-    A(f"    const {T}* __restrict__ gp = g + z * {O}ll;")
+    A(f"    const TI* __restrict__ xp = x + z * {X}ll;")
+    A(f"    const TI* __restrict__ gp = g + z * {O}ll;")
     _row_request(A, "    ", st, T, st.layout_x, x_read, "xp", "xr", True)
     _row_request(A, "    ", st, T, st.layout_out, range(st.nseg_out), "gp", "gr", True)
     _row_unpack(A, "    ", st, T, st.layout_x, x_read, "xr", "xv")
@@ -384,7 +388,7 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
         A("      }")
         A("    }")
     A("    if (NEED_DX) {")
-    A(f"      {T}* __restrict__ dp = dx + z * {X}ll;")
+    A(f"      TI* __restrict__ dp = dx + z * {X}ll;")
     _row_store(A, "      ", st, T, st.layout_x, st.nseg_x, "dp", lambda a: f"dxa{a}" if a in x_used else f"{T}(0)")
     A("    }")
     A("  }")
@@ -396,7 +400,7 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("// [q0, q1) contributes its head partial when a <= q0 < b (e is its first group) and its tail partial when only its")
     A("// last position lies in [a, b).  One block = 64 weight columns x 16 slot lanes; the 16 partial sums are added in lane")
     A("// order (fixed, so the result does not change from run to run).")
-    A(f"__global__ void __launch_bounds__(1024) fold_kernel(const {T}* __restrict__ part, {T}* __restrict__ dw,")
+    A(f"__global__ void __launch_bounds__(1024) fold_kernel(const {T}* __restrict__ part, TI* __restrict__ dw,")
     A("    const int64_t* __restrict__ csr_offsets, int64_t batch, int64_t nslots, int64_t row0) {")
     A(f"  __shared__ {T} s_acc[16][64];")
     A("  __shared__ int s_any[16];")
@@ -405,7 +409,7 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("  const int j = blockIdx.x * 64 + jl;")
     A(f"  const bool live = j < {W};")
     A("  const int64_t a = csr_offsets[e], b = csr_offsets[e + 1];")
-    A(f"  if (a == b) {{ if (sl == 0 && live) dw[e * {W}ll + j] = 0; return; }}")
+    A(f"  if (a == b) {{ if (sl == 0 && live) io_st({T}(0), dw + e * {W}ll + j); return; }}")
     A("  // slots whose range [s * batch / nslots, (s + 1) * batch / nslots) meets [a, b)")
     A("  int64_t s_lo = a * nslots / batch, s_hi = (b - 1) * nslots / batch;")
     A("  while (s_lo > 0 && (s_lo * batch / nslots) > a) --s_lo;")
@@ -426,16 +430,12 @@ def emit_unit(st: SymmetricStructure, T: str, name: str, fwd_hash: int, bwd_hash
     A("  if (sl == 0 && live) {")
     A(f"    {T} total = 0; int seen = 0;")
     A("    for (int t = 0; t < 16; ++t) { total += s_acc[t][jl]; seen |= s_any[t]; }")
-    A(f"    if (seen) dw[e * {W}ll + j] = total;")
+    A(f"    if (seen) io_st(total, dw + e * {W}ll + j);")
     A("  }")
     A("}")
     A("")
-    code = f"dtype_code<{T}>::value"
     A(f"""
-static bool all_dtype(const cueq_u1d_buffer* b, int n) {{
-  for (int i = 0; i < n; ++i) if (b[i].dtype != {code}) return false;
-  return true;
-}}
+static bool all_dtype(const cueq_u1d_buffer* b, int n) {{ return common_dtype(b, n) == {io_code}; }}
 
 static int64_t slots_for(int64_t batch, int waves) {{
   int64_t n = wave_slots(waves) / {nch};
@@ -450,10 +450,10 @@ static int run_fwd(const SpecCall& c) {{
   if (b[1].batch_dim != CUEQ_BATCH_BATCHED || b[2].batch_dim != CUEQ_BATCH_BATCHED) return CUEQ_ERR_UNSUPPORTED;
   if (c.batch == 0) return CUEQ_OK;
   const dim3 grid(static_cast<unsigned>(slots_for(c.batch, {fwd_waves}) * {nch})), t(64);
-  const {T}* w = static_cast<const {T}*>(b[0].data);
-  const {T}* x = static_cast<const {T}*>(b[1].data);
-  {T}* o = static_cast<{T}*>(b[2].data);
-  KernelTimer timer("{name}_fwd_{T}", c.stream);
+  const TI* w = static_cast<const TI*>(b[0].data);
+  const TI* x = static_cast<const TI*>(b[1].data);
+  TI* o = static_cast<TI*>(b[2].data);
+  KernelTimer timer("{name}_fwd_{tag}", c.stream);
   if (b[0].batch_dim == CUEQ_BATCH_INDEXED)
     hipLaunchKernelGGL(fwd_kernel<1>, grid, t, 0, c.stream, w, x, o, b[0].index, b[0].index_is_64, c.batch);
   else if (b[0].batch_dim == CUEQ_BATCH_SHARED)
@@ -483,11 +483,11 @@ static int run_bwd(const SpecCall& c) {{
   if (bdw && (bdw->batch_dim != CUEQ_BATCH_INDEXED || bdw->index != b[0].index || bdw->rows != b[0].rows || !bdw->csr_offsets))
     return CUEQ_ERR_UNSUPPORTED;
   const int64_t batch = c.batch;
-  {T}* dw = bdw ? static_cast<{T}*>(bdw->data) : nullptr;
+  TI* dw = bdw ? static_cast<TI*>(bdw->data) : nullptr;
   if (batch == 0) {{
     if (bdw && bdw->rows > 0) {{
       const int64_t nn = bdw->rows * {W}ll;
-      hipLaunchKernelGGL(fill_zero<{T}>, dim3(fill_blocks<{T}>(nn)), dim3(256), 0, c.stream, dw, nn);
+      hipLaunchKernelGGL(fill_zero<TI>, dim3(fill_blocks<TI>(nn)), dim3(256), 0, c.stream, dw, nn);
       CUEQ_CHECK_HIP(hipGetLastError());
     }}
     return CUEQ_OK;
@@ -498,10 +498,10 @@ static int run_bwd(const SpecCall& c) {{
   {T}* part = static_cast<{T}*>(c.workspace);
   const int64_t* perm = bdw ? bdw->csr_perm : nullptr;
   {{
-    KernelTimer timer("{name}_bwd_{T}", c.stream);
+    KernelTimer timer("{name}_bwd_{tag}", c.stream);
     hipLaunchKernelGGL((bwd_kernel<NEED_DW, NEED_DX>), dim3(static_cast<unsigned>(nslots * {nch})), dim3(64), 0, c.stream,
-                       static_cast<const {T}*>(b[0].data), static_cast<const {T}*>(b[1].data), static_cast<const {T}*>(b[2].data), dw,
-                       bdx ? static_cast<{T}*>(bdx->data) : nullptr, part, b[0].index, b[0].index_is_64, perm, batch);
+                       static_cast<const TI*>(b[0].data), static_cast<const TI*>(b[1].data), static_cast<const TI*>(b[2].data), dw,
+                       bdx ? static_cast<TI*>(bdx->data) : nullptr, part, b[0].index, b[0].index_is_64, perm, batch);
   }}
   CUEQ_CHECK_HIP(hipGetLastError());
   if (NEED_DW) {{
@@ -516,13 +516,13 @@ static int run_bwd(const SpecCall& c) {{
   return CUEQ_OK;
 }}
 
-static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{T}", run_fwd, nullptr}};
+static const U1dSpec spec_fwd = {{0x{fwd_hash:016x}ull, "{name}_fwd_{tag}", run_fwd, nullptr, {io_code}}};
 static SpecRegistrar reg_fwd(&spec_fwd);""")
     for (ndw, ndx), h in sorted(bwd_hashes.items()):
-        tag = ("w" if ndw else "") + ("x" if ndx else "")
+        which = ("w" if ndw else "") + ("x" if ndx else "")
         tb = f"<{str(ndw).lower()}, {str(ndx).lower()}>"
-        A(f'static const U1dSpec spec_bwd_{tag} = {{0x{h:016x}ull, "{name}_bwd_{tag}_{T}", run_bwd{tb}, bwd_workspace{tb}}};')
-        A(f"static SpecRegistrar reg_bwd_{tag}(&spec_bwd_{tag});")
+        A(f'static const U1dSpec spec_bwd_{which} = {{0x{h:016x}ull, "{name}_bwd_{which}_{tag}", run_bwd{tb}, bwd_workspace{tb}, {io_code}}};')
+        A(f"static SpecRegistrar reg_bwd_{which}(&spec_bwd_{which});")
     A("")
     A(f"}}  // namespace {ns}")
     A("}  // namespace cueq")

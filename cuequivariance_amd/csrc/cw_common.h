@@ -32,6 +32,60 @@ __device__ __forceinline__ T wave_sum(T v) {
   return v;
 }
 
+// ---- element types of the buffers ----------------------------------------------------------------
+// The generated kernels compute in `float` or `double`; their buffers hold that type or, for `float` arithmetic, 16-bit
+// elements (bfloat16 as its bits, IEEE half) that are widened when loaded and rounded to nearest even when stored.
+struct bf16_t { uint16_t bits; };
+using f16_t = _Float16;
+
+template <typename TI> struct math_of { using type = TI; };  // the arithmetic type that goes with an element type
+template <> struct math_of<bf16_t> { using type = float; };
+template <> struct math_of<f16_t> { using type = float; };
+
+template <typename T> struct dtype_code;
+template <> struct dtype_code<float> { static constexpr int value = CUEQ_F32; };
+template <> struct dtype_code<double> { static constexpr int value = CUEQ_F64; };
+template <> struct dtype_code<bf16_t> { static constexpr int value = CUEQ_BF16; };
+template <> struct dtype_code<f16_t> { static constexpr int value = CUEQ_F16; };
+
+__device__ __forceinline__ float io_ld(const float* p) { return *p; }
+__device__ __forceinline__ double io_ld(const double* p) { return *p; }
+__device__ __forceinline__ float io_ld(const bf16_t* p) { return bf16_bits_to_float(p->bits); }
+__device__ __forceinline__ float io_ld(const f16_t* p) { return static_cast<float>(*p); }
+__device__ __forceinline__ void io_st(float v, float* p) { *p = v; }
+__device__ __forceinline__ void io_st(double v, double* p) { *p = v; }
+// (float -> bfloat16: the hardware's conversion, round to nearest even, one instruction)
+__device__ __forceinline__ uint16_t io_bf16_bits(float v) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(v)); }
+__device__ __forceinline__ void io_st(float v, bf16_t* p) { p->bits = io_bf16_bits(v); }
+__device__ __forceinline__ void io_st(float v, f16_t* p) { *p = static_cast<f16_t>(v); }
+// the same for data read or written once per launch (non-temporal: they do not displace gathered rows in the caches)
+#ifndef CUEQ_CW_NO_STREAM
+__device__ __forceinline__ float io_ldnt(const float* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ double io_ldnt(const double* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ float io_ldnt(const bf16_t* p) { return bf16_bits_to_float(__builtin_nontemporal_load(&p->bits)); }
+__device__ __forceinline__ float io_ldnt(const f16_t* p) { return static_cast<float>(__builtin_nontemporal_load(p)); }
+__device__ __forceinline__ void io_stnt(float v, float* p) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void io_stnt(double v, double* p) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ void io_stnt(float v, bf16_t* p) { __builtin_nontemporal_store(io_bf16_bits(v), &p->bits); }
+__device__ __forceinline__ void io_stnt(float v, f16_t* p) { __builtin_nontemporal_store(static_cast<f16_t>(v), p); }
+#else
+template <typename TI> __device__ __forceinline__ auto io_ldnt(const TI* p) { return io_ld(p); }
+template <typename M, typename TI> __device__ __forceinline__ void io_stnt(M v, TI* p) { io_st(v, p); }
+#endif
+
+// the element type shared by buffers [0, n), as a CUEQ_* code, or -1 when they differ
+inline int common_dtype(const cueq_u1d_buffer* b, int n) {
+  for (int i = 1; i < n; ++i) if (b[i].dtype != b[0].dtype) return -1;
+  return b[0].dtype;
+}
+
+// out[i] = in[i] rounded to TO (the gradient of a gathered operand is summed in the arithmetic type and rounded once)
+template <typename M, typename TO>
+__global__ void __launch_bounds__(256) round_rows(const M* __restrict__ in, int64_t n, TO* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) io_st(in[i], out + i);
+}
+
 // ---- finishing kernels ------------------------------------------------------------------------
 // out[r, :] = sum over zz in [offsets[r], offsets[r+1]) of partial[perm[zz], :]   (width elements per row)
 template <typename T>
@@ -42,9 +96,9 @@ __global__ void __launch_bounds__(256) segment_sum_rows(const T* __restrict__ pa
   const int64_t r = tid / width;
   if (r >= nrows) return;
   const int c = static_cast<int>(tid - r * width);
-  T acc = 0;
-  for (int64_t zz = offsets[r]; zz < offsets[r + 1]; ++zz) acc += partial[perm[zz] * width + c];
-  out[tid] = acc;
+  typename math_of<T>::type acc = 0;
+  for (int64_t zz = offsets[r]; zz < offsets[r + 1]; ++zz) acc += io_ld(partial + perm[zz] * width + c);
+  io_st(acc, out + tid);
 }
 
 // The same sum for rows whose width is a multiple of 4 elements (16-byte aligned rows): a thread owns 4 consecutive
@@ -58,7 +112,7 @@ __global__ void __launch_bounds__(256) segment_sum_rows_vec(const T* __restrict_
   const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
   if (c >= width) return;
   const int64_t z0 = offsets[r], z1 = offsets[r + 1];
-  T acc[4] = {0, 0, 0, 0};
+  typename math_of<T>::type acc[4] = {0, 0, 0, 0};
   int64_t zz = z0;
   for (; zz + 8 <= z1; zz += 8) {
     V4 x[8];
@@ -67,30 +121,30 @@ __global__ void __launch_bounds__(256) segment_sum_rows_vec(const T* __restrict_
 #pragma unroll
     for (int k = 0; k < 8; ++k)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] += x[k].v[e];
+      for (int e = 0; e < 4; ++e) acc[e] += io_ld(&x[k].v[e]);
   }
   for (; zz < z1; ++zz) {
     const V4 x = *reinterpret_cast<const V4*>(partial + perm[zz] * width + c);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] += x.v[e];
+    for (int e = 0; e < 4; ++e) acc[e] += io_ld(&x.v[e]);
   }
   V4 o;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) o.v[e] = acc[e];
+  for (int e = 0; e < 4; ++e) io_st(acc[e], &o.v[e]);
   *reinterpret_cast<V4*>(out + r * width + c) = o;
 }
 
-// out[z, j] = sum over c in [0, nparts) of partial[(z * nparts + c), j]
-template <typename T>
+// out[z, j] = sum over c in [0, nparts) of partial[(z * nparts + c), j]   (partials in the arithmetic type)
+template <typename T, typename TO = T>
 __global__ void __launch_bounds__(256) fold_parts(const T* __restrict__ partial, int64_t n, int nparts, int width,
-                                                  T* __restrict__ out) {
+                                                  TO* __restrict__ out) {
   const int64_t tid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tid >= n * width) return;
   const int64_t z = tid / width;
   const int j = static_cast<int>(tid - z * width);
   T acc = 0;
   for (int c = 0; c < nparts; ++c) acc += partial[(z * nparts + c) * width + j];
-  out[tid] = acc;
+  io_st(acc, out + tid);
 }
 
 // p[0 .. n) = 0, 16 bytes per thread (element by element when p is not 16-byte aligned, and for the tail);
@@ -103,7 +157,7 @@ __global__ void __launch_bounds__(256) fill_zero(T* __restrict__ p, int64_t n) {
   if (i + V <= n && reinterpret_cast<uintptr_t>(p) % 16 == 0) {
     *reinterpret_cast<uint4*>(p + i) = make_uint4(0u, 0u, 0u, 0u);
   } else {
-    for (int64_t k = i; k < n && k < i + V; ++k) p[k] = 0;
+    for (int64_t k = i; k < n && k < i + V; ++k) p[k] = T{};
   }
 }
 
@@ -136,9 +190,5 @@ inline unsigned blocks_for(int64_t n, int per_block = 256) { return static_cast<
 // followed by a gather-sum in index order (bit-reproducible, one extra pass over batch x row).
 // A process-wide option (cueq_set_option("deterministic", ...); initial value from CUEQ_DETERMINISTIC, read once).
 bool deterministic_scatter();
-
-template <typename T> struct dtype_code;
-template <> struct dtype_code<float> { static constexpr int value = CUEQ_F32; };
-template <> struct dtype_code<double> { static constexpr int value = CUEQ_F64; };
 
 }  // namespace cueq

@@ -4,8 +4,9 @@
 // library is built, straight-line kernels are generated (cuequivariance_amd/codegen) with the
 // path table baked into the instruction stream; each generated translation unit registers
 // itself here under a content hash of the descriptor tables.  cueq_u1d_plan_create computes the
-// same hash and, when it finds an entry, cueq_u1d_run tries it first; the entry may decline a
-// call shape (returns CUEQ_ERR_UNSUPPORTED), in which case the generic kernels run.
+// same hash and, when it finds entries, cueq_u1d_run tries them first; an entry may decline a
+// call shape (returns CUEQ_ERR_UNSUPPORTED), in which case the generic kernels run.  One descriptor may have several
+// entries: one per element type of the buffers (the arithmetic type itself, and 16-bit elements for float arithmetic).
 #pragma once
 
 #include <cstdint>
@@ -27,10 +28,12 @@ struct U1dSpec {
   const char* name;
   int (*run)(const SpecCall& call);                                    // CUEQ_OK / CUEQ_ERR_UNSUPPORTED / error
   int64_t (*workspace)(const cueq_u1d_buffer* buffers, int64_t batch);  // bytes, may be null
+  int io_dtype;  // CUEQ_* code of the buffers this entry takes (all buffers of a call hold the same type)
 };
 
 void register_u1d_spec(const U1dSpec* spec);
-const U1dSpec* find_u1d_spec(uint64_t hash);
+// the entry for `hash` whose buffers hold `io_dtype`; io_dtype < 0: the one whose buffers hold the arithmetic type
+const U1dSpec* find_u1d_spec(uint64_t hash, int io_dtype = -1);
 
 // FNV-1a over a stream of 64-bit words (little endian bytes); the generator computes the same.
 struct Fnv64 {

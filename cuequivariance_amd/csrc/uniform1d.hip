@@ -40,14 +40,19 @@ static std::mutex& spec_mutex() {
   static std::mutex m;
   return m;
 }
+static std::atomic<uint64_t> g_spec_version{1};  // bumped by every registration: plans look their entries up again
 void register_u1d_spec(const U1dSpec* spec) {
   std::lock_guard<std::mutex> lock(spec_mutex());
   spec_list().push_back(spec);
+  g_spec_version.fetch_add(1, std::memory_order_release);
 }
-const U1dSpec* find_u1d_spec(uint64_t hash) {
+static bool spec_takes(const U1dSpec* s, int io_dtype) {
+  return io_dtype < 0 ? (s->io_dtype == CUEQ_F32 || s->io_dtype == CUEQ_F64) : s->io_dtype == io_dtype;
+}
+const U1dSpec* find_u1d_spec(uint64_t hash, int io_dtype) {
   std::lock_guard<std::mutex> lock(spec_mutex());
   for (const U1dSpec* s : spec_list())
-    if (s->hash == hash) return s;
+    if (s->hash == hash && spec_takes(s, io_dtype)) return s;
   return nullptr;
 }
 
@@ -294,11 +299,30 @@ struct cueq_u1d_plan {
   std::vector<int32_t> buffer_dim, buffer_nseg;
   std::vector<OutTables> out;  // one per output buffer
   std::vector<const int32_t*> seg_base, seg_stride;  // per buffer, device pointers (null: default layout)
-  const cueq::U1dSpec* spec = nullptr;  // descriptor-specialised kernels, if any were built
+  // descriptor-specialised kernels registered for these tables (one entry per element type of the buffers); looked up again
+  // whenever the registry has grown since, because units compiled at first use arrive while plans exist
+  static constexpr int kMaxSpecs = 4;
+  mutable std::atomic<const cueq::U1dSpec*> specs[kMaxSpecs] = {};
+  mutable std::atomic<int> nspecs{0};
+  mutable std::atomic<uint64_t> specs_version{0};
   uint64_t hash = 0;
   void* device_blob = nullptr;
   int device = 0;
 };
+
+// Number of entries of plan->specs, after looking them up again when the registry has changed since the last look.
+static int plan_specs(const cueq_u1d_plan* plan) {
+  const uint64_t now = g_spec_version.load(std::memory_order_acquire);
+  if (plan->specs_version.load(std::memory_order_acquire) != now) {
+    std::lock_guard<std::mutex> lock(spec_mutex());
+    int n = 0;  // (the registry only grows and keeps its order: entries already published keep their place)
+    for (const U1dSpec* sp : spec_list())
+      if (sp->hash == plan->hash && n < cueq_u1d_plan::kMaxSpecs) plan->specs[n++].store(sp, std::memory_order_relaxed);
+    plan->nspecs.store(n, std::memory_order_release);
+    plan->specs_version.store(g_spec_version.load(std::memory_order_acquire), std::memory_order_release);
+  }
+  return plan->nspecs.load(std::memory_order_acquire);
+}
 
 extern "C" const char* cueq_last_error(void) { return g_error.c_str(); }
 
@@ -503,9 +527,15 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
       plan->seg_stride[b] = plan->seg_base[b] + d->buffer_num_segments[b];
     }
   plan->hash = hash_u1d_desc(d);
-  plan->spec = find_u1d_spec(plan->hash);
+  (void)plan_specs(plan);
   *out_plan = plan;
   return CUEQ_OK;
+}
+
+// 1 when kernels generated for these tables are registered for buffers of `io_dtype` (a CUEQ_* code), else 0.  Host-only.
+extern "C" int cueq_u1d_desc_serves(const cueq_u1d_desc* d, int32_t io_dtype) {
+  if (!d || io_dtype < 0) return 0;
+  return find_u1d_spec(hash_u1d_desc(d), io_dtype) ? 1 : 0;
 }
 
 // Host-only: content hash of the descriptor tables and whether specialised kernels are linked in.
@@ -520,7 +550,10 @@ extern "C" int cueq_u1d_desc_info(const cueq_u1d_desc* d, uint64_t* hash) {
 extern "C" int cueq_u1d_plan_info(const cueq_u1d_plan* plan, uint64_t* hash) {
   if (!plan) return 0;
   if (hash) *hash = plan->hash;
-  return plan->spec ? 1 : 0;
+  const int n = plan_specs(plan);
+  for (int i = 0; i < n; ++i)
+    if (spec_takes(plan->specs[i].load(std::memory_order_relaxed), -1)) return 1;
+  return 0;
 }
 
 extern "C" void cueq_u1d_plan_destroy(cueq_u1d_plan* plan) {
@@ -535,7 +568,10 @@ extern "C" int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq
   if (!plan || !buffers) return 0;
   const int msize = plan->math_dtype == CUEQ_F64 ? 8 : 4;
   int64_t need = 0;
-  if (plan->spec && plan->spec->workspace) need = plan->spec->workspace(buffers, batch);
+  for (int i = 0, n = plan_specs(plan); i < n; ++i) {
+    const U1dSpec* sp = plan->specs[i].load(std::memory_order_relaxed);
+    if (sp->workspace) need = std::max<int64_t>(need, sp->workspace(buffers, batch));
+  }
   for (int ob = 0; ob < plan->num_outputs; ++ob) {
     const int b = plan->num_inputs + ob;
     if (buffers[b].batch_dim != CUEQ_BATCH_SHARED) continue;
@@ -642,10 +678,12 @@ extern "C" int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* bu
   CUEQ_REQUIRE(plan && buffers, CUEQ_ERR_INVALID, "null argument");
   CUEQ_REQUIRE(batch >= 0, CUEQ_ERR_INVALID, "negative batch size");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (plan->spec && !opt_force_generic().load(std::memory_order_relaxed)) {
+  if (!opt_force_generic().load(std::memory_order_relaxed)) {
     SpecCall call{buffers, batch, workspace, workspace_bytes, s};
-    const int rc = plan->spec->run(call);
-    if (rc != CUEQ_ERR_UNSUPPORTED) return rc;
+    for (int i = 0, n = plan_specs(plan); i < n; ++i) {
+      const int rc = plan->specs[i].load(std::memory_order_relaxed)->run(call);
+      if (rc != CUEQ_ERR_UNSUPPORTED) return rc;
+    }
   }
   if (plan->math_dtype == CUEQ_F64) return run_typed<double>(plan, buffers, batch, workspace, workspace_bytes, s);
   return run_typed<float>(plan, buffers, batch, workspace, workspace_bytes, s);

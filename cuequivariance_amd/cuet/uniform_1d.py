@@ -76,6 +76,7 @@ class Uniform1dPlan:
         self._handles: dict[int, int] = {}
         self._backward: dict[tuple, "Uniform1dPlan"] = {}
         self._choice: dict = {}
+        self._io_seen: set = set()  # 16-bit element types whose kernels were looked for (and compiled, when that is on)
         self.jit_root = None  # for a backward plan: the forward plan, whose translation unit holds its kernels
         self.polynomial = None  # the flattened polynomial the tables came from, when the caller has it
         self.origin = None      # the polynomial that one was flattened from (a fully connected product's descriptor)
@@ -130,6 +131,24 @@ class Uniform1dPlan:
                     "off (CUEQ_AMD_JIT=0 / cuequivariance_amd.jit.enable(False))",
                     stacklevel=2)
             return out.value
+
+    def ensure_io(self, dtype: torch.dtype) -> None:
+        """Kernels for buffers that all hold the 16-bit ``dtype`` while the arithmetic is float32: a unit of their own, linked
+        into the library for the registered descriptors, compiled at first use for others (when that is switched on).  The
+        device plans find such a unit as soon as it is registered."""
+        if self.math_dtype != torch.float32 or dtype not in (torch.bfloat16, torch.float16) or dtype in self._io_seen:
+            return
+        with self._lock:
+            if dtype not in self._io_seen:
+                if _jit.enabled():
+                    root = self.jit_root or self
+                    _jit.ensure_plan(self.tables, _DTYPE_CODE[self.math_dtype], root.tables, root.polynomial, root.origin,
+                                     io_code=_DTYPE_CODE[dtype])
+                self._io_seen.add(dtype)
+
+    def serves(self, dtype: torch.dtype) -> bool:
+        """True when kernels generated for exactly these tables and buffers of ``dtype`` are registered with the library."""
+        return _jit._has_spec(self.tables, _DTYPE_CODE[self.math_dtype], _DTYPE_CODE[dtype])
 
     def __del__(self):
         try:
@@ -326,6 +345,8 @@ def _launch(plan: Uniform1dPlan, cfg: _CallConfig, inputs: Sequence[torch.Tensor
         rec = pool.pop()  # (a record is used by one launch at a time: list.pop / append are atomic)
     except IndexError:
         rec = _LaunchRecord(plan, cfg, sig[0], sig[1])
+        if nin and sig[0][0].itemsize == 2 and all(d == sig[0][0] for d in sig[0]):
+            plan.ensure_io(sig[0][0])
     modes, widths = cfg.modes, plan.widths
     with _on_device(device):
         handle = plan._handles.get(device.index)

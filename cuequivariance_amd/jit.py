@@ -111,9 +111,16 @@ def _tuning(st, T: str) -> dict:
     return dict(fwd, **bwd)
 
 
-def _has_spec(t: U1dTables, code: int) -> bool:
+_IO_NAME = {_lib.BF16: "bf16", _lib.F16: "f16"}  # element types of buffers that differ from the (float) arithmetic type
+
+
+def _has_spec(t: U1dTables, code: int, io_code: Optional[int] = None) -> bool:
+    """Whether kernels generated for these tables are registered with the library: for buffers of the arithmetic type
+    ``code``, or of the 16-bit type ``io_code``."""
     desc, keep = _lib.make_desc(t, code)
-    return bool(_lib.load().cueq_u1d_desc_info(C.byref(desc), None))
+    if io_code is None or io_code == code:
+        return bool(_lib.load().cueq_u1d_desc_info(C.byref(desc), None))
+    return bool(_lib.load().cueq_u1d_desc_serves(C.byref(desc), io_code))
 
 
 def is_symmetric_contraction(poly) -> bool:
@@ -174,49 +181,59 @@ def has_fused_backward(t: U1dTables, polynomial=None, origin=None) -> bool:
 
 
 def ensure_plan(tables: U1dTables, math_code: int, root_tables: Optional[U1dTables] = None, root_polynomial=None,
-                root_origin=None) -> bool:
+                root_origin=None, io_code: Optional[int] = None) -> bool:
     """Kernels for one plan: first the family unit of its root (the forward plan of a channel-wise product or symmetric
     contraction holds the kernels of its backward plans too), then, if the plan still has none, a unit of its own from
-    the general generator (``codegen/general.py``: second derivatives, harmonics, flattened dense products, ...)."""
-    if _has_spec(tables, math_code):
+    the general generator (``codegen/general.py``: second derivatives, harmonics, flattened dense products, ...).
+    ``io_code``: the element type of the buffers when it is not the arithmetic type (bfloat16 / half with float arithmetic:
+    a unit of its own per element type)."""
+    if io_code == math_code:
+        io_code = None
+    if io_code is not None and (math_code != _lib.F32 or io_code not in _IO_NAME):
+        return False
+    if _has_spec(tables, math_code, io_code):
         return True
     if not enabled():
         return False
     if root_tables is not None and _family(root_tables, root_polynomial, root_origin):
-        ensure_specialised(root_tables, math_code, root_polynomial, origin=root_origin)
-        if _has_spec(tables, math_code):
+        ensure_specialised(root_tables, math_code, root_polynomial, origin=root_origin, io_code=io_code)
+        if _has_spec(tables, math_code, io_code):
             return True
-    return ensure_specialised(tables, math_code, None, general=True)
+    return ensure_specialised(tables, math_code, None, general=True, io_code=io_code)
 
 
-def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, general: bool = False, origin=None) -> bool:
+def ensure_specialised(tables: U1dTables, math_code: int, polynomial=None, general: bool = False, origin=None,
+                       io_code: Optional[int] = None) -> bool:
     """Make sure specialised kernels for ``tables`` (forward) and for its backward are registered with the library,
     compiling them if this module is enabled and the descriptor is a channel-wise product or (given the flattened
     ``polynomial`` the tables came from) a symmetric contraction - or, with ``general``, anything the general generator
     covers.  Returns whether they are."""
     from .codegen import general as gen
 
-    if _has_spec(tables, math_code):
+    if _has_spec(tables, math_code, io_code):
         return True
     family = _family(tables, polynomial, origin)
     if not enabled() or not (family or (general and gen.supported(tables))):
         return False
+    if io_code is not None and family == "fc_rows":
+        return False  # (that family is generated for buffers of the arithmetic type only)
     key = tables.content_hash(math_code)
+    slot = key if io_code is None else (key, io_code)
     with _lock:
-        if key in _loaded or _has_spec(tables, math_code):
+        if slot in _loaded or _has_spec(tables, math_code, io_code):
             return True
-        if key in _failed:
+        if slot in _failed:
             return False
         try:
-            _loaded[key] = _build_and_load(tables, math_code, key, polynomial, origin)
+            _loaded[slot] = _build_and_load(tables, math_code, key, polynomial, origin, _IO_NAME.get(io_code))
         except Exception as e:  # compilation is an optimisation: the table-driven kernels still serve the plan
-            _failed.add(key)
+            _failed.add(slot)
             print(f"[cueq_amd.jit] specialised kernels for descriptor {key:016x} not built: {e}", file=sys.stderr, flush=True)
             return False
-    return _has_spec(tables, math_code)
+    return _has_spec(tables, math_code, io_code)
 
 
-def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None, origin=None):
+def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None, origin=None, io: Optional[str] = None):
     from .codegen import channelwise as cw
     from .codegen import symmetric as sc
 
@@ -227,19 +244,19 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None, origin=N
     if family is None:
         from .codegen import general as gen
 
-        src = gen.emit_unit(t, T, name, key)
+        src = gen.emit_unit(t, T, name, key, io=io)
         what = f"general plan, {sum(t.num_paths)} paths, extent {t.operand_extent}"
     elif family == "channelwise":
         _, paths = t.operation(0)
         st = cw.analyze(t.operand_extent, t.buffer_num_segments, [(*idx, c) for idx, c in paths], t.layout(1), t.layout(3))
         tb = t.backward((True, True, True))
-        src = cw.emit_unit(st, T, name, key, tb.content_hash(code), **_tuning(st, T))
+        src = cw.emit_unit(st, T, name, key, tb.content_hash(code), io=io, **_tuning(st, T))
         what = f"{st.num_paths} paths, extent {st.extent}"
     elif family == "channelwise_sh":
         tp = U1dTables.from_polynomial(origin.product)
         _, paths = tp.operation(0)
         st = cw.analyze(tp.operand_extent, tp.buffer_num_segments, [(*idx, c) for idx, c in paths], t.layout(1), t.layout(3), origin.terms)
-        src = cw.emit_unit(st, T, name, key, t.backward((True, True, True)).content_hash(code), **_tuning(st, T))
+        src = cw.emit_unit(st, T, name, key, t.backward((True, True, True)).content_hash(code), io=io, **_tuning(st, T))
         what = f"{st.num_paths} paths, extent {st.extent}, spherical harmonics of degrees {list(origin.ls)} in the kernels"
     elif family == "fc_rows":
         from .codegen import fullyconnected_rows as fcr
@@ -250,11 +267,11 @@ def _build_and_load(t: U1dTables, code: int, key: int, polynomial=None, origin=N
     else:
         st = sc.analyze(polynomial, t.layout(1), t.layout(2))
         bwd = {(dw, dx): t.backward((dw, dx)).content_hash(code) for dw, dx in ((True, True), (True, False), (False, True))}
-        src = sc.emit_unit(st, T, name, key, bwd)
+        src = sc.emit_unit(st, T, name, key, bwd, io=io)
         what = f"symmetric contraction, {len(st.terms)} folded terms, extent {st.extent}"
-    so = cache_dir() / f"u1d_{name}_{T}_{hashlib.sha1(src.encode()).hexdigest()[:10]}.so"
+    so = cache_dir() / f"u1d_{name}_{io or T}_{hashlib.sha1(src.encode()).hexdigest()[:10]}.so"
     if not so.exists():
-        _compile(src, so, f"descriptor {key:016x} ({T}, {what})")
+        _compile(src, so, f"descriptor {key:016x} ({T}{', buffers of ' + io if io else ''}, {what})")
     _lib.load()  # the library the object links against is already in the process
     return C.CDLL(str(so))
 

@@ -131,6 +131,11 @@ void cueq_u1d_plan_destroy(cueq_u1d_plan* plan);
 int cueq_u1d_plan_info(const cueq_u1d_plan* plan, uint64_t* hash);
 /* Same answer from the tables alone; touches no device (usable on a host without a GPU). */
 int cueq_u1d_desc_info(const cueq_u1d_desc* desc, uint64_t* hash);
+/* The same question for buffers of one element type (a CUEQ_* code): the specialised kernels of a descriptor exist per
+ * element type of the buffers - the arithmetic type itself (what cueq_u1d_desc_info reports) and, for float arithmetic,
+ * bfloat16 and half (loaded and stored as 16-bit elements, computed in float: the reference's math_dtype=float32 with
+ * 16-bit tensors, cuequivariance_torch/primitives/segmented_polynomial_uniform_1d.py:254-260).  Host-only. */
+int cueq_u1d_desc_serves(const cueq_u1d_desc* desc, int32_t io_dtype);
 
 /* Bytes of device workspace cueq_u1d_run needs for this call shape (0 if none). */
 int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size);
