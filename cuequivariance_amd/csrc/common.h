@@ -38,6 +38,55 @@ __host__ __device__ inline int dtype_size(int dt) {
   return dt == CUEQ_F64 ? 8 : (dt == CUEQ_F32 ? 4 : 2);
 }
 
+// ---- 2-byte element formats of the matrix-core kernels ---------------------------------------------------------------
+// Those kernels move 2-byte elements as words; only the product instruction and the rounding of results depend on the
+// format.  The element type selects it: uint16_t = bfloat16 (as its bits), f16bits = IEEE half (as its bits).
+struct f16bits { uint16_t bits; };
+typedef float mm_floatx16 __attribute__((ext_vector_type(16)));
+typedef float mm_floatx4 __attribute__((ext_vector_type(4)));
+typedef float mm_floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 mm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 mm_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 mm_f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 mm_f16x2 __attribute__((ext_vector_type(2)));
+template <typename TI> struct is_half_bits { static constexpr bool value = false; };
+template <> struct is_half_bits<f16bits> { static constexpr bool value = true; };
+
+// acc += A (32 x 16) B (16 x 32), eight 2-byte elements per lane and operand
+template <typename TI>
+__device__ __forceinline__ mm_floatx16 mm_32x32x16(uint4 a, uint4 b, mm_floatx16 acc) {
+  if constexpr (is_half_bits<TI>::value)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(mm_f16x8, a), __builtin_bit_cast(mm_f16x8, b), acc, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(mm_bf16x8, a), __builtin_bit_cast(mm_bf16x8, b), acc, 0, 0, 0);
+}
+// acc += A (16 x 32) B (32 x 16)
+template <typename TI>
+__device__ __forceinline__ mm_floatx4 mm_16x16x32(uint4 a, uint4 b, mm_floatx4 acc) {
+  if constexpr (is_half_bits<TI>::value)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mm_f16x8, a), __builtin_bit_cast(mm_f16x8, b), acc, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mm_bf16x8, a), __builtin_bit_cast(mm_bf16x8, b), acc, 0, 0, 0);
+}
+// two floats rounded to nearest even and packed, `lo` in the low half (one conversion instruction)
+template <typename TI>
+__device__ __forceinline__ uint32_t mm_pack(float lo, float hi) {
+  const mm_floatx2 f = {lo, hi};
+  if constexpr (is_half_bits<TI>::value) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, mm_f16x2));
+  else return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, mm_bf16x2));
+}
+// one element widened to float / one float rounded to the format
+template <typename TI>
+__device__ __forceinline__ float mm_widen(uint16_t bits) {
+  if constexpr (is_half_bits<TI>::value) return static_cast<float>(__builtin_bit_cast(_Float16, bits));
+  else return __uint_as_float(static_cast<uint32_t>(bits) << 16);
+}
+template <typename TI>
+__device__ __forceinline__ uint16_t mm_round(float v) {
+  if constexpr (is_half_bits<TI>::value) return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+  else return __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
+}
+
 // bf16 <-> f32 by bit manipulation (round to nearest even on the way down).
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
   return __uint_as_float(static_cast<uint32_t>(b) << 16);

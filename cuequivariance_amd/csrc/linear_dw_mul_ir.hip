@@ -24,7 +24,6 @@ namespace cueq {
 namespace {
 
 typedef float dw_floatx16 __attribute__((ext_vector_type(16)));
-typedef __bf16 dw_bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kDwMaxParts = 32;
 // Blocks of up to this many components request their rows two steps ahead (two register sets); with five components the
@@ -176,7 +175,7 @@ __device__ __forceinline__ void dw_body(const TI* __restrict__ A, int64_t lda, c
 #pragma unroll
           for (int b = 0; b < TB; ++b) {
             if constexpr (ES == 2) {
-              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(dw_bf16x8, fa[a]), __builtin_bit_cast(dw_bf16x8, fb[b]), acc[a][b], 0, 0, 0);
+              acc[a][b] = mm_32x32x16<TI>(fa[a], fb[b], acc[a][b]);
             } else {
               acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(fa[a].x), __uint_as_float(fb[b].x), acc[a][b], 0, 0, 0);
               acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(fa[a].y), __uint_as_float(fb[b].y), acc[a][b], 0, 0, 0);
@@ -300,7 +299,7 @@ extern "C" int cueq_linear_dw_mul_ir(int32_t dtype, int64_t K, int64_t N, int64_
                                      const int64_t* table, int32_t nparts, float* partials, double alpha, void* stream_) {
   using namespace cueq;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "linear_dw_mul_ir: bfloat16 or float32");
+  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F16 || dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "linear_dw_mul_ir: bfloat16, half or float32");
   CUEQ_REQUIRE(rows >= 0 && nparts >= 1 && nparts <= kDwMaxParts, CUEQ_ERR_INVALID, "linear_dw_mul_ir: 1 to %d parts", kDwMaxParts);
   CUEQ_REQUIRE(K > 0 && N > 0 && K % 32 == 0 && N % 32 == 0 && K <= 128 && N <= 128, CUEQ_ERR_UNSUPPORTED,
                "linear_dw_mul_ir: K and N must be 32, 64, 96 or 128");
@@ -333,7 +332,7 @@ extern "C" int cueq_linear_dw_mul_ir(int32_t dtype, int64_t K, int64_t N, int64_
   } while (0)
 #define DW_D(TI_)                                                                         \
   switch (dmax) { case 1: DW(TI_, 1); break; case 3: DW(TI_, 3); break; case 5: DW(TI_, 5); break; default: DW(TI_, 7); break; }
-  if (dtype == CUEQ_F32) { DW_D(float) } else { DW_D(uint16_t) }
+  if (dtype == CUEQ_F32) { DW_D(float) } else if (dtype == CUEQ_F16) { DW_D(f16bits) } else { DW_D(uint16_t) }
 #undef DW_D
 #undef DW
   CUEQ_CHECK_HIP(hipGetLastError());

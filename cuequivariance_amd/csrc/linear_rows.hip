@@ -101,7 +101,7 @@ __device__ __forceinline__ void lr_unit(uint4 (&xs)[NV], const char* wl, char* s
       }
 #pragma unroll
       for (int v = 0; v < NV; ++v)
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(lr_bf16x8, af[t & 1][v]), __builtin_bit_cast(lr_bf16x8, xf[v]), acc, 0, 0, 0);
+        acc = mm_32x32x16<TI>(af[t & 1][v], xf[v], acc);
     } else {
 #pragma unroll
       for (int v = 0; v < NV; ++v) {
@@ -116,7 +116,7 @@ __device__ __forceinline__ void lr_unit(uint4 (&xs)[NV], const char* wl, char* s
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       if constexpr (ES == 2) {
-        const uint2 v = make_uint2(lr_pack(alpha * acc[4 * a], alpha * acc[4 * a + 1]), lr_pack(alpha * acc[4 * a + 2], alpha * acc[4 * a + 3]));
+        const uint2 v = make_uint2(mm_pack<TI>(alpha * acc[4 * a], alpha * acc[4 * a + 1]), mm_pack<TI>(alpha * acc[4 * a + 2], alpha * acc[4 * a + 3]));
         *reinterpret_cast<uint2*>(stage + c * SRS + ((t * 32) % SC + 8 * a + 4 * h) * 2) = v;
       } else {
         *reinterpret_cast<float4*>(stage + c * SRS + (8 * a + 4 * h) * 4) =
@@ -242,7 +242,7 @@ extern "C" int cueq_linear_rows(int32_t dtype, int32_t w_contraction_major, int6
                                 const void* W, int64_t w_numel, void* C, int64_t ldc, const int64_t* table, int64_t nparts, double alpha, void* stream_) {
   using namespace cueq;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "linear_rows: bfloat16 or float32");
+  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F16 || dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "linear_rows: bfloat16, half or float32");
   CUEQ_REQUIRE(M >= 0 && N > 0 && K > 0 && nparts >= 0, CUEQ_ERR_INVALID, "linear_rows: bad extents");
   CUEQ_REQUIRE(N % 32 == 0 && K % 32 == 0 && N <= 128 && K <= 128, CUEQ_ERR_UNSUPPORTED, "linear_rows: K and N must be 32, 64, 96 or 128");
   CUEQ_REQUIRE(nparts <= kLrMaxParts, CUEQ_ERR_TOO_LARGE, "linear_rows: at most %d parts per launch", kLrMaxParts);
@@ -292,7 +292,7 @@ extern "C" int cueq_linear_rows(int32_t dtype, int32_t w_contraction_major, int6
     case 3: LR_N(TI_, 3); break;   \
     default: LR_N(TI_, 4); break;  \
   }
-  if (dtype == CUEQ_F32) { LR_K(float) } else { LR_K(uint16_t) }
+  if (dtype == CUEQ_F32) { LR_K(float) } else if (dtype == CUEQ_F16) { LR_K(f16bits) } else { LR_K(uint16_t) }
 #undef LR_K
 #undef LR_N
 #undef LR

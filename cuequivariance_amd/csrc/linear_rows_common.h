@@ -9,9 +9,7 @@ namespace cueq {
 namespace {
 
 typedef float lr_floatx16 __attribute__((ext_vector_type(16)));
-typedef __bf16 lr_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float lr_floatx2 __attribute__((ext_vector_type(2)));
-typedef __bf16 lr_bf16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t lr_u32x4 __attribute__((ext_vector_type(4)));
 
 // 16-byte accesses marked as streams: every byte of A and C is touched once
@@ -35,11 +33,6 @@ struct LrParts {
   LrPart part[kLrMaxParts];
   int64_t w_off[kLrMaxSlots];
 };
-
-__device__ __forceinline__ uint32_t lr_pack(float lo, float hi) {
-  const lr_floatx2 f = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, lr_bf16x2));
-}
 
 // The weight blocks of a launch into LDS as rows of K elements (one row per result column, WRS bytes apart), 16-byte
 // vectors requested in batches of four before the first is stored (one wait per batch instead of one per vector).

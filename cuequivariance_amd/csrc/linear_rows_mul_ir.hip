@@ -143,7 +143,7 @@ struct MiWork {
           wk += 16 * WRS;
 #pragma unroll
           for (int i = 0; i < D; ++i)
-            acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lr_bf16x8, wf), __builtin_bit_cast(lr_bf16x8, xop[i]), acc[i][t], 0, 0, 0);
+            acc[i][t] = mm_16x16x32<TI>(wf, xop[i], acc[i][t]);
           if (t % 2 == 1) __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -193,7 +193,7 @@ struct MiWork {
         if constexpr (ES == 2) {
 #pragma unroll
           for (int w = 0; w < D; ++w)
-            *reinterpret_cast<uint2*>(dst + 8 * w) = make_uint2(lr_pack(val[4 * w], val[4 * w + 1]), lr_pack(val[4 * w + 2], val[4 * w + 3]));
+            *reinterpret_cast<uint2*>(dst + 8 * w) = make_uint2(mm_pack<TI>(val[4 * w], val[4 * w + 1]), mm_pack<TI>(val[4 * w + 2], val[4 * w + 3]));
         } else {
 #pragma unroll
           for (int w = 0; w < D; ++w)
@@ -351,7 +351,7 @@ extern "C" int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_majo
                                        void* stream_) {
   using namespace cueq;
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "linear_rows_mul_ir: bfloat16 or float32");
+  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F16 || dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "linear_rows_mul_ir: bfloat16, half or float32");
   CUEQ_REQUIRE(M >= 0 && N > 0 && K > 0 && nparts >= 0, CUEQ_ERR_INVALID, "linear_rows_mul_ir: bad extents");
   const int es = dtype == CUEQ_F32 ? 4 : 2, epv = 16 / es, us = 128 / es;
   CUEQ_REQUIRE(N % 32 == 0 && N <= 128 && K % us == 0 && K <= 128, CUEQ_ERR_UNSUPPORTED,
@@ -435,7 +435,7 @@ extern "C" int cueq_linear_rows_mul_ir(int32_t dtype, int32_t w_contraction_majo
     case 5: MI_N(TI_, 5); break;  \
     default: MI_N(TI_, 7); break; \
   }
-  if (dtype == CUEQ_F32) { MI_D(float) } else { MI_D(uint16_t) }
+  if (dtype == CUEQ_F32) { MI_D(float) } else if (dtype == CUEQ_F16) { MI_D(f16bits) } else { MI_D(uint16_t) }
 #undef MI_D
 #undef MI_N
 #undef MI
