@@ -26,8 +26,12 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ float tri_load(const float* p, int64_t i) { return p[i]; }
 __device__ __forceinline__ float tri_load(const uint16_t* p, int64_t i) { return bf16_bits_to_float(p[i]); }
+__device__ __forceinline__ float tri_load(const f16bits* p, int64_t i) { return mm_widen<f16bits>(p[i].bits); }
+__device__ __forceinline__ uint16_t raw16(uint16_t v) { return v; }  // the bits of a 2-byte element
+__device__ __forceinline__ uint16_t raw16(f16bits v) { return v.bits; }
 __device__ __forceinline__ void tri_store(float* p, int64_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void tri_store(uint16_t* p, int64_t i, float v) { p[i] = float_to_bf16_bits(v); }
+__device__ __forceinline__ void tri_store(f16bits* p, int64_t i, float v) { p[i].bits = mm_round<f16bits>(v); }
 
 // ------------------------------------------------------------------------------------------------
 // C[b] (M x N) = alpha * A[b] (M x K, row stride lda) * B[b]^T (N x K, row stride ldb)  (+ C[b])
@@ -61,9 +65,19 @@ __device__ __forceinline__ void xcd_tile(int& bx, int& by, int& bz) {
 // ------------------------------------------------------------------------------------------------
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {  // round to nearest even, one v_cvt_pk_bf16_f32
-  const floatx2_t f = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+// Two floats rounded to nearest even and packed (one conversion instruction), and the halves of such a word as floats;
+// F selects the 2-byte format: uint16_t = bfloat16, f16bits = half.
+template <typename F>
+__device__ __forceinline__ uint32_t pack16(float lo, float hi) { return mm_pack<F>(lo, hi); }
+template <typename F>
+__device__ __forceinline__ float lo16(uint32_t w) {
+  if constexpr (is_half_bits<F>::value) return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w & 0xffffu)));
+  else return __uint_as_float(w << 16);
+}
+template <typename F>
+__device__ __forceinline__ float hi16(uint32_t w) {
+  if constexpr (is_half_bits<F>::value) return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16)));
+  else return __uint_as_float(w & 0xffff0000u);
 }
 
 // The value again, as far as the compiler can tell a new one: the two floats of a packed pair are then unpacked where they
@@ -93,16 +107,15 @@ __device__ __forceinline__ float ln_rstd(float sumsq, float inv_d, float eps) { 
 __device__ __forceinline__ float ln_affine(float centered, float rs, float gm, float bt) {
   return __fadd_rn(__fmul_rn(__fmul_rn(centered, rs), gm), bt);
 }
-__device__ __forceinline__ float lo_bf16(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float hi_bf16(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
 template <typename TO>
 __device__ __forceinline__ void stage_put(char* tile, int row_stride, int col, int h, const floatx16& acc, float alpha) {
+  using F = TO;
 #pragma unroll
   for (int v = 0; v < 16; v += 2) {
     char* p = tile + (8 * (v >> 2) + 4 * h + (v & 3)) * row_stride + col * static_cast<int>(sizeof(TO));
     if constexpr (sizeof(TO) == 2) {
-      const uint32_t w = pack_bf16(alpha * acc[v], alpha * acc[v + 1]);
+      const uint32_t w = pack16<F>(alpha * acc[v], alpha * acc[v + 1]);
       *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(w & 0xffffu);
       *reinterpret_cast<uint16_t*>(p + row_stride) = static_cast<uint16_t>(w >> 16);
     } else {
@@ -114,13 +127,14 @@ __device__ __forceinline__ void stage_put(char* tile, int row_stride, int col, i
 
 template <typename TO>
 __device__ __forceinline__ uint4 add_vec(uint4 a, uint4 b) {
+  using F = TO;
   if constexpr (sizeof(TO) == 2) {
     const uint32_t x[4] = {a.x, a.y, a.z, a.w}, y[4] = {b.x, b.y, b.z, b.w};
     uint32_t r[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      r[e] = pack_bf16(__uint_as_float(x[e] << 16) + __uint_as_float(y[e] << 16),
-                       __uint_as_float(x[e] & 0xffff0000u) + __uint_as_float(y[e] & 0xffff0000u));
+      r[e] = pack16<F>(lo16<F>(x[e]) + lo16<F>(y[e]),
+                       hi16<F>(x[e]) + hi16<F>(y[e]));
     return make_uint4(r[0], r[1], r[2], r[3]);
   } else {
     return make_uint4(__float_as_uint(__uint_as_float(a.x) + __uint_as_float(b.x)), __float_as_uint(__uint_as_float(a.y) + __uint_as_float(b.y)),
@@ -200,6 +214,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
                                                    float alpha, int accumulate, int vec_out, int64_t k_total, int nparts, int64_t pA,
                                                    int64_t pB, int64_t pC, const int64_t* __restrict__ goff, int ngroups, int gmode,
                                                    int64_t gsB, int64_t gsC) {
+  using F = TI;
   constexpr int EPV = 16 / sizeof(TI);  // elements per 16-byte vector
   constexpr int BK = KB / sizeof(TI);   // k extent of one step
   constexpr int RB = KB + 16;           // bytes between the rows of a contraction-contiguous tile
@@ -316,8 +331,7 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_kernel(const TI* __restrict
         for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[i][q]),
-                                                                __builtin_bit_cast(bf16x8_t, fb[j][q]), acc[i][j], 0, 0, 0);
+            acc[i][j] = mm_32x32x16<F>(fa[i][q], fb[j][q], acc[i][j]);
       } else {
 #pragma unroll
         for (int s = 0; s < 4; ++s)
@@ -383,13 +397,14 @@ __device__ __forceinline__ void tn_load8(const float* p, float* r) {
   const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
   r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w; r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
 }
-__device__ __forceinline__ void tn_load8(const uint16_t* p, float* r) {
+template <typename F>
+__device__ __forceinline__ void tn_load8(const F* p, float* r) {
   const uint4 a = *reinterpret_cast<const uint4*>(p);
   const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    r[2 * e] = __uint_as_float(w[e] << 16);
-    r[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+    r[2 * e] = lo16<F>(w[e]);
+    r[2 * e + 1] = hi16<F>(w[e]);
   }
 }
 
@@ -397,6 +412,7 @@ template <typename TI, bool VEC>
 __global__ void __launch_bounds__(256) gemm_tn_kernel(const TI* __restrict__ A, int64_t lda, int64_t sA, const TI* __restrict__ B,
                                                       int64_t ldb, int64_t sB, float* __restrict__ P, int M, int N, int64_t rows,
                                                       int64_t rows_per_chunk, int nparts, float alpha) {
+  using F = TI;
   __shared__ __align__(16) float sa[kTnRows][kTile + 4];
   __shared__ __align__(16) float sb[kTnRows][kTile + 4];
   const int tid = threadIdx.x;
@@ -496,6 +512,7 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
                                                            const TI* __restrict__ mask, int mask_axis, const TI* __restrict__ dC,
                                                            TI* __restrict__ out1, TI* __restrict__ out2, int64_t ldc, int M, int N, int K,
                                                            int vec_out) {
+  using F = TI;
   // 8 wavefronts of 64 x 32 (both products): half the accumulators per wavefront of the plain GEMM tiling, so two
   // blocks fit a CU and one block's epilogue overlaps the other's loads.
   constexpr int EPV = 16 / sizeof(TI);
@@ -570,8 +587,7 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
         if constexpr (sizeof(TI) == 2) {
 #pragma unroll
           for (int q = 0; q < 2; ++q)
-            acc[p][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa[i][q]),
-                                                                __builtin_bit_cast(bf16x8_t, fb[q]), acc[p][i], 0, 0, 0);
+            acc[p][i] = mm_32x32x16<F>(fa[i][q], fb[q], acc[p][i]);
         } else {
 #pragma unroll
           for (int q = 0; q < 2; ++q) {
@@ -653,8 +669,9 @@ __global__ void __launch_bounds__(512, 4) dual_gate_kernel(const TI* __restrict_
 // ------------------------------------------------------------------------------------------------
 template <typename TI>
 __device__ __forceinline__ void mma_step(floatx16& acc, const uint4& a, const uint4& b) {
+  using F = TI;
   if constexpr (sizeof(TI) == 2) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+    acc = mm_32x32x16<F>(a, b, acc);
   } else {
     const float* pa = reinterpret_cast<const float*>(&a);
     const float* pb = reinterpret_cast<const float*>(&b);
@@ -707,6 +724,7 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
                           const TI* __restrict__ bias1, const TI* __restrict__ bias2, const TI* __restrict__ mask,
                           const TI* __restrict__ dC, int64_t ldc, TI* __restrict__ dX1, TI* __restrict__ dX2,
                           int64_t lddx, int accumulate, TI* __restrict__ dU, TI* __restrict__ dV, int C, int M) {
+  using F = TI;
   constexpr bool BF = sizeof(TI) == 2;
   constexpr int EPV = 16 / sizeof(TI);
   constexpr int K = 32 * KT;
@@ -755,7 +773,7 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
     if (tid < 64) {
       float bv = 0.f;
       if (has_bias) {
-        if constexpr (BF) bv = bf16_bits_to_float(stb);
+        if constexpr (BF) bv = mm_widen<F>(raw16(stb));
         else bv = stb;
       }
       *reinterpret_cast<float*>(&smem[buf][BIAS + tid * 4]) = bv;
@@ -817,9 +835,9 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
   auto dc_value = [&](int v) -> float {
     if constexpr (!BF) return __uint_as_float(dcr[v]);
     else {
-      if constexpr (DC_BY_ROW) return __uint_as_float(dcr[v] << 16);
+      if constexpr (DC_BY_ROW) return lo16<F>(dcr[v]);
       const uint32_t w = dcr[4 * (v >> 2) + ((v & 3) >> 1)];
-      return (v & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+      return (v & 1) ? hi16<F>(w) : lo16<F>(w);
     }
   };
 
@@ -884,8 +902,8 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
         }
       }
       if constexpr (BF) {
-        pu[2 * a] = pack_bf16(du[0], du[1]); pu[2 * a + 1] = pack_bf16(du[2], du[3]);
-        pv[2 * a] = pack_bf16(dv[0], dv[1]); pv[2 * a + 1] = pack_bf16(dv[2], dv[3]);
+        pu[2 * a] = pack16<F>(du[0], du[1]); pu[2 * a + 1] = pack16<F>(du[2], du[3]);
+        pv[2 * a] = pack16<F>(dv[0], dv[1]); pv[2 * a + 1] = pack16<F>(dv[2], dv[3]);
       }
     }
     // second product: rows m (lanes of the operand), contraction over the 32 rows c of the chunk
@@ -969,17 +987,17 @@ __global__ void __launch_bounds__((gbi_threads<TI, SPLIT>()), (gbi_waves_per_sim
 // goes on to the gradient with respect to those input rows - the lane has half of the gradient row in registers, so the two
 // row sums of the LayerNorm backward are sums over its own values completed by one exchange - and writes that to dX1.
 // ------------------------------------------------------------------------------------------------
-template <int KT, bool SPLIT, bool DC_BY_ROW, bool LNB = false>
+template <typename F, int KT, bool SPLIT, bool DC_BY_ROW, bool LNB = false>
 __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
-    gate_bwd_input_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X1,
-                              const uint16_t* __restrict__ X2, int64_t ldx, const uint16_t* __restrict__ bias1,
-                              const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask, const uint16_t* __restrict__ dC,
-                              int64_t ldc, uint16_t* __restrict__ dX1, uint16_t* __restrict__ dX2, int64_t lddx, int accumulate,
-                              uint16_t* __restrict__ dU, uint16_t* __restrict__ dV, int C, int M, const uint16_t* __restrict__ ln_x = nullptr,
+    gate_bwd_input_res_kernel(const F* __restrict__ W1, const F* __restrict__ W2, int64_t ldw, const F* __restrict__ X1,
+                              const F* __restrict__ X2, int64_t ldx, const F* __restrict__ bias1,
+                              const F* __restrict__ bias2, const F* __restrict__ mask, const F* __restrict__ dC,
+                              int64_t ldc, F* __restrict__ dX1, F* __restrict__ dX2, int64_t lddx, int accumulate,
+                              F* __restrict__ dU, F* __restrict__ dV, int C, int M, const F* __restrict__ ln_x = nullptr,
                               int64_t ldlx = 0, const float* __restrict__ ln_mean = nullptr, const float* __restrict__ ln_rstd = nullptr,
-                              const uint16_t* __restrict__ ln_gamma = nullptr) {
+                              const F* __restrict__ ln_gamma = nullptr) {
   static_assert(!(LNB && SPLIT), "the LayerNorm backward goes with the one-input form");
-  using TI = uint16_t;
+  using TI = F;
   constexpr int ES = 2, EPV = 8;
   constexpr int K = 32 * KT, ROWB = K * ES, NS = ROWB / 64, VPR = ROWB / 16;
   // weight rows in LDS: 256-byte rows keep their 16-byte units XOR-swizzled by a rotation of the row's low four bits
@@ -1057,7 +1075,7 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   };
   auto dc_value = [&](int v) -> float {
     const uint32_t w = dcr[v >> 1];
-    return (v & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+    return (v & 1) ? hi16<F>(w) : lo16<F>(w);
   };
   // the rows of X of a tile, one row per lane, and its mask value (as stored: converted where it is used, so that the
   // request is not followed by a wait).  The registers are free once the last chunk's first product has read them:
@@ -1073,7 +1091,7 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
         xf1[s2][q] = *reinterpret_cast<const uint4*>(X1 + o);
         if constexpr (SPLIT) xf2[s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
       }
-    if (mask) mraw = mask[mld];
+    if (mask) mraw = raw16(mask[mld]);
   };
   int64_t tile = ptile;
   if (tile < ntiles) request_x(tile_row(tile));
@@ -1082,7 +1100,7 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
   for (; tile < ntiles; tile += tstep) {
     const int mrow0 = static_cast<int>(tile * 32);
     const int mcol = mrow0 + c;
-    const float mk = mask ? __uint_as_float(mraw << 16) : 1.0f;
+    const float mk = mask ? lo16<F>(mraw) : 1.0f;
     floatx16 ax1[KT], ax2[SPLIT ? KT : 1];
 #pragma unroll
     for (int t = 0; t < KT; ++t) ax1[t] = floatx16{0};
@@ -1134,8 +1152,8 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
           dv[b] = dc_value(v) * mk * sg;
           du[b] = dv[b] * fmaf(-av[v], sg, av[v]);
         }
-        pu[2 * a] = pack_bf16(du[0], du[1]); pu[2 * a + 1] = pack_bf16(du[2], du[3]);
-        pv[2 * a] = pack_bf16(dv[0], dv[1]); pv[2 * a + 1] = pack_bf16(dv[2], dv[3]);
+        pu[2 * a] = pack16<F>(du[0], du[1]); pu[2 * a + 1] = pack16<F>(du[2], du[3]);
+        pv[2 * a] = pack16<F>(dv[0], dv[1]); pv[2 * a + 1] = pack16<F>(dv[2], dv[3]);
         if (dU != nullptr) {
           const int row = c0 + 8 * a + 4 * h;
           if constexpr (!DC_BY_ROW) {
@@ -1202,14 +1220,14 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
       // other form, 32 bytes per row and instruction, measure 5 % slower here.)
 #pragma unroll
       for (int which = 0; which < 2; ++which) {
-        uint16_t* dst = which == 0 ? dX1 : dX2;
+        F* dst = which == 0 ? dX1 : dX2;
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
           __builtin_amdgcn_wave_barrier();
 #pragma unroll
           for (int ds = 0; ds < KT; ++ds) {
             const floatx16& acc = (which == 0) ? ax1[ds] : ax2[ds];
-            const uint32_t w01 = pack_bf16(acc[4 * a], acc[4 * a + 1]), w23 = pack_bf16(acc[4 * a + 2], acc[4 * a + 3]);
+            const uint32_t w01 = pack16<F>(acc[4 * a], acc[4 * a + 1]), w23 = pack16<F>(acc[4 * a + 2], acc[4 * a + 3]);
             char* p = stage + (4 * h) * SSTR + (ds * 32 + c) * 2;
             *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(w01 & 0xffffu);
             *reinterpret_cast<uint16_t*>(p + SSTR) = static_cast<uint16_t>(w01 >> 16);
@@ -1269,9 +1287,9 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               float d = acc[8 * j + e];
-              if (accumulate) d += (e & 1) ? hi_bf16(ow[e >> 1]) : lo_bf16(ow[e >> 1]);
+              if (accumulate) d += (e & 1) ? hi16<F>(ow[e >> 1]) : lo16<F>(ow[e >> 1]);
               const float g = d * gm[e];
-              const float xn = (((e & 1) ? hi_bf16(xw[e >> 1]) : lo_bf16(xw[e >> 1])) - mu) * rs;
+              const float xn = (((e & 1) ? hi16<F>(xw[e >> 1]) : lo16<F>(xw[e >> 1])) - mu) * rs;
               s1 += g;
               s2 = fmaf(g, xn, s2);
               acc[8 * j + e] = g;
@@ -1289,8 +1307,8 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
             uint32_t o[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              const float x0 = (lo_bf16(xw[e]) - mu) * rs, x1 = (hi_bf16(xw[e]) - mu) * rs;
-              o[e] = pack_bf16(rs * (acc[8 * j + 2 * e] - s1 - x0 * s2), rs * (acc[8 * j + 2 * e + 1] - s1 - x1 * s2));
+              const float x0 = (lo16<F>(xw[e]) - mu) * rs, x1 = (hi16<F>(xw[e]) - mu) * rs;
+              o[e] = pack16<F>(rs * (acc[8 * j + 2 * e] - s1 - x0 * s2), rs * (acc[8 * j + 2 * e + 1] - s1 - x1 * s2));
             }
             val[ds][j] = make_uint4(o[0], o[1], o[2], o[3]);
           }
@@ -1301,8 +1319,8 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
         const floatx16& acc = ax1[ds];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          const uint32_t p0 = pack_bf16(acc[8 * j], acc[8 * j + 1]), p1 = pack_bf16(acc[8 * j + 2], acc[8 * j + 3]);
-          const uint32_t p2 = pack_bf16(acc[8 * j + 4], acc[8 * j + 5]), p3 = pack_bf16(acc[8 * j + 6], acc[8 * j + 7]);
+          const uint32_t p0 = pack16<F>(acc[8 * j], acc[8 * j + 1]), p1 = pack16<F>(acc[8 * j + 2], acc[8 * j + 3]);
+          const uint32_t p2 = pack16<F>(acc[8 * j + 4], acc[8 * j + 5]), p3 = pack16<F>(acc[8 * j + 6], acc[8 * j + 7]);
           const auto s0 = __builtin_amdgcn_permlane32_swap(p0, p2, false, false);
           const auto s1 = __builtin_amdgcn_permlane32_swap(p1, p3, false, false);
           val[ds][j] = make_uint4(s0[0], s1[0], s0[1], s1[1]);
@@ -1336,14 +1354,14 @@ __global__ void __launch_bounds__((SPLIT ? 256 : 512), (SPLIT ? 1 : 2))
 // normalised in the registers, rounded to the 2-byte type - the operand of the products, exactly what a separate
 // LayerNorm launch would have written - and stored with their mean and 1 / std for the later stages.
 // ------------------------------------------------------------------------------------------------
-template <int KT, bool LN, bool ROWS>
+template <typename F, int KT, bool LN, bool ROWS>
 __global__ void __launch_bounds__(512, 2)
-    dual_gate_res_kernel(const uint16_t* __restrict__ W1, const uint16_t* __restrict__ W2, int64_t ldw, const uint16_t* __restrict__ X,
-                         const uint16_t* __restrict__ X2, int64_t ldx, const uint16_t* __restrict__ bias1, const uint16_t* __restrict__ bias2, const uint16_t* __restrict__ mask,
-                         uint16_t* __restrict__ out, int64_t ldc, int C, int M, const uint16_t* __restrict__ gamma,
-                         const uint16_t* __restrict__ beta, float eps, uint16_t* __restrict__ xhat, int64_t ldxh, float* __restrict__ mean,
+    dual_gate_res_kernel(const F* __restrict__ W1, const F* __restrict__ W2, int64_t ldw, const F* __restrict__ X,
+                         const F* __restrict__ X2, int64_t ldx, const F* __restrict__ bias1, const F* __restrict__ bias2, const F* __restrict__ mask,
+                         F* __restrict__ out, int64_t ldc, int C, int M, const F* __restrict__ gamma,
+                         const F* __restrict__ beta, float eps, F* __restrict__ xhat, int64_t ldxh, float* __restrict__ mean,
                          float* __restrict__ rstd) {
-  using TI = uint16_t;
+  using TI = F;
   constexpr int ES = 2, EPV = 8;
   constexpr int K = 32 * KT, ROWB = K * ES, NS = ROWB / 64, VPR = ROWB / 16;
   constexpr bool SWZ = KT == 4;  // (same layout of the weight rows as gate_bwd_input_res_kernel)
@@ -1399,7 +1417,7 @@ __global__ void __launch_bounds__(512, 2)
           xn[t][s2][q] = *reinterpret_cast<const uint4*>(X + o);
           if constexpr (ROWS) xn2[t][s2][q] = *reinterpret_cast<const uint4*>(X2 + o);
         }
-      if (mask) mraw[t] = mask[mld];
+      if (mask) mraw[t] = raw16(mask[mld]);
     }
   };
   // (tiles dealt out wavefront-major: the tiles worked on at one time lie next to each other in memory and are spread over
@@ -1420,7 +1438,7 @@ __global__ void __launch_bounds__(512, 2)
           xf[t][s2][q] = xn[t][s2][q];
           if constexpr (ROWS) xf2[t][s2][q] = xn2[t][s2][q];
         }
-      mk[t] = mask ? __uint_as_float(mraw[t] << 16) : 1.0f;
+      mk[t] = mask ? lo16<F>(mraw[t]) : 1.0f;
     }
     request_x(min(tile + tstep, ntiles - 1));  // (past the end: the last tile again, so that the request is unconditional)
     if constexpr (LN) {
@@ -1447,7 +1465,7 @@ __global__ void __launch_bounds__(512, 2)
 #pragma unroll
           for (int q = 0; q < 2; ++q) {
             const uint32_t w[4] = {xf[t][s2][q].x, xf[t][s2][q].y, xf[t][s2][q].z, xf[t][s2][q].w};
-            const float v[8] = {lo_bf16(w[0]), hi_bf16(w[0]), lo_bf16(w[1]), hi_bf16(w[1]), lo_bf16(w[2]), hi_bf16(w[2]), lo_bf16(w[3]), hi_bf16(w[3])};
+            const float v[8] = {lo16<F>(w[0]), hi16<F>(w[0]), lo16<F>(w[1]), hi16<F>(w[1]), lo16<F>(w[2]), hi16<F>(w[2]), lo16<F>(w[3]), hi16<F>(w[3])};
             gs[s2][q] = ln_sum8(v);
           }
         const float mu = __fmul_rn(tree(gs), 1.0f / K);
@@ -1456,7 +1474,7 @@ __global__ void __launch_bounds__(512, 2)
 #pragma unroll
           for (int q = 0; q < 2; ++q) {
             const uint32_t w[4] = {again(xf[t][s2][q].x), again(xf[t][s2][q].y), again(xf[t][s2][q].z), again(xf[t][s2][q].w)};
-            float v[8] = {lo_bf16(w[0]), hi_bf16(w[0]), lo_bf16(w[1]), hi_bf16(w[1]), lo_bf16(w[2]), hi_bf16(w[2]), lo_bf16(w[3]), hi_bf16(w[3])};
+            float v[8] = {lo16<F>(w[0]), hi16<F>(w[0]), lo16<F>(w[1]), hi16<F>(w[1]), lo16<F>(w[2]), hi16<F>(w[2]), lo16<F>(w[3]), hi16<F>(w[3])};
             gs[s2][q] = ln_center_sq8(v, mu);
           }
         const float rs = ln_rstd(tree(gs), 1.0f / K, eps);
@@ -1474,8 +1492,8 @@ __global__ void __launch_bounds__(512, 2)
             uint32_t o[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              o[e] = pack_bf16(ln_affine(__fsub_rn(lo_bf16(w[e]), mu), rs, gm[2 * e], bt[2 * e]),
-                               ln_affine(__fsub_rn(hi_bf16(w[e]), mu), rs, gm[2 * e + 1], bt[2 * e + 1]));
+              o[e] = pack16<F>(ln_affine(__fsub_rn(lo16<F>(w[e]), mu), rs, gm[2 * e], bt[2 * e]),
+                               ln_affine(__fsub_rn(hi16<F>(w[e]), mu), rs, gm[2 * e + 1], bt[2 * e + 1]));
             xf[t][s2][q] = make_uint4(o[0], o[1], o[2], o[3]);
             if (mcol[t] < M) *reinterpret_cast<uint4*>(xhat + static_cast<int64_t>(mld) * ldxh + (s2 * 64 + h * 32 + q * 16) / ES) = xf[t][s2][q];
             __builtin_amdgcn_sched_barrier(0);  // one piece at a time: its gamma / beta values die here
@@ -1525,8 +1543,8 @@ __global__ void __launch_bounds__(512, 2)
             const int v = 4 * a + b;
             g[b] = __builtin_amdgcn_rcpf(1.0f + __expf(-au[0][v])) * av[0][v] * mk[0];
           }
-          pk[2 * a] = pack_bf16(g[0], g[1]);
-          pk[2 * a + 1] = pack_bf16(g[2], g[3]);
+          pk[2 * a] = pack16<F>(g[0], g[1]);
+          pk[2 * a + 1] = pack16<F>(g[2], g[3]);
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -1546,7 +1564,7 @@ __global__ void __launch_bounds__(512, 2)
             const int v = 4 * a + b;
             g[b] = __builtin_amdgcn_rcpf(1.0f + __expf(-au[t][v])) * av[t][v] * mk[t];
           }
-          const uint32_t own[2] = {pack_bf16(g[0], g[1]), pack_bf16(g[2], g[3])};
+          const uint32_t own[2] = {pack16<F>(g[0], g[1]), pack16<F>(g[2], g[3])};
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
             const uint32_t other = static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(own[j]), 0xB1, 0xF, 0xF, true));
@@ -1745,12 +1763,13 @@ __device__ __forceinline__ void ln_store8(float* p, const float* r) {
   *reinterpret_cast<float4*>(p) = make_float4(r[0], r[1], r[2], r[3]);
   *reinterpret_cast<float4*>(p + 4) = make_float4(r[4], r[5], r[6], r[7]);
 }
-__device__ __forceinline__ void ln_store8(uint16_t* p, const float* r) {
+template <typename F>
+__device__ __forceinline__ void ln_store8(F* p, const float* r) {
   uint4 o;
-  o.x = float_to_bf16_bits(r[0]) | (static_cast<uint32_t>(float_to_bf16_bits(r[1])) << 16);
-  o.y = float_to_bf16_bits(r[2]) | (static_cast<uint32_t>(float_to_bf16_bits(r[3])) << 16);
-  o.z = float_to_bf16_bits(r[4]) | (static_cast<uint32_t>(float_to_bf16_bits(r[5])) << 16);
-  o.w = float_to_bf16_bits(r[6]) | (static_cast<uint32_t>(float_to_bf16_bits(r[7])) << 16);
+  o.x = mm_round<F>(r[0]) | (static_cast<uint32_t>(mm_round<F>(r[1])) << 16);
+  o.y = mm_round<F>(r[2]) | (static_cast<uint32_t>(mm_round<F>(r[3])) << 16);
+  o.z = mm_round<F>(r[4]) | (static_cast<uint32_t>(mm_round<F>(r[5])) << 16);
+  o.w = mm_round<F>(r[6]) | (static_cast<uint32_t>(mm_round<F>(r[7])) << 16);
   *reinterpret_cast<uint4*>(p) = o;
 }
 template <int L>
@@ -1768,6 +1787,7 @@ template <typename T, int L>
 __global__ void __launch_bounds__(256) ln_fwd_rows8(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
                                                     T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd, int64_t rows,
                                                     float eps) {
+  using F = T;
   constexpr int D = 8 * L, RPW = 64 / L;
   const int lane = threadIdx.x & 63, sub = lane / L, col = (lane % L) * 8;
   const int64_t row = (static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6)) * RPW + sub;
@@ -1799,6 +1819,7 @@ template <typename T, int L>
 __global__ void __launch_bounds__(256) ln_bwd_rows8(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ mean,
                                                     const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
                                                     float* __restrict__ part, int64_t rows, int rows_per_block) {
+  using F = T;
   constexpr int D = 8 * L, RPW = 64 / L;
   extern __shared__ float sred[];  // [4 waves][2][D]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane / L, col = (lane % L) * 8;
@@ -1882,7 +1903,8 @@ struct LnT {
 
 template <typename T>
 __device__ __forceinline__ float lnt_tile(const char* tile, int d, int m) {
-  if constexpr (sizeof(T) == 2) return bf16_bits_to_float(*reinterpret_cast<const uint16_t*>(tile + d * LnT<T>::RS + m * 2));
+  using F = T;
+  if constexpr (sizeof(T) == 2) return mm_widen<F>(*reinterpret_cast<const uint16_t*>(tile + d * LnT<T>::RS + m * 2));
   else return *reinterpret_cast<const float*>(tile + d * LnT<T>::RS + m * 4);
 }
 
@@ -1904,6 +1926,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) ln_t_fwd_kernel(const T* __restrict__ xt, const T* __restrict__ gamma, const T* __restrict__ beta,
                                                        T* __restrict__ y, float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int D,
                                                        float eps) {
+  using F = T;
   using L = LnT<T>;
   extern __shared__ __align__(16) char lnt_dyn[];  // D * RS bytes: the x tile
   char* tile = lnt_dyn;
@@ -1963,7 +1986,7 @@ __global__ void __launch_bounds__(256) ln_t_fwd_kernel(const T* __restrict__ xt,
       o[e] = (lnt_tile<T>(tile, d, r) - mu2) * rs * sgam[d] + sbet[d];
     }
     uint4 out;
-    if constexpr (sizeof(T) == 2) out = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+    if constexpr (sizeof(T) == 2) out = make_uint4(pack16<F>(o[0], o[1]), pack16<F>(o[2], o[3]), pack16<F>(o[4], o[5]), pack16<F>(o[6], o[7]));
     else out = make_uint4(__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3]));
     *reinterpret_cast<uint4*>(y + (m0 + r) * D + v * L::EPV) = out;
   }
@@ -1973,6 +1996,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) ln_t_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ xt, const float* __restrict__ mean,
                                                        const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dxt,
                                                        float* __restrict__ part, int64_t M, int D, int64_t ntiles, int need_affine) {
+  using F = T;
   using L = LnT<T>;
   constexpr int PW = 4 / sizeof(T);  // elements per 4-byte store along m
   extern __shared__ __align__(16) char lnt_dyn[];  // the x tile (D * RS bytes, rounded up to 16), then the dy tile (MT * DS)
@@ -1986,7 +2010,7 @@ __global__ void __launch_bounds__(256) ln_t_bwd_kernel(const T* __restrict__ dy,
   const int DS = D * static_cast<int>(sizeof(T)) + 4;  // bytes between rows of the dy tile
   const int vpr = D / L::EPV;
   auto dyv = [&](int m, int d) -> float {
-    if constexpr (sizeof(T) == 2) return bf16_bits_to_float(*reinterpret_cast<const uint16_t*>(dtile + m * DS + d * 2));
+    if constexpr (sizeof(T) == 2) return mm_widen<F>(*reinterpret_cast<const uint16_t*>(dtile + m * DS + d * 2));
     else return *reinterpret_cast<const float*>(dtile + m * DS + d * 4);
   };
   float sg[(kLnTMaxD + 255) / 256] = {0}, sb[(kLnTMaxD + 255) / 256] = {0};  // this thread's d: partial dgamma / dbeta
@@ -2051,7 +2075,7 @@ __global__ void __launch_bounds__(256) ln_t_bwd_kernel(const T* __restrict__ dy,
             o[e] = rs[e] * (dyv(mm, d) * gmm - k1[e] - xh * k2[e]);
           }
           uint32_t w;
-          if constexpr (sizeof(T) == 2) w = pack_bf16(o[0], o[1]);
+          if constexpr (sizeof(T) == 2) w = pack16<F>(o[0], o[1]);
           else w = __float_as_uint(o[0]);
           *reinterpret_cast<uint32_t*>(dxt + static_cast<int64_t>(d) * M + mg) = w;
         }
@@ -2116,8 +2140,8 @@ struct LnCols {
 // the H dwords of lane (cp, dh) for the tile at column m0 (which every lane of the wavefront shares); LAST: nothing reads
 // x_t after this kernel (the backward: marked as a stream 45 instead of 47 us; in the forward, which reads what the
 // contraction has just written, the mark costs 9 us)
-template <int D, bool LAST = false>
-__device__ __forceinline__ void lncols_request(uint32_t (&xv)[D / 2], const uint16_t* xt, int64_t m0, int64_t row_bytes, uint32_t voff) {
+template <int D, bool LAST = false, typename F>
+__device__ __forceinline__ void lncols_request(uint32_t (&xv)[D / 2], const F* xt, int64_t m0, int64_t row_bytes, uint32_t voff) {
   // (one scalar base that walks down the rows; the scheduling barriers keep every address next to its load - computed
   // all at once, the D / 2 bases would not fit the scalar registers)
   const char* src = uniform_ptr(xt + m0);
@@ -2129,9 +2153,9 @@ __device__ __forceinline__ void lncols_request(uint32_t (&xv)[D / 2], const uint
   }
 }
 
-template <int D>
-__global__ void __launch_bounds__(256, 2) ln_t_fwd_cols_kernel(const uint16_t* __restrict__ xt, const uint16_t* __restrict__ gamma,
-                                                               const uint16_t* __restrict__ beta, uint16_t* __restrict__ y, float* __restrict__ mean,
+template <typename F, int D>
+__global__ void __launch_bounds__(256, 2) ln_t_fwd_cols_kernel(const F* __restrict__ xt, const F* __restrict__ gamma,
+                                                               const F* __restrict__ beta, F* __restrict__ y, float* __restrict__ mean,
                                                                float* __restrict__ rstd, int64_t M, float eps) {
   using L = LnCols<D>;
   constexpr int H = L::H, RS = L::RS;
@@ -2159,7 +2183,7 @@ __global__ void __launch_bounds__(256, 2) ln_t_fwd_cols_kernel(const uint16_t* _
     const int64_t m0 = tile * 64;
     float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-    for (int i = 0; i < H; ++i) { s0 += lo_bf16(xv[i]); s1 += hi_bf16(xv[i]); }
+    for (int i = 0; i < H; ++i) { s0 += lo16<F>(xv[i]); s1 += hi16<F>(xv[i]); }
     s0 += __shfl_xor(s0, 32, 64);
     s1 += __shfl_xor(s1, 32, 64);
     const float mu0 = s0 * (1.0f / D), mu1 = s1 * (1.0f / D);
@@ -2167,7 +2191,7 @@ __global__ void __launch_bounds__(256, 2) ln_t_fwd_cols_kernel(const uint16_t* _
 #pragma unroll
     for (int i = 0; i < H; ++i) {
       const uint32_t w = again(xv[i]);
-      const float c0 = lo_bf16(w) - mu0, c1 = hi_bf16(w) - mu1;
+      const float c0 = lo16<F>(w) - mu0, c1 = hi16<F>(w) - mu1;
       q0 = fmaf(c0, c0, q0);
       q1 = fmaf(c1, c1, q1);
     }
@@ -2186,8 +2210,8 @@ __global__ void __launch_bounds__(256, 2) ln_t_fwd_cols_kernel(const uint16_t* _
         const int i = p * 8 + 2 * e;
         const float ga = gam[i], gb = gam[i + 1], ba = bet[i], bb = bet[i + 1];
         const uint32_t xa_ = again(xv[i]), xb_ = again(xv[i + 1]);
-        w0[e] = pack_bf16((lo_bf16(xa_) - mu0) * r0 * ga + ba, (lo_bf16(xb_) - mu0) * r0 * gb + bb);
-        w1[e] = pack_bf16((hi_bf16(xa_) - mu1) * r1 * ga + ba, (hi_bf16(xb_) - mu1) * r1 * gb + bb);
+        w0[e] = pack16<F>((lo16<F>(xa_) - mu0) * r0 * ga + ba, (lo16<F>(xb_) - mu0) * r0 * gb + bb);
+        w1[e] = pack16<F>((hi16<F>(xa_) - mu1) * r1 * ga + ba, (hi16<F>(xb_) - mu1) * r1 * gb + bb);
       }
       *reinterpret_cast<uint4*>(stage + cp * RS + dh * D + p * 16) = make_uint4(w0[0], w0[1], w0[2], w0[3]);
       *reinterpret_cast<uint4*>(stage + (32 + cp) * RS + dh * D + p * 16) = make_uint4(w1[0], w1[1], w1[2], w1[3]);
@@ -2226,10 +2250,10 @@ __global__ void __launch_bounds__(256, 2) ln_t_fwd_cols_kernel(const uint16_t* _
   if (mine % 2) work(xa, tile);
 }
 
-template <int D>
-__global__ void __launch_bounds__(256, 2) ln_t_bwd_cols_kernel(const uint16_t* __restrict__ dy, const uint16_t* __restrict__ xt,
+template <typename F, int D>
+__global__ void __launch_bounds__(256, 2) ln_t_bwd_cols_kernel(const F* __restrict__ dy, const F* __restrict__ xt,
                                                                const float* __restrict__ mean, const float* __restrict__ rstd,
-                                                               const uint16_t* __restrict__ gamma, uint16_t* __restrict__ dxt, int64_t M) {
+                                                               const F* __restrict__ gamma, F* __restrict__ dxt, int64_t M) {
   using L = LnCols<D>;
   constexpr int H = L::H, RS = L::RS;
   extern __shared__ __align__(16) char lntc_dyn[];  // 4 wavefronts x WAVE_LDS
@@ -2279,12 +2303,12 @@ __global__ void __launch_bounds__(256, 2) ln_t_bwd_cols_kernel(const uint16_t* _
     auto dy_at = [&](int j, int i) -> float {  // value i of the lane's half
       const uint4 q = dv[j][i >> 3];
       const uint32_t w = ((i >> 1) & 3) == 0 ? q.x : ((i >> 1) & 3) == 1 ? q.y : ((i >> 1) & 3) == 2 ? q.z : q.w;
-      return (i & 1) ? hi_bf16(w) : lo_bf16(w);
+      return (i & 1) ? hi16<F>(w) : lo16<F>(w);
     };
     auto dy_at2 = [&](int j, int i) -> float {  // the same for the second pass
       const uint4 q = dv[j][i >> 3];
       const uint32_t w = again(((i >> 1) & 3) == 0 ? q.x : ((i >> 1) & 3) == 1 ? q.y : ((i >> 1) & 3) == 2 ? q.z : q.w);
-      return (i & 1) ? hi_bf16(w) : lo_bf16(w);
+      return (i & 1) ? hi16<F>(w) : lo16<F>(w);
     };
     float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
 #pragma unroll
@@ -2293,8 +2317,8 @@ __global__ void __launch_bounds__(256, 2) ln_t_bwd_cols_kernel(const uint16_t* _
       const float g0 = dy_at(0, i) * g, g1 = dy_at(1, i) * g;
       a0 += g0;
       a1 += g1;
-      b0 = fmaf(g0, (lo_bf16(xv[i]) - mu.x) * rs.x, b0);
-      b1 = fmaf(g1, (hi_bf16(xv[i]) - mu.y) * rs.y, b1);
+      b0 = fmaf(g0, (lo16<F>(xv[i]) - mu.x) * rs.x, b0);
+      b1 = fmaf(g1, (hi16<F>(xv[i]) - mu.y) * rs.y, b1);
       if (i % 8 == 7) __builtin_amdgcn_sched_barrier(0);
     }
     a0 += __shfl_xor(a0, 32, 64);
@@ -2308,9 +2332,9 @@ __global__ void __launch_bounds__(256, 2) ln_t_bwd_cols_kernel(const uint16_t* _
       for (int i = 0; i < H; ++i) {
         const float g = gam[i];
         const uint32_t w = again(xv[i]);
-        const float xh0 = (lo_bf16(w) - mu.x) * rs.x, xh1 = (hi_bf16(w) - mu.y) * rs.y;
+        const float xh0 = (lo16<F>(w) - mu.x) * rs.x, xh1 = (hi16<F>(w) - mu.y) * rs.y;
         const float o0 = rs.x * (dy_at2(0, i) * g - k10 - xh0 * k20), o1 = rs.y * (dy_at2(1, i) * g - k11 - xh1 * k21);
-        store_global<uint32_t>(dst, voff, pack_bf16(o0, o1));
+        store_global<uint32_t>(dst, voff, pack16<F>(o0, o1));
         dst += row_bytes;
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -2425,7 +2449,7 @@ __global__ void __launch_bounds__(256) fold_partials_kernel(const float* __restr
   tri_store(out, i, s);
 }
 
-static bool is_io(int dt) { return dt == CUEQ_F32 || dt == CUEQ_BF16; }
+static bool is_io(int dt) { return dt == CUEQ_F32 || dt == CUEQ_BF16 || dt == CUEQ_F16; }
 // rows one launch takes when its row tiles sit on grid.y (65535 tiles of 128; a multiple of every tile height used)
 constexpr int64_t kRowSlab = 65280ll * 128;
 
@@ -2433,16 +2457,18 @@ constexpr int64_t kRowSlab = 65280ll * 128;
 
 using namespace cueq;
 
-#define TRI_DISPATCH(dt, CALL_F32, CALL_BF16)      \
+// 2-byte element types: uint16_t = bfloat16 as its bits, f16bits = half as its bits
+#define TRI_DISPATCH(dt, CALL_F32, CALL_BF16, CALL_F16)      \
   do {                                             \
-    if ((dt) == CUEQ_F32) { CALL_F32; } else { CALL_BF16; } \
+    if ((dt) == CUEQ_F32) { CALL_F32; } else if ((dt) == CUEQ_F16) { CALL_F16; } else { CALL_BF16; } \
   } while (0)
 
 extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, int32_t trans_b, int64_t M, int64_t N, int64_t K,
                          const void* A, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b, void* C,
                          int64_t ldc, int64_t stride_c, int64_t batch, double alpha, int32_t accumulate, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm: dtypes must be float32 or bfloat16");
+  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm: dtypes must be float32, bfloat16 or half");
+  CUEQ_REQUIRE(in_dtype == out_dtype || in_dtype == CUEQ_F32 || out_dtype == CUEQ_F32, CUEQ_ERR_UNSUPPORTED, "gemm: bfloat16 and half do not mix");
   CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 0, CUEQ_ERR_INVALID, "gemm: negative extent");
   if (M == 0 || N == 0 || batch == 0) return CUEQ_OK;
   CUEQ_REQUIRE(A && B && C, CUEQ_ERR_INVALID, "gemm: null operand");
@@ -2476,7 +2502,7 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
   const float al = static_cast<float>(alpha);
   const int m = static_cast<int>(M), n = static_cast<int>(N), k = static_cast<int>(K);
   const bool mixed = in_dtype != out_dtype;
-  const bool mixed_ok = !mixed || (!trans_a && !trans_b) || (in_dtype == CUEQ_BF16 && out_dtype == CUEQ_F32 && !trans_a && trans_b);
+  const bool mixed_ok = !mixed || (!trans_a && !trans_b) || (in_dtype != CUEQ_F32 && out_dtype == CUEQ_F32 && !trans_a && trans_b);
   if (aligned && mixed_ok) {
     const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(batch));
     CUEQ_REQUIRE(grid.y < 65536, CUEQ_ERR_TOO_LARGE, "gemm: too many row tiles (M <= 8388480)");
@@ -2485,15 +2511,18 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
     // 256 x 256 tiles when both extents are multiples of 256 and there are enough of them to fill the chip
     const bool big = !mixed && M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) * batch >= 2 * static_cast<int64_t>(device_cus());
     // (the timing label names the tile size, so a test can tell which kernel a shape ran on)
-    KernelTimer timer(in_dtype == CUEQ_F32 ? (big ? "gemm_nt_f32_256" : "gemm_nt_f32") : (big ? "gemm_nt_bf16_256" : "gemm_nt_bf16"), stream);
+    KernelTimer timer(in_dtype == CUEQ_F32 ? (big ? "gemm_nt_f32_256" : "gemm_nt_f32") : in_dtype == CUEQ_F16 ? (big ? "gemm_nt_f16_256" : "gemm_nt_f16") : (big ? "gemm_nt_bf16_256" : "gemm_nt_bf16"), stream);
     const dim3 grid_big(static_cast<unsigned>(N / 256), static_cast<unsigned>(M / 256), static_cast<unsigned>(batch));
 #define GEMM_ARGS(TI, TO) static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate, vec_out, 0, 1, 0, 0, 0, nullptr, 0, 0, 0, 0
 #define GEMM_LAUNCH(TI, TO, TA, TB) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, GEMM_ARGS(TI, TO))
 #define GEMM_SZ(TI, TA, TB) do { if (big) hipLaunchKernelGGL((gemm_kernel<TI, TI, TA, TB, 4, 4, (sizeof(TI) == 2 ? 128 : 64)>), grid_big, dim3(1024), 0, stream, GEMM_ARGS(TI, TI)); else GEMM_LAUNCH(TI, TI, TA, TB); } while (0)
 #define GEMM_TR(TI) do { if (trans_a && trans_b) GEMM_SZ(TI, true, true); else if (trans_a) GEMM_SZ(TI, true, false); else if (trans_b) GEMM_SZ(TI, false, true); else GEMM_SZ(TI, false, false); } while (0)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_TR(float);
+    else if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F16) GEMM_LAUNCH(float, f16bits, false, false);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t, false, false);
+    else if (in_dtype == CUEQ_F16 && out_dtype == CUEQ_F32) { if (trans_b) GEMM_LAUNCH(f16bits, float, false, true); else GEMM_LAUNCH(f16bits, float, false, false); }
     else if (out_dtype == CUEQ_F32) { if (trans_b) GEMM_LAUNCH(uint16_t, float, false, true); else GEMM_LAUNCH(uint16_t, float, false, false); }
+    else if (in_dtype == CUEQ_F16) GEMM_TR(f16bits);
     else GEMM_TR(uint16_t);
 #undef GEMM_TR
 #undef GEMM_SZ
@@ -2507,8 +2536,11 @@ extern "C" int cueq_gemm(int32_t in_dtype, int32_t out_dtype, int32_t trans_a, i
     const int64_t rsa = trans_a ? 1 : lda, ksa = trans_a ? lda : 1, rsb = trans_b ? 1 : ldb, ksb = trans_b ? ldb : 1;
 #define GEMM_LAUNCH(TI, TO) hipLaunchKernelGGL((gemm_simple<TI, TO>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), rsa, ksa, stride_a, static_cast<const TI*>(B), rsb, ksb, stride_b, static_cast<TO*>(C), ldc, stride_c, m, n, k, al, accumulate)
     if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F32) GEMM_LAUNCH(float, float);
+    else if (in_dtype == CUEQ_F32 && out_dtype == CUEQ_F16) GEMM_LAUNCH(float, f16bits);
     else if (in_dtype == CUEQ_F32) GEMM_LAUNCH(float, uint16_t);
+    else if (in_dtype == CUEQ_F16 && out_dtype == CUEQ_F32) GEMM_LAUNCH(f16bits, float);
     else if (out_dtype == CUEQ_F32) GEMM_LAUNCH(uint16_t, float);
+    else if (in_dtype == CUEQ_F16) GEMM_LAUNCH(f16bits, f16bits);
     else GEMM_LAUNCH(uint16_t, uint16_t);
 #undef GEMM_LAUNCH
   }
@@ -2527,7 +2559,7 @@ extern "C" int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t tran
                                int64_t nparts, int64_t k_chunks, int64_t chunk_stride_c, double alpha, int32_t accumulate, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   CUEQ_REQUIRE(is_io(in_dtype) && (out_dtype == in_dtype || out_dtype == CUEQ_F32), CUEQ_ERR_UNSUPPORTED,
-               "gemm_table: float32 or bfloat16 operands, result of the same type or float32");
+               "gemm_table: float32, bfloat16 or half operands, result of the same type or float32");
   CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && nparts >= 0 && k_chunks >= 1, CUEQ_ERR_INVALID, "gemm_table: bad extents");
   if (M == 0 || N == 0 || nparts == 0) return CUEQ_OK;
   CUEQ_REQUIRE(A && B && C && table, CUEQ_ERR_INVALID, "gemm_table: null operand");
@@ -2565,6 +2597,7 @@ extern "C" int cueq_gemm_table(int32_t in_dtype, int32_t out_dtype, int32_t tran
 #define GT(TI, TO, TA, TB) do { if (skinny) hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB, 4, 1>), grid_s, dim3(256), 0, stream, GT_ARGS(TI, TO)); else hipLaunchKernelGGL((gemm_kernel<TI, TO, TA, TB>), grid, dim3(256), 0, stream, GT_ARGS(TI, TO)); } while (0)
 #define GT_T(TI, TO) do { if (small) hipLaunchKernelGGL((gemm_kernel<TI, TO, true, true, 1, 1>), grid_1, dim3(64), 0, stream, GT_ARGS(TI, TO)); else if (trans_a && trans_b) GT(TI, TO, true, true); else if (trans_b) GT(TI, TO, false, true); else GT(TI, TO, false, false); } while (0)
   if (in_dtype == CUEQ_F32) GT_T(float, float);
+  else if (in_dtype == CUEQ_F16) { if (out_dtype == CUEQ_F32) GT_T(f16bits, float); else GT_T(f16bits, f16bits); }
   else if (out_dtype == CUEQ_F32) GT_T(uint16_t, float);
   else GT_T(uint16_t, uint16_t);
 #undef GT_T
@@ -2579,7 +2612,7 @@ extern "C" int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mo
                                  int64_t batch, const int64_t* offsets, int64_t ngroups, int32_t trans_b, int64_t group_stride, double alpha,
                                  int32_t accumulate, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm_grouped: dtypes must be float32 or bfloat16");
+  CUEQ_REQUIRE(is_io(in_dtype) && is_io(out_dtype), CUEQ_ERR_UNSUPPORTED, "gemm_grouped: dtypes must be float32, bfloat16 or half");
   CUEQ_REQUIRE(mode == 1 || mode == 2, CUEQ_ERR_INVALID, "gemm_grouped: mode must be 1 (rows grouped) or 2 (contraction grouped)");
   CUEQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch >= 1 && ngroups >= 0, CUEQ_ERR_INVALID, "gemm_grouped: bad extents");
   if (M == 0 || N == 0 || ngroups == 0) return CUEQ_OK;
@@ -2603,6 +2636,7 @@ extern "C" int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mo
     const int vec_out = (reinterpret_cast<uintptr_t>(C) % 16 == 0 && (ldc * out_es) % 16 == 0 && (stride_c * out_es) % 16 == 0) ? 1 : 0;
 #define GG(TI, TB) hipLaunchKernelGGL((gemm_kernel<TI, TI, false, TB>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, static_cast<TI*>(C), ldc, stride_c, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), al, accumulate, vec_out, 0, 1, 0, 0, 0, offsets, static_cast<int>(ngroups), 1, group_stride, 0)
     if (in_dtype == CUEQ_F32) { if (trans_b) GG(float, true); else GG(float, false); }
+    else if (in_dtype == CUEQ_F16) { if (trans_b) GG(f16bits, true); else GG(f16bits, false); }
     else { if (trans_b) GG(uint16_t, true); else GG(uint16_t, false); }
 #undef GG
   } else {
@@ -2614,6 +2648,7 @@ extern "C" int cueq_gemm_grouped(int32_t in_dtype, int32_t out_dtype, int32_t mo
     const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile), static_cast<unsigned>((M + kTile - 1) / kTile), static_cast<unsigned>(ngroups * batch));
 #define GK(TI, TO) hipLaunchKernelGGL((gemm_kernel<TI, TO, true, true>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, 0, static_cast<const TI*>(B), ldb, 0, static_cast<TO*>(C), ldc, 0, static_cast<int>(M), static_cast<int>(N), 0, al, accumulate, 0, 0, static_cast<int>(batch), stride_a, stride_b, stride_c, offsets, static_cast<int>(ngroups), 2, 0, group_stride)
     if (in_dtype == CUEQ_F32) GK(float, float);
+    else if (in_dtype == CUEQ_F16) { if (out_dtype == CUEQ_F32) GK(f16bits, float); else GK(f16bits, f16bits); }
     else if (out_dtype == CUEQ_F32) GK(uint16_t, float);
     else GK(uint16_t, uint16_t);
 #undef GK
@@ -2633,19 +2668,21 @@ static bool dual_gate_res_fits(int64_t C, int64_t M, int64_t K, const void* out,
 }
 static int launch_dual_gate_res(int64_t C, int64_t M, int64_t K, const void* W1, const void* W2, int64_t ldw, const void* X, const void* X2,
                                 int64_t ldx, const void* bias1, const void* bias2, const void* mask, void* out, int64_t ldc, const void* gamma,
-                                const void* beta, float eps, void* xhat, int64_t ldxh, float* mean, float* rstd, hipStream_t stream) {
+                                const void* beta, float eps, void* xhat, int64_t ldxh, float* mean, float* rstd, bool half, hipStream_t stream) {
   const bool by_rows = X2 != nullptr;
   const size_t lds = dual_gate_res_lds(C, K, xhat != nullptr);
   const int64_t ntiles = (M + (by_rows ? 31 : 63)) / (by_rows ? 32 : 64);
   int64_t gx = (ntiles + 7) / 8;
   if (gx > device_cus()) gx = device_cus();
-#define DGR(KT, LN, RW) do { auto kfn = dual_gate_res_kernel<KT, LN, RW>; \
+#define DGR_F(FT, KT, LN, RW) do { auto kfn = dual_gate_res_kernel<FT, KT, LN, RW>; \
     CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<uint16_t*>(out), ldc, static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), eps, static_cast<uint16_t*>(xhat), ldxh, mean, rstd); } while (0)
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const FT*>(W1), static_cast<const FT*>(W2), ldw, static_cast<const FT*>(X), static_cast<const FT*>(X2), ldx, static_cast<const FT*>(bias1), static_cast<const FT*>(bias2), static_cast<const FT*>(mask), static_cast<FT*>(out), ldc, static_cast<int>(C), static_cast<int>(M), static_cast<const FT*>(gamma), static_cast<const FT*>(beta), eps, static_cast<FT*>(xhat), ldxh, mean, rstd); } while (0)
+#define DGR(KT, LN, RW) do { if (half) DGR_F(f16bits, KT, LN, RW); else DGR_F(uint16_t, KT, LN, RW); } while (0)
 #define DGR_K(LN, RW) do { switch (K / 32) { case 1: DGR(1, LN, RW); break; case 2: DGR(2, LN, RW); break; case 3: DGR(3, LN, RW); break; default: DGR(4, LN, RW); break; } } while (0)
   if (by_rows) DGR_K(false, true); else if (xhat) DGR_K(true, false); else DGR_K(false, false);
 #undef DGR_K
 #undef DGR
+#undef DGR_F
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }
@@ -2683,19 +2720,19 @@ extern "C" int cueq_dual_gate(int32_t dtype, int32_t backward, int64_t M, int64_
   KernelTimer timer(backward ? "dual_gate_bwd" : "dual_gate_fwd", stream);
   // forward with one shared right operand, biases along the rows and the mask along the columns, in a 2-byte type:
   // the left operands (the weights, M rows) stay resident in LDS when they fit
-  if (dtype == CUEQ_BF16 && !backward && share && (!(bias1 || bias2) || bias_axis == 0) && (!mask || mask_axis == 1) &&
+  if (dtype != CUEQ_F32 && !backward && share && (!(bias1 || bias2) || bias_axis == 0) && (!mask || mask_axis == 1) &&
       dual_gate_res_fits(M, N, K, out1, ldc, false, false)) {
-    return launch_dual_gate_res(M, N, K, A1, A2, lda, B1, nullptr, ldb, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, stream);
+    return launch_dual_gate_res(M, N, K, A1, A2, lda, B1, nullptr, ldb, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, dtype == CUEQ_F16, stream);
   }
   // the mirrored case - two left operands of many rows, the weights on the right, biases along the columns and the mask
   // along the rows: the same kernel with the weights (N rows) resident, two inputs and the result by rows
-  if (dtype == CUEQ_BF16 && !backward && !share && A2 != A1 && (!(bias1 || bias2) || bias_axis == 1) && (!mask || mask_axis == 0) && M <= kRowSlab &&
+  if (dtype != CUEQ_F32 && !backward && !share && A2 != A1 && (!(bias1 || bias2) || bias_axis == 1) && (!mask || mask_axis == 0) && M <= kRowSlab &&
       dual_gate_res_fits(N, M, K, out1, ldc, false, true)) {
-    return launch_dual_gate_res(N, M, K, B1, B2, ldb, A1, A2, lda, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, stream);
+    return launch_dual_gate_res(N, M, K, B1, B2, ldb, A1, A2, lda, bias1, bias2, mask, out1, ldc, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, dtype == CUEQ_F16, stream);
   }
 #define DG(TI, BW, SH) hipLaunchKernelGGL((dual_gate_kernel<TI, BW, SH>), grid, dim3(512), 0, stream, static_cast<const TI*>(A1), static_cast<const TI*>(A2), lda, static_cast<const TI*>(B1), static_cast<const TI*>(B2), ldb, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), bias_axis, static_cast<const TI*>(mask), mask_axis, static_cast<const TI*>(dC), static_cast<TI*>(out1), static_cast<TI*>(out2), ldc, static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), vec_out)
 #define DG_T(TI) do { if (backward) { if (share) DG(TI, true, true); else DG(TI, true, false); } else { if (share) DG(TI, false, true); else DG(TI, false, false); } } while (0)
-  TRI_DISPATCH(dtype, DG_T(float), DG_T(uint16_t));
+  TRI_DISPATCH(dtype, DG_T(float), DG_T(uint16_t), DG_T(f16bits));
 #undef DG_T
 #undef DG
   CUEQ_CHECK_HIP(hipGetLastError());
@@ -2706,7 +2743,7 @@ extern "C" int cueq_ln_dual_gate(int32_t dtype, int64_t C, int64_t M, int64_t K,
                                  int64_t ldx, const void* gamma, const void* beta, double eps, const void* bias1, const void* bias2,
                                  const void* mask, void* out, int64_t ldc, void* xhat, int64_t ldxh, float* mean, float* rstd, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(dtype == CUEQ_BF16, CUEQ_ERR_UNSUPPORTED, "ln_dual_gate: built for bfloat16 (compose cueq_layer_norm_fwd and cueq_dual_gate otherwise)");
+  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F16, CUEQ_ERR_UNSUPPORTED, "ln_dual_gate: built for bfloat16 and half (compose cueq_layer_norm_fwd and cueq_dual_gate otherwise)");
   CUEQ_REQUIRE(C > 0 && M >= 0 && K > 0, CUEQ_ERR_INVALID, "ln_dual_gate: bad extents");
   if (M == 0) return CUEQ_OK;
   CUEQ_REQUIRE(W1 && W2 && X && out && xhat && mean && rstd, CUEQ_ERR_INVALID, "ln_dual_gate: null operand");
@@ -2717,7 +2754,7 @@ extern "C" int cueq_ln_dual_gate(int32_t dtype, int64_t C, int64_t M, int64_t K,
   CUEQ_REQUIRE(dual_gate_res_fits(C, M, K, out, ldc, true, false), CUEQ_ERR_UNSUPPORTED,
                "ln_dual_gate: needs K = 32, 64, 96 or 128, C a multiple of 32 that fits the local data share, an even M of at least 4096 and an even ldc");
   KernelTimer timer("ln_dual_gate_fwd", stream);
-  return launch_dual_gate_res(C, M, K, W1, W2, ldw, X, nullptr, ldx, bias1, bias2, mask, out, ldc, gamma, beta, static_cast<float>(eps), xhat, ldxh, mean, rstd, stream);
+  return launch_dual_gate_res(C, M, K, W1, W2, ldw, X, nullptr, ldx, bias1, bias2, mask, out, ldc, gamma, beta, static_cast<float>(eps), xhat, ldxh, mean, rstd, dtype == CUEQ_F16, stream);
 }
 
 // ln_x != NULL: the LayerNorm backward in the same kernel (cueq_gate_bwd_input_ln)
@@ -2734,7 +2771,7 @@ static int gate_bwd_input_impl(int32_t dtype, int64_t C, int64_t M, int64_t K, c
   CUEQ_REQUIRE(C % 32 == 0 && C > 0, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: C must be a positive multiple of 32");
   CUEQ_REQUIRE(M < (1ll << 31) - kTile && C < (1ll << 31), CUEQ_ERR_TOO_LARGE, "gate_bwd_input: extent too large");
   CUEQ_REQUIRE(W1 && W2 && X1 && dC && dX1 && (!dU == !dV), CUEQ_ERR_INVALID, "gate_bwd_input: null operand");
-  const bool bf = dtype == CUEQ_BF16;
+  const bool bf = dtype != CUEQ_F32, half = dtype == CUEQ_F16;
   const bool split = X2 != nullptr && X2 != X1;
   CUEQ_REQUIRE(!split || dX2, CUEQ_ERR_INVALID, "gate_bwd_input: two inputs need two gradients");
   CUEQ_REQUIRE(!(split && accumulate), CUEQ_ERR_UNSUPPORTED, "gate_bwd_input: accumulate needs a single input");
@@ -2774,18 +2811,22 @@ static int gate_bwd_input_impl(int32_t dtype, int64_t C, int64_t M, int64_t K, c
       const int64_t ntiles = (M + 31) / 32;
       int64_t gx = (ntiles + nwaves - 1) / nwaves;
       if (gx > device_cus()) gx = device_cus();
-#define GBR(KT, SP) do { auto kfn = gate_bwd_input_res_kernel<KT, SP, !SP, false>; \
+#define GBR_F(FT, KT, SP) do { auto kfn = gate_bwd_input_res_kernel<FT, KT, SP, !SP, false>; \
         CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(SP ? 256 : 512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X1), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<const uint16_t*>(dC), ldc, static_cast<uint16_t*>(dX1), static_cast<uint16_t*>(dX2), lddx, accumulate, static_cast<uint16_t*>(dU), static_cast<uint16_t*>(dV), static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(nullptr), int64_t(0), static_cast<const float*>(nullptr), static_cast<const float*>(nullptr), static_cast<const uint16_t*>(nullptr)); } while (0)
+        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(SP ? 256 : 512), lds, stream, static_cast<const FT*>(W1), static_cast<const FT*>(W2), ldw, static_cast<const FT*>(X1), static_cast<const FT*>(X2), ldx, static_cast<const FT*>(bias1), static_cast<const FT*>(bias2), static_cast<const FT*>(mask), static_cast<const FT*>(dC), ldc, static_cast<FT*>(dX1), static_cast<FT*>(dX2), lddx, accumulate, static_cast<FT*>(dU), static_cast<FT*>(dV), static_cast<int>(C), static_cast<int>(M), static_cast<const FT*>(nullptr), int64_t(0), static_cast<const float*>(nullptr), static_cast<const float*>(nullptr), static_cast<const FT*>(nullptr)); } while (0)
+#define GBR(KT, SP) do { if (half) GBR_F(f16bits, KT, SP); else GBR_F(uint16_t, KT, SP); } while (0)
 #define GBR_K(SP) do { switch (K / 32) { case 1: GBR(1, SP); break; case 2: GBR(2, SP); break; case 3: GBR(3, SP); break; default: GBR(4, SP); break; } } while (0)
-#define GBL(KT) do { auto kfn = gate_bwd_input_res_kernel<KT, false, true, true>; \
+#define GBL_F(FT, KT) do { auto kfn = gate_bwd_input_res_kernel<FT, KT, false, true, true>; \
         CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const uint16_t*>(W1), static_cast<const uint16_t*>(W2), ldw, static_cast<const uint16_t*>(X1), static_cast<const uint16_t*>(X2), ldx, static_cast<const uint16_t*>(bias1), static_cast<const uint16_t*>(bias2), static_cast<const uint16_t*>(mask), static_cast<const uint16_t*>(dC), ldc, static_cast<uint16_t*>(dX1), static_cast<uint16_t*>(dX2), lddx, accumulate, static_cast<uint16_t*>(dU), static_cast<uint16_t*>(dV), static_cast<int>(C), static_cast<int>(M), static_cast<const uint16_t*>(ln_x), ldlx, ln_mean, ln_rstd, static_cast<const uint16_t*>(ln_gamma)); } while (0)
+        hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(gx)), dim3(512), lds, stream, static_cast<const FT*>(W1), static_cast<const FT*>(W2), ldw, static_cast<const FT*>(X1), static_cast<const FT*>(X2), ldx, static_cast<const FT*>(bias1), static_cast<const FT*>(bias2), static_cast<const FT*>(mask), static_cast<const FT*>(dC), ldc, static_cast<FT*>(dX1), static_cast<FT*>(dX2), lddx, accumulate, static_cast<FT*>(dU), static_cast<FT*>(dV), static_cast<int>(C), static_cast<int>(M), static_cast<const FT*>(ln_x), ldlx, ln_mean, ln_rstd, static_cast<const FT*>(ln_gamma)); } while (0)
+#define GBL(KT) do { if (half) GBL_F(f16bits, KT); else GBL_F(uint16_t, KT); } while (0)
       if (ln_x) { switch (K / 32) { case 1: GBL(1); break; case 2: GBL(2); break; case 3: GBL(3); break; default: GBL(4); break; } }
       else if (split) GBR_K(true); else GBR_K(false);
 #undef GBL
+#undef GBL_F
 #undef GBR_K
 #undef GBR
+#undef GBR_F
       CUEQ_CHECK_HIP(hipGetLastError());
       return CUEQ_OK;
     }
@@ -2794,7 +2835,7 @@ static int gate_bwd_input_impl(int32_t dtype, int64_t C, int64_t M, int64_t K, c
 #define GBI(TI, KT, SP) hipLaunchKernelGGL((gate_bwd_input_kernel<TI, KT, SP, !SP>), dim3(static_cast<unsigned>((M + gbi_threads<TI, SP>() / 2 - 1) / (gbi_threads<TI, SP>() / 2))), dim3(gbi_threads<TI, SP>()), 0, stream, static_cast<const TI*>(W1), static_cast<const TI*>(W2), ldw, static_cast<const TI*>(X1), static_cast<const TI*>(X2), ldx, static_cast<const TI*>(bias1), static_cast<const TI*>(bias2), static_cast<const TI*>(mask), static_cast<const TI*>(dC), ldc, static_cast<TI*>(dX1), static_cast<TI*>(dX2), lddx, accumulate, static_cast<TI*>(dU), static_cast<TI*>(dV), static_cast<int>(C), static_cast<int>(M))
 #define GBI_K(TI, SP) do { switch (K / 32) { case 1: GBI(TI, 1, SP); break; case 2: GBI(TI, 2, SP); break; case 3: GBI(TI, 3, SP); break; default: GBI(TI, 4, SP); break; } } while (0)
 #define GBI_T(TI) do { if (split) GBI_K(TI, true); else GBI_K(TI, false); } while (0)
-  TRI_DISPATCH(dtype, GBI_T(float), GBI_T(uint16_t));
+  TRI_DISPATCH(dtype, GBI_T(float), GBI_T(uint16_t), GBI_T(f16bits));
 #undef GBI_T
 #undef GBI_K
 #undef GBI
@@ -2815,7 +2856,7 @@ extern "C" int cueq_gate_bwd_input_ln(int32_t dtype, int64_t C, int64_t M, int64
                                       int64_t ldx, const void* bias1, const void* bias2, const void* mask, const void* dC, int64_t ldc,
                                       void* dX, int64_t lddx, int32_t accumulate, const void* ln_x, int64_t ldlx, const float* ln_mean,
                                       const float* ln_rstd, const void* ln_gamma, void* stream_) {
-  CUEQ_REQUIRE(dtype == CUEQ_BF16, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input_ln: built for bfloat16");
+  CUEQ_REQUIRE(dtype == CUEQ_BF16 || dtype == CUEQ_F16, CUEQ_ERR_UNSUPPORTED, "gate_bwd_input_ln: built for bfloat16 and half");
   CUEQ_REQUIRE(ln_x && ln_mean && ln_rstd, CUEQ_ERR_INVALID, "gate_bwd_input_ln: null operand");
   CUEQ_REQUIRE(reinterpret_cast<uintptr_t>(ln_x) % 16 == 0 && ldlx % 8 == 0 && ldlx >= K, CUEQ_ERR_UNSUPPORTED,
                "gate_bwd_input_ln: the LayerNorm input rows must be 16-byte aligned");
@@ -2847,18 +2888,21 @@ extern "C" int cueq_gemm_tn(int32_t in_dtype, int64_t M, int64_t N, int64_t rows
   const bool vec = M % 8 == 0 && N % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && stride_a % 8 == 0 && stride_b % 8 == 0 &&
                    reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0;
   KernelTimer timer("gemm_tn", stream);
-  if (in_dtype == CUEQ_BF16 && vec && rows > 0) {
-    // 2-byte inputs: bf16 MFMA on contraction-major tiles (transposing LDS reads); batch items = (row chunk, part)
+  if (in_dtype != CUEQ_F32 && vec && rows > 0) {
+    // 2-byte inputs: MFMA on contraction-major tiles (transposing LDS reads); batch items = (row chunk, part)
     const int64_t rpc32 = (((rows + chunks - 1) / chunks + 31) / 32) * 32;
-    hipLaunchKernelGGL((gemm_kernel<uint16_t, float, true, true>), grid, dim3(256), 0, stream, static_cast<const uint16_t*>(A), lda,
-                       rpc32 * lda, static_cast<const uint16_t*>(B), ldb, rpc32 * ldb, partials, N, static_cast<int64_t>(M) * N,
-                       static_cast<int>(M), static_cast<int>(N), static_cast<int>(rpc32), static_cast<float>(alpha), 0, 0, rows, nparts,
-                       stride_a, stride_b, chunks * static_cast<int64_t>(M) * N, nullptr, 0, 0, 0, 0);
+#define TN2(FT) hipLaunchKernelGGL((gemm_kernel<FT, float, true, true>), grid, dim3(256), 0, stream, static_cast<const FT*>(A), lda, \
+                       rpc32 * lda, static_cast<const FT*>(B), ldb, rpc32 * ldb, partials, N, static_cast<int64_t>(M) * N, \
+                       static_cast<int>(M), static_cast<int>(N), static_cast<int>(rpc32), static_cast<float>(alpha), 0, 0, rows, nparts, \
+                       stride_a, stride_b, chunks * static_cast<int64_t>(M) * N, nullptr, 0, 0, 0, 0)
+    if (in_dtype == CUEQ_F16) TN2(f16bits); else TN2(uint16_t);
+#undef TN2
     CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }
 #define TN_LAUNCH(TI, V) hipLaunchKernelGGL((gemm_tn_kernel<TI, V>), grid, dim3(256), 0, stream, static_cast<const TI*>(A), lda, stride_a, static_cast<const TI*>(B), ldb, stride_b, partials, static_cast<int>(M), static_cast<int>(N), rows, rpc, nparts, static_cast<float>(alpha))
   if (in_dtype == CUEQ_F32) { if (vec) TN_LAUNCH(float, true); else TN_LAUNCH(float, false); }
+  else if (in_dtype == CUEQ_F16) { if (vec) TN_LAUNCH(f16bits, true); else TN_LAUNCH(f16bits, false); }
   else { if (vec) TN_LAUNCH(uint16_t, true); else TN_LAUNCH(uint16_t, false); }
 #undef TN_LAUNCH
   CUEQ_CHECK_HIP(hipGetLastError());
@@ -2871,7 +2915,7 @@ extern "C" int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_
   if (batch <= 0 || rows <= 0 || cols <= 0) return CUEQ_OK;
   CUEQ_REQUIRE(in && out, CUEQ_ERR_INVALID, "transpose: null operand");
   CUEQ_REQUIRE(rows < (1ll << 31) && cols < (1ll << 31), CUEQ_ERR_TOO_LARGE, "transpose: extent too large");
-  if (dtype == CUEQ_BF16 && rows % 2 == 0 && cols % 2 == 0 && reinterpret_cast<uintptr_t>(in) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0) {
+  if (dtype != CUEQ_F32 && rows % 2 == 0 && cols % 2 == 0 && reinterpret_cast<uintptr_t>(in) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 4 == 0) {
     int64_t gy2 = (rows + 63) / 64, gx2 = (cols + 63) / 64;
     const int rows_on_x = gy2 >= 65536 ? 1 : 0;
     if (rows_on_x) { const int64_t t = gx2; gx2 = gy2; gy2 = t; }
@@ -2890,7 +2934,8 @@ extern "C" int cueq_transpose(int32_t dtype, int64_t batch, int64_t rows, int64_
   KernelTimer timer("transpose", stream);
   TRI_DISPATCH(dtype,
                hipLaunchKernelGGL(transpose_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), static_cast<float*>(out), static_cast<int>(rows), static_cast<int>(cols), rows_on_x),
-               hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols), rows_on_x));
+               hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), static_cast<uint16_t*>(out), static_cast<int>(rows), static_cast<int>(cols), rows_on_x),
+               hipLaunchKernelGGL(transpose_kernel<f16bits>, grid, dim3(256), 0, stream, static_cast<const f16bits*>(in), static_cast<f16bits*>(out), static_cast<int>(rows), static_cast<int>(cols), rows_on_x));
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }
@@ -2912,7 +2957,7 @@ extern "C" int cueq_layer_norm_fwd(int32_t dtype, int64_t rows, int64_t D, const
     const dim3 g8(static_cast<unsigned>((rows + rpb - 1) / rpb));
 #define LN8(T, LL) hipLaunchKernelGGL((ln_fwd_rows8<T, LL>), g8, dim3(256), 0, stream, static_cast<const T*>(x), static_cast<const T*>(gamma), static_cast<const T*>(beta), static_cast<T*>(y), mean, rstd, rows, static_cast<float>(eps))
 #define LN8_L(T) do { switch (L) { case 4: LN8(T, 4); break; case 8: LN8(T, 8); break; case 16: LN8(T, 16); break; case 32: LN8(T, 32); break; default: LN8(T, 64); } } while (0)
-    TRI_DISPATCH(dtype, LN8_L(float), LN8_L(uint16_t));
+    TRI_DISPATCH(dtype, LN8_L(float), LN8_L(uint16_t), LN8_L(f16bits));
 #undef LN8_L
 #undef LN8
     CUEQ_CHECK_HIP(hipGetLastError());
@@ -2921,7 +2966,7 @@ extern "C" int cueq_layer_norm_fwd(int32_t dtype, int64_t rows, int64_t D, const
   const int nq = static_cast<int>((D + 63) / 64);
 #define LN_FWD(T, NQ) hipLaunchKernelGGL((ln_fwd_kernel<T, NQ>), grid, dim3(256), 0, stream, static_cast<const T*>(x), static_cast<const T*>(gamma), static_cast<const T*>(beta), static_cast<T*>(y), mean, rstd, rows, static_cast<int>(D), static_cast<float>(eps))
 #define LN_FWD_NQ(T) do { if (nq <= 1) LN_FWD(T, 1); else if (nq <= 2) LN_FWD(T, 2); else if (nq <= 4) LN_FWD(T, 4); else if (nq <= 8) LN_FWD(T, 8); else LN_FWD(T, 16); } while (0)
-  TRI_DISPATCH(dtype, LN_FWD_NQ(float), LN_FWD_NQ(uint16_t));
+  TRI_DISPATCH(dtype, LN_FWD_NQ(float), LN_FWD_NQ(uint16_t), LN_FWD_NQ(f16bits));
 #undef LN_FWD_NQ
 #undef LN_FWD
   CUEQ_CHECK_HIP(hipGetLastError());
@@ -2963,13 +3008,13 @@ extern "C" int cueq_layer_norm_bwd(int32_t dtype, int64_t rows, int64_t D, const
       const int L = static_cast<int>(D / 8);
 #define LNB8(T, LL) hipLaunchKernelGGL((ln_bwd_rows8<T, LL>), dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const T*>(dy), static_cast<const T*>(x), mean, rstd, static_cast<const T*>(gamma), static_cast<T*>(dx), part, rows, rpb)
 #define LNB8_L(T) do { switch (L) { case 4: LNB8(T, 4); break; case 8: LNB8(T, 8); break; case 16: LNB8(T, 16); break; case 32: LNB8(T, 32); break; default: LNB8(T, 64); } } while (0)
-      TRI_DISPATCH(dtype, LNB8_L(float), LNB8_L(uint16_t));
+      TRI_DISPATCH(dtype, LNB8_L(float), LNB8_L(uint16_t), LNB8_L(f16bits));
 #undef LNB8_L
 #undef LNB8
     } else {
 #define LN_BWD(T, NQ) hipLaunchKernelGGL((ln_bwd_kernel<T, NQ>), dim3(static_cast<unsigned>(nb)), dim3(256), sh, stream, static_cast<const T*>(dy), static_cast<const T*>(x), mean, rstd, static_cast<const T*>(gamma), static_cast<T*>(dx), part, rows, static_cast<int>(D), rpb)
 #define LN_BWD_NQ(T) do { if (nq <= 1) LN_BWD(T, 1); else if (nq <= 2) LN_BWD(T, 2); else if (nq <= 4) LN_BWD(T, 4); else if (nq <= 8) LN_BWD(T, 8); else LN_BWD(T, 16); } while (0)
-    TRI_DISPATCH(dtype, LN_BWD_NQ(float), LN_BWD_NQ(uint16_t));
+    TRI_DISPATCH(dtype, LN_BWD_NQ(float), LN_BWD_NQ(uint16_t), LN_BWD_NQ(f16bits));
 #undef LN_BWD_NQ
 #undef LN_BWD
     }
@@ -3002,28 +3047,32 @@ extern "C" int cueq_layer_norm_t_fwd(int32_t dtype, int64_t M, int64_t D, const 
   CUEQ_REQUIRE(ntiles < (1ll << 31), CUEQ_ERR_TOO_LARGE, "layer_norm_t: too many rows");
   const size_t fwd_lds = static_cast<size_t>(D) * 132;
   KernelTimer timer("layer_norm_t_fwd", stream);
-  if (dtype == CUEQ_BF16 && (D == 64 || D == 128) && D * M + 256 < (1ll << 32) &&
+  const bool half = dtype == CUEQ_F16;
+  if (dtype != CUEQ_F32 && (D == 64 || D == 128) && D * M + 256 < (1ll << 32) &&
       ((reinterpret_cast<uintptr_t>(mean) | reinterpret_cast<uintptr_t>(rstd)) & 7) == 0) {
     // one lane per column pair and half of d, 64 columns per wavefront, four wavefronts per block, two blocks per CU
     int64_t nb = (ntiles + 3) / 4;
     if (nb > 2 * device_cus()) nb = 2 * device_cus();
     const size_t lds = static_cast<size_t>(4 * 64) * (2 * D + 16);
-#define LNTC(DD)                                                                                                                             \
+#define LNTC_F(FT, DD)                                                                                                                             \
   do {                                                                                                                                       \
-    auto kfn = ln_t_fwd_cols_kernel<DD>;                                                                                                     \
+    auto kfn = ln_t_fwd_cols_kernel<FT, DD>;                                                                                                     \
     CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(nb)), dim3(256), lds, stream, static_cast<const uint16_t*>(x_t),                       \
-                       static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, M,    \
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(nb)), dim3(256), lds, stream, static_cast<const FT*>(x_t),                       \
+                       static_cast<const FT*>(gamma), static_cast<const FT*>(beta), static_cast<FT*>(y), mean, rstd, M,    \
                        static_cast<float>(eps));                                                                                             \
   } while (0)
+#define LNTC(DD) do { if (half) LNTC_F(f16bits, DD); else LNTC_F(uint16_t, DD); } while (0)
     if (D == 64) LNTC(64); else LNTC(128);
 #undef LNTC
+#undef LNTC_F
     CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }
   TRI_DISPATCH(dtype,
                hipLaunchKernelGGL(ln_t_fwd_kernel<float>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const float*>(x_t), static_cast<const float*>(gamma), static_cast<const float*>(beta), static_cast<float*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)),
-               hipLaunchKernelGGL(ln_t_fwd_kernel<uint16_t>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const uint16_t*>(x_t), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)));
+               hipLaunchKernelGGL(ln_t_fwd_kernel<uint16_t>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const uint16_t*>(x_t), static_cast<const uint16_t*>(gamma), static_cast<const uint16_t*>(beta), static_cast<uint16_t*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)),
+               hipLaunchKernelGGL(ln_t_fwd_kernel<f16bits>, dim3(static_cast<unsigned>(ntiles)), dim3(256), fwd_lds, stream, static_cast<const f16bits*>(x_t), static_cast<const f16bits*>(gamma), static_cast<const f16bits*>(beta), static_cast<f16bits*>(y), mean, rstd, M, static_cast<int>(D), static_cast<float>(eps)));
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }
@@ -3060,22 +3109,25 @@ extern "C" int cueq_layer_norm_t_bwd(int32_t dtype, int64_t M, int64_t D, const 
   const int64_t nb = ln_t_bwd_blocks(dtype, M);
   float* part = static_cast<float*>(workspace);
   const int64_t es = dtype == CUEQ_F32 ? 4 : 2;
-  if (dtype == CUEQ_BF16 && !need_affine && (D == 64 || D == 128) && D * M + 256 < (1ll << 32) &&
+  const bool half = dtype == CUEQ_F16;
+  if (dtype != CUEQ_F32 && !need_affine && (D == 64 || D == 128) && D * M + 256 < (1ll << 32) &&
       ((reinterpret_cast<uintptr_t>(mean) | reinterpret_cast<uintptr_t>(rstd)) & 7) == 0) {
     // one lane per column pair and half of d, 64 columns per wavefront, four wavefronts per block, two blocks per CU
     int64_t nbc = (ntiles + 3) / 4;
     if (nbc > 2 * device_cus()) nbc = 2 * device_cus();
     const size_t lds = static_cast<size_t>(4 * 64) * (2 * D + 16);
     KernelTimer timer("layer_norm_t_bwd", stream);
-#define LNTC(DD)                                                                                                                             \
+#define LNTC_F(FT, DD)                                                                                                                             \
   do {                                                                                                                                       \
-    auto kfn = ln_t_bwd_cols_kernel<DD>;                                                                                                     \
+    auto kfn = ln_t_bwd_cols_kernel<FT, DD>;                                                                                                     \
     CUEQ_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds))); \
-    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(nbc)), dim3(256), lds, stream, static_cast<const uint16_t*>(dy),                       \
-                       static_cast<const uint16_t*>(x_t), mean, rstd, static_cast<const uint16_t*>(gamma), static_cast<uint16_t*>(dx_t), M); \
+    hipLaunchKernelGGL(kfn, dim3(static_cast<unsigned>(nbc)), dim3(256), lds, stream, static_cast<const FT*>(dy),                       \
+                       static_cast<const FT*>(x_t), mean, rstd, static_cast<const FT*>(gamma), static_cast<FT*>(dx_t), M); \
   } while (0)
+#define LNTC(DD) do { if (half) LNTC_F(f16bits, DD); else LNTC_F(uint16_t, DD); } while (0)
     if (D == 64) LNTC(64); else LNTC(128);
 #undef LNTC
+#undef LNTC_F
     CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }
@@ -3084,7 +3136,8 @@ extern "C" int cueq_layer_norm_t_bwd(int32_t dtype, int64_t M, int64_t D, const 
     KernelTimer timer("layer_norm_t_bwd", stream);
     TRI_DISPATCH(dtype,
                  hipLaunchKernelGGL(ln_t_bwd_kernel<float>, dim3(static_cast<unsigned>(nb)), dim3(256), bwd_lds, stream, static_cast<const float*>(dy), static_cast<const float*>(x_t), mean, rstd, static_cast<const float*>(gamma), static_cast<float*>(dx_t), part, M, static_cast<int>(D), ntiles, need_affine),
-                 hipLaunchKernelGGL(ln_t_bwd_kernel<uint16_t>, dim3(static_cast<unsigned>(nb)), dim3(256), bwd_lds, stream, static_cast<const uint16_t*>(dy), static_cast<const uint16_t*>(x_t), mean, rstd, static_cast<const uint16_t*>(gamma), static_cast<uint16_t*>(dx_t), part, M, static_cast<int>(D), ntiles, need_affine));
+                 hipLaunchKernelGGL(ln_t_bwd_kernel<uint16_t>, dim3(static_cast<unsigned>(nb)), dim3(256), bwd_lds, stream, static_cast<const uint16_t*>(dy), static_cast<const uint16_t*>(x_t), mean, rstd, static_cast<const uint16_t*>(gamma), static_cast<uint16_t*>(dx_t), part, M, static_cast<int>(D), ntiles, need_affine),
+                 hipLaunchKernelGGL(ln_t_bwd_kernel<f16bits>, dim3(static_cast<unsigned>(nb)), dim3(256), bwd_lds, stream, static_cast<const f16bits*>(dy), static_cast<const f16bits*>(x_t), mean, rstd, static_cast<const f16bits*>(gamma), static_cast<f16bits*>(dx_t), part, M, static_cast<int>(D), ntiles, need_affine));
   }
   CUEQ_CHECK_HIP(hipGetLastError());
   const unsigned g = static_cast<unsigned>((D + 255) / 256);
@@ -3107,7 +3160,8 @@ extern "C" int cueq_gate_fwd(int32_t dtype, int64_t rows, int64_t cols, const fl
   KernelTimer timer("gate_fwd", stream);
   TRI_DISPATCH(dtype,
                hipLaunchKernelGGL(gate_fwd_kernel<float>, grid, dim3(256), 0, stream, u, v, static_cast<const float*>(bias_u), static_cast<const float*>(bias_v), bias_axis, static_cast<const float*>(mask), mask_axis, static_cast<float*>(out), rows, cols),
-               hipLaunchKernelGGL(gate_fwd_kernel<uint16_t>, grid, dim3(256), 0, stream, u, v, static_cast<const uint16_t*>(bias_u), static_cast<const uint16_t*>(bias_v), bias_axis, static_cast<const uint16_t*>(mask), mask_axis, static_cast<uint16_t*>(out), rows, cols));
+               hipLaunchKernelGGL(gate_fwd_kernel<uint16_t>, grid, dim3(256), 0, stream, u, v, static_cast<const uint16_t*>(bias_u), static_cast<const uint16_t*>(bias_v), bias_axis, static_cast<const uint16_t*>(mask), mask_axis, static_cast<uint16_t*>(out), rows, cols),
+               hipLaunchKernelGGL(gate_fwd_kernel<f16bits>, grid, dim3(256), 0, stream, u, v, static_cast<const f16bits*>(bias_u), static_cast<const f16bits*>(bias_v), bias_axis, static_cast<const f16bits*>(mask), mask_axis, static_cast<f16bits*>(out), rows, cols));
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }
@@ -3124,7 +3178,8 @@ extern "C" int cueq_gate_bwd(int32_t dtype, int64_t rows, int64_t cols, const vo
   KernelTimer timer("gate_bwd", stream);
   TRI_DISPATCH(dtype,
                hipLaunchKernelGGL(gate_bwd_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(dout), u, v, static_cast<const float*>(bias_u), static_cast<const float*>(bias_v), bias_axis, static_cast<const float*>(mask), mask_axis, static_cast<float*>(du), static_cast<float*>(dv), rows, cols),
-               hipLaunchKernelGGL(gate_bwd_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(dout), u, v, static_cast<const uint16_t*>(bias_u), static_cast<const uint16_t*>(bias_v), bias_axis, static_cast<const uint16_t*>(mask), mask_axis, static_cast<uint16_t*>(du), static_cast<uint16_t*>(dv), rows, cols));
+               hipLaunchKernelGGL(gate_bwd_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(dout), u, v, static_cast<const uint16_t*>(bias_u), static_cast<const uint16_t*>(bias_v), bias_axis, static_cast<const uint16_t*>(mask), mask_axis, static_cast<uint16_t*>(du), static_cast<uint16_t*>(dv), rows, cols),
+               hipLaunchKernelGGL(gate_bwd_kernel<f16bits>, grid, dim3(256), 0, stream, static_cast<const f16bits*>(dout), u, v, static_cast<const f16bits*>(bias_u), static_cast<const f16bits*>(bias_v), bias_axis, static_cast<const f16bits*>(mask), mask_axis, static_cast<f16bits*>(du), static_cast<f16bits*>(dv), rows, cols));
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }
@@ -3138,7 +3193,8 @@ extern "C" int cueq_sum_cols(int32_t dtype, int64_t rows, int64_t cols, const vo
   const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
   TRI_DISPATCH(dtype,
                hipLaunchKernelGGL(sum_cols_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), out, rows, cols),
-               hipLaunchKernelGGL(sum_cols_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), out, rows, cols));
+               hipLaunchKernelGGL(sum_cols_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), out, rows, cols),
+               hipLaunchKernelGGL(sum_cols_kernel<f16bits>, grid, dim3(256), 0, stream, static_cast<const f16bits*>(in), out, rows, cols));
   CUEQ_CHECK_HIP(hipGetLastError());
   return CUEQ_OK;
 }
@@ -3171,7 +3227,8 @@ extern "C" int cueq_sum_rows(int32_t dtype, int64_t rows, int64_t cols, const vo
     const dim3 grid1(static_cast<unsigned>((cols + 63) / 64));
     TRI_DISPATCH(dtype,
                  hipLaunchKernelGGL(sum_rows_lds_kernel<float>, grid1, dim3(1024), 0, stream, static_cast<const float*>(in), out, rows, cols),
-                 hipLaunchKernelGGL(sum_rows_lds_kernel<uint16_t>, grid1, dim3(1024), 0, stream, static_cast<const uint16_t*>(in), out, rows, cols));
+                 hipLaunchKernelGGL(sum_rows_lds_kernel<uint16_t>, grid1, dim3(1024), 0, stream, static_cast<const uint16_t*>(in), out, rows, cols),
+                 hipLaunchKernelGGL(sum_rows_lds_kernel<f16bits>, grid1, dim3(1024), 0, stream, static_cast<const f16bits*>(in), out, rows, cols));
     CUEQ_CHECK_HIP(hipGetLastError());
     return CUEQ_OK;
   }
@@ -3181,7 +3238,8 @@ extern "C" int cueq_sum_rows(int32_t dtype, int64_t rows, int64_t cols, const vo
   const dim3 grid(static_cast<unsigned>((cols + 255) / 256), static_cast<unsigned>(nb));
   TRI_DISPATCH(dtype,
                hipLaunchKernelGGL(sum_rows_partial_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(in), part, rows, cols, rpb),
-               hipLaunchKernelGGL(sum_rows_partial_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), part, rows, cols, rpb));
+               hipLaunchKernelGGL(sum_rows_partial_kernel<uint16_t>, grid, dim3(256), 0, stream, static_cast<const uint16_t*>(in), part, rows, cols, rpb),
+               hipLaunchKernelGGL(sum_rows_partial_kernel<f16bits>, grid, dim3(256), 0, stream, static_cast<const f16bits*>(in), part, rows, cols, rpb));
   CUEQ_CHECK_HIP(hipGetLastError());
   hipLaunchKernelGGL(fold_partials_kernel<float>, dim3(static_cast<unsigned>((cols + 255) / 256)), dim3(256), 0, stream, part, out, nb, cols, 0);
   CUEQ_CHECK_HIP(hipGetLastError());

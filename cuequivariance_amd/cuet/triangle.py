@@ -41,7 +41,8 @@ class TriMulPrecision(enum.IntEnum):
     IEEE = 3
 
 
-_CODE = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
+_CODE = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+_TWO_BYTE = (torch.bfloat16, torch.float16)  # the matrix-core kernels for 2-byte elements take either format
 
 
 def _stream(t: torch.Tensor):
@@ -219,7 +220,7 @@ def ln_dual_gate_fwd(x, gamma, beta, eps: float, W1, W2, bias1, bias2, mask):
     (then :func:`layer_norm_fwd` and :func:`dual_gate_fwd` do the same in two launches)."""
     M, K = x.shape
     Cn = W1.shape[0]
-    if x.dtype != torch.bfloat16 or K % 32 or K > 128 or Cn % 32 or M % 2 or M < 4096 or M > 65280 * 128:
+    if x.dtype not in _TWO_BYTE or K % 32 or K > 128 or Cn % 32 or M % 2 or M < 4096 or M > 65280 * 128:
         return None
     if 2 * Cn * (2 * K if K == 128 else 2 * K + 16) + 8 * Cn + 8 * K > 160 * 1024 or not _fusable(x, W1, W2):
         return None
@@ -290,7 +291,7 @@ def gate_bwd_input_ln(dC, W1, W2, X, bias1, bias2, mask, dX, ln_x, ln_mean, ln_r
     Cn, K = W1.shape
     M = X.shape[0]
     T = W1.dtype
-    if T != torch.bfloat16 or K % 32 or K > 128 or Cn % 32 or M % 2 or dC.stride(0) % 2 or dC.data_ptr() % 4:
+    if T not in _TWO_BYTE or K % 32 or K > 128 or Cn % 32 or M % 2 or dC.stride(0) % 2 or dC.data_ptr() % 4:
         return None
     if 2 * Cn * (2 * K if K == 128 else 2 * K + 16) + 8 * Cn + 4 * K > 160 * 1024 or not _fusable(W1, W2, X, dX, ln_x):
         return None
@@ -339,7 +340,7 @@ def gemm_long_k(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
     sum of the partial products (no atomics)."""
     P, K = A.shape
     Q = B.shape[0]
-    n = _split_k_chunks(K, 8 if A.dtype == torch.bfloat16 else 4)
+    n = _split_k_chunks(K, 8 if A.dtype in _TWO_BYTE else 4)
     if n == 1:
         return gemm_nt(A, B, torch.float32)
     ck = K // n
@@ -611,7 +612,7 @@ def triangle_multiplicative_update(
     if not x.is_cuda:
         raise ValueError("triangle_multiplicative_update runs on the GPU only: x is on " + str(x.device))
     if x.dtype not in _CODE:
-        raise ValueError(f"x must be float32 or bfloat16, got {x.dtype}")
+        raise ValueError(f"x must be float32, bfloat16 or float16, got {x.dtype}")
     T, dev = x.dtype, x.device
     if mask is not None and tuple(mask.shape) != tuple(lead) + (N, N):
         raise ValueError(f"mask must have shape {tuple(lead) + (N, N)}, got {tuple(mask.shape)}")

@@ -4,8 +4,10 @@ The reference's torch entry point forwards to a closed kernel and its own test c
 (``cuequivariance_torch/tests/primitives/triangle_test.py:97-118``); the algorithm is the open one in
 ``cuequivariance_jax/cuequivariance_jax/triangle/_triangle_multiplicative_update.py:371-417``.  The oracle restates it
 with torch; here it is pinned against library routines (``F.layer_norm``, ``F.linear``) and an explicit loop for the
-triangular contraction.  GPU tolerances: float32 ``1e-5 * max|ref|``, bfloat16 ``2e-2 * max|ref|`` against the
-float64 oracle evaluated on the inputs rounded to the tested dtype.
+triangular contraction.  GPU tolerances: float32 ``1e-5 * max|ref|``, bfloat16 ``2e-2 * max|ref|``, float16
+``4e-3 * max|ref|`` (intermediates are stored in the input type: a few roundings to 8 / 11 bits each; a kernel that read
+half as bfloat16 or the reverse would be off by orders of magnitude) against the float64 oracle evaluated on the inputs
+rounded to the tested dtype.
 """
 
 import pytest
@@ -15,7 +17,7 @@ import torch.nn.functional as F
 from oracle.triangle import triangle_multiplicative_update as oracle_trimul
 from cuequivariance_amd import _lib
 
-TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 4e-3}
 
 
 def make_case(Bsz, N, D, dtype, seed, bias=True, Do=None):
@@ -84,7 +86,7 @@ def rel_err(got, ref):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("direction", ["outgoing", "incoming"])
 @pytest.mark.parametrize("shape", [(1, 32, 32, None), (2, 48, 64, None), (1, 40, 128, 64), (1, 33, 32, None), (1, 20, 64, None),
                                    (1, 66, 96, None)])
@@ -184,7 +186,7 @@ def test_layer_norm_fused_into_the_gated_projection(device, M, K, C, affine, bia
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("dims", [(3, 256, 128, 192), (2, 136, 200, 72), (1, 33, 47, 21), (160, 512, 256, 96),
                                   (128, 512, 512, 512)])
@@ -202,7 +204,7 @@ def test_gemm_operand_orders(device, dtype, trans_a, trans_b, dims):
     big = M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) * batch >= 2 * cus
     if dims == (128, 512, 512, 512):
         assert big or cus > 256, "the benchmark's contraction shape must run on the 256 x 256 tiles"
-    label = ("gemm_nt_f32" if dtype == torch.float32 else "gemm_nt_bf16") + ("_256" if big else "") if aligned else "gemm_nt_simple"
+    label = {torch.float32: "gemm_nt_f32", torch.bfloat16: "gemm_nt_bf16", torch.float16: "gemm_nt_f16"}[dtype] + ("_256" if big else "") if aligned else "gemm_nt_simple"
     g = torch.Generator().manual_seed(M * 7 + N)
     A = torch.randn((batch, K, M) if trans_a else (batch, M, K), generator=g).to(dtype)
     B = torch.randn((batch, K, N) if trans_b else (batch, N, K), generator=g).to(dtype)
@@ -220,7 +222,7 @@ def test_gemm_operand_orders(device, dtype, trans_a, trans_b, dims):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(1, 40, 128, None), (1, 33, 96, 64), (1, 16, 160, None)])
 def test_input_gradient_only(device, dtype, shape):
     """Only x asks for a gradient (the benchmark's case): the gate gradients then stay in registers (D <= 128) or go
@@ -264,29 +266,33 @@ def test_defaults_shapes_and_errors(device):
 
 
 @pytest.mark.gpu
-def test_benchmark_size_against_oracle(device):
-    """The benchmarked case itself (one 512 x 512 pair tensor, 128 channels, bfloat16, outgoing, Bernoulli(0.9) mask):
-    forward and the gradient with respect to the pair tensor against the float64 oracle evaluated on the
-    bfloat16-rounded inputs, 2e-2 * max|ref|.  This is the only size at which the 256 x 256 contraction tiles, the
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_benchmark_size_against_oracle(device, dtype):
+    """The benchmarked case itself (one 512 x 512 pair tensor, 128 channels, bfloat16 - and the same in half -, outgoing,
+    Bernoulli(0.9) mask): forward and the gradient with respect to the pair tensor against the float64 oracle evaluated on
+    the rounded inputs, 2e-2 (bfloat16) / 4e-3 (half) * max|ref|.  This is the only size at which the 256 x 256 contraction tiles, the
     LDS-resident gate backward on 262 144 rows and the LayerNorm with layout change run inside the composed update."""
     from cuequivariance_amd import _lib, cuet
 
-    p, cot = make_case(1, 512, 128, torch.bfloat16, 7)
+    p, cot = make_case(1, 512, 128, dtype, 7)
     pr = {k: v.clone() for k, v in p.items()}
     pr["x"].requires_grad_(True)
     ref = oracle_trimul(direction="outgoing", **pr)
     (want,) = torch.autograd.grad(ref, [pr["x"]], cot)
     ref = ref.detach()
-    pg = {k: v.to(torch.bfloat16).to(device) for k, v in p.items()}
+    pg = {k: v.to(dtype).to(device) for k, v in p.items()}
     pg["x"].requires_grad_(True)
     _lib.timing_begin()
     out = cuet.triangle_multiplicative_update(direction="outgoing", **pg)
-    (got,) = torch.autograd.grad(out, [pg["x"]], cot.to(torch.bfloat16).to(device))
+    (got,) = torch.autograd.grad(out, [pg["x"]], cot.to(dtype).to(device))
     ran = _lib.timing_end()
     if torch.cuda.get_device_properties(device).multi_processor_count <= 256:
-        assert ran.get("gemm_nt_bf16_256", (0, 0))[0] == 3, ran  # the contraction and its two gradients
-    assert rel_err(out, ref) <= 2e-2, ("out", rel_err(out, ref))
-    assert rel_err(got, want) <= 2e-2, ("dx", rel_err(got, want))
+        label = "gemm_nt_bf16_256" if dtype == torch.bfloat16 else "gemm_nt_f16_256"
+        assert ran.get(label, (0, 0))[0] == 3, ran  # the contraction and its two gradients
+    # the stages with the weights resident in the local data share serve both 2-byte formats
+    assert "ln_dual_gate_fwd" in ran and "gate_bwd_input_ln" in ran, ran
+    assert rel_err(out, ref) <= TOL[dtype], ("out", rel_err(out, ref))
+    assert rel_err(got, want) <= TOL[dtype], ("dx", rel_err(got, want))
 
 
 @pytest.mark.gpu
@@ -314,7 +320,7 @@ def test_full_size_properties(device):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("split", [False, True])
 @pytest.mark.parametrize("M", [2048 * 32 + 37 * 32 + 8, 3 * 32 + 8])
 def test_gate_bwd_input_many_tiles(device, dtype, split, M):
@@ -399,7 +405,7 @@ def test_gate_bwd_input_through_the_layer_norm(device, M, K, C, with_prior, affi
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("N", [64 * 2048 + 64 * 5 + 2, 4096 + 34])
 @pytest.mark.parametrize("with_bias", [True, False])
 def test_dual_gate_many_column_tiles(device, dtype, N, with_bias):
@@ -457,7 +463,7 @@ def test_dual_gate_two_inputs_result_by_rows(device, M, K, C, with_bias, masked)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", [(513, 16384), (37, 8200), (3000, 700), (70000, 130), (1, 8192), (5, 3)])
 def test_sum_rows_paths(device, dtype, shape):
     """Column sums of a (rows, cols) matrix in float32: the single-launch kernel (few rows, many columns), the two-stage
