@@ -47,11 +47,20 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
+
+// 2-byte element types: uint16_t = bfloat16 as its bits, f16bits = IEEE half as its bits
+struct f16bits { uint16_t bits; };
+template <typename TI> struct is_half { static constexpr bool value = false; };
+template <> struct is_half<f16bits> { static constexpr bool value = true; };
 
 template <typename TI>
 __device__ __forceinline__ void mma_step(floatx16& acc, const uint4& a, const uint4& b) {
-  if constexpr (sizeof(TI) == 2) {
+  if constexpr (is_half<TI>::value) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), acc, 0, 0, 0);
+  } else if constexpr (sizeof(TI) == 2) {
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
   } else {
     const float* pa = reinterpret_cast<const float*>(&a);
@@ -60,28 +69,45 @@ __device__ __forceinline__ void mma_step(floatx16& acc, const uint4& a, const ui
     for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[e], pb[e], acc, 0, 0, 0);
   }
 }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+// two floats rounded to nearest even into one word of the 2-byte format, and the halves of such a word as floats
+template <typename TI>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   const floatx2_t f = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+  if constexpr (is_half<TI>::value) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2_t));
+  else return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+template <typename TI>
+__device__ __forceinline__ float lo2(uint32_t w) {
+  if constexpr (is_half<TI>::value) return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w & 0xffffu)));
+  else return __uint_as_float(w << 16);
+}
+template <typename TI>
+__device__ __forceinline__ float hi2(uint32_t w) {
+  if constexpr (is_half<TI>::value) return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16)));
+  else return __uint_as_float(w & 0xffff0000u);
 }
 __device__ __forceinline__ float to_f(float v) { return v; }
-__device__ __forceinline__ float to_f(uint16_t v) { return __uint_as_float(static_cast<uint32_t>(v) << 16); }
+__device__ __forceinline__ float to_f(uint16_t v) { return lo2<uint16_t>(v); }
+__device__ __forceinline__ float to_f(f16bits v) { return lo2<f16bits>(v.bits); }
 // four adjacent elements of a row
 __device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
   const float4 t = *reinterpret_cast<const float4*>(p);
   v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
 }
-__device__ __forceinline__ void load4(const uint16_t* p, float (&v)[4]) {
+template <typename TI>
+__device__ __forceinline__ void load4(const TI* p, float (&v)[4]) {
   const uint2 t = *reinterpret_cast<const uint2*>(p);
-  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
-  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+  v[0] = lo2<TI>(t.x); v[1] = hi2<TI>(t.x);
+  v[2] = lo2<TI>(t.y); v[3] = hi2<TI>(t.y);
 }
 __device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) { *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d); }
-__device__ __forceinline__ void store4(uint16_t* p, float a, float b, float c, float d) {
-  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16(a, b), pack_bf16(c, d));
+template <typename TI>
+__device__ __forceinline__ void store4(TI* p, float a, float b, float c, float d) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack2<TI>(a, b), pack2<TI>(c, d));
 }
 __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
-__device__ __forceinline__ void store1(uint16_t* p, float v) { *p = static_cast<uint16_t>(pack_bf16(v, 0.f) & 0xffffu); }
+template <typename TI>
+__device__ __forceinline__ void store1(TI* p, float v) { *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(pack2<TI>(v, 0.f) & 0xffffu); }
 
 constexpr int kWaves = 8;
 '''
@@ -381,9 +407,10 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int, x_
     A(f"// dw: {len(units)} units over 8 wavefronts, MFMAs per pair of rows: {[load[i] for i in slots]}")
     A(f"constexpr int kdwLds = {2 * stride * 4};")
     A("__device__ __forceinline__ void stage(float* dst, const uint4& v, const float*) { *reinterpret_cast<uint4*>(dst) = v; }")
-    A("__device__ __forceinline__ void stage(float* dst, const uint4& v, const uint16_t*) {")
-    A("  *reinterpret_cast<float4*>(dst) = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));")
-    A("  *reinterpret_cast<float4*>(dst + 4) = make_float4(__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xffff0000u), __uint_as_float(v.w << 16), __uint_as_float(v.w & 0xffff0000u));")
+    A("template <typename TI>")
+    A("__device__ __forceinline__ void stage(float* dst, const uint4& v, const TI*) {")
+    A("  *reinterpret_cast<float4*>(dst) = make_float4(lo2<TI>(v.x), hi2<TI>(v.x), lo2<TI>(v.y), hi2<TI>(v.y));")
+    A("  *reinterpret_cast<float4*>(dst + 4) = make_float4(lo2<TI>(v.z), hi2<TI>(v.z), lo2<TI>(v.w), hi2<TI>(v.w));")
     A("}")
     A(f"__global__ void __launch_bounds__(64 * kWaves, 1) dw_kernel(const {T}* __restrict__ X, int64_t ldx, const {T}* __restrict__ S, int64_t lds_, "
       f"const {T}* __restrict__ G, int64_t ldg, float* __restrict__ PART, int64_t numel, int Z, int chunk) {{")
@@ -419,7 +446,7 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int, x_
                 elif fast16 and name == "xr":
                     A(f"          *reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(buf) + row * {XSTR} + col * 2) = static_cast<uint16_t>(w4[e >> 1] >> (16 * (e & 1)));")
                 else:
-                    A(f"          buf[{base} + row * {W} + col] = __uint_as_float((w4[e >> 1] >> (16 * (e & 1))) << 16);")
+                    A(f"          buf[{base} + row * {W} + col] = lo2<{T}>(w4[e >> 1] >> (16 * (e & 1)));")
                 A("        }")
                 A("      }")
                 A("    }")
@@ -476,10 +503,10 @@ def _emit_dw_kernel(A, T: str, paths, n2: int, width_in: int, width_out: int, x_
                     A("#pragma unroll")
                     terms = " + ".join(f"({coeff!r}f * s{j}[e]) * g{c_off + 32 * nt}[e]" for j, coeff, c_off in uses)
                     A(f"          for (int e = 0; e < 8; ++e) hv[e] = {terms};")
-                    A("          const uint4 hb = make_uint4(pack_bf16(hv[0], hv[1]), pack_bf16(hv[2], hv[3]), pack_bf16(hv[4], hv[5]), pack_bf16(hv[6], hv[7]));")
+                    A(f"          const uint4 hb = make_uint4(pack2<{T}>(hv[0], hv[1]), pack2<{T}>(hv[2], hv[3]), pack2<{T}>(hv[4], hv[5]), pack2<{T}>(hv[6], hv[7]));")
                     for kt in range(K // 32):
                         a = acc_of[(w_off, K, N, nt, kt)]
-                        A(f"          mma_step<uint16_t>(acc{a}, x{a_off + 32 * kt}, hb);")
+                        A(f"          mma_step<{T}>(acc{a}, x{a_off + 32 * kt}, hb);")
                     A("        }")
             A("      } break;")
             continue

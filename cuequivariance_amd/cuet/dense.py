@@ -29,7 +29,9 @@ from .. import _lib, cue
 
 __all__ = ["SegmentedPolynomialDense"]
 
-_DTYPE_CODE = {torch.float32: _lib.F32, torch.float64: _lib.F64, torch.bfloat16: _lib.BF16}
+_DTYPE_CODE = {torch.float32: _lib.F32, torch.float64: _lib.F64, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}
+_MATRIX_CORE = (torch.float32, torch.bfloat16, torch.float16)  # element types of the matrix-core kernels (float32 accumulation)
+_FC_ELEMENT = {torch.float32: "float", torch.bfloat16: "uint16_t", torch.float16: "f16bits"}  # their names in the generated units
 
 
 class _Path:
@@ -276,9 +278,9 @@ class _MulIrPlan:
         return _MulIrPlan(blocks)
 
     def accepts(self, dtype) -> bool:
-        if dtype not in (torch.float32, torch.bfloat16):
+        if dtype not in _MATRIX_CORE:
             return False
-        us = 64 if dtype == torch.bfloat16 else 32  # channels per slice of the row-streaming launch
+        us = 32 if dtype == torch.float32 else 64  # channels per slice of the row-streaming launch
         return all(d == 1 or (K % us == 0 and N % us == 0) for _, _, _, K, N, d, _ in self.blocks)
 
     def tables(self, es: int):
@@ -385,7 +387,7 @@ def _run_merged(dtype, A, B, Cout, launches, forward: bool):
     stream = torch.cuda.current_stream(A.device).cuda_stream
     code = _DTYPE_CODE[dtype]
     for K, N, coeff, fwd_tab, dx_tab, rows in launches:
-        if rows is not None and dtype in (torch.bfloat16, torch.float32):
+        if rows is not None and dtype in _MATRIX_CORE:
             for fwd_host, dx_host, nparts in rows[A.element_size()]:
                 if forward:
                     _lib.check(lib.cueq_linear_rows(code, 1, A.shape[0], N, K, A.data_ptr(), A.stride(0), B.data_ptr(), B.numel(), Cout.data_ptr(),
@@ -1255,7 +1257,7 @@ class SegmentedPolynomialDense(nn.Module):
     def fused_unit(self, dtype, *row_tensors):
         """The kernels generated for this product (``codegen/fullyconnected.py``; compiled at first use), or ``None``:
         then the table-driven GEMMs run.  Rows are read and written in 16-byte pieces."""
-        if dtype not in (torch.float32, torch.bfloat16) or not self.has_x2:
+        if dtype not in _MATRIX_CORE or not self.has_x2:
             return None
         if any(t.data_ptr() % 16 or (t.stride(0) * t.element_size()) % 16 or t.stride(1) != 1 for t in row_tensors):
             return None
@@ -1265,7 +1267,7 @@ class SegmentedPolynomialDense(nn.Module):
         if key not in self._fused:
             blocks = self.fc_blocks or (None, None)
             self._fused[key] = jit.fully_connected_unit(self.paths, self.input_sizes[2], self.input_sizes[1], self.out_size,
-                                                          "float" if dtype == torch.float32 else "uint16_t", blocks[0], blocks[1])
+                                                          _FC_ELEMENT[dtype], blocks[0], blocks[1])
         return self._fused[key]
 
     def mul_ir_ready(self, dtype) -> bool:
@@ -1274,19 +1276,19 @@ class SegmentedPolynomialDense(nn.Module):
             return False
         if self.mul_ir is not None:
             return self.mul_ir.accepts(dtype)
-        if dtype not in (torch.float32, torch.bfloat16) or not self.fc_plan.ok:
+        if dtype not in _MATRIX_CORE or not self.fc_plan.ok:
             return False
         from .. import jit
 
         key = (dtype, jit.enabled())
         if key not in self._fused:
             self._fused[key] = jit.fully_connected_unit(self.paths, self.input_sizes[2], self.input_sizes[1], self.out_size,
-                                                          "float" if dtype == torch.float32 else "uint16_t", *self.fc_blocks)
+                                                          _FC_ELEMENT[dtype], *self.fc_blocks)
         return self._fused[key] is not None
 
     def tiled(self, dtype, A: torch.Tensor, Cout: torch.Tensor) -> bool:
         """The tiled kernel serves fp32 / bf16 contractions without a per-row scale."""
-        return (not self.has_x2) and dtype in (torch.float32, torch.bfloat16)
+        return (not self.has_x2) and dtype in _MATRIX_CORE
 
     def transposed_weights(self, wd: torch.Tensor) -> torch.Tensor:
         """Every ``K x N`` weight block transposed in place of itself (same offsets) by ``cueq_transpose``."""
@@ -1319,8 +1321,8 @@ class SegmentedPolynomialDense(nn.Module):
             raise NotImplementedError("indexed_linear: only the 3-operand (Linear) form is supported")
         if x1.device.type != "cuda":
             raise RuntimeError("indexed_linear runs on the GPU only; got tensors on " + str(x1.device))
-        if x1.dtype not in (torch.float32, torch.bfloat16):
-            raise NotImplementedError(f"indexed_linear: float32 and bfloat16 are implemented, got {x1.dtype}")
+        if x1.dtype not in _MATRIX_CORE:
+            raise NotImplementedError(f"indexed_linear: float32, bfloat16 and float16 are implemented, got {x1.dtype}")
         if index.ndim != 1 or index.shape[0] != x1.shape[0]:
             raise ValueError("indexed_linear: the index must have one entry per batch row")
         Cn = w.shape[0]
@@ -1356,7 +1358,7 @@ class SegmentedPolynomialDense(nn.Module):
             raise NotImplementedError(f"fused_tp: rows='mul_ir' does not take {x1.dtype} with these multiplicities")
         if self.rows_mul_ir and self.fc_blocks is not None and not self.mul_ir_ready(x1.dtype):
             raise NotImplementedError("fused_tp: rows='mul_ir' of a fully connected product runs on the generated fused kernels only "
-                                      "(float32 / bfloat16, compilation at first use switched on or the product prebuilt)")
+                                      "(float32 / bfloat16 / float16, compilation at first use switched on or the product prebuilt)")
         if self.math_dtype == torch.float32 and x1.dtype == torch.float64:
             raise ValueError("Fused TP does not support float32 math_dtype with float64 inputs.")
         if x2 is not None:
@@ -1366,6 +1368,10 @@ class SegmentedPolynomialDense(nn.Module):
                 x2 = x2.expand(x1.shape[0], x2.shape[1])
             elif x1.shape[0] == 1 and x2.shape[0] != 1:
                 x1 = x1.expand(x2.shape[0], x1.shape[1])
-        if x2 is not None and self.fc_plan.ok and x1.dtype in (torch.float32, torch.bfloat16):
+        if x2 is not None and x1.dtype == torch.float16 and not (self.fc_plan.ok and self.fused_unit(torch.float16, _aligned(x1.detach())) is not None):
+            # half runs on the generated fused kernels only (the table-driven kernels behind them know float32 and bfloat16):
+            # anything else is computed in float32 - every half is a float - and rounded once
+            return [self.forward([w.float(), x1.float(), x2.float()], input_indices, output_shapes, output_indices)[0].to(torch.float16)]
+        if x2 is not None and self.fc_plan.ok and x1.dtype in _MATRIX_CORE:
             return [_apply_dense(1, self, w, x1, x2)]
         return [_apply_dense(0, self, w, x1, x2)]

@@ -155,7 +155,7 @@ class SegmentedPolynomialFusedTP(nn.Module):
         for k in output_indices:
             assert k in output_shapes, "output shapes must be provided for output indices"
         if (self.dense is not None and not input_indices and not output_indices and not output_shapes
-                and inputs[self.dense_perm[0]].shape[0] == 1 and inputs[0].dtype in (torch.float32, torch.float64, torch.bfloat16)
+                and inputs[self.dense_perm[0]].shape[0] == 1 and inputs[0].dtype in (torch.float32, torch.float64, torch.bfloat16, torch.float16)
                 and all(t.dtype == inputs[0].dtype for t in inputs)):
             return self.dense([inputs[i] for i in self.dense_perm], input_indices, output_shapes, output_indices)
         if self._rows_orig == "mul_ir":

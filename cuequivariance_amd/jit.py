@@ -321,7 +321,7 @@ def prebuild_fully_connected(force: bool = False) -> list:
         # both row orders of the first operand and the output: ir_mul (the kernels' own) and mul_ir (the modules' default)
         mul_ir = ([(o, mul, ir.dim) for o, (mul, ir) in zip(_starts(m.irreps_in1), m.irreps_in1)],
                   [(o, mul, ir.dim) for o, (mul, ir) in zip(_starts(m.irreps_out), m.irreps_out)])
-        for T in ("float", "uint16_t"):
+        for T in ("float", "uint16_t", "f16bits"):
             for blocks, tag in (((None, None), ""), (mul_ir, ", mul_ir rows")):
                 src = fc.emit_unit(dense.paths, dense.input_sizes[2], dense.input_sizes[1], dense.out_size, T, *blocks)
                 so = PREBUILT / f"fc_{hashlib.sha1(src.encode()).hexdigest()[:16]}_{T}.so"

@@ -58,9 +58,9 @@ def test_dense_entries_refuse_bad_arguments_before_any_launch():
     lib = _lib.load()
     F32, F64, BF16 = _lib.F32, _lib.F64, _lib.BF16
     p = 4096  # a fake, 16-byte aligned address: never dereferenced by a refused call
-    # dtype outside float32 / bfloat16
+    # dtype outside float32 / bfloat16 / half
     assert lib.cueq_gemm(F64, F64, 0, 0, 8, 8, 8, p, 8, 0, p, 8, 0, p, 8, 0, 1, 1.0, 0, None) == -2
-    assert b"float32 or bfloat16" in lib.cueq_last_error()
+    assert b"float32, bfloat16 or half" in lib.cueq_last_error()
     # negative extent, null operand
     assert lib.cueq_gemm(F32, F32, 0, 0, -1, 8, 8, p, 8, 0, p, 8, 0, p, 8, 0, 1, 1.0, 0, None) == -1
     assert lib.cueq_gemm(F32, F32, 0, 0, 8, 8, 8, None, 8, 0, p, 8, 0, p, 8, 0, 1, 1.0, 0, None) == -1

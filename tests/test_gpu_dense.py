@@ -5,7 +5,7 @@
 ``cuequivariance_torch/tests/operations/tensor_product_test.py:30-108``): outputs and first
 derivatives, several dtypes, shared and batched weights.
 
-Tolerances (max-norm relative to ``max|ref|``): float64 1e-12, float32 1e-5, bfloat16 2e-2.  The
+Tolerances (max-norm relative to ``max|ref|``): float64 1e-12, float32 1e-5, bfloat16 2e-2, float16 2e-3.  The
 float64 oracle is evaluated on the inputs after rounding to the tested dtype.
 """
 
@@ -17,7 +17,7 @@ from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
 
 pytestmark = pytest.mark.gpu
 
-TOL = {torch.float64: 1e-12, torch.float32: 1e-5, torch.bfloat16: 2e-2}
+TOL = {torch.float64: 1e-12, torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-3}
 
 
 def rel_err(got, ref):
@@ -52,7 +52,7 @@ def linear_module(irreps_in, irreps_out, **kw):
                        internal_weights=False, method="fused_tp", **kw)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 @pytest.mark.parametrize(
     "irreps_in,irreps_out,Z",
     [
@@ -70,7 +70,7 @@ def test_linear_matches_oracle(device, dtype, irreps_in, irreps_out, Z):
     check_against_oracle(device, m, [w, x], dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
 def test_fully_connected_matches_oracle(device, dtype):
     from cuequivariance_amd import cuet
 
@@ -86,7 +86,7 @@ def test_fully_connected_matches_oracle(device, dtype):
 
 
 @pytest.mark.parametrize("layout", [cue.ir_mul, cue.mul_ir])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_fully_connected_benchmark_size(device, dtype, layout):
     """At the benchmark's size (50 000 rows, 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o): rows drawn from all over the batch
     (the first, the last and those of the last, partly filled tile among them) against the float64 oracle, outputs and
@@ -188,7 +188,7 @@ def test_linear_full_size_properties(device):
     assert abs((gx.double() * x.detach().double()).sum().item() - lhs) <= 1e-4 * abs(lhs) + 1e-3 * scale
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize(
     "irreps,classes,sizes",
     [

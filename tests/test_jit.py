@@ -221,7 +221,7 @@ def test_fully_connected_generator_limits():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("i1,i2,i3,Z", [
     ("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o", 777),   # ragged: the last 32-row tile holds 9 rows
     ("32x0e+64x1o", "0e+1o", "96x0e+32x1o", 2500),     # mixed block shapes, a wavefront walks more than one tile on few CUs
@@ -255,8 +255,8 @@ def test_fused_fully_connected_matches_oracle_and_tables(device, dtype, i1, i2, 
     assert d._fused.get((dtype, True)) is not None, "the generated kernels were not built"
     jit.enable(False)
     tables = run()
-    assert d._fused.get((dtype, False)) is None
-    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert d._fused.get((dtype, False)) is None  # (half: computed in float32 by the table-driven kernels, rounded once)
+    tol = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-3}[dtype]
     for name, u, v, t in zip(("out", "dw", "dx1", "dx2"), got, want, tables):
         assert u.dtype == dtype and u.shape == v.shape
         scale = max(v.abs().max().item(), 1e-30)

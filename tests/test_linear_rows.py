@@ -14,7 +14,7 @@ import torch
 
 from cuequivariance_amd import _lib, cue
 
-BF16, F32, F64 = 3, 0, 1
+BF16, F16, F32, F64 = 3, 2, 0, 1
 
 
 def _table(rows):
@@ -55,7 +55,7 @@ def _reference(A, W, parts, K, N, contraction_major, alpha, ldc):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("contraction_major", [1, 0])
 @pytest.mark.parametrize(
     "M,K,N,nblocks,nparts",
@@ -75,7 +75,7 @@ def test_linear_rows_against_float64_product(device, dtype, contraction_major, M
     lib = _lib.load()
     g = torch.Generator(device=device).manual_seed(M + K + N)
     lda, ldc = nparts * K + 8, nparts * N + 16
-    es = 2 if dtype == torch.bfloat16 else 4
+    es = 4 if dtype == torch.float32 else 2
     nblocks = min(nblocks, (160 * 1024 - 8 * 32 * 144) // (N * (es * K + 16)))  # what the local data share holds
     A = torch.randn(M, lda, device=device, generator=g).to(dtype)
     W = torch.randn(nblocks * K * N + 8, device=device, generator=g).to(dtype)
@@ -85,7 +85,7 @@ def test_linear_rows_against_float64_product(device, dtype, contraction_major, M
     out = torch.full((M, ldc), 7.0, device=device).to(dtype)
     alpha = 0.37
     stream = torch.cuda.current_stream(device).cuda_stream
-    code = BF16 if dtype == torch.bfloat16 else F32
+    code = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}[dtype]
     _lib.check(lib.cueq_linear_rows(code, contraction_major, M, N, K, A.data_ptr(), lda, W.data_ptr(), W.numel(), out.data_ptr(), ldc, _table(parts),
                                     nparts, alpha, stream), "cueq_linear_rows")
     ref = _reference(A, W, parts, K, N, contraction_major, alpha, ldc)
@@ -95,7 +95,7 @@ def test_linear_rows_against_float64_product(device, dtype, contraction_major, M
     got = out.double()
     assert (got[:, ~written] == 7.0).all()  # columns of no part stay as they were
     err = (got[:, written] - ref[:, written]).abs().max().item()
-    tol = 2.0 ** -8 if dtype == torch.bfloat16 else 1e-5
+    tol = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 1e-5}[dtype]
     assert err <= tol * ref.abs().max().item(), err
 
 

@@ -13,7 +13,7 @@ import torch
 
 from cuequivariance_amd import _lib
 
-BF16, F32, F64 = 3, 0, 1
+BF16, F16, F32, F64 = 3, 2, 0, 1
 
 
 def _table(rows):
@@ -51,7 +51,7 @@ def _reference(A, W, parts, K, N, contraction_major, alpha, ldc):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("contraction_major", [1, 0])
 @pytest.mark.parametrize(
     "M,K,N,dims",
@@ -72,8 +72,8 @@ def _reference(A, W, parts, K, N, contraction_major, alpha, ldc):
     ],
 )
 def test_against_float64_product(device, dtype, contraction_major, M, K, N, dims):
-    if dtype == torch.bfloat16 and K % 64:
-        pytest.skip("a bfloat16 slice is 64 channels")
+    if dtype != torch.float32 and K % 64:
+        pytest.skip("a slice of 2-byte elements is 64 channels")
     lib = _lib.load()
     g = torch.Generator(device=device).manual_seed(M + K + N + sum(dims))
     nparts = len(dims)
@@ -89,7 +89,7 @@ def test_against_float64_product(device, dtype, contraction_major, M, K, N, dims
     out = torch.full((M, ldc), 7.0, device=device).to(dtype)
     alpha = 0.37
     stream = torch.cuda.current_stream(device).cuda_stream
-    code = BF16 if dtype == torch.bfloat16 else F32
+    code = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}[dtype]
     _lib.check(lib.cueq_linear_rows_mul_ir(code, contraction_major, M, N, K, A.data_ptr(), lda, W.data_ptr(), W.numel(), out.data_ptr(), ldc,
                                            _table(parts), nparts, alpha, stream), "cueq_linear_rows_mul_ir")
     ref = _reference(A, W, parts, K, N, contraction_major, alpha, ldc)
@@ -99,12 +99,12 @@ def test_against_float64_product(device, dtype, contraction_major, M, K, N, dims
     got = out.double()
     assert (got[:, ~written] == 7.0).all()  # columns of no part stay as they were
     err = (got[:, written] - ref[:, written]).abs().max().item()
-    tol = 2.0 ** -8 if dtype == torch.bfloat16 else 1e-5
+    tol = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 1e-5}[dtype]
     assert err <= tol * ref.abs().max().item(), err
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize(
     "rows,K,N,dims",
     [
@@ -133,7 +133,7 @@ def test_weight_gradient_against_float64_product(device, dtype, rows, K, N, dims
     part = torch.full((items, K * N), float("nan"), device=device)
     alpha = 0.61
     stream = torch.cuda.current_stream(device).cuda_stream
-    code = BF16 if dtype == torch.bfloat16 else F32
+    code = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32}[dtype]
     _lib.check(lib.cueq_linear_dw_mul_ir(code, K, N, rows, A.data_ptr(), lda, G.data_ptr(), ldg, table, len(dims), part.data_ptr(), alpha, stream),
                "cueq_linear_dw_mul_ir")
     for p, (a, c, d) in enumerate(zip(a_offs, c_offs, dims)):
