@@ -33,7 +33,9 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # published dense peaks, TFLOP/s: matrix cores per input type, and the fp32 vector units
-MFMA_PEAK = {"bf16": 2500.0, "f32": 157.3}
+MFMA_PEAK = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
+_DTYPES = {"bf16": "bfloat16", "fp16": "float16", "fp32": "float32", None: "float32"}
+_DT_NAME = {"bfloat16": "bf16", "float16": "f16", "float32": "f32"}
 VALU_PEAK_F32 = 157.3
 
 # Bytes that left the L2 per launch at the default workload (5000 nodes, 100000 edges, fp32), from two
@@ -171,7 +173,7 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
                 "50000 nodes, int32 element index, fwd + bwd (dw, dx)" + ("; buffers of bfloat16, arithmetic in float32" if es == 2 else ""))
     elif wl in ("cfg4", "cfg4mi"):
         Z = 200_000
-        dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
+        dtype = getattr(torch, _DTYPES[dtype_name])
         irreps = cue.Irreps("O3", "128x0e+128x1o+128x2e")
         # cfg4mi: the same Linear on mul_ir rows (the module's default layout), addressed inside the dense kernels
         m = cuet.Linear(irreps, irreps, layout=cue.mul_ir if wl == "cfg4mi" else cue.ir_mul, internal_weights=False, method="fused_tp")
@@ -183,8 +185,8 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         def step():
             return torch.autograd.grad(m(x, w), [w, x], cot)
 
-        unit, units, dt = "rows/s", Z, "bf16" if dtype == torch.bfloat16 else "f32"
-        es = 2 if dtype == torch.bfloat16 else 4
+        unit, units, dt = "rows/s", Z, _DT_NAME[str(dtype).replace("torch.", "")]
+        es = 4 if dtype == torch.float32 else 2
         f = 2 * Z * 128 * 128 * 9
         flops = {"fwd": f, "bwd": 2 * f}
         # fwd reads x, writes out; bwd reads x and g, writes dx (weights 49152 elements negligible)
@@ -195,7 +197,7 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
             desc += "; rows in mul_ir, addressed as they lie by the dense kernels (no transposition pass)"
     elif wl in ("cfg4fc", "cfg4fcmi"):
         Z = 50_000
-        dtype = torch.bfloat16 if dtype_name == "bf16" else torch.float32
+        dtype = getattr(torch, _DTYPES[dtype_name])
         i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e")
         # cfg4fcmi: the same product on mul_ir rows (the module's default layout), taken as they lie by the fused kernels
         m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.mul_ir if wl == "cfg4fcmi" else cue.ir_mul, internal_weights=False)
@@ -208,8 +210,8 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         def step():
             return torch.autograd.grad(m(x1, x2, w), [w, x1, x2], cot)
 
-        unit, units, dt = "rows/s", Z, "bf16" if dtype == torch.bfloat16 else "f32"
-        es = 2 if dtype == torch.bfloat16 else 4
+        unit, units, dt = "rows/s", Z, _DT_NAME[str(dtype).replace("torch.", "")]
+        es = 4 if dtype == torch.float32 else 2
         # every distinct element once: fwd reads x1, x2 and writes out; bwd reads x1, x2, g and writes dx1, dx2 (weights 20480 negligible)
         alg = {"fwd": Z * (256 + 9 + 256) * es, "bwd": Z * (256 + 9 + 256 + 256 + 9) * es}
         # 11 distinct (weight block, x1 component) products of 64 x 64 per row; forward, dx1, dx2 and dw contract each once
@@ -274,7 +276,7 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         desc = ("next row (FullyConnectedTensorProductConv's product): 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, a weight row per edge, "
                 "20000 edges, 2000 nodes, x1 gathered by source, output summed by destination, fwd + bwd (dw, dx1, dx2)")
     elif wl == "cfg5":
-        dtype = torch.float32 if dtype_name == "fp32" else torch.bfloat16
+        dtype = getattr(torch, _DTYPES[dtype_name or "bf16"])
         n, D = 512, 128
         g = torch.Generator(device=dev).manual_seed(0)
 
@@ -292,8 +294,8 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         def step():
             return torch.autograd.grad(cuet.triangle_multiplicative_update(x, "outgoing", **kw), [x], cot)
 
-        unit, units, dt = "pair rows/s", n * n, "bf16" if dtype == torch.bfloat16 else "f32"
-        es = 2 if dtype == torch.bfloat16 else 4
+        unit, units, dt = "pair rows/s", n * n, _DT_NAME[str(dtype).replace("torch.", "")]
+        es = 4 if dtype == torch.float32 else 2
         f = 2 * n * n * D * 4 * D + 2 * D * n ** 3 + 2 * n * n * D * 2 * D  # projections in, contraction, projections out
         flops = {"fwd": f, "bwd": 2 * f}
         # fwd reads z and the mask, writes the update; bwd reads z, the mask and the cotangent, writes dz
@@ -460,15 +462,20 @@ def setup_costs(torch, cue, cuet, _lib, dev, N: int, E: int, compile_probe: bool
     m = cuet.ChannelWiseTensorProduct(cue.Irreps("O3", "128x0e+128x1o+128x2e+128x3o"), cue.Irreps("O3", "0e+1o+2e+3o"), "0e+1o+2e+3o",
                                       layout=cue.ir_mul, shared_weights=False)
     out["module_build_ms"] = (time.perf_counter() - t0) * 1e3
-    plan = m.f.m._plan(torch.float32)
+    import importlib
+
+    u1d = importlib.import_module("cuequivariance_amd.cuet.uniform_1d")  # (the package also exports a function of this name)
+    cached = m.f.m._plan(torch.float32)
+    # a plan object of its own (the module's is shared through a cache and exists since the timed steps): the tables of the
+    # backward derived on the host, both sets uploaded, the generated kernels looked up
+    plan = u1d.Uniform1dPlan(cached.tables, torch.float32)
+    plan.polynomial, plan.origin = cached.polynomial, cached.origin
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     plan.handle(dev)
     plan.backward_plan((True, True, True)).handle(dev)
     torch.cuda.synchronize()
     out["plan_create_ms"] = (time.perf_counter() - t0) * 1e3
-    import importlib
-
-    u1d = importlib.import_module("cuequivariance_amd.cuet.uniform_1d")  # (the package also exports a function of this name)
 
     g = torch.Generator().manual_seed(1)
     sorted_ids = torch.sort(torch.randint(0, N, (E,), generator=g, dtype=torch.int32))[0].to(dev)
@@ -580,7 +587,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--dtype", choices=["fp32", "fp64", "bf16"], default=None,
+    ap.add_argument("--dtype", choices=["fp32", "fp64", "bf16", "fp16"], default=None,
                     help="cfg2: fp32 (default) or fp64; cfg3: fp32; cfg4: fp32 (default) or bf16; cfg5: bf16 (default) or fp32")
     ap.add_argument("--nodes", type=int, default=5000)
     ap.add_argument("--edges", type=int, default=100_000)
@@ -679,7 +686,8 @@ def main() -> int:
                             ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_linear_fp32_mul_ir", "cfg4mi", "fp32"),
                             ("cfg4_linear_bf16_mul_ir", "cfg4mi", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("cfg4_fc_fp32_mul_ir", "cfg4fcmi", "fp32"),
                             ("cfg4_fc_bf16_mul_ir", "cfg4fcmi", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
-                            ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp32", "cfg5", "fp32")):
+                            ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp16", "cfg5", "fp16"), ("cfg5_fp32", "cfg5", "fp32"),
+                            ("cfg4_linear_fp16", "cfg4", "fp16"), ("cfg4_fc_fp16", "cfg4fc", "fp16")):
             add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))
             if key in ("cfg1_fp32", "cfg4_fc_bf16", "cfg4_fc_bf16_mul_ir") and "error" not in sec[key]:
                 # workloads whose eager step is bound by the host's launch path: the same step replayed as one HIP graph
