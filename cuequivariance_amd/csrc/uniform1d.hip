@@ -71,6 +71,16 @@ static std::atomic<int>& opt_force_generic() {
 }
 bool deterministic_scatter() { return opt_deterministic().load(std::memory_order_relaxed) != 0; }
 
+// Groups of one segment each are the default row layout: such a buffer counts as having none (the Python table builder
+// drops them the same way), so that both spellings of the same rows find the same generated kernels.
+static bool has_row_layout(const cueq_u1d_desc* d, int b, int64_t first_group) {
+  if (!d->layout_num_groups || d->layout_num_groups[b] <= 0) return false;
+  if (!d->layout_group_dims) return true;  // (refused by cueq_u1d_plan_create)
+  for (int g = 0; g < d->layout_num_groups[b]; ++g)
+    if (d->layout_group_dims[first_group + g] != 1) return true;
+  return false;
+}
+
 uint64_t hash_u1d_desc(const cueq_u1d_desc* d) {
   Fnv64 f;
   const int nbuf = d->num_inputs + d->num_outputs;
@@ -99,15 +109,21 @@ uint64_t hash_u1d_desc(const cueq_u1d_desc* d) {
   }
   // row layouts (descriptors without any hash as they always did)
   bool any_layout = false;
-  if (d->layout_num_groups)
-    for (int b = 0; b < nbuf; ++b) any_layout |= d->layout_num_groups[b] > 0;
+  if (d->layout_num_groups) {
+    int64_t g0 = 0;
+    for (int b = 0; b < nbuf; ++b) {
+      any_layout |= has_row_layout(d, b, g0);
+      g0 += d->layout_num_groups[b] > 0 ? d->layout_num_groups[b] : 0;
+    }
+  }
   if (any_layout) {
     f.word(0x6C61796F757473ull);
     int64_t g0 = 0;
     for (int b = 0; b < nbuf; ++b) {
-      const int ng = d->layout_num_groups[b];
-      f.word(static_cast<uint64_t>(ng));
-      for (int g = 0; g < ng; ++g) f.word(static_cast<uint64_t>(d->layout_group_dims[g0 + g]));
+      const int ng = d->layout_num_groups[b] > 0 ? d->layout_num_groups[b] : 0;
+      const bool lay = has_row_layout(d, b, g0);
+      f.word(static_cast<uint64_t>(lay ? ng : 0));
+      for (int g = 0; lay && g < ng; ++g) f.word(static_cast<uint64_t>(d->layout_group_dims[g0 + g]));
       g0 += ng;
     }
   }
@@ -476,7 +492,7 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
           delete plan;
           CUEQ_REQUIRE(false, CUEQ_ERR_INVALID, "layout groups of buffer %d do not partition its %d channel segments", b, nseg);
         }
-        lay_off[b] = reserve(t.size() * sizeof(int32_t));
+        if (has_row_layout(d, b, g0)) lay_off[b] = reserve(t.size() * sizeof(int32_t));  // (groups of one segment: the default rows)
       }
       g0 += ng;
     }

@@ -34,9 +34,9 @@ class _FlattenedOperation(nn.Module):
     """One operation of a polynomial on the uniform-1d kernels: every mode but the last one of its output flattened
     away, that one split down to a common extent.  Built at first use."""
 
-    def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype):
+    def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype, output_dtype_map=None):
         super().__init__()
-        self._polynomial, self._math_dtype = polynomial, math_dtype
+        self._polynomial, self._math_dtype, self._output_dtype_map = polynomial, math_dtype, output_dtype_map
         self.f = None
 
     def _build(self):
@@ -59,7 +59,7 @@ class _FlattenedOperation(nn.Module):
             extents = sorted(q.operations[0][1].get_dims(keep))
             if len(extents) > 1:
                 q = q.split_mode(keep, math.gcd(*extents))
-        return SegmentedPolynomial(q, method="uniform_1d", math_dtype=self._math_dtype)
+        return SegmentedPolynomial(q, method="uniform_1d", math_dtype=self._math_dtype, output_dtype_map=self._output_dtype_map)
 
     def forward(self, inputs, input_indices, output_shapes, output_indices):
         if self.f is None:
@@ -133,7 +133,10 @@ class SegmentedPolynomialFusedTP(nn.Module):
             local = [ins.index(b) if b < self.num_inputs else len(ins) for b in ope.buffers]
             sub = cue.SegmentedPolynomial([polynomial.inputs[b] for b in ins], [polynomial.outputs[b_out - self.num_inputs]],
                                           [(cue.Operation(local), stp)])
-            self.ops.append(_FlattenedOperation(sub, math_dtype))
+            # the operation's result in the type the polynomial's output is to have (the reference sums in that type): the
+            # input it inherits from when the operation reads it, else the arithmetic type - rounded once, after the sum
+            src = self.dtypes[b_out]
+            self.ops.append(_FlattenedOperation(sub, math_dtype, [ins.index(src) if src in ins else -1]))
             self.op_inputs.append(ins)
             self.op_output.append(b_out - self.num_inputs)
 

@@ -181,6 +181,10 @@ class FullyConnectedTensorProductConv(nn.Module):
     def forward(self, src_features: torch.Tensor, edge_sh: torch.Tensor, edge_emb: torch.Tensor,
                 graph: tuple, src_scalars: Optional[torch.Tensor] = None, dst_scalars: Optional[torch.Tensor] = None,
                 reduce: str = "mean", edge_envelope: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Arguments as in the reference (``layers/tp_conv_fully_connected.py:156-276``).  Destination ids outside
+        ``[0, num_dst_nodes)`` raise an error in eager mode; while the current stream is being captured into a HIP graph the
+        grouping of the edges by destination is recorded as device work that cannot report them: such edges are left out of
+        every destination row, at capture and at every replay."""
         edge_width = edge_emb.size(-1)
         if self.mlp is None:
             if self.tp.weight_numel != edge_width:

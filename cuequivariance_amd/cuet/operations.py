@@ -189,6 +189,9 @@ class ChannelWiseTensorProduct(torch.nn.Module):
         indices_out: Optional[torch.Tensor] = None,
         size_out: Optional[int] = None,
     ) -> torch.Tensor:
+        """Arguments as in the reference (``operations/tp_channel_wise.py:186-258``).  Row ids outside ``[0, size_out)`` in ``indices_out`` raise an error in eager mode; while the current stream is being
+        captured into a HIP graph the grouping of the batch rows by output row is recorded as device work that cannot report
+        them: such batch rows are left out of every output row, at capture and at every replay."""
         x1 = apply_layout(self.transpose_in1, x1)
         x2 = apply_layout(self.transpose_in2, x2)
         indices_in: Dict[int, torch.Tensor] = {}
@@ -397,7 +400,10 @@ class FullyConnectedTensorProduct(torch.nn.Module):
                 indices_1: Optional[torch.Tensor] = None, indices_out: Optional[torch.Tensor] = None,
                 size_out: Optional[int] = None) -> torch.Tensor:
         """``indices_1`` (rows of ``x1`` per batch element) and ``indices_out`` / ``size_out`` (output row per batch
-        element, summed) are extensions over the reference's signature: gather and scatter-sum inside the kernel."""
+        element, summed) are extensions over the reference's signature: gather and scatter-sum inside the kernel.
+        Row ids outside ``[0, size_out)`` in ``indices_out`` raise an error in eager mode; while the current stream is being
+        captured into a HIP graph the grouping of the batch rows by output row is recorded as device work that cannot report
+        them: such batch rows are left out of every output row, at capture and at every replay."""
         if self.weight is not None:
             if weight is not None:
                 raise ValueError("Internal weights are used, weight should be None")

@@ -152,7 +152,9 @@ int cueq_u1d_run(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int6
  * but the workspace is a static device array of cueq_u1d_static_scratch_bytes() (32 MiB) that every device running
  * the library holds until the process ends; the call allocates nothing.  A call shape whose
  * cueq_u1d_workspace_size exceeds that returns CUEQ_ERR_TOO_LARGE.  All calls on one device share the array:
- * calls that overlap on one device (different streams or threads) race; calls on one stream do not. */
+ * calls that overlap on one device (different streams or threads) race; calls on one stream do not.  The first call on a
+ * device looks the array's address up (a host-side query, not a stream operation): make one call on each device before
+ * recording the entry point into a HIP graph. */
 int64_t cueq_u1d_static_scratch_bytes(void);
 int cueq_u1d_run_static(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch_size, void* stream);
 

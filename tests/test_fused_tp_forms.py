@@ -120,6 +120,31 @@ def test_several_operations_and_outputs(device, dtype):
           expect_dense=False)
 
 
+@pytest.mark.gpu
+def test_operations_sum_in_the_type_of_the_output(device):
+    """Mixed element types: bfloat16 features, float32 weights, the output mapped to the float32 input.  Two operations add
+    into that output, one of them reads bfloat16 inputs only: its share must reach the sum in float32 (the reference sums in
+    the mapped output type), not rounded to bfloat16 first - a rounding there would show as an error of 2^-9, a hundred
+    times the bound of 1e-5 * max|ref| held here (the products of bfloat16 values are formed in float32)."""
+    from cuequivariance_amd import cuet
+
+    a_ = random_stp("u,u,u", seed=21)
+    b_ = random_stp("u,u,u", seed=22)
+    x, y, w, out = a_.operands[0], a_.operands[1], b_.operands[1], a_.operands[2]
+    assert b_.operands[0] == x and b_.operands[2] == out
+    poly = cue.SegmentedPolynomial([x, y, w], [out], [(cue.Operation([0, 1, 3]), a_), (cue.Operation([0, 2, 3]), b_)])
+    g = torch.Generator().manual_seed(4)
+    Z = 41
+    ins = [torch.randn(Z, x.size, dtype=torch.float64, generator=g).bfloat16(), torch.randn(Z, y.size, dtype=torch.float64, generator=g).bfloat16(),
+           torch.randn(Z, w.size, dtype=torch.float64, generator=g).float()]
+    m = cuet.SegmentedPolynomial(poly, method="fused_tp", math_dtype=torch.float32, output_dtype_map=[2])
+    assert m.m.dense is None
+    ref = naive_segmented_polynomial(spec_from_polynomial(poly), [t.double() for t in ins])[0]
+    got = m([t.to(device) for t in ins])[0]
+    assert got.dtype == torch.float32
+    assert rel_err(got, ref) <= 1e-5, rel_err(got, ref)
+
+
 def test_refusals_match_the_reference():
     from cuequivariance_amd import cuet
 

@@ -90,6 +90,30 @@ def test_table_hash_with_layouts_agrees_between_python_and_c(math_code):
     assert len(seen) == 5
 
 
+@pytest.mark.parametrize("math_code", [0, 1])
+def test_groups_of_one_segment_hash_as_the_default_rows(math_code):
+    """A descriptor handed to the C ABI with every group of a buffer one segment long describes the default rows: its hash
+    (and with it the generated kernels it finds) is that of the descriptor without a layout."""
+    lib = _lib.load()
+    _, t, groups = channelwise_tables()
+    plain, keep0 = _lib.make_desc(t, math_code)
+    want = ctypes.c_uint64()
+    has_plain = lib.cueq_u1d_desc_info(ctypes.byref(plain), ctypes.byref(want))
+    nbuf = t.num_inputs + t.num_outputs
+    # spelled out by hand: buffers 1 and 3 in groups of one, then buffer 1 in groups of one next to a real layout of buffer 3
+    for lay in ({1: [1] * t.buffer_num_segments[1], 3: [1] * t.buffer_num_segments[3]}, {1: [1] * t.buffer_num_segments[1], 3: list(groups[3])}):
+        desc, keep = _lib.make_desc(t, math_code)
+        n = _lib.int32_array([len(lay.get(b, ())) for b in range(nbuf)])
+        d = _lib.int32_array([x for b in range(nbuf) for x in lay.get(b, ())])
+        desc.layout_num_groups, desc.layout_group_dims = n, d
+        got = ctypes.c_uint64()
+        has = lib.cueq_u1d_desc_info(ctypes.byref(desc), ctypes.byref(got))
+        same = t.with_layouts(lay)
+        assert got.value == same.content_hash(math_code)
+        if not same.layouts:
+            assert got.value == want.value and has == has_plain == 1
+
+
 def test_channelwise_module_drops_its_transpositions():
     from cuequivariance_amd import cuet
 

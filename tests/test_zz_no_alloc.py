@@ -49,7 +49,12 @@ def _run_both(plan, tables, inputs, modes, out_rows, batch):
         need = lib.cueq_u1d_workspace_size(plan, bufs, batch)
         assert 0 < need <= lib.cueq_u1d_static_scratch_bytes()
         if static:
+            # the entry point's contract: nothing is allocated - neither through torch nor underneath it
+            torch.cuda.synchronize(dev)
+            before = (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev), torch.cuda.mem_get_info(dev)[0])
             _lib.check(lib.cueq_u1d_run_static(plan, bufs, batch, stream), "cueq_u1d_run_static")
+            torch.cuda.synchronize(dev)
+            assert (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev), torch.cuda.mem_get_info(dev)[0]) == before
         else:
             ws = torch.empty(need, dtype=torch.uint8, device=dev)
             _lib.check(lib.cueq_u1d_run(plan, bufs, batch, ws.data_ptr(), need, stream), "cueq_u1d_run")
@@ -84,6 +89,28 @@ def test_static_scratch_matches_workspace_run(device):
             ref, got = _run_both(plan_b, bwd_w, ins, [S, B, B, B, S], [1], batch_b)
             assert not torch.isnan(got[0]).any()
             assert torch.equal(ref[0], got[0]), f"batch-reduced output, batch {batch_b}"
+        # recorded into a HIP graph (after the eager calls above, which looked the array's address up on this device):
+        # every replay gives what the eager call gives
+        batch_c = 300
+        ins = [torch.randn(batch_c, bwd.width(b), generator=g).to(device) for b in range(4)]
+        ref, _ = _run_both(plan_a, bwd, ins, [B] * 7, [batch_c] * 3, batch_c)
+        outs = [torch.zeros(batch_c, bwd.width(4 + o), device=device) for o in range(3)]
+        bufs_c = _buffers([*ins, *outs], [B] * 7)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                _lib.check(lib.cueq_u1d_run_static(plan_a, bufs_c, batch_c, torch.cuda.current_stream().cuda_stream), "cueq_u1d_run_static")
+        torch.cuda.current_stream().wait_stream(side)
+        for replay in range(3):
+            for o in outs:
+                o.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for name, r, q in zip(("dw", "dx1", "dx2"), ref, outs):
+                assert torch.equal(r, q), f"graph replay {replay}: {name}"
         # beyond the static array: refused with a clear error, nothing launched
         batch = 400_000  # 400 000 rows x 2 halves x 16 floats = 51 MB of partials
         bufs = (_lib.U1dBuffer * 7)()
