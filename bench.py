@@ -48,6 +48,24 @@ MEASURED_TRAFFIC_BYTES = {
     ("c128_l3_fwd_float", 5000, 100_000): 2.143e9,
 }
 
+# What the memory system of this part delivers to kernels of the access shape used here (64-thread workgroups, a dword per
+# lane and instruction; `python bench.py --calibrate`, profiles/memory_system_calibration.txt): a read stream, a copy (bytes
+# read + written) and float atomic adds.  With the measured traffic above they give the least time this decomposition of the
+# headline step can take: forward = its L2-miss traffic at the read rate; backward = the longer of its 2.05e8 atomic adds
+# (edges x 2048 values of the node gradient) at the atomic rate and its L2-miss traffic at the copy rate.
+CAL_READ_BPS, CAL_COPY_BPS, CAL_ATOMIC_ADDS_PER_S = 7.09e12, 5.81e12, 3.2e11
+CAL_SOURCE = ("profiles/memory_system_calibration.txt (read 7.09 TB/s, copy 5.81 TB/s, 3.2e11 float atomic adds/s) with the traffic of "
+              "profiles/channelwise_c128_l3_fp32_cfg2_hbm_traffic.txt")
+
+
+def design_ceiling(N: int, E: int, alg: dict):
+    """Least times (s) of forward and backward of the default headline workload for this decomposition on this part, or None."""
+    f, b = MEASURED_TRAFFIC_BYTES.get(("c128_l3_fwd_float", N, E)), MEASURED_TRAFFIC_BYTES.get(("c128_l3_bwd_float", N, E))
+    if f is None or b is None:
+        return None
+    return {"fwd": f / CAL_READ_BPS, "bwd": max(E * 2048 / CAL_ATOMIC_ADDS_PER_S, b / CAL_COPY_BPS)}
+
+
 # Vector (wave64) instructions the generated kernels execute per batch element (sample, edge, node), forward and backward,
 # counted with rocprofv3 --pmc SQ_INSTS_VALU over one launch each and divided by the batch size (summary and command:
 # profiles/uniform1d_fp32_valu_instruction_counts.txt).  A wave64 instruction is at most 64 fused multiply-adds =
@@ -409,6 +427,7 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
         }
     dominant = max(per_kernel.items(), key=lambda kv: kv[1]["avg_ms"]) if per_kernel else None
     roofline = None
+    ceiling = design_ceiling(N, E, alg) if (dtype == torch.float32 and not deterministic) else None
     if dominant is not None:
         a = dominant[1]["achieved_GBps"]
         traffic = MEASURED_TRAFFIC_BYTES.get((dominant[0], N, E)) if not deterministic else None
@@ -418,6 +437,12 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
             "kernel": dominant[0], "avg_ms": dominant[1]["avg_ms"],
             "algorithmic_bytes_per_launch": dominant[1]["algorithmic_bytes"],
         }
+        if ceiling is not None and traffic:
+            # the fraction of the 8 TB/s roofline this kernel would reach at its least time (see design_ceiling)
+            kind = "fwd" if "_fwd_" in dominant[0] else "bwd"
+            roofline["design_ceiling_frac"] = dominant[1]["algorithmic_bytes"] / ceiling[kind] / 1e9 / HBM_PEAK_GBS
+            roofline["design_ceiling_ms"] = ceiling[kind] * 1e3
+            roofline["design_ceiling_source"] = CAL_SOURCE
     total_alg = alg["fwd"] + alg["bwd"]
     valu_flops = E * sum(VALU_INSTS_PER_ELEMENT["cfg2"]) * 128  # executed vector instructions x 128 flops
     line = {
@@ -443,6 +468,7 @@ def run_cfg2(torch, cue, cuet, _lib, dev, dtype, N: int, E: int, steps: int, war
         },
         "roofline": roofline,
         "step_roofline_frac": (total_alg / (elapsed / steps)) / 1e9 / HBM_PEAK_GBS,
+        "step_design_ceiling_frac": (total_alg / (ceiling["fwd"] + ceiling["bwd"])) / 1e9 / HBM_PEAK_GBS if ceiling else None,
         "step_valu_frac": valu_flops / (elapsed / steps) / 1e12 / (78.6 if dtype == torch.float64 else VALU_PEAK_F32),
         "valu_source": VALU_SOURCE,
         "kernels": per_kernel,
