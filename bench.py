@@ -320,6 +320,12 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         alg = {"fwd": (2 * n * n * D + n * n) * es, "bwd": (3 * n * n * D + n * n) * es}
         flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = "configs[4]: triangle multiplicative update, outgoing, z [1,512,512,128], mask Bernoulli(0.9), fwd + bwd w.r.t. z"
+        # What the stages of this decomposition move at the least (the normalised input, a, b, t, y and their cotangents live
+        # in HBM between the launches): per pair row and channel, in elements - forward: x read, x-hat written, a|b (2)
+        # written and read, t written and read, y written, x-hat and y read, out written = 12; backward: dout, x-hat, y read,
+        # dx-hat and dy written, dy and t read, dt written, dt read twice with a and b, da|db (2) written and read, x and
+        # x-hat and dx-hat read, dx written = 20.
+        extra = {"decomposition_traffic_bytes": (12 + 20) * n * n * D * es}
     else:
         raise ValueError(wl)
     if graph:
@@ -358,6 +364,9 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
     if graph:
         desc += "; the step replayed as one HIP graph"
     roofs = _roofs(alg["fwd"] + alg["bwd"], flops["fwd"] + flops["bwd"], elapsed, flop_peak, flop_roof)
+    more = dict(extra) if wl == "cfg5" else {}
+    if more:  # the step against 8 TB/s on the bytes its own stages must move (the binding roof of the 2-byte step as decomposed)
+        more["hbm_frac_of_decomposition_traffic"] = more["decomposition_traffic_bytes"] / elapsed / 1e9 / HBM_PEAK_GBS
     achieved = ((alg["fwd"] + alg["bwd"]) / elapsed / 1e9) if roofs["bound"] == "hbm" else ((flops["fwd"] + flops["bwd"]) / elapsed / 1e12)
     return {
         "metric": f"{unit.split('/')[0]}/sec, {wl} fwd+bwd (secondary workload)", "value": units / elapsed, "unit": unit, "n_gpus": 1,
@@ -366,7 +375,7 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         "roofline": {"bound": roofs["bound"], "achieved": achieved, "peak": HBM_PEAK_GBS if roofs["bound"] == "hbm" else flop_peak,
                      "unit": "GB/s" if roofs["bound"] == "hbm" else "TFLOP/s", "frac": roofs["frac"], "traffic": None,
                      "hbm_frac": roofs["hbm_frac"], f"{flop_roof}_frac": roofs[f"{flop_roof}_frac"],
-                     "algorithmic_bytes": roofs["algorithmic_bytes"], "flops": roofs["flops"],
+                     "algorithmic_bytes": roofs["algorithmic_bytes"], "flops": roofs["flops"], **more,
                      "scope": "whole step: algorithmic bytes and flops of forward + backward over the step time, against 8 TB/s and the "
                               f"{flop_roof} peak ({flop_peak} TFLOP/s); bound = the roof with the longer minimum time"
                               + ("; flops = 2 (2 l3 + 1) per weight, forward once and backward twice (algorithmic)" if wl == "fcconv" else
@@ -602,7 +611,7 @@ def _compact(line: dict) -> dict:
     r = line["roofline"]
     out = {"ms_per_step": line["ms_per_step"], "value": line["value"], "unit": line["unit"], "dtype": line["dtype"],
            "bound": r["bound"], "frac": r["frac"], "workload": line["config"]["workload"]}
-    for k in ("hbm_frac", "mfma_frac", "valu_frac"):
+    for k in ("hbm_frac", "mfma_frac", "valu_frac", "decomposition_traffic_bytes", "hbm_frac_of_decomposition_traffic"):
         if k in r:
             out[k] = r[k]
     return out
