@@ -33,3 +33,15 @@ def _kernels_at_first_use_off():
     jit.enable(False)
     yield
 
+
+
+@pytest.fixture
+def jit_on(tmp_path, monkeypatch):
+    """Compilation at first use switched on for one test, into an empty cache; the previous state comes back afterwards."""
+    from cuequivariance_amd import jit
+
+    was = jit.enabled()
+    monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
+    jit.enable(True)
+    yield
+    jit.enable(was)

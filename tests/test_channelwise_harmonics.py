@@ -111,15 +111,16 @@ def test_cfg2_descriptor_with_harmonics_in_the_kernels(device, dtype, determinis
 def test_other_descriptor_with_harmonics(device, first_use, tmp_path, monkeypatch):
     """48 channels, degrees 0..2, unnormalised vectors: the table-driven kernels run the substituted polynomial as it is; with
     compilation at first use the channel-wise generator makes the unit."""
+    was = jit.enabled()
     if first_use:
         monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
-        jit.enable(True)
+    jit.enable(first_use)
     try:
         for dtype in (torch.float64, torch.float32):
             m = run_case(device, "48x0e+48x1o+48x1e", [0, 1, 2], ["0e", "1o", "1e", "2o"], 40, 333, dtype, seed=42, normalize=False)
             assert m.f.m._plan(dtype).specialised(device) == first_use
     finally:
-        jit.enable(False)
+        jit.enable(was)
 
 
 @pytest.mark.gpu
@@ -135,6 +136,7 @@ def test_harmonics_with_mul_ir_rows(device, tmp_path, monkeypatch):
         return torch.cat(outs, 1)
 
     monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
+    was = jit.enabled()
     jit.enable(True)
     try:
         i1 = cue.Irreps("O3", "32x0e+32x1o+32x2e")
@@ -151,7 +153,7 @@ def test_harmonics_with_mul_ir_rows(device, tmp_path, monkeypatch):
         assert (to_mul_ir(ya.cpu(), a.irreps_out) - yb.cpu()).abs().max().item() <= 1e-12 * ya.abs().max().item()
         assert b.f.m._plan(torch.float64).specialised(device)
     finally:
-        jit.enable(False)
+        jit.enable(was)
 
 
 @pytest.mark.gpu

@@ -12,14 +12,6 @@ from cuequivariance_amd.cue import descriptors
 from cuequivariance_amd.tables import U1dTables
 
 
-@pytest.fixture
-def jit_on(tmp_path, monkeypatch):
-    monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
-    jit.enable(True)
-    yield
-    jit.enable(False)
-
-
 def flattened_tables(polynomial):
     from cuequivariance_amd.codegen.registry import flattened_fully_connected_tables
 

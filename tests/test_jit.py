@@ -10,14 +10,6 @@ from cuequivariance_amd.tables import U1dTables
 from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
 
 
-@pytest.fixture
-def jit_on(tmp_path, monkeypatch):
-    monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
-    jit.enable(True)
-    yield
-    jit.enable(False)
-
-
 def test_compile_load_and_register(jit_on):
     """A 24-channel l <= 1 product: not in the build's registry; after ``ensure_specialised`` the library reports
     specialised kernels for the forward tables and for the full backward tables, and a second call finds the cached

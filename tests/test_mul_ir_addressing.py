@@ -251,16 +251,6 @@ def test_second_derivative_mul_ir(device):
 
 
 # --------------------------------------------------------------------------- kernels generated at first use
-@pytest.fixture
-def jit_on(tmp_path, monkeypatch):
-    from cuequivariance_amd import jit
-
-    monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
-    jit.enable(True)
-    yield
-    jit.enable(False)
-
-
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,ir1,lmax", [(torch.float32, "40x0e+40x1o+40x2e", 2), (torch.float64, "24x0e+24x1o+24x2e+24x3o", 3)])
 def test_first_use_kernels_mul_ir(device, dtype, ir1, lmax, jit_on):
@@ -321,11 +311,12 @@ def test_symmetric_contraction_other_descriptor_mul_ir(device, first_use, tmp_pa
     """48 channels, degree 2: the table-driven kernels, and a unit compiled at first use."""
     from cuequivariance_amd import jit
 
+    was = jit.enabled()
     if first_use:
         monkeypatch.setenv("CUEQ_AMD_JIT_CACHE", str(tmp_path))
-        jit.enable(True)
+    jit.enable(first_use)
     try:
         m = run_symmetric_case(device, "48x0e+48x1o+48x2e", "48x0e+48x1o", 2, 3, 77, torch.float64, seed=32)
         assert m.f.m._plan(torch.float64).specialised(device) == first_use
     finally:
-        jit.enable(False)
+        jit.enable(was)
