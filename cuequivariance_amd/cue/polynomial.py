@@ -240,6 +240,27 @@ class SegmentedPolynomial:
     def __hash__(self):
         return hash((self.inputs, self.outputs, self.operations))
 
+    def pack(self) -> str:
+        """The polynomial as one line of text (operand shapes, and per operation its buffers and the tensor product's own
+        ``to_base64``); ``unpack`` rebuilds an equal polynomial.  Traced graphs carry it in place of the object."""
+        import json
+
+        def shape(o):
+            return [o.ndim, [list(seg) for seg in o.segments]]
+
+        return json.dumps({"inputs": [shape(o) for o in self.inputs], "outputs": [shape(o) for o in self.outputs],
+                           "operations": [[list(ope.buffers), stp.to_base64()] for ope, stp in self.operations]},
+                          separators=(",", ":"))
+
+    @classmethod
+    def unpack(cls, text: str) -> "SegmentedPolynomial":
+        import json
+
+        data = json.loads(text)
+        inputs = [SegmentedOperand(seg, ndim=ndim) for ndim, seg in data["inputs"]]
+        outputs = [SegmentedOperand(seg, ndim=ndim) for ndim, seg in data["outputs"]]
+        return cls(inputs, outputs, [(Operation(b), SegmentedTensorProduct.from_base64(t)) for b, t in data["operations"]])
+
     def __eq__(self, o):
         if not isinstance(o, SegmentedPolynomial):
             return NotImplemented

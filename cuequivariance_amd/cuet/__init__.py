@@ -6,6 +6,7 @@ from .operations import ChannelWiseSphericalTensorProduct, ChannelWiseTensorProd
 from .uniform_1d import uniform_1d
 from .triangle import triangle_multiplicative_update, TriMulPrecision
 from . import layers
+from . import dense as _dense  # noqa: F401  (defines the operators dense_fwd / dense_bwd that saved graphs of Linear and the fully connected product call)
 
 __all__ = [
     "TransposeSegments",

@@ -17,9 +17,9 @@ those kernels refuse go through ``cueq_seg_gemm`` / ``cueq_seg_outer`` / ``cueq_
 from __future__ import annotations
 
 import ctypes as C
-import itertools
+import json
 import threading
-import weakref
+from collections import OrderedDict
 from typing import Dict, List, Optional
 
 import torch
@@ -1110,9 +1110,9 @@ class _IndexedDw(torch.autograd.Function):
 
 # ---------------------------------------------------------------------- traced execution (torch.compile / export)
 # Forward and backward of the two shared-weight functions as opaque operators.  They call the static methods above with
-# a plain object in place of the autograd context; the module travels as a small integer.
-_traced_modules: dict = {}
-_traced_ids = itertools.count()
+# a plain object in place of the autograd context; the module travels as the text of its constructor's arguments, so
+# that a graph saved by one process can be loaded by another (the module is then built again from that text).
+_traced_modules: "OrderedDict[str, SegmentedPolynomialDense]" = OrderedDict()
 _traced_lock = threading.Lock()
 _FUNCTIONS = (_DenseFunction, _FcFunction)
 
@@ -1122,28 +1122,39 @@ class _PlainContext:
         self.saved_tensors = tensors
 
 
-def _module_by_id(mod_id: int) -> "SegmentedPolynomialDense":
-    mod = _traced_modules[mod_id]()
-    if mod is None:
-        raise RuntimeError("fused_tp: the module this graph was traced from no longer exists")
-    return mod
+def _module_by_key(key: str) -> "SegmentedPolynomialDense":
+    with _traced_lock:
+        mod = _traced_modules.get(key)
+        if mod is not None:
+            _traced_modules.move_to_end(key)
+            return mod
+    a = json.loads(key)
+    return SegmentedPolynomialDense(cue.SegmentedPolynomial.unpack(a["polynomial"]), a["math_dtype"], a["output_dtype_map"], a["name"],
+                                    a["method"], a["rows"], a["row_blocks"])  # (registers itself under the same text)
+
+
+def _remember_traced(key: str, mod: "SegmentedPolynomialDense") -> None:
+    with _traced_lock:
+        _traced_modules[key] = mod
+        while len(_traced_modules) > 256:
+            _traced_modules.popitem(last=False)
 
 
 @torch.library.custom_op("cuequivariance_amd::dense_fwd", mutates_args=(), device_types="cuda")
-def _dense_fwd_op(mod_id: int, kind: int, w: torch.Tensor, x1: torch.Tensor, x2: Optional[torch.Tensor]) -> torch.Tensor:
-    return _FUNCTIONS[kind].forward(_PlainContext(), _module_by_id(mod_id), w, x1, x2)
+def _dense_fwd_op(mod_key: str, kind: int, w: torch.Tensor, x1: torch.Tensor, x2: Optional[torch.Tensor]) -> torch.Tensor:
+    return _FUNCTIONS[kind].forward(_PlainContext(), _module_by_key(mod_key), w, x1, x2)
 
 
 @_dense_fwd_op.register_fake
-def _dense_fwd_fake(mod_id, kind, w, x1, x2):
-    return x1.new_empty(x1.shape[0], _module_by_id(mod_id).out_size)
+def _dense_fwd_fake(mod_key, kind, w, x1, x2):
+    return x1.new_empty(x1.shape[0], _module_by_key(mod_key).out_size)
 
 
 @torch.library.custom_op("cuequivariance_amd::dense_bwd", mutates_args=(), device_types="cuda")
-def _dense_bwd_op(mod_id: int, kind: int, w: torch.Tensor, x1: torch.Tensor, x2: Optional[torch.Tensor], g: torch.Tensor,
+def _dense_bwd_op(mod_key: str, kind: int, w: torch.Tensor, x1: torch.Tensor, x2: Optional[torch.Tensor], g: torch.Tensor,
                   need: List[bool]) -> List[torch.Tensor]:
     ctx = _PlainContext()
-    ctx.mod, ctx.has_x2 = _module_by_id(mod_id), x2 is not None
+    ctx.mod, ctx.has_x2 = _module_by_key(mod_key), x2 is not None
     ctx.saved_tensors = (w, x1, x2 if (x2 is not None or kind == 1) else torch.empty(0))
     ctx.needs_input_grad = (False, *need)
     if kind == 0:
@@ -1154,22 +1165,22 @@ def _dense_bwd_op(mod_id: int, kind: int, w: torch.Tensor, x1: torch.Tensor, x2:
 
 
 @_dense_bwd_op.register_fake
-def _dense_bwd_fake(mod_id, kind, w, x1, x2, g, need):
+def _dense_bwd_fake(mod_key, kind, w, x1, x2, g, need):
     return [torch.empty_like(t) if (n and t is not None) else x1.new_empty(0) for t, n in zip((w, x1, x2), need)]
 
 
 def _dense_setup_context(ctx, inputs, output):
-    mod_id, kind, w, x1, x2 = inputs
-    ctx.meta = (mod_id, kind, x2 is not None)
+    mod_key, kind, w, x1, x2 = inputs
+    ctx.meta = (mod_key, kind, x2 is not None)
     ctx.save_for_backward(w, x1, *([x2] if x2 is not None else []))
 
 
 def _dense_autograd(ctx, g):
-    mod_id, kind, has_x2 = ctx.meta
+    mod_key, kind, has_x2 = ctx.meta
     w, x1 = ctx.saved_tensors[:2]
     x2 = ctx.saved_tensors[2] if has_x2 else None
     need = [bool(n) for n in ctx.needs_input_grad[2:5]]
-    got = _dense_bwd_op(mod_id, kind, w, x1, x2, g.contiguous(), need)
+    got = _dense_bwd_op(mod_key, kind, w, x1, x2, g.contiguous(), need)
     gw, gx1, gx2 = [t if t.numel() > 0 else None for t in got]
     return None, None, gw, gx1, gx2
 
@@ -1178,8 +1189,8 @@ torch.library.register_autograd("cuequivariance_amd::dense_fwd", _dense_autograd
 
 
 def _apply_dense(kind: int, mod: "SegmentedPolynomialDense", w, x1, x2):
-    if torch.compiler.is_compiling() or type(x1) not in (torch.Tensor, torch.nn.Parameter):
-        return _dense_fwd_op(mod.traced_id, kind, w, x1, x2)
+    if torch.compiler.is_compiling() or torch.jit.is_tracing() or type(x1) not in (torch.Tensor, torch.nn.Parameter):
+        return _dense_fwd_op(mod.traced_key, kind, w, x1, x2)
     return _FUNCTIONS[kind].apply(mod, w, x1, x2)
 
 
@@ -1250,9 +1261,13 @@ class SegmentedPolynomialDense(nn.Module):
                 raise NotImplementedError("fused_tp: rows='mul_ir' of a 4-operand contraction needs row_blocks")
             self.fc_blocks = (starts(row_blocks[0], self.input_sizes[1]), starts(row_blocks[1], self.out_size))
         self.rows_mul_ir = rows == "mul_ir"
-        with _traced_lock:  # the integer under which a traced graph names this module
-            self.traced_id = next(_traced_ids)
-            _traced_modules[self.traced_id] = weakref.ref(self)
+        # the text under which a traced graph names this module: the arguments it was built from
+        self.traced_key = json.dumps({
+            "polynomial": polynomial.pack(), "math_dtype": None if math_dtype is None else str(math_dtype).split(".")[-1],
+            "output_dtype_map": None if output_dtype_map is None else [int(i) for i in output_dtype_map], "name": name, "method": method,
+            "rows": rows, "row_blocks": None if row_blocks is None else [[[int(m), int(d)] for m, d in blocks] for blocks in row_blocks]},
+            separators=(",", ":"))
+        _remember_traced(self.traced_key, self)
 
     def fused_unit(self, dtype, *row_tensors):
         """The kernels generated for this product (``codegen/fullyconnected.py``; compiled at first use), or ``None``:

@@ -493,13 +493,14 @@ class _TriMul(torch.autograd.Function):
 
 # ---------------------------------------------------------------------- traced execution (torch.compile / export)
 # Two opaque operators, forward and backward, around the same two functions.  Optional tensors travel as empty
-# placeholders plus a presence list (operator schemas have no optional entries inside tensor lists).
+# placeholders plus a presence list (operator schemas have no optional entries inside tensor lists; the list holds
+# integers because torch.jit.trace does not take lists of booleans).
 def _placeholders(ref: torch.Tensor, tensors):
-    return [ref.new_empty(0) if t is None else t for t in tensors], [t is not None for t in tensors]
+    return [ref.new_empty(0) if t is None else t for t in tensors], [int(t is not None) for t in tensors]
 
 
 @torch.library.custom_op("cuequivariance_amd::trimul_fwd", mutates_args=(), device_types="cuda")
-def _trimul_fwd_op(x: torch.Tensor, tensors: List[torch.Tensor], present: List[bool], outgoing: bool, eps: float) -> List[torch.Tensor]:
+def _trimul_fwd_op(x: torch.Tensor, tensors: List[torch.Tensor], present: List[int], outgoing: bool, eps: float) -> List[torch.Tensor]:
     args = [t if p else None for t, p in zip(tensors, present)]  # mask, then the 12 weights
     out, saved, _, _ = _trimul_fwd(x, *args, outgoing, eps)
     return [out, *saved[12:]]  # + xh, mean1, rstd1, ab, t2, mean2, rstd2, y
@@ -516,7 +517,7 @@ def _trimul_fwd_fake(x, tensors, present, outgoing, eps):
 
 
 @torch.library.custom_op("cuequivariance_amd::trimul_bwd", mutates_args=(), device_types="cuda")
-def _trimul_bwd_op(dout: torch.Tensor, x: torch.Tensor, tensors: List[torch.Tensor], computed: List[torch.Tensor], present: List[bool],
+def _trimul_bwd_op(dout: torch.Tensor, x: torch.Tensor, tensors: List[torch.Tensor], computed: List[torch.Tensor], present: List[int],
                    need: List[bool], outgoing: bool) -> List[torch.Tensor]:
     mask, nin_w, nin_b, p_in_w, p_in_b, g_in_w, g_in_b, nout_w, nout_b, p_out_w, p_out_b, g_out_w, g_out_b = [
         t if p else None for t, p in zip(tensors, present)]
@@ -650,7 +651,7 @@ def triangle_multiplicative_update(
         Bsz *= s
     xf = x.reshape(Bsz, N, N, D).contiguous()
     mf = None if mask is None else mask.reshape(Bsz, N, N).to(T).contiguous()
-    if torch.compiler.is_compiling() or type(xf) not in (torch.Tensor, torch.nn.Parameter):
+    if torch.compiler.is_compiling() or torch.jit.is_tracing() or type(xf) not in (torch.Tensor, torch.nn.Parameter):
         tensors, present = _placeholders(xf, [mf, *args])
         out = _trimul_fwd_op(xf, tensors, present, direction == "outgoing", float(eps))[0]
     else:

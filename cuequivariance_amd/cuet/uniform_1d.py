@@ -18,10 +18,8 @@ Everything executes through the C ABI in ``libcueq_amd.so``; CPU tensors are rej
 from __future__ import annotations
 
 import ctypes as C
-import itertools
 import threading
 import warnings
-import weakref
 from collections import OrderedDict
 from typing import List, Optional, Sequence
 
@@ -49,17 +47,31 @@ _DTYPE_CODE = {
 }
 
 
-_traced_plans: dict = {}
-_traced_ids = itertools.count()
+_traced_plans: "OrderedDict[str, Uniform1dPlan]" = OrderedDict()
 _PLAIN_TENSORS = (torch.Tensor, torch.nn.Parameter)
 _traced_lock = threading.Lock()
+_DTYPE_BY_NAME = {"float32": torch.float32, "float64": torch.float64}
 
 
-def _plan_by_id(plan_id: int) -> "Uniform1dPlan":
-    plan = _traced_plans[plan_id]()
-    if plan is None:
-        raise RuntimeError("uniform_1d: the module this graph was traced from no longer exists")
+def _plan_by_key(key: str) -> "Uniform1dPlan":
+    """The plan a traced graph names: the one that wrote the key while it is known here, else one built from the key (a
+    graph saved by one process and loaded by another carries everything the plan is made of)."""
+    with _traced_lock:
+        plan = _traced_plans.get(key)
+        if plan is not None:
+            _traced_plans.move_to_end(key)
+            return plan
+    name, dtype_name, packed = key.split("|", 2)
+    plan = _cached_plan(Uniform1dPlan(U1dTables.unpack(packed), _DTYPE_BY_NAME[dtype_name], name=name))
+    _remember_traced(key, plan)
     return plan
+
+
+def _remember_traced(key: str, plan: "Uniform1dPlan") -> None:
+    with _traced_lock:
+        _traced_plans[key] = plan
+        while len(_traced_plans) > 256:
+            _traced_plans.popitem(last=False)
 
 
 class Uniform1dPlan:
@@ -81,10 +93,10 @@ class Uniform1dPlan:
         self.polynomial = None  # the flattened polynomial the tables came from, when the caller has it
         self.origin = None      # the polynomial that one was flattened from (a fully connected product's descriptor)
         self._lock = threading.Lock()
-        # small integer under which a traced graph (torch.compile / export) names this plan
-        with _traced_lock:
-            self.traced_id = next(_traced_ids)  # (never reused: entries of plans that are gone are dropped)
-            _traced_plans[self.traced_id] = weakref.ref(self)
+        # under this text a traced graph (torch.compile, torch.export, torch.jit.trace) names the plan: operator name,
+        # arithmetic type and the packed tables, so that a saved graph stays valid where this object does not exist
+        self.traced_key = f"{name.replace('|', '/')}|{str(math_dtype).split('.')[-1]}|{tables.pack()}"
+        _remember_traced(self.traced_key, self)
 
     def __getattr__(self, item):
         # table fields (operand_extent, num_inputs, buffer_dim, ...) read through
@@ -98,6 +110,7 @@ class Uniform1dPlan:
 
     def key(self) -> tuple:
         return (self.math_dtype, self.tables)
+
 
     def specialised(self, device: torch.device) -> bool:
         """True when kernels generated for exactly these tables are linked into the library."""
@@ -152,11 +165,6 @@ class Uniform1dPlan:
 
     def __del__(self):
         try:
-            with _traced_lock:
-                _traced_plans.pop(self.traced_id, None)
-        except Exception:
-            pass
-        try:
             lib = _lib.load()
             for h in self._handles.values():
                 lib.cueq_u1d_plan_destroy(h)
@@ -200,6 +208,9 @@ def _backward_choice(plan: Uniform1dPlan, needs: tuple, device: torch.device) ->
 
 _plan_cache: "OrderedDict[tuple, Uniform1dPlan]" = OrderedDict()
 _plan_cache_lock = threading.Lock()
+
+
+_seam_plans: dict = {}  # argument lists of ``uniform_1d`` (as tuples) -> plan
 
 
 def _cached_plan(plan: Uniform1dPlan) -> Uniform1dPlan:
@@ -434,17 +445,17 @@ class _Uniform1dFunction(torch.autograd.Function):
 # Under torch.compile / torch.export the launch is one opaque operator (the Python above it - resolving batch modes
 # and row counts - is traced as ordinary integer arithmetic); eager calls keep the lighter autograd.Function path.
 @torch.library.custom_op("cuequivariance_amd::u1d_launch", mutates_args=(), device_types="cuda")
-def _u1d_launch_op(plan_id: int, modes: List[int], index_of: List[int], rows: List[int], batch: int,
+def _u1d_launch_op(plan_key: str, modes: List[int], index_of: List[int], rows: List[int], batch: int,
                    tensors: List[torch.Tensor]) -> List[torch.Tensor]:
-    plan = _plan_by_id(plan_id)
+    plan = _plan_by_key(plan_key)
     nin = plan.num_inputs
     outs = _launch(plan, _CallConfig(modes, index_of, rows, batch), [t.detach() for t in tensors[:nin]], tensors[nin:])
     return list(outs)
 
 
 @_u1d_launch_op.register_fake
-def _u1d_launch_fake(plan_id, modes, index_of, rows, batch, tensors):
-    plan = _plan_by_id(plan_id)
+def _u1d_launch_fake(plan_key, modes, index_of, rows, batch, tensors):
+    plan = _plan_by_key(plan_key)
     nin = plan.num_inputs
     outs = []
     for o in range(plan.num_outputs):
@@ -454,14 +465,14 @@ def _u1d_launch_fake(plan_id, modes, index_of, rows, batch, tensors):
 
 
 def _u1d_setup_context(ctx, inputs, output):
-    plan_id, modes, index_of, rows, batch, tensors = inputs
-    ctx.meta = (plan_id, tuple(modes), tuple(index_of), tuple(rows), batch)
+    plan_key, modes, index_of, rows, batch, tensors = inputs
+    ctx.meta = (plan_key, tuple(modes), tuple(index_of), tuple(rows), batch)
     ctx.save_for_backward(*tensors)
 
 
 def _u1d_backward(ctx, grad_outputs):
-    plan_id, modes, index_of, rows, batch = ctx.meta
-    plan = _plan_by_id(plan_id)
+    plan_key, modes, index_of, rows, batch = ctx.meta
+    plan = _plan_by_key(plan_key)
     nin = plan.num_inputs
     tensors = ctx.saved_tensors
     inputs, indices = tensors[:nin], tensors[nin:]
@@ -480,7 +491,7 @@ def _u1d_backward(ctx, grad_outputs):
                                 dtype=plan.math_dtype if src < 0 else inputs[src].dtype)
             cots.append(g)
         flagged = [i for i, n in enumerate(computed) if n]
-        got = _u1d_launch_op(bplan.traced_id, list(modes) + [modes[i] for i in flagged], list(index_of) + [index_of[i] for i in flagged],
+        got = _u1d_launch_op(bplan.traced_key, list(modes) + [modes[i] for i in flagged], list(index_of) + [index_of[i] for i in flagged],
                              list(rows) + [rows[i] for i in flagged], batch, [*inputs, *cots, *indices])
         for g, i in zip(got, flagged):
             if needs[i]:
@@ -542,8 +553,10 @@ def run_plan(plan: Uniform1dPlan, batch_dim: Sequence[int], index_buffer: Sequen
             modes[b] = BATCH_DIM_BATCHED
             rows[b] = batch
     # (traced: under Dynamo, or called with the tracer's tensor subclasses when a composite operator is decomposed)
-    if torch.compiler.is_compiling() or (inputs and type(inputs[0]) not in _PLAIN_TENSORS):
-        return list(_u1d_launch_op(plan.traced_id, modes, list(index_buffer[: nin + nout]), rows, batch, [*inputs, *indices]))
+    if torch.jit.is_tracing():  # (the tracer hands out sizes as tensors: row counts become constants of the trace)
+        rows, batch = [int(r) for r in rows], int(batch)
+    if torch.compiler.is_compiling() or torch.jit.is_tracing() or (inputs and type(inputs[0]) not in _PLAIN_TENSORS):
+        return list(_u1d_launch_op(plan.traced_key, modes, list(index_buffer[: nin + nout]), rows, batch, [*inputs, *indices]))
     cfg = _CallConfig(modes, list(index_buffer[: nin + nout]), rows, batch)
     if len(plan._configs) >= 64:  # (call shapes of a module are few; a stream of ever new batch sizes starts over)
         plan._configs.clear()
@@ -584,14 +597,25 @@ def uniform_1d(
     """
     if len(num_operands) != num_operations:
         raise ValueError("uniform_1d: num_operations does not match num_operands")
-    plan = _cached_plan(
-        Uniform1dPlan(
-            U1dTables.make(
-                operand_extent, num_inputs, num_outputs, buffer_dim, buffer_num_segments, dtypes, num_operands,
-                operations, num_paths, path_indices_start, path_coefficients_start, path_indices, path_coefficients,
-            ),
-            math_dtype,
-            name=name,
+    # the frontend passes the same lists on every call: the plan is looked up by their values (tuples hash in a few
+    # microseconds; building and hashing the tables takes a hundred and more for a few hundred paths)
+    key = (name, math_dtype, operand_extent, num_inputs, num_outputs, tuple(buffer_dim), tuple(buffer_num_segments), tuple(dtypes),
+           tuple(num_operands), tuple(operations), tuple(num_paths), tuple(path_indices_start), tuple(path_coefficients_start),
+           tuple(path_indices), tuple(path_coefficients))
+    plan = _seam_plans.get(key)
+    if plan is None:
+        plan = _cached_plan(
+            Uniform1dPlan(
+                U1dTables.make(
+                    operand_extent, num_inputs, num_outputs, buffer_dim, buffer_num_segments, dtypes, num_operands,
+                    operations, num_paths, path_indices_start, path_coefficients_start, path_indices, path_coefficients,
+                ),
+                math_dtype,
+                name=name,
+            )
         )
-    )
+        with _plan_cache_lock:
+            if len(_seam_plans) >= 256:
+                _seam_plans.pop(next(iter(_seam_plans)))
+            _seam_plans[key] = plan
     return run_plan(plan, batch_dim, index_buffer, batch_size, num_index, tensors)

@@ -181,6 +181,60 @@ class U1dTables:
             out = out.with_layouts(lay)
         return out
 
+    def pack(self) -> str:
+        """The tables as one line of text (two base64 fields of deflated bytes: the integers as little-endian int64, the
+        coefficients as float64): what a traced graph carries in place of the object, so that a saved graph can be loaded
+        where the object does not exist.  ``unpack`` inverts it exactly."""
+        import base64
+        import zlib
+
+        nbuf = self.num_inputs + self.num_outputs
+        lay = []
+        for b in range(nbuf if self.layouts else 0):
+            lay += [len(self.layouts[b]), *self.layouts[b]]
+        ints = [self.operand_extent, self.num_inputs, self.num_outputs, len(self.num_operands), len(self.operations),
+                len(self.path_indices), len(self.path_coefficients), len(lay),
+                *self.buffer_dim, *self.buffer_num_segments, *self.dtypes, *self.num_operands, *self.operations, *self.num_paths,
+                *self.path_indices_start, *self.path_coefficients_start, *self.path_indices, *lay]
+        a = base64.b64encode(zlib.compress(struct.pack(f"<{len(ints)}q", *ints), 6)).decode("ascii")
+        c = base64.b64encode(zlib.compress(struct.pack(f"<{len(self.path_coefficients)}d", *self.path_coefficients), 6)).decode("ascii")
+        return a + ":" + c
+
+    @classmethod
+    def unpack(cls, text: str) -> "U1dTables":
+        import base64
+        import zlib
+
+        a, c = text.split(":")
+        raw = zlib.decompress(base64.b64decode(a))
+        ints = list(struct.unpack(f"<{len(raw) // 8}q", raw))
+        extent, nin, nout, nops, noperations, nidx, ncoef, nlay = ints[:8]
+        pos = [8]
+
+        def take(n):
+            out = ints[pos[0]: pos[0] + n]
+            pos[0] += n
+            return out
+
+        nbuf = nin + nout
+        buffer_dim, nseg, dtypes = take(nbuf), take(nbuf), take(nbuf)
+        num_operands, operations, num_paths, pis, pcs = take(nops), take(noperations), take(nops), take(nops), take(nops)
+        path_indices, lay = take(nidx), take(nlay)
+        if pos[0] != len(ints):
+            raise ValueError("uniform_1d: packed tables of unexpected length")
+        raw = zlib.decompress(base64.b64decode(c))
+        coefficients = struct.unpack(f"<{ncoef}d", raw)
+        t = cls.make(extent, nin, nout, buffer_dim, nseg, dtypes, num_operands, operations, num_paths, pis, pcs, path_indices, coefficients)
+        if lay:
+            groups, k = {}, 0
+            for b in range(nbuf):
+                n = lay[k]
+                if n:
+                    groups[b] = lay[k + 1: k + 1 + n]
+                k += 1 + n
+            t = t.with_layouts(groups)
+        return t
+
     def content_hash(self, math_code: int) -> int:
         """FNV-1a 64 over the table contents; equals ``cueq::hash_u1d_desc`` of the C library."""
         words = [math_code, self.operand_extent, self.num_inputs, self.num_outputs, *self.buffer_dim,

@@ -41,6 +41,29 @@ def test_registration_and_schema():
     assert [p.value for p in ops_torch.TriMulPrecision] == [-1, 0, 1, 2, 3]
 
 
+def test_uniform_1d_plan_lookup_by_argument_values(monkeypatch):
+    """``uniform_1d`` finds its plan by the values of the lists it is given: equal lists (other objects) meet the same
+    plan, a changed coefficient or another arithmetic type meets another one."""
+    import importlib
+
+    u = importlib.import_module("cuequivariance_amd.cuet.uniform_1d")
+    seen = []
+    monkeypatch.setattr(u, "run_plan", lambda plan, *a, **k: seen.append(plan) or [])
+    t = U1dTables.from_polynomial(channelwise_poly().flatten_coefficient_modes().squeeze_modes())
+
+    def call(coefficients, math_dtype=torch.float32):
+        return u.uniform_1d(
+            "lookup", math_dtype, t.operand_extent, t.num_inputs, t.num_outputs, 0, list(t.buffer_dim), list(t.buffer_num_segments),
+            [0] * 4, [-1] * 4, list(t.dtypes), len(t.num_operands), list(t.num_operands), list(t.operations), list(t.num_paths),
+            list(t.path_indices_start), list(t.path_coefficients_start), list(t.path_indices), coefficients, 0, [])
+
+    c = list(t.path_coefficients)
+    call(c), call(list(c)), call([2.0 * c[0]] + c[1:]), call(c, torch.float64)
+    assert seen[0] is seen[1]
+    assert seen[2] is not seen[0] and seen[2].tables.path_coefficients[0] == 2.0 * c[0]
+    assert seen[3] is not seen[0] and seen[3].math_dtype == torch.float64
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_uniform_1d_through_torch_ops(device, dtype):
