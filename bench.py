@@ -236,6 +236,9 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         f = 2 * Z * 64 * 64 * 11
         flops = {"fwd": f, "bwd": 3 * f}
         flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
+        if dtype == torch.float32:
+            # the float32 kernels form the products g W^T once for both input gradients: three contractions are executed
+            fc_executed_flops = 3 * f
         desc = ("configs[3]: FullyConnectedTensorProduct 64x0e+64x1o (x) 0e+1o+2e -> 64x0e+64x1o, batch 50000, shared weights, "
                 "fwd + bwd (dw, dx1, dx2)")
         if wl == "cfg4fcmi":
@@ -367,6 +370,10 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
     more = dict(extra) if wl == "cfg5" else {}
     if more:  # the step against 8 TB/s on the bytes its own stages must move (the binding roof of the 2-byte step as decomposed)
         more["hbm_frac_of_decomposition_traffic"] = more["decomposition_traffic_bytes"] / elapsed / 1e9 / HBM_PEAK_GBS
+    if wl in ("cfg4fc", "cfg4fcmi") and dt == "f32":
+        # `flops` counts the four contractions of the step (forward, dx1, dx2, dw); the matrix instructions executed are fewer
+        more["executed_matrix_flops"] = fc_executed_flops
+        more["mfma_frac_executed"] = fc_executed_flops / elapsed / 1e12 / flop_peak
     achieved = ((alg["fwd"] + alg["bwd"]) / elapsed / 1e9) if roofs["bound"] == "hbm" else ((flops["fwd"] + flops["bwd"]) / elapsed / 1e12)
     return {
         "metric": f"{unit.split('/')[0]}/sec, {wl} fwd+bwd (secondary workload)", "value": units / elapsed, "unit": unit, "n_gpus": 1,
@@ -611,7 +618,8 @@ def _compact(line: dict) -> dict:
     r = line["roofline"]
     out = {"ms_per_step": line["ms_per_step"], "value": line["value"], "unit": line["unit"], "dtype": line["dtype"],
            "bound": r["bound"], "frac": r["frac"], "workload": line["config"]["workload"]}
-    for k in ("hbm_frac", "mfma_frac", "valu_frac", "decomposition_traffic_bytes", "hbm_frac_of_decomposition_traffic"):
+    for k in ("hbm_frac", "mfma_frac", "valu_frac", "decomposition_traffic_bytes", "hbm_frac_of_decomposition_traffic",
+              "executed_matrix_flops", "mfma_frac_executed"):
         if k in r:
             out[k] = r[k]
     return out

@@ -144,6 +144,114 @@ def _products(paths, transposed: bool):
     return prods
 
 
+def _emit_staging(A, T: str, blocks, lds_off, transposed: bool, threads: int):
+    """The weight blocks from memory into LDS (``lds_off[w_off] = (offset, rows, columns, row stride in bytes)``): every
+    thread requests all its 16-byte pieces before it writes the first one, so the block starts after one trip to memory
+    instead of one per weight block.  ``transposed``: element (k, n) of a block goes to row n, column k."""
+    es = 4 if T == "float" else 2
+    epv = 16 // es
+    plan, total = [], 0
+    for w_off, K, N in blocks:
+        nvec = K * N // epv
+        cnt = (nvec + threads - 1) // threads
+        plan.append((w_off, K, N, nvec, cnt, total))
+        total += cnt
+    A("  {")
+    A(f"    uint4 stg[{total}];")
+    for w_off, K, N, nvec, cnt, base in plan:
+        for i in range(cnt):
+            guard = "" if (i + 1) * threads <= nvec else f"(tid + {i * threads} >= {nvec}) ? make_uint4(0, 0, 0, 0) : "
+            A(f"    stg[{base + i}] = {guard}*reinterpret_cast<const uint4*>(W + {w_off} + (tid + {i * threads}) * {epv});")
+    for w_off, K, N, nvec, cnt, base in plan:
+        o, R, C, RS = lds_off[w_off]
+        for i in range(cnt):
+            guard = "" if (i + 1) * threads <= nvec else f"if (tid + {i * threads} < {nvec}) "
+            A(f"    {guard}{{ const int e = (tid + {i * threads}) * {epv}, k = e / {N}, n = e % {N};")
+            if not transposed:
+                A(f"      *reinterpret_cast<uint4*>(smem + {o} + k * {RS} + n * {es}) = stg[{base + i}]; }}")
+            elif es == 4:
+                A(f"      char* q = smem + {o} + n * {RS} + k * 4;")
+                A(f"      *reinterpret_cast<uint32_t*>(q) = stg[{base + i}].x; *reinterpret_cast<uint32_t*>(q + {RS}) = stg[{base + i}].y;")
+                A(f"      *reinterpret_cast<uint32_t*>(q + {2 * RS}) = stg[{base + i}].z; *reinterpret_cast<uint32_t*>(q + {3 * RS}) = stg[{base + i}].w; }}")
+            else:
+                A(f"      char* q = smem + {o} + n * {RS} + k * 2;")
+                for c, comp in enumerate("xyzw"):
+                    A(f"      *reinterpret_cast<uint16_t*>(q + {2 * c * RS}) = static_cast<uint16_t>(stg[{base + i}].{comp} & 0xffffu); "
+                      f"*reinterpret_cast<uint16_t*>(q + {(2 * c + 1) * RS}) = static_cast<uint16_t>(stg[{base + i}].{comp} >> 16);")
+                A("    }")
+    A("  }")
+
+
+def _operand_groups(A, prods, transposed: bool, in_blocks, es: int, single: bool = False):
+    """Declares the operand registers of a kernel and returns ``(groups, contraction, request, fragment)``: the products
+    grouped by the segment of the row operand ``IN`` they contract with, ``request(gi)`` emits the loads of group ``gi``
+    (into one of two register sets, so that a group can be requested while the previous one is worked on) and
+    ``fragment(gi, comp, s2, q)`` is the expression of one 16-byte MFMA operand.  ``single``: one register set only - a
+    group is requested when the last product of the previous one has read its operands."""
+    # products grouped by operand segment so that its fragments are loaded once
+    by_seg = OrderedDict()
+    for (w_off, K, N, in_off), uses in prods.items():
+        by_seg.setdefault(in_off, []).append((w_off, K, N, uses))
+    segs = list(by_seg.items())
+    if in_blocks:
+        segs.sort(key=lambda it: it[0])  # the segments of a block next to each other
+    contraction = {in_off: (pl[0][1] if transposed else pl[0][2]) for in_off, pl in segs}
+    for in_off, pl in segs:
+        assert all((p[1] if transposed else p[2]) == contraction[in_off] for p in pl), "one operand segment, one contraction length"
+    # Operand groups: a segment on its own, or the segments of one mul_ir block together - the lane's channels of such a
+    # block with all their components are one contiguous run of the row, loaded once and taken apart in registers.
+    groups = []
+    for in_off, pl in segs:
+        blk = _block_at(in_off, in_blocks)
+        if blk is not None and groups and groups[-1][0] is not None and groups[-1][0][:3] == blk[:3]:
+            groups[-1][1].append((in_off, pl, blk[3]))
+        else:
+            groups.append((blk, [(in_off, pl, blk[3] if blk else 0)]))
+    def nraw(g):  # 16-byte vectors a lane holds for the group
+        blk, members = g
+        C = contraction[members[0][0]]
+        return (C * es // 64) * 2 * (blk[2] if blk else 1)
+    if single:
+        A(f"    uint4 rawa[{max(nraw(g) for g in groups)}];")
+    else:
+        A(f"    uint4 rawa[{max(nraw(g) for g in groups[0::2])}], rawb[{max([nraw(g) for g in groups[1::2]] or [1])}];")
+
+    def request(gi):
+        blk, members = groups[gi]
+        C = contraction[members[0][0]]
+        name = "rawa" if (gi % 2 == 0 or single) else "rawb"
+        if blk is None:
+            in_off = members[0][0]
+            for s2 in range(C * es // 64):
+                for q in range(2):
+                    A(f"    {name}[{2 * s2 + q}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {in_off}) + {s2 * 64} + h * 32 + {q * 16});")
+        else:
+            s0, mul, d, _ = blk
+            for s2 in range(C * es // 64):
+                for m in range(2 * d):
+                    A(f"    {name}[{2 * d * s2 + m}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {s0}) + ({s2 * 64} + h * 32) * {d} + {16 * m});")
+
+    def fragment(gi, comp, s2, q):
+        """Expression of the MFMA operand (s2, q) of component ``comp`` of group ``gi``: 16 bytes of consecutive channels."""
+        blk, members = groups[gi]
+        name = "rawa" if (gi % 2 == 0 or single) else "rawb"
+        if blk is None:
+            return f"{name}[{2 * s2 + q}]"
+        d = blk[2]
+        word = lambda e: f"{name}[{2 * d * s2 + (e // (4 if es == 4 else 8))}].{'xyzw'[(e // (1 if es == 4 else 2)) % 4]}"
+        if es == 4:  # elements (4 q + e) * d + comp of the run, e < 4
+            return "make_uint4(" + ", ".join(word((4 * q + e) * d + comp) for e in range(4)) + ")"
+        parts = []
+        for j in range(4):  # dword j: elements (8 q + 2 j) * d + comp (low half) and the next channel's (high half)
+            e0 = (8 * q + 2 * j) * d + comp
+            e1 = e0 + d
+            sel = (0x0302 if e0 & 1 else 0x0100) | ((0x0706 if e1 & 1 else 0x0504) << 16)
+            parts.append(f"__builtin_amdgcn_perm({word(e1)}, {word(e0)}, 0x{sel:08x}u)")
+        return "make_uint4(" + ", ".join(parts) + ")"
+
+    return groups, contraction, request, fragment
+
+
 def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, width_res: int, n2: int, in_blocks=None, res_blocks=None):
     """One kernel.  ``transposed``: the blocks sit in LDS as W^T (rows n, contraction k).  ``rowdot``: instead of
     accumulating the scaled products into result columns, they are multiplied element-wise with G and summed per row.
@@ -167,14 +275,7 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
     A(f"__global__ void __launch_bounds__(64 * kWaves, 1) {name}_kernel({args}) {{")
     A("  extern __shared__ __align__(16) char smem[];")
     A("  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;")
-    for w_off, K, N in blocks:
-        o, R, C, RS = lds_off[w_off]
-        if transposed:  # global block is K x N (k major): element (k, n) goes to row n, column k
-            A(f"  for (int e = tid; e < {K * N}; e += 64 * kWaves) {{ const int k = e / {N}, n = e % {N}; "
-              f"*reinterpret_cast<{T}*>(smem + {o} + n * {RS} + k * {es}) = W[{w_off} + e]; }}")
-        else:
-            A(f"  for (int e = tid; e < {K * N}; e += 64 * kWaves) {{ const int k = e / {N}, n = e % {N}; "
-              f"*reinterpret_cast<{T}*>(smem + {o} + k * {RS} + n * {es}) = W[{w_off} + e]; }}")
+    _emit_staging(A, T, blocks, lds_off, transposed, 64 * 8)
     A("  __syncthreads();")
     A("  const int ntiles = (Z + 31) / 32;")
     A("  // tile t goes to block t mod grid, wavefront (t / grid) mod 8: a short batch spreads over every CU first")
@@ -218,64 +319,7 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
     else:
         for t in range(ntiles):
             A(f"    floatx16 o{t} = floatx16{{0}};")
-    # products grouped by operand segment so that its fragments are loaded once
-    by_seg = OrderedDict()
-    for (w_off, K, N, in_off), uses in prods.items():
-        by_seg.setdefault(in_off, []).append((w_off, K, N, uses))
-    segs = list(by_seg.items())
-    if in_blocks:
-        segs.sort(key=lambda it: it[0])  # the segments of a block next to each other
-    contraction = {in_off: (pl[0][1] if transposed else pl[0][2]) for in_off, pl in segs}
-    for in_off, pl in segs:
-        assert all((p[1] if transposed else p[2]) == contraction[in_off] for p in pl), "one operand segment, one contraction length"
-    # Operand groups: a segment on its own, or the segments of one mul_ir block together - the lane's channels of such a
-    # block with all their components are one contiguous run of the row, loaded once and taken apart in registers.
-    groups = []
-    for in_off, pl in segs:
-        blk = _block_at(in_off, in_blocks)
-        if blk is not None and groups and groups[-1][0] is not None and groups[-1][0][:3] == blk[:3]:
-            groups[-1][1].append((in_off, pl, blk[3]))
-        else:
-            groups.append((blk, [(in_off, pl, blk[3] if blk else 0)]))
-    def nraw(g):  # 16-byte vectors a lane holds for the group
-        blk, members = g
-        C = contraction[members[0][0]]
-        return (C * es // 64) * 2 * (blk[2] if blk else 1)
-    A(f"    uint4 rawa[{max(nraw(g) for g in groups[0::2])}], rawb[{max([nraw(g) for g in groups[1::2]] or [1])}];")
-
-    def request(gi):
-        blk, members = groups[gi]
-        C = contraction[members[0][0]]
-        name = "rawa" if gi % 2 == 0 else "rawb"
-        if blk is None:
-            in_off = members[0][0]
-            for s2 in range(C * es // 64):
-                for q in range(2):
-                    A(f"    {name}[{2 * s2 + q}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {in_off}) + {s2 * 64} + h * 32 + {q * 16});")
-        else:
-            s0, mul, d, _ = blk
-            for s2 in range(C * es // 64):
-                for m in range(2 * d):
-                    A(f"    {name}[{2 * d * s2 + m}] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(IN + z * ldi + {s0}) + ({s2 * 64} + h * 32) * {d} + {16 * m});")
-
-    def fragment(gi, comp, s2, q):
-        """Expression of the MFMA operand (s2, q) of component ``comp`` of group ``gi``: 16 bytes of consecutive channels."""
-        blk, members = groups[gi]
-        name = "rawa" if gi % 2 == 0 else "rawb"
-        if blk is None:
-            return f"{name}[{2 * s2 + q}]"
-        d = blk[2]
-        word = lambda e: f"{name}[{2 * d * s2 + (e // (4 if es == 4 else 8))}].{'xyzw'[(e // (1 if es == 4 else 2)) % 4]}"
-        if es == 4:  # elements (4 q + e) * d + comp of the run, e < 4
-            return "make_uint4(" + ", ".join(word((4 * q + e) * d + comp) for e in range(4)) + ")"
-        parts = []
-        for j in range(4):  # dword j: elements (8 q + 2 j) * d + comp (low half) and the next channel's (high half)
-            e0 = (8 * q + 2 * j) * d + comp
-            e1 = e0 + d
-            sel = (0x0302 if e0 & 1 else 0x0100) | ((0x0706 if e1 & 1 else 0x0504) << 16)
-            parts.append(f"__builtin_amdgcn_perm({word(e1)}, {word(e0)}, 0x{sel:08x}u)")
-        return "make_uint4(" + ", ".join(parts) + ")"
-
+    groups, contraction, request, fragment = _operand_groups(A, prods, transposed, in_blocks, es)
     request(0)
     for gi, (blk, members) in enumerate(groups):
         # the operands of the next group are requested before the products of the current one are worked on
@@ -346,6 +390,170 @@ def _emit_kernel(A, name: str, T: str, paths, transposed: bool, rowdot: bool, wi
                       + ", ".join(val(a, 4 * m4 + e) for e in range(4)) + ");")
         A("    }")
     A("  }")
+    A("}")
+    A("")
+
+
+def dx12_supported(paths, width_in: int) -> bool:
+    """The kernel that forms both input gradients splits the rows of every product between two wavefronts: multiplicities
+    of the first operand multiples of 64, its segments covering the row exactly."""
+    segs = {}
+    for p in paths:
+        if p.K % 64 or segs.setdefault(p.a_off, p.K) != p.K:
+            return False
+    pos = 0
+    for a_off in sorted(segs):
+        if a_off != pos:
+            return False
+        pos += segs[a_off]
+    return pos == width_in
+
+
+def _emit_dx12_kernel(A, T: str, paths, width_in: int, n2: int, g_blocks=None, x_blocks=None):
+    """Both input gradients from one pass over the products ``R = W_b g_seg^T`` (result rows k = channels of the first
+    operand, one batch row per lane): ``dx1[z, a_off + k] += c x2[z, j] R[k, z]`` and ``dx2[z, j] += c sum_k x1[z, a_off + k]
+    R[k, z]`` - a quarter of the step's matrix products less than the two separate kernels.  The accumulators of dx1 and the
+    row of x1 would not fit one wavefront's registers side by side, so a unit of work is (32-row tile, half of the channels
+    of every segment): 64 + 64 registers, two wavefronts per SIMD as in the other kernels, and twice as many units to deal
+    out.  The two halves of a row's dx2 go to ``PART[z][half][j]`` (float) and are added by ``dx12_fold_kernel``: no
+    atomics, the same bits every run.  ``g_blocks`` / ``x_blocks``: blocks of g / of x1 and dx1 in ``mul_ir`` order."""
+    es = 4 if T == "float" else 2
+    g_blocks, x_blocks = _mul_ir_blocks(g_blocks), _mul_ir_blocks(x_blocks)
+    blocks = sorted({(p.w_off, p.K, p.N) for p in paths})
+    lds_off, off = {}, 0
+    for w_off, K, N in blocks:
+        lds_off[w_off] = (off, K, N, N * es + 16)
+        off += K * (N * es + 16)
+    prods = _products(paths, False)
+    js = sorted({u[0] for us in prods.values() for u in us})
+    seg_len = {p.a_off: p.K for p in paths}
+    A(f"// dx12: {len(prods)} products, {sum(len(u) for u in prods.values())} uses (each twice), {off} bytes of weights in LDS")
+    A(f"constexpr int kdx12Lds = {off};")
+    A(f"__global__ void __launch_bounds__(64 * kWaves, 1) dx12_kernel(const {T}* __restrict__ W, const {T}* __restrict__ IN, int64_t ldi, "
+      f"const {T}* __restrict__ S, int64_t lds_, const {T}* __restrict__ X, int64_t ldx, {T}* __restrict__ OUT, int64_t ldo, "
+      f"float* __restrict__ PART, int Z) {{")
+    A("  extern __shared__ __align__(16) char smem[];")
+    A("  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;")
+    _emit_staging(A, T, blocks, lds_off, False, 64 * 8)
+    A("  __syncthreads();")
+    A("  const int nunits = 2 * ((Z + 31) / 32);")
+    A("  // unit u = (tile u / 2, channel half u mod 2) goes to block u mod grid, slot (u / grid) mod 8; the slots are dealt to the")
+    A("  // wavefronts in the order 0 3 5 6 1 2 4 7, so that a round that fills only the first four slots puts one unit on every")
+    A("  // SIMD whether the hardware places wavefront w on SIMD w mod 4 or on SIMD w / 2")
+    A("  const int slot = (0x73261540u >> (4 * wave)) & 7;  // wave 0 1 2 3 4 5 6 7 -> slot 0 4 5 1 6 2 3 7")
+    A("  for (int unit = blockIdx.x + gridDim.x * slot; unit < nunits; unit += gridDim.x * kWaves) {")
+    A("    const int hlf = unit & 1;")
+    A("    const int zrow = (unit >> 1) * 32 + c;")
+    A("    const int64_t z = zrow < Z ? zrow : Z - 1;  // (lanes past the end repeat the last row)")
+    for j in js:
+        A(f"    const float s{j} = to_f(S[z * lds_ + {j}]);")
+        A(f"    float d{j} = 0.f;")
+    # this unit's channels of segment a_off: tiles tl < K / 64 at channel 32 * (hlf * K / 64 + tl); a lane holds 16 of the 32
+    # (8 a + 4 h + r), as accumulator o_<a_off>_<tl> and as the row of x1 x_<a_off>_<tl>
+    for a_off, K in sorted(seg_len.items()):
+        for tl in range(K // 64):
+            A(f"    floatx16 o_{a_off}_{tl} = floatx16{{0}};")
+            A(f"    float x_{a_off}_{tl}[16];")
+    done = set()
+    for a_off, K in sorted(seg_len.items()):
+        KH = K // 64
+        blk = _block_at(a_off, x_blocks)
+        for tl in range(KH):
+            if blk is None:
+                A("#pragma unroll")
+                A(f"    for (int a = 0; a < 4; ++a) {{ float v4[4]; load4(X + z * ldx + {a_off} + 32 * (hlf * {KH} + {tl}) + 4 * h + 8 * a, v4); "
+                  f"x_{a_off}_{tl}[4 * a] = v4[0]; x_{a_off}_{tl}[4 * a + 1] = v4[1]; x_{a_off}_{tl}[4 * a + 2] = v4[2]; x_{a_off}_{tl}[4 * a + 3] = v4[3]; }}")
+                continue
+            # mul_ir block: the lane's channels 8 a + 4 h + r of a tile with all d components are 4 d consecutive elements
+            s0, mul, d, _ = blk
+            if (s0, tl) in done:
+                continue
+            done.add((s0, tl))
+            for a in range(4):
+                A(f"    {{ float gv[{4 * d}];")
+                for m in range(d):
+                    A(f"      {{ float q4[4]; load4(X + z * ldx + {s0} + (32 * (hlf * {KH} + {tl}) + {8 * a} + 4 * h) * {d} + {4 * m}, q4); "
+                      f"gv[{4 * m}] = q4[0]; gv[{4 * m + 1}] = q4[1]; gv[{4 * m + 2}] = q4[2]; gv[{4 * m + 3}] = q4[3]; }}")
+                for kc in range(d):
+                    for r in range(4):
+                        A(f"      x_{s0 + kc * mul}_{tl}[{4 * a + r}] = gv[{r * d + kc}];")
+                A("    }")
+    # one set of operand registers (two do not fit beside the accumulators and the row of x1, and made no difference when
+    # timed): the next group is requested as soon as the last product of the current one has issued its matrix
+    # instructions, ahead of that product's uses
+    groups, contraction, request, fragment = _operand_groups(A, prods, False, g_blocks, es, single=True)
+    request(0)
+    for gi, (blk, members) in enumerate(groups):
+        for mi, (in_off, plist, comp) in enumerate(members):
+            ns = contraction[in_off] * es // 64
+            A("    {")
+            for s2 in range(ns):
+                for q in range(2):
+                    A(f"      const uint4 xf_{s2}_{q} = {fragment(gi, comp, s2, q)};")
+            for pi, (w_off, K, N, uses) in enumerate(plist):
+                o, R, Cc, RS = lds_off[w_off]
+                KH = K // 64
+                for tl in range(KH):
+                    A("      {")
+                    A("        floatx16 T = floatx16{0};")
+                    A(f"        const char* wr = smem + {o} + (32 * (hlf * {KH} + {tl}) + c) * {RS} + h * 32;")
+                    for s2 in range(ns):
+                        for q in range(2):
+                            A(f"        mma_step<{T}>(T, *reinterpret_cast<const uint4*>(wr + {s2 * 64 + q * 16}), xf_{s2}_{q});")
+                    if gi + 1 < len(groups) and mi == len(members) - 1 and pi == len(plist) - 1 and tl == KH - 1:
+                        A("        __builtin_amdgcn_sched_barrier(0);")
+                        request(gi + 1)
+                    for j, coeff, a_off in uses:
+                        A(f"        {{ const float sc = {coeff!r}f * s{j};")
+                        A("#pragma unroll")
+                        A(f"          for (int v = 0; v < 16; ++v) o_{a_off}_{tl}[v] = fmaf(sc, T[v], o_{a_off}_{tl}[v]);")
+                        A("          float p = 0.f;")
+                        A("#pragma unroll")
+                        A(f"          for (int v = 0; v < 16; ++v) p = fmaf(T[v], x_{a_off}_{tl}[v], p);")
+                        A(f"          d{j} = fmaf({coeff!r}f, p, d{j});")
+                        A(f'          asm volatile("" : "+v"(d{j}));  // finish this use here: a product\'s result is not kept for later')
+                        A("        }")
+                    A("      }")
+                    A("      __builtin_amdgcn_sched_barrier(0);  // keep the loads of later products from piling up ahead of this one")
+            A("    }")
+    # rows past the end were clamped to the last row: those lanes hold its values and store them again (the same bits to
+    # the same place), see the other kernels
+    A("    {")
+    for j in range(n2):
+        if j in js:
+            A(f"      {{ const float tot = d{j} + __shfl_xor(d{j}, 32, 64); if (h == 0) PART[(z * 2 + hlf) * {n2} + {j}] = tot; }}")
+        else:
+            A(f"      if (h == 0) PART[(z * 2 + hlf) * {n2} + {j}] = 0.f;")
+    done = set()
+    for a_off, K in sorted(seg_len.items()):
+        KH = K // 64
+        blk = _block_at(a_off, x_blocks)
+        for tl in range(KH):
+            if blk is None:
+                A("#pragma unroll")
+                A(f"      for (int a = 0; a < 4; ++a) store4(OUT + z * ldo + {a_off} + 32 * (hlf * {KH} + {tl}) + 4 * h + 8 * a, "
+                  f"o_{a_off}_{tl}[4 * a], o_{a_off}_{tl}[4 * a + 1], o_{a_off}_{tl}[4 * a + 2], o_{a_off}_{tl}[4 * a + 3]);")
+                continue
+            s0, mul, d, _ = blk
+            if (s0, tl) in done:
+                continue
+            done.add((s0, tl))
+            val = lambda a, m: f"o_{s0 + (m % d) * mul}_{tl}[{4 * a + m // d}]"
+            for a in range(4):
+                for m4 in range(d):
+                    A(f"      store4(OUT + z * ldo + {s0} + (32 * (hlf * {KH} + {tl}) + {8 * a} + 4 * h) * {d} + {4 * m4}, "
+                      + ", ".join(val(a, 4 * m4 + e) for e in range(4)) + ");")
+    A("    }")
+    A("  }")
+    A("}")
+    A("")
+    A("// dx2[z][j] = PART[z][0][j] + PART[z][1][j]")
+    A(f"__global__ void __launch_bounds__(256) dx12_fold_kernel(const float* __restrict__ PART, {T}* __restrict__ OUT2, int64_t ldo2, int Z) {{")
+    A(f"  const int64_t e = blockIdx.x * 256ll + threadIdx.x;")
+    A(f"  if (e >= int64_t(Z) * {n2}) return;")
+    A(f"  const int64_t z = e / {n2};")
+    A(f"  const int j = static_cast<int>(e % {n2});")
+    A(f"  store1(OUT2 + z * ldo2 + j, PART[(z * 2) * {n2} + j] + PART[(z * 2 + 1) * {n2} + j]);")
     A("}")
     A("")
 
@@ -562,6 +770,11 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=N
     _emit_kernel(A, "fwd", T, paths, True, False, width_out, n2, in_blocks, out_blocks)
     _emit_kernel(A, "dx1", T, paths, False, False, width_in, n2, out_blocks, in_blocks)
     _emit_kernel(A, "dx2", T, paths, True, True, width_out, n2, in_blocks, out_blocks)
+    # (2-byte types keep the two separate kernels: they are bound by memory latency, not by the matrix cores, and ran
+    # 39 + 5 us against 22 + 18 us with the one-pass kernel on the 64-channel benchmark product)
+    has_dx12 = T == "float" and dx12_supported(paths, width_in)
+    if has_dx12:
+        _emit_dx12_kernel(A, T, paths, width_in, n2, out_blocks, in_blocks)
     _emit_dw_kernel(A, T, paths, n2, width_in, width_out, in_blocks, out_blocks)
     A("// compute units of the current device (asked once per device: the query is slow)")
     A("int grid_for(int64_t Z) {")
@@ -585,7 +798,7 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=N
     A("  __atomic_store_n(&done[dev], 1, __ATOMIC_RELEASE);")
     A("  return 0;")
     A("}")
-    A("int done_fwd[64], done_dx1[64], done_dx2[64], done_dw[64];")
+    A("int done_fwd[64], done_dx1[64], done_dx2[64], done_dx12[64], done_dw[64];")
     A("}  // namespace")
     A("")
     A(f'extern "C" int fcj_fwd(int64_t Z, const void* W, const void* X, int64_t ldx, const void* S, int64_t lds_, void* OUT, int64_t ldo, void* stream) {{')
@@ -608,6 +821,23 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=N
     A(f"  hipLaunchKernelGGL(dx2_kernel, dim3(grid_for(Z)), dim3(64 * kWaves), kdx2Lds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(W), "
       f"static_cast<const {T}*>(X), ldx, static_cast<const {T}*>(S), lds_, static_cast<const {T}*>(G), ldg, static_cast<{T}*>(DX2), ld2, static_cast<int>(Z));")
     A("  return hipGetLastError() == hipSuccess ? 0 : -1;")
+    A("}")
+    A("// both input gradients in one pass; PART: 2 * n2 floats per row of scratch.  -2: this product has no such kernel")
+    A(f'extern "C" int fcj_dx12(int64_t Z, const void* W, const void* G, int64_t ldg, const void* S, int64_t lds_, const void* X, int64_t ldx, '
+      f'void* DX1, int64_t ldd, void* DX2, int64_t ld2, float* PART, void* stream) {{')
+    if has_dx12:
+        A("  if (Z <= 0) return 0;")
+        A("  if (prepare(dx12_kernel, kdx12Lds, done_dx12)) return -1;")
+        A("  const int64_t units = 2 * ((Z + 31) / 32);")
+        A("  const int cus = grid_for(int64_t(1) << 40);")
+        A(f"  hipLaunchKernelGGL(dx12_kernel, dim3(static_cast<unsigned>(units < cus ? units : cus)), dim3(64 * kWaves), kdx12Lds, static_cast<hipStream_t>(stream), "
+          f"static_cast<const {T}*>(W), static_cast<const {T}*>(G), ldg, static_cast<const {T}*>(S), lds_, static_cast<const {T}*>(X), ldx, "
+          f"static_cast<{T}*>(DX1), ldd, PART, static_cast<int>(Z));")
+        A(f"  hipLaunchKernelGGL(dx12_fold_kernel, dim3(static_cast<unsigned>((Z * {n2} + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream), "
+          f"PART, static_cast<{T}*>(DX2), ld2, static_cast<int>(Z));")
+        A("  return hipGetLastError() == hipSuccess ? 0 : -1;")
+    else:
+        A("  return -2;")
     A("}")
     A("// number of per-block partial sums fcj_dw writes for a batch of Z rows (the caller sizes PART with it)")
     A('extern "C" int fcj_dw_blocks(int64_t Z) {')

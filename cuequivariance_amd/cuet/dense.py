@@ -832,7 +832,16 @@ class _FcFunction(torch.autograd.Function):
                 gx1 = (torch.empty_like if mod.dx1_covers_input or unit is not None else torch.zeros_like)(x1d)
             if need_x2:
                 gx2 = (torch.empty_like if unit is not None else torch.zeros_like)(x2d)
-            if unit is not None:
+            both = -2
+            if unit is not None and need_x1 and need_x2:  # one pass over the products g W^T serves both (-2: not for this product)
+                part = torch.empty(Z, 2 * x2d.shape[1], dtype=torch.float32, device=dev)
+                both = unit.fcj_dx12(Z, wd.data_ptr(), g.data_ptr(), g.stride(0), x2d.data_ptr(), x2d.stride(0), x1d.data_ptr(), x1d.stride(0),
+                                     gx1.data_ptr(), gx1.stride(0), gx2.data_ptr(), gx2.stride(0), part.data_ptr(), stream)
+                if both not in (0, -2):
+                    raise RuntimeError("fused fully connected gradients (both operands): launch failed")
+            if both == 0:
+                pass
+            elif unit is not None:
                 if need_x1 and unit.fcj_dx1(Z, wd.data_ptr(), g.data_ptr(), g.stride(0), x2d.data_ptr(), x2d.stride(0), gx1.data_ptr(),
                                             gx1.stride(0), stream) != 0:
                     raise RuntimeError("fused fully connected gradient (first operand): launch failed")

@@ -337,7 +337,7 @@ def prebuild_fully_connected(force: bool = False) -> list:
 def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=None, out_blocks=None):
     """The fused kernels of ``codegen/fullyconnected.py`` for one fully connected product and element type (``float`` or
     ``uint16_t`` for bfloat16), compiled at first use and loaded: a ``ctypes`` handle with ``fcj_fwd``, ``fcj_dx1``,
-    ``fcj_dx2`` and ``fcj_dw``, or ``None`` when this module is off, the product is outside what the generator covers, or the compiler
+    ``fcj_dx2``, ``fcj_dx12`` (both input gradients in one pass; returns -2 for products it does not cover) and ``fcj_dw``, or ``None`` when this module is off, the product is outside what the generator covers, or the compiler
     failed (the caller then runs the table-driven GEMMs)."""
     from .codegen import fullyconnected as fc
 
@@ -361,9 +361,10 @@ def fully_connected_unit(paths, n2: int, width_in: int, width_out: int, T: str, 
             h.fcj_fwd.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp]
             h.fcj_dx1.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp]
             h.fcj_dx2.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp]
+            h.fcj_dx12.argtypes = [i64, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp]
             h.fcj_dw_blocks.argtypes = [i64]
             h.fcj_dw.argtypes = [i64, vp, i64, vp, i64, vp, i64, vp, i64, vp]
-            for f in (h.fcj_fwd, h.fcj_dx1, h.fcj_dx2, h.fcj_dw_blocks, h.fcj_dw):
+            for f in (h.fcj_fwd, h.fcj_dx1, h.fcj_dx2, h.fcj_dx12, h.fcj_dw_blocks, h.fcj_dw):
                 f.restype = C.c_int
             _loaded[key] = h
             return h

@@ -39,6 +39,12 @@ int fcj_dx1(int64_t Z, const void* W, const void* g, int64_t ld_g, const void* x
 int fcj_dx2(int64_t Z, const void* W, const void* x1, int64_t ld_x1, const void* x2, int64_t ld_x2, const void* g, int64_t ld_g,
             void* dx2, int64_t ld_dx2, void* stream);
 
+/* dx1 and dx2 from one pass over their common products g W^T (float objects whose multiplicities are multiples of 64;
+ * every other object returns -2 and the caller uses fcj_dx1 and fcj_dx2).  part: 2 * (columns of x2) floats per row of
+ * scratch that the caller provides; the two halves of every dx2 row are added in a fixed order (no atomics). */
+int fcj_dx12(int64_t Z, const void* W, const void* g, int64_t ld_g, const void* x2, int64_t ld_x2, const void* x1, int64_t ld_x1,
+             void* dx1, int64_t ld_dx1, void* dx2, int64_t ld_dx2, float* part, void* stream);
+
 /* Weight gradient as per-block partial sums: fcj_dw writes part[b, 0 .. numel) (float, numel = number of weights) for
  * b < fcj_dw_blocks(Z); the caller provides part and sums its rows (cueq_sum_rows).  Weights no path touches are not
  * written: clear part first when the paths do not cover W. */

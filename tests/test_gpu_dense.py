@@ -135,6 +135,43 @@ def test_fully_connected_benchmark_size(device, dtype, layout):
         assert abs((grad.double() * operand.detach().double()).sum().item() - lhs) <= slack, (grad.shape, lhs, slack)
 
 
+@pytest.mark.parametrize("layout", [cue.ir_mul, cue.mul_ir])
+def test_fully_connected_input_gradients_in_one_pass_and_apart(device, layout, jit_on):
+    """Asked for together, the two input gradients of a float32 product come from one kernel that forms the products g W^T
+    once (two wavefronts share the channels of a 32-row tile; the halves of dx2 are added in a fixed order); asked for one
+    at a time, each comes from its own kernel (the generated kernels of this product are built with the library; the suite
+    runs with them switched off unless asked, hence ``jit_on``).  Both ways against each other (different summation orders: 1e-5), the
+    one-pass way twice (the same bits), on a batch that ends inside a tile."""
+    from cuequivariance_amd import cuet
+
+    m = cuet.FullyConnectedTensorProduct(
+        cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "0e+1o+2e"), cue.Irreps("O3", "64x0e+64x1o"),
+        layout=layout, internal_weights=False,
+    )
+    Z = 4_133
+    g = torch.Generator().manual_seed(17)
+    w = (0.2 * torch.randn(1, m.weight_numel, generator=g)).to(device)
+    x1 = torch.randn(Z, 256, generator=g).to(device).requires_grad_(True)
+    x2 = torch.randn(Z, 9, generator=g).to(device).requires_grad_(True)
+    cot = torch.randn(Z, 256, generator=g).to(device)
+    both = torch.autograd.grad(m(x1, x2, w), [x1, x2], cot)
+    again = torch.autograd.grad(m(x1, x2, w), [x1, x2], cot)
+    only1 = torch.autograd.grad(m(x1, x2, w), [x1], cot)[0]
+    only2 = torch.autograd.grad(m(x1, x2, w), [x2], cot)[0]
+    assert torch.equal(both[0], again[0]) and torch.equal(both[1], again[1])
+    assert rel_err(both[0], only1) <= 1e-5 and rel_err(both[1], only2) <= 1e-5
+    dense = next(x for x in m.modules() if type(x).__name__ == "SegmentedPolynomialDense" and x.rows_mul_ir == (layout == cue.mul_ir))
+    unit = dense.fused_unit(torch.float32, x1.detach(), cot)
+    assert unit is not None, "the generated kernels of the benchmark product are built with the library"
+    part = torch.empty(1, 18, device=device)
+    out1, out2 = torch.empty(1, 256, device=device), torch.empty(1, 9, device=device)
+    status = unit.fcj_dx12(1, w.data_ptr(), cot.data_ptr(), 256, x2.data_ptr(), 9, x1.data_ptr(), 256, out1.data_ptr(), 256,
+                           out2.data_ptr(), 9, part.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert status == 0, "the one-pass kernel serves this product (multiplicities of 64)"
+    assert rel_err(out1, both[0][:1]) <= 1e-5 and rel_err(out2, both[1][:1]) <= 1e-5
+
+
 def _starts(irreps):
     out, off = [], 0
     for mul, ir in irreps:

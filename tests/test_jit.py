@@ -193,15 +193,21 @@ def test_fully_connected_generator_limits():
     d = dense("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o")
     assert fc.supported(d.paths, 9, 256, 256, 4) and fc.supported(d.paths, 9, 256, 256, 2)
     src = fc.emit_unit(d.paths, 9, 256, 256, "float")
-    for name in ("fwd_kernel", "dx1_kernel", "dx2_kernel", "dw_kernel"):
+    for name in ("fwd_kernel", "dx1_kernel", "dx2_kernel", "dx12_kernel", "dw_kernel"):
         assert name in src
+    # both input gradients in one pass: float objects with multiplicities that are multiples of 64 only
+    assert fc.dx12_supported(d.paths, 256)
+    assert "dx12_kernel" not in fc.emit_unit(d.paths, 9, 256, 256, "uint16_t")
+    mixed = dense("32x0e+64x1o", "0e+1o", "96x0e+32x1o")
+    assert not fc.dx12_supported(mixed.paths, mixed.input_sizes[1])
+    assert "return -2;" in fc.emit_unit(mixed.paths, mixed.input_sizes[2], mixed.input_sizes[1], mixed.out_size, "float")
     # every entry point the header of the generated objects declares is defined, with the declared number of arguments
     import pathlib
     import re
 
     header = (pathlib.Path(__file__).resolve().parent.parent / "include" / "cueq_amd_generated.h").read_text()
     declared = re.findall(r"^int (fcj_\w+)\(([^;]*)\);", header, flags=re.M | re.S)
-    assert {n for n, _ in declared} == {"fcj_fwd", "fcj_dx1", "fcj_dx2", "fcj_dw_blocks", "fcj_dw"}
+    assert {n for n, _ in declared} == {"fcj_fwd", "fcj_dx1", "fcj_dx2", "fcj_dx12", "fcj_dw_blocks", "fcj_dw"}
     for name, args in declared:
         m = re.search(r'extern "C" int %s\(([^)]*)\)' % name, src)
         assert m, name
