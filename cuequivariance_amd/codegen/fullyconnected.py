@@ -437,11 +437,8 @@ def _emit_dx12_kernel(A, T: str, paths, width_in: int, n2: int, g_blocks=None, x
     _emit_staging(A, T, blocks, lds_off, False, 64 * 8)
     A("  __syncthreads();")
     A("  const int nunits = 2 * ((Z + 31) / 32);")
-    A("  // unit u = (tile u / 2, channel half u mod 2) goes to block u mod grid, slot (u / grid) mod 8; the slots are dealt to the")
-    A("  // wavefronts in the order 0 3 5 6 1 2 4 7, so that a round that fills only the first four slots puts one unit on every")
-    A("  // SIMD whether the hardware places wavefront w on SIMD w mod 4 or on SIMD w / 2")
-    A("  const int slot = (0x73261540u >> (4 * wave)) & 7;  // wave 0 1 2 3 4 5 6 7 -> slot 0 4 5 1 6 2 3 7")
-    A("  for (int unit = blockIdx.x + gridDim.x * slot; unit < nunits; unit += gridDim.x * kWaves) {")
+    A("  // unit u = (tile u / 2, channel half u mod 2) goes to block u mod grid, wavefront (u / grid) mod 8")
+    A("  for (int unit = blockIdx.x + gridDim.x * wave; unit < nunits; unit += gridDim.x * kWaves) {")
     A("    const int hlf = unit & 1;")
     A("    const int zrow = (unit >> 1) * 32 + c;")
     A("    const int64_t z = zrow < Z ? zrow : Z - 1;  // (lanes past the end repeat the last row)")
