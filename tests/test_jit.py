@@ -224,6 +224,7 @@ def test_fully_connected_generator_limits():
     ("64x0e+64x1o", "0e+1o+2e", "64x0e+64x1o", 777),   # ragged: the last 32-row tile holds 9 rows
     ("32x0e+64x1o", "0e+1o", "96x0e+32x1o", 2500),     # mixed block shapes, a wavefront walks more than one tile on few CUs
     ("32x0e", "0e+1o", "32x1o", 1),
+    ("128x0e+64x0e", "0e+1o", "64x0e+64x1o", 333),     # a segment of 128 channels: two tiles per half in the one-pass input gradients
 ])
 def test_fused_fully_connected_matches_oracle_and_tables(device, dtype, i1, i2, i3, Z, jit_on):
     """The generated fully connected kernels (weights resident in LDS, products scaled in registers) against the CPU
