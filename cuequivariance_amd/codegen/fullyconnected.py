@@ -555,7 +555,7 @@ def _emit_dx12_kernel(A, T: str, paths, width_in: int, n2: int, g_blocks=None, x
     A("")
 
 
-DW_ROWS = 16  # batch rows per staged tile of the weight-gradient kernel
+DW_ROWS = 16  # batch rows per staged tile of the weight-gradient kernel (8 and 32 measured 2 - 3 us slower in float)
 
 
 def _emit_colmap(A, name: str, blocks):
