@@ -106,8 +106,10 @@ __device__ __forceinline__ void dw_body(const TI* __restrict__ A, int64_t lda, c
   // (a vector past the row piece - extents below 128 only - repeats the lane's last one that exists)
   const int xlim = VRX - 1 - line0 * 8 - l8 >= 0 ? ((VRX - 1 - line0 * 8 - l8) / (8 * (32 / ZR))) * (32 / ZR) * EPL : 0;
   const int glim = VRG - 1 - line0 * 8 - l8 >= 0 ? ((VRG - 1 - line0 * 8 - l8) / (8 * (32 / ZR))) * (32 / ZR) * EPL : 0;
-  const TI* xp = A + E0;
-  const TI* gp = G + E0;
+  // (a lane whose first vector lies past the row piece - pieces shorter than 128 elements - requests the piece's first
+  // vector instead: nothing is read outside the piece, which for the last row of a tensor would be outside the tensor)
+  const TI* xp = A + (line0 * 8 + l8 < VRX ? E0 : 0);
+  const TI* gp = G + (line0 * 8 + l8 < VRG ? E0 : 0);
   auto load_step = [&](uint4 (&qx)[D], uint4 (&qg)[D], bool& ok, int64_t z) {
     ok = z + row < z_end;
     const int64_t zz = ok ? z + row : z_end - 1;

@@ -145,6 +145,28 @@ def test_weight_gradient_against_float64_product(device, dtype, rows, K, N, dims
         assert err <= 2e-6 * max(1.0, (x.abs().max() * y.abs().max()).item()) * (rows * d) ** 0.5 + 1e-5 * ref.abs().max().item(), (p, err)
 
 
+@pytest.mark.parametrize("es", [2, 4])
+@pytest.mark.parametrize("extent", [32, 64, 96, 128])
+@pytest.mark.parametrize("d", [1, 3, 5, 7])
+def test_weight_gradient_requests_stay_inside_the_row_piece(es, extent, d):
+    """The requests of ``cueq_linear_dw_mul_ir`` carry no condition (``csrc/linear_dw_mul_ir.hip``, ``dw_body``): thread ``tid``
+    asks for the 16-byte vectors ``E0 + min(v * step, lim)`` of its row's piece, ``E0`` replaced by 0 when the thread's first
+    vector lies past the piece.  Restated here for every supported extent and block size: no request may reach past the
+    ``extent * d`` elements of the piece - for the last row of a tensor that would be past the tensor (a piece of 32 floats
+    was read up to its element 127 before ``E0`` was replaced)."""
+    epv = 16 // es
+    zr, epl = 2 * epv, 128 // es
+    vectors = extent * d // epv
+    for tid in range(256):
+        line0, l8 = (tid >> 3) // zr, tid & 7
+        has = line0 * 8 + l8 < vectors
+        lim = ((vectors - 1 - line0 * 8 - l8) // (8 * (32 // zr))) * (32 // zr) * epl if has else 0
+        e0 = line0 * epl + l8 * epv if has else 0
+        for v in range(d):
+            first = e0 + min(v * (32 // zr) * epl, lim)
+            assert first % epv == 0 and first + epv <= extent * d, (tid, v, first)
+
+
 def test_weight_gradient_argument_checks_without_a_device():
     lib = _lib.load()
     buf = (C.c_char * 4096)()
