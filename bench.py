@@ -141,7 +141,8 @@ def _roofs(bytes_, flops, seconds, flop_peak_tflops, flop_roof: str) -> dict:
             "algorithmic_bytes": bytes_, "flops": flops}
 
 
-def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warmup: int, graph: bool = False) -> dict:
+def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warmup: int, graph: bool = False,
+              calling_thread_autograd: bool = False) -> dict:
     """One secondary workload (BASELINE.json configs[0], [2], [3], [4]); same timing discipline as the headline line.
     Both roofs are reported: algorithmic bytes against 8 TB/s and flops against the matrix-core peak of the input type
     (dense workloads) or the fp32 vector peak (path-table workloads)."""
@@ -346,14 +347,18 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         run = cuda_graph.replay
     else:
         run = step
-    for _ in range(warmup):
-        run()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        run()
-    torch.cuda.synchronize()
-    elapsed = (time.perf_counter() - t0) / steps
+    # calling_thread_autograd: PyTorch hands the backward of GPU tensors to a worker thread of the device and waits for it;
+    # torch.autograd.set_multithreading_enabled(False) runs it on the calling thread (a process-wide setting a single-GPU
+    # user may choose).  The hand-over is most of the host's time in the launch-bound workloads.
+    with torch.autograd.set_multithreading_enabled(not calling_thread_autograd):
+        for _ in range(warmup):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            run()
+        torch.cuda.synchronize()
+        elapsed = (time.perf_counter() - t0) / steps
     # per-kernel durations from a second pass of the same steps with HIP events around the library's kernels: the events cost
     # a few microseconds per kernel on the device (0.09 ms on the eleven launches of the triangle update), so they stay out
     # of the timed region of these workloads
@@ -366,6 +371,8 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         kernels = {n_: {"launches": l, "avg_ms": t / max(l, 1), "ms_per_step": t / steps} for n_, (l, t) in _lib.timing_end().items()}
     if graph:
         desc += "; the step replayed as one HIP graph"
+    if calling_thread_autograd:
+        desc += "; backward on the calling thread (torch.autograd.set_multithreading_enabled(False))"
     roofs = _roofs(alg["fwd"] + alg["bwd"], flops["fwd"] + flops["bwd"], elapsed, flop_peak, flop_roof)
     more = dict(extra) if wl == "cfg5" else {}
     if more:  # the step against 8 TB/s on the bytes its own stages must move (the binding roof of the 2-byte step as decomposed)
@@ -648,6 +655,8 @@ def main() -> int:
                     help="ordered (bit-reproducible) scatter of the node-feature gradient instead of fp atomics")
     ap.add_argument("--graph", action="store_true",
                     help="secondary workloads only: capture the step into a HIP graph and time its replays")
+    ap.add_argument("--calling-thread-autograd", action="store_true",
+                    help="secondary workloads only: time the step with torch.autograd.set_multithreading_enabled(False)")
     ap.add_argument("--workload", choices=["cfg1", "cfg2", "cfg2sh", "cfg3", "cfg4", "cfg4mi", "cfg4fc", "cfg4fcmi", "fcconv", "cfg5"], default=None,
                     help="default: the headline metric (cfg2, fp32) with every other configuration in a 'secondary' object.  "
                          "Naming a workload prints one line for it alone: cfg2 the headline, cfg1 the reference's CPU-sized "
@@ -698,7 +707,8 @@ def main() -> int:
         print(json.dumps({"calibration": "copy", "bytes_read": n * 4, "bytes_written": n * 4, "launches": 5}))
         return 0
     if args.workload not in (None, "cfg2"):
-        print(json.dumps(secondary(torch, cue, cuet, _lib, dev, args.workload, args.dtype, args.steps, args.warmup, args.graph)))
+        print(json.dumps(secondary(torch, cue, cuet, _lib, dev, args.workload, args.dtype, args.steps, args.warmup, args.graph,
+                                   args.calling_thread_autograd)))
         return 0
     # (bf16: buffers of bfloat16, arithmetic in float32 - a secondary measurement, the headline is float32 throughout)
     dtype = {"fp64": torch.float64, "bf16": torch.bfloat16}.get(args.dtype, torch.float32)
@@ -733,12 +743,19 @@ def main() -> int:
                             ("cfg4_linear_fp16", "cfg4", "fp16"), ("cfg4_fc_fp16", "cfg4fc", "fp16")):
             add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))
             if key in ("cfg1_fp32", "cfg4_fc_bf16", "cfg4_fc_bf16_mul_ir") and "error" not in sec[key]:
-                # workloads whose eager step is bound by the host's launch path: the same step replayed as one HIP graph
+                # workloads whose eager step is bound by the host's launch path: the same step replayed as one HIP graph, and
+                # the eager step with the backward on the calling thread instead of PyTorch's device worker thread
                 try:
                     sec[key]["graph_ms_per_step"] = secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm, graph=True)["ms_per_step"]
                 except Exception as e:
                     sec[key]["graph_ms_per_step"] = None
                     sec[key]["graph_error"] = f"{type(e).__name__}: {e}"
+                try:
+                    sec[key]["calling_thread_autograd_ms_per_step"] = secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm,
+                                                                                calling_thread_autograd=True)["ms_per_step"]
+                except Exception as e:
+                    sec[key]["calling_thread_autograd_ms_per_step"] = None
+                    sec[key]["calling_thread_autograd_error"] = f"{type(e).__name__}: {e}"
         if not args.no_cpu_baseline:
             # more CPU baselines (the oracle on this box's host cores, bounded samples): the headline workload on one
             # thread, the dense workloads on the box's share of cores
