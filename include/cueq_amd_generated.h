@@ -16,7 +16,8 @@
  * Every call launches asynchronously on `stream` (a hipStream_t), allocates
  * nothing, and returns 0, or -1 when the launch failed.  Rows are read and written
  * in 16-byte pieces: pointers and row strides of x1, out, g and dx1 must be
- * multiples of 16 bytes.
+ * multiples of 16 bytes, and so must the pointer W (the weight blocks are brought
+ * into the local data share in 16-byte pieces).
  */
 #ifndef CUEQ_AMD_GENERATED_H
 #define CUEQ_AMD_GENERATED_H
