@@ -800,6 +800,7 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=N
     A("")
     A(f'extern "C" int fcj_fwd(int64_t Z, const void* W, const void* X, int64_t ldx, const void* S, int64_t lds_, void* OUT, int64_t ldo, void* stream) {{')
     A("  if (Z <= 0) return 0;")
+    A("  if (reinterpret_cast<uintptr_t>(W) % 16) return -1;  // (the weight blocks are staged in 16-byte pieces)")
     A("  if (prepare(fwd_kernel, kfwdLds, done_fwd)) return -1;")
     A(f"  hipLaunchKernelGGL(fwd_kernel, dim3(grid_for(Z)), dim3(64 * kWaves), kfwdLds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(W), "
       f"static_cast<const {T}*>(X), ldx, static_cast<const {T}*>(S), lds_, static_cast<{T}*>(OUT), ldo, static_cast<int>(Z));")
@@ -807,6 +808,7 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=N
     A("}")
     A(f'extern "C" int fcj_dx1(int64_t Z, const void* W, const void* G, int64_t ldg, const void* S, int64_t lds_, void* DX1, int64_t ldd, void* stream) {{')
     A("  if (Z <= 0) return 0;")
+    A("  if (reinterpret_cast<uintptr_t>(W) % 16) return -1;  // (the weight blocks are staged in 16-byte pieces)")
     A("  if (prepare(dx1_kernel, kdx1Lds, done_dx1)) return -1;")
     A(f"  hipLaunchKernelGGL(dx1_kernel, dim3(grid_for(Z)), dim3(64 * kWaves), kdx1Lds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(W), "
       f"static_cast<const {T}*>(G), ldg, static_cast<const {T}*>(S), lds_, static_cast<{T}*>(DX1), ldd, static_cast<int>(Z));")
@@ -814,6 +816,7 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=N
     A("}")
     A(f'extern "C" int fcj_dx2(int64_t Z, const void* W, const void* X, int64_t ldx, const void* S, int64_t lds_, const void* G, int64_t ldg, void* DX2, int64_t ld2, void* stream) {{')
     A("  if (Z <= 0) return 0;")
+    A("  if (reinterpret_cast<uintptr_t>(W) % 16) return -1;  // (the weight blocks are staged in 16-byte pieces)")
     A("  if (prepare(dx2_kernel, kdx2Lds, done_dx2)) return -1;")
     A(f"  hipLaunchKernelGGL(dx2_kernel, dim3(grid_for(Z)), dim3(64 * kWaves), kdx2Lds, static_cast<hipStream_t>(stream), static_cast<const {T}*>(W), "
       f"static_cast<const {T}*>(X), ldx, static_cast<const {T}*>(S), lds_, static_cast<const {T}*>(G), ldg, static_cast<{T}*>(DX2), ld2, static_cast<int>(Z));")
@@ -824,6 +827,7 @@ def emit_unit(paths, n2: int, width_in: int, width_out: int, T: str, in_blocks=N
       f'void* DX1, int64_t ldd, void* DX2, int64_t ld2, float* PART, void* stream) {{')
     if has_dx12:
         A("  if (Z <= 0) return 0;")
+        A("  if (reinterpret_cast<uintptr_t>(W) % 16) return -1;  // (the weight blocks are staged in 16-byte pieces)")
         A("  if (prepare(dx12_kernel, kdx12Lds, done_dx12)) return -1;")
         A("  const int64_t units = 2 * ((Z + 31) / 32);")
         A("  const int cus = grid_for(int64_t(1) << 40);")
