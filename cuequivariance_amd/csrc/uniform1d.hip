@@ -201,6 +201,10 @@ struct KernelArgs {
   int32_t out_nseg;
   int32_t extent;
   int32_t chunk;
+  // an indexed output whose rows collect very many batch rows: every row is worked on in `zsplit` pieces of its range
+  // (launch row c * rows_real + r = piece c of output row r, written to a partial buffer and added up in order afterwards)
+  int32_t zsplit;
+  int64_t rows_real;
   const int32_t* out_seg_base;  // layout of the output rows (null: default)
   const int32_t* out_seg_stride;
 };
@@ -228,7 +232,17 @@ __device__ __forceinline__ M path_product(const KernelArgs& a, int p, int64_t z,
 template <typename M>
 __device__ __forceinline__ void z_range(const KernelArgs& a, int64_t r, int64_t& z0, int64_t& z1) {
   if (a.out_mode == CUEQ_BATCH_BATCHED) { z0 = r; z1 = r + 1; }
-  else if (a.out_mode == CUEQ_BATCH_INDEXED) { z0 = a.csr_offsets[r]; z1 = a.csr_offsets[r + 1]; }
+  else if (a.out_mode == CUEQ_BATCH_INDEXED) {
+    if (a.zsplit > 1) {
+      const int64_t rr = r % a.rows_real, c = r / a.rows_real;
+      const int64_t lo = a.csr_offsets[rr], len = a.csr_offsets[rr + 1] - lo;
+      z0 = lo + len * c / a.zsplit;
+      z1 = lo + len * (c + 1) / a.zsplit;
+    } else {
+      z0 = a.csr_offsets[r];
+      z1 = a.csr_offsets[r + 1];
+    }
+  }
   else { z0 = r * a.chunk; z1 = min(z0 + a.chunk, a.batch); }
 }
 
@@ -254,12 +268,68 @@ __global__ void __launch_bounds__(256) u1d_generic_elem(KernelArgs a) {
   store_as<M>(a.out, a.out_dtype, where, acc);
 }
 
+// The product of one path for the lanes of a wavefront that differ in the channel only (`u`; p, z the same for all lanes):
+// tables, batch modes, indices and row addresses are then scalar work and a path costs one load per operand and lane.
+template <typename M>
+__device__ __forceinline__ M path_product_lanes(const KernelArgs& a, int p, int64_t z, int u) {
+  M prod = static_cast<M>(a.coeff[p]);
+  const int n = a.nin[p];
+  for (int k = 0; k < n; ++k) {
+    const int32_t packed = a.in[p * kMaxInOperands + k];
+    const DevBuffer& b = a.buf[packed >> 24];
+    const int seg = packed & 0xffffff;
+    int64_t row = 0;
+    if (b.mode == CUEQ_BATCH_BATCHED) row = z;
+    else if (b.mode == CUEQ_BATCH_INDEXED) row = load_index(b.index, b.index_is_64, z);
+    if (b.dim) {
+      const int64_t base = row * (static_cast<int64_t>(b.nseg) * a.extent);
+      const int64_t off = b.seg_base ? base + b.seg_base[seg] + static_cast<int64_t>(u) * b.seg_stride[seg] : base + static_cast<int64_t>(seg) * a.extent + u;
+      prod *= load_as<M>(b.data, b.dtype, off);
+    } else {
+      prod *= load_as<M>(b.data, b.dtype, row * b.nseg + seg);  // (one value for the wavefront)
+    }
+  }
+  return prod;
+}
+
+// One wavefront per (output row, output segment, 64 channels) of an output that carries the channel mode: the lanes are
+// the channels, everything else is the same for the whole wavefront (its number is read into a scalar register, so that the
+// compiler keeps tables, modes and row addresses in scalar registers).
+template <typename M>
+__global__ void __launch_bounds__(256) u1d_generic_rowseg(KernelArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int64_t wid = static_cast<int64_t>(blockIdx.x) * 4 + wv;
+  const int nuc = (a.extent + 63) / 64;
+  if (wid >= a.out_rows * a.out_nseg * nuc) return;
+  const int uc = static_cast<int>(wid % nuc);
+  const int64_t rs = wid / nuc;
+  const int s = static_cast<int>(rs % a.out_nseg);
+  const int64_t r = rs / a.out_nseg;
+  const int u = uc * 64 + lane;
+  const int ul = u < a.extent ? u : a.extent - 1;  // (lanes past the extent compute the last channel again and store nothing)
+  int64_t z0, z1;
+  z_range<M>(a, r, z0, z1);
+  const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
+  M acc = 0;
+  for (int64_t zz = z0; zz < z1; ++zz) {
+    const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
+    for (int p = p0; p < p1; ++p) acc += path_product_lanes<M>(a, p, z, ul);
+  }
+  if (u < a.extent) {
+    const int64_t per_row = static_cast<int64_t>(a.out_nseg) * a.extent;
+    const int64_t where = a.out_seg_base ? r * per_row + a.out_seg_base[s] + static_cast<int64_t>(u) * a.out_seg_stride[s]
+                                         : r * per_row + static_cast<int64_t>(s) * a.extent + u;
+    store_as<M>(a.out, a.out_dtype, where, acc);
+  }
+}
+
 // One wavefront per scalar output element (row, segment): lanes stride over the channel
 // mode, then a fixed-shape butterfly reduction.
 template <typename M>
 __global__ void __launch_bounds__(256) u1d_generic_wave(KernelArgs a) {
   const int lane = threadIdx.x & 63;
-  const int64_t wid = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+  const int64_t wid = static_cast<int64_t>(blockIdx.x) * 4 + __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   if (wid >= a.out_rows * a.out_nseg) return;
   const int64_t r = wid / a.out_nseg;
   const int s = static_cast<int>(wid - r * a.out_nseg);
@@ -274,9 +344,14 @@ __global__ void __launch_bounds__(256) u1d_generic_wave(KernelArgs a) {
       bool has_channel = false;
       for (int k = 0; k < a.nin[p]; ++k) has_channel |= a.buf[a.in[p * kMaxInOperands + k] >> 24].dim != 0;
       if (has_channel) {
-        for (int u = lane; u < a.extent; u += 64) acc += path_product<M>(a, p, z, u);
-      } else if (lane == 0) {
-        acc += path_product<M>(a, p, z, 0);
+        for (int u0 = 0; u0 < a.extent; u0 += 64) {  // (u0 the same for all lanes; a lane past the extent adds nothing)
+          const int u = u0 + lane;
+          const M v = path_product_lanes<M>(a, p, z, u < a.extent ? u : a.extent - 1);
+          acc += u < a.extent ? v : static_cast<M>(0);
+        }
+      } else {
+        const M v = path_product_lanes<M>(a, p, z, 0);
+        acc += lane == 0 ? v : static_cast<M>(0);
       }
     }
   }
@@ -580,6 +655,13 @@ extern "C" void cueq_u1d_plan_destroy(cueq_u1d_plan* plan) {
 
 static int64_t share_chunks(int64_t batch) { return (batch + kShareChunk - 1) / kShareChunk; }
 
+// Pieces per row of an indexed output: 1 unless its rows collect a thousand batch rows and more on average (a weight
+// gradient indexed by a handful of classes), then about 256 batch rows a piece, at most 64 pieces.
+static int64_t row_splits(int64_t batch, int64_t rows) {
+  if (rows <= 0 || batch / rows < 1024) return 1;
+  return std::min<int64_t>(64, (batch / rows + 255) / 256);
+}
+
 extern "C" int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch) {
   if (!plan || !buffers) return 0;
   const int msize = plan->math_dtype == CUEQ_F64 ? 8 : 4;
@@ -590,10 +672,15 @@ extern "C" int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq
   }
   for (int ob = 0; ob < plan->num_outputs; ++ob) {
     const int b = plan->num_inputs + ob;
+    const int64_t width = static_cast<int64_t>(plan->buffer_nseg[b]) * (plan->buffer_dim[b] ? plan->extent : 1);
+    if (buffers[b].batch_dim == CUEQ_BATCH_INDEXED) {
+      const int64_t splits = row_splits(batch, buffers[b].rows);
+      if (splits > 1) need = std::max<int64_t>(need, splits * buffers[b].rows * width * msize);
+      continue;
+    }
     if (buffers[b].batch_dim != CUEQ_BATCH_SHARED) continue;
     const int64_t nch = share_chunks(batch);
     if (nch <= 1) continue;
-    const int64_t width = static_cast<int64_t>(plan->buffer_nseg[b]) * (plan->buffer_dim[b] ? plan->extent : 1);
     need = std::max<int64_t>(need, nch * width * msize);
   }
   return need;
@@ -659,6 +746,17 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
     a.out_seg_base = plan->seg_base[b];
     a.out_seg_stride = plan->seg_stride[b];
     int64_t nchunks = 0;
+    a.zsplit = 1;
+    a.rows_real = o.rows;
+    if (o.batch_dim == CUEQ_BATCH_INDEXED && row_splits(batch, o.rows) > 1) {
+      const int64_t splits = row_splits(batch, o.rows);
+      const int64_t need = splits * o.rows * width * static_cast<int64_t>(sizeof(M));
+      CUEQ_REQUIRE(workspace != nullptr && workspace_bytes >= need, CUEQ_ERR_INVALID, "workspace too small: need %lld bytes", (long long)need);
+      a.out = workspace;
+      a.out_dtype = sizeof(M) == 8 ? CUEQ_F64 : CUEQ_F32;
+      a.out_rows = splits * o.rows;
+      a.zsplit = static_cast<int32_t>(splits);
+    }
     if (o.batch_dim == CUEQ_BATCH_SHARED) {
       nchunks = share_chunks(batch);
       if (nchunks > 1) {
@@ -676,13 +774,27 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
     const int64_t work = a.out_rows * (wave ? static_cast<int64_t>(a.out_nseg) * 64 : width);
     const int64_t blocks = (work + 255) / 256;
     CUEQ_REQUIRE(blocks < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "output %d too large for one launch", ob);
-    if (wave) hipLaunchKernelGGL(u1d_generic_wave<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    // outputs that carry the channel mode (at least half a wavefront of channels): a wavefront per (row, segment, 64 channels)
+    const bool rowseg = !wave && plan->buffer_dim[b] && plan->extent >= 32;
+    if (rowseg) {
+      const int64_t waves = a.out_rows * a.out_nseg * ((plan->extent + 63) / 64);
+      const int64_t rblocks = (waves + 3) / 4;
+      CUEQ_REQUIRE(rblocks < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "output %d too large for one launch", ob);
+      hipLaunchKernelGGL(u1d_generic_rowseg<M>, dim3(static_cast<unsigned>(rblocks)), dim3(256), 0, stream, a);
+    } else if (wave) hipLaunchKernelGGL(u1d_generic_wave<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
     else hipLaunchKernelGGL(u1d_generic_elem<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
     CUEQ_CHECK_HIP(hipGetLastError());
     if (nchunks > 1) {
       const int64_t fb = (width + 255) / 256;
       hipLaunchKernelGGL(u1d_fold_chunks<M>, dim3(static_cast<unsigned>(fb)), dim3(256), 0, stream,
                          static_cast<const M*>(workspace), nchunks, width, o.data, o.dtype);
+      CUEQ_CHECK_HIP(hipGetLastError());
+    }
+    if (a.zsplit > 1) {  // the pieces of every row, added in order
+      const int64_t elems = o.rows * width, fb = (elems + 255) / 256;
+      CUEQ_REQUIRE(fb < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "output %d too large for one launch", ob);
+      hipLaunchKernelGGL(u1d_fold_chunks<M>, dim3(static_cast<unsigned>(fb)), dim3(256), 0, stream,
+                         static_cast<const M*>(workspace), static_cast<int64_t>(a.zsplit), elems, o.data, o.dtype);
       CUEQ_CHECK_HIP(hipGetLastError());
     }
   }

@@ -121,6 +121,19 @@ def test_channelwise_non_registered_descriptor_uses_table_driven_kernels(device)
         assert not m.f.m._plan(torch.float32).specialised(device)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_table_driven_kernels_split_very_long_output_rows(device, dtype, monkeypatch):
+    """Three output rows that collect 1 400 edges each (a gradient indexed by a handful of classes looks like this): the
+    table-driven kernels work on such a row in pieces of its edge range and add the pieces in order.  48 and 96 channels
+    (one wavefront per 64 channels of a row segment, the second one partly filled), every gradient, twice for the same bits."""
+    monkeypatch.setenv("CUEQ_FORCE_GENERIC", "1")
+    for channels in (48, 96):
+        m = cw_module(f"{channels}x0e+{channels}x1o", "0e+1o", "0e+1o")
+        out, grads = run_cw_case(device, m, N=3, Z=4200, dtype=dtype, seed=11 + channels, sort_receivers=False)
+        out2, grads2 = run_cw_case(device, m, N=3, Z=4200, dtype=dtype, seed=11 + channels, sort_receivers=False)
+        assert torch.equal(out, out2) and all(torch.equal(a, b) for a, b in zip(grads, grads2))
+
+
 def test_channelwise_mul_ir_layout_and_shared_internal_weights(device):
     from cuequivariance_amd import cuet
 
