@@ -183,8 +183,22 @@ struct DevBuffer {
   const int32_t* seg_stride;
 };
 
+// One path as the wavefront-uniform kernels read it - 80 bytes in one piece (the separate arrays below cost three requests
+// and leave the buffer's mode, type and layout to be looked up per operand): operand k is element off[k] + u * stride[k] of
+// the row of buffer buf[k] (stride 0: a scalar operand; the row layout of the buffer is worked into off and stride).
+struct PathRow {
+  double coeff;
+  int32_t nin;
+  int32_t channel;             // 1 when one of the inputs carries the channel mode
+  uint8_t buf[8];
+  int32_t off[kMaxInOperands];
+  int32_t stride[kMaxInOperands];
+};
+static_assert(sizeof(PathRow) == 80, "a path row is 80 bytes");
+
 struct KernelArgs {
   DevBuffer buf[kMaxBuffers];
+  const PathRow* rows;      // the paths once more, packed
   // path tables of the output buffer being computed
   const double* coeff;
   const int32_t* nin;       // inputs of each path
@@ -205,6 +219,7 @@ struct KernelArgs {
   // (launch row c * rows_real + r = piece c of output row r, written to a partial buffer and added up in order afterwards)
   int32_t zsplit;
   int64_t rows_real;
+  int32_t same_type;  // every buffer holds elements of the arithmetic type: operands are loaded without a switch on the type
   const int32_t* out_seg_base;  // layout of the output rows (null: default)
   const int32_t* out_seg_stride;
 };
@@ -292,6 +307,69 @@ __device__ __forceinline__ M path_product_lanes(const KernelArgs& a, int p, int6
   return prod;
 }
 
+// Path row p, the same for the whole wavefront, read through the constant address space: the table is written once when the
+// plan is made and never by a kernel, so the read may go through the scalar unit into scalar registers (read as ordinary global
+// memory it costs every lane a vector load, and a readfirstlane per field).
+__device__ __forceinline__ PathRow load_path_row(const PathRow* rows, int p) {
+  typedef const __attribute__((address_space(4))) uint32_t* ConstWords;
+  ConstWords q = (ConstWords)(reinterpret_cast<uintptr_t>(rows + p));
+  uint32_t w[sizeof(PathRow) / 4];
+#pragma unroll
+  for (int k = 0; k < static_cast<int>(sizeof(PathRow) / 4); ++k) w[k] = q[k];
+  PathRow r;
+  __builtin_memcpy(&r, w, sizeof(PathRow));
+  return r;
+}
+
+// The row of every buffer for batch row z as a pointer, one lane per buffer, into `srow` (LDS, private to the wavefront): the
+// batch mode and the index of a buffer are looked at once per batch row, not once per path and operand.  Every buffer holds
+// elements of type M here (KernelArgs::same_type).
+// (The pointers are kept as pointers into global memory: a load through a generic pointer counts as an LDS access as well, and the
+// wait for the next row pointer would then wait for the operand loads in flight.)
+template <typename M>
+using GlobalRow = const __attribute__((address_space(1))) M*;
+
+template <typename M>
+__device__ __forceinline__ void row_pointers(const KernelArgs& a, int64_t z, int lane, GlobalRow<M>* srow) {
+  if (lane < kMaxBuffers) {
+    const DevBuffer& b = a.buf[lane];
+    int64_t row = 0;
+    if (b.mode == CUEQ_BATCH_BATCHED) row = z;
+    else if (b.mode == CUEQ_BATCH_INDEXED && b.index != nullptr) row = load_index(b.index, b.index_is_64, z);
+    srow[lane] = (GlobalRow<M>)(reinterpret_cast<uintptr_t>(b.data)) + row * (b.dim ? static_cast<int64_t>(b.nseg) * a.extent : static_cast<int64_t>(b.nseg));
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // (the same wavefront reads what it wrote: LDS works in order)
+  __builtin_amdgcn_wave_barrier();
+}
+
+// The product of a path with N operands: the N loads are issued together, then multiplied in the order of the table (the same
+// order, hence the same bits, as path_product_lanes).  No branch, nothing looked up per operand but the row pointer.
+template <typename M, int N>
+__device__ __forceinline__ M path_product_same(const PathRow& r, int u, const GlobalRow<M>* srow) {
+  M v[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) v[k] = srow[r.buf[k]][r.off[k] + u * r.stride[k]];
+  M prod = static_cast<M>(r.coeff);
+#pragma unroll
+  for (int k = 0; k < N; ++k) prod *= v[k];
+  return prod;
+}
+
+// One path (its packed row `r`) for the lanes of a wavefront, the rows of the batch row in `srow`.
+template <typename M>
+__device__ __forceinline__ M path_product_row(const PathRow& r, int u, const GlobalRow<M>* srow) {
+  switch (r.nin) {
+    case 0: return static_cast<M>(r.coeff);
+    case 1: return path_product_same<M, 1>(r, u, srow);
+    case 2: return path_product_same<M, 2>(r, u, srow);
+    case 3: return path_product_same<M, 3>(r, u, srow);
+    case 4: return path_product_same<M, 4>(r, u, srow);
+    case 5: return path_product_same<M, 5>(r, u, srow);
+    case 6: return path_product_same<M, 6>(r, u, srow);
+    default: return path_product_same<M, 7>(r, u, srow);
+  }
+}
+
 // One wavefront per (output row, output segment, 64 channels) of an output that carries the channel mode: the lanes are
 // the channels, everything else is the same for the whole wavefront (its number is read into a scalar register, so that the
 // compiler keeps tables, modes and row addresses in scalar registers).
@@ -311,10 +389,23 @@ __global__ void __launch_bounds__(256) u1d_generic_rowseg(KernelArgs a) {
   int64_t z0, z1;
   z_range<M>(a, r, z0, z1);
   const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
+  __shared__ GlobalRow<M> srow_all[4][kMaxBuffers];
+  GlobalRow<M>* srow = srow_all[wv];
   M acc = 0;
   for (int64_t zz = z0; zz < z1; ++zz) {
     const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
-    for (int p = p0; p < p1; ++p) acc += path_product_lanes<M>(a, p, z, ul);
+    if (a.same_type) {
+      row_pointers<M>(a, z, lane, srow);
+      PathRow next = load_path_row(a.rows, p0 < p1 ? p0 : 0);  // (the row of the next path is requested while this one is worked on)
+      for (int p = p0; p < p1; ++p) {
+        const PathRow cur = next;
+        next = load_path_row(a.rows, p + 1 < p1 ? p + 1 : p);
+        acc += path_product_row<M>(cur, ul, srow);
+      }
+    } else {
+      for (int p = p0; p < p1; ++p) acc += path_product_lanes<M>(a, p, z, ul);
+    }
+    __builtin_amdgcn_wave_barrier();  // (the next batch row overwrites the offsets)
   }
   if (u < a.extent) {
     const int64_t per_row = static_cast<int64_t>(a.out_nseg) * a.extent;
@@ -336,9 +427,31 @@ __global__ void __launch_bounds__(256) u1d_generic_wave(KernelArgs a) {
   int64_t z0, z1;
   z_range<M>(a, r, z0, z1);
   const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
+  __shared__ GlobalRow<M> srow_all[4][kMaxBuffers];
+  GlobalRow<M>* srow = srow_all[wid & 3];
   M acc = 0;
   for (int64_t zz = z0; zz < z1; ++zz) {
     const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
+    if (a.same_type) {  // the same sums in the same order, the paths read as packed rows
+      row_pointers<M>(a, z, lane, srow);
+      PathRow next = load_path_row(a.rows, p0 < p1 ? p0 : 0);
+      for (int p = p0; p < p1; ++p) {
+        const PathRow cur = next;
+        next = load_path_row(a.rows, p + 1 < p1 ? p + 1 : p);
+        if (cur.channel) {
+          for (int u0 = 0; u0 < a.extent; u0 += 64) {
+            const int u = u0 + lane;
+            const M v = path_product_row<M>(cur, u < a.extent ? u : a.extent - 1, srow);
+            acc += u < a.extent ? v : static_cast<M>(0);
+          }
+        } else {
+          const M v = path_product_row<M>(cur, 0, srow);
+          acc += lane == 0 ? v : static_cast<M>(0);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      continue;
+    }
     for (int p = p0; p < p1; ++p) {
       // a path sums over the channel mode only when one of its inputs carries it; a path of scalars contributes once
       bool has_channel = false;
@@ -375,6 +488,7 @@ struct OutTables {
   double* coeff = nullptr;
   int32_t* nin = nullptr;
   int32_t* in = nullptr;
+  PathRow* rows = nullptr;
   int32_t* seg_start = nullptr;
   bool contracts_channel = false;  // scalar output fed by channel-carrying inputs
 };
@@ -531,7 +645,7 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
   // Lay all tables out in one host blob, then one upload.
   size_t total = 0;
   auto reserve = [&](size_t bytes) { size_t o = total; total += (bytes + 15) & ~size_t(15); return o; };
-  struct Off { size_t coeff, nin, in, seg; };
+  struct Off { size_t coeff, nin, in, rows, seg; };
   std::vector<Off> offs(d->num_outputs);
   for (int ob = 0; ob < d->num_outputs; ++ob) {
     auto& v = per_out[ob];
@@ -540,6 +654,7 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
     offs[ob].coeff = reserve(v.size() * sizeof(double));
     offs[ob].nin = reserve(v.size() * sizeof(int32_t));
     offs[ob].in = reserve(v.size() * kMaxInOperands * sizeof(int32_t));
+    offs[ob].rows = reserve((v.size() + 1) * sizeof(PathRow));
     offs[ob].seg = reserve((nseg + 1) * sizeof(int32_t));
   }
   // row layouts: per buffer the base offset and channel stride of every segment
@@ -582,11 +697,31 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
     auto* nin = reinterpret_cast<int32_t*>(host.data() + offs[ob].nin);
     auto* in = reinterpret_cast<int32_t*>(host.data() + offs[ob].in);
     auto* seg = reinterpret_cast<int32_t*>(host.data() + offs[ob].seg);
+    auto* rows = reinterpret_cast<PathRow*>(host.data() + offs[ob].rows);
     std::vector<int32_t> count(nseg + 1, 0);
     for (size_t p = 0; p < v.size(); ++p) {
       coeff[p] = v[p].c;
       nin[p] = v[p].nin;
       std::memcpy(in + p * kMaxInOperands, v[p].in, sizeof(v[p].in));
+      rows[p].coeff = v[p].c;
+      rows[p].nin = v[p].nin;
+      rows[p].channel = 0;
+      for (int k = 0; k < v[p].nin; ++k) {
+        const int bi = v[p].in[k] >> 24, sg = v[p].in[k] & 0xffffff;
+        rows[p].buf[k] = static_cast<uint8_t>(bi);
+        if (d->buffer_dim[bi] == 0) {  // a scalar per segment
+          rows[p].off[k] = sg;
+          rows[p].stride[k] = 0;
+        } else if (lay_off[bi] != SIZE_MAX) {  // rows in groups: base and channel stride of the segment
+          rows[p].off[k] = lay_tab[bi][sg];
+          rows[p].stride[k] = lay_tab[bi][d->buffer_num_segments[bi] + sg];
+          rows[p].channel = 1;
+        } else {
+          rows[p].off[k] = sg * static_cast<int32_t>(d->operand_extent);
+          rows[p].stride[k] = 1;
+          rows[p].channel = 1;
+        }
+      }
       count[v[p].out_seg + 1]++;
     }
     seg[0] = 0;
@@ -607,6 +742,7 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
     t.coeff = reinterpret_cast<double*>(base + offs[ob].coeff);
     t.nin = reinterpret_cast<int32_t*>(base + offs[ob].nin);
     t.in = reinterpret_cast<int32_t*>(base + offs[ob].in);
+    t.rows = reinterpret_cast<PathRow*>(base + offs[ob].rows);
     t.seg_start = reinterpret_cast<int32_t*>(base + offs[ob].seg);
     t.contracts_channel = contracts[ob];
   }
@@ -723,6 +859,9 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
   a.batch = batch;
   a.extent = plan->extent;
   a.chunk = kShareChunk;
+  a.same_type = 1;
+  for (int b = 0; b < plan->num_inputs; ++b)
+    if (buffers[b].dtype != (sizeof(M) == 8 ? CUEQ_F64 : CUEQ_F32)) a.same_type = 0;
 
   for (int ob = 0; ob < plan->num_outputs; ++ob) {
     const int b = plan->num_inputs + ob;
@@ -734,6 +873,7 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
     a.coeff = t.coeff;
     a.nin = t.nin;
     a.in = t.in;
+    a.rows = t.rows;
     a.seg_start = t.seg_start;
     a.out_dim = plan->buffer_dim[b];
     a.out_nseg = plan->buffer_nseg[b];
