@@ -389,23 +389,90 @@ __global__ void __launch_bounds__(256) u1d_generic_rowseg(KernelArgs a) {
   int64_t z0, z1;
   z_range<M>(a, r, z0, z1);
   const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
-  __shared__ GlobalRow<M> srow_all[4][kMaxBuffers];
-  GlobalRow<M>* srow = srow_all[wv];
   M acc = 0;
   for (int64_t zz = z0; zz < z1; ++zz) {
     const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
-    if (a.same_type) {
+    for (int p = p0; p < p1; ++p) acc += path_product_lanes<M>(a, p, z, ul);
+  }
+  if (u < a.extent) {
+    const int64_t per_row = static_cast<int64_t>(a.out_nseg) * a.extent;
+    const int64_t where = a.out_seg_base ? r * per_row + a.out_seg_base[s] + static_cast<int64_t>(u) * a.out_seg_stride[s]
+                                         : r * per_row + static_cast<int64_t>(s) * a.extent + u;
+    store_as<M>(a.out, a.out_dtype, where, acc);
+  }
+}
+
+// 1 in global memory: what the operands past the last one of a path read in u1d_rowseg_paths.
+__device__ const float kOneFloat = 1.0f;
+__device__ const double kOneDouble = 1.0;
+template <typename M>
+__device__ __forceinline__ GlobalRow<M> pointer_to_one() {
+  if constexpr (sizeof(M) == 8) return (GlobalRow<M>)(reinterpret_cast<uintptr_t>(&kOneDouble));
+  else return (GlobalRow<M>)(reinterpret_cast<uintptr_t>(&kOneFloat));
+}
+
+template <typename M, int N>
+__device__ __forceinline__ void request_operands(const PathRow& r, int u, const GlobalRow<M>* srow, M (&v)[N]) {
+#pragma unroll
+  for (int k = 0; k < N; ++k) v[k] = srow[r.buf[k]][r.off[k] + u * r.stride[k]];
+}
+
+template <typename M, int N>
+__device__ __forceinline__ M product_of(const PathRow& r, const M (&v)[N]) {
+  M prod = static_cast<M>(r.coeff);
+#pragma unroll
+  for (int k = 0; k < N; ++k) prod *= v[k];
+  return prod;
+}
+
+// u1d_generic_rowseg for buffers that all hold the math type, every path read as exactly N operands (N: the most operands of a
+// path of this output; a path with fewer has the rest point at a 1 in memory - multiplying by 1 changes no bit).  With the count
+// fixed there is no branch in the walk, and the operands of a path are requested while the path before it still waits for its
+// own: two paths in flight per wavefront, where the memory latency of one (row pointer from LDS, then the operand from L2) is
+// what a path costs.  Sums in the order of the table, as u1d_generic_rowseg.
+template <typename M, int N>
+__global__ void __launch_bounds__(256) u1d_rowseg_paths(KernelArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int64_t wid = static_cast<int64_t>(blockIdx.x) * 4 + wv;
+  const int nuc = (a.extent + 63) / 64;
+  if (wid >= a.out_rows * a.out_nseg * nuc) return;
+  const int uc = static_cast<int>(wid % nuc);
+  const int64_t rs = wid / nuc;
+  const int s = static_cast<int>(rs % a.out_nseg);
+  const int64_t r = rs / a.out_nseg;
+  const int u = uc * 64 + lane;
+  const int ul = u < a.extent ? u : a.extent - 1;
+  int64_t z0, z1;
+  z_range<M>(a, r, z0, z1);
+  const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
+  __shared__ GlobalRow<M> srow_all[4][kMaxBuffers + 1];
+  GlobalRow<M>* srow = srow_all[wv];
+  M acc = 0;
+  if (p0 < p1) {
+    for (int64_t zz = z0; zz < z1; ++zz) {
+      const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
+      if (lane == kMaxBuffers) srow[kMaxBuffers] = pointer_to_one<M>();
       row_pointers<M>(a, z, lane, srow);
-      PathRow next = load_path_row(a.rows, p0 < p1 ? p0 : 0);  // (the row of the next path is requested while this one is worked on)
-      for (int p = p0; p < p1; ++p) {
-        const PathRow cur = next;
-        next = load_path_row(a.rows, p + 1 < p1 ? p + 1 : p);
-        acc += path_product_row<M>(cur, ul, srow);
+      PathRow ra = load_path_row(a.rows, p0);
+      PathRow rb = load_path_row(a.rows, p0 + 1 < p1 ? p0 + 1 : p0);
+      M va[N], vb[N];
+      request_operands<M, N>(ra, ul, srow, va);
+      for (int p = p0; p < p1; p += 2) {  // ra, va: path p; rb: path p + 1 (or the last path once more, then not added)
+        request_operands<M, N>(rb, ul, srow, vb);
+        __builtin_amdgcn_sched_barrier(0);  // (a scalar read asked for earlier would be waited for together with the LDS reads)
+        const PathRow rn = load_path_row(a.rows, p + 2 < p1 ? p + 2 : p1 - 1);
+        acc += product_of<M, N>(ra, va);
+        request_operands<M, N>(rn, ul, srow, va);
+        __builtin_amdgcn_sched_barrier(0);
+        const PathRow rm = load_path_row(a.rows, p + 3 < p1 ? p + 3 : p1 - 1);
+        const M second = product_of<M, N>(rb, vb);
+        acc += p + 1 < p1 ? second : static_cast<M>(0);
+        ra = rn;
+        rb = rm;
       }
-    } else {
-      for (int p = p0; p < p1; ++p) acc += path_product_lanes<M>(a, p, z, ul);
+      __builtin_amdgcn_wave_barrier();  // (the next batch row overwrites the pointers)
     }
-    __builtin_amdgcn_wave_barrier();  // (the next batch row overwrites the offsets)
   }
   if (u < a.extent) {
     const int64_t per_row = static_cast<int64_t>(a.out_nseg) * a.extent;
@@ -490,6 +557,7 @@ struct OutTables {
   int32_t* in = nullptr;
   PathRow* rows = nullptr;
   int32_t* seg_start = nullptr;
+  int max_nin = 1;                 // the most input operands of a path (at least 1)
   bool contracts_channel = false;  // scalar output fed by channel-carrying inputs
 };
 
@@ -706,6 +774,7 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
       rows[p].coeff = v[p].c;
       rows[p].nin = v[p].nin;
       rows[p].channel = 0;
+      for (int k = v[p].nin; k < kMaxInOperands; ++k) rows[p].buf[k] = kMaxBuffers;  // (the slot of the 1; offset and stride 0)
       for (int k = 0; k < v[p].nin; ++k) {
         const int bi = v[p].in[k] >> 24, sg = v[p].in[k] & 0xffffff;
         rows[p].buf[k] = static_cast<uint8_t>(bi);
@@ -745,6 +814,7 @@ extern "C" int cueq_u1d_plan_create(const cueq_u1d_desc* d, cueq_u1d_plan** out_
     t.rows = reinterpret_cast<PathRow*>(base + offs[ob].rows);
     t.seg_start = reinterpret_cast<int32_t*>(base + offs[ob].seg);
     t.contracts_channel = contracts[ob];
+    for (const auto& path : per_out[ob]) t.max_nin = std::max<int>(t.max_nin, path.nin);
   }
   plan->seg_base.assign(nbuf, nullptr);
   plan->seg_stride.assign(nbuf, nullptr);
@@ -792,10 +862,11 @@ extern "C" void cueq_u1d_plan_destroy(cueq_u1d_plan* plan) {
 static int64_t share_chunks(int64_t batch) { return (batch + kShareChunk - 1) / kShareChunk; }
 
 // Pieces per row of an indexed output: 1 unless its rows collect a thousand batch rows and more on average (a weight
-// gradient indexed by a handful of classes), then about 256 batch rows a piece, at most 64 pieces.
+// gradient indexed by a handful of classes: few rows, hence few wavefronts, each with a long walk), then about 64 batch rows a
+// piece, at most 64 pieces.
 static int64_t row_splits(int64_t batch, int64_t rows) {
   if (rows <= 0 || batch / rows < 1024) return 1;
-  return std::min<int64_t>(64, (batch / rows + 255) / 256);
+  return std::min<int64_t>(64, (batch / rows + 63) / 64);
 }
 
 extern "C" int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch) {
@@ -920,7 +991,17 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
       const int64_t waves = a.out_rows * a.out_nseg * ((plan->extent + 63) / 64);
       const int64_t rblocks = (waves + 3) / 4;
       CUEQ_REQUIRE(rblocks < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "output %d too large for one launch", ob);
-      hipLaunchKernelGGL(u1d_generic_rowseg<M>, dim3(static_cast<unsigned>(rblocks)), dim3(256), 0, stream, a);
+      const dim3 rgrid(static_cast<unsigned>(rblocks));
+      if (!a.same_type) hipLaunchKernelGGL(u1d_generic_rowseg<M>, rgrid, dim3(256), 0, stream, a);
+      else switch (t.max_nin) {
+        case 1: hipLaunchKernelGGL((u1d_rowseg_paths<M, 1>), rgrid, dim3(256), 0, stream, a); break;
+        case 2: hipLaunchKernelGGL((u1d_rowseg_paths<M, 2>), rgrid, dim3(256), 0, stream, a); break;
+        case 3: hipLaunchKernelGGL((u1d_rowseg_paths<M, 3>), rgrid, dim3(256), 0, stream, a); break;
+        case 4: hipLaunchKernelGGL((u1d_rowseg_paths<M, 4>), rgrid, dim3(256), 0, stream, a); break;
+        case 5: hipLaunchKernelGGL((u1d_rowseg_paths<M, 5>), rgrid, dim3(256), 0, stream, a); break;
+        case 6: hipLaunchKernelGGL((u1d_rowseg_paths<M, 6>), rgrid, dim3(256), 0, stream, a); break;
+        default: hipLaunchKernelGGL((u1d_rowseg_paths<M, 7>), rgrid, dim3(256), 0, stream, a); break;
+      }
     } else if (wave) hipLaunchKernelGGL(u1d_generic_wave<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
     else hipLaunchKernelGGL(u1d_generic_elem<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
     CUEQ_CHECK_HIP(hipGetLastError());
