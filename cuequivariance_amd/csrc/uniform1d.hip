@@ -342,34 +342,6 @@ __device__ __forceinline__ void row_pointers(const KernelArgs& a, int64_t z, int
   __builtin_amdgcn_wave_barrier();
 }
 
-// The product of a path with N operands: the N loads are issued together, then multiplied in the order of the table (the same
-// order, hence the same bits, as path_product_lanes).  No branch, nothing looked up per operand but the row pointer.
-template <typename M, int N>
-__device__ __forceinline__ M path_product_same(const PathRow& r, int u, const GlobalRow<M>* srow) {
-  M v[N];
-#pragma unroll
-  for (int k = 0; k < N; ++k) v[k] = srow[r.buf[k]][r.off[k] + u * r.stride[k]];
-  M prod = static_cast<M>(r.coeff);
-#pragma unroll
-  for (int k = 0; k < N; ++k) prod *= v[k];
-  return prod;
-}
-
-// One path (its packed row `r`) for the lanes of a wavefront, the rows of the batch row in `srow`.
-template <typename M>
-__device__ __forceinline__ M path_product_row(const PathRow& r, int u, const GlobalRow<M>* srow) {
-  switch (r.nin) {
-    case 0: return static_cast<M>(r.coeff);
-    case 1: return path_product_same<M, 1>(r, u, srow);
-    case 2: return path_product_same<M, 2>(r, u, srow);
-    case 3: return path_product_same<M, 3>(r, u, srow);
-    case 4: return path_product_same<M, 4>(r, u, srow);
-    case 5: return path_product_same<M, 5>(r, u, srow);
-    case 6: return path_product_same<M, 6>(r, u, srow);
-    default: return path_product_same<M, 7>(r, u, srow);
-  }
-}
-
 // One wavefront per (output row, output segment, 64 channels) of an output that carries the channel mode: the lanes are
 // the channels, everything else is the same for the whole wavefront (its number is read into a scalar register, so that the
 // compiler keeps tables, modes and row addresses in scalar registers).
@@ -425,11 +397,38 @@ __device__ __forceinline__ M product_of(const PathRow& r, const M (&v)[N]) {
   return prod;
 }
 
-// u1d_generic_rowseg for buffers that all hold the math type, every path read as exactly N operands (N: the most operands of a
-// path of this output; a path with fewer has the rest point at a 1 in memory - multiplying by 1 changes no bit).  With the count
-// fixed there is no branch in the walk, and the operands of a path are requested while the path before it still waits for its
-// own: two paths in flight per wavefront, where the memory latency of one (row pointer from LDS, then the operand from L2) is
-// what a path costs.  Sums in the order of the table, as u1d_generic_rowseg.
+// The paths p0 <= p < p1 (p0 < p1) of one batch row for the lanes of a wavefront, every path read as exactly N operands (N: the
+// most operands of a path of this output; a path with fewer has the rest point at a 1 in memory - multiplying by 1 changes no
+// bit).  With the count fixed there is no branch in the walk, and the operands of a path are requested while the path before it
+// still waits for its own: two paths in flight per wavefront, where the memory latency of one (row pointer from LDS, then the
+// operand from L2) is what a path costs.  Returns acc + the products in the order of the table.  Reduce: the lanes are summed
+// afterwards, so a path adds only where it should count - in the lanes inside the extent when it carries the channel mode,
+// in the first lane of the first 64 channels otherwise.
+template <typename M, int N, bool Reduce>
+__device__ __forceinline__ M walk_paths(const PathRow* rows, int p0, int p1, int u, bool inside, bool first, const GlobalRow<M>* srow,
+                                        M acc) {
+  PathRow ra = load_path_row(rows, p0);
+  PathRow rb = load_path_row(rows, p0 + 1 < p1 ? p0 + 1 : p0);
+  M va[N], vb[N];
+  request_operands<M, N>(ra, u, srow, va);
+  for (int p = p0; p < p1; p += 2) {  // ra, va: path p; rb: path p + 1 (or the last path once more, then not added)
+    request_operands<M, N>(rb, u, srow, vb);
+    __builtin_amdgcn_sched_barrier(0);  // (a scalar read asked for earlier would be waited for together with the LDS reads)
+    const PathRow rn = load_path_row(rows, p + 2 < p1 ? p + 2 : p1 - 1);
+    const M one = product_of<M, N>(ra, va);
+    acc += !Reduce || (ra.channel ? inside : first) ? one : static_cast<M>(0);
+    request_operands<M, N>(rn, u, srow, va);
+    __builtin_amdgcn_sched_barrier(0);
+    const PathRow rm = load_path_row(rows, p + 3 < p1 ? p + 3 : p1 - 1);
+    const M two = product_of<M, N>(rb, vb);
+    acc += p + 1 < p1 && (!Reduce || (rb.channel ? inside : first)) ? two : static_cast<M>(0);
+    ra = rn;
+    rb = rm;
+  }
+  return acc;
+}
+
+// u1d_generic_rowseg for buffers that all hold the math type (walk_paths).
 template <typename M, int N>
 __global__ void __launch_bounds__(256) u1d_rowseg_paths(KernelArgs a) {
   const int lane = threadIdx.x & 63;
@@ -454,23 +453,7 @@ __global__ void __launch_bounds__(256) u1d_rowseg_paths(KernelArgs a) {
       const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
       if (lane == kMaxBuffers) srow[kMaxBuffers] = pointer_to_one<M>();
       row_pointers<M>(a, z, lane, srow);
-      PathRow ra = load_path_row(a.rows, p0);
-      PathRow rb = load_path_row(a.rows, p0 + 1 < p1 ? p0 + 1 : p0);
-      M va[N], vb[N];
-      request_operands<M, N>(ra, ul, srow, va);
-      for (int p = p0; p < p1; p += 2) {  // ra, va: path p; rb: path p + 1 (or the last path once more, then not added)
-        request_operands<M, N>(rb, ul, srow, vb);
-        __builtin_amdgcn_sched_barrier(0);  // (a scalar read asked for earlier would be waited for together with the LDS reads)
-        const PathRow rn = load_path_row(a.rows, p + 2 < p1 ? p + 2 : p1 - 1);
-        acc += product_of<M, N>(ra, va);
-        request_operands<M, N>(rn, ul, srow, va);
-        __builtin_amdgcn_sched_barrier(0);
-        const PathRow rm = load_path_row(a.rows, p + 3 < p1 ? p + 3 : p1 - 1);
-        const M second = product_of<M, N>(rb, vb);
-        acc += p + 1 < p1 ? second : static_cast<M>(0);
-        ra = rn;
-        rb = rm;
-      }
+      acc = walk_paths<M, N, false>(a.rows, p0, p1, ul, true, true, srow, acc);
       __builtin_amdgcn_wave_barrier();  // (the next batch row overwrites the pointers)
     }
   }
@@ -480,6 +463,38 @@ __global__ void __launch_bounds__(256) u1d_rowseg_paths(KernelArgs a) {
                                          : r * per_row + static_cast<int64_t>(s) * a.extent + u;
     store_as<M>(a.out, a.out_dtype, where, acc);
   }
+}
+
+// u1d_generic_wave for buffers that all hold the math type: per batch row the channels 64 at a time, all paths for each
+// (walk_paths), then the butterfly over the lanes.
+template <typename M, int N>
+__global__ void __launch_bounds__(256) u1d_reduce_paths(KernelArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int64_t wid = static_cast<int64_t>(blockIdx.x) * 4 + wv;
+  if (wid >= a.out_rows * a.out_nseg) return;
+  const int64_t r = wid / a.out_nseg;
+  const int s = static_cast<int>(wid - r * a.out_nseg);
+  int64_t z0, z1;
+  z_range<M>(a, r, z0, z1);
+  const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
+  __shared__ GlobalRow<M> srow_all[4][kMaxBuffers + 1];
+  GlobalRow<M>* srow = srow_all[wv];
+  M acc = 0;
+  if (p0 < p1) {
+    for (int64_t zz = z0; zz < z1; ++zz) {
+      const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
+      if (lane == kMaxBuffers) srow[kMaxBuffers] = pointer_to_one<M>();
+      row_pointers<M>(a, z, lane, srow);
+      for (int u0 = 0; u0 < a.extent; u0 += 64) {  // (at least once: the extent is at least 1)
+        const int u = u0 + lane;
+        acc = walk_paths<M, N, true>(a.rows, p0, p1, u < a.extent ? u : a.extent - 1, u < a.extent, u == 0, srow, acc);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 64);
+  if (lane == 0) store_as<M>(a.out, a.out_dtype, wid, acc);
 }
 
 // One wavefront per scalar output element (row, segment): lanes stride over the channel
@@ -494,31 +509,9 @@ __global__ void __launch_bounds__(256) u1d_generic_wave(KernelArgs a) {
   int64_t z0, z1;
   z_range<M>(a, r, z0, z1);
   const int p0 = a.seg_start[s], p1 = a.seg_start[s + 1];
-  __shared__ GlobalRow<M> srow_all[4][kMaxBuffers];
-  GlobalRow<M>* srow = srow_all[wid & 3];
   M acc = 0;
   for (int64_t zz = z0; zz < z1; ++zz) {
     const int64_t z = (a.out_mode == CUEQ_BATCH_INDEXED) ? a.csr_perm[zz] : zz;
-    if (a.same_type) {  // the same sums in the same order, the paths read as packed rows
-      row_pointers<M>(a, z, lane, srow);
-      PathRow next = load_path_row(a.rows, p0 < p1 ? p0 : 0);
-      for (int p = p0; p < p1; ++p) {
-        const PathRow cur = next;
-        next = load_path_row(a.rows, p + 1 < p1 ? p + 1 : p);
-        if (cur.channel) {
-          for (int u0 = 0; u0 < a.extent; u0 += 64) {
-            const int u = u0 + lane;
-            const M v = path_product_row<M>(cur, u < a.extent ? u : a.extent - 1, srow);
-            acc += u < a.extent ? v : static_cast<M>(0);
-          }
-        } else {
-          const M v = path_product_row<M>(cur, 0, srow);
-          acc += lane == 0 ? v : static_cast<M>(0);
-        }
-      }
-      __builtin_amdgcn_wave_barrier();
-      continue;
-    }
     for (int p = p0; p < p1; ++p) {
       // a path sums over the channel mode only when one of its inputs carries it; a path of scalars contributes once
       bool has_channel = false;
@@ -893,6 +886,32 @@ extern "C" int64_t cueq_u1d_workspace_size(const cueq_u1d_plan* plan, const cueq
   return need;
 }
 
+// The kernels with a fixed operand count, as functors over the count.
+struct RowsegPaths {
+  template <typename M, int N>
+  static void launch(dim3 grid, hipStream_t stream, const KernelArgs& a) {
+    hipLaunchKernelGGL((u1d_rowseg_paths<M, N>), grid, dim3(256), 0, stream, a);
+  }
+};
+struct ReducePaths {
+  template <typename M, int N>
+  static void launch(dim3 grid, hipStream_t stream, const KernelArgs& a) {
+    hipLaunchKernelGGL((u1d_reduce_paths<M, N>), grid, dim3(256), 0, stream, a);
+  }
+};
+template <typename M, typename K>
+static void launch_by_operands(int most, dim3 grid, hipStream_t stream, const KernelArgs& a) {
+  switch (most) {
+    case 1: K::template launch<M, 1>(grid, stream, a); break;
+    case 2: K::template launch<M, 2>(grid, stream, a); break;
+    case 3: K::template launch<M, 3>(grid, stream, a); break;
+    case 4: K::template launch<M, 4>(grid, stream, a); break;
+    case 5: K::template launch<M, 5>(grid, stream, a); break;
+    case 6: K::template launch<M, 6>(grid, stream, a); break;
+    default: K::template launch<M, 7>(grid, stream, a); break;
+  }
+}
+
 template <typename M>
 static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, int64_t batch, void* workspace,
                      int64_t workspace_bytes, hipStream_t stream) {
@@ -993,16 +1012,12 @@ static int run_typed(const cueq_u1d_plan* plan, const cueq_u1d_buffer* buffers, 
       CUEQ_REQUIRE(rblocks < (int64_t(1) << 31), CUEQ_ERR_TOO_LARGE, "output %d too large for one launch", ob);
       const dim3 rgrid(static_cast<unsigned>(rblocks));
       if (!a.same_type) hipLaunchKernelGGL(u1d_generic_rowseg<M>, rgrid, dim3(256), 0, stream, a);
-      else switch (t.max_nin) {
-        case 1: hipLaunchKernelGGL((u1d_rowseg_paths<M, 1>), rgrid, dim3(256), 0, stream, a); break;
-        case 2: hipLaunchKernelGGL((u1d_rowseg_paths<M, 2>), rgrid, dim3(256), 0, stream, a); break;
-        case 3: hipLaunchKernelGGL((u1d_rowseg_paths<M, 3>), rgrid, dim3(256), 0, stream, a); break;
-        case 4: hipLaunchKernelGGL((u1d_rowseg_paths<M, 4>), rgrid, dim3(256), 0, stream, a); break;
-        case 5: hipLaunchKernelGGL((u1d_rowseg_paths<M, 5>), rgrid, dim3(256), 0, stream, a); break;
-        case 6: hipLaunchKernelGGL((u1d_rowseg_paths<M, 6>), rgrid, dim3(256), 0, stream, a); break;
-        default: hipLaunchKernelGGL((u1d_rowseg_paths<M, 7>), rgrid, dim3(256), 0, stream, a); break;
-      }
-    } else if (wave) hipLaunchKernelGGL(u1d_generic_wave<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+      else launch_by_operands<M, RowsegPaths>(t.max_nin, rgrid, stream, a);
+    } else if (wave) {
+      const dim3 wgrid(static_cast<unsigned>(blocks));
+      if (!a.same_type) hipLaunchKernelGGL(u1d_generic_wave<M>, wgrid, dim3(256), 0, stream, a);
+      else launch_by_operands<M, ReducePaths>(t.max_nin, wgrid, stream, a);
+    }
     else hipLaunchKernelGGL(u1d_generic_elem<M>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
     CUEQ_CHECK_HIP(hipGetLastError());
     if (nchunks > 1) {
