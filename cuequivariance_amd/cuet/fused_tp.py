@@ -11,10 +11,13 @@ Here two executors stand behind the same interface:
 
 * the matrix-core executor (``cuet/dense.py``) for what the high-level layers produce - one operation ``uv,iu,iv``
   (Linear) or ``uvw,iu,jv,kw`` with ``v = 1`` (fully connected product), weights shared over the batch, no index tensors;
-* everything else - the other contraction forms, several operations, per-sample or indexed operands - on the
+* the same executor behind an element-wise stage (``_MatrixWithElementwiseStage``) for the other forms with a matrix shape
+  and shared weights: ``u_v_uvw_w`` with any ``v`` and ``u_u_uw_w`` (the products of the two row operands first, then their
+  Linear map), ``u_v_uv_u`` and ``u_v_uv_v`` (the Linear map of one row operand first, then its product with the other);
+* everything else - element-wise and outer products, several operations, per-sample or indexed operands - on the
   uniform-1d kernels: every operation is flattened down to one channel mode (the last mode of its output, split to a
   common extent), which keeps gathers and scatters inside the kernels.  Correct for all the reference's forms, generated
-  straight-line kernels at first use; these forms are element-wise / outer products without a matrix-core shape.
+  straight-line kernels at first use.
 """
 
 from __future__ import annotations
@@ -65,6 +68,151 @@ class _FlattenedOperation(nn.Module):
         if self.f is None:
             self.f = self._build()
         return self.f(inputs, input_indices=input_indices, output_shapes=output_shapes, output_indices=output_indices)
+
+
+class _MatrixWithElementwiseStage(nn.Module):
+    """One 4-operand operation whose weights (the input with two or three modes) are shared over the batch, as a Linear map
+    on the matrix-core executor and an element-wise stage; ``W`` stands for the weights, ``a`` and ``b`` for the two row
+    operands in the order of the inputs, the names of the modes are free:
+
+    * ``W[x y o], a[x], b[y] -> out[o]`` (``u_v_uvw_w``) and ``W[c o], a[c], b[c] -> out[o]`` (``u_u_uw_w``): the products
+      ``P[z, (x, y)] = a[z, x] b[z, y]`` (or ``a[z, c] b[z, c]``) per distinct pair of segments, formed by broadcasting,
+      then ``out = P W`` with ``W`` read as the ``(x y) x o`` matrix it is in memory - the paths and coefficients of the
+      operation become those of a Linear map.  ``P`` has ``x y`` values per pair and row: the rows are worked on in
+      pieces that keep it under 1 GiB.
+    * ``W[m0 m1], a, b -> out`` with one row operand carrying the contracted mode and the other the mode of the output
+      (``u_v_uv_u``, ``u_v_uv_v``): ``T = g W`` (or ``g W^T``: the weights are gathered into that order first) per distinct
+      (weight segment, segment of ``g``), then ``out += c e * T`` on the uniform-1d kernels.
+
+    Everything between the stages is differentiable torch code; 2-byte inputs are computed in float32.  Raises
+    ``NotImplementedError`` when the operation has none of these shapes."""
+
+    def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype, name: str):
+        super().__init__()
+        import numpy as np
+
+        from .dense import SegmentedPolynomialDense
+
+        if len(polynomial.operations) != 1 or polynomial.num_inputs != 3 or polynomial.num_outputs != 1:
+            raise NotImplementedError("one operation with three inputs and one output")
+        ope, stp = polynomial.operations[0]
+        if tuple(ope.buffers) != (0, 1, 2, 3) or stp.num_paths == 0:
+            raise NotImplementedError("operands in buffer order")
+        found = None
+        for iw in range(3):
+            sw = stp.subscripts.operands[iw]
+            try:
+                d = stp.flatten_modes([m for m in stp.subscripts.modes() if m not in sw])
+            except ValueError:
+                continue
+            ia, ib = [i for i in range(3) if i != iw]
+            W, a, b, o = (d.subscripts.operands[i] for i in (iw, ia, ib, 3))
+            if len(W) == 3 and o == W[2] and {a, b} == {W[0], W[1]} and a != b:
+                found = ("outer", d, iw, ia, ib, a == W[0])
+            elif len(W) == 2 and a == b == W[0] and o == W[1]:
+                found = ("same", d, iw, ia, ib, True)
+            elif len(W) == 2 and len(a) == len(b) == 1 and {a, b} == {W[0], W[1]} and a != b and o in (a, b):
+                g, e = (ia, ib) if o == b else (ib, ia)  # g carries the contracted mode, e the mode of the output
+                found = ("after", d, iw, g, e, d.subscripts.operands[g] == W[0])
+            if found:
+                break
+        if found is None:
+            raise NotImplementedError(f"no matrix shape with shared weights in {stp.subscripts}")
+        self.kind, d, self.iw, self.i1, self.i2, self.flag = found
+        self.size = [o.size for o in d.operands]
+        offs = [o.segment_offsets() for o in d.operands]
+        lin = cue.SegmentedTensorProduct.from_subscripts("uv,u,v")
+        paths = [(p.indices, float(p.coefficients)) for p in d.paths if float(p.coefficients) != 0.0]
+        if not paths:
+            raise NotImplementedError("no path with a coefficient")
+        self.w_gather = None
+        if self.kind in ("outer", "same"):
+            for seg in d.operands[self.iw]:
+                lin.add_segment(0, (int(np.prod(seg[:-1])), seg[-1]))
+            pairs = sorted({(idx[self.i1], idx[self.i2]) for idx, _ in paths})
+            # pairs of one shape are formed together: (first columns of a, of b, their extents, how many pairs)
+            groups, where = {}, {}
+            for pa, pb in pairs:
+                groups.setdefault((d.operands[self.i1][pa][0], d.operands[self.i2][pb][0]), []).append((pa, pb))
+            self.groups = []
+            for (na, nb), members in sorted(groups.items()):
+                for pa, pb in members:
+                    where[(pa, pb)] = lin.add_segment(1, (na * nb if self.kind == "outer" else na,))
+                self.groups.append((torch.tensor([[offs[self.i1][pa] + k for k in range(na)] for pa, _ in members]),
+                                    torch.tensor([[offs[self.i2][pb] + k for k in range(nb)] for _, pb in members])))
+            for seg in d.operands[3]:
+                lin.add_segment(2, tuple(seg))
+            for idx, c in paths:
+                lin.add_path(idx[self.iw], where[(idx[self.i1], idx[self.i2])], idx[3], c=c)
+            self.after = None
+        else:
+            transposed = not self.flag  # the weights lie (output mode, contracted mode): gathered into the other order
+            if transposed:
+                gather = np.arange(self.size[self.iw])
+                for seg, off in zip(d.operands[self.iw], offs[self.iw]):
+                    gather[off:off + seg[0] * seg[1]] = off + np.arange(seg[0] * seg[1]).reshape(seg[0], seg[1]).T.reshape(-1)
+                self.w_gather = torch.from_numpy(gather)
+            for seg in d.operands[self.iw]:
+                lin.add_segment(0, (seg[1], seg[0]) if transposed else tuple(seg))
+            for seg in d.operands[self.i1]:
+                lin.add_segment(1, tuple(seg))
+            uses = sorted({(idx[self.iw], idx[self.i1]) for idx, _ in paths})
+            el = cue.SegmentedTensorProduct.from_subscripts("u,u,u")
+            for seg in d.operands[self.i2]:
+                el.add_segment(0, tuple(seg))
+            for t, (pw, pg) in enumerate(uses):
+                n = lin.operands[0][pw][1]
+                lin.add_segment(2, (n,))
+                el.add_segment(1, (n,))
+                lin.add_path(pw, pg, t, c=1.0)
+            for seg in d.operands[3]:
+                el.add_segment(2, tuple(seg))
+            for idx, c in paths:
+                el.add_path(idx[self.i2], uses.index((idx[self.iw], idx[self.i1])), idx[3], c=c)
+            self.groups = []
+            self.after = _FlattenedOperation(
+                cue.SegmentedPolynomial([el.operands[0], el.operands[1]], [el.operands[2]], [(cue.Operation([0, 1, 2]), el)]), math_dtype)
+        self.p_size = lin.operands[1].size
+        self.linear = SegmentedPolynomialDense(
+            cue.SegmentedPolynomial([lin.operands[0], lin.operands[1]], [lin.operands[2]], [(cue.Operation([0, 1, 2]), lin)]),
+            math_dtype, None, name)
+        self._on_device: dict = {}
+
+    def _tables(self, device):
+        t = self._on_device.get(device)
+        if t is None:
+            t = self._on_device[device] = ([(ga.to(device), gb.to(device)) for ga, gb in self.groups],
+                                           None if self.w_gather is None else self.w_gather.to(device))
+        return t
+
+    def forward(self, inputs: List[torch.Tensor]) -> torch.Tensor:
+        if inputs[0].dtype in (torch.bfloat16, torch.float16):
+            inputs = [t.float() for t in inputs]
+        w, x1, x2 = inputs[self.iw], inputs[self.i1], inputs[self.i2]
+        groups, w_gather = self._tables(w.device)
+        Z = max(x1.shape[0], x2.shape[0])
+        if self.kind == "after":
+            if w_gather is not None:
+                w = w[:, w_gather]
+            t = self.linear([w, x1.contiguous()], {}, {}, {})[0]
+            return self.after([x2, t], {}, {}, {})[0]
+        step = max(1, (1 << 30) // max(1, self.p_size * w.element_size()))
+        outs = []
+        for z0 in range(0, Z, step):
+            a = x1 if x1.shape[0] == 1 else x1[z0:z0 + step]
+            b = x2 if x2.shape[0] == 1 else x2[z0:z0 + step]
+            rows = min(step, Z - z0)
+            parts = []
+            for ga, gb in groups:
+                if self.kind == "same":
+                    prod = a[:, ga] * b[:, gb]
+                elif self.flag:  # the mode of a comes first in the weights
+                    prod = a[:, ga][:, :, :, None] * b[:, gb][:, :, None, :]
+                else:
+                    prod = b[:, gb][:, :, :, None] * a[:, ga][:, :, None, :]
+                parts.append(prod.expand(rows, *prod.shape[1:]).reshape(rows, -1))
+            outs.append(self.linear([w, parts[0] if len(parts) == 1 else torch.cat(parts, 1)], {}, {}, {})[0])
+        return outs[0] if len(outs) == 1 else torch.cat(outs, 0)
 
 
 def _permute_inputs(polynomial: cue.SegmentedPolynomial, perm) -> cue.SegmentedPolynomial:
@@ -122,6 +270,13 @@ class SegmentedPolynomialFusedTP(nn.Module):
                     break
                 except NotImplementedError:
                     continue
+        # the other forms with a matrix shape: a Linear map on the same executor and an element-wise stage
+        self.composed = None
+        if self.dense is None and rows != "mul_ir":
+            try:
+                self.composed = _MatrixWithElementwiseStage(polynomial, math_dtype, name)
+            except NotImplementedError:
+                self.composed = None
         if rows == "mul_ir" and self.dense is None:
             raise NotImplementedError("fused_tp: rows='mul_ir' is served by the matrix-core executor only")
         # one flattened executor per operation: (module, input buffers it reads, output it adds to)
@@ -161,6 +316,14 @@ class SegmentedPolynomialFusedTP(nn.Module):
                 and inputs[self.dense_perm[0]].shape[0] == 1 and inputs[0].dtype in (torch.float32, torch.float64, torch.bfloat16, torch.float16)
                 and all(t.dtype == inputs[0].dtype for t in inputs)):
             return self.dense([inputs[i] for i in self.dense_perm], input_indices, output_shapes, output_indices)
+        if (self.composed is not None and not input_indices and not output_indices and not output_shapes and inputs[0].is_cuda
+                and inputs[self.composed.iw].shape[0] == 1 and inputs[0].dtype in (torch.float32, torch.float64, torch.bfloat16, torch.float16)
+                and all(t.dtype == inputs[0].dtype for t in inputs)
+                and len({t.shape[0] for i, t in enumerate(inputs) if i != self.composed.iw} - {1}) <= 1):
+            out = self.composed(inputs)
+            src = self.dtypes[self.num_inputs]
+            dtype = (self.math_dtype or torch.float32) if src < 0 else inputs[src].dtype
+            return [out if out.dtype == dtype else out.to(dtype)]
         if self._rows_orig == "mul_ir":
             raise NotImplementedError("fused_tp: rows='mul_ir' takes shared weights, no index tensors and one dtype for all inputs")
         device = inputs[0].device

@@ -361,9 +361,10 @@ class FullyConnectedTensorProduct(torch.nn.Module):
         self.method = _method_from_fallback(method, use_fallback, "fused_tp")
         self.f_per_sample = _FlattenedUniform(e.polynomial, math_dtype)  # weights of shape (batch, weight_numel)
         self.f = SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
-        if getattr(self.f.m, "dense", True) is None:
-            # the matrix-core executor takes a second operand of multiplicity one; others run on the uniform-1d kernels of
-            # the flattened descriptor, with the weight row shared by the batch
+        if getattr(self.f.m, "dense", True) is None and getattr(self.f.m, "composed", None) is None:
+            # the matrix-core executor takes a second operand of multiplicity one directly, any other behind a stage that
+            # forms the products of the two operands; what neither takes runs on the uniform-1d kernels of the flattened
+            # descriptor, with the weight row shared by the batch
             self.f = None
         # mul_ir rows of the first operand and of the output taken as they lie by the generated fused kernels (no
         # transposition pass) when those kernels serve the call; everything else keeps the passes
@@ -378,17 +379,6 @@ class FullyConnectedTensorProduct(torch.nn.Module):
                                                                [(mul, ir.dim) for mul, ir in e.outputs[0].irreps])})
             except (NotImplementedError, ValueError):
                 self.f_rows = None
-        # A second operand of V invariant scalars ("10x0e" node attributes): the product is the Linear map of the
-        # features x1[i, u] * x2[v] (multiplicity u * V) with the very same weights - same paths, same weight layout
-        # (u, v, w) = (u * V + v, w), same coefficients - and runs on the dense 3-operand kernels.
-        self.f_outer, self._outer_segments = None, None
-        if self.f is None and len(irreps_in2) == 1 and irreps_in2[0].ir.is_scalar() and irreps_in2[0].mul > 1:
-            V = irreps_in2[0].mul
-            big = cue.Irreps(irreps_in1.irrep_class, [(mul * V, ir) for mul, ir in irreps_in1])
-            lin = descriptors.linear(big, irreps_out)
-            if lin.polynomial.inputs[0].size == self.weight_numel:
-                self.f_outer = SegmentedPolynomial(lin.polynomial, method=self.method, math_dtype=math_dtype)
-                self._outer_segments = [(ir.dim, mul) for mul, ir in irreps_in1]
 
     def extra_repr(self) -> str:
         return (
@@ -422,12 +412,6 @@ class FullyConnectedTensorProduct(torch.nn.Module):
                 {} if indices_out is None else {0: torch.empty(size_out, 1, device="meta")},
                 {} if indices_out is None else {0: indices_out})
             return apply_layout(self.transpose_out, out[0])
-        if self.f_outer is not None and weight.shape[0] == 1:
-            Z, off, parts = x1.shape[0], 0, []
-            for d, u in self._outer_segments:  # ir_mul rows: (component, channel) -> (component, channel * V + v)
-                parts.append((x1[:, off:off + d * u].reshape(Z, d, u, 1) * x2.reshape(x2.shape[0], 1, 1, -1)).reshape(Z, -1))
-                off += d * u
-            return apply_layout(self.transpose_out, self.f_outer([weight, torch.cat(parts, 1)])[0])
         if weight.shape[0] != 1 or self.f is None:
             return apply_layout(self.transpose_out, self.f_per_sample([weight, x1, x2])[0])
         return apply_layout(self.transpose_out, self.f([weight, x1, x2])[0])

@@ -39,12 +39,15 @@ def rel_err(got, ref):
     return (got.detach().cpu().double() - ref.double()).abs().max().item() / max(ref.abs().max().item(), 1e-30)
 
 
-def check(device, poly, inputs, dtype, input_indices=None, output_shapes=None, output_indices=None, expect_dense=None):
+def check(device, poly, inputs, dtype, input_indices=None, output_shapes=None, output_indices=None, expect_dense=None,
+          expect_stages=None):
     from cuequivariance_amd import cuet
 
     m = cuet.SegmentedPolynomial(poly, method="fused_tp", math_dtype=dtype)
     if expect_dense is not None:
         assert (m.m.dense is not None) == expect_dense
+    if expect_stages is not None:
+        assert (m.m.composed.kind if m.m.composed is not None else None) == expect_stages
     spec = spec_from_polynomial(poly)
     a = [t.clone().requires_grad_(True) for t in inputs]
     sizes = {k: v.shape[0] for k, v in (output_shapes or {}).items()}
@@ -74,6 +77,84 @@ def test_every_reference_form(device, form, dtype):
     Z = 37
     inputs = [torch.randn(Z, o.size, dtype=torch.float64, generator=g).to(dtype) for o in poly.inputs]
     check(device, poly, inputs, dtype)
+
+
+STAGED = {"u,v,uvw,w": "outer", "u,u,uw,w": "same", "u,v,uv,u": "after", "u,v,uv,v": "after",
+          "v,u,uvw,w": "outer", "v,u,uv,u": "after"}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("shared_row", [None, 0, 1])
+@pytest.mark.parametrize("form", sorted(STAGED))
+def test_forms_with_a_matrix_shape_run_on_the_matrix_cores_when_the_weights_are_shared(device, form, shared_row, dtype):
+    """The weights (the operand with two or three modes) as one row: a Linear map on the matrix-core executor with an
+    element-wise stage before or after it, not the flattened uniform-1d kernels - also with the two row operands in the other
+    order, and with one of them shared over the batch as well.  Results and all three gradients against the oracle."""
+    d = random_stp(form, seed=3 + sum(map(ord, form)), nseg=3)
+    poly = cue.SegmentedPolynomial.eval_last_operand(d)
+    g = torch.Generator().manual_seed(5)
+    Z = 203
+    rows = [Z, Z, 1]
+    if shared_row is not None:
+        rows[shared_row] = 1
+    inputs = [torch.randn(r, o.size, dtype=torch.float64, generator=g).to(dtype) for r, o in zip(rows, poly.inputs)]
+    check(device, poly, inputs, dtype, expect_dense=False, expect_stages=STAGED[form])
+
+
+@pytest.mark.gpu
+def test_fully_connected_product_of_general_multiplicities(device):
+    """``cuet.FullyConnectedTensorProduct`` with a second operand of multiplicity above one (``uvw,iu,jv,kw`` as it comes from
+    the descriptor, mixed multiplicities), float32 and bfloat16, against the oracle in float64 (bfloat16: on the rounded
+    inputs, 2e-2): runs as products of the two operands followed by a Linear map.  Rows in ``mul_ir`` against the same
+    module in ``ir_mul`` on transposed rows; rows in pieces when the products of all rows would not fit 1 GiB."""
+    from cuequivariance_amd import cuet
+    from cuequivariance_amd.cuet.fused_tp import _MatrixWithElementwiseStage
+
+    i1, i2, io = cue.Irreps("O3", "32x0e+16x1o"), cue.Irreps("O3", "8x0e+8x1o"), cue.Irreps("O3", "32x0e+32x1o+16x1e")
+    e = cue.descriptors.fully_connected_tensor_product(i1, i2, io)
+    m = cuet.FullyConnectedTensorProduct(i1, i2, io, layout=cue.ir_mul, shared_weights=True, internal_weights=False, device=device)
+    assert isinstance(m.f.m.composed, _MatrixWithElementwiseStage) and m.f.m.composed.kind == "outer"
+    g = torch.Generator().manual_seed(8)
+    Z = 300
+    x1, x2 = torch.randn(Z, i1.dim, generator=g), torch.randn(Z, i2.dim, generator=g)
+    w = torch.randn(1, m.weight_numel, generator=g)
+    cot = torch.randn(Z, io.dim, generator=g)
+    spec = spec_from_polynomial(e.polynomial)
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)):
+        b = [t.to(dtype).to(device).requires_grad_(True) for t in (w, x1, x2)]
+        a = [t.detach().cpu().double().requires_grad_(True) for t in b]
+        ref = naive_segmented_polynomial(spec, a)[0]
+        c = cot.to(dtype)
+        ref_grads = torch.autograd.grad(ref, a, c.double())
+        got = m(b[1], b[2], b[0])
+        assert got.dtype == dtype and rel_err(got, ref.detach()) <= tol, (dtype, rel_err(got, ref.detach()))
+        grads = torch.autograd.grad(got, b, c.to(device))
+        for g_, r_ in zip(grads, ref_grads):
+            assert rel_err(g_, r_) <= tol, (dtype, rel_err(g_, r_))
+    # mul_ir rows
+    mm = cuet.FullyConnectedTensorProduct(i1, i2, io, layout=cue.mul_ir, shared_weights=True, internal_weights=False, device=device)
+    to_mul_ir = [cuet.TransposeIrrepsLayout(ir, source=cue.ir_mul, target=cue.mul_ir, device=device) for ir in (i1, i2, io)]
+    x1d, x2d, wd = x1.to(device), x2.to(device), w.to(device)
+    got = mm(to_mul_ir[0](x1d), to_mul_ir[1](x2d), wd)
+    assert rel_err(got, to_mul_ir[2](m(x1d, x2d, wd)).cpu()) <= 1e-6
+    # traced as a whole: the stages are torch code around the opaque operators of the matrix-core executor
+    compiled = torch.compile(m, fullgraph=True)
+    xg = [t.clone().requires_grad_(True) for t in (x1d, x2d, wd)]
+    out_c = compiled(xg[0], xg[1], xg[2])
+    assert rel_err(out_c, m(x1d, x2d, wd).cpu()) <= 1e-6
+    gc = torch.autograd.grad(out_c, xg, cot.to(device))
+    xe = [t.clone().requires_grad_(True) for t in (x1d, x2d, wd)]
+    ge = torch.autograd.grad(m(xe[0], xe[1], xe[2]), xe, cot.to(device))
+    for g_, r_ in zip(gc, ge):
+        assert rel_err(g_, r_.cpu()) <= 1e-5
+    # rows in pieces
+    st = m.f.m.composed
+    rows = (1 << 30) // (st.p_size * 4) + 77
+    x1d, x2d = torch.randn(rows, i1.dim, device=device), torch.randn(rows, i2.dim, device=device)
+    whole = m(x1d, x2d, wd)
+    tail = m(x1d[-100:], x2d[-100:], wd)
+    assert whole.shape == (rows, io.dim) and rel_err(whole[-100:], tail.cpu()) <= 1e-6
 
 
 @pytest.mark.gpu
