@@ -173,6 +173,8 @@ class _MatrixWithElementwiseStage(nn.Module):
             self.after = _FlattenedOperation(
                 cue.SegmentedPolynomial([el.operands[0], el.operands[1]], [el.operands[2]], [(cue.Operation([0, 1, 2]), el)]), math_dtype)
         self.p_size = lin.operands[1].size
+        # what the flattened operation would have to walk per row: one scalar path per contracted index of every path
+        self.scalar_paths = sum(lin.operands[0][p.indices[0]][0] for p in lin.paths)
         self.linear = SegmentedPolynomialDense(
             cue.SegmentedPolynomial([lin.operands[0], lin.operands[1]], [lin.operands[2]], [(cue.Operation([0, 1, 2]), lin)]),
             math_dtype, None, name)
@@ -270,7 +272,11 @@ class SegmentedPolynomialFusedTP(nn.Module):
                     break
                 except NotImplementedError:
                     continue
-        # the other forms with a matrix shape: a Linear map on the same executor and an element-wise stage
+        # the other forms with a matrix shape: a Linear map on the same executor and an element-wise stage, taken when the
+        # flattened operation would have `stages_from` scalar paths or more (small multiplicities are one cheap launch of a
+        # generated uniform-1d kernel; beyond a few thousand paths that kernel takes minutes to compile and the matrix
+        # cores are far ahead)
+        self.stages_from = 2048
         self.composed = None
         if self.dense is None and rows != "mul_ir":
             try:
@@ -316,7 +322,7 @@ class SegmentedPolynomialFusedTP(nn.Module):
                 and inputs[self.dense_perm[0]].shape[0] == 1 and inputs[0].dtype in (torch.float32, torch.float64, torch.bfloat16, torch.float16)
                 and all(t.dtype == inputs[0].dtype for t in inputs)):
             return self.dense([inputs[i] for i in self.dense_perm], input_indices, output_shapes, output_indices)
-        if (self.composed is not None and not input_indices and not output_indices and not output_shapes and inputs[0].is_cuda
+        if (self.composed is not None and self.composed.scalar_paths >= self.stages_from and not input_indices and not output_indices and not output_shapes and inputs[0].is_cuda
                 and inputs[self.composed.iw].shape[0] == 1 and inputs[0].dtype in (torch.float32, torch.float64, torch.bfloat16, torch.float16)
                 and all(t.dtype == inputs[0].dtype for t in inputs)
                 and len({t.shape[0] for i, t in enumerate(inputs) if i != self.composed.iw} - {1}) <= 1):

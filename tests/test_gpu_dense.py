@@ -398,6 +398,7 @@ def test_fully_connected_with_scalar_attributes_matches_oracle(device, dtype, la
     i1, i2, i3 = cue.Irreps("O3", "16x0e+16x1o+8x0e"), cue.Irreps("O3", "5x0e"), cue.Irreps("O3", "16x0e+8x1o")
     m = cuet.FullyConnectedTensorProduct(i1, i2, i3, layout=layout, internal_weights=False)
     assert m.f is not None and m.f.m.dense is None and m.f.m.composed.kind == "outer"
+    m.f.m.stages_from = 0  # (these small multiplicities would otherwise take the flattened operation)
     g = torch.Generator().manual_seed(13)
     Z = 45
     ins = [torch.randn(1, m.weight_numel, dtype=torch.float64, generator=g), torch.randn(Z, i1.dim, dtype=torch.float64, generator=g),
