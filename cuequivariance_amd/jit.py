@@ -1,7 +1,7 @@
 """Descriptor-specialised kernels at first use.
 
 The library ships straight-line kernels for the descriptors listed in ``codegen/registry.py``; every other descriptor
-would run on the table-driven kernels, which are tens of times slower.  Unless this module is switched off
+would run on the table-driven kernels, which are twenty to a hundred times slower on large workloads.  Unless this module is switched off
 (``CUEQ_AMD_JIT=0`` in the environment, or ``enable(False)``), the first plan of a descriptor that has no specialised
 kernels yet generates a translation unit - the same kind the build generates for channel-wise products
 (``codegen/channelwise.py``) and symmetric contractions (``codegen/symmetric.py``), a general straight-line one
