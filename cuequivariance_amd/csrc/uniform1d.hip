@@ -2,8 +2,10 @@
 //
 // A plan regroups the descriptor's paths by (output buffer, output segment) and uploads
 // them once.  In the table-driven kernels of this file every output element is owned by one
-// thread (or one wavefront when a scalar output contracts the channel mode), which walks the
-// batch rows that contribute to it and the paths of its segment in a fixed order: no atomics,
+// thread - a lane of a wavefront that works on 64 channels of one output segment, where the output
+// carries at least 32 channels - or by one wavefront when a scalar output contracts the channel
+// mode; the owner walks the batch rows that contribute to it and the paths of its segment in a
+// fixed order (very long rows of an indexed output in pieces that are added in order): no atomics,
 // results are bit-reproducible from run to run.  (The generated channel-wise backward scatters
 // the gradient of a gathered operand with floating-point atomics unless the "deterministic"
 // option is set; everything else there is bit-reproducible too.)
