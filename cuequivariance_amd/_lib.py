@@ -53,6 +53,8 @@ EXPORTED_SYMBOLS = (
     "cueq_linear_dw_mul_ir",
     "cueq_fc_combine",
     "cueq_fc_rowdot",
+    "cueq_outer_rows",
+    "cueq_outer_rows_contract",
     "cueq_gemm_grouped",
     "cueq_segmented_transpose",
     "cueq_layer_norm_t_fwd",
@@ -227,6 +229,10 @@ def load() -> C.CDLL:
         lib.cueq_fc_combine.restype = C.c_int
         lib.cueq_fc_rowdot.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, i32, ptr, i32, i32, ptr]
         lib.cueq_fc_rowdot.restype = C.c_int
+        lib.cueq_outer_rows.argtypes = [i32, i64, ptr, i64, ptr, i64, ptr, i64, ptr, i32, i32, i32, i32, ptr]
+        lib.cueq_outer_rows.restype = C.c_int
+        lib.cueq_outer_rows_contract.argtypes = [i32, i32, i64, ptr, i64, ptr, i64, ptr, i64, ptr, ptr, ptr, i32, i32, i32, i32, ptr]
+        lib.cueq_outer_rows_contract.restype = C.c_int
         lib.cueq_segmented_transpose.argtypes = [i32, i64, i64, ptr, ptr, ptr, ptr]
         lib.cueq_segmented_transpose.restype = C.c_int
         lib.cueq_layer_norm_t_fwd.argtypes = [i32, i64, i64, ptr, ptr, ptr, f64, ptr, ptr, ptr, ptr]

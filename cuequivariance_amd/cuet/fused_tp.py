@@ -77,9 +77,11 @@ class _MatrixWithElementwiseStage(nn.Module):
 
     * ``W[x y o], a[x], b[y] -> out[o]`` (``u_v_uvw_w``) and ``W[c o], a[c], b[c] -> out[o]`` (``u_u_uw_w``): the products
       ``P[z, (x, y)] = a[z, x] b[z, y]`` (or ``a[z, c] b[z, c]``) per distinct pair of segments, formed by broadcasting,
-      then ``out = P W`` with ``W`` read as the ``(x y) x o`` matrix it is in memory - the paths and coefficients of the
-      operation become those of a Linear map.  ``P`` has ``x y`` values per pair and row: the rows are worked on in
-      pieces that keep it under 1 GiB.
+      then ``out = P W`` with ``W`` read as the ``(x y) x o`` matrix it is in memory.  The paths that add into one output
+      segment become one path of the Linear map (their products side by side, their weight blocks stacked, each times its
+      coefficient: a gather of the weight row), so no two paths write the same columns and the executor sends all paths of one
+      contraction length out in one launch.  ``P`` has ``x y`` values per path and row: the rows are worked on in pieces that
+      keep it under 1 GiB.
     * ``W[m0 m1], a, b -> out`` with one row operand carrying the contracted mode and the other the mode of the output
       (``u_v_uv_u``, ``u_v_uv_v``): ``T = g W`` (or ``g W^T``: the weights are gathered into that order first) per distinct
       (weight segment, segment of ``g``), then ``out += c e * T`` on the uniform-1d kernels.
@@ -125,25 +127,39 @@ class _MatrixWithElementwiseStage(nn.Module):
         paths = [(p.indices, float(p.coefficients)) for p in d.paths if float(p.coefficients) != 0.0]
         if not paths:
             raise NotImplementedError("no path with a coefficient")
-        self.w_gather = None
+        self.w_gather, self.w_scale = None, None
         if self.kind in ("outer", "same"):
-            for seg in d.operands[self.iw]:
-                lin.add_segment(0, (int(np.prod(seg[:-1])), seg[-1]))
-            pairs = sorted({(idx[self.i1], idx[self.i2]) for idx, _ in paths})
-            # pairs of one shape are formed together: (first columns of a, of b, their extents, how many pairs)
-            groups, where = {}, {}
-            for pa, pb in pairs:
-                groups.setdefault((d.operands[self.i1][pa][0], d.operands[self.i2][pb][0]), []).append((pa, pb))
-            self.groups = []
-            for (na, nb), members in sorted(groups.items()):
-                for pa, pb in members:
-                    where[(pa, pb)] = lin.add_segment(1, (na * nb if self.kind == "outer" else na,))
-                self.groups.append((torch.tensor([[offs[self.i1][pa] + k for k in range(na)] for pa, _ in members]),
-                                    torch.tensor([[offs[self.i2][pb] + k for k in range(nb)] for _, pb in members])))
+            # The paths that add into one output segment are one product: out[:, c] = [P_1 | P_2 | ...] [c_1 W_1; c_2 W_2; ...]
+            # (their products side by side, their weight blocks stacked, each times its coefficient), so the Linear map has one
+            # path per output segment, no two of them write the same columns, and all of one contraction length go out in one
+            # table-driven launch.  Products are formed together per shape (extent of a, extent of b): with mixed shapes an
+            # output segment has one such path per shape.
+            by_shape = {}
+            for idx, c in paths:
+                na, nb = d.operands[self.i1][idx[self.i1]][0], d.operands[self.i2][idx[self.i2]][0]
+                by_shape.setdefault((na, nb), {}).setdefault(idx[3], []).append((idx, c))
             for seg in d.operands[3]:
                 lin.add_segment(2, tuple(seg))
-            for idx, c in paths:
-                lin.add_path(idx[self.iw], where[(idx[self.i1], idx[self.i2])], idx[3], c=c)
+            self.groups, gather, scale = [], [], []
+            self.parts, cursor = [], 0  # (kind "outer": every product as (offset in a, in b, in P, extent of a, of b), in the order of P)
+            for (na, nb), by_out in sorted(by_shape.items()):
+                k = na * nb if self.kind == "outer" else na
+                rows_a, rows_b = [], []
+                for out_seg, members in sorted(by_out.items()):
+                    n = d.operands[3][out_seg][0]
+                    sw = lin.add_segment(0, (k * len(members), n))
+                    sp = lin.add_segment(1, (k * len(members),))
+                    lin.add_path(sw, sp, out_seg, c=1.0)
+                    for idx, c in members:
+                        rows_a.append([offs[self.i1][idx[self.i1]] + t for t in range(na)])
+                        rows_b.append([offs[self.i2][idx[self.i2]] + t for t in range(nb)])
+                        self.parts.append((offs[self.i1][idx[self.i1]], offs[self.i2][idx[self.i2]], cursor, na, nb))
+                        cursor += k
+                        gather.append(offs[self.iw][idx[self.iw]] + np.arange(k * n))
+                        scale.append(np.full(k * n, c))
+                self.groups.append((torch.tensor(rows_a), torch.tensor(rows_b)))
+            self.w_gather = torch.from_numpy(np.concatenate(gather))
+            self.w_scale = torch.from_numpy(np.concatenate(scale))
             self.after = None
         else:
             transposed = not self.flag  # the weights lie (output mode, contracted mode): gathered into the other order
@@ -184,26 +200,55 @@ class _MatrixWithElementwiseStage(nn.Module):
         t = self._on_device.get(device)
         if t is None:
             t = self._on_device[device] = ([(ga.to(device), gb.to(device)) for ga, gb in self.groups],
-                                           None if self.w_gather is None else self.w_gather.to(device))
+                                           None if self.w_gather is None else self.w_gather.to(device),
+                                           None if self.w_scale is None else self.w_scale.to(device))
+        return t
+
+    def outer_tables(self, device):
+        """Device tables of ``cueq_outer_rows`` / ``cueq_outer_rows_contract`` for the products of this stage: the parts, and
+        per row operand the parts that read each of its segments (in the order of P: the order the sums take)."""
+        key = ("outer", device)
+        t = self._on_device.get(key)
+        if t is None:
+            parts = torch.tensor(self.parts, dtype=torch.int32)
+            lists = []
+            for col in (0, 1):  # segments of a, of b
+                by_seg = {}
+                for q, part in enumerate(self.parts):
+                    by_seg.setdefault(part[col], []).append(q)
+                start, members = [0], []
+                for _, qs in sorted(by_seg.items()):
+                    members += qs
+                    start.append(len(members))
+                lists.append((torch.tensor(start, dtype=torch.int32).to(device), torch.tensor(members, dtype=torch.int32).to(device),
+                              len(start) - 1, max(self.parts[qs[0]][3 + col] for qs in by_seg.values())))
+            vec = all(v % 4 == 0 for part in self.parts for v in part)
+            t = self._on_device[key] = (parts.to(device), len(self.parts), max(na * nb for _, _, _, na, nb in self.parts), lists, vec)
         return t
 
     def forward(self, inputs: List[torch.Tensor]) -> torch.Tensor:
         if inputs[0].dtype in (torch.bfloat16, torch.float16):
             inputs = [t.float() for t in inputs]
         w, x1, x2 = inputs[self.iw], inputs[self.i1], inputs[self.i2]
-        groups, w_gather = self._tables(w.device)
+        groups, w_gather, w_scale = self._tables(w.device)
         Z = max(x1.shape[0], x2.shape[0])
         if self.kind == "after":
             if w_gather is not None:
                 w = w[:, w_gather]
             t = self.linear([w, x1.contiguous()], {}, {}, {})[0]
             return self.after([x2, t], {}, {}, {})[0]
+        w = w[:, w_gather] * w_scale.to(w.dtype)  # the weight blocks of every path, stacked per output segment, times the coefficients
         step = max(1, (1 << 30) // max(1, self.p_size * w.element_size()))
         outs = []
         for z0 in range(0, Z, step):
             a = x1 if x1.shape[0] == 1 else x1[z0:z0 + step]
             b = x2 if x2.shape[0] == 1 else x2[z0:z0 + step]
             rows = min(step, Z - z0)
+            if self.kind == "outer" and not (torch.compiler.is_compiling() or torch.jit.is_tracing()):
+                # (the kernels of csrc/outer_rows.hip; a traced graph keeps the torch code below)
+                prod = _OuterRows.apply(self, a.expand(rows, -1), b.expand(rows, -1))
+                outs.append(self.linear([w, prod], {}, {}, {})[0])
+                continue
             parts = []
             for ga, gb in groups:
                 if self.kind == "same":
@@ -215,6 +260,76 @@ class _MatrixWithElementwiseStage(nn.Module):
                 parts.append(prod.expand(rows, *prod.shape[1:]).reshape(rows, -1))
             outs.append(self.linear([w, parts[0] if len(parts) == 1 else torch.cat(parts, 1)], {}, {}, {})[0])
         return outs[0] if len(outs) == 1 else torch.cat(outs, 0)
+
+
+def _outer_launch(st: "_MatrixWithElementwiseStage", a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    from .. import _lib
+
+    a, b = a.contiguous(), b.contiguous()
+    rows = a.shape[0]
+    parts, nparts, max_part, _, vec = st.outer_tables(a.device)
+    out = torch.empty(rows, st.p_size, dtype=a.dtype, device=a.device)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.load().cueq_outer_rows(
+            _lib.F64 if a.dtype == torch.float64 else _lib.F32, rows, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), out.data_ptr(),
+            out.stride(0), parts.data_ptr(), nparts, max_part, 1 if st.flag else 0, 1 if vec else 0,
+            torch.cuda.current_stream(a.device).cuda_stream), "cueq_outer_rows")
+    return out
+
+
+def _contract_launch(st: "_MatrixWithElementwiseStage", which: int, q: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    from .. import _lib
+
+    q, x = q.contiguous(), x.contiguous()
+    rows = q.shape[0]
+    parts, _, _, lists, vec = st.outer_tables(q.device)
+    start, members, nsegs, max_extent = lists[which]
+    out = torch.zeros(rows, st.size[st.i1 if which == 0 else st.i2], dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().cueq_outer_rows_contract(
+            _lib.F64 if q.dtype == torch.float64 else _lib.F32, which, rows, q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0),
+            out.data_ptr(), out.stride(0), parts.data_ptr(), start.data_ptr(), members.data_ptr(), nsegs, max_extent,
+            1 if st.flag else 0, 1 if vec else 0, torch.cuda.current_stream(q.device).cuda_stream), "cueq_outer_rows_contract")
+    return out
+
+
+class _OuterRows(torch.autograd.Function):
+    """``P = a (x) b`` per part (``cueq_outer_rows``).  Its gradients are the two contractions of ``_ContractRows``, whose
+    gradients are this product and the other contraction: derivatives of any order stay on the three kernels."""
+
+    @staticmethod
+    def forward(ctx, st, a, b):
+        ctx.st = st
+        ctx.save_for_backward(a, b)
+        return _outer_launch(st, a.detach(), b.detach())
+
+    @staticmethod
+    def backward(ctx, g):
+        a, b = ctx.saved_tensors
+        return (None, _ContractRows.apply(ctx.st, 0, g, b) if ctx.needs_input_grad[1] else None,
+                _ContractRows.apply(ctx.st, 1, g, a) if ctx.needs_input_grad[2] else None)
+
+
+class _ContractRows(torch.autograd.Function):
+    """``which = 0``: ``out[z, u] = sum_p sum_v q[z, p, u, v] x[z, v]`` (``x`` in the place of ``b``); ``which = 1``: the sum over
+    ``u`` with ``x`` in the place of ``a`` (``cueq_outer_rows_contract``)."""
+
+    @staticmethod
+    def forward(ctx, st, which, q, x):
+        ctx.st, ctx.which = st, which
+        ctx.save_for_backward(q, x)
+        return _contract_launch(st, which, q.detach(), x.detach())
+
+    @staticmethod
+    def backward(ctx, c):
+        q, x = ctx.saved_tensors
+        st, which = ctx.st, ctx.which
+        gq = gx = None
+        if ctx.needs_input_grad[2]:
+            gq = _OuterRows.apply(st, c, x) if which == 0 else _OuterRows.apply(st, x, c)
+        if ctx.needs_input_grad[3]:
+            gx = _ContractRows.apply(st, 1 - which, q, c)
+        return None, None, gq, gx
 
 
 def _permute_inputs(polynomial: cue.SegmentedPolynomial, perm) -> cue.SegmentedPolynomial:

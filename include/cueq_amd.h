@@ -230,6 +230,28 @@ int cueq_fc_combine(int32_t dtype, int32_t t_dtype, int64_t rows, const void* S,
 int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, const void* X, int64_t ldx, const void* G, int64_t ldg, void* D,
                    int64_t ldd, int32_t n2, const void* uses, int32_t num_uses, int32_t vectorised, void* stream);
 
+/* Element-wise stage of the fully connected contraction with a second operand of any multiplicity (form u_v_uvw_w of
+ * FusedTensorProductOp4, primitives/segmented_polynomial_fused_tp.py:40-48, list of forms :114-129): the row-wise outer
+ * products of operand segments, which a Linear map (cueq_gemm_table / cueq_gemm_nt) then contracts with the weights read as
+ * (u v) x w matrices, and the two contractions that are its gradients.  parts: device array of nparts records
+ * {int32 a_off, b_off, p_off, na, nb} (element offsets inside a row of A, B, P; extents of the two segments).
+ *   cueq_outer_rows:           P[z, p_off + u * nb + v] = A[z, a_off + u] * B[z, b_off + v]   (a_major != 0)
+ *                              P[z, p_off + v * na + u] = the same product                    (a_major == 0)
+ *   cueq_outer_rows_contract:  which == 0:  O[z, a_off + u] = sum over the parts p of the segment and v of P[z, ..] * X[z, b_off_p + v]
+ *                              which == 1:  O[z, b_off + v] = sum over the parts p of the segment and u of P[z, ..] * X[z, a_off_p + u]
+ * Segments (of A for which == 0, of B for which == 1): seg_start (device, nsegs + 1 entries) delimits, in seg_parts (device),
+ * the parts that read the segment; they are added in that order.  Columns of O outside the listed segments are not written.
+ * max_part: the largest na * nb; max_extent: the largest extent of a listed segment (they size the grids).  Row strides in
+ * elements; a row stride of 0 reads one row for every z.  dtype: float32 or float64 (all tensors).
+ * vectorised != 0: the caller states that every offset and every extent of the fast index of P (nb if a_major, else na) in
+ * the table is a multiple of four (then, with matching row strides and pointers, a thread moves four adjacent elements at a
+ * time).  The three operations are closed under differentiation: the gradients of each are the other two. */
+int cueq_outer_rows(int32_t dtype, int64_t rows, const void* A, int64_t lda, const void* B, int64_t ldb, void* P, int64_t ldp,
+                    const void* parts, int32_t nparts, int32_t max_part, int32_t a_major, int32_t vectorised, void* stream);
+int cueq_outer_rows_contract(int32_t dtype, int32_t which, int64_t rows, const void* Q, int64_t ldq, const void* X, int64_t ldx, void* O,
+                             int64_t ldo, const void* parts, const int32_t* seg_start, const int32_t* seg_parts, int32_t nsegs,
+                             int32_t max_extent, int32_t a_major, int32_t vectorised, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* triangle multiplicative update: the stages behind                           */
 /*   cuequivariance_torch/cuequivariance_torch/primitives/triangle.py:138-262   */

@@ -104,6 +104,46 @@ def test_forms_with_a_matrix_shape_run_on_the_matrix_cores_when_the_weights_are_
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("dims", [dict(u=8, v=4, w=16), dict(u=5, v=3, w=8), dict(u=16, v=12, w=8)])
+@pytest.mark.parametrize("form", ["u,v,uvw,w", "v,u,uvw,w"])
+def test_outer_product_kernels_against_their_definition(device, form, dims, dtype):
+    """``cueq_outer_rows`` and the two ``cueq_outer_rows_contract`` sums through the C ABI against the same sums written with
+    index arithmetic in float64 - both orders of the two indices in P, extents that are and are not multiples of four (the
+    vector and the scalar kernels), segments read by several parts.  float64 1e-13, float32 1e-5 of the largest value."""
+    from cuequivariance_amd.cuet.fused_tp import _MatrixWithElementwiseStage, _contract_launch, _outer_launch
+
+    saved = dict(DIMS)
+    DIMS.update(dims)
+    try:
+        d = random_stp(form, seed=17, nseg=3)
+    finally:
+        DIMS.clear()
+        DIMS.update(saved)
+    st = _MatrixWithElementwiseStage(cue.SegmentedPolynomial.eval_last_operand(d), dtype, "t")
+    assert st.kind == "outer" and len(st.parts) > 3
+    g = torch.Generator().manual_seed(6)
+    Z = 77
+    a = torch.randn(Z, st.size[st.i1], dtype=torch.float64, generator=g)
+    b = torch.randn(Z, st.size[st.i2], dtype=torch.float64, generator=g)
+    q = torch.randn(Z, st.p_size, dtype=torch.float64, generator=g)
+    P = torch.zeros(Z, st.p_size, dtype=torch.float64)
+    ca, cb = torch.zeros_like(a), torch.zeros_like(b)
+    for a_off, b_off, p_off, na, nb in st.parts:
+        x, y = a[:, a_off:a_off + na], b[:, b_off:b_off + nb]
+        block = x[:, :, None] * y[:, None, :] if st.flag else y[:, :, None] * x[:, None, :]
+        P[:, p_off:p_off + na * nb] = block.reshape(Z, -1)
+        qb = q[:, p_off:p_off + na * nb].reshape(Z, na, nb) if st.flag else q[:, p_off:p_off + na * nb].reshape(Z, nb, na).transpose(1, 2)
+        ca[:, a_off:a_off + na] += (qb * y[:, None, :]).sum(2)
+        cb[:, b_off:b_off + nb] += (qb * x[:, :, None]).sum(1)
+    tol = 1e-13 if dtype == torch.float64 else 1e-5
+    ad, bd, qd = (t.to(dtype).to(device) for t in (a, b, q))
+    assert rel_err(_outer_launch(st, ad, bd), P) <= tol
+    assert rel_err(_contract_launch(st, 0, qd, bd), ca) <= tol
+    assert rel_err(_contract_launch(st, 1, qd, ad), cb) <= tol
+
+
+@pytest.mark.gpu
 def test_fully_connected_product_of_general_multiplicities(device):
     """``cuet.FullyConnectedTensorProduct`` with a second operand of multiplicity above one (``uvw,iu,jv,kw`` as it comes from
     the descriptor, mixed multiplicities), float32 and bfloat16, against the oracle in float64 (bfloat16: on the rounded
