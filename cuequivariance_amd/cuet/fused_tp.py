@@ -237,6 +237,8 @@ class _MatrixWithElementwiseStage(nn.Module):
                 w = w[:, w_gather]
             t = self.linear([w, x1.contiguous()], {}, {}, {})[0]
             return self.after([x2, t], {}, {}, {})[0]
+        if Z == 0:  # (no rows: nothing to launch; the result still hangs on the inputs)
+            return x1.new_zeros((0, self.size[3])) + 0 * (x1.sum() + x2.sum() + w.sum())
         w = w[:, w_gather] * w_scale.to(w.dtype)  # the weight blocks of every path, stacked per output segment, times the coefficients
         step = max(1, (1 << 30) // max(1, self.p_size * w.element_size()))
         outs = []

@@ -189,6 +189,12 @@ def test_fully_connected_product_of_general_multiplicities(device):
     ge = torch.autograd.grad(m(xe[0], xe[1], xe[2]), xe, cot.to(device))
     for g_, r_ in zip(gc, ge):
         assert rel_err(g_, r_.cpu()) <= 1e-5
+    # no rows at all
+    e1, e2 = torch.zeros(0, i1.dim, device=device, requires_grad=True), torch.zeros(0, i2.dim, device=device)
+    we = wd.clone().requires_grad_(True)
+    empty = m(e1, e2, we)
+    assert empty.shape == (0, io.dim)
+    assert all(float(g_.abs().sum()) == 0.0 for g_ in torch.autograd.grad(empty.sum(), [e1, we]))
     # rows in pieces
     st = m.f.m.composed
     rows = (1 << 30) // (st.p_size * 4) + 77
