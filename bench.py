@@ -248,26 +248,28 @@ def secondary(torch, cue, cuet, _lib, dev, wl: str, dtype_name, steps: int, warm
         # a fully connected product whose second operand has multiplicity above one (no BASELINE config; sizes chosen here): the
         # products of the two operands in HBM, then a Linear map on the matrix cores
         Z = 50_000
+        dtype = getattr(torch, _DTYPES[dtype_name])
         i1, i2 = cue.Irreps("O3", "64x0e+64x1o"), cue.Irreps("O3", "16x0e+16x1o")
         m = cuet.FullyConnectedTensorProduct(i1, i2, i1, layout=cue.ir_mul, internal_weights=False)
         g = torch.Generator(device=dev).manual_seed(0)
-        x1 = torch.randn(Z, i1.dim, device=dev, generator=g, requires_grad=True)
-        x2 = torch.randn(Z, i2.dim, device=dev, generator=g, requires_grad=True)
-        w = torch.randn(1, m.weight_numel, device=dev, generator=g, requires_grad=True)
-        cot = torch.randn(Z, i1.dim, device=dev, generator=g)
+        x1 = torch.randn(Z, i1.dim, device=dev, generator=g).to(dtype).requires_grad_(True)
+        x2 = torch.randn(Z, i2.dim, device=dev, generator=g).to(dtype).requires_grad_(True)
+        w = torch.randn(1, m.weight_numel, device=dev, generator=g).to(dtype).requires_grad_(True)
+        cot = torch.randn(Z, i1.dim, device=dev, generator=g).to(dtype)
 
         def step():
             return torch.autograd.grad(m(x1, x2, w), [w, x1, x2], cot)
 
-        unit, units, dt = "rows/s", Z, "f32"
-        # every distinct element once: fwd reads x1, x2 and writes out; bwd reads x1, x2, g and writes dx1, dx2 (weights 655360 = 2.6 MB)
-        alg = {"fwd": Z * (256 + 64 + 256) * 4, "bwd": Z * (256 + 64 + 256 + 256 + 64) * 4}
+        unit, units, dt = "rows/s", Z, _DT_NAME[str(dtype).replace("torch.", "")]
+        es = 4 if dtype == torch.float32 else 2
+        # every distinct element once: fwd reads x1, x2 and writes out; bwd reads x1, x2, g and writes dx1, dx2 (weights 655360 elements)
+        alg = {"fwd": Z * (256 + 64 + 256) * es, "bwd": Z * (256 + 64 + 256 + 256 + 64) * es}
         # 10 flattened paths, each a (64 * 16) x 64 contraction per row; forward, product gradient and weight gradient contract each once
         f = 2 * Z * 64 * 16 * 64 * 10
         flops = {"fwd": f, "bwd": 2 * f}
         flop_roof, flop_peak = "mfma", MFMA_PEAK[dt]
         desc = ("next row (the general fully connected form u_v_uvw_w): FullyConnectedTensorProduct 64x0e+64x1o (x) 16x0e+16x1o -> "
-                "64x0e+64x1o, batch 50000, shared weights, fwd + bwd (dw, dx1, dx2); products of the two operands in HBM (10240 floats per "
+                "64x0e+64x1o, batch 50000, shared weights, fwd + bwd (dw, dx1, dx2); products of the two operands in HBM (10240 values per "
                 "row), then a Linear map on the matrix cores")
     elif wl == "cfg2sh":
         # configs[1] with the spherical harmonics of the edge vectors evaluated inside the edge kernels (the step before the
@@ -763,7 +765,7 @@ def main() -> int:
         for key, wl, dn in (("cfg1_fp32", "cfg1", None), ("cfg3_fp32", "cfg3", None), ("cfg3_bf16_io", "cfg3", "bf16"), ("cfg4_linear_fp32", "cfg4", "fp32"),
                             ("cfg4_linear_bf16", "cfg4", "bf16"), ("cfg4_linear_fp32_mul_ir", "cfg4mi", "fp32"),
                             ("cfg4_linear_bf16_mul_ir", "cfg4mi", "bf16"), ("cfg4_fc_fp32", "cfg4fc", "fp32"), ("cfg4_fc_bf16", "cfg4fc", "bf16"), ("cfg4_fc_fp32_mul_ir", "cfg4fcmi", "fp32"),
-                            ("cfg4_fc_bf16_mul_ir", "cfg4fcmi", "bf16"), ("fc_general_fp32", "fcgen", "fp32"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
+                            ("cfg4_fc_bf16_mul_ir", "cfg4fcmi", "bf16"), ("fc_general_fp32", "fcgen", "fp32"), ("fc_general_bf16", "fcgen", "bf16"), ("fc_conv_rows_fp32", "fcconv", "fp32"), ("cfg2_fp32_harmonics_in_kernels", "cfg2sh", "fp32"),
                             ("cfg5_bf16", "cfg5", "bf16"), ("cfg5_fp16", "cfg5", "fp16"), ("cfg5_fp32", "cfg5", "fp32"),
                             ("cfg4_linear_fp16", "cfg4", "fp16"), ("cfg4_fc_fp16", "cfg4fc", "fp16")):
             add(key, lambda wl=wl, dn=dn: _compact(secondary(torch, cue, cuet, _lib, dev, wl, dn, ssteps, swarm)))

@@ -7,7 +7,8 @@
 //   contract 1: O[z, seg_off + v] = sum over the parts p of the segment, in list order, and u of P[z, ..] * X[z, a_off_p + u]
 // The three are closed under differentiation (each one's gradients are the other two), so the stage is differentiable to any
 // order on these kernels.  All of them are bound by the bytes of P: every element is written, or read, once; sums run in a
-// fixed order (no atomics).
+// fixed order (no atomics).  Elements of float64, float32, bfloat16 or half; the 2-byte types are multiplied and summed in
+// float32 and rounded once.
 
 #include "common.h"
 #include "cw_common.h"
@@ -19,16 +20,58 @@ struct OuterPart {
   int32_t a_off, b_off, p_off, na, nb;
 };
 
+// Element access: T is the type in memory (float, double, or the bits of a bfloat16 / half), Math<T> the type the products
+// and sums are formed in (the same, or float for the 2-byte types: widened on load, rounded once on store).
 template <typename T>
-struct Vec4;
-template <>
-struct Vec4<float> {
-  typedef float4 type;
+struct Math {
+  typedef T type;
 };
 template <>
-struct Vec4<double> {
-  typedef double4 type;
+struct Math<uint16_t> {
+  typedef float type;
 };
+template <>
+struct Math<f16bits> {
+  typedef float type;
+};
+template <typename T>
+__device__ __forceinline__ typename Math<T>::type ld1(const T* p) {
+  if constexpr (sizeof(T) == 2) return mm_widen<T>(*reinterpret_cast<const uint16_t*>(p));
+  else return *p;
+}
+template <typename T>
+__device__ __forceinline__ void st1(T* p, typename Math<T>::type v) {
+  if constexpr (sizeof(T) == 2) *reinterpret_cast<uint16_t*>(p) = mm_round<T>(v);
+  else *p = v;
+}
+// four adjacent elements (p on a boundary of four elements)
+template <typename T>
+__device__ __forceinline__ void ld4(const T* p, typename Math<T>::type (&v)[4]) {
+  if constexpr (sizeof(T) == 2) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    v[0] = mm_widen<T>(static_cast<uint16_t>(w.x & 0xffffu)), v[1] = mm_widen<T>(static_cast<uint16_t>(w.x >> 16));
+    v[2] = mm_widen<T>(static_cast<uint16_t>(w.y & 0xffffu)), v[3] = mm_widen<T>(static_cast<uint16_t>(w.y >> 16));
+  } else if constexpr (sizeof(T) == 4) {
+    const float4 w = *reinterpret_cast<const float4*>(p);
+    v[0] = w.x, v[1] = w.y, v[2] = w.z, v[3] = w.w;
+  } else {
+    const double4 w = *reinterpret_cast<const double4*>(p);
+    v[0] = w.x, v[1] = w.y, v[2] = w.z, v[3] = w.w;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void st4(T* p, const typename Math<T>::type (&v)[4]) {
+  if constexpr (sizeof(T) == 2) {
+    uint2 w;
+    w.x = static_cast<uint32_t>(mm_round<T>(v[0])) | (static_cast<uint32_t>(mm_round<T>(v[1])) << 16);
+    w.y = static_cast<uint32_t>(mm_round<T>(v[2])) | (static_cast<uint32_t>(mm_round<T>(v[3])) << 16);
+    *reinterpret_cast<uint2*>(p) = w;
+  } else if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+    *reinterpret_cast<double4*>(p) = make_double4(v[0], v[1], v[2], v[3]);
+  }
+}
 
 // One part per blockIdx.y; a thread makes V adjacent elements of P for one row (V = 4: the fast index has an extent that is a
 // multiple of four and every offset and row stride is too).
@@ -46,15 +89,15 @@ __global__ void __launch_bounds__(256) outer_rows_kernel(const T* __restrict__ A
     const T* slow = AMAJOR ? A + z * lda + part.a_off : B + z * ldb + part.b_off;
     const T* fast = AMAJOR ? B + z * ldb + part.b_off : A + z * lda + part.a_off;
     T* out = P + z * ldp + part.p_off + static_cast<int64_t>(s) * fast_n + f;
-    const T x = slow[s];
+    const typename Math<T>::type x = ld1<T>(slow + s);
     if constexpr (V == 4) {
-      typedef typename Vec4<T>::type V4;
-      const V4 y = *reinterpret_cast<const V4*>(fast + f);
-      V4 r;
-      r.x = x * y.x, r.y = x * y.y, r.z = x * y.z, r.w = x * y.w;
-      *reinterpret_cast<V4*>(out) = r;
+      typename Math<T>::type y[4];
+      ld4<T>(fast + f, y);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) y[k] *= x;
+      st4<T>(out, y);
     } else {
-      out[0] = x * fast[f];
+      st1<T>(out, x * ld1<T>(fast + f));
     }
   }
 }
@@ -78,7 +121,8 @@ __global__ void __launch_bounds__(256) outer_contract_kernel(const T* __restrict
   for (int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; t < total; t += static_cast<int64_t>(gridDim.x) * 256) {
     const int64_t z = t / n;
     const int i = static_cast<int>(t - z * n);
-    T acc = 0;
+    typedef typename Math<T>::type MT;
+    MT acc = 0;
     for (int q = q0; q < q1; ++q) {
       const OuterPart part = parts[seg_parts[q]];
       const int m = WHICH == 0 ? part.nb : part.na;  // extent of the contracted index
@@ -87,23 +131,22 @@ __global__ void __launch_bounds__(256) outer_contract_kernel(const T* __restrict
       if constexpr (kContractedIsFast) {
         p += static_cast<int64_t>(i) * m;
         if constexpr (V == 4) {
-          typedef typename Vec4<T>::type V4;
           for (int k = 0; k < m; k += 4) {
-            const V4 a = *reinterpret_cast<const V4*>(p + k), b = *reinterpret_cast<const V4*>(x + k);
-            acc += a.x * b.x;
-            acc += a.y * b.y;
-            acc += a.z * b.z;
-            acc += a.w * b.w;
+            MT a[4], b[4];
+            ld4<T>(p + k, a);
+            ld4<T>(x + k, b);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc += a[e] * b[e];
           }
         } else {
-          for (int k = 0; k < m; ++k) acc += p[k] * x[k];
+          for (int k = 0; k < m; ++k) acc += ld1<T>(p + k) * ld1<T>(x + k);
         }
       } else {
         p += i;  // the threads of a wavefront read adjacent elements
-        for (int k = 0; k < m; ++k) acc += p[static_cast<int64_t>(k) * n] * x[k];
+        for (int k = 0; k < m; ++k) acc += ld1<T>(p + static_cast<int64_t>(k) * n) * ld1<T>(x + k);
       }
     }
-    O[z * ldo + seg_off + i] = acc;
+    st1<T>(O + z * ldo + seg_off + i, acc);
   }
 }
 
@@ -125,12 +168,12 @@ using namespace cueq;
 extern "C" int cueq_outer_rows(int32_t dtype, int64_t rows, const void* A, int64_t lda, const void* B, int64_t ldb, void* P, int64_t ldp,
                                const void* parts, int32_t nparts, int32_t max_part, int32_t a_major, int32_t vectorised, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(dtype == CUEQ_F32 || dtype == CUEQ_F64, CUEQ_ERR_UNSUPPORTED, "outer_rows: float32 or float64");
+  CUEQ_REQUIRE(dtype == CUEQ_F32 || dtype == CUEQ_F64 || dtype == CUEQ_BF16 || dtype == CUEQ_F16, CUEQ_ERR_UNSUPPORTED, "outer_rows: unknown dtype");
   CUEQ_REQUIRE(rows >= 0 && nparts >= 0 && nparts < 65536 && max_part >= 0 && lda >= 0 && ldb >= 0 && ldp >= 0, CUEQ_ERR_INVALID,
                "outer_rows: negative extent, or 65 536 parts and more");
   if (rows == 0 || nparts == 0 || max_part == 0) return CUEQ_OK;
   CUEQ_REQUIRE(A && B && P && parts, CUEQ_ERR_INVALID, "outer_rows: null operand");
-  const int es = dtype == CUEQ_F64 ? 8 : 4;
+  const int es = dtype_size(dtype);
   const bool vec = vectorised != 0 && rows_aligned(A, lda, es) && rows_aligned(B, ldb, es) && rows_aligned(P, ldp, es);
   const dim3 grid(grid_for(rows * (max_part / (vec ? 4 : 1))), static_cast<unsigned>(nparts));
   KernelTimer timer("outer_rows", stream);
@@ -140,7 +183,9 @@ extern "C" int cueq_outer_rows(int32_t dtype, int64_t rows, const void* A, int64
 #define BY_ORDER(T, V) do { if (a_major) LAUNCH(T, V, true); else LAUNCH(T, V, false); } while (0)
 #define BY_VEC(T) do { if (vec) BY_ORDER(T, 4); else BY_ORDER(T, 1); } while (0)
   if (dtype == CUEQ_F32) BY_VEC(float);
-  else BY_VEC(double);
+  else if (dtype == CUEQ_F64) BY_VEC(double);
+  else if (dtype == CUEQ_BF16) BY_VEC(uint16_t);
+  else BY_VEC(f16bits);
 #undef BY_VEC
 #undef BY_ORDER
 #undef LAUNCH
@@ -152,13 +197,13 @@ extern "C" int cueq_outer_rows_contract(int32_t dtype, int32_t which, int64_t ro
                                         void* O, int64_t ldo, const void* parts, const int32_t* seg_start, const int32_t* seg_parts,
                                         int32_t nsegs, int32_t max_extent, int32_t a_major, int32_t vectorised, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  CUEQ_REQUIRE(dtype == CUEQ_F32 || dtype == CUEQ_F64, CUEQ_ERR_UNSUPPORTED, "outer_rows_contract: float32 or float64");
+  CUEQ_REQUIRE(dtype == CUEQ_F32 || dtype == CUEQ_F64 || dtype == CUEQ_BF16 || dtype == CUEQ_F16, CUEQ_ERR_UNSUPPORTED, "outer_rows_contract: unknown dtype");
   CUEQ_REQUIRE(which == 0 || which == 1, CUEQ_ERR_INVALID, "outer_rows_contract: which is 0 (sum over the index of b) or 1 (of a)");
   CUEQ_REQUIRE(rows >= 0 && nsegs >= 0 && nsegs < 65536 && max_extent >= 0 && ldq >= 0 && ldx >= 0 && ldo >= 0, CUEQ_ERR_INVALID,
                "outer_rows_contract: negative extent, or 65 536 segments and more");
   if (rows == 0 || nsegs == 0 || max_extent == 0) return CUEQ_OK;
   CUEQ_REQUIRE(Q && X && O && parts && seg_start && seg_parts, CUEQ_ERR_INVALID, "outer_rows_contract: null operand");
-  const int es = dtype == CUEQ_F64 ? 8 : 4;
+  const int es = dtype_size(dtype);
   const bool fast = (which == 0) == (a_major != 0);
   const bool vec = fast && vectorised != 0 && rows_aligned(Q, ldq, es) && rows_aligned(X, ldx, es);
   const dim3 grid(grid_for(rows * max_extent), static_cast<unsigned>(nsegs));
@@ -177,7 +222,9 @@ extern "C" int cueq_outer_rows_contract(int32_t dtype, int32_t which, int64_t ro
     else LAUNCH(T, 1, 1, false);                           \
   } while (0)
   if (dtype == CUEQ_F32) BY_SHAPE(float);
-  else BY_SHAPE(double);
+  else if (dtype == CUEQ_F64) BY_SHAPE(double);
+  else if (dtype == CUEQ_BF16) BY_SHAPE(uint16_t);
+  else BY_SHAPE(f16bits);
 #undef BY_SHAPE
 #undef LAUNCH
   CUEQ_CHECK_HIP(hipGetLastError());

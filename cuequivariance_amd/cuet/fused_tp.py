@@ -86,7 +86,8 @@ class _MatrixWithElementwiseStage(nn.Module):
       (``u_v_uv_u``, ``u_v_uv_v``): ``T = g W`` (or ``g W^T``: the weights are gathered into that order first) per distinct
       (weight segment, segment of ``g``), then ``out += c e * T`` on the uniform-1d kernels.
 
-    Everything between the stages is differentiable torch code; 2-byte inputs are computed in float32.  Raises
+    Everything between the stages is differentiable; 2-byte inputs stay 2-byte tensors on the first form (products and sums
+    in float32, every tensor rounded once) and are computed in float32 on the others.  Raises
     ``NotImplementedError`` when the operation has none of these shapes."""
 
     def __init__(self, polynomial: cue.SegmentedPolynomial, math_dtype, name: str):
@@ -227,7 +228,10 @@ class _MatrixWithElementwiseStage(nn.Module):
         return t
 
     def forward(self, inputs: List[torch.Tensor]) -> torch.Tensor:
-        if inputs[0].dtype in (torch.bfloat16, torch.float16):
+        traced = torch.compiler.is_compiling() or torch.jit.is_tracing()
+        if inputs[0].dtype in (torch.bfloat16, torch.float16) and (self.kind != "outer" or traced):
+            # (2-byte inputs stay what they are on the product kernels and the matrix cores only: products and sums in float32,
+            # every tensor rounded once; the stages in torch code are computed in float32 throughout)
             inputs = [t.float() for t in inputs]
         w, x1, x2 = inputs[self.iw], inputs[self.i1], inputs[self.i2]
         groups, w_gather, w_scale = self._tables(w.device)
@@ -239,14 +243,15 @@ class _MatrixWithElementwiseStage(nn.Module):
             return self.after([x2, t], {}, {}, {})[0]
         if Z == 0:  # (no rows: nothing to launch; the result still hangs on the inputs)
             return x1.new_zeros((0, self.size[3])) + 0 * (x1.sum() + x2.sum() + w.sum())
-        w = w[:, w_gather] * w_scale.to(w.dtype)  # the weight blocks of every path, stacked per output segment, times the coefficients
+        # the weight blocks of every path, stacked per output segment, times the coefficients (2-byte weights: rounded once)
+        w = (w.float()[:, w_gather] * w_scale.float()).to(w.dtype) if w.dtype in (torch.bfloat16, torch.float16) else w[:, w_gather] * w_scale.to(w.dtype)
         step = max(1, (1 << 30) // max(1, self.p_size * w.element_size()))
         outs = []
         for z0 in range(0, Z, step):
             a = x1 if x1.shape[0] == 1 else x1[z0:z0 + step]
             b = x2 if x2.shape[0] == 1 else x2[z0:z0 + step]
             rows = min(step, Z - z0)
-            if self.kind == "outer" and not (torch.compiler.is_compiling() or torch.jit.is_tracing()):
+            if self.kind == "outer" and not traced:
                 # (the kernels of csrc/outer_rows.hip; a traced graph keeps the torch code below)
                 prod = _OuterRows.apply(self, a.expand(rows, -1), b.expand(rows, -1))
                 outs.append(self.linear([w, prod], {}, {}, {})[0])
@@ -264,6 +269,12 @@ class _MatrixWithElementwiseStage(nn.Module):
         return outs[0] if len(outs) == 1 else torch.cat(outs, 0)
 
 
+def _code(dtype):
+    from .. import _lib
+
+    return {torch.float32: _lib.F32, torch.float64: _lib.F64, torch.bfloat16: _lib.BF16, torch.float16: _lib.F16}[dtype]
+
+
 def _outer_launch(st: "_MatrixWithElementwiseStage", a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     from .. import _lib
 
@@ -273,7 +284,7 @@ def _outer_launch(st: "_MatrixWithElementwiseStage", a: torch.Tensor, b: torch.T
     out = torch.empty(rows, st.p_size, dtype=a.dtype, device=a.device)
     with torch.cuda.device(a.device):
         _lib.check(_lib.load().cueq_outer_rows(
-            _lib.F64 if a.dtype == torch.float64 else _lib.F32, rows, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), out.data_ptr(),
+            _code(a.dtype), rows, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), out.data_ptr(),
             out.stride(0), parts.data_ptr(), nparts, max_part, 1 if st.flag else 0, 1 if vec else 0,
             torch.cuda.current_stream(a.device).cuda_stream), "cueq_outer_rows")
     return out
@@ -289,7 +300,7 @@ def _contract_launch(st: "_MatrixWithElementwiseStage", which: int, q: torch.Ten
     out = torch.zeros(rows, st.size[st.i1 if which == 0 else st.i2], dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
         _lib.check(_lib.load().cueq_outer_rows_contract(
-            _lib.F64 if q.dtype == torch.float64 else _lib.F32, which, rows, q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0),
+            _code(q.dtype), which, rows, q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0),
             out.data_ptr(), out.stride(0), parts.data_ptr(), start.data_ptr(), members.data_ptr(), nsegs, max_extent,
             1 if st.flag else 0, 1 if vec else 0, torch.cuda.current_stream(q.device).cuda_stream), "cueq_outer_rows_contract")
     return out

@@ -242,7 +242,8 @@ int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, const void* X, 
  * Segments (of A for which == 0, of B for which == 1): seg_start (device, nsegs + 1 entries) delimits, in seg_parts (device),
  * the parts that read the segment; they are added in that order.  Columns of O outside the listed segments are not written.
  * max_part: the largest na * nb; max_extent: the largest extent of a listed segment (they size the grids).  Row strides in
- * elements; a row stride of 0 reads one row for every z.  dtype: float32 or float64 (all tensors).
+ * elements; a row stride of 0 reads one row for every z.  dtype (all tensors): float64, float32, or bfloat16 / half with
+ * products and sums in float32, rounded once.
  * vectorised != 0: the caller states that every offset and every extent of the fast index of P (nb if a_major, else na) in
  * the table is a multiple of four (then, with matching row strides and pointers, a thread moves four adjacent elements at a
  * time).  The three operations are closed under differentiation: the gradients of each are the other two. */

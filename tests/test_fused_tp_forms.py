@@ -104,13 +104,15 @@ def test_forms_with_a_matrix_shape_run_on_the_matrix_cores_when_the_weights_are_
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("dims", [dict(u=8, v=4, w=16), dict(u=5, v=3, w=8), dict(u=16, v=12, w=8)])
 @pytest.mark.parametrize("form", ["u,v,uvw,w", "v,u,uvw,w"])
 def test_outer_product_kernels_against_their_definition(device, form, dims, dtype):
     """``cueq_outer_rows`` and the two ``cueq_outer_rows_contract`` sums through the C ABI against the same sums written with
     index arithmetic in float64 - both orders of the two indices in P, extents that are and are not multiples of four (the
-    vector and the scalar kernels), segments read by several parts.  float64 1e-13, float32 1e-5 of the largest value."""
+    vector and the scalar kernels), segments read by several parts.  float64 1e-13, float32 1e-5 of the largest value; bfloat16
+    and half on inputs rounded to the type: products and sums are formed in float32 and rounded once, half a unit in the last
+    place of the largest value (2^-8, 2^-11)."""
     from cuequivariance_amd.cuet.fused_tp import _MatrixWithElementwiseStage, _contract_launch, _outer_launch
 
     saved = dict(DIMS)
@@ -120,13 +122,13 @@ def test_outer_product_kernels_against_their_definition(device, form, dims, dtyp
     finally:
         DIMS.clear()
         DIMS.update(saved)
-    st = _MatrixWithElementwiseStage(cue.SegmentedPolynomial.eval_last_operand(d), dtype, "t")
+    st = _MatrixWithElementwiseStage(cue.SegmentedPolynomial.eval_last_operand(d), torch.float64 if dtype == torch.float64 else torch.float32, "t")
     assert st.kind == "outer" and len(st.parts) > 3
     g = torch.Generator().manual_seed(6)
     Z = 77
-    a = torch.randn(Z, st.size[st.i1], dtype=torch.float64, generator=g)
-    b = torch.randn(Z, st.size[st.i2], dtype=torch.float64, generator=g)
-    q = torch.randn(Z, st.p_size, dtype=torch.float64, generator=g)
+    a = torch.randn(Z, st.size[st.i1], dtype=torch.float64, generator=g).to(dtype).double()
+    b = torch.randn(Z, st.size[st.i2], dtype=torch.float64, generator=g).to(dtype).double()
+    q = torch.randn(Z, st.p_size, dtype=torch.float64, generator=g).to(dtype).double()
     P = torch.zeros(Z, st.p_size, dtype=torch.float64)
     ca, cb = torch.zeros_like(a), torch.zeros_like(b)
     for a_off, b_off, p_off, na, nb in st.parts:
@@ -136,7 +138,7 @@ def test_outer_product_kernels_against_their_definition(device, form, dims, dtyp
         qb = q[:, p_off:p_off + na * nb].reshape(Z, na, nb) if st.flag else q[:, p_off:p_off + na * nb].reshape(Z, nb, na).transpose(1, 2)
         ca[:, a_off:a_off + na] += (qb * y[:, None, :]).sum(2)
         cb[:, b_off:b_off + nb] += (qb * x[:, :, None]).sum(1)
-    tol = 1e-13 if dtype == torch.float64 else 1e-5
+    tol = {torch.float64: 1e-13, torch.float32: 1e-5, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
     ad, bd, qd = (t.to(dtype).to(device) for t in (a, b, q))
     assert rel_err(_outer_launch(st, ad, bd), P) <= tol
     assert rel_err(_contract_launch(st, 0, qd, bd), ca) <= tol
