@@ -73,8 +73,37 @@ __device__ __forceinline__ void st4(T* p, const typename Math<T>::type (&v)[4]) 
   }
 }
 
-// One part per blockIdx.y; a thread makes V adjacent elements of P for one row (V = 4: the fast index has an extent that is a
-// multiple of four and every offset and row stride is too).
+// V adjacent elements (p on a boundary of V elements); V = 8 is for the 2-byte types: one 16-byte access
+template <typename T, int V>
+__device__ __forceinline__ void ldv(const T* p, typename Math<T>::type (&v)[V]) {
+  if constexpr (V == 8) {
+    static_assert(sizeof(T) == 2, "eight elements at a time for 2-byte types only");
+    const uint4 w = *reinterpret_cast<const uint4*>(p);
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = mm_widen<T>(static_cast<uint16_t>(words[k] & 0xffffu));
+      v[2 * k + 1] = mm_widen<T>(static_cast<uint16_t>(words[k] >> 16));
+    }
+  } else {
+    ld4<T>(p, v);
+  }
+}
+template <typename T, int V>
+__device__ __forceinline__ void stv(T* p, const typename Math<T>::type (&v)[V]) {
+  if constexpr (V == 8) {
+    uint32_t words[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      words[k] = static_cast<uint32_t>(mm_round<T>(v[2 * k])) | (static_cast<uint32_t>(mm_round<T>(v[2 * k + 1])) << 16);
+    *reinterpret_cast<uint4*>(p) = make_uint4(words[0], words[1], words[2], words[3]);
+  } else {
+    st4<T>(p, v);
+  }
+}
+
+// One part per blockIdx.y; a thread makes V adjacent elements of P for one row (V = 4 or 8: the fast index has an extent that
+// is a multiple of V and every offset and row stride is too).
 template <typename T, int V, bool AMAJOR>
 __global__ void __launch_bounds__(256) outer_rows_kernel(const T* __restrict__ A, int64_t lda, const T* __restrict__ B, int64_t ldb,
                                                          T* __restrict__ P, int64_t ldp, const OuterPart* __restrict__ parts, int64_t rows) {
@@ -90,12 +119,12 @@ __global__ void __launch_bounds__(256) outer_rows_kernel(const T* __restrict__ A
     const T* fast = AMAJOR ? B + z * ldb + part.b_off : A + z * lda + part.a_off;
     T* out = P + z * ldp + part.p_off + static_cast<int64_t>(s) * fast_n + f;
     const typename Math<T>::type x = ld1<T>(slow + s);
-    if constexpr (V == 4) {
-      typename Math<T>::type y[4];
-      ld4<T>(fast + f, y);
+    if constexpr (V > 1) {
+      typename Math<T>::type y[V];
+      ldv<T, V>(fast + f, y);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) y[k] *= x;
-      st4<T>(out, y);
+      for (int k = 0; k < V; ++k) y[k] *= x;
+      stv<T, V>(out, y);
     } else {
       st1<T>(out, x * ld1<T>(fast + f));
     }
@@ -130,13 +159,13 @@ __global__ void __launch_bounds__(256) outer_contract_kernel(const T* __restrict
       const T* p = Q + z * ldq + part.p_off;
       if constexpr (kContractedIsFast) {
         p += static_cast<int64_t>(i) * m;
-        if constexpr (V == 4) {
-          for (int k = 0; k < m; k += 4) {
-            MT a[4], b[4];
-            ld4<T>(p + k, a);
-            ld4<T>(x + k, b);
+        if constexpr (V > 1) {
+          for (int k = 0; k < m; k += V) {
+            MT a[V], b[V];
+            ldv<T, V>(p + k, a);
+            ldv<T, V>(x + k, b);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc += a[e] * b[e];
+            for (int e = 0; e < V; ++e) acc += a[e] * b[e];
           }
         } else {
           for (int k = 0; k < m; ++k) acc += ld1<T>(p + k) * ld1<T>(x + k);
@@ -157,8 +186,8 @@ static unsigned grid_for(int64_t items) {
   return static_cast<unsigned>(blocks < 1 ? 1 : blocks);
 }
 
-static bool rows_aligned(const void* p, int64_t ld, int es) {
-  return reinterpret_cast<uintptr_t>(p) % (4 * es) == 0 && ld % 4 == 0;
+static bool rows_aligned(const void* p, int64_t ld, int es, int v) {
+  return reinterpret_cast<uintptr_t>(p) % (v * es) == 0 && ld % v == 0;
 }
 
 }  // namespace cueq
@@ -174,18 +203,22 @@ extern "C" int cueq_outer_rows(int32_t dtype, int64_t rows, const void* A, int64
   if (rows == 0 || nparts == 0 || max_part == 0) return CUEQ_OK;
   CUEQ_REQUIRE(A && B && P && parts, CUEQ_ERR_INVALID, "outer_rows: null operand");
   const int es = dtype_size(dtype);
-  const bool vec = vectorised != 0 && rows_aligned(A, lda, es) && rows_aligned(B, ldb, es) && rows_aligned(P, ldp, es);
-  const dim3 grid(grid_for(rows * (max_part / (vec ? 4 : 1))), static_cast<unsigned>(nparts));
+  // vectorised: 0, or the number (4 or 8) that every offset and fast extent of the table is a multiple of
+  const int v = (vectorised >= 8 && es == 2 && rows_aligned(A, lda, es, 8) && rows_aligned(B, ldb, es, 8) && rows_aligned(P, ldp, es, 8)) ? 8
+                : (vectorised >= 4 && rows_aligned(A, lda, es, 4) && rows_aligned(B, ldb, es, 4) && rows_aligned(P, ldp, es, 4)) ? 4 : 1;
+  const dim3 grid(grid_for(rows * (max_part / v)), static_cast<unsigned>(nparts));
   KernelTimer timer("outer_rows", stream);
 #define LAUNCH(T, V, AM)                                                                                                        \
   hipLaunchKernelGGL((outer_rows_kernel<T, V, AM>), grid, dim3(256), 0, stream, static_cast<const T*>(A), lda, static_cast<const T*>(B), \
                      ldb, static_cast<T*>(P), ldp, static_cast<const OuterPart*>(parts), rows)
 #define BY_ORDER(T, V) do { if (a_major) LAUNCH(T, V, true); else LAUNCH(T, V, false); } while (0)
-#define BY_VEC(T) do { if (vec) BY_ORDER(T, 4); else BY_ORDER(T, 1); } while (0)
+#define BY_VEC(T) do { if (v == 4) BY_ORDER(T, 4); else BY_ORDER(T, 1); } while (0)
+#define BY_VEC2(T) do { if (v == 8) BY_ORDER(T, 8); else BY_VEC(T); } while (0)
   if (dtype == CUEQ_F32) BY_VEC(float);
   else if (dtype == CUEQ_F64) BY_VEC(double);
-  else if (dtype == CUEQ_BF16) BY_VEC(uint16_t);
-  else BY_VEC(f16bits);
+  else if (dtype == CUEQ_BF16) BY_VEC2(uint16_t);
+  else BY_VEC2(f16bits);
+#undef BY_VEC2
 #undef BY_VEC
 #undef BY_ORDER
 #undef LAUNCH
@@ -205,26 +238,30 @@ extern "C" int cueq_outer_rows_contract(int32_t dtype, int32_t which, int64_t ro
   CUEQ_REQUIRE(Q && X && O && parts && seg_start && seg_parts, CUEQ_ERR_INVALID, "outer_rows_contract: null operand");
   const int es = dtype_size(dtype);
   const bool fast = (which == 0) == (a_major != 0);
-  const bool vec = fast && vectorised != 0 && rows_aligned(Q, ldq, es) && rows_aligned(X, ldx, es);
+  const int v = !fast ? 1
+                : (vectorised >= 8 && es == 2 && rows_aligned(Q, ldq, es, 8) && rows_aligned(X, ldx, es, 8)) ? 8
+                : (vectorised >= 4 && rows_aligned(Q, ldq, es, 4) && rows_aligned(X, ldx, es, 4)) ? 4 : 1;
   const dim3 grid(grid_for(rows * max_extent), static_cast<unsigned>(nsegs));
   KernelTimer timer("outer_rows_contract", stream);
 #define LAUNCH(T, V, W, AM)                                                                                                        \
   hipLaunchKernelGGL((outer_contract_kernel<T, V, W, AM>), grid, dim3(256), 0, stream, static_cast<const T*>(Q), ldq,            \
                      static_cast<const T*>(X), ldx, static_cast<T*>(O), ldo, static_cast<const OuterPart*>(parts), seg_start, seg_parts, rows)
-#define BY_SHAPE(T)                                        \
+#define BY_SHAPE(T, V8)                                    \
   do {                                                     \
     if (which == 0 && a_major) {                           \
-      if (vec) LAUNCH(T, 4, 0, true);                      \
+      if (v == 8) LAUNCH(T, V8, 0, true);                  \
+      else if (v == 4) LAUNCH(T, 4, 0, true);              \
       else LAUNCH(T, 1, 0, true);                          \
     } else if (which == 0) LAUNCH(T, 1, 0, false);         \
     else if (a_major) LAUNCH(T, 1, 1, true);               \
-    else if (vec) LAUNCH(T, 4, 1, false);                  \
+    else if (v == 8) LAUNCH(T, V8, 1, false);              \
+    else if (v == 4) LAUNCH(T, 4, 1, false);               \
     else LAUNCH(T, 1, 1, false);                           \
   } while (0)
-  if (dtype == CUEQ_F32) BY_SHAPE(float);
-  else if (dtype == CUEQ_F64) BY_SHAPE(double);
-  else if (dtype == CUEQ_BF16) BY_SHAPE(uint16_t);
-  else BY_SHAPE(f16bits);
+  if (dtype == CUEQ_F32) BY_SHAPE(float, 4);
+  else if (dtype == CUEQ_F64) BY_SHAPE(double, 4);
+  else if (dtype == CUEQ_BF16) BY_SHAPE(uint16_t, 8);
+  else BY_SHAPE(f16bits, 8);
 #undef BY_SHAPE
 #undef LAUNCH
   CUEQ_CHECK_HIP(hipGetLastError());

@@ -223,7 +223,7 @@ class _MatrixWithElementwiseStage(nn.Module):
                     start.append(len(members))
                 lists.append((torch.tensor(start, dtype=torch.int32).to(device), torch.tensor(members, dtype=torch.int32).to(device),
                               len(start) - 1, max(self.parts[qs[0]][3 + col] for qs in by_seg.values())))
-            vec = all(v % 4 == 0 for part in self.parts for v in part)
+            vec = 8 if all(v % 8 == 0 for part in self.parts for v in part) else 4 if all(v % 4 == 0 for part in self.parts for v in part) else 0
             t = self._on_device[key] = (parts.to(device), len(self.parts), max(na * nb for _, _, _, na, nb in self.parts), lists, vec)
         return t
 
@@ -285,7 +285,7 @@ def _outer_launch(st: "_MatrixWithElementwiseStage", a: torch.Tensor, b: torch.T
     with torch.cuda.device(a.device):
         _lib.check(_lib.load().cueq_outer_rows(
             _code(a.dtype), rows, a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), out.data_ptr(),
-            out.stride(0), parts.data_ptr(), nparts, max_part, 1 if st.flag else 0, 1 if vec else 0,
+            out.stride(0), parts.data_ptr(), nparts, max_part, 1 if st.flag else 0, vec,
             torch.cuda.current_stream(a.device).cuda_stream), "cueq_outer_rows")
     return out
 
@@ -302,7 +302,7 @@ def _contract_launch(st: "_MatrixWithElementwiseStage", which: int, q: torch.Ten
         _lib.check(_lib.load().cueq_outer_rows_contract(
             _code(q.dtype), which, rows, q.data_ptr(), q.stride(0), x.data_ptr(), x.stride(0),
             out.data_ptr(), out.stride(0), parts.data_ptr(), start.data_ptr(), members.data_ptr(), nsegs, max_extent,
-            1 if st.flag else 0, 1 if vec else 0, torch.cuda.current_stream(q.device).cuda_stream), "cueq_outer_rows_contract")
+            1 if st.flag else 0, vec, torch.cuda.current_stream(q.device).cuda_stream), "cueq_outer_rows_contract")
     return out
 
 

@@ -244,9 +244,9 @@ int cueq_fc_rowdot(int32_t dtype, int32_t g_dtype, int64_t rows, const void* X, 
  * max_part: the largest na * nb; max_extent: the largest extent of a listed segment (they size the grids).  Row strides in
  * elements; a row stride of 0 reads one row for every z.  dtype (all tensors): float64, float32, or bfloat16 / half with
  * products and sums in float32, rounded once.
- * vectorised != 0: the caller states that every offset and every extent of the fast index of P (nb if a_major, else na) in
- * the table is a multiple of four (then, with matching row strides and pointers, a thread moves four adjacent elements at a
- * time).  The three operations are closed under differentiation: the gradients of each are the other two. */
+ * vectorised = 4 or 8: the caller states that every offset and every extent of the fast index of P (nb if a_major, else na) in
+ * the table is a multiple of that number (then, with matching row strides and pointers, a thread moves four adjacent elements
+ * at a time, eight of a 2-byte type); 0: no such statement.  The three operations are closed under differentiation: the gradients of each are the other two. */
 int cueq_outer_rows(int32_t dtype, int64_t rows, const void* A, int64_t lda, const void* B, int64_t ldb, void* P, int64_t ldp,
                     const void* parts, int32_t nparts, int32_t max_part, int32_t a_major, int32_t vectorised, void* stream);
 int cueq_outer_rows_contract(int32_t dtype, int32_t which, int64_t rows, const void* Q, int64_t ldq, const void* X, int64_t ldx, void* O,

@@ -105,7 +105,7 @@ def test_forms_with_a_matrix_shape_run_on_the_matrix_cores_when_the_weights_are_
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32, torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("dims", [dict(u=8, v=4, w=16), dict(u=5, v=3, w=8), dict(u=16, v=12, w=8)])
+@pytest.mark.parametrize("dims", [dict(u=8, v=4, w=16), dict(u=5, v=3, w=8), dict(u=16, v=12, w=8), dict(u=16, v=8, w=8)])
 @pytest.mark.parametrize("form", ["u,v,uvw,w", "v,u,uvw,w"])
 def test_outer_product_kernels_against_their_definition(device, form, dims, dtype):
     """``cueq_outer_rows`` and the two ``cueq_outer_rows_contract`` sums through the C ABI against the same sums written with
