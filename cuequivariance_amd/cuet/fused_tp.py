@@ -81,7 +81,7 @@ class _MatrixWithElementwiseStage(nn.Module):
       segment become one path of the Linear map (their products side by side, their weight blocks stacked, each times its
       coefficient: a gather of the weight row), so no two paths write the same columns and the executor sends all paths of one
       contraction length out in one launch.  ``P`` has ``x y`` values per path and row: the rows are worked on in pieces that
-      keep it under 1 GiB.
+      keep it under 4 GiB (``piece_bytes``).
     * ``W[m0 m1], a, b -> out`` with one row operand carrying the contracted mode and the other the mode of the output
       (``u_v_uv_u``, ``u_v_uv_v``): ``T = g W`` (or ``g W^T``: the weights are gathered into that order first) per distinct
       (weight segment, segment of ``g``), then ``out += c e * T`` on the uniform-1d kernels.
@@ -196,6 +196,9 @@ class _MatrixWithElementwiseStage(nn.Module):
             cue.SegmentedPolynomial([lin.operands[0], lin.operands[1]], [lin.operands[2]], [(cue.Operation([0, 1, 2]), lin)]),
             math_dtype, None, name)
         self._on_device: dict = {}
+        # rows are worked on in pieces whose products take at most this many bytes (large pieces fill the chip better: the
+        # Linear map has few, long contractions)
+        self.piece_bytes = 4 << 30
 
     def _tables(self, device):
         t = self._on_device.get(device)
@@ -245,7 +248,7 @@ class _MatrixWithElementwiseStage(nn.Module):
             return x1.new_zeros((0, self.size[3])) + 0 * (x1.sum() + x2.sum() + w.sum())
         # the weight blocks of every path, stacked per output segment, times the coefficients (2-byte weights: rounded once)
         w = (w.float()[:, w_gather] * w_scale.float()).to(w.dtype) if w.dtype in (torch.bfloat16, torch.float16) else w[:, w_gather] * w_scale.to(w.dtype)
-        step = max(1, (1 << 30) // max(1, self.p_size * w.element_size()))
+        step = max(1, self.piece_bytes // max(1, self.p_size * w.element_size()))
         outs = []
         for z0 in range(0, Z, step):
             a = x1 if x1.shape[0] == 1 else x1[z0:z0 + step]

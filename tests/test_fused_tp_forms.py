@@ -150,7 +150,7 @@ def test_fully_connected_product_of_general_multiplicities(device):
     """``cuet.FullyConnectedTensorProduct`` with a second operand of multiplicity above one (``uvw,iu,jv,kw`` as it comes from
     the descriptor, mixed multiplicities), float32 and bfloat16, against the oracle in float64 (bfloat16: on the rounded
     inputs, 2e-2): runs as products of the two operands followed by a Linear map.  Rows in ``mul_ir`` against the same
-    module in ``ir_mul`` on transposed rows; rows in pieces when the products of all rows would not fit 1 GiB."""
+    module in ``ir_mul`` on transposed rows; rows in pieces when the products of all rows exceed the piece size (lowered here)."""
     from cuequivariance_amd import cuet
     from cuequivariance_amd.cuet.fused_tp import _MatrixWithElementwiseStage
 
@@ -199,7 +199,8 @@ def test_fully_connected_product_of_general_multiplicities(device):
     assert all(float(g_.abs().sum()) == 0.0 for g_ in torch.autograd.grad(empty.sum(), [e1, we]))
     # rows in pieces
     st = m.f.m.composed
-    rows = (1 << 30) // (st.p_size * 4) + 77
+    st.piece_bytes = 64 << 20
+    rows = st.piece_bytes // (st.p_size * 4) + 77
     x1d, x2d = torch.randn(rows, i1.dim, device=device), torch.randn(rows, i2.dim, device=device)
     whole = m(x1d, x2d, wd)
     tail = m(x1d[-100:], x2d[-100:], wd)
