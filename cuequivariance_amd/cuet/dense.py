@@ -60,9 +60,11 @@ def _analyse(polynomial: cue.SegmentedPolynomial):
         if not (len(ss[0]) == 2 and ss[1] == ss[0][0] and ss[2] == ss[0][1]):
             raise NotImplementedError(f"fused_tp does not support {d.subscripts} (expected uv,u,v)")
     else:
-        if not (len(ss[0]) == 3 and ss[1] == ss[0][0] and ss[2] == ss[0][1] and ss[3] == ss[0][2]):
+        # (uw,u,,w is the same contraction with the mode of extent one left out: the second operand is one scalar per segment)
+        squeezed = len(ss[0]) == 2 and ss[1] == ss[0][0] and ss[2] == "" and ss[3] == ss[0][1]
+        if not squeezed and not (len(ss[0]) == 3 and ss[1] == ss[0][0] and ss[2] == ss[0][1] and ss[3] == ss[0][2]):
             raise NotImplementedError(f"fused_tp does not support {d.subscripts} (expected uvw,u,v,w)")
-        if d.get_dims(ss[2]) - {1}:
+        if not squeezed and d.get_dims(ss[2]) - {1}:
             raise NotImplementedError(
                 "fused_tp: the second operand of a 4-operand contraction must have multiplicity 1 "
                 f"(got extents {sorted(d.get_dims(ss[2]))})"

@@ -10,7 +10,8 @@ indexed inputs and ``scatter_add_`` into indexed outputs (``:186-262``).
 Here two executors stand behind the same interface:
 
 * the matrix-core executor (``cuet/dense.py``) for what the high-level layers produce - one operation ``uv,iu,iv``
-  (Linear) or ``uvw,iu,jv,kw`` with ``v = 1`` (fully connected product), weights shared over the batch, no index tensors;
+  (Linear) or ``uvw,iu,jv,kw`` with ``v = 1`` (fully connected product; also with that mode left out of the subscripts:
+  ``u__uw_w``, ``_v_vw_w``), weights shared over the batch, no index tensors;
 * the same executor behind an element-wise stage (``_MatrixWithElementwiseStage``) for the other forms with a matrix shape
   and shared weights: ``u_v_uvw_w`` with any ``v`` and ``u_u_uw_w`` (the products of the two row operands first, then their
   Linear map), ``u_v_uv_u`` and ``u_v_uv_v`` (the Linear map of one row operand first, then its product with the other);

@@ -104,6 +104,20 @@ def test_forms_with_a_matrix_shape_run_on_the_matrix_cores_when_the_weights_are_
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float32])
+@pytest.mark.parametrize("form", ["u,,uw,w", ",v,vw,w"])
+def test_fully_connected_form_without_its_unit_mode_runs_on_the_matrix_core_executor(device, form, dtype):
+    """``u__uw_w`` / ``_v_vw_w``: the fully connected contraction with the mode of extent one left out of the subscripts (one
+    operand is a scalar per segment).  With the weights as one row the wrapper finds the order of the inputs that the
+    matrix-core executor takes; results and gradients against the oracle."""
+    d = random_stp(form, seed=5 + sum(map(ord, form)), nseg=3)
+    poly = cue.SegmentedPolynomial.eval_last_operand(d)
+    g = torch.Generator().manual_seed(12)
+    inputs = [torch.randn(r, o.size, dtype=torch.float64, generator=g).to(dtype) for r, o in zip((131, 131, 1), poly.inputs)]
+    check(device, poly, inputs, dtype, expect_dense=True)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("dims", [dict(u=8, v=4, w=16), dict(u=5, v=3, w=8), dict(u=16, v=12, w=8), dict(u=16, v=8, w=8)])
 @pytest.mark.parametrize("form", ["u,v,uvw,w", "v,u,uvw,w"])
