@@ -82,7 +82,8 @@ class _MatrixWithElementwiseStage(nn.Module):
       segment become one path of the Linear map (their products side by side, their weight blocks stacked, each times its
       coefficient: a gather of the weight row), so no two paths write the same columns and the executor sends all paths of one
       contraction length out in one launch.  ``P`` has ``x y`` values per path and row: the rows are worked on in pieces that
-      keep it under 4 GiB (``piece_bytes``).
+      keep it under 4 GiB (``piece_bytes``); in training the products of all rows are kept for the weight gradient up to
+      32 GiB (``keep_bytes``), beyond that every piece forms them again in the backward.
     * ``W[m0 m1], a, b -> out`` with one row operand carrying the contracted mode and the other the mode of the output
       (``u_v_uv_u``, ``u_v_uv_v``): ``T = g W`` (or ``g W^T``: the weights are gathered into that order first) per distinct
       (weight segment, segment of ``g``), then ``out += c e * T`` on the uniform-1d kernels.
@@ -200,6 +201,8 @@ class _MatrixWithElementwiseStage(nn.Module):
         # rows are worked on in pieces whose products take at most this many bytes (large pieces fill the chip better: the
         # Linear map has few, long contractions)
         self.piece_bytes = 4 << 30
+        # products of all rows beyond this many bytes are not kept for the backward but formed again there
+        self.keep_bytes = 32 << 30
 
     def _tables(self, device):
         t = self._on_device.get(device)
@@ -250,16 +253,12 @@ class _MatrixWithElementwiseStage(nn.Module):
         # the weight blocks of every path, stacked per output segment, times the coefficients (2-byte weights: rounded once)
         w = (w.float()[:, w_gather] * w_scale.float()).to(w.dtype) if w.dtype in (torch.bfloat16, torch.float16) else w[:, w_gather] * w_scale.to(w.dtype)
         step = max(1, self.piece_bytes // max(1, self.p_size * w.element_size()))
-        outs = []
-        for z0 in range(0, Z, step):
-            a = x1 if x1.shape[0] == 1 else x1[z0:z0 + step]
-            b = x2 if x2.shape[0] == 1 else x2[z0:z0 + step]
-            rows = min(step, Z - z0)
+
+        def piece(a, b, w):
+            rows = max(a.shape[0], b.shape[0])
             if self.kind == "outer" and not traced:
                 # (the kernels of csrc/outer_rows.hip; a traced graph keeps the torch code below)
-                prod = _OuterRows.apply(self, a.expand(rows, -1), b.expand(rows, -1))
-                outs.append(self.linear([w, prod], {}, {}, {})[0])
-                continue
+                return self.linear([w, _OuterRows.apply(self, a.expand(rows, -1), b.expand(rows, -1))], {}, {}, {})[0]
             parts = []
             for ga, gb in groups:
                 if self.kind == "same":
@@ -269,7 +268,24 @@ class _MatrixWithElementwiseStage(nn.Module):
                 else:
                     prod = b[:, gb][:, :, :, None] * a[:, ga][:, :, None, :]
                 parts.append(prod.expand(rows, *prod.shape[1:]).reshape(rows, -1))
-            outs.append(self.linear([w, parts[0] if len(parts) == 1 else torch.cat(parts, 1)], {}, {}, {})[0])
+            return self.linear([w, parts[0] if len(parts) == 1 else torch.cat(parts, 1)], {}, {}, {})[0]
+
+        # The weight gradient needs the products again: autograd keeps them, all pieces of them, until the backward.  Beyond
+        # `keep_bytes` they are formed a second time in the backward instead, piece by piece (one more product kernel per piece).
+        again = (not traced and torch.is_grad_enabled() and Z * self.p_size * w.element_size() > self.keep_bytes
+                 and any(t.requires_grad for t in (x1, x2, w)))
+        outs = []
+        for z0 in range(0, Z, step):
+            a = x1 if x1.shape[0] == 1 else x1[z0:z0 + step]
+            b = x2 if x2.shape[0] == 1 else x2[z0:z0 + step]
+            if x1.shape[0] == 1 and x2.shape[0] == 1:
+                b = b.expand(min(step, Z - z0), -1)
+            if again:
+                from torch.utils.checkpoint import checkpoint
+
+                outs.append(checkpoint(piece, a, b, w, use_reentrant=False))
+            else:
+                outs.append(piece(a, b, w))
         return outs[0] if len(outs) == 1 else torch.cat(outs, 0)
 
 

@@ -219,6 +219,18 @@ def test_fully_connected_product_of_general_multiplicities(device):
     whole = m(x1d, x2d, wd)
     tail = m(x1d[-100:], x2d[-100:], wd)
     assert whole.shape == (rows, io.dim) and rel_err(whole[-100:], tail.cpu()) <= 1e-6
+    # products not kept for the backward but formed again there, piece by piece: the same gradients, and second derivatives
+    xs = [t.clone().requires_grad_(True) for t in (x1d[:5000], x2d[:5000], wd)]
+    ct = torch.randn(5000, io.dim, device=device)
+
+    def grads_and_second(keep):
+        st.keep_bytes, st.piece_bytes = keep, 8 << 20
+        first = torch.autograd.grad(m(xs[0], xs[1], xs[2]), xs, ct, create_graph=True)
+        second = torch.autograd.grad(sum((f * f).sum() for f in first), xs)
+        return [f.detach() for f in first] + list(second)
+
+    for kept, again in zip(grads_and_second(32 << 30), grads_and_second(0)):
+        assert rel_err(again, kept.cpu()) <= 1e-6
 
 
 @pytest.mark.gpu
