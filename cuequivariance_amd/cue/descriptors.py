@@ -7,6 +7,8 @@ Reference behaviour followed (``cuequivariance/cuequivariance/group_theory/descr
 * ``irreps_tp.py:505-545``  linear                          ``"uv,iu,iv"``
 * ``spherical_harmonics_.py:23-85,119-156`` spherical-harmonics polynomial, recursion and normalisation
 * ``symmetric_contractions.py:20-134``  symmetric_contraction  ``"w_a_b_c_i+abciw"`` per degree
+* ``rotations.py:23-252``  rotations about fixed axes with the angle given as ``[cos(l t) .. cos(t), 1, sin(t) .. sin(l t)]``,
+  their compositions ``xy``, ``yx``, ``yxy``, a rotation by a known angle about a known axis, and the inversion
 
 All descriptors use the ``ir_mul`` layout (component index outside, multiplicity inside).
 """
@@ -31,6 +33,13 @@ __all__ = [
     "spherical_harmonics",
     "spherical_harmonics_values",
     "symmetric_contraction",
+    "fixed_axis_angle_rotation",
+    "x_rotation",
+    "y_rotation",
+    "xy_rotation",
+    "yx_rotation",
+    "yxy_rotation",
+    "inversion",
 ]
 
 
@@ -332,3 +341,131 @@ def spherical_harmonics(ir_vec: Irrep, ls, layout=ir_mul) -> EquivariantPolynomi
     return EquivariantPolynomial(
         [IrrepsAndLayout(Irreps(type(ir_vec), [(1, ir_vec)]), ir_mul)], [IrrepsAndLayout(irreps_out, ir_mul)], poly
     )
+
+
+# ---- rotations and the inversion -------------------------------------------------------------------------------------
+# A rotation by the angle t about a coordinate axis acts on an irrep of degree l through D(t) = expm(t X_axis), whose entries
+# are linear combinations of cos(m t), sin(m t), m <= l.  The descriptors take the angle as the vector
+#   encoding(t) = [cos(L t), cos((L - 1) t), ..., cos(t), 1, sin(t), ..., sin(L t)],   L = lmax,
+# so D(t) = sum_e encoding(t)[e] C[e]: the constant matrices C[e] are read off D at sampled angles (a linear system with the
+# 2 L + 1 functions as unknowns per entry - exact, the entries lie in their span), not typed in per degree.  Rotations are
+# active and right-handed on the components (x, y, z) of a vector: about x by t takes y towards z, about y takes z towards x.
+
+
+def _rotation_generators(ir: Irrep) -> np.ndarray:
+    if type(ir).__name__ not in ("SO3", "O3", "O3_e3nn"):
+        raise ValueError(f"Unsupported irrep class {type(ir).__name__}. Must be SO3 or O3.")
+    return np.asarray(ir.continuous_generators(), dtype=np.float64)
+
+
+def _expm(a: np.ndarray) -> np.ndarray:
+    from scipy.linalg import expm
+
+    return expm(a)
+
+
+@functools.lru_cache(maxsize=None)
+def _axis_rotation_tensor(ir: Irrep, axis: int, lmax: int) -> np.ndarray:
+    """``C[e, j, k]`` with ``D(t)[k, j] = sum_e encoding(t)[e] C[e, j, k]`` for the rotation about coordinate axis ``axis``."""
+    if ir.l > lmax:
+        raise ValueError(f"lmax = {lmax} is below the degree of {ir}")
+    X = _rotation_generators(ir)[axis]
+    ts = np.linspace(0.0, 2.0 * np.pi, 4 * lmax + 5, endpoint=False) + 0.1234
+    m = np.arange(1, lmax + 1)
+    enc = np.concatenate([np.cos(ts[:, None] * m[::-1]), np.ones((len(ts), 1)), np.sin(ts[:, None] * m)], axis=1)
+    D = np.stack([_expm(t * X) for t in ts])  # (samples, k, j)
+    sol, *_ = np.linalg.lstsq(enc, D.reshape(len(ts), -1), rcond=None)
+    assert np.abs(enc @ sol - D.reshape(len(ts), -1)).max() < 1e-10
+    C = sol.reshape(2 * lmax + 1, ir.dim, ir.dim).transpose(0, 2, 1)  # (e, j, k)
+    C[np.abs(C) < 1e-12] = 0.0
+    return C
+
+
+def _lmax_of(irreps: Irreps, lmax: Optional[int]) -> int:
+    for _, ir in irreps:
+        _rotation_generators(ir)
+    return max(ir.l for _, ir in irreps) if lmax is None else int(lmax)
+
+
+def _rotation_polynomial(irreps: Irreps, tensors, num_angles: int, lmax: int) -> EquivariantPolynomial:
+    """``angle encodings (num_angles of them), input[u] -> output[u]`` with the constant tensor ``tensors(ir)[e1, .., j, k]`` per
+    irrep: every encoding component is a scalar segment, every component of an irrep a segment of its multiplicity."""
+    d = SegmentedTensorProduct.from_subscripts(",".join([""] * num_angles + ["u", "u"]))
+    for a in range(num_angles):
+        for _ in range(2 * lmax + 1):
+            d.add_segment(a, ())
+    for mul, ir in irreps:
+        first = d.operands[num_angles].num_segments
+        for _ in range(ir.dim):
+            d.add_segment(num_angles, (mul,))
+            d.add_segment(num_angles + 1, (mul,))
+        T = tensors(ir)
+        for idx in zip(*np.nonzero(T)):
+            *es, j, k = (int(v) for v in idx)
+            d.add_path(*es, first + j, first + k, c=float(T[idx]))
+    enc = [IrrepsAndLayout(irreps.new_scalars(2 * lmax + 1), ir_mul) for _ in range(num_angles)]
+    return EquivariantPolynomial(enc + [IrrepsAndLayout(irreps, ir_mul)], [IrrepsAndLayout(irreps, ir_mul)],
+                                 SegmentedPolynomial.eval_last_operand(d))
+
+
+def _clean(T: np.ndarray) -> np.ndarray:
+    T = T.copy()
+    T[np.abs(T) < 1e-12] = 0.0
+    return T
+
+
+def y_rotation(irreps: Irreps, lmax: Optional[int] = None) -> EquivariantPolynomial:
+    """``phi[], input[u] -> output[u]``: rotation about the y axis, the angle as ``encoding(phi)`` (reference ``rotations.py:131-199``)."""
+    L = _lmax_of(irreps, lmax)
+    return _rotation_polynomial(irreps, lambda ir: _axis_rotation_tensor(ir, 1, L), 1, L)
+
+
+def x_rotation(irreps: Irreps, lmax: Optional[int] = None) -> EquivariantPolynomial:
+    """``phi[], input[u] -> output[u]``: rotation about the x axis (reference ``rotations.py:202-232``)."""
+    L = _lmax_of(irreps, lmax)
+    return _rotation_polynomial(irreps, lambda ir: _axis_rotation_tensor(ir, 0, L), 1, L)
+
+
+def xy_rotation(irreps: Irreps, lmax: Optional[int] = None) -> EquivariantPolynomial:
+    """``gamma[], beta[], input[u] -> output[u]``: about y by gamma, then about x by beta (reference ``rotations.py:87-107``)."""
+    L = _lmax_of(irreps, lmax)
+    return _rotation_polynomial(
+        irreps, lambda ir: _clean(np.einsum("cja,bak->cbjk", _axis_rotation_tensor(ir, 1, L), _axis_rotation_tensor(ir, 0, L))), 2, L)
+
+
+def yx_rotation(irreps: Irreps, lmax: Optional[int] = None) -> EquivariantPolynomial:
+    """``phi[], theta[], input[u] -> output[u]``: about x by phi, then about y by theta (reference ``rotations.py:110-128``)."""
+    L = _lmax_of(irreps, lmax)
+    return _rotation_polynomial(
+        irreps, lambda ir: _clean(np.einsum("cja,bak->cbjk", _axis_rotation_tensor(ir, 0, L), _axis_rotation_tensor(ir, 1, L))), 2, L)
+
+
+def yxy_rotation(irreps: Irreps, lmax: Optional[int] = None) -> EquivariantPolynomial:
+    """``gamma[], beta[], alpha[], input[u] -> output[u]``: about y by gamma, then about x by beta, then about y by alpha
+    (reference ``rotations.py:49-84``)."""
+    L = _lmax_of(irreps, lmax)
+
+    def tensor(ir):
+        Y, X = _axis_rotation_tensor(ir, 1, L), _axis_rotation_tensor(ir, 0, L)
+        return _clean(np.einsum("cja,bad,edk->cbejk", Y, X, Y))
+
+    return _rotation_polynomial(irreps, tensor, 3, L)
+
+
+def fixed_axis_angle_rotation(irreps: Irreps, axis: np.ndarray, angle: float) -> EquivariantPolynomial:
+    """``input[u] -> output[u]``: rotation by a known angle about a known axis (reference ``rotations.py:23-46``)."""
+    axis = np.asarray(axis, dtype=np.float64)
+    axis = axis / np.linalg.norm(axis)
+
+    def tensor(ir):
+        D = _expm(float(angle) * np.einsum("a,aij->ij", axis, _rotation_generators(ir)))
+        return _clean(D.T)  # (j, k)
+
+    return _rotation_polynomial(irreps, tensor, 0, 0)
+
+
+def inversion(irreps: Irreps) -> EquivariantPolynomial:
+    """``input[u] -> output[u]``: the inversion ``x -> -x`` of O(3): every irrep times its parity (reference ``rotations.py:235-252``)."""
+    if irreps.irrep_class.__name__ not in ("O3", "O3_e3nn"):
+        raise ValueError(f"Unsupported irrep class {irreps.irrep_class.__name__}. Must be O3.")
+    return _rotation_polynomial(irreps, lambda ir: float(ir.p) * np.eye(ir.dim), 0, 0)

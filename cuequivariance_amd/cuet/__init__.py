@@ -2,7 +2,8 @@
 
 from .transpose import TransposeSegments, TransposeIrrepsLayout
 from .segmented_polynomial import SegmentedPolynomial
-from .operations import ChannelWiseSphericalTensorProduct, ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction, SphericalHarmonics
+from .operations import (ChannelWiseSphericalTensorProduct, ChannelWiseTensorProduct, FullyConnectedTensorProduct, Linear, SymmetricContraction,
+                         SphericalHarmonics, Rotation, Inversion, encode_rotation_angle, vector_to_euler_angles)
 from .uniform_1d import uniform_1d
 from .triangle import triangle_multiplicative_update, TriMulPrecision
 from . import layers
@@ -18,6 +19,10 @@ __all__ = [
     "Linear",
     "SymmetricContraction",
     "SphericalHarmonics",
+    "Rotation",
+    "Inversion",
+    "encode_rotation_angle",
+    "vector_to_euler_angles",
     "uniform_1d",
     "triangle_multiplicative_update",
     "TriMulPrecision",

@@ -26,7 +26,8 @@ from ..cue import descriptors
 from .segmented_polynomial import SegmentedPolynomial
 from .transpose import TransposeIrrepsLayout, apply_layout
 
-__all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear", "SymmetricContraction", "SphericalHarmonics"]
+__all__ = ["ChannelWiseTensorProduct", "FullyConnectedTensorProduct", "Linear", "SymmetricContraction", "SphericalHarmonics",
+           "Rotation", "Inversion", "encode_rotation_angle", "vector_to_euler_angles"]
 
 
 def _default_irreps(*irreps_list):
@@ -616,3 +617,105 @@ class SphericalHarmonics(torch.nn.Module):
             vectors = torch.nn.functional.normalize(vectors, dim=1)
         [output] = self.f([vectors])
         return output
+
+
+class Rotation(torch.nn.Module):
+    """Rotation of SO(3) / O(3) features (``cuequivariance_torch/operations/rotation.py:29-157`` in the reference):
+    ``forward(gamma, beta, alpha, x)`` applies the rotation about y by ``gamma``, then about x by ``beta``, then about y by
+    ``alpha`` to every irrep of ``x`` - ``R = R_y(alpha) R_x(beta) R_y(gamma)``, active and right-handed on the components
+    ``(x, y, z)`` of a vector.  Angles: one per row of ``x``, or a single one for all rows.  One uniform-1d polynomial with the three
+    angle encodings and ``x`` as inputs (``descriptors.yxy_rotation``)."""
+
+    def __init__(
+        self,
+        irreps: cue.Irreps,
+        *,
+        layout: Optional[cue.IrrepsLayout] = None,
+        layout_in: Optional[cue.IrrepsLayout] = None,
+        layout_out: Optional[cue.IrrepsLayout] = None,
+        device: Optional[torch.device] = None,
+        math_dtype=None,
+        use_fallback: Optional[bool] = None,
+        method: Optional[str] = None,
+    ):
+        super().__init__()
+        (irreps,) = _default_irreps(irreps)
+        if irreps.irrep_class not in [cue.SO3, cue.O3]:
+            raise ValueError(f"Unsupported irrep class {irreps.irrep_class}. Must be SO3 or O3.")
+        e = descriptors.yxy_rotation(irreps)
+        self.irreps = irreps
+        self.lmax = max(ir.l for _, ir in irreps)
+        self.transpose_in = TransposeIrrepsLayout(
+            e.inputs[3].irreps, source=_default_layout(layout_in or layout), target=e.inputs[3].layout, device=device
+        )
+        self.transpose_out = TransposeIrrepsLayout(
+            e.outputs[0].irreps, source=e.outputs[0].layout, target=_default_layout(layout_out or layout), device=device
+        )
+        self.method = _method_from_fallback(method, use_fallback, "uniform_1d")
+        # (multiplicities that differ: the channel mode split down to their common divisor)
+        self.f = (SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+                  if e.polynomial.all_same_segment_shape() or self.method != "uniform_1d" else _FlattenedUniform(e.polynomial, math_dtype))
+
+    def forward(self, gamma: torch.Tensor, beta: torch.Tensor, alpha: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+        encodings = []
+        for angle in (gamma, beta, alpha):
+            angle = torch.as_tensor(angle, dtype=x.dtype, device=x.device)
+            enc = encode_rotation_angle(angle, self.lmax)
+            encodings.append(enc.reshape(-1, enc.shape[-1]))  # (1 or batch, 2 lmax + 1)
+        out = self.f([*encodings, apply_layout(self.transpose_in, x)])
+        return apply_layout(self.transpose_out, out[0])
+
+
+def encode_rotation_angle(angle: torch.Tensor, ell: int) -> torch.Tensor:
+    """``[cos(ell a), cos((ell - 1) a), ..., cos(a), 1, sin(a), sin(2 a), ..., sin(ell a)]`` along a new last axis: the form in
+    which the rotation polynomials take an angle (``operations/rotation.py:160-176`` in the reference)."""
+    angle = torch.as_tensor(angle).unsqueeze(-1)
+    m = torch.arange(1, ell + 1, device=angle.device, dtype=angle.dtype)
+    return torch.cat([torch.cos(m.flip(0) * angle), torch.ones_like(angle), torch.sin(m * angle)], dim=-1)
+
+
+def vector_to_euler_angles(vector: torch.Tensor):
+    """``(beta, alpha)`` with ``R_y(alpha) R_x(beta) e_y = vector / |vector|`` (``operations/rotation.py:179-208`` in the
+    reference): ``beta`` is the angle to the y axis, ``alpha`` the azimuth from z towards x (0 on the y axis itself)."""
+    assert vector.shape[-1] == 3
+    x, y, z = torch.nn.functional.normalize(vector.reshape(-1, 3), dim=-1).unbind(-1)
+    on_axis = (x == 0.0) & (z == 0.0)
+    beta = torch.acos(torch.clamp(torch.where(on_axis, torch.sign(y), y), -1.0, 1.0))
+    alpha = torch.atan2(torch.where(on_axis, torch.zeros_like(x), x), torch.where(on_axis, torch.ones_like(z), z))
+    return beta.reshape(vector.shape[:-1]), alpha.reshape(vector.shape[:-1])
+
+
+class Inversion(torch.nn.Module):
+    """Inversion ``x -> -x`` of O(3) features: every irrep times its parity (``operations/rotation.py:211-310`` in the
+    reference)."""
+
+    def __init__(
+        self,
+        irreps: cue.Irreps,
+        *,
+        layout: Optional[cue.IrrepsLayout] = None,
+        layout_in: Optional[cue.IrrepsLayout] = None,
+        layout_out: Optional[cue.IrrepsLayout] = None,
+        device: Optional[torch.device] = None,
+        math_dtype=None,
+        use_fallback: Optional[bool] = None,
+        method: Optional[str] = None,
+    ):
+        super().__init__()
+        (irreps,) = _default_irreps(irreps)
+        if irreps.irrep_class not in [cue.O3]:
+            raise ValueError(f"Unsupported irrep class {irreps.irrep_class}. Must be O3.")
+        e = descriptors.inversion(irreps)
+        self.irreps = irreps
+        self.transpose_in = TransposeIrrepsLayout(
+            e.inputs[0].irreps, source=_default_layout(layout_in or layout), target=e.inputs[0].layout, device=device
+        )
+        self.transpose_out = TransposeIrrepsLayout(
+            e.outputs[0].irreps, source=e.outputs[0].layout, target=_default_layout(layout_out or layout), device=device
+        )
+        self.method = _method_from_fallback(method, use_fallback, "uniform_1d")
+        self.f = (SegmentedPolynomial(e.polynomial, method=self.method, math_dtype=math_dtype)
+                  if e.polynomial.all_same_segment_shape() or self.method != "uniform_1d" else _FlattenedUniform(e.polynomial, math_dtype))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return apply_layout(self.transpose_out, self.f([apply_layout(self.transpose_in, x)])[0])
