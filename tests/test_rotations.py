@@ -179,3 +179,12 @@ def test_vector_to_euler_angles_points_the_y_axis_at_the_vector():
     assert cuet.vector_to_euler_angles(torch.zeros(2, 4, 3))[0].shape == (2, 4)
     enc = cuet.encode_rotation_angle(torch.tensor([0.25, -1.0], dtype=torch.float64), 3)
     assert enc.shape == (2, 7) and np.allclose(enc[0].numpy(), encode(0.25, 3)[0]) and np.allclose(enc[1].numpy(), encode(-1.0, 3)[0])
+
+
+def test_removed_names_refuse_with_their_replacement():
+    """The four classes the reference keeps as stubs (``primitives/deprecated.py``): importable, not constructible."""
+    from cuequivariance_amd import cuet
+
+    for name in ("TensorProduct", "EquivariantTensorProduct", "SymmetricTensorProduct", "IWeightedSymmetricTensorProduct"):
+        with pytest.raises(ImportError, match="SegmentedPolynomial"):
+            getattr(cuet, name)(None)
