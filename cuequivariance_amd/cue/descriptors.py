@@ -5,6 +5,9 @@ Reference behaviour followed (``cuequivariance/cuequivariance/group_theory/descr
 * ``irreps_tp.py:22-91``    fully_connected_tensor_product  ``"uvw,iu,jv,kw+ijk"``
 * ``irreps_tp.py:232-321``  channelwise_tensor_product      ``"uv,iu,jv,kuv+ijk"``
 * ``irreps_tp.py:505-545``  linear                          ``"uv,iu,iv"``
+* ``irreps_tp.py:127-195``  full_tensor_product             ``"iu,jv,kuv+ijk"`` (the channel-wise product without weights)
+* ``irreps_tp.py:364-461``  elementwise_tensor_product      ``"iu,ju,ku+ijk"`` (equal channels multiplied, multiplicities aligned)
+* ``transposition.py:18-36``  transpose                     ``"ui,iu"`` / ``"iu,ui"`` between the two layouts
 * ``spherical_harmonics_.py:23-85,119-156`` spherical-harmonics polynomial, recursion and normalisation
 * ``symmetric_contractions.py:20-134``  symmetric_contraction  ``"w_a_b_c_i+abciw"`` per degree
 * ``rotations.py:23-252``  rotations about fixed axes with the angle given as ``[cos(l t) .. cos(t), 1, sin(t) .. sin(l t)]``,
@@ -30,6 +33,9 @@ __all__ = [
     "channelwise_tensor_product",
     "fully_connected_tensor_product",
     "linear",
+    "full_tensor_product",
+    "elementwise_tensor_product",
+    "transpose",
     "spherical_harmonics",
     "spherical_harmonics_values",
     "symmetric_contraction",
@@ -153,6 +159,88 @@ def linear(irreps_in: Irreps, irreps_out: Irreps) -> EquivariantPolynomial:
         [IrrepsAndLayout(irreps_out, ir_mul)],
         poly,
     )
+
+
+def full_tensor_product(irreps1: Irreps, irreps2: Irreps, irreps3_filter=None) -> EquivariantPolynomial:
+    """``lhs[iu], rhs[jv] -> output[kuv]``: the channel-wise product without weights - every pair of channels of every allowed
+    (ir1, ir2, ir3) gets an output channel.  Output irreps stable-sorted like those of the channel-wise product."""
+    G = irreps1.irrep_class
+    if irreps3_filter is not None:
+        irreps3_filter = into_list_of_irrep(G, irreps3_filter)
+    d = SegmentedTensorProduct.from_subscripts("iu,jv,kuv+ijk")
+    for mul, ir in irreps1:
+        d.add_segment(0, (ir.dim, mul))
+    for mul, ir in irreps2:
+        d.add_segment(1, (ir.dim, mul))
+    out = []
+    for (i1, (mul1, ir1)), (i2, (mul2, ir2)) in itertools.product(enumerate(irreps1), enumerate(irreps2)):
+        for ir3 in ir1 * ir2:
+            if irreps3_filter is not None and ir3 not in irreps3_filter:
+                continue
+            for cg in clebsch_gordan(ir1, ir2, ir3):
+                d.add_path(i1, i2, None, c=cg)
+                out.append((mul1 * mul2, ir3))
+    irreps3, _perm, inv = Irreps(G, out).sort()
+    d = d.permute_segments(2, inv).normalize_paths_for_operand(-1)
+    return EquivariantPolynomial(
+        [IrrepsAndLayout(irreps1, ir_mul), IrrepsAndLayout(irreps2, ir_mul)], [IrrepsAndLayout(irreps3, ir_mul)],
+        SegmentedPolynomial.eval_last_operand(d))
+
+
+def _cut_to_common_multiplicities(irreps1: Irreps, irreps2: Irreps):
+    """Both lists of (multiplicity, irrep) cut so that entry k of one has the multiplicity of entry k of the other: the longer
+    entry is split into the common part and the rest, which meets the next entry of the other list.  In ``ir_mul`` rows a split
+    keeps the memory order only for irreps of dimension one."""
+    if irreps1.num_irreps != irreps2.num_irreps:
+        raise ValueError(f"The input irreps must have the same number of irreps, got {irreps1} and {irreps2}")
+    a, b = [(m, ir) for m, ir in irreps1], [(m, ir) for m, ir in irreps2]
+    k = 0
+    while k < min(len(a), len(b)):
+        (m1, ir1), (m2, ir2) = a[k], b[k]
+        if m1 < m2:
+            assert ir2.dim == 1, "splitting the channels of an irrep of dimension above one does not keep ir_mul rows in order"
+            b[k:k + 1] = [(m1, ir2), (m2 - m1, ir2)]
+        elif m2 < m1:
+            assert ir1.dim == 1, "splitting the channels of an irrep of dimension above one does not keep ir_mul rows in order"
+            a[k:k + 1] = [(m2, ir1), (m1 - m2, ir1)]
+        k += 1
+    assert [m for m, _ in a] == [m for m, _ in b], (a, b)
+    return Irreps(irreps1.irrep_class, a), Irreps(irreps2.irrep_class, b)
+
+
+def elementwise_tensor_product(irreps1: Irreps, irreps2: Irreps, irreps3_filter=None) -> EquivariantPolynomial:
+    """``lhs[iu], rhs[ju] -> output[ku]``: channel n of the first operand with channel n of the second (the operands must hold
+    the same number of irreps; multiplicities are aligned by cutting).  The output keeps the order of the products."""
+    G = irreps1.irrep_class
+    if irreps3_filter is not None:
+        irreps3_filter = into_list_of_irrep(G, irreps3_filter)
+    cut1, cut2 = _cut_to_common_multiplicities(irreps1, irreps2)
+    d = SegmentedTensorProduct.from_subscripts("iu,ju,ku+ijk")
+    out = []
+    for (mul, ir1), (_, ir2) in zip(cut1, cut2):
+        i1, i2 = d.add_segment(0, (ir1.dim, mul)), d.add_segment(1, (ir2.dim, mul))
+        for ir3 in ir1 * ir2:
+            if irreps3_filter is not None and ir3 not in irreps3_filter:
+                continue
+            for cg in clebsch_gordan(ir1, ir2, ir3):
+                d.add_path(i1, i2, None, c=cg)
+                out.append((mul, ir3))
+    d = d.normalize_paths_for_operand(-1)
+    return EquivariantPolynomial(
+        [IrrepsAndLayout(cut1, ir_mul), IrrepsAndLayout(cut2, ir_mul)], [IrrepsAndLayout(Irreps(G, out), ir_mul)],
+        SegmentedPolynomial.eval_last_operand(d))
+
+
+def transpose(irreps: Irreps, source, target) -> EquivariantPolynomial:
+    """``input -> output``: the same features in the other layout (``mul_ir``: component inside, ``ir_mul``: channel inside); one
+    path of coefficient one per irrep."""
+    from .irreps import mul_ir
+
+    d = SegmentedTensorProduct.from_subscripts(("ui" if source == mul_ir else "iu") + "," + ("ui" if target == mul_ir else "iu"))
+    for mul, ir in irreps:
+        d.add_path(None, None, c=1.0, dims={"u": mul, "i": ir.dim})
+    return EquivariantPolynomial([IrrepsAndLayout(irreps, source)], [IrrepsAndLayout(irreps, target)],
+                                 SegmentedPolynomial.eval_last_operand(d))
 
 
 def spherical_harmonics_values(ir_vec: Irrep, ls: Sequence[int], vectors: np.ndarray) -> np.ndarray:

@@ -380,3 +380,47 @@ def test_spherical_harmonics_polynomial():
     for ell in ls:
         np.testing.assert_allclose((y[:, off: off + 2 * ell + 1] ** 2).sum(1), 2 * ell + 1, atol=1e-12)
         off += 2 * ell + 1
+
+
+def test_weightless_products_and_the_transpose_descriptor():
+    """``full_tensor_product`` is the channel-wise product with every weight one (that descriptor is pinned to the reference's
+    expectations above); ``elementwise_tensor_product`` is its diagonal in the two channel indices, with the multiplicities of
+    the two operands cut to match; ``transpose`` moves every element between the two layouts.  Evaluated by the oracle."""
+    import torch
+
+    from oracle.naive import naive_segmented_polynomial, spec_from_polynomial
+
+    def run(e, *xs):
+        return naive_segmented_polynomial(spec_from_polynomial(e.polynomial), [torch.as_tensor(x) for x in xs])[0].numpy()
+
+    rng = np.random.default_rng(5)
+    a, b = cue.Irreps("O3", "2x0e+3x1o+1x2e"), cue.Irreps("O3", "1x0e+2x1o")
+    full = cue.descriptors.full_tensor_product(a, b, ["0e", "1o", "2e"])
+    cw = cue.descriptors.channelwise_tensor_product(a, b, ["0e", "1o", "2e"])
+    assert full.outputs[0].irreps == cw.outputs[0].irreps and full.polynomial.operations[0][1].subscripts == "iu,jv,kuv+ijk"
+    x1, x2 = rng.normal(size=(4, a.dim)), rng.normal(size=(4, b.dim))
+    assert np.allclose(run(full, x1, x2), run(cw, np.ones((4, cw.inputs[0].irreps.dim)), x1, x2), atol=1e-13)
+
+    c, d = cue.Irreps("O3", "3x1o+4x0e"), cue.Irreps("O3", "3x1o+2x0e+2x0o")
+    el = cue.descriptors.elementwise_tensor_product(c, d)
+    assert str(el.inputs[0].irreps) == "3x1o+2x0e+2x0e" and str(el.inputs[1].irreps) == "3x1o+2x0e+2x0o"
+    assert str(el.outputs[0].irreps) == "3x0e+3x1e+3x2e+2x0e+2x0o" and el.polynomial.operations[0][1].subscripts == "iu,ju,ku+ijk"
+    y1, y2 = rng.normal(size=(2, c.dim)), rng.normal(size=(2, d.dim))
+    got = run(el, y1, y2)
+    # the first three output irreps against the diagonal of the full product of 3x1o with 3x1o (ir_mul rows: (component, u, v))
+    f = run(cue.descriptors.full_tensor_product(cue.Irreps("O3", "3x1o"), cue.Irreps("O3", "3x1o")), y1[:, :9], y2[:, :9])
+    off_f = off_g = 0
+    for dim in (1, 3, 5):
+        block = f[:, off_f:off_f + dim * 9].reshape(2, dim, 3, 3)
+        assert np.allclose(got[:, off_g:off_g + dim * 3].reshape(2, dim, 3), np.einsum("zkuu->zku", block), atol=1e-13)
+        off_f, off_g = off_f + dim * 9, off_g + dim * 3
+    assert np.allclose(got[:, off_g:off_g + 2], y1[:, 9:11] * y2[:, 9:11]) and np.allclose(got[:, off_g + 2:], y1[:, 11:13] * y2[:, 11:13])
+    with pytest.raises(ValueError):
+        cue.descriptors.elementwise_tensor_product(cue.Irreps("O3", "2x0e"), cue.Irreps("O3", "1x0e+2x1o"))
+
+    t = cue.descriptors.transpose(a, cue.mul_ir, cue.ir_mul)
+    z = rng.normal(size=(3, a.dim))
+    want = np.concatenate([z[:, o:o + m * ir.dim].reshape(3, m, ir.dim).transpose(0, 2, 1).reshape(3, -1)
+                           for (m, ir), o in zip(a, np.cumsum([0] + [m * ir.dim for m, ir in a]))], axis=1)
+    assert np.array_equal(run(t, z), want)
+    assert np.array_equal(run(cue.descriptors.transpose(a, cue.ir_mul, cue.mul_ir), want), z)
