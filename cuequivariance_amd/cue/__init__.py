@@ -25,8 +25,11 @@ from .reduced_basis import (
     selection_rule_product,
     selection_rule_power,
 )
+from .irreps import assume, get_irrep_scope, get_layout_scope
 from . import descriptors
 from . import mace
+
+__version__ = "0.1.0"
 
 __all__ = [
     "Irrep", "SU2", "SO3", "O3", "O3_e3nn", "MulIrrep", "Irreps", "IrrepsLayout", "mul_ir", "ir_mul",
@@ -34,4 +37,5 @@ __all__ = [
     "Path", "SegmentedTensorProduct", "Operation", "SegmentedPolynomial", "EquivariantPolynomial",
     "descriptors", "mace", "IrrepsArray", "reduced_tensor_product_basis", "reduced_symmetric_tensor_product_basis",
     "reduced_antisymmetric_tensor_product_basis", "selection_rule_product", "selection_rule_power",
+    "assume", "get_irrep_scope", "get_layout_scope", "__version__",
 ]

@@ -385,6 +385,53 @@ def clebsch_gordan(r1: Irrep, r2: Irrep, r3: Irrep) -> np.ndarray:
 # --------------------------------------------------------------------------
 # Irreps container
 # --------------------------------------------------------------------------
+# ---- assumed irrep class and layout (reference: irreps_array/context_irrep_class.py, context_layout.py, context_decorator.py) ----
+_assumed = {"irrep_class": None, "layout": None}
+
+
+def get_irrep_scope(raising: bool = True):
+    """The irrep class assumed by the enclosing ``with cue.assume(...)`` (a name such as ``"O3"`` is looked up)."""
+    value = _assumed["irrep_class"]
+    if raising and value is None:
+        raise ValueError("No irrep class set in the context. Please specify the irrep class explicitly or use ``with cue.assume(irrep):``.")
+    return _IRREP_CLASSES[value] if isinstance(value, str) else value
+
+
+def get_layout_scope(raising: bool = True):
+    """The layout assumed by the enclosing ``with cue.assume(...)``."""
+    value = _assumed["layout"]
+    if raising and value is None:
+        raise ValueError("No layout set in the context. Please specify the layout explicitly or use ``with cue.assume(layout):``.")
+    return value
+
+
+class assume:
+    """Context manager and decorator: inside, ``cue.Irreps("2x1")`` takes the given irrep class and a layout left out (``None``)
+    is the given one.  ``cue.assume(cue.SO3, cue.ir_mul)``, ``cue.assume("O3")``, ``cue.assume(cue.mul_ir)``."""
+
+    def __init__(self, irrep_class=None, layout=None):
+        if isinstance(irrep_class, IrrepsLayout) and layout is None:
+            irrep_class, layout = None, irrep_class
+        self.irrep_class, self.layout = irrep_class, layout
+
+    def __enter__(self):
+        self._before = dict(_assumed)
+        _assumed["irrep_class"], _assumed["layout"] = self.irrep_class, self.layout
+        return self
+
+    def __exit__(self, *exc):
+        _assumed.update(self._before)
+        return False
+
+    def __call__(self, func):
+        @functools.wraps(func)
+        def wrapper(*args, **kwargs):
+            with self:
+                return func(*args, **kwargs)
+
+        return wrapper
+
+
 @dataclasses.dataclass(frozen=True)
 class MulIrrep:
     mul: int
@@ -418,9 +465,13 @@ class Irreps:
         elif len(args) == 1 and isinstance(args[0], Irrep):
             args = (type(args[0]), [(1, args[0])])
         elif len(args) == 1:
-            # Without an explicit group the string decides: "0e"/"1o" is O3, bare integers SO3.
+            # Without an explicit group: the one assumed by the enclosing ``with cue.assume(...)``, else the string decides
+            # ("0e" / "1o" is O3, bare integers SO3).
             text = args[0]
-            if isinstance(text, str):
+            scope = get_irrep_scope(raising=False)
+            if scope is not None:
+                args = (scope, text)
+            elif isinstance(text, str):
                 args = (O3 if re.search(r"\d[eo]", text) else SO3, text)
             else:
                 raise ValueError("Irreps needs an irrep class")
@@ -665,8 +716,9 @@ class IrrepsLayout(Enum):
     def as_layout(layout) -> "IrrepsLayout":
         if isinstance(layout, IrrepsLayout):
             return layout
-        if layout is None:
-            return IrrepsLayout.mul_ir
+        if layout is None:  # the layout assumed by the enclosing ``with cue.assume(...)``, else the e3nn layout
+            scope = get_layout_scope(raising=False)
+            return IrrepsLayout.mul_ir if scope is None else scope
         try:
             return IrrepsLayout[layout]
         except KeyError:

@@ -55,6 +55,9 @@ def _transposition_moves(irreps) -> bool:
 
 def _default_layout(layout) -> cue.IrrepsLayout:
     if layout is None:
+        assumed = cue.get_layout_scope(raising=False)  # (inside ``with cue.assume(layout):``)
+        if assumed is not None:
+            return assumed
         warnings.warn("layout is not specified, defaulting to cue.mul_ir (the e3nn layout)")
         return cue.mul_ir
     return cue.IrrepsLayout.as_layout(layout)

@@ -424,3 +424,27 @@ def test_weightless_products_and_the_transpose_descriptor():
                            for (m, ir), o in zip(a, np.cumsum([0] + [m * ir.dim for m, ir in a]))], axis=1)
     assert np.array_equal(run(t, z), want)
     assert np.array_equal(run(cue.descriptors.transpose(a, cue.ir_mul, cue.mul_ir), want), z)
+
+
+def test_assumed_irrep_class_and_layout():
+    """``cue.assume`` as context manager and decorator (reference ``irreps_array/context_decorator.py:33-84``): the irrep class of
+    ``cue.Irreps("2x1")`` and the layout of ``cue.IrrepsAndLayout`` without one; scopes nest and are restored."""
+    with pytest.raises(ValueError):
+        cue.get_irrep_scope()
+    assert cue.get_irrep_scope(raising=False) is None and cue.get_layout_scope(raising=False) is None
+    with cue.assume(cue.SO3, cue.mul_ir):
+        rep = cue.IrrepsAndLayout("2x1")
+        assert rep.irreps == cue.Irreps("SO3", "2x1") and rep.layout == cue.mul_ir
+        with cue.assume("O3", cue.ir_mul):
+            assert cue.Irreps("2x1o").irrep_class is cue.O3 and cue.IrrepsAndLayout("1e").layout == cue.ir_mul
+            assert cue.get_irrep_scope() is cue.O3 and cue.get_layout_scope() == cue.ir_mul
+        assert cue.get_irrep_scope() is cue.SO3 and cue.get_layout_scope() == cue.mul_ir
+    assert cue.get_irrep_scope(raising=False) is None
+
+    @cue.assume(cue.SU2)
+    def half():
+        return cue.Irreps("3x1/2")
+
+    assert half().irrep_class is cue.SU2
+    with cue.assume(cue.ir_mul):  # a layout alone
+        assert cue.get_layout_scope() == cue.ir_mul and cue.get_irrep_scope(raising=False) is None
