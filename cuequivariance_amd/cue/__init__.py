@@ -28,6 +28,8 @@ from .reduced_basis import (
 from .irreps import assume, get_irrep_scope, get_layout_scope
 from . import descriptors
 from . import mace
+from . import segmented_polynomials
+from . import group_theory
 
 __version__ = "0.1.0"
 
@@ -37,5 +39,5 @@ __all__ = [
     "Path", "SegmentedTensorProduct", "Operation", "SegmentedPolynomial", "EquivariantPolynomial",
     "descriptors", "mace", "IrrepsArray", "reduced_tensor_product_basis", "reduced_symmetric_tensor_product_basis",
     "reduced_antisymmetric_tensor_product_basis", "selection_rule_product", "selection_rule_power",
-    "assume", "get_irrep_scope", "get_layout_scope", "__version__",
+    "assume", "get_irrep_scope", "get_layout_scope", "__version__", "segmented_polynomials", "group_theory",
 ]

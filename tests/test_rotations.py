@@ -188,3 +188,26 @@ def test_removed_names_refuse_with_their_replacement():
     for name in ("TensorProduct", "EquivariantTensorProduct", "SymmetricTensorProduct", "IWeightedSymmetricTensorProduct"):
         with pytest.raises(ImportError, match="SegmentedPolynomial"):
             getattr(cuet, name)(None)
+
+
+def test_composition_of_descriptors_by_dot():
+    """``cue.segmented_polynomials.dot`` as the reference uses it to build its rotations (``rotations.py:70-77,94-96``): the y
+    rotation composed with the x rotation over the intermediate features, operands moved into the order ``gamma, beta, input,
+    output``, evaluates like ``xy_rotation``; with no pair given ``dot`` is the plain product of two descriptors."""
+    irreps = cue.Irreps("O3", "2x0e+2x1o+2x2e")
+    y = descriptors.y_rotation(irreps).polynomial.operations[0][1]   # gamma, input, A
+    x = descriptors.x_rotation(irreps).polynomial.operations[0][1]   # beta, A, output
+    d = cue.segmented_polynomials.dot(y, x, (2, 1)).move_operand(1, 2)  # gamma, input, beta, output -> gamma, beta, input, output
+    assert d.subscripts == ",,u,u" and d.num_operands == 4
+    g, b = 0.7, -0.4
+    feats = np.random.default_rng(6).normal(size=(3, irreps.dim))
+    got = naive_segmented_polynomial(spec_from_polynomial(cue.SegmentedPolynomial.eval_last_operand(d)),
+                                     [torch.as_tensor(encode(g, 2)), torch.as_tensor(encode(b, 2)), torch.as_tensor(feats)])[0].numpy()
+    assert np.allclose(got, evaluate(descriptors.xy_rotation(irreps), encode(g, 2), encode(b, 2), feats), atol=1e-12)
+    a = cue.SegmentedTensorProduct.from_subscripts("i,j+ij")
+    a.add_path(None, None, c=np.arange(6.0).reshape(2, 3))
+    p = cue.segmented_polynomials.dot(a, a)
+    assert p.num_operands == 4 and p.num_paths == 1 and p.coefficient_subscripts == "ij"
+    with pytest.raises(ValueError):
+        cue.segmented_polynomials.dot(y, x, (0, 1))
+    assert hasattr(cue.group_theory, "clebsch_gordan") and cue.group_theory.descriptors is descriptors
