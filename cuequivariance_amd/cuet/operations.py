@@ -23,6 +23,7 @@ import torch
 
 from .. import cue
 from ..cue import descriptors
+from .script import scriptable
 from .segmented_polynomial import SegmentedPolynomial
 from .transpose import TransposeIrrepsLayout, apply_layout
 
@@ -100,6 +101,7 @@ class _FlattenedUniform(torch.nn.Module):
                       output_indices=output_indices or {})
 
 
+@scriptable("with_weight")
 class ChannelWiseTensorProduct(torch.nn.Module):
     """``out[k u v] = w[u v] * sum_ij C[i j k] x1[i u] x2[j v]`` for every allowed irrep triple.
 
@@ -315,6 +317,7 @@ class ChannelWiseSphericalTensorProduct(torch.nn.Module):
         return apply_layout(self.transpose_out, out[0])
 
 
+@scriptable("fully_connected")
 class FullyConnectedTensorProduct(torch.nn.Module):
     """``out[k w] = sum_{u v i j} w[u v w] C[i j k] x1[i u] x2[j v]`` over every allowed irrep triple."""
 
@@ -426,6 +429,7 @@ class FullyConnectedTensorProduct(torch.nn.Module):
                 and x1.shape[0] == x2.shape[0] and dense.mul_ir_ready(x1.dtype))
 
 
+@scriptable("linear")
 class Linear(torch.nn.Module):
     """Equivariant linear map: one ``mul_in x mul_out`` weight block per pair of equal irreps, scaled ``1/sqrt(mul_in)``.
 
@@ -519,6 +523,7 @@ class Linear(torch.nn.Module):
         return apply_layout(self.transpose_out, out[0])
 
 
+@scriptable("contraction")
 class SymmetricContraction(torch.nn.Module):
     """Symmetric contraction of MACE (https://arxiv.org/abs/2206.07697): for every degree ``n`` up to
     ``contraction_degree`` the symmetric part of ``x ⊗ ... ⊗ x`` (``n`` factors) is mapped onto ``irreps_out`` with
@@ -599,6 +604,7 @@ class SymmetricContraction(torch.nn.Module):
         return apply_layout(self.transpose_out, out[0])
 
 
+@scriptable("vectors")
 class SphericalHarmonics(torch.nn.Module):
     """Spherical harmonics of 3-vectors: ``forward(vectors (batch, 3)) -> (batch, sum(2l+1))`` for the degrees ``ls``
     (ascending, unique); component normalisation, ``Y_1 = sqrt(3) x``.  ``normalize=True`` divides the vectors by their
@@ -622,6 +628,7 @@ class SphericalHarmonics(torch.nn.Module):
         return output
 
 
+@scriptable("rotation")
 class Rotation(torch.nn.Module):
     """Rotation of SO(3) / O(3) features (``cuequivariance_torch/operations/rotation.py:29-157`` in the reference):
     ``forward(gamma, beta, alpha, x)`` applies the rotation about y by ``gamma``, then about x by ``beta``, then about y by
@@ -688,6 +695,7 @@ def vector_to_euler_angles(vector: torch.Tensor):
     return beta.reshape(vector.shape[:-1]), alpha.reshape(vector.shape[:-1])
 
 
+@scriptable("x")
 class Inversion(torch.nn.Module):
     """Inversion ``x -> -x`` of O(3) features: every irrep times its parity (``operations/rotation.py:211-310`` in the
     reference)."""

@@ -21,6 +21,7 @@ import torch.nn as nn
 from .. import cue
 from ..tables import U1dTables
 from . import uniform_1d as u1d
+from .script import scriptable
 
 __all__ = ["SegmentedPolynomial", "SegmentedPolynomialFromUniform1d"]
 
@@ -181,6 +182,7 @@ class SegmentedPolynomialFromUniform1d(nn.Module):
         return u1d.run_plan(self._plan(math_dtype), batch_dim, index_buffer, batch_size, num_index, tensors)
 
 
+@scriptable("polynomial")
 class SegmentedPolynomial(nn.Module):
     """Executes a ``cue.SegmentedPolynomial`` on tensors of shape ``(batch | 1 | index range, operand_size)``.
 

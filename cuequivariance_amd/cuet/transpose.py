@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from .. import _lib, cue
+from .script import scriptable
 
 __all__ = ["TransposeSegments", "TransposeIrrepsLayout"]
 
@@ -88,6 +89,7 @@ class TransposeSegments(torch.nn.Module):
         return _Permute.apply(x, fwd, bwd)
 
 
+@scriptable("x")
 class TransposeIrrepsLayout(torch.nn.Module):
     """Change the layout of a tensor of the given irreps from ``source`` to ``target``."""
 
