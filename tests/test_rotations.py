@@ -211,3 +211,22 @@ def test_composition_of_descriptors_by_dot():
     with pytest.raises(ValueError):
         cue.segmented_polynomials.dot(y, x, (0, 1))
     assert hasattr(cue.group_theory, "clebsch_gordan") and cue.group_theory.descriptors is descriptors
+
+
+@pytest.mark.gpu
+def test_rotation_traced_as_a_whole(device):
+    """``torch.compile(fullgraph=True)`` and ``torch.export`` of ``cuet.Rotation`` (angle encodings in torch code, the polynomial
+    through the opaque uniform-1d operator) against the eager module."""
+    from cuequivariance_amd import cuet
+
+    irreps = cue.Irreps("O3", "4x0e+4x1o+4x2e")
+    rot = cuet.Rotation(irreps, layout=cue.ir_mul, device=device)
+    g = torch.Generator(device=device).manual_seed(7)
+    x = torch.randn(11, irreps.dim, device=device, generator=g)
+    a = torch.randn(3, 11, device=device, generator=g)
+    want = rot(a[0], a[1], a[2], x)
+    got = torch.compile(rot, fullgraph=True)(a[0], a[1], a[2], x)
+    assert (got - want).abs().max().item() <= 1e-6 * want.abs().max().item()
+    program = torch.export.export(rot, (a[0].clone(), a[1].clone(), a[2].clone(), x.clone()))
+    out = program.module()(a[0], a[1], a[2], x)
+    assert (out - want).abs().max().item() <= 1e-6 * want.abs().max().item()
